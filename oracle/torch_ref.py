@@ -1,0 +1,320 @@
+"""CPU oracle for the attention + RG-LRU step, restated with plain torch ops.
+
+TEST INFRASTRUCTURE ONLY.  Nothing that ships (the package, its kernels, its
+modules) may import this file; it exists so that tests, the smoke check and the
+CPU-baseline leg of the benchmark have an independent statement of what the
+reference computes.  Every function is written from the text of the reference
+and cites the lines it follows (paths relative to the reference checkout,
+``src/boost_and_broadside/``).
+
+All functions are pure: weights come in as a flat ``dict`` keyed by the
+reference's ``state_dict`` names, so the oracle shares no module code with the
+product.  Dtype behaviour is whatever torch's own type promotion gives for the
+dtypes passed in, which is exactly how the reference behaves under autocast:
+feed bf16 gate pre-activations and the sigmoids come out bf16, the decay
+``sigmoid(log_lambda) ** (c * r)`` promotes to fp32, and so on.
+
+How each function is pinned (see tests/test_oracle_pins.py):
+
+* ``sdpa_masked``      library routine (torch SDPA) + fp64 brute force
+                       (oracle/bruteforce.py) + closed forms (all-alive,
+                       single alive key, all dead => mean of V, dead-key
+                       perturbation invariance, permutation equivariance).
+* ``rglru_step``       closed forms from the recurrence (x=0, h=0, lambda=0
+                       with r=1, r=0 => clamp floor) + the C restatement.
+* ``temporal_step``    step == sequence, with the sequence path built on the
+                       library ``F.conv1d`` (fixes tap order and buffer order).
+* ``field_step``, ``block_step``, ``pack/unpack/reset``  invariants the
+                       reference's own tests state (fields ignore state, reset
+                       zeroes exactly the done environments, env-major rows).
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+CONV_TAPS = 4  # models/yemong/griffin.py:22
+
+
+# --------------------------------------------------------------------------
+# Level K: the two operations the HIP kernels replace
+# --------------------------------------------------------------------------
+
+def key_bias(alive: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """Additive key bias (B,1,1,NM) in ``dtype``: 0 where alive, finfo.min/2 where dead.
+
+    Follows models/yemong/attention.py:101-112.
+    """
+    keep = alive.reshape(alive.shape[0], 1, 1, alive.shape[-1]).to(dtype)
+    return (1.0 - keep) * (torch.finfo(dtype).min / 2)
+
+
+def sdpa_masked(qkv: torch.Tensor, alive: torch.Tensor | None, n_heads: int) -> torch.Tensor:
+    """Masked multi-head attention over one packed projection buffer.
+
+    ``qkv`` is (B, NM, 3*D) with columns [Q | K | V], each third split head-major
+    into ``n_heads`` runs of D/n_heads columns.  Returns (B, NM, D) with the heads
+    merged back head-major, i.e. the tensor the reference hands to ``out_proj``.
+    Follows models/yemong/attention.py:136-147 and :168.
+    """
+    B, NM, D3 = qkv.shape
+    D = D3 // 3
+    dh = D // n_heads
+    q, k, v = (t.reshape(B, NM, n_heads, dh).transpose(1, 2) for t in qkv.split(D, dim=-1))
+    bias = None if alive is None else key_bias(alive, q.dtype)
+    o = F.scaled_dot_product_attention(q, k, v, attn_mask=bias, dropout_p=0.0)
+    return o.transpose(1, 2).reshape(B, NM, D)
+
+
+def rglru_step(
+    x: torch.Tensor,
+    gates_pre: torch.Tensor,
+    log_lambda: torch.Tensor,
+    c: float,
+    h: torch.Tensor,
+) -> torch.Tensor:
+    """One RG-LRU update given the two gate pre-activations.
+
+    ``gates_pre`` is (R, 2*D): columns [0,D) are ``linear_a(x)``, columns [D,2D)
+    are ``linear_x(x)`` (bias included).  Returns the new state, which is also the
+    layer output.  Follows models/yemong/griffin.py:179-186 (identical to the T=1
+    scan, griffin.py:206-212 with :45-64 degenerating to ``a*h0 + b``).
+    """
+    D = x.shape[-1]
+    r = torch.sigmoid(gates_pre[..., :D])
+    i = torch.sigmoid(gates_pre[..., D:])
+    a = torch.sigmoid(log_lambda) ** (c * r)
+    g = torch.sqrt(torch.clamp((1.0 - a) * (1.0 + a), min=1e-6))
+    return a * h + g * (i * x)
+
+
+# --------------------------------------------------------------------------
+# Level M pieces (torch library ops around the two kernels)
+# --------------------------------------------------------------------------
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``nn.RMSNorm(D)`` with its default ``eps=None`` (=> finfo(x.dtype).eps)."""
+    return F.rms_norm(x, (x.shape[-1],), weight, None)
+
+
+def gated_mlp(p: dict, prefix: str, x: torch.Tensor) -> torch.Tensor:
+    """down(gelu(gate(x)) * up(x)); models/yemong/attention.py:21-37."""
+    gate = F.gelu(F.linear(x, p[prefix + "gate_proj.weight"]))
+    return F.linear(gate * F.linear(x, p[prefix + "up_proj.weight"]), p[prefix + "down_proj.weight"])
+
+
+def spatial_sublayer(p: dict, prefix: str, x: torch.Tensor, alive: torch.Tensor | None, n_heads: int) -> torch.Tensor:
+    """Pre-norm attention + FFN block without bullets; models/yemong/attention.py:76-99,114-169."""
+    n = rms_norm(x, p[prefix + "norm1.weight"])
+    merged = sdpa_masked(F.linear(n, p[prefix + "qkv.weight"]), alive, n_heads)
+    x = x + F.linear(merged, p[prefix + "out_proj.weight"])
+    return x + gated_mlp(p, prefix + "ffn.", rms_norm(x, p[prefix + "norm2.weight"]))
+
+
+def rglru_gates(p: dict, prefix: str, x: torch.Tensor) -> torch.Tensor:
+    """[linear_a(x) | linear_x(x)] as one (R, 2D) tensor; models/yemong/griffin.py:166-167."""
+    return torch.cat(
+        [
+            F.linear(x, p[prefix + "linear_a.weight"], p[prefix + "linear_a.bias"]),
+            F.linear(x, p[prefix + "linear_x.weight"], p[prefix + "linear_x.bias"]),
+        ],
+        dim=-1,
+    )
+
+
+def temporal_step(p: dict, prefix: str, x: torch.Tensor, h: torch.Tensor, conv_buf: torch.Tensor):
+    """Griffin temporal sublayer for one timestep.
+
+    x (R,D), h (R,D), conv_buf (R,3,D) oldest -> newest.  Returns
+    (x_out, h_new, conv_buf_new).  Follows models/yemong/griffin.py:269-286 with
+    T=1 and done_mask=None; the tap at weight index k multiplies padded[:, k]
+    (griffin.py:131-137), so the current input meets weight index 3.
+    """
+    n = rms_norm(x, p[prefix + "norm1.weight"])
+    b1 = F.linear(n, p[prefix + "linear1.weight"])
+    w = p[prefix + "conv.weight"].squeeze(1)  # (D, 4)
+    padded = torch.cat([conv_buf, b1.unsqueeze(1)], dim=1)  # (R, 4, D)
+    v = (padded * w.t().unsqueeze(0)).sum(dim=1) + p[prefix + "conv.bias"]
+    lam = p[prefix + "rg_lru.log_lambda"]
+    h_new = rglru_step(v, rglru_gates(p, prefix + "rg_lru.", v), lam, 8.0, h)
+    b2 = F.gelu(F.linear(n, p[prefix + "linear2.weight"]))
+    x1 = x + F.linear(h_new * b2, p[prefix + "linear_out.weight"])
+    x2 = x1 + gated_mlp(p, prefix + "gated_mlp.", rms_norm(x1, p[prefix + "norm2.weight"]))
+    return x2, h_new, padded[:, 1:, :]
+
+
+def temporal_sequence(
+    p: dict,
+    prefix: str,
+    x_seq: torch.Tensor,
+    h0: torch.Tensor,
+    conv_buf: torch.Tensor,
+    done: torch.Tensor | None = None,
+):
+    """Same sublayer over (R,T,D), written independently of ``temporal_step``.
+
+    The depthwise causal conv goes through the library ``F.conv1d`` (the reference
+    states its tap loop is that cross-correlation, griffin.py:131-134) and the
+    recurrence is a plain loop over T, so a wrong tap or buffer order in
+    ``temporal_step`` cannot hide here.  ``done`` (R,T) follows griffin.py:213-218:
+    done at t cuts the state (and the conv taps reaching back across it,
+    griffin.py:67-93) for steps after t.
+    """
+    R, T, D = x_seq.shape
+    n = rms_norm(x_seq, p[prefix + "norm1.weight"])
+    b1 = F.linear(n, p[prefix + "linear1.weight"])
+    padded = torch.cat([conv_buf, b1], dim=1)  # (R, T+3, D)
+    if done is None:
+        v = F.conv1d(padded.transpose(1, 2), p[prefix + "conv.weight"], p[prefix + "conv.bias"], groups=D)
+        v = v.transpose(1, 2)
+    else:
+        # episode id of every padded position; a tap contributes only inside one episode
+        starts = torch.zeros(R, T, dtype=torch.long)
+        starts[:, 1:] = done[:, :-1].long()
+        epi = torch.cat([torch.zeros(R, CONV_TAPS - 1, dtype=torch.long), starts.cumsum(1)], dim=1)
+        w = p[prefix + "conv.weight"].squeeze(1)
+        v = torch.zeros_like(b1)
+        for t in range(T):
+            for k in range(CONV_TAPS):
+                same = (epi[:, t + k] == epi[:, t + CONV_TAPS - 1]).to(b1.dtype).unsqueeze(-1)
+                v[:, t] = v[:, t] + padded[:, t + k] * w[:, k] * same
+        v = v + p[prefix + "conv.bias"]
+    lam = p[prefix + "rg_lru.log_lambda"]
+    gates = rglru_gates(p, prefix + "rg_lru.", v)
+    h, ys = h0, []
+    for t in range(T):
+        if done is not None and t > 0:
+            h = h * (~done[:, t - 1]).to(h.dtype).unsqueeze(-1)
+        h = rglru_step(v[:, t], gates[:, t], lam, 8.0, h)
+        ys.append(h)
+    y = torch.stack(ys, dim=1)
+    b2 = F.gelu(F.linear(n, p[prefix + "linear2.weight"]))
+    x1 = x_seq + F.linear(y * b2, p[prefix + "linear_out.weight"])
+    x2 = x1 + gated_mlp(p, prefix + "gated_mlp.", rms_norm(x1, p[prefix + "norm2.weight"]))
+    return x2, h, padded[:, -(CONV_TAPS - 1):, :]
+
+
+def field_step(p: dict, prefix: str, sub_weight: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """Temporal sublayer for state-free (field) tokens; models/yemong/griffin.py:288-317."""
+    n = rms_norm(x, p[prefix + "norm1.weight"])
+    b1 = F.linear(F.linear(n, p[prefix + "linear1.weight"]), sub_weight)
+    b2 = F.gelu(F.linear(n, p[prefix + "linear2.weight"]))
+    x1 = x + F.linear(b1 * b2, p[prefix + "linear_out.weight"])
+    return x1 + gated_mlp(p, prefix + "gated_mlp.", rms_norm(x1, p[prefix + "norm2.weight"]))
+
+
+def block_step(
+    p: dict,
+    prefix: str,
+    n_spatial: int,
+    n_temporal: int,
+    n_heads: int,
+    x: torch.Tensor,
+    alive: torch.Tensor,
+    h: torch.Tensor,
+    conv_buf: torch.Tensor,
+    n_rec: int | None = None,
+):
+    """One Yemong block for one timestep; models/yemong/griffin.py:376-417.
+
+    x (B,NM,D), alive (B,NM), h (n_temporal, B*n_rec, D), conv_buf
+    (n_temporal, B*n_rec, 3, D).  Recurrent rows are env-major (b*n_rec + n).
+    """
+    B, NM, D = x.shape
+    n_rec = NM if n_rec is None else n_rec
+    for s in range(n_spatial):
+        x = spatial_sublayer(p, f"{prefix}spatial.{s}.", x, alive, n_heads)
+    hs, cbs = [], []
+    for j in range(n_temporal):
+        tp = f"{prefix}temporal.{j}."
+        ships = x[:, :n_rec].reshape(B * n_rec, D)
+        out, h_new, cb_new = temporal_step(p, tp, ships, h[j], conv_buf[j])
+        parts = [out.reshape(B, n_rec, D)]
+        if NM > n_rec:
+            parts.append(field_step(p, tp, p[f"{prefix}field_sub.{j}.weight"], x[:, n_rec:]))
+        x = torch.cat(parts, dim=1)
+        hs.append(h_new)
+        cbs.append(cb_new)
+    if not hs:
+        return x, h[:0], conv_buf[:0]
+    return x, torch.stack(hs), torch.stack(cbs)
+
+
+def unpack_hidden(hidden: torch.Tensor, d_model: int):
+    """(L, R, 4D) -> h (L,R,D), conv_buf (L,R,3,D); models/yemong/policy.py:323-324."""
+    L, R, _ = hidden.shape
+    return hidden[:, :, :d_model], hidden[:, :, d_model:].reshape(L, R, CONV_TAPS - 1, d_model)
+
+
+def pack_hidden(h: torch.Tensor, conv_buf: torch.Tensor) -> torch.Tensor:
+    """Inverse of ``unpack_hidden``; models/yemong/policy.py:346-354."""
+    L, R, D = h.shape
+    return torch.cat([h, conv_buf.reshape(L, R, (CONV_TAPS - 1) * D)], dim=-1)
+
+
+def reset_hidden(hidden: torch.Tensor, done: torch.Tensor, n_rec: int) -> torch.Tensor:
+    """Zero every recurrent row of finished environments; models/yemong/policy.py:268-285."""
+    keep = (~done.repeat_interleave(n_rec)).to(hidden.dtype)
+    return hidden * keep[None, :, None]
+
+
+def trunk_step(
+    p: dict,
+    n_blocks: int,
+    n_spatial: int,
+    n_temporal: int,
+    n_heads: int,
+    x: torch.Tensor,
+    alive: torch.Tensor,
+    hidden: torch.Tensor,
+):
+    """The block loop of ``get_action_and_value``; models/yemong/policy.py:311-354."""
+    B, NM, D = x.shape
+    n_rec = hidden.shape[1] // B
+    h_all, cb_all = unpack_hidden(hidden, D)
+    hs, cbs = [], []
+    for i in range(n_blocks):
+        sl = slice(i * n_temporal, (i + 1) * n_temporal)
+        x, h_new, cb_new = block_step(
+            p, f"yemong_layers.{i}.", n_spatial, n_temporal, n_heads, x, alive, h_all[sl], cb_all[sl], n_rec
+        )
+        hs.append(h_new)
+        cbs.append(cb_new)
+    if not hs or hs[0].shape[0] == 0:
+        return x, hidden
+    return x, pack_hidden(torch.cat(hs), torch.cat(cbs))
+
+
+# --------------------------------------------------------------------------
+# The measured composition (two kernels + the four projections around them)
+# --------------------------------------------------------------------------
+
+def harness_step(p: dict, tokens: torch.Tensor, alive: torch.Tensor, state: torch.Tensor, n_heads: int = 4):
+    """Minimal attention + RG-LRU step on (B,NM,D) tokens.
+
+    ``p`` holds ``qkv.weight`` (3D,D), ``out_proj.weight`` (D,D), ``linear_a.*``,
+    ``linear_x.*`` and ``log_lambda``; ``state`` is (B*N, D) fp32 for the first N
+    tokens of every environment (ships); the trailing NM-N tokens (fields) skip
+    the recurrence as in models/yemong/griffin.py:406-413.
+    Returns (hidden (B,NM,D), new_state (B*N,D)).
+    """
+    B, NM, D = tokens.shape
+    N = state.shape[0] // B
+    u = F.linear(sdpa_masked(F.linear(tokens, p["qkv.weight"]), alive, n_heads), p["out_proj.weight"])
+    ships = u[:, :N].reshape(B * N, D)
+    h_new = rglru_step(ships, rglru_gates(p, "", ships), p["log_lambda"], 8.0, state)
+    y = h_new.to(u.dtype).reshape(B, N, D)
+    return torch.cat([y, u[:, N:]], dim=1), h_new
+
+
+def sigma_lambda_reference(d_model: int) -> torch.Tensor:
+    """log_lambda as the reference initialises it; models/yemong/griffin.py:165."""
+    return torch.linspace(0.0, 4.0, d_model)
+
+
+def softplus_neg(x: float) -> float:
+    """log(sigmoid(x)) for a python float, used by closed-form checks."""
+    return -math.log1p(math.exp(-x))

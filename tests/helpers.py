@@ -1,0 +1,83 @@
+"""Shared test utilities: seeded weights keyed by the reference's state_dict names, error metrics."""
+
+from __future__ import annotations
+
+import math
+import os
+import sys
+
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def _xavier(gen: torch.Generator, out_f: int, in_f: int) -> torch.Tensor:
+    bound = math.sqrt(6.0 / (in_f + out_f))
+    return (torch.rand(out_f, in_f, generator=gen) * 2 - 1) * bound
+
+
+def _uniform(gen: torch.Generator, n: int, fan_in: int) -> torch.Tensor:
+    bound = 1.0 / math.sqrt(fan_in)
+    return (torch.rand(n, generator=gen) * 2 - 1) * bound
+
+
+def spatial_params(gen: torch.Generator, prefix: str, D: int) -> dict:
+    """Weights of one spatial sublayer (names: models/yemong/attention.py:60-74)."""
+    return {
+        prefix + "norm1.weight": 1.0 + 0.1 * torch.randn(D, generator=gen),
+        prefix + "qkv.weight": _xavier(gen, 3 * D, D),
+        prefix + "out_proj.weight": _xavier(gen, D, D),
+        prefix + "norm2.weight": 1.0 + 0.1 * torch.randn(D, generator=gen),
+        prefix + "ffn.gate_proj.weight": _xavier(gen, 4 * D, D),
+        prefix + "ffn.up_proj.weight": _xavier(gen, 4 * D, D),
+        prefix + "ffn.down_proj.weight": _xavier(gen, D, 4 * D),
+    }
+
+
+def temporal_params(gen: torch.Generator, prefix: str, D: int) -> dict:
+    """Weights of one temporal sublayer (names: models/yemong/griffin.py:165-167,238-247)."""
+    return {
+        prefix + "norm1.weight": 1.0 + 0.1 * torch.randn(D, generator=gen),
+        prefix + "linear1.weight": _xavier(gen, D, D),
+        prefix + "conv.weight": 0.5 * torch.randn(D, 1, 4, generator=gen),
+        prefix + "conv.bias": 0.1 * torch.randn(D, generator=gen),
+        prefix + "rg_lru.log_lambda": torch.linspace(0.0, 4.0, D),
+        prefix + "rg_lru.linear_a.weight": _xavier(gen, D, D),
+        prefix + "rg_lru.linear_a.bias": _uniform(gen, D, D),
+        prefix + "rg_lru.linear_x.weight": _xavier(gen, D, D),
+        prefix + "rg_lru.linear_x.bias": _uniform(gen, D, D),
+        prefix + "linear2.weight": _xavier(gen, D, D),
+        prefix + "linear_out.weight": _xavier(gen, D, D),
+        prefix + "norm2.weight": 1.0 + 0.1 * torch.randn(D, generator=gen),
+        prefix + "gated_mlp.gate_proj.weight": _xavier(gen, 4 * D, D),
+        prefix + "gated_mlp.up_proj.weight": _xavier(gen, 4 * D, D),
+        prefix + "gated_mlp.down_proj.weight": _xavier(gen, D, 4 * D),
+    }
+
+
+def block_params(gen: torch.Generator, prefix: str, D: int, n_spatial: int, n_temporal: int) -> dict:
+    """Weights of one Yemong block (names: models/yemong/griffin.py:340-368)."""
+    p: dict = {}
+    for s in range(n_spatial):
+        p.update(spatial_params(gen, f"{prefix}spatial.{s}.", D))
+    for j in range(n_temporal):
+        p.update(temporal_params(gen, f"{prefix}temporal.{j}.", D))
+        # the reference starts field_sub at identity; perturb it so a wrong wiring shows
+        p[f"{prefix}field_sub.{j}.weight"] = torch.eye(D) + 0.05 * torch.randn(D, D, generator=gen)
+    return p
+
+
+def trunk_params(seed: int, D: int, n_blocks: int, n_spatial: int, n_temporal: int) -> dict:
+    gen = torch.Generator().manual_seed(seed)
+    p: dict = {}
+    for i in range(n_blocks):
+        p.update(block_params(gen, f"yemong_layers.{i}.", D, n_spatial, n_temporal))
+    return p
+
+
+def max_rel(y: torch.Tensor, ref: torch.Tensor) -> float:
+    """max|y - ref| / max|ref| over the whole tensor (the parity metric of the step)."""
+    y, ref = y.double(), ref.double()
+    return float((y - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
