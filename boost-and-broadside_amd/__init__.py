@@ -1,0 +1,30 @@
+"""MI355X (gfx950) implementation of the Yemong trunk's per-timestep hot path.
+
+Masked multi-head attention over each environment's entity tokens followed by the
+per-entity RG-LRU recurrence step, as hand-written HIP kernels behind a C ABI
+(``include/bnb_amd.h`` -> ``_lib/libbnb_amd.so``), plus torch modules that keep the
+reference policy's layer interfaces and ``state_dict`` names.
+
+    ops       sdpa_masked, rglru_step                       (the two kernels)
+    trunk     TransformerBlock, RGLRU, GriffinTemporalBlock, YemongBlock, YemongTrunk
+    harness   benchmark workloads, traffic model, AttnRglruStep
+    build     compiles the HIP sources
+"""
+
+from . import _native, harness, ops, trunk
+from .ops import rglru_step, sdpa_masked
+from .trunk import (
+    CONV_KERNEL,
+    GatedMLP,
+    GriffinTemporalBlock,
+    ModelConfig,
+    RGLRU,
+    TransformerBlock,
+    YemongBlock,
+    YemongTrunk,
+)
+
+__all__ = [
+    "CONV_KERNEL", "GatedMLP", "GriffinTemporalBlock", "ModelConfig", "RGLRU", "TransformerBlock",
+    "YemongBlock", "YemongTrunk", "rglru_step", "sdpa_masked", "ops", "trunk", "harness",
+]

@@ -1,0 +1,60 @@
+"""Compiles the HIP sources of this package into ``_lib/libbnb_amd.so`` for gfx950.
+
+Run as ``python boost-and-broadside_amd/build.py``; also called by the repository's
+build entry point.  hipcc cross-compiles, so no GPU is needed.
+"""
+
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG_DIR, "csrc")
+INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
+LIB_DIR = os.path.join(PKG_DIR, "_lib")
+LIB_PATH = os.path.join(LIB_DIR, "libbnb_amd.so")
+SOURCES = ("abi.hip", "rglru_step.hip", "sdpa_masked.hip")
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-fno-gpu-rdc",
+    # packed-fp32 VALU forms are kept out of the generated code on purpose
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def build(verbose: bool = False) -> str:
+    """Compile every source and link the shared library; returns its path."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    os.makedirs(LIB_DIR, exist_ok=True)
+    objects = []
+    for src in SOURCES:
+        obj = os.path.join(LIB_DIR, src.replace(".hip", ".o"))
+        cmd = [hipcc, *HIPCC_FLAGS, "-I", INCLUDE, "-I", CSRC, "-c", os.path.join(CSRC, src), "-o", obj]
+        _run(cmd, verbose)
+        objects.append(obj)
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objects], verbose)
+    return LIB_PATH
+
+
+def _run(cmd: list[str], verbose: bool) -> None:
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(line for line in proc.stderr.splitlines() if noise not in line)
+    if proc.returncode != 0:
+        raise RuntimeError(f"command failed ({proc.returncode}): {' '.join(cmd)}\n{err}")
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

@@ -1,0 +1,92 @@
+// Shared device helpers for the gfx950 kernels: raw bf16 handling and vector types.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "bnb_amd.h"
+
+namespace bnb {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// bf16 is carried as raw 16-bit patterns outside the MFMA operands.
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+
+// Round-to-nearest-even fp32 -> bf16, the rounding torch applies when it stores bf16.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float v)
+{
+    __bf16 b = (__bf16)v;  // v_cvt_pk_bf16_f32 on gfx950
+    return (uint32_t)__builtin_bit_cast(uint16_t, b);
+}
+
+__device__ __forceinline__ float round_to_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
+{
+    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+// Eight consecutive channels of one row, widened to fp32.
+struct Row8 {
+    float v[8];
+};
+
+__device__ __forceinline__ Row8 load8(const float *p)
+{
+    const f32x4 a = *reinterpret_cast<const f32x4 *>(p);
+    const f32x4 b = *reinterpret_cast<const f32x4 *>(p + 4);
+    return Row8{{a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w}};
+}
+
+__device__ __forceinline__ Row8 load8(const uint16_t *p)
+{
+    const u32x4 w = *reinterpret_cast<const u32x4 *>(p);
+    Row8 r;
+    r.v[0] = __uint_as_float(w.x << 16);
+    r.v[1] = __uint_as_float(w.x & 0xffff0000u);
+    r.v[2] = __uint_as_float(w.y << 16);
+    r.v[3] = __uint_as_float(w.y & 0xffff0000u);
+    r.v[4] = __uint_as_float(w.z << 16);
+    r.v[5] = __uint_as_float(w.z & 0xffff0000u);
+    r.v[6] = __uint_as_float(w.w << 16);
+    r.v[7] = __uint_as_float(w.w & 0xffff0000u);
+    return r;
+}
+
+__device__ __forceinline__ void store8(float *p, const Row8 &r)
+{
+    *reinterpret_cast<f32x4 *>(p) = f32x4{r.v[0], r.v[1], r.v[2], r.v[3]};
+    *reinterpret_cast<f32x4 *>(p + 4) = f32x4{r.v[4], r.v[5], r.v[6], r.v[7]};
+}
+
+__device__ __forceinline__ void store8(uint16_t *p, const Row8 &r)
+{
+    *reinterpret_cast<u32x4 *>(p) = u32x4{pack_bf16x2(r.v[0], r.v[1]), pack_bf16x2(r.v[2], r.v[3]),
+                                          pack_bf16x2(r.v[4], r.v[5]), pack_bf16x2(r.v[6], r.v[7])};
+}
+
+__device__ __forceinline__ float load1(const float *p) { return *p; }
+__device__ __forceinline__ float load1(const uint16_t *p) { return bf16_bits_to_f32(*p); }
+__device__ __forceinline__ void store1(float *p, float v) { *p = v; }
+__device__ __forceinline__ void store1(uint16_t *p, float v) { *p = (uint16_t)f32_to_bf16_bits(v); }
+
+template <typename T>
+struct is_bf16 {
+    static constexpr bool value = false;
+};
+template <>
+struct is_bf16<uint16_t> {
+    static constexpr bool value = true;
+};
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace bnb

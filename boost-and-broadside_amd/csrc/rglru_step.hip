@@ -1,0 +1,186 @@
+// RG-LRU recurrence step for gfx950: one coalesced pass over the entity rows.
+//
+// Per element (reference: models/yemong/griffin.py:179-185):
+//   r = sigmoid(ga), i = sigmoid(gx), a = sigmoid(lambda)^(c r),
+//   h' = a h + sqrt(max((1-a)(1+a), 1e-6)) (i x)
+// The kernel is bound by HBM traffic (x, two gate pre-activations and the old state in,
+// the new state and its optional low-precision copy out), so the design is a plain
+// streaming loop: every lane owns 8 consecutive channels of a row, moves them with
+// 16-byte accesses and keeps everything between load and store in registers.
+
+#include "common.h"
+
+namespace bnb {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kRglruThreads = 256;
+constexpr int kRglruRowsInFlight = 4;  // rows each lane has loads outstanding for
+
+__device__ __forceinline__ float fast_sigmoid(float v)
+{
+    // 1 / (1 + 2^(-v log2 e)); v_exp_f32 and v_rcp_f32 are 1-ulp approximations
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-kLog2e * v));
+}
+
+// log2(sigmoid(lambda)) computed with the precise library routines (once per block).
+__device__ __forceinline__ float log2_sigmoid(float lam) { return -log1pf(expf(-lam)) * kLog2e; }
+
+template <bool G_BF16, bool X_BF16>
+__device__ __forceinline__ float rglru_element(float x, float ga, float gx, float l2sig, float c, float h)
+{
+    float r = fast_sigmoid(ga);
+    float i = fast_sigmoid(gx);
+    float cr = c * r;
+    if (G_BF16) {
+        // autocast keeps the sigmoid outputs and the python-scalar product c*r in bf16
+        r = round_to_bf16(r);
+        i = round_to_bf16(i);
+        cr = round_to_bf16(c * r);
+    }
+    const float a = __builtin_amdgcn_exp2f(cr * l2sig);
+    const float gate = __builtin_amdgcn_sqrtf(fmaxf((1.0f - a) * (1.0f + a), 1e-6f));
+    float ix = i * x;
+    if (G_BF16 && X_BF16) ix = round_to_bf16(ix);
+    return a * h + gate * ix;
+}
+
+template <typename XT, typename GT, typename YT, bool HAS_Y>
+__global__ __launch_bounds__(kRglruThreads) void rglru_step_vec8_kernel(
+    const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
+    const float *h_in, int64_t h_in_stride, float *h_out, int64_t h_out_stride, YT *__restrict__ y,
+    int64_t R, int D, int rows_per_pass)
+{
+    extern __shared__ float s_l2sig[];  // D entries
+    for (int d = threadIdx.x; d < D; d += kRglruThreads) s_l2sig[d] = log2_sigmoid(log_lambda[d]);
+    __syncthreads();
+
+    const int vecs_per_row = D >> 3;
+    const int local_row = threadIdx.x / vecs_per_row;
+    if (local_row >= rows_per_pass) return;
+    const int d0 = (threadIdx.x - local_row * vecs_per_row) << 3;
+
+    float l2sig[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) l2sig[e] = s_l2sig[d0 + e];
+
+    const int64_t block_rows = (int64_t)rows_per_pass * kRglruRowsInFlight;
+    const int64_t row0 = (int64_t)blockIdx.x * block_rows + local_row;
+
+    Row8 xv[kRglruRowsInFlight], ga[kRglruRowsInFlight], gx[kRglruRowsInFlight], hv[kRglruRowsInFlight];
+#pragma unroll
+    for (int k = 0; k < kRglruRowsInFlight; ++k) {
+        const int64_t row = row0 + (int64_t)k * rows_per_pass;
+        if (row < R) {
+            xv[k] = load8(x + row * D + d0);
+            ga[k] = load8(gates + row * 2 * D + d0);
+            gx[k] = load8(gates + row * 2 * D + D + d0);
+            hv[k] = load8(h_in + row * h_in_stride + d0);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kRglruRowsInFlight; ++k) {
+        const int64_t row = row0 + (int64_t)k * rows_per_pass;
+        if (row < R) {
+            Row8 out;
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                out.v[e] = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(
+                    xv[k].v[e], ga[k].v[e], gx[k].v[e], l2sig[e], c, hv[k].v[e]);
+            store8(h_out + row * h_out_stride + d0, out);
+            if (HAS_Y) store8(y + row * D + d0, out);
+        }
+    }
+}
+
+// Any D, any alignment: one lane per element.
+template <typename XT, typename GT, typename YT, bool HAS_Y>
+__global__ __launch_bounds__(kRglruThreads) void rglru_step_scalar_kernel(
+    const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
+    const float *h_in, int64_t h_in_stride, float *h_out, int64_t h_out_stride, YT *__restrict__ y,
+    int64_t R, int D)
+{
+    const int64_t idx = (int64_t)blockIdx.x * kRglruThreads + threadIdx.x;
+    if (idx >= R * D) return;
+    const int64_t row = idx / D;
+    const int d = (int)(idx - row * D);
+    const float out = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(
+        load1(x + idx), load1(gates + row * 2 * D + d), load1(gates + row * 2 * D + D + d),
+        log2_sigmoid(log_lambda[d]), c, h_in[row * h_in_stride + d]);
+    h_out[row * h_out_stride + d] = out;
+    if (HAS_Y) store1(y + idx, out);
+}
+
+template <typename XT, typename GT, typename YT, bool HAS_Y>
+static int launch_rglru(const void *x, const void *gates, const float *log_lambda, float c, const float *h_in,
+                        int64_t h_in_stride, float *h_out, int64_t h_out_stride, void *y, int64_t R, int D,
+                        hipStream_t stream)
+{
+    const bool vec = (D % 8 == 0) && (D / 8 <= kRglruThreads) && aligned16(x) && aligned16(gates) &&
+                     aligned16(h_in) && aligned16(h_out) && (!HAS_Y || aligned16(y)) &&
+                     (h_in_stride % 4 == 0) && (h_out_stride % 4 == 0);
+    if (vec) {
+        const int rows_per_pass = kRglruThreads / (D / 8);
+        const int64_t block_rows = (int64_t)rows_per_pass * kRglruRowsInFlight;
+        const int64_t blocks = (R + block_rows - 1) / block_rows;
+        if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL((rglru_step_vec8_kernel<XT, GT, YT, HAS_Y>), dim3((unsigned)blocks),
+                           dim3(kRglruThreads), (size_t)D * sizeof(float), stream, (const XT *)x,
+                           (const GT *)gates, log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y,
+                           R, D, rows_per_pass);
+    } else {
+        const int64_t blocks = (R * D + kRglruThreads - 1) / kRglruThreads;
+        if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL((rglru_step_scalar_kernel<XT, GT, YT, HAS_Y>), dim3((unsigned)blocks),
+                           dim3(kRglruThreads), 0, stream, (const XT *)x, (const GT *)gates, log_lambda, c,
+                           h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D);
+    }
+    return (int)hipGetLastError();
+}
+
+template <typename XT, typename GT>
+static int dispatch_y(const void *x, const void *gates, const float *log_lambda, float c, const float *h_in,
+                      int64_t h_in_stride, float *h_out, int64_t h_out_stride, void *y, int y_dtype, int64_t R,
+                      int D, hipStream_t stream)
+{
+    if (y == nullptr)
+        return launch_rglru<XT, GT, float, false>(x, gates, log_lambda, c, h_in, h_in_stride, h_out,
+                                                  h_out_stride, nullptr, R, D, stream);
+    if (y_dtype == BNB_F32)
+        return launch_rglru<XT, GT, float, true>(x, gates, log_lambda, c, h_in, h_in_stride, h_out,
+                                                 h_out_stride, y, R, D, stream);
+    return launch_rglru<XT, GT, uint16_t, true>(x, gates, log_lambda, c, h_in, h_in_stride, h_out,
+                                                h_out_stride, y, R, D, stream);
+}
+
+}  // namespace bnb
+
+extern "C" int bnb_rglru_step_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
+                                  const float *log_lambda, float c, const float *h_in,
+                                  int64_t h_in_row_stride, float *h_out, int64_t h_out_row_stride, void *y,
+                                  int y_dtype, int64_t R, int D, void *stream)
+{
+    using namespace bnb;
+    if (R < 0 || D < 1) return BNB_ERR_BAD_SHAPE;
+    if (R == 0) return 0;
+    if (!x || !gates_pre || !log_lambda || !h_in || !h_out) return BNB_ERR_NULL_POINTER;
+    if ((x_dtype != BNB_F32 && x_dtype != BNB_BF16) || (g_dtype != BNB_F32 && g_dtype != BNB_BF16) ||
+        (y && y_dtype != BNB_F32 && y_dtype != BNB_BF16))
+        return BNB_ERR_BAD_DTYPE;
+    if (h_in_row_stride < D || h_out_row_stride < D) return BNB_ERR_BAD_SHAPE;
+    if ((reinterpret_cast<uintptr_t>(h_in) | reinterpret_cast<uintptr_t>(h_out) |
+         reinterpret_cast<uintptr_t>(log_lambda)) & 3u)
+        return BNB_ERR_MISALIGNED;
+    hipStream_t s = (hipStream_t)stream;
+    const bool xb = x_dtype == BNB_BF16, gb = g_dtype == BNB_BF16;
+    if (!xb && !gb)
+        return dispatch_y<float, float>(x, gates_pre, log_lambda, c, h_in, h_in_row_stride, h_out,
+                                        h_out_row_stride, y, y_dtype, R, D, s);
+    if (xb && gb)
+        return dispatch_y<uint16_t, uint16_t>(x, gates_pre, log_lambda, c, h_in, h_in_row_stride, h_out,
+                                              h_out_row_stride, y, y_dtype, R, D, s);
+    if (!xb && gb)
+        return dispatch_y<float, uint16_t>(x, gates_pre, log_lambda, c, h_in, h_in_row_stride, h_out,
+                                           h_out_row_stride, y, y_dtype, R, D, s);
+    return dispatch_y<uint16_t, float>(x, gates_pre, log_lambda, c, h_in, h_in_row_stride, h_out,
+                                       h_out_row_stride, y, y_dtype, R, D, s);
+}

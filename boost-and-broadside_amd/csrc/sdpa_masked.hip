@@ -1,0 +1,464 @@
+// Masked multi-head attention over each environment's entity tokens, for gfx950.
+//
+// out[b,i,h,:] = sum_j softmax_j(q[b,i,h].k[b,j,h] / sqrt(dh) + bias[b,j]) v[b,j,h,:]
+// (reference: models/yemong/attention.py:101-112,136-147,168).  The additive bias of the
+// reference (0 for a live key, finfo.min/2 for a dead one) has two exact consequences that
+// the kernels implement directly instead of adding a huge constant:
+//   * an environment with at least one live key gives every dead key weight exactly 0, so
+//     dead keys are dropped from the key list before any arithmetic (their K/V rows are
+//     never even read);
+//   * an environment with no live key has every score rounded to the same constant, i.e.
+//     an exactly uniform softmax over ALL keys: the output is the mean of V.
+// Queries are never masked.
+//
+// Two kernels:
+//   sdpa_valu_kernel   any dtype, dh in {8,16,32,64}, any NM that fits LDS; one lane per
+//                      (environment, head, query) row, K/V of a group of environments
+//                      staged in LDS as fp32, chunked online softmax.  This is the 4v4 /
+//                      8v11 path (NM < 32) and the fp32 path.
+//   sdpa_mfma_kernel   bf16, dh = 32, 32 <= NM <= 160; one wavefront per (environment,
+//                      head); S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16_bf16 so
+//                      that the softmax reductions over keys stay inside a lane.
+
+#include "common.h"
+
+namespace bnb {
+
+constexpr float kLog2eA = 1.4426950408889634f;
+constexpr int kValuThreads = 256;
+constexpr int kValuEnvPad = 16;   // floats between environments in LDS (bank spreading)
+constexpr int kValuHeadPad = 4;   // floats after every head row in LDS (bank spreading)
+
+// ------------------------------------------------------------------------------------
+// VALU kernel
+// ------------------------------------------------------------------------------------
+
+// LDS: K then V, each [G][NM][nh][DH + pad] fp32 (+ env pad), then alive bytes [G][NM],
+// then one "has a live key" flag per environment.
+template <typename T, int DH>
+__global__ __launch_bounds__(kValuThreads) void sdpa_valu_kernel(
+    const T *__restrict__ qkv, int64_t row_stride, const uint8_t *__restrict__ alive, T *__restrict__ out,
+    int B, int NM, int H, int G, int nh, float scale_log2e)
+{
+    extern __shared__ __align__(16) unsigned char s_raw[];
+    constexpr int HP = DH + kValuHeadPad;
+    const int D = H * DH;
+    const int env_pitch = NM * nh * HP + kValuEnvPad;  // floats
+    float *s_k = reinterpret_cast<float *>(s_raw);
+    float *s_v = s_k + (size_t)G * env_pitch;
+    uint8_t *s_alive = reinterpret_cast<uint8_t *>(s_v + (size_t)G * env_pitch);
+    int *s_any = reinterpret_cast<int *>(s_alive + (((size_t)G * NM + 15) & ~(size_t)15));
+
+    const int env0 = blockIdx.x * G;
+    const int h0 = blockIdx.y * nh;
+    const int tid = threadIdx.x;
+
+    if (tid < G) s_any[tid] = (alive == nullptr) ? 1 : 0;
+    __syncthreads();
+
+    // alive bytes (benign race on s_any: every writer stores 1)
+    for (int idx = tid; idx < G * NM; idx += kValuThreads) {
+        const int g = idx / NM;
+        const int env = env0 + g;
+        uint8_t a = 1;
+        if (alive != nullptr) a = (env < B) ? alive[(int64_t)env * NM + (idx - g * NM)] : 1;
+        s_alive[idx] = a;
+        if (a) s_any[g] = 1;
+    }
+
+    // K and V tiles, 8 elements per lane per trip
+    constexpr int V8 = DH / 8;
+    const int per_mat = G * NM * nh * V8;
+    for (int idx = tid; idx < 2 * per_mat; idx += kValuThreads) {
+        const int mat = idx / per_mat;
+        int rem = idx - mat * per_mat;
+        const int c8 = rem % V8;
+        rem /= V8;
+        const int hh = rem % nh;
+        rem /= nh;
+        const int j = rem % NM;
+        const int g = rem / NM;
+        const int env = env0 + g;
+        Row8 r;
+        if (env < B) {
+            r = load8(qkv + ((int64_t)env * NM + j) * row_stride + (1 + mat) * D + (h0 + hh) * DH + c8 * 8);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) r.v[e] = 0.0f;
+        }
+        float *dst = (mat ? s_v : s_k) + (size_t)g * env_pitch + (j * nh + hh) * HP + c8 * 8;
+        *reinterpret_cast<f32x4 *>(dst) = f32x4{r.v[0], r.v[1], r.v[2], r.v[3]};
+        *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{r.v[4], r.v[5], r.v[6], r.v[7]};
+    }
+    __syncthreads();
+
+    const int rows = G * nh * NM;
+    for (int row = tid; row < rows; row += kValuThreads) {
+        const int g = row / (nh * NM);
+        const int rem = row - g * (nh * NM);
+        const int hh = rem / NM;
+        const int i = rem - hh * NM;
+        const int env = env0 + g;
+        if (env >= B) continue;
+
+        float q[DH];
+        const T *qp = qkv + ((int64_t)env * NM + i) * row_stride + (h0 + hh) * DH;
+#pragma unroll
+        for (int c8 = 0; c8 < V8; ++c8) {
+            const Row8 r = load8(qp + c8 * 8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) q[c8 * 8 + e] = r.v[e] * scale_log2e;
+        }
+
+        const bool any = s_any[g] != 0;
+        const uint8_t *al = s_alive + g * NM;
+        const float *kbase = s_k + (size_t)g * env_pitch + hh * HP;
+        const float *vbase = s_v + (size_t)g * env_pitch + hh * HP;
+
+        float m = -INFINITY, l = 0.0f;
+        float o[DH];
+#pragma unroll
+        for (int d = 0; d < DH; ++d) o[d] = 0.0f;
+
+        for (int j0 = 0; j0 < NM; j0 += 4) {
+            float s[4];
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                const int j = j0 + jj;
+                s[jj] = -INFINITY;
+                if (j < NM) {
+                    const float *kr = kbase + (size_t)j * nh * HP;
+                    float dot = 0.0f;
+#pragma unroll
+                    for (int d4 = 0; d4 < DH / 4; ++d4) {
+                        const f32x4 kv = *reinterpret_cast<const f32x4 *>(kr + d4 * 4);
+                        dot = fmaf(q[d4 * 4 + 0], kv.x, dot);
+                        dot = fmaf(q[d4 * 4 + 1], kv.y, dot);
+                        dot = fmaf(q[d4 * 4 + 2], kv.z, dot);
+                        dot = fmaf(q[d4 * 4 + 3], kv.w, dot);
+                    }
+                    s[jj] = any ? (al[j] ? dot : -INFINITY) : 0.0f;
+                }
+            }
+            const float m_new = fmaxf(fmaxf(m, fmaxf(s[0], s[1])), fmaxf(s[2], s[3]));
+            if (m_new == -INFINITY) continue;  // nothing live seen yet
+            const float alpha = __builtin_amdgcn_exp2f(m - m_new);  // 0 when m = -inf
+            l *= alpha;
+#pragma unroll
+            for (int d = 0; d < DH; ++d) o[d] *= alpha;
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                const int j = j0 + jj;
+                if (j < NM) {
+                    const float p = __builtin_amdgcn_exp2f(s[jj] - m_new);
+                    l += p;
+                    const float *vr = vbase + (size_t)j * nh * HP;
+#pragma unroll
+                    for (int d4 = 0; d4 < DH / 4; ++d4) {
+                        const f32x4 vv = *reinterpret_cast<const f32x4 *>(vr + d4 * 4);
+                        o[d4 * 4 + 0] = fmaf(p, vv.x, o[d4 * 4 + 0]);
+                        o[d4 * 4 + 1] = fmaf(p, vv.y, o[d4 * 4 + 1]);
+                        o[d4 * 4 + 2] = fmaf(p, vv.z, o[d4 * 4 + 2]);
+                        o[d4 * 4 + 3] = fmaf(p, vv.w, o[d4 * 4 + 3]);
+                    }
+                }
+            }
+            m = m_new;
+        }
+
+        const float inv_l = 1.0f / l;
+        T *op = out + ((int64_t)env * NM + i) * D + (h0 + hh) * DH;
+#pragma unroll
+        for (int c8 = 0; c8 < V8; ++c8) {
+            Row8 r;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) r.v[e] = o[c8 * 8 + e] * inv_l;
+            store8(op + c8 * 8, r);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// MFMA kernel (bf16, dh = 32)
+// ------------------------------------------------------------------------------------
+//
+// v_mfma_f32_32x32x16_bf16, wave64: lane = 32*half + m.
+//   A (32 x 16): lane supplies row m,    contraction slots 8*half .. 8*half+7
+//   B (16 x 32): lane supplies column m, contraction slots 8*half .. 8*half+7
+//   D (32 x 32): lane holds column m, rows 8*(v/4) + 4*half + (v%4) for v = 0..15
+// S^T block (keys x queries) = K_blk (A) * Q_blk^T (B): a lane ends up with 16 scores of
+// ONE query per key block, so max and sum over keys are in-lane plus one exchange between
+// the two halves.  O^T (dh x queries) = V^T (A) * P^T (B): the probabilities a lane holds
+// are exactly the B operand it must supply, provided the A operand (V^T from LDS) lists the
+// keys in the same order: slot e of MFMA (kb,t) is key 32*kb + 16*t + 8*(e/4) + 4*half + e%4.
+
+constexpr int kDh = 32;
+
+template <int NKB>
+__global__ __launch_bounds__(kWave) void sdpa_mfma_kernel(
+    const uint16_t *__restrict__ qkv, int64_t row_stride, const uint8_t *__restrict__ alive,
+    uint16_t *__restrict__ out, int B, int NM, int H, float scale_log2e)
+{
+    constexpr int KCAP = NKB * 32;
+    constexpr int VP = KCAP + 4;  // halfs per V^T row: 8-byte aligned, bank-spread
+    __shared__ __align__(16) uint16_t s_vt[kDh * VP];
+    __shared__ uint16_t s_kidx[KCAP];
+
+    // Work-groups are dealt round-robin to the 8 XCDs; hand each XCD a contiguous run of
+    // (environment, head) pairs so the 4 heads of an environment share one L2.
+    const int chunk = gridDim.x >> 3;
+    const int logical = (blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
+    if (logical >= B * H) return;
+    const int env = logical / H;
+    const int head = logical - env * H;
+    const int D = H * kDh;
+
+    const int lane = threadIdx.x;
+    const int m = lane & 31;
+    const int half = lane >> 5;
+
+    // ---- compacted list of live keys (all keys when none is alive) ----
+    int cnt = 0;
+    for (int base = 0; base < NM; base += kWave) {
+        const int key = base + lane;
+        bool a = key < NM;
+        if (a && alive != nullptr) a = alive[(int64_t)env * NM + key] != 0;
+        const uint64_t mask = __ballot(a);
+        const int before = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
+                                                     __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+        if (a) s_kidx[cnt + before] = (uint16_t)key;
+        cnt += __popcll(mask);
+    }
+    const bool uniform = (cnt == 0);
+    if (uniform) {
+        cnt = NM;
+        for (int key = lane; key < NM; key += kWave) s_kidx[key] = (uint16_t)key;
+    }
+    __syncthreads();
+    const int nkb = (cnt + 31) >> 5;
+
+    const uint16_t *env_base = qkv + (int64_t)env * NM * row_stride;
+
+    // ---- V^T into LDS: lane -> (position pos, 8 channels) ----
+    for (int pos0 = 0; pos0 < nkb * 32; pos0 += 16) {
+        const int pos = pos0 + (lane >> 2);
+        const int c8 = (lane & 3) * 8;
+        u32x4 w = {0u, 0u, 0u, 0u};
+        if (pos < cnt) {
+            const int key = s_kidx[pos];
+            w = *reinterpret_cast<const u32x4 *>(env_base + (int64_t)key * row_stride + 2 * D + head * kDh + c8);
+        }
+        uint16_t *dst = s_vt + c8 * VP + pos;
+        dst[0 * VP] = (uint16_t)(w.x & 0xffffu);
+        dst[1 * VP] = (uint16_t)(w.x >> 16);
+        dst[2 * VP] = (uint16_t)(w.y & 0xffffu);
+        dst[3 * VP] = (uint16_t)(w.y >> 16);
+        dst[4 * VP] = (uint16_t)(w.z & 0xffffu);
+        dst[5 * VP] = (uint16_t)(w.z >> 16);
+        dst[6 * VP] = (uint16_t)(w.w & 0xffffu);
+        dst[7 * VP] = (uint16_t)(w.w >> 16);
+    }
+
+    // ---- K operand in registers: row = key position, 8 channels per half per t ----
+    bf16x8 ka[NKB][2];
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb) {
+        u32x4 w0 = {0u, 0u, 0u, 0u}, w1 = {0u, 0u, 0u, 0u};
+        const int pos = kb * 32 + m;
+        if (kb < nkb && pos < cnt) {
+            const int key = s_kidx[pos];
+            const uint16_t *kp = env_base + (int64_t)key * row_stride + D + head * kDh + half * 8;
+            w0 = *reinterpret_cast<const u32x4 *>(kp);
+            w1 = *reinterpret_cast<const u32x4 *>(kp + 16);
+        }
+        ka[kb][0] = __builtin_bit_cast(bf16x8, w0);
+        ka[kb][1] = __builtin_bit_cast(bf16x8, w1);
+    }
+    __syncthreads();  // V^T visible
+
+    const int nqb = (NM + 31) >> 5;
+    for (int qb = 0; qb < nqb; ++qb) {
+        const int qrow = qb * 32 + m;
+        const int qsafe = qrow < NM ? qrow : NM - 1;
+        const uint16_t *qp = env_base + (int64_t)qsafe * row_stride + head * kDh + half * 8;
+        const bf16x8 qb0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(qp));
+        const bf16x8 qb1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(qp + 16));
+
+        f32x16 acc[NKB];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb) {
+            if (kb < nkb) {
+                f32x16 z = {0.0f};
+                z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kb][0], qb0, z, 0, 0, 0);
+                z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kb][1], qb1, z, 0, 0, 0);
+                if (uniform) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) z[v] = 0.0f;
+                }
+                if (kb == nkb - 1) {
+                    // positions past the live count are padding
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int pos = kb * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+                        if (pos >= cnt) z[v] = -INFINITY;
+                    }
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
+                acc[kb] = z;
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float mc = mx * scale_log2e;
+
+        float sum = 0.0f;
+        f32x16 o = {0.0f};
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb) {
+            if (kb < nkb) {
+                float p[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    p[v] = __builtin_amdgcn_exp2f(fmaf(acc[kb][v], scale_log2e, -mc));
+                    sum += p[v];
+                }
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    bf16x8 pb;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * t + e];
+                    const uint16_t *vp = s_vt + m * VP + kb * 32 + 16 * t + 4 * half;
+                    const u32x2 lo = *reinterpret_cast<const u32x2 *>(vp);
+                    const u32x2 hi = *reinterpret_cast<const u32x2 *>(vp + 8);
+                    const u32x4 vw = {lo.x, lo.y, hi.x, hi.y};
+                    o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vw), pb, o, 0, 0, 0);
+                }
+            }
+        }
+        sum += __shfl_xor(sum, 32);
+        const float inv = __builtin_amdgcn_rcpf(sum);
+
+        if (qrow < NM) {
+            uint16_t *op = out + ((int64_t)env * NM + qrow) * D + head * kDh + 4 * half;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const u32x2 w = {pack_bf16x2(o[4 * i + 0] * inv, o[4 * i + 1] * inv),
+                                 pack_bf16x2(o[4 * i + 2] * inv, o[4 * i + 3] * inv)};
+                *reinterpret_cast<u32x2 *>(op + 8 * i) = w;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------
+
+constexpr size_t kLdsDefault = 64 * 1024;
+constexpr size_t kLdsMax = 160 * 1024;
+
+static size_t valu_lds_bytes(int G, int NM, int nh, int DH)
+{
+    const size_t env_pitch = (size_t)NM * nh * (DH + kValuHeadPad) + kValuEnvPad;
+    return 2 * (size_t)G * env_pitch * sizeof(float) + (((size_t)G * NM + 15) & ~(size_t)15) + (size_t)G * sizeof(int);
+}
+
+template <typename T, int DH>
+static int launch_valu(const void *qkv, int64_t row_stride, const uint8_t *alive, void *out, int B, int NM,
+                       int H, hipStream_t stream)
+{
+    // all heads of an environment in one block when they fit, else one head per block
+    int nh = H;
+    if (valu_lds_bytes(1, NM, H, DH) > kLdsDefault) nh = 1;
+    int G = kValuThreads / (nh * NM);
+    if (G < 1) G = 1;
+    if (G > 8) G = 8;
+    while (G > 1 && valu_lds_bytes(G, NM, nh, DH) > kLdsDefault) --G;
+    if (G > B) G = B;
+    const size_t lds = valu_lds_bytes(G, NM, nh, DH);
+    if (lds > kLdsMax) return BNB_ERR_UNSUPPORTED;
+    auto kernel = sdpa_valu_kernel<T, DH>;
+    if (lds > kLdsDefault) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsMax);
+        if (e != hipSuccess) return (int)e;
+    }
+    const dim3 grid((unsigned)((B + G - 1) / G), (unsigned)(H / nh));
+    const float scale_log2e = kLog2eA / sqrtf((float)DH);
+    hipLaunchKernelGGL(kernel, grid, dim3(kValuThreads), lds, stream, (const T *)qkv, row_stride, alive,
+                       (T *)out, B, NM, H, G, nh, scale_log2e);
+    return (int)hipGetLastError();
+}
+
+template <typename T>
+static int dispatch_valu(const void *qkv, int64_t row_stride, const uint8_t *alive, void *out, int B, int NM,
+                         int H, int dh, hipStream_t stream)
+{
+    switch (dh) {
+        case 8: return launch_valu<T, 8>(qkv, row_stride, alive, out, B, NM, H, stream);
+        case 16: return launch_valu<T, 16>(qkv, row_stride, alive, out, B, NM, H, stream);
+        case 32: return launch_valu<T, 32>(qkv, row_stride, alive, out, B, NM, H, stream);
+        case 64: return launch_valu<T, 64>(qkv, row_stride, alive, out, B, NM, H, stream);
+        default: return BNB_ERR_UNSUPPORTED;
+    }
+}
+
+template <int NKB>
+static int launch_mfma(const void *qkv, int64_t row_stride, const uint8_t *alive, void *out, int B, int NM,
+                       int H, hipStream_t stream)
+{
+    const int64_t pairs = (int64_t)B * H;
+    const int64_t blocks = (pairs + 7) / 8 * 8;
+    if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+    const float scale_log2e = kLog2eA / sqrtf((float)kDh);
+    hipLaunchKernelGGL((sdpa_mfma_kernel<NKB>), dim3((unsigned)blocks), dim3(kWave), 0, stream,
+                       (const uint16_t *)qkv, row_stride, alive, (uint16_t *)out, B, NM, H, scale_log2e);
+    return (int)hipGetLastError();
+}
+
+static int dispatch_mfma(const void *qkv, int64_t row_stride, const uint8_t *alive, void *out, int B, int NM,
+                         int H, hipStream_t stream)
+{
+    switch ((NM + 31) / 32) {
+        case 1: return launch_mfma<1>(qkv, row_stride, alive, out, B, NM, H, stream);
+        case 2: return launch_mfma<2>(qkv, row_stride, alive, out, B, NM, H, stream);
+        case 3: return launch_mfma<3>(qkv, row_stride, alive, out, B, NM, H, stream);
+        case 4: return launch_mfma<4>(qkv, row_stride, alive, out, B, NM, H, stream);
+        case 5: return launch_mfma<5>(qkv, row_stride, alive, out, B, NM, H, stream);
+        default: return BNB_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace bnb
+
+extern "C" int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive,
+                                        void *out, int B, int NM, int H, int dh, int dtype, int path,
+                                        void *stream)
+{
+    using namespace bnb;
+    if (B < 0 || NM < 0 || H < 1 || dh < 1) return BNB_ERR_BAD_SHAPE;
+    if (dtype != BNB_F32 && dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
+    if (path < BNB_SDPA_PATH_AUTO || path > BNB_SDPA_PATH_MFMA) return BNB_ERR_UNSUPPORTED;
+    if (B == 0 || NM == 0) return 0;
+    if (!qkv || !out) return BNB_ERR_NULL_POINTER;
+    if (qkv_row_stride < (int64_t)3 * H * dh) return BNB_ERR_BAD_SHAPE;
+    if (NM > 512) return BNB_ERR_UNSUPPORTED;
+    const size_t esize = dtype == BNB_BF16 ? 2 : 4;
+    if (!aligned16(qkv) || !aligned16(out) || (qkv_row_stride * esize) % 16 != 0) return BNB_ERR_MISALIGNED;
+    hipStream_t s = (hipStream_t)stream;
+
+    const bool mfma_ok = dtype == BNB_BF16 && dh == kDh && NM <= 160;
+    if (path == BNB_SDPA_PATH_MFMA && !mfma_ok) return BNB_ERR_UNSUPPORTED;
+    const bool use_mfma = path == BNB_SDPA_PATH_MFMA || (path == BNB_SDPA_PATH_AUTO && mfma_ok && NM >= 32);
+    if (use_mfma) return dispatch_mfma(qkv, qkv_row_stride, alive, out, B, NM, H, s);
+    if (dtype == BNB_BF16) return dispatch_valu<uint16_t>(qkv, qkv_row_stride, alive, out, B, NM, H, dh, s);
+    return dispatch_valu<float>(qkv, qkv_row_stride, alive, out, B, NM, H, dh, s);
+}
+
+extern "C" int bnb_sdpa_masked_fwd(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, void *out,
+                                   int B, int NM, int H, int dh, int dtype, void *stream)
+{
+    return bnb_sdpa_masked_fwd_path(qkv, qkv_row_stride, alive, out, B, NM, H, dh, dtype, BNB_SDPA_PATH_AUTO,
+                                    stream);
+}

@@ -1,0 +1,178 @@
+"""Tensor-level front ends of the two HIP kernels.
+
+``sdpa_masked`` stands in for the key-bias + ``F.scaled_dot_product_attention`` +
+head-merge copy of the reference (models/yemong/attention.py:136-147,168);
+``rglru_step`` stands in for the element-wise chain of ``RGLRU._step``
+(models/yemong/griffin.py:179-185).  Both launch on torch's current stream, allocate
+their outputs with torch and never synchronise.  They are forward-only and run on a
+ROCm device only: anything else raises.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _native
+
+_DTYPE_CODE = {torch.float32: _native.F32, torch.bfloat16: _native.BF16}
+_PATH_CODE = {"auto": _native.PATH_AUTO, "valu": _native.PATH_VALU, "mfma": _native.PATH_MFMA}
+
+
+def _need_device(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"{name} is on {t.device}; the attention/RG-LRU kernels only exist as HIP code for gfx950 "
+            "and have no host fallback"
+        )
+
+
+def _code(t: torch.Tensor, name: str) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise TypeError(f"{name} must be float32 or bfloat16, got {t.dtype}") from None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def sdpa_masked(
+    qkv: torch.Tensor,
+    alive: torch.Tensor | None,
+    n_heads: int,
+    *,
+    path: str = "auto",
+) -> torch.Tensor:
+    """Masked multi-head attention over each environment's tokens.
+
+    Args:
+        qkv:     (B, NM, 3*D) packed projection, columns [Q | K | V], heads head-major
+                 inside each third.  float32 or bfloat16; last dim contiguous, rows of an
+                 environment and environments themselves evenly spaced (any row stride).
+        alive:   (B, NM) bool (or uint8), True = the entity exists, or None for no mask.
+                 Dead keys get weight 0; an environment with no live key averages V over
+                 all keys; dead queries are still computed.
+        n_heads: H; D must be divisible by it.
+        path:    "auto" | "valu" | "mfma" — kernel selection, for tests and benchmarks.
+
+    Returns:
+        (B, NM, D) in qkv's dtype, heads merged head-major (the input of ``out_proj``).
+    """
+    if qkv.dim() != 3 or qkv.shape[-1] % 3:
+        raise ValueError(f"qkv must be (B, NM, 3*D), got {tuple(qkv.shape)}")
+    _need_device(qkv, "qkv")
+    dtype = _code(qkv, "qkv")
+    B, NM, D3 = qkv.shape
+    D = D3 // 3
+    if n_heads < 1 or D % n_heads:
+        raise ValueError(f"d_model={D} must be divisible by n_heads={n_heads}")
+    if path not in _PATH_CODE:
+        raise ValueError(f"path must be one of {sorted(_PATH_CODE)}, got {path!r}")
+    if qkv.requires_grad and torch.is_grad_enabled():
+        raise RuntimeError("sdpa_masked is forward-only; call it under torch.no_grad()")
+    if B and NM and (qkv.stride(-1) != 1 or (B > 1 and qkv.stride(0) != NM * qkv.stride(1))):
+        qkv = qkv.contiguous()
+    mask_ptr = None
+    if alive is not None:
+        if alive.shape != (B, NM):
+            raise ValueError(f"alive must be {(B, NM)}, got {tuple(alive.shape)}")
+        if alive.dtype not in (torch.bool, torch.uint8):
+            raise TypeError(f"alive must be bool or uint8, got {alive.dtype}")
+        if alive.device != qkv.device:
+            raise RuntimeError(f"alive is on {alive.device}, qkv on {qkv.device}")
+        alive = alive.contiguous()
+        mask_ptr = alive.data_ptr()
+    out = torch.empty((B, NM, D), dtype=qkv.dtype, device=qkv.device)
+    if B == 0 or NM == 0:
+        return out
+    with torch.cuda.device(qkv.device):
+        rc = _native.load().bnb_sdpa_masked_fwd_path(
+            qkv.data_ptr(), qkv.stride(1), mask_ptr, out.data_ptr(), B, NM, n_heads, D // n_heads, dtype,
+            _PATH_CODE[path], _stream(),
+        )
+    _native.check(rc, "bnb_sdpa_masked_fwd")
+    return out
+
+
+def rglru_step(
+    x: torch.Tensor,
+    gates_pre: torch.Tensor,
+    log_lambda: torch.Tensor,
+    c: float,
+    h: torch.Tensor,
+    *,
+    h_out: torch.Tensor | None = None,
+    y_dtype: torch.dtype | None = None,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """One RG-LRU step given the two gate pre-activations.
+
+    Args:
+        x:          (R, D) input rows, float32 or bfloat16.
+        gates_pre:  (R, 2*D): ``[linear_a(x) | linear_x(x)]`` with biases, float32 or bfloat16.
+        log_lambda: (D,) float32 parameter.
+        c:          exponent constant (8.0 in the reference).
+        h:          (R, D) float32 previous state; rows may be strided (a view into the
+                    packed (.., 4*D) hidden tensor works), the last dim must be contiguous.
+        h_out:      optional float32 (R, D) destination (rows may be strided; may be ``h``
+                    itself for an in-place update).  Default: a new contiguous tensor.
+        y_dtype:    dtype of the returned layer output.  None or float32 returns the new
+                    state itself; bfloat16 makes the kernel write a rounded copy as well.
+
+    Returns:
+        (y, h_new): layer output and new state (the same tensor unless y_dtype is bfloat16).
+    """
+    if x.dim() != 2 or gates_pre.dim() != 2 or h.dim() != 2:
+        raise ValueError("x, gates_pre and h must be 2-D (rows, channels)")
+    R, D = x.shape
+    if gates_pre.shape != (R, 2 * D) or h.shape != (R, D) or log_lambda.shape != (D,):
+        raise ValueError(
+            f"shape mismatch: x {tuple(x.shape)}, gates_pre {tuple(gates_pre.shape)}, h {tuple(h.shape)}, "
+            f"log_lambda {tuple(log_lambda.shape)}"
+        )
+    for name, t in (("x", x), ("gates_pre", gates_pre), ("log_lambda", log_lambda), ("h", h)):
+        _need_device(t, name)
+    if h.dtype != torch.float32 or log_lambda.dtype != torch.float32:
+        raise TypeError("h and log_lambda must be float32 (the recurrent state is never stored narrower)")
+    if torch.is_grad_enabled() and (x.requires_grad or gates_pre.requires_grad or h.requires_grad):
+        raise RuntimeError("rglru_step is forward-only; call it under torch.no_grad()")
+    x_code, g_code = _code(x, "x"), _code(gates_pre, "gates_pre")
+    x = x.contiguous()
+    gates_pre = gates_pre.contiguous()
+    log_lambda = log_lambda.detach().contiguous()
+    if R and h.stride(-1) != 1:
+        h = h.contiguous()
+    if h_out is None:
+        h_out = torch.empty((R, D), dtype=torch.float32, device=x.device)
+    else:
+        if h_out.shape != (R, D) or h_out.dtype != torch.float32 or h_out.device != x.device:
+            raise ValueError("h_out must be a float32 (R, D) tensor on x's device")
+        if R and h_out.stride(-1) != 1:
+            raise ValueError("h_out must be contiguous in its last dim")
+    y = None
+    if y_dtype is not None and y_dtype != torch.float32:
+        if y_dtype != torch.bfloat16:
+            raise TypeError(f"y_dtype must be float32 or bfloat16, got {y_dtype}")
+        y = torch.empty((R, D), dtype=torch.bfloat16, device=x.device)
+    if R == 0:
+        return (h_out if y is None else y), h_out
+    with torch.cuda.device(x.device):
+        rc = _native.load().bnb_rglru_step_fwd(
+            x.data_ptr(), x_code, gates_pre.data_ptr(), g_code, log_lambda.data_ptr(), float(c),
+            h.data_ptr(), h.stride(0), h_out.data_ptr(), h_out.stride(0),
+            None if y is None else y.data_ptr(), _native.BF16, R, D, _stream(),
+        )
+    _native.check(rc, "bnb_rglru_step_fwd")
+    return (h_out if y is None else y), h_out
+
+
+def copy_bytes(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """Device copy through the library's 16-byte copy kernel (bandwidth yardstick)."""
+    _need_device(src, "src")
+    _need_device(dst, "dst")
+    n = src.numel() * src.element_size()
+    if n != dst.numel() * dst.element_size() or not (src.is_contiguous() and dst.is_contiguous()):
+        raise ValueError("src and dst must be contiguous and of equal byte size")
+    with torch.cuda.device(src.device):
+        rc = _native.load().bnb_copy_bytes(src.data_ptr(), dst.data_ptr(), n, _stream())
+    _native.check(rc, "bnb_copy_bytes")

@@ -1,0 +1,369 @@
+"""Drop-in trunk layers for the Yemong policy, running on the gfx950 kernels.
+
+Every class keeps the constructor arguments, method signatures, tensor layouts and
+``state_dict`` keys of the layer it replaces, so a reference checkpoint loads with
+``load_state_dict`` and a reference policy can swap its ``yemong_layers`` for these:
+
+    TransformerBlock        models/yemong/attention.py:40-169
+    GatedMLP                models/yemong/attention.py:21-37
+    RGLRU                   models/yemong/griffin.py:143-219
+    GriffinTemporalBlock    models/yemong/griffin.py:222-317
+    YemongBlock             models/yemong/griffin.py:320-472
+    ModelConfig             config/core.py:213-275
+    YemongTrunk             the block loop and hidden-state handling of
+                            models/yemong/policy.py:234-254, 268-285, 311-354
+
+What runs where: the attention core (key masking, softmax, head merge) and the RG-LRU
+element-wise recurrence are the HIP kernels in ``ops``; projections, norms, GELUs and the
+depthwise conv taps are torch library calls on the same stream.  The layers are
+forward-only (rollout / evaluation); they refuse tensors that need gradients and they
+refuse to run off-GPU.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops
+
+CONV_KERNEL = 4  # taps of the causal depthwise conv; the state keeps the last CONV_KERNEL-1 inputs
+
+
+@dataclass(frozen=True)
+class ModelConfig:
+    """Trunk architecture; field names and checks follow config/core.py:213-275."""
+
+    d_model: int
+    n_heads: int
+    n_yemong_blocks: int
+    n_spatial_per_block: int = 1
+    n_temporal_per_block: int = 1
+    encoder_split: bool = False
+    n_bullet_cross_per_block: int = 0
+    bullet_encoder_hidden: int = 64
+    grad_checkpoint: bool = False
+
+    @property
+    def n_hidden_layers(self) -> int:
+        return self.n_yemong_blocks * self.n_temporal_per_block
+
+    @property
+    def reads_bullets(self) -> bool:
+        return self.n_bullet_cross_per_block > 0 and self.n_yemong_blocks > 0
+
+    def __post_init__(self) -> None:
+        if self.d_model % self.n_heads:
+            raise ValueError(f"d_model={self.d_model} must be divisible by n_heads={self.n_heads}")
+        for name in ("n_yemong_blocks", "n_spatial_per_block", "n_temporal_per_block"):
+            if getattr(self, name) < 0:
+                raise ValueError(f"{name} must be >= 0, got {getattr(self, name)}")
+        if not 0 <= self.n_bullet_cross_per_block <= self.n_spatial_per_block:
+            raise ValueError(
+                f"n_bullet_cross_per_block must lie in [0, {self.n_spatial_per_block}], "
+                f"got {self.n_bullet_cross_per_block}"
+            )
+
+
+class GatedMLP(nn.Module):
+    """``down_proj(gelu(gate_proj(x)) * up_proj(x))`` with a 4x hidden width by default."""
+
+    def __init__(self, d_model: int, expand: int = 4) -> None:
+        super().__init__()
+        self.gate_proj = nn.Linear(d_model, expand * d_model, bias=False)
+        self.up_proj = nn.Linear(d_model, expand * d_model, bias=False)
+        self.down_proj = nn.Linear(expand * d_model, d_model, bias=False)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.down_proj(F.gelu(self.gate_proj(x)) * self.up_proj(x))
+
+
+class TransformerBlock(nn.Module):
+    """Pre-norm attention + FFN over the entity tokens of each environment.
+
+    ``forward(x (B,N,D), alive_mask (B,N) bool | None, bullets, bullet_mask) -> (B,N,D)``.
+    """
+
+    def __init__(self, model_config: ModelConfig, reads_bullets: bool = False) -> None:
+        super().__init__()
+        D = model_config.d_model
+        self.d_model = D
+        self.n_heads = model_config.n_heads
+        self.head_dim = D // model_config.n_heads
+        self.reads_bullets = reads_bullets
+        self.norm1 = nn.RMSNorm(D)
+        self.qkv = nn.Linear(D, 3 * D, bias=False)
+        self.out_proj = nn.Linear(D, D, bias=False)
+        if reads_bullets:
+            self.norm_bullet = nn.RMSNorm(D)
+            self.kv_bullet = nn.Linear(D, 2 * D, bias=False)
+        self.norm2 = nn.RMSNorm(D)
+        self.ffn = GatedMLP(D)
+
+    def forward(self, x, alive_mask=None, bullets=None, bullet_mask=None):
+        x = x + self._attn(self.norm1(x), alive_mask, bullets, bullet_mask)
+        return x + self.ffn(self.norm2(x))
+
+    def _attn(self, x, alive_mask, bullets=None, bullet_mask=None):
+        qkv = self.qkv(x)  # (B, N, 3D), fp32 or bf16 under autocast
+        merged = ops.sdpa_masked(qkv, alive_mask, self.n_heads)  # (B, N, D) head-major
+        if self.reads_bullets and bullets is not None:
+            merged = merged + self._bullet_read(qkv, bullets, bullet_mask)
+        return self.out_proj(merged)
+
+    def _bullet_read(self, qkv, bullets, bullet_mask):
+        """Cross-attention of the entity queries to bullet key/values (attention.py:149-166).
+
+        Not one of the two kernels of this package: it goes through torch's SDPA on the
+        device, with the reference's additive bias and its all-inactive gate.
+        """
+        B, N, _ = qkv.shape
+        H, dh, D = self.n_heads, self.head_dim, self.d_model
+        NB = bullets.shape[1]
+        q = qkv[..., :D].reshape(B, N, H, dh).transpose(1, 2)
+        kv = self.kv_bullet(self.norm_bullet(bullets))
+        kb = kv[..., :D].reshape(B, NB, H, dh).transpose(1, 2)
+        vb = kv[..., D:].reshape(B, NB, H, dh).transpose(1, 2)
+        bias = None
+        if bullet_mask is not None:
+            keep = bullet_mask.reshape(B, 1, 1, NB).to(q.dtype)
+            bias = (1.0 - keep) * (torch.finfo(q.dtype).min / 2)
+        o = F.scaled_dot_product_attention(q, kb, vb, attn_mask=bias, dropout_p=0.0)
+        if bullet_mask is not None:
+            o = o * bullet_mask.any(dim=-1).reshape(B, 1, 1, 1).to(o.dtype)
+        return o.transpose(1, 2).reshape(B, N, D)
+
+
+class RGLRU(nn.Module):
+    """Real-gated linear recurrent unit; parameters ``log_lambda``, ``linear_a``, ``linear_x``."""
+
+    def __init__(self, d_model: int, c: float = 8.0) -> None:
+        super().__init__()
+        self.c = c
+        self.log_lambda = nn.Parameter(torch.linspace(0.0, 4.0, d_model))
+        self.linear_a = nn.Linear(d_model, d_model, bias=True)
+        self.linear_x = nn.Linear(d_model, d_model, bias=True)
+        self._fused: tuple | None = None  # (key, weight (2D,D), bias (2D,))
+
+    def _gate_preactivations(self, x: torch.Tensor) -> torch.Tensor:
+        """``[linear_a(x) | linear_x(x)]`` as one (R, 2D) GEMM over concatenated weights."""
+        wa, wx, ba, bx = self.linear_a.weight, self.linear_x.weight, self.linear_a.bias, self.linear_x.bias
+        key = (wa._version, wx._version, ba._version, bx._version, wa.data_ptr(), wx.data_ptr(), wa.device)
+        if self._fused is None or self._fused[0] != key:
+            with torch.no_grad():
+                self._fused = (key, torch.cat([wa, wx], dim=0), torch.cat([ba, bx], dim=0))
+        return F.linear(x, self._fused[1], self._fused[2])
+
+    def _step(self, x: torch.Tensor, h: torch.Tensor) -> torch.Tensor:
+        """(R,D), (R,D) -> new state (R,D) float32 (also the layer output)."""
+        return self.step(x, h)[1]
+
+    def step(self, x: torch.Tensor, h: torch.Tensor, y_dtype: torch.dtype | None = None):
+        """One kernel launch: returns (output in ``y_dtype`` or the state itself, new state)."""
+        return ops.rglru_step(x, self._gate_preactivations(x), self.log_lambda, self.c, h, y_dtype=y_dtype)
+
+    def forward_sequence(self, x_seq, h0, done_mask=None):
+        """(R,T,D), (R,D) -> ((R,T,D) states, (R,D) last state).
+
+        T = 1 is the rollout path (one launch).  Longer sequences advance step by step;
+        ``done_mask[:, t]`` cuts the state after step t (griffin.py:213-218).
+        """
+        T = x_seq.shape[1]
+        if T == 1 and done_mask is None:
+            h = self._step(x_seq[:, 0], h0)
+            return h.unsqueeze(1), h
+        h, ys = h0, []
+        for t in range(T):
+            if done_mask is not None and t > 0:
+                h = h * (~done_mask[:, t - 1]).to(h.dtype).unsqueeze(-1)
+            h = self._step(x_seq[:, t], h)
+            ys.append(h)
+        return torch.stack(ys, dim=1), h
+
+
+class GriffinTemporalBlock(nn.Module):
+    """norm -> (linear1 -> causal conv -> RG-LRU) * gelu(linear2) -> linear_out, then a gated MLP."""
+
+    def __init__(self, d_model: int) -> None:
+        super().__init__()
+        self.norm1 = nn.RMSNorm(d_model)
+        self.linear1 = nn.Linear(d_model, d_model, bias=False)
+        self.conv = nn.Conv1d(d_model, d_model, kernel_size=CONV_KERNEL, groups=d_model, bias=True)
+        self.rg_lru = RGLRU(d_model)
+        self.linear2 = nn.Linear(d_model, d_model, bias=False)
+        self.linear_out = nn.Linear(d_model, d_model, bias=False)
+        self.norm2 = nn.RMSNorm(d_model)
+        self.gated_mlp = GatedMLP(d_model)
+
+    def forward_sequence(self, x_seq, h0, conv_buf, done_mask=None):
+        """(R,T,D), (R,D), (R,3,D) [, (R,T) bool] -> (out (R,T,D), new_h (R,D), new_conv_buf (R,3,D))."""
+        T = x_seq.shape[1]
+        normed = self.norm1(x_seq)
+        b1 = self.linear1(normed)
+        padded = torch.cat([conv_buf, b1], dim=1)  # (R, T+3, D); fp32 buffer promotes a bf16 b1
+        w = self.conv.weight.squeeze(1)  # (D, 4); tap k meets padded[:, t+k]
+        if done_mask is None:
+            conv_out = sum(padded[:, k:k + T] * w[:, k] for k in range(CONV_KERNEL)) + self.conv.bias
+        else:
+            conv_out = _conv_within_episodes(padded, w, self.conv.bias, done_mask)
+        y, new_h = self.rg_lru.forward_sequence(conv_out, h0, done_mask)
+        b2 = F.gelu(self.linear2(normed))
+        x1 = x_seq + self.linear_out(y * b2)
+        x2 = x1 + self.gated_mlp(self.norm2(x1))
+        return x2, new_h, padded[:, T:]
+
+    def forward_nonrecurrent(self, x, sub):
+        """Same block with ``sub`` (a Linear) in place of conv + RG-LRU; no state."""
+        normed = self.norm1(x)
+        b1 = sub(self.linear1(normed))
+        b2 = F.gelu(self.linear2(normed))
+        x1 = x + self.linear_out(b1 * b2)
+        return x1 + self.gated_mlp(self.norm2(x1))
+
+
+def _conv_within_episodes(padded, w, bias, done_mask):
+    """Depthwise causal conv whose taps stop at episode ends (griffin.py:67-140).
+
+    ``done_mask[:, t]`` ends an episode at t.  A tap contributes to output t only if the
+    input it reads lies in the same episode as t; the stored buffer counts as belonging
+    to the episode running at t = 0.
+    """
+    R, T = done_mask.shape
+    starts = torch.zeros_like(done_mask, dtype=torch.long)
+    starts[:, 1:] = done_mask[:, :-1].long()
+    episode = torch.cat([starts.new_zeros(R, CONV_KERNEL - 1), starts.cumsum(dim=1)], dim=1)  # (R, T+3)
+    here = episode[:, CONV_KERNEL - 1:]
+    out = 0
+    for k in range(CONV_KERNEL):
+        same = (episode[:, k:k + T] == here).to(padded.dtype).unsqueeze(-1)
+        out = out + padded[:, k:k + T] * w[:, k] * same
+    return out + bias
+
+
+class YemongBlock(nn.Module):
+    """``n_spatial_per_block`` attention sublayers, then ``n_temporal_per_block`` recurrent ones."""
+
+    def __init__(self, model_config: ModelConfig) -> None:
+        super().__init__()
+        D = model_config.d_model
+        self.spatial = nn.ModuleList(
+            TransformerBlock(model_config, reads_bullets=i < model_config.n_bullet_cross_per_block)
+            for i in range(model_config.n_spatial_per_block)
+        )
+        self.temporal = nn.ModuleList(GriffinTemporalBlock(D) for _ in range(model_config.n_temporal_per_block))
+        self.field_sub = nn.ModuleList(nn.Linear(D, D, bias=False) for _ in range(model_config.n_temporal_per_block))
+        for sub in self.field_sub:
+            nn.init.eye_(sub.weight)
+
+    @property
+    def n_temporal(self) -> int:
+        return len(self.temporal)
+
+    def step(self, x, alive, h, conv_buf, num_recurrent=None, bullets=None, bullet_mask=None):
+        """One timestep.
+
+        x (B,NM,D); alive (B,NM) bool; h (n_temporal, B*n_rec, D); conv_buf
+        (n_temporal, B*n_rec, 3, D).  The first ``num_recurrent`` tokens of every
+        environment are recurrent (state row b*n_rec + n), the rest take the state-free
+        path.  Returns (x, new_h, new_conv_buf) as new tensors.
+        """
+        B, NM, D = x.shape
+        n_rec = NM if num_recurrent is None else num_recurrent
+        for layer in self.spatial:
+            x = layer(x, alive, bullets, bullet_mask)
+        new_h, new_cb = [], []
+        for j, layer in enumerate(self.temporal):
+            ships = x[:, :n_rec].reshape(B * n_rec, 1, D)
+            out, h_j, cb_j = layer.forward_sequence(ships, h[j], conv_buf[j])
+            parts = [out.reshape(B, n_rec, D)]
+            if NM > n_rec:
+                parts.append(layer.forward_nonrecurrent(x[:, n_rec:], self.field_sub[j]))
+            x = torch.cat(parts, dim=1) if len(parts) > 1 else parts[0]
+            new_h.append(h_j)
+            new_cb.append(cb_j)
+        if not new_h:
+            return x, h[:0], conv_buf[:0]
+        return x, torch.stack(new_h), torch.stack(new_cb)
+
+    def sequence(self, x, alive_mask, h0, conv_buf0, done_mask=None, num_recurrent=None, bullets=None,
+                 bullet_mask=None):
+        """(T,B,NM,D) variant of ``step`` for re-evaluating a stored rollout (no gradients)."""
+        T, B, NM, D = x.shape
+        n_rec = NM if num_recurrent is None else num_recurrent
+        for layer in self.spatial:
+            x = layer(x.reshape(T * B, NM, D), alive_mask.reshape(T * B, NM), bullets, bullet_mask)
+            x = x.reshape(T, B, NM, D)
+        done_rows = None if done_mask is None else done_mask.t().repeat_interleave(n_rec, dim=0)  # (B*n_rec, T)
+        new_h, new_cb = [], []
+        for j, layer in enumerate(self.temporal):
+            ships = x[:, :, :n_rec].permute(1, 2, 0, 3).reshape(B * n_rec, T, D)
+            out, h_j, cb_j = layer.forward_sequence(ships, h0[j], conv_buf0[j], done_rows)
+            parts = [out.reshape(B, n_rec, T, D).permute(2, 0, 1, 3)]
+            if NM > n_rec:
+                parts.append(layer.forward_nonrecurrent(x[:, :, n_rec:], self.field_sub[j]))
+            x = torch.cat(parts, dim=2) if len(parts) > 1 else parts[0]
+            new_h.append(h_j)
+            new_cb.append(cb_j)
+        if not new_h:
+            return x, h0[:0], conv_buf0[:0]
+        return x, torch.stack(new_h), torch.stack(new_cb)
+
+
+class YemongTrunk(nn.Module):
+    """The recurrent trunk: ``forward(tokens, alive_mask, recurrent_state) -> (hidden, new_state)``.
+
+    ``recurrent_state`` is the packed tensor (n_layers, B*n_rec, 4*D) float32 of the
+    reference policy: ``[..., :D]`` is the RG-LRU state, ``[..., D:]`` the last three conv
+    inputs, oldest first.  ``n_rec`` is read off its row count, so a state sized with N
+    sends the trailing M tokens down the state-free path and one sized with N+M makes every
+    token recurrent.  The submodule list is named ``yemong_layers`` as in the policy.
+    """
+
+    def __init__(self, model_config: ModelConfig) -> None:
+        super().__init__()
+        self.config = model_config
+        self.yemong_layers = nn.ModuleList(YemongBlock(model_config) for _ in range(model_config.n_yemong_blocks))
+
+    @property
+    def n_hidden_layers(self) -> int:
+        return self.config.n_hidden_layers
+
+    def initial_hidden(self, num_envs: int, num_recurrent_tokens: int, device) -> torch.Tensor:
+        return torch.zeros(
+            self.n_hidden_layers, num_envs * num_recurrent_tokens, CONV_KERNEL * self.config.d_model, device=device
+        )
+
+    @staticmethod
+    def reset_hidden_for_envs(hidden: torch.Tensor, done_mask: torch.Tensor, num_recurrent_tokens: int):
+        """Zero all rows of finished environments (rows are env-major)."""
+        keep = (~done_mask.repeat_interleave(num_recurrent_tokens)).to(hidden.dtype)
+        return hidden * keep[None, :, None]
+
+    @torch.no_grad()
+    def forward(self, tokens, alive_mask, recurrent_state, bullets=None, bullet_mask=None):
+        B, NM, D = tokens.shape
+        L, rows, width = recurrent_state.shape
+        if L != self.n_hidden_layers or width != CONV_KERNEL * D or (B and rows % B):
+            raise ValueError(
+                f"recurrent_state {tuple(recurrent_state.shape)} does not fit {self.n_hidden_layers} layers, "
+                f"{B} environments and d_model {D}"
+            )
+        n_rec = rows // B if B else 0
+        n_t = self.config.n_temporal_per_block
+        h_all = recurrent_state[:, :, :D]
+        cb_all = recurrent_state[:, :, D:].reshape(L, rows, CONV_KERNEL - 1, D)
+        x, hs, cbs = tokens, [], []
+        for i, block in enumerate(self.yemong_layers):
+            sl = slice(i * n_t, (i + 1) * n_t)
+            x, h_i, cb_i = block.step(x, alive_mask, h_all[sl], cb_all[sl], n_rec, bullets, bullet_mask)
+            hs.append(h_i)
+            cbs.append(cb_i)
+        if L == 0:
+            return x, recurrent_state
+        new_state = torch.cat(
+            [torch.cat(hs, dim=0), torch.cat(cbs, dim=0).reshape(L, rows, (CONV_KERNEL - 1) * D)], dim=-1
+        )
+        return x, new_state

@@ -1,0 +1,133 @@
+/*
+ * C ABI of libbnb_amd.so: the masked-attention and RG-LRU step kernels for gfx950.
+ *
+ * The reference has no FFI or operator registry; the seam it offers is two Python
+ * call sites inside its policy trunk.  Each entry point below names the reference
+ * lines it stands in for (paths relative to the reference checkout,
+ * src/boost_and_broadside/).
+ *
+ * Conventions shared by every entry point
+ *   - every pointer is a DEVICE pointer owned by the caller; nothing is allocated,
+ *     freed or copied to the host, and no call synchronises the stream;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); work is
+ *     enqueued on it and the call returns immediately;
+ *   - the return value is 0 on success, a BNB_ERR_* code for a rejected argument, or
+ *     a hipError_t value if the launch itself failed; bnb_error_string() names it;
+ *   - calls are re-entrant and keep no state between calls.
+ */
+#ifndef BNB_AMD_H
+#define BNB_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BNB_ABI_VERSION 1
+
+/* element types of activation buffers */
+#define BNB_F32 0
+#define BNB_BF16 1
+
+/* argument errors (kept clear of the hipError_t range) */
+#define BNB_ERR_NULL_POINTER 10001  /* a required pointer is NULL */
+#define BNB_ERR_BAD_DTYPE 10002     /* dtype is neither BNB_F32 nor BNB_BF16 */
+#define BNB_ERR_BAD_SHAPE 10003     /* negative size, H*dh mismatch, stride smaller than a row */
+#define BNB_ERR_UNSUPPORTED 10004   /* shape outside what the kernels cover (see each entry point) */
+#define BNB_ERR_MISALIGNED 10005    /* pointer or stride breaks the stated alignment */
+
+/* Bumped on any change of a signature or of the meaning of an argument. */
+int bnb_abi_version(void);
+
+/* Architecture the device code was compiled for ("gfx950"). */
+const char *bnb_build_arch(void);
+
+/* Static, human-readable name of a code returned by the entry points below. */
+const char *bnb_error_string(int code);
+
+/*
+ * Masked multi-head attention over each environment's entity tokens.
+ *
+ * Replaces, in models/yemong/attention.py: the key-bias construction (:101-112,
+ * :142-145), F.scaled_dot_product_attention(q, k, v, attn_mask=bias) (:147) and the
+ * head-merge copy permute(0,2,1,3).reshape(B,N,D) (:168).  The packed projection
+ * `qkv = self.qkv(x)` (:135) goes in as it is, the tensor handed to `out_proj` (:169)
+ * comes out.
+ *
+ *   qkv    (B, NM, 3*H*dh) rows of `qkv_row_stride` elements, columns [Q | K | V],
+ *          each third split into H runs of dh columns; environments follow each other
+ *          every NM rows
+ *   alive  (B, NM) bytes, non-zero = the entity exists; NULL = no masking.  A dead key
+ *          receives weight exactly 0 whenever its environment has a live key; an
+ *          environment with no live key averages V uniformly over all NM keys (what the
+ *          reference's additive finfo.min/2 bias produces); dead queries are computed
+ *   out    (B, NM, H*dh) contiguous, heads merged head-major, same dtype as qkv
+ *   dtype  BNB_F32 or BNB_BF16 (bf16 in/out, fp32 scores, softmax and accumulation)
+ *
+ * Requirements: dh in {8,16,32,64}; NM <= 512 and NM*(dh+4)*8 bytes of K/V for one head
+ * within 160 KB of LDS (else BNB_ERR_UNSUPPORTED); qkv, out and the row stride aligned to
+ * 16 bytes.  B == 0 or NM == 0 is a no-op.
+ */
+int bnb_sdpa_masked_fwd(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, void *out,
+                        int B, int NM, int H, int dh, int dtype, void *stream);
+
+/*
+ * Same as bnb_sdpa_masked_fwd with the kernel chosen by the caller instead of by shape;
+ * used by tests and the benchmark to run both kernels on one input.  No reference
+ * counterpart beyond the one above.
+ *   BNB_SDPA_PATH_AUTO  what bnb_sdpa_masked_fwd does: the matrix-core kernel for bf16,
+ *                       dh == 32 and 32 <= NM <= 160, the vector-ALU kernel otherwise
+ *   BNB_SDPA_PATH_VALU  vector-ALU kernel (any supported shape and dtype)
+ *   BNB_SDPA_PATH_MFMA  matrix-core kernel (bf16, dh == 32, NM <= 160; else BNB_ERR_UNSUPPORTED)
+ */
+#define BNB_SDPA_PATH_AUTO 0
+#define BNB_SDPA_PATH_VALU 1
+#define BNB_SDPA_PATH_MFMA 2
+int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, void *out,
+                             int B, int NM, int H, int dh, int dtype, int path, void *stream);
+
+/*
+ * One RG-LRU recurrence step over R = B*n_rec entity rows of D channels.
+ *
+ * Replaces the element-wise chain of models/yemong/griffin.py:179-185 (RGLRU._step),
+ * equally :208-212 plus the T=1 scan of :45-64 (out = a*h0 + b): the two sigmoids,
+ * a = sigmoid(log_lambda)^(c*r), gate = sqrt(clamp((1-a)(1+a), 1e-6)),
+ * h' = a*h + gate*(i*x).  The two gate projections linear_a / linear_x (:166-167)
+ * stay GEMMs on the caller's side and arrive as one (R, 2*D) buffer.
+ *
+ *   x          (R, D) contiguous, x_dtype
+ *   gates_pre  (R, 2*D) contiguous, g_dtype: [linear_a(x) | linear_x(x)], biases included
+ *   log_lambda (D) fp32
+ *   c          the exponent constant (8 in the reference)
+ *   h_in       previous state, fp32, row r at h_in + r*h_in_row_stride (floats); a stride
+ *              of 4*D addresses the packed hidden tensor of models/yemong/policy.py:323
+ *   h_out      new state, fp32, same addressing; may equal h_in (in-place update)
+ *   y          optional (R, D) copy of the new state in y_dtype (the layer output under
+ *              bf16 autocast); NULL to skip it
+ *
+ * With bf16 gate pre-activations the roundings of the reference's autocast path are
+ * reproduced (r, i and c*r are rounded to bf16; i*x is rounded to bf16 when x is bf16
+ * too); state, decay and gate are always fp32.
+ *
+ * Requirements: D >= 1; R >= 0.  Rows whose pointers and strides are 16-byte aligned
+ * with D % 8 == 0 take the vector path; anything else takes a scalar path.
+ */
+int bnb_rglru_step_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
+                       const float *log_lambda, float c,
+                       const float *h_in, int64_t h_in_row_stride,
+                       float *h_out, int64_t h_out_row_stride,
+                       void *y, int y_dtype, int64_t R, int D, void *stream);
+
+/*
+ * Plain device-to-device copy of `bytes` bytes (multiple of 16, 16-byte aligned) by a
+ * grid of 16-byte loads and stores.  It has no counterpart in the reference: it is the
+ * yardstick the benchmark uses for achievable HBM bandwidth and for scaling hardware
+ * byte counters.
+ */
+int bnb_copy_bytes(const void *src, void *dst, int64_t bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BNB_AMD_H */

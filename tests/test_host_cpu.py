@@ -1,0 +1,154 @@
+"""CPU-side checks: the C ABI library loads and exports what the header declares, the host
+wrappers validate their arguments, the layer classes keep the reference's state_dict names,
+and the workload generators / traffic model give the documented figures.  No kernel runs."""
+
+import os
+import re
+
+import pytest
+import torch
+
+from helpers import ROOT, trunk_params
+
+import boost_and_broadside_amd as bnb
+from boost_and_broadside_amd import _native, harness, ops
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "bnb_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(bnb_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _native.load()
+    names = _declared_functions()
+    assert {"bnb_sdpa_masked_fwd", "bnb_rglru_step_fwd", "bnb_abi_version"} <= set(names)
+    for name in names:
+        assert hasattr(lib, name), name
+    assert sorted(_native.SIGNATURES) == names  # the ctypes table covers the header exactly
+
+
+def test_library_identity_and_error_names():
+    lib = _native.load()
+    assert lib.bnb_abi_version() == _native.ABI_VERSION == 1
+    assert lib.bnb_build_arch() == b"gfx950"
+    assert lib.bnb_error_string(0) == b"success"
+    assert b"NULL" in lib.bnb_error_string(10001)
+    assert b"alignment" in lib.bnb_error_string(10005)
+
+
+def test_header_constants_match_loader():
+    text = open(os.path.join(ROOT, "include", "bnb_amd.h")).read()
+    consts = dict(re.findall(r"#define\s+(BNB_[A-Z0-9_]+)\s+(\d+)", text))
+    assert int(consts["BNB_ABI_VERSION"]) == _native.ABI_VERSION
+    assert (int(consts["BNB_F32"]), int(consts["BNB_BF16"])) == (_native.F32, _native.BF16)
+    assert [int(consts[f"BNB_SDPA_PATH_{n}"]) for n in ("AUTO", "VALU", "MFMA")] == [0, 1, 2]
+
+
+def test_ops_refuse_host_tensors_and_bad_arguments():
+    with pytest.raises(RuntimeError, match="no host fallback"):
+        ops.sdpa_masked(torch.zeros(1, 2, 48), None, 4)
+    with pytest.raises(ValueError):
+        ops.sdpa_masked(torch.zeros(1, 2, 50), None, 4)  # not 3*D
+    with pytest.raises(RuntimeError, match="no host fallback"):
+        ops.rglru_step(torch.zeros(2, 8), torch.zeros(2, 16), torch.zeros(8), 8.0, torch.zeros(2, 8))
+    with pytest.raises(ValueError):
+        ops.rglru_step(torch.zeros(2, 8), torch.zeros(2, 8), torch.zeros(8), 8.0, torch.zeros(2, 8))
+
+
+def test_model_config_validation_matches_reference_rules():
+    # config/core.py:262-275 and tests/models/test_encoder.py:571-589
+    cfg = bnb.ModelConfig(d_model=64, n_heads=4, n_yemong_blocks=2)
+    assert (cfg.n_spatial_per_block, cfg.n_temporal_per_block, cfg.n_hidden_layers) == (1, 1, 2)
+    for kwargs in ({"n_yemong_blocks": -1}, {"n_spatial_per_block": -1}, {"n_temporal_per_block": -1}):
+        kw = {"n_yemong_blocks": 2, **kwargs}
+        with pytest.raises(ValueError):
+            bnb.ModelConfig(d_model=64, n_heads=4, **kw)
+    with pytest.raises(ValueError):
+        bnb.ModelConfig(d_model=66, n_heads=4, n_yemong_blocks=1)
+    with pytest.raises(ValueError):
+        bnb.ModelConfig(d_model=64, n_heads=4, n_yemong_blocks=1, n_spatial_per_block=1, n_bullet_cross_per_block=2)
+
+
+@pytest.mark.parametrize("n_blocks,n_spatial,n_temporal", [(2, 1, 1), (2, 2, 1), (1, 4, 2), (2, 2, 0)])
+def test_state_dict_keys_are_the_reference_names(n_blocks, n_spatial, n_temporal):
+    cfg = bnb.ModelConfig(d_model=32, n_heads=4, n_yemong_blocks=n_blocks, n_spatial_per_block=n_spatial,
+                          n_temporal_per_block=n_temporal)
+    trunk = bnb.YemongTrunk(cfg)
+    want = trunk_params(0, 32, n_blocks, n_spatial, n_temporal)
+    have = trunk.state_dict()
+    assert sorted(have) == sorted(want)
+    for k in want:
+        assert tuple(have[k].shape) == tuple(want[k].shape), k
+    trunk.load_state_dict(want, strict=True)
+    for block in trunk.yemong_layers:
+        assert len(block.spatial) == n_spatial and len(block.temporal) == n_temporal
+
+
+def test_bullet_reading_layers_carry_the_extra_reference_parameters():
+    cfg = bnb.ModelConfig(d_model=32, n_heads=4, n_yemong_blocks=1, n_spatial_per_block=2, n_bullet_cross_per_block=1)
+    keys = set(bnb.YemongBlock(cfg).state_dict())
+    assert {"spatial.0.norm_bullet.weight", "spatial.0.kv_bullet.weight"} <= keys
+    assert "spatial.1.kv_bullet.weight" not in keys
+
+
+def test_fresh_layers_follow_reference_initialisation():
+    cfg = bnb.ModelConfig(d_model=32, n_heads=4, n_yemong_blocks=1)
+    block = bnb.YemongBlock(cfg)
+    assert torch.equal(block.field_sub[0].weight, torch.eye(32))  # griffin.py:365-368
+    assert torch.allclose(block.temporal[0].rg_lru.log_lambda, torch.linspace(0, 4, 32))  # griffin.py:165
+    assert block.temporal[0].conv.weight.shape == (32, 1, 4) and block.temporal[0].rg_lru.c == 8.0
+
+
+def test_hidden_state_shape_and_reset_are_env_major():
+    # tests/models/test_encoder.py:272-303, :384-405
+    cfg = bnb.ModelConfig(d_model=16, n_heads=4, n_yemong_blocks=2, n_temporal_per_block=2)
+    trunk = bnb.YemongTrunk(cfg)
+    B, N = 3, 4
+    hidden = trunk.initial_hidden(B, N, torch.device("cpu"))
+    assert hidden.shape == (4, B * N, 4 * 16) and hidden.dtype == torch.float32 and not hidden.any()
+    hidden = torch.randn_like(hidden)
+    done = torch.tensor([False, True, False])
+    out = trunk.reset_hidden_for_envs(hidden, done, N)
+    assert (out[:, N:2 * N] == 0).all()
+    assert torch.equal(out[:, :N], hidden[:, :N]) and torch.equal(out[:, 2 * N:], hidden[:, 2 * N:])
+
+
+def test_workloads_and_traffic_model():
+    w = harness.WORKLOADS
+    assert [x.tokens_per_step for x in w.values()] == [12288, 98304, 94208, 344064, 655360]
+    got = {k: harness.algorithmic_bytes(v)["step"] for k, v in w.items()}
+    assert got == {
+        "c0_4v4_fp32": 1024 * (24588 + 20480),
+        "c1_4v4_rollout_bf16": 8192 * (12300 + 16384),
+        "c2_8v11_bf16": 4096 * (23575 + 38912),
+        "c3_32v48_bf16": 4096 * (86100 + 163840),
+        "c4_64v88_bf16": 4096 * (164000 + 311296),
+    }
+    assert harness.attention_flops(w["c4_64v88_bf16"]) == 4096 * 4 * 160 * 160 * 128
+
+
+def test_alive_generators():
+    w = harness.WORKLOADS
+    a0 = harness.make_alive(w["c0_4v4_fp32"])
+    assert a0.shape == (1, 1024, 12) and a0[..., 8:].all()
+    assert 0.8 < a0[..., :8].float().mean() < 0.9
+    a1 = harness.make_alive(w["c1_4v4_rollout_bf16"], steps=16, B=512)
+    assert a1[0].all()
+    assert (a1[1:] <= a1[:-1]).all()  # monotone dying
+    assert a1[-1].float().mean() < 1.0
+    a4 = harness.make_alive(w["c4_64v88_bf16"], steps=2, B=2048)
+    live = a4[0].sum(-1)
+    assert live.min() >= 16 and live.max() <= 160 and a4[0, :, 152:].all() and torch.equal(a4[0], a4[1])
+    assert torch.equal(harness.make_alive(w["c2_8v11_bf16"]), harness.make_alive(w["c2_8v11_bf16"]))  # seeded
+
+
+def test_inputs_are_seeded_and_typed():
+    w = harness.WORKLOADS["c1_4v4_rollout_bf16"]
+    t1, s1 = harness.make_inputs(w, B=8)
+    t2, s2 = harness.make_inputs(w, B=8)
+    assert torch.equal(t1, t2) and torch.equal(s1, s2)
+    assert t1.dtype == torch.bfloat16 and s1.dtype == torch.float32 and s1.shape == (64, 128)
+    p = harness.make_weights(w.seed, w.dtype)
+    assert p["qkv.weight"].shape == (384, 128) and p["log_lambda"].dtype == torch.float32

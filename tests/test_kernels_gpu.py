@@ -1,0 +1,345 @@
+"""Parity of the two HIP kernels (through the C ABI) against the CPU oracle.
+
+Bars: float32 max relative error <= 1e-5, bfloat16 <= 2e-2 (both as max|y-ref|/max|ref|
+against the float32 oracle evaluated on the same, already rounded, inputs), identical
+alive-masking behaviour (dead keys weigh exactly nothing, an all-dead environment is the
+mean of V, dead queries are computed).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import max_rel
+from oracle import c_ref, torch_ref
+
+from boost_and_broadside_amd import harness, ops
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 1e-5
+BF16_TOL = 2e-2
+DEV = "cuda:0"
+
+
+def _qkv(seed, B, NM, D, dtype, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (scale * torch.randn(B, NM, 3 * D, generator=g)).to(dtype)
+
+
+def _alive(seed, B, NM, p):
+    g = torch.Generator().manual_seed(seed + 99)
+    return torch.rand(B, NM, generator=g) < p
+
+
+def _run_sdpa(qkv, alive, H, path="auto"):
+    out = ops.sdpa_masked(qkv.to(DEV), None if alive is None else alive.to(DEV), H, path=path)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+# ------------------------------------------------------------------ masked attention, fp32
+
+
+@pytest.mark.parametrize(
+    "B,NM,H,dh",
+    [(3, 12, 4, 32), (5, 23, 4, 32), (2, 1, 4, 32), (7, 8, 4, 32), (2, 31, 4, 32), (3, 84, 4, 32),
+     (2, 160, 4, 32), (1, 200, 4, 32), (4, 9, 4, 16), (4, 6, 4, 8), (2, 10, 2, 64), (65, 12, 4, 32)],
+)
+def test_sdpa_fp32_matches_oracle(B, NM, H, dh):
+    qkv = _qkv(B * 1000 + NM, B, NM, H * dh, torch.float32)
+    alive = _alive(NM, B, NM, 0.75)
+    alive[:, 0] = True
+    got = _run_sdpa(qkv, alive, H)
+    ref = torch_ref.sdpa_masked(qkv, alive, H)
+    assert max_rel(got, ref) <= F32_TOL
+    assert torch.allclose(got, ref, rtol=1e-4, atol=2e-6)
+    if B * NM * NM <= 40000:  # the plain-C statement as a second, torch-free witness
+        cc = torch.from_numpy(c_ref.sdpa_masked(qkv.numpy(), alive.numpy(), H))
+        assert max_rel(got, cc) <= F32_TOL
+
+
+def test_sdpa_fp32_large_scores_stay_exact():
+    # scores of magnitude ~50 exercise the running-max rescaling
+    qkv = _qkv(5, 4, 23, 128, torch.float32, scale=3.0)
+    alive = _alive(5, 4, 23, 0.6)
+    alive[:, 3] = True
+    assert max_rel(_run_sdpa(qkv, alive, 4), torch_ref.sdpa_masked(qkv, alive, 4)) <= F32_TOL
+
+
+def test_sdpa_no_mask_equals_all_alive():
+    qkv = _qkv(6, 3, 12, 128, torch.float32)
+    a = _run_sdpa(qkv, None, 4)
+    b = _run_sdpa(qkv, torch.ones(3, 12, dtype=torch.bool), 4)
+    assert torch.equal(a, b)
+    assert max_rel(a, torch_ref.sdpa_masked(qkv, None, 4)) <= F32_TOL
+
+
+@pytest.mark.parametrize("dtype,path,NM", [(torch.float32, "valu", 12), (torch.bfloat16, "valu", 12),
+                                          (torch.bfloat16, "mfma", 84), (torch.bfloat16, "mfma", 160)])
+def test_all_dead_environment_is_mean_of_values(dtype, path, NM):
+    B, H, D = 3, 4, 128
+    qkv = _qkv(7, B, NM, D, dtype)
+    alive = torch.ones(B, NM, dtype=torch.bool)
+    alive[1] = False  # everyone dead in env 1
+    got = _run_sdpa(qkv, alive, H, path).float()
+    assert torch.isfinite(got).all()
+    mean_v = qkv[1, :, 2 * D:].float().mean(dim=0, keepdim=True).expand(NM, D)
+    tol = 2e-6 if dtype == torch.float32 else 1.6e-2
+    assert (got[1] - mean_v).abs().max() <= tol
+    ref = torch_ref.sdpa_masked(qkv.float(), alive, H)
+    assert max_rel(got, ref) <= (F32_TOL if dtype == torch.float32 else BF16_TOL)
+
+
+@pytest.mark.parametrize("dtype,path,NM", [(torch.float32, "valu", 12), (torch.bfloat16, "valu", 23),
+                                          (torch.bfloat16, "mfma", 84), (torch.bfloat16, "mfma", 33)])
+def test_dead_keys_have_exactly_zero_weight(dtype, path, NM):
+    B, H, D = 4, 4, 128
+    qkv = _qkv(8, B, NM, D, dtype)
+    alive = _alive(8, B, NM, 0.6)
+    alive[:, 1] = True
+    base = _run_sdpa(qkv, alive, H, path)
+    pert = qkv.clone()
+    dead = ~alive
+    pert[..., D:][dead] = pert[..., D:][dead] * -3.0 + 17.0  # K and V rows of dead tokens only
+    again = _run_sdpa(pert, alive, H, path)
+    assert torch.equal(base, again)
+    assert base[dead].float().abs().max() > 0  # dead queries still produce rows
+
+
+def test_single_live_key_broadcasts_its_value_row():
+    B, NM, H, D = 2, 12, 4, 128
+    qkv = _qkv(9, B, NM, D, torch.float32)
+    alive = torch.zeros(B, NM, dtype=torch.bool)
+    alive[0, 7] = True
+    alive[1, 0] = True
+    got = _run_sdpa(qkv, alive, H)
+    assert torch.allclose(got[0], qkv[0, 7, 2 * D:].expand(NM, D), atol=1e-6)
+    assert torch.allclose(got[1], qkv[1, 0, 2 * D:].expand(NM, D), atol=1e-6)
+
+
+def test_sdpa_accepts_padded_rows_and_uint8_mask():
+    B, NM, H, D = 3, 12, 4, 128
+    qkv = _qkv(10, B, NM, D, torch.float32)
+    wide = torch.zeros(B, NM, 3 * D + 64)
+    wide[..., : 3 * D] = qkv
+    alive = _alive(10, B, NM, 0.7)
+    alive[:, 2] = True
+    view = wide.to(DEV)[..., : 3 * D]  # row stride 448 elements
+    got = ops.sdpa_masked(view, alive.to(DEV).to(torch.uint8), H).cpu()
+    assert max_rel(got, torch_ref.sdpa_masked(qkv, alive, H)) <= F32_TOL
+
+
+def test_sdpa_empty_and_rejected_inputs():
+    assert ops.sdpa_masked(torch.zeros(0, 12, 384, device=DEV), None, 4).shape == (0, 12, 128)
+    assert ops.sdpa_masked(torch.zeros(2, 0, 384, device=DEV), None, 4).shape == (2, 0, 128)
+    with pytest.raises(RuntimeError, match="outside what the kernels cover"):
+        ops.sdpa_masked(torch.zeros(1, 4, 3 * 4 * 24, device=DEV), None, 4)  # head_dim 24
+    with pytest.raises(RuntimeError, match="outside what the kernels cover"):
+        ops.sdpa_masked(torch.zeros(1, 600, 384, device=DEV), None, 4)  # more tokens than supported
+    with pytest.raises(RuntimeError, match="outside what the kernels cover"):
+        ops.sdpa_masked(torch.zeros(1, 12, 384, device=DEV), None, 4, path="mfma")  # fp32 on the bf16 kernel
+    with pytest.raises(TypeError):
+        ops.sdpa_masked(torch.zeros(1, 4, 384, device=DEV, dtype=torch.float16), None, 4)
+
+
+# ------------------------------------------------------------------ masked attention, bf16
+
+
+@pytest.mark.parametrize(
+    "B,NM,path",
+    [(5, 12, "valu"), (4, 23, "valu"), (3, 31, "valu"), (3, 12, "mfma"), (3, 23, "mfma"), (3, 32, "mfma"),
+     (3, 33, "mfma"), (4, 84, "mfma"), (3, 96, "mfma"), (2, 129, "mfma"), (3, 160, "mfma"), (2, 160, "valu"),
+     (3, 84, "auto"), (9, 12, "auto")],
+)
+def test_sdpa_bf16_matches_fp32_oracle(B, NM, path):
+    H, D = 4, 128
+    qkv = _qkv(B * 77 + NM, B, NM, D, torch.bfloat16)
+    alive = _alive(NM + 1, B, NM, 0.7)
+    alive[:, NM // 2] = True
+    got = _run_sdpa(qkv, alive, H, path)
+    assert got.dtype == torch.bfloat16
+    truth = torch_ref.sdpa_masked(qkv.float(), alive, H)
+    assert max_rel(got.float(), truth) <= BF16_TOL
+    # no worse than the reference's own bf16 path (library SDPA on bf16 tensors) by more than rounding
+    lib16 = torch_ref.sdpa_masked(qkv, alive, H).float()
+    assert max_rel(got.float(), truth) <= max_rel(lib16, truth) + 8e-3
+
+
+def test_sdpa_bf16_both_kernels_agree():
+    B, NM, H, D = 6, 84, 4, 128
+    qkv = _qkv(21, B, NM, D, torch.bfloat16)
+    alive = _alive(21, B, NM, 0.7)
+    alive[:, 0] = True
+    a = _run_sdpa(qkv, alive, H, "valu").float()
+    b = _run_sdpa(qkv, alive, H, "mfma").float()
+    assert max_rel(a, b) <= 1.2e-2
+
+
+def test_sdpa_mfma_live_counts_across_block_edges():
+    # live keys 1, 31, 32, 33, 64, 65, 159, 160 of NM = 160: every padding/compaction edge
+    NM, H, D = 160, 4, 128
+    counts = [1, 31, 32, 33, 64, 65, 159, 160]
+    B = len(counts)
+    qkv = _qkv(22, B, NM, D, torch.bfloat16)
+    g = torch.Generator().manual_seed(22)
+    alive = torch.zeros(B, NM, dtype=torch.bool)
+    for b, c in enumerate(counts):
+        alive[b, torch.randperm(NM, generator=g)[:c]] = True
+    got = _run_sdpa(qkv, alive, H, "mfma").float()
+    truth = torch_ref.sdpa_masked(qkv.float(), alive, H)
+    for b in range(B):
+        assert max_rel(got[b], truth[b]) <= BF16_TOL, counts[b]
+
+
+def test_sdpa_environment_permutation_is_bitwise_equivariant_at_full_size():
+    # full 64v88 batch: shuffling environments must shuffle outputs bit for bit
+    w = harness.WORKLOADS["c4_64v88_bf16"]
+    g = torch.Generator(device=DEV).manual_seed(3)
+    qkv = torch.randn(w.B, w.NM, 384, device=DEV, generator=g).bfloat16()
+    alive = harness.make_alive(w, steps=1)[0].to(DEV)
+    perm = torch.randperm(w.B, device=DEV)
+    a = ops.sdpa_masked(qkv, alive, 4)
+    b = ops.sdpa_masked(qkv[perm].contiguous(), alive[perm].contiguous(), 4)
+    assert torch.equal(a[perm], b)
+    # and a sample of environments against the CPU oracle
+    pick = torch.arange(0, w.B, 257)
+    truth = torch_ref.sdpa_masked(qkv[pick].float().cpu(), alive[pick].cpu(), 4)
+    assert max_rel(a[pick].float().cpu(), truth) <= BF16_TOL
+
+
+# ------------------------------------------------------------------ RG-LRU step
+
+
+def _rglru_inputs(seed, R, D, xdt, gdt):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(R, D, generator=g).to(xdt)
+    gates = (1.5 * torch.randn(R, 2 * D, generator=g)).to(gdt)
+    h = 0.5 * torch.randn(R, D, generator=g)
+    return x, gates, torch.linspace(0.0, 4.0, D), h
+
+
+@pytest.mark.parametrize("R,D", [(1, 128), (17, 128), (1000, 128), (4097, 128), (33, 32), (9, 64), (5, 12), (3, 136)])
+def test_rglru_fp32_matches_oracle(R, D):
+    x, gates, lam, h = _rglru_inputs(R + D, R, D, torch.float32, torch.float32)
+    y, h_new = ops.rglru_step(x.to(DEV), gates.to(DEV), lam.to(DEV), 8.0, h.to(DEV))
+    assert y is h_new and h_new.dtype == torch.float32
+    ref = torch_ref.rglru_step(x, gates, lam, 8.0, h)
+    assert max_rel(h_new.cpu(), ref) <= F32_TOL
+    assert torch.allclose(h_new.cpu(), ref, rtol=2e-5, atol=2e-6)
+    cc = torch.from_numpy(c_ref.rglru_step(x.numpy(), gates.numpy(), lam.numpy(), 8.0, h.numpy()))
+    assert max_rel(h_new.cpu(), cc) <= F32_TOL
+
+
+def test_rglru_known_answers_on_device():
+    D = 128
+    lam = torch.linspace(0.0, 4.0, D)
+    h = torch.full((2, D), 2.0)
+    x = torch.full((2, D), 0.5)
+    big = 40.0
+    gates = torch.cat([torch.full((2, D), -big), torch.full((2, D), big)], dim=-1)  # r -> 0, i -> 1
+    _, out = ops.rglru_step(x.to(DEV), gates.to(DEV), lam.to(DEV), 8.0, h.to(DEV))
+    assert torch.allclose(out.cpu(), h + 1e-3 * x, rtol=1e-6)  # a = 1, clamp floor => gate = 1e-3
+    gates = torch.full((2, 2 * D), big)  # r -> 1
+    _, out = ops.rglru_step(torch.zeros(2, D, device=DEV), gates.to(DEV), lam.to(DEV), 8.0, h.to(DEV))
+    assert float(out[0, 0]) == pytest.approx(2.0 * 0.5 ** 8, rel=1e-6)  # lambda = 0 => a = 0.5^8
+
+
+def test_rglru_reads_and_writes_the_packed_hidden_in_place():
+    # state rows live inside a (R, 4D) tensor, as in the policy's packed hidden (policy.py:323)
+    R, D = 50, 128
+    x, gates, lam, h = _rglru_inputs(3, R, D, torch.float32, torch.float32)
+    packed = torch.randn(R, 4 * D)
+    packed[:, :D] = h
+    dev = packed.to(DEV)
+    view = dev[:, :D]
+    y, h_new = ops.rglru_step(x.to(DEV), gates.to(DEV), lam.to(DEV), 8.0, view, h_out=view)
+    ref = torch_ref.rglru_step(x, gates, lam, 8.0, h)
+    assert h_new.data_ptr() == dev.data_ptr()
+    assert max_rel(dev[:, :D].cpu(), ref) <= F32_TOL
+    assert torch.equal(dev[:, D:].cpu(), packed[:, D:])  # conv-buffer columns untouched
+
+
+@pytest.mark.parametrize("xdt,gdt", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.bfloat16),
+                                     (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("R,D", [(257, 128), (6, 20)])
+def test_rglru_bf16_follows_autocast_dtype_flow(xdt, gdt, R, D):
+    x, gates, lam, h = _rglru_inputs(R, R, D, xdt, gdt)
+    y, h_new = ops.rglru_step(x.to(DEV), gates.to(DEV), lam.to(DEV), 8.0, h.to(DEV), y_dtype=torch.bfloat16)
+    assert y.dtype == torch.bfloat16 and h_new.dtype == torch.float32
+    truth = torch_ref.rglru_step(x.float(), gates.float(), lam, 8.0, h)
+    assert max_rel(h_new.cpu(), truth) <= BF16_TOL
+    assert max_rel(y.float().cpu(), truth) <= BF16_TOL
+    # same operations in the same dtypes on the CPU: only transcendental rounding may differ
+    mirror = torch_ref.rglru_step(x, gates, lam, 8.0, h)
+    assert mirror.dtype == torch.float32
+    assert max_rel(h_new.cpu(), mirror) <= 4e-3
+    assert torch.equal(y.cpu(), h_new.cpu().bfloat16())
+
+
+def test_rglru_empty_and_rejected_inputs():
+    lam = torch.linspace(0, 4, 128, device=DEV)
+    y, h = ops.rglru_step(torch.zeros(0, 128, device=DEV), torch.zeros(0, 256, device=DEV), lam, 8.0,
+                          torch.zeros(0, 128, device=DEV))
+    assert h.shape == (0, 128)
+    with pytest.raises(TypeError):
+        ops.rglru_step(torch.zeros(2, 128, device=DEV), torch.zeros(2, 256, device=DEV), lam, 8.0,
+                       torch.zeros(2, 128, device=DEV, dtype=torch.bfloat16))
+
+
+def test_rglru_rollout_of_full_size_state_matches_oracle_on_sampled_rows():
+    # 64v88 state (622,592 rows), 4 carried steps; rows sampled across the tensor go through the oracle
+    w = harness.WORKLOADS["c4_64v88_bf16"]
+    R, D, T = w.B * w.N, 128, 4
+    g = torch.Generator(device=DEV).manual_seed(11)
+    lam = torch.linspace(0, 4, D, device=DEV)
+    h = 0.5 * torch.randn(R, D, device=DEV, generator=g)
+    pick = torch.arange(0, R, 9973, device=DEV)
+    h_ref = h[pick].cpu()
+    for t in range(T):
+        x = torch.randn(R, D, device=DEV, generator=g).bfloat16()
+        gates = torch.randn(R, 2 * D, device=DEV, generator=g).bfloat16()
+        y, h = ops.rglru_step(x, gates, lam, 8.0, h, y_dtype=torch.bfloat16)
+        h_ref = torch_ref.rglru_step(x[pick].float().cpu(), gates[pick].float().cpu(), lam.cpu(), 8.0, h_ref)
+        assert max_rel(h[pick].cpu(), h_ref) <= BF16_TOL, t
+    assert torch.isfinite(h).all()
+
+
+# ------------------------------------------------------------------ the measured step
+
+
+@pytest.mark.parametrize("name,B", [("c0_4v4_fp32", None), ("c1_4v4_rollout_bf16", 256), ("c2_8v11_bf16", 128),
+                                    ("c3_32v48_bf16", 32), ("c4_64v88_bf16", 16)])
+def test_step_matches_oracle_on_benchmark_workloads(name, B):
+    w = harness.WORKLOADS[name]
+    B = w.B if B is None else B
+    p = harness.make_weights(w.seed, w.dtype)
+    tokens, state = harness.make_inputs(w, B=B)
+    alive = harness.make_alive(w, steps=1, B=B)[0]
+    step = harness.AttnRglruStep.from_weights(p, DEV)
+    hidden, new_state = step(tokens.to(DEV), alive.to(DEV), state.to(DEV))
+    p32 = {k: v.float() for k, v in p.items()}
+    ref_hidden, ref_state = torch_ref.harness_step(p32, tokens.float(), alive, state)
+    tol = F32_TOL if w.dtype == torch.float32 else BF16_TOL
+    assert hidden.dtype == w.dtype and new_state.dtype == torch.float32
+    assert max_rel(hidden.float().cpu(), ref_hidden) <= tol
+    assert max_rel(new_state.cpu(), ref_state) <= tol
+
+
+def test_step_carried_rollout_with_dying_ships():
+    # 4v4 rollout shape, 12 carried steps, ships dying along the way
+    w = harness.WORKLOADS["c1_4v4_rollout_bf16"]
+    B, T = 64, 12
+    p = harness.make_weights(w.seed, w.dtype)
+    step = harness.AttnRglruStep.from_weights(p, DEV)
+    p32 = {k: v.float() for k, v in p.items()}
+    alive = harness.make_alive(w, steps=T, B=B)
+    _, state = harness.make_inputs(w, B=B)
+    dev_state, ref_state = state.to(DEV), state
+    g = torch.Generator().manual_seed(5)
+    for t in range(T):
+        tokens = torch.randn(B, w.NM, 128, generator=g).bfloat16()
+        hidden, dev_state = step(tokens.to(DEV), alive[t].to(DEV), dev_state)
+        ref_hidden, ref_state = torch_ref.harness_step(p32, tokens.float(), alive[t], ref_state)
+        assert max_rel(hidden.float().cpu(), ref_hidden) <= BF16_TOL, t
+    assert max_rel(dev_state.cpu(), ref_state) <= BF16_TOL
