@@ -1,0 +1,332 @@
+"""Benchmark of the attention + RG-LRU step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+One "step" is one pass of the two kernels over one batch of synthetic input that is already
+resident in HBM: masked attention over every environment's packed q/k/v rows, then the
+RG-LRU update of every ship row with the recurrent state carried from step to step.  The
+projections around the kernels (4 GEMMs) are torch library calls and are reported
+separately (``module``), as are the same two regions run through eager PyTorch on the GPU
+(``torch_gpu_baseline``) and on the host cores (``cpu_baseline``).  Rank 0 prints one JSON
+line.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+import torch.nn.functional as F
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "entity-tokens/sec through attention+RG-LRU step; % of HBM roofline"
+POOL = 4  # distinct input batches cycled through the timed steps
+
+
+def parse_args():
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default: the workload's rollout length, at least 32)")
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--workload", default=None, help="one of the harness workloads (default: the 64v88 headline)")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU-baseline leg; 0 skips it")
+    ap.add_argument("--no-torch-baseline", action="store_true")
+    ap.add_argument("--no-module", action="store_true")
+    return ap.parse_args()
+
+
+# ---------------------------------------------------------------------------------------------
+# reference-style eager PyTorch statements of the two regions (the GPU baseline being beaten);
+# written out here so that the benchmark's GPU legs do not touch the CPU checker
+# ---------------------------------------------------------------------------------------------
+
+
+def torch_attention_region(qkv, alive, n_heads):
+    B, NM, D3 = qkv.shape
+    D = D3 // 3
+    dh = D // n_heads
+    q, k, v = qkv.chunk(3, dim=-1)
+    q = q.view(B, NM, n_heads, dh).permute(0, 2, 1, 3)
+    k = k.view(B, NM, n_heads, dh).permute(0, 2, 1, 3)
+    v = v.view(B, NM, n_heads, dh).permute(0, 2, 1, 3)
+    keep = alive.view(B, 1, 1, NM).to(q.dtype)
+    bias = (1.0 - keep) * (torch.finfo(q.dtype).min / 2)
+    out = F.scaled_dot_product_attention(q, k, v, attn_mask=bias, dropout_p=0.0)
+    return out.permute(0, 2, 1, 3).reshape(B, NM, D)
+
+
+def torch_rglru_region(x, gates, log_lambda, c, h):
+    D = x.shape[-1]
+    r = torch.sigmoid(gates[:, :D])
+    i = torch.sigmoid(gates[:, D:])
+    a = torch.sigmoid(log_lambda) ** (c * r)
+    gate = torch.sqrt(torch.clamp((1.0 - a) * (1.0 + a), min=1e-6))
+    return a * h + gate * (i * x)
+
+
+# ---------------------------------------------------------------------------------------------
+
+
+def timed_loop(fn, steps, warmup):
+    """Run fn(t) for warmup + steps iterations; wall-clock seconds of the timed part."""
+    for t in range(warmup):
+        fn(t)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t in range(steps):
+        fn(warmup + t)
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def event_split(launch_a, launch_b, steps, warmup):
+    """Average device time of the two launches, from events on the stream they run on."""
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    for t in range(warmup):
+        launch_a(t)
+        launch_b(t)
+    torch.cuda.synchronize()
+    for t in range(steps):
+        ev[t][0].record()
+        launch_a(warmup + t)
+        ev[t][1].record()
+        launch_b(warmup + t)
+        ev[t][2].record()
+    torch.cuda.synchronize()
+    ta = sum(e[0].elapsed_time(e[1]) for e in ev) / steps * 1e-3
+    tb = sum(e[1].elapsed_time(e[2]) for e in ev) / steps * 1e-3
+    return ta, tb
+
+
+def cpu_baseline(w, p, budget_s):
+    """The CPU checker (torch restatement of the reference ops) timed on the host cores.
+
+    Same two regions as the GPU figure (attention incl. bias and head merge; RG-LRU
+    element-wise chain), float32, on a slice of the workload's environments sized so the
+    leg stays within ``budget_s`` seconds.
+    """
+    from oracle import torch_ref
+
+    from boost_and_broadside_amd import harness
+
+    threads = torch.get_num_threads()
+    B = min(w.B, 256)
+    p32 = {k: v.float() for k, v in p.items()}
+    tokens, state = harness.make_inputs(w, B=B)
+    alive = harness.make_alive(w, steps=1, B=B)[0]
+    tokens = tokens.float()
+    qkv = F.linear(tokens, p32["qkv.weight"])
+    u = F.linear(torch_ref.sdpa_masked(qkv, alive, harness.N_HEADS), p32["out_proj.weight"])
+    ships = u[:, : w.N].reshape(B * w.N, -1).contiguous()
+    gates = torch_ref.rglru_gates(p32, "", ships)
+
+    def once():
+        torch_ref.sdpa_masked(qkv, alive, harness.N_HEADS)
+        return torch_ref.rglru_step(ships, gates, p32["log_lambda"], 8.0, state)
+
+    once()
+    t0 = time.perf_counter()
+    once()
+    one = max(time.perf_counter() - t0, 1e-6)
+    reps = int(max(3, min(200, budget_s / one)))
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        once()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": B * w.NM / med,
+        "unit": "entity-tokens/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{B} of {w.B} environments of {w.name}, float32, {reps} repetitions of the two regions "
+                  f"(torch SDPA with additive key bias + head merge; RG-LRU element-wise chain), median",
+        "ms_per_step_sample": med * 1e3,
+        "cpu_model": _cpu_model(),
+    }
+
+
+def _cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def load_traffic(kernel, workload):
+    """Measured HBM bytes per launch, if a counter summary has been recorded for this pair."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        table = json.load(open(path))
+    except (OSError, ValueError):
+        return None
+    return table.get(f"{kernel}:{workload}")
+
+
+def main():
+    args = parse_args()
+    world = int(os.environ.get("WORLD_SIZE", "1"))
+    if args.gpus != 1 or world != 1:
+        print(
+            "bench.py measures one GPU: environments are independent, so more GPUs would only shard the batch "
+            f"with no exchange; run it with --gpus 1 (got --gpus {args.gpus}, WORLD_SIZE {world}).",
+            file=sys.stderr,
+        )
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a ROCm GPU (the kernels have no host fallback)", file=sys.stderr)
+        sys.exit(2)
+
+    import boost_and_broadside_amd as bnb
+    from boost_and_broadside_amd import harness, ops
+
+    bnb._native.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = harness.WORKLOADS[args.workload or harness.HEADLINE]
+    steps = args.steps if args.steps is not None else max(w.steps, 32)
+    warmup = args.warmup
+    H, D = harness.N_HEADS, harness.D_MODEL
+    bf16 = w.dtype == torch.bfloat16
+
+    # ---- synthetic inputs, resident in HBM before anything is timed ----
+    p = harness.make_weights(w.seed, w.dtype)
+    step_module = harness.AttnRglruStep.from_weights(p, dev)
+    alive_steps = harness.make_alive(w, steps=min(max(w.steps, 1), warmup + steps)).to(dev)
+    n_alive = alive_steps.shape[0]
+    gen = torch.Generator(device=dev).manual_seed(w.seed)
+    tokens_pool = [torch.randn(w.B, w.NM, D, device=dev, generator=gen).to(w.dtype) for _ in range(POOL)]
+    state0 = 0.5 * torch.randn(w.B * w.N, D, device=dev, generator=gen)
+    lam = step_module.log_lambda.detach()
+
+    # kernel inputs exactly as the projections produce them
+    qkv_pool, x_pool, gates_pool = [], [], []
+    with torch.no_grad():
+        for i in range(POOL):
+            qkv = step_module.qkv(tokens_pool[i])
+            merged = ops.sdpa_masked(qkv, alive_steps[0], H)
+            ships = step_module.out_proj(merged)[:, : w.N].reshape(w.B * w.N, D).contiguous()
+            qkv_pool.append(qkv)
+            x_pool.append(ships)
+            gates_pool.append(step_module.gates(ships))
+    o_buf = torch.empty(w.B, w.NM, D, dtype=w.dtype, device=dev)
+    y_buf = torch.empty(w.B * w.N, D, dtype=torch.bfloat16, device=dev) if bf16 else None
+    h_bufs = [state0.clone(), torch.empty_like(state0)]
+    y_dtype = torch.bfloat16 if bf16 else None
+
+    def launch_attn(t):
+        ops.sdpa_masked(qkv_pool[t % POOL], alive_steps[t % n_alive], H, out=o_buf)
+
+    def launch_rglru(t):
+        ops.rglru_step(x_pool[t % POOL], gates_pool[t % POOL], lam, 8.0, h_bufs[t & 1], h_out=h_bufs[(t + 1) & 1],
+                       y_dtype=y_dtype, y_out=y_buf)
+
+    def kernel_step(t):
+        launch_attn(t)
+        launch_rglru(t)
+
+    wall = timed_loop(kernel_step, steps, warmup)
+    t_attn, t_rglru = event_split(launch_attn, launch_rglru, steps, warmup)
+    assert torch.isfinite(h_bufs[0]).all() and torch.isfinite(o_buf.float()).all()
+
+    tokens = w.tokens_per_step
+    ab = harness.algorithmic_bytes(w)
+    peak = harness.HBM_PEAK_BYTES_PER_S
+
+    def roof(kernel, nbytes, seconds):
+        return {
+            "kernel": kernel, "bound": "hbm", "achieved": nbytes / seconds / 1e9, "peak": peak / 1e9, "unit": "GB/s",
+            "frac": nbytes / seconds / peak, "algorithmic_bytes_per_launch": nbytes, "avg_launch_us": seconds * 1e6,
+            "traffic": load_traffic(kernel, w.name),
+        }
+
+    attn_kernel = "sdpa_mfma_kernel" if (bf16 and 32 <= w.NM <= 160) else "sdpa_valu_kernel"
+    roofs = {"attention": roof(attn_kernel, ab["attn"], t_attn), "rglru": roof("rglru_step_vec8_kernel", ab["rglru"], t_rglru)}
+    dominant = "attention" if t_attn >= t_rglru else "rglru"
+
+    result = {
+        "metric": METRIC,
+        "value": tokens * steps / wall,
+        "unit": "entity-tokens/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": wall / steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if bf16 else "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{w.name}: {w.B} environments x ({w.N} ship + {w.M} field tokens), d_model {D}, "
+                        f"{H} heads x {D // H}, alive mask '{w.alive}', fp32 recurrent state carried over the steps",
+            "region": "masked attention kernel + RG-LRU step kernel (the 4 projections are reported under 'module')",
+            "tokens_per_step": tokens,
+        },
+        "roofline": roofs[dominant],
+        "roofline_step": {
+            "bound": "hbm", "achieved": ab["step"] / (t_attn + t_rglru) / 1e9, "peak": peak / 1e9, "unit": "GB/s",
+            "frac": ab["step"] / (t_attn + t_rglru) / peak, "algorithmic_bytes_per_step": ab["step"],
+            "kernel_us_per_step": (t_attn + t_rglru) * 1e6,
+        },
+        "kernels": roofs,
+    }
+
+    # ---- yardstick: plain copy through the library's copy kernel ----
+    n_copy = 1 << 30
+    src = torch.empty(n_copy, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    t_copy = timed_loop(lambda t: ops.copy_bytes(src, dst), 20, 3) / 20
+    result["copy_kernel"] = {"GBps_read_plus_write": 2 * n_copy / t_copy / 1e9, "bytes": n_copy}
+    del src, dst
+
+    # ---- the same two regions through eager PyTorch on the GPU ----
+    if not args.no_torch_baseline:
+        hb = [state0.clone()]
+
+        def torch_step(t):
+            torch_attention_region(qkv_pool[t % POOL], alive_steps[t % n_alive], H)
+            hb[0] = torch_rglru_region(x_pool[t % POOL], gates_pool[t % POOL], lam, 8.0, hb[0])
+
+        n_t = max(4, min(steps, 16))
+        wall_t = timed_loop(torch_step, n_t, 2)
+        result["torch_gpu_baseline"] = {
+            "value": tokens * n_t / wall_t, "unit": "entity-tokens/s", "ms_per_step": wall_t / n_t * 1e3,
+            "steps": n_t, "speedup_of_this_build": (tokens * steps / wall) / (tokens * n_t / wall_t),
+            "what": "F.scaled_dot_product_attention with additive key bias + head-merge copy, and the eager "
+                    "RG-LRU element-wise chain, same inputs, same dtype",
+        }
+
+    # ---- whole module step: 4 projections + the two kernels ----
+    if not args.no_module:
+        st = [state0.clone()]
+
+        def module_step(t):
+            _, st[0] = step_module(tokens_pool[t % POOL], alive_steps[t % n_alive], st[0])
+
+        wall_m = timed_loop(module_step, steps, warmup)
+        result["module"] = {"value": tokens * steps / wall_m, "unit": "entity-tokens/s", "ms_per_step": wall_m / steps * 1e3}
+
+    # free the device before the host leg
+    if args.cpu_seconds > 0:
+        result["cpu_baseline"] = cpu_baseline(w, p, args.cpu_seconds)
+    else:
+        result["cpu_baseline"] = None
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -43,6 +43,7 @@ def sdpa_masked(
     n_heads: int,
     *,
     path: str = "auto",
+    out: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Masked multi-head attention over each environment's tokens.
 
@@ -55,6 +56,7 @@ def sdpa_masked(
                  all keys; dead queries are still computed.
         n_heads: H; D must be divisible by it.
         path:    "auto" | "valu" | "mfma" — kernel selection, for tests and benchmarks.
+        out:     optional preallocated contiguous (B, NM, D) destination in qkv's dtype.
 
     Returns:
         (B, NM, D) in qkv's dtype, heads merged head-major (the input of ``out_proj``).
@@ -83,7 +85,10 @@ def sdpa_masked(
             raise RuntimeError(f"alive is on {alive.device}, qkv on {qkv.device}")
         alive = alive.contiguous()
         mask_ptr = alive.data_ptr()
-    out = torch.empty((B, NM, D), dtype=qkv.dtype, device=qkv.device)
+    if out is None:
+        out = torch.empty((B, NM, D), dtype=qkv.dtype, device=qkv.device)
+    elif out.shape != (B, NM, D) or out.dtype != qkv.dtype or out.device != qkv.device or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous {(B, NM, D)} {qkv.dtype} tensor on {qkv.device}")
     if B == 0 or NM == 0:
         return out
     with torch.cuda.device(qkv.device):
@@ -104,6 +109,7 @@ def rglru_step(
     *,
     h_out: torch.Tensor | None = None,
     y_dtype: torch.dtype | None = None,
+    y_out: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """One RG-LRU step given the two gate pre-activations.
 
@@ -118,6 +124,7 @@ def rglru_step(
                     itself for an in-place update).  Default: a new contiguous tensor.
         y_dtype:    dtype of the returned layer output.  None or float32 returns the new
                     state itself; bfloat16 makes the kernel write a rounded copy as well.
+        y_out:      optional preallocated contiguous bfloat16 (R, D) destination for that copy.
 
     Returns:
         (y, h_new): layer output and new state (the same tensor unless y_dtype is bfloat16).
@@ -153,7 +160,12 @@ def rglru_step(
     if y_dtype is not None and y_dtype != torch.float32:
         if y_dtype != torch.bfloat16:
             raise TypeError(f"y_dtype must be float32 or bfloat16, got {y_dtype}")
-        y = torch.empty((R, D), dtype=torch.bfloat16, device=x.device)
+        if y_out is None:
+            y = torch.empty((R, D), dtype=torch.bfloat16, device=x.device)
+        elif y_out.shape != (R, D) or y_out.dtype != torch.bfloat16 or y_out.device != x.device or not y_out.is_contiguous():
+            raise ValueError("y_out must be a contiguous bfloat16 (R, D) tensor on x's device")
+        else:
+            y = y_out
     if R == 0:
         return (h_out if y is None else y), h_out
     with torch.cuda.device(x.device):
