@@ -16,9 +16,10 @@
 //                      (environment, head, query) row, K/V of a group of environments
 //                      staged in LDS as fp32, chunked online softmax.  This is the 4v4 /
 //                      8v11 path (NM < 32) and the fp32 path.
-//   sdpa_mfma_kernel   bf16, dh = 32, 32 <= NM <= 160; one wavefront per (environment,
-//                      head); S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_32x32x16_bf16 so
-//                      that the softmax reductions over keys stay inside a lane.
+//   sdpa_mfma_kernel   bf16, dh = 32, 32 <= NM <= 160; one work-group per (environment,
+//                      head), one wavefront per 32 queries; S^T = K Q^T and O^T = V^T P^T on
+//                      v_mfma_f32_32x32x16_bf16 so that the softmax reductions over keys
+//                      stay inside a lane.
 
 #include "common.h"
 
@@ -193,16 +194,21 @@ __global__ __launch_bounds__(kValuThreads) void sdpa_valu_kernel(
 // keys in the same order: slot e of MFMA (kb,t) is key 32*kb + 16*t + 8*(e/4) + 4*half + e%4.
 
 constexpr int kDh = 32;
+constexpr int kKeyPitch = kDh + 8;  // halfs per K row in LDS: 80 bytes, 16-byte aligned, bank-spread
 
+// One work-group per (environment, head); wave w owns queries 32w .. 32w+31 and all waves
+// share the K rows and the transposed V rows of the live keys in LDS.
 template <int NKB>
-__global__ __launch_bounds__(kWave) void sdpa_mfma_kernel(
+__global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
     const uint16_t *__restrict__ qkv, int64_t row_stride, const uint8_t *__restrict__ alive,
     uint16_t *__restrict__ out, int B, int NM, int H, float scale_log2e)
 {
     constexpr int KCAP = NKB * 32;
     constexpr int VP = KCAP + 4;  // halfs per V^T row: 8-byte aligned, bank-spread
+    constexpr int NT = kWave * NKB;
+    __shared__ __align__(16) uint16_t s_k[KCAP * kKeyPitch];
     __shared__ __align__(16) uint16_t s_vt[kDh * VP];
-    __shared__ uint16_t s_kidx[KCAP];
+    __shared__ uint16_t s_cnt[2 * NKB];  // live keys per 16-key slice, in key order
 
     // Work-groups are dealt round-robin to the 8 XCDs; hand each XCD a contiguous run of
     // (environment, head) pairs so the 4 heads of an environment share one L2.
@@ -213,140 +219,163 @@ __global__ __launch_bounds__(kWave) void sdpa_mfma_kernel(
     const int head = logical - env * H;
     const int D = H * kDh;
 
-    const int lane = threadIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
     const int m = lane & 31;
     const int half = lane >> 5;
 
-    // ---- compacted list of live keys (all keys when none is alive) ----
-    int cnt = 0;
-    for (int base = 0; base < NM; base += kWave) {
-        const int key = base + lane;
-        bool a = key < NM;
-        if (a && alive != nullptr) a = alive[(int64_t)env * NM + key] != 0;
-        const uint64_t mask = __ballot(a);
-        const int before = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
-                                                     __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
-        if (a) s_kidx[cnt + before] = (uint16_t)key;
-        cnt += __popcll(mask);
-    }
-    const bool uniform = (cnt == 0);
-    if (uniform) {
-        cnt = NM;
-        for (int key = lane; key < NM; key += kWave) s_kidx[key] = (uint16_t)key;
-    }
-    __syncthreads();
-    const int nkb = (cnt + 31) >> 5;
-
     const uint16_t *env_base = qkv + (int64_t)env * NM * row_stride;
 
-    // ---- V^T into LDS: lane -> (position pos, 8 channels) ----
-    for (int pos0 = 0; pos0 < nkb * 32; pos0 += 16) {
-        const int pos = pos0 + (lane >> 2);
-        const int c8 = (lane & 3) * 8;
-        u32x4 w = {0u, 0u, 0u, 0u};
-        if (pos < cnt) {
-            const int key = s_kidx[pos];
-            w = *reinterpret_cast<const u32x4 *>(env_base + (int64_t)key * row_stride + 2 * D + head * kDh + c8);
+    // ---- this wave's queries: issue the loads before anything else ----
+    const int qrow = wave * 32 + m;
+    const int qsafe = qrow < NM ? qrow : NM - 1;
+    const uint16_t *qp = env_base + (int64_t)qsafe * row_stride + head * kDh + half * 8;
+    const u32x4 qw0 = *reinterpret_cast<const u32x4 *>(qp);
+    const u32x4 qw1 = *reinterpret_cast<const u32x4 *>(qp + 16);
+
+    // ---- K rows and V^T of the live keys into LDS, compacted ----
+    // Thread -> (key, 8 channels), two items per thread.  A thread reads its key's alive
+    // byte, starts its K/V loads at once if the key is live, and only then works out the
+    // key's position among the live keys (ballot inside the wave, per-wave counts through
+    // LDS), so the position arithmetic overlaps the loads.
+    const uint8_t *alive_env = alive == nullptr ? nullptr : alive + (int64_t)env * NM;
+    int cnt = 0;
+    bool uniform = false;
+    for (int pass = 0; pass < 2; ++pass) {
+        bool live[2];
+        u32x4 kw[2], vw[2];
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int key = (tid + it * NT) >> 2;
+            live[it] = key < NM;
+            if (live[it] && alive_env != nullptr && !uniform) live[it] = alive_env[key] != 0;
         }
-        uint16_t *dst = s_vt + c8 * VP + pos;
-        dst[0 * VP] = (uint16_t)(w.x & 0xffffu);
-        dst[1 * VP] = (uint16_t)(w.x >> 16);
-        dst[2 * VP] = (uint16_t)(w.y & 0xffffu);
-        dst[3 * VP] = (uint16_t)(w.y >> 16);
-        dst[4 * VP] = (uint16_t)(w.z & 0xffffu);
-        dst[5 * VP] = (uint16_t)(w.z >> 16);
-        dst[6 * VP] = (uint16_t)(w.w & 0xffffu);
-        dst[7 * VP] = (uint16_t)(w.w >> 16);
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            if (live[it]) {
+                const int idx = tid + it * NT;
+                const uint16_t *rp = env_base + (int64_t)(idx >> 2) * row_stride + head * kDh + (idx & 3) * 8;
+                kw[it] = *reinterpret_cast<const u32x4 *>(rp + D);
+                vw[it] = *reinterpret_cast<const u32x4 *>(rp + 2 * D);
+            }
+        }
+        int before[2];
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const uint64_t mask = __ballot(live[it] && (lane & 3) == 0);  // one bit per live key
+            before[it] = __popcll(mask & ((1ull << (lane & ~3)) - 1ull));
+            if (lane == 0) s_cnt[it * NKB + wave] = (uint16_t)__popcll(mask);
+        }
+        __syncthreads();
+        int base0 = 0, base1 = 0;
+        cnt = 0;
+#pragma unroll
+        for (int ch = 0; ch < 2 * NKB; ++ch) {
+            const int c = s_cnt[ch];
+            if (ch < wave) base0 += c;
+            if (ch < NKB + wave) base1 += c;
+            cnt += c;
+        }
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            if (live[it]) {
+                // live keys fill the END of the nkb*32 positions; the padding sits in front
+                const int pos = (((cnt + 31) & ~31) - cnt) + (it ? base1 : base0) + before[it];
+                const int c8 = (tid & 3) * 8;
+                *reinterpret_cast<u32x4 *>(s_k + pos * kKeyPitch + c8) = kw[it];
+                uint16_t *dst = s_vt + c8 * VP + pos;
+                dst[0 * VP] = (uint16_t)(vw[it].x & 0xffffu);
+                dst[1 * VP] = (uint16_t)(vw[it].x >> 16);
+                dst[2 * VP] = (uint16_t)(vw[it].y & 0xffffu);
+                dst[3 * VP] = (uint16_t)(vw[it].y >> 16);
+                dst[4 * VP] = (uint16_t)(vw[it].z & 0xffffu);
+                dst[5 * VP] = (uint16_t)(vw[it].z >> 16);
+                dst[6 * VP] = (uint16_t)(vw[it].w & 0xffffu);
+                dst[7 * VP] = (uint16_t)(vw[it].w >> 16);
+            }
+        }
+        if (cnt != 0) break;
+        // no live key at all: every key takes part with the same weight; stage them all
+        uniform = true;
+        __syncthreads();  // s_cnt is rewritten by the second pass
     }
-
-    // ---- K operand in registers: row = key position, 8 channels per half per t ----
-    bf16x8 ka[NKB][2];
+    const int nkb = (cnt + 31) >> 5;
+    const int pad = nkb * 32 - cnt;  // positions [0, pad) of key block 0 hold no key
+    for (int idx = tid; idx < pad * 4; idx += NT) {
+        const int pos = idx >> 2;
+        const int c8 = (idx & 3) * 8;
+        *reinterpret_cast<u32x4 *>(s_k + pos * kKeyPitch + c8) = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
-    for (int kb = 0; kb < NKB; ++kb) {
-        u32x4 w0 = {0u, 0u, 0u, 0u}, w1 = {0u, 0u, 0u, 0u};
-        const int pos = kb * 32 + m;
-        if (kb < nkb && pos < cnt) {
-            const int key = s_kidx[pos];
-            const uint16_t *kp = env_base + (int64_t)key * row_stride + D + head * kDh + half * 8;
-            w0 = *reinterpret_cast<const u32x4 *>(kp);
-            w1 = *reinterpret_cast<const u32x4 *>(kp + 16);
-        }
-        ka[kb][0] = __builtin_bit_cast(bf16x8, w0);
-        ka[kb][1] = __builtin_bit_cast(bf16x8, w1);
+        for (int e = 0; e < 8; ++e) s_vt[(c8 + e) * VP + pos] = 0;
     }
-    __syncthreads();  // V^T visible
+    __syncthreads();
 
-    const int nqb = (NM + 31) >> 5;
-    for (int qb = 0; qb < nqb; ++qb) {
-        const int qrow = qb * 32 + m;
-        const int qsafe = qrow < NM ? qrow : NM - 1;
-        const uint16_t *qp = env_base + (int64_t)qsafe * row_stride + head * kDh + half * 8;
-        const bf16x8 qb0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(qp));
-        const bf16x8 qb1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(qp + 16));
+    // ---- S^T = K Q^T for this wave's 32 queries ----
+    // With no live key every score is the same constant: zero queries give exactly that.
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    const bf16x8 qb0 = __builtin_bit_cast(bf16x8, uniform ? zero4 : qw0);
+    const bf16x8 qb1 = __builtin_bit_cast(bf16x8, uniform ? zero4 : qw1);
+    // Padding is confined to key block 0, where it enters as the initial accumulator.
+    f32x16 bias0;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) bias0[v] = (8 * (v >> 2) + 4 * half + (v & 3) < pad) ? -INFINITY : 0.0f;
 
-        f32x16 acc[NKB];
-        float mx = -INFINITY;
+    // Two sweeps over the key blocks instead of keeping all NKB*16 scores per lane: the
+    // matrix cores idle most of the time, registers are what limits the work-groups in
+    // flight, and a second K Q^T costs less than the occupancy the scores would take.
+    auto scores = [&](int kb) -> f32x16 {
+        const uint16_t *kp = s_k + (kb * 32 + m) * kKeyPitch + half * 8;
+        const bf16x8 ka0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp));
+        const bf16x8 ka1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + 16));
+        f32x16 z = {0.0f};
+        if (kb == 0) z = bias0;
+        z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0, qb0, z, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka1, qb1, z, 0, 0, 0);
+    };
+
+    float mx = -INFINITY;
+    for (int kb = 0; kb < nkb; ++kb) {
+        const f32x16 z = scores(kb);
 #pragma unroll
-        for (int kb = 0; kb < NKB; ++kb) {
-            if (kb < nkb) {
-                f32x16 z = {0.0f};
-                z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kb][0], qb0, z, 0, 0, 0);
-                z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kb][1], qb1, z, 0, 0, 0);
-                if (uniform) {
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float mc = mx * scale_log2e;
+
+    // ---- P = exp2(scale (S - max)), O^T = V^T P^T ----
+    float sum = 0.0f;
+    f32x16 o = {0.0f};
+    for (int kb = 0; kb < nkb; ++kb) {
+        const f32x16 z = scores(kb);
+        float p[16];
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) z[v] = 0.0f;
-                }
-                if (kb == nkb - 1) {
-                    // positions past the live count are padding
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int pos = kb * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
-                        if (pos >= cnt) z[v] = -INFINITY;
-                    }
-                }
-#pragma unroll
-                for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
-                acc[kb] = z;
-            }
+        for (int v = 0; v < 16; ++v) {
+            p[v] = __builtin_amdgcn_exp2f(fmaf(z[v], scale_log2e, -mc));
+            sum += p[v];
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float mc = mx * scale_log2e;
-
-        float sum = 0.0f;
-        f32x16 o = {0.0f};
 #pragma unroll
-        for (int kb = 0; kb < NKB; ++kb) {
-            if (kb < nkb) {
-                float p[16];
+        for (int t = 0; t < 2; ++t) {
+            bf16x8 pb;
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    p[v] = __builtin_amdgcn_exp2f(fmaf(acc[kb][v], scale_log2e, -mc));
-                    sum += p[v];
-                }
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    bf16x8 pb;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * t + e];
-                    const uint16_t *vp = s_vt + m * VP + kb * 32 + 16 * t + 4 * half;
-                    const u32x2 lo = *reinterpret_cast<const u32x2 *>(vp);
-                    const u32x2 hi = *reinterpret_cast<const u32x2 *>(vp + 8);
-                    const u32x4 vw = {lo.x, lo.y, hi.x, hi.y};
-                    o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vw), pb, o, 0, 0, 0);
-                }
-            }
+            for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * t + e];
+            const uint16_t *vp = s_vt + m * VP + kb * 32 + 16 * t + 4 * half;
+            const u32x2 lo = *reinterpret_cast<const u32x2 *>(vp);
+            const u32x2 hi = *reinterpret_cast<const u32x2 *>(vp + 8);
+            const u32x4 vw = {lo.x, lo.y, hi.x, hi.y};
+            o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vw), pb, o, 0, 0, 0);
         }
-        sum += __shfl_xor(sum, 32);
-        const float inv = __builtin_amdgcn_rcpf(sum);
+    }
+    sum += __shfl_xor(sum, 32);
+    const float inv = __builtin_amdgcn_rcpf(sum);
 
-        if (qrow < NM) {
-            uint16_t *op = out + ((int64_t)env * NM + qrow) * D + head * kDh + 4 * half;
+    if (qrow < NM) {
+        uint16_t *op = out + ((int64_t)env * NM + qrow) * D + head * kDh + 4 * half;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const u32x2 w = {pack_bf16x2(o[4 * i + 0] * inv, o[4 * i + 1] * inv),
-                                 pack_bf16x2(o[4 * i + 2] * inv, o[4 * i + 3] * inv)};
-                *reinterpret_cast<u32x2 *>(op + 8 * i) = w;
-            }
+        for (int i = 0; i < 4; ++i) {
+            const u32x2 w = {pack_bf16x2(o[4 * i + 0] * inv, o[4 * i + 1] * inv),
+                             pack_bf16x2(o[4 * i + 2] * inv, o[4 * i + 3] * inv)};
+            *reinterpret_cast<u32x2 *>(op + 8 * i) = w;
         }
     }
 }
@@ -412,7 +441,7 @@ static int launch_mfma(const void *qkv, int64_t row_stride, const uint8_t *alive
     const int64_t blocks = (pairs + 7) / 8 * 8;
     if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
     const float scale_log2e = kLog2eA / sqrtf((float)kDh);
-    hipLaunchKernelGGL((sdpa_mfma_kernel<NKB>), dim3((unsigned)blocks), dim3(kWave), 0, stream,
+    hipLaunchKernelGGL((sdpa_mfma_kernel<NKB>), dim3((unsigned)blocks), dim3(kWave * NKB), 0, stream,
                        (const uint16_t *)qkv, row_stride, alive, (uint16_t *)out, B, NM, H, scale_log2e);
     return (int)hipGetLastError();
 }
