@@ -29,9 +29,13 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float v)
 
 __device__ __forceinline__ float round_to_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
 
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// Two fp32 -> one dword of two bf16 (lo in bits 0..15): a single v_cvt_pk_bf16_f32.
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
 {
-    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
 }
 
 // Eight consecutive channels of one row, widened to fp32.

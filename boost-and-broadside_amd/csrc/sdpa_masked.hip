@@ -221,7 +221,7 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it scalar
     const int m = lane & 31;
     const int half = lane >> 5;
 
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
     // ---- this wave's queries: issue the loads before anything else ----
     const int qrow = wave * 32 + m;
     const int qsafe = qrow < NM ? qrow : NM - 1;
-    const uint16_t *qp = env_base + (int64_t)qsafe * row_stride + head * kDh + half * 8;
+    const uint16_t *qp = env_base + (uint32_t)qsafe * (uint32_t)row_stride + (uint32_t)(head * kDh + half * 8);
     const u32x4 qw0 = *reinterpret_cast<const u32x4 *>(qp);
     const u32x4 qw1 = *reinterpret_cast<const u32x4 *>(qp + 16);
 
@@ -243,22 +243,28 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
     int cnt = 0;
     bool uniform = false;
     for (int pass = 0; pass < 2; ++pass) {
+        // Branch-free on purpose: every lane issues its alive-byte loads back to back, then
+        // its K/V loads back to back; a lane whose key is dead or out of range reads key
+        // row 0 instead (one cached row) and discards it.
         bool live[2];
         u32x4 kw[2], vw[2];
+        uint32_t ab[2] = {1u, 1u};
+        if (alive_env != nullptr && !uniform) {
+#pragma unroll
+            for (int it = 0; it < 2; ++it) {
+                const int key = (tid + it * NT) >> 2;
+                ab[it] = alive_env[key < NM ? key : NM - 1];
+            }
+        }
+        const uint32_t stride32 = (uint32_t)row_stride;
+        const uint16_t *kv_base = env_base + D + head * kDh + (tid & 3) * 8;
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
             const int key = (tid + it * NT) >> 2;
-            live[it] = key < NM;
-            if (live[it] && alive_env != nullptr && !uniform) live[it] = alive_env[key] != 0;
-        }
-#pragma unroll
-        for (int it = 0; it < 2; ++it) {
-            if (live[it]) {
-                const int idx = tid + it * NT;
-                const uint16_t *rp = env_base + (int64_t)(idx >> 2) * row_stride + head * kDh + (idx & 3) * 8;
-                kw[it] = *reinterpret_cast<const u32x4 *>(rp + D);
-                vw[it] = *reinterpret_cast<const u32x4 *>(rp + 2 * D);
-            }
+            live[it] = key < NM && ab[it] != 0;
+            const uint32_t off = (live[it] ? (uint32_t)key : 0u) * stride32;
+            kw[it] = *reinterpret_cast<const u32x4 *>(kv_base + off);
+            vw[it] = *reinterpret_cast<const u32x4 *>(kv_base + off + D);
         }
         int before[2];
 #pragma unroll
@@ -477,7 +483,8 @@ extern "C" int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride,
     if (!aligned16(qkv) || !aligned16(out) || (qkv_row_stride * esize) % 16 != 0) return BNB_ERR_MISALIGNED;
     hipStream_t s = (hipStream_t)stream;
 
-    const bool mfma_ok = dtype == BNB_BF16 && dh == kDh && NM <= 160;
+    // the matrix-core kernel addresses rows inside one environment with 32-bit offsets
+    const bool mfma_ok = dtype == BNB_BF16 && dh == kDh && NM <= 160 && (int64_t)NM * qkv_row_stride < (1LL << 30);
     if (path == BNB_SDPA_PATH_MFMA && !mfma_ok) return BNB_ERR_UNSUPPORTED;
     const bool use_mfma = path == BNB_SDPA_PATH_MFMA || (path == BNB_SDPA_PATH_AUTO && mfma_ok && NM >= 32);
     if (use_mfma) return dispatch_mfma(qkv, qkv_row_stride, alive, out, B, NM, H, s);
