@@ -1,0 +1,318 @@
+"""The drop-in trunk layers on the GPU against the CPU oracle fed the same state_dict.
+
+These mirror the reference's own layer tests (tests/models/test_encoder.py): shape and
+finiteness of the attention block incl. the all-dead mask (:106-140), the RG-LRU sequence
+against its step loop (:198-268), step == sequence across sublayer layouts and an episode
+boundary (:466-569), the field path (:1041-1203) and hidden-state handling (:272-303,
+:384-405).  Numeric bars: float32 1e-5, bf16 autocast 2e-2 (max|y-ref|/max|ref|); GEMMs,
+norms and GELUs are library calls on both sides.
+"""
+
+import pytest
+import torch
+
+from helpers import block_params, max_rel, temporal_params, trunk_params
+from oracle import torch_ref
+
+import boost_and_broadside_amd as bnb
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+F32_TOL = 1e-5
+BF16_TOL = 2e-2
+
+
+def _strip(p, prefix):
+    return {k[len(prefix):]: v for k, v in p.items() if k.startswith(prefix)}
+
+
+def _cfg(D=64, H=4, blocks=1, spatial=1, temporal=1, bullets=0):
+    return bnb.ModelConfig(d_model=D, n_heads=H, n_yemong_blocks=blocks, n_spatial_per_block=spatial,
+                           n_temporal_per_block=temporal, n_bullet_cross_per_block=bullets)
+
+
+# ------------------------------------------------------------------ TransformerBlock
+
+
+@pytest.mark.parametrize("D,H,B,N", [(64, 4, 3, 8), (128, 4, 5, 12), (128, 4, 2, 23), (32, 4, 2, 4)])
+def test_transformer_block_matches_oracle_fp32(D, H, B, N):
+    gen = torch.Generator().manual_seed(D + N)
+    p = block_params(gen, "b.", D, 1, 0)
+    layer = bnb.TransformerBlock(_cfg(D, H)).eval()
+    layer.load_state_dict(_strip(p, "b.spatial.0."))
+    layer.to(DEV)
+    x = torch.randn(B, N, D, generator=gen)
+    alive = torch.rand(B, N, generator=gen) < 0.7
+    alive[:, 0] = True
+    with torch.no_grad():
+        got = layer(x.to(DEV), alive_mask=alive.to(DEV)).cpu()
+        got_nomask = layer(x.to(DEV)).cpu()
+    assert got.shape == (B, N, D)
+    assert max_rel(got, torch_ref.spatial_sublayer(p, "b.spatial.0.", x, alive, H)) <= F32_TOL
+    assert max_rel(got_nomask, torch_ref.spatial_sublayer(p, "b.spatial.0.", x, None, H)) <= F32_TOL
+
+
+def test_transformer_block_all_dead_mask_is_finite():
+    layer = bnb.TransformerBlock(_cfg()).to(DEV).eval()
+    x = torch.randn(1, 4, 64, device=DEV)
+    with torch.no_grad():
+        out = layer(x, alive_mask=torch.zeros(1, 4, dtype=torch.bool, device=DEV))
+    assert not torch.isnan(out).any() and torch.isfinite(out).all()
+
+
+def test_transformer_block_under_bf16_autocast_feeds_bf16_to_the_kernel(monkeypatch):
+    # under autocast the qkv Linear emits bf16 while the norm keeps x fp32 (test_encoder.py:142-176):
+    # the kernel must see the bf16 projection and the residual stream must stay fp32
+    gen = torch.Generator().manual_seed(3)
+    D, H, B, N = 128, 4, 4, 12
+    p = block_params(gen, "b.", D, 1, 0)
+    layer = bnb.TransformerBlock(_cfg(D, H)).eval()
+    layer.load_state_dict(_strip(p, "b.spatial.0."))
+    layer.to(DEV)
+    seen = {}
+    real = bnb.ops.sdpa_masked
+
+    def spy(qkv, alive, n_heads, **kw):
+        seen["dtype"] = qkv.dtype
+        return real(qkv, alive, n_heads, **kw)
+
+    monkeypatch.setattr(bnb.trunk.ops, "sdpa_masked", spy)
+    x = torch.randn(B, N, D, generator=gen)
+    alive = torch.rand(B, N, generator=gen) < 0.8
+    alive[:, 1] = True
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        got = layer(x.to(DEV), alive_mask=alive.to(DEV))
+    assert seen["dtype"] == torch.bfloat16 and got.dtype == torch.float32
+    assert max_rel(got.cpu(), torch_ref.spatial_sublayer(p, "b.spatial.0.", x, alive, H)) <= BF16_TOL
+
+
+def test_layers_refuse_gradients_and_host_tensors():
+    layer = bnb.TransformerBlock(_cfg()).to(DEV)
+    with pytest.raises(RuntimeError, match="forward-only"):
+        layer(torch.randn(1, 4, 64, device=DEV))  # grad mode on, parameters require grad
+    with pytest.raises(RuntimeError, match="no host fallback"):
+        with torch.no_grad():
+            bnb.TransformerBlock(_cfg())(torch.randn(1, 4, 64))
+
+
+def test_bullet_cross_attention_matches_manual_composition():
+    # attention.py:149-166: separate softmax over bullet keys, gated off when no bullet is active
+    gen = torch.Generator().manual_seed(5)
+    D, H, B, N, NB = 64, 4, 3, 6, 10
+    layer = bnb.TransformerBlock(_cfg(D, H, spatial=1, bullets=1), reads_bullets=True).to(DEV).eval()
+    x = torch.randn(B, N, D, generator=gen).to(DEV)
+    alive = torch.ones(B, N, dtype=torch.bool, device=DEV)
+    bullets = torch.randn(B, NB, D, generator=gen).to(DEV)
+    bmask = (torch.rand(B, NB, generator=gen) < 0.5).to(DEV)
+    bmask[0] = False  # nothing in flight in env 0: contribution must vanish there
+    with torch.no_grad():
+        with_b = layer(x, alive, bullets, bmask)
+        without = layer(x, alive)
+    assert torch.allclose(with_b[0], without[0], atol=1e-6)
+    assert not torch.allclose(with_b[1], without[1], atol=1e-4)
+
+
+# ------------------------------------------------------------------ RG-LRU and temporal block
+
+
+def test_rglru_sequence_equals_step_loop_and_oracle():
+    # test_encoder.py:198-225 at D=32, T=1 and T=16
+    torch.manual_seed(0)
+    D, R = 32, 8
+    unit = bnb.RGLRU(D).to(DEV).eval()
+    p = {k: v.detach().cpu() for k, v in unit.state_dict().items()}
+    gen = torch.Generator().manual_seed(2)
+    for T in (1, 16):
+        x_seq = torch.randn(R, T, D, generator=gen)
+        h0 = torch.randn(R, D, generator=gen)
+        with torch.no_grad():
+            out, h_last = unit.forward_sequence(x_seq.to(DEV), h0.to(DEV))
+        assert out.shape == (R, T, D)
+        h = h0
+        for t in range(T):
+            h = torch_ref.rglru_step(x_seq[:, t], torch_ref.rglru_gates(p, "", x_seq[:, t]), p["log_lambda"], 8.0, h)
+            assert torch.allclose(out[:, t].cpu(), h, atol=1e-5)
+        assert torch.allclose(h_last.cpu(), h, atol=1e-5)
+
+
+def test_rglru_done_mask_cuts_the_state():
+    # test_encoder.py:227-256
+    torch.manual_seed(0)
+    D, R, T = 32, 2, 8
+    unit = bnb.RGLRU(D).to(DEV).eval()
+    gen = torch.Generator().manual_seed(4)
+    x_seq = torch.randn(R, T, D, generator=gen).to(DEV)
+    h0 = torch.randn(R, D, generator=gen).to(DEV)
+    done = torch.zeros(R, T, dtype=torch.bool, device=DEV)
+    done[0, 3] = True
+    with torch.no_grad():
+        with_done, _ = unit.forward_sequence(x_seq, h0, done)
+        no_done, _ = unit.forward_sequence(x_seq, h0)
+        fresh, _ = unit.forward_sequence(x_seq[:, 4:], torch.zeros(R, D, device=DEV))
+    assert torch.allclose(with_done[0, :4], no_done[0, :4], atol=1e-6)
+    assert not torch.allclose(with_done[0, 4:], no_done[0, 4:], atol=1e-6)
+    assert torch.allclose(with_done[1], no_done[1], atol=1e-6)
+    assert torch.allclose(with_done[0, 4:], fresh[0], atol=1e-5)
+
+
+@pytest.mark.parametrize("D,R", [(64, 10), (128, 33)])
+def test_temporal_block_step_matches_oracle(D, R):
+    gen = torch.Generator().manual_seed(D)
+    p = temporal_params(gen, "t.", D)
+    layer = bnb.GriffinTemporalBlock(D).eval()
+    layer.load_state_dict(_strip(p, "t."))
+    layer.to(DEV)
+    x = torch.randn(R, D, generator=gen)
+    h0 = 0.5 * torch.randn(R, D, generator=gen)
+    cb = torch.randn(R, 3, D, generator=gen)
+    with torch.no_grad():
+        out, h1, cb1 = layer.forward_sequence(x.unsqueeze(1).to(DEV), h0.to(DEV), cb.to(DEV))
+    ref_out, ref_h, ref_cb = torch_ref.temporal_step(p, "t.", x, h0, cb)
+    assert out.shape == (R, 1, D) and cb1.shape == (R, 3, D)
+    assert max_rel(out[:, 0].cpu(), ref_out) <= F32_TOL
+    assert max_rel(h1.cpu(), ref_h) <= F32_TOL
+    assert max_rel(cb1.cpu(), ref_cb) <= F32_TOL
+
+
+def test_temporal_block_sequence_with_done_matches_oracle_sequence():
+    D, R, T = 64, 6, 7
+    gen = torch.Generator().manual_seed(8)
+    p = temporal_params(gen, "t.", D)
+    layer = bnb.GriffinTemporalBlock(D).eval()
+    layer.load_state_dict(_strip(p, "t."))
+    layer.to(DEV)
+    x_seq = torch.randn(R, T, D, generator=gen)
+    h0 = 0.5 * torch.randn(R, D, generator=gen)
+    cb = torch.randn(R, 3, D, generator=gen)
+    done = torch.zeros(R, T, dtype=torch.bool)
+    done[:3, 2] = True
+    with torch.no_grad():
+        out, h1, cb1 = layer.forward_sequence(x_seq.to(DEV), h0.to(DEV), cb.to(DEV), done.to(DEV))
+    ref_out, ref_h, ref_cb = torch_ref.temporal_sequence(p, "t.", x_seq, h0, cb, done)
+    assert max_rel(out.cpu(), ref_out) <= 2e-5
+    assert max_rel(h1.cpu(), ref_h) <= 2e-5 and torch.allclose(cb1.cpu(), ref_cb, atol=1e-5)
+
+
+# ------------------------------------------------------------------ block and trunk
+
+
+@pytest.mark.parametrize("spatial,temporal,N,M", [(1, 1, 3, 2), (2, 1, 8, 4), (3, 2, 5, 0), (2, 0, 4, 2)])
+def test_block_step_matches_oracle(spatial, temporal, N, M):
+    D, H, B = 64, 4, 3
+    gen = torch.Generator().manual_seed(spatial * 10 + temporal)
+    p = block_params(gen, "b.", D, spatial, temporal)
+    block = bnb.YemongBlock(_cfg(D, H, 1, spatial, temporal)).eval()
+    block.load_state_dict(_strip(p, "b."))
+    block.to(DEV)
+    x = torch.randn(B, N + M, D, generator=gen)
+    alive = torch.rand(B, N + M, generator=gen) < 0.8
+    alive[:, N:] = True
+    alive[:, 0] = True
+    h = 0.5 * torch.randn(temporal, B * N, D, generator=gen)
+    cb = torch.randn(temporal, B * N, 3, D, generator=gen)
+    with torch.no_grad():
+        out, h1, cb1 = block.step(x.to(DEV), alive.to(DEV), h.to(DEV), cb.to(DEV), N)
+    ref_out, ref_h, ref_cb = torch_ref.block_step(p, "b.", spatial, temporal, H, x, alive, h, cb, N)
+    assert out.shape == x.shape and h1.shape == h.shape and cb1.shape == cb.shape
+    assert max_rel(out.cpu(), ref_out) <= 2e-5
+    if temporal:
+        assert max_rel(h1.cpu(), ref_h) <= 2e-5 and max_rel(cb1.cpu(), ref_cb) <= 2e-5
+
+
+@pytest.mark.parametrize("blocks,spatial,temporal", [(2, 1, 1), (2, 2, 1), (1, 3, 2)])
+def test_trunk_step_equals_sequence_and_oracle(blocks, spatial, temporal):
+    # the load-bearing property of the trunk (test_encoder.py:466-514): rolling out step by step
+    # and re-evaluating the stored sequence agree
+    D, H, B, N, M, T = 64, 4, 2, 3, 2, 6
+    p = trunk_params(blocks * 7 + spatial, D, blocks, spatial, temporal)
+    trunk = bnb.YemongTrunk(_cfg(D, H, blocks, spatial, temporal)).eval()
+    trunk.load_state_dict(p)
+    trunk.to(DEV)
+    gen = torch.Generator().manual_seed(7)
+    xs = torch.randn(T, B, N + M, D, generator=gen)
+    alive = torch.ones(T, B, N + M, dtype=torch.bool)
+    alive[2:, 0, 1] = False
+    hidden0 = trunk.initial_hidden(B, N, DEV)
+    assert hidden0.shape == (blocks * temporal, B * N, 4 * D)
+
+    hidden, ref_hidden, outs = hidden0, hidden0.cpu(), []
+    for t in range(T):
+        out, hidden = trunk(xs[t].to(DEV), alive[t].to(DEV), hidden)
+        ref_out, ref_hidden = torch_ref.trunk_step(p, blocks, spatial, temporal, H, xs[t], alive[t], ref_hidden)
+        assert max_rel(out.cpu(), ref_out) <= 5e-5, t
+        outs.append(out)
+    assert max_rel(hidden.cpu(), ref_hidden) <= 5e-5
+
+    # sequence path over the same inputs
+    x = xs.to(DEV)
+    h_all, cb_all = hidden0[:, :, :D], hidden0[:, :, D:].reshape(blocks * temporal, B * N, 3, D)
+    with torch.no_grad():
+        for i, block in enumerate(trunk.yemong_layers):
+            sl = slice(i * temporal, (i + 1) * temporal)
+            x, _, _ = block.sequence(x, alive.to(DEV), h_all[sl], cb_all[sl], None, N)
+    assert torch.allclose(x, torch.stack(outs), atol=1e-4)
+
+
+def test_trunk_reset_between_steps_equals_done_aware_sequence():
+    # test_encoder.py:516-569: zeroing the packed state after a done env == sequence path with done_mask
+    D, H, B, N, M, T = 64, 4, 2, 3, 2, 8
+    p = trunk_params(11, D, 2, 2, 1)
+    trunk = bnb.YemongTrunk(_cfg(D, H, 2, 2, 1)).eval()
+    trunk.load_state_dict(p)
+    trunk.to(DEV)
+    gen = torch.Generator().manual_seed(11)
+    xs = torch.randn(T, B, N + M, D, generator=gen).to(DEV)
+    alive = torch.ones(T, B, N + M, dtype=torch.bool, device=DEV)
+    done = torch.zeros(T, B, dtype=torch.bool, device=DEV)
+    done[3] = True
+    hidden0 = trunk.initial_hidden(B, N, DEV)
+    hidden, outs = hidden0, []
+    for t in range(T):
+        out, hidden = trunk(xs[t], alive[t], hidden)
+        outs.append(out)
+        hidden = trunk.reset_hidden_for_envs(hidden, done[t], N)
+    x = xs
+    h_all, cb_all = hidden0[:, :, :D], hidden0[:, :, D:].reshape(2, B * N, 3, D)
+    with torch.no_grad():
+        for i, block in enumerate(trunk.yemong_layers):
+            x, _, _ = block.sequence(x, alive, h_all[i:i + 1], cb_all[i:i + 1], done, N)
+    assert torch.allclose(x, torch.stack(outs), atol=1e-4)
+
+
+def test_state_sized_with_all_tokens_makes_fields_recurrent():
+    # policy.py:318-322: n_rec is read off the hidden tensor
+    D, H, B, N, M = 64, 4, 2, 3, 2
+    p = trunk_params(3, D, 1, 1, 1)
+    trunk = bnb.YemongTrunk(_cfg(D, H, 1, 1, 1)).eval()
+    trunk.load_state_dict(p)
+    trunk.to(DEV)
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn(B, N + M, D, generator=gen)
+    alive = torch.ones(B, N + M, dtype=torch.bool)
+    hidden = torch.randn(1, B * (N + M), 4 * D, generator=gen)
+    out, new_hidden = trunk(x.to(DEV), alive.to(DEV), hidden.to(DEV))
+    ref_out, ref_hidden = torch_ref.trunk_step(p, 1, 1, 1, H, x, alive, hidden)
+    assert new_hidden.shape == hidden.shape
+    assert max_rel(out.cpu(), ref_out) <= 2e-5 and max_rel(new_hidden.cpu(), ref_hidden) <= 2e-5
+
+
+def test_trunk_under_autocast_matches_oracle_within_bf16_bar():
+    # rollout configuration: 2 blocks x (2 spatial + 1 temporal), d_model 128, bf16 autocast
+    D, H, B, N, M = 128, 4, 16, 8, 4
+    p = trunk_params(21, D, 2, 2, 1)
+    trunk = bnb.YemongTrunk(_cfg(D, H, 2, 2, 1)).eval()
+    trunk.load_state_dict(p)
+    trunk.to(DEV)
+    gen = torch.Generator().manual_seed(21)
+    hidden, ref_hidden = trunk.initial_hidden(B, N, DEV), torch.zeros(2, B * N, 4 * D)
+    alive = torch.ones(B, N + M, dtype=torch.bool)
+    for t in range(4):
+        x = torch.randn(B, N + M, D, generator=gen)
+        alive[:, :N] &= torch.rand(B, N, generator=gen) > 0.1
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out, hidden = trunk(x.to(DEV), alive.to(DEV), hidden)
+        ref_out, ref_hidden = torch_ref.trunk_step(p, 2, 2, 1, H, x, alive, ref_hidden)
+        assert hidden.dtype == torch.float32
+        assert max_rel(out.float().cpu(), ref_out) <= BF16_TOL, t
+        assert max_rel(hidden.cpu(), ref_hidden) <= BF16_TOL, t
