@@ -6,11 +6,13 @@ namespace bnb {
 
 constexpr int kCopyThreads = 256;
 
+// One 16-byte nontemporal move per lane: the fastest plain copy measured on MI355X
+// (deeper per-lane unrolling and grid-stride loops both stream slower).
 __global__ __launch_bounds__(kCopyThreads) void copy16_kernel(const u32x4 *__restrict__ src,
                                                               u32x4 *__restrict__ dst, int64_t n16)
 {
-    const int64_t stride = (int64_t)gridDim.x * kCopyThreads;
-    for (int64_t i = (int64_t)blockIdx.x * kCopyThreads + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+    const int64_t i = (int64_t)blockIdx.x * kCopyThreads + threadIdx.x;
+    if (i < n16) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
 }  // namespace bnb
@@ -40,9 +42,7 @@ extern "C" int bnb_copy_bytes(const void *src, void *dst, int64_t bytes, void *s
     if (!src || !dst) return BNB_ERR_NULL_POINTER;
     if (!aligned16(src) || !aligned16(dst)) return BNB_ERR_MISALIGNED;
     const int64_t n16 = bytes >> 4;
-    // four 16-byte moves per lane keeps the grid a few waves deep on 256 CUs
-    int64_t blocks = (n16 + (int64_t)kCopyThreads * 4 - 1) / ((int64_t)kCopyThreads * 4);
-    if (blocks < 1) blocks = 1;
+    const int64_t blocks = (n16 + kCopyThreads - 1) / kCopyThreads;
     if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(kCopyThreads), 0, (hipStream_t)stream,
                        (const u32x4 *)src, (u32x4 *)dst, n16);

@@ -77,6 +77,42 @@ __device__ __forceinline__ void store8(uint16_t *p, const Row8 &r)
                                           pack_bf16x2(r.v[4], r.v[5]), pack_bf16x2(r.v[6], r.v[7])};
 }
 
+// Streaming variants: nontemporal accesses for data that is touched once per launch.
+__device__ __forceinline__ Row8 load8_stream(const float *p)
+{
+    const f32x4 a = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p));
+    const f32x4 b = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p + 4));
+    return Row8{{a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w}};
+}
+
+__device__ __forceinline__ Row8 load8_stream(const uint16_t *p)
+{
+    const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+    Row8 r;
+    r.v[0] = __uint_as_float(w.x << 16);
+    r.v[1] = __uint_as_float(w.x & 0xffff0000u);
+    r.v[2] = __uint_as_float(w.y << 16);
+    r.v[3] = __uint_as_float(w.y & 0xffff0000u);
+    r.v[4] = __uint_as_float(w.z << 16);
+    r.v[5] = __uint_as_float(w.z & 0xffff0000u);
+    r.v[6] = __uint_as_float(w.w << 16);
+    r.v[7] = __uint_as_float(w.w & 0xffff0000u);
+    return r;
+}
+
+__device__ __forceinline__ void store8_stream(float *p, const Row8 &r)
+{
+    __builtin_nontemporal_store(f32x4{r.v[0], r.v[1], r.v[2], r.v[3]}, reinterpret_cast<f32x4 *>(p));
+    __builtin_nontemporal_store(f32x4{r.v[4], r.v[5], r.v[6], r.v[7]}, reinterpret_cast<f32x4 *>(p + 4));
+}
+
+__device__ __forceinline__ void store8_stream(uint16_t *p, const Row8 &r)
+{
+    __builtin_nontemporal_store(u32x4{pack_bf16x2(r.v[0], r.v[1]), pack_bf16x2(r.v[2], r.v[3]),
+                                      pack_bf16x2(r.v[4], r.v[5]), pack_bf16x2(r.v[6], r.v[7])},
+                                reinterpret_cast<u32x4 *>(p));
+}
+
 __device__ __forceinline__ float load1(const float *p) { return *p; }
 __device__ __forceinline__ float load1(const uint16_t *p) { return bf16_bits_to_f32(*p); }
 __device__ __forceinline__ void store1(float *p, float v) { *p = v; }

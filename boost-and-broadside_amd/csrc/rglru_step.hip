@@ -5,16 +5,18 @@
 //   h' = a h + sqrt(max((1-a)(1+a), 1e-6)) (i x)
 // The kernel is bound by HBM traffic (x, two gate pre-activations and the old state in,
 // the new state and its optional low-precision copy out), so the design is a plain
-// streaming loop: every lane owns 8 consecutive channels of a row, moves them with
-// 16-byte accesses and keeps everything between load and store in registers.
+// streaming pass: every lane owns 8 consecutive channels of ONE row, moves them with
+// 16-byte nontemporal accesses and keeps everything between load and store in registers.
+// Measured on MI355X, one row per lane in large blocks streams faster than several rows in
+// flight per lane (more, shorter waves beat deeper per-lane unrolling on this memory system).
 
 #include "common.h"
 
 namespace bnb {
 
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr int kRglruThreads = 256;
-constexpr int kRglruRowsInFlight = 4;  // rows each lane has loads outstanding for
+constexpr int kRglruThreads = 256;     // scalar path, and the vector path on small inputs
+constexpr int kRglruBigThreads = 1024;  // vector path once the grid is large enough to fill the chip
 
 __device__ __forceinline__ float fast_sigmoid(float v)
 {
@@ -44,52 +46,34 @@ __device__ __forceinline__ float rglru_element(float x, float ga, float gx, floa
     return a * h + gate * ix;
 }
 
-template <typename XT, typename GT, typename YT, bool HAS_Y>
-__global__ __launch_bounds__(kRglruThreads) void rglru_step_vec8_kernel(
+template <int THREADS, typename XT, typename GT, typename YT, bool HAS_Y>
+__global__ __launch_bounds__(THREADS) void rglru_step_vec8_kernel(
     const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
     const float *h_in, int64_t h_in_stride, float *h_out, int64_t h_out_stride, YT *__restrict__ y,
-    int64_t R, int D, int rows_per_pass)
+    int64_t R, int D, int rows_per_block)
 {
     extern __shared__ float s_l2sig[];  // D entries
-    for (int d = threadIdx.x; d < D; d += kRglruThreads) s_l2sig[d] = log2_sigmoid(log_lambda[d]);
+    for (int d = threadIdx.x; d < D; d += THREADS) s_l2sig[d] = log2_sigmoid(log_lambda[d]);
     __syncthreads();
 
     const int vecs_per_row = D >> 3;
     const int local_row = threadIdx.x / vecs_per_row;
-    if (local_row >= rows_per_pass) return;
+    const int64_t row = (int64_t)blockIdx.x * rows_per_block + local_row;
+    if (local_row >= rows_per_block || row >= R) return;
     const int d0 = (threadIdx.x - local_row * vecs_per_row) << 3;
 
-    float l2sig[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) l2sig[e] = s_l2sig[d0 + e];
+    const Row8 xv = load8_stream(x + row * D + d0);
+    const Row8 ga = load8_stream(gates + row * 2 * D + d0);
+    const Row8 gx = load8_stream(gates + row * 2 * D + D + d0);
+    const Row8 hv = load8_stream(h_in + row * h_in_stride + d0);
 
-    const int64_t block_rows = (int64_t)rows_per_pass * kRglruRowsInFlight;
-    const int64_t row0 = (int64_t)blockIdx.x * block_rows + local_row;
-
-    Row8 xv[kRglruRowsInFlight], ga[kRglruRowsInFlight], gx[kRglruRowsInFlight], hv[kRglruRowsInFlight];
+    Row8 out;
 #pragma unroll
-    for (int k = 0; k < kRglruRowsInFlight; ++k) {
-        const int64_t row = row0 + (int64_t)k * rows_per_pass;
-        if (row < R) {
-            xv[k] = load8(x + row * D + d0);
-            ga[k] = load8(gates + row * 2 * D + d0);
-            gx[k] = load8(gates + row * 2 * D + D + d0);
-            hv[k] = load8(h_in + row * h_in_stride + d0);
-        }
-    }
-#pragma unroll
-    for (int k = 0; k < kRglruRowsInFlight; ++k) {
-        const int64_t row = row0 + (int64_t)k * rows_per_pass;
-        if (row < R) {
-            Row8 out;
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                out.v[e] = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(
-                    xv[k].v[e], ga[k].v[e], gx[k].v[e], l2sig[e], c, hv[k].v[e]);
-            store8(h_out + row * h_out_stride + d0, out);
-            if (HAS_Y) store8(y + row * D + d0, out);
-        }
-    }
+    for (int e = 0; e < 8; ++e)
+        out.v[e] = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(xv.v[e], ga.v[e], gx.v[e],
+                                                                          s_l2sig[d0 + e], c, hv.v[e]);
+    store8_stream(h_out + row * h_out_stride + d0, out);
+    if (HAS_Y) store8_stream(y + row * D + d0, out);
 }
 
 // Any D, any alignment: one lane per element.
@@ -119,14 +103,23 @@ static int launch_rglru(const void *x, const void *gates, const float *log_lambd
                      aligned16(h_in) && aligned16(h_out) && (!HAS_Y || aligned16(y)) &&
                      (h_in_stride % 4 == 0) && (h_out_stride % 4 == 0);
     if (vec) {
-        const int rows_per_pass = kRglruThreads / (D / 8);
-        const int64_t block_rows = (int64_t)rows_per_pass * kRglruRowsInFlight;
-        const int64_t blocks = (R + block_rows - 1) / block_rows;
+        const int vecs_per_row = D / 8;
+        // big blocks amortise the per-block log2 sigmoid(lambda) table; keep small inputs spread out
+        const bool big = vecs_per_row <= kRglruBigThreads && R * vecs_per_row >= (int64_t)kRglruBigThreads * 2048;
+        const int threads = big ? kRglruBigThreads : kRglruThreads;
+        const int rows_per_block = threads / vecs_per_row;
+        const int64_t blocks = (R + rows_per_block - 1) / rows_per_block;
         if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
-        hipLaunchKernelGGL((rglru_step_vec8_kernel<XT, GT, YT, HAS_Y>), dim3((unsigned)blocks),
-                           dim3(kRglruThreads), (size_t)D * sizeof(float), stream, (const XT *)x,
-                           (const GT *)gates, log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y,
-                           R, D, rows_per_pass);
+        if (big)
+            hipLaunchKernelGGL((rglru_step_vec8_kernel<kRglruBigThreads, XT, GT, YT, HAS_Y>), dim3((unsigned)blocks),
+                               dim3(threads), (size_t)D * sizeof(float), stream, (const XT *)x, (const GT *)gates,
+                               log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D,
+                               rows_per_block);
+        else
+            hipLaunchKernelGGL((rglru_step_vec8_kernel<kRglruThreads, XT, GT, YT, HAS_Y>), dim3((unsigned)blocks),
+                               dim3(threads), (size_t)D * sizeof(float), stream, (const XT *)x, (const GT *)gates,
+                               log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D,
+                               rows_per_block);
     } else {
         const int64_t blocks = (R * D + kRglruThreads - 1) / kRglruThreads;
         if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
