@@ -172,7 +172,8 @@ def load_traffic(kernel, workload):
         table = json.load(open(path))
     except (OSError, ValueError):
         return None
-    return table.get(f"{kernel}:{workload}")
+    entry = table.get(f"{kernel}:{workload}")
+    return None if entry is None else entry["total_bytes"]
 
 
 def main():
