@@ -208,6 +208,7 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
     constexpr int NT = kWave * NKB;
     __shared__ __align__(16) uint16_t s_k[KCAP * kKeyPitch];
     __shared__ __align__(16) uint16_t s_vt[kDh * VP];
+    __shared__ uint16_t s_cnt[2 * NKB];  // live keys per 16-key slice, in key order
 
     // Work-groups are dealt round-robin to the 8 XCDs; hand each XCD a contiguous run of
     // (environment, head) pairs so the 4 heads of an environment share one L2.
@@ -234,71 +235,63 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
     const u32x4 qw1 = *reinterpret_cast<const u32x4 *>(qp + 16);
 
     // ---- K rows and V^T of the live keys into LDS, compacted ----
-    // Every wave reads the whole alive row of the environment (NM <= 160 bytes: up to three
-    // byte loads per lane) and derives from wave ballots both its own keys' liveness and
-    // their positions among the live keys, so no cross-wave exchange or barrier is needed
-    // before the K/V loads can be issued.  Thread -> (key, 8 channels), two items per thread.
+    // Thread -> (key, 8 channels), two items per thread.  A thread reads its key's alive
+    // byte, starts its K/V loads at once if the key is live, and only then works out the
+    // key's position among the live keys (ballot inside the wave, per-wave counts through
+    // LDS), so the position arithmetic overlaps the loads.
     const uint8_t *alive_env = alive == nullptr ? nullptr : alive + (int64_t)env * NM;
-    constexpr int NMASK = (KCAP + 63) / 64;
-    uint32_t ab[NMASK];
-#pragma unroll
-    for (int j = 0; j < NMASK; ++j) {
-        const int key = j * 64 + lane;
-        ab[j] = 1u;
-        if (alive_env != nullptr) ab[j] = alive_env[key < NM ? key : NM - 1];
-    }
-    uint64_t mask[NMASK];
     int cnt = 0;
+    bool uniform = false;
+    for (int pass = 0; pass < 2; ++pass) {
+        // Branch-free on purpose: every lane issues its alive-byte loads back to back, then
+        // its K/V loads back to back; a lane whose key is dead or out of range reads key
+        // row 0 instead (one cached row) and discards it.
+        bool live[2];
+        u32x4 kw[2], vw[2];
+        uint32_t ab[2] = {1u, 1u};
+        if (alive_env != nullptr && !uniform) {
 #pragma unroll
-    for (int j = 0; j < NMASK; ++j) {
-        mask[j] = __ballot(j * 64 + lane < NM && ab[j] != 0);
-        cnt += __popcll(mask[j]);
-    }
-    const bool uniform = (cnt == 0);  // no live key: every key takes part with the same weight
-    if (uniform) {
-        cnt = NM;
-#pragma unroll
-        for (int j = 0; j < NMASK; ++j) {
-            const int left = NM - j * 64;
-            mask[j] = left >= 64 ? ~0ull : (left > 0 ? (1ull << left) - 1ull : 0ull);
+            for (int it = 0; it < 2; ++it) {
+                const int key = (tid + it * NT) >> 2;
+                ab[it] = alive_env[key < NM ? key : NM - 1];
+            }
         }
-    }
-    const int pad_front = (((cnt + 31) & ~31) - cnt);  // live keys fill the END of the nkb*32 positions
-    {
         const uint32_t stride32 = (uint32_t)row_stride;
         const uint16_t *kv_base = env_base + D + head * kDh + (tid & 3) * 8;
-        bool live[2];
-        int pos[2];
-        u32x4 kw[2], vw[2];
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
             const int key = (tid + it * NT) >> 2;
-            // bit `key` of the alive mask and the number of live keys before it
-            bool l = false;
-            int before = 0;
-#pragma unroll
-            for (int j = 0; j < NMASK; ++j) {
-                const int rel = key - j * 64;
-                if (rel >= 64) before += __popcll(mask[j]);
-                if (rel >= 0 && rel < 64) {
-                    l = (mask[j] >> rel) & 1ull;
-                    before += __popcll(mask[j] & ((1ull << rel) - 1ull));
-                }
-            }
-            live[it] = l;
-            pos[it] = pad_front + before;
-            // branch-free: a lane whose key is dead or out of range reads key row 0 and discards it
-            const uint32_t off = (l ? (uint32_t)key : 0u) * stride32;
+            live[it] = key < NM && ab[it] != 0;
+            const uint32_t off = (live[it] ? (uint32_t)key : 0u) * stride32;
             kw[it] = *reinterpret_cast<const u32x4 *>(kv_base + off);
             vw[it] = *reinterpret_cast<const u32x4 *>(kv_base + off + D);
+        }
+        int before[2];
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const uint64_t mask = __ballot(live[it] && (lane & 3) == 0);  // one bit per live key
+            before[it] = __popcll(mask & ((1ull << (lane & ~3)) - 1ull));
+            if (lane == 0) s_cnt[it * NKB + wave] = (uint16_t)__popcll(mask);
+        }
+        __syncthreads();
+        int base0 = 0, base1 = 0;
+        cnt = 0;
+#pragma unroll
+        for (int ch = 0; ch < 2 * NKB; ++ch) {
+            const int c = s_cnt[ch];
+            if (ch < wave) base0 += c;
+            if (ch < NKB + wave) base1 += c;
+            cnt += c;
         }
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
             if (live[it]) {
+                // live keys fill the END of the nkb*32 positions; the padding sits in front
+                const int pos = (((cnt + 31) & ~31) - cnt) + (it ? base1 : base0) + before[it];
                 const int c8 = (tid & 3) * 8;
-                *reinterpret_cast<u32x4 *>(s_k + pos[it] * kKeyPitch + c8) = kw[it];
+                *reinterpret_cast<u32x4 *>(s_k + pos * kKeyPitch + c8) = kw[it];
                 // channel d = c8 + e goes to V^T row vt_row(d) (see the output stage)
-                uint16_t *dst = s_vt + (16 * (c8 >> 4) + 4 * ((c8 >> 3) & 1)) * VP + pos[it];
+                uint16_t *dst = s_vt + (16 * (c8 >> 4) + 4 * ((c8 >> 3) & 1)) * VP + pos;
                 dst[0 * VP] = (uint16_t)(vw[it].x & 0xffffu);
                 dst[1 * VP] = (uint16_t)(vw[it].x >> 16);
                 dst[2 * VP] = (uint16_t)(vw[it].y & 0xffffu);
@@ -309,6 +302,10 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
                 dst[11 * VP] = (uint16_t)(vw[it].w >> 16);
             }
         }
+        if (cnt != 0) break;
+        // no live key at all: every key takes part with the same weight; stage them all
+        uniform = true;
+        __syncthreads();  // s_cnt is rewritten by the second pass
     }
     const int nkb = (cnt + 31) >> 5;
     const int pad = nkb * 32 - cnt;  // positions [0, pad) of key block 0 hold no key
@@ -317,7 +314,7 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
         const int c8 = (idx & 3) * 8;
         *reinterpret_cast<u32x4 *>(s_k + pos * kKeyPitch + c8) = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int e = 0; e < 8; ++e) s_vt[(c8 + e) * VP + pos] = 0;  // all 32 rows get covered, order is irrelevant
+        for (int e = 0; e < 8; ++e) s_vt[(c8 + e) * VP + pos] = 0;
     }
     __syncthreads();
 
