@@ -227,12 +227,12 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
 
     const uint16_t *env_base = qkv + (int64_t)env * NM * row_stride;
 
-    // ---- this wave's queries: issue the loads before anything else ----
+    // ---- this wave's queries (loaded together with the K/V rows, after the alive bytes: the
+    //      alive row is tiny and usually an L2 hit, and nothing else can start before it) ----
     const int qrow = wave * 32 + m;
     const int qsafe = qrow < NM ? qrow : NM - 1;
     const uint16_t *qp = env_base + (uint32_t)qsafe * (uint32_t)row_stride + (uint32_t)(head * kDh + half * 8);
-    const u32x4 qw0 = *reinterpret_cast<const u32x4 *>(qp);
-    const u32x4 qw1 = *reinterpret_cast<const u32x4 *>(qp + 16);
+    u32x4 qw0 = {0u, 0u, 0u, 0u}, qw1 = {0u, 0u, 0u, 0u};
 
     // ---- K rows and V^T of the live keys into LDS, compacted ----
     // Thread -> (key, 8 channels), two items per thread.  A thread reads its key's alive
@@ -265,6 +265,10 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
             const uint32_t off = (live[it] ? (uint32_t)key : 0u) * stride32;
             kw[it] = *reinterpret_cast<const u32x4 *>(kv_base + off);
             vw[it] = *reinterpret_cast<const u32x4 *>(kv_base + off + D);
+        }
+        if (pass == 0) {
+            qw0 = *reinterpret_cast<const u32x4 *>(qp);
+            qw1 = *reinterpret_cast<const u32x4 *>(qp + 16);
         }
         int before[2];
 #pragma unroll
