@@ -53,12 +53,13 @@ __global__ __launch_bounds__(kValuThreads) void sdpa_valu_kernel(
     const int env0 = blockIdx.x * G;
     const int h0 = blockIdx.y * nh;
     const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;  // a multiple of 64, at most kValuThreads
 
     if (tid < G) s_any[tid] = (alive == nullptr) ? 1 : 0;
     __syncthreads();
 
     // alive bytes (benign race on s_any: every writer stores 1)
-    for (int idx = tid; idx < G * NM; idx += kValuThreads) {
+    for (int idx = tid; idx < G * NM; idx += nthreads) {
         const int g = idx / NM;
         const int env = env0 + g;
         uint8_t a = 1;
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(kValuThreads) void sdpa_valu_kernel(
     // K and V tiles, 8 elements per lane per trip
     constexpr int V8 = DH / 8;
     const int per_mat = G * NM * nh * V8;
-    for (int idx = tid; idx < 2 * per_mat; idx += kValuThreads) {
+    for (int idx = tid; idx < 2 * per_mat; idx += nthreads) {
         const int mat = idx / per_mat;
         int rem = idx - mat * per_mat;
         const int c8 = rem % V8;
@@ -94,7 +95,7 @@ __global__ __launch_bounds__(kValuThreads) void sdpa_valu_kernel(
     __syncthreads();
 
     const int rows = G * nh * NM;
-    for (int row = tid; row < rows; row += kValuThreads) {
+    for (int row = tid; row < rows; row += nthreads) {
         const int g = row / (nh * NM);
         const int rem = row - g * (nh * NM);
         const int hh = rem / NM;
@@ -423,6 +424,10 @@ static int launch_valu(const void *qkv, int64_t row_stride, const uint8_t *alive
     if (G > 8) G = 8;
     while (G > 1 && valu_lds_bytes(G, NM, nh, DH) > kLdsDefault) --G;
     if (G > B) G = B;
+    // small batches: fewer environments per block so that every CU still gets several blocks
+    while (G > 1 && (int64_t)((B + G - 1) / G) * (H / nh) < 1024) --G;
+    int threads = (G * nh * NM + kWave - 1) / kWave * kWave;
+    if (threads > kValuThreads) threads = kValuThreads;
     const size_t lds = valu_lds_bytes(G, NM, nh, DH);
     if (lds > kLdsMax) return BNB_ERR_UNSUPPORTED;
     auto kernel = sdpa_valu_kernel<T, DH>;
@@ -433,7 +438,7 @@ static int launch_valu(const void *qkv, int64_t row_stride, const uint8_t *alive
     }
     const dim3 grid((unsigned)((B + G - 1) / G), (unsigned)(H / nh));
     const float scale_log2e = kLog2eA / sqrtf((float)DH);
-    hipLaunchKernelGGL(kernel, grid, dim3(kValuThreads), lds, stream, (const T *)qkv, row_stride, alive,
+    hipLaunchKernelGGL(kernel, grid, dim3(threads), lds, stream, (const T *)qkv, row_stride, alive,
                        (T *)out, B, NM, H, G, nh, scale_log2e);
     return (int)hipGetLastError();
 }

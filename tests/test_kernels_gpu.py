@@ -192,6 +192,45 @@ def test_sdpa_mfma_live_counts_across_block_edges():
         assert max_rel(got[b], truth[b]) <= BF16_TOL, counts[b]
 
 
+@pytest.mark.parametrize("NM,path", [(161, "auto"), (200, "auto"), (320, "auto")])
+def test_sdpa_bf16_beyond_matrix_core_range_uses_the_vector_kernel(NM, path):
+    # crossover evaluation reaches 320 ships (modes/crossover.py:92); more than 160 tokens in bf16
+    # falls back to the vector-ALU kernel
+    B, H, D = 2, 4, 128
+    qkv = _qkv(NM, B, NM, D, torch.bfloat16)
+    alive = _alive(NM, B, NM, 0.6)
+    alive[:, 5] = True
+    got = _run_sdpa(qkv, alive, H, path).float()
+    assert max_rel(got, torch_ref.sdpa_masked(qkv.float(), alive, H)) <= BF16_TOL
+    with pytest.raises(RuntimeError, match="outside what the kernels cover"):
+        _run_sdpa(qkv, alive, H, "mfma")
+
+
+@pytest.mark.parametrize("NM", [12, 84])
+def test_sdpa_mfma_padded_rows_no_mask_and_uint8_mask(NM):
+    B, H, D = 5, 4, 128
+    qkv = _qkv(31 + NM, B, NM, D, torch.bfloat16)
+    wide = torch.zeros(B, NM, 3 * D + 64, dtype=torch.bfloat16)
+    wide[..., : 3 * D] = qkv
+    view = wide.to(DEV)[..., : 3 * D]  # row stride 448 elements
+    truth = torch_ref.sdpa_masked(qkv.float(), None, H)
+    assert max_rel(ops.sdpa_masked(view, None, H, path="mfma").float().cpu(), truth) <= BF16_TOL
+    alive = _alive(NM, B, NM, 0.5)
+    alive[:, 0] = True
+    a = ops.sdpa_masked(view, alive.to(DEV).to(torch.uint8), H, path="mfma")
+    b = ops.sdpa_masked(qkv.to(DEV), alive.to(DEV), H, path="mfma")
+    assert torch.equal(a, b)
+
+
+def test_sdpa_small_batches_fp32():
+    # one and a handful of environments (crossover runs 48..256, modes/crossover.py:37-47)
+    for B in (1, 2, 48):
+        qkv = _qkv(B, B, 12, 128, torch.float32)
+        alive = _alive(B, B, 12, 0.8)
+        alive[:, 0] = True
+        assert max_rel(_run_sdpa(qkv, alive, 4), torch_ref.sdpa_masked(qkv, alive, 4)) <= F32_TOL
+
+
 def test_sdpa_environment_permutation_is_bitwise_equivariant_at_full_size():
     # full 64v88 batch: shuffling environments must shuffle outputs bit for bit
     w = harness.WORKLOADS["c4_64v88_bf16"]
