@@ -1,0 +1,150 @@
+// Causal depthwise conv tap sum + conv-buffer shift for one timestep, for gfx950.
+//
+// Per row (reference: models/yemong/griffin.py:275-277 with the tap loop of :127-139 at T = 1):
+//   padded = [p0, p1, p2, b1]            p* = the three previous linear1 outputs, oldest first
+//   v      = sum_k padded[k] * w[:, k] + bias
+//   new buffer = [p1, p2, b1]
+// The previous buffer is read from, and the new one written into, the conv columns of a
+// packed (.., 4D) state row (models/yemong/policy.py:323-324, :346-354), so neither the
+// `cat` that builds `padded`, the eight element-wise tap kernels, nor the `cat` that repacks
+// the state exist any more.  Pure HBM streaming: 8 channels of one row per lane, 16-byte
+// nontemporal accesses, fp32 arithmetic in the reference's order (taps 0..3, then the bias).
+
+#include "common.h"
+
+namespace bnb {
+
+constexpr int kConvThreads = 256;
+constexpr int kConvBigThreads = 1024;
+constexpr int kTaps = 4;
+
+template <int THREADS, typename BT>
+__global__ __launch_bounds__(THREADS) void conv_step_vec8_kernel(
+    const BT *__restrict__ b1, const float *conv_in, int64_t conv_in_stride, const float *__restrict__ weight,
+    const float *__restrict__ bias, const uint8_t *__restrict__ reset, int rows_per_env, float *__restrict__ v_out,
+    float *conv_out, int64_t conv_out_stride, int64_t R, int D, int rows_per_block)
+{
+    extern __shared__ float s_wb[];  // D*4 tap weights (as stored: [d][k]) then D biases
+    for (int i = threadIdx.x; i < D * kTaps; i += THREADS) s_wb[i] = weight[i];
+    for (int i = threadIdx.x; i < D; i += THREADS) s_wb[D * kTaps + i] = bias != nullptr ? bias[i] : 0.0f;
+    __syncthreads();
+
+    const int vecs_per_row = D >> 3;
+    const int local_row = threadIdx.x / vecs_per_row;
+    const int64_t row = (int64_t)blockIdx.x * rows_per_block + local_row;
+    if (local_row >= rows_per_block || row >= R) return;
+    const int d0 = (threadIdx.x - local_row * vecs_per_row) << 3;
+
+    const Row8 cur = load8_stream(b1 + row * D + d0);
+    const float *pin = conv_in + row * conv_in_stride + d0;
+    Row8 p0 = load8_stream(pin), p1 = load8_stream(pin + D), p2 = load8_stream(pin + 2 * D);
+    if (reset != nullptr && reset[row / rows_per_env]) {
+        // the environment was reset before this step: its stored inputs read as zero
+#pragma unroll
+        for (int e = 0; e < 8; ++e) p0.v[e] = p1.v[e] = p2.v[e] = 0.0f;
+    }
+
+    Row8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float *w = s_wb + (d0 + e) * kTaps;
+        float acc = p0.v[e] * w[0];
+        acc += p1.v[e] * w[1];
+        acc += p2.v[e] * w[2];
+        acc += cur.v[e] * w[3];
+        v.v[e] = acc + s_wb[D * kTaps + d0 + e];
+    }
+    store8_stream(v_out + row * D + d0, v);
+    float *pout = conv_out + row * conv_out_stride + d0;
+    store8_stream(pout, p1);
+    store8_stream(pout + D, p2);
+    store8_stream(pout + 2 * D, cur);
+}
+
+// Any D, any alignment: one lane per element.
+template <typename BT>
+__global__ __launch_bounds__(kConvThreads) void conv_step_scalar_kernel(
+    const BT *__restrict__ b1, const float *conv_in, int64_t conv_in_stride, const float *__restrict__ weight,
+    const float *__restrict__ bias, const uint8_t *__restrict__ reset, int rows_per_env, float *__restrict__ v_out,
+    float *conv_out, int64_t conv_out_stride, int64_t R, int D)
+{
+    const int64_t idx = (int64_t)blockIdx.x * kConvThreads + threadIdx.x;
+    if (idx >= R * D) return;
+    const int64_t row = idx / D;
+    const int d = (int)(idx - row * D);
+    const bool zero = reset != nullptr && reset[row / rows_per_env];
+    const float *pin = conv_in + row * conv_in_stride + d;
+    const float p0 = zero ? 0.0f : pin[0], p1 = zero ? 0.0f : pin[D], p2 = zero ? 0.0f : pin[2 * D];
+    const float cur = load1(b1 + idx);
+    const float *w = weight + (int64_t)d * kTaps;
+    float acc = p0 * w[0];
+    acc += p1 * w[1];
+    acc += p2 * w[2];
+    acc += cur * w[3];
+    v_out[idx] = acc + (bias != nullptr ? bias[d] : 0.0f);
+    float *pout = conv_out + row * conv_out_stride + d;
+    pout[0] = p1;
+    pout[D] = p2;
+    pout[2 * D] = cur;
+}
+
+template <typename BT>
+static int launch_conv(const void *b1, const float *conv_in, int64_t conv_in_stride, const float *weight,
+                       const float *bias, const uint8_t *reset, int rows_per_env, float *v_out, float *conv_out,
+                       int64_t conv_out_stride, int64_t R, int D, hipStream_t stream)
+{
+    const bool vec = (D % 8 == 0) && (D / 8 <= kConvThreads) && aligned16(b1) && aligned16(conv_in) &&
+                     aligned16(conv_out) && aligned16(v_out) && (conv_in_stride % 4 == 0) &&
+                     (conv_out_stride % 4 == 0) && (size_t)D * (kTaps + 1) * sizeof(float) <= 48 * 1024;
+    if (vec) {
+        const int vecs_per_row = D / 8;
+        const bool big = R * vecs_per_row >= (int64_t)kConvBigThreads * 2048;
+        const int threads = big ? kConvBigThreads : kConvThreads;
+        const int rows_per_block = threads / vecs_per_row;
+        const int64_t blocks = (R + rows_per_block - 1) / rows_per_block;
+        if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+        const size_t lds = (size_t)D * (kTaps + 1) * sizeof(float);
+        if (big)
+            hipLaunchKernelGGL((conv_step_vec8_kernel<kConvBigThreads, BT>), dim3((unsigned)blocks), dim3(threads), lds,
+                               stream, (const BT *)b1, conv_in, conv_in_stride, weight, bias, reset, rows_per_env,
+                               v_out, conv_out, conv_out_stride, R, D, rows_per_block);
+        else
+            hipLaunchKernelGGL((conv_step_vec8_kernel<kConvThreads, BT>), dim3((unsigned)blocks), dim3(threads), lds,
+                               stream, (const BT *)b1, conv_in, conv_in_stride, weight, bias, reset, rows_per_env,
+                               v_out, conv_out, conv_out_stride, R, D, rows_per_block);
+    } else {
+        const int64_t blocks = (R * D + kConvThreads - 1) / kConvThreads;
+        if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL((conv_step_scalar_kernel<BT>), dim3((unsigned)blocks), dim3(kConvThreads), 0, stream,
+                           (const BT *)b1, conv_in, conv_in_stride, weight, bias, reset, rows_per_env, v_out,
+                           conv_out, conv_out_stride, R, D);
+    }
+    return (int)hipGetLastError();
+}
+
+}  // namespace bnb
+
+extern "C" int bnb_conv_step_fwd(const void *b1, int b1_dtype, const float *conv_in, int64_t conv_in_row_stride,
+                                 const float *weight, const float *bias, const uint8_t *reset, int rows_per_env,
+                                 float *v_out, float *conv_out, int64_t conv_out_row_stride, int64_t R, int D,
+                                 void *stream)
+{
+    using namespace bnb;
+    if (R < 0 || D < 1) return BNB_ERR_BAD_SHAPE;
+    if (R == 0) return 0;
+    if (!b1 || !conv_in || !weight || !v_out || !conv_out) return BNB_ERR_NULL_POINTER;
+    if (b1_dtype != BNB_F32 && b1_dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
+    if (conv_in_row_stride < 3 * (int64_t)D || conv_out_row_stride < 3 * (int64_t)D) return BNB_ERR_BAD_SHAPE;
+    if (reset != nullptr && rows_per_env < 1) return BNB_ERR_BAD_SHAPE;
+    if ((reinterpret_cast<uintptr_t>(conv_in) | reinterpret_cast<uintptr_t>(conv_out) |
+         reinterpret_cast<uintptr_t>(v_out) | reinterpret_cast<uintptr_t>(weight) |
+         reinterpret_cast<uintptr_t>(bias)) & 3u)
+        return BNB_ERR_MISALIGNED;
+    if (reset == nullptr) rows_per_env = 1;
+    hipStream_t s = (hipStream_t)stream;
+    if (b1_dtype == BNB_BF16)
+        return launch_conv<uint16_t>(b1, conv_in, conv_in_row_stride, weight, bias, reset, rows_per_env, v_out,
+                                     conv_out, conv_out_row_stride, R, D, s);
+    return launch_conv<float>(b1, conv_in, conv_in_row_stride, weight, bias, reset, rows_per_env, v_out, conv_out,
+                              conv_out_row_stride, R, D, s);
+}

@@ -50,7 +50,7 @@ template <int THREADS, typename XT, typename GT, typename YT, bool HAS_Y>
 __global__ __launch_bounds__(THREADS) void rglru_step_vec8_kernel(
     const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
     const float *h_in, int64_t h_in_stride, float *h_out, int64_t h_out_stride, YT *__restrict__ y,
-    int64_t R, int D, int rows_per_block)
+    int64_t R, int D, int rows_per_block, const uint8_t *__restrict__ reset, int rows_per_env)
 {
     extern __shared__ float s_l2sig[];  // D entries
     for (int d = threadIdx.x; d < D; d += THREADS) s_l2sig[d] = log2_sigmoid(log_lambda[d]);
@@ -65,7 +65,12 @@ __global__ __launch_bounds__(THREADS) void rglru_step_vec8_kernel(
     const Row8 xv = load8_stream(x + row * D + d0);
     const Row8 ga = load8_stream(gates + row * 2 * D + d0);
     const Row8 gx = load8_stream(gates + row * 2 * D + D + d0);
-    const Row8 hv = load8_stream(h_in + row * h_in_stride + d0);
+    Row8 hv = load8_stream(h_in + row * h_in_stride + d0);
+    if (reset != nullptr && reset[row / rows_per_env]) {
+        // the environment was reset before this step: its previous state reads as zero
+#pragma unroll
+        for (int e = 0; e < 8; ++e) hv.v[e] = 0.0f;
+    }
 
     Row8 out;
 #pragma unroll
@@ -81,15 +86,16 @@ template <typename XT, typename GT, typename YT, bool HAS_Y>
 __global__ __launch_bounds__(kRglruThreads) void rglru_step_scalar_kernel(
     const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
     const float *h_in, int64_t h_in_stride, float *h_out, int64_t h_out_stride, YT *__restrict__ y,
-    int64_t R, int D)
+    int64_t R, int D, const uint8_t *__restrict__ reset, int rows_per_env)
 {
     const int64_t idx = (int64_t)blockIdx.x * kRglruThreads + threadIdx.x;
     if (idx >= R * D) return;
     const int64_t row = idx / D;
     const int d = (int)(idx - row * D);
+    const float h_prev = (reset != nullptr && reset[row / rows_per_env]) ? 0.0f : h_in[row * h_in_stride + d];
     const float out = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(
         load1(x + idx), load1(gates + row * 2 * D + d), load1(gates + row * 2 * D + D + d),
-        log2_sigmoid(log_lambda[d]), c, h_in[row * h_in_stride + d]);
+        log2_sigmoid(log_lambda[d]), c, h_prev);
     h_out[row * h_out_stride + d] = out;
     if (HAS_Y) store1(y + idx, out);
 }
@@ -97,7 +103,7 @@ __global__ __launch_bounds__(kRglruThreads) void rglru_step_scalar_kernel(
 template <typename XT, typename GT, typename YT, bool HAS_Y>
 static int launch_rglru(const void *x, const void *gates, const float *log_lambda, float c, const float *h_in,
                         int64_t h_in_stride, float *h_out, int64_t h_out_stride, void *y, int64_t R, int D,
-                        hipStream_t stream)
+                        const uint8_t *reset, int rows_per_env, hipStream_t stream)
 {
     const bool vec = (D % 8 == 0) && (D / 8 <= kRglruThreads) && aligned16(x) && aligned16(gates) &&
                      aligned16(h_in) && aligned16(h_out) && (!HAS_Y || aligned16(y)) &&
@@ -114,18 +120,18 @@ static int launch_rglru(const void *x, const void *gates, const float *log_lambd
             hipLaunchKernelGGL((rglru_step_vec8_kernel<kRglruBigThreads, XT, GT, YT, HAS_Y>), dim3((unsigned)blocks),
                                dim3(threads), (size_t)D * sizeof(float), stream, (const XT *)x, (const GT *)gates,
                                log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D,
-                               rows_per_block);
+                               rows_per_block, reset, rows_per_env);
         else
             hipLaunchKernelGGL((rglru_step_vec8_kernel<kRglruThreads, XT, GT, YT, HAS_Y>), dim3((unsigned)blocks),
                                dim3(threads), (size_t)D * sizeof(float), stream, (const XT *)x, (const GT *)gates,
                                log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D,
-                               rows_per_block);
+                               rows_per_block, reset, rows_per_env);
     } else {
         const int64_t blocks = (R * D + kRglruThreads - 1) / kRglruThreads;
         if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
         hipLaunchKernelGGL((rglru_step_scalar_kernel<XT, GT, YT, HAS_Y>), dim3((unsigned)blocks),
                            dim3(kRglruThreads), 0, stream, (const XT *)x, (const GT *)gates, log_lambda, c,
-                           h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D);
+                           h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D, reset, rows_per_env);
     }
     return (int)hipGetLastError();
 }
@@ -133,24 +139,25 @@ static int launch_rglru(const void *x, const void *gates, const float *log_lambd
 template <typename XT, typename GT>
 static int dispatch_y(const void *x, const void *gates, const float *log_lambda, float c, const float *h_in,
                       int64_t h_in_stride, float *h_out, int64_t h_out_stride, void *y, int y_dtype, int64_t R,
-                      int D, hipStream_t stream)
+                      int D, const uint8_t *reset, int rows_per_env, hipStream_t stream)
 {
     if (y == nullptr)
         return launch_rglru<XT, GT, float, false>(x, gates, log_lambda, c, h_in, h_in_stride, h_out,
-                                                  h_out_stride, nullptr, R, D, stream);
+                                                  h_out_stride, nullptr, R, D, reset, rows_per_env, stream);
     if (y_dtype == BNB_F32)
         return launch_rglru<XT, GT, float, true>(x, gates, log_lambda, c, h_in, h_in_stride, h_out,
-                                                 h_out_stride, y, R, D, stream);
+                                                 h_out_stride, y, R, D, reset, rows_per_env, stream);
     return launch_rglru<XT, GT, uint16_t, true>(x, gates, log_lambda, c, h_in, h_in_stride, h_out,
-                                                h_out_stride, y, R, D, stream);
+                                                h_out_stride, y, R, D, reset, rows_per_env, stream);
 }
 
 }  // namespace bnb
 
-extern "C" int bnb_rglru_step_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
-                                  const float *log_lambda, float c, const float *h_in,
-                                  int64_t h_in_row_stride, float *h_out, int64_t h_out_row_stride, void *y,
-                                  int y_dtype, int64_t R, int D, void *stream)
+extern "C" int bnb_rglru_step_reset_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
+                                        const float *log_lambda, float c, const float *h_in,
+                                        int64_t h_in_row_stride, float *h_out, int64_t h_out_row_stride,
+                                        void *y, int y_dtype, const uint8_t *reset, int rows_per_env, int64_t R,
+                                        int D, void *stream)
 {
     using namespace bnb;
     if (R < 0 || D < 1) return BNB_ERR_BAD_SHAPE;
@@ -160,20 +167,31 @@ extern "C" int bnb_rglru_step_fwd(const void *x, int x_dtype, const void *gates_
         (y && y_dtype != BNB_F32 && y_dtype != BNB_BF16))
         return BNB_ERR_BAD_DTYPE;
     if (h_in_row_stride < D || h_out_row_stride < D) return BNB_ERR_BAD_SHAPE;
+    if (reset != nullptr && rows_per_env < 1) return BNB_ERR_BAD_SHAPE;
     if ((reinterpret_cast<uintptr_t>(h_in) | reinterpret_cast<uintptr_t>(h_out) |
          reinterpret_cast<uintptr_t>(log_lambda)) & 3u)
         return BNB_ERR_MISALIGNED;
+    if (reset == nullptr) rows_per_env = 1;
     hipStream_t s = (hipStream_t)stream;
     const bool xb = x_dtype == BNB_BF16, gb = g_dtype == BNB_BF16;
     if (!xb && !gb)
         return dispatch_y<float, float>(x, gates_pre, log_lambda, c, h_in, h_in_row_stride, h_out,
-                                        h_out_row_stride, y, y_dtype, R, D, s);
+                                        h_out_row_stride, y, y_dtype, R, D, reset, rows_per_env, s);
     if (xb && gb)
         return dispatch_y<uint16_t, uint16_t>(x, gates_pre, log_lambda, c, h_in, h_in_row_stride, h_out,
-                                              h_out_row_stride, y, y_dtype, R, D, s);
+                                              h_out_row_stride, y, y_dtype, R, D, reset, rows_per_env, s);
     if (!xb && gb)
         return dispatch_y<float, uint16_t>(x, gates_pre, log_lambda, c, h_in, h_in_row_stride, h_out,
-                                           h_out_row_stride, y, y_dtype, R, D, s);
+                                           h_out_row_stride, y, y_dtype, R, D, reset, rows_per_env, s);
     return dispatch_y<uint16_t, float>(x, gates_pre, log_lambda, c, h_in, h_in_row_stride, h_out,
-                                       h_out_row_stride, y, y_dtype, R, D, s);
+                                       h_out_row_stride, y, y_dtype, R, D, reset, rows_per_env, s);
+}
+
+extern "C" int bnb_rglru_step_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
+                                  const float *log_lambda, float c, const float *h_in,
+                                  int64_t h_in_row_stride, float *h_out, int64_t h_out_row_stride, void *y,
+                                  int y_dtype, int64_t R, int D, void *stream)
+{
+    return bnb_rglru_step_reset_fwd(x, x_dtype, gates_pre, g_dtype, log_lambda, c, h_in, h_in_row_stride, h_out,
+                                    h_out_row_stride, y, y_dtype, nullptr, 1, R, D, stream);
 }

@@ -3,9 +3,10 @@
 ``sdpa_masked`` stands in for the key-bias + ``F.scaled_dot_product_attention`` +
 head-merge copy of the reference (models/yemong/attention.py:136-147,168);
 ``rglru_step`` stands in for the element-wise chain of ``RGLRU._step``
-(models/yemong/griffin.py:179-185).  Both launch on torch's current stream, allocate
-their outputs with torch and never synchronise.  They are forward-only and run on a
-ROCm device only: anything else raises.
+(models/yemong/griffin.py:179-185); ``conv_step`` for the padded ``cat``, the depthwise tap
+loop and the buffer shift of the temporal block at T = 1 (griffin.py:127-139, 275-277).
+All launch on torch's current stream, allocate their outputs with torch and never
+synchronise.  They are forward-only and run on a ROCm device only: anything else raises.
 """
 
 from __future__ import annotations
@@ -110,6 +111,8 @@ def rglru_step(
     h_out: torch.Tensor | None = None,
     y_dtype: torch.dtype | None = None,
     y_out: torch.Tensor | None = None,
+    reset: torch.Tensor | None = None,
+    rows_per_env: int = 1,
 ) -> tuple[torch.Tensor, torch.Tensor]:
     """One RG-LRU step given the two gate pre-activations.
 
@@ -125,6 +128,9 @@ def rglru_step(
         y_dtype:    dtype of the returned layer output.  None or float32 returns the new
                     state itself; bfloat16 makes the kernel write a rounded copy as well.
         y_out:      optional preallocated contiguous bfloat16 (R, D) destination for that copy.
+        reset:      optional (R / rows_per_env,) bool: environments whose previous state must
+                    read as zero (``reset_hidden_for_envs`` folded into this step).
+        rows_per_env: consecutive rows that belong to one environment (rows are env-major).
 
     Returns:
         (y, h_new): layer output and new state (the same tensor unless y_dtype is bfloat16).
@@ -166,16 +172,96 @@ def rglru_step(
             raise ValueError("y_out must be a contiguous bfloat16 (R, D) tensor on x's device")
         else:
             y = y_out
+    reset_ptr = _reset_pointer(reset, R, rows_per_env, x.device)
     if R == 0:
         return (h_out if y is None else y), h_out
     with torch.cuda.device(x.device):
-        rc = _native.load().bnb_rglru_step_fwd(
+        rc = _native.load().bnb_rglru_step_reset_fwd(
             x.data_ptr(), x_code, gates_pre.data_ptr(), g_code, log_lambda.data_ptr(), float(c),
             h.data_ptr(), h.stride(0), h_out.data_ptr(), h_out.stride(0),
-            None if y is None else y.data_ptr(), _native.BF16, R, D, _stream(),
+            None if y is None else y.data_ptr(), _native.BF16, reset_ptr, int(rows_per_env), R, D, _stream(),
         )
     _native.check(rc, "bnb_rglru_step_fwd")
     return (h_out if y is None else y), h_out
+
+
+def _reset_pointer(reset, R: int, rows_per_env: int, device) -> int | None:
+    """Validate an optional per-environment reset mask and return its device address."""
+    if reset is None:
+        return None
+    if rows_per_env < 1 or R % rows_per_env:
+        raise ValueError(f"rows_per_env={rows_per_env} does not divide the {R} rows")
+    if reset.shape != (R // rows_per_env,) or reset.dtype not in (torch.bool, torch.uint8):
+        raise ValueError(f"reset must be a bool ({R // rows_per_env},) tensor, got {tuple(reset.shape)} {reset.dtype}")
+    if reset.device != device or not reset.is_contiguous():
+        raise ValueError("reset must be contiguous and on the same device as the rows")
+    return reset.data_ptr()
+
+
+def conv_step(
+    b1: torch.Tensor,
+    conv_buf: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None,
+    *,
+    conv_out: torch.Tensor | None = None,
+    reset: torch.Tensor | None = None,
+    rows_per_env: int = 1,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """Causal depthwise conv of one timestep and the shift of the stored inputs.
+
+    Args:
+        b1:       (R, D) this step's ``linear1`` output, float32 or bfloat16.
+        conv_buf: (R, 3, D) float32 previous inputs, oldest first; each row's 3*D values must
+                  be contiguous, rows may be strided (a view of the packed hidden works).
+        weight:   (D, 4) or (D, 1, 4) float32 depthwise taps (``conv.weight``).
+        bias:     (D,) float32 or None.
+        conv_out: optional (R, 3, D) float32 destination with the same layout rules (may be
+                  ``conv_buf`` itself).  Default: a new contiguous tensor.
+        reset, rows_per_env: as in ``rglru_step``: environments whose stored inputs read as zero.
+
+    Returns:
+        (v, new_conv_buf): conv output (R, D) float32 and the shifted buffer ``[p1, p2, b1]``.
+    """
+    if b1.dim() != 2 or conv_buf.dim() != 3:
+        raise ValueError("b1 must be (R, D) and conv_buf (R, 3, D)")
+    R, D = b1.shape
+    if conv_buf.shape != (R, 3, D):
+        raise ValueError(f"conv_buf must be {(R, 3, D)}, got {tuple(conv_buf.shape)}")
+    for name, t in (("b1", b1), ("conv_buf", conv_buf), ("weight", weight)):
+        _need_device(t, name)
+    if conv_buf.dtype != torch.float32 or weight.dtype != torch.float32 or (bias is not None and bias.dtype != torch.float32):
+        raise TypeError("conv_buf, weight and bias must be float32")
+    if torch.is_grad_enabled() and (b1.requires_grad or conv_buf.requires_grad):
+        raise RuntimeError("conv_step is forward-only; call it under torch.no_grad()")
+    b_code = _code(b1, "b1")
+    weight = weight.detach().reshape(D, 4).contiguous()
+    bias_ptr = None
+    if bias is not None:
+        bias = bias.detach().contiguous()
+        bias_ptr = bias.data_ptr()
+    b1 = b1.contiguous()
+
+    def rows_ok(t):
+        return R == 0 or (t.stride(2) == 1 and t.stride(1) == D)
+
+    if not rows_ok(conv_buf):
+        conv_buf = conv_buf.contiguous()
+    if conv_out is None:
+        conv_out = torch.empty((R, 3, D), dtype=torch.float32, device=b1.device)
+    elif conv_out.shape != (R, 3, D) or conv_out.dtype != torch.float32 or conv_out.device != b1.device or not rows_ok(conv_out):
+        raise ValueError("conv_out must be a float32 (R, 3, D) tensor on b1's device with contiguous rows")
+    v = torch.empty((R, D), dtype=torch.float32, device=b1.device)
+    reset_ptr = _reset_pointer(reset, R, rows_per_env, b1.device)
+    if R == 0:
+        return v, conv_out
+    with torch.cuda.device(b1.device):
+        rc = _native.load().bnb_conv_step_fwd(
+            b1.data_ptr(), b_code, conv_buf.data_ptr(), conv_buf.stride(0), weight.data_ptr(), bias_ptr,
+            reset_ptr, int(rows_per_env), v.data_ptr(), conv_out.data_ptr(), conv_out.stride(0), R, D, _stream(),
+        )
+    _native.check(rc, "bnb_conv_step_fwd")
+    return v, conv_out
 
 
 def copy_bytes(src: torch.Tensor, dst: torch.Tensor) -> None:

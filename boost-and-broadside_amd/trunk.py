@@ -13,11 +13,13 @@ Every class keeps the constructor arguments, method signatures, tensor layouts a
     YemongTrunk             the block loop and hidden-state handling of
                             models/yemong/policy.py:234-254, 268-285, 311-354
 
-What runs where: the attention core (key masking, softmax, head merge) and the RG-LRU
-element-wise recurrence are the HIP kernels in ``ops``; projections, norms, GELUs and the
-depthwise conv taps are torch library calls on the same stream.  The layers are
-forward-only (rollout / evaluation); they refuse tensors that need gradients and they
-refuse to run off-GPU.
+What runs where: the attention core (key masking, softmax, head merge), the RG-LRU
+element-wise recurrence and the one-step causal conv with its buffer shift are the HIP
+kernels in ``ops``; projections, norms and GELUs are torch library calls on the same stream
+(so is the conv over longer sequences).  ``YemongTrunk.forward`` steps the packed hidden
+tensor in place of the reference's unpack / ``cat`` / re-pack and can fold the done-environment
+reset into the same kernels.  The layers are forward-only (rollout / evaluation); they refuse
+tensors that need gradients and they refuse to run off-GPU.
 """
 
 from __future__ import annotations
@@ -161,9 +163,17 @@ class RGLRU(nn.Module):
         """(R,D), (R,D) -> new state (R,D) float32 (also the layer output)."""
         return self.step(x, h)[1]
 
-    def step(self, x: torch.Tensor, h: torch.Tensor, y_dtype: torch.dtype | None = None):
-        """One kernel launch: returns (output in ``y_dtype`` or the state itself, new state)."""
-        return ops.rglru_step(x, self._gate_preactivations(x), self.log_lambda, self.c, h, y_dtype=y_dtype)
+    def step(self, x, h, y_dtype=None, *, h_out=None, reset=None, rows_per_env=1):
+        """One kernel launch: returns (output in ``y_dtype`` or the state itself, new state).
+
+        ``h_out`` lets the new state land in place (e.g. in the RG-LRU columns of a packed
+        hidden tensor); ``reset`` (one bool per environment of ``rows_per_env`` rows) makes the
+        previous state of those environments read as zero.
+        """
+        return ops.rglru_step(
+            x, self._gate_preactivations(x), self.log_lambda, self.c, h, y_dtype=y_dtype, h_out=h_out,
+            reset=reset, rows_per_env=rows_per_env,
+        )
 
     def forward_sequence(self, x_seq, h0, done_mask=None):
         """(R,T,D), (R,D) -> ((R,T,D) states, (R,D) last state).
@@ -201,6 +211,13 @@ class GriffinTemporalBlock(nn.Module):
     def forward_sequence(self, x_seq, h0, conv_buf, done_mask=None):
         """(R,T,D), (R,D), (R,3,D) [, (R,T) bool] -> (out (R,T,D), new_h (R,D), new_conv_buf (R,3,D))."""
         T = x_seq.shape[1]
+        if T == 1 and done_mask is None:
+            # rollout: the conv taps and the buffer shift are one kernel, the recurrence another
+            x = x_seq[:, 0]
+            normed = self.norm1(x)
+            v, new_conv_buf = ops.conv_step(self.linear1(normed), conv_buf, self.conv.weight, self.conv.bias)
+            y, new_h = self.rg_lru.step(v, h0)
+            return self._finish(x, normed, y).unsqueeze(1), new_h, new_conv_buf
         normed = self.norm1(x_seq)
         b1 = self.linear1(normed)
         padded = torch.cat([conv_buf, b1], dim=1)  # (R, T+3, D); fp32 buffer promotes a bf16 b1
@@ -210,10 +227,31 @@ class GriffinTemporalBlock(nn.Module):
         else:
             conv_out = _conv_within_episodes(padded, w, self.conv.bias, done_mask)
         y, new_h = self.rg_lru.forward_sequence(conv_out, h0, done_mask)
-        b2 = F.gelu(self.linear2(normed))
-        x1 = x_seq + self.linear_out(y * b2)
-        x2 = x1 + self.gated_mlp(self.norm2(x1))
-        return x2, new_h, padded[:, T:]
+        return self._finish(x_seq, normed, y), new_h, padded[:, T:]
+
+    def _finish(self, x, normed, y):
+        """Gate branch, output projection and the gated MLP, both residuals."""
+        x1 = x + self.linear_out(y * F.gelu(self.linear2(normed)))
+        return x1 + self.gated_mlp(self.norm2(x1))
+
+    def step_packed(self, x, state_in, state_out, reset=None, rows_per_env=1):
+        """One timestep on packed state rows, written where they live.
+
+        x (R, D); ``state_in`` / ``state_out`` (R, 4*D) float32 rows ``[h | p0 | p1 | p2]`` of the
+        policy's packed hidden tensor (rows may be strided).  The conv kernel writes the shifted
+        inputs into ``state_out[:, D:]`` and the RG-LRU kernel writes the new state into
+        ``state_out[:, :D]``: no ``cat`` builds the padded sequence or re-packs the state, and a
+        ``reset`` mask (one bool per environment) stands in for zeroing the state beforehand.
+        Returns the sublayer output (R, D).
+        """
+        R, D = x.shape
+        normed = self.norm1(x)
+        v, _ = ops.conv_step(
+            self.linear1(normed), state_in[:, D:].view(R, CONV_KERNEL - 1, D), self.conv.weight, self.conv.bias,
+            conv_out=state_out[:, D:].view(R, CONV_KERNEL - 1, D), reset=reset, rows_per_env=rows_per_env,
+        )
+        y, _ = self.rg_lru.step(v, state_in[:, :D], h_out=state_out[:, :D], reset=reset, rows_per_env=rows_per_env)
+        return self._finish(x, normed, y)
 
     def forward_nonrecurrent(self, x, sub):
         """Same block with ``sub`` (a Linear) in place of conv + RG-LRU; no state."""
@@ -288,6 +326,25 @@ class YemongBlock(nn.Module):
             return x, h[:0], conv_buf[:0]
         return x, torch.stack(new_h), torch.stack(new_cb)
 
+    def step_packed(self, x, alive, state_in, state_out, num_recurrent, reset=None, bullets=None,
+                    bullet_mask=None):
+        """``step`` on this block's slots of the packed hidden tensor.
+
+        ``state_in`` / ``state_out`` are (n_temporal, B*n_rec, 4*D) views; the new state is
+        written into ``state_out`` by the kernels.  Returns the updated tokens (B, NM, D).
+        """
+        B, NM, D = x.shape
+        n_rec = num_recurrent
+        for layer in self.spatial:
+            x = layer(x, alive, bullets, bullet_mask)
+        for j, layer in enumerate(self.temporal):
+            ships = layer.step_packed(x[:, :n_rec].reshape(B * n_rec, D), state_in[j], state_out[j], reset, n_rec)
+            parts = [ships.reshape(B, n_rec, D)]
+            if NM > n_rec:
+                parts.append(layer.forward_nonrecurrent(x[:, n_rec:], self.field_sub[j]))
+            x = torch.cat(parts, dim=1) if len(parts) > 1 else parts[0]
+        return x
+
     def sequence(self, x, alive_mask, h0, conv_buf0, done_mask=None, num_recurrent=None, bullets=None,
                  bullet_mask=None):
         """(T,B,NM,D) variant of ``step`` for re-evaluating a stored rollout (no gradients)."""
@@ -343,7 +400,16 @@ class YemongTrunk(nn.Module):
         return hidden * keep[None, :, None]
 
     @torch.no_grad()
-    def forward(self, tokens, alive_mask, recurrent_state, bullets=None, bullet_mask=None):
+    def forward(self, tokens, alive_mask, recurrent_state, bullets=None, bullet_mask=None, *, reset_mask=None,
+                out_state=None):
+        """tokens (B,NM,D), alive_mask (B,NM) bool, recurrent_state (L, B*n_rec, 4D) -> (hidden, new_state).
+
+        ``reset_mask`` (B,) bool, optional: environments whose incoming state is to be read as
+        zero, i.e. ``forward(x, a, reset_hidden_for_envs(state, reset_mask, n_rec))`` without the
+        extra pass over the state.  ``out_state``: optional preallocated destination for the new
+        state (must not alias ``recurrent_state``); by default a new tensor is returned and the
+        input state is left untouched, as in the reference.
+        """
         B, NM, D = tokens.shape
         L, rows, width = recurrent_state.shape
         if L != self.n_hidden_layers or width != CONV_KERNEL * D or (B and rows % B):
@@ -351,19 +417,21 @@ class YemongTrunk(nn.Module):
                 f"recurrent_state {tuple(recurrent_state.shape)} does not fit {self.n_hidden_layers} layers, "
                 f"{B} environments and d_model {D}"
             )
+        if recurrent_state.dtype != torch.float32:
+            raise TypeError("the recurrent state is float32")
         n_rec = rows // B if B else 0
         n_t = self.config.n_temporal_per_block
-        h_all = recurrent_state[:, :, :D]
-        cb_all = recurrent_state[:, :, D:].reshape(L, rows, CONV_KERNEL - 1, D)
-        x, hs, cbs = tokens, [], []
+        if out_state is None:
+            out_state = torch.empty_like(recurrent_state)
+        elif out_state.shape != recurrent_state.shape or out_state.dtype != torch.float32 or (
+            out_state.data_ptr() == recurrent_state.data_ptr() and L
+        ):
+            raise ValueError("out_state must be a separate float32 tensor shaped like recurrent_state")
+        if reset_mask is not None:
+            reset_mask = reset_mask.contiguous()
+        x = tokens
         for i, block in enumerate(self.yemong_layers):
             sl = slice(i * n_t, (i + 1) * n_t)
-            x, h_i, cb_i = block.step(x, alive_mask, h_all[sl], cb_all[sl], n_rec, bullets, bullet_mask)
-            hs.append(h_i)
-            cbs.append(cb_i)
-        if L == 0:
-            return x, recurrent_state
-        new_state = torch.cat(
-            [torch.cat(hs, dim=0), torch.cat(cbs, dim=0).reshape(L, rows, (CONV_KERNEL - 1) * D)], dim=-1
-        )
-        return x, new_state
+            x = block.step_packed(x, alive_mask, recurrent_state[sl], out_state[sl], n_rec, reset_mask, bullets,
+                                  bullet_mask)
+        return x, out_state

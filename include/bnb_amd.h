@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 1
+#define BNB_ABI_VERSION 2
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -118,6 +118,51 @@ int bnb_rglru_step_fwd(const void *x, int x_dtype, const void *gates_pre, int g_
                        const float *h_in, int64_t h_in_row_stride,
                        float *h_out, int64_t h_out_row_stride,
                        void *y, int y_dtype, int64_t R, int D, void *stream);
+
+/*
+ * bnb_rglru_step_fwd with an optional per-environment reset folded into the read of the
+ * previous state: rows r with reset[r / rows_per_env] != 0 use h = 0.  This is the effect of
+ * the reference's reset_hidden_for_envs (models/yemong/policy.py:268-285, a full read+write of
+ * the packed state after every step) applied to the RG-LRU columns, without that pass.
+ * reset == NULL behaves exactly like bnb_rglru_step_fwd; reset holds one byte per environment
+ * and rows are environment-major (models/yemong/griffin.py:408).
+ */
+int bnb_rglru_step_reset_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
+                             const float *log_lambda, float c,
+                             const float *h_in, int64_t h_in_row_stride,
+                             float *h_out, int64_t h_out_row_stride,
+                             void *y, int y_dtype, const uint8_t *reset, int rows_per_env,
+                             int64_t R, int D, void *stream);
+
+/*
+ * Causal depthwise conv (kernel 4) for one timestep plus the shift of the stored inputs.
+ *
+ * Replaces, in models/yemong/griffin.py at T = 1: `padded = cat([conv_buf, b1])` (:275), the
+ * tap loop of _causal_depthwise_conv (:127-139: out = sum_k padded[:, k] * weight[:, k] + bias)
+ * and `new_conv_buf = padded[:, -3:]` (:277); and, in models/yemong/policy.py, the re-packing
+ * cat of the conv columns (:346-354) because the new inputs are written where they live.
+ *
+ *   b1        (R, D) contiguous, b1_dtype: this step's linear1 output (bf16 under autocast)
+ *   conv_in   previous three inputs of row r at conv_in + r*conv_in_row_stride, laid out
+ *             [p0 | p1 | p2] (oldest first), D floats each; a stride of 4*D with conv_in =
+ *             state + D addresses the packed hidden tensor (policy.py:324)
+ *   weight    (D, 4) fp32 = conv.weight.squeeze(1); tap k multiplies padded[:, k], so the
+ *             current input meets weight[:, 3]
+ *   bias      (D) fp32 or NULL
+ *   reset     optional, one byte per environment of rows_per_env rows: a non-zero byte makes
+ *             the stored inputs read as zero (reset_hidden_for_envs folded in)
+ *   v_out     (R, D) fp32 contiguous: the conv output (input of the RG-LRU and its gates)
+ *   conv_out  new stored inputs [p1 | p2 | b1], same addressing as conv_in; may equal conv_in
+ *
+ * Requirements: D >= 1, strides >= 3*D.  16-byte aligned rows with D % 8 == 0 take the vector
+ * path; anything else takes a scalar path.
+ */
+int bnb_conv_step_fwd(const void *b1, int b1_dtype,
+                      const float *conv_in, int64_t conv_in_row_stride,
+                      const float *weight, const float *bias,
+                      const uint8_t *reset, int rows_per_env,
+                      float *v_out, float *conv_out, int64_t conv_out_row_stride,
+                      int64_t R, int D, void *stream);
 
 /*
  * Plain device-to-device copy of `bytes` bytes (multiple of 16, 16-byte aligned) by a

@@ -344,6 +344,79 @@ def test_rglru_rollout_of_full_size_state_matches_oracle_on_sampled_rows():
     assert torch.isfinite(h).all()
 
 
+# ------------------------------------------------------------------ conv step and folded reset
+
+
+def _conv_ref(b1, conv_buf, weight, bias):
+    """padded = [p0,p1,p2,b1]; v = sum_k padded[k] * w[:,k] + bias; buffer shifts (griffin.py:127-139,275-277)."""
+    padded = torch.cat([conv_buf, b1.float().unsqueeze(1)], dim=1)
+    v = (padded * weight.reshape(-1, 4).t().unsqueeze(0)).sum(dim=1)
+    return (v + bias if bias is not None else v), padded[:, 1:]
+
+
+@pytest.mark.parametrize("R,D,dtype", [(1, 128, torch.float32), (77, 128, torch.bfloat16), (5000, 128, torch.bfloat16),
+                                       (9, 32, torch.float32), (7, 12, torch.bfloat16), (3, 136, torch.float32)])
+def test_conv_step_matches_tap_formula(R, D, dtype):
+    g = torch.Generator().manual_seed(R + D)
+    b1 = torch.randn(R, D, generator=g).to(dtype)
+    buf = torch.randn(R, 3, D, generator=g)
+    w = 0.5 * torch.randn(D, 1, 4, generator=g)
+    bias = 0.1 * torch.randn(D, generator=g)
+    v, new_buf = ops.conv_step(b1.to(DEV), buf.to(DEV), w.to(DEV), bias.to(DEV))
+    ref_v, ref_buf = _conv_ref(b1, buf, w, bias)
+    assert v.dtype == torch.float32 and new_buf.shape == (R, 3, D)
+    assert max_rel(v.cpu(), ref_v) <= F32_TOL
+    assert torch.equal(new_buf.cpu(), ref_buf)  # a pure shift: bit exact
+    # the library depthwise conv as an independent statement of the tap order
+    lib = torch.nn.functional.conv1d(torch.cat([buf, b1.float().unsqueeze(1)], 1).transpose(1, 2), w, bias, groups=D)[:, :, 0]
+    assert max_rel(v.cpu(), lib) <= F32_TOL
+    v2, _ = ops.conv_step(b1.to(DEV), buf.to(DEV), w.to(DEV), None)
+    assert max_rel(v2.cpu(), ref_v - bias) <= F32_TOL
+
+
+def test_conv_and_rglru_step_update_the_packed_state_in_place_with_reset():
+    # rows of the policy's packed hidden (R, 4D) = [h | p0 | p1 | p2]; environments 1 and 3 were reset
+    B, n_rec, D = 5, 3, 128
+    R = B * n_rec
+    g = torch.Generator().manual_seed(9)
+    state = torch.randn(R, 4 * D, generator=g)
+    b1 = torch.randn(R, D, generator=g).bfloat16()
+    w, bias = 0.5 * torch.randn(D, 1, 4, generator=g), 0.1 * torch.randn(D, generator=g)
+    gates = torch.randn(R, 2 * D, generator=g).bfloat16()
+    lam = torch.linspace(0, 4, D)
+    done = torch.tensor([False, True, False, True, False])
+    dev_in, dev_out = state.to(DEV), torch.full((R, 4 * D), float("nan"), device=DEV)
+    v, _ = ops.conv_step(b1.to(DEV), dev_in[:, D:].view(R, 3, D), w.to(DEV), bias.to(DEV),
+                         conv_out=dev_out[:, D:].view(R, 3, D), reset=done.to(DEV), rows_per_env=n_rec)
+    y, _ = ops.rglru_step(v, gates.to(DEV), lam.to(DEV), 8.0, dev_in[:, :D], h_out=dev_out[:, :D],
+                          reset=done.to(DEV), rows_per_env=n_rec)
+    assert torch.equal(dev_in.cpu(), state)  # the incoming state is never written
+    zeroed = torch_ref.reset_hidden(state.unsqueeze(0), done, n_rec)[0]
+    ref_v, ref_buf = _conv_ref(b1, zeroed[:, D:].reshape(R, 3, D), w, bias)
+    ref_h = torch_ref.rglru_step(ref_v, gates, lam, 8.0, zeroed[:, :D])
+    assert max_rel(v.cpu(), ref_v) <= F32_TOL
+    assert torch.equal(dev_out[:, D:].cpu(), ref_buf.reshape(R, 3 * D))
+    assert max_rel(dev_out[:, :D].cpu(), ref_h) <= 4e-3  # bf16 gate flow, fp32 oracle of the same dtypes
+    assert y.data_ptr() == dev_out.data_ptr()
+
+
+def test_conv_step_full_size_rows_sampled_against_formula():
+    w_ = harness.WORKLOADS["c4_64v88_bf16"]
+    R, D = w_.B * w_.N, 128
+    g = torch.Generator(device=DEV).manual_seed(4)
+    state = torch.randn(R, 4 * D, device=DEV, generator=g)
+    b1 = torch.randn(R, D, device=DEV, generator=g).bfloat16()
+    w = 0.5 * torch.randn(D, 1, 4, device=DEV, generator=g)
+    bias = 0.1 * torch.randn(D, device=DEV, generator=g)
+    new_state = torch.empty_like(state)
+    v, _ = ops.conv_step(b1, state[:, D:].view(R, 3, D), w, bias, conv_out=new_state[:, D:].view(R, 3, D))
+    pick = torch.arange(0, R, 7919, device=DEV)
+    ref_v, ref_buf = _conv_ref(b1[pick].cpu(), state[pick, D:].reshape(-1, 3, D).cpu(), w.cpu(), bias.cpu())
+    assert max_rel(v[pick].cpu(), ref_v) <= F32_TOL
+    assert torch.equal(new_state[pick, D:].cpu(), ref_buf.reshape(-1, 3 * D))
+    assert torch.equal(new_state[:, D:2 * D], state[:, 2 * D:3 * D])  # whole-tensor shift property
+
+
 # ------------------------------------------------------------------ the measured step
 
 

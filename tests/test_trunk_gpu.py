@@ -316,3 +316,32 @@ def test_trunk_under_autocast_matches_oracle_within_bf16_bar():
         assert hidden.dtype == torch.float32
         assert max_rel(out.float().cpu(), ref_out) <= BF16_TOL, t
         assert max_rel(hidden.cpu(), ref_hidden) <= BF16_TOL, t
+
+
+def test_trunk_folded_reset_equals_reset_then_step_and_leaves_input_state_alone():
+    # policy.py:268-285 zeroes the packed state of finished environments in a separate pass;
+    # reset_mask folds that into the step kernels
+    D, H, B, N, M = 128, 4, 6, 8, 4
+    p = trunk_params(31, D, 2, 2, 1)
+    trunk = bnb.YemongTrunk(_cfg(D, H, 2, 2, 1)).eval()
+    trunk.load_state_dict(p)
+    trunk.to(DEV)
+    gen = torch.Generator().manual_seed(31)
+    x = torch.randn(B, N + M, D, generator=gen)
+    alive = torch.ones(B, N + M, dtype=torch.bool)
+    alive[2, 3] = False
+    hidden = torch.randn(2, B * N, 4 * D, generator=gen)
+    done = torch.tensor([False, True, False, False, True, False])
+    dev_hidden = hidden.to(DEV)
+    out_a, state_a = trunk(x.to(DEV), alive.to(DEV), dev_hidden, reset_mask=done.to(DEV))
+    assert torch.equal(dev_hidden.cpu(), hidden)
+    out_b, state_b = trunk(x.to(DEV), alive.to(DEV), trunk.reset_hidden_for_envs(dev_hidden, done.to(DEV), N))
+    assert torch.equal(out_a, out_b) and torch.equal(state_a, state_b)
+    ref_out, ref_state = torch_ref.trunk_step(p, 2, 2, 1, H, x, alive, torch_ref.reset_hidden(hidden, done, N))
+    assert max_rel(out_a.cpu(), ref_out) <= 5e-5 and max_rel(state_a.cpu(), ref_state) <= 5e-5
+    # preallocated destination
+    dest = torch.empty_like(dev_hidden)
+    _, state_c = trunk(x.to(DEV), alive.to(DEV), dev_hidden, reset_mask=done.to(DEV), out_state=dest)
+    assert state_c.data_ptr() == dest.data_ptr() and torch.equal(dest, state_a)
+    with pytest.raises(ValueError):
+        trunk(x.to(DEV), alive.to(DEV), dev_hidden, out_state=dev_hidden)
