@@ -39,6 +39,7 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU-baseline leg; 0 skips it")
     ap.add_argument("--no-torch-baseline", action="store_true")
     ap.add_argument("--no-module", action="store_true")
+    ap.add_argument("--no-trunk", action="store_true", help="skip the whole-trunk leg (2 blocks x (2 spatial + 1 temporal))")
     return ap.parse_args()
 
 
@@ -69,6 +70,71 @@ def torch_rglru_region(x, gates, log_lambda, c, h):
     a = torch.sigmoid(log_lambda) ** (c * r)
     gate = torch.sqrt(torch.clamp((1.0 - a) * (1.0 + a), min=1e-6))
     return a * h + gate * (i * x)
+
+
+def torch_conv_region(b1, conv_buf, weight, bias):
+    padded = torch.cat([conv_buf, b1.unsqueeze(1)], dim=1)
+    w = weight.reshape(-1, 4)
+    out = torch.zeros_like(padded[:, :1])
+    for k in range(4):
+        out = out + padded[:, k:k + 1] * w[:, k]
+    return (out + bias)[:, 0], padded[:, 1:]
+
+
+class eager_kernels:
+    """Context manager: the trunk layers run the reference-style eager PyTorch regions above
+    instead of the HIP kernels (same modules, same weights) - the GPU baseline of the trunk leg."""
+
+    def __enter__(self):
+        from boost_and_broadside_amd import ops
+
+        self.ops = ops
+        self.saved = (ops.sdpa_masked, ops.rglru_step, ops.conv_step, ops.add_rmsnorm, ops.gelu_mul)
+
+        def sdpa(qkv, alive, n_heads, **kw):
+            if alive is None:
+                alive = torch.ones(qkv.shape[:2], dtype=torch.bool, device=qkv.device)
+            return torch_attention_region(qkv, alive, n_heads)
+
+        def rglru(x, gates, lam, c, h, **kw):
+            out = torch_rglru_region(x, gates, lam, c, h)
+            return out, out
+
+        def conv(b1, conv_buf, weight, bias, also_bf16=False, **kw):
+            v, buf = torch_conv_region(b1, conv_buf, weight, bias)
+            return (v, buf, v.to(torch.bfloat16)) if also_bf16 else (v, buf)
+
+        def add_rmsnorm(x, weight, delta=None, eps=None, out_dtype=torch.float32):
+            s = x if delta is None else x + delta
+            return s, F.rms_norm(s, (s.shape[-1],), weight, eps).to(out_dtype)
+
+        def gelu_mul(a, b, out_dtype=None):
+            out = F.gelu(a) * b
+            return out if out_dtype is None else out.to(out_dtype)
+
+        ops.sdpa_masked, ops.rglru_step, ops.conv_step, ops.add_rmsnorm, ops.gelu_mul = sdpa, rglru, conv, add_rmsnorm, gelu_mul
+        return self
+
+    def __exit__(self, *exc):
+        o = self.ops
+        o.sdpa_masked, o.rglru_step, o.conv_step, o.add_rmsnorm, o.gelu_mul = self.saved
+        return False
+
+
+def reference_style_trunk_step(trunk, x, alive, hidden, n_rec):
+    """The block loop as the reference writes it: unpack views, per-block step, cat and re-pack
+    (models/yemong/policy.py:316-354)."""
+    L, rows, width = hidden.shape
+    D = width // 4
+    n_t = trunk.config.n_temporal_per_block
+    h_all, cb_all = hidden[:, :, :D], hidden[:, :, D:].reshape(L, rows, 3, D)
+    hs, cbs = [], []
+    for i, block in enumerate(trunk.yemong_layers):
+        sl = slice(i * n_t, (i + 1) * n_t)
+        x, h_i, cb_i = block.step(x, alive, h_all[sl], cb_all[sl], n_rec)
+        hs.append(h_i)
+        cbs.append(cb_i)
+    return x, torch.cat([torch.cat(hs, 0), torch.cat(cbs, 0).reshape(L, rows, 3 * D)], dim=-1)
 
 
 # ---------------------------------------------------------------------------------------------
@@ -319,6 +385,60 @@ def main():
 
         wall_m = timed_loop(module_step, steps, warmup)
         result["module"] = {"value": tokens * steps / wall_m, "unit": "entity-tokens/s", "ms_per_step": wall_m / steps * 1e3}
+
+    # ---- conv-step kernel (temporal block's causal conv + buffer shift on the packed state) ----
+    R = w.B * w.N
+    packed = [torch.randn(R, 4 * D, device=dev, generator=gen), None]
+    packed[1] = torch.empty_like(packed[0])
+    b1_pool = [x_pool[i] for i in range(POOL)]  # same shape and dtype as linear1's output
+    conv_w = 0.5 * torch.randn(D, 1, 4, device=dev, generator=gen)
+    conv_b = 0.1 * torch.randn(D, device=dev, generator=gen)
+
+    def launch_conv(t):
+        src, dst = packed[t & 1], packed[(t + 1) & 1]
+        ops.conv_step(b1_pool[t % POOL], src[:, D:].view(R, 3, D), conv_w, conv_b, conv_out=dst[:, D:].view(R, 3, D))
+
+    t_conv = timed_loop(launch_conv, steps, warmup) / steps
+    s_act = 2 if bf16 else 4
+    conv_bytes = R * (D * s_act + 3 * D * 4 + D * 4 + 3 * D * 4)
+    result["conv_step_kernel"] = {
+        "avg_launch_us": t_conv * 1e6, "algorithmic_bytes_per_launch": conv_bytes, "achieved_GBps": conv_bytes / t_conv / 1e9,
+        "frac_of_hbm_peak": conv_bytes / t_conv / peak,
+        "what": "read linear1 output + 3 stored inputs, write conv output + shifted inputs into the packed state",
+    }
+    del packed
+
+    # ---- whole trunk (reference default: 2 blocks x (2 spatial + 1 temporal)), state carried ----
+    if not args.no_trunk:
+        cfg = bnb.ModelConfig(d_model=D, n_heads=H, n_yemong_blocks=2, n_spatial_per_block=2, n_temporal_per_block=1)
+        torch.manual_seed(w.seed)
+        trunk = bnb.YemongTrunk(cfg).to(dev).eval()
+        x32 = [t.float() for t in tokens_pool[:2]]
+        n_tr = max(4, min(steps, 16))
+        hid = [trunk.initial_hidden(w.B, w.N, dev), None]
+        hid[1] = torch.empty_like(hid[0])
+
+        def trunk_step(t):
+            with torch.autocast("cuda", dtype=torch.bfloat16, enabled=bf16):
+                trunk(x32[t & 1], alive_steps[t % n_alive], hid[t & 1], out_state=hid[(t + 1) & 1])
+
+        wall_tr = timed_loop(trunk_step, n_tr, 10)  # first calls pay GEMM heuristics and code loading
+        ref_h = [trunk.initial_hidden(w.B, w.N, dev)]
+
+        def trunk_step_eager(t):
+            with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16, enabled=bf16):
+                _, ref_h[0] = reference_style_trunk_step(trunk, x32[t & 1], alive_steps[t % n_alive], ref_h[0], w.N)
+
+        with eager_kernels():
+            wall_te = timed_loop(trunk_step_eager, n_tr, 10)
+        result["trunk"] = {
+            "value": tokens * n_tr / wall_tr, "unit": "entity-tokens/s", "ms_per_step": wall_tr / n_tr * 1e3,
+            "steps": n_tr, "eager_torch_ms_per_step": wall_te / n_tr * 1e3, "speedup_over_eager_torch": wall_te / wall_tr,
+            "what": "YemongTrunk.forward, 2 blocks x (2 attention + 1 temporal sublayer), d_model 128, packed fp32 state "
+                    "carried, " + ("bf16 autocast" if bf16 else "fp32") + "; eager = same modules with the kernels "
+                    "replaced by the reference's torch ops and its unpack/cat/re-pack of the state",
+        }
+        del trunk, hid, ref_h
 
     # free the device before the host leg
     if args.cpu_seconds > 0:

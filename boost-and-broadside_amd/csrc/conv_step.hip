@@ -22,7 +22,7 @@ template <int THREADS, typename BT>
 __global__ __launch_bounds__(THREADS) void conv_step_vec8_kernel(
     const BT *__restrict__ b1, const float *conv_in, int64_t conv_in_stride, const float *__restrict__ weight,
     const float *__restrict__ bias, const uint8_t *__restrict__ reset, int rows_per_env, float *__restrict__ v_out,
-    float *conv_out, int64_t conv_out_stride, int64_t R, int D, int rows_per_block)
+    uint16_t *__restrict__ v_bf16_out, float *conv_out, int64_t conv_out_stride, int64_t R, int D, int rows_per_block)
 {
     extern __shared__ float s_wb[];  // D*4 tap weights (as stored: [d][k]) then D biases
     for (int i = threadIdx.x; i < D * kTaps; i += THREADS) s_wb[i] = weight[i];
@@ -55,6 +55,7 @@ __global__ __launch_bounds__(THREADS) void conv_step_vec8_kernel(
         v.v[e] = acc + s_wb[D * kTaps + d0 + e];
     }
     store8_stream(v_out + row * D + d0, v);
+    if (v_bf16_out != nullptr) store8_stream(v_bf16_out + row * D + d0, v);
     float *pout = conv_out + row * conv_out_stride + d0;
     store8_stream(pout, p1);
     store8_stream(pout + D, p2);
@@ -66,7 +67,7 @@ template <typename BT>
 __global__ __launch_bounds__(kConvThreads) void conv_step_scalar_kernel(
     const BT *__restrict__ b1, const float *conv_in, int64_t conv_in_stride, const float *__restrict__ weight,
     const float *__restrict__ bias, const uint8_t *__restrict__ reset, int rows_per_env, float *__restrict__ v_out,
-    float *conv_out, int64_t conv_out_stride, int64_t R, int D)
+    uint16_t *__restrict__ v_bf16_out, float *conv_out, int64_t conv_out_stride, int64_t R, int D)
 {
     const int64_t idx = (int64_t)blockIdx.x * kConvThreads + threadIdx.x;
     if (idx >= R * D) return;
@@ -81,7 +82,9 @@ __global__ __launch_bounds__(kConvThreads) void conv_step_scalar_kernel(
     acc += p1 * w[1];
     acc += p2 * w[2];
     acc += cur * w[3];
-    v_out[idx] = acc + (bias != nullptr ? bias[d] : 0.0f);
+    const float v = acc + (bias != nullptr ? bias[d] : 0.0f);
+    v_out[idx] = v;
+    if (v_bf16_out != nullptr) store1(v_bf16_out + idx, v);
     float *pout = conv_out + row * conv_out_stride + d;
     pout[0] = p1;
     pout[D] = p2;
@@ -90,11 +93,11 @@ __global__ __launch_bounds__(kConvThreads) void conv_step_scalar_kernel(
 
 template <typename BT>
 static int launch_conv(const void *b1, const float *conv_in, int64_t conv_in_stride, const float *weight,
-                       const float *bias, const uint8_t *reset, int rows_per_env, float *v_out, float *conv_out,
-                       int64_t conv_out_stride, int64_t R, int D, hipStream_t stream)
+                       const float *bias, const uint8_t *reset, int rows_per_env, float *v_out, uint16_t *v_bf16_out,
+                       float *conv_out, int64_t conv_out_stride, int64_t R, int D, hipStream_t stream)
 {
     const bool vec = (D % 8 == 0) && (D / 8 <= kConvThreads) && aligned16(b1) && aligned16(conv_in) &&
-                     aligned16(conv_out) && aligned16(v_out) && (conv_in_stride % 4 == 0) &&
+                     aligned16(conv_out) && aligned16(v_out) && aligned16(v_bf16_out) && (conv_in_stride % 4 == 0) &&
                      (conv_out_stride % 4 == 0) && (size_t)D * (kTaps + 1) * sizeof(float) <= 48 * 1024;
     if (vec) {
         const int vecs_per_row = D / 8;
@@ -107,17 +110,17 @@ static int launch_conv(const void *b1, const float *conv_in, int64_t conv_in_str
         if (big)
             hipLaunchKernelGGL((conv_step_vec8_kernel<kConvBigThreads, BT>), dim3((unsigned)blocks), dim3(threads), lds,
                                stream, (const BT *)b1, conv_in, conv_in_stride, weight, bias, reset, rows_per_env,
-                               v_out, conv_out, conv_out_stride, R, D, rows_per_block);
+                               v_out, v_bf16_out, conv_out, conv_out_stride, R, D, rows_per_block);
         else
             hipLaunchKernelGGL((conv_step_vec8_kernel<kConvThreads, BT>), dim3((unsigned)blocks), dim3(threads), lds,
                                stream, (const BT *)b1, conv_in, conv_in_stride, weight, bias, reset, rows_per_env,
-                               v_out, conv_out, conv_out_stride, R, D, rows_per_block);
+                               v_out, v_bf16_out, conv_out, conv_out_stride, R, D, rows_per_block);
     } else {
         const int64_t blocks = (R * D + kConvThreads - 1) / kConvThreads;
         if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
         hipLaunchKernelGGL((conv_step_scalar_kernel<BT>), dim3((unsigned)blocks), dim3(kConvThreads), 0, stream,
                            (const BT *)b1, conv_in, conv_in_stride, weight, bias, reset, rows_per_env, v_out,
-                           conv_out, conv_out_stride, R, D);
+                           v_bf16_out, conv_out, conv_out_stride, R, D);
     }
     return (int)hipGetLastError();
 }
@@ -126,8 +129,8 @@ static int launch_conv(const void *b1, const float *conv_in, int64_t conv_in_str
 
 extern "C" int bnb_conv_step_fwd(const void *b1, int b1_dtype, const float *conv_in, int64_t conv_in_row_stride,
                                  const float *weight, const float *bias, const uint8_t *reset, int rows_per_env,
-                                 float *v_out, float *conv_out, int64_t conv_out_row_stride, int64_t R, int D,
-                                 void *stream)
+                                 float *v_out, void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride,
+                                 int64_t R, int D, void *stream)
 {
     using namespace bnb;
     if (R < 0 || D < 1) return BNB_ERR_BAD_SHAPE;
@@ -140,11 +143,12 @@ extern "C" int bnb_conv_step_fwd(const void *b1, int b1_dtype, const float *conv
          reinterpret_cast<uintptr_t>(v_out) | reinterpret_cast<uintptr_t>(weight) |
          reinterpret_cast<uintptr_t>(bias)) & 3u)
         return BNB_ERR_MISALIGNED;
+    if (reinterpret_cast<uintptr_t>(v_bf16_out) & 1u) return BNB_ERR_MISALIGNED;
     if (reset == nullptr) rows_per_env = 1;
     hipStream_t s = (hipStream_t)stream;
     if (b1_dtype == BNB_BF16)
         return launch_conv<uint16_t>(b1, conv_in, conv_in_row_stride, weight, bias, reset, rows_per_env, v_out,
-                                     conv_out, conv_out_row_stride, R, D, s);
-    return launch_conv<float>(b1, conv_in, conv_in_row_stride, weight, bias, reset, rows_per_env, v_out, conv_out,
-                              conv_out_row_stride, R, D, s);
+                                     (uint16_t *)v_bf16_out, conv_out, conv_out_row_stride, R, D, s);
+    return launch_conv<float>(b1, conv_in, conv_in_row_stride, weight, bias, reset, rows_per_env, v_out,
+                              (uint16_t *)v_bf16_out, conv_out, conv_out_row_stride, R, D, s);
 }

@@ -207,7 +207,8 @@ def conv_step(
     conv_out: torch.Tensor | None = None,
     reset: torch.Tensor | None = None,
     rows_per_env: int = 1,
-) -> tuple[torch.Tensor, torch.Tensor]:
+    also_bf16: bool = False,
+):
     """Causal depthwise conv of one timestep and the shift of the stored inputs.
 
     Args:
@@ -219,9 +220,12 @@ def conv_step(
         conv_out: optional (R, 3, D) float32 destination with the same layout rules (may be
                   ``conv_buf`` itself).  Default: a new contiguous tensor.
         reset, rows_per_env: as in ``rglru_step``: environments whose stored inputs read as zero.
+        also_bf16: also write a bfloat16 copy of the conv output (the input autocast would
+                  feed the gate projections) and return it as a third value.
 
     Returns:
-        (v, new_conv_buf): conv output (R, D) float32 and the shifted buffer ``[p1, p2, b1]``.
+        (v, new_conv_buf[, v_bf16]): conv output (R, D) float32, the shifted buffer
+        ``[p1, p2, b1]``, and the bfloat16 copy when asked for.
     """
     if b1.dim() != 2 or conv_buf.dim() != 3:
         raise ValueError("b1 must be (R, D) and conv_buf (R, 3, D)")
@@ -252,16 +256,104 @@ def conv_step(
     elif conv_out.shape != (R, 3, D) or conv_out.dtype != torch.float32 or conv_out.device != b1.device or not rows_ok(conv_out):
         raise ValueError("conv_out must be a float32 (R, 3, D) tensor on b1's device with contiguous rows")
     v = torch.empty((R, D), dtype=torch.float32, device=b1.device)
+    v_lp = torch.empty((R, D), dtype=torch.bfloat16, device=b1.device) if also_bf16 else None
     reset_ptr = _reset_pointer(reset, R, rows_per_env, b1.device)
-    if R == 0:
-        return v, conv_out
-    with torch.cuda.device(b1.device):
-        rc = _native.load().bnb_conv_step_fwd(
-            b1.data_ptr(), b_code, conv_buf.data_ptr(), conv_buf.stride(0), weight.data_ptr(), bias_ptr,
-            reset_ptr, int(rows_per_env), v.data_ptr(), conv_out.data_ptr(), conv_out.stride(0), R, D, _stream(),
-        )
-    _native.check(rc, "bnb_conv_step_fwd")
-    return v, conv_out
+    if R:
+        with torch.cuda.device(b1.device):
+            rc = _native.load().bnb_conv_step_fwd(
+                b1.data_ptr(), b_code, conv_buf.data_ptr(), conv_buf.stride(0), weight.data_ptr(), bias_ptr,
+                reset_ptr, int(rows_per_env), v.data_ptr(), None if v_lp is None else v_lp.data_ptr(),
+                conv_out.data_ptr(), conv_out.stride(0), R, D, _stream(),
+            )
+        _native.check(rc, "bnb_conv_step_fwd")
+    return (v, conv_out, v_lp) if also_bf16 else (v, conv_out)
+
+
+_F32_EPS = float(torch.finfo(torch.float32).eps)
+_NORM_WIDTHS = (8, 16, 32, 64, 128, 256, 512)
+
+
+def add_rmsnorm(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    *,
+    delta: torch.Tensor | None = None,
+    eps: float | None = None,
+    out_dtype: torch.dtype = torch.float32,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """``s = x + delta`` (if given) and ``rmsnorm(s) * weight`` in one pass.
+
+    x (..., D) float32 with contiguous rows; delta same shape, float32 or bfloat16; weight (D,)
+    float32; eps defaults to ``finfo(float32).eps`` (``nn.RMSNorm(D)`` with eps=None).
+    Returns (s, normed): s is x itself when there is no delta; normed has ``out_dtype``.
+    """
+    D = x.shape[-1]
+    if x.dtype != torch.float32 or weight.dtype != torch.float32 or weight.shape != (D,):
+        raise TypeError("x and weight must be float32 and weight must be (D,)")
+    if D not in _NORM_WIDTHS:
+        raise ValueError(f"add_rmsnorm supports D in {_NORM_WIDTHS}, got {D}")
+    _need_device(x, "x")
+    if torch.is_grad_enabled() and (x.requires_grad or (delta is not None and delta.requires_grad)):
+        raise RuntimeError("add_rmsnorm is forward-only; call it under torch.no_grad()")
+    x2 = x.reshape(-1, D)
+    if x2.numel() and x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    R = x2.shape[0]
+    d_ptr, d_code, s_out = None, _native.F32, None
+    if delta is not None:
+        if delta.shape != x.shape:
+            raise ValueError(f"delta must be {tuple(x.shape)}, got {tuple(delta.shape)}")
+        delta = delta.reshape(-1, D).contiguous()
+        d_ptr, d_code = delta.data_ptr(), _code(delta, "delta")
+        s_out = torch.empty((R, D), dtype=torch.float32, device=x.device)
+    normed = torch.empty((R, D), dtype=out_dtype, device=x.device)
+    o_code = _code(normed, "out_dtype")
+    if R:
+        with torch.cuda.device(x.device):
+            rc = _native.load().bnb_add_rmsnorm_fwd(
+                x2.data_ptr(), x2.stride(0), d_ptr, d_code, weight.detach().contiguous().data_ptr(),
+                _F32_EPS if eps is None else float(eps), None if s_out is None else s_out.data_ptr(),
+                normed.data_ptr(), o_code, R, D, _stream(),
+            )
+        _native.check(rc, "bnb_add_rmsnorm_fwd")
+    return (x if s_out is None else s_out.reshape(x.shape)), normed.reshape(x.shape)
+
+
+def gelu_mul(a: torch.Tensor, b: torch.Tensor, *, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """``gelu(a) * b`` (erf GELU) for (..., H) tensors whose rows may be strided.
+
+    The gelu is rounded to a's dtype (as ``F.gelu`` returns it), the product once to
+    ``out_dtype`` (default: torch's promotion of a and b).
+    """
+    if a.shape != b.shape:
+        raise ValueError(f"a {tuple(a.shape)} and b {tuple(b.shape)} differ")
+    H = a.shape[-1]
+    if H % 8:
+        raise ValueError(f"gelu_mul needs a multiple of 8 channels, got {H}")
+    _need_device(a, "a")
+    _need_device(b, "b")
+    if torch.is_grad_enabled() and (a.requires_grad or b.requires_grad):
+        raise RuntimeError("gelu_mul is forward-only; call it under torch.no_grad()")
+    if out_dtype is None:
+        out_dtype = torch.promote_types(a.dtype, b.dtype)
+
+    def rows(t):
+        t2 = t.reshape(-1, H) if t.dim() != 2 else t
+        if t2.numel() and t2.stride(-1) != 1:
+            t2 = t2.contiguous()
+        return t2
+
+    a2, b2 = rows(a), rows(b)
+    R = a2.shape[0]
+    out = torch.empty((R, H), dtype=out_dtype, device=a.device)
+    if R:
+        with torch.cuda.device(a.device):
+            rc = _native.load().bnb_gelu_mul_fwd(
+                a2.data_ptr(), _code(a2, "a"), a2.stride(0), b2.data_ptr(), _code(b2, "b"), b2.stride(0),
+                out.data_ptr(), _code(out, "out_dtype"), R, H, _stream(),
+            )
+        _native.check(rc, "bnb_gelu_mul_fwd")
+    return out.reshape(a.shape)
 
 
 def copy_bytes(src: torch.Tensor, dst: torch.Tensor) -> None:

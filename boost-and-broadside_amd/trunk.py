@@ -34,6 +34,47 @@ from . import ops
 
 CONV_KERNEL = 4  # taps of the causal depthwise conv; the state keeps the last CONV_KERNEL-1 inputs
 
+_FUSED_WIDTHS = (8, 16, 32, 64, 128, 256, 512)  # d_model values the fused norm kernel covers
+
+
+def _projection_dtype() -> torch.dtype:
+    """dtype a Linear computes in right now: the autocast dtype if autocast is on, else float32."""
+    if torch.is_autocast_enabled("cuda"):
+        return torch.get_autocast_dtype("cuda")
+    return torch.float32
+
+
+def _fused_ok(x: torch.Tensor, act: torch.dtype) -> bool:
+    """Whether the fused norm / gelu kernels apply: fp32 residual stream on the GPU, a covered
+    width, fp32 or bf16 projections.  Anything else takes the plain torch composition."""
+    return (
+        x.is_cuda and x.dtype == torch.float32 and x.shape[-1] in _FUSED_WIDTHS
+        and act in (torch.float32, torch.bfloat16)
+    )
+
+
+def _cached_cast(owner: nn.Module, slot: str, tensors: tuple, dtype: torch.dtype, build):
+    """``build()`` (a tensor derived from ``tensors`` in ``dtype``) cached on ``owner`` until one
+    of the source tensors is modified or replaced.  Saves the per-step weight casts autocast
+    would otherwise repeat."""
+    key = (dtype,) + tuple((t._version, t.data_ptr(), t.device) for t in tensors)
+    hit = owner.__dict__.get(slot)
+    if hit is None or hit[0] != key:
+        with torch.no_grad():
+            hit = (key, build())
+        owner.__dict__[slot] = hit
+    return hit[1]
+
+
+def _project(layer: nn.Linear, x: torch.Tensor) -> torch.Tensor:
+    """``layer(x)`` for an activation that already has the projection dtype."""
+    w, b = layer.weight, layer.bias
+    if x.dtype == w.dtype:
+        return F.linear(x, w, b)
+    wc = _cached_cast(layer, "_bnb_w", (w,), x.dtype, lambda: w.detach().to(x.dtype))
+    bc = None if b is None else _cached_cast(layer, "_bnb_b", (b,), x.dtype, lambda: b.detach().to(x.dtype))
+    return F.linear(x, wc, bc)
+
 
 @dataclass(frozen=True)
 class ModelConfig:
@@ -80,7 +121,16 @@ class GatedMLP(nn.Module):
         self.down_proj = nn.Linear(expand * d_model, d_model, bias=False)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.down_proj(F.gelu(self.gate_proj(x)) * self.up_proj(x))
+        hidden = self.gate_proj.out_features
+        if not x.is_cuda or hidden % 8 or x.dtype not in (torch.float32, torch.bfloat16) or (
+            torch.is_grad_enabled() and x.requires_grad
+        ):
+            return self.down_proj(F.gelu(self.gate_proj(x)) * self.up_proj(x))
+        # one GEMM for [gate | up], one kernel for gelu(gate) * up, one GEMM down
+        wg, wu = self.gate_proj.weight, self.up_proj.weight
+        w = _cached_cast(self, "_bnb_gate_up", (wg, wu), x.dtype, lambda: torch.cat([wg, wu], dim=0).detach().to(x.dtype))
+        gu = F.linear(x, w)
+        return _project(self.down_proj, ops.gelu_mul(gu[..., :hidden], gu[..., hidden:], out_dtype=x.dtype))
 
 
 class TransformerBlock(nn.Module):
@@ -106,15 +156,22 @@ class TransformerBlock(nn.Module):
         self.ffn = GatedMLP(D)
 
     def forward(self, x, alive_mask=None, bullets=None, bullet_mask=None):
-        x = x + self._attn(self.norm1(x), alive_mask, bullets, bullet_mask)
-        return x + self.ffn(self.norm2(x))
+        act = _projection_dtype()
+        if not _fused_ok(x, act):
+            x = x + self._attn(self.norm1(x), alive_mask, bullets, bullet_mask)
+            return x + self.ffn(self.norm2(x))
+        # norm (+ cast) -> qkv -> attention kernel -> out_proj -> add + norm (+ cast) -> FFN
+        _, n1 = ops.add_rmsnorm(x, self.norm1.weight, eps=self.norm1.eps, out_dtype=act)
+        attn = self._attn(n1, alive_mask, bullets, bullet_mask)
+        x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=attn, eps=self.norm2.eps, out_dtype=act)
+        return x1 + self.ffn(n2)
 
     def _attn(self, x, alive_mask, bullets=None, bullet_mask=None):
-        qkv = self.qkv(x)  # (B, N, 3D), fp32 or bf16 under autocast
+        qkv = _project(self.qkv, x)  # (B, N, 3D), fp32 or bf16 under autocast
         merged = ops.sdpa_masked(qkv, alive_mask, self.n_heads)  # (B, N, D) head-major
         if self.reads_bullets and bullets is not None:
             merged = merged + self._bullet_read(qkv, bullets, bullet_mask)
-        return self.out_proj(merged)
+        return _project(self.out_proj, merged)
 
     def _bullet_read(self, qkv, bullets, bullet_mask):
         """Cross-attention of the entity queries to bullet key/values (attention.py:149-166).
@@ -148,22 +205,24 @@ class RGLRU(nn.Module):
         self.log_lambda = nn.Parameter(torch.linspace(0.0, 4.0, d_model))
         self.linear_a = nn.Linear(d_model, d_model, bias=True)
         self.linear_x = nn.Linear(d_model, d_model, bias=True)
-        self._fused: tuple | None = None  # (key, weight (2D,D), bias (2D,))
 
-    def _gate_preactivations(self, x: torch.Tensor) -> torch.Tensor:
-        """``[linear_a(x) | linear_x(x)]`` as one (R, 2D) GEMM over concatenated weights."""
+    def _gate_preactivations(self, x: torch.Tensor, x_act: torch.Tensor | None = None) -> torch.Tensor:
+        """``[linear_a(x) | linear_x(x)]`` as one (R, 2D) GEMM over concatenated weights.
+
+        ``x_act``: the same rows already in the projection dtype (saves the cast)."""
+        act = _projection_dtype()
+        if x_act is None or x_act.dtype != act:
+            x_act = x.to(act)
         wa, wx, ba, bx = self.linear_a.weight, self.linear_x.weight, self.linear_a.bias, self.linear_x.bias
-        key = (wa._version, wx._version, ba._version, bx._version, wa.data_ptr(), wx.data_ptr(), wa.device)
-        if self._fused is None or self._fused[0] != key:
-            with torch.no_grad():
-                self._fused = (key, torch.cat([wa, wx], dim=0), torch.cat([ba, bx], dim=0))
-        return F.linear(x, self._fused[1], self._fused[2])
+        w = _cached_cast(self, "_bnb_gw", (wa, wx), act, lambda: torch.cat([wa, wx], dim=0).detach().to(act))
+        b = _cached_cast(self, "_bnb_gb", (ba, bx), act, lambda: torch.cat([ba, bx], dim=0).detach().to(act))
+        return F.linear(x_act, w, b)
 
     def _step(self, x: torch.Tensor, h: torch.Tensor) -> torch.Tensor:
         """(R,D), (R,D) -> new state (R,D) float32 (also the layer output)."""
         return self.step(x, h)[1]
 
-    def step(self, x, h, y_dtype=None, *, h_out=None, reset=None, rows_per_env=1):
+    def step(self, x, h, y_dtype=None, *, h_out=None, reset=None, rows_per_env=1, x_act=None):
         """One kernel launch: returns (output in ``y_dtype`` or the state itself, new state).
 
         ``h_out`` lets the new state land in place (e.g. in the RG-LRU columns of a packed
@@ -171,7 +230,7 @@ class RGLRU(nn.Module):
         previous state of those environments read as zero.
         """
         return ops.rglru_step(
-            x, self._gate_preactivations(x), self.log_lambda, self.c, h, y_dtype=y_dtype, h_out=h_out,
+            x, self._gate_preactivations(x, x_act), self.log_lambda, self.c, h, y_dtype=y_dtype, h_out=h_out,
             reset=reset, rows_per_env=rows_per_env,
         )
 
@@ -214,12 +273,10 @@ class GriffinTemporalBlock(nn.Module):
         if T == 1 and done_mask is None:
             # rollout: the conv taps and the buffer shift are one kernel, the recurrence another
             x = x_seq[:, 0]
-            normed = self.norm1(x)
-            v, new_conv_buf = ops.conv_step(self.linear1(normed), conv_buf, self.conv.weight, self.conv.bias)
-            y, new_h = self.rg_lru.step(v, h0)
-            return self._finish(x, normed, y).unsqueeze(1), new_h, new_conv_buf
-        normed = self.norm1(x_seq)
-        b1 = self.linear1(normed)
+            out, new_h, new_conv_buf = self._step(x, h0, conv_buf, None, None, None, 1)
+            return out.unsqueeze(1), new_h, new_conv_buf
+        normed = self._norm_in(x_seq)
+        b1 = _project(self.linear1, normed)
         padded = torch.cat([conv_buf, b1], dim=1)  # (R, T+3, D); fp32 buffer promotes a bf16 b1
         w = self.conv.weight.squeeze(1)  # (D, 4); tap k meets padded[:, t+k]
         if done_mask is None:
@@ -229,10 +286,37 @@ class GriffinTemporalBlock(nn.Module):
         y, new_h = self.rg_lru.forward_sequence(conv_out, h0, done_mask)
         return self._finish(x_seq, normed, y), new_h, padded[:, T:]
 
+    def _norm_in(self, x):
+        """norm1(x) in the projection dtype (one kernel with the cast when the fused path applies)."""
+        act = _projection_dtype()
+        if _fused_ok(x, act):
+            return ops.add_rmsnorm(x, self.norm1.weight, eps=self.norm1.eps, out_dtype=act)[1]
+        return self.norm1(x)
+
     def _finish(self, x, normed, y):
         """Gate branch, output projection and the gated MLP, both residuals."""
-        x1 = x + self.linear_out(y * F.gelu(self.linear2(normed)))
+        act = _projection_dtype()
+        gate_in = _project(self.linear2, normed)
+        if _fused_ok(x, act) and gate_in.dtype == act:
+            # gelu(linear2) * y in one kernel, residual add + norm2 (+ cast) in one kernel
+            r = _project(self.linear_out, ops.gelu_mul(gate_in, y, out_dtype=act))
+            x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=r, eps=self.norm2.eps, out_dtype=act)
+            return x1 + self.gated_mlp(n2)
+        x1 = x + self.linear_out(y * F.gelu(gate_in))
         return x1 + self.gated_mlp(self.norm2(x1))
+
+    def _step(self, x, h_in, conv_in, h_out, conv_out, reset, rows_per_env):
+        """One timestep: x (R,D), h_in (R,D), conv_in (R,3,D) -> (out, new_h, new_conv_buf)."""
+        act = _projection_dtype()
+        normed = self._norm_in(x)
+        b1 = _project(self.linear1, normed)
+        want_lp = act == torch.bfloat16
+        res = ops.conv_step(b1, conv_in, self.conv.weight, self.conv.bias, conv_out=conv_out, reset=reset,
+                            rows_per_env=rows_per_env, also_bf16=want_lp)
+        v, new_conv_buf = res[0], res[1]
+        y, new_h = self.rg_lru.step(v, h_in, h_out=h_out, reset=reset, rows_per_env=rows_per_env,
+                                    x_act=res[2] if want_lp else None)
+        return self._finish(x, normed, y), new_h, new_conv_buf
 
     def step_packed(self, x, state_in, state_out, reset=None, rows_per_env=1):
         """One timestep on packed state rows, written where they live.
@@ -245,20 +329,22 @@ class GriffinTemporalBlock(nn.Module):
         Returns the sublayer output (R, D).
         """
         R, D = x.shape
-        normed = self.norm1(x)
-        v, _ = ops.conv_step(
-            self.linear1(normed), state_in[:, D:].view(R, CONV_KERNEL - 1, D), self.conv.weight, self.conv.bias,
-            conv_out=state_out[:, D:].view(R, CONV_KERNEL - 1, D), reset=reset, rows_per_env=rows_per_env,
-        )
-        y, _ = self.rg_lru.step(v, state_in[:, :D], h_out=state_out[:, :D], reset=reset, rows_per_env=rows_per_env)
-        return self._finish(x, normed, y)
+        return self._step(
+            x, state_in[:, :D], state_in[:, D:].view(R, CONV_KERNEL - 1, D), state_out[:, :D],
+            state_out[:, D:].view(R, CONV_KERNEL - 1, D), reset, rows_per_env,
+        )[0]
 
     def forward_nonrecurrent(self, x, sub):
         """Same block with ``sub`` (a Linear) in place of conv + RG-LRU; no state."""
-        normed = self.norm1(x)
-        b1 = sub(self.linear1(normed))
-        b2 = F.gelu(self.linear2(normed))
-        x1 = x + self.linear_out(b1 * b2)
+        act = _projection_dtype()
+        normed = self._norm_in(x)
+        b1 = _project(sub, _project(self.linear1, normed))
+        gate_in = _project(self.linear2, normed)
+        if _fused_ok(x, act) and gate_in.dtype == act:
+            r = _project(self.linear_out, ops.gelu_mul(gate_in, b1, out_dtype=act))
+            x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=r, eps=self.norm2.eps, out_dtype=act)
+            return x1 + self.gated_mlp(n2)
+        x1 = x + self.linear_out(b1 * F.gelu(gate_in))
         return x1 + self.gated_mlp(self.norm2(x1))
 
 

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 2
+#define BNB_ABI_VERSION 3
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -151,7 +151,9 @@ int bnb_rglru_step_reset_fwd(const void *x, int x_dtype, const void *gates_pre, 
  *   bias      (D) fp32 or NULL
  *   reset     optional, one byte per environment of rows_per_env rows: a non-zero byte makes
  *             the stored inputs read as zero (reset_hidden_for_envs folded in)
- *   v_out     (R, D) fp32 contiguous: the conv output (input of the RG-LRU and its gates)
+ *   v_out     (R, D) fp32 contiguous: the conv output (input of the RG-LRU)
+ *   v_bf16_out optional (R, D) bf16 contiguous copy of v_out (what autocast would feed the
+ *             gate projections), or NULL
  *   conv_out  new stored inputs [p1 | p2 | b1], same addressing as conv_in; may equal conv_in
  *
  * Requirements: D >= 1, strides >= 3*D.  16-byte aligned rows with D % 8 == 0 take the vector
@@ -161,8 +163,38 @@ int bnb_conv_step_fwd(const void *b1, int b1_dtype,
                       const float *conv_in, int64_t conv_in_row_stride,
                       const float *weight, const float *bias,
                       const uint8_t *reset, int rows_per_env,
-                      float *v_out, float *conv_out, int64_t conv_out_row_stride,
+                      float *v_out, void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride,
                       int64_t R, int D, void *stream);
+
+/*
+ * Residual add + RMSNorm (+ the cast in front of the next projection) in one pass:
+ *     s = x + delta            (delta optional)
+ *     n = s * rsqrt(mean(s^2) + eps) * weight
+ * Replaces `x = x + <sublayer output>` followed by `self.norm*(x)` in
+ * models/yemong/attention.py:97-98 and models/yemong/griffin.py:269,284-285 (nn.RMSNorm(D),
+ * eps = finfo(float32).eps), and the fp32 -> bf16 copy autocast puts before the next Linear.
+ *
+ *   x         (R, D) fp32 residual stream, row r at x + r*x_row_stride
+ *   delta     optional (R, D) contiguous, delta_dtype (a bf16 Linear output under autocast)
+ *   weight    (D) fp32
+ *   sum_out   optional (R, D) fp32 contiguous: s (only with delta)
+ *   norm_out  (R, D) contiguous in out_dtype
+ * Requirements: D in {8,16,32,64,128,256,512}; 16-byte aligned pointers.
+ */
+int bnb_add_rmsnorm_fwd(const float *x, int64_t x_row_stride, const void *delta, int delta_dtype,
+                        const float *weight, float eps, float *sum_out, void *norm_out, int out_dtype,
+                        int64_t R, int D, void *stream);
+
+/*
+ * out = gelu(a) * b with the exact (erf) GELU, the gelu rounded to a's dtype as F.gelu does and
+ * the product rounded once to out_dtype.  Replaces `F.gelu(gate_proj(x)) * up_proj(x)`
+ * (models/yemong/attention.py:36-37) and `b1_out * F.gelu(linear2(normed))`
+ * (models/yemong/griffin.py:281-282).  a and b are (R, H) with row strides in elements (the
+ * two halves of one (R, 2H) projection output work), out is (R, H) contiguous.
+ * Requirements: H % 8 == 0; 16-byte aligned rows.
+ */
+int bnb_gelu_mul_fwd(const void *a, int a_dtype, int64_t a_row_stride, const void *b, int b_dtype,
+                     int64_t b_row_stride, void *out, int out_dtype, int64_t R, int H, void *stream);
 
 /*
  * Plain device-to-device copy of `bytes` bytes (multiple of 16, 16-byte aligned) by a

@@ -417,6 +417,62 @@ def test_conv_step_full_size_rows_sampled_against_formula():
     assert torch.equal(new_state[:, D:2 * D], state[:, 2 * D:3 * D])  # whole-tensor shift property
 
 
+# ------------------------------------------------------------------ fused norm and gelu-gate kernels
+
+
+@pytest.mark.parametrize("R,D", [(1, 128), (37, 128), (3000, 128), (9, 64), (5, 32), (4, 512), (6, 8)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_add_rmsnorm_matches_library_rms_norm(R, D, out_dtype):
+    g = torch.Generator().manual_seed(R * 7 + D)
+    x = 2.0 * torch.randn(R, D, generator=g)
+    w = 1.0 + 0.1 * torch.randn(D, generator=g)
+    delta = torch.randn(R, D, generator=g).bfloat16()
+    tol = F32_TOL if out_dtype == torch.float32 else 4e-3
+    # norm only: nn.RMSNorm(D) semantics (eps = finfo(float32).eps)
+    same, n = ops.add_rmsnorm(x.to(DEV), w.to(DEV), out_dtype=out_dtype)
+    assert same.data_ptr() != 0 and n.dtype == out_dtype
+    ref = torch.nn.functional.rms_norm(x, (D,), w, None)
+    assert max_rel(n.float().cpu(), ref) <= tol
+    assert torch.allclose(n.float().cpu(), ref.to(out_dtype).float(), rtol=1e-2 if out_dtype == torch.bfloat16 else 1e-5, atol=1e-5)
+    # add + norm: fp32 residual + bf16 branch output
+    s_, n2 = ops.add_rmsnorm(x.to(DEV), w.to(DEV), delta=delta.to(DEV), out_dtype=out_dtype)
+    ref_s = x + delta
+    assert torch.equal(s_.cpu(), ref_s)  # fp32 + bf16 -> fp32, one rounding: bit exact
+    assert max_rel(n2.float().cpu(), torch.nn.functional.rms_norm(ref_s, (D,), w, None)) <= tol
+
+
+def test_add_rmsnorm_keeps_leading_shape_and_rejects_uncovered_widths():
+    x = torch.randn(3, 5, 128, device=DEV)
+    w = torch.ones(128, device=DEV)
+    s_, n = ops.add_rmsnorm(x, w, delta=torch.zeros_like(x))
+    assert s_.shape == x.shape and n.shape == x.shape and torch.equal(s_, x)
+    with pytest.raises(ValueError):
+        ops.add_rmsnorm(torch.randn(2, 24, device=DEV), torch.ones(24, device=DEV))
+
+
+@pytest.mark.parametrize("adt,bdt,odt", [(torch.float32, torch.float32, torch.float32),
+                                         (torch.bfloat16, torch.bfloat16, torch.bfloat16),
+                                         (torch.bfloat16, torch.float32, torch.bfloat16)])
+@pytest.mark.parametrize("R,H", [(3, 512), (1000, 512), (7, 128), (5, 8)])
+def test_gelu_mul_matches_torch_with_its_rounding_points(adt, bdt, odt, R, H):
+    g = torch.Generator().manual_seed(R + H)
+    both = (2.0 * torch.randn(R, 2 * H, generator=g)).to(adt)
+    a = both[:, :H]  # the two halves of one projection output: row stride 2H
+    b = both[:, H:].to(bdt) if bdt == adt else torch.randn(R, H, generator=g).to(bdt)
+    dev_both = both.to(DEV)
+    dev_b = dev_both[:, H:] if bdt == adt else b.to(DEV)
+    out = ops.gelu_mul(dev_both[:, :H], dev_b, out_dtype=odt)
+    assert out.dtype == odt and out.is_contiguous()
+    ref = (torch.nn.functional.gelu(a) * b).to(odt)  # torch rounds gelu to a's dtype, then the product
+    truth = torch.nn.functional.gelu(a.double()) * b.double()
+    assert max_rel(out.float().cpu(), truth.float()) <= (F32_TOL if odt == torch.float32 else BF16_TOL)
+    if odt == torch.float32:
+        assert torch.allclose(out.cpu(), ref, rtol=1e-5, atol=2e-6)
+    else:
+        # identical rounding points: at most one bf16 ulp apart where erf rounding differs
+        assert (out.float().cpu() - ref.float()).abs().max() <= 2 ** -7 * ref.float().abs().max()
+
+
 # ------------------------------------------------------------------ the measured step
 
 
