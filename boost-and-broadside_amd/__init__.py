@@ -6,7 +6,7 @@ per-entity RG-LRU recurrence step, as hand-written HIP kernels behind a C ABI
 reference policy's layer interfaces and ``state_dict`` names.
 
     ops       sdpa_masked, rglru_step, conv_step             (the kernels)
-    trunk     TransformerBlock, RGLRU, GriffinTemporalBlock, YemongBlock, YemongTrunk
+    trunk     TransformerBlock, RGLRU, GriffinTemporalBlock, YemongBlock, YemongTrunk, GraphedTrunk
     harness   benchmark workloads, traffic model, AttnRglruStep
     build     compiles the HIP sources
 """
@@ -16,6 +16,7 @@ from .ops import conv_step, rglru_step, sdpa_masked
 from .trunk import (
     CONV_KERNEL,
     GatedMLP,
+    GraphedTrunk,
     GriffinTemporalBlock,
     ModelConfig,
     RGLRU,
@@ -25,6 +26,6 @@ from .trunk import (
 )
 
 __all__ = [
-    "CONV_KERNEL", "GatedMLP", "GriffinTemporalBlock", "ModelConfig", "RGLRU", "TransformerBlock",
+    "CONV_KERNEL", "GatedMLP", "GraphedTrunk", "GriffinTemporalBlock", "ModelConfig", "RGLRU", "TransformerBlock",
     "YemongBlock", "YemongTrunk", "conv_step", "rglru_step", "sdpa_masked", "ops", "trunk", "harness",
 ]

@@ -521,3 +521,81 @@ class YemongTrunk(nn.Module):
             x = block.step_packed(x, alive_mask, recurrent_state[sl], out_state[sl], n_rec, reset_mask, bullets,
                                   bullet_mask)
         return x, out_state
+
+
+class GraphedTrunk:
+    """``YemongTrunk.forward`` for one fixed shape, captured into two HIP graphs and replayed.
+
+    At rollout scale of a few thousand tokens a trunk step is ~100 short launches and the
+    host, not the GPU, sets the pace (the reference notes the same of its own rollout).
+    Capturing the step removes that: ``step(tokens, alive_mask, reset_mask)`` copies the inputs
+    into static buffers, replays one graph and returns the static output and state tensors.
+    The packed state lives in two buffers that alternate as input and output, hence two
+    graphs.  Outputs are overwritten by the next ``step``; clone what must outlive it.
+
+    Args:
+        trunk: the module to capture (weights are read at replay time, so in-place weight
+            updates are seen; replacing parameter tensors requires a new capture).
+        num_envs, num_tokens, num_recurrent: B, N+M and n_rec of every later call.
+        autocast_dtype: ``torch.bfloat16`` to capture under autocast, None for fp32.
+        use_reset: capture with a ``reset_mask`` input (all-False masks are then cheap no-ops).
+    """
+
+    def __init__(self, trunk: YemongTrunk, num_envs: int, num_tokens: int, num_recurrent: int, *,
+                 autocast_dtype: torch.dtype | None = None, use_reset: bool = True, device=None) -> None:
+        dev = torch.device(device) if device is not None else next(trunk.parameters()).device
+        D = trunk.config.d_model
+        self.trunk, self.autocast_dtype = trunk, autocast_dtype
+        self.tokens = torch.zeros(num_envs, num_tokens, D, device=dev)
+        self.alive = torch.ones(num_envs, num_tokens, dtype=torch.bool, device=dev)
+        self.reset = torch.zeros(num_envs, dtype=torch.bool, device=dev) if use_reset else None
+        self.states = [trunk.initial_hidden(num_envs, num_recurrent, dev) for _ in range(2)]
+        self.cur = 0  # index of the buffer holding the current state
+        self.graphs, self.outputs = [], []
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):
+            for _ in range(3):  # warm-up outside capture: weight caches, GEMM heuristics, code loading
+                self._run(0)
+                self._run(1)
+        torch.cuda.current_stream(dev).wait_stream(side)
+        torch.cuda.synchronize(dev)
+        for src in (0, 1):
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                out = self._run(src)
+            self.graphs.append(graph)
+            self.outputs.append(out)
+        for s in self.states:
+            s.zero_()
+
+    def _run(self, src: int) -> torch.Tensor:
+        with torch.autocast("cuda", dtype=self.autocast_dtype or torch.bfloat16, enabled=self.autocast_dtype is not None):
+            out, _ = self.trunk(self.tokens, self.alive, self.states[src], reset_mask=self.reset,
+                                out_state=self.states[1 - src])
+        return out
+
+    @property
+    def state(self) -> torch.Tensor:
+        """The current packed recurrent state (a static buffer)."""
+        return self.states[self.cur]
+
+    def load_state(self, state: torch.Tensor) -> None:
+        self.states[self.cur].copy_(state)
+
+    @torch.no_grad()
+    def step(self, tokens, alive_mask, reset_mask=None):
+        """One trunk step on the captured shape; returns (hidden, new_state) static tensors."""
+        self.tokens.copy_(tokens)
+        self.alive.copy_(alive_mask)
+        if self.reset is not None:
+            if reset_mask is None:
+                self.reset.fill_(False)
+            else:
+                self.reset.copy_(reset_mask)
+        elif reset_mask is not None:
+            raise ValueError("this capture was made without a reset input")
+        self.graphs[self.cur].replay()
+        out = self.outputs[self.cur]
+        self.cur = 1 - self.cur
+        return out, self.states[self.cur]

@@ -345,3 +345,29 @@ def test_trunk_folded_reset_equals_reset_then_step_and_leaves_input_state_alone(
     assert state_c.data_ptr() == dest.data_ptr() and torch.equal(dest, state_a)
     with pytest.raises(ValueError):
         trunk(x.to(DEV), alive.to(DEV), dev_hidden, out_state=dev_hidden)
+
+
+@pytest.mark.parametrize("autocast_dtype", [None, torch.bfloat16])
+def test_graphed_trunk_replays_match_eager_steps(autocast_dtype):
+    # every replay is checked against the eager step, with eager work and synchronisations in between
+    D, H, B, N, M = 128, 4, 32, 8, 4
+    p = trunk_params(41, D, 2, 2, 1)
+    trunk = bnb.YemongTrunk(_cfg(D, H, 2, 2, 1)).eval()
+    trunk.load_state_dict(p)
+    trunk.to(DEV)
+    graphed = bnb.GraphedTrunk(trunk, B, N + M, N, autocast_dtype=autocast_dtype)
+    gen = torch.Generator().manual_seed(41)
+    eager_state = trunk.initial_hidden(B, N, DEV)
+    alive = torch.ones(B, N + M, dtype=torch.bool)
+    for t in range(6):
+        x = torch.randn(B, N + M, D, generator=gen).to(DEV)
+        alive[:, :N] &= torch.rand(B, N, generator=gen) > 0.1
+        done = torch.rand(B, generator=gen) < 0.2 if t in (2, 4) else None
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast_dtype is not None):
+            ref_out, eager_state = trunk(x, alive.to(DEV), eager_state,
+                                         reset_mask=None if done is None else done.to(DEV))
+        torch.cuda.synchronize()
+        out, state = graphed.step(x, alive.to(DEV), None if done is None else done.to(DEV))
+        assert torch.equal(out, ref_out), t
+        assert torch.equal(state, eager_state), t
+        assert state.data_ptr() == graphed.state.data_ptr()
