@@ -199,10 +199,18 @@ constexpr int kKeyPitch = kDh + 8;  // halfs per K row in LDS: 80 bytes, 16-byte
 
 // One work-group per (environment, head); wave w owns queries 32w .. 32w+31 and all waves
 // share the K rows and the transposed V rows of the live keys in LDS.
-template <int NKB>
+//
+// The same kernel serves self-attention over the entity tokens (q, k, v are the three thirds
+// of one packed buffer, NQ == NK) and, with CROSS, the read of bullet key/values by the entity
+// queries (models/yemong/attention.py:149-166): keys and values come from a second buffer,
+// an environment without any live key contributes nothing (the reference gates it off
+// instead of letting the uniform average through), and the result is added to `accum`.
+// NKB = key blocks and waves of the work-group: max(ceil(NK/32), ceil(NQ/32)).
+template <int NKB, bool CROSS>
 __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
-    const uint16_t *__restrict__ qkv, int64_t row_stride, const uint8_t *__restrict__ alive,
-    uint16_t *__restrict__ out, int B, int NM, int H, float scale_log2e)
+    const uint16_t *__restrict__ q, int64_t q_stride, const uint16_t *__restrict__ k,
+    const uint16_t *__restrict__ v, int64_t kv_stride, const uint8_t *__restrict__ alive,
+    const uint16_t *accum, uint16_t *out, int B, int NQ, int NK, int H, float scale_log2e)
 {
     constexpr int KCAP = NKB * 32;
     constexpr int VP = KCAP + 4;  // halfs per V^T row: 8-byte aligned, bank-spread
@@ -226,13 +234,13 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
     const int m = lane & 31;
     const int half = lane >> 5;
 
-    const uint16_t *env_base = qkv + (int64_t)env * NM * row_stride;
+    const uint16_t *q_base = q + (int64_t)env * NQ * q_stride;
 
     // ---- this wave's queries (loaded together with the K/V rows, after the alive bytes: the
     //      alive row is tiny and usually an L2 hit, and nothing else can start before it) ----
     const int qrow = wave * 32 + m;
-    const int qsafe = qrow < NM ? qrow : NM - 1;
-    const uint16_t *qp = env_base + (uint32_t)qsafe * (uint32_t)row_stride + (uint32_t)(head * kDh + half * 8);
+    const int qsafe = qrow < NQ ? qrow : NQ - 1;
+    const uint16_t *qp = q_base + (uint32_t)qsafe * (uint32_t)q_stride + (uint32_t)(head * kDh + half * 8);
     u32x4 qw0 = {0u, 0u, 0u, 0u}, qw1 = {0u, 0u, 0u, 0u};
 
     // ---- K rows and V^T of the live keys into LDS, compacted ----
@@ -240,7 +248,7 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
     // byte, starts its K/V loads at once if the key is live, and only then works out the
     // key's position among the live keys (ballot inside the wave, per-wave counts through
     // LDS), so the position arithmetic overlaps the loads.
-    const uint8_t *alive_env = alive == nullptr ? nullptr : alive + (int64_t)env * NM;
+    const uint8_t *alive_env = alive == nullptr ? nullptr : alive + (int64_t)env * NK;
     int cnt = 0;
     bool uniform = false;
     for (int pass = 0; pass < 2; ++pass) {
@@ -254,18 +262,20 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
 #pragma unroll
             for (int it = 0; it < 2; ++it) {
                 const int key = (tid + it * NT) >> 2;
-                ab[it] = alive_env[key < NM ? key : NM - 1];
+                ab[it] = alive_env[key < NK ? key : NK - 1];
             }
         }
-        const uint32_t stride32 = (uint32_t)row_stride;
-        const uint16_t *kv_base = env_base + D + head * kDh + (tid & 3) * 8;
+        const uint32_t stride32 = (uint32_t)kv_stride;
+        const int64_t kv_env = (int64_t)env * NK * kv_stride + head * kDh + (tid & 3) * 8;
+        const uint16_t *k_base = k + kv_env;
+        const uint16_t *v_base = v + kv_env;
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
             const int key = (tid + it * NT) >> 2;
-            live[it] = key < NM && ab[it] != 0;
+            live[it] = key < NK && ab[it] != 0;
             const uint32_t off = (live[it] ? (uint32_t)key : 0u) * stride32;
-            kw[it] = *reinterpret_cast<const u32x4 *>(kv_base + off);
-            vw[it] = *reinterpret_cast<const u32x4 *>(kv_base + off + D);
+            kw[it] = *reinterpret_cast<const u32x4 *>(k_base + off);
+            vw[it] = *reinterpret_cast<const u32x4 *>(v_base + off);
         }
         if (pass == 0) {
             qw0 = *reinterpret_cast<const u32x4 *>(qp);
@@ -307,7 +317,7 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
                 dst[11 * VP] = (uint16_t)(vw[it].w >> 16);
             }
         }
-        if (cnt != 0) break;
+        if (cnt != 0 || CROSS) break;
         // no live key at all: every key takes part with the same weight; stage them all
         uniform = true;
         __syncthreads();  // s_cnt is rewritten by the second pass
@@ -322,6 +332,7 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
         for (int e = 0; e < 8; ++e) s_vt[(c8 + e) * VP + pos] = 0;
     }
     __syncthreads();
+    if (wave * 32 >= NQ) return;  // waves that only helped staging (more key blocks than query blocks)
 
     // ---- S^T = K Q^T for this wave's 32 queries ----
     // With no live key every score is the same constant: zero queries give exactly that.
@@ -379,22 +390,30 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
         }
     }
     sum += __shfl_xor(sum, 32);
-    const float inv = __builtin_amdgcn_rcpf(sum);
+    // CROSS with no live key: nkb == 0, o == 0 and the contribution is exactly zero
+    const float inv = (CROSS && cnt == 0) ? 0.0f : __builtin_amdgcn_rcpf(sum);
 
     // The MFMA leaves a lane with rows 8i + 4*half + j (i, j = 0..3) of O^T.  V^T was stored
     // with its rows permuted so that MFMA row 8i + 4*half + j is channel
     // 16*(i/2) + 8*half + 4*(i%2) + j: the lane then owns two runs of 8 consecutive channels
     // and stores 16 bytes at a time, lanes m and m+32 side by side (32 contiguous bytes per
     // row and store instruction instead of scattered 8-byte pieces).
-    if (qrow < NM) {
-        uint16_t *op = out + ((int64_t)env * NM + qrow) * D + head * kDh + 8 * half;
+    if (qrow < NQ) {
+        const int64_t o_off = ((int64_t)env * NQ + qrow) * D + head * kDh + 8 * half;
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
-            const u32x4 w = {pack_bf16x2(o[8 * g + 0] * inv, o[8 * g + 1] * inv),
-                             pack_bf16x2(o[8 * g + 2] * inv, o[8 * g + 3] * inv),
-                             pack_bf16x2(o[8 * g + 4] * inv, o[8 * g + 5] * inv),
-                             pack_bf16x2(o[8 * g + 6] * inv, o[8 * g + 7] * inv)};
-            *reinterpret_cast<u32x4 *>(op + 16 * g) = w;
+            float r[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) r[e] = o[8 * g + e] * inv;
+            if (CROSS && accum != nullptr) {
+                // bf16 + bf16 as torch adds them: the read result is rounded first, then the sum
+                const Row8 a = load8(accum + o_off + 16 * g);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) r[e] = a.v[e] + round_to_bf16(r[e]);
+            }
+            const u32x4 w = {pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3]), pack_bf16x2(r[4], r[5]),
+                             pack_bf16x2(r[6], r[7])};
+            *reinterpret_cast<u32x4 *>(out + o_off + 16 * g) = w;
         }
     }
 }
@@ -456,28 +475,33 @@ static int dispatch_valu(const void *qkv, int64_t row_stride, const uint8_t *ali
     }
 }
 
-template <int NKB>
-static int launch_mfma(const void *qkv, int64_t row_stride, const uint8_t *alive, void *out, int B, int NM,
-                       int H, hipStream_t stream)
+template <int NKB, bool CROSS>
+static int launch_mfma(const void *q, int64_t q_stride, const void *k, const void *v, int64_t kv_stride,
+                       const uint8_t *alive, const void *accum, void *out, int B, int NQ, int NK, int H,
+                       hipStream_t stream)
 {
     const int64_t pairs = (int64_t)B * H;
     const int64_t blocks = (pairs + 7) / 8 * 8;
     if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
     const float scale_log2e = kLog2eA / sqrtf((float)kDh);
-    hipLaunchKernelGGL((sdpa_mfma_kernel<NKB>), dim3((unsigned)blocks), dim3(kWave * NKB), 0, stream,
-                       (const uint16_t *)qkv, row_stride, alive, (uint16_t *)out, B, NM, H, scale_log2e);
+    hipLaunchKernelGGL((sdpa_mfma_kernel<NKB, CROSS>), dim3((unsigned)blocks), dim3(kWave * NKB), 0, stream,
+                       (const uint16_t *)q, q_stride, (const uint16_t *)k, (const uint16_t *)v, kv_stride, alive,
+                       (const uint16_t *)accum, (uint16_t *)out, B, NQ, NK, H, scale_log2e);
     return (int)hipGetLastError();
 }
 
-static int dispatch_mfma(const void *qkv, int64_t row_stride, const uint8_t *alive, void *out, int B, int NM,
-                         int H, hipStream_t stream)
+template <bool CROSS>
+static int dispatch_mfma(const void *q, int64_t q_stride, const void *k, const void *v, int64_t kv_stride,
+                         const uint8_t *alive, const void *accum, void *out, int B, int NQ, int NK, int H,
+                         hipStream_t stream)
 {
-    switch ((NM + 31) / 32) {
-        case 1: return launch_mfma<1>(qkv, row_stride, alive, out, B, NM, H, stream);
-        case 2: return launch_mfma<2>(qkv, row_stride, alive, out, B, NM, H, stream);
-        case 3: return launch_mfma<3>(qkv, row_stride, alive, out, B, NM, H, stream);
-        case 4: return launch_mfma<4>(qkv, row_stride, alive, out, B, NM, H, stream);
-        case 5: return launch_mfma<5>(qkv, row_stride, alive, out, B, NM, H, stream);
+    const int blocks = ((NQ > NK ? NQ : NK) + 31) / 32;
+    switch (blocks) {
+        case 1: return launch_mfma<1, CROSS>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
+        case 2: return launch_mfma<2, CROSS>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
+        case 3: return launch_mfma<3, CROSS>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
+        case 4: return launch_mfma<4, CROSS>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
+        case 5: return launch_mfma<5, CROSS>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
         default: return BNB_ERR_UNSUPPORTED;
     }
 }
@@ -506,7 +530,12 @@ extern "C" int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride,
     // measured on MI355X the matrix-core kernel wins at every token count it covers, 4v4 included
     // (12 tokens: 24.7 us vs 45.5 us for 8192 environments), so AUTO takes it whenever it applies
     const bool use_mfma = path == BNB_SDPA_PATH_MFMA || (path == BNB_SDPA_PATH_AUTO && mfma_ok);
-    if (use_mfma) return dispatch_mfma(qkv, qkv_row_stride, alive, out, B, NM, H, s);
+    if (use_mfma) {
+        const uint16_t *base = (const uint16_t *)qkv;
+        const int D = H * dh;
+        return dispatch_mfma<false>(base, qkv_row_stride, base + D, base + 2 * D, qkv_row_stride, alive, nullptr, out,
+                                    B, NM, NM, H, s);
+    }
     if (dtype == BNB_BF16) return dispatch_valu<uint16_t>(qkv, qkv_row_stride, alive, out, B, NM, H, dh, s);
     return dispatch_valu<float>(qkv, qkv_row_stride, alive, out, B, NM, H, dh, s);
 }
@@ -516,4 +545,24 @@ extern "C" int bnb_sdpa_masked_fwd(const void *qkv, int64_t qkv_row_stride, cons
 {
     return bnb_sdpa_masked_fwd_path(qkv, qkv_row_stride, alive, out, B, NM, H, dh, dtype, BNB_SDPA_PATH_AUTO,
                                     stream);
+}
+
+extern "C" int bnb_sdpa_cross_fwd(const void *q, int64_t q_row_stride, int NQ, const void *k, const void *v,
+                                  int64_t kv_row_stride, int NK, const uint8_t *key_mask, const void *accum,
+                                  void *out, int B, int H, int dh, int dtype, void *stream)
+{
+    using namespace bnb;
+    if (B < 0 || NQ < 0 || NK < 0 || H < 1 || dh < 1) return BNB_ERR_BAD_SHAPE;
+    if (dtype != BNB_BF16 || dh != kDh || NQ > 160 || NK > 160) return BNB_ERR_UNSUPPORTED;
+    if (NK == 0) return BNB_ERR_UNSUPPORTED;  // nothing to read: the caller keeps `accum` as it is
+    if (B == 0 || NQ == 0) return 0;
+    if (!q || !out || !k || !v) return BNB_ERR_NULL_POINTER;
+    if (q_row_stride < (int64_t)H * dh || kv_row_stride < (int64_t)H * dh) return BNB_ERR_BAD_SHAPE;
+    if ((int64_t)NQ * q_row_stride >= (1LL << 30) || (int64_t)NK * kv_row_stride >= (1LL << 30))
+        return BNB_ERR_UNSUPPORTED;
+    if (!aligned16(q) || !aligned16(out) || (accum && !aligned16(accum)) || (q_row_stride * 2) % 16 != 0 ||
+        !aligned16(k) || !aligned16(v) || (kv_row_stride * 2) % 16 != 0)
+        return BNB_ERR_MISALIGNED;
+    return dispatch_mfma<true>(q, q_row_stride, k, v, kv_row_stride, key_mask, accum, out, B, NQ, NK, H,
+                               (hipStream_t)stream);
 }

@@ -101,6 +101,69 @@ def sdpa_masked(
     return out
 
 
+def cross_supported(q: torch.Tensor, kv: torch.Tensor, n_heads: int) -> bool:
+    """Whether ``sdpa_cross`` covers these shapes (bf16, head size 32, 1..160 keys, <= 160 queries)."""
+    D = kv.shape[-1] // 2
+    return (
+        q.is_cuda and q.dtype == torch.bfloat16 and kv.dtype == torch.bfloat16 and D % n_heads == 0
+        and D // n_heads == 32 and 1 <= kv.shape[1] <= 160 and q.shape[1] <= 160
+    )
+
+
+def sdpa_cross(
+    qkv: torch.Tensor,
+    kv: torch.Tensor,
+    key_mask: torch.Tensor | None,
+    n_heads: int,
+    *,
+    accum: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Entity queries reading a second key/value set (the bullet read), on the matrix-core kernel.
+
+    Args:
+        qkv:      (B, NQ, 3*D) packed entity projection; only its Q third is read.
+        kv:       (B, NK, 2*D) ``[K | V]`` of the other set (``kv_bullet``'s output).
+        key_mask: (B, NK) bool, True = active, or None.  Inactive keys get weight 0; an
+                  environment with no active key contributes exactly zero.
+        accum:    optional (B, NQ, D) contiguous tensor the result is added to (and written
+                  into); default: the bare result in a new tensor.
+
+    Returns (B, NQ, D) bfloat16.
+    """
+    B, NQ, D3 = qkv.shape
+    D = D3 // 3
+    NK = kv.shape[1]
+    if kv.shape != (B, NK, 2 * D):
+        raise ValueError(f"kv must be {(B, NK, 2 * D)}, got {tuple(kv.shape)}")
+    if not cross_supported(qkv, kv, n_heads):
+        raise RuntimeError("sdpa_cross covers bfloat16, head size 32, 1..160 keys and at most 160 queries")
+    if torch.is_grad_enabled() and (qkv.requires_grad or kv.requires_grad):
+        raise RuntimeError("sdpa_cross is forward-only; call it under torch.no_grad()")
+    if B and NQ and (qkv.stride(-1) != 1 or (B > 1 and qkv.stride(0) != NQ * qkv.stride(1))):
+        qkv = qkv.contiguous()
+    if B and (kv.stride(-1) != 1 or (B > 1 and kv.stride(0) != NK * kv.stride(1))):
+        kv = kv.contiguous()
+    mask_ptr = None
+    if key_mask is not None:
+        if key_mask.shape != (B, NK) or key_mask.dtype not in (torch.bool, torch.uint8):
+            raise ValueError(f"key_mask must be a bool {(B, NK)} tensor")
+        key_mask = key_mask.contiguous()
+        mask_ptr = key_mask.data_ptr()
+    if accum is not None and (accum.shape != (B, NQ, D) or accum.dtype != torch.bfloat16 or not accum.is_contiguous()):
+        raise ValueError("accum must be a contiguous bfloat16 (B, NQ, D) tensor")
+    out = accum if accum is not None else torch.empty((B, NQ, D), dtype=torch.bfloat16, device=qkv.device)
+    if B == 0 or NQ == 0:
+        return out
+    with torch.cuda.device(qkv.device):
+        rc = _native.load().bnb_sdpa_cross_fwd(
+            qkv.data_ptr(), qkv.stride(1), NQ, kv.data_ptr(), kv.data_ptr() + D * kv.element_size(), kv.stride(1), NK,
+            mask_ptr, None if accum is None else accum.data_ptr(), out.data_ptr(), B, n_heads, D // n_heads,
+            _native.BF16, _stream(),
+        )
+    _native.check(rc, "bnb_sdpa_cross_fwd")
+    return out
+
+
 def rglru_step(
     x: torch.Tensor,
     gates_pre: torch.Tensor,

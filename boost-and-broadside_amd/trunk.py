@@ -170,20 +170,29 @@ class TransformerBlock(nn.Module):
         qkv = _project(self.qkv, x)  # (B, N, 3D), fp32 or bf16 under autocast
         merged = ops.sdpa_masked(qkv, alive_mask, self.n_heads)  # (B, N, D) head-major
         if self.reads_bullets and bullets is not None:
-            merged = merged + self._bullet_read(qkv, bullets, bullet_mask)
+            kv = _project(self.kv_bullet, self._norm_bullets(bullets, qkv.dtype))
+            if ops.cross_supported(qkv, kv, self.n_heads):
+                merged = ops.sdpa_cross(qkv, kv, bullet_mask, self.n_heads, accum=merged)
+            else:
+                merged = merged + self._bullet_read(qkv, kv, bullet_mask)
         return _project(self.out_proj, merged)
 
-    def _bullet_read(self, qkv, bullets, bullet_mask):
-        """Cross-attention of the entity queries to bullet key/values (attention.py:149-166).
+    def _norm_bullets(self, bullets, act):
+        """norm_bullet(bullets) in the projection dtype."""
+        if _fused_ok(bullets, act):
+            return ops.add_rmsnorm(bullets, self.norm_bullet.weight, eps=self.norm_bullet.eps, out_dtype=act)[1]
+        n = self.norm_bullet(bullets)
+        return n if n.dtype == act else n.to(act)
 
-        Not one of the two kernels of this package: it goes through torch's SDPA on the
-        device, with the reference's additive bias and its all-inactive gate.
-        """
+    def _bullet_read(self, qkv, kv, bullet_mask):
+        """Cross-attention of the entity queries to bullet key/values (attention.py:149-166) for
+        the shapes the matrix-core kernel does not cover (fp32, more than 160 bullets, other
+        head sizes): torch's SDPA on the device, with the reference's additive bias and its
+        all-inactive gate.  ``kv`` is ``kv_bullet(norm_bullet(bullets))``."""
         B, N, _ = qkv.shape
         H, dh, D = self.n_heads, self.head_dim, self.d_model
-        NB = bullets.shape[1]
+        NB = kv.shape[1]
         q = qkv[..., :D].reshape(B, N, H, dh).transpose(1, 2)
-        kv = self.kv_bullet(self.norm_bullet(bullets))
         kb = kv[..., :D].reshape(B, NB, H, dh).transpose(1, 2)
         vb = kv[..., D:].reshape(B, NB, H, dh).transpose(1, 2)
         bias = None

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 3
+#define BNB_ABI_VERSION 4
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -86,6 +86,30 @@ int bnb_sdpa_masked_fwd(const void *qkv, int64_t qkv_row_stride, const uint8_t *
 #define BNB_SDPA_PATH_MFMA 2
 int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, void *out,
                              int B, int NM, int H, int dh, int dtype, int path, void *stream);
+
+/*
+ * Cross-attention of the entity queries to a second set of key/value rows (the bullet read),
+ * on the matrix-core kernel.
+ *
+ * Replaces, in models/yemong/attention.py:149-166: the head split of kb/vb (:152-153), the key
+ * bias (:154), F.scaled_dot_product_attention(q, kb, vb, attn_mask=bias) (:155-157), the
+ * `any_active` gate (:158-165: an environment without an active key contributes exactly 0
+ * instead of the uniform average) and `out = out + bullet_out` (:166).
+ *
+ *   q        (B, NQ, >= H*dh) rows of q_row_stride elements: the Q third of the packed
+ *            projection, heads head-major
+ *   k, v     (B, NK, >= H*dh) rows of kv_row_stride elements each (the two halves of
+ *            kv_bullet's output work: v = k + H*dh)
+ *   key_mask (B, NK) bytes, non-zero = active; NULL = all active
+ *   accum    optional (B, NQ, H*dh) contiguous: the self-attention output to add to (bf16
+ *            addition as torch performs it); may equal out
+ *   out      (B, NQ, H*dh) contiguous
+ * Requirements: dtype BNB_BF16, dh == 32, 1 <= NK <= 160, NQ <= 160, 16-byte aligned rows;
+ * anything else returns BNB_ERR_UNSUPPORTED and the caller keeps its library path.
+ */
+int bnb_sdpa_cross_fwd(const void *q, int64_t q_row_stride, int NQ, const void *k, const void *v,
+                       int64_t kv_row_stride, int NK, const uint8_t *key_mask, const void *accum,
+                       void *out, int B, int H, int dh, int dtype, void *stream);
 
 /*
  * One RG-LRU recurrence step over R = B*n_rec entity rows of D channels.

@@ -69,6 +69,28 @@ def sdpa_masked(qkv: torch.Tensor, alive: torch.Tensor | None, n_heads: int) -> 
     return o.transpose(1, 2).reshape(B, NM, D)
 
 
+def bullet_read(qkv: torch.Tensor, kv: torch.Tensor, bullet_mask: torch.Tensor | None, n_heads: int) -> torch.Tensor:
+    """Cross-attention of the entity queries to bullet key/values, merged head-major.
+
+    ``qkv`` (B, N, 3D) is the entity projection (only its Q third is used), ``kv`` (B, NB, 2D)
+    is ``kv_bullet(norm_bullet(bullets))`` = [K | V].  Inactive bullets get the additive
+    finfo.min/2 bias; an environment with no active bullet is gated to exactly zero instead of
+    the uniform average the bias alone would give.  Follows models/yemong/attention.py:149-165.
+    """
+    B, N, D3 = qkv.shape
+    D = D3 // 3
+    dh = D // n_heads
+    NB = kv.shape[1]
+    q = qkv[..., :D].reshape(B, N, n_heads, dh).transpose(1, 2)
+    kb = kv[..., :D].reshape(B, NB, n_heads, dh).transpose(1, 2)
+    vb = kv[..., D:].reshape(B, NB, n_heads, dh).transpose(1, 2)
+    bias = None if bullet_mask is None else key_bias(bullet_mask, q.dtype)
+    o = F.scaled_dot_product_attention(q, kb, vb, attn_mask=bias, dropout_p=0.0)
+    if bullet_mask is not None:
+        o = o * bullet_mask.any(dim=-1).reshape(B, 1, 1, 1).to(o.dtype)
+    return o.transpose(1, 2).reshape(B, N, D)
+
+
 def rglru_step(
     x: torch.Tensor,
     gates_pre: torch.Tensor,
@@ -106,10 +128,15 @@ def gated_mlp(p: dict, prefix: str, x: torch.Tensor) -> torch.Tensor:
     return F.linear(gate * F.linear(x, p[prefix + "up_proj.weight"]), p[prefix + "down_proj.weight"])
 
 
-def spatial_sublayer(p: dict, prefix: str, x: torch.Tensor, alive: torch.Tensor | None, n_heads: int) -> torch.Tensor:
-    """Pre-norm attention + FFN block without bullets; models/yemong/attention.py:76-99,114-169."""
+def spatial_sublayer(p: dict, prefix: str, x: torch.Tensor, alive: torch.Tensor | None, n_heads: int,
+                     bullets: torch.Tensor | None = None, bullet_mask: torch.Tensor | None = None) -> torch.Tensor:
+    """Pre-norm attention (+ optional bullet read) + FFN block; models/yemong/attention.py:76-99,114-169."""
     n = rms_norm(x, p[prefix + "norm1.weight"])
-    merged = sdpa_masked(F.linear(n, p[prefix + "qkv.weight"]), alive, n_heads)
+    qkv = F.linear(n, p[prefix + "qkv.weight"])
+    merged = sdpa_masked(qkv, alive, n_heads)
+    if bullets is not None and (prefix + "kv_bullet.weight") in p:
+        kv = F.linear(rms_norm(bullets, p[prefix + "norm_bullet.weight"]), p[prefix + "kv_bullet.weight"])
+        merged = merged + bullet_read(qkv, kv, bullet_mask, n_heads)
     x = x + F.linear(merged, p[prefix + "out_proj.weight"])
     return x + gated_mlp(p, prefix + "ffn.", rms_norm(x, p[prefix + "norm2.weight"]))
 

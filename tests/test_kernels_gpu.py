@@ -247,6 +247,45 @@ def test_sdpa_environment_permutation_is_bitwise_equivariant_at_full_size():
     assert max_rel(a[pick].float().cpu(), truth) <= BF16_TOL
 
 
+# ------------------------------------------------------------------ bullet read (cross-attention)
+
+
+@pytest.mark.parametrize("B,NQ,NK", [(4, 12, 80), (3, 20, 160), (5, 12, 7), (2, 84, 40), (3, 33, 33), (2, 160, 1)])
+def test_sdpa_cross_matches_oracle(B, NQ, NK):
+    H, D = 4, 128
+    g = torch.Generator().manual_seed(NQ * 200 + NK)
+    qkv = torch.randn(B, NQ, 3 * D, generator=g).bfloat16()
+    kv = torch.randn(B, NK, 2 * D, generator=g).bfloat16()
+    mask = torch.rand(B, NK, generator=g) < 0.5
+    mask[0] = False  # nothing active in env 0
+    mask[1, 0] = True
+    merged = torch.randn(B, NQ, D, generator=g).bfloat16()
+    truth = torch_ref.bullet_read(qkv.float(), kv.float(), mask, H)
+    bare = ops.sdpa_cross(qkv.to(DEV), kv.to(DEV), mask.to(DEV), H).float().cpu()
+    assert bare[0].abs().max() == 0  # gated off exactly
+    assert max_rel(bare, truth) <= BF16_TOL
+    acc = merged.to(DEV).clone()
+    out = ops.sdpa_cross(qkv.to(DEV), kv.to(DEV), mask.to(DEV), H, accum=acc)
+    assert out.data_ptr() == acc.data_ptr()
+    want = (merged + bare.bfloat16()).float()  # bf16 + bf16 as torch adds them
+    assert torch.equal(out.float().cpu(), want)
+    assert torch.equal(out[0].cpu(), merged[0])  # env 0 untouched
+    # inactive slots cannot influence the result
+    kv2 = kv.clone()
+    kv2[~mask] = kv2[~mask] * -2.0 + 9.0
+    assert torch.equal(ops.sdpa_cross(qkv.to(DEV), kv2.to(DEV), mask.to(DEV), H).float().cpu(), bare)
+    no_mask = ops.sdpa_cross(qkv.to(DEV), kv.to(DEV), None, H).float().cpu()
+    assert max_rel(no_mask, torch_ref.bullet_read(qkv.float(), kv.float(), None, H)) <= BF16_TOL
+
+
+def test_sdpa_cross_limits():
+    qkv = torch.zeros(1, 12, 384, device=DEV, dtype=torch.bfloat16)
+    assert not ops.cross_supported(qkv, torch.zeros(1, 161, 256, device=DEV, dtype=torch.bfloat16), 4)
+    assert not ops.cross_supported(qkv.float(), torch.zeros(1, 80, 256, device=DEV), 4)
+    with pytest.raises(RuntimeError):
+        ops.sdpa_cross(qkv, torch.zeros(1, 200, 256, device=DEV, dtype=torch.bfloat16), None, 4)
+
+
 # ------------------------------------------------------------------ RG-LRU step
 
 

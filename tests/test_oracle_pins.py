@@ -162,6 +162,32 @@ def test_mask_dtype_follows_query_dtype(monkeypatch):
     assert seen["q"] == torch.bfloat16 and seen["m"] == torch.bfloat16
 
 
+def test_bullet_read_is_masked_softmax_over_bullets_with_an_empty_gate():
+    # attention.py:149-165: separate softmax over bullet keys; all-inactive environment => exactly 0
+    B, N, NB, H, dh = 3, 4, 6, 2, 8
+    D = H * dh
+    g = torch.Generator().manual_seed(11)
+    qkv = torch.randn(B, N, 3 * D, generator=g)
+    kv = torch.randn(B, NB, 2 * D, generator=g)
+    mask = torch.tensor([[True, False, True, True, False, True], [False] * 6, [False, False, False, True, False, False]])
+    got = torch_ref.bullet_read(qkv, kv, mask, H)
+    assert got[1].abs().max() == 0  # nothing in flight: gated off, not a uniform average
+    assert torch.allclose(got[2], kv[2, 3, D:].expand(N, D), atol=1e-6)  # single active bullet: its V row
+    # fp64 loops: same definition as masked attention with Q from one buffer and K/V from the other
+    fake = torch.zeros(1, max(N, NB), 3 * D, dtype=torch.float64)
+    fake[0, :N, :D] = qkv[0, :, :D]
+    fake[0, :NB, D:] = kv[0]
+    alive = torch.zeros(1, max(N, NB), dtype=torch.bool)
+    alive[0, :NB] = mask[0]
+    brute = bruteforce.sdpa_masked_loops(fake.numpy(), alive.numpy(), H)[0, :N]
+    assert np.abs(got[0].double().numpy() - brute).max() < 5e-6
+    # inactive slots cannot influence anything (tests/models/test_encoder.py:700-720)
+    kv2 = kv.clone()
+    kv2[~mask] += 500.0
+    assert torch.equal(torch_ref.bullet_read(qkv, kv2, mask, H), got)
+    assert torch.allclose(torch_ref.bullet_read(qkv, kv, None, H), torch_ref.bullet_read(qkv, kv, torch.ones(B, NB, dtype=torch.bool), H))
+
+
 # ---------------------------------------------------------------- RG-LRU step
 
 

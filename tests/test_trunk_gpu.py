@@ -371,3 +371,26 @@ def test_graphed_trunk_replays_match_eager_steps(autocast_dtype):
         assert torch.equal(out, ref_out), t
         assert torch.equal(state, eager_state), t
         assert state.data_ptr() == graphed.state.data_ptr()
+
+
+@pytest.mark.parametrize("autocast", [False, True])
+def test_bullet_reading_block_matches_oracle(autocast):
+    # fp32 goes through the library SDPA path, bf16 autocast through the matrix-core cross kernel
+    D, H, B, N, NB = 128, 4, 4, 12, 80
+    gen = torch.Generator().manual_seed(17)
+    p = block_params(gen, "b.", D, 1, 0)
+    p["b.spatial.0.norm_bullet.weight"] = 1.0 + 0.1 * torch.randn(D, generator=gen)
+    p["b.spatial.0.kv_bullet.weight"] = 0.1 * torch.randn(2 * D, D, generator=gen)
+    layer = bnb.TransformerBlock(_cfg(D, H, spatial=1, bullets=1), reads_bullets=True).eval()
+    layer.load_state_dict(_strip(p, "b.spatial.0."))
+    layer.to(DEV)
+    x = torch.randn(B, N, D, generator=gen)
+    alive = torch.rand(B, N, generator=gen) < 0.8
+    alive[:, 0] = True
+    bullets = torch.randn(B, NB, D, generator=gen)
+    bmask = torch.rand(B, NB, generator=gen) < 0.3
+    bmask[0] = False
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+        got = layer(x.to(DEV), alive.to(DEV), bullets.to(DEV), bmask.to(DEV))
+    ref = torch_ref.spatial_sublayer(p, "b.spatial.0.", x, alive, H, bullets, bmask)
+    assert max_rel(got.float().cpu(), ref) <= (BF16_TOL if autocast else F32_TOL)
