@@ -419,6 +419,273 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
 }
 
 // ------------------------------------------------------------------------------------
+// Streaming MFMA kernel for the bullet read with many keys (bf16, dh = 32)
+// ------------------------------------------------------------------------------------
+//
+// The bullet axis is N*K slots long (80 .. 1520 in the shipped scenarios) and mostly
+// empty: only bullets in flight are keys.  One work-group per (environment, head), one
+// wave per 32 queries.  The work-group first compacts the indices of the live bullets
+// into LDS, then walks them in tiles of 32*NQB keys: the K rows and transposed V rows of
+// the next tile are gathered from global memory into registers while the matrix cores
+// work on the current tile out of LDS (two LDS buffers, one barrier per tile), with the
+// running maximum / sum / output of an online softmax carried across tiles.  Key
+// positions, operand layouts and the output stage are those of sdpa_mfma_kernel.
+
+constexpr int kStreamMaxKeys = 2048;
+
+template <int NQB>
+__global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
+    const uint16_t *__restrict__ q, int64_t q_stride, const uint16_t *__restrict__ k,
+    const uint16_t *__restrict__ v, int64_t kv_stride, const uint8_t *__restrict__ alive,
+    const uint16_t *accum, uint16_t *out, int B, int NQ, int NK, int H, float scale_log2e)
+{
+    constexpr int TK = 32 * NQB;  // keys per tile
+    constexpr int VP = TK + 4;    // halfs per V^T row: 8-byte aligned, bank-spread
+    constexpr int NT = kWave * NQB;
+    __shared__ __align__(16) uint16_t s_k[2][TK * kKeyPitch];
+    __shared__ __align__(16) uint16_t s_vt[2][kDh * VP];
+    __shared__ uint16_t s_idx[kStreamMaxKeys];  // indices of the live keys, ascending
+    __shared__ int s_wcnt[NQB];
+
+    const int chunk = gridDim.x >> 3;
+    const int logical = (blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
+    if (logical >= B * H) return;
+    const int env = logical / H;
+    const int head = logical - env * H;
+    const int D = H * kDh;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m = lane & 31;
+    const int half = lane >> 5;
+
+    // ---- live-key index list: wave w scans keys [w*J*64, (w+1)*J*64), 64 per ballot ----
+    const uint8_t *alive_env = alive == nullptr ? nullptr : alive + (int64_t)env * NK;
+    const int J = (NK + NT - 1) / NT;  // <= 32 because NK <= kStreamMaxKeys
+    const int key0 = wave * J * 64 + lane;
+    uint32_t bits = 0;
+    int mine = 0;
+    for (int j0 = 0; j0 < J; j0 += 8) {
+        // eight independent byte loads in flight, then their ballots
+        uint32_t a[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int key = key0 + (j0 + u) * 64;
+            const bool in = j0 + u < J && key < NK;
+            a[u] = 1u;
+            if (alive_env != nullptr) a[u] = alive_env[key < NK ? key : NK - 1];  // branch-free: no wait between the loads
+            a[u] = in ? a[u] : 0u;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const bool on = a[u] != 0;
+            bits |= (on ? 1u : 0u) << ((j0 + u) & 31);
+            mine += (int)__popcll(__ballot(on));
+        }
+    }
+    if (lane == 0) s_wcnt[wave] = mine;
+
+    // this wave's queries, in flight while the index list is built
+    const int qrow = wave * 32 + m;
+    const int qsafe = qrow < NQ ? qrow : NQ - 1;
+    const uint16_t *qp = q + (int64_t)env * NQ * q_stride + (uint32_t)qsafe * (uint32_t)q_stride +
+                         (uint32_t)(head * kDh + half * 8);
+    const u32x4 qw0 = *reinterpret_cast<const u32x4 *>(qp);
+    const u32x4 qw1 = *reinterpret_cast<const u32x4 *>(qp + 16);
+
+    __syncthreads();
+    int base = 0, cnt = 0;
+#pragma unroll
+    for (int w = 0; w < NQB; ++w) {
+        const int c = s_wcnt[w];
+        if (w < wave) base += c;
+        cnt += c;
+    }
+    // nothing in flight in this environment: the read contributes exactly zero
+    if (cnt == 0 && accum == out) return;
+    for (int j = 0; j < J; ++j) {
+        const bool a = (bits >> j) & 1u;
+        const uint64_t mask = __ballot(a);
+        if (a) s_idx[base + (int)__popcll(mask & ((1ull << lane) - 1ull))] = (uint16_t)(key0 + j * 64);
+        base += (int)__popcll(mask);
+    }
+    __syncthreads();
+
+    const int nkb = (cnt + 31) >> 5;
+    const int pad = nkb * 32 - cnt;  // positions [0, pad) of the first key block hold no key
+    const int ntiles = (nkb + NQB - 1) / NQB;
+
+    // thread -> (position in tile, 8 channels), two items per thread
+    const uint32_t stride32 = (uint32_t)kv_stride;
+    const int64_t kv_env = (int64_t)env * NK * kv_stride + head * kDh + (tid & 3) * 8;
+    const uint16_t *k_base = k + kv_env;
+    const uint16_t *v_base = v + kv_env;
+    u32x4 kw[2], vw[2];
+    auto gather = [&](int t) {
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int li = t * TK + ((tid + it * NT) >> 2) - pad;  // index among the live keys
+            const uint32_t key = s_idx[(li >= 0 && li < cnt) ? li : 0];
+            kw[it] = *reinterpret_cast<const u32x4 *>(k_base + key * stride32);
+            vw[it] = *reinterpret_cast<const u32x4 *>(v_base + key * stride32);
+        }
+    };
+    auto stash = [&](int t, int buf) {
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int lp = (tid + it * NT) >> 2;
+            const int li = t * TK + lp - pad;
+            if (li < cnt) {
+                const u32x4 zero4 = {0u, 0u, 0u, 0u};
+                const u32x4 kk = li >= 0 ? kw[it] : zero4;  // padding: zero K and V rows
+                const u32x4 vv = li >= 0 ? vw[it] : zero4;
+                const int c8 = (tid & 3) * 8;
+                *reinterpret_cast<u32x4 *>(&s_k[buf][lp * kKeyPitch + c8]) = kk;
+                uint16_t *dst = &s_vt[buf][(16 * (c8 >> 4) + 4 * ((c8 >> 3) & 1)) * VP + lp];
+                dst[0 * VP] = (uint16_t)(vv.x & 0xffffu);
+                dst[1 * VP] = (uint16_t)(vv.x >> 16);
+                dst[2 * VP] = (uint16_t)(vv.y & 0xffffu);
+                dst[3 * VP] = (uint16_t)(vv.y >> 16);
+                dst[8 * VP] = (uint16_t)(vv.z & 0xffffu);
+                dst[9 * VP] = (uint16_t)(vv.z >> 16);
+                dst[10 * VP] = (uint16_t)(vv.w & 0xffffu);
+                dst[11 * VP] = (uint16_t)(vv.w >> 16);
+            }
+        }
+    };
+
+    const bf16x8 qb0 = __builtin_bit_cast(bf16x8, qw0);
+    const bf16x8 qb1 = __builtin_bit_cast(bf16x8, qw1);
+    float mx = -INFINITY, sum = 0.0f;
+    f32x16 o = {0.0f};
+
+    // the rows this lane will add its result to, fetched while the first tile is gathered
+    const int64_t o_off = ((int64_t)env * NQ + qsafe) * D + head * kDh + 8 * half;
+    u32x4 acc0 = {0u, 0u, 0u, 0u}, acc1 = {0u, 0u, 0u, 0u};
+    if (accum != nullptr) {
+        acc0 = *reinterpret_cast<const u32x4 *>(accum + o_off);
+        acc1 = *reinterpret_cast<const u32x4 *>(accum + o_off + 16);
+    }
+    if (ntiles > 0) {
+        gather(0);
+        stash(0, 0);
+    }
+    // Every load issued so far has to be back before the loop: otherwise the compiler guards
+    // the first use of the query registers inside the loop with a wait for ALL outstanding
+    // loads, and that wait would also stall every iteration on the next tile's gather.
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), expcnt/lgkmcnt untouched
+    __syncthreads();
+    for (int t = 0; t < ntiles; ++t) {
+        const int buf = t & 1;
+        if (t + 1 < ntiles) gather(t + 1);
+        int nb = nkb - t * NQB;
+        nb = nb < NQB ? nb : NQB;
+        // K Q^T of key block kb.  Only the very first key block can hold padding positions; they
+        // get -inf there.  The empty asm keeps that rare fix-up a real branch: folded into
+        // selects it would cost 16 extra instructions in every key block.
+        auto scores = [&](int kb) -> f32x16 {
+            const uint16_t *kp = &s_k[buf][(kb * 32 + m) * kKeyPitch + half * 8];
+            const bf16x8 ka0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp));
+            const bf16x8 ka1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + 16));
+            f32x16 z = {0.0f};
+            z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0, qb0, z, 0, 0, 0);
+            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka1, qb1, z, 0, 0, 0);
+        };
+        auto mask_padding = [&](f32x16 &z) {
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                if (8 * (e >> 2) + 4 * half + (e & 3) < pad) z[e] = -INFINITY;
+        };
+        auto weigh = [&](int kb, const f32x16 &z, float mc) {
+            float p[16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                p[e] = __builtin_amdgcn_exp2f(fmaf(z[e], scale_log2e, -mc));
+                sum += p[e];
+            }
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2) {
+                bf16x8 pb;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * h2 + e];
+                const uint16_t *vp = &s_vt[buf][m * VP + kb * 32 + 16 * h2 + 4 * half];
+                const u32x2 lo = *reinterpret_cast<const u32x2 *>(vp);
+                const u32x2 hi = *reinterpret_cast<const u32x2 *>(vp + 8);
+                const u32x4 vq = {lo.x, lo.y, hi.x, hi.y};
+                o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vq), pb, o, 0, 0, 0);
+            }
+        };
+        if (wave * 32 < NQ) {
+            // two key blocks per iteration: two independent MFMA chains in flight
+            float tmx = -INFINITY;
+            int kb = 0;
+            for (; kb + 1 < nb; kb += 2) {
+                f32x16 z0 = scores(kb);
+                const f32x16 z1 = scores(kb + 1);
+                if (t == 0 && kb == 0 && pad != 0) mask_padding(z0);
+#pragma unroll
+                for (int e = 0; e < 16; ++e) tmx = fmaxf(tmx, fmaxf(z0[e], z1[e]));
+            }
+            if (kb < nb) {
+                f32x16 z0 = scores(kb);
+                if (t == 0 && kb == 0 && pad != 0) mask_padding(z0);
+#pragma unroll
+                for (int e = 0; e < 16; ++e) tmx = fmaxf(tmx, z0[e]);
+            }
+            tmx = fmaxf(tmx, __shfl_xor(tmx, 32));
+            const float mnew = fmaxf(mx, tmx);  // finite: every key block holds at least one live key
+            const float alpha = __builtin_amdgcn_exp2f((mx - mnew) * scale_log2e);
+            mx = mnew;
+            sum *= alpha;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[e] *= alpha;
+            const float mc = mx * scale_log2e;
+            kb = 0;
+            for (; kb + 1 < nb; kb += 2) {
+                f32x16 z0 = scores(kb);
+                const f32x16 z1 = scores(kb + 1);
+                if (t == 0 && kb == 0 && pad != 0) mask_padding(z0);
+                weigh(kb, z0, mc);
+                weigh(kb + 1, z1, mc);
+            }
+            if (kb < nb) {
+                f32x16 z0 = scores(kb);
+                if (t == 0 && kb == 0 && pad != 0) mask_padding(z0);
+                weigh(kb, z0, mc);
+            }
+        }
+        if (t + 1 < ntiles) stash(t + 1, buf ^ 1);
+        __syncthreads();
+    }
+    sum += __shfl_xor(sum, 32);
+    const float inv = cnt == 0 ? 0.0f : __builtin_amdgcn_rcpf(sum);
+
+    if (qrow < NQ) {
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+            float r[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) r[e] = o[8 * g + e] * inv;
+            if (accum != nullptr) {
+                // bf16 + bf16 as torch adds them: the read result is rounded first, then the sum
+                const u32x4 aw = g ? acc1 : acc0;
+                const uint32_t a2[4] = {aw.x, aw.y, aw.z, aw.w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float a = __uint_as_float((e & 1) ? (a2[e >> 1] & 0xffff0000u) : (a2[e >> 1] << 16));
+                    r[e] = a + round_to_bf16(r[e]);
+                }
+            }
+            const u32x4 w = {pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3]), pack_bf16x2(r[4], r[5]),
+                             pack_bf16x2(r[6], r[7])};
+            *reinterpret_cast<u32x4 *>(out + o_off + 16 * g) = w;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------
 
@@ -506,6 +773,35 @@ static int dispatch_mfma(const void *q, int64_t q_stride, const void *k, const v
     }
 }
 
+template <int NQB>
+static int launch_cross_stream(const void *q, int64_t q_stride, const void *k, const void *v, int64_t kv_stride,
+                               const uint8_t *alive, const void *accum, void *out, int B, int NQ, int NK, int H,
+                               hipStream_t stream)
+{
+    const int64_t pairs = (int64_t)B * H;
+    const int64_t blocks = (pairs + 7) / 8 * 8;
+    if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+    const float scale_log2e = kLog2eA / sqrtf((float)kDh);
+    hipLaunchKernelGGL((sdpa_cross_stream_kernel<NQB>), dim3((unsigned)blocks), dim3(kWave * NQB), 0, stream,
+                       (const uint16_t *)q, q_stride, (const uint16_t *)k, (const uint16_t *)v, kv_stride, alive,
+                       (const uint16_t *)accum, (uint16_t *)out, B, NQ, NK, H, scale_log2e);
+    return (int)hipGetLastError();
+}
+
+static int dispatch_cross_stream(const void *q, int64_t q_stride, const void *k, const void *v, int64_t kv_stride,
+                                 const uint8_t *alive, const void *accum, void *out, int B, int NQ, int NK, int H,
+                                 hipStream_t stream)
+{
+    switch ((NQ + 31) / 32) {
+        case 1: return launch_cross_stream<1>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
+        case 2: return launch_cross_stream<2>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
+        case 3: return launch_cross_stream<3>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
+        case 4: return launch_cross_stream<4>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
+        case 5: return launch_cross_stream<5>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
+        default: return BNB_ERR_UNSUPPORTED;
+    }
+}
+
 }  // namespace bnb
 
 extern "C" int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive,
@@ -553,7 +849,7 @@ extern "C" int bnb_sdpa_cross_fwd(const void *q, int64_t q_row_stride, int NQ, c
 {
     using namespace bnb;
     if (B < 0 || NQ < 0 || NK < 0 || H < 1 || dh < 1) return BNB_ERR_BAD_SHAPE;
-    if (dtype != BNB_BF16 || dh != kDh || NQ > 160 || NK > 160) return BNB_ERR_UNSUPPORTED;
+    if (dtype != BNB_BF16 || dh != kDh || NQ > 160 || NK > kStreamMaxKeys) return BNB_ERR_UNSUPPORTED;
     if (NK == 0) return BNB_ERR_UNSUPPORTED;  // nothing to read: the caller keeps `accum` as it is
     if (B == 0 || NQ == 0) return 0;
     if (!q || !out || !k || !v) return BNB_ERR_NULL_POINTER;
@@ -563,6 +859,9 @@ extern "C" int bnb_sdpa_cross_fwd(const void *q, int64_t q_row_stride, int NQ, c
     if (!aligned16(q) || !aligned16(out) || (accum && !aligned16(accum)) || (q_row_stride * 2) % 16 != 0 ||
         !aligned16(k) || !aligned16(v) || (kv_row_stride * 2) % 16 != 0)
         return BNB_ERR_MISALIGNED;
+    if (NK > 160)
+        return dispatch_cross_stream(q, q_row_stride, k, v, kv_row_stride, key_mask, accum, out, B, NQ, NK, H,
+                                     (hipStream_t)stream);
     return dispatch_mfma<true>(q, q_row_stride, k, v, kv_row_stride, key_mask, accum, out, B, NQ, NK, H,
                                (hipStream_t)stream);
 }

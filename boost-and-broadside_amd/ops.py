@@ -102,11 +102,11 @@ def sdpa_masked(
 
 
 def cross_supported(q: torch.Tensor, kv: torch.Tensor, n_heads: int) -> bool:
-    """Whether ``sdpa_cross`` covers these shapes (bf16, head size 32, 1..160 keys, <= 160 queries)."""
+    """Whether ``sdpa_cross`` covers these shapes (bf16, head size 32, 1..2048 keys, <= 160 queries)."""
     D = kv.shape[-1] // 2
     return (
         q.is_cuda and q.dtype == torch.bfloat16 and kv.dtype == torch.bfloat16 and D % n_heads == 0
-        and D // n_heads == 32 and 1 <= kv.shape[1] <= 160 and q.shape[1] <= 160
+        and D // n_heads == 32 and 1 <= kv.shape[1] <= 2048 and q.shape[1] <= 160
     )
 
 
@@ -117,6 +117,7 @@ def sdpa_cross(
     n_heads: int,
     *,
     accum: torch.Tensor | None = None,
+    out: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Entity queries reading a second key/value set (the bullet read), on the matrix-core kernel.
 
@@ -125,8 +126,9 @@ def sdpa_cross(
         kv:       (B, NK, 2*D) ``[K | V]`` of the other set (``kv_bullet``'s output).
         key_mask: (B, NK) bool, True = active, or None.  Inactive keys get weight 0; an
                   environment with no active key contributes exactly zero.
-        accum:    optional (B, NQ, D) contiguous tensor the result is added to (and written
-                  into); default: the bare result in a new tensor.
+        accum:    optional (B, NQ, D) contiguous tensor the result is added to (and, unless
+                  ``out`` is given, written into); default: the bare result in a new tensor.
+        out:      optional (B, NQ, D) contiguous bfloat16 destination.
 
     Returns (B, NQ, D) bfloat16.
     """
@@ -136,7 +138,7 @@ def sdpa_cross(
     if kv.shape != (B, NK, 2 * D):
         raise ValueError(f"kv must be {(B, NK, 2 * D)}, got {tuple(kv.shape)}")
     if not cross_supported(qkv, kv, n_heads):
-        raise RuntimeError("sdpa_cross covers bfloat16, head size 32, 1..160 keys and at most 160 queries")
+        raise RuntimeError("sdpa_cross covers bfloat16, head size 32, 1..2048 keys and at most 160 queries")
     if torch.is_grad_enabled() and (qkv.requires_grad or kv.requires_grad):
         raise RuntimeError("sdpa_cross is forward-only; call it under torch.no_grad()")
     if B and NQ and (qkv.stride(-1) != 1 or (B > 1 and qkv.stride(0) != NQ * qkv.stride(1))):
@@ -151,7 +153,10 @@ def sdpa_cross(
         mask_ptr = key_mask.data_ptr()
     if accum is not None and (accum.shape != (B, NQ, D) or accum.dtype != torch.bfloat16 or not accum.is_contiguous()):
         raise ValueError("accum must be a contiguous bfloat16 (B, NQ, D) tensor")
-    out = accum if accum is not None else torch.empty((B, NQ, D), dtype=torch.bfloat16, device=qkv.device)
+    if out is not None and (out.shape != (B, NQ, D) or out.dtype != torch.bfloat16 or not out.is_contiguous()):
+        raise ValueError("out must be a contiguous bfloat16 (B, NQ, D) tensor")
+    if out is None:
+        out = accum if accum is not None else torch.empty((B, NQ, D), dtype=torch.bfloat16, device=qkv.device)
     if B == 0 or NQ == 0:
         return out
     with torch.cuda.device(qkv.device):

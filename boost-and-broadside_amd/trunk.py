@@ -186,7 +186,7 @@ class TransformerBlock(nn.Module):
 
     def _bullet_read(self, qkv, kv, bullet_mask):
         """Cross-attention of the entity queries to bullet key/values (attention.py:149-166) for
-        the shapes the matrix-core kernel does not cover (fp32, more than 160 bullets, other
+        the shapes the matrix-core kernel does not cover (fp32, more than 2048 bullets, other
         head sizes): torch's SDPA on the device, with the reference's additive bias and its
         all-inactive gate.  ``kv`` is ``kv_bullet(norm_bullet(bullets))``."""
         B, N, _ = qkv.shape

@@ -278,12 +278,43 @@ def test_sdpa_cross_matches_oracle(B, NQ, NK):
     assert max_rel(no_mask, torch_ref.bullet_read(qkv.float(), kv.float(), None, H)) <= BF16_TOL
 
 
+@pytest.mark.parametrize("B,NQ,NK,p_live", [(4, 12, 161, 0.5), (3, 84, 800, 0.3), (2, 156, 1520, 1.0), (3, 156, 1520, 0.1),
+                                           (2, 33, 2048, 0.7), (3, 20, 500, 0.02), (2, 160, 193, 0.17)])
+def test_sdpa_cross_streams_long_key_axes(B, NQ, NK, p_live):
+    # more keys than fit in LDS at once: tiles of live keys with an online softmax across them
+    H, D = 4, 128
+    g = torch.Generator().manual_seed(NQ * 3000 + NK)
+    qkv = torch.randn(B, NQ, 3 * D, generator=g).bfloat16()
+    kv = torch.randn(B, NK, 2 * D, generator=g).bfloat16()
+    kv[:, :, :D] *= 3.0  # peaked softmax rows: the running maximum has to move between tiles
+    mask = torch.rand(B, NK, generator=g) < p_live
+    mask[0] = False
+    mask[1, NK - 1] = True
+    merged = torch.randn(B, NQ, D, generator=g).bfloat16()
+    truth = torch_ref.bullet_read(qkv.float(), kv.float(), mask, H)
+    bare = ops.sdpa_cross(qkv.to(DEV), kv.to(DEV), mask.to(DEV), H).float().cpu()
+    assert bare[0].abs().max() == 0
+    assert max_rel(bare, truth) <= BF16_TOL
+    acc = merged.to(DEV).clone()
+    out = ops.sdpa_cross(qkv.to(DEV), kv.to(DEV), mask.to(DEV), H, accum=acc)
+    assert out.data_ptr() == acc.data_ptr()
+    assert torch.equal(out.float().cpu(), (merged + bare.bfloat16()).float())
+    other = torch.empty_like(acc)  # accum != out: environments without a live key copy accum through
+    got = ops.sdpa_cross(qkv.to(DEV), kv.to(DEV), mask.to(DEV), H, accum=merged.to(DEV), out=other)
+    assert torch.equal(got.cpu(), out.cpu())
+    kv2 = kv.clone()
+    kv2[~mask] = kv2[~mask] * -2.0 + 9.0
+    assert torch.equal(ops.sdpa_cross(qkv.to(DEV), kv2.to(DEV), mask.to(DEV), H).float().cpu(), bare)
+    no_mask = ops.sdpa_cross(qkv.to(DEV), kv.to(DEV), None, H).float().cpu()
+    assert max_rel(no_mask, torch_ref.bullet_read(qkv.float(), kv.float(), None, H)) <= BF16_TOL
+
+
 def test_sdpa_cross_limits():
     qkv = torch.zeros(1, 12, 384, device=DEV, dtype=torch.bfloat16)
-    assert not ops.cross_supported(qkv, torch.zeros(1, 161, 256, device=DEV, dtype=torch.bfloat16), 4)
+    assert not ops.cross_supported(qkv, torch.zeros(1, 2049, 256, device=DEV, dtype=torch.bfloat16), 4)
     assert not ops.cross_supported(qkv.float(), torch.zeros(1, 80, 256, device=DEV), 4)
     with pytest.raises(RuntimeError):
-        ops.sdpa_cross(qkv, torch.zeros(1, 200, 256, device=DEV, dtype=torch.bfloat16), None, 4)
+        ops.sdpa_cross(qkv, torch.zeros(1, 2100, 256, device=DEV, dtype=torch.bfloat16), None, 4)
 
 
 # ------------------------------------------------------------------ RG-LRU step
