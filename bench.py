@@ -39,6 +39,7 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU-baseline leg; 0 skips it")
     ap.add_argument("--no-torch-baseline", action="store_true")
     ap.add_argument("--no-module", action="store_true")
+    ap.add_argument("--no-bullets", action="store_true", help="skip the bullet-read leg")
     ap.add_argument("--no-trunk", action="store_true", help="skip the whole-trunk leg (2 blocks x (2 spatial + 1 temporal))")
     return ap.parse_args()
 
@@ -407,6 +408,40 @@ def main():
         "what": "read linear1 output + 3 stored inputs, write conv output + shifted inputs into the packed state",
     }
     del packed
+
+    # ---- bullet read (entity queries attending to the bullets in flight; 10 slots per ship) ----
+    if bf16 and not args.no_bullets:
+        NB = w.N * 10
+        live_p = 0.25
+        kv_b = (0.7 * torch.randn(w.B, NB, 2 * D, device=dev, generator=gen)).to(w.dtype)
+        b_mask = torch.rand(w.B, NB, device=dev, generator=gen) < live_p
+        merged = [torch.zeros(w.B, w.NM, D, device=dev, dtype=w.dtype) for _ in range(2)]
+        qkv_b = qkv_pool[0]
+        n_b = max(4, min(steps, 16))
+        t_read = timed_loop(lambda t: ops.sdpa_cross(qkv_b, kv_b, b_mask, H, accum=merged[t & 1]), n_b, 3) / n_b
+
+        def torch_read(t):
+            q = qkv_b[..., :D].reshape(w.B, w.NM, H, D // H).transpose(1, 2)
+            kb = kv_b[..., :D].reshape(w.B, NB, H, D // H).transpose(1, 2)
+            vb = kv_b[..., D:].reshape(w.B, NB, H, D // H).transpose(1, 2)
+            bias = (1.0 - b_mask.reshape(w.B, 1, 1, NB).to(q.dtype)) * (torch.finfo(q.dtype).min / 2)
+            o = torch.nn.functional.scaled_dot_product_attention(q, kb, vb, attn_mask=bias)
+            o = o * b_mask.any(-1).reshape(w.B, 1, 1, 1).to(o.dtype)
+            merged[t & 1] += o.transpose(1, 2).reshape(w.B, w.NM, D)
+
+        t_read_torch = None if args.no_torch_baseline else timed_loop(torch_read, 3, 1) / 3
+        live = int(b_mask.sum().item())
+        read_bytes = live * 2 * D * 2 + w.B * NB + 3 * w.B * w.NM * D * 2
+        result["bullet_read"] = {
+            "avg_launch_us": t_read * 1e6, "slots_per_env": NB, "live_fraction": live_p,
+            "algorithmic_bytes_per_launch": read_bytes, "achieved_GBps": read_bytes / t_read / 1e9,
+            "frac_of_hbm_peak": read_bytes / t_read / peak,
+            "tflops": 4 * live * w.NM * D / t_read / 1e12,
+            "eager_torch_us": None if t_read_torch is None else t_read_torch * 1e6,
+            "what": "bnb_sdpa_cross_fwd added into the self-attention output: K/V rows of the live bullets, the slot "
+                    "mask, Q, accumulator in and out; exp-throughput-bound rather than HBM-bound when many bullets are live",
+        }
+        del kv_b, b_mask, merged
 
     # ---- whole trunk (reference default: 2 blocks x (2 spatial + 1 temporal)), state carried ----
     if not args.no_trunk:
