@@ -1,0 +1,371 @@
+// Temporal sublayer over a whole sequence for gfx950: the causal depthwise conv and the
+// RG-LRU recurrence, each as ONE pass over (rows, T, D).
+//
+// Reference: models/yemong/griffin.py:96-140 (tap loop with episode-aware validity,
+// :67-93) and :188-219 (gates, decay, Hillis-Steele scan :25-64).  The reference evaluates
+// h_t = a_t h_{t-1} + b_t with a log-depth scan, log2(T) rounds of full-tensor element-wise
+// kernels over padded copies of a and b; here every lane owns 8 channels of one row and
+// simply walks t = 0..T-1 with the state in registers: x and the gate pre-activations are
+// read once, y is written once, a and b never exist in memory.  `done[r, t]` ends an episode
+// at t: step t+1 starts from a zero state (:213-218) and its conv taps do not reach back
+// across the boundary (:67-93).  Loads for several timesteps are issued before the
+// dependent arithmetic, so the sequential recurrence does not serialise the memory traffic.
+
+#include "common.h"
+#include "rglru_math.h"
+
+namespace bnb {
+
+constexpr int kSeqThreads = 256;
+constexpr int kSeqTaps = 4;
+constexpr int kSeqAhead = 4;  // timesteps whose operands are in flight together
+
+// ------------------------------------------------------------------------------------
+// RG-LRU over T steps
+// ------------------------------------------------------------------------------------
+
+template <typename XT, typename GT, typename YT>
+__global__ __launch_bounds__(kSeqThreads) void rglru_scan_vec8_kernel(
+    const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
+    const float *__restrict__ h0, int64_t h0_stride, const uint8_t *__restrict__ done, YT *__restrict__ y,
+    float *__restrict__ h_last, int64_t h_last_stride, int64_t R, int T, int D, int64_t rs, int64_t ts, int rows_per_block)
+{
+    extern __shared__ float s_l2sig[];  // D entries
+    for (int d = threadIdx.x; d < D; d += kSeqThreads) s_l2sig[d] = log2_sigmoid(log_lambda[d]);
+    __syncthreads();
+
+    const int vecs_per_row = D >> 3;
+    const int local_row = threadIdx.x / vecs_per_row;
+    const int64_t row = (int64_t)blockIdx.x * rows_per_block + local_row;
+    if (local_row >= rows_per_block || row >= R) return;
+    const int d0 = (threadIdx.x - local_row * vecs_per_row) << 3;
+
+    float l2[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) l2[e] = s_l2sig[d0 + e];
+    Row8 h = load8(h0 + row * h0_stride + d0);
+    const XT *xp = x + row * rs + d0;
+    const GT *gp = gates + row * 2 * rs + d0;
+    YT *yp = y + row * rs + d0;
+    const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
+
+    for (int t0 = 0; t0 < T; t0 += kSeqAhead) {
+        Row8 xv[kSeqAhead], ga[kSeqAhead], gx[kSeqAhead];
+        uint32_t cut[kSeqAhead];
+#pragma unroll
+        for (int u = 0; u < kSeqAhead; ++u) {
+            // past the end: re-read the last step (discarded) so the loads stay branch-free
+            const int t = t0 + u < T ? t0 + u : T - 1;
+            xv[u] = load8_stream(xp + t * ts);
+            ga[u] = load8_stream(gp + t * 2 * ts);
+            gx[u] = load8_stream(gp + t * 2 * ts + D);
+            cut[u] = 0;
+            if (dn != nullptr) cut[u] = dn[t > 0 ? t - 1 : 0];
+            if (t == 0) cut[u] = 0;  // the first step continues the stored state
+        }
+#pragma unroll
+        for (int u = 0; u < kSeqAhead; ++u) {
+            if (t0 + u < T) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float prev = cut[u] ? 0.0f : h.v[e];
+                    h.v[e] = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(xv[u].v[e], ga[u].v[e], gx[u].v[e],
+                                                                                    l2[e], c, prev);
+                }
+                store8_stream(yp + (t0 + u) * ts, h);
+            }
+        }
+    }
+    store8(h_last + row * h_last_stride + d0, h);
+}
+
+// Any D, any alignment, and small inputs (eight times the lanes): one lane per (row, channel).
+template <typename XT, typename GT, typename YT>
+__global__ __launch_bounds__(kSeqThreads) void rglru_scan_scalar_kernel(
+    const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
+    const float *__restrict__ h0, int64_t h0_stride, const uint8_t *__restrict__ done, YT *__restrict__ y,
+    float *__restrict__ h_last, int64_t h_last_stride, int64_t R, int T, int D, int64_t rs, int64_t ts)
+{
+    const int64_t idx = (int64_t)blockIdx.x * kSeqThreads + threadIdx.x;
+    if (idx >= R * D) return;
+    const int64_t row = idx / D;
+    const int d = (int)(idx - row * D);
+    const float l2 = log2_sigmoid(log_lambda[d]);
+    float h = h0[row * h0_stride + d];
+    const XT *xp = x + row * rs + d;
+    const GT *gp = gates + row * 2 * rs + d;
+    YT *yp = y + row * rs + d;
+    const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
+    for (int t0 = 0; t0 < T; t0 += kSeqAhead) {
+        float xv[kSeqAhead], ga[kSeqAhead], gx[kSeqAhead];
+        uint32_t cut[kSeqAhead];
+#pragma unroll
+        for (int u = 0; u < kSeqAhead; ++u) {
+            const int t = t0 + u < T ? t0 + u : T - 1;
+            xv[u] = load1(xp + t * ts);
+            ga[u] = load1(gp + t * 2 * ts);
+            gx[u] = load1(gp + t * 2 * ts + D);
+            cut[u] = 0;
+            if (dn != nullptr) cut[u] = dn[t > 0 ? t - 1 : 0];
+            if (t == 0) cut[u] = 0;
+        }
+#pragma unroll
+        for (int u = 0; u < kSeqAhead; ++u) {
+            if (t0 + u < T) {
+                h = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(xv[u], ga[u], gx[u], l2, c,
+                                                                          cut[u] ? 0.0f : h);
+                store1(yp + (t0 + u) * ts, h);
+            }
+        }
+    }
+    h_last[row * h_last_stride + d] = h;
+}
+
+template <typename XT, typename GT, typename YT>
+static int launch_scan(const void *x, const void *gates, const float *log_lambda, float c, const float *h0,
+                       int64_t h0_stride, const uint8_t *done, void *y, float *h_last, int64_t h_last_stride,
+                       int64_t R, int T, int D, int time_major, hipStream_t stream)
+{
+    // element strides of one row / one timestep: (R, T, D) or (T, R, D)
+    const int64_t rs = time_major ? D : (int64_t)T * D, ts = time_major ? R * D : D;
+    const bool vec_ok = (D % 8 == 0) && (D / 8 <= kSeqThreads) && aligned16(x) && aligned16(gates) && aligned16(h0) &&
+                        aligned16(h_last) && aligned16(y) && (h0_stride % 4 == 0) && (h_last_stride % 4 == 0);
+    // the wide lanes need enough rows to fill the chip; below that one lane per channel
+    const bool vec = vec_ok && R * (D / 8) >= (int64_t)256 * kSeqThreads * 2;
+    if (vec) {
+        const int rows_per_block = kSeqThreads / (D / 8);
+        const int64_t blocks = (R + rows_per_block - 1) / rows_per_block;
+        if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL((rglru_scan_vec8_kernel<XT, GT, YT>), dim3((unsigned)blocks), dim3(kSeqThreads),
+                           (size_t)D * sizeof(float), stream, (const XT *)x, (const GT *)gates, log_lambda, c, h0,
+                           h0_stride, done, (YT *)y, h_last, h_last_stride, R, T, D, rs, ts, rows_per_block);
+    } else {
+        const int64_t blocks = (R * D + kSeqThreads - 1) / kSeqThreads;
+        if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL((rglru_scan_scalar_kernel<XT, GT, YT>), dim3((unsigned)blocks), dim3(kSeqThreads), 0,
+                           stream, (const XT *)x, (const GT *)gates, log_lambda, c, h0, h0_stride, done, (YT *)y,
+                           h_last, h_last_stride, R, T, D, rs, ts);
+    }
+    return (int)hipGetLastError();
+}
+
+template <typename XT, typename GT>
+static int scan_dispatch_y(const void *x, const void *gates, const float *log_lambda, float c, const float *h0,
+                           int64_t h0_stride, const uint8_t *done, void *y, int y_dtype, float *h_last,
+                           int64_t h_last_stride, int64_t R, int T, int D, int time_major, hipStream_t stream)
+{
+    if (y_dtype == BNB_F32)
+        return launch_scan<XT, GT, float>(x, gates, log_lambda, c, h0, h0_stride, done, y, h_last, h_last_stride, R,
+                                          T, D, time_major, stream);
+    return launch_scan<XT, GT, uint16_t>(x, gates, log_lambda, c, h0, h0_stride, done, y, h_last, h_last_stride, R, T,
+                                         D, time_major, stream);
+}
+
+// ------------------------------------------------------------------------------------
+// causal depthwise conv over T steps
+// ------------------------------------------------------------------------------------
+
+// `hist` counts how many of the three previous inputs belong to the running episode: the
+// stored buffer belongs to the episode running at t = 0, a boundary clears the history.
+template <typename BT>
+__global__ __launch_bounds__(kSeqThreads) void conv_seq_vec8_kernel(
+    const BT *__restrict__ b1, const float *__restrict__ conv_in, int64_t conv_in_stride,
+    const float *__restrict__ weight, const float *__restrict__ bias, const uint8_t *__restrict__ done,
+    float *__restrict__ v_out, uint16_t *__restrict__ v_bf16_out, float *__restrict__ conv_out,
+    int64_t conv_out_stride, int64_t R, int T, int D, int64_t rs, int64_t ts, int rows_per_block)
+{
+    const int vecs_per_row = D >> 3;
+    const int local_row = threadIdx.x / vecs_per_row;
+    const int64_t row = (int64_t)blockIdx.x * rows_per_block + local_row;
+    if (local_row >= rows_per_block || row >= R) return;
+    const int d0 = (threadIdx.x - local_row * vecs_per_row) << 3;
+
+    float w[8][kSeqTaps], bs[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const f32x4 wv = *reinterpret_cast<const f32x4 *>(weight + (int64_t)(d0 + e) * kSeqTaps);
+        w[e][0] = wv.x;
+        w[e][1] = wv.y;
+        w[e][2] = wv.z;
+        w[e][3] = wv.w;
+        bs[e] = bias != nullptr ? bias[d0 + e] : 0.0f;
+    }
+    const float *pin = conv_in + row * conv_in_stride + d0;
+    Row8 p0 = load8(pin), p1 = load8(pin + D), p2 = load8(pin + 2 * D);
+    const BT *bp = b1 + row * rs + d0;
+    const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
+    int hist = 3;
+
+    for (int t0 = 0; t0 < T; t0 += kSeqAhead) {
+        Row8 cur[kSeqAhead];
+        uint32_t cut[kSeqAhead];
+#pragma unroll
+        for (int u = 0; u < kSeqAhead; ++u) {
+            const int t = t0 + u < T ? t0 + u : T - 1;
+            cur[u] = load8_stream(bp + t * ts);
+            cut[u] = 0;
+            if (dn != nullptr) cut[u] = dn[t > 0 ? t - 1 : 0];
+            if (t == 0) cut[u] = 0;
+        }
+#pragma unroll
+        for (int u = 0; u < kSeqAhead; ++u) {
+            if (t0 + u < T) {
+                if (cut[u]) hist = 0;
+                Row8 v;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    // inputs from before the boundary read as zero; the reference's order:
+                    // taps 0..3 (oldest input first), then the bias
+                    float acc = (hist >= 3 ? p0.v[e] : 0.0f) * w[e][0];
+                    acc += (hist >= 2 ? p1.v[e] : 0.0f) * w[e][1];
+                    acc += (hist >= 1 ? p2.v[e] : 0.0f) * w[e][2];
+                    acc += cur[u].v[e] * w[e][3];
+                    v.v[e] = acc + bs[e];
+                }
+                const int64_t off = row * rs + (t0 + u) * ts + d0;
+                store8_stream(v_out + off, v);
+                if (v_bf16_out != nullptr) store8_stream(v_bf16_out + off, v);
+                p0 = p1;
+                p1 = p2;
+                p2 = cur[u];
+                hist = hist < 3 ? hist + 1 : 3;
+            }
+        }
+    }
+    // the last three inputs, whatever episode they belong to (griffin.py:277)
+    float *pout = conv_out + row * conv_out_stride + d0;
+    store8(pout, p0);
+    store8(pout + D, p1);
+    store8(pout + 2 * D, p2);
+}
+
+template <typename BT>
+__global__ __launch_bounds__(kSeqThreads) void conv_seq_scalar_kernel(
+    const BT *__restrict__ b1, const float *__restrict__ conv_in, int64_t conv_in_stride,
+    const float *__restrict__ weight, const float *__restrict__ bias, const uint8_t *__restrict__ done,
+    float *__restrict__ v_out, uint16_t *__restrict__ v_bf16_out, float *__restrict__ conv_out,
+    int64_t conv_out_stride, int64_t R, int T, int D, int64_t rs, int64_t ts)
+{
+    const int64_t idx = (int64_t)blockIdx.x * kSeqThreads + threadIdx.x;
+    if (idx >= R * D) return;
+    const int64_t row = idx / D;
+    const int d = (int)(idx - row * D);
+    const float *wp = weight + (int64_t)d * kSeqTaps;
+    const float w0 = wp[0], w1 = wp[1], w2 = wp[2], w3 = wp[3];
+    const float bs = bias != nullptr ? bias[d] : 0.0f;
+    const float *pin = conv_in + row * conv_in_stride + d;
+    float p0 = pin[0], p1 = pin[D], p2 = pin[2 * D];
+    const BT *bp = b1 + row * rs + d;
+    const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
+    int hist = 3;
+    for (int t = 0; t < T; ++t) {
+        const float cur = load1(bp + t * ts);
+        if (dn != nullptr && t > 0 && dn[t - 1]) hist = 0;
+        float acc = (hist >= 3 ? p0 : 0.0f) * w0;
+        acc += (hist >= 2 ? p1 : 0.0f) * w1;
+        acc += (hist >= 1 ? p2 : 0.0f) * w2;
+        acc += cur * w3;
+        const float v = acc + bs;
+        v_out[row * rs + t * ts + d] = v;
+        if (v_bf16_out != nullptr) store1(v_bf16_out + row * rs + t * ts + d, v);
+        p0 = p1;
+        p1 = p2;
+        p2 = cur;
+        hist = hist < 3 ? hist + 1 : 3;
+    }
+    float *pout = conv_out + row * conv_out_stride + d;
+    pout[0] = p0;
+    pout[D] = p1;
+    pout[2 * D] = p2;
+}
+
+template <typename BT>
+static int launch_conv_seq(const void *b1, const float *conv_in, int64_t conv_in_stride, const float *weight,
+                           const float *bias, const uint8_t *done, float *v_out, uint16_t *v_bf16_out,
+                           float *conv_out, int64_t conv_out_stride, int64_t R, int T, int D, int time_major,
+                           hipStream_t stream)
+{
+    const int64_t rs = time_major ? D : (int64_t)T * D, ts = time_major ? R * D : D;
+    const bool vec_ok = (D % 8 == 0) && (D / 8 <= kSeqThreads) && aligned16(b1) && aligned16(conv_in) &&
+                        aligned16(conv_out) && aligned16(v_out) && aligned16(v_bf16_out) && aligned16(weight) &&
+                        (conv_in_stride % 4 == 0) && (conv_out_stride % 4 == 0);
+    const bool vec = vec_ok && R * (D / 8) >= (int64_t)256 * kSeqThreads * 2;
+    if (vec) {
+        const int rows_per_block = kSeqThreads / (D / 8);
+        const int64_t blocks = (R + rows_per_block - 1) / rows_per_block;
+        if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL((conv_seq_vec8_kernel<BT>), dim3((unsigned)blocks), dim3(kSeqThreads), 0, stream,
+                           (const BT *)b1, conv_in, conv_in_stride, weight, bias, done, v_out, v_bf16_out, conv_out,
+                           conv_out_stride, R, T, D, rs, ts, rows_per_block);
+    } else {
+        const int64_t blocks = (R * D + kSeqThreads - 1) / kSeqThreads;
+        if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL((conv_seq_scalar_kernel<BT>), dim3((unsigned)blocks), dim3(kSeqThreads), 0, stream,
+                           (const BT *)b1, conv_in, conv_in_stride, weight, bias, done, v_out, v_bf16_out, conv_out,
+                           conv_out_stride, R, T, D, rs, ts);
+    }
+    return (int)hipGetLastError();
+}
+
+}  // namespace bnb
+
+extern "C" int bnb_rglru_scan_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
+                                  const float *log_lambda, float c, const float *h0, int64_t h0_row_stride,
+                                  const uint8_t *done, void *y, int y_dtype, float *h_last,
+                                  int64_t h_last_row_stride, int64_t R, int T, int D, int time_major, void *stream)
+{
+    using namespace bnb;
+    if (R < 0 || T < 0 || D < 1) return BNB_ERR_BAD_SHAPE;
+    if (R == 0) return 0;
+    if (!log_lambda || !h0 || !h_last) return BNB_ERR_NULL_POINTER;
+    if (h0_row_stride < D || h_last_row_stride < D) return BNB_ERR_BAD_SHAPE;
+    if ((x_dtype != BNB_F32 && x_dtype != BNB_BF16) || (g_dtype != BNB_F32 && g_dtype != BNB_BF16) ||
+        (y_dtype != BNB_F32 && y_dtype != BNB_BF16))
+        return BNB_ERR_BAD_DTYPE;
+    if ((reinterpret_cast<uintptr_t>(h0) | reinterpret_cast<uintptr_t>(h_last) |
+         reinterpret_cast<uintptr_t>(log_lambda)) & 3u)
+        return BNB_ERR_MISALIGNED;
+    hipStream_t s = (hipStream_t)stream;
+    if (T == 0) {  // nothing to advance: the state passes through
+        if (h0 == h_last && h0_row_stride == h_last_row_stride) return 0;
+        return (int)hipMemcpy2DAsync(h_last, (size_t)h_last_row_stride * sizeof(float), h0,
+                                     (size_t)h0_row_stride * sizeof(float), (size_t)D * sizeof(float), (size_t)R,
+                                     hipMemcpyDeviceToDevice, s);
+    }
+    if (!x || !gates_pre || !y) return BNB_ERR_NULL_POINTER;
+    const bool xb = x_dtype == BNB_BF16, gb = g_dtype == BNB_BF16;
+    if (!xb && !gb)
+        return scan_dispatch_y<float, float>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype, h_last,
+                                             h_last_row_stride, R, T, D, time_major != 0, s);
+    if (xb && gb)
+        return scan_dispatch_y<uint16_t, uint16_t>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype,
+                                                   h_last, h_last_row_stride, R, T, D, time_major != 0, s);
+    if (!xb && gb)
+        return scan_dispatch_y<float, uint16_t>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype,
+                                                h_last, h_last_row_stride, R, T, D, time_major != 0, s);
+    return scan_dispatch_y<uint16_t, float>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype, h_last,
+                                            h_last_row_stride, R, T, D, time_major != 0, s);
+}
+
+extern "C" int bnb_conv_seq_fwd(const void *b1, int b1_dtype, const float *conv_in, int64_t conv_in_row_stride,
+                                const float *weight, const float *bias, const uint8_t *done, float *v_out,
+                                void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride, int64_t R, int T,
+                                int D, int time_major, void *stream)
+{
+    using namespace bnb;
+    if (R < 0 || T < 1 || D < 1) return BNB_ERR_BAD_SHAPE;
+    if (R == 0) return 0;
+    if (!b1 || !conv_in || !weight || !v_out || !conv_out) return BNB_ERR_NULL_POINTER;
+    if (b1_dtype != BNB_F32 && b1_dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
+    if (conv_in_row_stride < 3 * (int64_t)D || conv_out_row_stride < 3 * (int64_t)D) return BNB_ERR_BAD_SHAPE;
+    if ((reinterpret_cast<uintptr_t>(conv_in) | reinterpret_cast<uintptr_t>(conv_out) |
+         reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(v_out) |
+         reinterpret_cast<uintptr_t>(bias)) & 3u)
+        return BNB_ERR_MISALIGNED;
+    hipStream_t s = (hipStream_t)stream;
+    if (b1_dtype == BNB_BF16)
+        return launch_conv_seq<uint16_t>(b1, conv_in, conv_in_row_stride, weight, bias, done, v_out,
+                                         (uint16_t *)v_bf16_out, conv_out, conv_out_row_stride, R, T, D, time_major != 0, s);
+    return launch_conv_seq<float>(b1, conv_in, conv_in_row_stride, weight, bias, done, v_out, (uint16_t *)v_bf16_out,
+                                  conv_out, conv_out_row_stride, R, T, D, time_major != 0, s);
+}

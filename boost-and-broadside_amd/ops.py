@@ -337,6 +337,161 @@ def conv_step(
     return (v, conv_out, v_lp) if also_bf16 else (v, conv_out)
 
 
+def _done_pointer(done, R, T, device):
+    """Contiguous byte view of an optional (R, T) episode-end mask; returns (keepalive, pointer)."""
+    if done is None:
+        return None, None
+    if done.shape != (R, T) or done.dtype not in (torch.bool, torch.uint8):
+        raise ValueError(f"done must be a bool {(R, T)} tensor")
+    if done.device != device:
+        raise ValueError("done must live on the same device as the inputs")
+    done = done.contiguous()
+    return done, done.data_ptr()
+
+
+def conv_seq(
+    b1: torch.Tensor,
+    conv_buf: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None,
+    done: torch.Tensor | None = None,
+    *,
+    conv_out: torch.Tensor | None = None,
+    also_bf16: bool = False,
+    time_major: bool = False,
+):
+    """Causal depthwise conv over a sequence, taps cut at episode ends (griffin.py:67-140).
+
+    Args:
+        b1:       (R, T, D) ``linear1`` outputs, float32 or bfloat16.
+        conv_buf: (R, 3, D) float32 inputs stored before the sequence (rows may be strided).
+        weight, bias: as in ``conv_step``.
+        done:     optional (R, T) bool; True at t ends an episode at t.
+        conv_out: optional (R, 3, D) float32 destination for the new stored inputs.
+        also_bf16: also return a bfloat16 copy of the conv output.
+        time_major: ``b1`` and the returned conv output are (T, R, D) instead of (R, T, D);
+                  ``done`` stays (R, T).
+
+    Returns:
+        (v, new_conv_buf[, v_bf16]): conv output (R, T, D) float32 and the last three entries
+        of ``[conv_buf, b1]``.
+    """
+    if b1.dim() != 3 or conv_buf.dim() != 3:
+        raise ValueError("b1 must be (R, T, D) and conv_buf (R, 3, D)")
+    R, T, D = b1.shape
+    if time_major:
+        T, R = R, T
+    if T < 1:
+        raise ValueError("conv_seq needs at least one timestep")
+    if conv_buf.shape != (R, 3, D):
+        raise ValueError(f"conv_buf must be {(R, 3, D)}, got {tuple(conv_buf.shape)}")
+    for name, t in (("b1", b1), ("conv_buf", conv_buf), ("weight", weight)):
+        _need_device(t, name)
+    if conv_buf.dtype != torch.float32 or weight.dtype != torch.float32 or (bias is not None and bias.dtype != torch.float32):
+        raise TypeError("conv_buf, weight and bias must be float32")
+    if torch.is_grad_enabled() and (b1.requires_grad or conv_buf.requires_grad):
+        raise RuntimeError("conv_seq is forward-only; call it under torch.no_grad()")
+    b_code = _code(b1, "b1")
+    weight = weight.detach().reshape(D, 4).contiguous()
+    bias_ptr = None
+    if bias is not None:
+        bias = bias.detach().contiguous()
+        bias_ptr = bias.data_ptr()
+    b1 = b1.contiguous()
+
+    def rows_ok(t):
+        return R == 0 or (t.stride(2) == 1 and t.stride(1) == D)
+
+    if not rows_ok(conv_buf):
+        conv_buf = conv_buf.contiguous()
+    if conv_out is None:
+        conv_out = torch.empty((R, 3, D), dtype=torch.float32, device=b1.device)
+    elif conv_out.shape != (R, 3, D) or conv_out.dtype != torch.float32 or conv_out.device != b1.device or not rows_ok(conv_out):
+        raise ValueError("conv_out must be a float32 (R, 3, D) tensor on b1's device with contiguous rows")
+    v = torch.empty(b1.shape, dtype=torch.float32, device=b1.device)
+    v_lp = torch.empty(b1.shape, dtype=torch.bfloat16, device=b1.device) if also_bf16 else None
+    keep, done_ptr = _done_pointer(done, R, T, b1.device)
+    if R:
+        with torch.cuda.device(b1.device):
+            rc = _native.load().bnb_conv_seq_fwd(
+                b1.data_ptr(), b_code, conv_buf.data_ptr(), conv_buf.stride(0), weight.data_ptr(), bias_ptr, done_ptr,
+                v.data_ptr(), None if v_lp is None else v_lp.data_ptr(), conv_out.data_ptr(), conv_out.stride(0),
+                R, T, D, int(time_major), _stream(),
+            )
+        _native.check(rc, "bnb_conv_seq_fwd")
+    del keep
+    return (v, conv_out, v_lp) if also_bf16 else (v, conv_out)
+
+
+def rglru_scan(
+    x: torch.Tensor,
+    gates_pre: torch.Tensor,
+    log_lambda: torch.Tensor,
+    c: float,
+    h0: torch.Tensor,
+    done: torch.Tensor | None = None,
+    *,
+    y_dtype: torch.dtype = torch.float32,
+    h_out: torch.Tensor | None = None,
+    time_major: bool = False,
+):
+    """RG-LRU over a whole sequence in one pass (griffin.py:188-219 without the log-depth scan).
+
+    Args:
+        x:          (R, T, D) float32 or bfloat16.
+        gates_pre:  (R, T, 2*D) ``[linear_a(x) | linear_x(x)]``.
+        log_lambda: (D,) float32.
+        h0:         (R, D) float32 state before the sequence (rows may be strided).
+        done:       optional (R, T) bool; True at t makes step t+1 start from a zero state.
+        y_dtype:    dtype of the returned states.
+        h_out:      optional (R, D) float32 destination of the final state.
+        time_major: ``x``, ``gates_pre`` and the returned states are (T, R, .) instead of
+                    (R, T, .); ``done`` stays (R, T).
+
+    Returns:
+        (y, h_last): all states (R, T, D) in ``y_dtype`` and the final state (R, D) float32.
+    """
+    if x.dim() != 3:
+        raise ValueError("x must be (R, T, D)")
+    R, T, D = x.shape
+    if gates_pre.shape != (R, T, 2 * D):
+        raise ValueError(f"gates_pre must be {(R, T, 2 * D)}, got {tuple(gates_pre.shape)}")
+    if time_major:
+        T, R = R, T
+    if h0.shape != (R, D) or h0.dtype != torch.float32:
+        raise ValueError(f"h0 must be a float32 {(R, D)} tensor")
+    if log_lambda.shape != (D,) or log_lambda.dtype != torch.float32:
+        raise ValueError(f"log_lambda must be a float32 {(D,)} tensor")
+    for name, t in (("x", x), ("gates_pre", gates_pre), ("h0", h0), ("log_lambda", log_lambda)):
+        _need_device(t, name)
+    if torch.is_grad_enabled() and (x.requires_grad or gates_pre.requires_grad or h0.requires_grad or log_lambda.requires_grad):
+        raise RuntimeError("rglru_scan is forward-only; call it under torch.no_grad()")
+    if y_dtype not in _DTYPE_CODE:
+        raise TypeError(f"y_dtype must be float32 or bfloat16, got {y_dtype}")
+    x_code, g_code = _code(x, "x"), _code(gates_pre, "gates_pre")
+    x = x.contiguous()
+    gates_pre = gates_pre.contiguous()
+    log_lambda = log_lambda.detach().contiguous()
+    if R and h0.stride(1) != 1:
+        h0 = h0.contiguous()
+    if h_out is None:
+        h_out = torch.empty((R, D), dtype=torch.float32, device=x.device)
+    elif h_out.shape != (R, D) or h_out.dtype != torch.float32 or h_out.device != x.device or (R and h_out.stride(1) != 1):
+        raise ValueError("h_out must be a float32 (R, D) tensor on x's device with contiguous rows")
+    y = torch.empty(x.shape, dtype=y_dtype, device=x.device)
+    keep, done_ptr = _done_pointer(done, R, T, x.device)
+    if R:
+        with torch.cuda.device(x.device):
+            rc = _native.load().bnb_rglru_scan_fwd(
+                x.data_ptr(), x_code, gates_pre.data_ptr(), g_code, log_lambda.data_ptr(), float(c), h0.data_ptr(),
+                h0.stride(0), done_ptr, y.data_ptr(), _DTYPE_CODE[y_dtype], h_out.data_ptr(), h_out.stride(0),
+                R, T, D, int(time_major), _stream(),
+            )
+        _native.check(rc, "bnb_rglru_scan_fwd")
+    del keep
+    return y, h_out
+
+
 _F32_EPS = float(torch.finfo(torch.float32).eps)
 _NORM_WIDTHS = (8, 16, 32, 64, 128, 256, 512)
 

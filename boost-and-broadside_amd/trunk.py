@@ -243,23 +243,19 @@ class RGLRU(nn.Module):
             reset=reset, rows_per_env=rows_per_env,
         )
 
-    def forward_sequence(self, x_seq, h0, done_mask=None):
-        """(R,T,D), (R,D) -> ((R,T,D) states, (R,D) last state).
+    def forward_sequence(self, x_seq, h0, done_mask=None, *, time_major=False, y_dtype=torch.float32, x_act=None,
+                         h_out=None):
+        """(R,T,D), (R,D) -> ((R,T,D) states, (R,D) last state), one pass over the sequence.
 
-        T = 1 is the rollout path (one launch).  Longer sequences advance step by step;
-        ``done_mask[:, t]`` cuts the state after step t (griffin.py:213-218).
+        The gate projections run as one GEMM over all R*T rows and one kernel walks the
+        recurrence in time order; ``done_mask[:, t]`` cuts the state after step t
+        (griffin.py:213-218).  ``time_major``: ``x_seq`` and the states are (T,R,D).
         """
-        T = x_seq.shape[1]
-        if T == 1 and done_mask is None:
-            h = self._step(x_seq[:, 0], h0)
-            return h.unsqueeze(1), h
-        h, ys = h0, []
-        for t in range(T):
-            if done_mask is not None and t > 0:
-                h = h * (~done_mask[:, t - 1]).to(h.dtype).unsqueeze(-1)
-            h = self._step(x_seq[:, t], h)
-            ys.append(h)
-        return torch.stack(ys, dim=1), h
+        D = x_seq.shape[-1]
+        flat_act = None if x_act is None else x_act.reshape(-1, D)
+        gates = self._gate_preactivations(x_seq.reshape(-1, D), flat_act).reshape(*x_seq.shape[:2], 2 * D)
+        return ops.rglru_scan(x_seq, gates, self.log_lambda, self.c, h0, done_mask, y_dtype=y_dtype, h_out=h_out,
+                              time_major=time_major)
 
 
 class GriffinTemporalBlock(nn.Module):
@@ -276,24 +272,29 @@ class GriffinTemporalBlock(nn.Module):
         self.norm2 = nn.RMSNorm(d_model)
         self.gated_mlp = GatedMLP(d_model)
 
-    def forward_sequence(self, x_seq, h0, conv_buf, done_mask=None):
-        """(R,T,D), (R,D), (R,3,D) [, (R,T) bool] -> (out (R,T,D), new_h (R,D), new_conv_buf (R,3,D))."""
-        T = x_seq.shape[1]
-        if T == 1 and done_mask is None:
+    def forward_sequence(self, x_seq, h0, conv_buf, done_mask=None, *, time_major=False):
+        """(R,T,D), (R,D), (R,3,D) [, (R,T) bool] -> (out (R,T,D), new_h (R,D), new_conv_buf (R,3,D)).
+
+        ``time_major``: ``x_seq`` and ``out`` are (T,R,D), the layout stored rollouts have.
+        """
+        T = x_seq.shape[0] if time_major else x_seq.shape[1]
+        if T == 1 and done_mask is None and not time_major:
             # rollout: the conv taps and the buffer shift are one kernel, the recurrence another
             x = x_seq[:, 0]
             out, new_h, new_conv_buf = self._step(x, h0, conv_buf, None, None, None, 1)
             return out.unsqueeze(1), new_h, new_conv_buf
+        # two passes over the sequence: conv taps (cut at episode ends), then the recurrence;
+        # the only tensors in between are the conv output and the gate pre-activations
+        act = _projection_dtype()
         normed = self._norm_in(x_seq)
         b1 = _project(self.linear1, normed)
-        padded = torch.cat([conv_buf, b1], dim=1)  # (R, T+3, D); fp32 buffer promotes a bf16 b1
-        w = self.conv.weight.squeeze(1)  # (D, 4); tap k meets padded[:, t+k]
-        if done_mask is None:
-            conv_out = sum(padded[:, k:k + T] * w[:, k] for k in range(CONV_KERNEL)) + self.conv.bias
-        else:
-            conv_out = _conv_within_episodes(padded, w, self.conv.bias, done_mask)
-        y, new_h = self.rg_lru.forward_sequence(conv_out, h0, done_mask)
-        return self._finish(x_seq, normed, y), new_h, padded[:, T:]
+        want_lp = act == torch.bfloat16
+        res = ops.conv_seq(b1, conv_buf, self.conv.weight, self.conv.bias, done_mask, also_bf16=want_lp,
+                           time_major=time_major)
+        y, new_h = self.rg_lru.forward_sequence(res[0], h0, done_mask, time_major=time_major,
+                                                y_dtype=act if _fused_ok(x_seq, act) else torch.float32,
+                                                x_act=res[2] if want_lp else None)
+        return self._finish(x_seq, normed, y), new_h, res[1]
 
     def _norm_in(self, x):
         """norm1(x) in the projection dtype (one kernel with the cast when the fused path applies)."""
@@ -355,25 +356,6 @@ class GriffinTemporalBlock(nn.Module):
             return x1 + self.gated_mlp(n2)
         x1 = x + self.linear_out(b1 * F.gelu(gate_in))
         return x1 + self.gated_mlp(self.norm2(x1))
-
-
-def _conv_within_episodes(padded, w, bias, done_mask):
-    """Depthwise causal conv whose taps stop at episode ends (griffin.py:67-140).
-
-    ``done_mask[:, t]`` ends an episode at t.  A tap contributes to output t only if the
-    input it reads lies in the same episode as t; the stored buffer counts as belonging
-    to the episode running at t = 0.
-    """
-    R, T = done_mask.shape
-    starts = torch.zeros_like(done_mask, dtype=torch.long)
-    starts[:, 1:] = done_mask[:, :-1].long()
-    episode = torch.cat([starts.new_zeros(R, CONV_KERNEL - 1), starts.cumsum(dim=1)], dim=1)  # (R, T+3)
-    here = episode[:, CONV_KERNEL - 1:]
-    out = 0
-    for k in range(CONV_KERNEL):
-        same = (episode[:, k:k + T] == here).to(padded.dtype).unsqueeze(-1)
-        out = out + padded[:, k:k + T] * w[:, k] * same
-    return out + bias
 
 
 class YemongBlock(nn.Module):
@@ -451,9 +433,10 @@ class YemongBlock(nn.Module):
         done_rows = None if done_mask is None else done_mask.t().repeat_interleave(n_rec, dim=0)  # (B*n_rec, T)
         new_h, new_cb = [], []
         for j, layer in enumerate(self.temporal):
-            ships = x[:, :, :n_rec].permute(1, 2, 0, 3).reshape(B * n_rec, T, D)
-            out, h_j, cb_j = layer.forward_sequence(ships, h0[j], conv_buf0[j], done_rows)
-            parts = [out.reshape(B, n_rec, T, D).permute(2, 0, 1, 3)]
+            # the sequence kernels read (T, rows, D) as stored: no transposed copies of the rollout
+            ships = x[:, :, :n_rec].reshape(T, B * n_rec, D)
+            out, h_j, cb_j = layer.forward_sequence(ships, h0[j], conv_buf0[j], done_rows, time_major=True)
+            parts = [out.reshape(T, B, n_rec, D)]
             if NM > n_rec:
                 parts.append(layer.forward_nonrecurrent(x[:, :, n_rec:], self.field_sub[j]))
             x = torch.cat(parts, dim=2) if len(parts) > 1 else parts[0]

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 4
+#define BNB_ABI_VERSION 5
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -192,6 +192,59 @@ int bnb_conv_step_fwd(const void *b1, int b1_dtype,
                       const uint8_t *reset, int rows_per_env,
                       float *v_out, void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride,
                       int64_t R, int D, void *stream);
+
+/*
+ * The same causal depthwise conv over a whole sequence of T steps per row, with episode
+ * boundaries.
+ *
+ * Replaces, in models/yemong/griffin.py: `padded = cat([conv_buf, b1], dim=1)` (:275),
+ * _causal_conv_tap_validity (:67-93), the tap loop of _causal_depthwise_conv (:127-139) and
+ * `new_conv_buf = padded[:, -3:]` (:277) of GriffinTemporalBlock.forward_sequence.
+ *
+ *   b1        (R, T, D) contiguous, b1_dtype; with time_major != 0 the sequence tensors
+ *             b1, v_out and v_bf16_out are (T, R, D) instead (every step's rows together,
+ *             the layout the policy keeps rollouts in); done stays (R, T)
+ *   conv_in   the three inputs stored before the sequence, [p0 | p1 | p2] per row as in
+ *             bnb_conv_step_fwd; they count as part of the episode running at t = 0
+ *   done      optional (R, T) bytes: non-zero at t ends an episode at t, so outputs after t
+ *             take no tap from inputs at or before t; NULL = no boundaries
+ *   v_out     (R, T, D) fp32 contiguous; v_bf16_out optional bf16 copy
+ *   conv_out  the last three entries of [conv_in, b1] per row (not cut at boundaries, as in
+ *             the reference); may equal conv_in
+ * Requirements: T >= 1, strides >= 3*D; vector path as for bnb_conv_step_fwd (weight 16-byte
+ * aligned), scalar path otherwise.
+ */
+int bnb_conv_seq_fwd(const void *b1, int b1_dtype,
+                     const float *conv_in, int64_t conv_in_row_stride,
+                     const float *weight, const float *bias, const uint8_t *done,
+                     float *v_out, void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride,
+                     int64_t R, int T, int D, int time_major, void *stream);
+
+/*
+ * RG-LRU over a whole sequence: T recurrence steps per row in one pass.
+ *
+ * Replaces RGLRU.forward_sequence, models/yemong/griffin.py:188-219: the gate sigmoids, the
+ * decay a = sigmoid(log_lambda)^(c r), b = sqrt(clamp((1-a)(1+a), 1e-6)) (i x), the reset of
+ * a after an episode end (:213-218) and the Hillis-Steele scan (:25-64) that evaluates
+ * h_t = a_t h_{t-1} + b_t in log2(T) rounds over padded copies of a and b.  Here the
+ * recurrence is evaluated in time order with the state in registers, so a and b are never
+ * stored; results agree with the scan to fp32 rounding (the order of the multiply-adds
+ * differs).  Element arithmetic and roundings as in bnb_rglru_step_fwd.
+ *
+ *   x          (R, T, D) contiguous, x_dtype; with time_major != 0, x, gates_pre and y are
+ *              (T, R, .) instead; done stays (R, T)
+ *   gates_pre  (R, T, 2*D) contiguous, g_dtype: [linear_a(x) | linear_x(x)] per step
+ *   h0         (R, D) fp32 state before the sequence, row stride h0_row_stride floats
+ *   done       optional (R, T) bytes: non-zero at t makes step t+1 start from a zero state
+ *   y          (R, T, D) contiguous in y_dtype: every state h_0 .. h_{T-1}
+ *   h_last     (R, D) fp32 state after the sequence (= h_{T-1}); may equal h0
+ * T == 0 copies h0 to h_last.
+ */
+int bnb_rglru_scan_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
+                       const float *log_lambda, float c,
+                       const float *h0, int64_t h0_row_stride, const uint8_t *done,
+                       void *y, int y_dtype, float *h_last, int64_t h_last_row_stride,
+                       int64_t R, int T, int D, int time_major, void *stream);
 
 /*
  * Residual add + RMSNorm (+ the cast in front of the next projection) in one pass:

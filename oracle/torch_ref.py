@@ -22,6 +22,10 @@ How each function is pinned (see tests/test_oracle_pins.py):
                        perturbation invariance, permutation equivariance).
 * ``rglru_step``       closed forms from the recurrence (x=0, h=0, lambda=0
                        with r=1, r=0 => clamp floor) + the C restatement.
+* ``conv_sequence``    library ``F.conv1d`` (no boundaries) and per-episode ``F.conv1d`` on
+                       zero history (with boundaries).
+* ``rglru_sequence``   the log-depth scan == a plain loop of the pinned ``rglru_step`` with
+                       the state zeroed after each episode end; fp64 agreement to 1e-12.
 * ``temporal_step``    step == sequence, with the sequence path built on the
                        library ``F.conv1d`` (fixes tap order and buffer order).
 * ``field_step``, ``block_step``, ``pack/unpack/reset``  invariants the
@@ -171,6 +175,71 @@ def temporal_step(p: dict, prefix: str, x: torch.Tensor, h: torch.Tensor, conv_b
     x1 = x + F.linear(h_new * b2, p[prefix + "linear_out.weight"])
     x2 = x1 + gated_mlp(p, prefix + "gated_mlp.", rms_norm(x1, p[prefix + "norm2.weight"]))
     return x2, h_new, padded[:, 1:, :]
+
+
+def conv_sequence(b1: torch.Tensor, conv_buf: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None,
+                  done: torch.Tensor | None = None):
+    """Causal depthwise conv over (R,T,D) with the stored buffer as left padding.
+
+    Tap k of the (D,1,4) weight meets padded[:, t+k], i.e. the input ``3-k`` steps back
+    (griffin.py:127-139).  ``done[:, t]`` ends an episode at t: a tap is dropped when an
+    episode started between the input it reads and the output step; the stored buffer belongs
+    to the episode running at t = 0 (griffin.py:67-93).  Returns (v (R,T,D), last three
+    entries of the padded sequence), griffin.py:275-277.
+    """
+    R, T, D = b1.shape
+    padded = torch.cat([conv_buf, b1], dim=1)
+    w = weight.reshape(D, CONV_TAPS)
+    v = torch.zeros(R, T, D, dtype=padded.dtype)
+    if done is not None:
+        begins = torch.zeros(R, T + CONV_TAPS - 1, dtype=torch.long)  # 1 where a padded position opens an episode
+        begins[:, CONV_TAPS:] = done[:, :-1].long()
+        opened = begins.cumsum(dim=1)  # episodes opened up to and including each padded position
+    for k in range(CONV_TAPS):
+        tap = padded[:, k:k + T] * w[:, k]
+        if done is not None:
+            inside = opened[:, k:k + T] == opened[:, CONV_TAPS - 1:CONV_TAPS - 1 + T]
+            tap = tap * inside.unsqueeze(-1).to(tap.dtype)
+        v = v + tap
+    if bias is not None:
+        v = v + bias
+    return v, padded[:, -(CONV_TAPS - 1):, :]
+
+
+def rglru_sequence(x: torch.Tensor, gates_pre: torch.Tensor, log_lambda: torch.Tensor, c: float, h0: torch.Tensor,
+                   done: torch.Tensor | None = None):
+    """RG-LRU over (R,T,D) the way the reference evaluates it: per-step a_t, b_t, then a
+    log-depth inclusive scan of the pairs under (a2,b2)o(a1,b1) = (a2 a1, a2 b1 + b2).
+
+    Follows griffin.py:206-219 (coefficients; ``a`` is zeroed at the step after an episode
+    end) and :25-64 (the scan: pad T to a power of two with the identity (1,0), log2 rounds
+    of shifted combines, h_t = A_t h0 + B_t).  Returns (all states (R,T,D), last state).
+    """
+    R, T, D = x.shape
+    r = torch.sigmoid(gates_pre[..., :D])
+    i = torch.sigmoid(gates_pre[..., D:])
+    a = torch.sigmoid(log_lambda) ** (c * r)
+    b = torch.sqrt(torch.clamp((1.0 - a) * (1.0 + a), min=1e-6)) * (i * x)
+    if done is not None:
+        fresh = torch.zeros(R, T, dtype=torch.bool)
+        fresh[:, 1:] = done[:, :-1]
+        a = a.masked_fill(fresh.unsqueeze(-1), 0.0)
+    width = 1
+    while width < T:
+        width *= 2
+    A = torch.ones(R, width, D, dtype=a.dtype)
+    Bc = torch.zeros(R, width, D, dtype=b.dtype)
+    A[:, :T], Bc[:, :T] = a, b
+    span = 1
+    while span < width:
+        A_prev = torch.ones_like(A)
+        B_prev = torch.zeros_like(Bc)
+        A_prev[:, span:], B_prev[:, span:] = A[:, :-span], Bc[:, :-span]
+        Bc = A * B_prev + Bc  # uses the not yet updated A
+        A = A * A_prev
+        span *= 2
+    states = (A * h0.unsqueeze(1) + Bc)[:, :T]
+    return states, states[:, -1]
 
 
 def temporal_sequence(

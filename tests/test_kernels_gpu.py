@@ -581,3 +581,133 @@ def test_step_carried_rollout_with_dying_ships():
         ref_hidden, ref_state = torch_ref.harness_step(p32, tokens.float(), alive[t], ref_state)
         assert max_rel(hidden.float().cpu(), ref_hidden) <= BF16_TOL, t
     assert max_rel(dev_state.cpu(), ref_state) <= BF16_TOL
+
+
+# ------------------------------------------------------------------ sequence path: conv + recurrence over T
+
+
+def _seq_inputs(seed, R, T, D, x_dtype, g_dtype, p_done):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(R, T, D, generator=g).to(x_dtype)
+    gates = (2.0 * torch.randn(R, T, 2 * D, generator=g)).to(g_dtype)
+    h0 = torch.randn(R, D, generator=g)
+    done = (torch.rand(R, T, generator=g) < p_done) if p_done > 0 else None
+    return x, gates, h0, done
+
+
+# R * D/8 >= 131072 lanes takes the 8-channels-per-lane kernel, smaller inputs one lane per channel
+@pytest.mark.parametrize("R,T,D", [(5, 1, 128), (7, 2, 128), (9, 3, 64), (33, 7, 128), (16, 128, 128), (3, 130, 40),
+                                   (8192, 5, 128), (8200, 9, 128)])
+@pytest.mark.parametrize("p_done", [0.0, 0.2])
+def test_rglru_scan_fp32_matches_oracle(R, T, D, p_done):
+    x, gates, h0, done = _seq_inputs(R + T, R, T, D, torch.float32, torch.float32, p_done)
+    lam = torch.linspace(0.0, 4.0, D)
+    want, want_last = torch_ref.rglru_sequence(x, gates, lam, 8.0, h0, done)
+    y, last = ops.rglru_scan(x.to(DEV), gates.to(DEV), lam.to(DEV), 8.0, h0.to(DEV), None if done is None else done.to(DEV))
+    assert y.dtype == torch.float32 and y.shape == (R, T, D)
+    assert max_rel(y.cpu(), want) <= F32_TOL
+    assert max_rel(last.cpu(), want_last) <= F32_TOL
+    assert torch.equal(last.cpu(), y[:, -1].cpu())
+
+
+@pytest.mark.parametrize("R,T", [(6, 4), (40, 128), (8192, 6)])
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+def test_rglru_scan_bf16_gates_match_oracle(R, T, x_dtype):
+    D = 128
+    x, gates, h0, done = _seq_inputs(R * 3 + T, R, T, D, x_dtype, torch.bfloat16, 0.1)
+    lam = torch.linspace(0.0, 4.0, D)
+    want, want_last = torch_ref.rglru_sequence(x, gates, lam, 8.0, h0, done)  # torch's own promotion, as under autocast
+    assert want.dtype == torch.float32
+    for y_dtype in (torch.float32, torch.bfloat16):
+        y, last = ops.rglru_scan(x.to(DEV), gates.to(DEV), lam.to(DEV), 8.0, h0.to(DEV), done.to(DEV), y_dtype=y_dtype)
+        assert y.dtype == y_dtype
+        assert max_rel(y.float().cpu(), want) <= BF16_TOL
+        assert max_rel(last.cpu(), want_last) <= BF16_TOL
+
+
+def test_rglru_scan_equals_the_step_kernel_applied_t_times():
+    # same element arithmetic in both kernels: bit-identical states
+    R, T, D = 64, 12, 128
+    x, gates, h0, done = _seq_inputs(5, R, T, D, torch.float32, torch.bfloat16, 0.25)
+    lam = torch.linspace(0.0, 4.0, D).to(DEV)
+    xd, gd, dd = x.to(DEV), gates.to(DEV), done.to(DEV)
+    y, last = ops.rglru_scan(xd, gd, lam, 8.0, h0.to(DEV), dd)
+    h = h0.to(DEV)
+    for t in range(T):
+        reset = dd[:, t - 1].contiguous() if t > 0 else None
+        _, h = ops.rglru_step(xd[:, t].contiguous(), gd[:, t].contiguous(), lam, 8.0, h, reset=reset, rows_per_env=1)
+        assert torch.equal(h, y[:, t])
+    assert torch.equal(h, last)
+
+
+def test_rglru_scan_strided_state_and_in_place_final_state():
+    R, T, D = 10, 6, 128
+    x, gates, h0, _ = _seq_inputs(8, R, T, D, torch.float32, torch.float32, 0.0)
+    lam = torch.linspace(0.0, 4.0, D).to(DEV)
+    packed = torch.randn(R, 4 * D, device=DEV)
+    packed[:, :D] = h0.to(DEV)
+    before = packed.clone()
+    y, last = ops.rglru_scan(x.to(DEV), gates.to(DEV), lam, 8.0, packed[:, :D], h_out=packed[:, :D])
+    want, want_last = torch_ref.rglru_sequence(x, gates, lam.cpu(), 8.0, h0)
+    assert last.data_ptr() == packed.data_ptr()
+    assert max_rel(packed[:, :D].cpu(), want_last) <= F32_TOL
+    assert torch.equal(packed[:, D:], before[:, D:])
+
+
+@pytest.mark.parametrize("R,T,D", [(5, 1, 128), (7, 2, 128), (6, 3, 64), (33, 9, 128), (12, 128, 128), (3, 20, 40),
+                                   (8192, 5, 128)])
+@pytest.mark.parametrize("p_done", [0.0, 0.3])
+@pytest.mark.parametrize("b_dtype", [torch.float32, torch.bfloat16])
+def test_conv_seq_matches_oracle(R, T, D, p_done, b_dtype):
+    g = torch.Generator().manual_seed(R * 7 + T)
+    b1 = torch.randn(R, T, D, generator=g).to(b_dtype)
+    buf = torch.randn(R, 3, D, generator=g)
+    w = 0.5 * torch.randn(D, 1, 4, generator=g)
+    bias = 0.1 * torch.randn(D, generator=g)
+    done = (torch.rand(R, T, generator=g) < p_done) if p_done > 0 else None
+    want, want_tail = torch_ref.conv_sequence(b1.float(), buf, w, bias, done)
+    v, tail, v_lp = ops.conv_seq(b1.to(DEV), buf.to(DEV), w.to(DEV), bias.to(DEV), None if done is None else done.to(DEV),
+                                 also_bf16=True)
+    assert v.dtype == torch.float32 and v_lp.dtype == torch.bfloat16
+    assert max_rel(v.cpu(), want) <= F32_TOL
+    assert torch.equal(tail.cpu(), want_tail)
+    assert torch.equal(v_lp.cpu(), v.cpu().bfloat16())
+
+
+def test_conv_seq_equals_the_step_kernel_applied_t_times():
+    R, T, D = 32, 7, 128
+    g = torch.Generator().manual_seed(3)
+    b1 = torch.randn(R, T, D, generator=g).bfloat16().to(DEV)
+    buf = torch.randn(R, 3, D, generator=g).to(DEV)
+    w = (0.5 * torch.randn(D, 1, 4, generator=g)).to(DEV)
+    bias = (0.1 * torch.randn(D, generator=g)).to(DEV)
+    done = (torch.rand(R, T, generator=g) < 0.3).to(DEV)
+    v, tail = ops.conv_seq(b1, buf, w, bias, done)
+    cur = buf
+    for t in range(T):
+        reset = done[:, t - 1].contiguous() if t > 0 else None
+        vt, cur = ops.conv_step(b1[:, t].contiguous(), cur, w, bias, reset=reset, rows_per_env=1)
+        assert torch.equal(vt, v[:, t])
+    # the step path zeroes the stored inputs of a finished episode, the sequence path keeps the raw tail
+    raw_tail = torch.cat([buf, b1.float()], dim=1)[:, -3:]
+    assert torch.equal(tail, raw_tail)
+
+
+@pytest.mark.parametrize("R,T", [(12, 9), (8192, 4)])
+def test_sequence_kernels_time_major_layout_gives_the_same_numbers(R, T):
+    D = 128
+    x, gates, h0, done = _seq_inputs(77 + R, R, T, D, torch.float32, torch.bfloat16, 0.2)
+    lam = torch.linspace(0.0, 4.0, D).to(DEV)
+    xd, gd, dd, hd = x.to(DEV), gates.to(DEV), done.to(DEV), h0.to(DEV)
+    y, last = ops.rglru_scan(xd, gd, lam, 8.0, hd, dd, y_dtype=torch.bfloat16)
+    yt, last_t = ops.rglru_scan(xd.transpose(0, 1).contiguous(), gd.transpose(0, 1).contiguous(), lam, 8.0, hd, dd,
+                                y_dtype=torch.bfloat16, time_major=True)
+    assert yt.shape == (T, R, D)
+    assert torch.equal(yt.transpose(0, 1), y) and torch.equal(last_t, last)
+    g = torch.Generator().manual_seed(1)
+    buf = torch.randn(R, 3, D, generator=g).to(DEV)
+    w = torch.randn(D, 1, 4, generator=g).to(DEV)
+    bias = torch.randn(D, generator=g).to(DEV)
+    v, tail, v_lp = ops.conv_seq(xd, buf, w, bias, dd, also_bf16=True)
+    vt, tail_t, vt_lp = ops.conv_seq(xd.transpose(0, 1).contiguous(), buf, w, bias, dd, also_bf16=True, time_major=True)
+    assert torch.equal(vt.transpose(0, 1), v) and torch.equal(tail_t, tail) and torch.equal(vt_lp.transpose(0, 1), v_lp)

@@ -411,3 +411,102 @@ def test_harness_step_matches_its_parts():
     ships = u[:, :N].reshape(B * N, D)
     want = torch_ref.rglru_step(ships, torch_ref.rglru_gates(p, "", ships), p["log_lambda"], 8.0, state)
     assert torch.equal(new_state, want)
+
+
+# ---------------------------------------------------------------- sequence path (conv + scan over T)
+
+
+def _episode_conv_bruteforce(b1, conv_buf, weight, bias, done):
+    """Per row, per episode: library conv1d on that episode's inputs with zero history
+    (the stored buffer is the history of the episode running at t = 0)."""
+    R, T, D = b1.shape
+    out = torch.zeros(R, T, D, dtype=b1.dtype)
+    for r in range(R):
+        start = 0
+        hist = conv_buf[r]
+        for t in range(T):
+            last = t == T - 1 or bool(done[r, t])
+            if last:
+                seg = torch.cat([hist, b1[r, start:t + 1]], dim=0)  # (3 + len, D)
+                y = F.conv1d(seg.t().unsqueeze(0), weight, bias, groups=D)[0].t()
+                out[r, start:t + 1] = y
+                start = t + 1
+                hist = torch.zeros(3, D, dtype=b1.dtype)
+    return out
+
+
+@pytest.mark.parametrize("T", [1, 2, 3, 4, 9, 33])
+def test_conv_sequence_is_the_library_conv_without_boundaries(T):
+    g = torch.Generator().manual_seed(T)
+    R, D = 3, 8
+    b1 = torch.randn(R, T, D, generator=g, dtype=torch.float64)
+    buf = torch.randn(R, 3, D, generator=g, dtype=torch.float64)
+    w = torch.randn(D, 1, 4, generator=g, dtype=torch.float64)
+    bias = torch.randn(D, generator=g, dtype=torch.float64)
+    v, tail = torch_ref.conv_sequence(b1, buf, w, bias)
+    lib = F.conv1d(torch.cat([buf, b1], 1).transpose(1, 2), w, bias, groups=D).transpose(1, 2)
+    assert (v - lib).abs().max() < 1e-12
+    assert torch.equal(tail, torch.cat([buf, b1], 1)[:, -3:])
+    none_done = torch.zeros(R, T, dtype=torch.bool)
+    assert torch.equal(torch_ref.conv_sequence(b1, buf, w, bias, none_done)[0], v)
+
+
+@pytest.mark.parametrize("T,p", [(1, 0.5), (2, 0.5), (5, 0.4), (16, 0.3), (40, 0.1), (12, 1.0)])
+def test_conv_sequence_cuts_taps_at_episode_ends(T, p):
+    g = torch.Generator().manual_seed(100 + T)
+    R, D = 4, 6
+    b1 = torch.randn(R, T, D, generator=g, dtype=torch.float64)
+    buf = torch.randn(R, 3, D, generator=g, dtype=torch.float64)
+    w = torch.randn(D, 1, 4, generator=g, dtype=torch.float64)
+    bias = torch.randn(D, generator=g, dtype=torch.float64)
+    done = torch.rand(R, T, generator=g) < p
+    v, tail = torch_ref.conv_sequence(b1, buf, w, bias, done)
+    assert (v - _episode_conv_bruteforce(b1, buf, w, bias, done)).abs().max() < 1e-12
+    assert torch.equal(tail, torch.cat([buf, b1], 1)[:, -3:])  # the stored inputs are not cut
+    # a done flag at the last step changes nothing inside the sequence
+    d2 = done.clone()
+    d2[:, -1] = ~d2[:, -1]
+    assert torch.equal(torch_ref.conv_sequence(b1, buf, w, bias, d2)[0], v)
+
+
+def _loop_of_steps(x, gates, lam, c, h0, done):
+    h, ys = h0, []
+    for t in range(x.shape[1]):
+        if done is not None and t > 0:
+            h = h * (~done[:, t - 1]).to(h.dtype).unsqueeze(-1)
+        h = torch_ref.rglru_step(x[:, t], gates[:, t], lam, c, h)
+        ys.append(h)
+    return torch.stack(ys, dim=1)
+
+
+@pytest.mark.parametrize("T,p", [(1, 0.0), (2, 0.5), (3, 0.0), (7, 0.3), (128, 0.05), (130, 0.0), (64, 1.0)])
+def test_rglru_sequence_scan_equals_the_step_loop(T, p):
+    # tests/models/test_encoder.py:179-268 asserts the same at T = 1 and T = 128
+    g = torch.Generator().manual_seed(200 + T)
+    R, D = 3, 16
+    x = torch.randn(R, T, D, generator=g, dtype=torch.float64)
+    gates = 2.0 * torch.randn(R, T, 2 * D, generator=g, dtype=torch.float64)
+    lam = torch.linspace(0.0, 4.0, D, dtype=torch.float64)
+    h0 = torch.randn(R, D, generator=g, dtype=torch.float64)
+    done = (torch.rand(R, T, generator=g) < p) if p > 0 else None
+    ys, last = torch_ref.rglru_sequence(x, gates, lam, 8.0, h0, done)
+    want = _loop_of_steps(x, gates, lam, 8.0, h0, done)
+    assert (ys - want).abs().max() < 1e-12
+    assert torch.equal(last, ys[:, -1])
+    ys32, _ = torch_ref.rglru_sequence(x.float(), gates.float(), lam.float(), 8.0, h0.float(), done)
+    assert (ys32.double() - want).abs().max() < 2e-5
+
+
+def test_rglru_sequence_forgets_everything_after_an_episode_end():
+    g = torch.Generator().manual_seed(7)
+    R, T, D = 2, 10, 8
+    x = torch.randn(R, T, D, generator=g)
+    gates = torch.randn(R, T, 2 * D, generator=g)
+    lam = torch.linspace(0.0, 4.0, D)
+    done = torch.zeros(R, T, dtype=torch.bool)
+    done[:, 4] = True
+    a, _ = torch_ref.rglru_sequence(x, gates, lam, 8.0, torch.randn(R, D, generator=g), done)
+    x2 = x.clone()
+    x2[:, :5] += 3.0
+    b, _ = torch_ref.rglru_sequence(x2, gates, lam, 8.0, torch.randn(R, D, generator=g), done)
+    assert torch.equal(a[:, 5:], b[:, 5:]) and not torch.equal(a[:, :5], b[:, :5])

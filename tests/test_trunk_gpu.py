@@ -194,6 +194,30 @@ def test_temporal_block_sequence_with_done_matches_oracle_sequence():
     assert max_rel(h1.cpu(), ref_h) <= 2e-5 and torch.allclose(cb1.cpu(), ref_cb, atol=1e-5)
 
 
+@pytest.mark.parametrize("time_major", [False, True])
+def test_temporal_block_sequence_under_autocast_matches_oracle(time_major):
+    # the update path's precision: bf16 projections around fp32 conv and recurrence, T = 128
+    D, R, T = 128, 24, 128
+    gen = torch.Generator().manual_seed(18)
+    p = temporal_params(gen, "t.", D)
+    layer = bnb.GriffinTemporalBlock(D).eval()
+    layer.load_state_dict(_strip(p, "t."))
+    layer.to(DEV)
+    x_seq = torch.randn(R, T, D, generator=gen)
+    h0 = 0.5 * torch.randn(R, D, generator=gen)
+    cb = torch.randn(R, 3, D, generator=gen)
+    done = torch.rand(R, T, generator=gen) < 0.03
+    xin = x_seq.transpose(0, 1).contiguous() if time_major else x_seq
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        out, h1, cb1 = layer.forward_sequence(xin.to(DEV), h0.to(DEV), cb.to(DEV), done.to(DEV), time_major=time_major)
+    if time_major:
+        out = out.transpose(0, 1)
+    ref_out, ref_h, ref_cb = torch_ref.temporal_sequence(p, "t.", x_seq, h0, cb, done)
+    assert max_rel(out.float().cpu(), ref_out) <= BF16_TOL
+    assert max_rel(h1.cpu(), ref_h) <= BF16_TOL
+    assert max_rel(cb1.cpu(), ref_cb) <= BF16_TOL
+
+
 # ------------------------------------------------------------------ block and trunk
 
 
