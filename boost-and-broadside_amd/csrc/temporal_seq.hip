@@ -10,6 +10,8 @@
 // at t: step t+1 starts from a zero state (:213-218) and its conv taps do not reach back
 // across the boundary (:67-93).  Loads for several timesteps are issued before the
 // dependent arithmetic, so the sequential recurrence does not serialise the memory traffic.
+// The recurrence also has a backward kernel (reverse-time walk) so that the update path of
+// training can use it.
 
 #include "common.h"
 #include "rglru_math.h"
@@ -159,6 +161,251 @@ static int scan_dispatch_y(const void *x, const void *gates, const float *log_la
                                           T, D, time_major, stream);
     return launch_scan<XT, GT, uint16_t>(x, gates, log_lambda, c, h0, h0_stride, done, y, h_last, h_last_stride, R, T,
                                          D, time_major, stream);
+}
+
+// ------------------------------------------------------------------------------------
+// RG-LRU over T steps, backward
+// ------------------------------------------------------------------------------------
+//
+// Reverse-time walk with the running state gradient in registers:
+//   G_t   = dy_t + a'_{t+1} G_{t+1}            (a' = 0 across an episode boundary)
+//   da_t  = G_t h_{t-1}  (0 at a boundary)  -  [s_t > 1e-6] G_t (i x)_t a_t / g_t
+//   d(ix) = G_t g_t,  dx = d(ix) i,  di = d(ix) x
+//   d ga  = da a ln(sigmoid(lambda)) c r (1 - r),   d gx = di i (1 - i)
+//   d lambda += da a (c r) (1 - sigmoid(lambda))
+// r, i, a, g are recomputed from the saved inputs exactly as the forward computed them
+// (roundings included); h_{t-1} is read from the saved states.
+
+struct RglruGrad {
+    float dx, dga, dgx, dlam, carry;
+};
+
+template <bool G_BF16, bool X_BF16>
+__device__ __forceinline__ RglruGrad rglru_element_bwd(float x, float ga, float gx, float l2sig, float one_minus_sig,
+                                                        float c, float h_prev, float G)
+{
+    float r = fast_sigmoid(ga);
+    float i = fast_sigmoid(gx);
+    float cr = c * r;
+    if (G_BF16) {
+        r = round_to_bf16(r);
+        i = round_to_bf16(i);
+        cr = round_to_bf16(c * r);
+    }
+    const float a = __builtin_amdgcn_exp2f(cr * l2sig);
+    const float s = (1.0f - a) * (1.0f + a);
+    const float gate = __builtin_amdgcn_sqrtf(fmaxf(s, 1e-6f));
+    float ix = i * x;
+    if (G_BF16 && X_BF16) ix = round_to_bf16(ix);
+    float da = G * h_prev;
+    if (s > 1e-6f) da -= G * ix * a * __builtin_amdgcn_rcpf(gate);
+    const float dix = G * gate;
+    RglruGrad out;
+    out.dx = dix * i;
+    out.dgx = dix * x * i * (1.0f - i);
+    const float da_a = da * a;
+    out.dga = da_a * (l2sig * 0.6931471805599453f) * c * r * (1.0f - r);
+    out.dlam = da_a * cr * one_minus_sig;
+    out.carry = a * G;
+    return out;
+}
+
+// 1 - sigmoid(lambda) = sigmoid(-lambda)
+__device__ __forceinline__ float sigmoid_neg(float lam) { return 1.0f / (1.0f + expf(lam)); }
+
+template <typename XT, typename GT, typename YT>
+__global__ __launch_bounds__(kSeqThreads) void rglru_scan_bwd_scalar_kernel(
+    const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
+    const float *__restrict__ h0, int64_t h0_stride, const uint8_t *__restrict__ done, const YT *__restrict__ y,
+    const YT *__restrict__ dy, const float *__restrict__ dh_last, int64_t dh_last_stride, XT *__restrict__ dx,
+    GT *__restrict__ dgates, float *__restrict__ dh0, float *__restrict__ dlam_rows, int64_t R, int T, int D,
+    int64_t rs, int64_t ts)
+{
+    const int64_t idx = (int64_t)blockIdx.x * kSeqThreads + threadIdx.x;
+    if (idx >= R * D) return;
+    const int64_t row = idx / D;
+    const int d = (int)(idx - row * D);
+    const float lam = log_lambda[d];
+    const float l2 = log2_sigmoid(lam), oms = sigmoid_neg(lam);
+    const XT *xp = x + row * rs + d;
+    const GT *gp = gates + row * 2 * rs + d;
+    const YT *yp = y + row * rs + d;
+    const YT *dyp = dy == nullptr ? nullptr : dy + row * rs + d;
+    XT *dxp = dx + row * rs + d;
+    GT *dgp = dgates + row * 2 * rs + d;
+    const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
+    const float h_first = h0[row * h0_stride + d];
+    float carry = dh_last == nullptr ? 0.0f : dh_last[row * dh_last_stride + d];
+    float dlam = 0.0f;
+    for (int t1 = T; t1 > 0; t1 -= kSeqAhead) {
+        float xv[kSeqAhead], ga[kSeqAhead], gx[kSeqAhead], dyv[kSeqAhead], hp[kSeqAhead];
+        uint32_t cut[kSeqAhead];
+#pragma unroll
+        for (int u = 0; u < kSeqAhead; ++u) {
+            const int t = t1 - 1 - u > 0 ? t1 - 1 - u : 0;  // before the start: re-read step 0 (discarded)
+            xv[u] = load1(xp + t * ts);
+            ga[u] = load1(gp + t * 2 * ts);
+            gx[u] = load1(gp + t * 2 * ts + D);
+            dyv[u] = dyp == nullptr ? 0.0f : load1(dyp + t * ts);
+            hp[u] = load1(yp + (t > 0 ? t - 1 : 0) * ts);
+            cut[u] = 0;
+            if (dn != nullptr) cut[u] = dn[t > 0 ? t - 1 : 0];
+            if (t == 0) {
+                cut[u] = 0;
+                hp[u] = h_first;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kSeqAhead; ++u) {
+            const int t = t1 - 1 - u;
+            if (t >= 0) {
+                const float G = dyv[u] + carry;
+                const RglruGrad g = rglru_element_bwd<is_bf16<GT>::value, is_bf16<XT>::value>(
+                    xv[u], ga[u], gx[u], l2, oms, c, cut[u] ? 0.0f : hp[u], G);
+                store1(dxp + t * ts, g.dx);
+                store1(dgp + t * 2 * ts, g.dga);
+                store1(dgp + t * 2 * ts + D, g.dgx);
+                dlam += g.dlam;
+                carry = cut[u] ? 0.0f : g.carry;
+            }
+        }
+    }
+    dh0[row * D + d] = carry;
+    dlam_rows[row * D + d] = dlam;
+}
+
+template <typename XT, typename GT, typename YT>
+__global__ __launch_bounds__(kSeqThreads) void rglru_scan_bwd_vec8_kernel(
+    const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
+    const float *__restrict__ h0, int64_t h0_stride, const uint8_t *__restrict__ done, const YT *__restrict__ y,
+    const YT *__restrict__ dy, const float *__restrict__ dh_last, int64_t dh_last_stride, XT *__restrict__ dx,
+    GT *__restrict__ dgates, float *__restrict__ dh0, float *__restrict__ dlam_rows, int64_t R, int T, int D,
+    int64_t rs, int64_t ts, int rows_per_block)
+{
+    extern __shared__ float s_lam[];  // D entries of log2 sigmoid(lambda), then D of 1 - sigmoid(lambda)
+    for (int d = threadIdx.x; d < D; d += kSeqThreads) {
+        const float lam = log_lambda[d];
+        s_lam[d] = log2_sigmoid(lam);
+        s_lam[D + d] = sigmoid_neg(lam);
+    }
+    __syncthreads();
+
+    const int vecs_per_row = D >> 3;
+    const int local_row = threadIdx.x / vecs_per_row;
+    const int64_t row = (int64_t)blockIdx.x * rows_per_block + local_row;
+    if (local_row >= rows_per_block || row >= R) return;
+    const int d0 = (threadIdx.x - local_row * vecs_per_row) << 3;
+
+    float l2[8], oms[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        l2[e] = s_lam[d0 + e];
+        oms[e] = s_lam[D + d0 + e];
+    }
+    const XT *xp = x + row * rs + d0;
+    const GT *gp = gates + row * 2 * rs + d0;
+    const YT *yp = y + row * rs + d0;
+    const YT *dyp = dy == nullptr ? nullptr : dy + row * rs + d0;
+    XT *dxp = dx + row * rs + d0;
+    GT *dgp = dgates + row * 2 * rs + d0;
+    const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
+    const Row8 h_first = load8(h0 + row * h0_stride + d0);
+    Row8 carry, dlam;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) carry.v[e] = dlam.v[e] = 0.0f;
+    if (dh_last != nullptr) carry = load8(dh_last + row * dh_last_stride + d0);
+
+    constexpr int AHEAD = 2;  // five operand rows per step: keep the register footprint moderate
+    for (int t1 = T; t1 > 0; t1 -= AHEAD) {
+        Row8 xv[AHEAD], ga[AHEAD], gx[AHEAD], dyv[AHEAD], hp[AHEAD];
+        uint32_t cut[AHEAD];
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u) {
+            const int t = t1 - 1 - u > 0 ? t1 - 1 - u : 0;
+            xv[u] = load8_stream(xp + t * ts);
+            ga[u] = load8_stream(gp + t * 2 * ts);
+            gx[u] = load8_stream(gp + t * 2 * ts + D);
+            if (dyp != nullptr) {
+                dyv[u] = load8_stream(dyp + t * ts);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) dyv[u].v[e] = 0.0f;
+            }
+            hp[u] = load8(yp + (t > 0 ? t - 1 : 0) * ts);
+            cut[u] = 0;
+            if (dn != nullptr) cut[u] = dn[t > 0 ? t - 1 : 0];
+            if (t == 0) {
+                cut[u] = 0;
+                hp[u] = h_first;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u) {
+            const int t = t1 - 1 - u;
+            if (t >= 0) {
+                Row8 ox, oa, og;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float G = dyv[u].v[e] + carry.v[e];
+                    const RglruGrad g = rglru_element_bwd<is_bf16<GT>::value, is_bf16<XT>::value>(
+                        xv[u].v[e], ga[u].v[e], gx[u].v[e], l2[e], oms[e], c, cut[u] ? 0.0f : hp[u].v[e], G);
+                    ox.v[e] = g.dx;
+                    oa.v[e] = g.dga;
+                    og.v[e] = g.dgx;
+                    dlam.v[e] += g.dlam;
+                    carry.v[e] = cut[u] ? 0.0f : g.carry;
+                }
+                store8_stream(dxp + t * ts, ox);
+                store8_stream(dgp + t * 2 * ts, oa);
+                store8_stream(dgp + t * 2 * ts + D, og);
+            }
+        }
+    }
+    store8(dh0 + row * D + d0, carry);
+    store8(dlam_rows + row * D + d0, dlam);
+}
+
+template <typename XT, typename GT, typename YT>
+static int launch_scan_bwd(const void *x, const void *gates, const float *log_lambda, float c, const float *h0,
+                           int64_t h0_stride, const uint8_t *done, const void *y, const void *dy,
+                           const float *dh_last, int64_t dh_last_stride, void *dx, void *dgates, float *dh0,
+                           float *dlam_rows, int64_t R, int T, int D, int time_major, hipStream_t stream)
+{
+    const int64_t rs = time_major ? D : (int64_t)T * D, ts = time_major ? R * D : D;
+    const bool vec_ok = (D % 8 == 0) && (D / 8 <= kSeqThreads) && aligned16(x) && aligned16(gates) && aligned16(h0) &&
+                        aligned16(y) && aligned16(dy) && aligned16(dh_last) && aligned16(dx) && aligned16(dgates) &&
+                        aligned16(dh0) && aligned16(dlam_rows) && (h0_stride % 4 == 0) && (dh_last_stride % 4 == 0);
+    const bool vec = vec_ok && R * (D / 8) >= (int64_t)256 * kSeqThreads * 2;
+    if (vec) {
+        const int rows_per_block = kSeqThreads / (D / 8);
+        const int64_t blocks = (R + rows_per_block - 1) / rows_per_block;
+        if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL((rglru_scan_bwd_vec8_kernel<XT, GT, YT>), dim3((unsigned)blocks), dim3(kSeqThreads),
+                           (size_t)2 * D * sizeof(float), stream, (const XT *)x, (const GT *)gates, log_lambda, c, h0,
+                           h0_stride, done, (const YT *)y, (const YT *)dy, dh_last, dh_last_stride, (XT *)dx,
+                           (GT *)dgates, dh0, dlam_rows, R, T, D, rs, ts, rows_per_block);
+    } else {
+        const int64_t blocks = (R * D + kSeqThreads - 1) / kSeqThreads;
+        if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL((rglru_scan_bwd_scalar_kernel<XT, GT, YT>), dim3((unsigned)blocks), dim3(kSeqThreads), 0,
+                           stream, (const XT *)x, (const GT *)gates, log_lambda, c, h0, h0_stride, done,
+                           (const YT *)y, (const YT *)dy, dh_last, dh_last_stride, (XT *)dx, (GT *)dgates, dh0,
+                           dlam_rows, R, T, D, rs, ts);
+    }
+    return (int)hipGetLastError();
+}
+
+template <typename XT, typename GT>
+static int scan_bwd_dispatch_y(const void *x, const void *gates, const float *log_lambda, float c, const float *h0,
+                               int64_t h0_stride, const uint8_t *done, const void *y, int y_dtype, const void *dy,
+                               const float *dh_last, int64_t dh_last_stride, void *dx, void *dgates, float *dh0,
+                               float *dlam_rows, int64_t R, int T, int D, int time_major, hipStream_t stream)
+{
+    if (y_dtype == BNB_F32)
+        return launch_scan_bwd<XT, GT, float>(x, gates, log_lambda, c, h0, h0_stride, done, y, dy, dh_last,
+                                              dh_last_stride, dx, dgates, dh0, dlam_rows, R, T, D, time_major, stream);
+    return launch_scan_bwd<XT, GT, uint16_t>(x, gates, log_lambda, c, h0, h0_stride, done, y, dy, dh_last,
+                                             dh_last_stride, dx, dgates, dh0, dlam_rows, R, T, D, time_major, stream);
 }
 
 // ------------------------------------------------------------------------------------
@@ -345,6 +592,44 @@ extern "C" int bnb_rglru_scan_fwd(const void *x, int x_dtype, const void *gates_
                                                 h_last, h_last_row_stride, R, T, D, time_major != 0, s);
     return scan_dispatch_y<uint16_t, float>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype, h_last,
                                             h_last_row_stride, R, T, D, time_major != 0, s);
+}
+
+extern "C" int bnb_rglru_scan_bwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
+                                  const float *log_lambda, float c, const float *h0, int64_t h0_row_stride,
+                                  const uint8_t *done, const void *y, int y_dtype, const void *dy,
+                                  const float *dh_last, int64_t dh_last_row_stride, void *dx, void *dgates,
+                                  float *dh0, float *dlam_rows, int64_t R, int T, int D, int time_major,
+                                  void *stream)
+{
+    using namespace bnb;
+    if (R < 0 || T < 1 || D < 1) return BNB_ERR_BAD_SHAPE;
+    if (R == 0) return 0;
+    if (!x || !gates_pre || !log_lambda || !h0 || !y || !dx || !dgates || !dh0 || !dlam_rows)
+        return BNB_ERR_NULL_POINTER;
+    if (h0_row_stride < D || (dh_last && dh_last_row_stride < D)) return BNB_ERR_BAD_SHAPE;
+    if ((x_dtype != BNB_F32 && x_dtype != BNB_BF16) || (g_dtype != BNB_F32 && g_dtype != BNB_BF16) ||
+        (y_dtype != BNB_F32 && y_dtype != BNB_BF16))
+        return BNB_ERR_BAD_DTYPE;
+    if ((reinterpret_cast<uintptr_t>(h0) | reinterpret_cast<uintptr_t>(dh_last) | reinterpret_cast<uintptr_t>(dh0) |
+         reinterpret_cast<uintptr_t>(dlam_rows) | reinterpret_cast<uintptr_t>(log_lambda)) & 3u)
+        return BNB_ERR_MISALIGNED;
+    hipStream_t s = (hipStream_t)stream;
+    const bool xb = x_dtype == BNB_BF16, gb = g_dtype == BNB_BF16;
+    if (!xb && !gb)
+        return scan_bwd_dispatch_y<float, float>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype, dy,
+                                                 dh_last, dh_last_row_stride, dx, dgates, dh0, dlam_rows, R, T, D,
+                                                 time_major != 0, s);
+    if (xb && gb)
+        return scan_bwd_dispatch_y<uint16_t, uint16_t>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y,
+                                                       y_dtype, dy, dh_last, dh_last_row_stride, dx, dgates, dh0,
+                                                       dlam_rows, R, T, D, time_major != 0, s);
+    if (!xb && gb)
+        return scan_bwd_dispatch_y<float, uint16_t>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype,
+                                                    dy, dh_last, dh_last_row_stride, dx, dgates, dh0, dlam_rows, R, T,
+                                                    D, time_major != 0, s);
+    return scan_bwd_dispatch_y<uint16_t, float>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype, dy,
+                                                dh_last, dh_last_row_stride, dx, dgates, dh0, dlam_rows, R, T, D,
+                                                time_major != 0, s);
 }
 
 extern "C" int bnb_conv_seq_fwd(const void *b1, int b1_dtype, const float *conv_in, int64_t conv_in_row_stride,

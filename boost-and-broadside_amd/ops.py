@@ -464,10 +464,14 @@ def rglru_scan(
         raise ValueError(f"log_lambda must be a float32 {(D,)} tensor")
     for name, t in (("x", x), ("gates_pre", gates_pre), ("h0", h0), ("log_lambda", log_lambda)):
         _need_device(t, name)
-    if torch.is_grad_enabled() and (x.requires_grad or gates_pre.requires_grad or h0.requires_grad or log_lambda.requires_grad):
-        raise RuntimeError("rglru_scan is forward-only; call it under torch.no_grad()")
     if y_dtype not in _DTYPE_CODE:
         raise TypeError(f"y_dtype must be float32 or bfloat16, got {y_dtype}")
+    if torch.is_grad_enabled() and (x.requires_grad or gates_pre.requires_grad or h0.requires_grad or log_lambda.requires_grad):
+        # training: forward and backward kernels behind autograd
+        if y_dtype != torch.float32 or h_out is not None:
+            raise RuntimeError("rglru_scan under autograd returns float32 states and owns its outputs")
+        keep, _ = _done_pointer(done, R, T, x.device)
+        return _RglruScan.apply(x, gates_pre, log_lambda, h0, keep, float(c), bool(time_major))
     x_code, g_code = _code(x, "x"), _code(gates_pre, "gates_pre")
     x = x.contiguous()
     gates_pre = gates_pre.contiguous()
@@ -490,6 +494,43 @@ def rglru_scan(
         _native.check(rc, "bnb_rglru_scan_fwd")
     del keep
     return y, h_out
+
+
+class _RglruScan(torch.autograd.Function):
+    """``rglru_scan`` with a backward: one reverse-time kernel pass instead of autograd through
+    the per-step coefficient chain and a log-depth scan."""
+
+    @staticmethod
+    def forward(ctx, x, gates_pre, log_lambda, h0, done, c, time_major):
+        with torch.no_grad():
+            y, h_last = rglru_scan(x, gates_pre, log_lambda, c, h0, done, time_major=time_major)
+        ctx.save_for_backward(x, gates_pre, log_lambda, h0, y)
+        ctx.done, ctx.c, ctx.time_major = done, c, time_major
+        return y, h_last
+
+    @staticmethod
+    def backward(ctx, dy, dh_last):
+        x, gates_pre, log_lambda, h0, y = ctx.saved_tensors
+        T, R = (x.shape[0], x.shape[1]) if ctx.time_major else (x.shape[1], x.shape[0])
+        D = x.shape[2]
+        x_c, g_c = x.contiguous(), gates_pre.contiguous()
+        h0_c = h0 if h0.stride(1) == 1 else h0.contiguous()
+        dy = dy.contiguous()
+        dh_last = dh_last.contiguous()
+        dx = torch.empty_like(x_c)
+        dgates = torch.empty_like(g_c)
+        dh0 = torch.empty((R, D), dtype=torch.float32, device=x.device)
+        dlam_rows = torch.empty((R, D), dtype=torch.float32, device=x.device)
+        done_ptr = None if ctx.done is None else ctx.done.data_ptr()
+        with torch.cuda.device(x.device):
+            rc = _native.load().bnb_rglru_scan_bwd(
+                x_c.data_ptr(), _DTYPE_CODE[x.dtype], g_c.data_ptr(), _DTYPE_CODE[gates_pre.dtype],
+                log_lambda.data_ptr(), ctx.c, h0_c.data_ptr(), h0_c.stride(0), done_ptr, y.data_ptr(),
+                _DTYPE_CODE[y.dtype], dy.data_ptr(), dh_last.data_ptr(), dh_last.stride(0), dx.data_ptr(),
+                dgates.data_ptr(), dh0.data_ptr(), dlam_rows.data_ptr(), R, T, D, int(ctx.time_major), _stream(),
+            )
+        _native.check(rc, "bnb_rglru_scan_bwd")
+        return dx, dgates, dlam_rows.sum(dim=0), dh0, None, None, None
 
 
 _F32_EPS = float(torch.finfo(torch.float32).eps)

@@ -48,7 +48,7 @@ def _fused_ok(x: torch.Tensor, act: torch.dtype) -> bool:
     """Whether the fused norm / gelu kernels apply: fp32 residual stream on the GPU, a covered
     width, fp32 or bf16 projections.  Anything else takes the plain torch composition."""
     return (
-        x.is_cuda and x.dtype == torch.float32 and x.shape[-1] in _FUSED_WIDTHS
+        not torch.is_grad_enabled() and x.is_cuda and x.dtype == torch.float32 and x.shape[-1] in _FUSED_WIDTHS
         and act in (torch.float32, torch.bfloat16)
     )
 
@@ -69,6 +69,8 @@ def _cached_cast(owner: nn.Module, slot: str, tensors: tuple, dtype: torch.dtype
 def _project(layer: nn.Linear, x: torch.Tensor) -> torch.Tensor:
     """``layer(x)`` for an activation that already has the projection dtype."""
     w, b = layer.weight, layer.bias
+    if torch.is_grad_enabled():
+        return layer(x)  # training: autocast's own (differentiable) casts
     if x.dtype == w.dtype:
         return F.linear(x, w, b)
     wc = _cached_cast(layer, "_bnb_w", (w,), x.dtype, lambda: w.detach().to(x.dtype))
@@ -122,9 +124,7 @@ class GatedMLP(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         hidden = self.gate_proj.out_features
-        if not x.is_cuda or hidden % 8 or x.dtype not in (torch.float32, torch.bfloat16) or (
-            torch.is_grad_enabled() and x.requires_grad
-        ):
+        if not x.is_cuda or hidden % 8 or x.dtype not in (torch.float32, torch.bfloat16) or torch.is_grad_enabled():
             return self.down_proj(F.gelu(self.gate_proj(x)) * self.up_proj(x))
         # one GEMM for [gate | up], one kernel for gelu(gate) * up, one GEMM down
         wg, wu = self.gate_proj.weight, self.up_proj.weight
@@ -168,6 +168,13 @@ class TransformerBlock(nn.Module):
 
     def _attn(self, x, alive_mask, bullets=None, bullet_mask=None):
         qkv = _project(self.qkv, x)  # (B, N, 3D), fp32 or bf16 under autocast
+        if torch.is_grad_enabled():
+            # training: the attention itself stays with torch's differentiable SDPA
+            merged = self._self_attention_autograd(qkv, alive_mask)
+            if self.reads_bullets and bullets is not None:
+                kv = self.kv_bullet(self.norm_bullet(bullets))
+                merged = merged + self._bullet_read(qkv, kv, bullet_mask)
+            return self.out_proj(merged)
         merged = ops.sdpa_masked(qkv, alive_mask, self.n_heads)  # (B, N, D) head-major
         if self.reads_bullets and bullets is not None:
             kv = _project(self.kv_bullet, self._norm_bullets(bullets, qkv.dtype))
@@ -176,6 +183,18 @@ class TransformerBlock(nn.Module):
             else:
                 merged = merged + self._bullet_read(qkv, kv, bullet_mask)
         return _project(self.out_proj, merged)
+
+    def _self_attention_autograd(self, qkv, alive_mask):
+        """Masked self-attention as the reference composes it (attention.py:136-147,168)."""
+        B, N, _ = qkv.shape
+        H, dh, D = self.n_heads, self.head_dim, self.d_model
+        q, k, v = (t.reshape(B, N, H, dh).transpose(1, 2) for t in qkv.split(D, dim=-1))
+        bias = None
+        if alive_mask is not None:
+            keep = alive_mask.reshape(B, 1, 1, N).to(q.dtype)
+            bias = (1.0 - keep) * (torch.finfo(q.dtype).min / 2)
+        o = F.scaled_dot_product_attention(q, k, v, attn_mask=bias, dropout_p=0.0)
+        return o.transpose(1, 2).reshape(B, N, D)
 
     def _norm_bullets(self, bullets, act):
         """norm_bullet(bullets) in the projection dtype."""
@@ -219,6 +238,8 @@ class RGLRU(nn.Module):
         """``[linear_a(x) | linear_x(x)]`` as one (R, 2D) GEMM over concatenated weights.
 
         ``x_act``: the same rows already in the projection dtype (saves the cast)."""
+        if torch.is_grad_enabled():
+            return torch.cat([self.linear_a(x), self.linear_x(x)], dim=-1)
         act = _projection_dtype()
         if x_act is None or x_act.dtype != act:
             x_act = x.to(act)
@@ -283,6 +304,8 @@ class GriffinTemporalBlock(nn.Module):
             x = x_seq[:, 0]
             out, new_h, new_conv_buf = self._step(x, h0, conv_buf, None, None, None, 1)
             return out.unsqueeze(1), new_h, new_conv_buf
+        if torch.is_grad_enabled():
+            return self._sequence_autograd(x_seq, h0, conv_buf, done_mask, time_major)
         # two passes over the sequence: conv taps (cut at episode ends), then the recurrence;
         # the only tensors in between are the conv output and the gate pre-activations
         act = _projection_dtype()
@@ -295,6 +318,20 @@ class GriffinTemporalBlock(nn.Module):
                                                 y_dtype=act if _fused_ok(x_seq, act) else torch.float32,
                                                 x_act=res[2] if want_lp else None)
         return self._finish(x_seq, normed, y), new_h, res[1]
+
+    def _sequence_autograd(self, x_seq, h0, conv_buf, done_mask, time_major):
+        """Training path: torch ops (differentiable) around the recurrence, which runs on its
+        forward and backward kernels."""
+        normed = self.norm1(x_seq)
+        b1 = self.linear1(normed)
+        rows_first = b1.transpose(0, 1) if time_major else b1  # (R, T, D) view
+        T = rows_first.shape[1]
+        padded = torch.cat([conv_buf, rows_first], dim=1)  # fp32 buffer promotes a bf16 b1
+        v = _conv_within_episodes(padded, self.conv.weight.squeeze(1), self.conv.bias, done_mask)
+        if time_major:
+            v = v.transpose(0, 1).contiguous()
+        y, new_h = self.rg_lru.forward_sequence(v, h0, done_mask, time_major=time_major)
+        return self._finish(x_seq, normed, y), new_h, padded[:, T:]
 
     def _norm_in(self, x):
         """norm1(x) in the projection dtype (one kernel with the cast when the fused path applies)."""
@@ -356,6 +393,28 @@ class GriffinTemporalBlock(nn.Module):
             return x1 + self.gated_mlp(n2)
         x1 = x + self.linear_out(b1 * F.gelu(gate_in))
         return x1 + self.gated_mlp(self.norm2(x1))
+
+
+def _conv_within_episodes(padded, w, bias, done_mask):
+    """Depthwise causal conv whose taps stop at episode ends (griffin.py:67-140), in torch ops.
+
+    ``padded`` (R, T+3, D), ``w`` (D, 4).  ``done_mask[:, t]`` ends an episode at t.  A tap
+    contributes to output t only if the input it reads lies in the same episode as t; the
+    stored buffer counts as belonging to the episode running at t = 0.
+    """
+    T = padded.shape[1] - (CONV_KERNEL - 1)
+    if done_mask is None:
+        return sum(padded[:, k:k + T] * w[:, k] for k in range(CONV_KERNEL)) + bias
+    R = done_mask.shape[0]
+    starts = torch.zeros_like(done_mask, dtype=torch.long)
+    starts[:, 1:] = done_mask[:, :-1].long()
+    episode = torch.cat([starts.new_zeros(R, CONV_KERNEL - 1), starts.cumsum(dim=1)], dim=1)  # (R, T+3)
+    here = episode[:, CONV_KERNEL - 1:]
+    out = 0
+    for k in range(CONV_KERNEL):
+        same = (episode[:, k:k + T] == here).to(padded.dtype).unsqueeze(-1)
+        out = out + padded[:, k:k + T] * w[:, k] * same
+    return out + bias
 
 
 class YemongBlock(nn.Module):
@@ -424,7 +483,11 @@ class YemongBlock(nn.Module):
 
     def sequence(self, x, alive_mask, h0, conv_buf0, done_mask=None, num_recurrent=None, bullets=None,
                  bullet_mask=None):
-        """(T,B,NM,D) variant of ``step`` for re-evaluating a stored rollout (no gradients)."""
+        """(T,B,NM,D) variant of ``step`` for re-evaluating a stored rollout.
+
+        Under ``torch.no_grad()`` every sublayer runs on the kernels.  With gradients enabled
+        (the PPO update) the projections, norms, attention and conv are torch ops and the
+        recurrence runs on its forward and backward kernels."""
         T, B, NM, D = x.shape
         n_rec = NM if num_recurrent is None else num_recurrent
         for layer in self.spatial:

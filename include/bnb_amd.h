@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 5
+#define BNB_ABI_VERSION 6
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -244,6 +244,31 @@ int bnb_rglru_scan_fwd(const void *x, int x_dtype, const void *gates_pre, int g_
                        const float *log_lambda, float c,
                        const float *h0, int64_t h0_row_stride, const uint8_t *done,
                        void *y, int y_dtype, float *h_last, int64_t h_last_row_stride,
+                       int64_t R, int T, int D, int time_major, void *stream);
+
+/*
+ * Backward of bnb_rglru_scan_fwd: what autograd computes through the reference's coefficient
+ * chain and log-depth scan (models/yemong/griffin.py:206-219, :25-64), as one reverse-time
+ * pass.  The forward's inputs and its states y are passed back in; r, i, a and the gate are
+ * recomputed from them.
+ *
+ *   x, gates_pre, log_lambda, c, h0, done, time_major   as given to the forward
+ *   y          the forward's states, y_dtype (float32 keeps h_{t-1} exact)
+ *   dy         gradient of y, same dtype and layout as y, or NULL (zero)
+ *   dh_last    optional (R, D) fp32 gradient of the final state
+ *   dx         out, x's dtype and layout
+ *   dgates     out, gates_pre's dtype and layout: [d linear_a | d linear_x]
+ *   dh0        out (R, D) fp32 contiguous
+ *   dlam_rows  out (R, D) fp32 contiguous: each row's contribution to d log_lambda; the
+ *              caller sums over rows (kept separate so that the sum has a fixed order)
+ * Requirements: T >= 1.
+ */
+int bnb_rglru_scan_bwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
+                       const float *log_lambda, float c,
+                       const float *h0, int64_t h0_row_stride, const uint8_t *done,
+                       const void *y, int y_dtype, const void *dy,
+                       const float *dh_last, int64_t dh_last_row_stride,
+                       void *dx, void *dgates, float *dh0, float *dlam_rows,
                        int64_t R, int T, int D, int time_major, void *stream);
 
 /*

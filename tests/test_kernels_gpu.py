@@ -711,3 +711,52 @@ def test_sequence_kernels_time_major_layout_gives_the_same_numbers(R, T):
     v, tail, v_lp = ops.conv_seq(xd, buf, w, bias, dd, also_bf16=True)
     vt, tail_t, vt_lp = ops.conv_seq(xd.transpose(0, 1).contiguous(), buf, w, bias, dd, also_bf16=True, time_major=True)
     assert torch.equal(vt.transpose(0, 1), v) and torch.equal(tail_t, tail) and torch.equal(vt_lp.transpose(0, 1), v_lp)
+
+
+# ------------------------------------------------------------------ recurrence backward
+
+
+def _scan_grads_oracle(x, gates, lam, h0, done, wy, wl, dtype64=True):
+    """Gradients of sum(y*wy) + sum(h_last*wl) through the oracle's scan, by torch autograd."""
+    up = (lambda t: t.double()) if dtype64 else (lambda t: t.clone())
+    leaves = [up(t).requires_grad_(True) for t in (x, gates, lam, h0)]
+    y, last = torch_ref.rglru_sequence(leaves[0], leaves[1], leaves[2], 8.0, leaves[3], done)
+    ((y * up(wy)).sum() + (last * up(wl)).sum()).backward()
+    return [t.grad for t in leaves]
+
+
+@pytest.mark.parametrize("R,T,D", [(4, 1, 128), (6, 5, 64), (9, 128, 128), (3, 7, 40), (8192, 6, 128)])
+@pytest.mark.parametrize("p_done", [0.0, 0.2])
+@pytest.mark.parametrize("time_major", [False, True])
+def test_rglru_scan_backward_fp32_matches_autograd_of_the_oracle(R, T, D, p_done, time_major):
+    x, gates, h0, done = _seq_inputs(R * 5 + T, R, T, D, torch.float32, torch.float32, p_done)
+    g = torch.Generator().manual_seed(T)
+    wy, wl = torch.randn(R, T, D, generator=g), torch.randn(R, D, generator=g)
+    lam = torch.linspace(0.0, 4.0, D)
+    want = _scan_grads_oracle(x, gates, lam, h0, done, wy, wl)
+    lay = (lambda t: t.transpose(0, 1).contiguous()) if time_major else (lambda t: t)
+    leaves = [t.to(DEV).requires_grad_(True) for t in (lay(x), lay(gates), lam, h0)]
+    y, last = ops.rglru_scan(leaves[0], leaves[1], leaves[2], 8.0, leaves[3], None if done is None else done.to(DEV),
+                             time_major=time_major)
+    ((y * lay(wy).to(DEV)).sum() + (last * wl.to(DEV)).sum()).backward()
+    got = [t.grad.cpu() for t in leaves]
+    assert max_rel(lay(got[0]) if time_major else got[0], want[0]) <= 2e-5
+    assert max_rel(lay(got[1]) if time_major else got[1], want[1]) <= 2e-5
+    assert max_rel(got[2], want[2]) <= 2e-5
+    assert max_rel(got[3], want[3]) <= 2e-5
+
+
+def test_rglru_scan_backward_with_bf16_gates():
+    # the update path's dtypes: fp32 conv output, bf16 gate pre-activations
+    R, T, D = 32, 64, 128
+    x, gates, h0, done = _seq_inputs(9, R, T, D, torch.float32, torch.bfloat16, 0.05)
+    g = torch.Generator().manual_seed(2)
+    wy, wl = torch.randn(R, T, D, generator=g), torch.randn(R, D, generator=g)
+    lam = torch.linspace(0.0, 4.0, D)
+    want = _scan_grads_oracle(x, gates.float(), lam, h0, done, wy, wl)  # exact gradients at the rounded inputs
+    leaves = [t.to(DEV).requires_grad_(True) for t in (x, gates, lam, h0)]
+    y, last = ops.rglru_scan(leaves[0], leaves[1], leaves[2], 8.0, leaves[3], done.to(DEV))
+    ((y * wy.to(DEV)).sum() + (last * wl.to(DEV)).sum()).backward()
+    assert leaves[1].grad.dtype == torch.bfloat16
+    for got, ref in zip((t.grad for t in leaves), want):
+        assert max_rel(got.float().cpu(), ref) <= BF16_TOL

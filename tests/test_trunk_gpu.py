@@ -87,10 +87,19 @@ def test_transformer_block_under_bf16_autocast_feeds_bf16_to_the_kernel(monkeypa
     assert max_rel(got.cpu(), torch_ref.spatial_sublayer(p, "b.spatial.0.", x, alive, H)) <= BF16_TOL
 
 
-def test_layers_refuse_gradients_and_host_tensors():
+def test_layers_train_through_torch_ops_and_refuse_host_tensors():
     layer = bnb.TransformerBlock(_cfg()).to(DEV)
+    x = torch.randn(2, 4, 64, device=DEV)
+    alive = torch.tensor([[True, True, False, True], [True, False, False, True]], device=DEV)
+    with torch.no_grad():
+        want = layer(x, alive)
+    got = layer(x, alive)  # grad mode on, parameters require grad: the differentiable composition
+    assert got.requires_grad and max_rel(got.detach().cpu(), want.cpu()) <= 2e-5
+    got.sum().backward()
+    assert all(p.grad is not None for p in layer.parameters())
+    qkv = torch.randn(1, 4, 192, device=DEV, requires_grad=True)
     with pytest.raises(RuntimeError, match="forward-only"):
-        layer(torch.randn(1, 4, 64, device=DEV))  # grad mode on, parameters require grad
+        bnb.sdpa_masked(qkv, None, 4)  # the kernels themselves have no backward
     with pytest.raises(RuntimeError, match="no host fallback"):
         with torch.no_grad():
             bnb.TransformerBlock(_cfg())(torch.randn(1, 4, 64))
@@ -418,3 +427,54 @@ def test_bullet_reading_block_matches_oracle(autocast):
         got = layer(x.to(DEV), alive.to(DEV), bullets.to(DEV), bmask.to(DEV))
     ref = torch_ref.spatial_sublayer(p, "b.spatial.0.", x, alive, H, bullets, bmask)
     assert max_rel(got.float().cpu(), ref) <= (BF16_TOL if autocast else F32_TOL)
+
+
+# ------------------------------------------------------------------ training path (gradients)
+
+
+def test_temporal_block_sequence_gradients_match_autograd_of_the_oracle():
+    D, R, T = 64, 5, 9
+    gen = torch.Generator().manual_seed(21)
+    p = temporal_params(gen, "t.", D)
+    layer = bnb.GriffinTemporalBlock(D)
+    layer.load_state_dict(_strip(p, "t."))
+    layer.to(DEV)
+    x_seq = torch.randn(R, T, D, generator=gen)
+    h0 = 0.5 * torch.randn(R, D, generator=gen)
+    cb = torch.randn(R, 3, D, generator=gen)
+    done = torch.zeros(R, T, dtype=torch.bool)
+    done[:2, 3] = True
+    wo = torch.randn(R, T, D, generator=gen)
+    xd = x_seq.to(DEV).requires_grad_(True)
+    out, h1, cb1 = layer.forward_sequence(xd, h0.to(DEV), cb.to(DEV), done.to(DEV))
+    ((out * wo.to(DEV)).sum() + h1.sum() + cb1.sum()).backward()
+    pr = {k: v.clone().double().requires_grad_(True) for k, v in p.items()}
+    xr = x_seq.double().requires_grad_(True)
+    ro, rh, rcb = torch_ref.temporal_sequence(pr, "t.", xr, h0.double(), cb.double(), done)
+    ((ro * wo.double()).sum() + rh.sum() + rcb.sum()).backward()
+    assert max_rel(xd.grad.cpu(), xr.grad) <= 5e-5
+    for name, param in layer.named_parameters():
+        assert max_rel(param.grad.cpu(), pr["t." + name].grad) <= 5e-5, name
+
+
+def test_block_sequence_trains_and_matches_the_no_grad_path():
+    cfg = _cfg(64, 4, spatial=1, temporal=1)
+    torch.manual_seed(5)
+    block = bnb.YemongBlock(cfg).to(DEV)
+    T, B, N, M, D = 6, 3, 4, 2, 64
+    gen = torch.Generator().manual_seed(6)
+    x = torch.randn(T, B, N + M, D, generator=gen).to(DEV)
+    alive = (torch.rand(T, B, N + M, generator=gen) < 0.8).to(DEV)
+    alive[..., 0] = True
+    h0 = torch.randn(1, B * N, D, generator=gen).to(DEV)
+    cb0 = torch.randn(1, B * N, 3, D, generator=gen).to(DEV)
+    done = (torch.rand(T, B, generator=gen) < 0.2).to(DEV)
+    with torch.no_grad():
+        want, want_h, want_cb = block.sequence(x, alive, h0, cb0, done, N)
+    got, got_h, got_cb = block.sequence(x, alive, h0, cb0, done, N)
+    assert max_rel(got.detach().cpu(), want.cpu()) <= 2e-5
+    assert max_rel(got_h.detach().cpu(), want_h.cpu()) <= 2e-5 and max_rel(got_cb.detach().cpu(), want_cb.cpu()) <= 2e-5
+    got.square().mean().backward()
+    grads = [p.grad for p in block.parameters()]
+    assert all(g is not None and torch.isfinite(g).all() for g in grads)
+    assert block.temporal[0].rg_lru.log_lambda.grad.abs().max() > 0
