@@ -40,6 +40,7 @@ def parse_args():
     ap.add_argument("--no-torch-baseline", action="store_true")
     ap.add_argument("--no-module", action="store_true")
     ap.add_argument("--no-bullets", action="store_true", help="skip the bullet-read leg")
+    ap.add_argument("--no-sequence", action="store_true", help="skip the update-path (T = 128) recurrence leg")
     ap.add_argument("--no-trunk", action="store_true", help="skip the whole-trunk leg (2 blocks x (2 spatial + 1 temporal))")
     return ap.parse_args()
 
@@ -71,6 +72,33 @@ def torch_rglru_region(x, gates, log_lambda, c, h):
     a = torch.sigmoid(log_lambda) ** (c * r)
     gate = torch.sqrt(torch.clamp((1.0 - a) * (1.0 + a), min=1e-6))
     return a * h + gate * (i * x)
+
+
+def torch_scan_region(x, gates, log_lambda, c, h0, done):
+    """The reference's sequence recurrence in torch ops (griffin.py:206-219 and the log-depth
+    scan :25-64): coefficients, reset of a after an episode end, shifted combines."""
+    D = x.shape[-1]
+    r = torch.sigmoid(gates[..., :D])
+    i = torch.sigmoid(gates[..., D:])
+    a = torch.sigmoid(log_lambda) ** (c * r)
+    b = torch.sqrt(torch.clamp((1.0 - a) * (1.0 + a), min=1e-6)) * (i * x)
+    fresh = done.roll(1, dims=1)
+    fresh[:, 0] = False
+    a = a.masked_fill(fresh.unsqueeze(-1), 0.0)
+    T = a.shape[1]
+    width = 1 << (T - 1).bit_length()
+    if width > T:
+        a = torch.nn.functional.pad(a, (0, 0, 0, width - T), value=1.0)
+        b = torch.nn.functional.pad(b, (0, 0, 0, width - T), value=0.0)
+    span = 1
+    while span < width:
+        a_prev = torch.nn.functional.pad(a[:, : width - span], (0, 0, span, 0), value=1.0)
+        b_prev = torch.nn.functional.pad(b[:, : width - span], (0, 0, span, 0), value=0.0)
+        b = a * b_prev + b
+        a = a * a_prev
+        span *= 2
+    out = (a * h0.unsqueeze(1) + b)[:, :T]
+    return out, out[:, -1]
 
 
 def torch_conv_region(b1, conv_buf, weight, bias):
@@ -442,6 +470,55 @@ def main():
                     "mask, Q, accumulator in and out; exp-throughput-bound rather than HBM-bound when many bullets are live",
         }
         del kv_b, b_mask, merged
+
+    # ---- update path: the recurrence over a stored rollout (T = 128), forward and backward ----
+    if not args.no_sequence:
+        Rs, Ts = 8192, 128  # 1024 environments x 8 ships, the rollout length of the reference's training run
+        g_dt = torch.bfloat16 if bf16 else torch.float32
+        xs = torch.randn(Ts, Rs, D, device=dev, generator=gen)
+        gs = torch.randn(Ts, Rs, 2 * D, device=dev, generator=gen).to(g_dt)
+        hs = torch.randn(Rs, D, device=dev, generator=gen)
+        dn = torch.rand(Rs, Ts, device=dev, generator=gen) < 0.02
+        lam_s = lam
+        t_scan = timed_loop(lambda t: ops.rglru_scan(xs, gs, lam_s, 8.0, hs, dn, y_dtype=g_dt, time_major=True), 8, 2) / 8
+        es = 2 if bf16 else 4
+        scan_bytes = Rs * Ts * D * (4 + 2 * es + es) + Rs * Ts
+        leaves = [t.clone().requires_grad_(True) for t in (xs, gs, lam_s, hs)]
+
+        def scan_train(t):
+            for leaf in leaves:
+                leaf.grad = None
+            with torch.enable_grad():
+                y, _ = ops.rglru_scan(leaves[0], leaves[1], leaves[2], 8.0, leaves[3], dn, time_major=True)
+                y.backward(xs)
+
+        t_train = timed_loop(scan_train, 4, 2) / 4
+        bwd_bytes = Rs * Ts * D * (4 + 2 * es + 4 + 4 + 4 + 2 * es)  # x, gates, y, dy in; dx, dgates out
+        t_ref = t_ref_train = None
+        if not args.no_torch_baseline:
+            xr, gr = xs.transpose(0, 1).contiguous(), gs.transpose(0, 1).contiguous()
+            t_ref = timed_loop(lambda t: torch_scan_region(xr, gr, lam_s, 8.0, hs, dn), 2, 1) / 2
+            rl = [t.clone().requires_grad_(True) for t in (xr, gr, lam_s, hs)]
+
+            def ref_train(t):
+                for leaf in rl:
+                    leaf.grad = None
+                with torch.enable_grad():
+                    torch_scan_region(rl[0], rl[1], rl[2], 8.0, rl[3], dn)[0].backward(xr)
+
+            t_ref_train = timed_loop(ref_train, 2, 1) / 2
+            del xr, gr, rl
+        result["sequence"] = {
+            "rows": Rs, "T": Ts, "scan_fwd_us": t_scan * 1e6, "scan_fwd_algorithmic_bytes": scan_bytes,
+            "scan_fwd_GBps": scan_bytes / t_scan / 1e9, "scan_fwd_frac_of_hbm_peak": scan_bytes / t_scan / peak,
+            "scan_fwd_bwd_us": t_train * 1e6, "scan_bwd_algorithmic_bytes": bwd_bytes,
+            "eager_torch_fwd_us": None if t_ref is None else t_ref * 1e6,
+            "eager_torch_fwd_bwd_us": None if t_ref_train is None else t_ref_train * 1e6,
+            "what": "bnb_rglru_scan_fwd / _bwd over (T, rows, D): x fp32, gate pre-activations and states in the "
+                    "projection dtype; eager = the reference's coefficient chain + Hillis-Steele scan in torch ops "
+                    "(and autograd through it)",
+        }
+        del xs, gs, hs, dn, leaves
 
     # ---- whole trunk (reference default: 2 blocks x (2 spatial + 1 temporal)), state carried ----
     if not args.no_trunk:
