@@ -5,14 +5,14 @@ per-entity RG-LRU recurrence step, as hand-written HIP kernels behind a C ABI
 (``include/bnb_amd.h`` -> ``_lib/libbnb_amd.so``), plus torch modules that keep the
 reference policy's layer interfaces and ``state_dict`` names.
 
-    ops       sdpa_masked, rglru_step, conv_step             (the kernels)
+    ops       sdpa_masked, sdpa_cross, rglru_step, conv_step, rglru_scan, conv_seq, add_rmsnorm, gelu_mul
     trunk     TransformerBlock, RGLRU, GriffinTemporalBlock, YemongBlock, YemongTrunk, GraphedTrunk
     harness   benchmark workloads, traffic model, AttnRglruStep
     build     compiles the HIP sources
 """
 
 from . import _native, harness, ops, trunk
-from .ops import conv_step, rglru_step, sdpa_masked
+from .ops import conv_seq, conv_step, rglru_scan, rglru_step, sdpa_cross, sdpa_masked
 from .trunk import (
     CONV_KERNEL,
     GatedMLP,
@@ -27,5 +27,6 @@ from .trunk import (
 
 __all__ = [
     "CONV_KERNEL", "GatedMLP", "GraphedTrunk", "GriffinTemporalBlock", "ModelConfig", "RGLRU", "TransformerBlock",
-    "YemongBlock", "YemongTrunk", "conv_step", "rglru_step", "sdpa_masked", "ops", "trunk", "harness",
+    "YemongBlock", "YemongTrunk", "conv_seq", "conv_step", "rglru_scan", "rglru_step", "sdpa_cross", "sdpa_masked", "ops",
+    "trunk", "harness",
 ]
