@@ -15,7 +15,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_DIR = os.path.join(PKG_DIR, "_lib")
 LIB_PATH = os.path.join(LIB_DIR, "libbnb_amd.so")
-SOURCES = ("abi.hip", "conv_step.hip", "elementwise.hip", "rglru_step.hip", "sdpa_masked.hip", "temporal_seq.hip")
+SOURCES = ("abi.hip", "conv_step.hip", "elementwise.hip", "ffn_fused.hip", "rglru_step.hip", "sdpa_masked.hip", "temporal_seq.hip")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -29,6 +29,14 @@ HIPCC_FLAGS = [
     "-Wno-unused-command-line-argument",
 ]
 
+# Per-source additions.  The fused FFN keeps 64 accumulators live across its chunk loop next
+# to two more MFMA results that the vector ALU consumes at once: with MFMA results in AGPRs
+# the compiler copies accumulators between the two register files every iteration, in VGPR
+# form it does not.
+EXTRA_FLAGS = {
+    "ffn_fused.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
+
 
 def build(verbose: bool = False) -> str:
     """Compile every source and link the shared library; returns its path."""
@@ -37,7 +45,7 @@ def build(verbose: bool = False) -> str:
     objects = []
     for src in SOURCES:
         obj = os.path.join(LIB_DIR, src.replace(".hip", ".o"))
-        cmd = [hipcc, *HIPCC_FLAGS, "-I", INCLUDE, "-I", CSRC, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc, *HIPCC_FLAGS, *EXTRA_FLAGS.get(src, []), "-I", INCLUDE, "-I", CSRC, "-c", os.path.join(CSRC, src), "-o", obj]
         _run(cmd, verbose)
         objects.append(obj)
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objects], verbose)

@@ -1,0 +1,265 @@
+// Residual add + RMSNorm + gated MLP + residual add as ONE kernel on the matrix cores (gfx950).
+//
+//   s   = x + delta                                   (fp32 residual stream, delta bf16)
+//   n   = bf16(s * rsqrt(mean(s^2) + eps) * w_norm)
+//   g,u = n Wg^T, n Wu^T                              (D = 128 -> hidden = 512, fp32 accumulators)
+//   h   = bf16(gelu(g) * u)
+//   out = s + h Wd^T                                  (fp32)
+// Reference: `x = x + attn(...)`, `x + self.ffn(self.norm2(x))` of models/yemong/attention.py:97-99
+// with GatedMLP :21-37, and the same tail of the temporal block, models/yemong/griffin.py:284-286,
+// as they run under bf16 autocast.
+//
+// As separate library GEMMs this sublayer moves the 1024-wide gate/up activations through
+// memory three times; here a wave owns 32 tokens and nothing but x, delta and out touches
+// HBM.  Everything is computed transposed so that results feed the next MFMA from registers:
+//   G^T (hidden x tokens) = Wg (A) * n^T (B),  out^T (channels x tokens) += Wd (A) * h^T (B).
+// v_mfma_f32_32x32x16_bf16 leaves a lane with one token column of G^T (16 hidden units), and
+// those 16 values are exactly the B operand the lane must supply for out^T when the A operand
+// (Wd) lists the hidden units in the same order; the weights are stored pre-arranged for that
+// (pack layout below).  The lane also owns its token's s values in the accumulator layout of
+// out^T, so `s` is simply the initial accumulator, and with the channel order chosen in the
+// pack the same registers are the B operand of the first GEMM after normalisation.
+// The weights (384 KB bf16) stream through LDS in 16 chunks of 32 hidden units (24 KB) with
+// three buffers: chunk c+2 travels from L2 through registers into LDS while chunk c is used,
+// and the gate/up operands of chunk c+1 are read from LDS a whole chunk ahead of their MFMAs
+// (with two waves per SIMD nothing else would hide the LDS latency); one barrier per chunk.
+//
+// Channel order: k-slot e of contraction step ks in a lane of half h stands for channel
+//   ch(ks, h, e) = 16ks + 8(e/4) + 4h + e%4
+// (the two lanes holding one token then own interleaved runs of four channels: 16-byte LDS
+// accesses on both sides of the staging area).  x, delta and out move between HBM and the
+// token-owning lanes through LDS, so that global accesses are whole rows: per-token 16-byte
+// pieces 512 bytes apart ran the same traffic at less than half the bandwidth.
+//
+// Pack layout (bf16, built once on the host side), chunk c = hidden units 32c..32c+31,
+// lane l = 32*h + m, e = 0..7:
+//   [c][0][ks][l][e] = Wg[32c + m][ch(ks, h, e)]                              ks = 0..7
+//   [c][1][ks][l][e] = Wu[32c + m][ch(ks, h, e)]
+//   [c][2][cb][t][l][e] = Wd[32cb + m][32c + 16t + 8(e/4) + 4h + e%4]         cb = 0..3, t = 0..1
+// i.e. every MFMA A operand is one contiguous 1 KB run read with a single ds_read_b128.
+
+#include "common.h"
+
+namespace bnb {
+
+constexpr int kFfnD = 128;
+constexpr int kFfnHidden = 512;
+constexpr int kFfnChunks = kFfnHidden / 32;
+constexpr int kFfnChunkHalfs = 3 * 32 * kFfnD;  // 12288 bf16 = 24 KB
+constexpr int kFfnWaves = 4;
+constexpr int kFfnThreads = kFfnWaves * kWave;
+constexpr int kFfnPrefetch = kFfnChunkHalfs / 8 / kFfnThreads;  // 16-byte pieces per thread per chunk
+
+// erf-GELU as v/2 + |v| (1/2 - q(|v|)) with q(z) = erfc(z / sqrt 2) / 2 from the three-term
+// Abramowitz-Stegun form 7.1.25 (|error of erfc| <= 2.5e-5, i.e. an error of at most
+// 1.3e-5 |v|, two orders of magnitude below the bf16 rounding of the product that follows).
+// The constants carry the 1/sqrt 2 and the 1/2.  12 vector-ALU operations per element: this
+// is what bounds the kernel.
+__device__ __forceinline__ float gelu_as(float v)
+{
+    const float t = __builtin_amdgcn_rcpf(fmaf(0.47047f * 0.70710678118654752f, fabsf(v), 1.0f));
+    float poly = fmaf(t, 0.5f * 0.7478556f, 0.5f * -0.0958798f);
+    poly = fmaf(t, poly, 0.5f * 0.3480242f);
+    const float e = __builtin_amdgcn_exp2f((v * v) * (-0.5f * 1.4426950408889634f));
+    return fmaf(fabsf(v), fmaf(-(poly * t), e, 0.5f), 0.5f * v);
+}
+
+template <bool HAS_DELTA>
+__global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void ffn_fused_kernel(
+    const float *__restrict__ x, int64_t x_stride, const uint16_t *__restrict__ delta,
+    const float *__restrict__ norm_w, float eps, const uint16_t *__restrict__ wpack, float *__restrict__ out,
+    int64_t R)
+{
+    // three weight buffers: chunk c is used while chunk c+1 is already complete (its operands
+    // are read one chunk ahead) and chunk c+2 is on its way in
+    __shared__ __align__(16) uint16_t s_w[3][kFfnChunkHalfs];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m = lane & 31;
+    const int half = lane >> 5;
+
+    u32x4 pre[kFfnPrefetch], pre1[kFfnPrefetch];
+    auto fetch = [&](int c, u32x4 (&dst)[kFfnPrefetch]) {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(wpack + (int64_t)c * kFfnChunkHalfs);
+#pragma unroll
+        for (int q = 0; q < kFfnPrefetch; ++q) dst[q] = src[tid + q * kFfnThreads];
+    };
+    auto stash = [&](int buf, const u32x4 (&src)[kFfnPrefetch]) {
+        u32x4 *dst = reinterpret_cast<u32x4 *>(s_w[buf]);
+#pragma unroll
+        for (int q = 0; q < kFfnPrefetch; ++q) dst[tid + q * kFfnThreads] = src[q];
+    };
+    fetch(0, pre);
+    fetch(1, pre1);
+
+    // ---- s = x + delta for this wave's 32 tokens ----
+    // Read as whole rows (a half-wave per 512-byte row, 16 bytes per lane) and handed to the
+    // lanes that own the tokens through this wave's slice of the still unused weight buffers:
+    // row r at r * kRowPitch floats, the pitch keeping the 32 row starts on different banks.
+    constexpr int kRowPitch = kFfnD + 4;
+    float *stage = reinterpret_cast<float *>(&s_w[0][0]) + wave * (32 * kRowPitch);
+    const int64_t row0 = ((int64_t)blockIdx.x * kFfnWaves + wave) * 32;
+    const int io_row = lane >> 5;        // which of the two rows of one instruction
+    const int io_col = (lane & 31) * 4;  // first of this lane's four channels
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int64_t r = row0 + 2 * j + io_row;
+        const int64_t rs = r < R ? r : R - 1;
+        f32x4 sv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(x + rs * x_stride + io_col));
+        if (HAS_DELTA) {
+            const u32x2 dv = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(delta + rs * kFfnD + io_col));
+            sv.x += __uint_as_float(dv.x << 16);
+            sv.y += __uint_as_float(dv.x & 0xffff0000u);
+            sv.z += __uint_as_float(dv.y << 16);
+            sv.w += __uint_as_float(dv.y & 0xffff0000u);
+        }
+        *reinterpret_cast<f32x4 *>(stage + (2 * j + io_row) * kRowPitch + io_col) = sv;
+    }
+    __syncthreads();
+
+    // the lane's own token in the accumulator layout, and its sum of squares
+    const int64_t row = row0 + m;
+    f32x16 acc[4];
+    float ss = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+        // k-slots 0..3 / 4..7 of step ks: channels 16ks + 4half + 0..3 and 16ks + 8 + 4half + 0..3;
+        // they are accumulator registers 8(ks%2) + 0..7 of channel block ks/2
+        const float *sp = stage + m * kRowPitch + 16 * ks + 4 * half;
+        const f32x4 lo = *reinterpret_cast<const f32x4 *>(sp);
+        const f32x4 hi = *reinterpret_cast<const f32x4 *>(sp + 8);
+        const float sv[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            acc[ks >> 1][8 * (ks & 1) + e] = sv[e];
+            ss = fmaf(sv[e], sv[e], ss);
+        }
+    }
+    ss += __shfl_xor(ss, 32);
+    const float rstd = rsqrtf(ss * (1.0f / kFfnD) + eps);
+
+    // ---- n = rmsnorm(s) as the B operand of the first GEMM (k-slot e of step ks = channel ch(ks, half, e)) ----
+    bf16x8 nb[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+        const f32x4 wl = *reinterpret_cast<const f32x4 *>(norm_w + 16 * ks + 4 * half);
+        const f32x4 wh = *reinterpret_cast<const f32x4 *>(norm_w + 16 * ks + 8 + 4 * half);
+        const float wv[8] = {wl.x, wl.y, wl.z, wl.w, wh.x, wh.y, wh.z, wh.w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) nb[ks][e] = (__bf16)((acc[ks >> 1][8 * (ks & 1) + e] * rstd) * wv[e]);
+    }
+
+    __syncthreads();  // every wave has its tokens out of the staging area
+    stash(0, pre);
+    stash(1, pre1);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // every load so far is back: no wait on them inside the loop
+    __syncthreads();
+
+    // gate/up operands of the chunk about to be used, read one chunk ahead of their use
+    u32x4 ag[8], au[8];
+    auto read_gate_up = [&](int buf) {
+        const uint16_t *wb = s_w[buf] + lane * 8;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            ag[ks] = *reinterpret_cast<const u32x4 *>(wb + ks * 512);
+            au[ks] = *reinterpret_cast<const u32x4 *>(wb + 4096 + ks * 512);
+        }
+    };
+    read_gate_up(0);
+
+    int buf = 0;  // c % 3
+    for (int c = 0; c < kFfnChunks; ++c) {
+        const int buf1 = buf == 2 ? 0 : buf + 1;
+        const int buf2 = buf1 == 2 ? 0 : buf1 + 1;
+        if (c + 2 < kFfnChunks) fetch(c + 2, pre);
+
+        f32x16 g = {0.0f}, u = {0.0f};
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            g = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ag[ks]), nb[ks], g, 0, 0, 0);
+            u = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, au[ks]), nb[ks], u, 0, 0, 0);
+        }
+        // the first half of the down-projection operands arrives while the vector ALU works
+        // on gelu(g) * u, the second half while the first four MFMAs run
+        const uint16_t *wd = s_w[buf] + lane * 8 + 8192;
+        u32x4 ad[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) ad[q] = *reinterpret_cast<const u32x4 *>(wd + q * 512);
+
+        // h = bf16(gelu(g) * u): one rounding where the library composition has four (GEMM
+        // outputs, F.gelu, product); this part is bound by vector-ALU issue, every op counts
+        bf16x8 hb[2];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) hb[v >> 3][v & 7] = (__bf16)(gelu_as(g[v]) * u[v]);
+
+        u32x4 ad2[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) ad2[q] = *reinterpret_cast<const u32x4 *>(wd + (4 + q) * 512);
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ad[cb * 2 + t]), hb[t],
+                                                                  acc[cb], 0, 0, 0);
+        }
+#pragma unroll
+        for (int cb = 2; cb < 4; ++cb) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ad2[(cb - 2) * 2 + t]),
+                                                                  hb[t], acc[cb], 0, 0, 0);
+        }
+        if (c + 1 < kFfnChunks) read_gate_up(buf1);  // complete in LDS since the previous barrier
+        if (c + 2 < kFfnChunks) stash(buf2, pre);
+        __syncthreads();
+        buf = buf1;
+    }
+
+    // ---- out: back through the staging area (the loop's last barrier has freed the weight
+    //      buffers) so that rows leave as whole 512-byte runs ----
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+        const f32x16 &a = acc[ks >> 1];
+        const int v0 = 8 * (ks & 1);
+        float *sp = stage + m * kRowPitch + 16 * ks + 4 * half;
+        *reinterpret_cast<f32x4 *>(sp) = f32x4{a[v0], a[v0 + 1], a[v0 + 2], a[v0 + 3]};
+        *reinterpret_cast<f32x4 *>(sp + 8) = f32x4{a[v0 + 4], a[v0 + 5], a[v0 + 6], a[v0 + 7]};
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int64_t r = row0 + 2 * j + io_row;
+        const f32x4 ov = *reinterpret_cast<const f32x4 *>(stage + (2 * j + io_row) * kRowPitch + io_col);
+        if (r < R) __builtin_nontemporal_store(ov, reinterpret_cast<f32x4 *>(out + r * kFfnD + io_col));
+    }
+}
+
+}  // namespace bnb
+
+extern "C" int bnb_ffn_fused_fwd(const float *x, int64_t x_row_stride, const void *delta, int delta_dtype,
+                                 const float *norm_weight, float eps, const void *weights_packed, float *out,
+                                 int64_t R, int D, int hidden, void *stream)
+{
+    using namespace bnb;
+    if (R < 0 || x_row_stride < D) return BNB_ERR_BAD_SHAPE;
+    if (D != kFfnD || hidden != kFfnHidden) return BNB_ERR_UNSUPPORTED;
+    if (R == 0) return 0;
+    if (!x || !norm_weight || !weights_packed || !out) return BNB_ERR_NULL_POINTER;
+    if (delta && delta_dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
+    if (!aligned16(x) || !aligned16(out) || !aligned16(norm_weight) || !aligned16(weights_packed) ||
+        (delta && !aligned16(delta)) || (x_row_stride % 4) != 0)
+        return BNB_ERR_MISALIGNED;
+    const int64_t blocks = (R + kFfnWaves * 32 - 1) / (kFfnWaves * 32);
+    if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    if (delta)
+        hipLaunchKernelGGL((ffn_fused_kernel<true>), dim3((unsigned)blocks), dim3(kFfnThreads), 0, s, x, x_row_stride,
+                           (const uint16_t *)delta, norm_weight, eps, (const uint16_t *)weights_packed, out, R);
+    else
+        hipLaunchKernelGGL((ffn_fused_kernel<false>), dim3((unsigned)blocks), dim3(kFfnThreads), 0, s, x,
+                           x_row_stride, (const uint16_t *)nullptr, norm_weight, eps,
+                           (const uint16_t *)weights_packed, out, R);
+    return (int)hipGetLastError();
+}

@@ -630,3 +630,92 @@ def copy_bytes(src: torch.Tensor, dst: torch.Tensor) -> None:
     with torch.cuda.device(src.device):
         rc = _native.load().bnb_copy_bytes(src.data_ptr(), dst.data_ptr(), n, _stream())
     _native.check(rc, "bnb_copy_bytes")
+
+
+FFN_WIDTH, FFN_HIDDEN = 128, 512
+
+
+def pack_ffn_weights(gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor) -> torch.Tensor:
+    """``gate_proj``/``up_proj`` (512, 128) and ``down_proj`` (128, 512) weights as the bfloat16
+    operand stream of ``ffn_fused``: 16 chunks of 32 hidden units, each
+    ``[gate (8, 64, 8) | up (8, 64, 8) | down (4, 2, 64, 8)]`` with the index meaning given in
+    ``include/bnb_amd.h`` (every matrix-core operand is one contiguous 1 KB run)."""
+    D, Hd = FFN_WIDTH, FFN_HIDDEN
+    if gate_w.shape != (Hd, D) or up_w.shape != (Hd, D) or down_w.shape != (D, Hd):
+        raise ValueError("ffn_fused covers d_model 128 with a hidden width of 512")
+    dev = gate_w.device
+    lane = torch.arange(64, device=dev)
+    m, half = lane % 32, lane // 32
+    e = torch.arange(8, device=dev)
+    c = torch.arange(Hd // 32, device=dev)
+    ks = torch.arange(8, device=dev)
+    rows = (32 * c[:, None, None, None] + m[None, None, :, None]).expand(-1, 8, -1, 8)  # (16, 8, 64, 8)
+    cols = (16 * ks[None, :, None, None] + 8 * (e // 4)[None, None, None, :] + 4 * half[None, None, :, None]
+            + (e % 4)[None, None, None, :]).expand(16, -1, -1, -1)
+    g = gate_w.detach().to(torch.bfloat16)[rows, cols]
+    u = up_w.detach().to(torch.bfloat16)[rows, cols]
+    cb = torch.arange(4, device=dev)
+    t = torch.arange(2, device=dev)
+    d_rows = (32 * cb[:, None] + m[None, :])[None, :, None, :, None].expand(16, -1, 2, -1, 8)  # (16, 4, 2, 64, 8)
+    d_cols = (32 * c[:, None, None, None, None] + 16 * t[None, None, :, None, None]
+              + 8 * (e // 4)[None, None, None, None, :] + 4 * half[None, None, None, :, None]
+              + (e % 4)[None, None, None, None, :]).expand(-1, 4, -1, -1, -1)
+    d = down_w.detach().to(torch.bfloat16)[d_rows, d_cols]
+    return torch.cat([g.reshape(16, -1), u.reshape(16, -1), d.reshape(16, -1)], dim=1).contiguous()
+
+
+def ffn_supported(x: torch.Tensor, hidden: int) -> bool:
+    """Whether ``ffn_fused`` covers this residual stream (fp32 on the GPU, width 128, hidden 512)."""
+    return x.is_cuda and x.dtype == torch.float32 and x.shape[-1] == FFN_WIDTH and hidden == FFN_HIDDEN
+
+
+def ffn_fused(
+    x: torch.Tensor,
+    delta: torch.Tensor | None,
+    norm_weight: torch.Tensor,
+    weights_packed: torch.Tensor,
+    *,
+    eps: float | None = None,
+    out: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """``s = x + delta; s + down(gelu(gate(n)) * up(n))`` with ``n = rmsnorm(s) * norm_weight``,
+    one matrix-core kernel with bfloat16 projections (what the sublayer tail computes under
+    bfloat16 autocast).
+
+    x (..., 128) float32 with contiguous rows; delta same shape, bfloat16, or None;
+    ``weights_packed`` from ``pack_ffn_weights``.  Returns (..., 128) float32.
+    """
+    D = x.shape[-1]
+    if not ffn_supported(x, FFN_HIDDEN):
+        raise RuntimeError("ffn_fused covers float32 (..., 128) residual streams on the GPU")
+    _need_device(x, "x")
+    if torch.is_grad_enabled() and (x.requires_grad or (delta is not None and delta.requires_grad)):
+        raise RuntimeError("ffn_fused is forward-only; call it under torch.no_grad()")
+    if weights_packed.dtype != torch.bfloat16 or weights_packed.numel() != 3 * FFN_HIDDEN * FFN_WIDTH or not weights_packed.is_contiguous():
+        raise ValueError("weights_packed must come from pack_ffn_weights")
+    if norm_weight.shape != (D,) or norm_weight.dtype != torch.float32:
+        raise ValueError(f"norm_weight must be a float32 {(D,)} tensor")
+    x2 = x.reshape(-1, D)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    R = x2.shape[0]
+    delta_ptr = None
+    if delta is not None:
+        if delta.shape != x.shape or delta.dtype != torch.bfloat16:
+            raise ValueError(f"delta must be a bfloat16 {tuple(x.shape)} tensor")
+        delta = delta.reshape(-1, D).contiguous()
+        delta_ptr = delta.data_ptr()
+    if out is None:
+        out = torch.empty((R, D), dtype=torch.float32, device=x.device)
+    elif out.numel() != R * D or out.dtype != torch.float32 or not out.is_contiguous() or out.device != x.device:
+        raise ValueError("out must be a contiguous float32 tensor of x's size on x's device")
+    norm_weight = norm_weight.detach().contiguous()
+    if R:
+        with torch.cuda.device(x.device):
+            rc = _native.load().bnb_ffn_fused_fwd(
+                x2.data_ptr(), x2.stride(0), delta_ptr, _native.BF16, norm_weight.data_ptr(),
+                float(_F32_EPS if eps is None else eps), weights_packed.data_ptr(), out.data_ptr(), R, D, FFN_HIDDEN,
+                _stream(),
+            )
+        _native.check(rc, "bnb_ffn_fused_fwd")
+    return out.reshape(x.shape)

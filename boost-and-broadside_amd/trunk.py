@@ -122,6 +122,22 @@ class GatedMLP(nn.Module):
         self.up_proj = nn.Linear(d_model, expand * d_model, bias=False)
         self.down_proj = nn.Linear(expand * d_model, d_model, bias=False)
 
+    def packed_weights(self) -> torch.Tensor:
+        """The three weight matrices as the fused sublayer-tail kernel's bf16 operand stream (cached)."""
+        ws = (self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight)
+        return _cached_cast(self, "_bnb_ffn_pack", ws, torch.bfloat16, lambda: ops.pack_ffn_weights(*ws))
+
+    def fused_tail(self, x: torch.Tensor, delta: torch.Tensor | None, norm: nn.RMSNorm) -> torch.Tensor | None:
+        """``s = x + delta; s + self(norm(s))`` as one kernel, or None when it does not apply
+        (it covers the bf16-autocast inference path at width 128 / hidden 512)."""
+        if (
+            torch.is_grad_enabled() or _projection_dtype() != torch.bfloat16
+            or not ops.ffn_supported(x, self.gate_proj.out_features)
+            or (delta is not None and delta.dtype != torch.bfloat16)
+        ):
+            return None
+        return ops.ffn_fused(x, delta, norm.weight, self.packed_weights(), eps=norm.eps)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         hidden = self.gate_proj.out_features
         if not x.is_cuda or hidden % 8 or x.dtype not in (torch.float32, torch.bfloat16) or torch.is_grad_enabled():
@@ -163,6 +179,9 @@ class TransformerBlock(nn.Module):
         # norm (+ cast) -> qkv -> attention kernel -> out_proj -> add + norm (+ cast) -> FFN
         _, n1 = ops.add_rmsnorm(x, self.norm1.weight, eps=self.norm1.eps, out_dtype=act)
         attn = self._attn(n1, alive_mask, bullets, bullet_mask)
+        fused = self.ffn.fused_tail(x, attn, self.norm2)
+        if fused is not None:
+            return fused
         x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=attn, eps=self.norm2.eps, out_dtype=act)
         return x1 + self.ffn(n2)
 
@@ -347,6 +366,9 @@ class GriffinTemporalBlock(nn.Module):
         if _fused_ok(x, act) and gate_in.dtype == act:
             # gelu(linear2) * y in one kernel, residual add + norm2 (+ cast) in one kernel
             r = _project(self.linear_out, ops.gelu_mul(gate_in, y, out_dtype=act))
+            fused = self.gated_mlp.fused_tail(x, r, self.norm2)
+            if fused is not None:
+                return fused
             x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=r, eps=self.norm2.eps, out_dtype=act)
             return x1 + self.gated_mlp(n2)
         x1 = x + self.linear_out(y * F.gelu(gate_in))
@@ -389,6 +411,9 @@ class GriffinTemporalBlock(nn.Module):
         gate_in = _project(self.linear2, normed)
         if _fused_ok(x, act) and gate_in.dtype == act:
             r = _project(self.linear_out, ops.gelu_mul(gate_in, b1, out_dtype=act))
+            fused = self.gated_mlp.fused_tail(x, r, self.norm2)
+            if fused is not None:
+                return fused
             x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=r, eps=self.norm2.eps, out_dtype=act)
             return x1 + self.gated_mlp(n2)
         x1 = x + self.linear_out(b1 * F.gelu(gate_in))

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 6
+#define BNB_ABI_VERSION 7
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -289,6 +289,33 @@ int bnb_rglru_scan_bwd(const void *x, int x_dtype, const void *gates_pre, int g_
 int bnb_add_rmsnorm_fwd(const float *x, int64_t x_row_stride, const void *delta, int delta_dtype,
                         const float *weight, float eps, float *sum_out, void *norm_out, int out_dtype,
                         int64_t R, int D, void *stream);
+
+/*
+ * Residual add + RMSNorm + gated MLP + residual add in one matrix-core kernel (bf16 compute):
+ *     s = x + delta;  n = rmsnorm(s) * norm_weight;  out = s + Wd (gelu(Wg n) * (Wu n))
+ * Replaces `x = x + <attention output>` and `x + self.ffn(self.norm2(x))` of
+ * models/yemong/attention.py:97-99 with GatedMLP (:21-37), and the same tail of the temporal
+ * block (models/yemong/griffin.py:284-286), as they run under bf16 autocast: the residual add,
+ * nn.RMSNorm, the casts, three Linear layers, F.gelu, the product and the last residual add.
+ *
+ *   x               (R, 128) fp32 residual stream, row stride x_row_stride floats
+ *   delta           optional (R, 128) bf16 contiguous (the sublayer output to add first); NULL = none
+ *   norm_weight     (128) fp32; eps as in nn.RMSNorm
+ *   weights_packed  gate_proj, up_proj (512 x 128) and down_proj (128 x 512) in bf16, arranged
+ *                   as the kernel's operand order (16 chunks of 32 hidden units, 24 KB each):
+ *                   [c][0][ks][l][e] = Wg[32c + l%32][16ks + 8(e/4) + 4(l/32) + e%4]
+ *                   [c][1][ks][l][e] = Wu[...same...]                          ks = 0..7
+ *                   [c][2][cb][t][l][e] = Wd[32cb + l%32][32c + 16t + 8(e/4) + 4(l/32) + e%4]
+ *                   with l = 0..63, e = 0..7, cb = 0..3, t = 0..1
+ *   out             (R, 128) fp32 contiguous; may equal x when x is contiguous
+ * Requirements: D == 128, hidden == 512 (else BNB_ERR_UNSUPPORTED), 16-byte aligned pointers.
+ * Operands of the three projections are bf16 as under autocast; between them the kernel rounds
+ * less often than the library composition (gate/up results stay fp32 until gelu(g) * u is
+ * rounded once; the down projection is added to s in fp32).
+ */
+int bnb_ffn_fused_fwd(const float *x, int64_t x_row_stride, const void *delta, int delta_dtype,
+                      const float *norm_weight, float eps, const void *weights_packed, float *out,
+                      int64_t R, int D, int hidden, void *stream);
 
 /*
  * out = gelu(a) * b with the exact (erf) GELU, the gelu rounded to a's dtype as F.gelu does and

@@ -760,3 +760,52 @@ def test_rglru_scan_backward_with_bf16_gates():
     assert leaves[1].grad.dtype == torch.bfloat16
     for got, ref in zip((t.grad for t in leaves), want):
         assert max_rel(got.float().cpu(), ref) <= BF16_TOL
+
+
+# ------------------------------------------------------------------ fused sublayer tail (add + norm + gated MLP + add)
+
+
+def _ffn_case(seed, R):
+    g = torch.Generator().manual_seed(seed)
+    D, Hd = 128, 512
+    x = torch.randn(R, D, generator=g)
+    delta = (0.5 * torch.randn(R, D, generator=g)).bfloat16()
+    nw = 1.0 + 0.1 * torch.randn(D, generator=g)
+    p = {"f.gate_proj.weight": torch.randn(Hd, D, generator=g) / D ** 0.5,
+         "f.up_proj.weight": torch.randn(Hd, D, generator=g) / D ** 0.5,
+         "f.down_proj.weight": torch.randn(D, Hd, generator=g) / Hd ** 0.5}
+    return x, delta, nw, p
+
+
+@pytest.mark.parametrize("R", [1, 31, 128, 129, 1000, 40000])
+@pytest.mark.parametrize("with_delta", [True, False])
+def test_ffn_fused_matches_oracle(R, with_delta):
+    x, delta, nw, p = _ffn_case(R, R)
+    rounded = {k: v.bfloat16().float() for k, v in p.items()}  # the projections run on bf16 weights
+    s = x + delta.float() if with_delta else x
+    want = s + torch_ref.gated_mlp(rounded, "f.", torch_ref.rms_norm(s, nw))
+    pk = ops.pack_ffn_weights(p["f.gate_proj.weight"].to(DEV), p["f.up_proj.weight"].to(DEV), p["f.down_proj.weight"].to(DEV))
+    got = ops.ffn_fused(x.to(DEV), delta.to(DEV) if with_delta else None, nw.to(DEV), pk)
+    assert got.shape == (R, 128) and got.dtype == torch.float32
+    assert max_rel(got.cpu(), want) <= BF16_TOL
+    # the MLP contribution alone (the residual would otherwise hide an error in it)
+    assert max_rel(got.cpu() - s, want - s) <= BF16_TOL
+
+
+def test_ffn_fused_every_weight_reaches_its_output():
+    # one-hot weights: hidden unit j and output channel k are hit exactly where the layout says
+    D, Hd = 128, 512
+    x = torch.zeros(64, D)
+    x[:, 5] = 1.0  # after the norm every channel but 5 is zero
+    nw = torch.ones(D)
+    for j, k in [(0, 0), (37, 100), (511, 127), (300, 9)]:
+        wg, wu, wd = torch.zeros(Hd, D), torch.zeros(Hd, D), torch.zeros(D, Hd)
+        wg[j, 5], wu[j, 5], wd[k, j] = 1.0, 2.0, 3.0
+        pk = ops.pack_ffn_weights(wg.to(DEV), wu.to(DEV), wd.to(DEV))
+        got = ops.ffn_fused(x.to(DEV), None, nw.to(DEV), pk).cpu() - x
+        n5 = torch_ref.rms_norm(x, nw)[0, 5].bfloat16().float()
+        h = (torch.nn.functional.gelu(n5).bfloat16().float() * (2.0 * n5).bfloat16().float()).bfloat16().float()
+        want = torch.zeros(D)
+        want[k] = 3.0 * h
+        assert torch.allclose(got[0], want, rtol=1e-2, atol=1e-6), (j, k)
+        assert torch.equal(got[0], got[63])
