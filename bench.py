@@ -39,6 +39,7 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU-baseline leg; 0 skips it")
     ap.add_argument("--no-torch-baseline", action="store_true")
     ap.add_argument("--no-module", action="store_true")
+    ap.add_argument("--no-ffn", action="store_true", help="skip the fused sublayer-tail leg")
     ap.add_argument("--no-bullets", action="store_true", help="skip the bullet-read leg")
     ap.add_argument("--no-sequence", action="store_true", help="skip the update-path (T = 128) recurrence leg")
     ap.add_argument("--no-trunk", action="store_true", help="skip the whole-trunk leg (2 blocks x (2 spatial + 1 temporal))")
@@ -437,6 +438,37 @@ def main():
         "what": "read linear1 output + 3 stored inputs, write conv output + shifted inputs into the packed state",
     }
     del packed
+
+    # ---- fused sublayer tail: add + RMSNorm + gated MLP + add on the matrix cores ----
+    if bf16 and not args.no_ffn:
+        Rf = w.B * w.NM
+        mlp = bnb.GatedMLP(D).to(dev).eval()
+        nw = torch.ones(D, device=dev)
+        pk = mlp.packed_weights()
+        xf = torch.randn(Rf, D, device=dev, generator=gen)
+        df = torch.randn(Rf, D, device=dev, generator=gen).to(torch.bfloat16)
+        of = torch.empty_like(xf)
+        n_f = max(4, min(steps, 16))
+        t_ffn = timed_loop(lambda t: ops.ffn_fused(xf, df, nw, pk, out=of), n_f, 3) / n_f
+
+        def ffn_library(t):
+            with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+                s = xf + df
+                n = F.rms_norm(s, (D,), nw, None)
+                return s + mlp.down_proj(F.gelu(mlp.gate_proj(n)) * mlp.up_proj(n))
+
+        t_ffn_lib = None if args.no_torch_baseline else timed_loop(ffn_library, n_f, 3) / n_f
+        ffn_flops = Rf * 2 * (D * 2 * 4 * D + 4 * D * D)
+        ffn_bytes = Rf * (4 * D + 2 * D + 4 * D)
+        result["ffn_fused_kernel"] = {
+            "rows": Rf, "avg_launch_us": t_ffn * 1e6, "tflops": ffn_flops / t_ffn / 1e12,
+            "frac_of_bf16_mfma_peak": ffn_flops / t_ffn / 2.5e15,
+            "algorithmic_bytes_per_launch": ffn_bytes, "achieved_GBps": ffn_bytes / t_ffn / 1e9,
+            "eager_torch_us": None if t_ffn_lib is None else t_ffn_lib * 1e6,
+            "what": "x + delta, RMSNorm, gate/up projections, gelu * up, down projection, residual add in one kernel; "
+                    "x fp32 and delta bf16 in, fp32 out; eager = the same composition in torch ops under bf16 autocast",
+        }
+        del xf, df, of, mlp
 
     # ---- bullet read (entity queries attending to the bullets in flight; 10 slots per ship) ----
     if bf16 and not args.no_bullets:
