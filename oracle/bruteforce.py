@@ -69,3 +69,96 @@ def rglru_step_loops(x, gates_pre, log_lambda, c, h) -> np.ndarray:
             gate = math.sqrt(max((1.0 - a) * (1.0 + a), 1e-6))
             out[row, d] = a * h[row, d] + gate * (i * x[row, d])
     return out
+
+
+def bullet_read_loops(q: np.ndarray, kv: np.ndarray, active: np.ndarray | None, n_heads: int) -> np.ndarray:
+    """Entity queries over bullet keys/values: softmax over the active bullets only, and an
+    environment without an active bullet contributes zero.
+
+    Definition being restated: models/yemong/attention.py:149-165.  ``q`` (B, N, D),
+    ``kv`` (B, NB, 2D) = [K | V].  With at least one active bullet the finfo.min/2 bias gives
+    inactive bullets weight exactly 0, which is what dropping them states.
+    """
+    q = np.asarray(q, dtype=np.float64)
+    kv = np.asarray(kv, dtype=np.float64)
+    B, N, D = q.shape
+    NB = kv.shape[1]
+    dh = D // n_heads
+    out = np.zeros((B, N, D), dtype=np.float64)
+    for b in range(B):
+        keys = [j for j in range(NB) if active is None or active[b, j]]
+        if not keys:
+            continue
+        for hd in range(n_heads):
+            lo = hd * dh
+            for i in range(N):
+                scores = [float(np.dot(q[b, i, lo:lo + dh], kv[b, j, lo:lo + dh])) / math.sqrt(dh) for j in keys]
+                m = max(scores)
+                w = [math.exp(s - m) for s in scores]
+                z = sum(w)
+                for wj, j in zip(w, keys):
+                    out[b, i, lo:lo + dh] += (wj / z) * kv[b, j, D + lo:D + lo + dh]
+    return out
+
+
+def conv_sequence_loops(b1, conv_buf, weight, bias, done) -> np.ndarray:
+    """out[r,t] = bias + sum_j w[:,3-j] * input[r,t-j] over the lags j that stay inside the
+    episode of step t; inputs before t = 0 come from the stored buffer (same episode as t = 0).
+
+    Definition being restated: models/yemong/griffin.py:67-93 (validity), :127-139 (taps).
+    """
+    b1 = np.asarray(b1, dtype=np.float64)
+    buf = np.asarray(conv_buf, dtype=np.float64)
+    w = np.asarray(weight, dtype=np.float64).reshape(b1.shape[-1], 4)
+    R, T, D = b1.shape
+    out = np.zeros((R, T, D), dtype=np.float64)
+    for r in range(R):
+        seq = [buf[r, 0], buf[r, 1], buf[r, 2]] + [b1[r, t] for t in range(T)]  # position p holds time p - 3
+        for t in range(T):
+            acc = np.zeros(D) if bias is None else np.asarray(bias, dtype=np.float64).copy()
+            for j in range(4):
+                # input at time t-j is in the episode of t iff no episode ended at t-j .. t-1
+                crossed = any(done is not None and 0 <= s < T and done[r, s] for s in range(t - j, t))
+                if not crossed:
+                    acc = acc + w[:, 3 - j] * seq[t - j + 3]
+            out[r, t] = acc
+    return out
+
+
+def rglru_sequence_loops(x, gates_pre, log_lambda, c, h0, done) -> np.ndarray:
+    """All states of the recurrence over T steps; the state is zero after an episode end.
+
+    Definition being restated: models/yemong/griffin.py:188-219.
+    """
+    x = np.asarray(x, dtype=np.float64)
+    R, T, D = x.shape
+    h = np.asarray(h0, dtype=np.float64).copy()
+    out = np.zeros((R, T, D), dtype=np.float64)
+    for t in range(T):
+        if t > 0 and done is not None:
+            for r in range(R):
+                if done[r, t - 1]:
+                    h[r] = 0.0
+        h = rglru_step_loops(x[:, t], np.asarray(gates_pre)[:, t], log_lambda, c, h)
+        out[:, t] = h
+    return out
+
+
+def ffn_tail_loops(x, delta, norm_w, gate_w, up_w, down_w, eps) -> np.ndarray:
+    """s = x + delta; s + Wd (gelu(Wg n) * (Wu n)), n = s / sqrt(mean(s^2) + eps) * norm_w, erf GELU.
+
+    Definition being restated: models/yemong/attention.py:21-37,97-99.
+    """
+    x = np.asarray(x, dtype=np.float64)
+    s = x if delta is None else x + np.asarray(delta, dtype=np.float64)
+    R, D = s.shape
+    gw, uw, dw = (np.asarray(a, dtype=np.float64) for a in (gate_w, up_w, down_w))
+    out = np.zeros((R, D), dtype=np.float64)
+    for r in range(R):
+        n = s[r] / math.sqrt(float(np.mean(s[r] * s[r])) + eps) * np.asarray(norm_w, dtype=np.float64)
+        hidden = np.zeros(gw.shape[0])
+        for j in range(gw.shape[0]):
+            g = float(np.dot(gw[j], n))
+            hidden[j] = 0.5 * g * (1.0 + math.erf(g / math.sqrt(2.0))) * float(np.dot(uw[j], n))
+        out[r] = s[r] + dw @ hidden
+    return out

@@ -1,4 +1,5 @@
-"""Writes tests/golden/step_vectors.npz: small seeded inputs and their expected outputs.
+"""Writes tests/golden/step_vectors.npz and widened_vectors.npz: small seeded inputs and their
+expected outputs.
 
 The reference keeps no stored numeric vectors for this path (its tests are property tests and
 its one golden file needs weights that are not in the checkout), and the reference was not
@@ -47,6 +48,67 @@ def main() -> None:
     out["rglru_out"] = bruteforce.rglru_step_loops(x, gates, lam, 8.0, h)
     np.savez_compressed(os.path.join(HERE, "step_vectors.npz"), **out)
     print("wrote", os.path.join(HERE, "step_vectors.npz"), {k: v.shape for k, v in out.items()})
+    widened()
+
+
+def widened() -> None:
+    """tests/golden/widened_vectors.npz: bullet read, sequence path and the sublayer tail."""
+    rng = np.random.default_rng(20240602)
+    out = {}
+
+    def bf16(a):
+        """Round to bfloat16 (nearest even), returned as float32."""
+        u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+        u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+        return u.view(np.float32)
+
+    def bits(a):
+        """bfloat16-exact float32 array -> its 16-bit patterns (halves the file)."""
+        return (np.ascontiguousarray(a, dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16)
+
+    # bullet read: env 0 has nothing in flight, env 1 a single bullet; 176 slots exercise the streamed path
+    for tag, (B, N, NB, H, dh) in {"read_small": (3, 6, 20, 4, 32), "read_long": (3, 5, 176, 4, 32)}.items():
+        D = H * dh
+        q = bf16(rng.standard_normal((B, N, D)))
+        kv = bf16(rng.standard_normal((B, NB, 2 * D)))
+        active = rng.random((B, NB)) < 0.4
+        active[0] = False
+        active[1] = False
+        active[1, NB - 1] = True
+        out[f"{tag}_q_bf16"], out[f"{tag}_kv_bf16"], out[f"{tag}_active"] = bits(q), bits(kv), active
+        out[f"{tag}_heads"] = np.int64(H)
+        out[f"{tag}_out"] = bruteforce.bullet_read_loops(q, kv, active, H)
+    # sequence path: conv with episode ends, recurrence with resets (T = 9 crosses the 4-step load groups)
+    R, T, D = 4, 9, 128
+    done = rng.random((R, T)) < 0.25
+    done[0] = False
+    done[1, 0] = True
+    b1 = rng.standard_normal((R, T, D)).astype(np.float32)
+    buf = rng.standard_normal((R, 3, D)).astype(np.float32)
+    w = (0.5 * rng.standard_normal((D, 1, 4))).astype(np.float32)
+    bias = (0.1 * rng.standard_normal(D)).astype(np.float32)
+    out["seq_done"], out["conv_b1"], out["conv_buf"], out["conv_w"], out["conv_bias"] = done, b1, buf, w, bias
+    out["conv_out"] = bruteforce.conv_sequence_loops(b1, buf, w, bias, done)
+    x = rng.standard_normal((R, T, D)).astype(np.float32)
+    gates = (2.0 * rng.standard_normal((R, T, 2 * D))).astype(np.float32)
+    h0 = (0.5 * rng.standard_normal((R, D))).astype(np.float32)
+    lam = np.linspace(0.0, 4.0, D, dtype=np.float32)
+    out["scan_x"], out["scan_gates"], out["scan_h0"], out["scan_lambda"] = x, gates, h0, lam
+    out["scan_out"] = bruteforce.rglru_sequence_loops(x, gates, lam, 8.0, h0, done)
+    # sublayer tail: weights already rounded to bf16 so that fp32 and bf16 paths see the same numbers
+    R, D, Hd = 5, 128, 512
+    out["ffn_x"] = rng.standard_normal((R, D)).astype(np.float32)
+    delta = bf16(0.5 * rng.standard_normal((R, D)))
+    out["ffn_norm_w"] = (1.0 + 0.1 * rng.standard_normal(D)).astype(np.float32)
+    gw = bf16(rng.standard_normal((Hd, D)) / np.sqrt(D))
+    uw = bf16(rng.standard_normal((Hd, D)) / np.sqrt(D))
+    dw = bf16(rng.standard_normal((D, Hd)) / np.sqrt(Hd))
+    out["ffn_delta_bf16"], out["ffn_gate_w_bf16"], out["ffn_up_w_bf16"], out["ffn_down_w_bf16"] = (
+        bits(delta), bits(gw), bits(uw), bits(dw))
+    out["ffn_out"] = bruteforce.ffn_tail_loops(out["ffn_x"], delta, out["ffn_norm_w"], gw, uw, dw,
+                                               float(np.finfo(np.float32).eps))
+    np.savez_compressed(os.path.join(HERE, "widened_vectors.npz"), **out)
+    print("wrote", os.path.join(HERE, "widened_vectors.npz"), {k: v.shape for k, v in out.items()})
 
 
 if __name__ == "__main__":

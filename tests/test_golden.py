@@ -60,3 +60,78 @@ def test_kernels_reproduce_rglru_vectors():
     x, g, h, lam = (torch.from_numpy(GOLD[k]).cuda() for k in ("rglru_x", "rglru_gates", "rglru_h", "rglru_lambda"))
     _, got = ops.rglru_step(x, g, lam, 8.0, h)
     assert max_rel(got.cpu(), torch.from_numpy(GOLD["rglru_out"])) <= 1e-5
+
+
+# ---------------------------------------------------------------- bullet read, sequence path, sublayer tail
+
+WIDE = np.load(os.path.join(ROOT, "tests", "golden", "widened_vectors.npz"))
+
+
+def _from_bits(name):
+    """bfloat16 bit patterns stored as uint16 -> float32 tensor."""
+    return torch.from_numpy((WIDE[name].astype(np.uint32) << 16).view(np.float32).copy())
+
+
+@pytest.mark.parametrize("tag", ["read_small", "read_long"])
+def test_oracle_reproduces_bullet_read_vectors(tag):
+    q, kv, active = _from_bits(f"{tag}_q_bf16"), _from_bits(f"{tag}_kv_bf16"), torch.from_numpy(WIDE[f"{tag}_active"])
+    H, want = int(WIDE[f"{tag}_heads"]), WIDE[f"{tag}_out"]
+    qkv = torch.cat([q, torch.zeros(*q.shape[:2], 2 * q.shape[-1])], dim=-1)  # only the Q third is read
+    got = torch_ref.bullet_read(qkv, kv, active, H).double().numpy()
+    assert np.abs(got - want).max() <= 5e-6
+    assert np.abs(want[0]).max() == 0  # nothing in flight
+    D = q.shape[-1]
+    assert np.abs(want[1] - kv[1, -1, D:].double().numpy()).max() <= 1e-12  # one bullet: its V row
+
+
+def test_oracle_reproduces_sequence_vectors():
+    done = torch.from_numpy(WIDE["seq_done"])
+    v, _ = torch_ref.conv_sequence(*(torch.from_numpy(WIDE[k]) for k in ("conv_b1", "conv_buf", "conv_w", "conv_bias")), done)
+    assert np.abs(v.double().numpy() - WIDE["conv_out"]).max() <= 5e-6
+    y, _ = torch_ref.rglru_sequence(torch.from_numpy(WIDE["scan_x"]), torch.from_numpy(WIDE["scan_gates"]),
+                                    torch.from_numpy(WIDE["scan_lambda"]), 8.0, torch.from_numpy(WIDE["scan_h0"]), done)
+    assert np.abs(y.double().numpy() - WIDE["scan_out"]).max() <= 5e-6
+
+
+def test_oracle_reproduces_sublayer_tail_vectors():
+    p = {"f.gate_proj.weight": _from_bits("ffn_gate_w_bf16"), "f.up_proj.weight": _from_bits("ffn_up_w_bf16"),
+         "f.down_proj.weight": _from_bits("ffn_down_w_bf16")}
+    s = torch.from_numpy(WIDE["ffn_x"]) + _from_bits("ffn_delta_bf16")
+    got = s + torch_ref.gated_mlp(p, "f.", torch_ref.rms_norm(s, torch.from_numpy(WIDE["ffn_norm_w"])))
+    assert np.abs(got.double().numpy() - WIDE["ffn_out"]).max() <= 2e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag", ["read_small", "read_long"])
+def test_kernels_reproduce_bullet_read_vectors(tag):
+    from boost_and_broadside_amd import ops
+
+    q, kv, active = _from_bits(f"{tag}_q_bf16"), _from_bits(f"{tag}_kv_bf16"), torch.from_numpy(WIDE[f"{tag}_active"])
+    qkv = torch.cat([q, torch.zeros(*q.shape[:2], 2 * q.shape[-1])], dim=-1).bfloat16()
+    got = ops.sdpa_cross(qkv.cuda(), kv.bfloat16().cuda(), active.cuda(), int(WIDE[f"{tag}_heads"])).float().cpu()
+    assert got[0].abs().max() == 0
+    assert max_rel(got, torch.from_numpy(WIDE[f"{tag}_out"])) <= 2e-2
+
+
+@pytest.mark.gpu
+def test_kernels_reproduce_sequence_vectors():
+    from boost_and_broadside_amd import ops
+
+    done = torch.from_numpy(WIDE["seq_done"]).cuda()
+    v, _ = ops.conv_seq(*(torch.from_numpy(WIDE[k]).cuda() for k in ("conv_b1", "conv_buf", "conv_w", "conv_bias")), done)
+    assert max_rel(v.cpu(), torch.from_numpy(WIDE["conv_out"])) <= 1e-5
+    y, last = ops.rglru_scan(torch.from_numpy(WIDE["scan_x"]).cuda(), torch.from_numpy(WIDE["scan_gates"]).cuda(),
+                             torch.from_numpy(WIDE["scan_lambda"]).cuda(), 8.0, torch.from_numpy(WIDE["scan_h0"]).cuda(), done)
+    assert max_rel(y.cpu(), torch.from_numpy(WIDE["scan_out"])) <= 1e-5
+    assert torch.equal(last, y[:, -1])
+
+
+@pytest.mark.gpu
+def test_kernels_reproduce_sublayer_tail_vectors():
+    from boost_and_broadside_amd import ops
+
+    pk = ops.pack_ffn_weights(_from_bits("ffn_gate_w_bf16").cuda(), _from_bits("ffn_up_w_bf16").cuda(),
+                              _from_bits("ffn_down_w_bf16").cuda())
+    got = ops.ffn_fused(torch.from_numpy(WIDE["ffn_x"]).cuda(), _from_bits("ffn_delta_bf16").bfloat16().cuda(),
+                        torch.from_numpy(WIDE["ffn_norm_w"]).cuda(), pk).cpu()
+    assert max_rel(got, torch.from_numpy(WIDE["ffn_out"])) <= 2e-2
