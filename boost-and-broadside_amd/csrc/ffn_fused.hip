@@ -20,9 +20,8 @@
 // out^T, so `s` is simply the initial accumulator, and with the channel order chosen in the
 // pack the same registers are the B operand of the first GEMM after normalisation.
 // The weights (384 KB bf16) stream through LDS in 16 chunks of 32 hidden units (24 KB) with
-// three buffers: chunk c+2 travels from L2 through registers into LDS while chunk c is used,
-// and the gate/up operands of chunk c+1 are read from LDS a whole chunk ahead of their MFMAs
-// (with two waves per SIMD nothing else would hide the LDS latency); one barrier per chunk.
+// three buffers: chunk c+2 travels from L2 through registers into LDS while the down projection
+// of chunk c and the gate/up products of chunk c+1 are formed; one barrier per chunk.
 //
 // Channel order: k-slot e of contraction step ks in a lane of half h stands for channel
 //   ch(ks, h, e) = 16ks + 8(e/4) + 4h + e%4
@@ -37,6 +36,8 @@
 //   [c][1][ks][l][e] = Wu[32c + m][ch(ks, h, e)]
 //   [c][2][cb][t][l][e] = Wd[32cb + m][32c + 16t + 8(e/4) + 4h + e%4]         cb = 0..3, t = 0..1
 // i.e. every MFMA A operand is one contiguous 1 KB run read with a single ds_read_b128.
+
+#include <type_traits>
 
 #include "common.h"
 
@@ -90,6 +91,19 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
         u32x4 *dst = reinterpret_cast<u32x4 *>(s_w[buf]);
 #pragma unroll
         for (int q = 0; q < kFfnPrefetch; ++q) dst[tid + q * kFfnThreads] = src[q];
+    };
+    // inside the loop a chunk comes in as two halves, so that only half of it occupies registers
+    constexpr int kHalfPre = kFfnPrefetch / 2;
+    u32x4 hp[kHalfPre];
+    auto fetch_half = [&](int c, int part) {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(wpack + (int64_t)c * kFfnChunkHalfs);
+#pragma unroll
+        for (int q = 0; q < kHalfPre; ++q) hp[q] = src[tid + (part * kHalfPre + q) * kFfnThreads];
+    };
+    auto stash_half = [&](int buf, int part) {
+        u32x4 *dst = reinterpret_cast<u32x4 *>(s_w[buf]);
+#pragma unroll
+        for (int q = 0; q < kHalfPre; ++q) dst[tid + (part * kHalfPre + q) * kFfnThreads] = hp[q];
     };
     fetch(0, pre);
     fetch(1, pre1);
@@ -157,65 +171,95 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
     __builtin_amdgcn_s_waitcnt(0x0f70);  // every load so far is back: no wait on them inside the loop
     __syncthreads();
 
-    // gate/up operands of the chunk about to be used, read one chunk ahead of their use
-    u32x4 ag[8], au[8];
-    auto read_gate_up = [&](int buf) {
-        const uint16_t *wb = s_w[buf] + lane * 8;
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-            ag[ks] = *reinterpret_cast<const u32x4 *>(wb + ks * 512);
-            au[ks] = *reinterpret_cast<const u32x4 *>(wb + 4096 + ks * 512);
-        }
+    // ---- the chunk loop, software-pipelined inside the wave ----
+    // Step c issues the gate/up MFMAs of chunk c+1 between the GELU arithmetic of chunk c
+    // (two elements per pair of MFMAs: about eight vector-ALU operations per MFMA, the ratio
+    // at which neither pipe waits for the other), then the down-projection MFMAs of chunk c.
+    // The LDS latency of the operand reads hides behind the same arithmetic.
+    auto gate_up_pair = [&](const uint16_t *wgu, int ks, f32x16 &gn, f32x16 &un) {
+        const bf16x8 a0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(wgu + ks * 512));
+        const bf16x8 a1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(wgu + 4096 + ks * 512));
+        gn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, nb[ks], gn, 0, 0, 0);
+        un = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, nb[ks], un, 0, 0, 0);
     };
-    read_gate_up(0);
+    f32x16 gA = {0.0f}, uA = {0.0f}, gB = {0.0f}, uB = {0.0f};
+    {
+        const uint16_t *wgu = s_w[0] + lane * 8;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) gate_up_pair(wgu, ks, gA, uA);
+    }
 
-    int buf = 0;  // c % 3
-    for (int c = 0; c < kFfnChunks; ++c) {
+    // FETCH: chunk c+2 exists and is brought in; NEXT: chunk c+1 exists and its gate/up products are formed
+    auto step = [&](auto fetch_tag, auto next_tag, int c, int buf, const f32x16 &g, const f32x16 &u, f32x16 &gn,
+                    f32x16 &un) {
+        constexpr bool FETCH = decltype(fetch_tag)::value, NEXT = decltype(next_tag)::value;
         const int buf1 = buf == 2 ? 0 : buf + 1;
         const int buf2 = buf1 == 2 ? 0 : buf1 + 1;
-        if (c + 2 < kFfnChunks) fetch(c + 2, pre);
-
-        f32x16 g = {0.0f}, u = {0.0f};
+        if (FETCH) fetch_half(c + 2, 0);
+        const uint16_t *wgu = s_w[buf1] + lane * 8;
+        const uint16_t *wd = s_w[buf] + lane * 8 + 8192;
+        bf16x8 hb[2];
+        if (NEXT) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) gn[v] = un[v] = 0.0f;
+        }
+        // operands are read one MFMA pair ahead of their use, the first down-projection operands
+        // during the last of the GELU arithmetic (into registers g and u give up)
+        u32x4 a0 = {0u, 0u, 0u, 0u}, a1 = a0, ad[8];
+        if (NEXT) {
+            a0 = *reinterpret_cast<const u32x4 *>(wgu);
+            a1 = *reinterpret_cast<const u32x4 *>(wgu + 4096);
+        }
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
-            g = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ag[ks]), nb[ks], g, 0, 0, 0);
-            u = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, au[ks]), nb[ks], u, 0, 0, 0);
+            u32x4 n0 = a0, n1 = a1;
+            if (NEXT && ks < 7) {
+                n0 = *reinterpret_cast<const u32x4 *>(wgu + (ks + 1) * 512);
+                n1 = *reinterpret_cast<const u32x4 *>(wgu + 4096 + (ks + 1) * 512);
+            }
+            if (NEXT) {
+                gn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a0), nb[ks], gn, 0, 0, 0);
+                un = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a1), nb[ks], un, 0, 0, 0);
+            }
+            // h = bf16(gelu(g) * u): one rounding where the library composition has four
+#pragma unroll
+            for (int v = 2 * ks; v < 2 * ks + 2; ++v) hb[v >> 3][v & 7] = (__bf16)(gelu_as(g[v]) * u[v]);
+            if (ks >= 6) {
+                ad[2 * (ks - 6)] = *reinterpret_cast<const u32x4 *>(wd + (2 * (ks - 6)) * 512);
+                ad[2 * (ks - 6) + 1] = *reinterpret_cast<const u32x4 *>(wd + (2 * (ks - 6) + 1) * 512);
+            }
+            a0 = n0;
+            a1 = n1;
+            if (FETCH && ks == 3) {
+                stash_half(buf2, 0);
+                fetch_half(c + 2, 1);
+            }
         }
-        // the first half of the down-projection operands arrives while the vector ALU works
-        // on gelu(g) * u, the second half while the first four MFMAs run
-        const uint16_t *wd = s_w[buf] + lane * 8 + 8192;
-        u32x4 ad[4];
+        // operand (cb, t) sits at index 2cb + t; blocks 0 and 1 are in, 2 and 3 follow while those MFMAs run
 #pragma unroll
-        for (int q = 0; q < 4; ++q) ad[q] = *reinterpret_cast<const u32x4 *>(wd + q * 512);
-
-        // h = bf16(gelu(g) * u): one rounding where the library composition has four (GEMM
-        // outputs, F.gelu, product); this part is bound by vector-ALU issue, every op counts
-        bf16x8 hb[2];
+        for (int q = 0; q < 4; ++q) ad[4 + q] = *reinterpret_cast<const u32x4 *>(wd + (4 + q) * 512);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) hb[v >> 3][v & 7] = (__bf16)(gelu_as(g[v]) * u[v]);
-
-        u32x4 ad2[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) ad2[q] = *reinterpret_cast<const u32x4 *>(wd + (4 + q) * 512);
-#pragma unroll
-        for (int cb = 0; cb < 2; ++cb) {
+        for (int cb = 0; cb < 4; ++cb) {
 #pragma unroll
             for (int t = 0; t < 2; ++t)
                 acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ad[cb * 2 + t]), hb[t],
                                                                   acc[cb], 0, 0, 0);
         }
-#pragma unroll
-        for (int cb = 2; cb < 4; ++cb) {
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ad2[(cb - 2) * 2 + t]),
-                                                                  hb[t], acc[cb], 0, 0, 0);
-        }
-        if (c + 1 < kFfnChunks) read_gate_up(buf1);  // complete in LDS since the previous barrier
-        if (c + 2 < kFfnChunks) stash(buf2, pre);
+        if (FETCH) stash_half(buf2, 1);
         __syncthreads();
-        buf = buf1;
+    };
+    using yes = std::integral_constant<bool, true>;
+    using no = std::integral_constant<bool, false>;
+    int buf = 0;  // chunk % 3
+    for (int c = 0; c < kFfnChunks - 2; c += 2) {
+        step(yes{}, yes{}, c, buf, gA, uA, gB, uB);
+        buf = buf == 2 ? 0 : buf + 1;
+        step(yes{}, yes{}, c + 1, buf, gB, uB, gA, uA);
+        buf = buf == 2 ? 0 : buf + 1;
     }
+    step(no{}, yes{}, kFfnChunks - 2, buf, gA, uA, gB, uB);
+    buf = buf == 2 ? 0 : buf + 1;
+    step(no{}, no{}, kFfnChunks - 1, buf, gB, uB, gA, uA);
 
     // ---- out: back through the staging area (the loop's last barrier has freed the weight
     //      buffers) so that rows leave as whole 512-byte runs ----
