@@ -22,7 +22,8 @@ template <int THREADS, typename XT, typename GT, typename YT, bool HAS_Y>
 __global__ __launch_bounds__(THREADS) void rglru_step_vec8_kernel(
     const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
     const float *h_in, int64_t h_in_stride, float *h_out, int64_t h_out_stride, YT *__restrict__ y,
-    int64_t R, int D, int rows_per_block, const uint8_t *__restrict__ reset, int rows_per_env)
+    int64_t R, int D, int rows_per_block, const uint8_t *__restrict__ reset, int rows_per_env,
+    int64_t y_group_stride)
 {
     extern __shared__ float s_l2sig[];  // D entries
     for (int d = threadIdx.x; d < D; d += THREADS) s_l2sig[d] = log2_sigmoid(log_lambda[d]);
@@ -38,7 +39,9 @@ __global__ __launch_bounds__(THREADS) void rglru_step_vec8_kernel(
     const Row8 ga = load8_stream(gates + row * 2 * D + d0);
     const Row8 gx = load8_stream(gates + row * 2 * D + D + d0);
     Row8 hv = load8_stream(h_in + row * h_in_stride + d0);
-    if (reset != nullptr && reset[row / rows_per_env]) {
+    // environment of the row: for the reset flag and for an output laid out per environment
+    const int64_t env = (reset != nullptr || y_group_stride != 0) ? row / rows_per_env : 0;
+    if (reset != nullptr && reset[env]) {
         // the environment was reset before this step: its previous state reads as zero
 #pragma unroll
         for (int e = 0; e < 8; ++e) hv.v[e] = 0.0f;
@@ -50,7 +53,11 @@ __global__ __launch_bounds__(THREADS) void rglru_step_vec8_kernel(
         out.v[e] = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(xv.v[e], ga.v[e], gx.v[e],
                                                                           s_l2sig[d0 + e], c, hv.v[e]);
     store8_stream(h_out + row * h_out_stride + d0, out);
-    if (HAS_Y) store8_stream(y + row * D + d0, out);
+    if (HAS_Y) {
+        // y rows either back to back or in groups of rows_per_env, y_group_stride elements apart
+        const int64_t y_off = y_group_stride != 0 ? env * y_group_stride + (row - env * rows_per_env) * D : row * D;
+        store8_stream(y + y_off + d0, out);
+    }
 }
 
 // Any D, any alignment: one lane per element.
@@ -58,24 +65,28 @@ template <typename XT, typename GT, typename YT, bool HAS_Y>
 __global__ __launch_bounds__(kRglruThreads) void rglru_step_scalar_kernel(
     const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
     const float *h_in, int64_t h_in_stride, float *h_out, int64_t h_out_stride, YT *__restrict__ y,
-    int64_t R, int D, const uint8_t *__restrict__ reset, int rows_per_env)
+    int64_t R, int D, const uint8_t *__restrict__ reset, int rows_per_env, int64_t y_group_stride)
 {
     const int64_t idx = (int64_t)blockIdx.x * kRglruThreads + threadIdx.x;
     if (idx >= R * D) return;
     const int64_t row = idx / D;
     const int d = (int)(idx - row * D);
-    const float h_prev = (reset != nullptr && reset[row / rows_per_env]) ? 0.0f : h_in[row * h_in_stride + d];
+    const int64_t env = (reset != nullptr || y_group_stride != 0) ? row / rows_per_env : 0;
+    const float h_prev = (reset != nullptr && reset[env]) ? 0.0f : h_in[row * h_in_stride + d];
     const float out = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(
         load1(x + idx), load1(gates + row * 2 * D + d), load1(gates + row * 2 * D + D + d),
         log2_sigmoid(log_lambda[d]), c, h_prev);
     h_out[row * h_out_stride + d] = out;
-    if (HAS_Y) store1(y + idx, out);
+    if (HAS_Y) {
+        const int64_t y_off = y_group_stride != 0 ? env * y_group_stride + (row - env * rows_per_env) * D : row * D;
+        store1(y + y_off + d, out);
+    }
 }
 
 template <typename XT, typename GT, typename YT, bool HAS_Y>
 static int launch_rglru(const void *x, const void *gates, const float *log_lambda, float c, const float *h_in,
                         int64_t h_in_stride, float *h_out, int64_t h_out_stride, void *y, int64_t R, int D,
-                        const uint8_t *reset, int rows_per_env, hipStream_t stream)
+                        const uint8_t *reset, int rows_per_env, int64_t y_group_stride, hipStream_t stream)
 {
     const bool vec = (D % 8 == 0) && (D / 8 <= kRglruThreads) && aligned16(x) && aligned16(gates) &&
                      aligned16(h_in) && aligned16(h_out) && (!HAS_Y || aligned16(y)) &&
@@ -92,18 +103,18 @@ static int launch_rglru(const void *x, const void *gates, const float *log_lambd
             hipLaunchKernelGGL((rglru_step_vec8_kernel<kRglruBigThreads, XT, GT, YT, HAS_Y>), dim3((unsigned)blocks),
                                dim3(threads), (size_t)D * sizeof(float), stream, (const XT *)x, (const GT *)gates,
                                log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D,
-                               rows_per_block, reset, rows_per_env);
+                               rows_per_block, reset, rows_per_env, y_group_stride);
         else
             hipLaunchKernelGGL((rglru_step_vec8_kernel<kRglruThreads, XT, GT, YT, HAS_Y>), dim3((unsigned)blocks),
                                dim3(threads), (size_t)D * sizeof(float), stream, (const XT *)x, (const GT *)gates,
                                log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D,
-                               rows_per_block, reset, rows_per_env);
+                               rows_per_block, reset, rows_per_env, y_group_stride);
     } else {
         const int64_t blocks = (R * D + kRglruThreads - 1) / kRglruThreads;
         if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
         hipLaunchKernelGGL((rglru_step_scalar_kernel<XT, GT, YT, HAS_Y>), dim3((unsigned)blocks),
                            dim3(kRglruThreads), 0, stream, (const XT *)x, (const GT *)gates, log_lambda, c,
-                           h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D, reset, rows_per_env);
+                           h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D, reset, rows_per_env, y_group_stride);
     }
     return (int)hipGetLastError();
 }
@@ -111,25 +122,25 @@ static int launch_rglru(const void *x, const void *gates, const float *log_lambd
 template <typename XT, typename GT>
 static int dispatch_y(const void *x, const void *gates, const float *log_lambda, float c, const float *h_in,
                       int64_t h_in_stride, float *h_out, int64_t h_out_stride, void *y, int y_dtype, int64_t R,
-                      int D, const uint8_t *reset, int rows_per_env, hipStream_t stream)
+                      int D, const uint8_t *reset, int rows_per_env, int64_t y_group_stride, hipStream_t stream)
 {
     if (y == nullptr)
         return launch_rglru<XT, GT, float, false>(x, gates, log_lambda, c, h_in, h_in_stride, h_out,
-                                                  h_out_stride, nullptr, R, D, reset, rows_per_env, stream);
+                                                  h_out_stride, nullptr, R, D, reset, rows_per_env, 0, stream);
     if (y_dtype == BNB_F32)
         return launch_rglru<XT, GT, float, true>(x, gates, log_lambda, c, h_in, h_in_stride, h_out,
-                                                 h_out_stride, y, R, D, reset, rows_per_env, stream);
+                                                 h_out_stride, y, R, D, reset, rows_per_env, y_group_stride, stream);
     return launch_rglru<XT, GT, uint16_t, true>(x, gates, log_lambda, c, h_in, h_in_stride, h_out,
-                                                h_out_stride, y, R, D, reset, rows_per_env, stream);
+                                                h_out_stride, y, R, D, reset, rows_per_env, y_group_stride, stream);
 }
 
 }  // namespace bnb
 
-extern "C" int bnb_rglru_step_reset_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
-                                        const float *log_lambda, float c, const float *h_in,
-                                        int64_t h_in_row_stride, float *h_out, int64_t h_out_row_stride,
-                                        void *y, int y_dtype, const uint8_t *reset, int rows_per_env, int64_t R,
-                                        int D, void *stream)
+extern "C" int bnb_rglru_step_rows_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
+                                       const float *log_lambda, float c, const float *h_in,
+                                       int64_t h_in_row_stride, float *h_out, int64_t h_out_row_stride, void *y,
+                                       int y_dtype, int64_t y_group_stride, const uint8_t *reset,
+                                       int rows_per_env, int64_t R, int D, void *stream)
 {
     using namespace bnb;
     if (R < 0 || D < 1) return BNB_ERR_BAD_SHAPE;
@@ -139,24 +150,36 @@ extern "C" int bnb_rglru_step_reset_fwd(const void *x, int x_dtype, const void *
         (y && y_dtype != BNB_F32 && y_dtype != BNB_BF16))
         return BNB_ERR_BAD_DTYPE;
     if (h_in_row_stride < D || h_out_row_stride < D) return BNB_ERR_BAD_SHAPE;
-    if (reset != nullptr && rows_per_env < 1) return BNB_ERR_BAD_SHAPE;
+    if ((reset != nullptr || y_group_stride != 0) && rows_per_env < 1) return BNB_ERR_BAD_SHAPE;
+    if (y_group_stride != 0 && (!y || y_group_stride < (int64_t)rows_per_env * D || y_group_stride % 8 != 0))
+        return BNB_ERR_BAD_SHAPE;
     if ((reinterpret_cast<uintptr_t>(h_in) | reinterpret_cast<uintptr_t>(h_out) |
          reinterpret_cast<uintptr_t>(log_lambda)) & 3u)
         return BNB_ERR_MISALIGNED;
-    if (reset == nullptr) rows_per_env = 1;
+    if (reset == nullptr && y_group_stride == 0) rows_per_env = 1;
     hipStream_t s = (hipStream_t)stream;
     const bool xb = x_dtype == BNB_BF16, gb = g_dtype == BNB_BF16;
     if (!xb && !gb)
         return dispatch_y<float, float>(x, gates_pre, log_lambda, c, h_in, h_in_row_stride, h_out,
-                                        h_out_row_stride, y, y_dtype, R, D, reset, rows_per_env, s);
+                                        h_out_row_stride, y, y_dtype, R, D, reset, rows_per_env, y_group_stride, s);
     if (xb && gb)
         return dispatch_y<uint16_t, uint16_t>(x, gates_pre, log_lambda, c, h_in, h_in_row_stride, h_out,
-                                              h_out_row_stride, y, y_dtype, R, D, reset, rows_per_env, s);
+                                              h_out_row_stride, y, y_dtype, R, D, reset, rows_per_env, y_group_stride, s);
     if (!xb && gb)
         return dispatch_y<float, uint16_t>(x, gates_pre, log_lambda, c, h_in, h_in_row_stride, h_out,
-                                           h_out_row_stride, y, y_dtype, R, D, reset, rows_per_env, s);
+                                           h_out_row_stride, y, y_dtype, R, D, reset, rows_per_env, y_group_stride, s);
     return dispatch_y<uint16_t, float>(x, gates_pre, log_lambda, c, h_in, h_in_row_stride, h_out,
-                                       h_out_row_stride, y, y_dtype, R, D, reset, rows_per_env, s);
+                                       h_out_row_stride, y, y_dtype, R, D, reset, rows_per_env, y_group_stride, s);
+}
+
+extern "C" int bnb_rglru_step_reset_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
+                                        const float *log_lambda, float c, const float *h_in,
+                                        int64_t h_in_row_stride, float *h_out, int64_t h_out_row_stride,
+                                        void *y, int y_dtype, const uint8_t *reset, int rows_per_env, int64_t R,
+                                        int D, void *stream)
+{
+    return bnb_rglru_step_rows_fwd(x, x_dtype, gates_pre, g_dtype, log_lambda, c, h_in, h_in_row_stride, h_out,
+                                   h_out_row_stride, y, y_dtype, 0, reset, rows_per_env, R, D, stream);
 }
 
 extern "C" int bnb_rglru_step_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,

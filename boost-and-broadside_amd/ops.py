@@ -195,7 +195,9 @@ def rglru_step(
                     itself for an in-place update).  Default: a new contiguous tensor.
         y_dtype:    dtype of the returned layer output.  None or float32 returns the new
                     state itself; bfloat16 makes the kernel write a rounded copy as well.
-        y_out:      optional preallocated contiguous bfloat16 (R, D) destination for that copy.
+        y_out:      optional preallocated destination of the layer output, float32 or bfloat16:
+                    contiguous (R, D), or a (B, rows_per_env, D) view into a wider token tensor
+                    (``tokens[:, :n]``), which the kernel then fills in place.
         reset:      optional (R / rows_per_env,) bool: environments whose previous state must
                     read as zero (``reset_hidden_for_envs`` folded into this step).
         rows_per_env: consecutive rows that belong to one environment (rows are env-major).
@@ -230,27 +232,47 @@ def rglru_step(
             raise ValueError("h_out must be a float32 (R, D) tensor on x's device")
         if R and h_out.stride(-1) != 1:
             raise ValueError("h_out must be contiguous in its last dim")
-    y = None
-    if y_dtype is not None and y_dtype != torch.float32:
+    y, y_group = None, 0
+    if y_out is not None:
+        # caller-owned destination in either dtype; a (B, n, D) view puts the rows of every
+        # environment into a wider token tensor
+        if y_out.dtype not in _DTYPE_CODE or y_out.device != x.device:
+            raise ValueError("y_out must be a float32 or bfloat16 tensor on x's device")
+        if y_dtype is not None and y_dtype != y_out.dtype:
+            raise ValueError("y_dtype and y_out disagree")
+        if y_out.dim() == 3:
+            y_group = _grouped_rows(y_out, R, D, rows_per_env, "y_out")
+        elif y_out.shape != (R, D) or not y_out.is_contiguous():
+            raise ValueError("y_out must be a contiguous (R, D) tensor or a (B, n, D) view")
+        y = y_out
+    elif y_dtype is not None and y_dtype != torch.float32:
         if y_dtype != torch.bfloat16:
             raise TypeError(f"y_dtype must be float32 or bfloat16, got {y_dtype}")
-        if y_out is None:
-            y = torch.empty((R, D), dtype=torch.bfloat16, device=x.device)
-        elif y_out.shape != (R, D) or y_out.dtype != torch.bfloat16 or y_out.device != x.device or not y_out.is_contiguous():
-            raise ValueError("y_out must be a contiguous bfloat16 (R, D) tensor on x's device")
-        else:
-            y = y_out
+        y = torch.empty((R, D), dtype=torch.bfloat16, device=x.device)
     reset_ptr = _reset_pointer(reset, R, rows_per_env, x.device)
     if R == 0:
         return (h_out if y is None else y), h_out
     with torch.cuda.device(x.device):
-        rc = _native.load().bnb_rglru_step_reset_fwd(
+        rc = _native.load().bnb_rglru_step_rows_fwd(
             x.data_ptr(), x_code, gates_pre.data_ptr(), g_code, log_lambda.data_ptr(), float(c),
             h.data_ptr(), h.stride(0), h_out.data_ptr(), h_out.stride(0),
-            None if y is None else y.data_ptr(), _native.BF16, reset_ptr, int(rows_per_env), R, D, _stream(),
+            None if y is None else y.data_ptr(), _native.BF16 if y is None else _DTYPE_CODE[y.dtype], int(y_group),
+            reset_ptr, int(rows_per_env), R, D, _stream(),
         )
     _native.check(rc, "bnb_rglru_step_fwd")
     return (h_out if y is None else y), h_out
+
+
+def _grouped_rows(t: torch.Tensor, R: int, D: int, rows_per_env: int, name: str) -> int:
+    """Group stride (elements) of a (B, n, D) view whose rows are the R = B*n rows of one
+    environment after the other inside a wider tensor: ``t[b, i]`` at ``b * stride(0) + i * D``."""
+    if t.dim() != 3 or t.shape[2] != D or t.shape[0] * t.shape[1] != R:
+        raise ValueError(f"{name} must be (R, D) or a (B, n, D) view with B*n == R")
+    if t.shape[1] != rows_per_env:
+        raise ValueError(f"{name} groups rows by {t.shape[1]}, rows_per_env is {rows_per_env}")
+    if R and (t.stride(2) != 1 or t.stride(1) != D or t.stride(0) < t.shape[1] * D or t.stride(0) % 8):
+        raise ValueError(f"{name} must have contiguous rows, D apart, and a group stride that is a multiple of 8")
+    return t.stride(0) if t.shape[0] > 1 else t.shape[1] * D
 
 
 def _reset_pointer(reset, R: int, rows_per_env: int, device) -> int | None:
@@ -280,7 +302,8 @@ def conv_step(
     """Causal depthwise conv of one timestep and the shift of the stored inputs.
 
     Args:
-        b1:       (R, D) this step's ``linear1`` output, float32 or bfloat16.
+        b1:       (R, D) this step's ``linear1`` output, float32 or bfloat16; or a
+                  (B, rows_per_env, D) view into a wider token tensor (``tokens[:, :n]``).
         conv_buf: (R, 3, D) float32 previous inputs, oldest first; each row's 3*D values must
                   be contiguous, rows may be strided (a view of the packed hidden works).
         weight:   (D, 4) or (D, 1, 4) float32 depthwise taps (``conv.weight``).
@@ -295,9 +318,10 @@ def conv_step(
         (v, new_conv_buf[, v_bf16]): conv output (R, D) float32, the shifted buffer
         ``[p1, p2, b1]``, and the bfloat16 copy when asked for.
     """
-    if b1.dim() != 2 or conv_buf.dim() != 3:
-        raise ValueError("b1 must be (R, D) and conv_buf (R, 3, D)")
-    R, D = b1.shape
+    if b1.dim() not in (2, 3) or conv_buf.dim() != 3:
+        raise ValueError("b1 must be (R, D) or a (B, rows_per_env, D) view, and conv_buf (R, 3, D)")
+    D = b1.shape[-1]
+    R = b1.numel() // D if D else 0
     if conv_buf.shape != (R, 3, D):
         raise ValueError(f"conv_buf must be {(R, 3, D)}, got {tuple(conv_buf.shape)}")
     for name, t in (("b1", b1), ("conv_buf", conv_buf), ("weight", weight)):
@@ -312,7 +336,11 @@ def conv_step(
     if bias is not None:
         bias = bias.detach().contiguous()
         bias_ptr = bias.data_ptr()
-    b1 = b1.contiguous()
+    b1_group = 0
+    if b1.dim() == 3 and not b1.is_contiguous():
+        b1_group = _grouped_rows(b1, R, D, rows_per_env, "b1")  # rows of every environment inside a wider tensor
+    else:
+        b1 = b1.contiguous()
 
     def rows_ok(t):
         return R == 0 or (t.stride(2) == 1 and t.stride(1) == D)
@@ -328,8 +356,8 @@ def conv_step(
     reset_ptr = _reset_pointer(reset, R, rows_per_env, b1.device)
     if R:
         with torch.cuda.device(b1.device):
-            rc = _native.load().bnb_conv_step_fwd(
-                b1.data_ptr(), b_code, conv_buf.data_ptr(), conv_buf.stride(0), weight.data_ptr(), bias_ptr,
+            rc = _native.load().bnb_conv_step_rows_fwd(
+                b1.data_ptr(), b_code, int(b1_group), conv_buf.data_ptr(), conv_buf.stride(0), weight.data_ptr(), bias_ptr,
                 reset_ptr, int(rows_per_env), v.data_ptr(), None if v_lp is None else v_lp.data_ptr(),
                 conv_out.data_ptr(), conv_out.stride(0), R, D, _stream(),
             )

@@ -271,7 +271,7 @@ class RGLRU(nn.Module):
         """(R,D), (R,D) -> new state (R,D) float32 (also the layer output)."""
         return self.step(x, h)[1]
 
-    def step(self, x, h, y_dtype=None, *, h_out=None, reset=None, rows_per_env=1, x_act=None):
+    def step(self, x, h, y_dtype=None, *, h_out=None, reset=None, rows_per_env=1, x_act=None, y_out=None):
         """One kernel launch: returns (output in ``y_dtype`` or the state itself, new state).
 
         ``h_out`` lets the new state land in place (e.g. in the RG-LRU columns of a packed
@@ -280,7 +280,7 @@ class RGLRU(nn.Module):
         """
         return ops.rglru_step(
             x, self._gate_preactivations(x, x_act), self.log_lambda, self.c, h, y_dtype=y_dtype, h_out=h_out,
-            reset=reset, rows_per_env=rows_per_env,
+            reset=reset, rows_per_env=rows_per_env, y_out=y_out,
         )
 
     def forward_sequence(self, x_seq, h0, done_mask=None, *, time_major=False, y_dtype=torch.float32, x_act=None,
@@ -403,6 +403,33 @@ class GriffinTemporalBlock(nn.Module):
             state_out[:, D:].view(R, CONV_KERNEL - 1, D), reset, rows_per_env,
         )[0]
 
+    def step_tokens(self, x, n_rec, state_in, state_out, reset, field_sub):
+        """One timestep over all tokens of every environment at once.
+
+        x (B, NM, D): the first ``n_rec`` tokens of an environment are recurrent (state rows
+        ``state_in`` / ``state_out`` (B*n_rec, 4*D) as in ``step_packed``), the rest go through
+        ``field_sub`` instead of conv + RG-LRU.  Norms, projections, gate and the sublayer tail
+        run once over all rows; the conv kernel reads its rows out of the (B, NM, D) projection
+        and the recurrence writes its output into the (B, NM, D) gate operand in place, so the
+        reference's slicing and concatenation of ship and field tokens (griffin.py:390-417)
+        costs nothing.  Returns (B, NM, D).
+        """
+        B, NM, D = x.shape
+        R = B * n_rec
+        act = _projection_dtype()
+        normed = self._norm_in(x)
+        b1 = _project(self.linear1, normed)
+        want_lp = act == torch.bfloat16
+        res = ops.conv_step(b1[:, :n_rec] if NM > n_rec else b1.reshape(R, D), state_in[:, D:].view(R, CONV_KERNEL - 1, D),
+                            self.conv.weight, self.conv.bias, conv_out=state_out[:, D:].view(R, CONV_KERNEL - 1, D),
+                            reset=reset, rows_per_env=n_rec, also_bf16=want_lp)
+        y = torch.empty((B, NM, D), dtype=act, device=x.device)
+        self.rg_lru.step(res[0], state_in[:, :D], h_out=state_out[:, :D], reset=reset, rows_per_env=n_rec,
+                         x_act=res[2] if want_lp else None, y_out=y[:, :n_rec] if NM > n_rec else y.view(R, D))
+        if NM > n_rec:
+            y[:, n_rec:] = _project(field_sub, b1[:, n_rec:])
+        return self._finish(x, normed, y)
+
     def forward_nonrecurrent(self, x, sub):
         """Same block with ``sub`` (a Linear) in place of conv + RG-LRU; no state."""
         act = _projection_dtype()
@@ -498,7 +525,11 @@ class YemongBlock(nn.Module):
         n_rec = num_recurrent
         for layer in self.spatial:
             x = layer(x, alive, bullets, bullet_mask)
+        act = _projection_dtype()
         for j, layer in enumerate(self.temporal):
+            if _fused_ok(x, act):
+                x = layer.step_tokens(x, n_rec, state_in[j], state_out[j], reset, self.field_sub[j] if NM > n_rec else None)
+                continue
             ships = layer.step_packed(x[:, :n_rec].reshape(B * n_rec, D), state_in[j], state_out[j], reset, n_rec)
             parts = [ships.reshape(B, n_rec, D)]
             if NM > n_rec:

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 7
+#define BNB_ABI_VERSION 8
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -162,6 +162,23 @@ int bnb_rglru_step_reset_fwd(const void *x, int x_dtype, const void *gates_pre, 
                              int64_t R, int D, void *stream);
 
 /*
+ * bnb_rglru_step_reset_fwd with the output y laid out per environment: with
+ * y_group_stride != 0, row r of y is at y + (r / rows_per_env) * y_group_stride +
+ * (r % rows_per_env) * D elements (y_group_stride >= rows_per_env * D, a multiple of 8), which
+ * addresses the ship tokens inside a (B, N+M, D) token tensor (models/yemong/griffin.py:390-417
+ * slices and concatenates ship and field tokens around the temporal operator; writing in
+ * place removes both copies).  y_group_stride == 0: contiguous (R, D).  rows_per_env is used
+ * for the grouping also when reset is NULL.
+ */
+int bnb_rglru_step_rows_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
+                            const float *log_lambda, float c,
+                            const float *h_in, int64_t h_in_row_stride,
+                            float *h_out, int64_t h_out_row_stride,
+                            void *y, int y_dtype, int64_t y_group_stride,
+                            const uint8_t *reset, int rows_per_env,
+                            int64_t R, int D, void *stream);
+
+/*
  * Causal depthwise conv (kernel 4) for one timestep plus the shift of the stored inputs.
  *
  * Replaces, in models/yemong/griffin.py at T = 1: `padded = cat([conv_buf, b1])` (:275), the
@@ -192,6 +209,18 @@ int bnb_conv_step_fwd(const void *b1, int b1_dtype,
                       const uint8_t *reset, int rows_per_env,
                       float *v_out, void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride,
                       int64_t R, int D, void *stream);
+
+/*
+ * bnb_conv_step_fwd with the input b1 laid out per environment: with b1_group_stride != 0,
+ * row r of b1 is at b1 + (r / rows_per_env) * b1_group_stride + (r % rows_per_env) * D elements
+ * (the ship tokens inside a (B, N+M, D) tensor of linear1 outputs).  0: contiguous (R, D).
+ */
+int bnb_conv_step_rows_fwd(const void *b1, int b1_dtype, int64_t b1_group_stride,
+                           const float *conv_in, int64_t conv_in_row_stride,
+                           const float *weight, const float *bias,
+                           const uint8_t *reset, int rows_per_env,
+                           float *v_out, void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride,
+                           int64_t R, int D, void *stream);
 
 /*
  * The same causal depthwise conv over a whole sequence of T steps per row, with episode

@@ -809,3 +809,39 @@ def test_ffn_fused_every_weight_reaches_its_output():
         want[k] = 3.0 * h
         assert torch.allclose(got[0], want, rtol=1e-2, atol=1e-6), (j, k)
         assert torch.equal(got[0], got[63])
+
+
+# ------------------------------------------------------------------ rows addressed inside a wider (B, N+M, D) token tensor
+
+
+@pytest.mark.parametrize("B,n,NM", [(3, 8, 12), (5, 19, 23), (1, 4, 9), (600, 8, 12)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_state_kernels_address_ship_rows_inside_the_token_tensor(B, n, NM, dtype):
+    D = 128
+    g = torch.Generator().manual_seed(B * 31 + NM)
+    tokens = torch.randn(B, NM, D, generator=g).to(dtype).to(DEV)   # linear1 outputs of all tokens
+    buf = torch.randn(B * n, 3, D, generator=g).to(DEV)
+    w = (0.5 * torch.randn(D, 1, 4, generator=g)).to(DEV)
+    bias = (0.1 * torch.randn(D, generator=g)).to(DEV)
+    reset = (torch.rand(B, generator=g) < 0.4).to(DEV)
+    view = tokens[:, :n]
+    v_a, buf_a = ops.conv_step(view, buf, w, bias, reset=reset, rows_per_env=n)
+    v_b, buf_b = ops.conv_step(view.reshape(B * n, D).contiguous(), buf, w, bias, reset=reset, rows_per_env=n)
+    assert torch.equal(v_a, v_b) and torch.equal(buf_a, buf_b)
+    # recurrence output written into the first n tokens of a wider tensor, the rest untouched
+    gates = torch.randn(B * n, 2 * D, generator=g).to(dtype).to(DEV)
+    h = torch.randn(B * n, D, generator=g).to(DEV)
+    lam = torch.linspace(0.0, 4.0, D).to(DEV)
+    for y_dtype in (torch.float32, torch.bfloat16):
+        wide = torch.full((B, NM, D), 7.0, dtype=y_dtype, device=DEV)
+        y, h_new = ops.rglru_step(v_a, gates, lam, 8.0, h, reset=reset, rows_per_env=n, y_out=wide[:, :n])
+        y_ref, h_ref = ops.rglru_step(v_a, gates, lam, 8.0, h, reset=reset, rows_per_env=n, y_dtype=y_dtype)
+        assert torch.equal(h_new, h_ref)
+        assert torch.equal(wide[:, :n].reshape(B * n, D), y_ref.to(y_dtype))
+        assert (wide[:, n:] == 7.0).all()
+    # no reset mask: the grouping alone still needs rows_per_env
+    wide = torch.zeros((B, NM, D), dtype=torch.float32, device=DEV)
+    ops.rglru_step(v_a, gates, lam, 8.0, h, rows_per_env=n, y_out=wide[:, :n])
+    assert torch.equal(wide[:, :n].reshape(B * n, D), ops.rglru_step(v_a, gates, lam, 8.0, h)[1])
+    with pytest.raises(ValueError):
+        ops.rglru_step(v_a, gates, lam, 8.0, h, rows_per_env=n + 1, y_out=wide[:, :n])
