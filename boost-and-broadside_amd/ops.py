@@ -747,3 +747,107 @@ def ffn_fused(
             )
         _native.check(rc, "bnb_ffn_fused_fwd")
     return out.reshape(x.shape)
+
+
+def pack_linear_weights(weight: torch.Tensor) -> torch.Tensor:
+    """A Linear weight (N, 128), N a multiple of 64, as the bfloat16 operand stream of
+    ``norm_linear``: ``[fb][ks][l][e]`` with the index meaning given in ``include/bnb_amd.h``
+    (every matrix-core operand one contiguous 1 KB run; a lane's 16 outputs per block of 32
+    features are two runs of 8 consecutive features)."""
+    N, D = weight.shape
+    if D != FFN_WIDTH or N % 64:
+        raise ValueError("norm_linear covers (N, 128) weights with N a multiple of 64")
+    dev = weight.device
+    lane = torch.arange(64, device=dev)
+    r, half = lane % 32, lane // 32
+    e = torch.arange(8, device=dev)
+    fb = torch.arange(N // 32, device=dev)
+    ks = torch.arange(8, device=dev)
+    feat = 16 * ((r // 8) // 2) + 8 * ((r // 4) % 2) + 4 * ((r // 8) % 2) + r % 4  # (64,)
+    rows = (32 * fb[:, None, None, None] + feat[None, None, :, None]).expand(-1, 8, -1, 8)
+    cols = (16 * ks[None, :, None, None] + 8 * (e // 4)[None, None, None, :] + 4 * half[None, None, :, None]
+            + (e % 4)[None, None, None, :]).expand(N // 32, -1, -1, -1)
+    return weight.detach().to(torch.bfloat16)[rows, cols].contiguous()
+
+
+class CompactRows:
+    """The set entries of a (B, n) bool mask as a device-side list: ``index`` (capacity B*n,
+    int32 flat positions b*n + j, ascending, the first ``offsets[B]`` valid) and ``offsets``
+    (B+1, int32 exclusive prefix of the per-row counts).  Built without any copy to the host."""
+
+    def __init__(self, mask: torch.Tensor) -> None:
+        if mask.dim() != 2 or mask.dtype not in (torch.bool, torch.uint8):
+            raise ValueError("mask must be a bool (B, n) tensor")
+        _need_device(mask, "mask")
+        mask = mask.contiguous()
+        B, n = mask.shape
+        if B * n >= 2 ** 31:
+            raise ValueError("mask too large for 32-bit row positions")
+        self.shape = (B, n)
+        counts = torch.empty(B, dtype=torch.int32, device=mask.device)
+        self.offsets = torch.zeros(B + 1, dtype=torch.int32, device=mask.device)
+        self.index = torch.empty(max(B * n, 1), dtype=torch.int32, device=mask.device)
+        if B and n:
+            lib = _native.load()
+            with torch.cuda.device(mask.device):
+                _native.check(lib.bnb_mask_count(mask.data_ptr(), counts.data_ptr(), B, n, _stream()), "bnb_mask_count")
+                torch.cumsum(counts, dim=0, dtype=torch.int32, out=self.offsets[1:])
+                _native.check(lib.bnb_mask_fill(mask.data_ptr(), self.offsets.data_ptr(), self.index.data_ptr(), B, n,
+                                                _stream()), "bnb_mask_fill")
+
+    @property
+    def total(self) -> torch.Tensor:
+        """Number of valid entries, as a one-element int32 device tensor."""
+        return self.offsets[-1:]
+
+
+def norm_linear(
+    x: torch.Tensor,
+    norm_weight: torch.Tensor,
+    weight_packed: torch.Tensor,
+    bias: torch.Tensor | None = None,
+    *,
+    eps: float | None = None,
+    rows: CompactRows | None = None,
+) -> torch.Tensor:
+    """``linear(rmsnorm(x) * norm_weight)`` in one matrix-core kernel with bfloat16 projection.
+
+    x (..., 128) float32 with contiguous rows; ``weight_packed`` from ``pack_linear_weights``
+    (N features).  With ``rows`` only the listed rows of the flattened x are projected, into
+    the leading ``rows.total`` rows of a (capacity, N) result in list order; the remaining
+    rows of the result are left unwritten.  Returns bfloat16 (..., N), or (capacity, N) with ``rows``.
+    """
+    D = x.shape[-1]
+    if not (x.is_cuda and x.dtype == torch.float32 and D == FFN_WIDTH):
+        raise RuntimeError("norm_linear covers float32 (..., 128) inputs on the GPU")
+    if torch.is_grad_enabled() and x.requires_grad:
+        raise RuntimeError("norm_linear is forward-only; call it under torch.no_grad()")
+    if weight_packed.dtype != torch.bfloat16 or weight_packed.dim() != 4 or not weight_packed.is_contiguous():
+        raise ValueError("weight_packed must come from pack_linear_weights")
+    N = weight_packed.shape[0] * 32
+    if norm_weight.shape != (D,) or norm_weight.dtype != torch.float32:
+        raise ValueError(f"norm_weight must be a float32 {(D,)} tensor")
+    x2 = x.reshape(-1, D)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    R = x2.shape[0]
+    if rows is not None and rows.shape[0] * rows.shape[1] != R:
+        raise ValueError("rows was built for a mask of a different size")
+    bias_ptr = None
+    if bias is not None:
+        if bias.shape != (N,):
+            raise ValueError(f"bias must have {N} entries")
+        bias = bias.detach().float().contiguous()
+        bias_ptr = bias.data_ptr()
+    out = torch.empty((R, N), dtype=torch.bfloat16, device=x.device)
+    norm_weight = norm_weight.detach().contiguous()
+    if R:
+        with torch.cuda.device(x.device):
+            rc = _native.load().bnb_norm_linear_fwd(
+                x2.data_ptr(), x2.stride(0), None if rows is None else rows.index.data_ptr(),
+                None if rows is None else rows.total.data_ptr(), norm_weight.data_ptr(),
+                float(_F32_EPS if eps is None else eps), weight_packed.data_ptr(), bias_ptr, out.data_ptr(), R, D, N,
+                _stream(),
+            )
+        _native.check(rc, "bnb_norm_linear_fwd")
+    return out if rows is not None else out.reshape(*x.shape[:-1], N)

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 8
+#define BNB_ABI_VERSION 9
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -318,6 +318,42 @@ int bnb_rglru_scan_bwd(const void *x, int x_dtype, const void *gates_pre, int g_
 int bnb_add_rmsnorm_fwd(const float *x, int64_t x_row_stride, const void *delta, int delta_dtype,
                         const float *weight, float eps, float *sum_out, void *norm_out, int out_dtype,
                         int64_t R, int D, void *stream);
+
+/*
+ * RMSNorm + Linear in one matrix-core kernel (bf16 projection), optionally over gathered rows:
+ *     out[r] = bf16( rmsnorm(x[src(r)]) * norm_weight @ W^T + bias ),   src(r) = row_index ? row_index[r] : r
+ * Replaces `self.kv_bullet(self.norm_bullet(bullets))` (models/yemong/attention.py:150-151),
+ * `self.qkv(self.norm1(x))` (:94-96,132) and `self.linear1(self.norm1(x))`
+ * (models/yemong/griffin.py:269-272) as they run under bf16 autocast.
+ *
+ *   x              fp32 rows of 128 channels, x_row_stride floats apart
+ *   row_index      optional int32 list: output row r reads x row row_index[r] (a compact list of
+ *                  the bullets in flight, see bnb_mask_fill); NULL = identity
+ *   n_rows         optional device-side int32 count: only the first *n_rows rows are produced
+ *                  (work-groups past it exit), so a data-dependent row count never reaches the
+ *                  host; NULL = R rows.  R is then the capacity the grid is sized for.
+ *   weight_packed  W (N, 128) in bf16, arranged as [fb][ks][l][e] =
+ *                  W[32fb + 16((r/8)/2) + 8((r/4)%2) + 4((r/8)%2) + r%4][16ks + 8(e/4) + 4(l/32) + e%4],
+ *                  r = l%32, fb = 0..N/32-1, ks = 0..7, l = 0..63, e = 0..7
+ *   bias           optional fp32 (N)
+ *   out            (R, N) bf16 contiguous
+ * Requirements: D == 128, N % 64 == 0, 16-byte aligned pointers.  The normalisation factor
+ * is applied to the products (a per-row scalar), the operand is bf16(x * norm_weight).
+ */
+int bnb_norm_linear_fwd(const float *x, int64_t x_row_stride, const int32_t *row_index,
+                        const int32_t *n_rows, const float *norm_weight, float eps,
+                        const void *weight_packed, const float *bias, void *out,
+                        int64_t R, int D, int N, void *stream);
+
+/*
+ * Compact list of the set entries of a byte mask (B, n), e.g. the bullets in flight of
+ * models/yemong/policy.py:222-228: bnb_mask_count writes the number of set bytes per row;
+ * the caller turns the counts into exclusive offsets (B+1, last = total); bnb_mask_fill writes
+ * index[offsets[b] + k] = b*n + j for the k-th set byte j of row b, ascending.  Nothing is
+ * copied to the host.
+ */
+int bnb_mask_count(const uint8_t *mask, int32_t *counts, int B, int n, void *stream);
+int bnb_mask_fill(const uint8_t *mask, const int32_t *offsets, int32_t *index, int B, int n, void *stream);
 
 /*
  * Residual add + RMSNorm + gated MLP + residual add in one matrix-core kernel (bf16 compute):

@@ -845,3 +845,59 @@ def test_state_kernels_address_ship_rows_inside_the_token_tensor(B, n, NM, dtype
     assert torch.equal(wide[:, :n].reshape(B * n, D), ops.rglru_step(v_a, gates, lam, 8.0, h)[1])
     with pytest.raises(ValueError):
         ops.rglru_step(v_a, gates, lam, 8.0, h, rows_per_env=n + 1, y_out=wide[:, :n])
+
+
+# ------------------------------------------------------------------ RMSNorm + Linear, compact row lists
+
+
+@pytest.mark.parametrize("R,N", [(1, 64), (33, 128), (128, 256), (1000, 384), (70000, 256)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_norm_linear_matches_oracle(R, N, with_bias):
+    g = torch.Generator().manual_seed(R + N)
+    D = 128
+    x = 2.0 * torch.randn(R, D, generator=g)
+    nw = 1.0 + 0.1 * torch.randn(D, generator=g)
+    W = torch.randn(N, D, generator=g) / D ** 0.5
+    bias = 0.2 * torch.randn(N, generator=g) if with_bias else None
+    want = torch.nn.functional.linear(torch_ref.rms_norm(x, nw), W.bfloat16().float(), bias)
+    got = ops.norm_linear(x.to(DEV), nw.to(DEV), ops.pack_linear_weights(W.to(DEV)), None if bias is None else bias.to(DEV))
+    assert got.shape == (R, N) and got.dtype == torch.bfloat16
+    assert max_rel(got.float().cpu(), want) <= BF16_TOL
+
+
+def test_norm_linear_one_hot_weights_hit_the_documented_positions():
+    D, N = 128, 128
+    x = torch.zeros(40, D)
+    x[:, 77] = 3.0
+    nw = torch.ones(D)
+    for f in (0, 5, 31, 64, 127):
+        W = torch.zeros(N, D)
+        W[f, 77] = 1.0
+        got = ops.norm_linear(x.to(DEV), nw.to(DEV), ops.pack_linear_weights(W.to(DEV))).float().cpu()
+        n77 = float(torch_ref.rms_norm(x, nw)[0, 77])
+        want = torch.zeros(N)
+        want[f] = n77
+        assert torch.allclose(got[0], want, rtol=1e-2, atol=1e-6), f
+        assert torch.equal(got[0], got[39])
+
+
+@pytest.mark.parametrize("B,n,p", [(1, 1, 1.0), (5, 80, 0.3), (7, 190, 0.0), (40, 1520, 0.25), (3, 2048, 1.0)])
+def test_compact_rows_and_gathered_projection(B, n, p):
+    g = torch.Generator().manual_seed(B * 7 + n)
+    mask = torch.rand(B, n, generator=g) < p
+    rows = ops.CompactRows(mask.to(DEV))
+    counts = mask.sum(1)
+    offs = torch.cat([torch.zeros(1, dtype=torch.long), counts.cumsum(0)])
+    assert torch.equal(rows.offsets.cpu().long(), offs)
+    total = int(offs[-1])
+    assert torch.equal(rows.index[:total].cpu().long(), mask.flatten().nonzero().flatten())
+    # projection over the listed rows only
+    D, N = 128, 256
+    x = torch.randn(B, n, D, generator=g)
+    nw = 1.0 + 0.1 * torch.randn(D, generator=g)
+    W = torch.randn(N, D, generator=g) / D ** 0.5
+    out = ops.norm_linear(x.to(DEV), nw.to(DEV), ops.pack_linear_weights(W.to(DEV)), rows=rows)
+    assert out.shape == (B * n, N)
+    if total:
+        want = torch.nn.functional.linear(torch_ref.rms_norm(x.reshape(-1, D)[mask.flatten()], nw), W.bfloat16().float())
+        assert max_rel(out[:total].float().cpu(), want) <= BF16_TOL
