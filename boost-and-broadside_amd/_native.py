@@ -12,7 +12,7 @@ import os
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "_lib", "libbnb_amd.so")
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 F32, BF16 = 0, 1
 PATH_AUTO, PATH_VALU, PATH_MFMA = 0, 1, 2
 
@@ -26,6 +26,7 @@ SIGNATURES = {
     "bnb_sdpa_masked_fwd": (_i, [_vp, _i64, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "bnb_sdpa_masked_fwd_path": (_i, [_vp, _i64, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "bnb_sdpa_cross_fwd": (_i, [_vp, _i64, _i, _vp, _vp, _i64, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "bnb_sdpa_cross_ranges_fwd": (_i, [_vp, _i64, _i, _vp, _i64, _vp, _i64, _vp, _vp, _i, _i, _i, _i, _vp]),
     "bnb_rglru_step_fwd": (_i, [_vp, _i, _vp, _i, _vp, _f, _vp, _i64, _vp, _i64, _vp, _i, _i64, _i, _vp]),
     "bnb_rglru_step_reset_fwd": (
         _i, [_vp, _i, _vp, _i, _vp, _f, _vp, _i64, _vp, _i64, _vp, _i, _vp, _i, _i64, _i, _vp]

@@ -437,7 +437,8 @@ template <int NQB>
 __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
     const uint16_t *__restrict__ q, int64_t q_stride, const uint16_t *__restrict__ k,
     const uint16_t *__restrict__ v, int64_t kv_stride, const uint8_t *__restrict__ alive,
-    const uint16_t *accum, uint16_t *out, int B, int NQ, int NK, int H, float scale_log2e)
+    const int32_t *__restrict__ ranges, const uint16_t *accum, uint16_t *out, int B, int NQ, int NK, int H,
+    float scale_log2e)
 {
     constexpr int TK = 32 * NQB;  // keys per tile
     constexpr int VP = TK + 4;    // halfs per V^T row: 8-byte aligned, bank-spread
@@ -460,33 +461,7 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
     const int m = lane & 31;
     const int half = lane >> 5;
 
-    // ---- live-key index list: wave w scans keys [w*J*64, (w+1)*J*64), 64 per ballot ----
-    const uint8_t *alive_env = alive == nullptr ? nullptr : alive + (int64_t)env * NK;
-    const int J = (NK + NT - 1) / NT;  // <= 32 because NK <= kStreamMaxKeys
-    const int key0 = wave * J * 64 + lane;
-    uint32_t bits = 0;
-    int mine = 0;
-    for (int j0 = 0; j0 < J; j0 += 8) {
-        // eight independent byte loads in flight, then their ballots
-        uint32_t a[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int key = key0 + (j0 + u) * 64;
-            const bool in = j0 + u < J && key < NK;
-            a[u] = 1u;
-            if (alive_env != nullptr) a[u] = alive_env[key < NK ? key : NK - 1];  // branch-free: no wait between the loads
-            a[u] = in ? a[u] : 0u;
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const bool on = a[u] != 0;
-            bits |= (on ? 1u : 0u) << ((j0 + u) & 31);
-            mine += (int)__popcll(__ballot(on));
-        }
-    }
-    if (lane == 0) s_wcnt[wave] = mine;
-
-    // this wave's queries, in flight while the index list is built
+    // this wave's queries, in flight while the key list is set up
     const int qrow = wave * 32 + m;
     const int qsafe = qrow < NQ ? qrow : NQ - 1;
     const uint16_t *qp = q + (int64_t)env * NQ * q_stride + (uint32_t)qsafe * (uint32_t)q_stride +
@@ -494,23 +469,60 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
     const u32x4 qw0 = *reinterpret_cast<const u32x4 *>(qp);
     const u32x4 qw1 = *reinterpret_cast<const u32x4 *>(qp + 16);
 
-    __syncthreads();
-    int base = 0, cnt = 0;
+    // Two ways to name the live keys of the environment: `ranges` (the K/V rows were already
+    // compacted: rows ranges[env] .. ranges[env+1]-1 of one list for all environments), or a
+    // mask over NK slots per environment, compacted here into an index list in LDS.
+    int cnt;
+    uint32_t first_row = 0;
+    if (ranges != nullptr) {
+        first_row = (uint32_t)ranges[env];
+        cnt = ranges[env + 1] - (int)first_row;
+        if (cnt == 0 && accum == out) return;
+    } else {
+        // wave w scans keys [w*J*64, (w+1)*J*64), 64 per ballot
+        const uint8_t *alive_env = alive == nullptr ? nullptr : alive + (int64_t)env * NK;
+        const int J = (NK + NT - 1) / NT;  // <= 32 because NK <= kStreamMaxKeys
+        const int key0 = wave * J * 64 + lane;
+        uint32_t bits = 0;
+        int mine = 0;
+        for (int j0 = 0; j0 < J; j0 += 8) {
+            // eight independent byte loads in flight, then their ballots
+            uint32_t a[8];
 #pragma unroll
-    for (int w = 0; w < NQB; ++w) {
-        const int c = s_wcnt[w];
-        if (w < wave) base += c;
-        cnt += c;
+            for (int u = 0; u < 8; ++u) {
+                const int key = key0 + (j0 + u) * 64;
+                const bool in = j0 + u < J && key < NK;
+                a[u] = 1u;
+                if (alive_env != nullptr) a[u] = alive_env[key < NK ? key : NK - 1];  // branch-free: no wait between the loads
+                a[u] = in ? a[u] : 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const bool on = a[u] != 0;
+                bits |= (on ? 1u : 0u) << ((j0 + u) & 31);
+                mine += (int)__popcll(__ballot(on));
+            }
+        }
+        if (lane == 0) s_wcnt[wave] = mine;
+        __syncthreads();
+        int base = 0;
+        cnt = 0;
+#pragma unroll
+        for (int w = 0; w < NQB; ++w) {
+            const int c = s_wcnt[w];
+            if (w < wave) base += c;
+            cnt += c;
+        }
+        // nothing in flight in this environment: the read contributes exactly zero
+        if (cnt == 0 && accum == out) return;
+        for (int j = 0; j < J; ++j) {
+            const bool a = (bits >> j) & 1u;
+            const uint64_t mask = __ballot(a);
+            if (a) s_idx[base + (int)__popcll(mask & ((1ull << lane) - 1ull))] = (uint16_t)(key0 + j * 64);
+            base += (int)__popcll(mask);
+        }
+        __syncthreads();
     }
-    // nothing in flight in this environment: the read contributes exactly zero
-    if (cnt == 0 && accum == out) return;
-    for (int j = 0; j < J; ++j) {
-        const bool a = (bits >> j) & 1u;
-        const uint64_t mask = __ballot(a);
-        if (a) s_idx[base + (int)__popcll(mask & ((1ull << lane) - 1ull))] = (uint16_t)(key0 + j * 64);
-        base += (int)__popcll(mask);
-    }
-    __syncthreads();
 
     const int nkb = (cnt + 31) >> 5;
     const int pad = nkb * 32 - cnt;  // positions [0, pad) of the first key block hold no key
@@ -518,7 +530,7 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
 
     // thread -> (position in tile, 8 channels), two items per thread
     const uint32_t stride32 = (uint32_t)kv_stride;
-    const int64_t kv_env = (int64_t)env * NK * kv_stride + head * kDh + (tid & 3) * 8;
+    const int64_t kv_env = (ranges != nullptr ? 0 : (int64_t)env * NK * kv_stride) + head * kDh + (tid & 3) * 8;
     const uint16_t *k_base = k + kv_env;
     const uint16_t *v_base = v + kv_env;
     u32x4 kw[2], vw[2];
@@ -526,7 +538,8 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
             const int li = t * TK + ((tid + it * NT) >> 2) - pad;  // index among the live keys
-            const uint32_t key = s_idx[(li >= 0 && li < cnt) ? li : 0];
+            const int lc = (li >= 0 && li < cnt) ? li : 0;
+            const uint32_t key = ranges != nullptr ? first_row + (uint32_t)lc : (uint32_t)s_idx[lc];
             kw[it] = *reinterpret_cast<const u32x4 *>(k_base + key * stride32);
             vw[it] = *reinterpret_cast<const u32x4 *>(v_base + key * stride32);
         }
@@ -775,8 +788,8 @@ static int dispatch_mfma(const void *q, int64_t q_stride, const void *k, const v
 
 template <int NQB>
 static int launch_cross_stream(const void *q, int64_t q_stride, const void *k, const void *v, int64_t kv_stride,
-                               const uint8_t *alive, const void *accum, void *out, int B, int NQ, int NK, int H,
-                               hipStream_t stream)
+                               const uint8_t *alive, const int32_t *ranges, const void *accum, void *out, int B,
+                               int NQ, int NK, int H, hipStream_t stream)
 {
     const int64_t pairs = (int64_t)B * H;
     const int64_t blocks = (pairs + 7) / 8 * 8;
@@ -784,20 +797,20 @@ static int launch_cross_stream(const void *q, int64_t q_stride, const void *k, c
     const float scale_log2e = kLog2eA / sqrtf((float)kDh);
     hipLaunchKernelGGL((sdpa_cross_stream_kernel<NQB>), dim3((unsigned)blocks), dim3(kWave * NQB), 0, stream,
                        (const uint16_t *)q, q_stride, (const uint16_t *)k, (const uint16_t *)v, kv_stride, alive,
-                       (const uint16_t *)accum, (uint16_t *)out, B, NQ, NK, H, scale_log2e);
+                       ranges, (const uint16_t *)accum, (uint16_t *)out, B, NQ, NK, H, scale_log2e);
     return (int)hipGetLastError();
 }
 
 static int dispatch_cross_stream(const void *q, int64_t q_stride, const void *k, const void *v, int64_t kv_stride,
-                                 const uint8_t *alive, const void *accum, void *out, int B, int NQ, int NK, int H,
-                                 hipStream_t stream)
+                                 const uint8_t *alive, const int32_t *ranges, const void *accum, void *out, int B,
+                                 int NQ, int NK, int H, hipStream_t stream)
 {
     switch ((NQ + 31) / 32) {
-        case 1: return launch_cross_stream<1>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
-        case 2: return launch_cross_stream<2>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
-        case 3: return launch_cross_stream<3>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
-        case 4: return launch_cross_stream<4>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
-        case 5: return launch_cross_stream<5>(q, q_stride, k, v, kv_stride, alive, accum, out, B, NQ, NK, H, stream);
+        case 1: return launch_cross_stream<1>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, B, NQ, NK, H, stream);
+        case 2: return launch_cross_stream<2>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, B, NQ, NK, H, stream);
+        case 3: return launch_cross_stream<3>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, B, NQ, NK, H, stream);
+        case 4: return launch_cross_stream<4>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, B, NQ, NK, H, stream);
+        case 5: return launch_cross_stream<5>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, B, NQ, NK, H, stream);
         default: return BNB_ERR_UNSUPPORTED;
     }
 }
@@ -860,8 +873,30 @@ extern "C" int bnb_sdpa_cross_fwd(const void *q, int64_t q_row_stride, int NQ, c
         !aligned16(k) || !aligned16(v) || (kv_row_stride * 2) % 16 != 0)
         return BNB_ERR_MISALIGNED;
     if (NK > 160)
-        return dispatch_cross_stream(q, q_row_stride, k, v, kv_row_stride, key_mask, accum, out, B, NQ, NK, H,
-                                     (hipStream_t)stream);
+        return dispatch_cross_stream(q, q_row_stride, k, v, kv_row_stride, key_mask, nullptr, accum, out, B, NQ, NK,
+                                     H, (hipStream_t)stream);
     return dispatch_mfma<true>(q, q_row_stride, k, v, kv_row_stride, key_mask, accum, out, B, NQ, NK, H,
                                (hipStream_t)stream);
+}
+
+extern "C" int bnb_sdpa_cross_ranges_fwd(const void *q, int64_t q_row_stride, int NQ, const void *kv_rows,
+                                         int64_t kv_row_stride, const int32_t *ranges, int64_t kv_capacity,
+                                         const void *accum, void *out, int B, int H, int dh, int dtype,
+                                         void *stream)
+{
+    using namespace bnb;
+    if (B < 0 || NQ < 0 || H < 1 || dh < 1 || kv_capacity < 0) return BNB_ERR_BAD_SHAPE;
+    if (dtype != BNB_BF16 || dh != kDh || NQ > 160) return BNB_ERR_UNSUPPORTED;
+    if (B == 0 || NQ == 0) return 0;
+    if (!q || !out || !kv_rows || !ranges) return BNB_ERR_NULL_POINTER;
+    if (q_row_stride < (int64_t)H * dh || kv_row_stride < (int64_t)2 * H * dh) return BNB_ERR_BAD_SHAPE;
+    // rows inside an environment (q) and inside the whole list (kv) are addressed with 32-bit offsets
+    if ((int64_t)NQ * q_row_stride >= (1LL << 30) || kv_capacity * kv_row_stride >= (1LL << 32))
+        return BNB_ERR_UNSUPPORTED;
+    if (!aligned16(q) || !aligned16(out) || (accum && !aligned16(accum)) || (q_row_stride * 2) % 16 != 0 ||
+        !aligned16(kv_rows) || (kv_row_stride * 2) % 16 != 0 || (reinterpret_cast<uintptr_t>(ranges) & 3u))
+        return BNB_ERR_MISALIGNED;
+    const uint16_t *kp = (const uint16_t *)kv_rows;
+    return dispatch_cross_stream(q, q_row_stride, kp, kp + (int64_t)H * dh, kv_row_stride, nullptr, ranges, accum, out, B,
+                                 NQ, 0, H, (hipStream_t)stream);
 }

@@ -784,6 +784,7 @@ class CompactRows:
         if B * n >= 2 ** 31:
             raise ValueError("mask too large for 32-bit row positions")
         self.shape = (B, n)
+        self.mask = mask
         counts = torch.empty(B, dtype=torch.int32, device=mask.device)
         self.offsets = torch.zeros(B + 1, dtype=torch.int32, device=mask.device)
         self.index = torch.empty(max(B * n, 1), dtype=torch.int32, device=mask.device)
@@ -851,3 +852,43 @@ def norm_linear(
             )
         _native.check(rc, "bnb_norm_linear_fwd")
     return out if rows is not None else out.reshape(*x.shape[:-1], N)
+
+
+def sdpa_cross_rows(
+    qkv: torch.Tensor,
+    kv_rows: torch.Tensor,
+    rows: CompactRows,
+    n_heads: int,
+    *,
+    accum: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """``sdpa_cross`` over key/value rows compacted beforehand: ``kv_rows`` (capacity, 2*D)
+    holds ``[K | V]`` of the entries listed in ``rows`` (e.g. ``norm_linear(bullets, ..., rows=rows)``),
+    environment b reading the rows ``rows.offsets[b] .. rows.offsets[b+1]-1``.  Same result as
+    ``sdpa_cross`` with the mask the list was built from, without scanning the mask again."""
+    B, NQ, D3 = qkv.shape
+    D = D3 // 3
+    if not (qkv.is_cuda and qkv.dtype == torch.bfloat16 and kv_rows.dtype == torch.bfloat16 and D % n_heads == 0
+            and D // n_heads == 32 and NQ <= 160):
+        raise RuntimeError("sdpa_cross_rows covers bfloat16, head size 32 and at most 160 queries")
+    if kv_rows.dim() != 2 or kv_rows.shape[1] != 2 * D or not kv_rows.is_contiguous():
+        raise ValueError(f"kv_rows must be a contiguous (capacity, {2 * D}) tensor")
+    if rows.shape[0] != B or kv_rows.shape[0] < rows.shape[0] * rows.shape[1]:
+        raise ValueError("rows was built for a different batch, or kv_rows is smaller than its capacity")
+    if torch.is_grad_enabled() and (qkv.requires_grad or kv_rows.requires_grad):
+        raise RuntimeError("sdpa_cross_rows is forward-only; call it under torch.no_grad()")
+    if B and NQ and (qkv.stride(-1) != 1 or (B > 1 and qkv.stride(0) != NQ * qkv.stride(1))):
+        qkv = qkv.contiguous()
+    if accum is not None and (accum.shape != (B, NQ, D) or accum.dtype != torch.bfloat16 or not accum.is_contiguous()):
+        raise ValueError("accum must be a contiguous bfloat16 (B, NQ, D) tensor")
+    out = accum if accum is not None else torch.empty((B, NQ, D), dtype=torch.bfloat16, device=qkv.device)
+    if B == 0 or NQ == 0:
+        return out
+    with torch.cuda.device(qkv.device):
+        rc = _native.load().bnb_sdpa_cross_ranges_fwd(
+            qkv.data_ptr(), qkv.stride(1), NQ, kv_rows.data_ptr(), kv_rows.stride(0), rows.offsets.data_ptr(),
+            kv_rows.shape[0], None if accum is None else accum.data_ptr(), out.data_ptr(), B, n_heads, D // n_heads,
+            _native.BF16, _stream(),
+        )
+    _native.check(rc, "bnb_sdpa_cross_ranges_fwd")
+    return out

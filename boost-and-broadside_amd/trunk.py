@@ -191,17 +191,39 @@ class TransformerBlock(nn.Module):
             # training: the attention itself stays with torch's differentiable SDPA
             merged = self._self_attention_autograd(qkv, alive_mask)
             if self.reads_bullets and bullets is not None:
+                if isinstance(bullet_mask, ops.CompactRows):
+                    bullet_mask = bullet_mask.mask
                 kv = self.kv_bullet(self.norm_bullet(bullets))
                 merged = merged + self._bullet_read(qkv, kv, bullet_mask)
             return self.out_proj(merged)
         merged = ops.sdpa_masked(qkv, alive_mask, self.n_heads)  # (B, N, D) head-major
         if self.reads_bullets and bullets is not None:
+            rows = bullet_mask if isinstance(bullet_mask, ops.CompactRows) else None
+            if rows is None and bullet_mask is not None and self._compact_read_ok(qkv, bullets):
+                rows = ops.CompactRows(bullet_mask)
+            if rows is not None and self._compact_read_ok(qkv, bullets):
+                # only the bullets in flight are normalised and projected (one kernel over a
+                # device-side list of them), and the read walks each environment's run of rows
+                w = self.kv_bullet.weight
+                pk = _cached_cast(self.kv_bullet, "_bnb_pack", (w,), torch.bfloat16, lambda: ops.pack_linear_weights(w))
+                kv_rows = ops.norm_linear(bullets, self.norm_bullet.weight, pk, eps=self.norm_bullet.eps, rows=rows)
+                return _project(self.out_proj, ops.sdpa_cross_rows(qkv, kv_rows, rows, self.n_heads, accum=merged))
+            if rows is not None:
+                bullet_mask = rows.mask
             kv = _project(self.kv_bullet, self._norm_bullets(bullets, qkv.dtype))
             if ops.cross_supported(qkv, kv, self.n_heads):
                 merged = ops.sdpa_cross(qkv, kv, bullet_mask, self.n_heads, accum=merged)
             else:
                 merged = merged + self._bullet_read(qkv, kv, bullet_mask)
         return _project(self.out_proj, merged)
+
+    def _compact_read_ok(self, qkv, bullets) -> bool:
+        """Whether the bullet read can run on the compacted list (bf16 projections, width 128,
+        heads of 32, at most 160 entity tokens, float32 bullet tokens on the GPU)."""
+        return (
+            qkv.dtype == torch.bfloat16 and self.d_model == ops.FFN_WIDTH and self.head_dim == 32 and qkv.shape[1] <= 160
+            and bullets.is_cuda and bullets.dtype == torch.float32 and self.kv_bullet.bias is None
+        )
 
     def _self_attention_autograd(self, qkv, alive_mask):
         """Masked self-attention as the reference composes it (attention.py:136-147,168)."""
@@ -626,11 +648,19 @@ class YemongTrunk(nn.Module):
             raise ValueError("out_state must be a separate float32 tensor shaped like recurrent_state")
         if reset_mask is not None:
             reset_mask = reset_mask.contiguous()
+        # the list of bullets in flight is built once and shared by every layer that reads them
+        bullet_rows = bullet_mask
+        if (
+            bullets is not None and bullet_mask is not None and self.config.reads_bullets and bullets.is_cuda
+            and bullets.dtype == torch.float32 and _projection_dtype() == torch.bfloat16 and D == ops.FFN_WIDTH
+            and D // self.config.n_heads == 32 and NM <= 160
+        ):
+            bullet_rows = ops.CompactRows(bullet_mask)
         x = tokens
         for i, block in enumerate(self.yemong_layers):
             sl = slice(i * n_t, (i + 1) * n_t)
             x = block.step_packed(x, alive_mask, recurrent_state[sl], out_state[sl], n_rec, reset_mask, bullets,
-                                  bullet_mask)
+                                  bullet_rows)
         return x, out_state
 
 

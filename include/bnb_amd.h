@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 9
+#define BNB_ABI_VERSION 10
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -113,6 +113,20 @@ int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride, const uint
 int bnb_sdpa_cross_fwd(const void *q, int64_t q_row_stride, int NQ, const void *k, const void *v,
                        int64_t kv_row_stride, int NK, const uint8_t *key_mask, const void *accum,
                        void *out, int B, int H, int dh, int dtype, void *stream);
+
+/*
+ * bnb_sdpa_cross_fwd over key/value rows that were compacted beforehand: kv_rows holds the
+ * [K | V] rows (2*H*dh wide, kv_row_stride elements apart) of the active keys of all
+ * environments back to back, and environment b owns rows ranges[b] .. ranges[b+1]-1 (int32,
+ * B+1 entries, e.g. the offsets of bnb_mask_fill with kv_rows = bnb_norm_linear_fwd over the
+ * same list).  No mask is scanned; an environment with an empty range contributes exactly 0.
+ * Any number of keys per environment; kv_capacity = rows allocated in kv_rows (addressed with
+ * 32-bit element offsets: kv_capacity * kv_row_stride < 2^32).  Other arguments and
+ * requirements as bnb_sdpa_cross_fwd.
+ */
+int bnb_sdpa_cross_ranges_fwd(const void *q, int64_t q_row_stride, int NQ, const void *kv_rows,
+                              int64_t kv_row_stride, const int32_t *ranges, int64_t kv_capacity,
+                              const void *accum, void *out, int B, int H, int dh, int dtype, void *stream);
 
 /*
  * One RG-LRU recurrence step over R = B*n_rec entity rows of D channels.

@@ -901,3 +901,30 @@ def test_compact_rows_and_gathered_projection(B, n, p):
     if total:
         want = torch.nn.functional.linear(torch_ref.rms_norm(x.reshape(-1, D)[mask.flatten()], nw), W.bfloat16().float())
         assert max_rel(out[:total].float().cpu(), want) <= BF16_TOL
+
+
+@pytest.mark.parametrize("B,NQ,NK,p", [(4, 12, 80, 0.5), (3, 84, 800, 0.3), (3, 156, 1520, 0.1), (2, 33, 3000, 0.6), (5, 20, 190, 0.0)])
+def test_sdpa_cross_over_compacted_rows_equals_the_masked_form(B, NQ, NK, p):
+    H, D = 4, 128
+    g = torch.Generator().manual_seed(NQ * 13 + NK)
+    qkv = torch.randn(B, NQ, 3 * D, generator=g).bfloat16().to(DEV)
+    kv = torch.randn(B, NK, 2 * D, generator=g).bfloat16().to(DEV)
+    mask = torch.rand(B, NK, generator=g) < p
+    mask[0] = False
+    if p > 0:
+        mask[1, NK - 1] = True
+    mask = mask.to(DEV)
+    rows = ops.CompactRows(mask)
+    kv_rows = torch.zeros(B * NK, 2 * D, dtype=torch.bfloat16, device=DEV)
+    total = int(rows.total.item())
+    kv_rows[:total] = kv.reshape(B * NK, 2 * D)[rows.index[:total].long()]
+    bare = ops.sdpa_cross_rows(qkv, kv_rows, rows, H)
+    truth = torch_ref.bullet_read(qkv.float().cpu(), kv.float().cpu(), mask.cpu(), H)
+    assert bare[0].abs().max() == 0
+    if truth.abs().max() > 0:
+        assert max_rel(bare.float().cpu(), truth) <= BF16_TOL
+    merged = torch.randn(B, NQ, D, generator=g).bfloat16().to(DEV)
+    got = ops.sdpa_cross_rows(qkv, kv_rows, rows, H, accum=merged.clone())
+    assert torch.equal(got, merged + bare)
+    if 160 < NK <= 2048:  # the masked form on the same kernel: same keys in the same order, bit for bit
+        assert torch.equal(got, ops.sdpa_cross(qkv, kv, mask, H, accum=merged.clone()))
