@@ -176,17 +176,24 @@ class TransformerBlock(nn.Module):
         if not _fused_ok(x, act):
             x = x + self._attn(self.norm1(x), alive_mask, bullets, bullet_mask)
             return x + self.ffn(self.norm2(x))
-        # norm (+ cast) -> qkv -> attention kernel -> out_proj -> add + norm (+ cast) -> FFN
-        _, n1 = ops.add_rmsnorm(x, self.norm1.weight, eps=self.norm1.eps, out_dtype=act)
-        attn = self._attn(n1, alive_mask, bullets, bullet_mask)
+        # norm + qkv (one kernel under bf16) -> attention kernel -> out_proj -> fused sublayer tail
+        if act == torch.bfloat16 and self.d_model == ops.FFN_WIDTH and self.qkv.bias is None:
+            w = self.qkv.weight
+            pk = _cached_cast(self.qkv, "_bnb_pack", (w,), torch.bfloat16, lambda: ops.pack_linear_weights(w))
+            attn = self._attn(None, alive_mask, bullets, bullet_mask,
+                              qkv=ops.norm_linear(x, self.norm1.weight, pk, eps=self.norm1.eps))
+        else:
+            _, n1 = ops.add_rmsnorm(x, self.norm1.weight, eps=self.norm1.eps, out_dtype=act)
+            attn = self._attn(n1, alive_mask, bullets, bullet_mask)
         fused = self.ffn.fused_tail(x, attn, self.norm2)
         if fused is not None:
             return fused
         x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=attn, eps=self.norm2.eps, out_dtype=act)
         return x1 + self.ffn(n2)
 
-    def _attn(self, x, alive_mask, bullets=None, bullet_mask=None):
-        qkv = _project(self.qkv, x)  # (B, N, 3D), fp32 or bf16 under autocast
+    def _attn(self, x, alive_mask, bullets=None, bullet_mask=None, qkv=None):
+        if qkv is None:
+            qkv = _project(self.qkv, x)  # (B, N, 3D), fp32 or bf16 under autocast
         if torch.is_grad_enabled():
             # training: the attention itself stays with torch's differentiable SDPA
             merged = self._self_attention_autograd(qkv, alive_mask)
