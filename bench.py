@@ -492,6 +492,28 @@ def main():
 
         t_read_torch = None if args.no_torch_baseline else timed_loop(torch_read, 3, 1) / 3
         live = int(b_mask.sum().item())
+
+        # the whole bullet branch of a layer, from raw bullet tokens: list of the bullets in flight,
+        # norm + kv projection over that list, read over per-environment row ranges ...
+        bullets_f = torch.randn(w.B, NB, D, device=dev, generator=gen)
+        layer_b = bnb.TransformerBlock(bnb.ModelConfig(d_model=D, n_heads=H, n_yemong_blocks=1, n_spatial_per_block=1, n_bullet_cross_per_block=1),
+                                       reads_bullets=True).to(dev).eval()
+        pk_kv = ops.pack_linear_weights(layer_b.kv_bullet.weight)
+
+        def branch_compact(t):
+            rows = ops.CompactRows(b_mask)
+            kv_rows = ops.norm_linear(bullets_f, layer_b.norm_bullet.weight, pk_kv, rows=rows)
+            ops.sdpa_cross_rows(qkv_b, kv_rows, rows, H, accum=merged[t & 1])
+
+        # ... against the same branch over every slot (norm kernel, library GEMM, masked read)
+        def branch_all_slots(t):
+            with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+                n = ops.add_rmsnorm(bullets_f, layer_b.norm_bullet.weight, out_dtype=torch.bfloat16)[1]
+                ops.sdpa_cross(qkv_b, layer_b.kv_bullet(n), b_mask, H, accum=merged[t & 1])
+
+        t_branch = timed_loop(branch_compact, n_b, 3) / n_b
+        t_branch_all = timed_loop(branch_all_slots, 4, 2) / 4
+        del bullets_f, layer_b
         read_bytes = live * 2 * D * 2 + w.B * NB + 3 * w.B * w.NM * D * 2
         result["bullet_read"] = {
             "avg_launch_us": t_read * 1e6, "slots_per_env": NB, "live_fraction": live_p,
@@ -499,6 +521,10 @@ def main():
             "frac_of_hbm_peak": read_bytes / t_read / peak,
             "tflops": 4 * live * w.NM * D / t_read / 1e12,
             "eager_torch_us": None if t_read_torch is None else t_read_torch * 1e6,
+            "branch_compact_us": t_branch * 1e6, "branch_all_slots_us": t_branch_all * 1e6,
+            "branch_what": "norm_bullet + kv_bullet + read from fp32 bullet tokens: compact = device-side list of the "
+                           "live bullets, bnb_norm_linear_fwd over it, bnb_sdpa_cross_ranges_fwd; all_slots = "
+                           "bnb_add_rmsnorm_fwd + library GEMM over every slot + bnb_sdpa_cross_fwd with the mask",
             "what": "bnb_sdpa_cross_fwd added into the self-attention output: K/V rows of the live bullets, the slot "
                     "mask, Q, accumulator in and out; exp-throughput-bound rather than HBM-bound when many bullets are live",
         }
