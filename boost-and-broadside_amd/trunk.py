@@ -456,7 +456,9 @@ class GriffinTemporalBlock(nn.Module):
         self.rg_lru.step(res[0], state_in[:, :D], h_out=state_out[:, :D], reset=reset, rows_per_env=n_rec,
                          x_act=res[2] if want_lp else None, y_out=y[:, :n_rec] if NM > n_rec else y.view(R, D))
         if NM > n_rec:
-            y[:, n_rec:] = _project(field_sub, b1[:, n_rec:])
+            # gathered into one (B*M, D) matrix first: on the strided view the library would run a
+            # batch of B tiny GEMMs
+            y[:, n_rec:] = _project(field_sub, b1[:, n_rec:].reshape(-1, D)).view(B, NM - n_rec, D)
         return self._finish(x, normed, y)
 
     def forward_nonrecurrent(self, x, sub):
