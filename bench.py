@@ -119,7 +119,8 @@ class eager_kernels:
         from boost_and_broadside_amd import ops
 
         self.ops = ops
-        self.saved = (ops.sdpa_masked, ops.rglru_step, ops.conv_step, ops.add_rmsnorm, ops.gelu_mul, ops.ffn_supported)
+        self.saved = (ops.sdpa_masked, ops.rglru_step, ops.conv_step, ops.add_rmsnorm, ops.gelu_mul, ops.ffn_supported,
+                      ops.FFN_WIDTH)
 
         def sdpa(qkv, alive, n_heads, **kw):
             if alive is None:
@@ -143,12 +144,14 @@ class eager_kernels:
             return out if out_dtype is None else out.to(out_dtype)
 
         ops.sdpa_masked, ops.rglru_step, ops.conv_step, ops.add_rmsnorm, ops.gelu_mul = sdpa, rglru, conv, add_rmsnorm, gelu_mul
-        ops.ffn_supported = lambda x, hidden: False  # the fused sublayer tail falls back to its library composition
+        # the matrix-core kernels (sublayer tail, norm + projection) fall back to their library compositions
+        ops.ffn_supported = lambda x, hidden: False
+        ops.FFN_WIDTH = -1
         return self
 
     def __exit__(self, *exc):
         o = self.ops
-        o.sdpa_masked, o.rglru_step, o.conv_step, o.add_rmsnorm, o.gelu_mul, o.ffn_supported = self.saved
+        o.sdpa_masked, o.rglru_step, o.conv_step, o.add_rmsnorm, o.gelu_mul, o.ffn_supported, o.FFN_WIDTH = self.saved
         return False
 
 

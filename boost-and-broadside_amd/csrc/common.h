@@ -127,6 +127,9 @@ struct is_bf16<uint16_t> {
     static constexpr bool value = true;
 };
 
+// Exact (erf) GELU, as torch's default F.gelu.
+__device__ __forceinline__ float gelu_erf(float v) { return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f)); }
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 }  // namespace bnb

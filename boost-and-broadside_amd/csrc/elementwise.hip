@@ -57,8 +57,6 @@ __global__ __launch_bounds__(kEwThreads) void add_rmsnorm_kernel(
 }
 
 // ---- out = gelu(a) * b -----------------------------------------------------------------------
-__device__ __forceinline__ float gelu_erf(float v) { return 0.5f * v * (1.0f + erff(v * 0.70710678118654752f)); }
-
 template <typename AT, typename BT, typename OT>
 __global__ __launch_bounds__(kEwThreads) void gelu_mul_kernel(const AT *__restrict__ a, int64_t a_stride,
                                                               const BT *__restrict__ b, int64_t b_stride,

@@ -65,12 +65,24 @@ __device__ __forceinline__ float gelu_as(float v)
     return fmaf(fabsf(v), fmaf(-(poly * t), e, 0.5f), 0.5f * v);
 }
 
-template <bool HAS_DELTA>
+// What is added to x before the norm (the output of the sublayer the tail belongs to):
+//   kDeltaNone  nothing;  kDeltaRows  the bf16 rows `delta`;
+//   kDeltaProj  rows_a Wp^T  (the block's output projection: attention.py:168-169 `out_proj`)
+//   kDeltaGate  (bf16(gelu(rows_a)) * rows_b) Wp^T  (griffin.py:281-283: `b1_out * gelu(linear2(..))`
+//               through `linear_out`), with the roundings torch's bf16 gelu and product have.
+// The projection is a 128 x 128 matrix product on the same MFMA layouts: its operand rows come
+// in through the staging area like x, the 32 KB of Wp sit in the weight buffers before the
+// chunk loop needs them, and the products accumulate straight onto x in the accumulators.
+enum { kDeltaNone = 0, kDeltaRows = 1, kDeltaProj = 2, kDeltaGate = 3 };
+constexpr int kProjPitch = kFfnD + 8;  // halfs per staged operand row (bank spread, 16-byte aligned)
+
+template <int MODE>
 __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void ffn_fused_kernel(
     const float *__restrict__ x, int64_t x_stride, const uint16_t *__restrict__ delta,
-    const float *__restrict__ norm_w, float eps, const uint16_t *__restrict__ wpack, float *__restrict__ out,
-    int64_t R)
+    const uint16_t *__restrict__ rows_b, const uint16_t *__restrict__ wproj, const float *__restrict__ norm_w,
+    float eps, const uint16_t *__restrict__ wpack, float *__restrict__ out, int64_t R)
 {
+    constexpr bool HAS_DELTA = MODE == kDeltaRows;
     // three weight buffers: chunk c is used while chunk c+1 is already complete (its operands
     // are read one chunk ahead) and chunk c+2 is on its way in
     __shared__ __align__(16) uint16_t s_w[3][kFfnChunkHalfs];
@@ -108,13 +120,46 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
     fetch(0, pre);
     fetch(1, pre1);
 
+    const int64_t row0 = ((int64_t)blockIdx.x * kFfnWaves + wave) * 32;
+    // ---- operand rows of the projection (modes Proj / Gate): whole 256-byte rows in, k-slot order out ----
+    bf16x8 mb[8];
+    if (MODE == kDeltaProj || MODE == kDeltaGate) {
+        uint16_t *stage_a = &s_w[0][0] + wave * (32 * kProjPitch);
+        const int a_row = lane >> 4;        // four rows per instruction
+        const int a_col = (lane & 15) * 8;  // this lane's eight channels
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int64_t r = row0 + 4 * j + a_row;
+            const int64_t rs = r < R ? r : R - 1;
+            u32x4 av = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(delta + rs * kFfnD + a_col));
+            if (MODE == kDeltaGate) {
+                const Row8 g = load8(reinterpret_cast<const uint16_t *>(&av));
+                const Row8 y = load8_stream(rows_b + rs * kFfnD + a_col);
+                float p[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) p[e] = round_to_bf16(gelu_erf(g.v[e])) * y.v[e];
+                av = u32x4{pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
+                           pack_bf16x2(p[6], p[7])};
+            }
+            *reinterpret_cast<u32x4 *>(stage_a + (4 * j + a_row) * kProjPitch + a_col) = av;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            const uint16_t *sp = stage_a + m * kProjPitch + 16 * ks + 4 * half;
+            const u32x2 lo = *reinterpret_cast<const u32x2 *>(sp);
+            const u32x2 hi = *reinterpret_cast<const u32x2 *>(sp + 8);
+            mb[ks] = __builtin_bit_cast(bf16x8, u32x4{lo.x, lo.y, hi.x, hi.y});
+        }
+        __syncthreads();
+    }
+
     // ---- s = x + delta for this wave's 32 tokens ----
     // Read as whole rows (a half-wave per 512-byte row, 16 bytes per lane) and handed to the
     // lanes that own the tokens through this wave's slice of the still unused weight buffers:
     // row r at r * kRowPitch floats, the pitch keeping the 32 row starts on different banks.
     constexpr int kRowPitch = kFfnD + 4;
     float *stage = reinterpret_cast<float *>(&s_w[0][0]) + wave * (32 * kRowPitch);
-    const int64_t row0 = ((int64_t)blockIdx.x * kFfnWaves + wave) * 32;
     const int io_row = lane >> 5;        // which of the two rows of one instruction
     const int io_col = (lane & 31) * 4;  // first of this lane's four channels
 #pragma unroll
@@ -146,10 +191,36 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
         const f32x4 hi = *reinterpret_cast<const f32x4 *>(sp + 8);
         const float sv[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            acc[ks >> 1][8 * (ks & 1) + e] = sv[e];
-            ss = fmaf(sv[e], sv[e], ss);
+        for (int e = 0; e < 8; ++e) acc[ks >> 1][8 * (ks & 1) + e] = sv[e];
+    }
+    if (MODE == kDeltaProj || MODE == kDeltaGate) {
+        // Wp (128 x 128 bf16, packed [cb][ks][lane][8] = Wp[32cb + lane%32][ch(ks, lane/32, .)]) into the
+        // weight buffers once everyone is done with the staging area, then 32 MFMAs onto x
+        __syncthreads();
+        {
+            const u32x4 *src = reinterpret_cast<const u32x4 *>(wproj);
+            u32x4 *dst = reinterpret_cast<u32x4 *>(&s_w[0][0]);
+            u32x4 t[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) t[q] = src[tid + q * kFfnThreads];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) dst[tid + q * kFfnThreads] = t[q];
         }
+        __syncthreads();
+        const uint16_t *wp = &s_w[0][0] + lane * 8;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+#pragma unroll
+            for (int cb = 0; cb < 4; ++cb) {
+                const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(wp + (cb * 8 + ks) * 512));
+                acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, mb[ks], acc[cb], 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) ss = fmaf(acc[cb][v], acc[cb][v], ss);
     }
     ss += __shfl_xor(ss, 32);
     const float rstd = rsqrtf(ss * (1.0f / kFfnD) + eps);
@@ -282,28 +353,66 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
 
 }  // namespace bnb
 
+namespace bnb {
+
+template <int MODE>
+static int launch_ffn(const float *x, int64_t x_stride, const void *rows_a, const void *rows_b, const void *wproj,
+                      const float *norm_weight, float eps, const void *weights_packed, float *out, int64_t R,
+                      hipStream_t s)
+{
+    const int64_t blocks = (R + kFfnWaves * 32 - 1) / (kFfnWaves * 32);
+    if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((ffn_fused_kernel<MODE>), dim3((unsigned)blocks), dim3(kFfnThreads), 0, s, x, x_stride,
+                       (const uint16_t *)rows_a, (const uint16_t *)rows_b, (const uint16_t *)wproj, norm_weight, eps,
+                       (const uint16_t *)weights_packed, out, R);
+    return (int)hipGetLastError();
+}
+
+static int ffn_common_checks(const float *x, int64_t x_row_stride, const float *norm_weight,
+                             const void *weights_packed, const float *out, int64_t R, int D, int hidden)
+{
+    if (R < 0 || x_row_stride < D) return BNB_ERR_BAD_SHAPE;
+    if (D != kFfnD || hidden != kFfnHidden) return BNB_ERR_UNSUPPORTED;
+    if (R == 0) return 0;
+    if (!x || !norm_weight || !weights_packed || !out) return BNB_ERR_NULL_POINTER;
+    if (!aligned16(x) || !aligned16(out) || !aligned16(norm_weight) || !aligned16(weights_packed) ||
+        (x_row_stride % 4) != 0)
+        return BNB_ERR_MISALIGNED;
+    return 0;
+}
+
+}  // namespace bnb
+
 extern "C" int bnb_ffn_fused_fwd(const float *x, int64_t x_row_stride, const void *delta, int delta_dtype,
                                  const float *norm_weight, float eps, const void *weights_packed, float *out,
                                  int64_t R, int D, int hidden, void *stream)
 {
     using namespace bnb;
-    if (R < 0 || x_row_stride < D) return BNB_ERR_BAD_SHAPE;
-    if (D != kFfnD || hidden != kFfnHidden) return BNB_ERR_UNSUPPORTED;
-    if (R == 0) return 0;
-    if (!x || !norm_weight || !weights_packed || !out) return BNB_ERR_NULL_POINTER;
+    const int rc = ffn_common_checks(x, x_row_stride, norm_weight, weights_packed, out, R, D, hidden);
+    if (rc != 0 || R == 0) return rc;
     if (delta && delta_dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
-    if (!aligned16(x) || !aligned16(out) || !aligned16(norm_weight) || !aligned16(weights_packed) ||
-        (delta && !aligned16(delta)) || (x_row_stride % 4) != 0)
-        return BNB_ERR_MISALIGNED;
-    const int64_t blocks = (R + kFfnWaves * 32 - 1) / (kFfnWaves * 32);
-    if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+    if (delta && !aligned16(delta)) return BNB_ERR_MISALIGNED;
     hipStream_t s = (hipStream_t)stream;
     if (delta)
-        hipLaunchKernelGGL((ffn_fused_kernel<true>), dim3((unsigned)blocks), dim3(kFfnThreads), 0, s, x, x_row_stride,
-                           (const uint16_t *)delta, norm_weight, eps, (const uint16_t *)weights_packed, out, R);
-    else
-        hipLaunchKernelGGL((ffn_fused_kernel<false>), dim3((unsigned)blocks), dim3(kFfnThreads), 0, s, x,
-                           x_row_stride, (const uint16_t *)nullptr, norm_weight, eps,
-                           (const uint16_t *)weights_packed, out, R);
-    return (int)hipGetLastError();
+        return launch_ffn<kDeltaRows>(x, x_row_stride, delta, nullptr, nullptr, norm_weight, eps, weights_packed, out,
+                                      R, s);
+    return launch_ffn<kDeltaNone>(x, x_row_stride, nullptr, nullptr, nullptr, norm_weight, eps, weights_packed, out, R, s);
+}
+
+extern "C" int bnb_ffn_fused_proj_fwd(const float *x, int64_t x_row_stride, const void *rows_a, const void *rows_b,
+                                      const void *proj_packed, const float *norm_weight, float eps,
+                                      const void *weights_packed, float *out, int64_t R, int D, int hidden,
+                                      void *stream)
+{
+    using namespace bnb;
+    const int rc = ffn_common_checks(x, x_row_stride, norm_weight, weights_packed, out, R, D, hidden);
+    if (rc != 0 || R == 0) return rc;
+    if (!rows_a || !proj_packed) return BNB_ERR_NULL_POINTER;
+    if (!aligned16(rows_a) || !aligned16(proj_packed) || (rows_b && !aligned16(rows_b))) return BNB_ERR_MISALIGNED;
+    hipStream_t s = (hipStream_t)stream;
+    if (rows_b)
+        return launch_ffn<kDeltaGate>(x, x_row_stride, rows_a, rows_b, proj_packed, norm_weight, eps, weights_packed,
+                                      out, R, s);
+    return launch_ffn<kDeltaProj>(x, x_row_stride, rows_a, nullptr, proj_packed, norm_weight, eps, weights_packed, out,
+                                  R, s);
 }

@@ -692,6 +692,23 @@ def pack_ffn_weights(gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Ten
     return torch.cat([g.reshape(16, -1), u.reshape(16, -1), d.reshape(16, -1)], dim=1).contiguous()
 
 
+def pack_proj_weights(weight: torch.Tensor) -> torch.Tensor:
+    """A (128, 128) output-projection weight as the bfloat16 operand stream of the projection
+    folded into ``ffn_fused``: ``[cb][ks][l][e] = W[32cb + l%32][16ks + 8(e/4) + 4(l/32) + e%4]``."""
+    if weight.shape != (FFN_WIDTH, FFN_WIDTH):
+        raise ValueError("the folded projection covers (128, 128) weights")
+    dev = weight.device
+    lane = torch.arange(64, device=dev)
+    m, half = lane % 32, lane // 32
+    e = torch.arange(8, device=dev)
+    cb = torch.arange(4, device=dev)
+    ks = torch.arange(8, device=dev)
+    rows = (32 * cb[:, None, None, None] + m[None, None, :, None]).expand(-1, 8, -1, 8)
+    cols = (16 * ks[None, :, None, None] + 8 * (e // 4)[None, None, None, :] + 4 * half[None, None, :, None]
+            + (e % 4)[None, None, None, :]).expand(4, -1, -1, -1)
+    return weight.detach().to(torch.bfloat16)[rows, cols].contiguous()
+
+
 def ffn_supported(x: torch.Tensor, hidden: int) -> bool:
     """Whether ``ffn_fused`` covers this residual stream (fp32 on the GPU, width 128, hidden 512)."""
     return x.is_cuda and x.dtype == torch.float32 and x.shape[-1] == FFN_WIDTH and hidden == FFN_HIDDEN
@@ -705,6 +722,7 @@ def ffn_fused(
     *,
     eps: float | None = None,
     out: torch.Tensor | None = None,
+    proj: tuple | None = None,
 ) -> torch.Tensor:
     """``s = x + delta; s + down(gelu(gate(n)) * up(n))`` with ``n = rmsnorm(s) * norm_weight``,
     one matrix-core kernel with bfloat16 projections (what the sublayer tail computes under
@@ -712,6 +730,11 @@ def ffn_fused(
 
     x (..., 128) float32 with contiguous rows; delta same shape, bfloat16, or None;
     ``weights_packed`` from ``pack_ffn_weights``.  Returns (..., 128) float32.
+
+    ``proj`` folds the sublayer's output projection in (then ``delta`` must be None):
+    ``(rows, wp)`` adds ``rows @ W^T``, ``(rows_g, rows_y, wp)`` adds
+    ``(gelu(rows_g) * rows_y) @ W^T``; rows are bfloat16 with x's shape, ``wp`` from
+    ``pack_proj_weights``.
     """
     D = x.shape[-1]
     if not ffn_supported(x, FFN_HIDDEN):
@@ -738,6 +761,28 @@ def ffn_fused(
     elif out.numel() != R * D or out.dtype != torch.float32 or not out.is_contiguous() or out.device != x.device:
         raise ValueError("out must be a contiguous float32 tensor of x's size on x's device")
     norm_weight = norm_weight.detach().contiguous()
+    if proj is not None:
+        if delta is not None:
+            raise ValueError("give either delta or proj")
+        *rows, wp = proj
+        if len(rows) not in (1, 2) or wp.dtype != torch.bfloat16 or wp.numel() != D * D or not wp.is_contiguous():
+            raise ValueError("proj must be (rows, packed) or (rows_g, rows_y, packed) with pack_proj_weights output")
+        flat = []
+        for t in rows:
+            if t.shape != x.shape or t.dtype != torch.bfloat16:
+                raise ValueError(f"projection operand rows must be bfloat16 {tuple(x.shape)} tensors")
+            if torch.is_grad_enabled() and t.requires_grad:
+                raise RuntimeError("ffn_fused is forward-only; call it under torch.no_grad()")
+            flat.append(t.reshape(-1, D).contiguous())
+        if R:
+            with torch.cuda.device(x.device):
+                rc = _native.load().bnb_ffn_fused_proj_fwd(
+                    x2.data_ptr(), x2.stride(0), flat[0].data_ptr(), flat[1].data_ptr() if len(flat) == 2 else None,
+                    wp.data_ptr(), norm_weight.data_ptr(), float(_F32_EPS if eps is None else eps),
+                    weights_packed.data_ptr(), out.data_ptr(), R, D, FFN_HIDDEN, _stream(),
+                )
+            _native.check(rc, "bnb_ffn_fused_proj_fwd")
+        return out.reshape(x.shape)
     if R:
         with torch.cuda.device(x.device):
             rc = _native.load().bnb_ffn_fused_fwd(

@@ -127,16 +127,31 @@ class GatedMLP(nn.Module):
         ws = (self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight)
         return _cached_cast(self, "_bnb_ffn_pack", ws, torch.bfloat16, lambda: ops.pack_ffn_weights(*ws))
 
-    def fused_tail(self, x: torch.Tensor, delta: torch.Tensor | None, norm: nn.RMSNorm) -> torch.Tensor | None:
-        """``s = x + delta; s + self(norm(s))`` as one kernel, or None when it does not apply
-        (it covers the bf16-autocast inference path at width 128 / hidden 512)."""
-        if (
-            torch.is_grad_enabled() or _projection_dtype() != torch.bfloat16
-            or not ops.ffn_supported(x, self.gate_proj.out_features)
-            or (delta is not None and delta.dtype != torch.bfloat16)
-        ):
+    def fused_tail_ok(self, x: torch.Tensor) -> bool:
+        """Whether the one-kernel sublayer tail applies (bf16-autocast inference, width 128, hidden 512)."""
+        return (
+            not torch.is_grad_enabled() and _projection_dtype() == torch.bfloat16
+            and ops.ffn_supported(x, self.gate_proj.out_features)
+        )
+
+    def fused_tail(self, x, delta, norm: nn.RMSNorm, *, proj_layer: nn.Linear | None = None, gate=None):
+        """``s = x + d; s + self(norm(s))`` as one kernel, or None when it does not apply.
+
+        ``d`` is ``delta`` itself, or with ``proj_layer`` (a bias-free 128 x 128 Linear)
+        ``proj_layer(delta)``, or with ``gate`` as well ``proj_layer(gelu(gate) * delta)``,
+        the projection then running inside the kernel."""
+        if not self.fused_tail_ok(x) or (delta is not None and delta.dtype != torch.bfloat16):
             return None
-        return ops.ffn_fused(x, delta, norm.weight, self.packed_weights(), eps=norm.eps)
+        if proj_layer is None:
+            return ops.ffn_fused(x, delta, norm.weight, self.packed_weights(), eps=norm.eps)
+        w = proj_layer.weight
+        if proj_layer.bias is not None or tuple(w.shape) != (ops.FFN_WIDTH, ops.FFN_WIDTH):
+            return None
+        if gate is not None and gate.dtype != torch.bfloat16:
+            return None
+        wp = _cached_cast(proj_layer, "_bnb_proj_pack", (w,), torch.bfloat16, lambda: ops.pack_proj_weights(w))
+        proj = (delta, wp) if gate is None else (gate, delta, wp)
+        return ops.ffn_fused(x, None, norm.weight, self.packed_weights(), eps=norm.eps, proj=proj)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         hidden = self.gate_proj.out_features
@@ -180,8 +195,16 @@ class TransformerBlock(nn.Module):
         if act == torch.bfloat16 and self.d_model == ops.FFN_WIDTH and self.qkv.bias is None:
             w = self.qkv.weight
             pk = _cached_cast(self.qkv, "_bnb_pack", (w,), torch.bfloat16, lambda: ops.pack_linear_weights(w))
-            attn = self._attn(None, alive_mask, bullets, bullet_mask,
-                              qkv=ops.norm_linear(x, self.norm1.weight, pk, eps=self.norm1.eps))
+            qkv = ops.norm_linear(x, self.norm1.weight, pk, eps=self.norm1.eps)
+            if self.ffn.fused_tail_ok(x) and self.out_proj.bias is None:
+                # the output projection runs inside the tail kernel, on the merged heads
+                merged = self._attn(None, alive_mask, bullets, bullet_mask, qkv=qkv, project=False)
+                fused = self.ffn.fused_tail(x, merged, self.norm2, proj_layer=self.out_proj)
+                if fused is not None:
+                    return fused
+                attn = _project(self.out_proj, merged)
+            else:
+                attn = self._attn(None, alive_mask, bullets, bullet_mask, qkv=qkv)
         else:
             _, n1 = ops.add_rmsnorm(x, self.norm1.weight, eps=self.norm1.eps, out_dtype=act)
             attn = self._attn(n1, alive_mask, bullets, bullet_mask)
@@ -191,7 +214,9 @@ class TransformerBlock(nn.Module):
         x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=attn, eps=self.norm2.eps, out_dtype=act)
         return x1 + self.ffn(n2)
 
-    def _attn(self, x, alive_mask, bullets=None, bullet_mask=None, qkv=None):
+    def _attn(self, x, alive_mask, bullets=None, bullet_mask=None, qkv=None, project=True):
+        """Attention sublayer without the residual; ``project=False`` returns the merged heads
+        before ``out_proj`` (inference path only)."""
         if qkv is None:
             qkv = _project(self.qkv, x)  # (B, N, 3D), fp32 or bf16 under autocast
         if torch.is_grad_enabled():
@@ -214,7 +239,8 @@ class TransformerBlock(nn.Module):
                 w = self.kv_bullet.weight
                 pk = _cached_cast(self.kv_bullet, "_bnb_pack", (w,), torch.bfloat16, lambda: ops.pack_linear_weights(w))
                 kv_rows = ops.norm_linear(bullets, self.norm_bullet.weight, pk, eps=self.norm_bullet.eps, rows=rows)
-                return _project(self.out_proj, ops.sdpa_cross_rows(qkv, kv_rows, rows, self.n_heads, accum=merged))
+                merged = ops.sdpa_cross_rows(qkv, kv_rows, rows, self.n_heads, accum=merged)
+                return _project(self.out_proj, merged) if project else merged
             if rows is not None:
                 bullet_mask = rows.mask
             kv = _project(self.kv_bullet, self._norm_bullets(bullets, qkv.dtype))
@@ -222,7 +248,7 @@ class TransformerBlock(nn.Module):
                 merged = ops.sdpa_cross(qkv, kv, bullet_mask, self.n_heads, accum=merged)
             else:
                 merged = merged + self._bullet_read(qkv, kv, bullet_mask)
-        return _project(self.out_proj, merged)
+        return _project(self.out_proj, merged) if project else merged
 
     def _compact_read_ok(self, qkv, bullets) -> bool:
         """Whether the bullet read can run on the compacted list (bf16 projections, width 128,
@@ -393,6 +419,11 @@ class GriffinTemporalBlock(nn.Module):
         act = _projection_dtype()
         gate_in = _project(self.linear2, normed)
         if _fused_ok(x, act) and gate_in.dtype == act:
+            if y.dtype == torch.bfloat16 and y.shape == gate_in.shape:
+                # gelu(linear2) * y, linear_out, both residual adds, norm2 and the gated MLP in one kernel
+                fused = self.gated_mlp.fused_tail(x, y, self.norm2, proj_layer=self.linear_out, gate=gate_in)
+                if fused is not None:
+                    return fused
             # gelu(linear2) * y in one kernel, residual add + norm2 (+ cast) in one kernel
             r = _project(self.linear_out, ops.gelu_mul(gate_in, y, out_dtype=act))
             fused = self.gated_mlp.fused_tail(x, r, self.norm2)

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 10
+#define BNB_ABI_VERSION 11
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -395,6 +395,22 @@ int bnb_mask_fill(const uint8_t *mask, const int32_t *offsets, int32_t *index, i
 int bnb_ffn_fused_fwd(const float *x, int64_t x_row_stride, const void *delta, int delta_dtype,
                       const float *norm_weight, float eps, const void *weights_packed, float *out,
                       int64_t R, int D, int hidden, void *stream);
+
+/*
+ * bnb_ffn_fused_fwd with the sublayer's output projection folded in: the tensor added to x
+ * before the norm is  rows_a Wp^T  (rows_b == NULL: `out_proj` of models/yemong/attention.py:168-169
+ * applied to the merged attention heads) or  (bf16(gelu(rows_a)) * rows_b) Wp^T  (the temporal
+ * block's `linear_out(b1_out * gelu(linear2(normed)))`, models/yemong/griffin.py:281-284),
+ * computed on the matrix cores and accumulated straight onto x; the projection's output never
+ * exists in memory.
+ *
+ *   rows_a, rows_b  (R, 128) bf16 contiguous
+ *   proj_packed     Wp (128, 128) in bf16 as [cb][ks][l][e] = Wp[32cb + l%32][16ks + 8(e/4) + 4(l/32) + e%4]
+ *   other arguments as bnb_ffn_fused_fwd
+ */
+int bnb_ffn_fused_proj_fwd(const float *x, int64_t x_row_stride, const void *rows_a, const void *rows_b,
+                           const void *proj_packed, const float *norm_weight, float eps,
+                           const void *weights_packed, float *out, int64_t R, int D, int hidden, void *stream);
 
 /*
  * out = gelu(a) * b with the exact (erf) GELU, the gelu rounded to a's dtype as F.gelu does and

@@ -928,3 +928,30 @@ def test_sdpa_cross_over_compacted_rows_equals_the_masked_form(B, NQ, NK, p):
     assert torch.equal(got, merged + bare)
     if 160 < NK <= 2048:  # the masked form on the same kernel: same keys in the same order, bit for bit
         assert torch.equal(got, ops.sdpa_cross(qkv, kv, mask, H, accum=merged.clone()))
+
+
+@pytest.mark.parametrize("R", [1, 130, 5000])
+@pytest.mark.parametrize("gated", [False, True])
+def test_ffn_fused_with_folded_projection_matches_oracle(R, gated):
+    x, _, nw, p = _ffn_case(R + 7, R)
+    g = torch.Generator().manual_seed(R)
+    D = 128
+    Wp = torch.randn(D, D, generator=g) / D ** 0.5
+    rows_a = torch.randn(R, D, generator=g).bfloat16()
+    rows_y = torch.randn(R, D, generator=g).bfloat16()
+    rounded = {k: v.bfloat16().float() for k, v in p.items()}
+    operand = rows_a.float()
+    if gated:
+        operand = (torch.nn.functional.gelu(rows_a.float()).bfloat16().float() * rows_y.float()).bfloat16().float()
+    s = x + operand @ Wp.bfloat16().float().t()
+    want = s + torch_ref.gated_mlp(rounded, "f.", torch_ref.rms_norm(s, nw))
+    pk = ops.pack_ffn_weights(p["f.gate_proj.weight"].to(DEV), p["f.up_proj.weight"].to(DEV), p["f.down_proj.weight"].to(DEV))
+    wp = ops.pack_proj_weights(Wp.to(DEV))
+    proj = (rows_a.to(DEV), rows_y.to(DEV), wp) if gated else (rows_a.to(DEV), wp)
+    got = ops.ffn_fused(x.to(DEV), None, nw.to(DEV), pk, proj=proj)
+    assert max_rel(got.cpu(), want) <= BF16_TOL
+    assert max_rel(got.cpu() - x, want - x) <= BF16_TOL
+    # the folded projection against the same projection done outside (bf16 GEMM output as delta)
+    delta = (operand @ Wp.bfloat16().float().t()).bfloat16()
+    two_step = ops.ffn_fused(x.to(DEV), delta.to(DEV), nw.to(DEV), pk)
+    assert max_rel(got.cpu(), two_step.cpu()) <= 1e-2
