@@ -12,7 +12,7 @@ import os
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "_lib", "libbnb_amd.so")
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 F32, BF16 = 0, 1
 PATH_AUTO, PATH_VALU, PATH_MFMA = 0, 1, 2
 
@@ -34,7 +34,7 @@ SIGNATURES = {
     "bnb_rglru_step_rows_fwd": (
         _i, [_vp, _i, _vp, _i, _vp, _f, _vp, _i64, _vp, _i64, _vp, _i, _i64, _vp, _i, _i64, _i, _vp]
     ),
-    "bnb_conv_step_rows_fwd": (_i, [_vp, _i, _i64, _vp, _i64, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _vp]),
+    "bnb_conv_step_rows_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _vp]),
     "bnb_conv_step_fwd": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _vp]),
     "bnb_conv_seq_fwd": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "bnb_rglru_scan_fwd": (_i, [_vp, _i, _vp, _i, _vp, _f, _vp, _i64, _vp, _vp, _i, _vp, _i64, _i64, _i, _i, _i, _vp]),
@@ -46,7 +46,7 @@ SIGNATURES = {
     "bnb_mask_count": (_i, [_vp, _vp, _i, _i, _vp]),
     "bnb_mask_fill": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "bnb_ffn_fused_fwd": (_i, [_vp, _i64, _vp, _i, _vp, _f, _vp, _vp, _i64, _i, _i, _vp]),
-    "bnb_ffn_fused_proj_fwd": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _f, _vp, _vp, _i64, _i, _i, _vp]),
+    "bnb_ffn_fused_proj_fwd": (_i, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _f, _vp, _vp, _i64, _i, _i, _vp]),
     "bnb_gelu_mul_fwd": (_i, [_vp, _i, _i64, _vp, _i, _i64, _vp, _i, _i64, _i, _vp]),
     "bnb_copy_bytes": (_i, [_vp, _vp, _i64, _vp]),
 }

@@ -23,7 +23,7 @@ __global__ __launch_bounds__(THREADS) void conv_step_vec8_kernel(
     const BT *__restrict__ b1, const float *conv_in, int64_t conv_in_stride, const float *__restrict__ weight,
     const float *__restrict__ bias, const uint8_t *__restrict__ reset, int rows_per_env, float *__restrict__ v_out,
     uint16_t *__restrict__ v_bf16_out, float *conv_out, int64_t conv_out_stride, int64_t R, int D, int rows_per_block,
-    int64_t b1_group_stride)
+    int64_t b1_group_stride, int64_t b1_row_stride)
 {
     extern __shared__ float s_wb[];  // D*4 tap weights (as stored: [d][k]) then D biases
     for (int i = threadIdx.x; i < D * kTaps; i += THREADS) s_wb[i] = weight[i];
@@ -39,7 +39,8 @@ __global__ __launch_bounds__(THREADS) void conv_step_vec8_kernel(
     // environment of the row: for the reset flag and for inputs laid out per environment
     // (groups of rows_per_env rows, b1_group_stride elements apart)
     const int64_t env = (reset != nullptr || b1_group_stride != 0) ? row / rows_per_env : 0;
-    const int64_t b1_off = b1_group_stride != 0 ? env * b1_group_stride + (row - env * rows_per_env) * D : row * D;
+    const int64_t b1_off =
+        b1_group_stride != 0 ? env * b1_group_stride + (row - env * rows_per_env) * b1_row_stride : row * b1_row_stride;
     const Row8 cur = load8_stream(b1 + b1_off + d0);
     const float *pin = conv_in + row * conv_in_stride + d0;
     Row8 p0 = load8_stream(pin), p1 = load8_stream(pin + D), p2 = load8_stream(pin + 2 * D);
@@ -73,14 +74,15 @@ __global__ __launch_bounds__(kConvThreads) void conv_step_scalar_kernel(
     const BT *__restrict__ b1, const float *conv_in, int64_t conv_in_stride, const float *__restrict__ weight,
     const float *__restrict__ bias, const uint8_t *__restrict__ reset, int rows_per_env, float *__restrict__ v_out,
     uint16_t *__restrict__ v_bf16_out, float *conv_out, int64_t conv_out_stride, int64_t R, int D,
-    int64_t b1_group_stride)
+    int64_t b1_group_stride, int64_t b1_row_stride)
 {
     const int64_t idx = (int64_t)blockIdx.x * kConvThreads + threadIdx.x;
     if (idx >= R * D) return;
     const int64_t row = idx / D;
     const int d = (int)(idx - row * D);
     const int64_t env = (reset != nullptr || b1_group_stride != 0) ? row / rows_per_env : 0;
-    const int64_t b1_off = b1_group_stride != 0 ? env * b1_group_stride + (row - env * rows_per_env) * D : row * D;
+    const int64_t b1_off =
+        b1_group_stride != 0 ? env * b1_group_stride + (row - env * rows_per_env) * b1_row_stride : row * b1_row_stride;
     const bool zero = reset != nullptr && reset[env];
     const float *pin = conv_in + row * conv_in_stride + d;
     const float p0 = zero ? 0.0f : pin[0], p1 = zero ? 0.0f : pin[D], p2 = zero ? 0.0f : pin[2 * D];
@@ -103,9 +105,9 @@ template <typename BT>
 static int launch_conv(const void *b1, const float *conv_in, int64_t conv_in_stride, const float *weight,
                        const float *bias, const uint8_t *reset, int rows_per_env, float *v_out, uint16_t *v_bf16_out,
                        float *conv_out, int64_t conv_out_stride, int64_t R, int D, int64_t b1_group_stride,
-                       hipStream_t stream)
+                       int64_t b1_row_stride, hipStream_t stream)
 {
-    const bool vec = (D % 8 == 0) && (D / 8 <= kConvThreads) && aligned16(b1) && aligned16(conv_in) &&
+    const bool vec = (D % 8 == 0) && (D / 8 <= kConvThreads) && aligned16(b1) && (b1_row_stride % 8 == 0) && aligned16(conv_in) &&
                      aligned16(conv_out) && aligned16(v_out) && aligned16(v_bf16_out) && (conv_in_stride % 4 == 0) &&
                      (conv_out_stride % 4 == 0) && (size_t)D * (kTaps + 1) * sizeof(float) <= 48 * 1024;
     if (vec) {
@@ -119,24 +121,25 @@ static int launch_conv(const void *b1, const float *conv_in, int64_t conv_in_str
         if (big)
             hipLaunchKernelGGL((conv_step_vec8_kernel<kConvBigThreads, BT>), dim3((unsigned)blocks), dim3(threads), lds,
                                stream, (const BT *)b1, conv_in, conv_in_stride, weight, bias, reset, rows_per_env,
-                               v_out, v_bf16_out, conv_out, conv_out_stride, R, D, rows_per_block, b1_group_stride);
+                               v_out, v_bf16_out, conv_out, conv_out_stride, R, D, rows_per_block, b1_group_stride, b1_row_stride);
         else
             hipLaunchKernelGGL((conv_step_vec8_kernel<kConvThreads, BT>), dim3((unsigned)blocks), dim3(threads), lds,
                                stream, (const BT *)b1, conv_in, conv_in_stride, weight, bias, reset, rows_per_env,
-                               v_out, v_bf16_out, conv_out, conv_out_stride, R, D, rows_per_block, b1_group_stride);
+                               v_out, v_bf16_out, conv_out, conv_out_stride, R, D, rows_per_block, b1_group_stride, b1_row_stride);
     } else {
         const int64_t blocks = (R * D + kConvThreads - 1) / kConvThreads;
         if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
         hipLaunchKernelGGL((conv_step_scalar_kernel<BT>), dim3((unsigned)blocks), dim3(kConvThreads), 0, stream,
                            (const BT *)b1, conv_in, conv_in_stride, weight, bias, reset, rows_per_env, v_out,
-                           v_bf16_out, conv_out, conv_out_stride, R, D, b1_group_stride);
+                           v_bf16_out, conv_out, conv_out_stride, R, D, b1_group_stride, b1_row_stride);
     }
     return (int)hipGetLastError();
 }
 
 }  // namespace bnb
 
-extern "C" int bnb_conv_step_rows_fwd(const void *b1, int b1_dtype, int64_t b1_group_stride, const float *conv_in,
+extern "C" int bnb_conv_step_rows_fwd(const void *b1, int b1_dtype, int64_t b1_group_stride, int64_t b1_row_stride,
+                                      const float *conv_in,
                                       int64_t conv_in_row_stride, const float *weight, const float *bias,
                                       const uint8_t *reset, int rows_per_env, float *v_out, void *v_bf16_out,
                                       float *conv_out, int64_t conv_out_row_stride, int64_t R, int D, void *stream)
@@ -148,7 +151,9 @@ extern "C" int bnb_conv_step_rows_fwd(const void *b1, int b1_dtype, int64_t b1_g
     if (b1_dtype != BNB_F32 && b1_dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
     if (conv_in_row_stride < 3 * (int64_t)D || conv_out_row_stride < 3 * (int64_t)D) return BNB_ERR_BAD_SHAPE;
     if ((reset != nullptr || b1_group_stride != 0) && rows_per_env < 1) return BNB_ERR_BAD_SHAPE;
-    if (b1_group_stride != 0 && (b1_group_stride < (int64_t)rows_per_env * D || b1_group_stride % 8 != 0))
+    if (b1_row_stride == 0) b1_row_stride = D;
+    if (b1_row_stride < D) return BNB_ERR_BAD_SHAPE;
+    if (b1_group_stride != 0 && (b1_group_stride < (int64_t)rows_per_env * b1_row_stride || b1_group_stride % 8 != 0))
         return BNB_ERR_BAD_SHAPE;
     if ((reinterpret_cast<uintptr_t>(conv_in) | reinterpret_cast<uintptr_t>(conv_out) |
          reinterpret_cast<uintptr_t>(v_out) | reinterpret_cast<uintptr_t>(weight) |
@@ -159,9 +164,11 @@ extern "C" int bnb_conv_step_rows_fwd(const void *b1, int b1_dtype, int64_t b1_g
     hipStream_t s = (hipStream_t)stream;
     if (b1_dtype == BNB_BF16)
         return launch_conv<uint16_t>(b1, conv_in, conv_in_row_stride, weight, bias, reset, rows_per_env, v_out,
-                                     (uint16_t *)v_bf16_out, conv_out, conv_out_row_stride, R, D, b1_group_stride, s);
+                                     (uint16_t *)v_bf16_out, conv_out, conv_out_row_stride, R, D, b1_group_stride,
+                                     b1_row_stride, s);
     return launch_conv<float>(b1, conv_in, conv_in_row_stride, weight, bias, reset, rows_per_env, v_out,
-                              (uint16_t *)v_bf16_out, conv_out, conv_out_row_stride, R, D, b1_group_stride, s);
+                              (uint16_t *)v_bf16_out, conv_out, conv_out_row_stride, R, D, b1_group_stride,
+                                     b1_row_stride, s);
 }
 
 extern "C" int bnb_conv_step_fwd(const void *b1, int b1_dtype, const float *conv_in, int64_t conv_in_row_stride,
@@ -169,6 +176,6 @@ extern "C" int bnb_conv_step_fwd(const void *b1, int b1_dtype, const float *conv
                                  float *v_out, void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride,
                                  int64_t R, int D, void *stream)
 {
-    return bnb_conv_step_rows_fwd(b1, b1_dtype, 0, conv_in, conv_in_row_stride, weight, bias, reset, rows_per_env,
+    return bnb_conv_step_rows_fwd(b1, b1_dtype, 0, 0, conv_in, conv_in_row_stride, weight, bias, reset, rows_per_env,
                                   v_out, v_bf16_out, conv_out, conv_out_row_stride, R, D, stream);
 }

@@ -241,7 +241,7 @@ def rglru_step(
         if y_dtype is not None and y_dtype != y_out.dtype:
             raise ValueError("y_dtype and y_out disagree")
         if y_out.dim() == 3:
-            y_group = _grouped_rows(y_out, R, D, rows_per_env, "y_out")
+            y_group, _ = _grouped_rows(y_out, R, D, rows_per_env, "y_out")
         elif y_out.shape != (R, D) or not y_out.is_contiguous():
             raise ValueError("y_out must be a contiguous (R, D) tensor or a (B, n, D) view")
         y = y_out
@@ -263,16 +263,20 @@ def rglru_step(
     return (h_out if y is None else y), h_out
 
 
-def _grouped_rows(t: torch.Tensor, R: int, D: int, rows_per_env: int, name: str) -> int:
-    """Group stride (elements) of a (B, n, D) view whose rows are the R = B*n rows of one
-    environment after the other inside a wider tensor: ``t[b, i]`` at ``b * stride(0) + i * D``."""
+def _grouped_rows(t: torch.Tensor, R: int, D: int, rows_per_env: int, name: str, pitch_ok: bool = False):
+    """(group stride, row stride) in elements of a (B, n, D) view whose rows are the R = B*n rows
+    of one environment after the other inside a wider tensor: ``t[b, i]`` at
+    ``b * stride(0) + i * stride(1)``.  ``pitch_ok`` allows rows further apart than D (a column
+    block of a wider matrix)."""
     if t.dim() != 3 or t.shape[2] != D or t.shape[0] * t.shape[1] != R:
         raise ValueError(f"{name} must be (R, D) or a (B, n, D) view with B*n == R")
     if t.shape[1] != rows_per_env:
         raise ValueError(f"{name} groups rows by {t.shape[1]}, rows_per_env is {rows_per_env}")
-    if R and (t.stride(2) != 1 or t.stride(1) != D or t.stride(0) < t.shape[1] * D or t.stride(0) % 8):
-        raise ValueError(f"{name} must have contiguous rows, D apart, and a group stride that is a multiple of 8")
-    return t.stride(0) if t.shape[0] > 1 else t.shape[1] * D
+    row = t.stride(1) if t.shape[1] > 1 else D
+    if R and (t.stride(2) != 1 or (row != D and not pitch_ok) or row < D or row % 8
+              or (t.shape[0] > 1 and (t.stride(0) < t.shape[1] * row or t.stride(0) % 8))):
+        raise ValueError(f"{name} must have contiguous rows at a regular pitch and a group stride that is a multiple of 8")
+    return (t.stride(0) if t.shape[0] > 1 else t.shape[1] * row), row
 
 
 def _reset_pointer(reset, R: int, rows_per_env: int, device) -> int | None:
@@ -336,9 +340,10 @@ def conv_step(
     if bias is not None:
         bias = bias.detach().contiguous()
         bias_ptr = bias.data_ptr()
-    b1_group = 0
+    b1_group, b1_row = 0, 0
     if b1.dim() == 3 and not b1.is_contiguous():
-        b1_group = _grouped_rows(b1, R, D, rows_per_env, "b1")  # rows of every environment inside a wider tensor
+        # rows of every environment inside a wider tensor (and possibly a column block of it)
+        b1_group, b1_row = _grouped_rows(b1, R, D, rows_per_env, "b1", pitch_ok=True)
     else:
         b1 = b1.contiguous()
 
@@ -357,7 +362,7 @@ def conv_step(
     if R:
         with torch.cuda.device(b1.device):
             rc = _native.load().bnb_conv_step_rows_fwd(
-                b1.data_ptr(), b_code, int(b1_group), conv_buf.data_ptr(), conv_buf.stride(0), weight.data_ptr(), bias_ptr,
+                b1.data_ptr(), b_code, int(b1_group), int(b1_row), conv_buf.data_ptr(), conv_buf.stride(0), weight.data_ptr(), bias_ptr,
                 reset_ptr, int(rows_per_env), v.data_ptr(), None if v_lp is None else v_lp.data_ptr(),
                 conv_out.data_ptr(), conv_out.stride(0), R, D, _stream(),
             )
@@ -709,6 +714,18 @@ def pack_proj_weights(weight: torch.Tensor) -> torch.Tensor:
     return weight.detach().to(torch.bfloat16)[rows, cols].contiguous()
 
 
+def _uniform_rows(t: torch.Tensor, D: int) -> bool:
+    """Whether ``t`` (..., D) can be viewed as rows at one regular pitch without a copy (a
+    column block of a contiguous wider matrix qualifies)."""
+    if t.stride(-1) != 1 or t.dim() < 2:
+        return False
+    try:
+        v = t.view(-1, D)
+    except RuntimeError:
+        return False
+    return v.stride(0) % 8 == 0 and v.stride(0) >= D and v.data_ptr() % 16 == 0
+
+
 def ffn_supported(x: torch.Tensor, hidden: int) -> bool:
     """Whether ``ffn_fused`` covers this residual stream (fp32 on the GPU, width 128, hidden 512)."""
     return x.is_cuda and x.dtype == torch.float32 and x.shape[-1] == FFN_WIDTH and hidden == FFN_HIDDEN
@@ -768,16 +785,18 @@ def ffn_fused(
         if len(rows) not in (1, 2) or wp.dtype != torch.bfloat16 or wp.numel() != D * D or not wp.is_contiguous():
             raise ValueError("proj must be (rows, packed) or (rows_g, rows_y, packed) with pack_proj_weights output")
         flat = []
-        for t in rows:
+        for k, t in enumerate(rows):
             if t.shape != x.shape or t.dtype != torch.bfloat16:
                 raise ValueError(f"projection operand rows must be bfloat16 {tuple(x.shape)} tensors")
             if torch.is_grad_enabled() and t.requires_grad:
                 raise RuntimeError("ffn_fused is forward-only; call it under torch.no_grad()")
-            flat.append(t.reshape(-1, D).contiguous())
+            t2 = t.reshape(-1, D) if (k == 0 and _uniform_rows(t, D)) else t.reshape(-1, D).contiguous()
+            flat.append(t2)
         if R:
             with torch.cuda.device(x.device):
                 rc = _native.load().bnb_ffn_fused_proj_fwd(
-                    x2.data_ptr(), x2.stride(0), flat[0].data_ptr(), flat[1].data_ptr() if len(flat) == 2 else None,
+                    x2.data_ptr(), x2.stride(0), flat[0].data_ptr(), flat[0].stride(0),
+                    flat[1].data_ptr() if len(flat) == 2 else None,
                     wp.data_ptr(), norm_weight.data_ptr(), float(_F32_EPS if eps is None else eps),
                     weights_packed.data_ptr(), out.data_ptr(), R, D, FFN_HIDDEN, _stream(),
                 )

@@ -414,10 +414,11 @@ class GriffinTemporalBlock(nn.Module):
             return ops.add_rmsnorm(x, self.norm1.weight, eps=self.norm1.eps, out_dtype=act)[1]
         return self.norm1(x)
 
-    def _finish(self, x, normed, y):
+    def _finish(self, x, normed, y, gate_in=None):
         """Gate branch, output projection and the gated MLP, both residuals."""
         act = _projection_dtype()
-        gate_in = _project(self.linear2, normed)
+        if gate_in is None:
+            gate_in = _project(self.linear2, normed)
         if _fused_ok(x, act) and gate_in.dtype == act:
             if y.dtype == torch.bfloat16 and y.shape == gate_in.shape:
                 # gelu(linear2) * y, linear_out, both residual adds, norm2 and the gated MLP in one kernel
@@ -477,10 +478,20 @@ class GriffinTemporalBlock(nn.Module):
         B, NM, D = x.shape
         R = B * n_rec
         act = _projection_dtype()
-        normed = self._norm_in(x)
-        b1 = _project(self.linear1, normed)
+        gate_in = normed = None
+        if act == torch.bfloat16 and D == ops.FFN_WIDTH and self.linear1.bias is None and self.linear2.bias is None:
+            # norm1, linear1 and linear2 as one kernel: [b1 | gate_in] side by side, read in place
+            ws = (self.linear1.weight, self.linear2.weight)
+            pk = _cached_cast(self, "_bnb_l12_pack", ws, torch.bfloat16,
+                              lambda: ops.pack_linear_weights(torch.cat([ws[0], ws[1]], dim=0)))
+            both = ops.norm_linear(x, self.norm1.weight, pk, eps=self.norm1.eps)  # (B, NM, 2D)
+            b1, gate_in = both[..., :D], both[..., D:]
+        else:
+            normed = self._norm_in(x)
+            b1 = _project(self.linear1, normed)
         want_lp = act == torch.bfloat16
-        res = ops.conv_step(b1[:, :n_rec] if NM > n_rec else b1.reshape(R, D), state_in[:, D:].view(R, CONV_KERNEL - 1, D),
+        res = ops.conv_step(b1[:, :n_rec] if (NM > n_rec or gate_in is not None) else b1.reshape(R, D),
+                            state_in[:, D:].view(R, CONV_KERNEL - 1, D),
                             self.conv.weight, self.conv.bias, conv_out=state_out[:, D:].view(R, CONV_KERNEL - 1, D),
                             reset=reset, rows_per_env=n_rec, also_bf16=want_lp)
         y = torch.empty((B, NM, D), dtype=act, device=x.device)
@@ -490,7 +501,7 @@ class GriffinTemporalBlock(nn.Module):
             # gathered into one (B*M, D) matrix first: on the strided view the library would run a
             # batch of B tiny GEMMs
             y[:, n_rec:] = _project(field_sub, b1[:, n_rec:].reshape(-1, D)).view(B, NM - n_rec, D)
-        return self._finish(x, normed, y)
+        return self._finish(x, normed, y, gate_in)
 
     def forward_nonrecurrent(self, x, sub):
         """Same block with ``sub`` (a Linear) in place of conv + RG-LRU; no state."""

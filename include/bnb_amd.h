@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 11
+#define BNB_ABI_VERSION 12
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -228,8 +228,10 @@ int bnb_conv_step_fwd(const void *b1, int b1_dtype,
  * bnb_conv_step_fwd with the input b1 laid out per environment: with b1_group_stride != 0,
  * row r of b1 is at b1 + (r / rows_per_env) * b1_group_stride + (r % rows_per_env) * D elements
  * (the ship tokens inside a (B, N+M, D) tensor of linear1 outputs).  0: contiguous (R, D).
+ * b1_row_stride (elements, 0 = D) is the distance between consecutive rows, for a b1 that is a
+ * column block of a wider projection output (e.g. [linear1 | linear2] computed together).
  */
-int bnb_conv_step_rows_fwd(const void *b1, int b1_dtype, int64_t b1_group_stride,
+int bnb_conv_step_rows_fwd(const void *b1, int b1_dtype, int64_t b1_group_stride, int64_t b1_row_stride,
                            const float *conv_in, int64_t conv_in_row_stride,
                            const float *weight, const float *bias,
                            const uint8_t *reset, int rows_per_env,
@@ -404,11 +406,13 @@ int bnb_ffn_fused_fwd(const float *x, int64_t x_row_stride, const void *delta, i
  * computed on the matrix cores and accumulated straight onto x; the projection's output never
  * exists in memory.
  *
- *   rows_a, rows_b  (R, 128) bf16 contiguous
+ *   rows_a, rows_b  (R, 128) bf16; rows_b contiguous, rows_a rows rows_a_stride elements apart
+ *                   (0 = 128; a column block of a wider projection output works)
  *   proj_packed     Wp (128, 128) in bf16 as [cb][ks][l][e] = Wp[32cb + l%32][16ks + 8(e/4) + 4(l/32) + e%4]
  *   other arguments as bnb_ffn_fused_fwd
  */
-int bnb_ffn_fused_proj_fwd(const float *x, int64_t x_row_stride, const void *rows_a, const void *rows_b,
+int bnb_ffn_fused_proj_fwd(const float *x, int64_t x_row_stride, const void *rows_a, int64_t rows_a_stride,
+                           const void *rows_b,
                            const void *proj_packed, const float *norm_weight, float eps,
                            const void *weights_packed, float *out, int64_t R, int D, int hidden, void *stream);
 

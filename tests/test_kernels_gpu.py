@@ -955,3 +955,25 @@ def test_ffn_fused_with_folded_projection_matches_oracle(R, gated):
     delta = (operand @ Wp.bfloat16().float().t()).bfloat16()
     two_step = ops.ffn_fused(x.to(DEV), delta.to(DEV), nw.to(DEV), pk)
     assert max_rel(got.cpu(), two_step.cpu()) <= 1e-2
+
+
+def test_column_block_operands_are_read_in_place():
+    # [linear1 | linear2] outputs side by side: the conv reads the left block, the tail's gate the right one
+    B, n, NM, D = 6, 8, 12, 128
+    g = torch.Generator().manual_seed(4)
+    both = torch.randn(B, NM, 2 * D, generator=g).bfloat16().to(DEV)
+    b1, gate = both[..., :D], both[..., D:]
+    buf = torch.randn(B * n, 3, D, generator=g).to(DEV)
+    w = (0.5 * torch.randn(D, 1, 4, generator=g)).to(DEV)
+    bias = (0.1 * torch.randn(D, generator=g)).to(DEV)
+    v_a, buf_a = ops.conv_step(b1[:, :n], buf, w, bias, rows_per_env=n)
+    v_b, buf_b = ops.conv_step(b1[:, :n].reshape(B * n, D).contiguous(), buf, w, bias)
+    assert torch.equal(v_a, v_b) and torch.equal(buf_a, buf_b)
+    x, _, nw, p = _ffn_case(3, B * NM)
+    pk = ops.pack_ffn_weights(p["f.gate_proj.weight"].to(DEV), p["f.up_proj.weight"].to(DEV), p["f.down_proj.weight"].to(DEV))
+    wp = ops.pack_proj_weights((torch.randn(D, D, generator=g) / D ** 0.5).to(DEV))
+    y = torch.randn(B, NM, D, generator=g).bfloat16().to(DEV)
+    xd = x.to(DEV).view(B, NM, D)
+    in_place = ops.ffn_fused(xd, None, nw.to(DEV), pk, proj=(gate, y, wp))
+    copied = ops.ffn_fused(xd, None, nw.to(DEV), pk, proj=(gate.contiguous(), y, wp))
+    assert torch.equal(in_place, copied)
