@@ -192,6 +192,44 @@ def test_sdpa_mfma_live_counts_across_block_edges():
         assert max_rel(got[b], truth[b]) <= BF16_TOL, counts[b]
 
 
+@pytest.mark.parametrize("NM", [1, 2, 5, 12, 15, 16])
+@pytest.mark.parametrize("H", [2, 4, 8, 3])
+def test_sdpa_two_heads_per_wave_for_up_to_16_tokens(NM, H):
+    # up to 16 tokens and an even head count take the kernel that shares one matrix-core tile
+    # between two heads (an odd head count keeps one head per wave); per environment: mixed,
+    # all alive, all dead, only the first and only the last token alive
+    B, D = 37, 32 * H
+    qkv = _qkv(300 + NM + H, B, NM, D, torch.bfloat16)
+    alive = _alive(300 + NM, B, NM, 0.6)
+    alive[0] = True
+    alive[1] = False
+    alive[2] = False
+    alive[2, 0] = True
+    alive[3] = False
+    alive[3, NM - 1] = True
+    got = _run_sdpa(qkv, alive, H, "mfma").float()
+    truth = torch_ref.sdpa_masked(qkv.float(), alive, H)
+    assert torch.isfinite(got).all()
+    for b in range(B):
+        assert max_rel(got[b], truth[b]) <= BF16_TOL, (b, alive[b])
+    mean_v = qkv[1, :, 2 * D:].float().mean(dim=0, keepdim=True).expand(NM, D)
+    assert (got[1] - mean_v).abs().max() <= 1.6e-2
+    assert torch.equal(got[3], qkv[3, NM - 1, 2 * D:].float().expand(NM, D))
+    # dead keys weigh exactly nothing: rewriting their K and V rows changes no output bit
+    pert = qkv.clone()
+    dead = ~alive
+    dead[~alive.any(dim=1)] = False  # an all-dead environment averages every row
+    pert[..., D:][dead] = pert[..., D:][dead] * -3.0 + 17.0
+    assert torch.equal(_run_sdpa(pert, alive, H, "mfma").float(), got)
+    # heads do not leak into each other: changing one head's inputs leaves the others' outputs alone
+    other = qkv.clone()
+    for part in range(3):
+        other[..., part * D: part * D + 32] = other[..., part * D: part * D + 32] * 2.0 + 1.0
+    again = _run_sdpa(other, alive, H, "mfma").float()
+    assert torch.equal(again[..., 32:], got[..., 32:])
+    assert not torch.equal(again[..., :32], got[..., :32])
+
+
 @pytest.mark.parametrize("NM,path", [(161, "auto"), (200, "auto"), (320, "auto")])
 def test_sdpa_bf16_beyond_matrix_core_range_uses_the_vector_kernel(NM, path):
     # crossover evaluation reaches 320 ships (modes/crossover.py:92); more than 160 tokens in bf16
