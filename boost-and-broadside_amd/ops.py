@@ -370,6 +370,142 @@ def conv_step(
     return (v, conv_out, v_lp) if also_bf16 else (v, conv_out)
 
 
+def pack_gate_weights(weight_a: torch.Tensor, weight_x: torch.Tensor) -> torch.Tensor:
+    """``linear_a.weight`` and ``linear_x.weight`` (128, 128 each) as the bfloat16 operand stream
+    of ``temporal_step``: ``[hf][q][ks][l][e]`` with the index meaning given in
+    ``include/bnb_amd.h`` (every matrix-core operand one contiguous 1 KB run; a lane's 16 outputs
+    per block of 32 channels are 16 consecutive channels)."""
+    D = FFN_WIDTH
+    if weight_a.shape != (D, D) or weight_x.shape != (D, D):
+        raise ValueError("temporal_step covers (128, 128) gate weights")
+    dev = weight_a.device
+    w = torch.cat([weight_a.detach(), weight_x.detach()], dim=0).to(torch.bfloat16)
+    hf = torch.arange(2, device=dev)[:, None, None, None, None]
+    q = torch.arange(4, device=dev)[None, :, None, None, None]
+    ks = torch.arange(8, device=dev)[None, None, :, None, None]
+    lane = torch.arange(64, device=dev)[None, None, None, :, None]
+    e = torch.arange(8, device=dev)[None, None, None, None, :]
+    r = lane % 32
+    rows = (q // 2) * D + 64 * hf + 32 * (q % 2) + 16 * ((r // 4) % 2) + 4 * (r // 8) + r % 4
+    cols = 16 * ks + 8 * (lane // 32) + e
+    rows, cols = torch.broadcast_tensors(rows, cols)
+    return w[rows, cols].contiguous()
+
+
+def temporal_step_supported(b1: torch.Tensor) -> bool:
+    """Whether ``temporal_step`` covers these linear1 outputs: bfloat16, 128 channels."""
+    return b1.is_cuda and b1.dtype == torch.bfloat16 and b1.shape[-1] == FFN_WIDTH
+
+
+def temporal_step(
+    b1: torch.Tensor,
+    conv_buf: torch.Tensor,
+    h: torch.Tensor,
+    conv_weight: torch.Tensor,
+    conv_bias: torch.Tensor | None,
+    gate_weight_packed: torch.Tensor,
+    gate_bias: torch.Tensor,
+    log_lambda: torch.Tensor,
+    c: float,
+    *,
+    conv_out: torch.Tensor | None = None,
+    h_out: torch.Tensor | None = None,
+    y_out: torch.Tensor | None = None,
+    reset: torch.Tensor | None = None,
+    rows_per_env: int = 1,
+):
+    """``conv_step`` -> gate projections -> ``rglru_step`` of one timestep as a single kernel
+    (bfloat16 autocast flow; the conv output and the gate pre-activations never reach memory).
+
+    Args:
+        b1:        (R, 128) bfloat16 ``linear1`` outputs, or a (B, rows_per_env, 128) view into a
+                   wider tensor (ship rows of a (B, N+M, ...) projection, possibly a column block).
+        conv_buf, conv_out: (R, 3, 128) float32 stored inputs and their destination, as in ``conv_step``.
+        h, h_out:  (R, 128) float32 state and its destination, as in ``rglru_step``.
+        conv_weight (128, 4) or (128, 1, 4), conv_bias (128,) or None: float32.
+        gate_weight_packed: ``pack_gate_weights(linear_a.weight, linear_x.weight)``.
+        gate_bias: (256,) float32 ``[linear_a.bias | linear_x.bias]``.
+        y_out:     optional bfloat16 destination of the layer output: contiguous (R, 128) or a
+                   (B, rows_per_env, 128) view into a wider token tensor.
+        reset, rows_per_env: as in ``rglru_step``.
+
+    Returns:
+        (y, h_new, new_conv_buf).
+    """
+    D = FFN_WIDTH
+    if b1.dim() not in (2, 3) or b1.shape[-1] != D or b1.dtype != torch.bfloat16:
+        raise ValueError("b1 must be bfloat16 (R, 128) or a (B, rows_per_env, 128) view")
+    R = b1.numel() // D
+    if conv_buf.shape != (R, 3, D) or h.shape != (R, D):
+        raise ValueError(f"conv_buf must be {(R, 3, D)} and h {(R, D)}, got {tuple(conv_buf.shape)}, {tuple(h.shape)}")
+    if gate_weight_packed.shape != (2, 4, 8, 64, 8) or gate_weight_packed.dtype != torch.bfloat16:
+        raise ValueError("gate_weight_packed must come from pack_gate_weights")
+    if gate_bias.shape != (2 * D,) or log_lambda.shape != (D,):
+        raise ValueError("gate_bias must be (256,) and log_lambda (128,)")
+    for name, t in (("b1", b1), ("conv_buf", conv_buf), ("h", h), ("conv_weight", conv_weight),
+                    ("gate_weight_packed", gate_weight_packed), ("gate_bias", gate_bias), ("log_lambda", log_lambda)):
+        _need_device(t, name)
+    for name, t in (("conv_buf", conv_buf), ("h", h), ("conv_weight", conv_weight), ("gate_bias", gate_bias),
+                    ("log_lambda", log_lambda)):
+        if t.dtype != torch.float32:
+            raise TypeError(f"{name} must be float32")
+    if conv_bias is not None and conv_bias.dtype != torch.float32:
+        raise TypeError("conv_bias must be float32")
+    if torch.is_grad_enabled() and (b1.requires_grad or conv_buf.requires_grad or h.requires_grad):
+        raise RuntimeError("temporal_step is forward-only; call it under torch.no_grad()")
+    dev = b1.device
+    conv_weight = conv_weight.detach().reshape(D, 4).contiguous()
+    conv_bias = None if conv_bias is None else conv_bias.detach().contiguous()
+    gate_weight_packed = gate_weight_packed.contiguous()
+    gate_bias = gate_bias.detach().contiguous()
+    log_lambda = log_lambda.detach().contiguous()
+    b1_group, b1_row = 0, D
+    if b1.dim() == 3 and not b1.is_contiguous():
+        b1_group, b1_row = _grouped_rows(b1, R, D, rows_per_env, "b1", pitch_ok=True)
+    else:
+        b1 = b1.contiguous()
+
+    def conv_rows_ok(t):
+        return R == 0 or (t.stride(2) == 1 and t.stride(1) == D)
+
+    if not conv_rows_ok(conv_buf):
+        conv_buf = conv_buf.contiguous()
+    if R and h.stride(-1) != 1:
+        h = h.contiguous()
+    if conv_out is None:
+        conv_out = torch.empty((R, 3, D), dtype=torch.float32, device=dev)
+    elif conv_out.shape != (R, 3, D) or conv_out.dtype != torch.float32 or conv_out.device != dev or not conv_rows_ok(conv_out):
+        raise ValueError("conv_out must be a float32 (R, 3, 128) tensor on b1's device with contiguous rows")
+    if h_out is None:
+        h_out = torch.empty((R, D), dtype=torch.float32, device=dev)
+    elif h_out.shape != (R, D) or h_out.dtype != torch.float32 or h_out.device != dev or (R and h_out.stride(-1) != 1):
+        raise ValueError("h_out must be a float32 (R, 128) tensor on b1's device, contiguous in its last dim")
+    y_group = 0
+    if y_out is None:
+        y_out = torch.empty((R, D), dtype=torch.bfloat16, device=dev)
+    else:
+        if y_out.dtype != torch.bfloat16 or y_out.device != dev:
+            raise ValueError("y_out must be a bfloat16 tensor on b1's device")
+        if y_out.dim() == 3:
+            y_group, _ = _grouped_rows(y_out, R, D, rows_per_env, "y_out")
+        elif y_out.shape != (R, D) or not y_out.is_contiguous():
+            raise ValueError("y_out must be a contiguous (R, 128) tensor or a (B, n, 128) view")
+    reset_ptr = _reset_pointer(reset, R, rows_per_env, dev)
+    if (b1_group or y_group) and (rows_per_env < 1 or R % rows_per_env):
+        raise ValueError(f"rows_per_env={rows_per_env} does not divide the {R} rows")
+    if R:
+        with torch.cuda.device(dev):
+            rc = _native.load().bnb_temporal_step_fwd(
+                b1.data_ptr(), int(b1_group), int(b1_row), conv_buf.data_ptr(), conv_buf.stride(0),
+                conv_out.data_ptr(), conv_out.stride(0), h.data_ptr(), h.stride(0), h_out.data_ptr(), h_out.stride(0),
+                conv_weight.data_ptr(), None if conv_bias is None else conv_bias.data_ptr(),
+                gate_weight_packed.data_ptr(), gate_bias.data_ptr(), log_lambda.data_ptr(), float(c),
+                y_out.data_ptr(), int(y_group), reset_ptr, int(rows_per_env), R, D, _stream(),
+            )
+        _native.check(rc, "bnb_temporal_step_fwd")
+    return y_out, h_out, conv_out
+
+
 def _done_pointer(done, R, T, device):
     """Contiguous byte view of an optional (R, T) episode-end mask; returns (keepalive, pointer)."""
     if done is None:

@@ -490,11 +490,27 @@ class GriffinTemporalBlock(nn.Module):
             normed = self._norm_in(x)
             b1 = _project(self.linear1, normed)
         want_lp = act == torch.bfloat16
-        res = ops.conv_step(b1[:, :n_rec] if (NM > n_rec or gate_in is not None) else b1.reshape(R, D),
-                            state_in[:, D:].view(R, CONV_KERNEL - 1, D),
+        y = torch.empty((B, NM, D), dtype=act, device=x.device)
+        ships_b1 = b1[:, :n_rec] if (NM > n_rec or gate_in is not None) else b1.reshape(R, D)
+        rg = self.rg_lru
+        if ops.temporal_step_supported(b1) and rg.linear_a.bias is not None and rg.linear_x.bias is not None:
+            # conv taps + buffer shift, both gate projections and the recurrence as one kernel:
+            # the conv output and the gate pre-activations never reach memory
+            gw = (rg.linear_a.weight, rg.linear_x.weight)
+            gb = (rg.linear_a.bias, rg.linear_x.bias)
+            gpk = _cached_cast(rg, "_bnb_gate_pack", gw, torch.bfloat16, lambda: ops.pack_gate_weights(*gw))
+            gbias = _cached_cast(rg, "_bnb_gate_bias", gb, torch.float32,
+                                 lambda: torch.cat([gb[0], gb[1]], dim=0).detach().float())
+            ops.temporal_step(ships_b1, state_in[:, D:].view(R, CONV_KERNEL - 1, D), state_in[:, :D],
+                              self.conv.weight, self.conv.bias, gpk, gbias, rg.log_lambda, rg.c,
+                              conv_out=state_out[:, D:].view(R, CONV_KERNEL - 1, D), h_out=state_out[:, :D],
+                              y_out=y[:, :n_rec] if NM > n_rec else y.view(R, D), reset=reset, rows_per_env=n_rec)
+            if NM > n_rec:
+                y[:, n_rec:] = _project(field_sub, b1[:, n_rec:].reshape(-1, D)).view(B, NM - n_rec, D)
+            return self._finish(x, normed, y, gate_in)
+        res = ops.conv_step(ships_b1, state_in[:, D:].view(R, CONV_KERNEL - 1, D),
                             self.conv.weight, self.conv.bias, conv_out=state_out[:, D:].view(R, CONV_KERNEL - 1, D),
                             reset=reset, rows_per_env=n_rec, also_bf16=want_lp)
-        y = torch.empty((B, NM, D), dtype=act, device=x.device)
         self.rg_lru.step(res[0], state_in[:, :D], h_out=state_out[:, :D], reset=reset, rows_per_env=n_rec,
                          x_act=res[2] if want_lp else None, y_out=y[:, :n_rec] if NM > n_rec else y.view(R, D))
         if NM > n_rec:

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 12
+#define BNB_ABI_VERSION 13
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -237,6 +237,47 @@ int bnb_conv_step_rows_fwd(const void *b1, int b1_dtype, int64_t b1_group_stride
                            const uint8_t *reset, int rows_per_env,
                            float *v_out, void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride,
                            int64_t R, int D, void *stream);
+
+/*
+ * One timestep of the temporal sublayer's state path in one launch: conv taps + buffer shift
+ * (bnb_conv_step_rows_fwd), the two RG-LRU gate projections, and the recurrence
+ * (bnb_rglru_step_rows_fwd), under the dtype flow of bfloat16 autocast.
+ *
+ * Replaces, in models/yemong/griffin.py at T = 1: :275-277 (cat, _causal_depthwise_conv :127-139,
+ * buffer slice) and RGLRU.forward_sequence :206-219 with its linear_a / linear_x (:166-167), i.e.
+ * everything between `linear1` and the `rglru_out * gate` product of :279-281.  The conv output
+ * and the gate pre-activations stay on chip (4608 instead of 7168 bytes of traffic per row).
+ *
+ *   b1, b1_group_stride, b1_row_stride   bf16 linear1 outputs, addressed as in bnb_conv_step_rows_fwd
+ *   conv_in / conv_out  [p0|p1|p2] per row, fp32, as in bnb_conv_step_fwd (may be the same buffer)
+ *   h_in / h_out        fp32 state rows, as in bnb_rglru_step_fwd (may be the same buffer)
+ *   conv_weight (D,4), conv_bias (D) or NULL, fp32
+ *   gate_weight_packed  bf16 [linear_a.weight ; linear_x.weight] (2D, D) in matrix-core operand
+ *                       order [hf][q][ks][l][e], 32768 entries: entry = W[row, col] with
+ *                       row = (q/2)*D + 64*hf + 32*(q%2) + 16*((l%32/4)%2) + 4*(l%32/8) + l%4,
+ *                       col = 16*ks + 8*(l/32) + e     (hf<2, q<4, ks<8, l<64, e<8)
+ *   gate_bias           fp32 (2D) = [linear_a.bias | linear_x.bias]; rounded to bf16 inside, as
+ *                       autocast hands it to the GEMM
+ *   log_lambda (D) fp32, c
+ *   y, y_group_stride   bf16 layer output = bf16(h'), addressed as in bnb_rglru_step_rows_fwd
+ *   reset, rows_per_env as in the two kernels it replaces
+ *
+ * Requirements: D == 128, R < 2^31, 16-byte aligned pointers, row strides multiples of 4 (fp32)
+ * or 8 (bf16) elements.  Gate pre-activations are accumulated in fp32 on the matrix cores and
+ * rounded to bf16 once (the library GEMM's rounding point); summation order differs from the
+ * library's, so single pre-activations may differ by one bf16 ulp.
+ */
+int bnb_temporal_step_fwd(const void *b1, int64_t b1_group_stride, int64_t b1_row_stride,
+                          const float *conv_in, int64_t conv_in_row_stride,
+                          float *conv_out, int64_t conv_out_row_stride,
+                          const float *h_in, int64_t h_in_row_stride,
+                          float *h_out, int64_t h_out_row_stride,
+                          const float *conv_weight, const float *conv_bias,
+                          const void *gate_weight_packed, const float *gate_bias,
+                          const float *log_lambda, float c,
+                          void *y, int64_t y_group_stride,
+                          const uint8_t *reset, int rows_per_env,
+                          int64_t R, int D, void *stream);
 
 /*
  * The same causal depthwise conv over a whole sequence of T steps per row, with episode

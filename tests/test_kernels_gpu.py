@@ -885,6 +885,136 @@ def test_state_kernels_address_ship_rows_inside_the_token_tensor(B, n, NM, dtype
         ops.rglru_step(v_a, gates, lam, 8.0, h, rows_per_env=n + 1, y_out=wide[:, :n])
 
 
+# ------------------------------------------------------------------ conv + gate projections + recurrence in one kernel
+
+
+def _temporal_inputs(seed, R, D=128):
+    g = torch.Generator().manual_seed(seed)
+    return dict(
+        b1=torch.randn(R, D, generator=g).to(torch.bfloat16),
+        buf=torch.randn(R, 3, D, generator=g),
+        h=0.5 * torch.randn(R, D, generator=g),
+        cw=0.5 * torch.randn(D, 1, 4, generator=g),
+        cb=0.1 * torch.randn(D, generator=g),
+        wa=torch.randn(D, D, generator=g) / D ** 0.5,
+        wx=torch.randn(D, D, generator=g) / D ** 0.5,
+        ba=0.3 * torch.randn(D, generator=g),
+        bx=0.3 * torch.randn(D, generator=g),
+        lam=torch.linspace(0.0, 4.0, D),
+    )
+
+
+def _temporal_truth(t, reset=None, rows_per_env=1):
+    """fp32 statement on the same (already rounded) inputs: conv taps, gate projections of the
+    unrounded conv output, recurrence.  Returns (h', shifted buffer)."""
+    b1 = t["b1"].float()
+    buf, h = t["buf"].clone(), t["h"].clone()
+    if reset is not None:
+        rows = reset.repeat_interleave(rows_per_env)
+        buf[rows] = 0.0
+        h[rows] = 0.0
+    w = t["cw"].reshape(-1, 4)
+    v = buf[:, 0] * w[:, 0] + buf[:, 1] * w[:, 1] + buf[:, 2] * w[:, 2] + b1 * w[:, 3] + t["cb"]
+    wa, wx = t["wa"].to(torch.bfloat16).float(), t["wx"].to(torch.bfloat16).float()
+    gates = torch.cat([v @ wa.t() + t["ba"], v @ wx.t() + t["bx"]], dim=1)
+    h_new = torch_ref.rglru_step(v, gates, t["lam"], 8.0, h)
+    return h_new, torch.stack([buf[:, 1], buf[:, 2], b1], dim=1)
+
+
+@pytest.mark.parametrize("R", [1, 31, 32, 33, 257, 5000, 70001])
+@pytest.mark.parametrize("with_reset", [False, True])
+def test_temporal_step_matches_oracle_and_the_three_kernel_composition(R, with_reset):
+    t = _temporal_inputs(R, R)
+    d = {k: v.to(DEV) for k, v in t.items()}
+    reset = None
+    if with_reset:
+        reset = torch.rand(R, generator=torch.Generator().manual_seed(R)) < 0.3
+    rdev = None if reset is None else reset.to(DEV)
+    pk = ops.pack_gate_weights(d["wa"], d["wx"])
+    gb = torch.cat([d["ba"], d["bx"]])
+    y, h_new, buf_new = ops.temporal_step(d["b1"], d["buf"], d["h"], d["cw"], d["cb"], pk, gb, d["lam"], 8.0, reset=rdev)
+    torch.cuda.synchronize()
+    h_true, buf_true = _temporal_truth(t, reset)
+    assert torch.equal(buf_new.cpu(), buf_true)  # the buffer shift only moves values
+    assert max_rel(h_new.cpu(), h_true) <= BF16_TOL
+    assert torch.equal(y, h_new.to(torch.bfloat16))
+    # the composition it replaces: conv kernel, library GEMM on the bf16 conv output, recurrence kernel
+    v, buf_c, v_lp = ops.conv_step(d["b1"], d["buf"], d["cw"], d["cb"], reset=rdev, also_bf16=True)
+    gates = torch.nn.functional.linear(v_lp, torch.cat([d["wa"], d["wx"]]).to(torch.bfloat16), gb.to(torch.bfloat16))
+    y_c, h_c = ops.rglru_step(v, gates, d["lam"], 8.0, d["h"], reset=rdev, y_dtype=torch.bfloat16)
+    assert torch.equal(buf_new, buf_c)
+    # same rounding points; the conv arithmetic may differ in the last fp32 bit and the summation
+    # order inside the projections now and then moves a pre-activation by one bf16 ulp
+    assert max_rel(h_new, h_c) <= 8e-3
+    assert (y == y_c).float().mean().item() >= 0.999
+    off = ((h_new - h_c).abs() > 1e-5 * h_c.abs().clamp_min(1e-2)).float().mean().item()
+    assert off <= 1e-3, off
+    assert max_rel(h_c.cpu(), h_true) <= BF16_TOL
+
+
+def test_temporal_step_every_gate_weight_reaches_its_channel():
+    # one-hot gate weights: channel j of gate g sees exactly conv-output channel perm[j]; any
+    # slip in the operand packing or in the channel order of the exchange shows as a mismatch
+    R, D = 64, 128
+    t = _temporal_inputs(5, R)
+    g = torch.Generator().manual_seed(6)
+    pa, px = torch.randperm(D, generator=g), torch.randperm(D, generator=g)
+    t["wa"] = torch.zeros(D, D)
+    t["wa"][torch.arange(D), pa] = 2.0
+    t["wx"] = torch.zeros(D, D)
+    t["wx"][torch.arange(D), px] = -1.5
+    d = {k: v.to(DEV) for k, v in t.items()}
+    _, h_new, _ = ops.temporal_step(d["b1"], d["buf"], d["h"], d["cw"], d["cb"], ops.pack_gate_weights(d["wa"], d["wx"]),
+                                    torch.cat([d["ba"], d["bx"]]), d["lam"], 8.0)
+    h_true, _ = _temporal_truth(t)
+    assert max_rel(h_new.cpu(), h_true) <= BF16_TOL
+    # elementwise too: a swapped pair of channels would hide inside a max-norm bound less easily here
+    assert torch.allclose(h_new.cpu(), h_true, rtol=3e-2, atol=3e-2)
+
+
+@pytest.mark.parametrize("B,n,NM", [(3, 8, 12), (5, 19, 23), (600, 8, 12), (7, 152, 160)])
+def test_temporal_step_reads_and_writes_ship_rows_inside_wider_tensors(B, n, NM):
+    D, R = 128, B * n
+    t = _temporal_inputs(B + NM, R)
+    d = {k: v.to(DEV) for k, v in t.items()}
+    g = torch.Generator().manual_seed(B)
+    both = torch.randn(B, NM, 2 * D, generator=g).to(torch.bfloat16).to(DEV)  # [linear1 | linear2] of all tokens
+    both[:, :n, :D] = d["b1"].view(B, n, D)
+    reset = (torch.rand(B, generator=g) < 0.4).to(DEV)
+    pk, gb = ops.pack_gate_weights(d["wa"], d["wx"]), torch.cat([d["ba"], d["bx"]])
+    # packed state rows [h | p0 | p1 | p2], read from one tensor and written into another
+    state_in = torch.cat([d["h"], d["buf"].reshape(R, 3 * D)], dim=1)
+    state_out = torch.full_like(state_in, 3.0)
+    wide = torch.full((B, NM, D), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.temporal_step(both[:, :n, :D], state_in[:, D:].view(R, 3, D), state_in[:, :D], d["cw"], d["cb"], pk, gb, d["lam"], 8.0,
+                      conv_out=state_out[:, D:].view(R, 3, D), h_out=state_out[:, :D], y_out=wide[:, :n], reset=reset,
+                      rows_per_env=n)
+    y_ref, h_ref, buf_ref = ops.temporal_step(d["b1"], d["buf"], d["h"], d["cw"], d["cb"], pk, gb, d["lam"], 8.0, reset=reset,
+                                              rows_per_env=n)
+    assert torch.equal(state_out[:, :D], h_ref) and torch.equal(state_out[:, D:].view(R, 3, D), buf_ref)
+    assert torch.equal(wide[:, :n].reshape(R, D), y_ref)
+    assert (wide[:, n:] == 7.0).all()
+    # in place: the state may be updated where it lives
+    ops.temporal_step(d["b1"], state_in[:, D:].view(R, 3, D), state_in[:, :D], d["cw"], d["cb"], pk, gb, d["lam"], 8.0,
+                      conv_out=state_in[:, D:].view(R, 3, D), h_out=state_in[:, :D], reset=reset, rows_per_env=n)
+    assert torch.equal(state_in, state_out)
+
+
+def test_temporal_step_rejects_what_it_does_not_cover():
+    t = {k: v.to(DEV) for k, v in _temporal_inputs(1, 4).items()}
+    pk, gb = ops.pack_gate_weights(t["wa"], t["wx"]), torch.cat([t["ba"], t["bx"]])
+    with pytest.raises(ValueError):
+        ops.temporal_step(t["b1"].float(), t["buf"], t["h"], t["cw"], t["cb"], pk, gb, t["lam"], 8.0)
+    with pytest.raises(ValueError):
+        ops.temporal_step(t["b1"], t["buf"][:3], t["h"], t["cw"], t["cb"], pk, gb, t["lam"], 8.0)
+    with pytest.raises(ValueError):
+        ops.temporal_step(t["b1"], t["buf"], t["h"], t["cw"], t["cb"], pk.reshape(-1), gb, t["lam"], 8.0)
+    with pytest.raises(ValueError):
+        ops.pack_gate_weights(torch.zeros(64, 64, device=DEV), torch.zeros(64, 64, device=DEV))
+    empty = ops.temporal_step(t["b1"][:0], t["buf"][:0], t["h"][:0], t["cw"], t["cb"], pk, gb, t["lam"], 8.0)
+    assert empty[0].shape == (0, 128) and empty[1].shape == (0, 128) and empty[2].shape == (0, 3, 128)
+
+
 # ------------------------------------------------------------------ RMSNorm + Linear, compact row lists
 
 
