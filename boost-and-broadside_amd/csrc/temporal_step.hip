@@ -30,14 +30,17 @@
 namespace bnb {
 
 constexpr int kTsD = 128;
-constexpr int kTsWaves = 8;
-constexpr int kTsThreads = kTsWaves * kWave;
+constexpr int kTsMaxWaves = 8;                    // waves of a work-group; fewer when there are few rows
 constexpr int kTsRows = 32;                       // rows of one wave's tile
 constexpr int kTsPitch = kTsD + 8;                // halfs per row of a wave's LDS tile: 272 bytes
 constexpr int kTsWeightHalfs = 2 * kTsD * kTsD;   // [Wa | Wx] in bf16: 64 KB
 constexpr int kTsTileHalfs = kTsRows * kTsPitch;
-constexpr size_t kTsLdsBytes = (size_t)kTsWeightHalfs * 2 + (size_t)kTsWaves * kTsTileHalfs * 2 +
-                               (size_t)(kTsD * 4 + kTsD + 2 * kTsD) * sizeof(float);
+constexpr int kTsTableFloats = kTsD * 4 + kTsD + 2 * kTsD + kTsD;  // conv taps, conv bias, gate bias, log2 sigmoid(lambda)
+
+static size_t ts_lds_bytes(int waves)
+{
+    return (size_t)kTsWeightHalfs * 2 + (size_t)kTsTableFloats * sizeof(float) + (size_t)waves * kTsTileHalfs * 2;
+}
 
 // LDS traffic between lanes of ONE wave: LDS operations of a wave complete in issue order, so
 // only the compiler has to be kept from moving accesses across the hand-over point.
@@ -48,27 +51,30 @@ __device__ __forceinline__ void wave_lds_handover()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-__global__ __launch_bounds__(kTsThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void temporal_step_kernel(
+__global__ __launch_bounds__(kTsMaxWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void temporal_step_kernel(
     const uint16_t *__restrict__ b1, int64_t b1_group_stride, int64_t b1_row_stride, const float *conv_in,
     int64_t conv_in_stride, float *conv_out, int64_t conv_out_stride, const float *h_in, int64_t h_in_stride,
     float *h_out, int64_t h_out_stride, const float *__restrict__ conv_weight, const float *__restrict__ conv_bias,
     const uint16_t *__restrict__ gate_weight_packed, const float *__restrict__ gate_bias,
     const float *__restrict__ log_lambda, float c, uint16_t *__restrict__ y, int64_t y_group_stride,
-    const uint8_t *__restrict__ reset, int rows_per_env, int64_t R)
+    const uint8_t *__restrict__ reset, int rows_per_env, int64_t R, int64_t full_rounds, int tail_rows_per_wave)
 {
     extern __shared__ __align__(16) unsigned char s_raw[];
     uint16_t *s_w = reinterpret_cast<uint16_t *>(s_raw);
-    uint16_t *s_tiles = s_w + kTsWeightHalfs;
-    float *s_conv_w = reinterpret_cast<float *>(s_tiles + kTsWaves * kTsTileHalfs);  // [d][k], as stored
+    float *s_conv_w = reinterpret_cast<float *>(s_w + kTsWeightHalfs);  // [d][k], as stored
     float *s_conv_b = s_conv_w + kTsD * 4;
     float *s_gate_b = s_conv_b + kTsD;  // [ba | bx], rounded to bf16 as autocast hands them to the GEMM
+    float *s_l2sig = s_gate_b + 2 * kTsD;
+    uint16_t *s_tiles = reinterpret_cast<uint16_t *>(s_l2sig + kTsD);
 
     const int tid = threadIdx.x;
-    for (int i = tid; i < kTsWeightHalfs / 8; i += kTsThreads)
+    const int threads = blockDim.x;
+    for (int i = tid; i < kTsWeightHalfs / 8; i += threads)
         reinterpret_cast<u32x4 *>(s_w)[i] = reinterpret_cast<const u32x4 *>(gate_weight_packed)[i];
-    for (int i = tid; i < kTsD * 4; i += kTsThreads) s_conv_w[i] = conv_weight[i];
-    for (int i = tid; i < kTsD; i += kTsThreads) s_conv_b[i] = conv_bias != nullptr ? conv_bias[i] : 0.0f;
-    for (int i = tid; i < 2 * kTsD; i += kTsThreads) s_gate_b[i] = round_to_bf16(gate_bias[i]);
+    for (int i = tid; i < kTsD * 4; i += threads) s_conv_w[i] = conv_weight[i];
+    for (int i = tid; i < kTsD; i += threads) s_conv_b[i] = conv_bias != nullptr ? conv_bias[i] : 0.0f;
+    for (int i = tid; i < 2 * kTsD; i += threads) s_gate_b[i] = round_to_bf16(gate_bias[i]);
+    for (int i = tid; i < kTsD; i += threads) s_l2sig[i] = log2_sigmoid(log_lambda[i]);
     __syncthreads();
 
     const int lane = tid & 63;
@@ -85,18 +91,33 @@ __global__ __launch_bounds__(kTsThreads) __attribute__((amdgpu_waves_per_eu(2, 2
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) l2s[hf][e] = log2_sigmoid(log_lambda[64 * hf + f8 + e]);
+        for (int e = 0; e < 8; ++e) l2s[hf][e] = s_l2sig[64 * hf + f8 + e];
 
-    const int64_t tiles = (R + kTsRows - 1) / kTsRows;
-    for (int64_t t = (int64_t)blockIdx.x * kTsWaves + wave; t < tiles; t += (int64_t)gridDim.x * kTsWaves) {
+    // Rounds of whole tiles are dealt to the waves of the grid in turn (at any time the grid works
+    // on one compact window of rows); what is left after the last whole round is split evenly
+    // between all waves in pieces of 8, 16 or 24 rows, so no wave has a whole tile more to do
+    // than another and a small input still spreads over the chip.
+    const int64_t grid_waves = (int64_t)gridDim.x * (threads >> 6);
+    const int64_t wave_global = (int64_t)blockIdx.x * (threads >> 6) + wave;
+    for (int64_t round = 0; round <= full_rounds; ++round) {
+        int64_t t0, t_end;
+        if (round < full_rounds) {
+            t0 = (round * grid_waves + wave_global) * kTsRows;
+            t_end = t0 + kTsRows;
+        } else {
+            t0 = full_rounds * grid_waves * kTsRows + wave_global * tail_rows_per_wave;
+            t_end = t0 + tail_rows_per_wave < R ? t0 + tail_rows_per_wave : R;
+            if (t0 >= t_end) break;
+        }
+        const int tile_rows = (int)(t_end - t0);  // wave-uniform
         // ---- the lane's four rows (rows past the end repeat the last row and store nothing) ----
         int64_t row[4], env[4];
         bool valid[4], zero[4];
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            const int64_t r = t * kTsRows + 8 * p + sub;
-            valid[p] = r < R;
-            row[p] = valid[p] ? r : R - 1;
+            const int64_t r = t0 + 8 * p + sub;
+            valid[p] = r < t_end;
+            row[p] = valid[p] ? r : t_end - 1;
             env[p] = (int64_t)((uint32_t)row[p] / (uint32_t)rows_per_env);  // R < 2^31, checked by the launcher
             zero[p] = reset != nullptr && reset[env[p]] != 0;
         }
@@ -116,6 +137,7 @@ __global__ __launch_bounds__(kTsThreads) __attribute__((amdgpu_waves_per_eu(2, 2
             // two rows at a time: all loads of the pair, then arithmetic and stores
 #pragma unroll
             for (int pg = 0; pg < 2; ++pg) {
+                if (16 * pg >= tile_rows) break;  // short tile: nothing in this pair of passes
                 Row8 p0[2], p1[2], p2[2], cur[2];
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
@@ -123,11 +145,11 @@ __global__ __launch_bounds__(kTsThreads) __attribute__((amdgpu_waves_per_eu(2, 2
                     const int64_t b1_off = b1_group_stride != 0
                                                ? env[p] * b1_group_stride + (row[p] - env[p] * rows_per_env) * b1_row_stride
                                                : row[p] * b1_row_stride;
-                    cur[i] = load8_stream(b1 + b1_off + d0);
+                    cur[i] = load8(b1 + b1_off + d0);
                     const float *pin = conv_in + row[p] * conv_in_stride + d0;
-                    p0[i] = load8_stream(pin);
-                    p1[i] = load8_stream(pin + kTsD);
-                    p2[i] = load8_stream(pin + 2 * kTsD);
+                    p0[i] = load8(pin);
+                    p1[i] = load8(pin + kTsD);
+                    p2[i] = load8(pin + 2 * kTsD);
                 }
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
@@ -147,9 +169,9 @@ __global__ __launch_bounds__(kTsThreads) __attribute__((amdgpu_waves_per_eu(2, 2
                     }
                     if (valid[p]) {
                         float *pout = conv_out + row[p] * conv_out_stride + d0;
-                        store8_stream(pout, p1[i]);
-                        store8_stream(pout + kTsD, p2[i]);
-                        store8_stream(pout + 2 * kTsD, cur[i]);
+                        store8(pout, p1[i]);
+                        store8(pout + kTsD, p2[i]);
+                        store8(pout + 2 * kTsD, cur[i]);
                     }
                     const float *vv = v[hf][p];
                     *reinterpret_cast<u32x4 *>(tile + (8 * p + sub) * kTsPitch + d0) =
@@ -173,7 +195,7 @@ __global__ __launch_bounds__(kTsThreads) __attribute__((amdgpu_waves_per_eu(2, 2
             // previous state of this half's channels: in flight while the matrix cores work
             Row8 hv[4];
 #pragma unroll
-            for (int p = 0; p < 4; ++p) hv[p] = load8_stream(h_in + row[p] * h_in_stride + d0);
+            for (int p = 0; p < 4; ++p) hv[p] = load8(h_in + row[p] * h_in_stride + d0);
 
             // ---- gate pre-activations of channels 64*hf .. +63: blocks q = 0,1 of Wa, 2,3 of Wx ----
             // A lane ends up with 16 consecutive channels per block: 32*(q%2) + 16*half + 0..15.
@@ -215,6 +237,7 @@ __global__ __launch_bounds__(kTsThreads) __attribute__((amdgpu_waves_per_eu(2, 2
             // ---- recurrence on the row mapping ----
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
+                if (8 * p >= tile_rows) break;
                 const uint16_t *gp = tile + (8 * p + sub) * kTsPitch + f8;
                 const Row8 ga = load8(gp);
                 const Row8 gx = load8(gp + 64);
@@ -224,11 +247,11 @@ __global__ __launch_bounds__(kTsThreads) __attribute__((amdgpu_waves_per_eu(2, 2
                     out.v[e] = rglru_element<true, false>(v[hf][p][e], ga.v[e], gx.v[e], l2s[hf][e], c,
                                                           zero[p] ? 0.0f : hv[p].v[e]);
                 if (valid[p]) {
-                    store8_stream(h_out + row[p] * h_out_stride + d0, out);
+                    store8(h_out + row[p] * h_out_stride + d0, out);
                     const int64_t y_off = y_group_stride != 0
                                               ? env[p] * y_group_stride + (row[p] - env[p] * rows_per_env) * kTsD
                                               : row[p] * kTsD;
-                    store8_stream(y + y_off + d0, out);
+                    store8(y + y_off + d0, out);
                 }
             }
             wave_lds_handover();
@@ -278,17 +301,23 @@ extern "C" int bnb_temporal_step_fwd(const void *b1, int64_t b1_group_stride, in
         (b1_group_stride % 8) != 0 || (y_group_stride % 8) != 0 || (conv_in_row_stride % 4) != 0 ||
         (conv_out_row_stride % 4) != 0 || (h_in_row_stride % 4) != 0 || (h_out_row_stride % 4) != 0)
         return BNB_ERR_MISALIGNED;
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(temporal_step_kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTsLdsBytes);
-    if (e != hipSuccess) return (int)e;
-    const int64_t tiles = (R + kTsRows - 1) / kTsRows;
-    int64_t blocks = (tiles + kTsWaves - 1) / kTsWaves;
+    // One work-group per CU at most (LDS), 8 waves each, every wave at least 8 rows.
     const int cus = ts_cu_count();
+    const int waves = kTsMaxWaves;
+    int64_t blocks = (R + (int64_t)waves * 8 - 1) / ((int64_t)waves * 8);
     if (blocks > cus) blocks = cus;
-    hipLaunchKernelGGL(temporal_step_kernel, dim3((unsigned)blocks), dim3(kTsThreads), kTsLdsBytes, (hipStream_t)stream,
+    const int64_t grid_waves = blocks * waves;
+    const int64_t full_rounds = R / (grid_waves * kTsRows);
+    const int64_t tail = R - full_rounds * grid_waves * kTsRows;
+    const int tail_rows_per_wave = (int)(((tail + grid_waves - 1) / grid_waves + 7) / 8 * 8);
+    const size_t lds = ts_lds_bytes(waves);
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(temporal_step_kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)ts_lds_bytes(kTsMaxWaves));
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(temporal_step_kernel, dim3((unsigned)blocks), dim3(waves * kWave), lds, (hipStream_t)stream,
                        (const uint16_t *)b1, b1_group_stride, b1_row_stride, conv_in, conv_in_row_stride, conv_out,
                        conv_out_row_stride, h_in, h_in_row_stride, h_out, h_out_row_stride, conv_weight, conv_bias,
                        (const uint16_t *)gate_weight_packed, gate_bias, log_lambda, c, (uint16_t *)y, y_group_stride,
-                       reset, rows_per_env, R);
+                       reset, rows_per_env, R, full_rounds, tail_rows_per_wave);
     return (int)hipGetLastError();
 }
