@@ -442,6 +442,36 @@ def main():
         "frac_of_hbm_peak": conv_bytes / t_conv / peak,
         "what": "read linear1 output + 3 stored inputs, write conv output + shifted inputs into the packed state",
     }
+    # ---- conv + gate projections + recurrence as one kernel, beside the three-kernel composition ----
+    if bf16:
+        gw_a = torch.randn(D, D, device=dev, generator=gen) / D ** 0.5
+        gw_x = torch.randn(D, D, device=dev, generator=gen) / D ** 0.5
+        g_bias = 0.3 * torch.randn(2 * D, device=dev, generator=gen)
+        g_pack = ops.pack_gate_weights(gw_a, gw_x)
+        g_w16, g_b16 = torch.cat([gw_a, gw_x]).to(torch.bfloat16), g_bias.to(torch.bfloat16)
+        y_ts = torch.empty(R, D, device=dev, dtype=torch.bfloat16)
+
+        def launch_fused(t):
+            src, dst = packed[t & 1], packed[(t + 1) & 1]
+            ops.temporal_step(b1_pool[t % POOL], src[:, D:].view(R, 3, D), src[:, :D], conv_w, conv_b, g_pack, g_bias, lam, 8.0,
+                              conv_out=dst[:, D:].view(R, 3, D), h_out=dst[:, :D], y_out=y_ts)
+
+        def launch_three(t):
+            src, dst = packed[t & 1], packed[(t + 1) & 1]
+            v, _, v16 = ops.conv_step(b1_pool[t % POOL], src[:, D:].view(R, 3, D), conv_w, conv_b,
+                                      conv_out=dst[:, D:].view(R, 3, D), also_bf16=True)
+            ops.rglru_step(v, F.linear(v16, g_w16, g_b16), lam, 8.0, src[:, :D], h_out=dst[:, :D], y_out=y_ts)
+
+        t_ts = timed_loop(launch_fused, steps, warmup) / steps
+        t_three = timed_loop(launch_three, steps, warmup) / steps
+        ts_bytes = R * (D * 2 + 2 * 3 * D * 4 + 2 * D * 4 + D * 2)
+        result["temporal_step_kernel"] = {
+            "rows": R, "avg_launch_us": t_ts * 1e6, "algorithmic_bytes_per_launch": ts_bytes, "achieved_GBps": ts_bytes / t_ts / 1e9,
+            "frac_of_hbm_peak": ts_bytes / t_ts / peak, "three_kernel_composition_us": t_three * 1e6,
+            "what": "conv taps + buffer shift, both gate projections (matrix cores) and the recurrence in one kernel: "
+                    "bf16 linear1 output, packed fp32 state in, packed fp32 state and bf16 layer output out; "
+                    "composition = conv kernel, library GEMM, recurrence kernel",
+        }
     del packed
 
     # ---- fused sublayer tail: add + RMSNorm + gated MLP + add on the matrix cores ----
