@@ -42,6 +42,7 @@ def parse_args():
     ap.add_argument("--no-ffn", action="store_true", help="skip the fused sublayer-tail leg")
     ap.add_argument("--no-bullets", action="store_true", help="skip the bullet-read leg")
     ap.add_argument("--no-sequence", action="store_true", help="skip the update-path (T = 128) recurrence leg")
+    ap.add_argument("--no-team-pool", action="store_true", help="skip the team pooling leg")
     ap.add_argument("--no-trunk", action="store_true", help="skip the whole-trunk leg (2 blocks x (2 spatial + 1 temporal))")
     return ap.parse_args()
 
@@ -564,6 +565,43 @@ def main():
                     "mask, Q, accumulator in and out; exp-throughput-bound rather than HBM-bound when many bullets are live",
         }
         del kv_b, b_mask, merged
+
+    # ---- team pooling over the ships (the value head's input), kernel beside the library composition ----
+    if not args.no_team_pool:
+        pma = bnb.TeamPMA(D, H).to(dev).eval()
+        with torch.no_grad():
+            pma.seeds.normal_(0.0, 0.02)
+        xs_t = torch.randn(w.B, w.NM, D, device=dev, generator=gen)
+        team_t = torch.randint(0, 2, (w.B, w.NM), device=dev, generator=gen, dtype=torch.int32)
+        alive_t = alive_steps[0]
+        ship_x, ship_team, ship_alive = xs_t[:, :w.N], team_t[:, :w.N], alive_t[:, :w.N]
+        n_p = max(4, min(steps, 16))
+        with torch.no_grad():
+            t_pool = timed_loop(lambda t: pma(ship_x, ship_team, ship_alive), n_p, 3) / n_p
+
+        def pool_library(t):
+            # the same function through the library: two attention calls with the seed as query
+            with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16, enabled=bf16):
+                team_pool = ship_x.new_zeros(w.B, 2, D)
+                for team in range(2):
+                    keys = (ship_team == team) & ship_alive
+                    o, _ = pma.attn(pma.seeds[team].view(1, 1, D).expand(w.B, 1, D), ship_x, ship_x,
+                                    key_padding_mask=~keys, need_weights=False)
+                    o = o.squeeze(1).nan_to_num(0.0) * keys.any(dim=1).unsqueeze(1).to(o.dtype)
+                    team_pool[:, team] = pma.norm(o)
+                return team_pool.gather(1, ship_team.clamp(0, 1).long().unsqueeze(-1).expand(w.B, w.N, D))
+
+        t_pool_lib = None if args.no_torch_baseline else timed_loop(pool_library, n_p, 3) / n_p
+        pool_bytes = w.B * w.N * (D * 4 + 4 + 1 + D * 4)
+        result["team_pool_kernel"] = {
+            "environments": w.B, "ships": w.N, "avg_launch_us": t_pool * 1e6, "algorithmic_bytes_per_launch": pool_bytes,
+            "achieved_GBps": pool_bytes / t_pool / 1e9, "frac_of_hbm_peak": pool_bytes / t_pool / peak,
+            "eager_torch_us": None if t_pool_lib is None else t_pool_lib * 1e6,
+            "what": "per-team attention pooling with a learned seed as the only query, out projection, RMSNorm and the "
+                    "broadcast back to the ships in one fp32 kernel: ship rows read once, (B, N, D) written once; eager = "
+                    "two nn.MultiheadAttention calls, norm and gather in torch ops (bf16 autocast on bf16 workloads)",
+        }
+        del xs_t
 
     # ---- update path: the recurrence over a stored rollout (T = 128), forward and backward ----
     if not args.no_sequence:

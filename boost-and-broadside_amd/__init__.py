@@ -5,8 +5,9 @@ per-entity RG-LRU recurrence step, as hand-written HIP kernels behind a C ABI
 (``include/bnb_amd.h`` -> ``_lib/libbnb_amd.so``), plus torch modules that keep the
 reference policy's layer interfaces and ``state_dict`` names.
 
-    ops       sdpa_masked, sdpa_cross, rglru_step, conv_step, rglru_scan, conv_seq, add_rmsnorm, gelu_mul
-    trunk     TransformerBlock, RGLRU, GriffinTemporalBlock, YemongBlock, YemongTrunk, GraphedTrunk
+    ops       sdpa_masked, sdpa_cross, rglru_step, conv_step, temporal_step, rglru_scan, conv_seq, add_rmsnorm,
+              gelu_mul, norm_linear, ffn_fused, team_pool
+    trunk     TransformerBlock, RGLRU, GriffinTemporalBlock, YemongBlock, YemongTrunk, GraphedTrunk, TeamPMA
     harness   benchmark workloads, traffic model, AttnRglruStep
     build     compiles the HIP sources
 """
@@ -20,13 +21,14 @@ from .trunk import (
     GriffinTemporalBlock,
     ModelConfig,
     RGLRU,
+    TeamPMA,
     TransformerBlock,
     YemongBlock,
     YemongTrunk,
 )
 
 __all__ = [
-    "CONV_KERNEL", "GatedMLP", "GraphedTrunk", "GriffinTemporalBlock", "ModelConfig", "RGLRU", "TransformerBlock",
+    "CONV_KERNEL", "GatedMLP", "GraphedTrunk", "GriffinTemporalBlock", "ModelConfig", "RGLRU", "TeamPMA", "TransformerBlock",
     "YemongBlock", "YemongTrunk", "conv_seq", "conv_step", "rglru_scan", "rglru_step", "sdpa_cross", "sdpa_masked", "ops",
     "trunk", "harness",
 ]

@@ -11,6 +11,8 @@ synchronise.  They are forward-only and run on a ROCm device only: anything else
 
 from __future__ import annotations
 
+import math
+
 import torch
 
 from . import _native
@@ -368,6 +370,101 @@ def conv_step(
             )
         _native.check(rc, "bnb_conv_step_fwd")
     return (v, conv_out, v_lp) if also_bf16 else (v, conv_out)
+
+
+def pack_team_pool_weights(seeds: torch.Tensor, in_proj_weight: torch.Tensor, out_proj_weight: torch.Tensor,
+                           n_heads: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """The constants ``team_pool`` needs, from TeamPMA's parameters (policy.py:88-92), float32:
+    the 2H score vectors ``W_k[hs]^T (W_q seeds[t])[hs] * log2(e) / sqrt(dh)`` (row ``t*H + h``) and
+    the (H*D, D) matrix whose rows ``h*D..`` are ``(out_proj.weight[:, hs] W_v[hs, :])^T``."""
+    D = seeds.shape[-1]
+    if seeds.shape != (2, D) or in_proj_weight.shape != (3 * D, D) or out_proj_weight.shape != (D, D) or D % n_heads:
+        raise ValueError("expected seeds (2, D), in_proj_weight (3D, D), out_proj_weight (D, D), D divisible by n_heads")
+    dh = D // n_heads
+    with torch.no_grad(), torch.autocast(seeds.device.type, enabled=False):  # these constants stay float32
+        w = in_proj_weight.detach().float()
+        wq, wk, wv = w[:D], w[D:2 * D], w[2 * D:]
+        q = (seeds.detach().float() @ wq.t()).view(2, n_heads, dh)                 # (t, h, dh)
+        u = torch.einsum("thd,hdc->thc", q, wk.view(n_heads, dh, D)) * (math.log2(math.e) / math.sqrt(dh))
+        wo = out_proj_weight.detach().float().view(D, n_heads, dh)                   # (o, h, dh)
+        m = torch.einsum("ohd,hdc->hco", wo, wv.view(n_heads, dh, D))                # (h, c, o) = (W_o[:, hs] W_v[hs, :])^T
+        return u.reshape(2 * n_heads, D).contiguous(), m.reshape(n_heads * D, D).contiguous()
+
+
+def team_pool_supported(x: torch.Tensor, n_heads: int) -> bool:
+    """Whether ``team_pool`` covers this input: float32 rows of 128 channels on the GPU, 2 or 4 heads."""
+    return x.is_cuda and x.dtype == torch.float32 and x.dim() == 3 and x.shape[-1] == FFN_WIDTH and n_heads in (2, 4)
+
+
+def team_pool(x: torch.Tensor, team_id: torch.Tensor, alive: torch.Tensor, score_vectors: torch.Tensor,
+              folded_projection: torch.Tensor, norm_weight: torch.Tensor, eps: float | None, n_heads: int, *,
+              broadcast: bool = True):
+    """Per-team attention pooling of the ship rows (TeamPMA.forward, policy.py:94-120): a kernel
+    that reads the ships once and leaves the weighted mean row per (team, head), one float32
+    library GEMM with the folded value/output projection, a kernel for RMSNorm and the hand-out.
+
+    Args:
+        x:        (B, N, 128) float32 ship rows; a ``tokens[:, :N]`` view of a wider tensor works.
+        team_id:  (B, N) integer team of every ship (0 / 1; anything else is nobody's key and
+                  reads team ``clamp(id, 0, 1)``'s vector).
+        alive:    (B, N) bool.
+        score_vectors, folded_projection: from ``pack_team_pool_weights``.
+        norm_weight: (128,) float32 RMSNorm weight; ``eps`` None means float32 machine epsilon.
+        broadcast: also return the (B, N, 128) tensor in which every ship holds its team's vector.
+
+    Returns:
+        (ships or None, pool): ``pool`` is (B, 2, 128), zero for a team without an alive ship.
+    """
+    if x.dim() != 3 or x.shape[-1] != FFN_WIDTH or x.dtype != torch.float32:
+        raise ValueError("x must be float32 (B, N, 128)")
+    B, N, D = x.shape
+    if team_id.shape != (B, N) or alive.shape != (B, N):
+        raise ValueError(f"team_id and alive must be {(B, N)}")
+    if alive.dtype not in (torch.bool, torch.uint8):
+        raise TypeError("alive must be bool")
+    if score_vectors.shape != (2 * n_heads, D) or folded_projection.shape != (n_heads * D, D):
+        raise ValueError("score_vectors / folded_projection must come from pack_team_pool_weights")
+    for name, t in (("x", x), ("team_id", team_id), ("alive", alive), ("score_vectors", score_vectors),
+                    ("folded_projection", folded_projection), ("norm_weight", norm_weight)):
+        _need_device(t, name)
+    for name, t in (("score_vectors", score_vectors), ("folded_projection", folded_projection), ("norm_weight", norm_weight)):
+        if t.dtype != torch.float32:
+            raise TypeError(f"{name} must be float32")
+    if torch.is_grad_enabled() and x.requires_grad:
+        raise RuntimeError("team_pool is forward-only; call it under torch.no_grad()")
+    if N and (x.stride(2) != 1 or x.stride(1) % 4 or (B > 1 and x.stride(0) % 4)):
+        x = x.contiguous()
+    if team_id.dtype != torch.int32 or (N and team_id.stride(1) != 1):
+        team_id = team_id.to(torch.int32).contiguous()
+    if N and alive.stride(1) != 1:
+        alive = alive.contiguous()
+    dev = x.device
+    pool = torch.empty((B, 2, D), dtype=torch.float32, device=dev)
+    ships = torch.empty((B, N, D), dtype=torch.float32, device=dev) if broadcast else None
+    if eps is None:
+        eps = torch.finfo(torch.float32).eps
+    if B:
+        def env_stride(t):
+            return t.stride(0) if B > 1 else t.shape[1] * (t.stride(1) if N else 1)
+
+        z = torch.empty((B * 2, n_heads * D), dtype=torch.float32, device=dev)
+        lib = _native.load()
+        with torch.cuda.device(dev):
+            rc = lib.bnb_team_attend_fwd(
+                x.data_ptr(), env_stride(x), x.stride(1) if N else D, team_id.data_ptr(), env_stride(team_id) if N else 0,
+                alive.data_ptr(), env_stride(alive) if N else 0, score_vectors.contiguous().data_ptr(), z.data_ptr(),
+                B, N, int(n_heads), D, _stream(),
+            )
+            _native.check(rc, "bnb_team_attend_fwd")
+            with torch.autocast("cuda", enabled=False):
+                pre = torch.mm(z, folded_projection)
+            rc = lib.bnb_team_norm_broadcast_fwd(
+                pre.data_ptr(), norm_weight.detach().contiguous().data_ptr(), float(eps), team_id.data_ptr(),
+                env_stride(team_id) if N else 0, pool.data_ptr(), None if ships is None else ships.data_ptr(), N * D, D,
+                B, N, D, _stream(),
+            )
+            _native.check(rc, "bnb_team_norm_broadcast_fwd")
+    return ships, pool
 
 
 def pack_gate_weights(weight_a: torch.Tensor, weight_x: torch.Tensor) -> torch.Tensor:

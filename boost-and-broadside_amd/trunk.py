@@ -9,6 +9,7 @@ Every class keeps the constructor arguments, method signatures, tensor layouts a
     RGLRU                   models/yemong/griffin.py:143-219
     GriffinTemporalBlock    models/yemong/griffin.py:222-317
     YemongBlock             models/yemong/griffin.py:320-472
+    TeamPMA                 models/yemong/policy.py:78-120
     ModelConfig             config/core.py:213-275
     YemongTrunk             the block loop and hidden-state handling of
                             models/yemong/policy.py:234-254, 268-285, 311-354
@@ -556,6 +557,57 @@ def _conv_within_episodes(padded, w, bias, done_mask):
         same = (episode[:, k:k + T] == here).to(padded.dtype).unsqueeze(-1)
         out = out + padded[:, k:k + T] * w[:, k] * same
     return out + bias
+
+
+class TeamPMA(nn.Module):
+    """Pooling by multi-head attention over each team's alive ships (policy.py:78-120).
+
+    Parameters and ``state_dict`` keys as in the reference: ``seeds`` (2, D), ``attn``
+    (``nn.MultiheadAttention``, bias-free, only its weights are used) and ``norm``.  ``forward``
+    returns (B, N, D): every ship holds the pooled, normalised vector of team
+    ``clamp(team_id, 0, 1)``; a team without an alive ship pools to zero.
+
+    Float32 rows of width 128 on the GPU without gradients run as one kernel (``ops.team_pool``),
+    which reads ``x`` once and never projects the ships to keys and values.  Everything else
+    (training, other widths) is one library attention call with both seeds as queries.
+    """
+
+    def __init__(self, d_model: int, n_heads: int) -> None:
+        super().__init__()
+        self.n_heads = n_heads
+        self.seeds = nn.Parameter(torch.zeros(2, d_model))
+        self.attn = nn.MultiheadAttention(d_model, n_heads, batch_first=True, bias=False)
+        self.norm = nn.RMSNorm(d_model)
+
+    def _folded(self):
+        srcs = (self.seeds, self.attn.in_proj_weight, self.attn.out_proj.weight)
+        return _cached_cast(self, "_bnb_pool_pack", srcs, torch.float32,
+                            lambda: ops.pack_team_pool_weights(*srcs, self.n_heads))
+
+    def pooled(self, x: torch.Tensor, team_id: torch.Tensor, alive: torch.Tensor) -> torch.Tensor:
+        """(B, 2, D) pooled team vectors without the broadcast back to the ships."""
+        if not torch.is_grad_enabled() and ops.team_pool_supported(x, self.n_heads):
+            return ops.team_pool(x, team_id, alive, *self._folded(), self.norm.weight, self.norm.eps, self.n_heads,
+                                 broadcast=False)[1]
+        return self._pooled_library(x, team_id, alive)
+
+    def _pooled_library(self, x, team_id, alive):
+        B, N, D = x.shape
+        keys = torch.stack([(team_id == 0) & alive, (team_id == 1) & alive], dim=1)  # (B, 2, N)
+        has_ship = keys.any(dim=-1, keepdim=True)
+        # a team without a ship may look at every row (keeps the softmax finite); its result is gated off
+        blocked = ~keys & has_ship
+        out, _ = self.attn(self.seeds.unsqueeze(0).expand(B, 2, D), x, x,
+                           attn_mask=blocked.repeat_interleave(self.n_heads, dim=0), need_weights=False)
+        out = out * has_ship.to(out.dtype)
+        return self.norm(out).to(x.dtype)
+
+    def forward(self, x: torch.Tensor, team_id: torch.Tensor, alive: torch.Tensor) -> torch.Tensor:
+        if not torch.is_grad_enabled() and ops.team_pool_supported(x, self.n_heads):
+            return ops.team_pool(x, team_id, alive, *self._folded(), self.norm.weight, self.norm.eps, self.n_heads)[0]
+        B, N, D = x.shape
+        pool = self._pooled_library(x, team_id, alive)
+        return pool.gather(1, team_id.clamp(0, 1).long().unsqueeze(-1).expand(B, N, D))
 
 
 class YemongBlock(nn.Module):

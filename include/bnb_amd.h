@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 13
+#define BNB_ABI_VERSION 14
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -237,6 +237,45 @@ int bnb_conv_step_rows_fwd(const void *b1, int b1_dtype, int64_t b1_group_stride
                            const uint8_t *reset, int rows_per_env,
                            float *v_out, void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride,
                            int64_t R, int D, void *stream);
+
+/*
+ * Pooling by multi-head attention over each team's alive ships, broadcast back to the ships:
+ * two kernels with one plain fp32 GEMM of the caller's between them.
+ *
+ * Together they replace TeamPMA.forward, models/yemong/policy.py:94-120: the two
+ * nn.MultiheadAttention calls with a learned seed as the only query (keys = alive ships of
+ * team t), nan_to_num, the has_ship gate, RMSNorm, and the gather that hands every ship the
+ * vector of team clamp(team_id, 0, 1).  The seed being a constant of the model, the caller folds
+ * the weights once per weight update (attn.in_proj_weight = [W_q; W_k; W_v], heads = slices hs):
+ *
+ *   score_vectors (2H, D) fp32: row t*H + h = W_k[hs, :]^T (W_q seeds[t])[hs] * log2(e) / sqrt(dh)
+ *   M             (H*D, D) fp32: rows h*D .. (h+1)*D = (attn.out_proj.weight[:, hs] W_v[hs, :])^T
+ *
+ * bnb_team_attend_fwd: z[b, t, h, :] = sum_j softmax_j(x[b, j] . score_vectors[t*H + h]) x[b, j]
+ * over the alive ships j of team t (all zero when there is none).
+ *   x        (B, N, D) fp32 ship rows: x[b, n] at b*x_env_stride + n*x_row_stride (a [:, :N]
+ *            view of the (B, N+M, D) trunk output works)
+ *   team_id  (B, N) int32, row b at b*team_env_stride; alive (B, N) bytes, likewise
+ *   z        (B, 2, H, D) fp32 contiguous
+ * The caller then forms pre = z.view(B*2, H*D) @ M (library GEMM, fp32).
+ *
+ * bnb_team_norm_broadcast_fwd: pool = RMSNorm(pre) (a zero row stays zero), out[b, n] =
+ * pool[b, clamp(team_id[b, n], 0, 1)].
+ *   pre      (B, 2, D) fp32 contiguous; norm_weight (D) fp32, eps
+ *   pool     (B, 2, D) fp32 or NULL; out (B, N, D) fp32 at b*out_env_stride + n*out_row_stride,
+ *            or NULL (then team_id may be NULL too)
+ *
+ * Requirements: D == 128, H in {2, 4}, 16-byte aligned x / out, strides multiples of 4 elements.
+ */
+int bnb_team_attend_fwd(const float *x, int64_t x_env_stride, int64_t x_row_stride,
+                        const int32_t *team_id, int64_t team_env_stride,
+                        const uint8_t *alive, int64_t alive_env_stride,
+                        const float *score_vectors, float *z,
+                        int B, int N, int H, int D, void *stream);
+int bnb_team_norm_broadcast_fwd(const float *pre, const float *norm_weight, float eps,
+                                const int32_t *team_id, int64_t team_env_stride,
+                                float *pool, float *out, int64_t out_env_stride, int64_t out_row_stride,
+                                int B, int N, int D, void *stream);
 
 /*
  * One timestep of the temporal sublayer's state path in one launch: conv taps + buffer shift

@@ -162,3 +162,38 @@ def ffn_tail_loops(x, delta, norm_w, gate_w, up_w, down_w, eps) -> np.ndarray:
             hidden[j] = 0.5 * g * (1.0 + math.erf(g / math.sqrt(2.0))) * float(np.dot(uw[j], n))
         out[r] = s[r] + dw @ hidden
     return out
+
+
+def team_pool_loops(x, team_id, alive, seeds, in_proj_weight, out_proj_weight, norm_weight, n_heads, eps) -> np.ndarray:
+    """Per team t in {0, 1}: softmax over the alive ships j of team t of (W_q seed_t)_h . (W_k x_j)_h / sqrt(dh),
+    weighted sum of (W_v x_j)_h, heads concatenated, W_o, RMSNorm; no such ship: zeros.  Returns the
+    pooled vectors (B, 2, D).
+
+    Definition being restated: models/yemong/policy.py:104-116 with torch's multi-head attention
+    (packed in-projection [W_q; W_k; W_v], heads = consecutive slices of the projected vectors).
+    """
+    x = np.asarray(x, dtype=np.float64)
+    B, N, D = x.shape
+    dh = D // n_heads
+    w_in = np.asarray(in_proj_weight, dtype=np.float64)
+    wq, wk, wv = w_in[:D], w_in[D:2 * D], w_in[2 * D:]
+    wo = np.asarray(out_proj_weight, dtype=np.float64)
+    pool = np.zeros((B, 2, D), dtype=np.float64)
+    for b in range(B):
+        for t in range(2):
+            keys = [j for j in range(N) if int(team_id[b, j]) == t and bool(alive[b, j])]
+            if not keys:
+                continue
+            q = wq @ np.asarray(seeds[t], dtype=np.float64)
+            merged = np.zeros(D)
+            for hd in range(n_heads):
+                lo, hi = hd * dh, (hd + 1) * dh
+                scores = [float(np.dot(q[lo:hi], (wk @ x[b, j])[lo:hi])) / math.sqrt(dh) for j in keys]
+                m = max(scores)
+                w = [math.exp(sc - m) for sc in scores]
+                z = sum(w)
+                for wj, j in zip(w, keys):
+                    merged[lo:hi] += (wj / z) * (wv @ x[b, j])[lo:hi]
+            out = wo @ merged
+            pool[b, t] = out / math.sqrt(float(np.mean(out * out)) + eps) * np.asarray(norm_weight, dtype=np.float64)
+    return pool

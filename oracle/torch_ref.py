@@ -26,6 +26,10 @@ How each function is pinned (see tests/test_oracle_pins.py):
                        zero history (with boundaries).
 * ``rglru_sequence``   the log-depth scan == a plain loop of the pinned ``rglru_step`` with
                        the state zeroed after each episode end; fp64 agreement to 1e-12.
+* ``team_pool``        library ``nn.MultiheadAttention`` + ``nn.RMSNorm`` composed as the
+                       reference's forward does + fp64 brute force + closed forms (one
+                       ship alive => that ship's projected row, empty team => zeros,
+                       other-team / dead perturbation invariance).
 * ``temporal_step``    step == sequence, with the sequence path built on the
                        library ``F.conv1d`` (fixes tap order and buffer order).
 * ``field_step``, ``block_step``, ``pack/unpack/reset``  invariants the
@@ -404,6 +408,38 @@ def harness_step(p: dict, tokens: torch.Tensor, alive: torch.Tensor, state: torc
     h_new = rglru_step(ships, rglru_gates(p, "", ships), p["log_lambda"], 8.0, state)
     y = h_new.to(u.dtype).reshape(B, N, D)
     return torch.cat([y, u[:, N:]], dim=1), h_new
+
+
+def team_pool(p: dict, prefix: str, x: torch.Tensor, team_id: torch.Tensor, alive: torch.Tensor, n_heads: int):
+    """Pooling by multi-head attention per team, broadcast back to the ships.
+
+    Follows models/yemong/policy.py:78-120: for team t in {0, 1} the learned seed ``seeds[t]`` is
+    the single query of a bias-free multi-head attention whose keys and values are the ship
+    rows ``x``, keys restricted to the alive ships of team t; a team without such a ship pools
+    to zero; the pooled vector goes through RMSNorm; every ship receives the pooled vector of
+    team ``clamp(team_id, 0, 1)``.  Weights: ``{prefix}seeds`` (2, D), ``{prefix}attn.in_proj_weight``
+    (3D, D) = [W_q; W_k; W_v], ``{prefix}attn.out_proj.weight`` (D, D), ``{prefix}norm.weight`` (D).
+    Returns (ships (B, N, D), pool (B, 2, D)).
+    """
+    B, N, D = x.shape
+    dh = D // n_heads
+    w_in = p[prefix + "attn.in_proj_weight"]
+    wq, wk, wv = w_in[:D], w_in[D:2 * D], w_in[2 * D:]
+    k = F.linear(x, wk).view(B, N, n_heads, dh)
+    v = F.linear(x, wv).view(B, N, n_heads, dh)
+    pool = x.new_zeros(B, 2, D)
+    for t in range(2):
+        keys = (team_id == t) & alive  # (B, N)
+        q = F.linear(p[prefix + "seeds"][t], wq).view(n_heads, dh)
+        scores = torch.einsum("hd,bnhd->bhn", q, k) / math.sqrt(dh)
+        scores = scores.masked_fill(~keys[:, None, :], float("-inf"))
+        weights = torch.softmax(scores, dim=-1).nan_to_num(0.0)  # no key at all: nothing is pooled
+        merged = torch.einsum("bhn,bnhd->bhd", weights, v).reshape(B, D)
+        out = F.linear(merged, p[prefix + "attn.out_proj.weight"])
+        out = out * keys.any(dim=1, keepdim=True).to(out.dtype)
+        pool[:, t] = rms_norm(out, p[prefix + "norm.weight"])
+    idx = team_id.clamp(0, 1).long().unsqueeze(-1).expand(B, N, D)
+    return pool.gather(1, idx), pool
 
 
 def sigma_lambda_reference(d_model: int) -> torch.Tensor:

@@ -1,5 +1,5 @@
-"""Writes tests/golden/step_vectors.npz and widened_vectors.npz: small seeded inputs and their
-expected outputs.
+"""Writes tests/golden/step_vectors.npz, widened_vectors.npz and team_pool_vectors.npz: small seeded
+inputs and their expected outputs.
 
 The reference keeps no stored numeric vectors for this path (its tests are property tests and
 its one golden file needs weights that are not in the checkout), and the reference was not
@@ -49,6 +49,7 @@ def main() -> None:
     np.savez_compressed(os.path.join(HERE, "step_vectors.npz"), **out)
     print("wrote", os.path.join(HERE, "step_vectors.npz"), {k: v.shape for k, v in out.items()})
     widened()
+    team_pool()
 
 
 def widened() -> None:
@@ -109,6 +110,31 @@ def widened() -> None:
                                                float(np.finfo(np.float32).eps))
     np.savez_compressed(os.path.join(HERE, "widened_vectors.npz"), **out)
     print("wrote", os.path.join(HERE, "widened_vectors.npz"), {k: v.shape for k, v in out.items()})
+
+
+def team_pool() -> None:
+    """tests/golden/team_pool_vectors.npz: per-team attention pooling (policy.py:78-120)."""
+    rng = np.random.default_rng(20240603)
+    B, N, D, H = 4, 9, 128, 4
+    out = {
+        "x": rng.standard_normal((B, N, D)).astype(np.float32),
+        "team_id": rng.integers(0, 2, (B, N)).astype(np.int32),
+        "alive": rng.random((B, N)) < 0.7,
+        "seeds": (0.5 * rng.standard_normal((2, D))).astype(np.float32),
+        "in_proj_weight": (rng.standard_normal((3 * D, D)) * np.sqrt(2.0 / D)).astype(np.float32),
+        "out_proj_weight": (rng.standard_normal((D, D)) / np.sqrt(D)).astype(np.float32),
+        "norm_weight": (1.0 + 0.1 * rng.standard_normal(D)).astype(np.float32),
+        "heads": np.int64(H),
+    }
+    out["team_id"][0] = 0       # nobody on team 1
+    out["alive"][1] = False     # everybody dead
+    out["alive"][2] = False
+    out["alive"][2, 4] = True   # a single ship alive
+    out["team_id"][3, 0] = 2    # a field id among the ships: nobody's key, reads team 1's vector
+    out["pool"] = bruteforce.team_pool_loops(out["x"], out["team_id"], out["alive"], out["seeds"], out["in_proj_weight"],
+                                             out["out_proj_weight"], out["norm_weight"], H, float(np.finfo(np.float32).eps))
+    np.savez_compressed(os.path.join(HERE, "team_pool_vectors.npz"), **out)
+    print("wrote", os.path.join(HERE, "team_pool_vectors.npz"), {k: v.shape for k, v in out.items()})
 
 
 if __name__ == "__main__":

@@ -81,3 +81,31 @@ def max_rel(y: torch.Tensor, ref: torch.Tensor) -> float:
     """max|y - ref| / max|ref| over the whole tensor (the parity metric of the step)."""
     y, ref = y.double(), ref.double()
     return float((y - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+
+
+def team_pool_params(gen: torch.Generator, prefix: str, D: int) -> dict:
+    """Weights of the team pooling layer (names: models/yemong/policy.py:88-92; scales as initialised at :218-220)."""
+    return {
+        prefix + "seeds": 0.5 * torch.randn(2, D, generator=gen),
+        prefix + "attn.in_proj_weight": torch.randn(3 * D, D, generator=gen) * math.sqrt(2.0 / D),
+        prefix + "attn.out_proj.weight": torch.randn(D, D, generator=gen) / math.sqrt(D),
+        prefix + "norm.weight": 1.0 + 0.1 * torch.randn(D, generator=gen),
+    }
+
+
+def team_case(seed: int, B: int, N: int, p_alive: float = 0.7):
+    """Seeded (team_id int32, alive bool) with the edge cases in the first environments: one team
+    absent, everybody dead, everybody alive, a single ship alive."""
+    g = torch.Generator().manual_seed(seed)
+    team = torch.randint(0, 2, (B, N), generator=g, dtype=torch.int32)
+    alive = torch.rand(B, N, generator=g) < p_alive
+    if B > 0 and N > 0:
+        team[0] = 0
+    if B > 1:
+        alive[1] = False
+    if B > 2:
+        alive[2] = True
+    if B > 3 and N > 0:
+        alive[3] = False
+        alive[3, N - 1] = True
+    return team, alive

@@ -135,3 +135,38 @@ def test_kernels_reproduce_sublayer_tail_vectors():
     got = ops.ffn_fused(torch.from_numpy(WIDE["ffn_x"]).cuda(), _from_bits("ffn_delta_bf16").bfloat16().cuda(),
                         torch.from_numpy(WIDE["ffn_norm_w"]).cuda(), pk).cpu()
     assert max_rel(got, torch.from_numpy(WIDE["ffn_out"])) <= 2e-2
+
+
+# ---------------------------------------------------------------- team pooling
+
+TEAM = np.load(os.path.join(ROOT, "tests", "golden", "team_pool_vectors.npz"))
+
+
+def _team_inputs():
+    p = {"tp.seeds": TEAM["seeds"], "tp.attn.in_proj_weight": TEAM["in_proj_weight"],
+         "tp.attn.out_proj.weight": TEAM["out_proj_weight"], "tp.norm.weight": TEAM["norm_weight"]}
+    p = {k: torch.from_numpy(v) for k, v in p.items()}
+    return p, torch.from_numpy(TEAM["x"]), torch.from_numpy(TEAM["team_id"]), torch.from_numpy(TEAM["alive"]), int(TEAM["heads"])
+
+
+def test_oracle_reproduces_team_pool_vectors():
+    p, x, team, alive, H = _team_inputs()
+    ships, pool = torch_ref.team_pool(p, "tp.", x, team, alive, H)
+    want = TEAM["pool"]
+    assert np.abs(pool.double().numpy() - want).max() <= 2e-5
+    assert np.abs(want[0, 1]).max() == 0 and np.abs(want[1]).max() == 0  # empty teams
+    assert torch.equal(ships[3, 0], pool[3, 1])  # the field id reads team 1's vector
+
+
+@pytest.mark.gpu
+def test_kernels_reproduce_team_pool_vectors():
+    from boost_and_broadside_amd import ops
+
+    p, x, team, alive, H = _team_inputs()
+    consts = ops.pack_team_pool_weights(p["tp.seeds"].cuda(), p["tp.attn.in_proj_weight"].cuda(),
+                                        p["tp.attn.out_proj.weight"].cuda(), H)
+    ships, pool = ops.team_pool(x.cuda(), team.cuda(), alive.cuda(), *consts, p["tp.norm.weight"].cuda(), None, H)
+    want = torch.from_numpy(TEAM["pool"]).float()
+    assert max_rel(pool.cpu(), want) <= 1e-5
+    assert torch.equal(pool.cpu() == 0, want == 0)
+    assert torch.equal(ships[3, 0], pool[3, 1])

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import max_rel
+from helpers import max_rel, team_case, team_pool_params
 from oracle import c_ref, torch_ref
 
 from boost_and_broadside_amd import harness, ops
@@ -1145,3 +1145,91 @@ def test_column_block_operands_are_read_in_place():
     in_place = ops.ffn_fused(xd, None, nw.to(DEV), pk, proj=(gate, y, wp))
     copied = ops.ffn_fused(xd, None, nw.to(DEV), pk, proj=(gate.contiguous(), y, wp))
     assert torch.equal(in_place, copied)
+
+
+# ------------------------------------------------------------------ team pooling
+
+
+def _team_pool_run(p, x, team, alive, H, broadcast=True):
+    consts = ops.pack_team_pool_weights(p["tp.seeds"].to(DEV), p["tp.attn.in_proj_weight"].to(DEV),
+                                        p["tp.attn.out_proj.weight"].to(DEV), H)
+    ships, pool = ops.team_pool(x.to(DEV), team.to(DEV), alive.to(DEV), *consts, p["tp.norm.weight"].to(DEV), None, H,
+                                broadcast=broadcast)
+    torch.cuda.synchronize()
+    return (None if ships is None else ships.cpu()), pool.cpu()
+
+
+@pytest.mark.parametrize("B,N", [(1, 1), (5, 8), (6, 19), (9, 64), (7, 65), (4, 152), (3, 320), (1030, 8)])
+@pytest.mark.parametrize("H", [4, 2])
+def test_team_pool_matches_oracle(B, N, H):
+    D = 128
+    g = torch.Generator().manual_seed(B * 7 + N)
+    p = team_pool_params(g, "tp.", D)
+    x = torch.randn(B, N, D, generator=g)
+    team, alive = team_case(B + N, B, N)
+    ships, pool = _team_pool_run(p, x, team, alive, H)
+    ref_ships, ref_pool = torch_ref.team_pool(p, "tp.", x, team, alive, H)
+    assert max_rel(pool, ref_pool) <= F32_TOL
+    assert torch.allclose(pool, ref_pool, rtol=1e-4, atol=2e-5)
+    # which teams are empty is reproduced exactly, and every ship carries its team's vector bit for bit
+    assert torch.equal(pool == 0, ref_pool == 0)
+    idx = team.clamp(0, 1).long().unsqueeze(-1).expand(B, N, D)
+    assert torch.equal(ships, pool.gather(1, idx))
+    if B * N <= 200:  # loop-only fp64 statement as a second witness
+        from oracle import bruteforce
+        loops = bruteforce.team_pool_loops(x.numpy(), team.numpy(), alive.numpy(), p["tp.seeds"].numpy(),
+                                           p["tp.attn.in_proj_weight"].numpy(), p["tp.attn.out_proj.weight"].numpy(),
+                                           p["tp.norm.weight"].numpy(), H, float(torch.finfo(torch.float32).eps))
+        assert max_rel(pool, torch.from_numpy(loops).float()) <= F32_TOL
+
+
+def test_team_pool_large_scores_and_masking_invariances():
+    B, N, D, H = 6, 40, 128, 4
+    g = torch.Generator().manual_seed(11)
+    p = team_pool_params(g, "tp.", D)
+    p["tp.seeds"] = 6.0 * torch.randn(2, D, generator=g)  # scores of magnitude ~50: the running maximum matters
+    x = 2.0 * torch.randn(B, N, D, generator=g)
+    team, alive = team_case(12, B, N)
+    _, pool = _team_pool_run(p, x, team, alive, H, broadcast=False)
+    _, ref = torch_ref.team_pool(p, "tp.", x, team, alive, H)
+    assert max_rel(pool, ref) <= F32_TOL
+    # dead ships are nobody's keys: rewriting their rows changes no bit
+    pert = x.clone()
+    pert[~alive] = pert[~alive] * -3.0 + 5.0
+    assert torch.equal(_team_pool_run(p, pert, team, alive, H, broadcast=False)[1], pool)
+    # team 0's vector does not depend on team 1's ships
+    pert = x.clone()
+    pert[team == 1] += 1.0
+    again = _team_pool_run(p, pert, team, alive, H, broadcast=False)[1]
+    assert torch.equal(again[:, 0], pool[:, 0]) and not torch.equal(again[:, 1], pool[:, 1])
+    # an id outside {0, 1} is no key and reads team 1's vector
+    odd = team.clone()
+    odd[2, 0] = 2
+    ships, pool_odd = _team_pool_run(p, x, odd, alive, H)
+    assert torch.equal(ships[2, 0], pool_odd[2, 1])
+    stay = alive.clone()
+    stay[2, 0] = False
+    assert torch.equal(_team_pool_run(p, x, team, stay, H, broadcast=False)[1][2], pool_odd[2])
+
+
+def test_team_pool_reads_ship_rows_inside_the_token_tensor_and_other_id_types():
+    B, N, M, D, H = 9, 8, 4, 128, 4
+    g = torch.Generator().manual_seed(13)
+    p = team_pool_params(g, "tp.", D)
+    tokens = torch.randn(B, N + M, D, generator=g).to(DEV)
+    team_all = torch.full((B, N + M), 2, dtype=torch.int32)
+    alive_all = torch.ones(B, N + M, dtype=torch.bool)
+    team_all[:, :N], alive_all[:, :N] = team_case(14, B, N)
+    team_all, alive_all = team_all.to(DEV), alive_all.to(DEV)
+    consts = ops.pack_team_pool_weights(p["tp.seeds"].to(DEV), p["tp.attn.in_proj_weight"].to(DEV),
+                                        p["tp.attn.out_proj.weight"].to(DEV), H)
+    nw = p["tp.norm.weight"].to(DEV)
+    a = ops.team_pool(tokens[:, :N], team_all[:, :N], alive_all[:, :N], *consts, nw, None, H)
+    b = ops.team_pool(tokens[:, :N].contiguous(), team_all[:, :N].long(), alive_all[:, :N].contiguous(), *consts, nw, None, H)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    with pytest.raises(ValueError):
+        ops.team_pool(tokens[:, :N], team_all, alive_all[:, :N], *consts, nw, None, H)
+    with pytest.raises(ValueError):
+        ops.team_pool(tokens[:, :N].bfloat16(), team_all[:, :N], alive_all[:, :N], *consts, nw, None, H)
+    empty = ops.team_pool(tokens[:0, :N], team_all[:0, :N], alive_all[:0, :N], *consts, nw, None, H)
+    assert empty[0].shape == (0, N, D) and empty[1].shape == (0, 2, D)

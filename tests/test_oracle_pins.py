@@ -510,3 +510,107 @@ def test_rglru_sequence_forgets_everything_after_an_episode_end():
     x2[:, :5] += 3.0
     b, _ = torch_ref.rglru_sequence(x2, gates, lam, 8.0, torch.randn(R, D, generator=g), done)
     assert torch.equal(a[:, 5:], b[:, 5:]) and not torch.equal(a[:, :5], b[:, :5])
+
+
+# ---------------------------------------------------------------- team pooling (policy.py:78-120)
+
+
+def _team_case(seed, B=4, N=7, D=32, H=4, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    p = {
+        "tp.seeds": 0.5 * torch.randn(2, D, generator=g, dtype=dtype),
+        "tp.attn.in_proj_weight": torch.randn(3 * D, D, generator=g, dtype=dtype) / D ** 0.5,
+        "tp.attn.out_proj.weight": torch.randn(D, D, generator=g, dtype=dtype) / D ** 0.5,
+        "tp.norm.weight": 1.0 + 0.2 * torch.randn(D, generator=g, dtype=dtype),
+    }
+    x = torch.randn(B, N, D, generator=g, dtype=dtype)
+    team = torch.randint(0, 2, (B, N), generator=g, dtype=torch.int32)
+    alive = torch.rand(B, N, generator=g) < 0.7
+    team[0] = 0            # env 0: nobody on team 1
+    alive[1] = False       # env 1: everyone dead
+    alive[2] = True
+    return p, x, team, alive, H
+
+
+def _reference_forward_with_library_modules(p, x, team_id, alive, H):
+    """The text of policy.py:94-120 on torch's own nn.MultiheadAttention / nn.RMSNorm."""
+    B, N, D = x.shape
+    attn = torch.nn.MultiheadAttention(D, H, batch_first=True, bias=False, dtype=x.dtype)
+    norm = torch.nn.RMSNorm(D, dtype=x.dtype)
+    with torch.no_grad():
+        attn.in_proj_weight.copy_(p["tp.attn.in_proj_weight"])
+        attn.out_proj.weight.copy_(p["tp.attn.out_proj.weight"])
+        norm.weight.copy_(p["tp.norm.weight"])
+        pool = x.new_zeros(B, 2, D)
+        for t in range(2):
+            mask = (team_id == t) & alive
+            seed = p["tp.seeds"][t].view(1, 1, D).expand(B, 1, D)
+            out, _ = attn(seed, x, x, key_padding_mask=~mask, need_weights=False)
+            out = out.squeeze(1).nan_to_num(0.0)
+            out = out * mask.any(dim=1).unsqueeze(1).to(out.dtype)
+            pool[:, t] = norm(out)
+        idx = team_id.clamp(0, 1).long().unsqueeze(-1).expand(B, N, D)
+        return pool.gather(1, idx), pool
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float64, 1e-12), (torch.float32, 2e-6)])
+def test_team_pool_is_the_library_attention_composition(dtype, tol):
+    p, x, team, alive, H = _team_case(3, dtype=dtype)
+    ships, pool = torch_ref.team_pool(p, "tp.", x, team, alive, H)
+    ships_lib, pool_lib = _reference_forward_with_library_modules(p, x, team, alive, H)
+    assert torch.allclose(pool, pool_lib, rtol=tol, atol=tol)
+    assert torch.allclose(ships, ships_lib, rtol=tol, atol=tol)
+
+
+def test_team_pool_matches_brute_force_and_closed_forms():
+    p, x, team, alive, H = _team_case(4)
+    ships, pool = torch_ref.team_pool(p, "tp.", x, team, alive, H)
+    eps = torch.finfo(torch.float64).eps
+    loops = bruteforce.team_pool_loops(x.numpy(), team.numpy(), alive.numpy(), p["tp.seeds"].numpy(),
+                                       p["tp.attn.in_proj_weight"].numpy(), p["tp.attn.out_proj.weight"].numpy(),
+                                       p["tp.norm.weight"].numpy(), H, eps)
+    assert np.allclose(pool.numpy(), loops, rtol=1e-10, atol=1e-12)
+    # empty teams pool to exactly zero; every ship carries the pooled vector of its (clamped) team
+    assert (pool[0, 1] == 0).all() and (pool[1] == 0).all()
+    B, N, D = x.shape
+    for b in range(B):
+        for n in range(N):
+            assert torch.equal(ships[b, n], pool[b, int(team[b, n].clamp(0, 1))])
+    # one alive ship on a team: softmax over one key is 1 whatever the seed says, so the pooled
+    # vector is RMSNorm(W_o W_v x_j)
+    one = alive.clone()
+    one[3] = False
+    one[3, 2] = True
+    t = int(team[3, 2])
+    _, pool_one = torch_ref.team_pool(p, "tp.", x, team, one, H)
+    D = x.shape[-1]
+    direct = p["tp.attn.out_proj.weight"] @ (p["tp.attn.in_proj_weight"][2 * D:] @ x[3, 2])
+    assert torch.allclose(pool_one[3, t], torch_ref.rms_norm(direct, p["tp.norm.weight"]), rtol=1e-10, atol=1e-12)
+    assert (pool_one[3, 1 - t] == 0).all()
+
+
+def test_team_pool_ignores_dead_ships_other_teams_and_field_ids():
+    p, x, team, alive, H = _team_case(5)
+    _, base = torch_ref.team_pool(p, "tp.", x, team, alive, H)
+    pert = x.clone()
+    pert[~alive] = pert[~alive] * -3.0 + 5.0  # dead ships are no keys of either team
+    _, again = torch_ref.team_pool(p, "tp.", pert, team, alive, H)
+    assert torch.equal(base, again)
+    # team 0's pool does not move when only team-1 ships change, and the other way round
+    pert = x.clone()
+    pert[team == 1] += 1.0
+    _, again = torch_ref.team_pool(p, "tp.", pert, team, alive, H)
+    assert torch.equal(base[:, 0], again[:, 0]) and not torch.equal(base[:, 1], again[:, 1])
+    # an id outside {0, 1} (field tokens carry 2) is nobody's key but reads team 1's pool
+    odd = team.clone()
+    odd[2, 0] = 2
+    ships, pool = torch_ref.team_pool(p, "tp.", x, odd, alive, H)
+    assert torch.equal(ships[2, 0], pool[2, 1])
+    stay = alive.clone()
+    stay[2, 0] = False
+    _, without = torch_ref.team_pool(p, "tp.", x, team, stay, H)
+    assert torch.allclose(pool[2], without[2], rtol=1e-12, atol=1e-12)
+    # ship order inside an environment does not matter for the pools
+    perm = torch.randperm(x.shape[1], generator=torch.Generator().manual_seed(1))
+    _, shuffled = torch_ref.team_pool(p, "tp.", x[:, perm], team[:, perm], alive[:, perm], H)
+    assert torch.allclose(base, shuffled, rtol=1e-10, atol=1e-12)

@@ -11,7 +11,7 @@ norms and GELUs are library calls on both sides.
 import pytest
 import torch
 
-from helpers import block_params, max_rel, temporal_params, trunk_params
+from helpers import block_params, max_rel, team_case, team_pool_params, temporal_params, trunk_params
 from oracle import torch_ref
 
 import boost_and_broadside_amd as bnb
@@ -478,3 +478,48 @@ def test_block_sequence_trains_and_matches_the_no_grad_path():
     grads = [p.grad for p in block.parameters()]
     assert all(g is not None and torch.isfinite(g).all() for g in grads)
     assert block.temporal[0].rg_lru.log_lambda.grad.abs().max() > 0
+
+
+@pytest.mark.parametrize("autocast", [False, True])
+@pytest.mark.parametrize("D,H", [(128, 4), (64, 4)])
+def test_team_pooling_layer_matches_oracle(autocast, D, H):
+    # width 128 runs on the kernel, width 64 on the library attention call; both must state the same function
+    B, N = 12, 19
+    g = torch.Generator().manual_seed(D + autocast)
+    p = team_pool_params(g, "tp.", D)
+    layer = bnb.TeamPMA(D, H).to(DEV).eval()
+    layer.load_state_dict(_strip(p, "tp."))
+    x = torch.randn(B, N, D, generator=g)
+    team, alive = team_case(3, B, N)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+        got = layer(x.to(DEV), team.to(DEV), alive.to(DEV))
+        pooled = layer.pooled(x.to(DEV), team.to(DEV), alive.to(DEV))
+    ref, ref_pool = torch_ref.team_pool(p, "tp.", x, team, alive, H)
+    assert got.shape == (B, N, D) and got.dtype == torch.float32
+    tol = 2e-2 if (autocast and D != 128) else 1e-5  # the kernel computes in fp32 whatever autocast says
+    assert max_rel(got.cpu(), ref) <= tol
+    assert max_rel(pooled.cpu(), ref_pool) <= tol
+    assert (got.cpu()[1] == 0).all()  # everybody dead in environment 1
+
+
+def test_team_pooling_layer_trains_through_the_library_path():
+    D, H, B, N = 128, 4, 5, 8
+    g = torch.Generator().manual_seed(21)
+    p = team_pool_params(g, "tp.", D)
+    layer = bnb.TeamPMA(D, H).to(DEV)
+    layer.load_state_dict(_strip(p, "tp."))
+    x = torch.randn(B, N, D, generator=g).to(DEV).requires_grad_()
+    # both teams present everywhere: with an empty team the oracle's softmax over no key is NaN
+    # and so is autograd through it, which leaves nothing to compare with
+    team = (torch.arange(N, dtype=torch.int32) % 2).repeat(B, 1)
+    alive = torch.rand(B, N, generator=g) < 0.6
+    alive[:, :2] = True
+    out = layer(x, team.to(DEV), alive.to(DEV))
+    out.square().sum().backward()
+    assert torch.isfinite(x.grad).all() and all(torch.isfinite(q.grad).all() for q in layer.parameters())
+    with torch.no_grad():
+        assert max_rel(layer(x.detach(), team.to(DEV), alive.to(DEV)), out.detach()) <= 1e-5
+    xr = x.detach().cpu().double().requires_grad_()
+    ref, _ = torch_ref.team_pool({k: v.double() for k, v in p.items()}, "tp.", xr, team, alive, H)
+    ref.square().sum().backward()
+    assert max_rel(x.grad.cpu(), xr.grad.float()) <= 1e-4
