@@ -236,7 +236,7 @@ def cpu_baseline(w, p, budget_s):
     t0 = time.perf_counter()
     once()
     one = max(time.perf_counter() - t0, 1e-6)
-    reps = int(max(3, min(200, budget_s / one)))
+    reps = int(max(3, min(5000, budget_s / one)))
     times = []
     for _ in range(reps):
         t0 = time.perf_counter()
@@ -597,8 +597,11 @@ def main():
             "environments": w.B, "ships": w.N, "avg_launch_us": t_pool * 1e6, "algorithmic_bytes_per_launch": pool_bytes,
             "achieved_GBps": pool_bytes / t_pool / 1e9, "frac_of_hbm_peak": pool_bytes / t_pool / peak,
             "eager_torch_us": None if t_pool_lib is None else t_pool_lib * 1e6,
+            "attend_algorithmic_bytes": w.B * w.N * (D * 4 + 4 + 1) + w.B * 2 * H * D * 4,
+            "handout_algorithmic_bytes": w.B * 2 * D * 4 + w.B * w.N * (4 + D * 4),
             "what": "per-team attention pooling with a learned seed as the only query, out projection, RMSNorm and the "
-                    "broadcast back to the ships in one fp32 kernel: ship rows read once, (B, N, D) written once; eager = "
+                    "broadcast back to the ships, fp32: a kernel that reads the ship rows once, one library GEMM on the pooled rows, a "
+                    "kernel that writes (B, N, D) once; eager = "
                     "two nn.MultiheadAttention calls, norm and gather in torch ops (bf16 autocast on bf16 workloads)",
         }
         del xs_t
