@@ -179,7 +179,6 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
     __syncthreads();
 
     // the lane's own token in the accumulator layout, and its sum of squares
-    const int64_t row = row0 + m;
     f32x16 acc[4];
     float ss = 0.0f;
 #pragma unroll
