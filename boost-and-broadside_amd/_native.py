@@ -12,7 +12,7 @@ import os
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "_lib", "libbnb_amd.so")
 
-ABI_VERSION = 14
+ABI_VERSION = 15
 F32, BF16 = 0, 1
 PATH_AUTO, PATH_VALU, PATH_MFMA = 0, 1, 2
 
@@ -38,8 +38,8 @@ SIGNATURES = {
     "bnb_team_attend_fwd": (_i, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i, _i, _i, _i, _vp]),
     "bnb_team_norm_broadcast_fwd": (_i, [_vp, _vp, _f, _vp, _i64, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "bnb_temporal_step_fwd": (
-        _i, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _f, _vp, _i64, _vp, _i,
-             _i64, _i, _vp]
+        _i, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _f, _vp, _i64, _i64,
+             _vp, _i, _i64, _i, _vp]
     ),
     "bnb_conv_step_fwd": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _vp]),
     "bnb_conv_seq_fwd": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
@@ -52,7 +52,7 @@ SIGNATURES = {
     "bnb_mask_count": (_i, [_vp, _vp, _i, _i, _vp]),
     "bnb_mask_fill": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "bnb_ffn_fused_fwd": (_i, [_vp, _i64, _vp, _i, _vp, _f, _vp, _vp, _i64, _i, _i, _vp]),
-    "bnb_ffn_fused_proj_fwd": (_i, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _f, _vp, _vp, _i64, _i, _i, _vp]),
+    "bnb_ffn_fused_proj_fwd": (_i, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _f, _vp, _vp, _i64, _i, _i, _vp]),
     "bnb_gelu_mul_fwd": (_i, [_vp, _i, _i64, _vp, _i, _i64, _vp, _i, _i64, _i, _vp]),
     "bnb_copy_bytes": (_i, [_vp, _vp, _i64, _vp]),
 }

@@ -80,7 +80,7 @@ template <int MODE>
 __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void ffn_fused_kernel(
     const float *__restrict__ x, int64_t x_stride, const uint16_t *__restrict__ delta,
     const uint16_t *__restrict__ rows_b, const uint16_t *__restrict__ wproj, const float *__restrict__ norm_w,
-    float eps, const uint16_t *__restrict__ wpack, float *__restrict__ out, int64_t R, int64_t rows_a_stride)
+    float eps, const uint16_t *__restrict__ wpack, float *__restrict__ out, int64_t R, int64_t rows_a_stride, int64_t rows_b_stride)
 {
     constexpr bool HAS_DELTA = MODE == kDeltaRows;
     // three weight buffers: chunk c is used while chunk c+1 is already complete (its operands
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
             u32x4 av = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(delta + rs * rows_a_stride + a_col));
             if (MODE == kDeltaGate) {
                 const Row8 g = load8(reinterpret_cast<const uint16_t *>(&av));
-                const Row8 y = load8_stream(rows_b + rs * kFfnD + a_col);
+                const Row8 y = load8_stream(rows_b + rs * rows_b_stride + a_col);
                 float p[8];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) p[e] = round_to_bf16(gelu_erf(g.v[e])) * y.v[e];
@@ -357,13 +357,13 @@ namespace bnb {
 template <int MODE>
 static int launch_ffn(const float *x, int64_t x_stride, const void *rows_a, const void *rows_b, const void *wproj,
                       const float *norm_weight, float eps, const void *weights_packed, float *out, int64_t R,
-                      int64_t rows_a_stride, hipStream_t s)
+                      int64_t rows_a_stride, int64_t rows_b_stride, hipStream_t s)
 {
     const int64_t blocks = (R + kFfnWaves * 32 - 1) / (kFfnWaves * 32);
     if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((ffn_fused_kernel<MODE>), dim3((unsigned)blocks), dim3(kFfnThreads), 0, s, x, x_stride,
                        (const uint16_t *)rows_a, (const uint16_t *)rows_b, (const uint16_t *)wproj, norm_weight, eps,
-                       (const uint16_t *)weights_packed, out, R, rows_a_stride);
+                       (const uint16_t *)weights_packed, out, R, rows_a_stride, rows_b_stride);
     return (int)hipGetLastError();
 }
 
@@ -394,13 +394,13 @@ extern "C" int bnb_ffn_fused_fwd(const float *x, int64_t x_row_stride, const voi
     hipStream_t s = (hipStream_t)stream;
     if (delta)
         return launch_ffn<kDeltaRows>(x, x_row_stride, delta, nullptr, nullptr, norm_weight, eps, weights_packed, out,
-                                      R, kFfnD, s);
+                                      R, kFfnD, kFfnD, s);
     return launch_ffn<kDeltaNone>(x, x_row_stride, nullptr, nullptr, nullptr, norm_weight, eps, weights_packed, out, R,
-                                  kFfnD, s);
+                                  kFfnD, kFfnD, s);
 }
 
 extern "C" int bnb_ffn_fused_proj_fwd(const float *x, int64_t x_row_stride, const void *rows_a, int64_t rows_a_stride,
-                                      const void *rows_b,
+                                      const void *rows_b, int64_t rows_b_stride,
                                       const void *proj_packed, const float *norm_weight, float eps,
                                       const void *weights_packed, float *out, int64_t R, int D, int hidden,
                                       void *stream)
@@ -410,13 +410,15 @@ extern "C" int bnb_ffn_fused_proj_fwd(const float *x, int64_t x_row_stride, cons
     if (rc != 0 || R == 0) return rc;
     if (!rows_a || !proj_packed) return BNB_ERR_NULL_POINTER;
     if (rows_a_stride == 0) rows_a_stride = kFfnD;
-    if (rows_a_stride < kFfnD) return BNB_ERR_BAD_SHAPE;
-    if (!aligned16(rows_a) || rows_a_stride % 8 != 0 || !aligned16(proj_packed) || (rows_b && !aligned16(rows_b)))
+    if (rows_b_stride == 0) rows_b_stride = kFfnD;
+    if (rows_a_stride < kFfnD || rows_b_stride < kFfnD) return BNB_ERR_BAD_SHAPE;
+    if (!aligned16(rows_a) || rows_a_stride % 8 != 0 || !aligned16(proj_packed) ||
+        (rows_b && (!aligned16(rows_b) || rows_b_stride % 8 != 0)))
         return BNB_ERR_MISALIGNED;
     hipStream_t s = (hipStream_t)stream;
     if (rows_b)
         return launch_ffn<kDeltaGate>(x, x_row_stride, rows_a, rows_b, proj_packed, norm_weight, eps, weights_packed,
-                                      out, R, rows_a_stride, s);
+                                      out, R, rows_a_stride, rows_b_stride, s);
     return launch_ffn<kDeltaProj>(x, x_row_stride, rows_a, nullptr, proj_packed, norm_weight, eps, weights_packed, out,
-                                  R, rows_a_stride, s);
+                                  R, rows_a_stride, kFfnD, s);
 }

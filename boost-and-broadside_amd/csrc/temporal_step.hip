@@ -57,7 +57,7 @@ __global__ __launch_bounds__(kTsMaxWaves * kWave) __attribute__((amdgpu_waves_pe
     float *h_out, int64_t h_out_stride, const float *__restrict__ conv_weight, const float *__restrict__ conv_bias,
     const uint16_t *__restrict__ gate_weight_packed, const float *__restrict__ gate_bias,
     const float *__restrict__ log_lambda, float c, uint16_t *__restrict__ y, int64_t y_group_stride,
-    const uint8_t *__restrict__ reset, int rows_per_env, int64_t R, int64_t full_rounds, int tail_rows_per_wave)
+    int64_t y_row_stride, const uint8_t *__restrict__ reset, int rows_per_env, int64_t R, int64_t full_rounds, int tail_rows_per_wave)
 {
     extern __shared__ __align__(16) unsigned char s_raw[];
     uint16_t *s_w = reinterpret_cast<uint16_t *>(s_raw);
@@ -249,8 +249,8 @@ __global__ __launch_bounds__(kTsMaxWaves * kWave) __attribute__((amdgpu_waves_pe
                 if (valid[p]) {
                     store8(h_out + row[p] * h_out_stride + d0, out);
                     const int64_t y_off = y_group_stride != 0
-                                              ? env[p] * y_group_stride + (row[p] - env[p] * rows_per_env) * kTsD
-                                              : row[p] * kTsD;
+                                              ? env[p] * y_group_stride + (row[p] - env[p] * rows_per_env) * y_row_stride
+                                              : row[p] * y_row_stride;
                     store8(y + y_off + d0, out);
                 }
             }
@@ -281,7 +281,7 @@ extern "C" int bnb_temporal_step_fwd(const void *b1, int64_t b1_group_stride, in
                                      float *h_out, int64_t h_out_row_stride, const float *conv_weight,
                                      const float *conv_bias, const void *gate_weight_packed, const float *gate_bias,
                                      const float *log_lambda, float c, void *y, int64_t y_group_stride,
-                                     const uint8_t *reset, int rows_per_env, int64_t R, int D, void *stream)
+                                     int64_t y_row_stride, const uint8_t *reset, int rows_per_env, int64_t R, int D, void *stream)
 {
     using namespace bnb;
     if (R < 0 || rows_per_env < 1) return BNB_ERR_BAD_SHAPE;
@@ -291,6 +291,8 @@ extern "C" int bnb_temporal_step_fwd(const void *b1, int64_t b1_group_stride, in
     if (!b1 || !conv_in || !conv_out || !h_in || !h_out || !conv_weight || !gate_weight_packed || !gate_bias ||
         !log_lambda || !y)
         return BNB_ERR_NULL_POINTER;
+    if (y_row_stride == 0) y_row_stride = D;
+    if (y_row_stride < D) return BNB_ERR_BAD_SHAPE;
     if (conv_in_row_stride < 3 * D || conv_out_row_stride < 3 * D || h_in_row_stride < D || h_out_row_stride < D ||
         b1_row_stride < D)
         return BNB_ERR_BAD_SHAPE;
@@ -298,7 +300,7 @@ extern "C" int bnb_temporal_step_fwd(const void *b1, int64_t b1_group_stride, in
         return BNB_ERR_BAD_SHAPE;
     if (!aligned16(b1) || !aligned16(conv_in) || !aligned16(conv_out) || !aligned16(h_in) || !aligned16(h_out) ||
         !aligned16(y) || !aligned16(conv_weight) || !aligned16(gate_weight_packed) || (b1_row_stride % 8) != 0 ||
-        (b1_group_stride % 8) != 0 || (y_group_stride % 8) != 0 || (conv_in_row_stride % 4) != 0 ||
+        (b1_group_stride % 8) != 0 || (y_group_stride % 8) != 0 || (y_row_stride % 8) != 0 || (conv_in_row_stride % 4) != 0 ||
         (conv_out_row_stride % 4) != 0 || (h_in_row_stride % 4) != 0 || (h_out_row_stride % 4) != 0)
         return BNB_ERR_MISALIGNED;
     // One work-group per CU at most (LDS), 8 waves each, every wave at least 8 rows.
@@ -318,6 +320,6 @@ extern "C" int bnb_temporal_step_fwd(const void *b1, int64_t b1_group_stride, in
                        (const uint16_t *)b1, b1_group_stride, b1_row_stride, conv_in, conv_in_row_stride, conv_out,
                        conv_out_row_stride, h_in, h_in_row_stride, h_out, h_out_row_stride, conv_weight, conv_bias,
                        (const uint16_t *)gate_weight_packed, gate_bias, log_lambda, c, (uint16_t *)y, y_group_stride,
-                       reset, rows_per_env, R, full_rounds, tail_rows_per_wave);
+                       y_row_stride, reset, rows_per_env, R, full_rounds, tail_rows_per_wave);
     return (int)hipGetLastError();
 }

@@ -523,7 +523,7 @@ def temporal_step(
         gate_weight_packed: ``pack_gate_weights(linear_a.weight, linear_x.weight)``.
         gate_bias: (256,) float32 ``[linear_a.bias | linear_x.bias]``.
         y_out:     optional bfloat16 destination of the layer output: contiguous (R, 128) or a
-                   (B, rows_per_env, 128) view into a wider token tensor.
+                   (B, rows_per_env, 128) view into a wider token tensor (possibly a column block).
         reset, rows_per_env: as in ``rglru_step``.
 
     Returns:
@@ -577,15 +577,15 @@ def temporal_step(
         h_out = torch.empty((R, D), dtype=torch.float32, device=dev)
     elif h_out.shape != (R, D) or h_out.dtype != torch.float32 or h_out.device != dev or (R and h_out.stride(-1) != 1):
         raise ValueError("h_out must be a float32 (R, 128) tensor on b1's device, contiguous in its last dim")
-    y_group = 0
+    y_group, y_row = 0, D
     if y_out is None:
         y_out = torch.empty((R, D), dtype=torch.bfloat16, device=dev)
     else:
         if y_out.dtype != torch.bfloat16 or y_out.device != dev:
             raise ValueError("y_out must be a bfloat16 tensor on b1's device")
-        if y_out.dim() == 3:
-            y_group, _ = _grouped_rows(y_out, R, D, rows_per_env, "y_out")
-        elif y_out.shape != (R, D) or not y_out.is_contiguous():
+        if y_out.dim() == 3 and not y_out.is_contiguous():
+            y_group, y_row = _grouped_rows(y_out, R, D, rows_per_env, "y_out", pitch_ok=True)
+        elif y_out.shape not in ((R, D), (R // max(rows_per_env, 1), rows_per_env, D)) or not y_out.is_contiguous():
             raise ValueError("y_out must be a contiguous (R, 128) tensor or a (B, n, 128) view")
     reset_ptr = _reset_pointer(reset, R, rows_per_env, dev)
     if (b1_group or y_group) and (rows_per_env < 1 or R % rows_per_env):
@@ -597,7 +597,7 @@ def temporal_step(
                 conv_out.data_ptr(), conv_out.stride(0), h.data_ptr(), h.stride(0), h_out.data_ptr(), h_out.stride(0),
                 conv_weight.data_ptr(), None if conv_bias is None else conv_bias.data_ptr(),
                 gate_weight_packed.data_ptr(), gate_bias.data_ptr(), log_lambda.data_ptr(), float(c),
-                y_out.data_ptr(), int(y_group), reset_ptr, int(rows_per_env), R, D, _stream(),
+                y_out.data_ptr(), int(y_group), int(y_row), reset_ptr, int(rows_per_env), R, D, _stream(),
             )
         _native.check(rc, "bnb_temporal_step_fwd")
     return y_out, h_out, conv_out
@@ -1023,13 +1023,12 @@ def ffn_fused(
                 raise ValueError(f"projection operand rows must be bfloat16 {tuple(x.shape)} tensors")
             if torch.is_grad_enabled() and t.requires_grad:
                 raise RuntimeError("ffn_fused is forward-only; call it under torch.no_grad()")
-            t2 = t.reshape(-1, D) if (k == 0 and _uniform_rows(t, D)) else t.reshape(-1, D).contiguous()
-            flat.append(t2)
+            flat.append(t.view(-1, D) if _uniform_rows(t, D) else t.reshape(-1, D).contiguous())
         if R:
             with torch.cuda.device(x.device):
                 rc = _native.load().bnb_ffn_fused_proj_fwd(
                     x2.data_ptr(), x2.stride(0), flat[0].data_ptr(), flat[0].stride(0),
-                    flat[1].data_ptr() if len(flat) == 2 else None,
+                    flat[1].data_ptr() if len(flat) == 2 else None, flat[1].stride(0) if len(flat) == 2 else 0,
                     wp.data_ptr(), norm_weight.data_ptr(), float(_F32_EPS if eps is None else eps),
                     weights_packed.data_ptr(), out.data_ptr(), R, D, FFN_HIDDEN, _stream(),
                 )

@@ -480,18 +480,37 @@ class GriffinTemporalBlock(nn.Module):
         R = B * n_rec
         act = _projection_dtype()
         gate_in = normed = None
+        y = None
         if act == torch.bfloat16 and D == ops.FFN_WIDTH and self.linear1.bias is None and self.linear2.bias is None:
-            # norm1, linear1 and linear2 as one kernel: [b1 | gate_in] side by side, read in place
-            ws = (self.linear1.weight, self.linear2.weight)
-            pk = _cached_cast(self, "_bnb_l12_pack", ws, torch.bfloat16,
-                              lambda: ops.pack_linear_weights(torch.cat([ws[0], ws[1]], dim=0)))
-            both = ops.norm_linear(x, self.norm1.weight, pk, eps=self.norm1.eps)  # (B, NM, 2D)
-            b1, gate_in = both[..., :D], both[..., D:]
+            # norm1, linear1 and linear2 as one kernel: [b1 | gate_in] side by side, read in place.
+            # With field tokens a third block carries field_sub(linear1(.)) as ONE projection
+            # (field_sub . linear1 folded; exact while field_sub is the identity it starts as, a
+            # bf16 rounding of b1 apart otherwise): the recurrence then writes the ship rows of the
+            # same block, and no gather, GEMM and scatter of the field rows remain.
+            rg = self.rg_lru
+            fold = (NM > n_rec and field_sub is not None and field_sub.bias is None
+                    and rg.linear_a.bias is not None and rg.linear_x.bias is not None)
+            ws = (self.linear1.weight, self.linear2.weight) + ((field_sub.weight,) if fold else ())
+
+            def packed():
+                blocks = [ws[0].detach().float(), ws[1].detach().float()]
+                if fold:
+                    with torch.autocast("cuda", enabled=False):  # the folded product is formed in float32
+                        blocks.append(ws[2].detach().float() @ blocks[0])
+                return ops.pack_linear_weights(torch.cat(blocks, dim=0))
+
+            pk = _cached_cast(self, "_bnb_l12f_pack" if fold else "_bnb_l12_pack", ws, torch.bfloat16, packed)
+            both = ops.norm_linear(x, self.norm1.weight, pk, eps=self.norm1.eps)  # (B, NM, 2D or 3D)
+            b1, gate_in = both[..., :D], both[..., D:2 * D]
+            if fold:
+                y = both[..., 2 * D:]
         else:
             normed = self._norm_in(x)
             b1 = _project(self.linear1, normed)
         want_lp = act == torch.bfloat16
-        y = torch.empty((B, NM, D), dtype=act, device=x.device)
+        fields_done = y is not None
+        if y is None:
+            y = torch.empty((B, NM, D), dtype=act, device=x.device)
         ships_b1 = b1[:, :n_rec] if (NM > n_rec or gate_in is not None) else b1.reshape(R, D)
         rg = self.rg_lru
         if ops.temporal_step_supported(b1) and rg.linear_a.bias is not None and rg.linear_x.bias is not None:
@@ -506,7 +525,7 @@ class GriffinTemporalBlock(nn.Module):
                               self.conv.weight, self.conv.bias, gpk, gbias, rg.log_lambda, rg.c,
                               conv_out=state_out[:, D:].view(R, CONV_KERNEL - 1, D), h_out=state_out[:, :D],
                               y_out=y[:, :n_rec] if NM > n_rec else y.view(R, D), reset=reset, rows_per_env=n_rec)
-            if NM > n_rec:
+            if NM > n_rec and not fields_done:
                 y[:, n_rec:] = _project(field_sub, b1[:, n_rec:].reshape(-1, D)).view(B, NM - n_rec, D)
             return self._finish(x, normed, y, gate_in)
         res = ops.conv_step(ships_b1, state_in[:, D:].view(R, CONV_KERNEL - 1, D),

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 14
+#define BNB_ABI_VERSION 15
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -298,7 +298,9 @@ int bnb_team_norm_broadcast_fwd(const float *pre, const float *norm_weight, floa
  *   gate_bias           fp32 (2D) = [linear_a.bias | linear_x.bias]; rounded to bf16 inside, as
  *                       autocast hands it to the GEMM
  *   log_lambda (D) fp32, c
- *   y, y_group_stride   bf16 layer output = bf16(h'), addressed as in bnb_rglru_step_rows_fwd
+ *   y, y_group_stride, y_row_stride   bf16 layer output = bf16(h'): row r at r*y_row_stride, or with
+ *                       y_group_stride != 0 at (r / rows_per_env)*y_group_stride + (r % rows_per_env)*y_row_stride
+ *                       (y_row_stride 0 = D; a column block of a wider tensor works)
  *   reset, rows_per_env as in the two kernels it replaces
  *
  * Requirements: D == 128, R < 2^31, 16-byte aligned pointers, row strides multiples of 4 (fp32)
@@ -314,7 +316,7 @@ int bnb_temporal_step_fwd(const void *b1, int64_t b1_group_stride, int64_t b1_ro
                           const float *conv_weight, const float *conv_bias,
                           const void *gate_weight_packed, const float *gate_bias,
                           const float *log_lambda, float c,
-                          void *y, int64_t y_group_stride,
+                          void *y, int64_t y_group_stride, int64_t y_row_stride,
                           const uint8_t *reset, int rows_per_env,
                           int64_t R, int D, void *stream);
 
@@ -486,13 +488,13 @@ int bnb_ffn_fused_fwd(const float *x, int64_t x_row_stride, const void *delta, i
  * computed on the matrix cores and accumulated straight onto x; the projection's output never
  * exists in memory.
  *
- *   rows_a, rows_b  (R, 128) bf16; rows_b contiguous, rows_a rows rows_a_stride elements apart
+ *   rows_a, rows_b  (R, 128) bf16, rows rows_a_stride / rows_b_stride elements apart
  *                   (0 = 128; a column block of a wider projection output works)
  *   proj_packed     Wp (128, 128) in bf16 as [cb][ks][l][e] = Wp[32cb + l%32][16ks + 8(e/4) + 4(l/32) + e%4]
  *   other arguments as bnb_ffn_fused_fwd
  */
 int bnb_ffn_fused_proj_fwd(const float *x, int64_t x_row_stride, const void *rows_a, int64_t rows_a_stride,
-                           const void *rows_b,
+                           const void *rows_b, int64_t rows_b_stride,
                            const void *proj_packed, const float *norm_weight, float eps,
                            const void *weights_packed, float *out, int64_t R, int D, int hidden, void *stream);
 

@@ -1147,6 +1147,32 @@ def test_column_block_operands_are_read_in_place():
     assert torch.equal(in_place, copied)
 
 
+def test_three_column_blocks_share_one_projection_output():
+    # [linear1 | linear2 | recurrence output] in one (B, NM, 3D) tensor: the fused state kernel
+    # writes the ship rows of the third block, the tail reads its gate and y operands in place
+    B, n, NM, D = 7, 8, 12, 128
+    t = {k: v.to(DEV) for k, v in _temporal_inputs(9, B * n).items()}
+    g = torch.Generator().manual_seed(5)
+    wide = torch.randn(B, NM, 3 * D, generator=g).bfloat16().to(DEV)
+    wide[:, :n, :D] = t["b1"].view(B, n, D)
+    before = wide.clone()
+    pk, gb = ops.pack_gate_weights(t["wa"], t["wx"]), torch.cat([t["ba"], t["bx"]])
+    y_ref, h_ref, buf_ref = ops.temporal_step(t["b1"], t["buf"], t["h"], t["cw"], t["cb"], pk, gb, t["lam"], 8.0, rows_per_env=n)
+    _, h_new, buf_new = ops.temporal_step(wide[:, :n, :D], t["buf"], t["h"], t["cw"], t["cb"], pk, gb, t["lam"], 8.0,
+                                          y_out=wide[:, :n, 2 * D:], rows_per_env=n)
+    assert torch.equal(h_new, h_ref) and torch.equal(buf_new, buf_ref)
+    assert torch.equal(wide[:, :n, 2 * D:].reshape(B * n, D), y_ref)
+    assert torch.equal(wide[..., :2 * D], before[..., :2 * D]) and torch.equal(wide[:, n:], before[:, n:])
+    x, _, nw, p = _ffn_case(6, B * NM)
+    ffn = ops.pack_ffn_weights(p["f.gate_proj.weight"].to(DEV), p["f.up_proj.weight"].to(DEV), p["f.down_proj.weight"].to(DEV))
+    wp = ops.pack_proj_weights((torch.randn(D, D, generator=g) / D ** 0.5).to(DEV))
+    xd = x.to(DEV).view(B, NM, D)
+    gate, y = wide[..., D:2 * D], wide[..., 2 * D:]
+    in_place = ops.ffn_fused(xd, None, nw.to(DEV), ffn, proj=(gate, y, wp))
+    copied = ops.ffn_fused(xd, None, nw.to(DEV), ffn, proj=(gate.contiguous(), y.contiguous(), wp))
+    assert torch.equal(in_place, copied)
+
+
 # ------------------------------------------------------------------ team pooling
 
 
