@@ -6,7 +6,8 @@
 // The kernel is bound by HBM traffic (x, two gate pre-activations and the old state in,
 // the new state and its optional low-precision copy out), so the design is a plain
 // streaming pass: every lane owns 8 consecutive channels of ONE row, moves them with
-// 16-byte nontemporal accesses and keeps everything between load and store in registers.
+// 16-byte accesses (nontemporal once the launch outgrows the last-level cache) and keeps
+// everything between load and store in registers.
 // Measured on MI355X, one row per lane in large blocks streams faster than several rows in
 // flight per lane (more, shorter waves beat deeper per-lane unrolling on this memory system).
 
@@ -18,7 +19,7 @@ namespace bnb {
 constexpr int kRglruThreads = 256;     // scalar path, and the vector path on small inputs
 constexpr int kRglruBigThreads = 1024;  // vector path once the grid is large enough to fill the chip
 
-template <int THREADS, typename XT, typename GT, typename YT, bool HAS_Y>
+template <int THREADS, typename XT, typename GT, typename YT, bool HAS_Y, bool STREAM>
 __global__ __launch_bounds__(THREADS) void rglru_step_vec8_kernel(
     const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
     const float *h_in, int64_t h_in_stride, float *h_out, int64_t h_out_stride, YT *__restrict__ y,
@@ -35,10 +36,12 @@ __global__ __launch_bounds__(THREADS) void rglru_step_vec8_kernel(
     if (local_row >= rows_per_block || row >= R) return;
     const int d0 = (threadIdx.x - local_row * vecs_per_row) << 3;
 
-    const Row8 xv = load8_stream(x + row * D + d0);
-    const Row8 ga = load8_stream(gates + row * 2 * D + d0);
-    const Row8 gx = load8_stream(gates + row * 2 * D + D + d0);
-    Row8 hv = load8_stream(h_in + row * h_in_stride + d0);
+    // STREAM: nontemporal accesses, best once the rows no longer fit the last-level cache; below
+    // that size cached accesses let the producer's output be picked up on chip
+    const Row8 xv = STREAM ? load8_stream(x + row * D + d0) : load8(x + row * D + d0);
+    const Row8 ga = STREAM ? load8_stream(gates + row * 2 * D + d0) : load8(gates + row * 2 * D + d0);
+    const Row8 gx = STREAM ? load8_stream(gates + row * 2 * D + D + d0) : load8(gates + row * 2 * D + D + d0);
+    Row8 hv = STREAM ? load8_stream(h_in + row * h_in_stride + d0) : load8(h_in + row * h_in_stride + d0);
     // environment of the row: for the reset flag and for an output laid out per environment
     const int64_t env = (reset != nullptr || y_group_stride != 0) ? row / rows_per_env : 0;
     if (reset != nullptr && reset[env]) {
@@ -52,11 +55,13 @@ __global__ __launch_bounds__(THREADS) void rglru_step_vec8_kernel(
     for (int e = 0; e < 8; ++e)
         out.v[e] = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(xv.v[e], ga.v[e], gx.v[e],
                                                                           s_l2sig[d0 + e], c, hv.v[e]);
-    store8_stream(h_out + row * h_out_stride + d0, out);
+    if (STREAM) store8_stream(h_out + row * h_out_stride + d0, out);
+    else store8(h_out + row * h_out_stride + d0, out);
     if (HAS_Y) {
         // y rows either back to back or in groups of rows_per_env, y_group_stride elements apart
         const int64_t y_off = y_group_stride != 0 ? env * y_group_stride + (row - env * rows_per_env) * D : row * D;
-        store8_stream(y + y_off + d0, out);
+        if (STREAM) store8_stream(y + y_off + d0, out);
+        else store8(y + y_off + d0, out);
     }
 }
 
@@ -99,16 +104,19 @@ static int launch_rglru(const void *x, const void *gates, const float *log_lambd
         const int rows_per_block = threads / vecs_per_row;
         const int64_t blocks = (R + rows_per_block - 1) / rows_per_block;
         if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
-        if (big)
-            hipLaunchKernelGGL((rglru_step_vec8_kernel<kRglruBigThreads, XT, GT, YT, HAS_Y>), dim3((unsigned)blocks),
-                               dim3(threads), (size_t)D * sizeof(float), stream, (const XT *)x, (const GT *)gates,
-                               log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D,
-                               rows_per_block, reset, rows_per_env, y_group_stride);
-        else
-            hipLaunchKernelGGL((rglru_step_vec8_kernel<kRglruThreads, XT, GT, YT, HAS_Y>), dim3((unsigned)blocks),
-                               dim3(threads), (size_t)D * sizeof(float), stream, (const XT *)x, (const GT *)gates,
-                               log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D,
-                               rows_per_block, reset, rows_per_env, y_group_stride);
+        // bytes the launch touches; MI355X keeps up to 256 MB in its last-level cache
+        const size_t bytes = (size_t)R * D * (sizeof(XT) + 2 * sizeof(GT) + 2 * sizeof(float) + (HAS_Y ? sizeof(YT) : 0));
+        const bool stream_hint = bytes > ((size_t)192 << 20);
+#define BNB_RGLRU_LAUNCH(T, S)                                                                                        \
+    hipLaunchKernelGGL((rglru_step_vec8_kernel<T, XT, GT, YT, HAS_Y, S>), dim3((unsigned)blocks), dim3(threads),         \
+                       (size_t)D * sizeof(float), stream, (const XT *)x, (const GT *)gates, log_lambda, c, h_in,         \
+                       h_in_stride, h_out, h_out_stride, (YT *)y, R, D, rows_per_block, reset, rows_per_env,             \
+                       y_group_stride)
+        if (big && stream_hint) BNB_RGLRU_LAUNCH(kRglruBigThreads, true);
+        else if (big) BNB_RGLRU_LAUNCH(kRglruBigThreads, false);
+        else if (stream_hint) BNB_RGLRU_LAUNCH(kRglruThreads, true);
+        else BNB_RGLRU_LAUNCH(kRglruThreads, false);
+#undef BNB_RGLRU_LAUNCH
     } else {
         const int64_t blocks = (R * D + kRglruThreads - 1) / kRglruThreads;
         if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
