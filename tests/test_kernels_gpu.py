@@ -1259,3 +1259,84 @@ def test_team_pool_reads_ship_rows_inside_the_token_tensor_and_other_id_types():
         ops.team_pool(tokens[:, :N].bfloat16(), team_all[:, :N], alive_all[:, :N], *consts, nw, None, H)
     empty = ops.team_pool(tokens[:0, :N], team_all[:0, :N], alive_all[:0, :N], *consts, nw, None, H)
     assert empty[0].shape == (0, N, D) and empty[1].shape == (0, 2, D)
+
+
+# ------------------------------------------------------------------ widened kernels at the headline size
+
+
+def test_full_size_temporal_step_on_sampled_rows_and_environment_permutation():
+    # 64v88: 4096 environments x 152 ships = 622,592 state rows, two carried steps on the packed state;
+    # sampled rows go through the fp32 statement, and permuting the environments permutes the result bit for bit
+    w = harness.WORKLOADS["c4_64v88_bf16"]
+    B, n, D = w.B, w.N, 128
+    R = B * n
+    g = torch.Generator(device=DEV).manual_seed(17)
+    small = {k: v.to(DEV) for k, v in _temporal_inputs(17, 4).items()}  # weights only
+    pk, gb = ops.pack_gate_weights(small["wa"], small["wx"]), torch.cat([small["ba"], small["bx"]])
+    state = torch.randn(R, 4 * D, device=DEV, generator=g) * 0.5
+    nxt = torch.empty_like(state)
+    y = torch.empty(R, D, device=DEV, dtype=torch.bfloat16)
+    pick = torch.arange(0, R, 7919, device=DEV)
+    ref = {"h": state[pick, :D].cpu(), "buf": state[pick, D:].view(-1, 3, D).cpu()}
+    cpu_w = {k: small[k].cpu() for k in ("cw", "cb", "wa", "wx", "ba", "bx", "lam")}
+    for t in range(2):
+        b1 = torch.randn(R, D, device=DEV, generator=g).bfloat16()
+        ops.temporal_step(b1, state[:, D:].view(R, 3, D), state[:, :D], small["cw"], small["cb"], pk, gb, small["lam"], 8.0,
+                          conv_out=nxt[:, D:].view(R, 3, D), h_out=nxt[:, :D], y_out=y)
+        h_true, buf_true = _temporal_truth({**cpu_w, "b1": b1[pick].cpu(), "h": ref["h"], "buf": ref["buf"]})
+        assert torch.equal(nxt[pick, D:].view(-1, 3, D).cpu(), buf_true), t
+        assert max_rel(nxt[pick, :D].cpu(), h_true) <= BF16_TOL, t
+        if t == 0:
+            perm = torch.randperm(B, device=DEV, generator=g)
+            rows = (perm[:, None] * n + torch.arange(n, device=DEV)[None, :]).reshape(-1)
+            st_p, nxt_p, y_p = state[rows].contiguous(), torch.empty_like(state), torch.empty_like(y)
+            ops.temporal_step(b1[rows].contiguous(), st_p[:, D:].view(R, 3, D), st_p[:, :D], small["cw"], small["cb"], pk, gb,
+                              small["lam"], 8.0, conv_out=nxt_p[:, D:].view(R, 3, D), h_out=nxt_p[:, :D], y_out=y_p)
+            assert torch.equal(nxt_p, nxt[rows]) and torch.equal(y_p, y[rows])
+            del st_p, nxt_p, y_p
+        ref = {"h": h_true, "buf": buf_true}  # carry the oracle's own state: errors must not need a reset to stay bounded
+        state, nxt = nxt, state
+    assert torch.isfinite(state).all()
+
+
+def test_full_size_sublayer_tail_and_projection_on_sampled_rows():
+    # 64v88: 655,360 token rows through the fused tail and through norm + qkv projection
+    w = harness.WORKLOADS["c4_64v88_bf16"]
+    R, D = w.B * w.NM, 128
+    g = torch.Generator(device=DEV).manual_seed(19)
+    _, _, nw, p = _ffn_case(19, 1)
+    x = torch.randn(R, D, device=DEV, generator=g)
+    delta = torch.randn(R, D, device=DEV, generator=g).bfloat16()
+    pk = ops.pack_ffn_weights(p["f.gate_proj.weight"].to(DEV), p["f.up_proj.weight"].to(DEV), p["f.down_proj.weight"].to(DEV))
+    out = ops.ffn_fused(x, delta, nw.to(DEV), pk)
+    pick = torch.arange(0, R, 6007, device=DEV)
+    rounded = {k: v.bfloat16().float() for k, v in p.items()}
+    s = x[pick].cpu() + delta[pick].float().cpu()
+    want = s + torch_ref.gated_mlp(rounded, "f.", torch_ref.rms_norm(s, nw))
+    assert max_rel(out[pick].cpu(), want) <= BF16_TOL
+    assert torch.isfinite(out).all()
+    # row permutation equivariance, bit for bit (every row is computed on its own)
+    perm = torch.randperm(R, device=DEV, generator=g)
+    assert torch.equal(ops.ffn_fused(x[perm], delta[perm], nw.to(DEV), pk), out[perm])
+    wq = torch.randn(3 * D, D, generator=torch.Generator().manual_seed(20)) / D ** 0.5
+    qkv = ops.norm_linear(x, nw.to(DEV), ops.pack_linear_weights(wq.to(DEV)))
+    want = torch_ref.rms_norm(x[pick].cpu(), nw) @ wq.bfloat16().float().t()
+    assert max_rel(qkv[pick].float().cpu(), want) <= BF16_TOL
+
+
+def test_full_size_team_pool_on_sampled_environments():
+    w = harness.WORKLOADS["c4_64v88_bf16"]
+    B, N, D, H = w.B, w.N, 128, 4
+    g = torch.Generator().manual_seed(23)
+    p = team_pool_params(g, "tp.", D)
+    gd = torch.Generator(device=DEV).manual_seed(23)
+    x = torch.randn(B, w.NM, D, device=DEV, generator=gd)
+    team, alive = team_case(24, B, N, p_alive=0.6)
+    consts = ops.pack_team_pool_weights(p["tp.seeds"].to(DEV), p["tp.attn.in_proj_weight"].to(DEV),
+                                        p["tp.attn.out_proj.weight"].to(DEV), H)
+    ships, pool = ops.team_pool(x[:, :N], team.to(DEV), alive.to(DEV), *consts, p["tp.norm.weight"].to(DEV), None, H)
+    pick = torch.arange(0, B, 97)
+    _, ref = torch_ref.team_pool(p, "tp.", x[pick, :N].cpu(), team[pick], alive[pick], H)
+    assert max_rel(pool[pick].cpu(), ref) <= F32_TOL
+    idx = team.clamp(0, 1).long().unsqueeze(-1).expand(B, N, D).to(DEV)
+    assert torch.equal(ships, pool.gather(1, idx))
