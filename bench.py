@@ -468,7 +468,8 @@ def main():
         ts_bytes = R * (D * 2 + 2 * 3 * D * 4 + 2 * D * 4 + D * 2)
         result["temporal_step_kernel"] = {
             "rows": R, "avg_launch_us": t_ts * 1e6, "algorithmic_bytes_per_launch": ts_bytes, "achieved_GBps": ts_bytes / t_ts / 1e9,
-            "frac_of_hbm_peak": ts_bytes / t_ts / peak, "three_kernel_composition_us": t_three * 1e6,
+            "frac_of_hbm_peak": ts_bytes / t_ts / peak, "traffic": load_traffic("temporal_step_kernel", w.name),
+            "three_kernel_composition_us": t_three * 1e6,
             "what": "conv taps + buffer shift, both gate projections (matrix cores) and the recurrence in one kernel: "
                     "bf16 linear1 output, packed fp32 state in, packed fp32 state and bf16 layer output out; "
                     "composition = conv kernel, library GEMM, recurrence kernel",
