@@ -19,127 +19,137 @@
 // All arithmetic is fp32 on the vector ALUs, which keeps the fp32 parity bar (the op also
 // serves evaluation without autocast).
 //
-// team_attend_kernel: ships come in chunks of 64 rows staged in LDS (the next chunk is already
-// in flight in registers):
-//   scores                    lane = ship, wave = a quarter of the channels, all heads of the
-//                             ship's own team (the other team's heads would be masked)
-//   online softmax            lane = ship, wave = head; the running maximum and sum of both
-//                             teams live in the wave's registers
-//   pooling                   thread = (channel, team): z(t, h)[d] for the H heads of its team
-
 #include "common.h"
 
 namespace bnb {
 
 constexpr int kTpD = 128;
 constexpr int kTpThreads = 256;
-constexpr int kTpChunk = 64;           // ship rows staged at a time
+constexpr int kTaRows = 16;            // ship rows a wave stages at a time
+constexpr int kTaWaves = 4;            // waves (environments) per work-group of the attend kernel
 constexpr int kTpPitch = kTpD + 4;     // floats per staged row: 16-byte aligned, bank-spread
 constexpr int kTpEnvs = 4;             // environments per work-group of the norm + hand-out kernel
 
-// max / sum over aligned groups of SEG lanes (SEG = 64: the whole wave)
-template <int SEG>
-__device__ __forceinline__ float seg_max(float v)
+// All-reduce over the aligned group of 16 lanes a lane belongs to, on the data-parallel
+// primitives (no LDS round trips): swap inside pairs, pairs inside quads, then mirror inside 8
+// and inside 16 (after the first two steps a quad is uniform, so mirroring exchanges quads).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
+__device__ __forceinline__ float row16_max(float v)
+{
+    v = fmaxf(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = fmaxf(v, dpp_move<0x141>(v));  // row_half_mirror
+    return fmaxf(v, dpp_move<0x140>(v));  // row_mirror
+}
+
+__device__ __forceinline__ float row16_sum(float v)
+{
+    v += dpp_move<0xB1>(v);
+    v += dpp_move<0x4E>(v);
+    v += dpp_move<0x141>(v);
+    return v + dpp_move<0x140>(v);
+}
+
+__device__ __forceinline__ float wave_sum(float v)
 {
 #pragma unroll
-    for (int o = SEG / 2; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o);
     return v;
 }
 
-template <int SEG>
-__device__ __forceinline__ float seg_sum(float v)
-{
-#pragma unroll
-    for (int o = SEG / 2; o >= 1; o >>= 1) v += __shfl_xor(v, o);
-    return v;
-}
-
-// SEG = lanes (staged rows) per environment in the score phase: 64 = one environment per
-// work-group, any number of ships in chunks of 64; 16 = four environments of up to 16 ships
-// side by side.  Writes z (B, 2, H, 128): the softmax-weighted mean of the ship rows per
-// (team, head), zero for a team without an alive ship.
-template <int H, int SEG>
-__global__ __launch_bounds__(kTpThreads) void team_attend_kernel(
+// One wavefront per environment, four per work-group, each on its own: after the score vectors
+// are in LDS no work-group barrier is left, only hand-overs inside the wave, so a CU keeps 16
+// independent waves busy.  Ships come in chunks of 16 rows through the wave's private LDS tile
+// (the next chunk is already in flight in registers).  Writes z (B, 2, H, 128): the
+// softmax-weighted mean of the ship rows per (team, head), zero for a team without an alive ship.
+//   scores     lane = (channel quarter g, ship s): partial dot products of ship s with the H
+//              score vectors of ITS team (the other team's would be masked) over channels
+//              32g .. 32g+31, summed over g with two cross-lane steps
+//   softmax    lane (g, s) keeps head g: online maximum / sum over the 16-lane group of head g,
+//              separately for the two teams
+//   pooling    lane l = channels 2l, 2l+1 of all 2H weighted sums
+template <int H>
+__global__ __launch_bounds__(kTaWaves * kWave) void team_attend_kernel(
     const float *__restrict__ x, int64_t x_env_stride, int64_t x_row_stride, const int32_t *__restrict__ team_id,
     int64_t team_env_stride, const uint8_t *__restrict__ alive, int64_t alive_env_stride,
     const float *__restrict__ score_vec, float *__restrict__ z_out, int B, int N)
 {
-    constexpr int NC = 2 * H;            // (team, head) pairs
-    constexpr int EPP = kTpChunk / SEG;  // environments per work-group
-    __shared__ __align__(16) float s_x[kTpChunk * kTpPitch];
-    constexpr int kTeamPitch = H * kTpD + 4;  // team 1's vectors start 16 bytes off team 0's banks
+    constexpr int NC = 2 * H;                  // (team, head) pairs
+    constexpr int kTeamPitch = H * kTpD + 4;   // team 1's vectors start 16 bytes off team 0's banks
     __shared__ __align__(16) float s_u[2 * kTeamPitch];
-    __shared__ __align__(16) float s_p[kTpChunk * NC];  // softmax numerators; 0 under the other team's heads
-    __shared__ __align__(16) float s_part[4 * kTpChunk * H];  // per channel quarter: partial scores
-    __shared__ float s_alpha[EPP * NC], s_l[EPP * NC];
+    __shared__ __align__(16) float s_x[kTaWaves][kTaRows * kTpPitch];
+    __shared__ __align__(16) float s_p[kTaWaves][kTaRows * NC];  // softmax numerators; 0 under the other team's heads
+    __shared__ float s_scale[kTaWaves][2 * NC];                   // per pair: rescale factor, then the final sum
 
     const int tid = threadIdx.x;
+    for (int i = tid; i < NC * kTpD; i += kTaWaves * kWave)
+        s_u[(i / (H * kTpD)) * kTeamPitch + i % (H * kTpD)] = score_vec[i];
+    __syncthreads();
+
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int d = tid & (kTpD - 1);  // pooling phase: channel
-    const int tm = wave >> 1;        // and team (wave-uniform)
-    for (int i = tid; i < NC * kTpD; i += kTpThreads) s_u[(i / (H * kTpD)) * kTeamPitch + i % (H * kTpD)] = score_vec[i];
+    const int env = blockIdx.x * kTaWaves + wave;
+    if (env >= B) return;
+    float *tile = s_x[wave];
+    float *ptile = s_p[wave];
+    float *scale = s_scale[wave];
+    const int g = lane >> 4;   // channel quarter in the score phase, head in the softmax
+    const int ship = lane & 15;
+    const float *xe = x + (int64_t)env * x_env_stride;
+    const int32_t *te = team_id + (int64_t)env * team_env_stride;
+    const uint8_t *ae = alive + (int64_t)env * alive_env_stride;
 
-    const int env_first = blockIdx.x * EPP;
-    const int seg = lane / SEG;      // environment of this lane inside the work-group
-    const int srow = lane % SEG;     // its ship inside the chunk
-    const int env_lane = env_first + seg;
-    float run_max[2] = {-INFINITY, -INFINITY}, run_sum[2] = {0.0f, 0.0f};  // of head `wave`, per team
-    float z[EPP][H];
+    float run_max[2] = {-INFINITY, -INFINITY}, run_sum[2] = {0.0f, 0.0f};  // head g, per team
+    float z[NC][2];
 #pragma unroll
-    for (int q = 0; q < EPP; ++q)
-#pragma unroll
-        for (int k = 0; k < H; ++k) z[q][k] = 0.0f;
+    for (int c = 0; c < NC; ++c) z[c][0] = z[c][1] = 0.0f;
 
-    // A thread's share of a chunk: 8 pieces of 16 bytes.  The next chunk is requested before the
-    // current one is worked on, so its latency hides under the arithmetic.
-    constexpr int kPieces = kTpChunk * (kTpD / 4) / kTpThreads;
+    // a lane's share of a chunk: 8 pieces of 16 bytes (piece = lane + 64*it: row piece/32)
+    constexpr int kPieces = kTaRows * (kTpD / 4) / kWave;
     f32x4 stage[kPieces];
+    int stage_team = -1, stage_alive = 0;  // of ship `ship` of the chunk in flight
     auto fetch = [&](int c0) {
-        const int rows = N - c0 < SEG ? N - c0 : SEG;
+        const int rows = N - c0 < kTaRows ? N - c0 : kTaRows;
+        const int sr = ship < rows ? ship : rows - 1;
+        stage_team = te[c0 + sr];
+        stage_alive = ae[c0 + sr];
 #pragma unroll
         for (int it = 0; it < kPieces; ++it) {
-            const int idx = tid + it * kTpThreads;
-            const int q4 = (idx & 31) * 4;
-            const int rr = idx >> 5;  // staged row: q * SEG + r
-            const int q = rr / SEG, r = rr % SEG;
-            const bool on = r < rows && env_first + q < B;
-            const int64_t off = on ? (int64_t)(env_first + q) * x_env_stride + (int64_t)(c0 + r) * x_row_stride + q4 : 0;
-            stage[it] = *reinterpret_cast<const f32x4 *>(x + off);
-        }
-    };
-    auto stash = [&](int c0) {
-        const int rows = N - c0 < SEG ? N - c0 : SEG;
-#pragma unroll
-        for (int it = 0; it < kPieces; ++it) {
-            const int idx = tid + it * kTpThreads;
-            const int q4 = (idx & 31) * 4;
-            const int rr = idx >> 5;
-            if (rr % SEG < rows) *reinterpret_cast<f32x4 *>(s_x + rr * kTpPitch + q4) = stage[it];
+            const int idx = lane + it * kWave;
+            const int r = idx >> 5, q4 = (idx & 31) * 4;
+            const int rr = r < rows ? r : rows - 1;  // rows past the end re-read the last one and are zeroed below
+            stage[it] = *reinterpret_cast<const f32x4 *>(xe + (int64_t)(c0 + rr) * x_row_stride + q4);
         }
     };
 
     if (N > 0) fetch(0);
-    for (int c0 = 0; c0 < N; c0 += SEG) {
-        const int rows = N - c0 < SEG ? N - c0 : SEG;
-        __syncthreads();  // previous chunk is done with s_x, s_p, s_alpha
-        stash(c0);
-        if (c0 + SEG < N) fetch(c0 + SEG);
-        __syncthreads();
-
-        // ---- scores of this lane's ship under the heads of ITS team (the other team's heads
-        //      would be masked anyway).  Each wave covers a quarter of the channels, so the
-        //      staged rows are read from LDS once, not once per head. ----
-        const bool present = srow < rows && env_lane < B;
-        const int ship_team = present ? team_id[(int64_t)env_lane * team_env_stride + c0 + srow] : -1;
-        const bool key = present && alive[(int64_t)env_lane * alive_env_stride + c0 + srow] != 0 &&
-                         (ship_team == 0 || ship_team == 1);
-        {
-            float part[H];
+    for (int c0 = 0; c0 < N; c0 += kTaRows) {
+        const int rows = N - c0 < kTaRows ? N - c0 : kTaRows;
+        // absent rows are stored as zeros: their weight is 0 and 0 * finite keeps the sums clean
 #pragma unroll
-            for (int k = 0; k < H; ++k) part[k] = 0.0f;
-            const float *xr = s_x + (present ? lane : 0) * kTpPitch + 32 * wave;
-            const float *ur = s_u + (key ? ship_team : 0) * kTeamPitch + 32 * wave;
+        for (int it = 0; it < kPieces; ++it) {
+            const int idx = lane + it * kWave;
+            const int r = idx >> 5, q4 = (idx & 31) * 4;
+            *reinterpret_cast<f32x4 *>(tile + r * kTpPitch + q4) = r < rows ? stage[it] : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+        const bool present = ship < rows;
+        const int ship_team = present ? stage_team : -1;
+        const bool key = present && stage_alive != 0 && (ship_team == 0 || ship_team == 1);
+        if (c0 + kTaRows < N) fetch(c0 + kTaRows);
+        wave_lds_handover();
+
+        // ---- partial scores over this lane's channel quarter, all heads of the ship's team ----
+        float part[H];
+#pragma unroll
+        for (int k = 0; k < H; ++k) part[k] = 0.0f;
+        {
+            const float *xr = tile + ship * kTpPitch + 32 * g;
+            const float *ur = s_u + (key ? ship_team : 0) * kTeamPitch + 32 * g;
 #pragma unroll
             for (int i = 0; i < 32; i += 4) {
                 const f32x4 xv = *reinterpret_cast<const f32x4 *>(xr + i);
@@ -149,78 +159,63 @@ __global__ __launch_bounds__(kTpThreads) void team_attend_kernel(
                     part[k] += xv.x * uv.x + xv.y * uv.y + xv.z * uv.z + xv.w * uv.w;
                 }
             }
-#pragma unroll
-            for (int k = 0; k < H; ++k) s_part[(wave * H + k) * kTpChunk + lane] = part[k];
         }
-        __syncthreads();
-
-        // ---- online softmax per environment and team: wave = head ----
-        if (wave < H) {
-            const int head = wave;
-            float dot = 0.0f;
+        // sum over the four channel quarters (lanes l, l^16, l^32, l^48); lane (g, s) keeps head g
+        float dot = 0.0f;
 #pragma unroll
-            for (int qw = 0; qw < 4; ++qw) dot += s_part[(qw * H + head) * kTpChunk + lane];
+        for (int k = 0; k < H; ++k) {
+            float v = part[k];
+            v += __shfl_xor(v, 16);
+            v += __shfl_xor(v, 32);
+            if (k == g) dot = v;
+        }
+
+        // ---- online softmax of head g over the 16 ships, per team ----
+        if (g < H) {
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 const bool mine = key && ship_team == t;
                 const float sc = mine ? dot : -INFINITY;
-                const float new_max = fmaxf(run_max[t], seg_max<SEG>(sc));
+                const float new_max = fmaxf(run_max[t], row16_max(sc));
                 const bool none = new_max == -INFINITY;  // no key of this team so far
                 const float pt = none ? 0.0f : __builtin_amdgcn_exp2f(sc - new_max);
                 const float alpha = none ? 1.0f : __builtin_amdgcn_exp2f(run_max[t] - new_max);
-                run_sum[t] = run_sum[t] * alpha + seg_sum<SEG>(pt);
+                run_sum[t] = run_sum[t] * alpha + row16_sum(pt);
                 run_max[t] = new_max;
-                s_p[lane * NC + t * H + head] = mine ? pt : 0.0f;
-                if (srow == 0) s_alpha[seg * NC + t * H + head] = alpha;
+                ptile[ship * NC + t * H + g] = mine ? pt : 0.0f;
+                if (ship == 0) scale[t * H + g] = alpha;
             }
         }
-        __syncthreads();
+        wave_lds_handover();
 
-        // ---- z(t, h)[d] = alpha z + sum_j p_j x_j[d] for the H heads of team tm.  Eight rows per
-        //      step, all their LDS reads issued before the arithmetic (the loop is bound by LDS
-        //      latency otherwise); rows past the chunk were never written and carry p = 0 only
-        //      if they are cleared, so the tail is done row by row. ----
+        // ---- z(t, h)[2l, 2l+1] = alpha z + sum_j p_j x_j ----
 #pragma unroll
-        for (int q = 0; q < EPP; ++q) {
+        for (int c = 0; c < NC; ++c) {
+            const float a = scale[c];
+            z[c][0] *= a, z[c][1] *= a;
+        }
+#pragma unroll 4
+        for (int j = 0; j < kTaRows; ++j) {
+            const f32x2 xv = *reinterpret_cast<const f32x2 *>(tile + j * kTpPitch + 2 * lane);
 #pragma unroll
-            for (int k = 0; k < H; ++k) z[q][k] *= s_alpha[q * NC + tm * H + k];
-            const float *xq = s_x + q * SEG * kTpPitch + d;
-            const float *pq = s_p + q * SEG * NC + tm * H;
-            int j = 0;
-            for (; j + 8 <= rows; j += 8) {
-                float xv[8], pv[8][H];
-#pragma unroll
-                for (int jj = 0; jj < 8; ++jj) {
-                    xv[jj] = xq[(j + jj) * kTpPitch];
-#pragma unroll
-                    for (int k = 0; k < H; ++k) pv[jj][k] = pq[(j + jj) * NC + k];
-                }
-#pragma unroll
-                for (int jj = 0; jj < 8; ++jj)
-#pragma unroll
-                    for (int k = 0; k < H; ++k) z[q][k] += pv[jj][k] * xv[jj];
-            }
-            for (; j < rows; ++j) {
-                const float xv = xq[j * kTpPitch];
-#pragma unroll
-                for (int k = 0; k < H; ++k) z[q][k] += pq[j * NC + k] * xv;
+            for (int c = 0; c < NC; ++c) {
+                const float pv = ptile[j * NC + c];
+                z[c][0] += pv * xv.x, z[c][1] += pv * xv.y;
             }
         }
+        wave_lds_handover();  // the tile is rewritten by the next chunk
     }
-    __syncthreads();
-    if (srow == 0 && wave < H) {
+    if (g < H && ship == 0) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t) s_l[seg * NC + t * H + wave] = run_sum[t];
+        for (int t = 0; t < 2; ++t) scale[NC + t * H + g] = run_sum[t];
     }
-    __syncthreads();
+    wave_lds_handover();
 #pragma unroll
-    for (int q = 0; q < EPP; ++q) {
-        if (env_first + q >= B) break;
-#pragma unroll
-        for (int k = 0; k < H; ++k) {
-            const float l = s_l[q * NC + tm * H + k];  // 0: no alive ship on this team
-            z_out[((int64_t)(env_first + q) * NC + tm * H + k) * kTpD + d] = l > 0.0f ? z[q][k] / l : 0.0f;
-        }
+    for (int c = 0; c < NC; ++c) {
+        const float l = scale[NC + c];  // 0: no alive ship on this team
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+        const f32x2 r = {z[c][0] * inv, z[c][1] * inv};
+        *reinterpret_cast<f32x2 *>(z_out + ((int64_t)env * NC + c) * kTpD + 2 * lane) = r;
     }
 }
 
@@ -242,7 +237,7 @@ __global__ __launch_bounds__(kTpThreads) void team_norm_broadcast_kernel(
 #pragma unroll
     for (int g = 0; g < kTpEnvs; ++g) {
         v[g] = env0 + g < B ? pre[((int64_t)(env0 + g) * 2 + tm) * kTpD + d] : 0.0f;
-        const float ss = seg_sum<64>(v[g] * v[g]);
+        const float ss = wave_sum(v[g] * v[g]);
         if (lane == 0) s_red[g * 4 + wave] = ss;
     }
     __syncthreads();
@@ -271,15 +266,14 @@ __global__ __launch_bounds__(kTpThreads) void team_norm_broadcast_kernel(
     }
 }
 
-template <int H, int SEG>
+template <int H>
 static int launch_team_attend(const float *x, int64_t x_env_stride, int64_t x_row_stride, const int32_t *team_id,
                               int64_t team_env_stride, const uint8_t *alive, int64_t alive_env_stride,
                               const float *score_vectors, float *z, int B, int N, hipStream_t s)
 {
-    constexpr int EPP = kTpChunk / SEG;
-    const int64_t blocks = ((int64_t)B + EPP - 1) / EPP;
+    const int64_t blocks = ((int64_t)B + kTaWaves - 1) / kTaWaves;
     if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((team_attend_kernel<H, SEG>), dim3((unsigned)blocks), dim3(kTpThreads), 0, s, x, x_env_stride,
+    hipLaunchKernelGGL((team_attend_kernel<H>), dim3((unsigned)blocks), dim3(kTaWaves * kWave), 0, s, x, x_env_stride,
                        x_row_stride, team_id, team_env_stride, alive, alive_env_stride, score_vectors, z, B, N);
     return (int)hipGetLastError();
 }
@@ -299,11 +293,11 @@ extern "C" int bnb_team_attend_fwd(const float *x, int64_t x_env_stride, int64_t
         return BNB_ERR_BAD_SHAPE;
     if (!aligned16(x) || (x_row_stride % 4) != 0 || (x_env_stride % 4) != 0) return BNB_ERR_MISALIGNED;
     hipStream_t s = (hipStream_t)stream;
-#define BNB_TP_ARGS x, x_env_stride, x_row_stride, team_id, team_env_stride, alive, alive_env_stride, score_vectors, z, B, N, s
-    // up to 16 ships: four environments share a work-group; otherwise one environment each
-    if (H == 4) return N <= 16 ? launch_team_attend<4, 16>(BNB_TP_ARGS) : launch_team_attend<4, 64>(BNB_TP_ARGS);
-    return N <= 16 ? launch_team_attend<2, 16>(BNB_TP_ARGS) : launch_team_attend<2, 64>(BNB_TP_ARGS);
-#undef BNB_TP_ARGS
+    if (H == 4)
+        return launch_team_attend<4>(x, x_env_stride, x_row_stride, team_id, team_env_stride, alive, alive_env_stride,
+                                     score_vectors, z, B, N, s);
+    return launch_team_attend<2>(x, x_env_stride, x_row_stride, team_id, team_env_stride, alive, alive_env_stride,
+                                 score_vectors, z, B, N, s);
 }
 
 extern "C" int bnb_team_norm_broadcast_fwd(const float *pre, const float *norm_weight, float eps, const int32_t *team_id,

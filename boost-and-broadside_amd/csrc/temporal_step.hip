@@ -42,15 +42,6 @@ static size_t ts_lds_bytes(int waves)
     return (size_t)kTsWeightHalfs * 2 + (size_t)kTsTableFloats * sizeof(float) + (size_t)waves * kTsTileHalfs * 2;
 }
 
-// LDS traffic between lanes of ONE wave: LDS operations of a wave complete in issue order, so
-// only the compiler has to be kept from moving accesses across the hand-over point.
-__device__ __forceinline__ void wave_lds_handover()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 __global__ __launch_bounds__(kTsMaxWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2))) void temporal_step_kernel(
     const uint16_t *__restrict__ b1, int64_t b1_group_stride, int64_t b1_row_stride, const float *conv_in,
     int64_t conv_in_stride, float *conv_out, int64_t conv_out_stride, const float *h_in, int64_t h_in_stride,
