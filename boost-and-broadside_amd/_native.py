@@ -61,7 +61,14 @@ _lib = None
 
 
 class NativeLibraryError(RuntimeError):
-    """The HIP library is missing, stale or returned an error code."""
+    """The HIP library is missing, stale or returned an error code (``code``, 0 when none)."""
+
+    def __init__(self, message: str, code: int = 0) -> None:
+        super().__init__(message)
+        self.code = code
+
+
+ERR_UNSUPPORTED = 10004  # BNB_ERR_UNSUPPORTED: a shape outside what the kernels cover
 
 
 def load() -> ctypes.CDLL:
@@ -92,4 +99,4 @@ def check(code: int, what: str) -> None:
     """Raise if an entry point returned a non-zero code."""
     if code != 0:
         msg = load().bnb_error_string(code).decode()
-        raise NativeLibraryError(f"{what} failed with code {code}: {msg}")
+        raise NativeLibraryError(f"{what} failed with code {code}: {msg}", code)

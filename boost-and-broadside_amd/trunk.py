@@ -31,7 +31,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from . import ops
+from . import _native, ops
 
 CONV_KERNEL = 4  # taps of the causal depthwise conv; the state keeps the last CONV_KERNEL-1 inputs
 
@@ -229,7 +229,14 @@ class TransformerBlock(nn.Module):
                 kv = self.kv_bullet(self.norm_bullet(bullets))
                 merged = merged + self._bullet_read(qkv, kv, bullet_mask)
             return self.out_proj(merged)
-        merged = ops.sdpa_masked(qkv, alive_mask, self.n_heads)  # (B, N, D) head-major
+        try:
+            merged = ops.sdpa_masked(qkv, alive_mask, self.n_heads)  # (B, N, D) head-major
+        except _native.NativeLibraryError as err:
+            if err.code != _native.ERR_UNSUPPORTED:
+                raise
+            # a shape the kernels do not cover (head sizes other than 8/16/32/64, more than 512
+            # tokens, float32 keys beyond what fits LDS): the library's attention on the device
+            merged = self._self_attention_autograd(qkv, alive_mask)
         if self.reads_bullets and bullets is not None:
             rows = bullet_mask if isinstance(bullet_mask, ops.CompactRows) else None
             if rows is None and bullet_mask is not None and self._compact_read_ok(qkv, bullets):

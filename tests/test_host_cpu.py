@@ -42,6 +42,7 @@ def test_header_constants_match_loader():
     text = open(os.path.join(ROOT, "include", "bnb_amd.h")).read()
     consts = dict(re.findall(r"#define\s+(BNB_[A-Z0-9_]+)\s+(\d+)", text))
     assert int(consts["BNB_ABI_VERSION"]) == _native.ABI_VERSION
+    assert int(consts["BNB_ERR_UNSUPPORTED"]) == _native.ERR_UNSUPPORTED
     assert (int(consts["BNB_F32"]), int(consts["BNB_BF16"])) == (_native.F32, _native.BF16)
     assert [int(consts[f"BNB_SDPA_PATH_{n}"]) for n in ("AUTO", "VALU", "MFMA")] == [0, 1, 2]
 

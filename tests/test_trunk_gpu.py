@@ -523,3 +523,22 @@ def test_team_pooling_layer_trains_through_the_library_path():
     ref, _ = torch_ref.team_pool({k: v.double() for k, v in p.items()}, "tp.", xr, team, alive, H)
     ref.square().sum().backward()
     assert max_rel(x.grad.cpu(), xr.grad.float()) <= 1e-4
+
+
+def test_attention_block_outside_kernel_coverage_uses_the_library_on_the_device():
+    # head size 24 is not one the kernels cover: the block must still compute the reference's function
+    D, H, B, N = 96, 4, 3, 10
+    g = torch.Generator().manual_seed(31)
+    blk = bnb.TransformerBlock(_cfg(D=D, H=H)).to(DEV).eval()
+    x = torch.randn(B, N, D, generator=g)
+    alive = torch.rand(B, N, generator=g) < 0.7
+    alive[0] = False
+    with torch.no_grad():
+        got = blk(x.to(DEV), alive.to(DEV)).cpu()
+    sd = {"s." + k: v.detach().cpu() for k, v in blk.state_dict().items()}
+    ref = torch_ref.spatial_sublayer(sd, "s.", x, alive, H)
+    assert max_rel(got, ref) <= 1e-5
+    from boost_and_broadside_amd import _native
+    with pytest.raises(_native.NativeLibraryError) as err:
+        bnb.ops.sdpa_masked(torch.zeros(1, 4, 3 * D, device=DEV), None, H)
+    assert err.value.code == _native.ERR_UNSUPPORTED
