@@ -562,6 +562,181 @@ __global__ __launch_bounds__(kWave) void sdpa_mfma_pair_kernel(
 }
 
 // ------------------------------------------------------------------------------------
+// fp32 on the matrix cores (dh = 32, up to 512 tokens): evaluation without autocast
+// ------------------------------------------------------------------------------------
+//
+// v_mfma_f32_32x32x2_f32 takes one fp32 per lane for A and for B (row / column l%32, k = l/32)
+// and accumulates in fp32, so the result meets the fp32 bar while the products leave the
+// vector ALUs (which the fp32 vector kernel saturates from ~64 tokens on).  Same formulation
+// as sdpa_mfma_kernel: one work-group per (environment, head), wave w owns queries 32w..32w+31,
+// live keys compacted to the end of the staged positions, S^T = K Q^T with keys on the M axis.
+// Differences that the operand shape allows:
+//   * the k index of a product may run in any order as long as A and B agree, so K Q^T walks
+//     channel 16*half + s at step s (a lane's 16 query values are one contiguous 64-byte load,
+//     K rows sit in LDS at an odd pitch) and V^T P^T walks key 8(s/4) + 4*half + s%4 -- exactly
+//     the key whose score the lane holds in accumulator register s, so P never moves and V is
+//     read from LDS as stored (32 consecutive channels per key: no transposed copy);
+//   * one sweep with a running maximum (the matrix cores are the bound here, 32 MFMAs of 64
+//     cycles per key block, and rescaling 16 accumulators per block is free next to that).
+constexpr int kF32KeyPitch = kDh + 1;  // floats per K row in LDS: odd, so 32 rows hit 32 banks
+
+__global__ __launch_bounds__(1024) void sdpa_mfma_f32_kernel(
+    const float *__restrict__ qkv, int64_t stride, const uint8_t *__restrict__ alive, float *__restrict__ out, int B,
+    int NM, int H, float scale_log2e)
+{
+    extern __shared__ __align__(16) float s_f32[];
+    const int nwaves = blockDim.x >> 6;
+    const int kcap = nwaves * 32;
+    float *s_k = s_f32;                         // [kcap][33]
+    float *s_v = s_k + kcap * kF32KeyPitch;     // [kcap][32]
+    int *s_cnt = reinterpret_cast<int *>(s_v + kcap * kDh);  // [2 * nwaves]
+
+    const int chunk = gridDim.x >> 3;
+    const int logical = (blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
+    if (logical >= B * H) return;
+    const int env = logical / H;
+    const int head = logical - env * H;
+    const int D = H * kDh;
+    const int tid = threadIdx.x;
+    const int NT = blockDim.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m = lane & 31;
+    const int half = lane >> 5;
+    const float *base = qkv + (int64_t)env * NM * stride;
+
+    // this lane's query values: channels 16*half .. +15 of query 32*wave + m
+    const int qrow = wave * 32 + m;
+    const float *qp = base + (int64_t)(qrow < NM ? qrow : NM - 1) * stride + head * kDh + 16 * half;
+    f32x4 qv[4];
+
+    // ---- K and V rows of the live keys into LDS, compacted (thread = key, 8 channels; two items) ----
+    const uint8_t *alive_env = alive == nullptr ? nullptr : alive + (int64_t)env * NM;
+    int cnt = 0;
+    bool uniform = false;
+    for (int pass = 0; pass < 2; ++pass) {
+        bool live[2];
+        f32x4 kw[2][2], vw[2][2];
+        uint32_t ab[2] = {1u, 1u};
+        if (alive_env != nullptr && !uniform) {
+#pragma unroll
+            for (int it = 0; it < 2; ++it) {
+                const int key = (tid + it * NT) >> 2;
+                ab[it] = alive_env[key < NM ? key : NM - 1];
+            }
+        }
+        const float *k_base = base + D + head * kDh + (tid & 3) * 8;
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int key = (tid + it * NT) >> 2;
+            live[it] = key < NM && ab[it] != 0;
+            const float *kp = k_base + (int64_t)(live[it] ? key : 0) * stride;
+            kw[it][0] = *reinterpret_cast<const f32x4 *>(kp);
+            kw[it][1] = *reinterpret_cast<const f32x4 *>(kp + 4);
+            vw[it][0] = *reinterpret_cast<const f32x4 *>(kp + D);
+            vw[it][1] = *reinterpret_cast<const f32x4 *>(kp + D + 4);
+        }
+        if (pass == 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) qv[i] = *reinterpret_cast<const f32x4 *>(qp + 4 * i);
+        }
+        int before[2];
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const uint64_t mask = __ballot(live[it] && (lane & 3) == 0);  // one bit per live key
+            before[it] = __popcll(mask & ((1ull << (lane & ~3)) - 1ull));
+            if (lane == 0) s_cnt[it * nwaves + wave] = (int)__popcll(mask);
+        }
+        __syncthreads();
+        int base0 = 0, base1 = 0;
+        cnt = 0;
+        for (int ch = 0; ch < 2 * nwaves; ++ch) {
+            const int c = s_cnt[ch];
+            if (ch < wave) base0 += c;
+            if (ch < nwaves + wave) base1 += c;
+            cnt += c;
+        }
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            if (live[it]) {
+                // live keys fill the END of the nkb*32 positions; the padding sits in front
+                const int pos = (((cnt + 31) & ~31) - cnt) + (it ? base1 : base0) + before[it];
+                const int c8 = (tid & 3) * 8;
+                float *kd = s_k + pos * kF32KeyPitch + c8;
+                kd[0] = kw[it][0].x, kd[1] = kw[it][0].y, kd[2] = kw[it][0].z, kd[3] = kw[it][0].w;
+                kd[4] = kw[it][1].x, kd[5] = kw[it][1].y, kd[6] = kw[it][1].z, kd[7] = kw[it][1].w;
+                *reinterpret_cast<f32x4 *>(s_v + pos * kDh + c8) = vw[it][0];
+                *reinterpret_cast<f32x4 *>(s_v + pos * kDh + c8 + 4) = vw[it][1];
+            }
+        }
+        if (cnt != 0) break;
+        // no live key at all: every key takes part with the same weight; stage them all
+        uniform = true;
+        __syncthreads();  // s_cnt is rewritten by the second pass
+    }
+    const int nkb = (cnt + 31) >> 5;
+    const int pad = nkb * 32 - cnt;  // positions [0, pad) of key block 0 hold no key
+    for (int idx = tid; idx < pad * kDh; idx += NT) {
+        const int pos = idx >> 5, c = idx & 31;
+        s_k[pos * kF32KeyPitch + c] = 0.0f;
+        s_v[pos * kDh + c] = 0.0f;
+    }
+    __syncthreads();
+    if (wave * 32 >= NM) return;  // waves that only helped staging
+
+    // with no live key every score is the same constant: zero queries give exactly that
+    float q[16];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        q[4 * i + 0] = uniform ? 0.0f : qv[i].x, q[4 * i + 1] = uniform ? 0.0f : qv[i].y;
+        q[4 * i + 2] = uniform ? 0.0f : qv[i].z, q[4 * i + 3] = uniform ? 0.0f : qv[i].w;
+    }
+
+    float run_max = -INFINITY, sum = 0.0f;
+    f32x16 o = {0.0f};
+    for (int kb = 0; kb < nkb; ++kb) {
+        f32x16 z = {0.0f};
+        if (kb == 0) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) z[v] = (8 * (v >> 2) + 4 * half + (v & 3) < pad) ? -INFINITY : 0.0f;
+        }
+        const float *kp = s_k + (kb * 32 + m) * kF32KeyPitch + 16 * half;
+#pragma unroll
+        for (int st = 0; st < 16; ++st) z = __builtin_amdgcn_mfma_f32_32x32x2f32(kp[st], q[st], z, 0, 0, 0);
+        float bmax = z[0];
+#pragma unroll
+        for (int v = 1; v < 16; ++v) bmax = fmaxf(bmax, z[v]);
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 32));
+        const float new_max = fmaxf(run_max, bmax);  // finite: every key block holds at least one live key
+        const float alpha = __builtin_amdgcn_exp2f((run_max - new_max) * scale_log2e);
+        run_max = new_max;
+        const float mc = new_max * scale_log2e;
+        sum *= alpha;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            o[v] *= alpha;
+            z[v] = __builtin_amdgcn_exp2f(fmaf(z[v], scale_log2e, -mc));
+            sum += z[v];
+        }
+        // V^T P^T: step st pairs accumulator register st (key 8(st/4) + 4*half + st%4) with that key's V row
+        const float *vp = s_v + (kb * 32 + 4 * half) * kDh + m;
+#pragma unroll
+        for (int st = 0; st < 16; ++st)
+            o = __builtin_amdgcn_mfma_f32_32x32x2f32(vp[(8 * (st >> 2) + (st & 3)) * kDh], z[st], o, 0, 0, 0);
+    }
+    sum += __shfl_xor(sum, 32);
+    const float inv = 1.0f / sum;
+    if (qrow < NM) {
+        // the lane holds channels 8a + 4*half + b (a, b = 0..3) of its query: four 16-byte pieces
+        float *op = out + ((int64_t)env * NM + qrow) * D + head * kDh + 4 * half;
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+            *reinterpret_cast<f32x4 *>(op + 8 * a) =
+                f32x4{o[4 * a + 0] * inv, o[4 * a + 1] * inv, o[4 * a + 2] * inv, o[4 * a + 3] * inv};
+    }
+}
+
+// ------------------------------------------------------------------------------------
 // Streaming MFMA kernel for the bullet read with many keys (bf16, dh = 32)
 // ------------------------------------------------------------------------------------
 //
@@ -998,6 +1173,27 @@ extern "C" int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride,
                                     B, NM, NM, H, s);
     }
     if (dtype == BNB_BF16) return dispatch_valu<uint16_t>(qkv, qkv_row_stride, alive, out, B, NM, H, dh, s);
+    // fp32, head size 32, more than one tile of tokens: the fp32 matrix-core kernel (measured against the
+    // vector kernel at 1024 environments: 84 tokens 129 -> 51 us, 160 tokens 404 -> 139 us, 320 tokens x 256
+    // environments 855 -> 132 us); taken by AUTO, the VALU path stays the vector kernel
+    if (dh == kDh && NM > 32 && path != BNB_SDPA_PATH_VALU && (int64_t)NM * qkv_row_stride < (1LL << 31)) {
+        const int nwaves = (NM + 31) / 32;
+        const size_t lds = (size_t)nwaves * 32 * (kF32KeyPitch + kDh) * sizeof(float) + (size_t)2 * nwaves * sizeof(int);
+        if (lds <= kLdsMax) {
+            const int64_t pairs = (int64_t)B * H;
+            const int64_t blocks = (pairs + 7) / 8 * 8;
+            if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+            if (lds > kLdsDefault) {
+                const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(sdpa_mfma_f32_kernel),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsMax);
+                if (e != hipSuccess) return (int)e;
+            }
+            hipLaunchKernelGGL(sdpa_mfma_f32_kernel, dim3((unsigned)blocks), dim3(nwaves * kWave), lds, s,
+                               (const float *)qkv, qkv_row_stride, alive, (float *)out, B, NM, H,
+                               kLog2eA / sqrtf((float)kDh));
+            return (int)hipGetLastError();
+        }
+    }
     return dispatch_valu<float>(qkv, qkv_row_stride, alive, out, B, NM, H, dh, s);
 }
 

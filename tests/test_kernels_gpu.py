@@ -59,6 +59,38 @@ def test_sdpa_fp32_matches_oracle(B, NM, H, dh):
         assert max_rel(got, cc) <= F32_TOL
 
 
+@pytest.mark.parametrize("NM", [33, 63, 64, 65, 100, 160, 161, 255, 320, 512])
+def test_sdpa_fp32_matrix_core_kernel_matches_oracle_and_the_vector_kernel(NM):
+    # fp32 with head size 32 and more than 32 tokens runs on the fp32 matrix-core kernel (AUTO);
+    # path="valu" forces the vector kernel on the same inputs
+    B, H, D = 5, 4, 128
+    qkv = _qkv(NM * 3, B, NM, D, torch.float32, scale=1.5)
+    alive = _alive(NM, B, NM, 0.6)
+    alive[0] = True
+    alive[1] = False            # nobody alive: mean of V
+    alive[2] = False
+    alive[2, NM - 1] = True     # a single key
+    got = _run_sdpa(qkv, alive, H)
+    ref = torch_ref.sdpa_masked(qkv, alive, H)
+    assert max_rel(got, ref) <= F32_TOL
+    assert torch.allclose(got, ref, rtol=1e-4, atol=2e-6)
+    assert max_rel(got, _run_sdpa(qkv, alive, H, "valu")) <= F32_TOL
+    assert (got[1] - qkv[1, :, 2 * D:].mean(dim=0, keepdim=True)).abs().max() <= 2e-6
+    assert torch.allclose(got[2], qkv[2, NM - 1, 2 * D:].expand(NM, D), atol=1e-6)
+    # dead keys weigh exactly nothing
+    pert = qkv.clone()
+    dead = ~alive
+    dead[1] = False
+    pert[..., D:][dead] = pert[..., D:][dead] * -3.0 + 17.0
+    assert torch.equal(_run_sdpa(pert, alive, H), got)
+    # padded rows (a view of a wider buffer) and no mask at all
+    wide = torch.zeros(B, NM, 3 * D + 64)
+    wide[..., : 3 * D] = qkv
+    view = wide.to(DEV)[..., : 3 * D]
+    assert torch.equal(ops.sdpa_masked(view, alive.to(DEV), H).cpu(), got)
+    assert max_rel(_run_sdpa(qkv, None, H), torch_ref.sdpa_masked(qkv, None, H)) <= F32_TOL
+
+
 def test_sdpa_fp32_large_scores_stay_exact():
     # scores of magnitude ~50 exercise the running-max rescaling
     qkv = _qkv(5, 4, 23, 128, torch.float32, scale=3.0)
