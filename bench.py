@@ -43,6 +43,7 @@ def parse_args():
     ap.add_argument("--no-bullets", action="store_true", help="skip the bullet-read leg")
     ap.add_argument("--no-sequence", action="store_true", help="skip the update-path (T = 128) recurrence leg")
     ap.add_argument("--no-team-pool", action="store_true", help="skip the team pooling leg")
+    ap.add_argument("--no-fp32-attention", action="store_true", help="skip the float32 attention leg")
     ap.add_argument("--no-trunk", action="store_true", help="skip the whole-trunk leg (2 blocks x (2 spatial + 1 temporal))")
     return ap.parse_args()
 
@@ -566,6 +567,33 @@ def main():
                     "mask, Q, accumulator in and out; exp-throughput-bound rather than HBM-bound when many bullets are live",
         }
         del kv_b, b_mask, merged
+
+    # ---- fp32 attention at an evaluation shape (crossover runs without autocast), kernel beside the library ----
+    if not args.no_fp32_attention:
+        Be, NMe = 1024, 160
+        qkv_e = torch.randn(Be, NMe, 3 * D, device=dev, generator=gen)
+        alive_e = torch.rand(Be, NMe, device=dev, generator=gen) < 0.7
+        alive_e[:, 0] = True
+        n_e = max(4, min(steps, 16))
+        t_e = timed_loop(lambda t: ops.sdpa_masked(qkv_e, alive_e, H), n_e, 3) / n_e
+        t_e_valu = timed_loop(lambda t: ops.sdpa_masked(qkv_e, alive_e, H, path="valu"), n_e, 3) / n_e
+
+        def attention_library(t):
+            q, k, v = (a.reshape(Be, NMe, H, D // H).transpose(1, 2) for a in qkv_e.split(D, dim=-1))
+            bias = (1.0 - alive_e.reshape(Be, 1, 1, NMe).float()) * (torch.finfo(torch.float32).min / 2)
+            return F.scaled_dot_product_attention(q, k, v, attn_mask=bias).transpose(1, 2).reshape(Be, NMe, D)
+
+        t_e_lib = None if args.no_torch_baseline else timed_loop(attention_library, n_e, 3) / n_e
+        flops_e = 4.0 * Be * NMe * NMe * D
+        result["fp32_attention_kernel"] = {
+            "environments": Be, "tokens": NMe, "avg_launch_us": t_e * 1e6, "tflops": flops_e / t_e / 1e12,
+            "frac_of_fp32_mfma_peak": flops_e / t_e / 157.3e12, "vector_kernel_us": t_e_valu * 1e6,
+            "eager_torch_us": None if t_e_lib is None else t_e_lib * 1e6,
+            "what": "masked attention in float32 on v_mfma_f32_32x32x2_f32 (flops counted over all keys, 70 % of them "
+                    "alive); vector_kernel = the float32 vector-ALU kernel on the same input; eager = torch SDPA with the "
+                    "additive key bias and the head-merge copy",
+        }
+        del qkv_e
 
     # ---- team pooling over the ships (the value head's input), kernel beside the library composition ----
     if not args.no_team_pool:
