@@ -355,7 +355,7 @@ def main():
             "traffic": load_traffic(kernel, w.name),
         }
 
-    attn_kernel = "sdpa_valu_kernel"
+    attn_kernel = "sdpa_mfma_f32_kernel" if D // H == 32 else "sdpa_valu_kernel"
     if bf16 and w.NM <= 160:
         attn_kernel = "sdpa_mfma_pair_kernel" if (w.NM <= 16 and H % 2 == 0) else "sdpa_mfma_kernel"
     roofs = {"attention": roof(attn_kernel, ab["attn"], t_attn), "rglru": roof("rglru_step_vec8_kernel", ab["rglru"], t_rglru)}

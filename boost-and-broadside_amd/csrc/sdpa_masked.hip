@@ -1173,10 +1173,10 @@ extern "C" int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride,
                                     B, NM, NM, H, s);
     }
     if (dtype == BNB_BF16) return dispatch_valu<uint16_t>(qkv, qkv_row_stride, alive, out, B, NM, H, dh, s);
-    // fp32, head size 32, more than one tile of tokens: the fp32 matrix-core kernel (measured against the
+    // fp32, head size 32: the fp32 matrix-core kernel (no slower at 12 tokens, and measured against the
     // vector kernel at 1024 environments: 84 tokens 129 -> 51 us, 160 tokens 404 -> 139 us, 320 tokens x 256
     // environments 855 -> 132 us); taken by AUTO, the VALU path stays the vector kernel
-    if (dh == kDh && NM > 32 && path != BNB_SDPA_PATH_VALU && (int64_t)NM * qkv_row_stride < (1LL << 31)) {
+    if (dh == kDh && NM > 0 && path != BNB_SDPA_PATH_VALU && (int64_t)NM * qkv_row_stride < (1LL << 31)) {
         const int nwaves = (NM + 31) / 32;
         const size_t lds = (size_t)nwaves * 32 * (kF32KeyPitch + kDh) * sizeof(float) + (size_t)2 * nwaves * sizeof(int);
         if (lds <= kLdsMax) {

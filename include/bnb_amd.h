@@ -78,7 +78,7 @@ int bnb_sdpa_masked_fwd(const void *qkv, int64_t qkv_row_stride, const uint8_t *
  * counterpart beyond the one above.
  *   BNB_SDPA_PATH_AUTO  what bnb_sdpa_masked_fwd does: the bf16 matrix-core kernel for bf16,
  *                       dh == 32 and NM <= 160; the fp32 matrix-core kernel for fp32, dh == 32
- *                       and 32 < NM <= 512; the vector-ALU kernel otherwise
+ *                       and NM <= 512; the vector-ALU kernel otherwise
  *   BNB_SDPA_PATH_VALU  vector-ALU kernel (any supported shape and dtype)
  *   BNB_SDPA_PATH_MFMA  bf16 matrix-core kernel (bf16, dh == 32, NM <= 160; else BNB_ERR_UNSUPPORTED)
  */
