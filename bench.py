@@ -684,6 +684,50 @@ def main():
         }
         del xs, gs, hs, dn, leaves
 
+        # weight gradients of the trunk's Linear layers over a stored rollout: rows = T x environments x tokens
+        if bf16:
+            Rw = 128 * 256 * 12  # T = 128, 256 environments of 4v4 (8 ships + 4 fields)
+            wg = {}
+            for name, (Nw, Kw) in (("qkv", (3 * D, D)), ("square", (D, D)), ("gate_or_up", (4 * D, D)), ("down", (D, 4 * D))):
+                dy_w = torch.randn(Rw, Nw, device=dev, generator=gen).to(torch.bfloat16)
+                x_w = torch.randn(Rw, Kw, device=dev, generator=gen).to(torch.bfloat16)
+                dw = torch.empty(Nw, Kw, device=dev)
+                t_w = timed_loop(lambda t: ops.linear_wgrad(dy_w, x_w, out=dw), 8, 3) / 8
+                t_w_lib = None if args.no_torch_baseline else timed_loop(lambda t: torch.mm(dy_w.t(), x_w), 4, 2) / 4
+                by = Rw * (Nw + Kw) * 2 + Nw * Kw * 4
+                wg[name] = {"N": Nw, "K": Kw, "us": t_w * 1e6, "algorithmic_bytes": by, "GBps": by / t_w / 1e9,
+                            "frac_of_hbm_peak": by / t_w / peak, "tflops": 2.0 * Rw * Nw * Kw / t_w / 1e12,
+                            "library_us": None if t_w_lib is None else t_w_lib * 1e6}
+                del dy_w, x_w, dw
+            cfg_u = bnb.ModelConfig(d_model=D, n_heads=H, n_yemong_blocks=1, n_spatial_per_block=2, n_temporal_per_block=1)
+            torch.manual_seed(w.seed)
+            blk = bnb.YemongBlock(cfg_u).to(dev)
+            Tu, Bu, Nu, Mu = 128, 256, 8, 4
+            xu = torch.randn(Tu, Bu, Nu + Mu, D, device=dev, generator=gen)
+            au = torch.rand(Tu, Bu, Nu + Mu, device=dev, generator=gen) < 0.9
+            hu = torch.zeros(1, Bu * Nu, D, device=dev)
+            cu = torch.zeros(1, Bu * Nu, 3, D, device=dev)
+            du = torch.rand(Tu, Bu, device=dev, generator=gen) < 0.02
+
+            def update_step(t):
+                blk.zero_grad(set_to_none=True)
+                with torch.enable_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+                    out_u = blk.sequence(xu, au, hu, cu, du, num_recurrent=Nu)[0]
+                out_u.float().square().mean().backward()
+
+            from boost_and_broadside_amd import trunk as trunk_module
+            t_up = timed_loop(update_step, 3, 2) / 3
+            with trunk_module.library_weight_gradients():
+                t_up_lib = timed_loop(update_step, 3, 2) / 3
+            result["update_path"] = {
+                "rows": Rw, "linear_wgrad": wg, "block_fwd_bwd_ms": t_up * 1e3, "block_fwd_bwd_library_wgrad_ms": t_up_lib * 1e3,
+                "what": "bnb_linear_wgrad_fwd (dW = dy^T x, bf16 in, fp32 out, rows split over the chip) beside the library "
+                        "GEMM on the same operands; block = one YemongBlock (2 attention + 1 temporal sublayer), T = 128 x 256 "
+                        "environments of 4v4, forward + backward under bf16 autocast, with the weight gradients on that "
+                        "kernel and on the library",
+            }
+            del blk, xu, au, hu, cu, du
+
     # ---- whole trunk (reference default: 2 blocks x (2 spatial + 1 temporal)), state carried ----
     if not args.no_trunk:
         cfg = bnb.ModelConfig(d_model=D, n_heads=H, n_yemong_blocks=2, n_spatial_per_block=2, n_temporal_per_block=1)

@@ -372,6 +372,80 @@ def conv_step(
     return (v, conv_out, v_lp) if also_bf16 else (v, conv_out)
 
 
+def linear_wgrad_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether ``linear_wgrad`` covers this layer: GPU, both weight dimensions multiples of 128."""
+    return x.is_cuda and weight.dim() == 2 and weight.shape[0] % 128 == 0 and weight.shape[1] % 128 == 0
+
+
+def linear_wgrad(dy: torch.Tensor, x: torch.Tensor, out: torch.Tensor | None = None, accumulate: bool = False) -> torch.Tensor:
+    """``dW = dy^T x`` for a Linear layer: ``dy`` (..., N) and ``x`` (..., K) bfloat16 with the same
+    leading shape, result (N, K) float32 (``out`` is overwritten, or added to with ``accumulate``).
+    Rows are reduced in a fixed order, so repeated calls give identical bits."""
+    N, K = dy.shape[-1], x.shape[-1]
+    if dy.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
+        raise TypeError("dy and x must be bfloat16")
+    if dy.shape[:-1] != x.shape[:-1]:
+        raise ValueError(f"dy {tuple(dy.shape)} and x {tuple(x.shape)} must share their leading shape")
+    if N % 128 or K % 128:
+        raise ValueError("linear_wgrad covers weight shapes whose dimensions are multiples of 128")
+    _need_device(dy, "dy")
+    _need_device(x, "x")
+    dy2 = dy.reshape(-1, N) if _uniform_rows(dy, N) else dy.reshape(-1, N).contiguous()
+    x2 = x.reshape(-1, K) if _uniform_rows(x, K) else x.reshape(-1, K).contiguous()
+    R = dy2.shape[0]
+    if out is None:
+        if accumulate:
+            raise ValueError("accumulate needs an existing out tensor")
+        out = torch.empty((N, K), dtype=torch.float32, device=dy.device)
+    elif out.shape != (N, K) or out.dtype != torch.float32 or not out.is_contiguous() or out.device != dy.device:
+        raise ValueError("out must be a contiguous float32 (N, K) tensor on dy's device")
+    lib = _native.load()
+    slices = int(lib.bnb_linear_wgrad_slices(R, N, K))
+    partials = torch.empty((slices, N, K), dtype=torch.float32, device=dy.device)
+    with torch.cuda.device(dy.device):
+        rc = lib.bnb_linear_wgrad_fwd(dy2.data_ptr(), dy2.stride(0) if R else N, x2.data_ptr(), x2.stride(0) if R else K,
+                                      partials.data_ptr(), slices, out.data_ptr(), int(bool(accumulate)), R, N, K, _stream())
+    _native.check(rc, "bnb_linear_wgrad_fwd")
+    return out
+
+
+class _LinearTrain(torch.autograd.Function):
+    """``F.linear`` under bfloat16 autocast whose weight gradient runs on ``linear_wgrad``."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        xb = x if x.dtype == torch.bfloat16 else x.to(torch.bfloat16)
+        wb = weight.to(torch.bfloat16)
+        ctx.save_for_backward(xb, wb)
+        ctx.x_dtype = x.dtype
+        ctx.has_bias = bias is not None
+        return torch.nn.functional.linear(xb, wb, None if bias is None else bias.to(torch.bfloat16))
+
+    @staticmethod
+    def backward(ctx, dy):
+        xb, wb = ctx.saved_tensors
+        dy = dy.contiguous() if dy.stride(-1) != 1 else dy
+        dyb = dy if dy.dtype == torch.bfloat16 else dy.to(torch.bfloat16)
+        dx = dw = db = None
+        if ctx.needs_input_grad[0]:
+            dx = torch.matmul(dyb, wb)
+            if dx.dtype != ctx.x_dtype:
+                dx = dx.to(ctx.x_dtype)
+        if ctx.needs_input_grad[1]:
+            dw = linear_wgrad(dyb, xb)
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            db = dyb.reshape(-1, dyb.shape[-1]).sum(dim=0, dtype=torch.float32)
+        return dx, dw, db
+
+
+def linear_train(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None) -> torch.Tensor:
+    """``F.linear(x, weight, bias)`` as bfloat16 autocast computes it, differentiable, with the weight
+    gradient accumulated in float32 by ``linear_wgrad`` instead of a library GEMM that contracts
+    over the (very long) row axis.  Use where ``linear_wgrad_supported`` holds."""
+    with torch.autocast("cuda", enabled=False):
+        return _LinearTrain.apply(x, weight, bias)
+
+
 def pack_team_pool_weights(seeds: torch.Tensor, in_proj_weight: torch.Tensor, out_proj_weight: torch.Tensor,
                            n_heads: int) -> tuple[torch.Tensor, torch.Tensor]:
     """The constants ``team_pool`` needs, from TeamPMA's parameters (policy.py:88-92), float32:

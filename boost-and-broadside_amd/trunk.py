@@ -25,6 +25,7 @@ tensors that need gradients and they refuse to run off-GPU.
 
 from __future__ import annotations
 
+import contextlib
 from dataclasses import dataclass
 
 import torch
@@ -36,6 +37,7 @@ from . import _native, ops
 CONV_KERNEL = 4  # taps of the causal depthwise conv; the state keeps the last CONV_KERNEL-1 inputs
 
 _FUSED_WIDTHS = (8, 16, 32, 64, 128, 256, 512)  # d_model values the fused norm kernel covers
+_WGRAD_MIN_ROWS = 8192  # below this many rows the library's weight-gradient GEMM is as fast as ops.linear_wgrad
 
 
 def _projection_dtype() -> torch.dtype:
@@ -52,6 +54,17 @@ def _fused_ok(x: torch.Tensor, act: torch.dtype) -> bool:
         not torch.is_grad_enabled() and x.is_cuda and x.dtype == torch.float32 and x.shape[-1] in _FUSED_WIDTHS
         and act in (torch.float32, torch.bfloat16)
     )
+
+
+@contextlib.contextmanager
+def library_weight_gradients():
+    """Inside the block every Linear weight gradient is left to the library GEMM (comparisons, debugging)."""
+    global _WGRAD_MIN_ROWS
+    keep, _WGRAD_MIN_ROWS = _WGRAD_MIN_ROWS, 1 << 62
+    try:
+        yield
+    finally:
+        _WGRAD_MIN_ROWS = keep
 
 
 def _cached_cast(owner: nn.Module, slot: str, tensors: tuple, dtype: torch.dtype, build):
@@ -71,6 +84,11 @@ def _project(layer: nn.Linear, x: torch.Tensor) -> torch.Tensor:
     """``layer(x)`` for an activation that already has the projection dtype."""
     w, b = layer.weight, layer.bias
     if torch.is_grad_enabled():
+        if (
+            w.requires_grad and w.dtype == torch.float32 and _projection_dtype() == torch.bfloat16
+            and x.numel() >= _WGRAD_MIN_ROWS * x.shape[-1] and ops.linear_wgrad_supported(x, w)
+        ):
+            return ops.linear_train(x, w, b)  # bf16 like autocast; weight gradient on the row-sliced kernel
         return layer(x)  # training: autocast's own (differentiable) casts
     if x.dtype == w.dtype:
         return F.linear(x, w, b)
@@ -157,7 +175,7 @@ class GatedMLP(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         hidden = self.gate_proj.out_features
         if not x.is_cuda or hidden % 8 or x.dtype not in (torch.float32, torch.bfloat16) or torch.is_grad_enabled():
-            return self.down_proj(F.gelu(self.gate_proj(x)) * self.up_proj(x))
+            return _project(self.down_proj, F.gelu(_project(self.gate_proj, x)) * _project(self.up_proj, x))
         # one GEMM for [gate | up], one kernel for gelu(gate) * up, one GEMM down
         wg, wu = self.gate_proj.weight, self.up_proj.weight
         w = _cached_cast(self, "_bnb_gate_up", (wg, wu), x.dtype, lambda: torch.cat([wg, wu], dim=0).detach().to(x.dtype))
@@ -226,9 +244,9 @@ class TransformerBlock(nn.Module):
             if self.reads_bullets and bullets is not None:
                 if isinstance(bullet_mask, ops.CompactRows):
                     bullet_mask = bullet_mask.mask
-                kv = self.kv_bullet(self.norm_bullet(bullets))
+                kv = _project(self.kv_bullet, self.norm_bullet(bullets))
                 merged = merged + self._bullet_read(qkv, kv, bullet_mask)
-            return self.out_proj(merged)
+            return _project(self.out_proj, merged)
         try:
             merged = ops.sdpa_masked(qkv, alive_mask, self.n_heads)  # (B, N, D) head-major
         except _native.NativeLibraryError as err:
@@ -321,7 +339,7 @@ class RGLRU(nn.Module):
 
         ``x_act``: the same rows already in the projection dtype (saves the cast)."""
         if torch.is_grad_enabled():
-            return torch.cat([self.linear_a(x), self.linear_x(x)], dim=-1)
+            return torch.cat([_project(self.linear_a, x), _project(self.linear_x, x)], dim=-1)
         act = _projection_dtype()
         if x_act is None or x_act.dtype != act:
             x_act = x.to(act)
@@ -405,7 +423,7 @@ class GriffinTemporalBlock(nn.Module):
         """Training path: torch ops (differentiable) around the recurrence, which runs on its
         forward and backward kernels."""
         normed = self.norm1(x_seq)
-        b1 = self.linear1(normed)
+        b1 = _project(self.linear1, normed)
         rows_first = b1.transpose(0, 1) if time_major else b1  # (R, T, D) view
         T = rows_first.shape[1]
         padded = torch.cat([conv_buf, rows_first], dim=1)  # fp32 buffer promotes a bf16 b1
@@ -440,7 +458,7 @@ class GriffinTemporalBlock(nn.Module):
                 return fused
             x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=r, eps=self.norm2.eps, out_dtype=act)
             return x1 + self.gated_mlp(n2)
-        x1 = x + self.linear_out(y * F.gelu(gate_in))
+        x1 = x + _project(self.linear_out, y * F.gelu(gate_in))
         return x1 + self.gated_mlp(self.norm2(x1))
 
     def _step(self, x, h_in, conv_in, h_out, conv_out, reset, rows_per_env):
@@ -559,7 +577,7 @@ class GriffinTemporalBlock(nn.Module):
                 return fused
             x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=r, eps=self.norm2.eps, out_dtype=act)
             return x1 + self.gated_mlp(n2)
-        x1 = x + self.linear_out(b1 * F.gelu(gate_in))
+        x1 = x + _project(self.linear_out, b1 * F.gelu(gate_in))
         return x1 + self.gated_mlp(self.norm2(x1))
 
 

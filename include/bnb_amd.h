@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 15
+#define BNB_ABI_VERSION 16
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -238,6 +238,31 @@ int bnb_conv_step_rows_fwd(const void *b1, int b1_dtype, int64_t b1_group_stride
                            const uint8_t *reset, int rows_per_env,
                            float *v_out, void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride,
                            int64_t R, int D, void *stream);
+
+/*
+ * Weight gradient of a bias-free or biased Linear layer:  dw[n][k] (+)= sum_r dy[r][n] * x[r][k],
+ * bf16 operands, fp32 accumulation on the matrix cores, fp32 result.
+ *
+ * Replaces what autograd computes for `weight.grad` of the trunk's nn.Linear layers
+ * (models/yemong/attention.py:60-74, models/yemong/griffin.py:165-167,238-247) when the PPO update
+ * back-propagates through them (train/rl/ppo.py:1417-1425): there the contraction runs over
+ * several hundred thousand token rows while N and K are 128..512, a shape the library GEMM
+ * runs far from the HBM bound.
+ *
+ *   dy       (R, N) bf16, rows dy_row_stride elements apart: gradient of the layer's output
+ *   x        (R, K) bf16, rows x_row_stride elements apart: the layer's input (as autocast cast it)
+ *   partials (slices, N, K) fp32 workspace owned by the caller; slices >= 1, a good value comes
+ *            from bnb_linear_wgrad_slices(R, N, K)
+ *   dw       (N, K) fp32 contiguous: overwritten, or added to when accumulate != 0
+ *
+ * The rows are split into `slices` ranges, one work-group per (128 x 128 output tile, slice);
+ * a second kernel adds the slices in a fixed order, so the result does not depend on timing.
+ * Requirements: N % 128 == 0, K % 128 == 0, 16-byte aligned pointers, strides multiples of 8.
+ */
+int bnb_linear_wgrad_slices(int64_t R, int N, int K);
+int bnb_linear_wgrad_fwd(const void *dy, int64_t dy_row_stride, const void *x, int64_t x_row_stride,
+                         float *partials, int slices, float *dw, int accumulate,
+                         int64_t R, int N, int K, void *stream);
 
 /*
  * Pooling by multi-head attention over each team's alive ships, broadcast back to the ships:

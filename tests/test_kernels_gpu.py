@@ -1372,3 +1372,110 @@ def test_full_size_team_pool_on_sampled_environments():
     assert max_rel(pool[pick].cpu(), ref) <= F32_TOL
     idx = team.clamp(0, 1).long().unsqueeze(-1).expand(B, N, D).to(DEV)
     assert torch.equal(ships, pool.gather(1, idx))
+
+
+# ------------------------------------------------------------------ Linear weight gradient
+
+
+def _wgrad_case(seed, R, N, K):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(R, N, generator=g).bfloat16(), torch.randn(R, K, generator=g).bfloat16()
+
+
+@pytest.mark.parametrize("R", [0, 1, 63, 64, 65, 1000, 20011, 140000])
+@pytest.mark.parametrize("N,K", [(128, 128), (384, 128), (128, 512), (256, 256)])
+def test_linear_wgrad_matches_float64_product(R, N, K):
+    """dW = dy^T x is fixed by the mathematics: the float64 product of the same bf16 operands is the truth
+    (what nn.Linear's backward, reference models/yemong/attention.py:60-74, computes for its weight)."""
+    if R == 140000 and (N, K) != (128, 128):
+        pytest.skip("the long case runs once")
+    dy, x = _wgrad_case(R + N + K, R, N, K)
+    got = ops.linear_wgrad(dy.to(DEV), x.to(DEV))
+    torch.cuda.synchronize()
+    ref = dy.double().t() @ x.double()
+    assert got.shape == (N, K) and got.dtype == torch.float32
+    if R == 0:
+        assert not got.any()
+        return
+    assert max_rel(got.cpu().double(), ref) <= F32_TOL
+    again = ops.linear_wgrad(dy.to(DEV), x.to(DEV))
+    assert torch.equal(got, again)  # fixed summation order
+
+
+def test_linear_wgrad_single_entries_land_where_the_definition_puts_them():
+    R, N, K = 777, 256, 128
+    dy = torch.zeros(R, N).bfloat16()
+    x = torch.zeros(R, K).bfloat16()
+    picks = [(0, 0, 0, 1.0), (63, 5, 127, 2.0), (64, 255, 1, -3.0), (776, 131, 64, 0.5), (400, 33, 97, 4.0), (401, 33, 97, 8.0)]
+    want = torch.zeros(N, K)
+    for r, n, k, v in picks:
+        dy[r, n] = v
+        x[r, k] = 1.0
+        want[n, k] += v
+    # every other product of the chosen rows that is not zero belongs to the truth too
+    want = dy.float().t() @ x.float()
+    assert want[33, 97] == 12.0 and want[255, 1] == -3.0 and want[5, 127] == 2.0
+    got = ops.linear_wgrad(dy.to(DEV), x.to(DEV)).cpu()
+    assert torch.equal(got, want)
+
+
+def test_linear_wgrad_reads_strided_rows_and_accumulates():
+    R, N, K = 5000, 128, 256
+    g = torch.Generator().manual_seed(5)
+    wide_dy = torch.randn(R, 3 * N, generator=g).bfloat16().to(DEV)
+    wide_x = torch.randn(R, K + 64, generator=g).bfloat16().to(DEV)
+    dy, x = wide_dy[:, N:2 * N], wide_x[:, 64:]
+    ref = dy.double().t() @ x.double()
+    out = torch.full((N, K), 2.0, device=DEV)
+    ops.linear_wgrad(dy, x, out=out)
+    assert max_rel(out.double(), ref) <= F32_TOL
+    ops.linear_wgrad(dy, x, out=out, accumulate=True)
+    assert max_rel(out.double(), 2 * ref) <= F32_TOL
+    lead = ops.linear_wgrad(dy.view(50, 100, N), x.view(50, 100, K))
+    assert torch.equal(lead, ops.linear_wgrad(dy, x))
+
+
+def test_linear_wgrad_rejects_what_it_does_not_cover():
+    dy, x = _wgrad_case(1, 10, 128, 128)
+    with pytest.raises(TypeError):
+        ops.linear_wgrad(dy.float().to(DEV), x.to(DEV))
+    with pytest.raises(ValueError):
+        ops.linear_wgrad(dy.to(DEV), x[:9].to(DEV))
+    with pytest.raises(ValueError):
+        ops.linear_wgrad(dy.to(DEV)[:, :64], x.to(DEV))
+    with pytest.raises(ValueError):
+        ops.linear_wgrad(dy.to(DEV), x.to(DEV), accumulate=True)
+    assert not ops.linear_wgrad_supported(x.to(DEV), torch.zeros(128, 96))
+
+
+@pytest.mark.parametrize("with_bias", [False, True])
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+def test_linear_train_gradients_match_autograd_of_the_same_bf16_linear(with_bias, x_dtype):
+    R, N, K = 9000, 256, 128
+    g = torch.Generator().manual_seed(11)
+    x0 = torch.randn(30, 300, K, generator=g).to(x_dtype)
+    w0 = torch.randn(N, K, generator=g) / K ** 0.5
+    b0 = torch.randn(N, generator=g) if with_bias else None
+    up = torch.randn(30, 300, N, generator=g)
+
+    x = x0.to(DEV).requires_grad_()
+    w = w0.to(DEV).requires_grad_()
+    b = b0.to(DEV).requires_grad_() if with_bias else None
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = ops.linear_train(x, w, b)
+    assert y.dtype == torch.bfloat16
+    (y.float() * up.to(DEV)).sum().backward()
+
+    # truth: the same bf16-rounded operands, float64 arithmetic
+    xd = x0.bfloat16().double().requires_grad_()
+    wd = w0.bfloat16().double().requires_grad_()
+    bd = b0.bfloat16().double().requires_grad_() if with_bias else None
+    yd = torch.nn.functional.linear(xd, wd, bd)
+    assert max_rel(y.detach().float().cpu().double(), yd.detach()) <= BF16_TOL
+    dyb = up.bfloat16().double()  # the gradient reaching the layer is rounded to its bf16 output
+    (yd * dyb).sum().backward()
+    assert x.grad.dtype == x_dtype and w.grad.dtype == torch.float32
+    assert max_rel(w.grad.cpu().double(), wd.grad) <= F32_TOL
+    assert max_rel(x.grad.float().cpu().double(), xd.grad) <= BF16_TOL
+    if with_bias:
+        assert max_rel(b.grad.cpu().double(), bd.grad) <= F32_TOL

@@ -542,3 +542,43 @@ def test_attention_block_outside_kernel_coverage_uses_the_library_on_the_device(
     with pytest.raises(_native.NativeLibraryError) as err:
         bnb.ops.sdpa_masked(torch.zeros(1, 4, 3 * D, device=DEV), None, H)
     assert err.value.code == _native.ERR_UNSUPPORTED
+
+
+def test_update_path_weight_gradients_agree_between_the_row_sliced_kernel_and_the_library(monkeypatch):
+    """Under bf16 autocast with gradients on, Linear layers with enough rows take ops.linear_train;
+    the parameter gradients must agree with the same update computed through nn.Linear alone."""
+    from boost_and_broadside_amd import ops, trunk
+
+    cfg = _cfg(128, 4, spatial=1, temporal=1)
+    torch.manual_seed(7)
+    block = bnb.YemongBlock(cfg).to(DEV)
+    T, B, N, M, D = 16, 48, 8, 4, 128  # 9,216 token rows, 6,144 recurrent rows
+    gen = torch.Generator().manual_seed(8)
+    x = torch.randn(T, B, N + M, D, generator=gen).to(DEV)
+    alive = (torch.rand(T, B, N + M, generator=gen) < 0.85).to(DEV)
+    alive[..., 0] = True
+    h0 = torch.zeros(1, B * N, D, device=DEV)
+    cb0 = torch.zeros(1, B * N, 3, D, device=DEV)
+    done = (torch.rand(T, B, generator=gen) < 0.1).to(DEV)
+
+    calls = []
+    real = ops.linear_wgrad
+    monkeypatch.setattr(ops, "linear_wgrad", lambda *a, **k: (calls.append(a[0].shape), real(*a, **k))[1])
+
+    def grads(min_rows):
+        monkeypatch.setattr(trunk, "_WGRAD_MIN_ROWS", min_rows)
+        block.zero_grad(set_to_none=True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out, h, cb = block.sequence(x, alive, h0, cb0, done, N)
+        (out.float().square().mean() + h.float().square().mean()).backward()
+        return {n: p.grad.detach().clone() for n, p in block.named_parameters()}
+
+    routed = grads(4096)
+    assert calls, "no Linear layer took the row-sliced weight gradient"
+    n_calls = len(calls)
+    with trunk.library_weight_gradients():
+        library = grads(4096)
+    assert len(calls) == n_calls
+    for name, g in routed.items():
+        assert torch.isfinite(g).all(), name
+        assert max_rel(g.cpu(), library[name].cpu()) <= BF16_TOL, name
