@@ -565,19 +565,20 @@ def test_update_path_weight_gradients_agree_between_the_row_sliced_kernel_and_th
     real = ops.linear_wgrad
     monkeypatch.setattr(ops, "linear_wgrad", lambda *a, **k: (calls.append(a[0].shape), real(*a, **k))[1])
 
-    def grads(min_rows):
-        monkeypatch.setattr(trunk, "_WGRAD_MIN_ROWS", min_rows)
+    monkeypatch.setattr(trunk, "_WGRAD_MIN_ROWS", 4096)
+
+    def grads():
         block.zero_grad(set_to_none=True)
         with torch.autocast("cuda", dtype=torch.bfloat16):
             out, h, cb = block.sequence(x, alive, h0, cb0, done, N)
         (out.float().square().mean() + h.float().square().mean()).backward()
         return {n: p.grad.detach().clone() for n, p in block.named_parameters()}
 
-    routed = grads(4096)
+    routed = grads()
     assert calls, "no Linear layer took the row-sliced weight gradient"
     n_calls = len(calls)
     with trunk.library_weight_gradients():
-        library = grads(4096)
+        library = grads()
     assert len(calls) == n_calls
     for name, g in routed.items():
         assert torch.isfinite(g).all(), name
