@@ -12,7 +12,7 @@ import os
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "_lib", "libbnb_amd.so")
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 F32, BF16 = 0, 1
 PATH_AUTO, PATH_VALU, PATH_MFMA = 0, 1, 2
 
@@ -37,6 +37,10 @@ SIGNATURES = {
     "bnb_conv_step_rows_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _vp]),
     "bnb_linear_wgrad_slices": (_i, [_i64, _i, _i]),
     "bnb_linear_wgrad_fwd": (_i, [_vp, _i64, _vp, _i64, _vp, _i, _vp, _i, _i64, _i, _i, _vp]),
+    "bnb_conv_seq_bwd_blocks": (_i, [_i64, _i, _i]),
+    "bnb_conv_seq_bwd": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _vp]),
+    "bnb_rmsnorm_bwd_blocks": (_i, [_i64, _i]),
+    "bnb_rmsnorm_bwd": (_i, [_vp, _i64, _vp, _i, _i64, _vp, _f, _vp, _vp, _vp, _i, _vp, _i64, _i, _vp]),
     "bnb_team_attend_fwd": (_i, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i, _i, _i, _i, _vp]),
     "bnb_team_norm_broadcast_fwd": (_i, [_vp, _vp, _f, _vp, _i64, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "bnb_temporal_step_fwd": (

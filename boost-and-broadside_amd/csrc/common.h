@@ -141,4 +141,9 @@ __device__ __forceinline__ void wave_lds_handover()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// out[i] (+)= sum over s of partials[s * elems + i], slices added in a fixed order (defined in
+// linear_wgrad.hip).  elems must be a multiple of 64; slices == 0 writes zeros (or leaves out alone
+// when accumulating).
+int launch_sum_slices(const float *partials, float *out, int64_t elems, int slices, int accumulate, hipStream_t stream);
+
 }  // namespace bnb

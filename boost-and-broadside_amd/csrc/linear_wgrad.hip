@@ -118,8 +118,8 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
 
 // dW (+)= sum over the slices in a fixed order: a work-group owns 64 consecutive elements (16 lanes x 4 floats);
 // its 16 lane groups each add every 16th slice, then group 0 adds the 16 sums in group order.
-__global__ __launch_bounds__(256) void linear_wgrad_reduce_kernel(const float *__restrict__ partials, float *__restrict__ dw,
-                                                                  int64_t elems, int slices, int accumulate)
+__global__ __launch_bounds__(256) void sum_slices_kernel(const float *__restrict__ partials, float *__restrict__ dw,
+                                                         int64_t elems, int slices, int accumulate)
 {
     __shared__ f32x4 s_sum[16][16];
     const int q = threadIdx.x & 15, g = threadIdx.x >> 4;
@@ -148,6 +148,14 @@ __global__ __launch_bounds__(256) void linear_wgrad_reduce_kernel(const float *_
         }
         *reinterpret_cast<f32x4 *>(dw + i) = t;
     }
+}
+
+int launch_sum_slices(const float *partials, float *out, int64_t elems, int slices, int accumulate, hipStream_t stream)
+{
+    if (elems <= 0 || elems % 64 != 0 || slices < 0) return BNB_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(sum_slices_kernel, dim3((unsigned)(elems / 64)), dim3(256), 0, stream, partials, out, elems, slices,
+                       accumulate);
+    return (int)hipGetLastError();
 }
 
 }  // namespace bnb
@@ -184,8 +192,5 @@ extern "C" int bnb_linear_wgrad_fwd(const void *dy, int64_t dy_row_stride, const
                        rows_per_slice > 0 ? rows_per_slice : kWgRows);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
-    const int64_t elems = (int64_t)N * K;
-    hipLaunchKernelGGL(linear_wgrad_reduce_kernel, dim3((unsigned)(elems / 64)), dim3(256), 0, s, partials, dw,
-                       elems, slices, accumulate);
-    return (int)hipGetLastError();
+    return launch_sum_slices(partials, dw, (int64_t)N * K, slices, accumulate, s);
 }

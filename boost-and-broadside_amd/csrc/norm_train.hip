@@ -1,0 +1,154 @@
+// RMSNorm backward for gfx950:  y = x * rsqrt(mean(x^2) + eps) * w
+//   dx = rstd * (dy * w) - x * rstd^3 * mean(dy * w * x)   (+ grad_sum, the gradient arriving on the
+//                                                           residual branch that bypasses the norm)
+//   dw = sum over rows of dy * x * rstd
+//
+// What autograd runs for every nn.RMSNorm of the trunk during the PPO update (reference:
+// train/rl/ppo.py:1417-1425 through models/yemong/attention.py:60,73,94-98 and
+// griffin.py:238,246,269,284-285).  The library does it in two kernels over fp32 tensors, after
+// a cast of the bf16 gradient to fp32 and before an add with the residual gradient; here one
+// streaming pass reads x (fp32) and dy (bf16 or fp32) once and writes dx once.  rstd is
+// recomputed from x, which is being read anyway.  Weight-gradient partial sums stay in
+// registers across a work-group's rows, are combined through LDS in a fixed order and written
+// one row per work-group; a second kernel adds those rows in a fixed order: no atomics, the
+// result does not depend on timing.
+// Bound: HBM.  8 channels per lane, 16-byte nontemporal accesses, fp32 arithmetic.
+
+#include "common.h"
+
+namespace bnb {
+
+constexpr int kNbThreads = 256;
+constexpr int kNbMaxBlocks = 2048;  // eight work-groups per CU keep enough loads in flight
+
+template <int LANES, typename GT, bool HAS_SUM>
+__global__ __launch_bounds__(kNbThreads) void rmsnorm_bwd_kernel(
+    const float *__restrict__ x, int64_t x_stride, const GT *__restrict__ dy, int64_t dy_stride,
+    const float *__restrict__ weight, float eps, const float *__restrict__ grad_sum, float *__restrict__ dx,
+    float *__restrict__ partials, int64_t R)
+{
+    constexpr int D = LANES * 8;
+    constexpr int ROWS = kNbThreads / LANES;
+    __shared__ float s_dw[ROWS * D];
+
+    const int local_row = threadIdx.x / LANES;
+    const int d0 = (threadIdx.x - local_row * LANES) << 3;
+    const int64_t step = (int64_t)gridDim.x * ROWS;
+    const Row8 w = load8(weight + d0);
+    float dw[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+
+    // every lane of a row group walks the same number of iterations (the butterflies need all of them)
+    int64_t row = (int64_t)blockIdx.x * ROWS + local_row;
+    int64_t r = row < R ? row : R - 1;
+    Row8 xn = load8_stream(x + r * x_stride + d0), gn = load8_stream(dy + r * dy_stride + d0);
+    for (int64_t base = (int64_t)blockIdx.x * ROWS; base < R; base += step) {
+        const Row8 xv = xn, gv = gn;
+        const int64_t cur = row;
+        const bool valid = cur < R;
+        row += step;
+        if (base + step < R) {
+            r = row < R ? row : R - 1;
+            xn = load8_stream(x + r * x_stride + d0), gn = load8_stream(dy + r * dy_stride + d0);
+        }
+        float ss = 0.0f, dot = 0.0f;
+        Row8 g;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            g.v[e] = gv.v[e] * w.v[e];
+            ss = fmaf(xv.v[e], xv.v[e], ss);
+            dot = fmaf(g.v[e], xv.v[e], dot);
+        }
+#pragma unroll
+        for (int off = 1; off < LANES; off <<= 1) {
+            ss += __shfl_xor(ss, off);
+            dot += __shfl_xor(dot, off);
+        }
+        if (!valid) continue;
+        const float rstd = rsqrtf(ss * (1.0f / D) + eps);
+        const float coef = dot * (1.0f / D) * rstd * rstd * rstd;
+        Row8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            o.v[e] = g.v[e] * rstd - xv.v[e] * coef;
+            dw[e] = fmaf(gv.v[e] * rstd, xv.v[e], dw[e]);
+        }
+        if (HAS_SUM) {
+            const Row8 s = load8_stream(grad_sum + cur * D + d0);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o.v[e] += s.v[e];
+        }
+        store8_stream(dx + cur * D + d0, o);
+    }
+
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s_dw[local_row * D + d0 + e] = dw[e];
+    __syncthreads();
+    for (int d = threadIdx.x; d < D; d += kNbThreads) {
+        float t = 0.0f;
+#pragma unroll
+        for (int j = 0; j < ROWS; ++j) t += s_dw[j * D + d];
+        partials[(int64_t)blockIdx.x * D + d] = t;
+    }
+}
+
+template <int LANES, typename GT>
+static int launch_norm_bwd(const float *x, int64_t x_stride, const void *dy, int64_t dy_stride, const float *weight, float eps,
+                           const float *grad_sum, float *dx, float *partials, int blocks, float *dw, int64_t R,
+                           hipStream_t stream)
+{
+    const dim3 g((unsigned)blocks), t(kNbThreads);
+    if (grad_sum)
+        hipLaunchKernelGGL((rmsnorm_bwd_kernel<LANES, GT, true>), g, t, 0, stream, x, x_stride, (const GT *)dy, dy_stride, weight,
+                           eps, grad_sum, dx, partials, R);
+    else
+        hipLaunchKernelGGL((rmsnorm_bwd_kernel<LANES, GT, false>), g, t, 0, stream, x, x_stride, (const GT *)dy, dy_stride, weight,
+                           eps, grad_sum, dx, partials, R);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    return launch_sum_slices(partials, dw, LANES * 8, blocks, 0, stream);
+}
+
+template <typename GT>
+static int dispatch_norm_bwd(int D, const float *x, int64_t x_stride, const void *dy, int64_t dy_stride, const float *weight,
+                             float eps, const float *grad_sum, float *dx, float *partials, int blocks, float *dw, int64_t R,
+                             hipStream_t s)
+{
+    switch (D) {
+        case 64: return launch_norm_bwd<8, GT>(x, x_stride, dy, dy_stride, weight, eps, grad_sum, dx, partials, blocks, dw, R, s);
+        case 128: return launch_norm_bwd<16, GT>(x, x_stride, dy, dy_stride, weight, eps, grad_sum, dx, partials, blocks, dw, R, s);
+        case 256: return launch_norm_bwd<32, GT>(x, x_stride, dy, dy_stride, weight, eps, grad_sum, dx, partials, blocks, dw, R, s);
+        case 512: return launch_norm_bwd<64, GT>(x, x_stride, dy, dy_stride, weight, eps, grad_sum, dx, partials, blocks, dw, R, s);
+        default: return BNB_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace bnb
+
+extern "C" int bnb_rmsnorm_bwd_blocks(int64_t R, int D)
+{
+    if (R <= 0 || D < 8) return 1;
+    const int rows = bnb::kNbThreads / (D / 8) > 0 ? bnb::kNbThreads / (D / 8) : 1;
+    const int64_t need = (R + rows - 1) / rows;
+    return (int)(need < bnb::kNbMaxBlocks ? need : bnb::kNbMaxBlocks);
+}
+
+extern "C" int bnb_rmsnorm_bwd(const float *x, int64_t x_row_stride, const void *dy, int dy_dtype, int64_t dy_row_stride,
+                               const float *weight, float eps, const float *grad_sum, float *dx, float *partials,
+                               int blocks, float *dw, int64_t R, int D, void *stream)
+{
+    using namespace bnb;
+    if (R < 0 || D < 1 || x_row_stride < D || dy_row_stride < D) return BNB_ERR_BAD_SHAPE;
+    if (D != 64 && D != 128 && D != 256 && D != 512) return BNB_ERR_UNSUPPORTED;
+    if (dy_dtype != BNB_F32 && dy_dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
+    if (!weight || !dw || !partials || (R > 0 && (!x || !dy || !dx))) return BNB_ERR_NULL_POINTER;
+    if (blocks < 1 || blocks > kNbMaxBlocks) return BNB_ERR_BAD_SHAPE;
+    if (!aligned16(weight) || !aligned16(dw) || !aligned16(partials) ||
+        (R > 0 && (!aligned16(x) || !aligned16(dy) || !aligned16(dx) || (grad_sum && !aligned16(grad_sum)))) ||
+        x_row_stride % 4 != 0 || dy_row_stride % 8 != 0)
+        return BNB_ERR_MISALIGNED;
+    hipStream_t s = (hipStream_t)stream;
+    if (R == 0) return launch_sum_slices(partials, dw, D, 0, 0, s);  // no rows: the weight gradient is zero
+    if (dy_dtype == BNB_BF16)
+        return dispatch_norm_bwd<uint16_t>(D, x, x_row_stride, dy, dy_row_stride, weight, eps, grad_sum, dx, partials, blocks, dw, R, s);
+    return dispatch_norm_bwd<float>(D, x, x_row_stride, dy, dy_row_stride, weight, eps, grad_sum, dx, partials, blocks, dw, R, s);
+}

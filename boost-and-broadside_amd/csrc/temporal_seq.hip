@@ -554,6 +554,141 @@ static int launch_conv_seq(const void *b1, const float *conv_in, int64_t conv_in
     return (int)hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------
+// backward of the causal depthwise conv over T steps
+// ------------------------------------------------------------------------------------
+//
+// With in[s] = stored input s + 3 for s in -3..-1 and b1[s] for s >= 0, the forward is
+//   v[t] = bias + sum_j w[3 - j] * in[t - j] * [no episode end in t-j .. t-1],   j = 0..3,
+// so every input's gradient depends on four output gradients only,
+//   d_in[s] = dv[s] w3 + m1 dv[s+1] w2 + m2 dv[s+2] w1 + m3 dv[s+3] w0,
+//   m1 = !done[s], m2 = m1 && !done[s+1], m3 = m2 && !done[s+2]   (done[s < 0] = false, dv[t >= T] = 0),
+// and the same products pair in[s] with the taps' gradients.  No recurrence: a work item is
+// (a group of rows, 16 consecutive s), a work-group walks items in a grid-stride loop with the
+// tap and bias gradients in registers, then adds its rows through LDS and writes one partial
+// row; the partial rows are added in a fixed order by sum_slices.
+constexpr int kCbChunk = 16;
+constexpr int kCbMaxBlocks = 2048;
+
+template <typename BT>
+__global__ __launch_bounds__(kSeqThreads) void conv_seq_bwd_kernel(
+    const BT *__restrict__ b1, const float *__restrict__ conv_in, int64_t conv_in_stride, const float *__restrict__ weight,
+    const uint8_t *__restrict__ done, const float *__restrict__ dv, const float *__restrict__ dconv_out,
+    BT *__restrict__ db1, float *__restrict__ dconv_in, float *__restrict__ partials, int64_t R, int T, int D, int64_t rs,
+    int64_t ts, int chunks, int64_t items)
+{
+    __shared__ float s_red[kSeqThreads * 8];
+    const int vecs = D >> 3;
+    const int rows_per_block = kSeqThreads / vecs;
+    const int local_row = threadIdx.x / vecs;
+    const int d0 = (threadIdx.x - local_row * vecs) << 3;
+
+    float w[8][kSeqTaps], dw[8][kSeqTaps], db[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const f32x4 wv = *reinterpret_cast<const f32x4 *>(weight + (int64_t)(d0 + e) * kSeqTaps);
+        w[e][0] = wv.x, w[e][1] = wv.y, w[e][2] = wv.z, w[e][3] = wv.w;
+        dw[e][0] = dw[e][1] = dw[e][2] = dw[e][3] = 0.0f;
+        db[e] = 0.0f;
+    }
+    const Row8 zero = {{0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f}};
+
+    for (int64_t item = blockIdx.x; item < items; item += gridDim.x) {
+        const int64_t group = item / chunks;
+        const int s0 = (int)(item - group * chunks) * kCbChunk - (kSeqTaps - 1);  // uniform over the work-group
+        const int64_t row = group * rows_per_block + local_row;
+        if (row >= R) continue;
+        const float *dvp = dv + row * rs + d0;
+        const BT *bp = b1 + row * rs + d0;
+        const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
+        auto grad_row = [&](int t) -> Row8 { return t >= 0 && t < T ? load8_stream(dvp + t * ts) : zero; };
+        auto ended = [&](int t) -> bool { return dn != nullptr && t >= 0 && t < T && dn[t] != 0; };
+
+        Row8 g0 = grad_row(s0), g1 = grad_row(s0 + 1), g2 = grad_row(s0 + 2);
+        bool f0 = ended(s0), f1 = ended(s0 + 1);
+        for (int u0 = 0; u0 < kCbChunk && s0 + u0 < T; u0 += kSeqAhead) {
+            Row8 gn[kSeqAhead], in[kSeqAhead];
+            bool fn[kSeqAhead];
+#pragma unroll
+            for (int u = 0; u < kSeqAhead; ++u) {
+                const int s = s0 + u0 + u;
+                gn[u] = grad_row(s + 3);
+                fn[u] = ended(s + 2);
+                if (s < 0)
+                    in[u] = load8(conv_in + row * conv_in_stride + (int64_t)(s + 3) * D + d0);
+                else
+                    in[u] = s < T ? load8_stream(bp + s * ts) : zero;
+            }
+#pragma unroll
+            for (int u = 0; u < kSeqAhead; ++u) {
+                const int s = s0 + u0 + u;
+                if (s < T) {
+                    const Row8 g3 = gn[u];
+                    const bool f2 = fn[u];
+                    const float m1 = f0 ? 0.0f : 1.0f, m2 = (f0 || f1) ? 0.0f : 1.0f, m3 = (f0 || f1 || f2) ? 0.0f : 1.0f;
+                    Row8 o;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float a1 = m1 * g1.v[e], a2 = m2 * g2.v[e], a3 = m3 * g3.v[e];
+                        o.v[e] = g0.v[e] * w[e][3] + a1 * w[e][2] + a2 * w[e][1] + a3 * w[e][0];
+                        const float x = in[u].v[e];
+                        dw[e][3] = fmaf(x, g0.v[e], dw[e][3]);
+                        dw[e][2] = fmaf(x, a1, dw[e][2]);
+                        dw[e][1] = fmaf(x, a2, dw[e][1]);
+                        dw[e][0] = fmaf(x, a3, dw[e][0]);
+                        db[e] += g0.v[e];
+                    }
+                    if (dconv_out != nullptr && s >= T - 3) {
+                        // this input is also entry s - (T - 3) of the stored inputs handed on
+                        const Row8 h = load8(dconv_out + row * 3 * (int64_t)D + (int64_t)(s - (T - 3)) * D + d0);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) o.v[e] += h.v[e];
+                    }
+                    if (s < 0)
+                        store8(dconv_in + row * 3 * (int64_t)D + (int64_t)(s + 3) * D + d0, o);
+                    else
+                        store8_stream(db1 + row * rs + s * ts + d0, o);
+                    g0 = g1, g1 = g2, g2 = g3;
+                    f0 = f1, f1 = f2;
+                }
+            }
+        }
+    }
+
+    // this work-group's tap and bias gradients: rows added in order, one partial row
+    // [ (d, tap) for all d | bias ] per work-group
+    float *part = partials + (int64_t)blockIdx.x * 5 * D;
+#pragma unroll
+    for (int q = 0; q < 5; ++q) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s_red[local_row * D + d0 + e] = q < 4 ? dw[e][q < 4 ? q : 0] : db[e];
+        __syncthreads();
+        for (int d = threadIdx.x; d < D; d += kSeqThreads) {
+            float t = 0.0f;
+            for (int j = 0; j < rows_per_block; ++j) t += s_red[j * D + d];
+            part[q < 4 ? d * kSeqTaps + q : 4 * D + d] = t;
+        }
+        __syncthreads();
+    }
+}
+
+template <typename BT>
+static int launch_conv_seq_bwd(const void *b1, const float *conv_in, int64_t conv_in_stride, const float *weight,
+                               const uint8_t *done, const float *dv, const float *dconv_out, void *db1, float *dconv_in,
+                               float *partials, int blocks, float *dwb, int64_t R, int T, int D, int time_major,
+                               hipStream_t stream)
+{
+    const int64_t rs = time_major ? D : (int64_t)T * D, ts = time_major ? R * D : D;
+    const int rows_per_block = kSeqThreads / (D / 8);
+    const int chunks = (T + (kSeqTaps - 1) + kCbChunk - 1) / kCbChunk;
+    const int64_t items = (R + rows_per_block - 1) / rows_per_block * chunks;
+    hipLaunchKernelGGL((conv_seq_bwd_kernel<BT>), dim3((unsigned)blocks), dim3(kSeqThreads), 0, stream, (const BT *)b1, conv_in,
+                       conv_in_stride, weight, done, dv, dconv_out, (BT *)db1, dconv_in, partials, R, T, D, rs, ts, chunks, items);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    return launch_sum_slices(partials, dwb, 5 * (int64_t)D, blocks, 0, stream);
+}
+
 }  // namespace bnb
 
 extern "C" int bnb_rglru_scan_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
@@ -653,4 +788,37 @@ extern "C" int bnb_conv_seq_fwd(const void *b1, int b1_dtype, const float *conv_
                                          (uint16_t *)v_bf16_out, conv_out, conv_out_row_stride, R, T, D, time_major != 0, s);
     return launch_conv_seq<float>(b1, conv_in, conv_in_row_stride, weight, bias, done, v_out, (uint16_t *)v_bf16_out,
                                   conv_out, conv_out_row_stride, R, T, D, time_major != 0, s);
+}
+
+extern "C" int bnb_conv_seq_bwd_blocks(int64_t R, int T, int D)
+{
+    if (R <= 0 || T < 1 || D < 8) return 1;
+    const int rows_per_block = bnb::kSeqThreads / (D / 8) > 0 ? bnb::kSeqThreads / (D / 8) : 1;
+    const int64_t items = (R + rows_per_block - 1) / rows_per_block * ((T + 3 + bnb::kCbChunk - 1) / bnb::kCbChunk);
+    return (int)(items < bnb::kCbMaxBlocks ? items : bnb::kCbMaxBlocks);
+}
+
+extern "C" int bnb_conv_seq_bwd(const void *b1, int b1_dtype, const float *conv_in, int64_t conv_in_row_stride,
+                                const float *weight, const uint8_t *done, const float *dv, const float *dconv_out,
+                                void *db1, float *dconv_in, float *partials, int blocks, float *dwb, int64_t R, int T,
+                                int D, int time_major, void *stream)
+{
+    using namespace bnb;
+    if (R < 0 || T < 1 || D < 1) return BNB_ERR_BAD_SHAPE;
+    if (D != 64 && D != 128 && D != 256 && D != 512) return BNB_ERR_UNSUPPORTED;
+    if (b1_dtype != BNB_F32 && b1_dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
+    if (!weight || !partials || !dwb || (R > 0 && (!b1 || !conv_in || !dv || !db1 || !dconv_in))) return BNB_ERR_NULL_POINTER;
+    if (conv_in_row_stride < 3 * (int64_t)D || blocks < 1 || blocks > kCbMaxBlocks) return BNB_ERR_BAD_SHAPE;
+    if (!aligned16(weight) || !aligned16(partials) || !aligned16(dwb) ||
+        (R > 0 && (!aligned16(b1) || !aligned16(conv_in) || !aligned16(dv) || !aligned16(db1) || !aligned16(dconv_in) ||
+                   (dconv_out && !aligned16(dconv_out)))) ||
+        conv_in_row_stride % 4 != 0)
+        return BNB_ERR_MISALIGNED;
+    hipStream_t s = (hipStream_t)stream;
+    if (R == 0) return launch_sum_slices(partials, dwb, 5 * (int64_t)D, 0, 0, s);
+    if (b1_dtype == BNB_BF16)
+        return launch_conv_seq_bwd<uint16_t>(b1, conv_in, conv_in_row_stride, weight, done, dv, dconv_out, db1, dconv_in,
+                                             partials, blocks, dwb, R, T, D, time_major != 0, s);
+    return launch_conv_seq_bwd<float>(b1, conv_in, conv_in_row_stride, weight, done, dv, dconv_out, db1, dconv_in, partials,
+                                      blocks, dwb, R, T, D, time_major != 0, s);
 }

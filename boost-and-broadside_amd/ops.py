@@ -763,6 +763,81 @@ def conv_seq(
     return (v, conv_out, v_lp) if also_bf16 else (v, conv_out)
 
 
+_CONV_TRAIN_WIDTHS = (64, 128, 256, 512)
+
+
+def conv_seq_bwd(b1, conv_buf, weight, done, dv, dconv_out=None, *, time_major: bool = False):
+    """Backward of ``conv_seq``: returns ``(db1, dconv_buf, dweight (D, 4), dbias (D,))``.
+
+    ``dv`` is the float32 gradient of the conv output (b1's layout), ``dconv_out`` the optional
+    gradient of the returned stored inputs; ``db1`` has b1's dtype.  Sums run in a fixed order."""
+    R, T, D = b1.shape
+    if time_major:
+        T, R = R, T
+    if D not in _CONV_TRAIN_WIDTHS:
+        raise ValueError(f"conv_seq_bwd supports D in {_CONV_TRAIN_WIDTHS}, got {D}")
+    if dv.shape != b1.shape or dv.dtype != torch.float32:
+        raise ValueError("dv must be float32 with b1's shape")
+    for name, t in (("b1", b1), ("conv_buf", conv_buf), ("weight", weight), ("dv", dv)):
+        _need_device(t, name)
+    b1 = b1.contiguous()
+    dv = dv.contiguous()
+    conv_buf = conv_buf if (R == 0 or (conv_buf.stride(2) == 1 and conv_buf.stride(1) == D)) else conv_buf.contiguous()
+    weight = weight.detach().reshape(D, 4).contiguous()
+    if dconv_out is not None:
+        if dconv_out.shape != (R, 3, D):
+            raise ValueError(f"dconv_out must be {(R, 3, D)}")
+        dconv_out = dconv_out.to(torch.float32).contiguous()
+    db1 = torch.empty_like(b1)
+    dconv = torch.empty((R, 3, D), dtype=torch.float32, device=b1.device)
+    dwb = torch.empty((5 * D,), dtype=torch.float32, device=b1.device)
+    lib = _native.load()
+    blocks = int(lib.bnb_conv_seq_bwd_blocks(R, T, D))
+    partials = torch.empty((blocks, 5 * D), dtype=torch.float32, device=b1.device)
+    keep, done_ptr = _done_pointer(done, R, T, b1.device)
+    with torch.cuda.device(b1.device):
+        rc = lib.bnb_conv_seq_bwd(b1.data_ptr(), _code(b1, "b1"), conv_buf.data_ptr(), conv_buf.stride(0) if R else 3 * D,
+                                  weight.data_ptr(), done_ptr, dv.data_ptr(), None if dconv_out is None else dconv_out.data_ptr(),
+                                  db1.data_ptr(), dconv.data_ptr(), partials.data_ptr(), blocks, dwb.data_ptr(), R, T, D,
+                                  int(time_major), _stream())
+    _native.check(rc, "bnb_conv_seq_bwd")
+    del keep
+    return db1, dconv, dwb[:4 * D].view(D, 4), dwb[4 * D:]
+
+
+class _ConvSeqTrain(torch.autograd.Function):
+    """``conv_seq`` with its backward kernel."""
+
+    @staticmethod
+    def forward(ctx, b1, conv_buf, weight, bias, done, time_major):
+        with torch.no_grad():
+            v, new_buf = conv_seq(b1, conv_buf, weight, bias, done, time_major=time_major)
+        ctx.save_for_backward(b1, conv_buf, weight)
+        ctx.done = done
+        ctx.time_major = time_major
+        ctx.has_bias = bias is not None
+        return v, new_buf
+
+    @staticmethod
+    def backward(ctx, dv, dbuf):
+        b1, conv_buf, weight = ctx.saved_tensors
+        if dv is None:
+            dv = torch.zeros(b1.shape, dtype=torch.float32, device=b1.device)
+        db1, dconv, dw, db = conv_seq_bwd(b1, conv_buf, weight, ctx.done, dv, dbuf, time_major=ctx.time_major)
+        return db1, dconv, dw.reshape(weight.shape), db if ctx.has_bias else None, None, None
+
+
+def conv_seq_train_supported(b1: torch.Tensor) -> bool:
+    """Whether ``conv_seq_train`` covers this input: a covered width on the GPU."""
+    return b1.is_cuda and b1.dim() == 3 and b1.shape[-1] in _CONV_TRAIN_WIDTHS and b1.dtype in (torch.float32, torch.bfloat16)
+
+
+def conv_seq_train(b1, conv_buf, weight, bias, done=None, *, time_major: bool = False):
+    """Differentiable ``conv_seq``: ``(v, new_conv_buf)`` with gradients for b1, conv_buf, weight and bias."""
+    with torch.autocast("cuda", enabled=False):
+        return _ConvSeqTrain.apply(b1, conv_buf, weight, bias, done, time_major)
+
+
 def rglru_scan(
     x: torch.Tensor,
     gates_pre: torch.Tensor,
@@ -921,6 +996,102 @@ def add_rmsnorm(
             )
         _native.check(rc, "bnb_add_rmsnorm_fwd")
     return (x if s_out is None else s_out.reshape(x.shape)), normed.reshape(x.shape)
+
+
+_NORM_TRAIN_WIDTHS = (64, 128, 256, 512)
+
+
+def rmsnorm_bwd(x: torch.Tensor, dy: torch.Tensor, weight: torch.Tensor, *, eps: float | None = None,
+                grad_sum: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
+    """Backward of ``y = rmsnorm(x) * weight``: returns ``(dx, dw)``, both float32.
+
+    x (..., D) float32 with contiguous rows; dy same shape, float32 or bfloat16; ``grad_sum`` (same
+    shape, float32) is added to dx: the gradient reaching x on the branch that bypasses the norm.
+    The rows are added into dw in a fixed order, so repeated calls give identical bits."""
+    D = x.shape[-1]
+    if x.dtype != torch.float32 or weight.dtype != torch.float32 or weight.shape != (D,):
+        raise TypeError("x and weight must be float32 and weight must be (D,)")
+    if D not in _NORM_TRAIN_WIDTHS:
+        raise ValueError(f"rmsnorm_bwd supports D in {_NORM_TRAIN_WIDTHS}, got {D}")
+    if dy.shape != x.shape or (grad_sum is not None and grad_sum.shape != x.shape):
+        raise ValueError("dy and grad_sum must have x's shape")
+    if grad_sum is not None and grad_sum.dtype != torch.float32:
+        raise TypeError("grad_sum must be float32")
+    _need_device(x, "x")
+    _need_device(dy, "dy")
+    x2 = x.reshape(-1, D) if _uniform_rows(x, D) else x.reshape(-1, D).contiguous()
+    dy2 = dy.reshape(-1, D) if _uniform_rows(dy, D) else dy.reshape(-1, D).contiguous()
+    gs = None if grad_sum is None else grad_sum.reshape(-1, D).contiguous()
+    R = x2.shape[0]
+    dx = torch.empty((R, D), dtype=torch.float32, device=x.device)
+    dw = torch.empty((D,), dtype=torch.float32, device=x.device)
+    lib = _native.load()
+    blocks = int(lib.bnb_rmsnorm_bwd_blocks(R, D))
+    partials = torch.empty((blocks, D), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.bnb_rmsnorm_bwd(x2.data_ptr(), x2.stride(0) if R else D, dy2.data_ptr(), _code(dy2, "dy"),
+                                 dy2.stride(0) if R else D, weight.detach().contiguous().data_ptr(),
+                                 _F32_EPS if eps is None else float(eps), None if gs is None else gs.data_ptr(),
+                                 dx.data_ptr(), partials.data_ptr(), blocks, dw.data_ptr(), R, D, _stream())
+    _native.check(rc, "bnb_rmsnorm_bwd")
+    return dx.reshape(x.shape), dw
+
+
+class _RmsNormTrain(torch.autograd.Function):
+    """``rmsnorm(x) * weight`` rounded once to ``out_dtype``; forward and backward one kernel each."""
+
+    @staticmethod
+    def forward(ctx, x, weight, eps, out_dtype):
+        with torch.no_grad():
+            n = add_rmsnorm(x, weight, eps=eps, out_dtype=out_dtype)[1]
+        ctx.save_for_backward(x, weight)
+        ctx.eps = eps
+        return n
+
+    @staticmethod
+    def backward(ctx, dn):
+        x, weight = ctx.saved_tensors
+        dx, dw = rmsnorm_bwd(x, dn, weight, eps=ctx.eps)
+        return dx, dw, None, None
+
+
+class _AddRmsNormTrain(torch.autograd.Function):
+    """``s = x + delta`` and ``rmsnorm(s) * weight``; the backward adds the gradient of ``s`` inside
+    the norm-backward kernel."""
+
+    @staticmethod
+    def forward(ctx, x, delta, weight, eps, out_dtype):
+        with torch.no_grad():
+            s, n = add_rmsnorm(x, weight, delta=delta, eps=eps, out_dtype=out_dtype)
+        ctx.save_for_backward(s, weight)
+        ctx.eps = eps
+        ctx.delta_dtype = delta.dtype
+        return s, n
+
+    @staticmethod
+    def backward(ctx, ds, dn):
+        s, weight = ctx.saved_tensors
+        if dn is None:
+            dn = torch.zeros_like(s)
+        dx, dw = rmsnorm_bwd(s, dn, weight, eps=ctx.eps, grad_sum=ds)
+        ddelta = dx if ctx.delta_dtype == torch.float32 else dx.to(ctx.delta_dtype)
+        return dx, ddelta, dw, None, None
+
+
+def rmsnorm_train_supported(x: torch.Tensor) -> bool:
+    """Whether ``rmsnorm_train`` covers this input: float32 rows of a covered width on the GPU."""
+    return x.is_cuda and x.dtype == torch.float32 and x.shape[-1] in _NORM_TRAIN_WIDTHS
+
+
+def rmsnorm_train(x: torch.Tensor, weight: torch.Tensor, *, delta: torch.Tensor | None = None, eps: float | None = None,
+                  out_dtype: torch.dtype = torch.float32):
+    """Differentiable ``add_rmsnorm``: returns ``normed`` without ``delta``, ``(x + delta, normed)`` with it.
+    ``normed`` is computed in float32 and rounded once to ``out_dtype`` (what ``nn.RMSNorm`` followed by
+    autocast's cast in front of the next Linear gives)."""
+    with torch.autocast("cuda", enabled=False):
+        if delta is None:
+            return _RmsNormTrain.apply(x, weight, eps, out_dtype)
+        return _AddRmsNormTrain.apply(x, delta, weight, eps, out_dtype)
 
 
 def gelu_mul(a: torch.Tensor, b: torch.Tensor, *, out_dtype: torch.dtype | None = None) -> torch.Tensor:

@@ -97,6 +97,25 @@ def _project(layer: nn.Linear, x: torch.Tensor) -> torch.Tensor:
     return F.linear(x, wc, bc)
 
 
+def _train_norm(norm: nn.RMSNorm, x: torch.Tensor, delta: torch.Tensor | None = None):
+    """``norm(x)``, or with ``delta`` the pair ``(x + delta, norm(x + delta))``, differentiable.
+
+    On the GPU with float32 rows of a covered width the norm's output is rounded once to the
+    projection dtype and forward and backward are one kernel each (``ops.rmsnorm_train``);
+    anything else is the module itself."""
+    act = _projection_dtype()
+    if (
+        torch.is_grad_enabled() and act in (torch.float32, torch.bfloat16) and ops.rmsnorm_train_supported(x)
+        and norm.weight is not None and norm.weight.dtype == torch.float32
+        and (delta is None or (delta.shape == x.shape and delta.dtype in (torch.float32, torch.bfloat16)))
+    ):
+        return ops.rmsnorm_train(x, norm.weight, delta=delta, eps=norm.eps, out_dtype=act)
+    if delta is None:
+        return norm(x)
+    s = x + delta
+    return s, norm(s)
+
+
 @dataclass(frozen=True)
 class ModelConfig:
     """Trunk architecture; field names and checks follow config/core.py:213-275."""
@@ -208,8 +227,8 @@ class TransformerBlock(nn.Module):
     def forward(self, x, alive_mask=None, bullets=None, bullet_mask=None):
         act = _projection_dtype()
         if not _fused_ok(x, act):
-            x = x + self._attn(self.norm1(x), alive_mask, bullets, bullet_mask)
-            return x + self.ffn(self.norm2(x))
+            x1, n2 = _train_norm(self.norm2, x, self._attn(_train_norm(self.norm1, x), alive_mask, bullets, bullet_mask))
+            return x1 + self.ffn(n2)
         # norm + qkv (one kernel under bf16) -> attention kernel -> out_proj -> fused sublayer tail
         if act == torch.bfloat16 and self.d_model == ops.FFN_WIDTH and self.qkv.bias is None:
             w = self.qkv.weight
@@ -422,8 +441,13 @@ class GriffinTemporalBlock(nn.Module):
     def _sequence_autograd(self, x_seq, h0, conv_buf, done_mask, time_major):
         """Training path: torch ops (differentiable) around the recurrence, which runs on its
         forward and backward kernels."""
-        normed = self.norm1(x_seq)
+        normed = _train_norm(self.norm1, x_seq)
         b1 = _project(self.linear1, normed)
+        if ops.conv_seq_train_supported(b1) and conv_buf.dtype == torch.float32 and self.conv.weight.dtype == torch.float32:
+            # conv forward and backward on their kernels (one pass each instead of a dozen element-wise ops per tap)
+            v, new_buf = ops.conv_seq_train(b1, conv_buf, self.conv.weight, self.conv.bias, done_mask, time_major=time_major)
+            y, new_h = self.rg_lru.forward_sequence(v, h0, done_mask, time_major=time_major)
+            return self._finish(x_seq, normed, y), new_h, new_buf
         rows_first = b1.transpose(0, 1) if time_major else b1  # (R, T, D) view
         T = rows_first.shape[1]
         padded = torch.cat([conv_buf, rows_first], dim=1)  # fp32 buffer promotes a bf16 b1
@@ -438,7 +462,7 @@ class GriffinTemporalBlock(nn.Module):
         act = _projection_dtype()
         if _fused_ok(x, act):
             return ops.add_rmsnorm(x, self.norm1.weight, eps=self.norm1.eps, out_dtype=act)[1]
-        return self.norm1(x)
+        return _train_norm(self.norm1, x)
 
     def _finish(self, x, normed, y, gate_in=None):
         """Gate branch, output projection and the gated MLP, both residuals."""
@@ -458,8 +482,8 @@ class GriffinTemporalBlock(nn.Module):
                 return fused
             x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=r, eps=self.norm2.eps, out_dtype=act)
             return x1 + self.gated_mlp(n2)
-        x1 = x + _project(self.linear_out, y * F.gelu(gate_in))
-        return x1 + self.gated_mlp(self.norm2(x1))
+        x1, n2 = _train_norm(self.norm2, x, _project(self.linear_out, y * F.gelu(gate_in)))
+        return x1 + self.gated_mlp(n2)
 
     def _step(self, x, h_in, conv_in, h_out, conv_out, reset, rows_per_env):
         """One timestep: x (R,D), h_in (R,D), conv_in (R,3,D) -> (out, new_h, new_conv_buf)."""
@@ -577,8 +601,8 @@ class GriffinTemporalBlock(nn.Module):
                 return fused
             x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=r, eps=self.norm2.eps, out_dtype=act)
             return x1 + self.gated_mlp(n2)
-        x1 = x + _project(self.linear_out, b1 * F.gelu(gate_in))
-        return x1 + self.gated_mlp(self.norm2(x1))
+        x1, n2 = _train_norm(self.norm2, x, _project(self.linear_out, b1 * F.gelu(gate_in)))
+        return x1 + self.gated_mlp(n2)
 
 
 def _conv_within_episodes(padded, w, bias, done_mask):

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 16
+#define BNB_ABI_VERSION 17
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -265,6 +265,30 @@ int bnb_linear_wgrad_fwd(const void *dy, int64_t dy_row_stride, const void *x, i
                          int64_t R, int N, int K, void *stream);
 
 /*
+ * RMSNorm backward:  y = x * rsqrt(mean(x^2) + eps) * weight
+ *   dx[r] = rstd * (dy[r] * weight) - x[r] * rstd^3 * mean(dy[r] * weight * x[r])  (+ grad_sum[r])
+ *   dw    = sum_r dy[r] * x[r] * rstd
+ *
+ * Replaces what autograd runs for the trunk's nn.RMSNorm modules (models/yemong/attention.py:60,73,
+ * 94-98; models/yemong/griffin.py:238,246,269,284-285) in the PPO update (train/rl/ppo.py:1417-1425):
+ * the cast of a bf16 gradient to fp32, the library's two norm-backward kernels and, with
+ * grad_sum, the add of the gradient that reaches x past the norm (the residual branch).
+ *
+ *   x        (R, D) fp32, rows x_row_stride elements apart: the norm's input
+ *   dy       (R, D) bf16 or fp32 (dy_dtype), rows dy_row_stride apart: gradient of the norm's output
+ *   grad_sum (R, D) fp32 contiguous or NULL
+ *   dx       (R, D) fp32 contiguous (may alias grad_sum)
+ *   partials (blocks, D) fp32 workspace of the caller; blocks from bnb_rmsnorm_bwd_blocks(R, D)
+ *   dw       (D) fp32, overwritten; rows are added in a fixed order (no atomics)
+ * Requirements: D in {64, 128, 256, 512}; 16-byte aligned pointers; x_row_stride % 4 == 0,
+ * dy_row_stride % 8 == 0.
+ */
+int bnb_rmsnorm_bwd_blocks(int64_t R, int D);
+int bnb_rmsnorm_bwd(const float *x, int64_t x_row_stride, const void *dy, int dy_dtype, int64_t dy_row_stride,
+                    const float *weight, float eps, const float *grad_sum, float *dx, float *partials, int blocks,
+                    float *dw, int64_t R, int D, void *stream);
+
+/*
  * Pooling by multi-head attention over each team's alive ships, broadcast back to the ships:
  * two kernels with one plain fp32 GEMM of the caller's between them.
  *
@@ -371,6 +395,27 @@ int bnb_conv_seq_fwd(const void *b1, int b1_dtype,
                      const float *conv_in, int64_t conv_in_row_stride,
                      const float *weight, const float *bias, const uint8_t *done,
                      float *v_out, void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride,
+                     int64_t R, int T, int D, int time_major, void *stream);
+
+/*
+ * Backward of bnb_conv_seq_fwd: what autograd computes through griffin.py:67-140,275-277 in the
+ * PPO update (train/rl/ppo.py:1417-1425), where the reference's tap loop becomes a dozen
+ * element-wise kernels per tap and direction.
+ *
+ *   b1, conv_in, weight, done, time_major  as passed to the forward
+ *   dv         gradient of v_out, fp32, b1's layout
+ *   dconv_out  gradient of conv_out, (R, 3, D) fp32 contiguous, or NULL
+ *   db1        gradient of b1, b1's dtype and layout
+ *   dconv_in   gradient of conv_in, (R, 3, D) fp32 contiguous
+ *   partials   (blocks, 5*D) fp32 workspace; blocks from bnb_conv_seq_bwd_blocks(R, T, D)
+ *   dwb        5*D floats, overwritten: the tap gradients as (D, 4), then the bias gradient (D);
+ *              rows and steps are added in a fixed order (no atomics)
+ * Requirements: D in {64, 128, 256, 512}, 16-byte aligned pointers, conv_in_row_stride % 4 == 0.
+ */
+int bnb_conv_seq_bwd_blocks(int64_t R, int T, int D);
+int bnb_conv_seq_bwd(const void *b1, int b1_dtype, const float *conv_in, int64_t conv_in_row_stride,
+                     const float *weight, const uint8_t *done, const float *dv, const float *dconv_out,
+                     void *db1, float *dconv_in, float *partials, int blocks, float *dwb,
                      int64_t R, int T, int D, int time_major, void *stream);
 
 /*

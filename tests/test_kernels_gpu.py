@@ -1479,3 +1479,169 @@ def test_linear_train_gradients_match_autograd_of_the_same_bf16_linear(with_bias
     assert max_rel(x.grad.float().cpu().double(), xd.grad) <= BF16_TOL
     if with_bias:
         assert max_rel(b.grad.cpu().double(), bd.grad) <= F32_TOL
+
+
+# ------------------------------------------------------------------ RMSNorm backward
+
+
+def _norm_truth(x, dy, w, eps, grad_sum=None):
+    """Autograd through the float64 definition (attention.py:60,73 use nn.RMSNorm(d_model), eps = finfo(float32).eps)."""
+    xd = x.double().requires_grad_()
+    wd = w.double().requires_grad_()
+    y = xd * torch.rsqrt(xd.square().mean(dim=-1, keepdim=True) + eps) * wd
+    (y * dy.double()).sum().backward()
+    dx = xd.grad if grad_sum is None else xd.grad + grad_sum.double()
+    return dx, wd.grad
+
+
+@pytest.mark.parametrize("D", [64, 128, 256, 512])
+@pytest.mark.parametrize("R", [0, 1, 31, 257, 5000, 70001])
+@pytest.mark.parametrize("dy_dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_bwd_matches_autograd_of_the_definition(D, R, dy_dtype):
+    if R == 70001 and D != 128:
+        pytest.skip("the long case runs at the trunk's width")
+    g = torch.Generator().manual_seed(R * 7 + D)
+    x = torch.randn(R, D, generator=g) * (0.2 + 3.0 * torch.rand(R, 1, generator=g))
+    dy = torch.randn(R, D, generator=g).to(dy_dtype)
+    w = 1.0 + 0.3 * torch.randn(D, generator=g)
+    eps = float(torch.finfo(torch.float32).eps)
+    dx, dw = ops.rmsnorm_bwd(x.to(DEV), dy.to(DEV), w.to(DEV))
+    torch.cuda.synchronize()
+    assert dx.shape == (R, D) and dw.shape == (D,) and dx.dtype == dw.dtype == torch.float32
+    if R == 0:
+        assert not dw.any()
+        return
+    ref_dx, ref_dw = _norm_truth(x, dy, w, eps)
+    assert max_rel(dx.cpu().double(), ref_dx) <= F32_TOL
+    assert max_rel(dw.cpu().double(), ref_dw) <= F32_TOL
+    dx2, dw2 = ops.rmsnorm_bwd(x.to(DEV), dy.to(DEV), w.to(DEV))
+    assert torch.equal(dx, dx2) and torch.equal(dw, dw2)
+
+
+def test_rmsnorm_bwd_adds_the_bypass_gradient_and_reads_strided_rows():
+    R, D = 3001, 128
+    g = torch.Generator().manual_seed(3)
+    wide = torch.randn(R, 3 * D, generator=g).to(DEV)
+    x = wide[:, D:2 * D]
+    dy = torch.randn(R, 2 * D, generator=g).bfloat16().to(DEV)[:, :D]
+    gs = torch.randn(R, D, generator=g).to(DEV)
+    w = (1.0 + 0.3 * torch.randn(D, generator=g)).to(DEV)
+    dx, dw = ops.rmsnorm_bwd(x, dy, w, eps=1e-5, grad_sum=gs)
+    ref_dx, ref_dw = _norm_truth(x.cpu(), dy.cpu(), w.cpu(), 1e-5, gs.cpu())
+    assert max_rel(dx.cpu().double(), ref_dx) <= F32_TOL and max_rel(dw.cpu().double(), ref_dw) <= F32_TOL
+    lead_dx, lead_dw = ops.rmsnorm_bwd(x.reshape(3001, 1, D), dy.reshape(3001, 1, D), w, eps=1e-5, grad_sum=gs.reshape(3001, 1, D))
+    assert torch.equal(lead_dx.reshape(R, D), dx) and torch.equal(lead_dw, dw)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("with_delta", [False, True])
+def test_rmsnorm_train_gradients_match_autograd_of_torch_rms_norm(out_dtype, with_delta):
+    R, D = 4000, 128
+    g = torch.Generator().manual_seed(17)
+    x0 = torch.randn(8, R // 8, D, generator=g)
+    d0 = torch.randn(8, R // 8, D, generator=g).bfloat16() if with_delta else None
+    w0 = 1.0 + 0.2 * torch.randn(D, generator=g)
+    up_n = torch.randn(8, R // 8, D, generator=g).to(out_dtype)
+    up_s = torch.randn(8, R // 8, D, generator=g)
+
+    x = x0.to(DEV).requires_grad_()
+    w = w0.to(DEV).requires_grad_()
+    d = d0.to(DEV).requires_grad_() if with_delta else None
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        res = ops.rmsnorm_train(x, w, delta=d, out_dtype=out_dtype)
+    if with_delta:
+        s, n = res
+        loss = (n.float() * up_n.to(DEV).float()).sum() + (s * up_s.to(DEV)).sum()
+    else:
+        n = res
+        loss = (n.float() * up_n.to(DEV).float()).sum()
+    assert n.dtype == out_dtype
+    loss.backward()
+
+    xr = x0.double().requires_grad_()
+    wr = w0.double().requires_grad_()
+    dr = d0.double().requires_grad_() if with_delta else None
+    sr = xr + dr if with_delta else xr
+    nr = torch.nn.functional.rms_norm(sr, (D,), wr, float(torch.finfo(torch.float32).eps))
+    lr = (nr * up_n.double()).sum() + ((sr * up_s.double()).sum() if with_delta else 0.0)
+    lr.backward()
+    tol = F32_TOL if out_dtype == torch.float32 else BF16_TOL
+    assert max_rel(n.detach().float().cpu().double(), nr.detach()) <= tol
+    assert max_rel(x.grad.cpu().double(), xr.grad) <= F32_TOL
+    assert max_rel(w.grad.cpu().double(), wr.grad) <= F32_TOL
+    if with_delta:
+        assert d.grad.dtype == torch.bfloat16
+        assert max_rel(d.grad.float().cpu().double(), dr.grad) <= BF16_TOL
+
+
+# ------------------------------------------------------------------ sequence conv backward
+
+
+def _conv_truth_grads(b1, buf, w, bias, done, up_v, up_tail):
+    """Autograd through the pinned oracle statement of the conv, float64."""
+    leaves = [t.double().requires_grad_() for t in (b1, buf, w, bias)]
+    v, tail = torch_ref.conv_sequence(leaves[0], leaves[1], leaves[2], leaves[3], done)
+    loss = (v * up_v.double()).sum()
+    if up_tail is not None:
+        loss = loss + (tail * up_tail.double()).sum()
+    loss.backward()
+    return [t.grad for t in leaves]
+
+
+@pytest.mark.parametrize("R,T,D", [(5, 1, 128), (7, 2, 128), (6, 3, 64), (33, 13, 128), (12, 128, 128), (9, 35, 256),
+                                   (3, 16, 512), (2100, 29, 128)])
+@pytest.mark.parametrize("p_done", [0.0, 0.35])
+@pytest.mark.parametrize("b_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("time_major", [False, True])
+def test_conv_seq_bwd_matches_autograd_of_the_oracle(R, T, D, p_done, b_dtype, time_major):
+    g = torch.Generator().manual_seed(R * 11 + T + D)
+    b1 = torch.randn(R, T, D, generator=g).to(b_dtype)
+    buf = torch.randn(R, 3, D, generator=g)
+    w = 0.5 * torch.randn(D, 1, 4, generator=g)
+    bias = 0.1 * torch.randn(D, generator=g)
+    done = (torch.rand(R, T, generator=g) < p_done) if p_done > 0 else None
+    up_v = torch.randn(R, T, D, generator=g)
+    up_tail = torch.randn(R, 3, D, generator=g) if (R + T) % 2 else None
+    want = _conv_truth_grads(b1.float(), buf, w, bias, done, up_v, up_tail)
+
+    def lay(t):
+        return t.transpose(0, 1).contiguous() if time_major else t
+
+    db1, dbuf, dw, dbias = ops.conv_seq_bwd(lay(b1).to(DEV), buf.to(DEV), w.to(DEV), None if done is None else done.to(DEV),
+                                            lay(up_v).to(DEV), None if up_tail is None else up_tail.to(DEV),
+                                            time_major=time_major)
+    torch.cuda.synchronize()
+    assert db1.dtype == b_dtype and dbuf.dtype == dw.dtype == dbias.dtype == torch.float32
+    got_b1 = db1.float().cpu()
+    got_b1 = got_b1.transpose(0, 1) if time_major else got_b1
+    assert max_rel(got_b1.double(), want[0]) <= (F32_TOL if b_dtype == torch.float32 else BF16_TOL)
+    assert max_rel(dbuf.cpu().double(), want[1]) <= F32_TOL
+    assert max_rel(dw.cpu().double(), want[2].reshape(D, 4)) <= F32_TOL
+    assert max_rel(dbias.cpu().double(), want[3]) <= F32_TOL
+    again = ops.conv_seq_bwd(lay(b1).to(DEV), buf.to(DEV), w.to(DEV), None if done is None else done.to(DEV),
+                             lay(up_v).to(DEV), None if up_tail is None else up_tail.to(DEV), time_major=time_major)
+    assert all(torch.equal(a, b) for a, b in zip((db1, dbuf, dw, dbias), again))
+
+
+def test_conv_seq_train_is_differentiable_and_equals_the_forward_kernel():
+    R, T, D = 40, 24, 128
+    g = torch.Generator().manual_seed(21)
+    b1 = torch.randn(T, R, D, generator=g).bfloat16().to(DEV).requires_grad_()
+    buf = torch.randn(R, 3, D, generator=g).to(DEV).requires_grad_()
+    w = (0.5 * torch.randn(D, 1, 4, generator=g)).to(DEV).requires_grad_()
+    bias = (0.1 * torch.randn(D, generator=g)).to(DEV).requires_grad_()
+    done = (torch.rand(R, T, generator=g) < 0.2).to(DEV)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        v, tail = ops.conv_seq_train(b1, buf, w, bias, done, time_major=True)
+    with torch.no_grad():
+        v0, tail0 = ops.conv_seq(b1.detach(), buf.detach(), w.detach(), bias.detach(), done, time_major=True)
+    assert torch.equal(v, v0) and torch.equal(tail, tail0)
+    up_v = torch.randn(T, R, D, generator=g).to(DEV)
+    (v * up_v).sum().backward()  # the handed-on inputs carry no gradient here
+    want = _conv_truth_grads(b1.detach().float().cpu().transpose(0, 1), buf.detach().cpu(), w.detach().cpu(),
+                             bias.detach().cpu(), done.cpu(), up_v.cpu().transpose(0, 1), None)
+    assert b1.grad.dtype == torch.bfloat16 and w.grad.shape == w.shape
+    assert max_rel(b1.grad.float().cpu().transpose(0, 1).double(), want[0]) <= BF16_TOL
+    assert max_rel(buf.grad.cpu().double(), want[1]) <= F32_TOL
+    assert max_rel(w.grad.cpu().double(), want[2]) <= F32_TOL
+    assert max_rel(bias.grad.cpu().double(), want[3]) <= F32_TOL
