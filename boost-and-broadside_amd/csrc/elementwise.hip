@@ -79,6 +79,38 @@ __global__ __launch_bounds__(kEwThreads) void gelu_mul_kernel(const AT *__restri
     store8_stream(out + row * H + c0, o);
 }
 
+// ---- backward of out = gelu(a) * b:  da = dout * b * gelu'(a),  db = dout * gelu(a) -----------
+// gelu'(v) = Phi(v) + v * phi(v); gelu(a) is rounded to a's dtype first, as the forward does.
+template <typename AT, typename BT, typename OT>
+__global__ __launch_bounds__(kEwThreads) void gelu_mul_bwd_kernel(const AT *__restrict__ a, int64_t a_stride,
+                                                                  const BT *__restrict__ b, int64_t b_stride,
+                                                                  const OT *__restrict__ dout, AT *__restrict__ da,
+                                                                  int64_t da_stride, BT *__restrict__ db, int64_t db_stride,
+                                                                  int64_t R, int H)
+{
+    const int vecs_per_row = H >> 3;
+    const int64_t idx = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+    if (idx >= R * vecs_per_row) return;
+    const int64_t row = idx / vecs_per_row;
+    const int c0 = (int)(idx - row * vecs_per_row) << 3;
+    const Row8 av = load8_stream(a + row * a_stride + c0);
+    const Row8 bv = load8_stream(b + row * b_stride + c0);
+    const Row8 gv = load8_stream(dout + row * H + c0);
+    Row8 ga, gb;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float v = av.v[e];
+        const float cdf = 0.5f * (1.0f + erff(v * 0.70710678118654752f));
+        const float pdf = 0.3989422804014327f * __expf(-0.5f * v * v);
+        float g = v * cdf;
+        if (is_bf16<AT>::value) g = round_to_bf16(g);
+        ga.v[e] = gv.v[e] * bv.v[e] * (cdf + v * pdf);
+        gb.v[e] = gv.v[e] * g;
+    }
+    store8_stream(da + row * da_stride + c0, ga);
+    store8_stream(db + row * db_stride + c0, gb);
+}
+
 template <int LANES, typename DT, typename OT>
 static int launch_norm(const float *x, int64_t x_stride, const void *delta, const float *weight, float eps,
                        float *sum_out, void *norm_out, int64_t R, hipStream_t stream)
@@ -122,6 +154,17 @@ static int launch_gelu_mul(const void *a, int64_t a_stride, const void *b, int64
     if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((gelu_mul_kernel<AT, BT, OT>), dim3((unsigned)blocks), dim3(kEwThreads), 0, stream,
                        (const AT *)a, a_stride, (const BT *)b, b_stride, (OT *)out, R, H);
+    return (int)hipGetLastError();
+}
+
+template <typename AT, typename BT, typename OT>
+static int launch_gelu_mul_bwd(const void *a, int64_t a_stride, const void *b, int64_t b_stride, const void *dout, void *da,
+                               int64_t da_stride, void *db, int64_t db_stride, int64_t R, int H, hipStream_t stream)
+{
+    const int64_t blocks = (R * (H / 8) + kEwThreads - 1) / kEwThreads;
+    if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((gelu_mul_bwd_kernel<AT, BT, OT>), dim3((unsigned)blocks), dim3(kEwThreads), 0, stream, (const AT *)a,
+                       a_stride, (const BT *)b, b_stride, (const OT *)dout, (AT *)da, da_stride, (BT *)db, db_stride, R, H);
     return (int)hipGetLastError();
 }
 
@@ -174,4 +217,36 @@ extern "C" int bnb_gelu_mul_fwd(const void *a, int a_dtype, int64_t a_row_stride
         case 6: return launch_gelu_mul<uint16_t, uint16_t, float>(a, a_row_stride, b, b_row_stride, out, R, H, s);
         default: return launch_gelu_mul<uint16_t, uint16_t, uint16_t>(a, a_row_stride, b, b_row_stride, out, R, H, s);
     }
+}
+
+extern "C" int bnb_gelu_mul_bwd(const void *a, int a_dtype, int64_t a_row_stride, const void *b, int b_dtype,
+                                int64_t b_row_stride, const void *dout, int out_dtype, void *da, int64_t da_row_stride,
+                                void *db, int64_t db_row_stride, int64_t R, int H, void *stream)
+{
+    using namespace bnb;
+    if (R < 0 || H < 1 || a_row_stride < H || b_row_stride < H || da_row_stride < H || db_row_stride < H) return BNB_ERR_BAD_SHAPE;
+    if (R == 0) return 0;
+    if (!a || !b || !dout || !da || !db) return BNB_ERR_NULL_POINTER;
+    for (int dt : {a_dtype, b_dtype, out_dtype})
+        if (dt != BNB_F32 && dt != BNB_BF16) return BNB_ERR_BAD_DTYPE;
+    if (H % 8) return BNB_ERR_UNSUPPORTED;
+    const int64_t ea = a_dtype == BNB_BF16 ? 2 : 4, eb = b_dtype == BNB_BF16 ? 2 : 4;
+    if (!aligned16(a) || !aligned16(b) || !aligned16(dout) || !aligned16(da) || !aligned16(db) || (a_row_stride * ea) % 16 ||
+        (b_row_stride * eb) % 16 || (da_row_stride * ea) % 16 || (db_row_stride * eb) % 16)
+        return BNB_ERR_MISALIGNED;
+    hipStream_t s = (hipStream_t)stream;
+#define BNB_GMB(AT, BT, OT) \
+    return launch_gelu_mul_bwd<AT, BT, OT>(a, a_row_stride, b, b_row_stride, dout, da, da_row_stride, db, db_row_stride, R, H, s)
+    const int key = (a_dtype << 2) | (b_dtype << 1) | out_dtype;
+    switch (key) {
+        case 0: BNB_GMB(float, float, float);
+        case 1: BNB_GMB(float, float, uint16_t);
+        case 2: BNB_GMB(float, uint16_t, float);
+        case 3: BNB_GMB(float, uint16_t, uint16_t);
+        case 4: BNB_GMB(uint16_t, float, float);
+        case 5: BNB_GMB(uint16_t, float, uint16_t);
+        case 6: BNB_GMB(uint16_t, uint16_t, float);
+        default: BNB_GMB(uint16_t, uint16_t, uint16_t);
+    }
+#undef BNB_GMB
 }

@@ -103,6 +103,66 @@ def sdpa_masked(
     return out
 
 
+def sdpa_train_supported(qkv: torch.Tensor, n_heads: int) -> bool:
+    """Whether ``sdpa_train`` covers this input: head size 32, at most 32 tokens and 8 heads, on the GPU."""
+    if not (qkv.is_cuda and qkv.dim() == 3 and qkv.dtype in (torch.float32, torch.bfloat16) and qkv.shape[-1] % 3 == 0):
+        return False
+    D = qkv.shape[-1] // 3
+    return D % n_heads == 0 and D // n_heads == 32 and 1 <= qkv.shape[1] <= 32 and n_heads <= 8
+
+
+def sdpa_masked_bwd(qkv: torch.Tensor, alive: torch.Tensor | None, n_heads: int, out: torch.Tensor,
+                    dout: torch.Tensor) -> torch.Tensor:
+    """Gradient of ``sdpa_masked`` with respect to ``qkv`` from the forward's result and its gradient."""
+    B, NM, D3 = qkv.shape
+    D = D3 // 3
+    if out.shape != (B, NM, D) or dout.shape != (B, NM, D) or out.dtype != qkv.dtype:
+        raise ValueError("out and dout must be (B, NM, D) in qkv's dtype")
+    for name, t in (("qkv", qkv), ("out", out), ("dout", dout)):
+        _need_device(t, name)
+    if B and (qkv.stride(-1) != 1 or (B > 1 and qkv.stride(0) != NM * qkv.stride(1))):
+        qkv = qkv.contiguous()
+    out = out.contiguous()
+    dout = dout.to(qkv.dtype).contiguous()
+    mask_ptr = None
+    if alive is not None:
+        if alive.shape != (B, NM) or alive.dtype not in (torch.bool, torch.uint8):
+            raise ValueError(f"alive must be a bool {(B, NM)} tensor")
+        alive = alive.contiguous()
+        mask_ptr = alive.data_ptr()
+    dqkv = torch.empty((B, NM, D3), dtype=qkv.dtype, device=qkv.device)
+    if B:
+        with torch.cuda.device(qkv.device):
+            rc = _native.load().bnb_sdpa_masked_bwd(qkv.data_ptr(), qkv.stride(1), mask_ptr, out.data_ptr(), dout.data_ptr(),
+                                                    dqkv.data_ptr(), B, NM, n_heads, D // n_heads, _code(qkv, "qkv"), _stream())
+        _native.check(rc, "bnb_sdpa_masked_bwd")
+    return dqkv
+
+
+class _SdpaTrain(torch.autograd.Function):
+    """``sdpa_masked`` with its backward kernel."""
+
+    @staticmethod
+    def forward(ctx, qkv, alive, n_heads):
+        with torch.no_grad():
+            out = sdpa_masked(qkv, alive, n_heads)
+        ctx.save_for_backward(qkv, out)
+        ctx.alive = alive
+        ctx.n_heads = n_heads
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        qkv, out = ctx.saved_tensors
+        return sdpa_masked_bwd(qkv, ctx.alive, ctx.n_heads, out, dout), None, None
+
+
+def sdpa_train(qkv: torch.Tensor, alive: torch.Tensor | None, n_heads: int) -> torch.Tensor:
+    """Differentiable ``sdpa_masked`` (use where ``sdpa_train_supported`` holds)."""
+    with torch.autocast("cuda", enabled=False):
+        return _SdpaTrain.apply(qkv, alive, n_heads)
+
+
 def cross_supported(q: torch.Tensor, kv: torch.Tensor, n_heads: int) -> bool:
     """Whether ``sdpa_cross`` covers these shapes (bf16, head size 32, 1..2048 keys, <= 160 queries)."""
     D = kv.shape[-1] // 2
@@ -1129,6 +1189,63 @@ def gelu_mul(a: torch.Tensor, b: torch.Tensor, *, out_dtype: torch.dtype | None 
             )
         _native.check(rc, "bnb_gelu_mul_fwd")
     return out.reshape(a.shape)
+
+
+def gelu_mul_bwd(a: torch.Tensor, b: torch.Tensor, dout: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Backward of ``gelu_mul``: ``(da, db)`` in a's and b's dtypes from the gradient of the product."""
+    H = a.shape[-1]
+    if a.shape != b.shape or dout.shape != a.shape or H % 8:
+        raise ValueError("a, b and dout must share a shape with a multiple of 8 channels")
+    for name, t in (("a", a), ("b", b), ("dout", dout)):
+        _need_device(t, name)
+
+    def rows(t):
+        t2 = t.reshape(-1, H) if t.dim() != 2 else t
+        if t2.numel() and t2.stride(-1) != 1:
+            t2 = t2.contiguous()
+        return t2
+
+    a2, b2, g2 = rows(a), rows(b), rows(dout).contiguous()
+    R = a2.shape[0]
+    da = torch.empty((R, H), dtype=a.dtype, device=a.device)
+    db = torch.empty((R, H), dtype=b.dtype, device=a.device)
+    if R:
+        with torch.cuda.device(a.device):
+            rc = _native.load().bnb_gelu_mul_bwd(
+                a2.data_ptr(), _code(a2, "a"), a2.stride(0), b2.data_ptr(), _code(b2, "b"), b2.stride(0),
+                g2.data_ptr(), _code(g2, "dout"), da.data_ptr(), H, db.data_ptr(), H, R, H, _stream(),
+            )
+        _native.check(rc, "bnb_gelu_mul_bwd")
+    return da.reshape(a.shape), db.reshape(a.shape)
+
+
+class _GeluMulTrain(torch.autograd.Function):
+    """``gelu(a) * b`` with one kernel forward and one backward."""
+
+    @staticmethod
+    def forward(ctx, a, b, out_dtype):
+        with torch.no_grad():
+            out = gelu_mul(a, b, out_dtype=out_dtype)
+        ctx.save_for_backward(a, b)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        a, b = ctx.saved_tensors
+        da, db = gelu_mul_bwd(a, b, dout)
+        return da, db, None
+
+
+def gelu_mul_train_supported(a: torch.Tensor, b: torch.Tensor) -> bool:
+    """Whether ``gelu_mul_train`` covers these operands."""
+    ok = (torch.float32, torch.bfloat16)
+    return a.is_cuda and b.is_cuda and a.shape == b.shape and a.shape[-1] % 8 == 0 and a.dtype in ok and b.dtype in ok
+
+
+def gelu_mul_train(a: torch.Tensor, b: torch.Tensor, *, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """Differentiable ``gelu_mul``."""
+    with torch.autocast("cuda", enabled=False):
+        return _GeluMulTrain.apply(a, b, out_dtype)
 
 
 def copy_bytes(src: torch.Tensor, dst: torch.Tensor) -> None:

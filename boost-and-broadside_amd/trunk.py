@@ -97,6 +97,16 @@ def _project(layer: nn.Linear, x: torch.Tensor) -> torch.Tensor:
     return F.linear(x, wc, bc)
 
 
+def _gelu_gate(gate: torch.Tensor, value: torch.Tensor) -> torch.Tensor:
+    """``gelu(gate) * value`` in grad mode: one kernel forward and one backward on the GPU (the product
+    rounded once to the projection dtype, which is what the next Linear would cast it to), torch ops elsewhere."""
+    act = _projection_dtype()
+    if ops.gelu_mul_train_supported(gate, value) and act in (torch.float32, torch.bfloat16):
+        out_dtype = act if act == torch.bfloat16 else torch.promote_types(gate.dtype, value.dtype)
+        return ops.gelu_mul_train(gate, value, out_dtype=out_dtype)
+    return F.gelu(gate) * value
+
+
 def _train_norm(norm: nn.RMSNorm, x: torch.Tensor, delta: torch.Tensor | None = None):
     """``norm(x)``, or with ``delta`` the pair ``(x + delta, norm(x + delta))``, differentiable.
 
@@ -194,7 +204,7 @@ class GatedMLP(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         hidden = self.gate_proj.out_features
         if not x.is_cuda or hidden % 8 or x.dtype not in (torch.float32, torch.bfloat16) or torch.is_grad_enabled():
-            return _project(self.down_proj, F.gelu(_project(self.gate_proj, x)) * _project(self.up_proj, x))
+            return _project(self.down_proj, _gelu_gate(_project(self.gate_proj, x), _project(self.up_proj, x)))
         # one GEMM for [gate | up], one kernel for gelu(gate) * up, one GEMM down
         wg, wu = self.gate_proj.weight, self.up_proj.weight
         w = _cached_cast(self, "_bnb_gate_up", (wg, wu), x.dtype, lambda: torch.cat([wg, wu], dim=0).detach().to(x.dtype))
@@ -258,8 +268,12 @@ class TransformerBlock(nn.Module):
         if qkv is None:
             qkv = _project(self.qkv, x)  # (B, N, 3D), fp32 or bf16 under autocast
         if torch.is_grad_enabled():
-            # training: the attention itself stays with torch's differentiable SDPA
-            merged = self._self_attention_autograd(qkv, alive_mask)
+            # training: forward and backward kernels for the small token counts of the update,
+            # torch's differentiable SDPA for the rest
+            if ops.sdpa_train_supported(qkv, self.n_heads):
+                merged = ops.sdpa_train(qkv, alive_mask, self.n_heads)
+            else:
+                merged = self._self_attention_autograd(qkv, alive_mask)
             if self.reads_bullets and bullets is not None:
                 if isinstance(bullet_mask, ops.CompactRows):
                     bullet_mask = bullet_mask.mask
@@ -482,7 +496,7 @@ class GriffinTemporalBlock(nn.Module):
                 return fused
             x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=r, eps=self.norm2.eps, out_dtype=act)
             return x1 + self.gated_mlp(n2)
-        x1, n2 = _train_norm(self.norm2, x, _project(self.linear_out, y * F.gelu(gate_in)))
+        x1, n2 = _train_norm(self.norm2, x, _project(self.linear_out, _gelu_gate(gate_in, y)))
         return x1 + self.gated_mlp(n2)
 
     def _step(self, x, h_in, conv_in, h_out, conv_out, reset, rows_per_env):
@@ -601,7 +615,7 @@ class GriffinTemporalBlock(nn.Module):
                 return fused
             x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=r, eps=self.norm2.eps, out_dtype=act)
             return x1 + self.gated_mlp(n2)
-        x1, n2 = _train_norm(self.norm2, x, _project(self.linear_out, b1 * F.gelu(gate_in)))
+        x1, n2 = _train_norm(self.norm2, x, _project(self.linear_out, _gelu_gate(gate_in, b1)))
         return x1 + self.gated_mlp(n2)
 
 

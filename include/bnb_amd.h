@@ -265,6 +265,24 @@ int bnb_linear_wgrad_fwd(const void *dy, int64_t dy_row_stride, const void *x, i
                          int64_t R, int N, int K, void *stream);
 
 /*
+ * Backward of bnb_sdpa_masked_fwd for small token counts: what autograd computes through
+ * models/yemong/attention.py:136-147 (head split, key bias on dead entities, SDPA, head merge)
+ * in the PPO update (train/rl/ppo.py:1417-1425).
+ *
+ *   qkv    (B, NM, 3*H*dh) as passed to the forward, rows qkv_row_stride elements apart
+ *          (environments NM rows apart)
+ *   alive  (B, NM) bytes or NULL, as in the forward
+ *   out    (B, NM, H*dh) contiguous: the forward's result
+ *   dout   (B, NM, H*dh) contiguous: its gradient
+ *   dqkv   (B, NM, 3*H*dh) contiguous: gradient of qkv
+ * all in `dtype` (BNB_F32 or BNB_BF16), arithmetic in fp32, every sum in a fixed order.
+ * Requirements: dh == 32, NM <= 32, H <= 8; 16-byte aligned rows.  Other shapes return
+ * BNB_ERR_UNSUPPORTED (the caller keeps the library's differentiable attention for them).
+ */
+int bnb_sdpa_masked_bwd(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, const void *out,
+                        const void *dout, void *dqkv, int64_t B, int NM, int H, int dh, int dtype, void *stream);
+
+/*
  * RMSNorm backward:  y = x * rsqrt(mean(x^2) + eps) * weight
  *   dx[r] = rstd * (dy[r] * weight) - x[r] * rstd^3 * mean(dy[r] * weight * x[r])  (+ grad_sum[r])
  *   dw    = sum_r dy[r] * x[r] * rstd
@@ -579,6 +597,17 @@ int bnb_ffn_fused_proj_fwd(const float *x, int64_t x_row_stride, const void *row
  */
 int bnb_gelu_mul_fwd(const void *a, int a_dtype, int64_t a_row_stride, const void *b, int b_dtype,
                      int64_t b_row_stride, void *out, int out_dtype, int64_t R, int H, void *stream);
+
+/*
+ * Backward of bnb_gelu_mul_fwd: da = dout * b * gelu'(a), db = dout * gelu(a), each rounded once
+ * to its tensor's dtype; what autograd runs as two multiplications and a gelu-backward kernel
+ * through attention.py:36-37 / griffin.py:281-282 in the PPO update (train/rl/ppo.py:1417-1425).
+ * dout is (R, H) contiguous in out_dtype; da and db are (R, H) with row strides in elements.
+ * Requirements as for the forward.
+ */
+int bnb_gelu_mul_bwd(const void *a, int a_dtype, int64_t a_row_stride, const void *b, int b_dtype,
+                     int64_t b_row_stride, const void *dout, int out_dtype, void *da, int64_t da_row_stride,
+                     void *db, int64_t db_row_stride, int64_t R, int H, void *stream);
 
 /*
  * Plain device-to-device copy of `bytes` bytes (multiple of 16, 16-byte aligned) by a

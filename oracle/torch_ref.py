@@ -20,6 +20,9 @@ How each function is pinned (see tests/test_oracle_pins.py):
                        (oracle/bruteforce.py) + closed forms (all-alive,
                        single alive key, all dead => mean of V, dead-key
                        perturbation invariance, permutation equivariance).
+* ``sdpa_masked_softmax``  the same function written out, for gradients: values and
+                       gradients equal ``sdpa_masked``'s wherever an environment has a live
+                       key, closed form (uniform weights) where it has none.
 * ``rglru_step``       closed forms from the recurrence (x=0, h=0, lambda=0
                        with r=1, r=0 => clamp floor) + the C restatement.
 * ``conv_sequence``    library ``F.conv1d`` (no boundaries) and per-episode ``F.conv1d`` on
@@ -74,6 +77,28 @@ def sdpa_masked(qkv: torch.Tensor, alive: torch.Tensor | None, n_heads: int) -> 
     q, k, v = (t.reshape(B, NM, n_heads, dh).transpose(1, 2) for t in qkv.split(D, dim=-1))
     bias = None if alive is None else key_bias(alive, q.dtype)
     o = F.scaled_dot_product_attention(q, k, v, attn_mask=bias, dropout_p=0.0)
+    return o.transpose(1, 2).reshape(B, NM, D)
+
+
+def sdpa_masked_softmax(qkv: torch.Tensor, alive: torch.Tensor | None, n_heads: int) -> torch.Tensor:
+    """``sdpa_masked`` with the attention written out (scores, bias, softmax, weighted sum) instead
+    of the library call of models/yemong/attention.py:147: the statement whose autograd is the
+    gradient truth.
+
+    The forward values are the same.  The gradients are the same wherever an environment has a
+    live key.  For an environment without one, the fused library backward recomputes the weights
+    from ``scores + bias - logsumexp`` with the finfo.min/2 bias absorbing ``log(NM)``, which turns
+    every weight into 1 instead of 1/NM (an artefact of that kernel, NM times the gradient of
+    the function it evaluated); this statement keeps the weights it used in the forward.
+    """
+    B, NM, D3 = qkv.shape
+    D = D3 // 3
+    dh = D // n_heads
+    q, k, v = (t.reshape(B, NM, n_heads, dh).transpose(1, 2) for t in qkv.split(D, dim=-1))
+    scores = q @ k.transpose(-1, -2) / (dh ** 0.5)
+    if alive is not None:
+        scores = scores + key_bias(alive, q.dtype)
+    o = torch.softmax(scores, dim=-1) @ v
     return o.transpose(1, 2).reshape(B, NM, D)
 
 

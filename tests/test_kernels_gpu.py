@@ -1645,3 +1645,99 @@ def test_conv_seq_train_is_differentiable_and_equals_the_forward_kernel():
     assert max_rel(buf.grad.cpu().double(), want[1]) <= F32_TOL
     assert max_rel(w.grad.cpu().double(), want[2]) <= F32_TOL
     assert max_rel(bias.grad.cpu().double(), want[3]) <= F32_TOL
+
+
+# ------------------------------------------------------------------ gelu(a) * b backward
+
+
+@pytest.mark.parametrize("R,H", [(1, 8), (37, 128), (1000, 512), (4099, 136)])
+@pytest.mark.parametrize("a_dtype,b_dtype,o_dtype", [(torch.float32, torch.float32, torch.float32),
+                                                     (torch.bfloat16, torch.bfloat16, torch.bfloat16),
+                                                     (torch.bfloat16, torch.float32, torch.bfloat16)])
+def test_gelu_mul_train_gradients_match_autograd_of_erf_gelu(R, H, a_dtype, b_dtype, o_dtype):
+    g = torch.Generator().manual_seed(R + H)
+    a0 = (2.0 * torch.randn(R, H, generator=g)).to(a_dtype)
+    b0 = torch.randn(R, H, generator=g).to(b_dtype)
+    up = torch.randn(R, H, generator=g).to(o_dtype)
+    a = a0.to(DEV).requires_grad_()
+    b = b0.to(DEV).requires_grad_()
+    out = ops.gelu_mul_train(a, b, out_dtype=o_dtype)
+    with torch.no_grad():
+        assert torch.equal(out, ops.gelu_mul(a.detach(), b.detach(), out_dtype=o_dtype))
+    out.backward(up.to(DEV))
+    ad = a0.double().requires_grad_()
+    bd = b0.double().requires_grad_()
+    (torch.nn.functional.gelu(ad) * bd * up.double()).sum().backward()
+    assert a.grad.dtype == a_dtype and b.grad.dtype == b_dtype
+    assert max_rel(a.grad.float().cpu().double(), ad.grad) <= (F32_TOL if a_dtype == torch.float32 else BF16_TOL)
+    assert max_rel(b.grad.float().cpu().double(), bd.grad) <= (F32_TOL if a_dtype == b_dtype == torch.float32 else BF16_TOL)
+
+
+def test_gelu_mul_bwd_reads_column_blocks_of_one_projection_output():
+    R, H = 300, 256
+    g = torch.Generator().manual_seed(9)
+    gu = torch.randn(R, 2 * H, generator=g).bfloat16().to(DEV)
+    dout = torch.randn(R, H, generator=g).bfloat16().to(DEV)
+    da, db = ops.gelu_mul_bwd(gu[:, :H], gu[:, H:], dout)
+    da2, db2 = ops.gelu_mul_bwd(gu[:, :H].contiguous(), gu[:, H:].contiguous(), dout)
+    assert torch.equal(da, da2) and torch.equal(db, db2)
+
+
+# ------------------------------------------------------------------ masked attention backward
+
+
+def _sdpa_truth_grad(qkv, alive, H, up):
+    """Autograd through the oracle's written-out statement of attention.py:136-147, float64 (pinned against the
+    library call in tests/test_oracle_pins.py; they differ only in the gradient of environments without a live key)."""
+    x = qkv.double().requires_grad_()
+    out = torch_ref.sdpa_masked_softmax(x, alive, H)
+    (out * up.double()).sum().backward()
+    return out.detach(), x.grad
+
+
+@pytest.mark.parametrize("B,NM,H", [(3, 12, 4), (70, 12, 4), (5, 27, 4), (4, 1, 4), (6, 32, 4), (9, 7, 2), (3, 20, 8), (1000, 12, 4)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("p_alive", [1.0, 0.7, 0.0])
+def test_sdpa_masked_bwd_matches_autograd_of_the_oracle(B, NM, H, dtype, p_alive):
+    D = 32 * H
+    qkv = _qkv(B * 31 + NM, B, NM, D, dtype, scale=1.5)
+    alive = None if p_alive == 1.0 else _alive(NM + B, B, NM, p_alive)
+    if alive is not None and p_alive > 0 and B > 2:
+        alive[1] = False  # one environment without a live key among live ones
+    g = torch.Generator().manual_seed(B + NM)
+    up = torch.randn(B, NM, D, generator=g).to(dtype)
+    ref_out, ref_grad = _sdpa_truth_grad(qkv, alive, H, up)
+    out = ops.sdpa_masked(qkv.to(DEV), None if alive is None else alive.to(DEV), H)
+    dqkv = ops.sdpa_masked_bwd(qkv.to(DEV), None if alive is None else alive.to(DEV), H, out, up.to(DEV))
+    torch.cuda.synchronize()
+    tol = F32_TOL if dtype == torch.float32 else BF16_TOL
+    assert dqkv.dtype == dtype and dqkv.shape == qkv.shape
+    assert max_rel(out.float().cpu().double(), ref_out) <= tol
+    # the bf16 forward result enters the backward (rowsum(dO * O)), so compare per third
+    for name, cols in (("dQ", slice(0, D)), ("dK", slice(D, 2 * D)), ("dV", slice(2 * D, 3 * D))):
+        if NM == 1 and name != "dV":  # a single key: the softmax is constant, dQ = dK = 0 up to float64 noise
+            assert dqkv[..., cols].float().abs().max() <= 1e-6 * ref_grad.abs().max(), name
+            continue
+        assert max_rel(dqkv[..., cols].float().cpu().double(), ref_grad[..., cols]) <= tol, name
+    if alive is not None and p_alive > 0:
+        dead = ~alive & alive.any(dim=1, keepdim=True)  # dead keys of environments that have live ones
+        assert not dqkv.cpu()[..., D:][dead].any()  # dead keys receive exactly nothing
+    again = ops.sdpa_masked_bwd(qkv.to(DEV), None if alive is None else alive.to(DEV), H, out, up.to(DEV))
+    assert torch.equal(dqkv, again)
+
+
+def test_sdpa_train_is_differentiable_and_reads_strided_rows():
+    B, NM, H, D = 33, 12, 4, 128
+    g = torch.Generator().manual_seed(4)
+    wide = (torch.randn(B, NM, 3 * D + 64, generator=g)).bfloat16().to(DEV).requires_grad_()
+    alive = (torch.rand(B, NM, generator=g) < 0.8).to(DEV)
+    up = torch.randn(B, NM, D, generator=g).to(DEV)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = ops.sdpa_train(wide[..., 64:], alive, H)
+    (out.float() * up).sum().backward()
+    ref_out, ref_grad = _sdpa_truth_grad(wide.detach()[..., 64:].float().cpu(), alive.cpu(), H, up.bfloat16().cpu())
+    assert max_rel(out.detach().float().cpu().double(), ref_out) <= BF16_TOL
+    assert not wide.grad[..., :64].any()
+    assert max_rel(wide.grad[..., 64:].float().cpu().double(), ref_grad) <= BF16_TOL
+    assert not ops.sdpa_train_supported(torch.zeros(2, 40, 384, device=DEV), 4)
+    assert not ops.sdpa_train_supported(torch.zeros(2, 12, 192, device=DEV), 4)

@@ -37,6 +37,43 @@ def test_bias_constants_per_dtype():
     assert float(b16[0, 0, 0, 1]) == pytest.approx(-1.6947656946257677e38, rel=1e-7)
 
 
+def test_written_out_attention_pins_values_and_gradients_of_the_library_call():
+    """The gradient truth of the attention-backward tests: same values as the library call everywhere,
+    same gradients wherever an environment has a live key; without one the library's fused backward
+    returns NM times the gradient of the function it evaluated (weights 1 instead of 1/NM)."""
+    B, NM, H, D = 6, 9, 4, 128
+    qkv = _qkv(5, B, NM, D, torch.float64)
+    g = torch.Generator().manual_seed(6)
+    alive = torch.rand(B, NM, generator=g) < 0.6
+    alive[:, 0] = True
+    alive[2] = False
+    up = torch.randn(B, NM, D, generator=g, dtype=torch.float64)
+    grads = []
+    for fn in (torch_ref.sdpa_masked, torch_ref.sdpa_masked_softmax):
+        x = qkv.clone().requires_grad_()
+        out = fn(x, alive, H)
+        (out * up).sum().backward()
+        grads.append((out.detach(), x.grad))
+    assert torch.allclose(grads[0][0], grads[1][0], rtol=1e-12, atol=1e-13)
+    some = alive.any(dim=1)
+    assert torch.allclose(grads[0][1][some], grads[1][1][some], rtol=1e-10, atol=1e-12)
+    # the all-dead environment, against the closed form with uniform weights 1/NM
+    q, k, v = (t.reshape(NM, H, 32).transpose(0, 1) for t in qkv[2].split(D, dim=-1))
+    do = up[2].reshape(NM, H, 32).transpose(0, 1)
+    P = torch.full((H, NM, NM), 1.0 / NM, dtype=torch.float64)
+    dP = do @ v.transpose(-1, -2)
+    dS = P * (dP - (P * dP).sum(-1, keepdim=True))
+    want = torch.cat([(dS @ k / 32 ** 0.5).transpose(0, 1).reshape(NM, D),
+                      (dS.transpose(-1, -2) @ q / 32 ** 0.5).transpose(0, 1).reshape(NM, D),
+                      (P.transpose(-1, -2) @ do).transpose(0, 1).reshape(NM, D)], dim=-1)
+    assert torch.allclose(grads[1][1][2], want, rtol=1e-10, atol=1e-12)
+    # and no-mask gradients agree as well
+    x0, x1 = qkv.clone().requires_grad_(), qkv.clone().requires_grad_()
+    (torch_ref.sdpa_masked(x0, None, H) * up).sum().backward()
+    (torch_ref.sdpa_masked_softmax(x1, None, H) * up).sum().backward()
+    assert torch.allclose(x0.grad, x1.grad, rtol=1e-10, atol=1e-12)
+
+
 def test_hand_computed_two_key_case():
     # one head, dh=2; scores 0 and ln 3 => weights 1/4, 3/4; V rows (4,0),(0,8) => (1,6)
     D = 2
