@@ -717,14 +717,49 @@ def main():
 
             from boost_and_broadside_amd import trunk as trunk_module
             t_up = timed_loop(update_step, 3, 2) / 3
-            with trunk_module.library_weight_gradients():
+            with trunk_module.library_update_path():
                 t_up_lib = timed_loop(update_step, 3, 2) / 3
+            # the other update-path kernels at the same size, each against its algorithmic bytes
+            def stream_leg(fn, nbytes, reps=8):
+                t = timed_loop(fn, reps, 3) / reps
+                return {"us": t * 1e6, "algorithmic_bytes": nbytes, "GBps": nbytes / t / 1e9, "frac_of_hbm_peak": nbytes / t / peak}
+
+            kern = {}
+            xn = torch.randn(Rw, D, device=dev, generator=gen)
+            dyn = torch.randn(Rw, D, device=dev, generator=gen).to(torch.bfloat16)
+            gsn = torch.randn(Rw, D, device=dev, generator=gen)
+            wn = torch.ones(D, device=dev)
+            kern["rmsnorm_bwd"] = stream_leg(lambda t: ops.rmsnorm_bwd(xn, dyn, wn, grad_sum=gsn), Rw * D * (4 + 2 + 4 + 4))
+            del xn, dyn, gsn
+            ag = torch.randn(Rw, 4 * D, device=dev, generator=gen).to(torch.bfloat16)
+            bg = torch.randn(Rw, 4 * D, device=dev, generator=gen).to(torch.bfloat16)
+            dg = torch.randn(Rw, 4 * D, device=dev, generator=gen).to(torch.bfloat16)
+            kern["gelu_mul_bwd"] = stream_leg(lambda t: ops.gelu_mul_bwd(ag, bg, dg), Rw * 4 * D * 2 * 5)
+            del ag, bg, dg
+            Ba = Tu * Bu
+            qa = torch.randn(Ba, Nu + Mu, 3 * D, device=dev, generator=gen).to(torch.bfloat16)
+            aa = torch.rand(Ba, Nu + Mu, device=dev, generator=gen) < 0.9
+            oa = ops.sdpa_masked(qa, aa, H)
+            da = torch.randn(Ba, Nu + Mu, D, device=dev, generator=gen).to(torch.bfloat16)
+            kern["sdpa_masked_bwd"] = stream_leg(lambda t: ops.sdpa_masked_bwd(qa, aa, H, oa, da), Ba * (Nu + Mu) * D * 2 * (3 + 1 + 1 + 3))
+            kern["sdpa_masked_fwd"] = stream_leg(lambda t: ops.sdpa_masked(qa, aa, H, out=oa), Ba * (Nu + Mu) * D * 2 * 4)
+            del qa, aa, oa, da
+            Rc = Bu * Nu
+            bc = torch.randn(Tu, Rc, D, device=dev, generator=gen).to(torch.bfloat16)
+            cc = torch.randn(Rc, 3, D, device=dev, generator=gen)
+            wc = torch.randn(D, 1, 4, device=dev, generator=gen)
+            dc = torch.rand(Rc, Tu, device=dev, generator=gen) < 0.02
+            dvc = torch.randn(Tu, Rc, D, device=dev, generator=gen)
+            kern["conv_seq_bwd"] = stream_leg(lambda t: ops.conv_seq_bwd(bc, cc, wc, dc, dvc, time_major=True), Tu * Rc * D * (2 + 4 + 2))
+            del bc, cc, dvc
             result["update_path"] = {
-                "rows": Rw, "linear_wgrad": wg, "block_fwd_bwd_ms": t_up * 1e3, "block_fwd_bwd_library_wgrad_ms": t_up_lib * 1e3,
+                "rows": Rw, "linear_wgrad": wg, "kernels": kern, "block_fwd_bwd_ms": t_up * 1e3,
+                "block_fwd_bwd_library_ms": t_up_lib * 1e3,
                 "what": "bnb_linear_wgrad_fwd (dW = dy^T x, bf16 in, fp32 out, rows split over the chip) beside the library "
-                        "GEMM on the same operands; block = one YemongBlock (2 attention + 1 temporal sublayer), T = 128 x 256 "
-                        "environments of 4v4, forward + backward under bf16 autocast, with the weight gradients on that "
-                        "kernel and on the library",
+                        "GEMM on the same operands; kernels = the norm, gelu-gate, attention and conv backward kernels at the "
+                        "sizes of the block below; block = one YemongBlock (2 attention + 1 temporal sublayer), T = 128 x 256 "
+                        "environments of 4v4, forward + backward under bf16 autocast, on the update-path kernels and with "
+                        "torch's own differentiable ops in their place (the recurrence keeps its kernels in both)",
             }
             del blk, xu, au, hu, cu, du
 

@@ -56,15 +56,19 @@ def _fused_ok(x: torch.Tensor, act: torch.dtype) -> bool:
     )
 
 
+_TRAIN_KERNELS = True  # grad-mode norms, gates, conv, attention and weight gradients on the library's own kernels when False
+
+
 @contextlib.contextmanager
-def library_weight_gradients():
-    """Inside the block every Linear weight gradient is left to the library GEMM (comparisons, debugging)."""
-    global _WGRAD_MIN_ROWS
-    keep, _WGRAD_MIN_ROWS = _WGRAD_MIN_ROWS, 1 << 62
+def library_update_path():
+    """Inside the block the grad-mode path uses torch's own differentiable ops only (norms, gelu gates,
+    conv taps, attention, weight-gradient GEMMs); the recurrence keeps its kernels.  For comparisons."""
+    global _TRAIN_KERNELS
+    keep, _TRAIN_KERNELS = _TRAIN_KERNELS, False
     try:
         yield
     finally:
-        _WGRAD_MIN_ROWS = keep
+        _TRAIN_KERNELS = keep
 
 
 def _cached_cast(owner: nn.Module, slot: str, tensors: tuple, dtype: torch.dtype, build):
@@ -85,7 +89,7 @@ def _project(layer: nn.Linear, x: torch.Tensor) -> torch.Tensor:
     w, b = layer.weight, layer.bias
     if torch.is_grad_enabled():
         if (
-            w.requires_grad and w.dtype == torch.float32 and _projection_dtype() == torch.bfloat16
+            _TRAIN_KERNELS and w.requires_grad and w.dtype == torch.float32 and _projection_dtype() == torch.bfloat16
             and x.numel() >= _WGRAD_MIN_ROWS * x.shape[-1] and ops.linear_wgrad_supported(x, w)
         ):
             return ops.linear_train(x, w, b)  # bf16 like autocast; weight gradient on the row-sliced kernel
@@ -101,7 +105,7 @@ def _gelu_gate(gate: torch.Tensor, value: torch.Tensor) -> torch.Tensor:
     """``gelu(gate) * value`` in grad mode: one kernel forward and one backward on the GPU (the product
     rounded once to the projection dtype, which is what the next Linear would cast it to), torch ops elsewhere."""
     act = _projection_dtype()
-    if ops.gelu_mul_train_supported(gate, value) and act in (torch.float32, torch.bfloat16):
+    if _TRAIN_KERNELS and ops.gelu_mul_train_supported(gate, value) and act in (torch.float32, torch.bfloat16):
         out_dtype = act if act == torch.bfloat16 else torch.promote_types(gate.dtype, value.dtype)
         return ops.gelu_mul_train(gate, value, out_dtype=out_dtype)
     return F.gelu(gate) * value
@@ -115,7 +119,7 @@ def _train_norm(norm: nn.RMSNorm, x: torch.Tensor, delta: torch.Tensor | None = 
     anything else is the module itself."""
     act = _projection_dtype()
     if (
-        torch.is_grad_enabled() and act in (torch.float32, torch.bfloat16) and ops.rmsnorm_train_supported(x)
+        _TRAIN_KERNELS and torch.is_grad_enabled() and act in (torch.float32, torch.bfloat16) and ops.rmsnorm_train_supported(x)
         and norm.weight is not None and norm.weight.dtype == torch.float32
         and (delta is None or (delta.shape == x.shape and delta.dtype in (torch.float32, torch.bfloat16)))
     ):
@@ -270,7 +274,7 @@ class TransformerBlock(nn.Module):
         if torch.is_grad_enabled():
             # training: forward and backward kernels for the small token counts of the update,
             # torch's differentiable SDPA for the rest
-            if ops.sdpa_train_supported(qkv, self.n_heads):
+            if _TRAIN_KERNELS and ops.sdpa_train_supported(qkv, self.n_heads):
                 merged = ops.sdpa_train(qkv, alive_mask, self.n_heads)
             else:
                 merged = self._self_attention_autograd(qkv, alive_mask)
@@ -457,7 +461,8 @@ class GriffinTemporalBlock(nn.Module):
         forward and backward kernels."""
         normed = _train_norm(self.norm1, x_seq)
         b1 = _project(self.linear1, normed)
-        if ops.conv_seq_train_supported(b1) and conv_buf.dtype == torch.float32 and self.conv.weight.dtype == torch.float32:
+        if (_TRAIN_KERNELS and ops.conv_seq_train_supported(b1) and conv_buf.dtype == torch.float32
+                and self.conv.weight.dtype == torch.float32):
             # conv forward and backward on their kernels (one pass each instead of a dozen element-wise ops per tap)
             v, new_buf = ops.conv_seq_train(b1, conv_buf, self.conv.weight, self.conv.bias, done_mask, time_major=time_major)
             y, new_h = self.rg_lru.forward_sequence(v, h0, done_mask, time_major=time_major)

@@ -544,9 +544,10 @@ def test_attention_block_outside_kernel_coverage_uses_the_library_on_the_device(
     assert err.value.code == _native.ERR_UNSUPPORTED
 
 
-def test_update_path_weight_gradients_agree_between_the_row_sliced_kernel_and_the_library(monkeypatch):
-    """Under bf16 autocast with gradients on, Linear layers with enough rows take ops.linear_train;
-    the parameter gradients must agree with the same update computed through nn.Linear alone."""
+def test_update_path_gradients_agree_between_the_kernels_and_the_library_ops(monkeypatch):
+    """Under bf16 autocast with gradients on, the block runs its norms, gates, conv, attention and Linear
+    weight gradients on the training kernels; every parameter gradient must agree with the same update
+    computed through torch's own differentiable ops."""
     from boost_and_broadside_amd import ops, trunk
 
     cfg = _cfg(128, 4, spatial=1, temporal=1)
@@ -577,7 +578,7 @@ def test_update_path_weight_gradients_agree_between_the_row_sliced_kernel_and_th
     routed = grads()
     assert calls, "no Linear layer took the row-sliced weight gradient"
     n_calls = len(calls)
-    with trunk.library_weight_gradients():
+    with trunk.library_update_path():
         library = grads()
     assert len(calls) == n_calls
     for name, g in routed.items():
