@@ -25,7 +25,7 @@ template <int LANES, typename GT, bool HAS_SUM>
 __global__ __launch_bounds__(kNbThreads) void rmsnorm_bwd_kernel(
     const float *__restrict__ x, int64_t x_stride, const GT *__restrict__ dy, int64_t dy_stride,
     const float *__restrict__ weight, float eps, const float *__restrict__ grad_sum, float *__restrict__ dx,
-    float *__restrict__ partials, int64_t R)
+    uint16_t *__restrict__ dx_bf16, float *__restrict__ partials, int64_t R)
 {
     constexpr int D = LANES * 8;
     constexpr int ROWS = kNbThreads / LANES;
@@ -78,6 +78,7 @@ __global__ __launch_bounds__(kNbThreads) void rmsnorm_bwd_kernel(
             for (int e = 0; e < 8; ++e) o.v[e] += s.v[e];
         }
         store8_stream(dx + cur * D + d0, o);
+        if (dx_bf16 != nullptr) store8_stream(dx_bf16 + cur * D + d0, o);
     }
 
 #pragma unroll
@@ -93,16 +94,16 @@ __global__ __launch_bounds__(kNbThreads) void rmsnorm_bwd_kernel(
 
 template <int LANES, typename GT>
 static int launch_norm_bwd(const float *x, int64_t x_stride, const void *dy, int64_t dy_stride, const float *weight, float eps,
-                           const float *grad_sum, float *dx, float *partials, int blocks, float *dw, int64_t R,
-                           hipStream_t stream)
+                           const float *grad_sum, float *dx, uint16_t *dx_bf16, float *partials, int blocks, float *dw,
+                           int64_t R, hipStream_t stream)
 {
     const dim3 g((unsigned)blocks), t(kNbThreads);
     if (grad_sum)
         hipLaunchKernelGGL((rmsnorm_bwd_kernel<LANES, GT, true>), g, t, 0, stream, x, x_stride, (const GT *)dy, dy_stride, weight,
-                           eps, grad_sum, dx, partials, R);
+                           eps, grad_sum, dx, dx_bf16, partials, R);
     else
         hipLaunchKernelGGL((rmsnorm_bwd_kernel<LANES, GT, false>), g, t, 0, stream, x, x_stride, (const GT *)dy, dy_stride, weight,
-                           eps, grad_sum, dx, partials, R);
+                           eps, grad_sum, dx, dx_bf16, partials, R);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
     return launch_sum_slices(partials, dw, LANES * 8, blocks, 0, stream);
@@ -110,14 +111,14 @@ static int launch_norm_bwd(const float *x, int64_t x_stride, const void *dy, int
 
 template <typename GT>
 static int dispatch_norm_bwd(int D, const float *x, int64_t x_stride, const void *dy, int64_t dy_stride, const float *weight,
-                             float eps, const float *grad_sum, float *dx, float *partials, int blocks, float *dw, int64_t R,
-                             hipStream_t s)
+                             float eps, const float *grad_sum, float *dx, uint16_t *dx_bf16, float *partials, int blocks,
+                             float *dw, int64_t R, hipStream_t s)
 {
     switch (D) {
-        case 64: return launch_norm_bwd<8, GT>(x, x_stride, dy, dy_stride, weight, eps, grad_sum, dx, partials, blocks, dw, R, s);
-        case 128: return launch_norm_bwd<16, GT>(x, x_stride, dy, dy_stride, weight, eps, grad_sum, dx, partials, blocks, dw, R, s);
-        case 256: return launch_norm_bwd<32, GT>(x, x_stride, dy, dy_stride, weight, eps, grad_sum, dx, partials, blocks, dw, R, s);
-        case 512: return launch_norm_bwd<64, GT>(x, x_stride, dy, dy_stride, weight, eps, grad_sum, dx, partials, blocks, dw, R, s);
+        case 64: return launch_norm_bwd<8, GT>(x, x_stride, dy, dy_stride, weight, eps, grad_sum, dx, dx_bf16, partials, blocks, dw, R, s);
+        case 128: return launch_norm_bwd<16, GT>(x, x_stride, dy, dy_stride, weight, eps, grad_sum, dx, dx_bf16, partials, blocks, dw, R, s);
+        case 256: return launch_norm_bwd<32, GT>(x, x_stride, dy, dy_stride, weight, eps, grad_sum, dx, dx_bf16, partials, blocks, dw, R, s);
+        case 512: return launch_norm_bwd<64, GT>(x, x_stride, dy, dy_stride, weight, eps, grad_sum, dx, dx_bf16, partials, blocks, dw, R, s);
         default: return BNB_ERR_UNSUPPORTED;
     }
 }
@@ -133,8 +134,8 @@ extern "C" int bnb_rmsnorm_bwd_blocks(int64_t R, int D)
 }
 
 extern "C" int bnb_rmsnorm_bwd(const float *x, int64_t x_row_stride, const void *dy, int dy_dtype, int64_t dy_row_stride,
-                               const float *weight, float eps, const float *grad_sum, float *dx, float *partials,
-                               int blocks, float *dw, int64_t R, int D, void *stream)
+                               const float *weight, float eps, const float *grad_sum, float *dx, void *dx_bf16,
+                               float *partials, int blocks, float *dw, int64_t R, int D, void *stream)
 {
     using namespace bnb;
     if (R < 0 || D < 1 || x_row_stride < D || dy_row_stride < D) return BNB_ERR_BAD_SHAPE;
@@ -143,12 +144,15 @@ extern "C" int bnb_rmsnorm_bwd(const float *x, int64_t x_row_stride, const void 
     if (!weight || !dw || !partials || (R > 0 && (!x || !dy || !dx))) return BNB_ERR_NULL_POINTER;
     if (blocks < 1 || blocks > kNbMaxBlocks) return BNB_ERR_BAD_SHAPE;
     if (!aligned16(weight) || !aligned16(dw) || !aligned16(partials) ||
-        (R > 0 && (!aligned16(x) || !aligned16(dy) || !aligned16(dx) || (grad_sum && !aligned16(grad_sum)))) ||
+        (R > 0 && (!aligned16(x) || !aligned16(dy) || !aligned16(dx) || (grad_sum && !aligned16(grad_sum)) ||
+                   (dx_bf16 && !aligned16(dx_bf16)))) ||
         x_row_stride % 4 != 0 || dy_row_stride % 8 != 0)
         return BNB_ERR_MISALIGNED;
     hipStream_t s = (hipStream_t)stream;
     if (R == 0) return launch_sum_slices(partials, dw, D, 0, 0, s);  // no rows: the weight gradient is zero
     if (dy_dtype == BNB_BF16)
-        return dispatch_norm_bwd<uint16_t>(D, x, x_row_stride, dy, dy_row_stride, weight, eps, grad_sum, dx, partials, blocks, dw, R, s);
-    return dispatch_norm_bwd<float>(D, x, x_row_stride, dy, dy_row_stride, weight, eps, grad_sum, dx, partials, blocks, dw, R, s);
+        return dispatch_norm_bwd<uint16_t>(D, x, x_row_stride, dy, dy_row_stride, weight, eps, grad_sum, dx, (uint16_t *)dx_bf16,
+                                           partials, blocks, dw, R, s);
+    return dispatch_norm_bwd<float>(D, x, x_row_stride, dy, dy_row_stride, weight, eps, grad_sum, dx, (uint16_t *)dx_bf16, partials,
+                                    blocks, dw, R, s);
 }

@@ -1062,8 +1062,9 @@ _NORM_TRAIN_WIDTHS = (64, 128, 256, 512)
 
 
 def rmsnorm_bwd(x: torch.Tensor, dy: torch.Tensor, weight: torch.Tensor, *, eps: float | None = None,
-                grad_sum: torch.Tensor | None = None) -> tuple[torch.Tensor, torch.Tensor]:
-    """Backward of ``y = rmsnorm(x) * weight``: returns ``(dx, dw)``, both float32.
+                grad_sum: torch.Tensor | None = None, also_bf16: bool = False):
+    """Backward of ``y = rmsnorm(x) * weight``: returns ``(dx, dw)``, both float32, and with
+    ``also_bf16`` a bfloat16 copy of dx as a third value (written by the same pass).
 
     x (..., D) float32 with contiguous rows; dy same shape, float32 or bfloat16; ``grad_sum`` (same
     shape, float32) is added to dx: the gradient reaching x on the branch that bypasses the norm.
@@ -1085,6 +1086,7 @@ def rmsnorm_bwd(x: torch.Tensor, dy: torch.Tensor, weight: torch.Tensor, *, eps:
     R = x2.shape[0]
     dx = torch.empty((R, D), dtype=torch.float32, device=x.device)
     dw = torch.empty((D,), dtype=torch.float32, device=x.device)
+    dx_lp = torch.empty((R, D), dtype=torch.bfloat16, device=x.device) if also_bf16 else None
     lib = _native.load()
     blocks = int(lib.bnb_rmsnorm_bwd_blocks(R, D))
     partials = torch.empty((blocks, D), dtype=torch.float32, device=x.device)
@@ -1092,13 +1094,17 @@ def rmsnorm_bwd(x: torch.Tensor, dy: torch.Tensor, weight: torch.Tensor, *, eps:
         rc = lib.bnb_rmsnorm_bwd(x2.data_ptr(), x2.stride(0) if R else D, dy2.data_ptr(), _code(dy2, "dy"),
                                  dy2.stride(0) if R else D, weight.detach().contiguous().data_ptr(),
                                  _F32_EPS if eps is None else float(eps), None if gs is None else gs.data_ptr(),
-                                 dx.data_ptr(), partials.data_ptr(), blocks, dw.data_ptr(), R, D, _stream())
+                                 dx.data_ptr(), None if dx_lp is None else dx_lp.data_ptr(), partials.data_ptr(), blocks,
+                                 dw.data_ptr(), R, D, _stream())
     _native.check(rc, "bnb_rmsnorm_bwd")
+    if also_bf16:
+        return dx.reshape(x.shape), dw, dx_lp.reshape(x.shape)
     return dx.reshape(x.shape), dw
 
 
 class _RmsNormTrain(torch.autograd.Function):
-    """``rmsnorm(x) * weight`` rounded once to ``out_dtype``; forward and backward one kernel each."""
+    """``(x, rmsnorm(x) * weight)``: x is handed through so that the gradient arriving on the residual
+    branch reaches the backward kernel, which adds it in the same pass."""
 
     @staticmethod
     def forward(ctx, x, weight, eps, out_dtype):
@@ -1106,18 +1112,20 @@ class _RmsNormTrain(torch.autograd.Function):
             n = add_rmsnorm(x, weight, eps=eps, out_dtype=out_dtype)[1]
         ctx.save_for_backward(x, weight)
         ctx.eps = eps
-        return n
+        return x.view_as(x), n
 
     @staticmethod
-    def backward(ctx, dn):
+    def backward(ctx, ds, dn):
         x, weight = ctx.saved_tensors
-        dx, dw = rmsnorm_bwd(x, dn, weight, eps=ctx.eps)
+        if dn is None:
+            dn = torch.zeros_like(x)
+        dx, dw = rmsnorm_bwd(x, dn, weight, eps=ctx.eps, grad_sum=ds)
         return dx, dw, None, None
 
 
 class _AddRmsNormTrain(torch.autograd.Function):
     """``s = x + delta`` and ``rmsnorm(s) * weight``; the backward adds the gradient of ``s`` inside
-    the norm-backward kernel."""
+    the norm-backward kernel and writes a bfloat16 delta's gradient in the same pass."""
 
     @staticmethod
     def forward(ctx, x, delta, weight, eps, out_dtype):
@@ -1133,8 +1141,11 @@ class _AddRmsNormTrain(torch.autograd.Function):
         s, weight = ctx.saved_tensors
         if dn is None:
             dn = torch.zeros_like(s)
-        dx, dw = rmsnorm_bwd(s, dn, weight, eps=ctx.eps, grad_sum=ds)
-        ddelta = dx if ctx.delta_dtype == torch.float32 else dx.to(ctx.delta_dtype)
+        if ctx.delta_dtype == torch.bfloat16:
+            dx, dw, ddelta = rmsnorm_bwd(s, dn, weight, eps=ctx.eps, grad_sum=ds, also_bf16=True)
+        else:
+            dx, dw = rmsnorm_bwd(s, dn, weight, eps=ctx.eps, grad_sum=ds)
+            ddelta = dx
         return dx, ddelta, dw, None, None
 
 
@@ -1145,9 +1156,10 @@ def rmsnorm_train_supported(x: torch.Tensor) -> bool:
 
 def rmsnorm_train(x: torch.Tensor, weight: torch.Tensor, *, delta: torch.Tensor | None = None, eps: float | None = None,
                   out_dtype: torch.dtype = torch.float32):
-    """Differentiable ``add_rmsnorm``: returns ``normed`` without ``delta``, ``(x + delta, normed)`` with it.
-    ``normed`` is computed in float32 and rounded once to ``out_dtype`` (what ``nn.RMSNorm`` followed by
-    autocast's cast in front of the next Linear gives)."""
+    """Differentiable ``add_rmsnorm``: returns ``(s, normed)`` with ``s = x + delta``, or ``s`` = x itself
+    (an alias, to be used for the residual connection so that its gradient is added inside the backward
+    kernel) without ``delta``.  ``normed`` is computed in float32 and rounded once to ``out_dtype`` (what
+    ``nn.RMSNorm`` followed by autocast's cast in front of the next Linear gives)."""
     with torch.autocast("cuda", enabled=False):
         if delta is None:
             return _RmsNormTrain.apply(x, weight, eps, out_dtype)
@@ -1234,6 +1246,51 @@ class _GeluMulTrain(torch.autograd.Function):
         a, b = ctx.saved_tensors
         da, db = gelu_mul_bwd(a, b, dout)
         return da, db, None
+
+
+class _GeluMulPackedTrain(torch.autograd.Function):
+    """``gelu(gu[..., :H]) * gu[..., H:]`` on one (..., 2H) projection output; the backward writes both
+    halves of its gradient in place (no slices to stitch)."""
+
+    @staticmethod
+    def forward(ctx, gu, out_dtype):
+        H = gu.shape[-1] // 2
+        with torch.no_grad():
+            out = gelu_mul(gu[..., :H], gu[..., H:], out_dtype=out_dtype)
+        ctx.save_for_backward(gu)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        (gu,) = ctx.saved_tensors
+        H = gu.shape[-1] // 2
+        g2 = gu.reshape(-1, 2 * H)
+        if g2.numel() and g2.stride(-1) != 1:
+            g2 = g2.contiguous()
+        d2 = dout.reshape(-1, H).contiguous()
+        R = g2.shape[0]
+        dgu = torch.empty((R, 2 * H), dtype=gu.dtype, device=gu.device)
+        if R:
+            code = _code(g2, "gu")
+            with torch.cuda.device(gu.device):
+                rc = _native.load().bnb_gelu_mul_bwd(
+                    g2.data_ptr(), code, g2.stride(0), g2.data_ptr() + H * g2.element_size(), code, g2.stride(0),
+                    d2.data_ptr(), _code(d2, "dout"), dgu.data_ptr(), 2 * H, dgu.data_ptr() + H * dgu.element_size(), 2 * H,
+                    R, H, _stream(),
+                )
+            _native.check(rc, "bnb_gelu_mul_bwd")
+        return dgu.reshape(gu.shape), None
+
+
+def gelu_mul_packed_train(gu: torch.Tensor, *, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """Differentiable ``gelu(gate) * up`` for ``gu = [gate | up]`` (..., 2H), the output of one projection
+    over concatenated weights.  Needs H % 8 == 0 and a float32 or bfloat16 tensor on the GPU."""
+    H2 = gu.shape[-1]
+    if H2 % 16 or gu.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("gu must be float32 or bfloat16 with 2H channels, H a multiple of 8")
+    _need_device(gu, "gu")
+    with torch.autocast("cuda", enabled=False):
+        return _GeluMulPackedTrain.apply(gu, gu.dtype if out_dtype is None else out_dtype)
 
 
 def gelu_mul_train_supported(a: torch.Tensor, b: torch.Tensor) -> bool:

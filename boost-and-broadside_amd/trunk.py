@@ -84,16 +84,22 @@ def _cached_cast(owner: nn.Module, slot: str, tensors: tuple, dtype: torch.dtype
     return hit[1]
 
 
+def _grad_linear(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None) -> torch.Tensor:
+    """``F.linear`` in grad mode: under bf16 autocast with enough rows the weight gradient runs on the
+    row-sliced kernel (``ops.linear_train``), otherwise autocast's own differentiable casts apply."""
+    if (
+        _TRAIN_KERNELS and w.requires_grad and w.dtype == torch.float32 and _projection_dtype() == torch.bfloat16
+        and x.numel() >= _WGRAD_MIN_ROWS * x.shape[-1] and ops.linear_wgrad_supported(x, w)
+    ):
+        return ops.linear_train(x, w, b)
+    return F.linear(x, w, b)
+
+
 def _project(layer: nn.Linear, x: torch.Tensor) -> torch.Tensor:
     """``layer(x)`` for an activation that already has the projection dtype."""
     w, b = layer.weight, layer.bias
     if torch.is_grad_enabled():
-        if (
-            _TRAIN_KERNELS and w.requires_grad and w.dtype == torch.float32 and _projection_dtype() == torch.bfloat16
-            and x.numel() >= _WGRAD_MIN_ROWS * x.shape[-1] and ops.linear_wgrad_supported(x, w)
-        ):
-            return ops.linear_train(x, w, b)  # bf16 like autocast; weight gradient on the row-sliced kernel
-        return layer(x)  # training: autocast's own (differentiable) casts
+        return _grad_linear(x, w, b)
     if x.dtype == w.dtype:
         return F.linear(x, w, b)
     wc = _cached_cast(layer, "_bnb_w", (w,), x.dtype, lambda: w.detach().to(x.dtype))
@@ -112,11 +118,12 @@ def _gelu_gate(gate: torch.Tensor, value: torch.Tensor) -> torch.Tensor:
 
 
 def _train_norm(norm: nn.RMSNorm, x: torch.Tensor, delta: torch.Tensor | None = None):
-    """``norm(x)``, or with ``delta`` the pair ``(x + delta, norm(x + delta))``, differentiable.
+    """``(s, norm(s))`` with ``s = x + delta`` (``s`` = x without ``delta``), differentiable.  Use the
+    returned ``s`` for the residual connection.
 
     On the GPU with float32 rows of a covered width the norm's output is rounded once to the
-    projection dtype and forward and backward are one kernel each (``ops.rmsnorm_train``);
-    anything else is the module itself."""
+    projection dtype, forward and backward are one kernel each and the backward adds the residual
+    branch's gradient in the same pass (``ops.rmsnorm_train``); anything else is the module itself."""
     act = _projection_dtype()
     if (
         _TRAIN_KERNELS and torch.is_grad_enabled() and act in (torch.float32, torch.bfloat16) and ops.rmsnorm_train_supported(x)
@@ -124,9 +131,7 @@ def _train_norm(norm: nn.RMSNorm, x: torch.Tensor, delta: torch.Tensor | None = 
         and (delta is None or (delta.shape == x.shape and delta.dtype in (torch.float32, torch.bfloat16)))
     ):
         return ops.rmsnorm_train(x, norm.weight, delta=delta, eps=norm.eps, out_dtype=act)
-    if delta is None:
-        return norm(x)
-    s = x + delta
+    s = x if delta is None else x + delta
     return s, norm(s)
 
 
@@ -208,6 +213,14 @@ class GatedMLP(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         hidden = self.gate_proj.out_features
         if not x.is_cuda or hidden % 8 or x.dtype not in (torch.float32, torch.bfloat16) or torch.is_grad_enabled():
+            if (
+                _TRAIN_KERNELS and torch.is_grad_enabled() and x.is_cuda and hidden % 8 == 0 and self.gate_proj.bias is None
+                and self.up_proj.bias is None and _projection_dtype() == torch.bfloat16
+            ):
+                # one projection over [gate | up] (one pass over x forward, one GEMM for its gradient backward),
+                # the gate product on its column blocks
+                gu = _grad_linear(x, torch.cat([self.gate_proj.weight, self.up_proj.weight], dim=0), None)
+                return _project(self.down_proj, ops.gelu_mul_packed_train(gu, out_dtype=torch.bfloat16))
             return _project(self.down_proj, _gelu_gate(_project(self.gate_proj, x), _project(self.up_proj, x)))
         # one GEMM for [gate | up], one kernel for gelu(gate) * up, one GEMM down
         wg, wu = self.gate_proj.weight, self.up_proj.weight
@@ -241,7 +254,8 @@ class TransformerBlock(nn.Module):
     def forward(self, x, alive_mask=None, bullets=None, bullet_mask=None):
         act = _projection_dtype()
         if not _fused_ok(x, act):
-            x1, n2 = _train_norm(self.norm2, x, self._attn(_train_norm(self.norm1, x), alive_mask, bullets, bullet_mask))
+            x0, n1 = _train_norm(self.norm1, x)
+            x1, n2 = _train_norm(self.norm2, x0, self._attn(n1, alive_mask, bullets, bullet_mask))
             return x1 + self.ffn(n2)
         # norm + qkv (one kernel under bf16) -> attention kernel -> out_proj -> fused sublayer tail
         if act == torch.bfloat16 and self.d_model == ops.FFN_WIDTH and self.qkv.bias is None:
@@ -446,7 +460,7 @@ class GriffinTemporalBlock(nn.Module):
         # two passes over the sequence: conv taps (cut at episode ends), then the recurrence;
         # the only tensors in between are the conv output and the gate pre-activations
         act = _projection_dtype()
-        normed = self._norm_in(x_seq)
+        x_seq, normed = self._norm_in(x_seq)
         b1 = _project(self.linear1, normed)
         want_lp = act == torch.bfloat16
         res = ops.conv_seq(b1, conv_buf, self.conv.weight, self.conv.bias, done_mask, also_bf16=want_lp,
@@ -459,7 +473,7 @@ class GriffinTemporalBlock(nn.Module):
     def _sequence_autograd(self, x_seq, h0, conv_buf, done_mask, time_major):
         """Training path: torch ops (differentiable) around the recurrence, which runs on its
         forward and backward kernels."""
-        normed = _train_norm(self.norm1, x_seq)
+        x_seq, normed = _train_norm(self.norm1, x_seq)
         b1 = _project(self.linear1, normed)
         if (_TRAIN_KERNELS and ops.conv_seq_train_supported(b1) and conv_buf.dtype == torch.float32
                 and self.conv.weight.dtype == torch.float32):
@@ -477,10 +491,11 @@ class GriffinTemporalBlock(nn.Module):
         return self._finish(x_seq, normed, y), new_h, padded[:, T:]
 
     def _norm_in(self, x):
-        """norm1(x) in the projection dtype (one kernel with the cast when the fused path applies)."""
+        """``(x, norm1(x))`` with the norm in the projection dtype (one kernel with the cast when the fused
+        path applies); the returned x is the one to use for the residual connection."""
         act = _projection_dtype()
         if _fused_ok(x, act):
-            return ops.add_rmsnorm(x, self.norm1.weight, eps=self.norm1.eps, out_dtype=act)[1]
+            return x, ops.add_rmsnorm(x, self.norm1.weight, eps=self.norm1.eps, out_dtype=act)[1]
         return _train_norm(self.norm1, x)
 
     def _finish(self, x, normed, y, gate_in=None):
@@ -507,7 +522,7 @@ class GriffinTemporalBlock(nn.Module):
     def _step(self, x, h_in, conv_in, h_out, conv_out, reset, rows_per_env):
         """One timestep: x (R,D), h_in (R,D), conv_in (R,3,D) -> (out, new_h, new_conv_buf)."""
         act = _projection_dtype()
-        normed = self._norm_in(x)
+        x, normed = self._norm_in(x)
         b1 = _project(self.linear1, normed)
         want_lp = act == torch.bfloat16
         res = ops.conv_step(b1, conv_in, self.conv.weight, self.conv.bias, conv_out=conv_out, reset=reset,
@@ -573,7 +588,7 @@ class GriffinTemporalBlock(nn.Module):
             if fold:
                 y = both[..., 2 * D:]
         else:
-            normed = self._norm_in(x)
+            x, normed = self._norm_in(x)
             b1 = _project(self.linear1, normed)
         want_lp = act == torch.bfloat16
         fields_done = y is not None
@@ -610,7 +625,7 @@ class GriffinTemporalBlock(nn.Module):
     def forward_nonrecurrent(self, x, sub):
         """Same block with ``sub`` (a Linear) in place of conv + RG-LRU; no state."""
         act = _projection_dtype()
-        normed = self._norm_in(x)
+        x, normed = self._norm_in(x)
         b1 = _project(sub, _project(self.linear1, normed))
         gate_in = _project(self.linear2, normed)
         if _fused_ok(x, act) and gate_in.dtype == act:

@@ -296,6 +296,7 @@ int bnb_sdpa_masked_bwd(const void *qkv, int64_t qkv_row_stride, const uint8_t *
  *   dy       (R, D) bf16 or fp32 (dy_dtype), rows dy_row_stride apart: gradient of the norm's output
  *   grad_sum (R, D) fp32 contiguous or NULL
  *   dx       (R, D) fp32 contiguous (may alias grad_sum)
+ *   dx_bf16  optional (R, D) bf16 contiguous copy of dx (the gradient of a bf16 residual delta), or NULL
  *   partials (blocks, D) fp32 workspace of the caller; blocks from bnb_rmsnorm_bwd_blocks(R, D)
  *   dw       (D) fp32, overwritten; rows are added in a fixed order (no atomics)
  * Requirements: D in {64, 128, 256, 512}; 16-byte aligned pointers; x_row_stride % 4 == 0,
@@ -303,8 +304,8 @@ int bnb_sdpa_masked_bwd(const void *qkv, int64_t qkv_row_stride, const uint8_t *
  */
 int bnb_rmsnorm_bwd_blocks(int64_t R, int D);
 int bnb_rmsnorm_bwd(const float *x, int64_t x_row_stride, const void *dy, int dy_dtype, int64_t dy_row_stride,
-                    const float *weight, float eps, const float *grad_sum, float *dx, float *partials, int blocks,
-                    float *dw, int64_t R, int D, void *stream);
+                    const float *weight, float eps, const float *grad_sum, float *dx, void *dx_bf16,
+                    float *partials, int blocks, float *dw, int64_t R, int D, void *stream);
 
 /*
  * Pooling by multi-head attention over each team's alive ships, broadcast back to the ships:

@@ -1526,7 +1526,8 @@ def test_rmsnorm_bwd_adds_the_bypass_gradient_and_reads_strided_rows():
     dy = torch.randn(R, 2 * D, generator=g).bfloat16().to(DEV)[:, :D]
     gs = torch.randn(R, D, generator=g).to(DEV)
     w = (1.0 + 0.3 * torch.randn(D, generator=g)).to(DEV)
-    dx, dw = ops.rmsnorm_bwd(x, dy, w, eps=1e-5, grad_sum=gs)
+    dx, dw, dx_lp = ops.rmsnorm_bwd(x, dy, w, eps=1e-5, grad_sum=gs, also_bf16=True)
+    assert torch.equal(dx_lp, dx.bfloat16())
     ref_dx, ref_dw = _norm_truth(x.cpu(), dy.cpu(), w.cpu(), 1e-5, gs.cpu())
     assert max_rel(dx.cpu().double(), ref_dx) <= F32_TOL and max_rel(dw.cpu().double(), ref_dw) <= F32_TOL
     lead_dx, lead_dw = ops.rmsnorm_bwd(x.reshape(3001, 1, D), dy.reshape(3001, 1, D), w, eps=1e-5, grad_sum=gs.reshape(3001, 1, D))
@@ -1548,13 +1549,10 @@ def test_rmsnorm_train_gradients_match_autograd_of_torch_rms_norm(out_dtype, wit
     w = w0.to(DEV).requires_grad_()
     d = d0.to(DEV).requires_grad_() if with_delta else None
     with torch.autocast("cuda", dtype=torch.bfloat16):
-        res = ops.rmsnorm_train(x, w, delta=d, out_dtype=out_dtype)
-    if with_delta:
-        s, n = res
-        loss = (n.float() * up_n.to(DEV).float()).sum() + (s * up_s.to(DEV)).sum()
-    else:
-        n = res
-        loss = (n.float() * up_n.to(DEV).float()).sum()
+        s, n = ops.rmsnorm_train(x, w, delta=d, out_dtype=out_dtype)
+    if not with_delta:
+        assert torch.equal(s, x)  # x handed through for the residual connection
+    loss = (n.float() * up_n.to(DEV).float()).sum() + (s * up_s.to(DEV)).sum()
     assert n.dtype == out_dtype
     loss.backward()
 
@@ -1563,7 +1561,7 @@ def test_rmsnorm_train_gradients_match_autograd_of_torch_rms_norm(out_dtype, wit
     dr = d0.double().requires_grad_() if with_delta else None
     sr = xr + dr if with_delta else xr
     nr = torch.nn.functional.rms_norm(sr, (D,), wr, float(torch.finfo(torch.float32).eps))
-    lr = (nr * up_n.double()).sum() + ((sr * up_s.double()).sum() if with_delta else 0.0)
+    lr = (nr * up_n.double()).sum() + (sr * up_s.double()).sum()
     lr.backward()
     tol = F32_TOL if out_dtype == torch.float32 else BF16_TOL
     assert max_rel(n.detach().float().cpu().double(), nr.detach()) <= tol
@@ -1741,3 +1739,19 @@ def test_sdpa_train_is_differentiable_and_reads_strided_rows():
     assert max_rel(wide.grad[..., 64:].float().cpu().double(), ref_grad) <= BF16_TOL
     assert not ops.sdpa_train_supported(torch.zeros(2, 40, 384, device=DEV), 4)
     assert not ops.sdpa_train_supported(torch.zeros(2, 12, 192, device=DEV), 4)
+
+
+def test_gelu_mul_packed_train_equals_the_two_operand_form():
+    R, H = 700, 512
+    g = torch.Generator().manual_seed(13)
+    gu0 = torch.randn(R, 2 * H, generator=g).bfloat16().to(DEV)
+    up = torch.randn(R, H, generator=g).bfloat16().to(DEV)
+    gu = gu0.clone().requires_grad_()
+    out = ops.gelu_mul_packed_train(gu.view(7, 100, 2 * H), out_dtype=torch.bfloat16)
+    out.backward(up.view(7, 100, H))
+    a = gu0[:, :H].clone().requires_grad_()
+    b = gu0[:, H:].clone().requires_grad_()
+    ref = ops.gelu_mul_train(a, b, out_dtype=torch.bfloat16)
+    ref.backward(up)
+    assert torch.equal(out.reshape(R, H), ref)
+    assert torch.equal(gu.grad[:, :H], a.grad) and torch.equal(gu.grad[:, H:], b.grad)
