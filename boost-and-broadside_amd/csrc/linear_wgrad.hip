@@ -7,7 +7,8 @@
 // GEMM picks a tiling for large M x N and runs these at 6-20x the time the operands need to
 // cross HBM once (393,216 rows, 128 x 128: 815 us against a 40 us floor).  Here the rows are
 // split into slices, one work-group per (128 x 128 output tile, slice), so the chip is filled
-// by the long dimension:
+// by the long dimension (the tiles of one slice placed on one XCD, so the operand rows they share
+// cross HBM once):
 //   * a work-group walks its slice in chunks of 64 rows.  A thread fetches an 8 x 8 block of one
 //     operand (eight coalesced 16-byte loads, the next chunk prefetched into registers),
 //     transposes it in registers (32 byte-permutes) and stores it column-major in LDS, because
@@ -34,7 +35,7 @@ __device__ __forceinline__ int wg_slot(int c, int rb) { return c * kWgRows + 8 *
 
 __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
     const uint16_t *__restrict__ dy, int64_t dy_stride, const uint16_t *__restrict__ x, int64_t x_stride,
-    float *__restrict__ partials, int64_t R, int N, int K, int64_t rows_per_slice)
+    float *__restrict__ partials, int64_t R, int N, int K, int64_t rows_per_slice, int slices)
 {
     __shared__ __align__(16) uint16_t s_t[2][kWgTile * kWgRows];  // [operand: dy, x][column][row], swizzled
 
@@ -43,8 +44,23 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int m = lane & 31;
     const int half = lane >> 5;
-    const int n0 = blockIdx.x * kWgTile, k0 = blockIdx.y * kWgTile;
-    const int64_t slice = blockIdx.z;
+    // work-group -> (output tile, slice): the tiles of one slice share the second operand's rows, so they
+    // are given ids that differ by multiples of 8 and close together: work-groups are dealt to the 8 XCDs in
+    // turn, which puts them on one XCD (one L2) at about the same time
+    const int tiles_n = N / kWgTile, tiles = tiles_n * (K / kWgTile);
+    const int full = slices / 8 * 8 * tiles;
+    int tile, slice_i;
+    if ((int)blockIdx.x < full) {
+        const int group = blockIdx.x / (8 * tiles), within = blockIdx.x - group * 8 * tiles;
+        tile = within >> 3;
+        slice_i = group * 8 + (within & 7);
+    } else {
+        const int r = blockIdx.x - full;
+        tile = r % tiles;
+        slice_i = slices / 8 * 8 + r / tiles;
+    }
+    const int n0 = (tile % tiles_n) * kWgTile, k0 = (tile / tiles_n) * kWgTile;
+    const int64_t slice = slice_i;
     const int64_t r_begin = slice * rows_per_slice;
     const int64_t r_end = r_begin + rows_per_slice < R ? r_begin + rows_per_slice : R;
 
@@ -56,8 +72,8 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
     const int64_t src_stride = operand ? x_stride : dy_stride;
     uint16_t *dst = s_t[operand];
 
-    u32x4 stage[8];
-    auto fetch = [&](int64_t row0) {
+    u32x4 stage_a[8];  // the next chunk's operand rows, in flight while this one is multiplied
+    auto fetch = [&](u32x4(&stage)[8], int64_t row0) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int64_t r = row0 + 8 * rg + j;
@@ -65,7 +81,7 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
             stage[j] = r < r_end ? v : u32x4{0u, 0u, 0u, 0u};  // rows past the slice add nothing
         }
     };
-    auto stash = [&]() {
+    auto stash = [&](const u32x4(&stage)[8]) {
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
             // column c of the block: rows 0..7 as four words of two halfs
@@ -89,11 +105,10 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
             for (int v = 0; v < 16; ++v) acc[i][t][v] = 0.0f;
 
     const int nw = 64 * (wave >> 1), kw = 64 * (wave & 1);  // this wave's quarter of the tile
-    if (r_begin < r_end) fetch(r_begin);
-    for (int64_t row0 = r_begin; row0 < r_end; row0 += kWgRows) {
+    auto chunk = [&](u32x4(&stage)[8], int64_t row0) {
         __syncthreads();  // everyone is done reading the previous chunk
-        stash();
-        if (row0 + kWgRows < r_end) fetch(row0 + kWgRows);
+        stash(stage);
+        if (row0 + kWgRows < r_end) fetch(stage, row0 + kWgRows);
         __syncthreads();
 #pragma unroll
         for (int ks = 0; ks < kWgRows / 16; ++ks) {
@@ -105,7 +120,9 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
             acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc[1][0], 0, 0, 0);
             acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc[1][1], 0, 0, 0);
         }
-    }
+    };
+    if (r_begin < r_end) fetch(stage_a, r_begin);
+    for (int64_t row0 = r_begin; row0 < r_end; row0 += kWgRows) chunk(stage_a, row0);
     // partial tile of this slice: lane holds column k = kw + 32t + m, rows n = nw + 32i + 8(v/4) + 4*half + v%4
     float *pt = partials + (slice * N + n0 + nw + 4 * half) * K + k0 + kw + m;
 #pragma unroll
@@ -162,10 +179,10 @@ int launch_sum_slices(const float *partials, float *out, int64_t elems, int slic
 
 extern "C" int bnb_linear_wgrad_slices(int64_t R, int N, int K)
 {
-    // slices such that tiles x slices is about two work-groups per CU (all resident at once), every slice at least 256 rows
+    // slices such that tiles x slices is about three work-groups per CU (all resident at once: 148 registers, 32 KB of LDS each), every slice at least 256 rows
     if (R <= 0 || N <= 0 || K <= 0) return 1;
     const int64_t tiles = (int64_t)(N / bnb::kWgTile) * (K / bnb::kWgTile);
-    int64_t s = 512 / (tiles > 0 ? tiles : 1);
+    int64_t s = 768 / (tiles > 0 ? tiles : 1);
     const int64_t by_rows = (R + 255) / 256;
     if (s > by_rows) s = by_rows;
     if (s < 1) s = 1;
@@ -187,9 +204,10 @@ extern "C" int bnb_linear_wgrad_fwd(const void *dy, int64_t dy_row_stride, const
         return BNB_ERR_MISALIGNED;
     hipStream_t s = (hipStream_t)stream;
     const int64_t rows_per_slice = ((R + slices - 1) / slices + kWgRows - 1) / kWgRows * kWgRows;
-    hipLaunchKernelGGL(linear_wgrad_kernel, dim3(N / kWgTile, K / kWgTile, slices), dim3(kWgThreads), 0, s,
-                       (const uint16_t *)dy, dy_row_stride, (const uint16_t *)x, x_row_stride, partials, R, N, K,
-                       rows_per_slice > 0 ? rows_per_slice : kWgRows);
+    const int64_t groups = (int64_t)(N / kWgTile) * (K / kWgTile) * slices;
+    if (groups > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(linear_wgrad_kernel, dim3((unsigned)groups), dim3(kWgThreads), 0, s, (const uint16_t *)dy, dy_row_stride,
+                       (const uint16_t *)x, x_row_stride, partials, R, N, K, rows_per_slice > 0 ? rows_per_slice : kWgRows, slices);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
     return launch_sum_slices(partials, dw, (int64_t)N * K, slices, accumulate, s);
