@@ -25,6 +25,7 @@ namespace bnb {
 constexpr int kSbDh = 32;          // head size
 constexpr int kSbHeadPitch = 36;   // floats between heads of one LDS row
 constexpr int kSbMaxTokens = 32;
+constexpr int kSbMfmaFrom = 11;  // AUTO: the matrix-core kernel above this many tokens (bf16); below, the vector kernel is as fast
 constexpr int kSbLdsBudget = 78 * 1024;  // two work-groups per CU
 
 struct SbShape {
@@ -228,14 +229,271 @@ static int launch_sdpa_bwd(const void *qkv, int64_t qkv_row_stride, const uint8_
     return (int)hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------
+// bf16 on the matrix cores, up to 160 tokens
+// ------------------------------------------------------------------------------------
+//
+// One work-group per (environment, head), one wave per block of 32 tokens.  Nothing is reduced
+// across waves: the products are formed twice, once per orientation.
+//   pass 0/1, wave = query block: S^T = K Q^T per key block (rows = keys, lane = query), row
+//     maximum and sum as in the forward kernel, L = log2-sum-exp and delta = rowsum(dO * O) per
+//     query (kept in LDS for pass 2); then P^T = exp2(S^T c - L), dP^T = V dO^T,
+//     dS^T = P^T (dP^T - delta) / sqrt(dh), and dQ^T += K^T dS^T with dS^T going from the
+//     accumulator registers straight into the B operand (the key order of the A operand, read
+//     from a transposed copy of K in LDS, follows the accumulator's row order);
+//   pass 2, wave = key block: S = Q K^T per query block (rows = queries, lane = key), P and dS from
+//     the per-query L and delta, dK^T += Q^T dS and dV^T += dO^T P the same way (transposed
+//     copies of Q and dO in LDS).
+// K, V (pass 1) and Q, dO (pass 2) share the same LDS.  Dead and padding keys enter as -inf in the
+// accumulator (P = 0 exactly); an environment without a live key uses zero scores over all its keys.
+// P and dS are rounded to bf16 for the second product of each pair, as the operands of the forward
+// kernel's second product are.
+
+constexpr int kMbPitch = kSbDh + 8;  // halfs per token row in LDS (80 bytes: 16-byte aligned, bank-spread)
+
+template <int NB>
+__global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
+    const uint16_t *__restrict__ qkv, int64_t qkv_row_stride, const uint8_t *__restrict__ alive,
+    const uint16_t *__restrict__ out, const uint16_t *__restrict__ dout, uint16_t *__restrict__ dqkv, int B, int NM, int H,
+    float scale)
+{
+    constexpr int CAP = NB * 32;
+    constexpr int TP = CAP + 4;  // halfs per row of a transposed copy
+    constexpr int NT = kWave * NB;
+    __shared__ __align__(16) uint16_t s_rows[2][CAP * kMbPitch];  // [K | V], later [Q | dO]: token-major
+    __shared__ __align__(16) uint16_t s_tr[2][kSbDh * TP];        // K^T, later [Q^T | dO^T]: channel-major
+    __shared__ __align__(16) float s_lse[CAP], s_delta[CAP];
+    __shared__ __align__(16) float s_bias[CAP];  // 0 for a key that takes part, -inf for a dead or padding key
+
+    const int chunk = gridDim.x >> 3;
+    const int logical = (blockIdx.x & 7) * chunk + (blockIdx.x >> 3);  // the heads of an environment on one XCD
+    if (logical >= B * H) return;
+    const int env = logical / H, head = logical - env * H;
+    const int D = H * kSbDh;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m = lane & 31, half = lane >> 5;
+    const float c = scale * 1.4426950408889634f;
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+
+    // token-major and channel-major copies of two (NM, 32) operands; rows past NM are zero.  The loads of
+    // both phases are issued at the start of the kernel, so their latency is paid once.
+    struct Staged {
+        u32x4 a[2], b[2];
+    };
+    auto stage_load = [&](const uint16_t *a, int64_t a_stride, const uint16_t *b, int64_t b_stride) -> Staged {
+        Staged r;
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int item = tid + it * NT;
+            const int tok = item >> 2, c8 = (item & 3) * 8;
+            const int safe = tok < NM ? tok : NM - 1;
+            const u32x4 aw = *reinterpret_cast<const u32x4 *>(a + ((int64_t)env * NM + safe) * a_stride + head * kSbDh + c8);
+            const u32x4 bw = *reinterpret_cast<const u32x4 *>(b + ((int64_t)env * NM + safe) * b_stride + head * kSbDh + c8);
+            r.a[it] = tok < NM ? aw : zero4;
+            r.b[it] = tok < NM ? bw : zero4;
+        }
+        return r;
+    };
+    auto stage_store = [&](const Staged &r, bool transpose_a, bool transpose_b) {
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int item = tid + it * NT;
+            const int tok = item >> 2, c8 = (item & 3) * 8;
+            *reinterpret_cast<u32x4 *>(s_rows[0] + tok * kMbPitch + c8) = r.a[it];
+            *reinterpret_cast<u32x4 *>(s_rows[1] + tok * kMbPitch + c8) = r.b[it];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t wa = r.a[it][e >> 1], wb = r.b[it][e >> 1];
+                if (transpose_a) s_tr[0][(c8 + e) * TP + tok] = (uint16_t)((e & 1) ? wa >> 16 : wa & 0xffffu);
+                if (transpose_b) s_tr[1][(c8 + e) * TP + tok] = (uint16_t)((e & 1) ? wb >> 16 : wb & 0xffffu);
+            }
+        }
+    };
+    // an operand of the first product of a pair: row (or column) tok, channels 8*half.. and 16 + 8*half..
+    auto row_operand = [&](const uint16_t *rows, int tok, bf16x8 &lo, bf16x8 &hi) {
+        const uint16_t *p = rows + tok * kMbPitch + half * 8;
+        lo = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(p));
+        hi = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(p + 16));
+    };
+    // the A operand of the second product: channel m, tokens in the order the accumulator rows 8t.. hold them
+    auto tr_operand = [&](const uint16_t *tr, int blk, int t) -> bf16x8 {
+        const uint16_t *p = tr + m * TP + blk * 32 + 16 * t + 4 * half;
+        const u32x2 lo = *reinterpret_cast<const u32x2 *>(p);
+        const u32x2 hi = *reinterpret_cast<const u32x2 *>(p + 8);
+        return __builtin_bit_cast(bf16x8, u32x4{lo.x, lo.y, hi.x, hi.y});
+    };
+    auto pack8 = [&](const float (&x)[16], int t) -> bf16x8 {
+        bf16x8 r;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r[e] = (__bf16)x[8 * t + e];
+        return r;
+    };
+    // a (32 channels x 32 tokens) accumulator to the rows of dqkv: lane = token, rows = channels 8i + 4*half + j
+    auto store_grad = [&](const f32x16 &acc, int tok, int third) {
+        if (tok >= NM) return;
+        uint16_t *dst = dqkv + ((int64_t)env * NM + tok) * 3 * D + third * D + head * kSbDh + 4 * half;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            *reinterpret_cast<u32x2 *>(dst + 8 * i) = u32x2{pack_bf16x2(acc[4 * i], acc[4 * i + 1]), pack_bf16x2(acc[4 * i + 2], acc[4 * i + 3])};
+    };
+
+    // ---- every global load of the kernel ----
+    const uint16_t *qp = qkv, *kp = qkv + D, *vp = qkv + 2 * D;
+    const int own = wave * 32 + m;
+    const int own_safe = own < NM ? own : NM - 1;
+    const int64_t own_row = (int64_t)env * NM + own_safe;
+    const int64_t own_q = own_row * qkv_row_stride + head * kSbDh + half * 8, own_o = own_row * D + head * kSbDh + half * 8;
+    bool any_live = false, my_live = false;
+    if (tid < CAP) {  // CAP <= NT
+        my_live = tid < NM && (alive == nullptr || alive[(int64_t)env * NM + tid] != 0);
+        any_live = my_live;
+    }
+    const Staged kv_in = stage_load(kp, qkv_row_stride, vp, qkv_row_stride);
+    u32x4 w0 = *reinterpret_cast<const u32x4 *>(qp + own_q), w1 = *reinterpret_cast<const u32x4 *>(qp + own_q + 16);
+    u32x4 g0 = *reinterpret_cast<const u32x4 *>(dout + own_o), g1 = *reinterpret_cast<const u32x4 *>(dout + own_o + 16);
+    const Row8 o0 = load8(out + own_o), o1 = load8(out + own_o + 16);
+    u32x4 kw0 = *reinterpret_cast<const u32x4 *>(kp + own_q), kw1 = *reinterpret_cast<const u32x4 *>(kp + own_q + 16);
+    u32x4 vw0 = *reinterpret_cast<const u32x4 *>(vp + own_q), vw1 = *reinterpret_cast<const u32x4 *>(vp + own_q + 16);
+    const Staged qd_in = stage_load(qp, qkv_row_stride, dout, D);
+
+    // ---- live keys ----
+    const bool uniform = __syncthreads_or(any_live ? 1 : 0) == 0;
+    if (tid < CAP) s_bias[tid] = (uniform ? tid < NM : my_live) ? 0.0f : -INFINITY;
+    stage_store(kv_in, true, false);
+    __syncthreads();
+
+    // ---- pass 0 and 1: this wave's queries ----
+    float delta;
+    {
+        const Row8 a0 = Row8{{__uint_as_float(g0.x << 16), __uint_as_float(g0.x & 0xffff0000u), __uint_as_float(g0.y << 16),
+                              __uint_as_float(g0.y & 0xffff0000u), __uint_as_float(g0.z << 16), __uint_as_float(g0.z & 0xffff0000u),
+                              __uint_as_float(g0.w << 16), __uint_as_float(g0.w & 0xffff0000u)}};
+        const Row8 a1 = Row8{{__uint_as_float(g1.x << 16), __uint_as_float(g1.x & 0xffff0000u), __uint_as_float(g1.y << 16),
+                              __uint_as_float(g1.y & 0xffff0000u), __uint_as_float(g1.z << 16), __uint_as_float(g1.z & 0xffff0000u),
+                              __uint_as_float(g1.w << 16), __uint_as_float(g1.w & 0xffff0000u)}};
+        float d = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) d = fmaf(a0.v[e], o0.v[e], fmaf(a1.v[e], o1.v[e], d));
+        delta = d + __shfl_xor(d, 32);
+    }
+    if (own >= NM) w0 = w1 = g0 = g1 = zero4, delta = 0.0f;  // padding queries: nothing flows through them
+    const bf16x8 qs0 = __builtin_bit_cast(bf16x8, uniform ? zero4 : w0), qs1 = __builtin_bit_cast(bf16x8, uniform ? zero4 : w1);
+    const bf16x8 gb0 = __builtin_bit_cast(bf16x8, g0), gb1 = __builtin_bit_cast(bf16x8, g1);
+
+    auto scores_t = [&](int kb) -> f32x16 {
+        f32x16 z;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const f32x4 b4 = *reinterpret_cast<const f32x4 *>(s_bias + kb * 32 + 8 * i + 4 * half);
+            z[4 * i] = b4.x, z[4 * i + 1] = b4.y, z[4 * i + 2] = b4.z, z[4 * i + 3] = b4.w;
+        }
+        bf16x8 k0, k1;
+        row_operand(s_rows[0], kb * 32 + m, k0, k1);
+        z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k0, qs0, z, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(k1, qs1, z, 0, 0, 0);
+    };
+    float mx = -INFINITY;
+    for (int kb = 0; kb < NB; ++kb) {
+        const f32x16 z = scores_t(kb);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float mc = mx * c;
+    float sum = 0.0f;
+    for (int kb = 0; kb < NB; ++kb) {
+        const f32x16 z = scores_t(kb);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sum += __builtin_amdgcn_exp2f(fmaf(z[v], c, -mc));
+    }
+    sum += __shfl_xor(sum, 32);
+    const float lse = mc + __builtin_amdgcn_logf(sum);  // log2 of the sum of exp2(z c)
+    if (half == 0) s_lse[own] = lse, s_delta[own] = delta;
+
+    f32x16 dq = {0.0f};
+    for (int kb = 0; kb < NB; ++kb) {
+        const f32x16 z = scores_t(kb);
+        bf16x8 v0, v1;
+        row_operand(s_rows[1], kb * 32 + m, v0, v1);
+        f32x16 dp = {0.0f};
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, gb0, dp, 0, 0, 0);
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, gb1, dp, 0, 0, 0);
+        float ds[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) ds[v] = __builtin_amdgcn_exp2f(fmaf(z[v], c, -lse)) * (dp[v] - delta) * scale;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_operand(s_tr[0], kb, t), pack8(ds, t), dq, 0, 0, 0);
+    }
+    store_grad(dq, own, 0);
+    __syncthreads();  // K, V and K^T are no longer needed; L and delta of every query are in LDS
+
+    // ---- pass 2: this wave's keys ----
+    stage_store(qd_in, true, true);
+    const float col_bias = s_bias[own];
+    if (own >= NM) kw0 = kw1 = vw0 = vw1 = zero4;
+    const bf16x8 ks0 = __builtin_bit_cast(bf16x8, uniform ? zero4 : kw0), ks1 = __builtin_bit_cast(bf16x8, uniform ? zero4 : kw1);
+    const bf16x8 vb0 = __builtin_bit_cast(bf16x8, vw0), vb1 = __builtin_bit_cast(bf16x8, vw1);
+    __syncthreads();
+
+    f32x16 dk = {0.0f}, dv = {0.0f};
+    for (int qb = 0; qb < NB; ++qb) {
+        f32x16 z;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) z[v] = col_bias;
+        bf16x8 a0, a1;
+        row_operand(s_rows[0], qb * 32 + m, a0, a1);
+        z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, ks0, z, 0, 0, 0);
+        z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, ks1, z, 0, 0, 0);
+        row_operand(s_rows[1], qb * 32 + m, a0, a1);
+        f32x16 dp = {0.0f};
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, vb0, dp, 0, 0, 0);
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, vb1, dp, 0, 0, 0);
+        float p[16], ds[16];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const f32x4 l4 = *reinterpret_cast<const f32x4 *>(s_lse + qb * 32 + 8 * i + 4 * half);
+            const f32x4 d4 = *reinterpret_cast<const f32x4 *>(s_delta + qb * 32 + 8 * i + 4 * half);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int v = 4 * i + j;
+                p[v] = __builtin_amdgcn_exp2f(fmaf(z[v], c, -l4[j]));
+                ds[v] = p[v] * (dp[v] - d4[j]) * scale;
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            dk = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_operand(s_tr[0], qb, t), pack8(ds, t), dk, 0, 0, 0);
+            dv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_operand(s_tr[1], qb, t), pack8(p, t), dv, 0, 0, 0);
+        }
+    }
+    store_grad(dk, own, 1);
+    store_grad(dv, own, 2);
+}
+
+template <int NB>
+static int launch_sdpa_bwd_mfma(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, const void *out, const void *dout,
+                                void *dqkv, int64_t B, int NM, int H, hipStream_t stream)
+{
+    const int64_t groups = (B * H + 7) / 8 * 8;  // a multiple of 8: the XCD mapping deals whole rounds
+    if (groups > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<NB>), dim3((unsigned)groups), dim3(kWave * NB), 0, stream, (const uint16_t *)qkv,
+                       qkv_row_stride, alive, (const uint16_t *)out, (const uint16_t *)dout, (uint16_t *)dqkv, (int)B, NM, H,
+                       1.0f / sqrtf((float)kSbDh));
+    return (int)hipGetLastError();
+}
+
 }  // namespace bnb
 
-extern "C" int bnb_sdpa_masked_bwd(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, const void *out,
-                                   const void *dout, void *dqkv, int64_t B, int NM, int H, int dh, int dtype, void *stream)
+extern "C" int bnb_sdpa_masked_bwd_path(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, const void *out,
+                                        const void *dout, void *dqkv, int64_t B, int NM, int H, int dh, int dtype, int path,
+                                        void *stream)
 {
     using namespace bnb;
     if (B < 0 || NM < 1 || H < 1 || dh < 1) return BNB_ERR_BAD_SHAPE;
-    if (dh != kSbDh || NM > kSbMaxTokens || H > 8 || NM * H > 256) return BNB_ERR_UNSUPPORTED;
+    const bool small = NM <= kSbMaxTokens && H <= 8 && NM * H <= 256;
+    const bool mfma = dtype == BNB_BF16 && NM <= 160 && B <= 0x7fffffffLL / (H > 0 ? H : 1);
+    if (dh != kSbDh || (!small && !mfma)) return BNB_ERR_UNSUPPORTED;
     if (dtype != BNB_F32 && dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
     if (qkv_row_stride < 3 * (int64_t)H * dh) return BNB_ERR_BAD_SHAPE;
     if (B == 0) return 0;
@@ -244,6 +502,24 @@ extern "C" int bnb_sdpa_masked_bwd(const void *qkv, int64_t qkv_row_stride, cons
     if (!aligned16(qkv) || !aligned16(out) || !aligned16(dout) || !aligned16(dqkv) || (qkv_row_stride * esz) % 16 != 0)
         return BNB_ERR_MISALIGNED;
     hipStream_t s = (hipStream_t)stream;
+    if (path != BNB_SDPA_PATH_AUTO && path != BNB_SDPA_PATH_VALU && path != BNB_SDPA_PATH_MFMA) return BNB_ERR_BAD_SHAPE;
+    if (path == BNB_SDPA_PATH_MFMA && !mfma) return BNB_ERR_UNSUPPORTED;
+    if (mfma && (path == BNB_SDPA_PATH_MFMA || (path == BNB_SDPA_PATH_AUTO && NM > kSbMfmaFrom))) {
+        switch ((NM + 31) / 32) {
+            case 1: return launch_sdpa_bwd_mfma<1>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
+            case 2: return launch_sdpa_bwd_mfma<2>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
+            case 3: return launch_sdpa_bwd_mfma<3>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
+            case 4: return launch_sdpa_bwd_mfma<4>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
+            default: return launch_sdpa_bwd_mfma<5>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
+        }
+    }
+    if (!small) return BNB_ERR_UNSUPPORTED;
     if (dtype == BNB_BF16) return launch_sdpa_bwd<uint16_t>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
     return launch_sdpa_bwd<float>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
+}
+
+extern "C" int bnb_sdpa_masked_bwd(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, const void *out,
+                                   const void *dout, void *dqkv, int64_t B, int NM, int H, int dh, int dtype, void *stream)
+{
+    return bnb_sdpa_masked_bwd_path(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, dh, dtype, BNB_SDPA_PATH_AUTO, stream);
 }

@@ -104,16 +104,21 @@ def sdpa_masked(
 
 
 def sdpa_train_supported(qkv: torch.Tensor, n_heads: int) -> bool:
-    """Whether ``sdpa_train`` covers this input: head size 32, at most 32 tokens and 8 heads, on the GPU."""
+    """Whether ``sdpa_train`` covers this input on the GPU: head size 32 and either at most 32 tokens and
+    8 heads (float32 or bfloat16) or bfloat16 with at most 160 tokens."""
     if not (qkv.is_cuda and qkv.dim() == 3 and qkv.dtype in (torch.float32, torch.bfloat16) and qkv.shape[-1] % 3 == 0):
         return False
     D = qkv.shape[-1] // 3
-    return D % n_heads == 0 and D // n_heads == 32 and 1 <= qkv.shape[1] <= 32 and n_heads <= 8
+    if D % n_heads or D // n_heads != 32 or qkv.shape[1] < 1:
+        return False
+    NM = qkv.shape[1]
+    return (NM <= 32 and n_heads <= 8) or (qkv.dtype == torch.bfloat16 and NM <= 160)
 
 
 def sdpa_masked_bwd(qkv: torch.Tensor, alive: torch.Tensor | None, n_heads: int, out: torch.Tensor,
-                    dout: torch.Tensor) -> torch.Tensor:
-    """Gradient of ``sdpa_masked`` with respect to ``qkv`` from the forward's result and its gradient."""
+                    dout: torch.Tensor, *, path: str = "auto") -> torch.Tensor:
+    """Gradient of ``sdpa_masked`` with respect to ``qkv`` from the forward's result and its gradient.
+    ``path``: "auto" | "valu" | "mfma" (kernel selection, for tests and benchmarks)."""
     B, NM, D3 = qkv.shape
     D = D3 // 3
     if out.shape != (B, NM, D) or dout.shape != (B, NM, D) or out.dtype != qkv.dtype:
@@ -133,8 +138,9 @@ def sdpa_masked_bwd(qkv: torch.Tensor, alive: torch.Tensor | None, n_heads: int,
     dqkv = torch.empty((B, NM, D3), dtype=qkv.dtype, device=qkv.device)
     if B:
         with torch.cuda.device(qkv.device):
-            rc = _native.load().bnb_sdpa_masked_bwd(qkv.data_ptr(), qkv.stride(1), mask_ptr, out.data_ptr(), dout.data_ptr(),
-                                                    dqkv.data_ptr(), B, NM, n_heads, D // n_heads, _code(qkv, "qkv"), _stream())
+            rc = _native.load().bnb_sdpa_masked_bwd_path(qkv.data_ptr(), qkv.stride(1), mask_ptr, out.data_ptr(), dout.data_ptr(),
+                                                         dqkv.data_ptr(), B, NM, n_heads, D // n_heads, _code(qkv, "qkv"),
+                                                         _PATH_CODE[path], _stream())
         _native.check(rc, "bnb_sdpa_masked_bwd")
     return dqkv
 

@@ -276,11 +276,17 @@ int bnb_linear_wgrad_fwd(const void *dy, int64_t dy_row_stride, const void *x, i
  *   dout   (B, NM, H*dh) contiguous: its gradient
  *   dqkv   (B, NM, 3*H*dh) contiguous: gradient of qkv
  * all in `dtype` (BNB_F32 or BNB_BF16), arithmetic in fp32, every sum in a fixed order.
- * Requirements: dh == 32, NM <= 32, H <= 8; 16-byte aligned rows.  Other shapes return
+ * Requirements: dh == 32 and either NM <= 32 with H <= 8 (vector-ALU kernel, fp32 or bf16) or bf16
+ * with NM <= 160 (matrix-core kernel); 16-byte aligned rows.  Other shapes return
  * BNB_ERR_UNSUPPORTED (the caller keeps the library's differentiable attention for them).
+ * bnb_sdpa_masked_bwd_path selects the kernel (BNB_SDPA_PATH_*; AUTO = vector-ALU kernel up to 32
+ * tokens, matrix cores above), for tests and benchmarks.
  */
 int bnb_sdpa_masked_bwd(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, const void *out,
                         const void *dout, void *dqkv, int64_t B, int NM, int H, int dh, int dtype, void *stream);
+int bnb_sdpa_masked_bwd_path(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, const void *out,
+                             const void *dout, void *dqkv, int64_t B, int NM, int H, int dh, int dtype, int path,
+                             void *stream);
 
 /*
  * RMSNorm backward:  y = x * rsqrt(mean(x^2) + eps) * weight

@@ -1755,3 +1755,33 @@ def test_gelu_mul_packed_train_equals_the_two_operand_form():
     ref.backward(up)
     assert torch.equal(out.reshape(R, H), ref)
     assert torch.equal(gu.grad[:, :H], a.grad) and torch.equal(gu.grad[:, H:], b.grad)
+
+
+@pytest.mark.parametrize("B,NM,H", [(3, 12, 4), (5, 27, 4), (4, 1, 4), (6, 32, 4), (5, 33, 4), (4, 64, 4), (3, 84, 4), (2, 152, 4),
+                                    (2, 160, 4), (3, 100, 2), (300, 40, 4)])
+@pytest.mark.parametrize("p_alive", [1.0, 0.7, 0.0])
+def test_sdpa_masked_bwd_on_the_matrix_cores_matches_autograd_of_the_oracle(B, NM, H, p_alive):
+    D = 32 * H
+    qkv = _qkv(B * 17 + NM, B, NM, D, torch.bfloat16, scale=1.5)
+    alive = None if p_alive == 1.0 else _alive(NM + B, B, NM, p_alive)
+    if alive is not None and p_alive > 0 and B > 2:
+        alive[1] = False
+    g = torch.Generator().manual_seed(B + NM)
+    up = torch.randn(B, NM, D, generator=g).bfloat16()
+    ref_out, ref_grad = _sdpa_truth_grad(qkv, alive, H, up)
+    mask = None if alive is None else alive.to(DEV)
+    out = ops.sdpa_masked(qkv.to(DEV), mask, H)
+    dqkv = ops.sdpa_masked_bwd(qkv.to(DEV), mask, H, out, up.to(DEV), path="mfma")
+    torch.cuda.synchronize()
+    for name, cols in (("dQ", slice(0, D)), ("dK", slice(D, 2 * D)), ("dV", slice(2 * D, 3 * D))):
+        if NM == 1 and name != "dV":
+            assert dqkv[..., cols].float().abs().max() <= 1e-6 * ref_grad.abs().max(), name
+            continue
+        assert max_rel(dqkv[..., cols].float().cpu().double(), ref_grad[..., cols]) <= BF16_TOL, name
+    if alive is not None and p_alive > 0:
+        dead = ~alive & alive.any(dim=1, keepdim=True)
+        assert not dqkv.cpu()[..., D:][dead].any()
+    assert torch.equal(dqkv, ops.sdpa_masked_bwd(qkv.to(DEV), mask, H, out, up.to(DEV), path="mfma"))
+    if NM <= 32:  # the two kernels against each other
+        other = ops.sdpa_masked_bwd(qkv.to(DEV), mask, H, out, up.to(DEV), path="valu")
+        assert max_rel(dqkv.float().cpu(), other.float().cpu()) <= BF16_TOL
