@@ -584,3 +584,36 @@ def test_update_path_gradients_agree_between_the_kernels_and_the_library_ops(mon
     for name, g in routed.items():
         assert torch.isfinite(g).all(), name
         assert max_rel(g.cpu(), library[name].cpu()) <= BF16_TOL, name
+
+
+def test_update_path_kernels_compose_with_activation_checkpointing():
+    """The reference can wrap each block's sequence pass in torch.utils.checkpoint (policy.py:452-466); the
+    training kernels' autograd Functions must give the same gradients when recomputed that way."""
+    from torch.utils.checkpoint import checkpoint
+
+    cfg = _cfg(128, 4, spatial=1, temporal=1)
+    torch.manual_seed(9)
+    block = bnb.YemongBlock(cfg).to(DEV)
+    T, B, N, M, D = 12, 64, 8, 4, 128
+    gen = torch.Generator().manual_seed(10)
+    x = torch.randn(T, B, N + M, D, generator=gen).to(DEV).requires_grad_()
+    alive = (torch.rand(T, B, N + M, generator=gen) < 0.85).to(DEV)
+    alive[..., 0] = True
+    h0 = torch.zeros(1, B * N, D, device=DEV)
+    cb0 = torch.zeros(1, B * N, 3, D, device=DEV)
+    done = (torch.rand(T, B, generator=gen) < 0.1).to(DEV)
+
+    def run(x_in):
+        return block.sequence(x_in, alive, h0, cb0, done, N)[0]
+
+    def grads(wrapped):
+        block.zero_grad(set_to_none=True)
+        x.grad = None
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = checkpoint(run, x, use_reentrant=False) if wrapped else run(x)
+        out.float().square().mean().backward()
+        return [x.grad.clone()] + [p.grad.clone() for p in block.parameters()]
+
+    plain, recomputed = grads(False), grads(True)
+    for a, b in zip(plain, recomputed):
+        assert torch.equal(a, b)  # same kernels, same order: identical bits
