@@ -754,14 +754,38 @@ def main():
             dvc = torch.randn(Tu, Rc, D, device=dev, generator=gen)
             kern["conv_seq_bwd"] = stream_leg(lambda t: ops.conv_seq_bwd(bc, cc, wc, dc, dvc, time_major=True), Tu * Rc * D * (2 + 4 + 2))
             del bc, cc, dvc
+            # the value head's team pooling over the same rollout, forward + backward
+            pma_u = bnb.TeamPMA(D, H).to(dev)
+            with torch.no_grad():
+                pma_u.seeds.normal_(0.0, 0.02)
+            xs_u = torch.randn(Tu * Bu, Nu, D, device=dev, generator=gen, requires_grad=True)
+            tm_u = torch.randint(0, 2, (Tu * Bu, Nu), device=dev, generator=gen, dtype=torch.int32)
+            al_u = torch.rand(Tu * Bu, Nu, device=dev, generator=gen) < 0.9
+            go_u = torch.randn(Tu * Bu, Nu, D, device=dev, generator=gen)
+
+            def pool_step(t):
+                pma_u.zero_grad(set_to_none=True)
+                xs_u.grad = None
+                with torch.enable_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+                    pma_u(xs_u, tm_u, al_u).backward(go_u)
+
+            t_pool_up = timed_loop(pool_step, 4, 2) / 4
+            t_pool_up_lib = None
+            if not args.no_torch_baseline:
+                with trunk_module.library_update_path():
+                    t_pool_up_lib = timed_loop(pool_step, 3, 2) / 3
+            del pma_u, xs_u, tm_u, al_u, go_u
             result["update_path"] = {
                 "rows": Rw, "linear_wgrad": wg, "kernels": kern, "block_fwd_bwd_ms": t_up * 1e3,
+                "team_pool_fwd_bwd_ms": t_pool_up * 1e3,
+                "team_pool_fwd_bwd_library_ms": None if t_pool_up_lib is None else t_pool_up_lib * 1e3,
                 "block_fwd_bwd_library_ms": None if t_up_lib is None else t_up_lib * 1e3,
                 "what": "bnb_linear_wgrad_fwd (dW = dy^T x, bf16 in, fp32 out, rows split over the chip) beside the library "
                         "GEMM on the same operands; kernels = the norm, gelu-gate, attention and conv backward kernels at the "
                         "sizes of the block below; block = one YemongBlock (2 attention + 1 temporal sublayer), T = 128 x 256 "
                         "environments of 4v4, forward + backward under bf16 autocast, on the update-path kernels and with "
-                        "torch's own differentiable ops in their place (the recurrence keeps its kernels in both)",
+                        "torch's own differentiable ops in their place (the recurrence keeps its kernels in both); team_pool = TeamPMA "
+                        "forward + backward over the ships of the same rollout (32,768 environments x 8 ships), kernels and library",
             }
             del blk, xu, au, hu, cu, du
 

@@ -45,6 +45,9 @@ SIGNATURES = {
     "bnb_rmsnorm_bwd_blocks": (_i, [_i64, _i]),
     "bnb_rmsnorm_bwd": (_i, [_vp, _i64, _vp, _i, _i64, _vp, _f, _vp, _vp, _vp, _vp, _i, _vp, _i64, _i, _vp]),
     "bnb_team_attend_fwd": (_i, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "bnb_team_attend_bwd": (_i, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "bnb_team_attend_bwd_partial_rows": (_i, []),
+    "bnb_team_gather_bwd": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i, _i, _i, _vp]),
     "bnb_team_norm_broadcast_fwd": (_i, [_vp, _vp, _f, _vp, _i64, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "bnb_temporal_step_fwd": (
         _i, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _f, _vp, _i64, _i64,

@@ -11,6 +11,7 @@ synchronise.  They are forward-only and run on a ROCm device only: anything else
 
 from __future__ import annotations
 
+import functools
 import math
 
 import torch
@@ -18,6 +19,17 @@ import torch
 from . import _native
 
 _DTYPE_CODE = {torch.float32: _native.F32, torch.bfloat16: _native.BF16}
+def _outside_autocast(backward):
+    """A custom Function's backward inherits the autocast state of the place ``.backward()`` is called
+    from; inside it torch GEMMs would return bfloat16 tensors where the kernels are handed float32
+    pointers.  Every backward here runs with autocast off and states its dtypes itself."""
+    @functools.wraps(backward)
+    def wrapped(ctx, *grads):
+        with torch.autocast("cuda", enabled=False):
+            return backward(ctx, *grads)
+    return wrapped
+
+
 _PATH_CODE = {"auto": _native.PATH_AUTO, "valu": _native.PATH_VALU, "mfma": _native.PATH_MFMA}
 
 
@@ -158,6 +170,7 @@ class _SdpaTrain(torch.autograd.Function):
         return out
 
     @staticmethod
+    @_outside_autocast
     def backward(ctx, dout):
         qkv, out = ctx.saved_tensors
         return sdpa_masked_bwd(qkv, ctx.alive, ctx.n_heads, out, dout), None, None
@@ -488,6 +501,7 @@ class _LinearTrain(torch.autograd.Function):
         return torch.nn.functional.linear(xb, wb, None if bias is None else bias.to(torch.bfloat16))
 
     @staticmethod
+    @_outside_autocast
     def backward(ctx, dy):
         xb, wb = ctx.saved_tensors
         dy = dy.contiguous() if dy.stride(-1) != 1 else dy
@@ -538,7 +552,7 @@ def team_pool_supported(x: torch.Tensor, n_heads: int) -> bool:
 
 def team_pool(x: torch.Tensor, team_id: torch.Tensor, alive: torch.Tensor, score_vectors: torch.Tensor,
               folded_projection: torch.Tensor, norm_weight: torch.Tensor, eps: float | None, n_heads: int, *,
-              broadcast: bool = True):
+              broadcast: bool = True, intermediates: bool = False):
     """Per-team attention pooling of the ship rows (TeamPMA.forward, policy.py:94-120): a kernel
     that reads the ships once and leaves the weighted mean row per (team, head), one float32
     library GEMM with the folded value/output projection, a kernel for RMSNorm and the hand-out.
@@ -553,7 +567,9 @@ def team_pool(x: torch.Tensor, team_id: torch.Tensor, alive: torch.Tensor, score
         broadcast: also return the (B, N, 128) tensor in which every ship holds its team's vector.
 
     Returns:
-        (ships or None, pool): ``pool`` is (B, 2, 128), zero for a team without an alive ship.
+        (ships or None, pool): ``pool`` is (B, 2, 128), zero for a team without an alive ship.  With
+        ``intermediates`` also the attention-weighted mean rows ``z`` (B*2, H*128) and the projected
+        rows before the norm (B*2, 128), which the backward needs.
     """
     if x.dim() != 3 or x.shape[-1] != FFN_WIDTH or x.dtype != torch.float32:
         raise ValueError("x must be float32 (B, N, 128)")
@@ -583,6 +599,7 @@ def team_pool(x: torch.Tensor, team_id: torch.Tensor, alive: torch.Tensor, score
     ships = torch.empty((B, N, D), dtype=torch.float32, device=dev) if broadcast else None
     if eps is None:
         eps = torch.finfo(torch.float32).eps
+    z = pre = None
     if B:
         def env_stride(t):
             return t.stride(0) if B > 1 else t.shape[1] * (t.stride(1) if N else 1)
@@ -604,7 +621,102 @@ def team_pool(x: torch.Tensor, team_id: torch.Tensor, alive: torch.Tensor, score
                 B, N, D, _stream(),
             )
             _native.check(rc, "bnb_team_norm_broadcast_fwd")
+    if intermediates:
+        if z is None:
+            z = torch.zeros((0, n_heads * D), dtype=torch.float32, device=dev)
+            pre = torch.zeros((0, D), dtype=torch.float32, device=dev)
+        return ships, pool, z, pre
     return ships, pool
+
+
+def team_pool_constants(seeds: torch.Tensor, in_proj_weight: torch.Tensor, out_proj_weight: torch.Tensor,
+                        n_heads: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """``pack_team_pool_weights`` as differentiable float32 torch ops on the (small) parameters, for the
+    update path: gradients of the two constants flow back to ``seeds`` and the attention weights."""
+    D = seeds.shape[-1]
+    dh = D // n_heads
+    with torch.autocast(seeds.device.type, enabled=False):
+        w = in_proj_weight.float()
+        wq, wk, wv = w[:D], w[D:2 * D], w[2 * D:]
+        q = (seeds.float() @ wq.t()).view(2, n_heads, dh)
+        u = torch.einsum("thd,hdc->thc", q, wk.view(n_heads, dh, D)) * (math.log2(math.e) / math.sqrt(dh))
+        wo = out_proj_weight.float().view(D, n_heads, dh)
+        m = torch.einsum("ohd,hdc->hco", wo, wv.view(n_heads, dh, D))
+        return u.reshape(2 * n_heads, D), m.reshape(n_heads * D, D)
+
+
+class _TeamPoolTrain(torch.autograd.Function):
+    """``team_pool`` (broadcast form) with a backward: the forward runs on the pooling kernels, the
+    backward on the norm-backward kernel, two small float32 GEMMs with the folded projection and the
+    attention-backward kernel (which recomputes the weights from the score vectors)."""
+
+    @staticmethod
+    def forward(ctx, x, team_id, alive, u, folded, norm_weight, eps, n_heads):
+        with torch.no_grad():
+            ships, _, z, pre = team_pool(x, team_id, alive, u, folded, norm_weight, eps, n_heads, intermediates=True)
+        ctx.save_for_backward(x, team_id, alive, u, folded, norm_weight, z, pre)
+        ctx.eps = eps
+        ctx.n_heads = n_heads
+        return ships
+
+    @staticmethod
+    @_outside_autocast
+    def backward(ctx, dships):
+        x, team_id, alive, u, folded, norm_weight, z, pre = ctx.saved_tensors
+        B, N, D = x.shape
+        H = ctx.n_heads
+        dev = x.device
+        u = u.float().contiguous()
+        folded = folded.float()
+        lib = _native.load()
+        dships = dships.float().contiguous()
+        if N and (x.stride(2) != 1 or x.stride(1) % 4 or (B > 1 and x.stride(0) % 4)):
+            x = x.contiguous()
+        if team_id.dtype != torch.int32 or (N and team_id.stride(1) != 1):
+            team_id = team_id.to(torch.int32).contiguous()
+        if N and alive.stride(1) != 1:
+            alive = alive.contiguous()
+
+        def env_stride(t):
+            return t.stride(0) if B > 1 else t.shape[1] * (t.stride(1) if N else 1)
+
+        dpool = torch.empty((B, 2, D), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            rc = lib.bnb_team_gather_bwd(dships.data_ptr(), team_id.data_ptr(), env_stride(team_id) if N else 0, alive.data_ptr(),
+                                         env_stride(alive) if N else 0, dpool.data_ptr(), B, N, D, _stream())
+        _native.check(rc, "bnb_team_gather_bwd")
+        dpre, dnorm = rmsnorm_bwd(pre.view(B, 2, D), dpool, norm_weight, eps=ctx.eps)
+        dpre = dpre.reshape(B * 2, D)
+        dz = (dpre @ folded.t()).float().contiguous()  # (B*2, H*D) float32: the kernel reads it through a float pointer
+        # z^T dpre contracts over 2B rows: batches of 1024 rows through the batched GEMM, then one sum
+        rows = B * 2
+        if rows >= 4096 and rows % 1024 == 0:
+            dfolded = torch.bmm(z.view(rows // 1024, 1024, H * D).transpose(1, 2), dpre.view(rows // 1024, 1024, D)).sum(dim=0)
+        else:
+            dfolded = z.t() @ dpre
+
+        for name, t, shape in (("z", z, (B * 2, H * D)), ("dz", dz, (B * 2, H * D)), ("score_vectors", u, (2 * H, D))):
+            if t.dtype != torch.float32 or tuple(t.shape) != shape or not t.is_contiguous():
+                raise TypeError(f"{name} must be a contiguous float32 {shape} tensor, got {t.dtype} {tuple(t.shape)}")
+        dx = torch.empty((B, N, D), dtype=torch.float32, device=dev)
+        ds = torch.empty((B * N, 2 * H), dtype=torch.float32, device=dev)
+        du = torch.empty((2 * H, D), dtype=torch.float32, device=dev)
+        partials = torch.empty((int(lib.bnb_team_attend_bwd_partial_rows()), 2 * H, D), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            rc = lib.bnb_team_attend_bwd(
+                x.data_ptr(), env_stride(x) if N else 0, x.stride(1) if N else D, team_id.data_ptr(), env_stride(team_id) if N else 0,
+                alive.data_ptr(), env_stride(alive) if N else 0, u.data_ptr(), z.data_ptr(), dz.data_ptr(),
+                dx.data_ptr(), ds.data_ptr(), partials.data_ptr(), du.data_ptr(), B, N, H, D, _stream(),
+            )
+        _native.check(rc, "bnb_team_attend_bwd")
+        return dx, None, None, du, dfolded, dnorm, None, None
+
+
+def team_pool_train(x, team_id, alive, score_vectors, folded_projection, norm_weight, eps, n_heads) -> torch.Tensor:
+    """Differentiable ``team_pool`` (the (B, N, 128) broadcast form); ``score_vectors`` and
+    ``folded_projection`` from ``team_pool_constants`` so that their gradients reach the parameters."""
+    with torch.autocast("cuda", enabled=False):
+        return _TeamPoolTrain.apply(x, team_id, alive, score_vectors, folded_projection, norm_weight, eps, n_heads)
 
 
 def pack_gate_weights(weight_a: torch.Tensor, weight_x: torch.Tensor) -> torch.Tensor:
@@ -885,6 +997,7 @@ class _ConvSeqTrain(torch.autograd.Function):
         return v, new_buf
 
     @staticmethod
+    @_outside_autocast
     def backward(ctx, dv, dbuf):
         b1, conv_buf, weight = ctx.saved_tensors
         if dv is None:
@@ -990,6 +1103,7 @@ class _RglruScan(torch.autograd.Function):
         return y, h_last
 
     @staticmethod
+    @_outside_autocast
     def backward(ctx, dy, dh_last):
         x, gates_pre, log_lambda, h0, y = ctx.saved_tensors
         T, R = (x.shape[0], x.shape[1]) if ctx.time_major else (x.shape[1], x.shape[0])
@@ -1121,6 +1235,7 @@ class _RmsNormTrain(torch.autograd.Function):
         return x.view_as(x), n
 
     @staticmethod
+    @_outside_autocast
     def backward(ctx, ds, dn):
         x, weight = ctx.saved_tensors
         if dn is None:
@@ -1143,6 +1258,7 @@ class _AddRmsNormTrain(torch.autograd.Function):
         return s, n
 
     @staticmethod
+    @_outside_autocast
     def backward(ctx, ds, dn):
         s, weight = ctx.saved_tensors
         if dn is None:
@@ -1248,6 +1364,7 @@ class _GeluMulTrain(torch.autograd.Function):
         return out
 
     @staticmethod
+    @_outside_autocast
     def backward(ctx, dout):
         a, b = ctx.saved_tensors
         da, db = gelu_mul_bwd(a, b, dout)
@@ -1267,6 +1384,7 @@ class _GeluMulPackedTrain(torch.autograd.Function):
         return out
 
     @staticmethod
+    @_outside_autocast
     def backward(ctx, dout):
         (gu,) = ctx.saved_tensors
         H = gu.shape[-1] // 2

@@ -705,8 +705,13 @@ class TeamPMA(nn.Module):
         return self.norm(out).to(x.dtype)
 
     def forward(self, x: torch.Tensor, team_id: torch.Tensor, alive: torch.Tensor) -> torch.Tensor:
-        if not torch.is_grad_enabled() and ops.team_pool_supported(x, self.n_heads):
-            return ops.team_pool(x, team_id, alive, *self._folded(), self.norm.weight, self.norm.eps, self.n_heads)[0]
+        if ops.team_pool_supported(x, self.n_heads):
+            if not torch.is_grad_enabled():
+                return ops.team_pool(x, team_id, alive, *self._folded(), self.norm.weight, self.norm.eps, self.n_heads)[0]
+            if _TRAIN_KERNELS and self.norm.weight.dtype == torch.float32:
+                # update path: the same kernels forward, gradients through the score vectors and the folded projection
+                u, folded = ops.team_pool_constants(self.seeds, self.attn.in_proj_weight, self.attn.out_proj.weight, self.n_heads)
+                return ops.team_pool_train(x, team_id, alive, u, folded, self.norm.weight, self.norm.eps, self.n_heads)
         B, N, D = x.shape
         pool = self._pooled_library(x, team_id, alive)
         return pool.gather(1, team_id.clamp(0, 1).long().unsqueeze(-1).expand(B, N, D))

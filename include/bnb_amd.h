@@ -353,6 +353,31 @@ int bnb_team_norm_broadcast_fwd(const float *pre, const float *norm_weight, floa
                                 int B, int N, int D, void *stream);
 
 /*
+ * Backward of bnb_team_attend_fwd for the update path (autograd through the attention weights of
+ * TeamPMA.forward, models/yemong/policy.py:94-120, in train/rl/ppo.py:1417-1425).
+ *
+ *   x, team_id, alive, score_vectors  as passed to the forward
+ *   z, dz     (B, 2, H, 128) fp32: the forward's result and its gradient
+ *   dx        (B, N, 128) fp32 contiguous: gradient of the ship rows
+ *   ds        (B*N, 2H) fp32 workspace/result: gradient of the base-2 scores (zero under the other team's heads)
+ *   partials  (bnb_team_attend_bwd_partial_rows(), 2H, 128) fp32 workspace
+ *   du        (2H, 128) fp32: gradient of score_vectors, rows added in a fixed order
+ */
+int bnb_team_attend_bwd(const float *x, int64_t x_env_stride, int64_t x_row_stride, const int32_t *team_id,
+                        int64_t team_env_stride, const uint8_t *alive, int64_t alive_env_stride,
+                        const float *score_vectors, const float *z, const float *dz, float *dx, float *ds,
+                        float *partials, float *du, int B, int N, int H, int D, void *stream);
+int bnb_team_attend_bwd_partial_rows(void);
+
+/*
+ * Backward of the hand-out of bnb_team_norm_broadcast_fwd: dpool (B, 2, 128) = per team the sum of
+ * dout (B, N, 128, contiguous) over the ships that hold that team's vector, zero for a team without
+ * an alive ship of its own.
+ */
+int bnb_team_gather_bwd(const float *dout, const int32_t *team_id, int64_t team_env_stride, const uint8_t *alive,
+                        int64_t alive_env_stride, float *dpool, int B, int N, int D, void *stream);
+
+/*
  * One timestep of the temporal sublayer's state path in one launch: conv taps + buffer shift
  * (bnb_conv_step_rows_fwd), the two RG-LRU gate projections, and the recurrence
  * (bnb_rglru_step_rows_fwd), under the dtype flow of bfloat16 autocast.

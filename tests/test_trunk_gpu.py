@@ -502,8 +502,11 @@ def test_team_pooling_layer_matches_oracle(autocast, D, H):
     assert (got.cpu()[1] == 0).all()  # everybody dead in environment 1
 
 
-def test_team_pooling_layer_trains_through_the_library_path():
-    D, H, B, N = 128, 4, 5, 8
+@pytest.mark.parametrize("kernels", [True, False])
+def test_team_pooling_layer_trains_and_matches_autograd_of_the_oracle(kernels):
+    from boost_and_broadside_amd import trunk
+
+    D, H, B, N = 128, 4, 37, 8
     g = torch.Generator().manual_seed(21)
     p = team_pool_params(g, "tp.", D)
     layer = bnb.TeamPMA(D, H).to(DEV)
@@ -514,15 +517,44 @@ def test_team_pooling_layer_trains_through_the_library_path():
     team = (torch.arange(N, dtype=torch.int32) % 2).repeat(B, 1)
     alive = torch.rand(B, N, generator=g) < 0.6
     alive[:, :2] = True
-    out = layer(x, team.to(DEV), alive.to(DEV))
-    out.square().sum().backward()
+    up = torch.randn(B, N, D, generator=g)
+
+    def run():
+        out = layer(x, team.to(DEV), alive.to(DEV))
+        (out * up.to(DEV)).sum().backward()
+        return out
+
+    if kernels:
+        out = run()
+    else:
+        with trunk.library_update_path():
+            out = run()
     assert torch.isfinite(x.grad).all() and all(torch.isfinite(q.grad).all() for q in layer.parameters())
     with torch.no_grad():
         assert max_rel(layer(x.detach(), team.to(DEV), alive.to(DEV)), out.detach()) <= 1e-5
     xr = x.detach().cpu().double().requires_grad_()
-    ref, _ = torch_ref.team_pool({k: v.double() for k, v in p.items()}, "tp.", xr, team, alive, H)
-    ref.square().sum().backward()
+    pr = {k: v.double().requires_grad_() for k, v in p.items()}
+    ref, _ = torch_ref.team_pool(pr, "tp.", xr, team, alive, H)
+    (ref * up.double()).sum().backward()
     assert max_rel(x.grad.cpu(), xr.grad.float()) <= 1e-4
+    for name, q in layer.named_parameters():
+        assert max_rel(q.grad.cpu().double(), pr["tp." + name].grad) <= 1e-4, name
+
+
+def test_team_pooling_gradients_with_empty_teams_are_finite_and_skip_them():
+    D, H, B, N = 128, 4, 16, 8
+    g = torch.Generator().manual_seed(23)
+    p = team_pool_params(g, "tp.", D)
+    layer = bnb.TeamPMA(D, H).to(DEV)
+    layer.load_state_dict(_strip(p, "tp."))
+    x = torch.randn(B, N, D, generator=g).to(DEV).requires_grad_()
+    team = torch.randint(0, 2, (B, N), generator=g, dtype=torch.int32)
+    alive = torch.rand(B, N, generator=g) < 0.5
+    team[0] = 0            # team 1 absent
+    alive[1] = False       # nobody alive
+    layer(x, team.to(DEV), alive.to(DEV)).square().sum().backward()
+    assert torch.isfinite(x.grad).all() and all(torch.isfinite(q.grad).all() for q in layer.parameters())
+    assert not x.grad[1].any()  # no key, no gradient
 
 
 def test_attention_block_outside_kernel_coverage_uses_the_library_on_the_device():
@@ -617,3 +649,45 @@ def test_update_path_kernels_compose_with_activation_checkpointing():
     plain, recomputed = grads(False), grads(True)
     for a, b in zip(plain, recomputed):
         assert torch.equal(a, b)  # same kernels, same order: identical bits
+
+
+def test_backward_called_inside_autocast_matches_backward_called_outside():
+    """``loss.backward()`` inside the autocast block hands its autocast state to every custom backward; the
+    kernels' backward code must not let a GEMM of its own turn bfloat16 there (a float32 pointer is what the
+    kernels are given).  Same gradients as with backward called outside."""
+    cfg = _cfg(128, 4, spatial=1, temporal=1)
+    torch.manual_seed(11)
+    block = bnb.YemongBlock(cfg).to(DEV)
+    pma = bnb.TeamPMA(128, 4).to(DEV)
+    with torch.no_grad():
+        pma.seeds.normal_(0.0, 0.02)
+    T, B, N, M, D = 8, 40, 8, 4, 128
+    gen = torch.Generator().manual_seed(12)
+    x = torch.randn(T, B, N + M, D, generator=gen).to(DEV).requires_grad_()
+    alive = (torch.rand(T, B, N + M, generator=gen) < 0.85).to(DEV)
+    alive[..., 0] = True
+    team = torch.randint(0, 2, (T * B, N), generator=gen, dtype=torch.int32).to(DEV)
+    h0 = torch.zeros(1, B * N, D, device=DEV)
+    cb0 = torch.zeros(1, B * N, 3, D, device=DEV)
+    done = (torch.rand(T, B, generator=gen) < 0.1).to(DEV)
+    params = list(block.parameters()) + list(pma.parameters())
+
+    def grads(inside):
+        for q in params:
+            q.grad = None
+        x.grad = None
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = block.sequence(x, alive, h0, cb0, done, N)[0]
+            pooled = pma(out[:, :, :N].reshape(T * B, N, D), team, alive[:, :, :N].reshape(T * B, N))
+            loss = out.float().square().mean() + pooled.float().square().mean()
+            if inside:
+                loss.backward()
+        if not inside:
+            loss.backward()
+        return [x.grad.clone()] + [q.grad.clone() for q in params]
+
+    for a, b in zip(grads(False), grads(True)):
+        # torch's own backward GEMMs (the small parameter einsums, F.linear) do change precision with the autocast
+        # state, so the comparison is at the bf16 bar, not bitwise
+        assert torch.isfinite(b).all()
+        assert max_rel(b.float().cpu(), a.float().cpu()) <= BF16_TOL
