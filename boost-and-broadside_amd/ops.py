@@ -1110,8 +1110,8 @@ class _RglruScan(torch.autograd.Function):
         D = x.shape[2]
         x_c, g_c = x.contiguous(), gates_pre.contiguous()
         h0_c = h0 if h0.stride(1) == 1 else h0.contiguous()
-        dy = dy.contiguous()
-        dh_last = dh_last.contiguous()
+        dy = dy.to(y.dtype).contiguous()          # the kernel reads dy in y's dtype and dh_last as float32
+        dh_last = dh_last.float().contiguous()
         dx = torch.empty_like(x_c)
         dgates = torch.empty_like(g_c)
         dh0 = torch.empty((R, D), dtype=torch.float32, device=x.device)
