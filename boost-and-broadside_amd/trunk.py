@@ -31,6 +31,7 @@ from dataclasses import dataclass
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
+import torch.utils.checkpoint
 
 from . import _native, ops
 
@@ -789,9 +790,10 @@ class YemongBlock(nn.Module):
                  bullet_mask=None):
         """(T,B,NM,D) variant of ``step`` for re-evaluating a stored rollout.
 
-        Under ``torch.no_grad()`` every sublayer runs on the kernels.  With gradients enabled
-        (the PPO update) the projections, norms, attention and conv are torch ops and the
-        recurrence runs on its forward and backward kernels."""
+        Under ``torch.no_grad()`` every sublayer runs on the inference kernels.  With gradients
+        enabled (the PPO update) the recurrence, the conv, the norms, the gelu gates, the attention
+        and the Linear weight gradients run on forward and backward kernels; the forward and
+        input-gradient GEMMs stay with the library."""
         T, B, NM, D = x.shape
         n_rec = NM if num_recurrent is None else num_recurrent
         for layer in self.spatial:
@@ -843,6 +845,35 @@ class YemongTrunk(nn.Module):
         """Zero all rows of finished environments (rows are env-major)."""
         keep = (~done_mask.repeat_interleave(num_recurrent_tokens)).to(hidden.dtype)
         return hidden * keep[None, :, None]
+
+    def sequence(self, x, alive_mask, initial_hidden, done_mask=None, bullets=None, bullet_mask=None, *,
+                 grad_checkpoint: bool = False) -> torch.Tensor:
+        """The trunk part of the rollout re-evaluation of the PPO update (policy.py:424-477): every block's
+        ``sequence`` over (T, B, NM, D) tokens from the rollout-start state, ``done_mask`` (T, B) resetting
+        the recurrence after an episode end.  ``initial_hidden`` is the packed (n_layers, B*n_rec, 4*D)
+        state; the final states are not needed by the update and not returned.  ``grad_checkpoint``
+        recomputes each block in the backward pass instead of keeping its activations, as the
+        reference's ``grad_checkpoint`` option does."""
+        T, B, NM, D = x.shape
+        n_layers, rows = initial_hidden.shape[0], initial_hidden.shape[1]
+        if n_layers != self.n_hidden_layers or rows % B:
+            raise ValueError(f"initial_hidden must be ({self.n_hidden_layers}, B*n_rec, {CONV_KERNEL * D})")
+        n_rec = rows // B
+        h_all = initial_hidden[:, :, :D]
+        cb_all = initial_hidden[:, :, D:].reshape(n_layers, rows, CONV_KERNEL - 1, D)
+        slot = 0
+        for layer in self.yemong_layers:
+            own = slice(slot, slot + layer.n_temporal)
+            slot += layer.n_temporal
+
+            def run(x_in, layer=layer, own=own):
+                return layer.sequence(x_in, alive_mask, h_all[own], cb_all[own], done_mask, n_rec, bullets, bullet_mask)[0]
+
+            if grad_checkpoint and torch.is_grad_enabled():
+                x = torch.utils.checkpoint.checkpoint(run, x, use_reentrant=False)
+            else:
+                x = run(x)
+        return x
 
     @torch.no_grad()
     def forward(self, tokens, alive_mask, recurrent_state, bullets=None, bullet_mask=None, *, reset_mask=None,

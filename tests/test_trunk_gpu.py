@@ -691,3 +691,48 @@ def test_backward_called_inside_autocast_matches_backward_called_outside():
         # state, so the comparison is at the bf16 bar, not bitwise
         assert torch.isfinite(b).all()
         assert max_rel(b.float().cpu(), a.float().cpu()) <= BF16_TOL
+
+
+@pytest.mark.parametrize("blocks,temporal", [(1, 1), (2, 1), (2, 2)])
+def test_trunk_sequence_is_the_loop_over_blocks_and_trains_with_and_without_checkpointing(blocks, temporal):
+    # the trunk part of policy.py:424-477: per block the slots [i*n_temporal, (i+1)*n_temporal) of the packed state
+    D, H, B, N, M, T = 128, 4, 6, 8, 4, 10
+    torch.manual_seed(31)
+    trunk = bnb.YemongTrunk(_cfg(D, H, blocks, 1, temporal)).to(DEV)
+    gen = torch.Generator().manual_seed(32)
+    xs = torch.randn(T, B, N + M, D, generator=gen).to(DEV)
+    alive = (torch.rand(T, B, N + M, generator=gen) < 0.85).to(DEV)
+    alive[..., 0] = True
+    done = (torch.rand(T, B, generator=gen) < 0.15).to(DEV)
+    hidden0 = 0.3 * torch.randn(blocks * temporal, B * N, 4 * D, generator=gen).to(DEV)
+
+    with torch.no_grad():
+        got = trunk.sequence(xs, alive, hidden0, done)
+        x = xs
+        h_all, cb_all = hidden0[:, :, :D], hidden0[:, :, D:].reshape(blocks * temporal, B * N, 3, D)
+        for i, block in enumerate(trunk.yemong_layers):
+            sl = slice(i * temporal, (i + 1) * temporal)
+            x = block.sequence(x, alive, h_all[sl], cb_all[sl], done, N)[0]
+        assert torch.equal(got, x)
+        # and step by step with the state reset after an episode end
+        hidden, outs = hidden0, []
+        for t in range(T):
+            out, hidden = trunk(xs[t], alive[t], hidden)
+            hidden = trunk.reset_hidden_for_envs(hidden, done[t], N)
+            outs.append(out)
+        assert max_rel(got, torch.stack(outs)) <= 5e-5
+
+    def grads(ckpt):
+        trunk.zero_grad(set_to_none=True)
+        xin = xs.clone().requires_grad_()
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = trunk.sequence(xin, alive, hidden0, done, grad_checkpoint=ckpt)
+        out.float().square().mean().backward()
+        return [xin.grad] + [q.grad.clone() for q in trunk.parameters()]
+
+    plain, recomputed = grads(False), grads(True)
+    assert all(torch.isfinite(g).all() for g in plain)
+    for a, b in zip(plain, recomputed):
+        assert torch.equal(a, b)
+    with pytest.raises(ValueError):
+        trunk.sequence(xs, alive, hidden0[:, :-1], done)
