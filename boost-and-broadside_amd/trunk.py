@@ -296,7 +296,7 @@ class TransformerBlock(nn.Module):
             if self.reads_bullets and bullets is not None:
                 if isinstance(bullet_mask, ops.CompactRows):
                     bullet_mask = bullet_mask.mask
-                kv = _project(self.kv_bullet, self.norm_bullet(bullets))
+                kv = _project(self.kv_bullet, _train_norm(self.norm_bullet, bullets)[1])
                 merged = merged + self._bullet_read(qkv, kv, bullet_mask)
             return _project(self.out_proj, merged)
         try:
