@@ -251,11 +251,17 @@ static int launch_sdpa_bwd(const void *qkv, int64_t qkv_row_stride, const uint8_
 
 constexpr int kMbPitch = kSbDh + 8;  // halfs per token row in LDS (80 bytes: 16-byte aligned, bank-spread)
 
-template <int NB>
+// NB = blocks of 32 tokens on the longer of the two axes (waves of the work-group).  CROSS: the keys and
+// values come from a second buffer kv (B, NK, 2*H*32) with its own mask (the bullet read,
+// models/yemong/attention.py:149-166): an environment without a live key contributed exactly nothing
+// in the forward (the reference gates it off), so all its gradients are zero; `out` is that read's own
+// result, before it was added to anything.
+template <int NB, bool CROSS>
 __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
-    const uint16_t *__restrict__ qkv, int64_t qkv_row_stride, const uint8_t *__restrict__ alive,
-    const uint16_t *__restrict__ out, const uint16_t *__restrict__ dout, uint16_t *__restrict__ dqkv, int B, int NM, int H,
-    float scale)
+    const uint16_t *__restrict__ q, int64_t q_row_stride, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
+    int64_t kv_row_stride, const uint8_t *__restrict__ alive, const uint16_t *__restrict__ out,
+    const uint16_t *__restrict__ dout, uint16_t *__restrict__ dq_out, int64_t dq_row_stride, uint16_t *__restrict__ dk_out,
+    uint16_t *__restrict__ dv_out, int64_t dkv_row_stride, int B, int NQ, int NK, int H, float scale)
 {
     constexpr int CAP = NB * 32;
     constexpr int TP = CAP + 4;  // halfs per row of a transposed copy
@@ -275,23 +281,24 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
     const int m = lane & 31, half = lane >> 5;
     const float c = scale * 1.4426950408889634f;
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    const int nqb = (NQ + 31) >> 5, nkb = (NK + 31) >> 5;  // <= NB
 
-    // token-major and channel-major copies of two (NM, 32) operands; rows past NM are zero.  The loads of
+    // token-major and channel-major copies of two (n, 32) operands; rows past n are zero.  The loads of
     // both phases are issued at the start of the kernel, so their latency is paid once.
     struct Staged {
         u32x4 a[2], b[2];
     };
-    auto stage_load = [&](const uint16_t *a, int64_t a_stride, const uint16_t *b, int64_t b_stride) -> Staged {
+    auto stage_load = [&](const uint16_t *a, int64_t a_stride, const uint16_t *b, int64_t b_stride, int n) -> Staged {
         Staged r;
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
             const int item = tid + it * NT;
             const int tok = item >> 2, c8 = (item & 3) * 8;
-            const int safe = tok < NM ? tok : NM - 1;
-            const u32x4 aw = *reinterpret_cast<const u32x4 *>(a + ((int64_t)env * NM + safe) * a_stride + head * kSbDh + c8);
-            const u32x4 bw = *reinterpret_cast<const u32x4 *>(b + ((int64_t)env * NM + safe) * b_stride + head * kSbDh + c8);
-            r.a[it] = tok < NM ? aw : zero4;
-            r.b[it] = tok < NM ? bw : zero4;
+            const int safe = tok < n ? tok : n - 1;
+            const u32x4 aw = *reinterpret_cast<const u32x4 *>(a + ((int64_t)env * n + safe) * a_stride + head * kSbDh + c8);
+            const u32x4 bw = *reinterpret_cast<const u32x4 *>(b + ((int64_t)env * n + safe) * b_stride + head * kSbDh + c8);
+            r.a[it] = tok < n ? aw : zero4;
+            r.b[it] = tok < n ? bw : zero4;
         }
         return r;
     };
@@ -329,37 +336,48 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
         for (int e = 0; e < 8; ++e) r[e] = (__bf16)x[8 * t + e];
         return r;
     };
-    // a (32 channels x 32 tokens) accumulator to the rows of dqkv: lane = token, rows = channels 8i + 4*half + j
-    auto store_grad = [&](const f32x16 &acc, int tok, int third) {
-        if (tok >= NM) return;
-        uint16_t *dst = dqkv + ((int64_t)env * NM + tok) * 3 * D + third * D + head * kSbDh + 4 * half;
+    // a (32 channels x 32 tokens) accumulator to rows of a gradient tensor: lane = token, rows = channels 8i + 4*half + j
+    auto store_grad = [&](const f32x16 &acc, uint16_t *base, int64_t row_stride, int tok, int n) {
+        if (tok >= n) return;
+        uint16_t *dst = base + ((int64_t)env * n + tok) * row_stride + head * kSbDh + 4 * half;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             *reinterpret_cast<u32x2 *>(dst + 8 * i) = u32x2{pack_bf16x2(acc[4 * i], acc[4 * i + 1]), pack_bf16x2(acc[4 * i + 2], acc[4 * i + 3])};
     };
 
     // ---- every global load of the kernel ----
-    const uint16_t *qp = qkv, *kp = qkv + D, *vp = qkv + 2 * D;
-    const int own = wave * 32 + m;
-    const int own_safe = own < NM ? own : NM - 1;
-    const int64_t own_row = (int64_t)env * NM + own_safe;
-    const int64_t own_q = own_row * qkv_row_stride + head * kSbDh + half * 8, own_o = own_row * D + head * kSbDh + half * 8;
+    const int own = wave * 32 + m;  // this lane's query in pass 1, its key in pass 2
+    const int64_t q_row = (int64_t)env * NQ + (own < NQ ? own : NQ - 1);
+    const int64_t k_row = (int64_t)env * NK + (own < NK ? own : NK - 1);
+    const int64_t own_q = q_row * q_row_stride + head * kSbDh + half * 8, own_o = q_row * D + head * kSbDh + half * 8;
+    const int64_t own_k = k_row * kv_row_stride + head * kSbDh + half * 8;
     bool any_live = false, my_live = false;
     if (tid < CAP) {  // CAP <= NT
-        my_live = tid < NM && (alive == nullptr || alive[(int64_t)env * NM + tid] != 0);
+        my_live = tid < NK && (alive == nullptr || alive[(int64_t)env * NK + tid] != 0);
         any_live = my_live;
     }
-    const Staged kv_in = stage_load(kp, qkv_row_stride, vp, qkv_row_stride);
-    u32x4 w0 = *reinterpret_cast<const u32x4 *>(qp + own_q), w1 = *reinterpret_cast<const u32x4 *>(qp + own_q + 16);
+    const Staged kv_in = stage_load(k, kv_row_stride, v, kv_row_stride, NK);
+    u32x4 w0 = *reinterpret_cast<const u32x4 *>(q + own_q), w1 = *reinterpret_cast<const u32x4 *>(q + own_q + 16);
     u32x4 g0 = *reinterpret_cast<const u32x4 *>(dout + own_o), g1 = *reinterpret_cast<const u32x4 *>(dout + own_o + 16);
     const Row8 o0 = load8(out + own_o), o1 = load8(out + own_o + 16);
-    u32x4 kw0 = *reinterpret_cast<const u32x4 *>(kp + own_q), kw1 = *reinterpret_cast<const u32x4 *>(kp + own_q + 16);
-    u32x4 vw0 = *reinterpret_cast<const u32x4 *>(vp + own_q), vw1 = *reinterpret_cast<const u32x4 *>(vp + own_q + 16);
-    const Staged qd_in = stage_load(qp, qkv_row_stride, dout, D);
+    u32x4 kw0 = *reinterpret_cast<const u32x4 *>(k + own_k), kw1 = *reinterpret_cast<const u32x4 *>(k + own_k + 16);
+    u32x4 vw0 = *reinterpret_cast<const u32x4 *>(v + own_k), vw1 = *reinterpret_cast<const u32x4 *>(v + own_k + 16);
+    const Staged qd_in = stage_load(q, q_row_stride, dout, D, NQ);
 
     // ---- live keys ----
-    const bool uniform = __syncthreads_or(any_live ? 1 : 0) == 0;
-    if (tid < CAP) s_bias[tid] = (uniform ? tid < NM : my_live) ? 0.0f : -INFINITY;
+    const bool none_live = __syncthreads_or(any_live ? 1 : 0) == 0;
+    if (CROSS && none_live) {
+        // the forward gated this environment off: nothing depends on its inputs
+        const f32x16 z16 = {0.0f};
+        if (wave < nqb) store_grad(z16, dq_out, dq_row_stride, own, NQ);
+        if (wave < nkb) {
+            store_grad(z16, dk_out, dkv_row_stride, own, NK);
+            store_grad(z16, dv_out, dkv_row_stride, own, NK);
+        }
+        return;
+    }
+    const bool uniform = none_live;  // self-attention without a live key: equal weights over all keys
+    if (tid < CAP) s_bias[tid] = (uniform ? tid < NK : my_live) ? 0.0f : -INFINITY;
     stage_store(kv_in, true, false);
     __syncthreads();
 
@@ -377,70 +395,73 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
         for (int e = 0; e < 8; ++e) d = fmaf(a0.v[e], o0.v[e], fmaf(a1.v[e], o1.v[e], d));
         delta = d + __shfl_xor(d, 32);
     }
-    if (own >= NM) w0 = w1 = g0 = g1 = zero4, delta = 0.0f;  // padding queries: nothing flows through them
+    if (own >= NQ) w0 = w1 = g0 = g1 = zero4, delta = 0.0f;  // padding queries: nothing flows through them
     const bf16x8 qs0 = __builtin_bit_cast(bf16x8, uniform ? zero4 : w0), qs1 = __builtin_bit_cast(bf16x8, uniform ? zero4 : w1);
     const bf16x8 gb0 = __builtin_bit_cast(bf16x8, g0), gb1 = __builtin_bit_cast(bf16x8, g1);
 
-    auto scores_t = [&](int kb) -> f32x16 {
-        f32x16 z;
+    if (wave < nqb) {
+        auto scores_t = [&](int kb) -> f32x16 {
+            f32x16 z;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const f32x4 b4 = *reinterpret_cast<const f32x4 *>(s_bias + kb * 32 + 8 * i + 4 * half);
-            z[4 * i] = b4.x, z[4 * i + 1] = b4.y, z[4 * i + 2] = b4.z, z[4 * i + 3] = b4.w;
+            for (int i = 0; i < 4; ++i) {
+                const f32x4 b4 = *reinterpret_cast<const f32x4 *>(s_bias + kb * 32 + 8 * i + 4 * half);
+                z[4 * i] = b4.x, z[4 * i + 1] = b4.y, z[4 * i + 2] = b4.z, z[4 * i + 3] = b4.w;
+            }
+            bf16x8 k0, k1;
+            row_operand(s_rows[0], kb * 32 + m, k0, k1);
+            z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k0, qs0, z, 0, 0, 0);
+            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(k1, qs1, z, 0, 0, 0);
+        };
+        float mx = -INFINITY;
+        for (int kb = 0; kb < nkb; ++kb) {
+            const f32x16 z = scores_t(kb);
+#pragma unroll
+            for (int vv = 0; vv < 16; ++vv) mx = fmaxf(mx, z[vv]);
         }
-        bf16x8 k0, k1;
-        row_operand(s_rows[0], kb * 32 + m, k0, k1);
-        z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k0, qs0, z, 0, 0, 0);
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(k1, qs1, z, 0, 0, 0);
-    };
-    float mx = -INFINITY;
-    for (int kb = 0; kb < NB; ++kb) {
-        const f32x16 z = scores_t(kb);
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float mc = mx * c;
+        float sum = 0.0f;
+        for (int kb = 0; kb < nkb; ++kb) {
+            const f32x16 z = scores_t(kb);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float mc = mx * c;
-    float sum = 0.0f;
-    for (int kb = 0; kb < NB; ++kb) {
-        const f32x16 z = scores_t(kb);
-#pragma unroll
-        for (int v = 0; v < 16; ++v) sum += __builtin_amdgcn_exp2f(fmaf(z[v], c, -mc));
-    }
-    sum += __shfl_xor(sum, 32);
-    const float lse = mc + __builtin_amdgcn_logf(sum);  // log2 of the sum of exp2(z c)
-    if (half == 0) s_lse[own] = lse, s_delta[own] = delta;
+            for (int vv = 0; vv < 16; ++vv) sum += __builtin_amdgcn_exp2f(fmaf(z[vv], c, -mc));
+        }
+        sum += __shfl_xor(sum, 32);
+        const float lse = mc + __builtin_amdgcn_logf(sum);  // log2 of the sum of exp2(z c)
+        if (half == 0) s_lse[own] = lse, s_delta[own] = delta;
 
-    f32x16 dq = {0.0f};
-    for (int kb = 0; kb < NB; ++kb) {
-        const f32x16 z = scores_t(kb);
-        bf16x8 v0, v1;
-        row_operand(s_rows[1], kb * 32 + m, v0, v1);
-        f32x16 dp = {0.0f};
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, gb0, dp, 0, 0, 0);
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, gb1, dp, 0, 0, 0);
-        float ds[16];
+        f32x16 dq = {0.0f};
+        for (int kb = 0; kb < nkb; ++kb) {
+            const f32x16 z = scores_t(kb);
+            bf16x8 v0, v1;
+            row_operand(s_rows[1], kb * 32 + m, v0, v1);
+            f32x16 dp = {0.0f};
+            dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, gb0, dp, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, gb1, dp, 0, 0, 0);
+            float ds[16];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) ds[v] = __builtin_amdgcn_exp2f(fmaf(z[v], c, -lse)) * (dp[v] - delta) * scale;
+            for (int vv = 0; vv < 16; ++vv) ds[vv] = __builtin_amdgcn_exp2f(fmaf(z[vv], c, -lse)) * (dp[vv] - delta) * scale;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_operand(s_tr[0], kb, t), pack8(ds, t), dq, 0, 0, 0);
+            for (int t = 0; t < 2; ++t) dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_operand(s_tr[0], kb, t), pack8(ds, t), dq, 0, 0, 0);
+        }
+        store_grad(dq, dq_out, dq_row_stride, own, NQ);
     }
-    store_grad(dq, own, 0);
     __syncthreads();  // K, V and K^T are no longer needed; L and delta of every query are in LDS
 
     // ---- pass 2: this wave's keys ----
     stage_store(qd_in, true, true);
     const float col_bias = s_bias[own];
-    if (own >= NM) kw0 = kw1 = vw0 = vw1 = zero4;
+    if (own >= NK) kw0 = kw1 = vw0 = vw1 = zero4;
     const bf16x8 ks0 = __builtin_bit_cast(bf16x8, uniform ? zero4 : kw0), ks1 = __builtin_bit_cast(bf16x8, uniform ? zero4 : kw1);
     const bf16x8 vb0 = __builtin_bit_cast(bf16x8, vw0), vb1 = __builtin_bit_cast(bf16x8, vw1);
     __syncthreads();
+    if (wave >= nkb) return;
 
     f32x16 dk = {0.0f}, dv = {0.0f};
-    for (int qb = 0; qb < NB; ++qb) {
+    for (int qb = 0; qb < nqb; ++qb) {
         f32x16 z;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) z[v] = col_bias;
+        for (int vv = 0; vv < 16; ++vv) z[vv] = col_bias;
         bf16x8 a0, a1;
         row_operand(s_rows[0], qb * 32 + m, a0, a1);
         z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, ks0, z, 0, 0, 0);
@@ -456,9 +477,9 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
             const f32x4 d4 = *reinterpret_cast<const f32x4 *>(s_delta + qb * 32 + 8 * i + 4 * half);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int v = 4 * i + j;
-                p[v] = __builtin_amdgcn_exp2f(fmaf(z[v], c, -l4[j]));
-                ds[v] = p[v] * (dp[v] - d4[j]) * scale;
+                const int vv = 4 * i + j;
+                p[vv] = __builtin_amdgcn_exp2f(fmaf(z[vv], c, -l4[j]));
+                ds[vv] = p[vv] * (dp[vv] - d4[j]) * scale;
             }
         }
 #pragma unroll
@@ -467,20 +488,42 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
             dv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_operand(s_tr[1], qb, t), pack8(p, t), dv, 0, 0, 0);
         }
     }
-    store_grad(dk, own, 1);
-    store_grad(dv, own, 2);
+    store_grad(dk, dk_out, dkv_row_stride, own, NK);
+    store_grad(dv, dv_out, dkv_row_stride, own, NK);
 }
 
-template <int NB>
-static int launch_sdpa_bwd_mfma(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, const void *out, const void *dout,
-                                void *dqkv, int64_t B, int NM, int H, hipStream_t stream)
+template <int NB, bool CROSS>
+static int launch_sdpa_bwd_mfma(const void *q, int64_t q_row_stride, const void *k, const void *v, int64_t kv_row_stride,
+                                const uint8_t *alive, const void *out, const void *dout, void *dq, int64_t dq_row_stride, void *dk,
+                                void *dv, int64_t dkv_row_stride, int64_t B, int NQ, int NK, int H, hipStream_t stream)
 {
     const int64_t groups = (B * H + 7) / 8 * 8;  // a multiple of 8: the XCD mapping deals whole rounds
     if (groups > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<NB>), dim3((unsigned)groups), dim3(kWave * NB), 0, stream, (const uint16_t *)qkv,
-                       qkv_row_stride, alive, (const uint16_t *)out, (const uint16_t *)dout, (uint16_t *)dqkv, (int)B, NM, H,
-                       1.0f / sqrtf((float)kSbDh));
+    hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<NB, CROSS>), dim3((unsigned)groups), dim3(kWave * NB), 0, stream, (const uint16_t *)q,
+                       q_row_stride, (const uint16_t *)k, (const uint16_t *)v, kv_row_stride, alive, (const uint16_t *)out,
+                       (const uint16_t *)dout, (uint16_t *)dq, dq_row_stride, (uint16_t *)dk, (uint16_t *)dv, dkv_row_stride, (int)B,
+                       NQ, NK, H, 1.0f / sqrtf((float)kSbDh));
     return (int)hipGetLastError();
+}
+
+template <bool CROSS>
+static int dispatch_sdpa_bwd_mfma(const void *q, int64_t q_row_stride, const void *k, const void *v, int64_t kv_row_stride,
+                                  const uint8_t *alive, const void *out, const void *dout, void *dq, int64_t dq_row_stride, void *dk,
+                                  void *dv, int64_t dkv_row_stride, int64_t B, int NQ, int NK, int H, hipStream_t s)
+{
+    const int nb = ((NQ > NK ? NQ : NK) + 31) / 32;
+#define BNB_SBM(NBV) \
+    return launch_sdpa_bwd_mfma<NBV, CROSS>(q, q_row_stride, k, v, kv_row_stride, alive, out, dout, dq, dq_row_stride, dk, dv, \
+                                            dkv_row_stride, B, NQ, NK, H, s)
+    switch (nb) {
+        case 1: BNB_SBM(1);
+        case 2: BNB_SBM(2);
+        case 3: BNB_SBM(3);
+        case 4: BNB_SBM(4);
+        case 5: BNB_SBM(5);
+        default: return BNB_ERR_UNSUPPORTED;
+    }
+#undef BNB_SBM
 }
 
 }  // namespace bnb
@@ -505,13 +548,11 @@ extern "C" int bnb_sdpa_masked_bwd_path(const void *qkv, int64_t qkv_row_stride,
     if (path != BNB_SDPA_PATH_AUTO && path != BNB_SDPA_PATH_VALU && path != BNB_SDPA_PATH_MFMA) return BNB_ERR_BAD_SHAPE;
     if (path == BNB_SDPA_PATH_MFMA && !mfma) return BNB_ERR_UNSUPPORTED;
     if (mfma && (path == BNB_SDPA_PATH_MFMA || (path == BNB_SDPA_PATH_AUTO && NM > kSbMfmaFrom))) {
-        switch ((NM + 31) / 32) {
-            case 1: return launch_sdpa_bwd_mfma<1>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
-            case 2: return launch_sdpa_bwd_mfma<2>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
-            case 3: return launch_sdpa_bwd_mfma<3>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
-            case 4: return launch_sdpa_bwd_mfma<4>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
-            default: return launch_sdpa_bwd_mfma<5>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
-        }
+        const uint16_t *p = (const uint16_t *)qkv;
+        const int D = H * dh;
+        uint16_t *g = (uint16_t *)dqkv;
+        return dispatch_sdpa_bwd_mfma<false>(p, qkv_row_stride, p + D, p + 2 * D, qkv_row_stride, alive, out, dout, g, 3 * (int64_t)D,
+                                             g + D, g + 2 * D, 3 * (int64_t)D, B, NM, NM, H, s);
     }
     if (!small) return BNB_ERR_UNSUPPORTED;
     if (dtype == BNB_BF16) return launch_sdpa_bwd<uint16_t>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
@@ -522,4 +563,25 @@ extern "C" int bnb_sdpa_masked_bwd(const void *qkv, int64_t qkv_row_stride, cons
                                    const void *dout, void *dqkv, int64_t B, int NM, int H, int dh, int dtype, void *stream)
 {
     return bnb_sdpa_masked_bwd_path(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, dh, dtype, BNB_SDPA_PATH_AUTO, stream);
+}
+
+extern "C" int bnb_sdpa_cross_bwd(const void *q, int64_t q_row_stride, int NQ, const void *kv, int64_t kv_row_stride, int NK,
+                                  const uint8_t *key_mask, const void *out, const void *dout, void *dq, void *dkv, int64_t B,
+                                  int H, int dh, int dtype, void *stream)
+{
+    using namespace bnb;
+    if (B < 0 || NQ < 1 || NK < 1 || H < 1 || dh < 1) return BNB_ERR_BAD_SHAPE;
+    if (dtype != BNB_BF16 || dh != kSbDh || NQ > 160 || NK > 160) return BNB_ERR_UNSUPPORTED;
+    const int D = H * dh;
+    if (q_row_stride < D || kv_row_stride < 2 * (int64_t)D) return BNB_ERR_BAD_SHAPE;
+    if (B == 0) return 0;
+    if (!q || !kv || !out || !dout || !dq || !dkv) return BNB_ERR_NULL_POINTER;
+    if (!aligned16(q) || !aligned16(kv) || !aligned16(out) || !aligned16(dout) || !aligned16(dq) || !aligned16(dkv) ||
+        (q_row_stride % 8) != 0 || (kv_row_stride % 8) != 0)
+        return BNB_ERR_MISALIGNED;
+    if (B > 0x7fffffffLL / H) return BNB_ERR_UNSUPPORTED;
+    const uint16_t *kp = (const uint16_t *)kv;
+    uint16_t *g = (uint16_t *)dkv;
+    return dispatch_sdpa_bwd_mfma<true>(q, q_row_stride, kp, kp + D, kv_row_stride, key_mask, out, dout, dq, D, g, g + D,
+                                        2 * (int64_t)D, B, NQ, NK, H, (hipStream_t)stream);
 }

@@ -250,6 +250,73 @@ def sdpa_cross(
     return out
 
 
+def sdpa_cross_train_supported(qkv: torch.Tensor, kv: torch.Tensor, n_heads: int) -> bool:
+    """Whether ``sdpa_cross_train`` covers these shapes: what ``sdpa_cross`` covers with at most 160 keys."""
+    return cross_supported(qkv, kv, n_heads) and kv.shape[1] <= 160 and kv.dim() == 3 and qkv.dim() == 3
+
+
+def sdpa_cross_bwd(qkv, kv, key_mask, n_heads, out, dout) -> tuple[torch.Tensor, torch.Tensor]:
+    """Gradients ``(dq (B, NQ, D), dkv (B, NK, 2D))`` of ``sdpa_cross`` (without accumulator) from its
+    result and that result's gradient; an environment without an active key gets zeros."""
+    B, NQ, D3 = qkv.shape
+    D = D3 // 3
+    NK = kv.shape[1]
+    for name, t in (("qkv", qkv), ("kv", kv), ("out", out), ("dout", dout)):
+        _need_device(t, name)
+        if t.dtype != torch.bfloat16:
+            raise TypeError(f"{name} must be bfloat16")
+    if kv.shape != (B, NK, 2 * D) or out.shape != (B, NQ, D) or dout.shape != (B, NQ, D):
+        raise ValueError("kv must be (B, NK, 2D), out and dout (B, NQ, D)")
+    if B and NQ and (qkv.stride(-1) != 1 or (B > 1 and qkv.stride(0) != NQ * qkv.stride(1))):
+        qkv = qkv.contiguous()
+    if B and (kv.stride(-1) != 1 or (B > 1 and kv.stride(0) != NK * kv.stride(1))):
+        kv = kv.contiguous()
+    out, dout = out.contiguous(), dout.contiguous()
+    mask_ptr = None
+    if key_mask is not None:
+        if key_mask.shape != (B, NK) or key_mask.dtype not in (torch.bool, torch.uint8):
+            raise ValueError(f"key_mask must be a bool {(B, NK)} tensor")
+        key_mask = key_mask.contiguous()
+        mask_ptr = key_mask.data_ptr()
+    dq = torch.empty((B, NQ, D), dtype=torch.bfloat16, device=qkv.device)
+    dkv = torch.empty((B, NK, 2 * D), dtype=torch.bfloat16, device=qkv.device)
+    if B:
+        with torch.cuda.device(qkv.device):
+            rc = _native.load().bnb_sdpa_cross_bwd(qkv.data_ptr(), qkv.stride(1), NQ, kv.data_ptr(), kv.stride(1), NK, mask_ptr,
+                                                   out.data_ptr(), dout.data_ptr(), dq.data_ptr(), dkv.data_ptr(), B, n_heads,
+                                                   D // n_heads, _native.BF16, _stream())
+        _native.check(rc, "bnb_sdpa_cross_bwd")
+    return dq, dkv
+
+
+class _SdpaCrossTrain(torch.autograd.Function):
+    """``sdpa_cross`` (the read's own result, nothing accumulated) with its backward kernel."""
+
+    @staticmethod
+    def forward(ctx, qkv, kv, key_mask, n_heads):
+        with torch.no_grad():
+            out = sdpa_cross(qkv, kv, key_mask, n_heads)
+        ctx.save_for_backward(qkv, kv, out)
+        ctx.key_mask = key_mask
+        ctx.n_heads = n_heads
+        return out
+
+    @staticmethod
+    @_outside_autocast
+    def backward(ctx, dout):
+        qkv, kv, out = ctx.saved_tensors
+        dq, dkv = sdpa_cross_bwd(qkv, kv, ctx.key_mask, ctx.n_heads, out, dout.to(torch.bfloat16))
+        dqkv = torch.zeros_like(qkv)
+        dqkv[..., : dq.shape[-1]] = dq
+        return dqkv, dkv, None, None
+
+
+def sdpa_cross_train(qkv: torch.Tensor, kv: torch.Tensor, key_mask: torch.Tensor | None, n_heads: int) -> torch.Tensor:
+    """Differentiable ``sdpa_cross``: the entity queries' read of a second key/value set, (B, NQ, D)."""
+    with torch.autocast("cuda", enabled=False):
+        return _SdpaCrossTrain.apply(qkv, kv, key_mask, n_heads)
+
+
 def rglru_step(
     x: torch.Tensor,
     gates_pre: torch.Tensor,

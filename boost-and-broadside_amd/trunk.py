@@ -297,7 +297,10 @@ class TransformerBlock(nn.Module):
                 if isinstance(bullet_mask, ops.CompactRows):
                     bullet_mask = bullet_mask.mask
                 kv = _project(self.kv_bullet, _train_norm(self.norm_bullet, bullets)[1])
-                merged = merged + self._bullet_read(qkv, kv, bullet_mask)
+                if _TRAIN_KERNELS and ops.sdpa_cross_train_supported(qkv, kv, self.n_heads):
+                    merged = merged + ops.sdpa_cross_train(qkv, kv, bullet_mask, self.n_heads)
+                else:
+                    merged = merged + self._bullet_read(qkv, kv, bullet_mask)
             return _project(self.out_proj, merged)
         try:
             merged = ops.sdpa_masked(qkv, alive_mask, self.n_heads)  # (B, N, D) head-major

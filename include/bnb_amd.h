@@ -289,6 +289,20 @@ int bnb_sdpa_masked_bwd_path(const void *qkv, int64_t qkv_row_stride, const uint
                              void *stream);
 
 /*
+ * Backward of bnb_sdpa_cross_fwd called without accumulator (autograd through the bullet read,
+ * models/yemong/attention.py:149-166, in the PPO update): bf16, dh == 32, NQ <= 160, NK <= 160.
+ *
+ *   q, kv, key_mask  as passed to the forward (q = the packed entity projection, only its first
+ *                    H*dh columns are read; kv = [K | V] rows)
+ *   out, dout        (B, NQ, H*dh) contiguous: the read's own result and its gradient
+ *   dq               (B, NQ, H*dh) contiguous;  dkv (B, NK, 2*H*dh) contiguous
+ * An environment without an active key was gated off in the forward: its gradients are zero.
+ */
+int bnb_sdpa_cross_bwd(const void *q, int64_t q_row_stride, int NQ, const void *kv, int64_t kv_row_stride, int NK,
+                       const uint8_t *key_mask, const void *out, const void *dout, void *dq, void *dkv,
+                       int64_t B, int H, int dh, int dtype, void *stream);
+
+/*
  * RMSNorm backward:  y = x * rsqrt(mean(x^2) + eps) * weight
  *   dx[r] = rstd * (dy[r] * weight) - x[r] * rstd^3 * mean(dy[r] * weight * x[r])  (+ grad_sum[r])
  *   dw    = sum_r dy[r] * x[r] * rstd

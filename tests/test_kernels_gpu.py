@@ -1785,3 +1785,61 @@ def test_sdpa_masked_bwd_on_the_matrix_cores_matches_autograd_of_the_oracle(B, N
     if NM <= 32:  # the two kernels against each other
         other = ops.sdpa_masked_bwd(qkv.to(DEV), mask, H, out, up.to(DEV), path="valu")
         assert max_rel(dqkv.float().cpu(), other.float().cpu()) <= BF16_TOL
+
+
+# ------------------------------------------------------------------ bullet read backward
+
+
+@pytest.mark.parametrize("B,NQ,NK,H", [(3, 12, 80, 4), (5, 23, 160, 4), (4, 1, 1, 4), (2, 84, 33, 4), (3, 160, 10, 4), (6, 12, 31, 2),
+                                       (200, 12, 80, 4)])
+@pytest.mark.parametrize("p_live", [1.0, 0.25, 0.0])
+def test_sdpa_cross_bwd_matches_autograd_of_the_oracle(B, NQ, NK, H, p_live):
+    D = 32 * H
+    g = torch.Generator().manual_seed(B * 13 + NQ + NK)
+    qkv = (1.2 * torch.randn(B, NQ, 3 * D, generator=g)).bfloat16()
+    kv = (1.2 * torch.randn(B, NK, 2 * D, generator=g)).bfloat16()
+    mask = None if p_live == 1.0 else torch.rand(B, NK, generator=g) < p_live
+    if mask is not None and p_live > 0 and B > 2:
+        mask[1] = False  # an environment without an active bullet among active ones
+        mask[0, 0] = True
+    up = torch.randn(B, NQ, D, generator=g).bfloat16()
+    xq = qkv.double().requires_grad_()
+    xkv = kv.double().requires_grad_()
+    ref = torch_ref.bullet_read(xq, xkv, mask, H)
+    (ref * up.double()).sum().backward()
+    dmask = None if mask is None else mask.to(DEV)
+    out = ops.sdpa_cross(qkv.to(DEV), kv.to(DEV), dmask, H)
+    dq, dkv = ops.sdpa_cross_bwd(qkv.to(DEV), kv.to(DEV), dmask, H, out, up.to(DEV))
+    torch.cuda.synchronize()
+    assert max_rel(out.float().cpu().double(), ref.detach()) <= BF16_TOL or not ref.detach().any()
+    for name, got, want in (("dQ", dq, xq.grad[..., :D]), ("dK", dkv[..., :D], xkv.grad[..., :D]), ("dV", dkv[..., D:], xkv.grad[..., D:])):
+        if want.abs().max() < 1e-12:  # gated-off environments only, or a single key
+            assert got.float().abs().max() <= 1e-6 * max(1.0, float(xkv.grad.abs().max())), name
+            continue
+        assert max_rel(got.float().cpu().double(), want) <= BF16_TOL, name
+    assert not xq.grad[..., D:].any()  # the read never touches the entity keys and values
+    if mask is not None:
+        off = ~mask.any(dim=1)
+        assert not dq.cpu()[off].any() and not dkv.cpu()[off].any()  # gated off: exactly nothing
+        dead = ~mask & mask.any(dim=1, keepdim=True)
+        assert not dkv.cpu()[dead].any()
+    again = ops.sdpa_cross_bwd(qkv.to(DEV), kv.to(DEV), dmask, H, out, up.to(DEV))
+    assert torch.equal(dq, again[0]) and torch.equal(dkv, again[1])
+
+
+def test_sdpa_cross_train_is_differentiable():
+    B, NQ, NK, H, D = 9, 12, 80, 4, 128
+    g = torch.Generator().manual_seed(2)
+    qkv = torch.randn(B, NQ, 3 * D, generator=g).bfloat16().to(DEV).requires_grad_()
+    kv = torch.randn(B, NK, 2 * D, generator=g).bfloat16().to(DEV).requires_grad_()
+    mask = (torch.rand(B, NK, generator=g) < 0.3).to(DEV)
+    up = torch.randn(B, NQ, D, generator=g).to(DEV)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = ops.sdpa_cross_train(qkv, kv, mask, H)
+        (out.float() * up).sum().backward()  # backward called inside autocast on purpose
+    xq = qkv.detach().cpu().double().requires_grad_()
+    xkv = kv.detach().cpu().double().requires_grad_()
+    (torch_ref.bullet_read(xq, xkv, mask.cpu(), H) * up.bfloat16().cpu().double()).sum().backward()
+    assert max_rel(qkv.grad.float().cpu().double(), xq.grad) <= BF16_TOL
+    assert max_rel(kv.grad.float().cpu().double(), xkv.grad) <= BF16_TOL
+    assert not ops.sdpa_cross_train_supported(qkv, torch.zeros(B, 200, 2 * D, device=DEV, dtype=torch.bfloat16), H)
