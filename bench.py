@@ -721,6 +721,29 @@ def main():
             if not args.no_torch_baseline:
                 with trunk_module.library_update_path():
                     t_up_lib = timed_loop(update_step, 3, 2) / 3
+            # the same block reading the bullets in flight (the reference's shipped default: one bullet-reading
+            # attention sublayer per block, 10 slots per ship, a quarter of them live)
+            cfg_b = bnb.ModelConfig(d_model=D, n_heads=H, n_yemong_blocks=1, n_spatial_per_block=2, n_temporal_per_block=1,
+                                    n_bullet_cross_per_block=1)
+            torch.manual_seed(w.seed)
+            blk_b = bnb.YemongBlock(cfg_b).to(dev)
+            bul_u = torch.randn(Tu * Bu, Nu * 10, D, device=dev, generator=gen, requires_grad=True)
+            bm_u = torch.rand(Tu * Bu, Nu * 10, device=dev, generator=gen) < 0.25
+
+            def update_step_bullets(t):
+                blk_b.zero_grad(set_to_none=True)
+                bul_u.grad = None
+                with torch.enable_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+                    out_b = blk_b.sequence(xu, au, hu, cu, du, Nu, bul_u, bm_u)[0]
+                out_b.float().square().mean().backward()
+
+            t_upb = timed_loop(update_step_bullets, 3, 2) / 3
+            t_upb_lib = None
+            if not args.no_torch_baseline:
+                with trunk_module.library_update_path():
+                    t_upb_lib = timed_loop(update_step_bullets, 2, 1) / 2
+            del blk_b, bul_u, bm_u
+
             # the other update-path kernels at the same size, each against its algorithmic bytes
             def stream_leg(fn, nbytes, reps=8):
                 t = timed_loop(fn, reps, 3) / reps
@@ -777,6 +800,8 @@ def main():
             del pma_u, xs_u, tm_u, al_u, go_u
             result["update_path"] = {
                 "rows": Rw, "linear_wgrad": wg, "kernels": kern, "block_fwd_bwd_ms": t_up * 1e3,
+                "block_with_bullets_fwd_bwd_ms": t_upb * 1e3,
+                "block_with_bullets_fwd_bwd_library_ms": None if t_upb_lib is None else t_upb_lib * 1e3,
                 "team_pool_fwd_bwd_ms": t_pool_up * 1e3,
                 "team_pool_fwd_bwd_library_ms": None if t_pool_up_lib is None else t_pool_up_lib * 1e3,
                 "block_fwd_bwd_library_ms": None if t_up_lib is None else t_up_lib * 1e3,
@@ -784,7 +809,8 @@ def main():
                         "GEMM on the same operands; kernels = the norm, gelu-gate, attention and conv backward kernels at the "
                         "sizes of the block below; block = one YemongBlock (2 attention + 1 temporal sublayer), T = 128 x 256 "
                         "environments of 4v4, forward + backward under bf16 autocast, on the update-path kernels and with "
-                        "torch's own differentiable ops in their place (the recurrence keeps its kernels in both); team_pool = TeamPMA "
+                        "torch's own differentiable ops in their place (the recurrence keeps its kernels in both); block_with_bullets = "
+                        "the same with one attention sublayer reading 80 bullet slots per environment, 25 % live; team_pool = TeamPMA "
                         "forward + backward over the ships of the same rollout (32,768 environments x 8 ships), kernels and library",
             }
             del blk, xu, au, hu, cu, du
