@@ -42,6 +42,7 @@ SIGNATURES = {
     "bnb_gelu_mul_bwd": (_i, [_vp, _i, _i64, _vp, _i, _i64, _vp, _i, _vp, _i64, _vp, _i64, _i64, _i, _vp]),
     "bnb_sdpa_masked_bwd": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp]),
     "bnb_sdpa_cross_bwd": (_i, [_vp, _i64, _i, _vp, _i64, _i, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
+    "bnb_sdpa_cross_ranges_bwd": (_i, [_vp, _i64, _i, _vp, _i64, _vp, _i64, _i, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
     "bnb_sdpa_masked_bwd_path": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _vp]),
     "bnb_rmsnorm_bwd_blocks": (_i, [_i64, _i]),
     "bnb_rmsnorm_bwd": (_i, [_vp, _i64, _vp, _i, _i64, _vp, _f, _vp, _vp, _vp, _vp, _i, _vp, _i64, _i, _vp]),

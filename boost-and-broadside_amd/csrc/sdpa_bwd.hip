@@ -259,9 +259,10 @@ constexpr int kMbPitch = kSbDh + 8;  // halfs per token row in LDS (80 bytes: 16
 template <int NB, bool CROSS>
 __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
     const uint16_t *__restrict__ q, int64_t q_row_stride, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
-    int64_t kv_row_stride, const uint8_t *__restrict__ alive, const uint16_t *__restrict__ out,
-    const uint16_t *__restrict__ dout, uint16_t *__restrict__ dq_out, int64_t dq_row_stride, uint16_t *__restrict__ dk_out,
-    uint16_t *__restrict__ dv_out, int64_t dkv_row_stride, int B, int NQ, int NK, int H, float scale)
+    int64_t kv_row_stride, const uint8_t *__restrict__ alive, const int32_t *__restrict__ ranges, int64_t kv_capacity,
+    const uint16_t *__restrict__ out, const uint16_t *__restrict__ dout, uint16_t *__restrict__ dq_out, int64_t dq_row_stride,
+    uint16_t *__restrict__ dk_out, uint16_t *__restrict__ dv_out, int64_t dkv_row_stride, int B, int NQ, int NK_all, int H,
+    float scale)
 {
     constexpr int CAP = NB * 32;
     constexpr int TP = CAP + 4;  // halfs per row of a transposed copy
@@ -281,6 +282,16 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
     const int m = lane & 31, half = lane >> 5;
     const float c = scale * 1.4426950408889634f;
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    // keys of this environment: rows env*NK_all .. of the key/value buffer, or with `ranges` (a list of the
+    // live rows only, CROSS) rows ranges[env] .. ranges[env+1]-1, all of them live
+    int64_t k_base = (int64_t)env * NK_all;
+    int NK = NK_all;
+    if (ranges != nullptr) {
+        k_base = ranges[env];
+        int64_t cnt = (int64_t)ranges[env + 1] - k_base;
+        if (cnt > kv_capacity - k_base) cnt = kv_capacity - k_base;
+        NK = cnt < 0 ? 0 : (cnt > CAP ? CAP : (int)cnt);
+    }
     const int nqb = (NQ + 31) >> 5, nkb = (NK + 31) >> 5;  // <= NB
 
     // token-major and channel-major copies of two (n, 32) operands; rows past n are zero.  The loads of
@@ -288,15 +299,16 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
     struct Staged {
         u32x4 a[2], b[2];
     };
-    auto stage_load = [&](const uint16_t *a, int64_t a_stride, const uint16_t *b, int64_t b_stride, int n) -> Staged {
+    auto stage_load = [&](const uint16_t *a, int64_t a_stride, const uint16_t *b, int64_t b_stride, int64_t base, int n) -> Staged {
         Staged r;
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
             const int item = tid + it * NT;
             const int tok = item >> 2, c8 = (item & 3) * 8;
-            const int safe = tok < n ? tok : n - 1;
-            const u32x4 aw = *reinterpret_cast<const u32x4 *>(a + ((int64_t)env * n + safe) * a_stride + head * kSbDh + c8);
-            const u32x4 bw = *reinterpret_cast<const u32x4 *>(b + ((int64_t)env * n + safe) * b_stride + head * kSbDh + c8);
+            const int safe = tok < n ? tok : (n > 0 ? n - 1 : 0);
+            const int64_t row = n > 0 ? base + safe : 0;  // an empty range reads row 0 of the buffer and discards it
+            const u32x4 aw = *reinterpret_cast<const u32x4 *>(a + row * a_stride + head * kSbDh + c8);
+            const u32x4 bw = *reinterpret_cast<const u32x4 *>(b + row * b_stride + head * kSbDh + c8);
             r.a[it] = tok < n ? aw : zero4;
             r.b[it] = tok < n ? bw : zero4;
         }
@@ -337,9 +349,9 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
         return r;
     };
     // a (32 channels x 32 tokens) accumulator to rows of a gradient tensor: lane = token, rows = channels 8i + 4*half + j
-    auto store_grad = [&](const f32x16 &acc, uint16_t *base, int64_t row_stride, int tok, int n) {
+    auto store_grad = [&](const f32x16 &acc, uint16_t *base, int64_t row_stride, int64_t first_row, int tok, int n) {
         if (tok >= n) return;
-        uint16_t *dst = base + ((int64_t)env * n + tok) * row_stride + head * kSbDh + 4 * half;
+        uint16_t *dst = base + (first_row + tok) * row_stride + head * kSbDh + 4 * half;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             *reinterpret_cast<u32x2 *>(dst + 8 * i) = u32x2{pack_bf16x2(acc[4 * i], acc[4 * i + 1]), pack_bf16x2(acc[4 * i + 2], acc[4 * i + 3])};
@@ -347,32 +359,33 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
 
     // ---- every global load of the kernel ----
     const int own = wave * 32 + m;  // this lane's query in pass 1, its key in pass 2
-    const int64_t q_row = (int64_t)env * NQ + (own < NQ ? own : NQ - 1);
-    const int64_t k_row = (int64_t)env * NK + (own < NK ? own : NK - 1);
+    const int64_t q_base = (int64_t)env * NQ;
+    const int64_t q_row = q_base + (own < NQ ? own : NQ - 1);
+    const int64_t k_row = NK > 0 ? k_base + (own < NK ? own : NK - 1) : 0;
     const int64_t own_q = q_row * q_row_stride + head * kSbDh + half * 8, own_o = q_row * D + head * kSbDh + half * 8;
     const int64_t own_k = k_row * kv_row_stride + head * kSbDh + half * 8;
     bool any_live = false, my_live = false;
     if (tid < CAP) {  // CAP <= NT
-        my_live = tid < NK && (alive == nullptr || alive[(int64_t)env * NK + tid] != 0);
+        my_live = tid < NK && (alive == nullptr || ranges != nullptr || alive[k_base + tid] != 0);
         any_live = my_live;
     }
-    const Staged kv_in = stage_load(k, kv_row_stride, v, kv_row_stride, NK);
+    const Staged kv_in = stage_load(k, kv_row_stride, v, kv_row_stride, k_base, NK);
     u32x4 w0 = *reinterpret_cast<const u32x4 *>(q + own_q), w1 = *reinterpret_cast<const u32x4 *>(q + own_q + 16);
     u32x4 g0 = *reinterpret_cast<const u32x4 *>(dout + own_o), g1 = *reinterpret_cast<const u32x4 *>(dout + own_o + 16);
     const Row8 o0 = load8(out + own_o), o1 = load8(out + own_o + 16);
     u32x4 kw0 = *reinterpret_cast<const u32x4 *>(k + own_k), kw1 = *reinterpret_cast<const u32x4 *>(k + own_k + 16);
     u32x4 vw0 = *reinterpret_cast<const u32x4 *>(v + own_k), vw1 = *reinterpret_cast<const u32x4 *>(v + own_k + 16);
-    const Staged qd_in = stage_load(q, q_row_stride, dout, D, NQ);
+    const Staged qd_in = stage_load(q, q_row_stride, dout, D, q_base, NQ);
 
     // ---- live keys ----
     const bool none_live = __syncthreads_or(any_live ? 1 : 0) == 0;
     if (CROSS && none_live) {
         // the forward gated this environment off: nothing depends on its inputs
         const f32x16 z16 = {0.0f};
-        if (wave < nqb) store_grad(z16, dq_out, dq_row_stride, own, NQ);
+        if (wave < nqb) store_grad(z16, dq_out, dq_row_stride, q_base, own, NQ);
         if (wave < nkb) {
-            store_grad(z16, dk_out, dkv_row_stride, own, NK);
-            store_grad(z16, dv_out, dkv_row_stride, own, NK);
+            store_grad(z16, dk_out, dkv_row_stride, k_base, own, NK);
+            store_grad(z16, dv_out, dkv_row_stride, k_base, own, NK);
         }
         return;
     }
@@ -444,7 +457,7 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
 #pragma unroll
             for (int t = 0; t < 2; ++t) dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_operand(s_tr[0], kb, t), pack8(ds, t), dq, 0, 0, 0);
         }
-        store_grad(dq, dq_out, dq_row_stride, own, NQ);
+        store_grad(dq, dq_out, dq_row_stride, q_base, own, NQ);
     }
     __syncthreads();  // K, V and K^T are no longer needed; L and delta of every query are in LDS
 
@@ -488,33 +501,35 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
             dv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr_operand(s_tr[1], qb, t), pack8(p, t), dv, 0, 0, 0);
         }
     }
-    store_grad(dk, dk_out, dkv_row_stride, own, NK);
-    store_grad(dv, dv_out, dkv_row_stride, own, NK);
+    store_grad(dk, dk_out, dkv_row_stride, k_base, own, NK);
+    store_grad(dv, dv_out, dkv_row_stride, k_base, own, NK);
 }
 
 template <int NB, bool CROSS>
 static int launch_sdpa_bwd_mfma(const void *q, int64_t q_row_stride, const void *k, const void *v, int64_t kv_row_stride,
-                                const uint8_t *alive, const void *out, const void *dout, void *dq, int64_t dq_row_stride, void *dk,
-                                void *dv, int64_t dkv_row_stride, int64_t B, int NQ, int NK, int H, hipStream_t stream)
+                                const uint8_t *alive, const int32_t *ranges, int64_t kv_capacity, const void *out, const void *dout,
+                                void *dq, int64_t dq_row_stride, void *dk, void *dv, int64_t dkv_row_stride, int64_t B, int NQ,
+                                int NK, int H, hipStream_t stream)
 {
     const int64_t groups = (B * H + 7) / 8 * 8;  // a multiple of 8: the XCD mapping deals whole rounds
     if (groups > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<NB, CROSS>), dim3((unsigned)groups), dim3(kWave * NB), 0, stream, (const uint16_t *)q,
-                       q_row_stride, (const uint16_t *)k, (const uint16_t *)v, kv_row_stride, alive, (const uint16_t *)out,
-                       (const uint16_t *)dout, (uint16_t *)dq, dq_row_stride, (uint16_t *)dk, (uint16_t *)dv, dkv_row_stride, (int)B,
+                       q_row_stride, (const uint16_t *)k, (const uint16_t *)v, kv_row_stride, alive, ranges, kv_capacity,
+                       (const uint16_t *)out, (const uint16_t *)dout, (uint16_t *)dq, dq_row_stride, (uint16_t *)dk, (uint16_t *)dv, dkv_row_stride, (int)B,
                        NQ, NK, H, 1.0f / sqrtf((float)kSbDh));
     return (int)hipGetLastError();
 }
 
 template <bool CROSS>
 static int dispatch_sdpa_bwd_mfma(const void *q, int64_t q_row_stride, const void *k, const void *v, int64_t kv_row_stride,
-                                  const uint8_t *alive, const void *out, const void *dout, void *dq, int64_t dq_row_stride, void *dk,
-                                  void *dv, int64_t dkv_row_stride, int64_t B, int NQ, int NK, int H, hipStream_t s)
+                                  const uint8_t *alive, const int32_t *ranges, int64_t kv_capacity, const void *out, const void *dout,
+                                  void *dq, int64_t dq_row_stride, void *dk, void *dv, int64_t dkv_row_stride, int64_t B, int NQ,
+                                  int NK, int H, hipStream_t s)
 {
     const int nb = ((NQ > NK ? NQ : NK) + 31) / 32;
 #define BNB_SBM(NBV) \
-    return launch_sdpa_bwd_mfma<NBV, CROSS>(q, q_row_stride, k, v, kv_row_stride, alive, out, dout, dq, dq_row_stride, dk, dv, \
-                                            dkv_row_stride, B, NQ, NK, H, s)
+    return launch_sdpa_bwd_mfma<NBV, CROSS>(q, q_row_stride, k, v, kv_row_stride, alive, ranges, kv_capacity, out, dout, dq, \
+                                            dq_row_stride, dk, dv, dkv_row_stride, B, NQ, NK, H, s)
     switch (nb) {
         case 1: BNB_SBM(1);
         case 2: BNB_SBM(2);
@@ -551,8 +566,8 @@ extern "C" int bnb_sdpa_masked_bwd_path(const void *qkv, int64_t qkv_row_stride,
         const uint16_t *p = (const uint16_t *)qkv;
         const int D = H * dh;
         uint16_t *g = (uint16_t *)dqkv;
-        return dispatch_sdpa_bwd_mfma<false>(p, qkv_row_stride, p + D, p + 2 * D, qkv_row_stride, alive, out, dout, g, 3 * (int64_t)D,
-                                             g + D, g + 2 * D, 3 * (int64_t)D, B, NM, NM, H, s);
+        return dispatch_sdpa_bwd_mfma<false>(p, qkv_row_stride, p + D, p + 2 * D, qkv_row_stride, alive, nullptr, 0, out, dout, g,
+                                             3 * (int64_t)D, g + D, g + 2 * D, 3 * (int64_t)D, B, NM, NM, H, s);
     }
     if (!small) return BNB_ERR_UNSUPPORTED;
     if (dtype == BNB_BF16) return launch_sdpa_bwd<uint16_t>(qkv, qkv_row_stride, alive, out, dout, dqkv, B, NM, H, s);
@@ -582,6 +597,27 @@ extern "C" int bnb_sdpa_cross_bwd(const void *q, int64_t q_row_stride, int NQ, c
     if (B > 0x7fffffffLL / H) return BNB_ERR_UNSUPPORTED;
     const uint16_t *kp = (const uint16_t *)kv;
     uint16_t *g = (uint16_t *)dkv;
-    return dispatch_sdpa_bwd_mfma<true>(q, q_row_stride, kp, kp + D, kv_row_stride, key_mask, out, dout, dq, D, g, g + D,
+    return dispatch_sdpa_bwd_mfma<true>(q, q_row_stride, kp, kp + D, kv_row_stride, key_mask, nullptr, 0, out, dout, dq, D, g, g + D,
                                         2 * (int64_t)D, B, NQ, NK, H, (hipStream_t)stream);
+}
+
+extern "C" int bnb_sdpa_cross_ranges_bwd(const void *q, int64_t q_row_stride, int NQ, const void *kv_rows, int64_t kv_row_stride,
+                                         const int32_t *ranges, int64_t capacity, int max_keys, const void *out, const void *dout,
+                                         void *dq, void *dkv_rows, int64_t B, int H, int dh, int dtype, void *stream)
+{
+    using namespace bnb;
+    if (B < 0 || NQ < 1 || H < 1 || dh < 1 || capacity < 1 || max_keys < 1) return BNB_ERR_BAD_SHAPE;  // an empty list: nothing to call
+    if (dtype != BNB_BF16 || dh != kSbDh || NQ > 160 || max_keys > 160) return BNB_ERR_UNSUPPORTED;
+    const int D = H * dh;
+    if (q_row_stride < D || kv_row_stride < 2 * (int64_t)D) return BNB_ERR_BAD_SHAPE;
+    if (B == 0) return 0;
+    if (!q || !ranges || !out || !dout || !dq || !kv_rows || !dkv_rows) return BNB_ERR_NULL_POINTER;
+    if (!aligned16(q) || !aligned16(kv_rows) || !aligned16(out) || !aligned16(dout) || !aligned16(dq) || !aligned16(dkv_rows) ||
+        (q_row_stride % 8) != 0 || (kv_row_stride % 8) != 0)
+        return BNB_ERR_MISALIGNED;
+    if (B > 0x7fffffffLL / H) return BNB_ERR_UNSUPPORTED;
+    const uint16_t *kp = (const uint16_t *)kv_rows;
+    uint16_t *g = (uint16_t *)dkv_rows;
+    return dispatch_sdpa_bwd_mfma<true>(q, q_row_stride, kp, kp + D, kv_row_stride, nullptr, ranges, capacity, out, dout, dq, D, g,
+                                        g + D, 2 * (int64_t)D, B, NQ, max_keys, H, (hipStream_t)stream);
 }

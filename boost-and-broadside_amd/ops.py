@@ -317,6 +317,66 @@ def sdpa_cross_train(qkv: torch.Tensor, kv: torch.Tensor, key_mask: torch.Tensor
         return _SdpaCrossTrain.apply(qkv, kv, key_mask, n_heads)
 
 
+def sdpa_cross_rows_bwd(qkv, kv_rows, rows: "CompactRows", n_heads, out, dout, total: int):
+    """Gradients ``(dq (B, NQ, D), dkv_rows (total, 2D))`` of ``sdpa_cross_rows`` (without accumulator);
+    ``total`` = ``rows.total_host()`` rows of ``kv_rows`` are valid."""
+    B, NQ, D3 = qkv.shape
+    D = D3 // 3
+    for name, t in (("qkv", qkv), ("kv_rows", kv_rows), ("out", out), ("dout", dout)):
+        _need_device(t, name)
+        if t.dtype != torch.bfloat16:
+            raise TypeError(f"{name} must be bfloat16")
+    if kv_rows.dim() != 2 or kv_rows.shape[1] != 2 * D or not kv_rows.is_contiguous() or kv_rows.shape[0] < total:
+        raise ValueError(f"kv_rows must be a contiguous (>= {total}, {2 * D}) tensor")
+    if rows.shape[0] != B or rows.shape[1] > 160 or out.shape != (B, NQ, D) or dout.shape != (B, NQ, D):
+        raise ValueError("rows must list at most 160 entries for each of the B environments; out and dout are (B, NQ, D)")
+    if B and NQ and (qkv.stride(-1) != 1 or (B > 1 and qkv.stride(0) != NQ * qkv.stride(1))):
+        qkv = qkv.contiguous()
+    out, dout = out.contiguous(), dout.contiguous()
+    dq = torch.empty((B, NQ, D), dtype=torch.bfloat16, device=qkv.device)
+    dkv = torch.empty((total, 2 * D), dtype=torch.bfloat16, device=qkv.device)
+    if total == 0:
+        return dq.zero_(), dkv
+    if B:
+        with torch.cuda.device(qkv.device):
+            rc = _native.load().bnb_sdpa_cross_ranges_bwd(qkv.data_ptr(), qkv.stride(1), NQ, kv_rows.data_ptr(), kv_rows.stride(0),
+                                                          rows.offsets.data_ptr(), total, rows.shape[1], out.data_ptr(), dout.data_ptr(),
+                                                          dq.data_ptr(), dkv.data_ptr(), B, n_heads, D // n_heads, _native.BF16, _stream())
+        _native.check(rc, "bnb_sdpa_cross_ranges_bwd")
+    return dq, dkv
+
+
+class _SdpaCrossRowsTrain(torch.autograd.Function):
+    """``sdpa_cross_rows`` (nothing accumulated) with its backward kernel."""
+
+    @staticmethod
+    def forward(ctx, qkv, kv_rows, rows, n_heads, total):
+        with torch.no_grad():
+            out = sdpa_cross_rows(qkv, kv_rows, rows, n_heads, total=total)
+        ctx.save_for_backward(qkv, kv_rows, out)
+        ctx.rows, ctx.n_heads, ctx.total = rows, n_heads, total
+        return out
+
+    @staticmethod
+    @_outside_autocast
+    def backward(ctx, dout):
+        qkv, kv_rows, out = ctx.saved_tensors
+        dq, dkv = sdpa_cross_rows_bwd(qkv, kv_rows, ctx.rows, ctx.n_heads, out, dout.to(torch.bfloat16), ctx.total)
+        dqkv = torch.zeros_like(qkv)
+        dqkv[..., : dq.shape[-1]] = dq
+        return dqkv, dkv, None, None, None
+
+
+def sdpa_cross_rows_train(qkv: torch.Tensor, kv_rows: torch.Tensor, rows: "CompactRows", n_heads: int) -> torch.Tensor:
+    """Differentiable ``sdpa_cross_rows``: ``kv_rows`` holds exactly ``rows.total_host()`` rows, ``[K | V]`` of the
+    listed entries in list order (bfloat16).  Needs head size 32, at most 160 queries and 160 entries per row of the mask."""
+    total = rows.total_host()
+    if kv_rows.shape[0] != total:
+        raise ValueError(f"kv_rows must hold the {total} listed rows")
+    with torch.autocast("cuda", enabled=False):
+        return _SdpaCrossRowsTrain.apply(qkv, kv_rows.contiguous(), rows, n_heads, total)
+
+
 def rglru_step(
     x: torch.Tensor,
     gates_pre: torch.Tensor,
@@ -1707,6 +1767,13 @@ class CompactRows:
         """Number of valid entries, as a one-element int32 device tensor."""
         return self.offsets[-1:]
 
+    def total_host(self) -> int:
+        """Number of valid entries as a Python int (one device-to-host copy, cached): what torch ops
+        over exactly the listed rows need to size their tensors."""
+        if getattr(self, "_total_host", None) is None:
+            self._total_host = int(self.offsets[-1].item())
+        return self._total_host
+
 
 def norm_linear(
     x: torch.Tensor,
@@ -1767,6 +1834,7 @@ def sdpa_cross_rows(
     n_heads: int,
     *,
     accum: torch.Tensor | None = None,
+    total: int | None = None,
 ) -> torch.Tensor:
     """``sdpa_cross`` over key/value rows compacted beforehand: ``kv_rows`` (capacity, 2*D)
     holds ``[K | V]`` of the entries listed in ``rows`` (e.g. ``norm_linear(bullets, ..., rows=rows)``),
@@ -1779,7 +1847,8 @@ def sdpa_cross_rows(
         raise RuntimeError("sdpa_cross_rows covers bfloat16, head size 32 and at most 160 queries")
     if kv_rows.dim() != 2 or kv_rows.shape[1] != 2 * D or not kv_rows.is_contiguous():
         raise ValueError(f"kv_rows must be a contiguous (capacity, {2 * D}) tensor")
-    if rows.shape[0] != B or kv_rows.shape[0] < rows.shape[0] * rows.shape[1]:
+    need = rows.shape[0] * rows.shape[1] if total is None else total  # without the host-side count: room for every entry
+    if rows.shape[0] != B or kv_rows.shape[0] < need:
         raise ValueError("rows was built for a different batch, or kv_rows is smaller than its capacity")
     if torch.is_grad_enabled() and (qkv.requires_grad or kv_rows.requires_grad):
         raise RuntimeError("sdpa_cross_rows is forward-only; call it under torch.no_grad()")
@@ -1790,6 +1859,8 @@ def sdpa_cross_rows(
     out = accum if accum is not None else torch.empty((B, NQ, D), dtype=torch.bfloat16, device=qkv.device)
     if B == 0 or NQ == 0:
         return out
+    if kv_rows.shape[0] == 0:  # an empty list: every environment reads nothing
+        return out if accum is not None else out.zero_()
     with torch.cuda.device(qkv.device):
         rc = _native.load().bnb_sdpa_cross_ranges_fwd(
             qkv.data_ptr(), qkv.stride(1), NQ, kv_rows.data_ptr(), kv_rows.stride(0), rows.offsets.data_ptr(),

@@ -294,13 +294,7 @@ class TransformerBlock(nn.Module):
             else:
                 merged = self._self_attention_autograd(qkv, alive_mask)
             if self.reads_bullets and bullets is not None:
-                if isinstance(bullet_mask, ops.CompactRows):
-                    bullet_mask = bullet_mask.mask
-                kv = _project(self.kv_bullet, _train_norm(self.norm_bullet, bullets)[1])
-                if _TRAIN_KERNELS and ops.sdpa_cross_train_supported(qkv, kv, self.n_heads):
-                    merged = merged + ops.sdpa_cross_train(qkv, kv, bullet_mask, self.n_heads)
-                else:
-                    merged = merged + self._bullet_read(qkv, kv, bullet_mask)
+                merged = merged + self._bullet_branch_autograd(qkv, bullets, bullet_mask)
             return _project(self.out_proj, merged)
         try:
             merged = ops.sdpa_masked(qkv, alive_mask, self.n_heads)  # (B, N, D) head-major
@@ -338,6 +332,37 @@ class TransformerBlock(nn.Module):
             qkv.dtype == torch.bfloat16 and self.d_model == ops.FFN_WIDTH and self.head_dim == 32 and qkv.shape[1] <= 160
             and bullets.is_cuda and bullets.dtype == torch.float32 and self.kv_bullet.bias is None
         )
+
+    def _bullet_branch_autograd(self, qkv, bullets, bullet_mask):
+        """The bullet read in grad mode, (B, N, D) to be added to the self-attention output.
+
+        With a mask, bf16 projections and at most 160 slots per environment only the bullets in
+        flight are normalised and projected: the list of live slots is built on the device, its
+        length read back once (torch needs it to size the gathered rows), ``norm_bullet`` and
+        ``kv_bullet`` run on the gathered rows and the read and its backward take the compacted
+        ``[K | V]`` rows with per-environment ranges.  Otherwise every slot is projected and the
+        read is the masked kernel pair, or torch's SDPA for the shapes the kernels do not cover."""
+        rows = bullet_mask if isinstance(bullet_mask, ops.CompactRows) else None
+        mask = rows.mask if rows is not None else bullet_mask
+        B, NB, D = bullets.shape
+        compact_ok = (
+            _TRAIN_KERNELS and mask is not None and qkv.is_cuda and qkv.dtype == torch.bfloat16 and NB <= 160
+            and self.head_dim == 32 and qkv.shape[1] <= 160 and self.kv_bullet.bias is None
+        )
+        if compact_ok:
+            if rows is None:
+                rows = ops.CompactRows(mask)
+            total = rows.total_host()
+            if total == 0:
+                return torch.zeros_like(qkv[..., :D])
+            live = bullets.reshape(B * NB, D).index_select(0, rows.index[:total].long())
+            kv_rows = _project(self.kv_bullet, _train_norm(self.norm_bullet, live)[1])
+            if kv_rows.dtype == torch.bfloat16:
+                return ops.sdpa_cross_rows_train(qkv, kv_rows, rows, self.n_heads)
+        kv = _project(self.kv_bullet, _train_norm(self.norm_bullet, bullets)[1])
+        if _TRAIN_KERNELS and ops.sdpa_cross_train_supported(qkv, kv, self.n_heads):
+            return ops.sdpa_cross_train(qkv, kv, mask, self.n_heads)
+        return self._bullet_read(qkv, kv, mask)
 
     def _self_attention_autograd(self, qkv, alive_mask):
         """Masked self-attention as the reference composes it (attention.py:136-147,168)."""

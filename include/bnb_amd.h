@@ -303,6 +303,16 @@ int bnb_sdpa_cross_bwd(const void *q, int64_t q_row_stride, int NQ, const void *
                        int64_t B, int H, int dh, int dtype, void *stream);
 
 /*
+ * The same backward over key/value rows compacted beforehand (the counterpart of
+ * bnb_sdpa_cross_ranges_fwd): environment b reads rows ranges[b] .. ranges[b+1]-1 of kv_rows
+ * (capacity rows of [K | V], all of them live), at most max_keys <= 160 per environment;
+ * dkv_rows has kv_rows' layout.  An environment with an empty range gets a zero dq.
+ */
+int bnb_sdpa_cross_ranges_bwd(const void *q, int64_t q_row_stride, int NQ, const void *kv_rows, int64_t kv_row_stride,
+                              const int32_t *ranges, int64_t capacity, int max_keys, const void *out, const void *dout,
+                              void *dq, void *dkv_rows, int64_t B, int H, int dh, int dtype, void *stream);
+
+/*
  * RMSNorm backward:  y = x * rsqrt(mean(x^2) + eps) * weight
  *   dx[r] = rstd * (dy[r] * weight) - x[r] * rstd^3 * mean(dy[r] * weight * x[r])  (+ grad_sum[r])
  *   dw    = sum_r dy[r] * x[r] * rstd

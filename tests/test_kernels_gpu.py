@@ -1843,3 +1843,48 @@ def test_sdpa_cross_train_is_differentiable():
     assert max_rel(qkv.grad.float().cpu().double(), xq.grad) <= BF16_TOL
     assert max_rel(kv.grad.float().cpu().double(), xkv.grad) <= BF16_TOL
     assert not ops.sdpa_cross_train_supported(qkv, torch.zeros(B, 200, 2 * D, device=DEV, dtype=torch.bfloat16), H)
+
+
+@pytest.mark.parametrize("B,NQ,NK,p_live", [(4, 12, 80, 0.25), (3, 23, 160, 0.1), (5, 12, 40, 1.0), (6, 84, 33, 0.5), (300, 12, 80, 0.25)])
+def test_sdpa_cross_rows_bwd_equals_the_masked_form(B, NQ, NK, p_live):
+    H, D = 4, 128
+    g = torch.Generator().manual_seed(B + NQ + NK)
+    qkv = torch.randn(B, NQ, 3 * D, generator=g).bfloat16().to(DEV)
+    kv = torch.randn(B, NK, 2 * D, generator=g).bfloat16().to(DEV)
+    mask = (torch.rand(B, NK, generator=g) < p_live).to(DEV)
+    if B > 2:
+        mask[1] = False
+    up = torch.randn(B, NQ, D, generator=g).bfloat16().to(DEV)
+    rows = ops.CompactRows(mask)
+    total = rows.total_host()
+    assert total == int(mask.sum())
+    kv_rows = kv.reshape(B * NK, 2 * D)[mask.reshape(-1)].contiguous()
+    out = ops.sdpa_cross(qkv, kv, mask, H)
+    out_rows = ops.sdpa_cross_rows(qkv, kv_rows, rows, H, total=total)
+    assert max_rel(out_rows.float().cpu(), out.float().cpu()) <= BF16_TOL  # two forward kernels (tile vs streamed keys)
+    dq, dkv = ops.sdpa_cross_bwd(qkv, kv, mask, H, out, up)
+    dq_r, dkv_r = ops.sdpa_cross_rows_bwd(qkv, kv_rows, rows, H, out, up, total)
+    # same keys, in the same order per environment: the live rows' gradients and dq agree to rounding of the
+    # sums' order (compaction moves keys to other accumulator rows), well inside the bf16 bar
+    assert max_rel(dq_r.float().cpu(), dq.float().cpu()) <= BF16_TOL
+    assert max_rel(dkv_r.float().cpu(), dkv.reshape(B * NK, 2 * D)[mask.reshape(-1)].float().cpu()) <= BF16_TOL
+    off = ~mask.any(dim=1)
+    assert not dq_r[off].any()
+
+
+def test_sdpa_cross_rows_train_matches_autograd_of_the_oracle():
+    B, NQ, NK, H, D = 7, 12, 80, 4, 128
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(B, NQ, 3 * D, generator=g).bfloat16().to(DEV).requires_grad_()
+    kv = torch.randn(B, NK, 2 * D, generator=g).bfloat16()
+    mask = torch.rand(B, NK, generator=g) < 0.3
+    up = torch.randn(B, NQ, D, generator=g)
+    rows = ops.CompactRows(mask.to(DEV))
+    kv_rows = kv.reshape(B * NK, 2 * D)[mask.reshape(-1)].to(DEV).requires_grad_()
+    out = ops.sdpa_cross_rows_train(qkv, kv_rows, rows, H)
+    (out.float() * up.to(DEV)).sum().backward()
+    xq = qkv.detach().cpu().double().requires_grad_()
+    xkv = kv.double().requires_grad_()
+    (torch_ref.bullet_read(xq, xkv, mask, H) * up.bfloat16().double()).sum().backward()
+    assert max_rel(qkv.grad.float().cpu().double(), xq.grad) <= BF16_TOL
+    assert max_rel(kv_rows.grad.float().cpu().double(), xkv.grad.reshape(B * NK, 2 * D)[mask.reshape(-1)]) <= BF16_TOL

@@ -736,3 +736,56 @@ def test_trunk_sequence_is_the_loop_over_blocks_and_trains_with_and_without_chec
         assert torch.equal(a, b)
     with pytest.raises(ValueError):
         trunk.sequence(xs, alive, hidden0[:, :-1], done)
+
+
+@pytest.mark.parametrize("p_live", [0.25, 0.0])
+def test_update_path_with_the_bullet_read_agrees_with_the_library_ops(p_live):
+    """Grad mode with bullets: only the bullets in flight are normalised and projected and the read runs on
+    its kernels; every gradient (parameters, tokens, bullets) must agree with torch's own differentiable ops."""
+    from boost_and_broadside_amd import trunk
+
+    cfg = _cfg(128, 4, spatial=2, temporal=1, bullets=1)
+    torch.manual_seed(13)
+    block = bnb.YemongBlock(cfg).to(DEV)
+    T, B, N, M, D = 8, 80, 8, 4, 128
+    NB = N * 10
+    gen = torch.Generator().manual_seed(14)
+    x = torch.randn(T, B, N + M, D, generator=gen).to(DEV).requires_grad_()
+    alive = (torch.rand(T, B, N + M, generator=gen) < 0.85).to(DEV)
+    alive[..., 0] = True
+    bullets = torch.randn(T * B, NB, D, generator=gen).to(DEV).requires_grad_()
+    bmask = (torch.rand(T * B, NB, generator=gen) < p_live).to(DEV)
+    if p_live > 0:
+        bmask[3] = False
+    h0 = torch.zeros(1, B * N, D, device=DEV)
+    cb0 = torch.zeros(1, B * N, 3, D, device=DEV)
+    done = (torch.rand(T, B, generator=gen) < 0.1).to(DEV)
+
+    def grads():
+        block.zero_grad(set_to_none=True)
+        x.grad = bullets.grad = None
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = block.sequence(x, alive, h0, cb0, done, N, bullets, bmask)[0]
+        out.float().square().mean().backward()
+        named = {n: p.grad for n, p in block.named_parameters() if p.grad is not None}
+        named["x"] = x.grad
+        if bullets.grad is not None:
+            named["bullets"] = bullets.grad
+        return {k: v.detach().clone() for k, v in named.items()}
+
+    fast = grads()
+    with trunk.library_update_path():
+        slow = grads()
+    assert ("bullets" in fast) == (p_live > 0) or "bullets" in fast
+    for name, g in slow.items():
+        if name not in fast:
+            assert not g.any(), name  # e.g. the bullet layers without any bullet in flight
+            continue
+        assert torch.isfinite(fast[name]).all(), name
+        if g.abs().max() == 0:
+            assert fast[name].abs().max() == 0, name
+        else:
+            assert max_rel(fast[name].float().cpu(), g.float().cpu()) <= BF16_TOL, name
+    if p_live > 0:
+        dead_rows = ~bmask.reshape(-1)
+        assert not fast["bullets"].reshape(-1, D)[dead_rows].any()  # bullets that are not in flight receive nothing
