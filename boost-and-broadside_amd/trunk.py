@@ -887,6 +887,9 @@ class YemongTrunk(nn.Module):
         if n_layers != self.n_hidden_layers or rows % B:
             raise ValueError(f"initial_hidden must be ({self.n_hidden_layers}, B*n_rec, {CONV_KERNEL * D})")
         n_rec = rows // B
+        if (bullets is not None and isinstance(bullet_mask, torch.Tensor) and bullet_mask.is_cuda
+                and bullet_mask.dtype == torch.bool and bullet_mask.dim() == 2):
+            bullet_mask = ops.CompactRows(bullet_mask)  # one list of the bullets in flight for every bullet-reading layer
         h_all = initial_hidden[:, :, :D]
         cb_all = initial_hidden[:, :, D:].reshape(n_layers, rows, CONV_KERNEL - 1, D)
         slot = 0

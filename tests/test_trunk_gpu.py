@@ -789,3 +789,29 @@ def test_update_path_with_the_bullet_read_agrees_with_the_library_ops(p_live):
     if p_live > 0:
         dead_rows = ~bmask.reshape(-1)
         assert not fast["bullets"].reshape(-1, D)[dead_rows].any()  # bullets that are not in flight receive nothing
+
+
+def test_trunk_sequence_with_bullets_shares_one_list_and_matches_the_block_loop():
+    D, H, B, N, M, T = 128, 4, 10, 8, 4, 6
+    torch.manual_seed(41)
+    trunk = bnb.YemongTrunk(_cfg(D, H, 2, 2, 1, bullets=1)).to(DEV)
+    gen = torch.Generator().manual_seed(42)
+    xs = torch.randn(T, B, N + M, D, generator=gen).to(DEV)
+    alive = (torch.rand(T, B, N + M, generator=gen) < 0.85).to(DEV)
+    alive[..., 0] = True
+    bullets = torch.randn(T * B, N * 10, D, generator=gen).to(DEV)
+    bmask = (torch.rand(T * B, N * 10, generator=gen) < 0.3).to(DEV)
+    done = (torch.rand(T, B, generator=gen) < 0.15).to(DEV)
+    hidden0 = torch.zeros(2, B * N, 4 * D, device=DEV)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        got = trunk.sequence(xs, alive, hidden0, done, bullets, bmask)
+        x = xs
+        for i, block in enumerate(trunk.yemong_layers):
+            x = block.sequence(x, alive, hidden0[i:i + 1, :, :D], hidden0[i:i + 1, :, D:].reshape(1, B * N, 3, D), done, N,
+                               bullets, bmask)[0]
+    assert max_rel(got.float().cpu(), x.float().cpu()) <= BF16_TOL
+    xin = xs.clone().requires_grad_()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = trunk.sequence(xin, alive, hidden0, done, bullets, bmask, grad_checkpoint=True)
+    out.float().square().mean().backward()
+    assert torch.isfinite(xin.grad).all() and all(q.grad is not None and torch.isfinite(q.grad).all() for q in trunk.parameters())
