@@ -340,7 +340,8 @@ def sdpa_cross_rows_bwd(qkv, kv_rows, rows: "CompactRows", n_heads, out, dout, t
     if B:
         with torch.cuda.device(qkv.device):
             rc = _native.load().bnb_sdpa_cross_ranges_bwd(qkv.data_ptr(), qkv.stride(1), NQ, kv_rows.data_ptr(), kv_rows.stride(0),
-                                                          rows.offsets.data_ptr(), total, rows.shape[1], out.data_ptr(), dout.data_ptr(),
+                                                          rows.offsets.data_ptr(), total, max(1, rows.max_count_host()), out.data_ptr(),
+                                                          dout.data_ptr(),
                                                           dq.data_ptr(), dkv.data_ptr(), B, n_heads, D // n_heads, _native.BF16, _stream())
         _native.check(rc, "bnb_sdpa_cross_ranges_bwd")
     return dq, dkv
@@ -1767,12 +1768,25 @@ class CompactRows:
         """Number of valid entries, as a one-element int32 device tensor."""
         return self.offsets[-1:]
 
+    def _host_counts(self) -> tuple[int, int]:
+        if getattr(self, "_host", None) is None:
+            B = self.shape[0]
+            if B == 0:
+                self._host = (0, 0)
+            else:
+                per_row = self.offsets[1:] - self.offsets[:-1]
+                both = torch.stack([self.offsets[-1], per_row.max()]).tolist()  # one device-to-host copy
+                self._host = (int(both[0]), int(both[1]))
+        return self._host
+
     def total_host(self) -> int:
         """Number of valid entries as a Python int (one device-to-host copy, cached): what torch ops
         over exactly the listed rows need to size their tensors."""
-        if getattr(self, "_total_host", None) is None:
-            self._total_host = int(self.offsets[-1].item())
-        return self._total_host
+        return self._host_counts()[0]
+
+    def max_count_host(self) -> int:
+        """Largest number of entries in one row of the mask, as a Python int (same copy, cached)."""
+        return self._host_counts()[1]
 
 
 def norm_linear(
