@@ -476,7 +476,7 @@ __global__ __launch_bounds__(256) void team_gather_bwd_kernel(const float *__res
 // du(pair) = sum over all ship rows of ds(row, pair) * x(row): rows dealt to the work-groups in
 // contiguous runs, a thread per (channel, half of the pairs), partial sums per work-group, then
 // sum_slices in a fixed order.
-constexpr int kDuBlocks = 512;
+constexpr int kDuBlocks = 2048;
 
 __global__ __launch_bounds__(256) void team_du_kernel(const float *__restrict__ x, int64_t x_env_stride, int64_t x_row_stride,
                                                       const float *__restrict__ ds, float *__restrict__ partials, int64_t rows,
@@ -492,8 +492,9 @@ __global__ __launch_bounds__(256) void team_du_kernel(const float *__restrict__ 
     for (int c = 0; c < 8; ++c) acc[c] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll 4
     for (int64_t r = r0 + rl; r < r1; r += 8) {
-        const uint32_t env = (uint32_t)(r / N);  // rows < 2^31 * N
-        const uint32_t n = (uint32_t)(r - (int64_t)env * N);
+        const uint32_t r32 = (uint32_t)r;  // B * N < 2^31: 32-bit division
+        const uint32_t env = r32 / (uint32_t)N;
+        const uint32_t n = r32 - env * (uint32_t)N;
         const f32x4 xv = *reinterpret_cast<const f32x4 *>(x + (int64_t)env * x_env_stride + (int64_t)n * x_row_stride + q4);
         const float *d = ds + r * NC;
 #pragma unroll
@@ -581,6 +582,7 @@ extern "C" int bnb_team_attend_bwd(const float *x, int64_t x_env_stride, int64_t
     hipStream_t s = (hipStream_t)stream;
     const int NC = 2 * H;
     if (B == 0 || N == 0) return launch_sum_slices(partials, du, (int64_t)NC * kTpD, 0, 0, s);
+    if ((int64_t)B * N >= (1LL << 31)) return BNB_ERR_UNSUPPORTED;
     if (!x || !team_id || !alive || !score_vectors || !z || !dz || !dx || !ds) return BNB_ERR_NULL_POINTER;
     if (x_row_stride < D || x_env_stride < (int64_t)N * D || team_env_stride < N || alive_env_stride < N)
         return BNB_ERR_BAD_SHAPE;
