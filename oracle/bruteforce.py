@@ -197,3 +197,90 @@ def team_pool_loops(x, team_id, alive, seeds, in_proj_weight, out_proj_weight, n
             out = wo @ merged
             pool[b, t] = out / math.sqrt(float(np.mean(out * out)) + eps) * np.asarray(norm_weight, dtype=np.float64)
     return pool
+
+
+# --------------------------------------------------------------------------
+# gradients of the update path, written out (not differentiated by a library)
+# --------------------------------------------------------------------------
+
+def sdpa_masked_grad_loops(qkv: np.ndarray, alive: np.ndarray | None, n_heads: int, dout: np.ndarray) -> np.ndarray:
+    """d(qkv) of ``sdpa_masked_loops`` for the output gradient ``dout`` (B, NM, D), float64.
+
+    Per environment and head, with P the weights the forward used (masked softmax; 1/NM for
+    every key when no key is alive, which is what equal biases on all keys evaluate to):
+        dV = P^T dO,  dP = dO V^T,  dS = P * (dP - rowsum(P * dP)),
+        dQ = dS K / sqrt(dh),  dK = dS^T Q / sqrt(dh).
+    Chain rule through models/yemong/attention.py:136-147 written out by hand.
+    """
+    qkv = np.asarray(qkv, dtype=np.float64)
+    dout = np.asarray(dout, dtype=np.float64)
+    B, NM, D3 = qkv.shape
+    D = D3 // 3
+    dh = D // n_heads
+    grad = np.zeros_like(qkv)
+    for b in range(B):
+        live = np.ones(NM, dtype=bool) if alive is None else np.asarray(alive[b], dtype=bool)
+        uniform = not live.any()
+        for h in range(n_heads):
+            cols = slice(h * dh, (h + 1) * dh)
+            Q, K, V = qkv[b, :, cols], qkv[b, :, D:][:, cols], qkv[b, :, 2 * D:][:, cols]
+            dO = dout[b, :, cols]
+            P = np.zeros((NM, NM))
+            for i in range(NM):
+                if uniform:
+                    P[i, :] = 1.0 / NM
+                    continue
+                s = np.array([np.dot(Q[i], K[j]) / math.sqrt(dh) if live[j] else -np.inf for j in range(NM)])
+                e = np.exp(s - s[live].max())
+                e[~live] = 0.0
+                P[i] = e / e.sum()
+            dP = dO @ V.T
+            dS = P * (dP - (P * dP).sum(axis=1, keepdims=True))
+            grad[b, :, cols] = dS @ K / math.sqrt(dh)
+            grad[b, :, D:][:, cols] = dS.T @ Q / math.sqrt(dh)
+            grad[b, :, 2 * D:][:, cols] = P.T @ dO
+    return grad
+
+
+def conv_sequence_grad_loops(b1, conv_buf, weight, done, dv, dtail=None):
+    """Gradients ``(db1, dconv_buf, dweight (D, 4), dbias (D,))`` of ``conv_sequence_loops`` for the output
+    gradient ``dv`` (R, T, D) and the gradient ``dtail`` (R, 3, D) of the three inputs handed on
+    (the last three of [conv_buf, b1], models/yemong/griffin.py:277), float64: every term
+    ``w[:, 3-j] * input[t-j]`` of the forward sends ``dv[t] * w`` to its input and ``dv[t] * input``
+    to its tap."""
+    b1 = np.asarray(b1, dtype=np.float64)
+    buf = np.asarray(conv_buf, dtype=np.float64)
+    dv = np.asarray(dv, dtype=np.float64)
+    R, T, D = b1.shape
+    w = np.asarray(weight, dtype=np.float64).reshape(D, 4)
+    dseq = np.zeros((R, T + 3, D))  # position p = time p - 3
+    dw = np.zeros((D, 4))
+    for r in range(R):
+        seq = np.concatenate([buf[r], b1[r]], axis=0)
+        for t in range(T):
+            for j in range(4):
+                crossed = any(done is not None and 0 <= s < T and done[r, s] for s in range(t - j, t))
+                if not crossed:
+                    dseq[r, t - j + 3] += dv[r, t] * w[:, 3 - j]
+                    dw[:, 3 - j] += dv[r, t] * seq[t - j + 3]
+        if dtail is not None:
+            dseq[r, T:] += np.asarray(dtail[r], dtype=np.float64)
+    return dseq[:, 3:], dseq[:, :3], dw, dv.sum(axis=(0, 1))
+
+
+def rms_norm_grad_loops(x, weight, eps, dy):
+    """``(dx, dweight)`` of ``y = x * rsqrt(mean(x^2) + eps) * weight`` (nn.RMSNorm, attention.py:60,73), float64,
+    row by row from the quotient rule."""
+    x = np.asarray(x, dtype=np.float64)
+    w = np.asarray(weight, dtype=np.float64)
+    dy = np.asarray(dy, dtype=np.float64)
+    R, D = x.shape
+    dx = np.zeros_like(x)
+    dw = np.zeros(D)
+    for r in range(R):
+        ms = float(np.dot(x[r], x[r])) / D + eps
+        rstd = 1.0 / math.sqrt(ms)
+        g = dy[r] * w
+        dx[r] = g * rstd - x[r] * (float(np.dot(g, x[r])) / D) * rstd ** 3
+        dw += dy[r] * x[r] * rstd
+    return dx, dw

@@ -1,5 +1,5 @@
-"""Writes tests/golden/step_vectors.npz, widened_vectors.npz and team_pool_vectors.npz: small seeded
-inputs and their expected outputs.
+"""Writes tests/golden/step_vectors.npz, widened_vectors.npz, team_pool_vectors.npz and update_vectors.npz:
+small seeded inputs and their expected outputs (update_vectors: expected gradients).
 
 The reference keeps no stored numeric vectors for this path (its tests are property tests and
 its one golden file needs weights that are not in the checkout), and the reference was not
@@ -50,6 +50,7 @@ def main() -> None:
     print("wrote", os.path.join(HERE, "step_vectors.npz"), {k: v.shape for k, v in out.items()})
     widened()
     team_pool()
+    update()
 
 
 def widened() -> None:
@@ -135,6 +136,51 @@ def team_pool() -> None:
                                              out["out_proj_weight"], out["norm_weight"], H, float(np.finfo(np.float32).eps))
     np.savez_compressed(os.path.join(HERE, "team_pool_vectors.npz"), **out)
     print("wrote", os.path.join(HERE, "team_pool_vectors.npz"), {k: v.shape for k, v in out.items()})
+
+
+
+
+def update() -> None:
+    """tests/golden/update_vectors.npz: gradients of the update path from the hand-written chain rules."""
+    rng = np.random.default_rng(20240604)
+    out = {}
+
+    def bf16(a):
+        u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+        return (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16).astype(np.uint32).view(np.float32)  # round to nearest even
+
+    # attention backward: inputs already bf16-representable so that both dtypes see the same numbers
+    for tag, (B, NM, H) in {"attn_4v4": (4, 12, 4), "attn_8v11": (3, 23, 4), "attn_wide": (2, 40, 4)}.items():
+        D = 32 * H
+        qkv = bf16(1.2 * rng.standard_normal((B, NM, 3 * D)))
+        alive = rng.random((B, NM)) < 0.7
+        alive[0] = False
+        alive[1] = False
+        alive[1, NM // 2] = True
+        dout = bf16(rng.standard_normal((B, NM, D)))
+        out[f"{tag}_qkv"], out[f"{tag}_alive"], out[f"{tag}_heads"], out[f"{tag}_dout"] = qkv, alive, np.int64(H), dout
+        out[f"{tag}_dqkv"] = bruteforce.sdpa_masked_grad_loops(qkv, alive, H, dout)
+    # sequence conv backward with episode ends and a gradient on the handed-on inputs
+    R, T, D = 5, 11, 128
+    b1 = bf16(rng.standard_normal((R, T, D)))
+    buf = rng.standard_normal((R, 3, D)).astype(np.float32)
+    w = (0.5 * rng.standard_normal((D, 1, 4))).astype(np.float32)
+    done = rng.random((R, T)) < 0.25
+    dv = rng.standard_normal((R, T, D)).astype(np.float32)
+    dtail = rng.standard_normal((R, 3, D)).astype(np.float32)
+    g = bruteforce.conv_sequence_grad_loops(b1, buf, w, done, dv, dtail)
+    out.update(conv_b1=b1, conv_buf=buf, conv_w=w, conv_done=done, conv_dv=dv, conv_dtail=dtail,
+               conv_db1=g[0], conv_dbuf=g[1], conv_dw=g[2], conv_dbias=g[3])
+    # RMSNorm backward
+    R, D = 9, 128
+    x = (rng.standard_normal((R, D)) * (0.2 + 3.0 * rng.random((R, 1)))).astype(np.float32)
+    nw = (1.0 + 0.3 * rng.standard_normal(D)).astype(np.float32)
+    dy = bf16(rng.standard_normal((R, D)))
+    eps = float(np.finfo(np.float32).eps)
+    gx, gw = bruteforce.rms_norm_grad_loops(x, nw, eps, dy)
+    out.update(norm_x=x, norm_w=nw, norm_dy=dy, norm_dx=gx, norm_dw=gw)
+    np.savez_compressed(os.path.join(HERE, "update_vectors.npz"), **out)
+    print("wrote", os.path.join(HERE, "update_vectors.npz"), {k: v.shape for k, v in out.items()})
 
 
 if __name__ == "__main__":

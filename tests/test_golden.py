@@ -170,3 +170,70 @@ def test_kernels_reproduce_team_pool_vectors():
     assert max_rel(pool.cpu(), want) <= 1e-5
     assert torch.equal(pool.cpu() == 0, want == 0)
     assert torch.equal(ships[3, 0], pool[3, 1])
+
+
+# ---------------------------------------------------------------- gradients of the update path
+
+UPD = np.load(os.path.join(ROOT, "tests", "golden", "update_vectors.npz"))
+UPD_ATTN = ("attn_4v4", "attn_8v11", "attn_wide")
+
+
+@pytest.mark.parametrize("tag", UPD_ATTN)
+def test_autograd_of_the_oracle_reproduces_attention_gradient_vectors(tag):
+    # the hand-written chain rule (oracle/bruteforce.py) and torch's differentiation of the written-out oracle agree
+    qkv = torch.from_numpy(UPD[f"{tag}_qkv"]).double().requires_grad_()
+    alive, H = torch.from_numpy(UPD[f"{tag}_alive"]), int(UPD[f"{tag}_heads"])
+    (torch_ref.sdpa_masked_softmax(qkv, alive, H) * torch.from_numpy(UPD[f"{tag}_dout"]).double()).sum().backward()
+    assert np.abs(qkv.grad.numpy() - UPD[f"{tag}_dqkv"]).max() <= 1e-10
+
+
+def test_autograd_of_the_oracle_reproduces_conv_and_norm_gradient_vectors():
+    lv = [torch.from_numpy(UPD[k]).double().requires_grad_() for k in ("conv_b1", "conv_buf", "conv_w")]
+    bias = torch.zeros(lv[0].shape[-1], dtype=torch.float64, requires_grad=True)
+    v, tail = torch_ref.conv_sequence(lv[0], lv[1], lv[2], bias, torch.from_numpy(UPD["conv_done"]))
+    ((v * torch.from_numpy(UPD["conv_dv"]).double()).sum() + (tail * torch.from_numpy(UPD["conv_dtail"]).double()).sum()).backward()
+    for t, key in zip(lv + [bias], ("conv_db1", "conv_dbuf", "conv_dw", "conv_dbias")):
+        assert np.abs(t.grad.numpy().reshape(UPD[key].shape) - UPD[key]).max() <= 1e-10, key
+    x = torch.from_numpy(UPD["norm_x"]).double().requires_grad_()
+    w = torch.from_numpy(UPD["norm_w"]).double().requires_grad_()
+    y = torch.nn.functional.rms_norm(x, (x.shape[-1],), w, float(np.finfo(np.float32).eps))
+    (y * torch.from_numpy(UPD["norm_dy"]).double()).sum().backward()
+    assert np.abs(x.grad.numpy() - UPD["norm_dx"]).max() <= 1e-10 and np.abs(w.grad.numpy() - UPD["norm_dw"]).max() <= 1e-10
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag", UPD_ATTN)
+@pytest.mark.parametrize("dtype,path", [(torch.float32, "valu"), (torch.bfloat16, "valu"), (torch.bfloat16, "mfma")])
+def test_kernels_reproduce_attention_gradient_vectors(tag, dtype, path):
+    from boost_and_broadside_amd import ops
+
+    qkv = torch.from_numpy(UPD[f"{tag}_qkv"]).to(dtype)  # stored values are bf16-representable: both dtypes see the same numbers
+    alive, H = torch.from_numpy(UPD[f"{tag}_alive"]), int(UPD[f"{tag}_heads"])
+    if path == "valu" and qkv.shape[1] > 32:
+        pytest.skip("the vector kernel covers up to 32 tokens")
+    dout = torch.from_numpy(UPD[f"{tag}_dout"]).to(dtype)
+    out = ops.sdpa_masked(qkv.cuda(), alive.cuda(), H)
+    got = ops.sdpa_masked_bwd(qkv.cuda(), alive.cuda(), H, out, dout.cuda(), path=path).float().cpu()
+    want = torch.from_numpy(UPD[f"{tag}_dqkv"])
+    D = qkv.shape[-1] // 3
+    for third in range(3):
+        cols = slice(third * D, (third + 1) * D)
+        assert max_rel(got[..., cols].double(), want[..., cols]) <= (1e-5 if dtype == torch.float32 else 2e-2), third
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("b_dtype", [torch.float32, torch.bfloat16])
+def test_kernels_reproduce_conv_and_norm_gradient_vectors(b_dtype):
+    from boost_and_broadside_amd import ops
+
+    b1 = torch.from_numpy(UPD["conv_b1"]).to(b_dtype).cuda()
+    got = ops.conv_seq_bwd(b1, torch.from_numpy(UPD["conv_buf"]).cuda(), torch.from_numpy(UPD["conv_w"]).cuda(),
+                           torch.from_numpy(UPD["conv_done"]).cuda(), torch.from_numpy(UPD["conv_dv"]).cuda(),
+                           torch.from_numpy(UPD["conv_dtail"]).cuda())
+    assert max_rel(got[0].float().cpu().double(), torch.from_numpy(UPD["conv_db1"])) <= (1e-5 if b_dtype == torch.float32 else 2e-2)
+    for g, key in zip(got[1:], ("conv_dbuf", "conv_dw", "conv_dbias")):
+        assert max_rel(g.cpu().double(), torch.from_numpy(UPD[key])) <= 1e-5, key
+    dx, dw = ops.rmsnorm_bwd(torch.from_numpy(UPD["norm_x"]).cuda(), torch.from_numpy(UPD["norm_dy"]).to(b_dtype).cuda(),
+                             torch.from_numpy(UPD["norm_w"]).cuda())
+    assert max_rel(dx.cpu().double(), torch.from_numpy(UPD["norm_dx"])) <= 1e-5
+    assert max_rel(dw.cpu().double(), torch.from_numpy(UPD["norm_dw"])) <= 1e-5
