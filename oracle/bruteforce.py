@@ -284,3 +284,34 @@ def rms_norm_grad_loops(x, weight, eps, dy):
         dx[r] = g * rstd - x[r] * (float(np.dot(g, x[r])) / D) * rstd ** 3
         dw += dy[r] * x[r] * rstd
     return dx, dw
+
+
+def bullet_read_grad_loops(q: np.ndarray, kv: np.ndarray, active: np.ndarray | None, n_heads: int, dout: np.ndarray):
+    """``(dq (B, N, D), dkv (B, NB, 2D))`` of ``bullet_read_loops`` for the output gradient ``dout``, float64: the same
+    chain rule as ``sdpa_masked_grad_loops`` over the active bullets only; an environment without an active bullet
+    was gated to zero (models/yemong/attention.py:161-164), so nothing flows back from it."""
+    q = np.asarray(q, dtype=np.float64)
+    kv = np.asarray(kv, dtype=np.float64)
+    dout = np.asarray(dout, dtype=np.float64)
+    B, N, D = q.shape
+    dh = D // n_heads
+    dq = np.zeros_like(q)
+    dkv = np.zeros_like(kv)
+    for b in range(B):
+        keys = [j for j in range(kv.shape[1]) if active is None or active[b, j]]
+        if not keys:
+            continue
+        for hd in range(n_heads):
+            cols = slice(hd * dh, (hd + 1) * dh)
+            Q, K, V, dO = q[b, :, cols], kv[b, keys][:, cols], kv[b, keys][:, D:][:, cols], dout[b, :, cols]
+            S = Q @ K.T / math.sqrt(dh)
+            E = np.exp(S - S.max(axis=1, keepdims=True))
+            P = E / E.sum(axis=1, keepdims=True)
+            dP = dO @ V.T
+            dS = P * (dP - (P * dP).sum(axis=1, keepdims=True))
+            dq[b, :, cols] = dS @ K / math.sqrt(dh)
+            dK, dV = dS.T @ Q / math.sqrt(dh), P.T @ dO
+            for n, j in enumerate(keys):
+                dkv[b, j, cols] = dK[n]
+                dkv[b, j, D:][cols] = dV[n]
+    return dq, dkv

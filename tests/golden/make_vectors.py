@@ -160,6 +160,19 @@ def update() -> None:
         dout = bf16(rng.standard_normal((B, NM, D)))
         out[f"{tag}_qkv"], out[f"{tag}_alive"], out[f"{tag}_heads"], out[f"{tag}_dout"] = qkv, alive, np.int64(H), dout
         out[f"{tag}_dqkv"] = bruteforce.sdpa_masked_grad_loops(qkv, alive, H, dout)
+    # bullet read backward: one environment without an active bullet, one with a single one
+    for tag, (B, N, NB, H) in {"cross_4v4": (4, 12, 80, 4), "cross_wide": (2, 40, 33, 4)}.items():
+        D = 32 * H
+        qkv = bf16(1.2 * rng.standard_normal((B, N, 3 * D)))
+        kv = bf16(1.2 * rng.standard_normal((B, NB, 2 * D)))
+        active = rng.random((B, NB)) < 0.3
+        active[0] = False
+        active[1] = False
+        active[1, NB // 3] = True
+        dout = bf16(rng.standard_normal((B, N, D)))
+        dq, dkv = bruteforce.bullet_read_grad_loops(qkv[..., :D], kv, active, H, dout)
+        out.update({f"{tag}_qkv": qkv, f"{tag}_kv": kv, f"{tag}_active": active, f"{tag}_heads": np.int64(H), f"{tag}_dout": dout,
+                    f"{tag}_dq": dq, f"{tag}_dkv": dkv})
     # sequence conv backward with episode ends and a gradient on the handed-on inputs
     R, T, D = 5, 11, 128
     b1 = bf16(rng.standard_normal((R, T, D)))

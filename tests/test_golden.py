@@ -237,3 +237,50 @@ def test_kernels_reproduce_conv_and_norm_gradient_vectors(b_dtype):
                              torch.from_numpy(UPD["norm_w"]).cuda())
     assert max_rel(dx.cpu().double(), torch.from_numpy(UPD["norm_dx"])) <= 1e-5
     assert max_rel(dw.cpu().double(), torch.from_numpy(UPD["norm_dw"])) <= 1e-5
+
+
+UPD_CROSS = ("cross_4v4", "cross_wide")
+
+
+@pytest.mark.parametrize("tag", UPD_CROSS)
+def test_autograd_of_the_oracle_reproduces_bullet_read_gradient_vectors(tag):
+    xq = torch.from_numpy(UPD[f"{tag}_qkv"]).double().requires_grad_()
+    xkv = torch.from_numpy(UPD[f"{tag}_kv"]).double().requires_grad_()
+    act, H = torch.from_numpy(UPD[f"{tag}_active"]), int(UPD[f"{tag}_heads"])
+    (torch_ref.bullet_read(xq, xkv, act, H) * torch.from_numpy(UPD[f"{tag}_dout"]).double()).sum().backward()
+    D = xkv.shape[-1] // 2
+    assert np.abs(xq.grad.numpy()[..., :D] - UPD[f"{tag}_dq"]).max() <= 1e-10 and not xq.grad[..., D:].any()
+    assert np.abs(xkv.grad.numpy() - UPD[f"{tag}_dkv"]).max() <= 1e-10
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tag", UPD_CROSS)
+@pytest.mark.parametrize("form", ["mask", "ranges"])
+def test_kernels_reproduce_bullet_read_gradient_vectors(tag, form):
+    from boost_and_broadside_amd import ops
+
+    qkv = torch.from_numpy(UPD[f"{tag}_qkv"]).bfloat16().cuda()
+    kv = torch.from_numpy(UPD[f"{tag}_kv"]).bfloat16().cuda()
+    act, H = torch.from_numpy(UPD[f"{tag}_active"]).cuda(), int(UPD[f"{tag}_heads"])
+    dout = torch.from_numpy(UPD[f"{tag}_dout"]).bfloat16().cuda()
+    want_dq, want_dkv = torch.from_numpy(UPD[f"{tag}_dq"]), torch.from_numpy(UPD[f"{tag}_dkv"])
+    B, NB, D2 = kv.shape
+    if form == "mask":
+        out = ops.sdpa_cross(qkv, kv, act, H)
+        dq, dkv = ops.sdpa_cross_bwd(qkv, kv, act, H, out, dout)
+        dkv = dkv.float().cpu()
+    else:
+        rows = ops.CompactRows(act)
+        total = rows.total_host()
+        kv_rows = kv.reshape(B * NB, D2)[act.reshape(-1)].contiguous()
+        out = ops.sdpa_cross_rows(qkv, kv_rows, rows, H, total=total)
+        dq, dkv_rows = ops.sdpa_cross_rows_bwd(qkv, kv_rows, rows, H, out, dout, total)
+        dkv = torch.zeros(B * NB, D2)
+        dkv[act.reshape(-1).cpu()] = dkv_rows.float().cpu()
+        dkv = dkv.reshape(B, NB, D2)
+    scale = float(want_dkv.abs().max())
+    # with a single active bullet the weights are constant and dq is zero up to float64 noise: measure against the
+    # gradients' common scale rather than dq's own maximum
+    assert float((dq.float().cpu().double() - want_dq).abs().max()) <= 2e-2 * max(float(want_dq.abs().max()), 1e-2 * scale)
+    assert max_rel(dkv.double(), want_dkv) <= 2e-2
+    assert not dq[0].any()  # no active bullet: gated off
