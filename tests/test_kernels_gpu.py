@@ -1888,3 +1888,76 @@ def test_sdpa_cross_rows_train_matches_autograd_of_the_oracle():
     (torch_ref.bullet_read(xq, xkv, mask, H) * up.bfloat16().double()).sum().backward()
     assert max_rel(qkv.grad.float().cpu().double(), xq.grad) <= BF16_TOL
     assert max_rel(kv_rows.grad.float().cpu().double(), xkv.grad.reshape(B * NK, 2 * D)[mask.reshape(-1)]) <= BF16_TOL
+
+
+# ------------------------------------------------------------------ element offsets past 2^31
+
+
+def _slices_of(n, width=2048):
+    return (slice(0, width), slice(n // 2, n // 2 + width), slice(n - width, n))
+
+
+def test_update_path_kernels_index_rows_whose_element_offsets_pass_2_31():
+    """Rollout-sized inputs (millions of token rows): the last rows must be as right as the first.
+
+    Every check compares a window at the start, the middle and the end of the rows against torch
+    on the same values; the weight gradient, a sum over all rows, against float64 in chunks.
+    """
+    import torch.nn.functional as F
+
+    gen = torch.Generator(device=DEV).manual_seed(11)
+    R = 2_300_000  # 1024 columns: offsets up to 2.36e9 elements
+    gu = torch.randn(R, 1024, device=DEV, generator=gen).bfloat16().requires_grad_()
+    out = ops.gelu_mul_packed_train(gu)
+    dout = torch.randn(R, 512, device=DEV, generator=gen).bfloat16()
+    out.backward(dout)
+    for sl in _slices_of(R):
+        g = gu.detach()[sl].float().requires_grad_()
+        ref = F.gelu(g[:, :512]).bfloat16().float() * g[:, 512:]
+        ref.backward(dout[sl].float())
+        assert max_rel(out[sl].detach().float(), ref.detach()) <= BF16_TOL
+        assert max_rel(gu.grad[sl].float(), g.grad) <= BF16_TOL
+
+    x = torch.randn(R, 128, device=DEV, generator=gen).bfloat16()
+    dy = gu.detach()[:, 512:]  # strided rows of the same buffer
+    got = ops.linear_wgrad(dy, x)
+    ref = torch.zeros(512, 128, device=DEV, dtype=torch.float64)
+    for s in range(0, R, 1 << 18):
+        ref += dy[s:s + (1 << 18)].double().t() @ x[s:s + (1 << 18)].double()
+    assert max_rel(got, ref) <= F32_TOL
+    del gu, out, dout, dy, x
+    torch.cuda.empty_cache()
+
+    R2 = 17_000_000  # 128 columns: offsets up to 2.18e9 elements
+    xs = torch.randn(R2, 128, device=DEV, generator=gen).requires_grad_()
+    w = (1 + 0.1 * torch.randn(128, device=DEV, generator=gen)).requires_grad_()
+    _, n = ops.rmsnorm_train(xs, w)
+    dn = torch.randn(R2, 128, device=DEV, generator=gen).to(n.dtype)
+    n.backward(dn)
+    eps = torch.finfo(torch.float32).eps
+    for sl in _slices_of(R2):
+        xr = xs.detach()[sl].clone().requires_grad_()
+        nr = F.rms_norm(xr, (128,), w.detach(), eps)
+        nr.backward(dn[sl].float())
+        assert max_rel(n[sl].detach().float(), nr.detach()) <= (BF16_TOL if n.dtype == torch.bfloat16 else F32_TOL)
+        assert max_rel(xs.grad[sl], xr.grad) <= F32_TOL
+    dw = torch.zeros(128, device=DEV, dtype=torch.float64)
+    for s in range(0, R2, 1 << 20):
+        xr = xs.detach()[s:s + (1 << 20)].double()
+        dw += (xr * torch.rsqrt(xr.square().mean(-1, keepdim=True) + eps) * dn[s:s + (1 << 20)].double()).sum(0)
+    assert max_rel(w.grad, dw) <= F32_TOL
+    del xs, n, dn
+    torch.cuda.empty_cache()
+
+    B, NM, H = 480_000, 12, 4  # 5.76 million token rows x 384 columns = 2.2e9 elements
+    qkv = torch.randn(B, NM, 384, device=DEV, generator=gen).bfloat16().requires_grad_()
+    alive = torch.rand(B, NM, device=DEV, generator=gen) < 0.8
+    o = ops.sdpa_train(qkv, alive, H)
+    do = torch.randn(B, NM, 128, device=DEV, generator=gen).bfloat16()
+    o.backward(do)
+    for sl in _slices_of(B, 256):
+        q = qkv.detach()[sl].float().cpu().requires_grad_()
+        r = torch_ref.sdpa_masked_softmax(q, alive[sl].cpu(), H)
+        r.backward(do[sl].float().cpu())
+        assert max_rel(o[sl].detach().float().cpu(), r.detach()) <= BF16_TOL
+        assert max_rel(qkv.grad[sl].float().cpu(), q.grad) <= BF16_TOL
