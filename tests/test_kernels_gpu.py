@@ -1961,3 +1961,73 @@ def test_update_path_kernels_index_rows_whose_element_offsets_pass_2_31():
         r.backward(do[sl].float().cpu())
         assert max_rel(o[sl].detach().float().cpu(), r.detach()) <= BF16_TOL
         assert max_rel(qkv.grad[sl].float().cpu(), q.grad) <= BF16_TOL
+
+
+def test_rollout_and_inference_kernels_index_rows_whose_element_offsets_pass_2_31():
+    """The same check for the sequence kernels, the bullet read (mask and list form), the sublayer tail
+    and norm + projection: a window at the start and one at the end of the rows against the oracle."""
+    import torch.nn.functional as F
+
+    gen = torch.Generator(device=DEV).manual_seed(12)
+
+    def randn(*shape):
+        return torch.randn(*shape, device=DEV, generator=gen)
+
+    R, T, D = 140_000, 128, 128  # 2.29e9 elements per (R, T, D) tensor
+    b1 = randn(R, T, D).bfloat16().requires_grad_()
+    cb = randn(R, 3, D).requires_grad_()
+    w, bias = randn(D, 4).requires_grad_(), randn(D).requires_grad_()
+    done = torch.rand(R, T, device=DEV, generator=gen) < 0.05
+    v, _ = ops.conv_seq_train(b1, cb, w, bias, done)
+    dv = randn(R, T, D)
+    v.backward(dv)
+    for sl in (slice(0, 48), slice(R - 48, R)):
+        b = b1.detach()[sl].float().cpu().requires_grad_()
+        c = cb.detach()[sl].cpu().requires_grad_()
+        r, _ = torch_ref.conv_sequence(b, c, w.detach().cpu(), bias.detach().cpu(), done[sl].cpu())
+        r.backward(dv[sl].cpu())
+        assert max_rel(v[sl].detach().cpu(), r.detach()) <= F32_TOL
+        assert max_rel(b1.grad[sl].float().cpu(), b.grad) <= BF16_TOL
+        assert max_rel(cb.grad[sl].cpu(), c.grad) <= F32_TOL
+    del b1, v, dv
+    torch.cuda.empty_cache()
+
+    x, gates = randn(R, T, D), randn(R, T, 2 * D)
+    lam, h0 = torch.linspace(0, 4, D, device=DEV), randn(R, D)
+    y, h_last = ops.rglru_scan(x, gates, lam, 8.0, h0, done)
+    for sl in (slice(0, 24), slice(R - 24, R)):
+        r, rh = torch_ref.rglru_sequence(x[sl].cpu(), gates[sl].cpu(), lam.cpu(), 8.0, h0[sl].cpu(), done[sl].cpu())
+        assert max_rel(y[sl].cpu(), r) <= 2e-5
+        assert max_rel(h_last[sl].cpu(), rh) <= 2e-5
+    del x, gates, y, h_last
+    torch.cuda.empty_cache()
+
+    B, NQ, NK, H = 6000, 12, 1520, 4  # keys and values: 2.33e9 elements
+    qkv, kv = randn(B, NQ, 384).bfloat16(), randn(B, NK, 256).bfloat16()
+    mask = torch.rand(B, NK, device=DEV, generator=gen) < 0.1
+    o = ops.sdpa_cross(qkv, kv, mask, H)
+    rows = ops.CompactRows(mask)
+    kv_rows = torch.zeros(B * NK, 256, device=DEV, dtype=torch.bfloat16)
+    kv_rows[: rows.total_host()] = kv.reshape(B * NK, 256)[mask.reshape(-1)]
+    o2 = ops.sdpa_cross_rows(qkv, kv_rows, rows, H)
+    for sl in (slice(0, 16), slice(B - 16, B)):
+        r = torch_ref.bullet_read(qkv[sl].float().cpu(), kv[sl].float().cpu(), mask[sl].cpu(), H)
+        assert max_rel(o[sl].float().cpu(), r) <= BF16_TOL
+        assert max_rel(o2[sl].float().cpu(), r) <= BF16_TOL
+    del qkv, kv, o, o2, kv_rows
+    torch.cuda.empty_cache()
+
+    R2 = 17_000_000  # 2.18e9 elements per (R2, 128) tensor
+    xs, delta, nw = randn(R2, 128), randn(R2, 128).bfloat16(), 1 + 0.1 * randn(128)
+    gw, uw, dw = randn(512, 128) / 11, randn(512, 128) / 11, randn(128, 512) / 22
+    wq = randn(384, 128) / 11
+    out = ops.ffn_fused(xs, delta, nw, ops.pack_ffn_weights(gw, uw, dw))
+    q = ops.norm_linear(xs, nw, ops.pack_linear_weights(wq))
+    eps = torch.finfo(torch.float32).eps
+    for sl in (slice(0, 2048), slice(R2 - 2048, R2)):
+        s = xs[sl] + delta[sl].float()
+        n = F.rms_norm(s, (128,), nw, eps).bfloat16()
+        hidden = F.gelu(F.linear(n, gw.bfloat16())) * F.linear(n, uw.bfloat16())
+        assert max_rel(out[sl], s + F.linear(hidden, dw.bfloat16()).float()) <= BF16_TOL
+        r = F.linear(F.rms_norm(xs[sl], (128,), nw, eps).bfloat16(), wq.bfloat16())
+        assert max_rel(q[sl].float(), r.float()) <= BF16_TOL
