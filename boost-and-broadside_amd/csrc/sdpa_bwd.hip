@@ -256,7 +256,11 @@ constexpr int kMbPitch = kSbDh + 8;  // halfs per token row in LDS (80 bytes: 16
 // models/yemong/attention.py:149-166): an environment without a live key contributed exactly nothing
 // in the forward (the reference gates it off), so all its gradients are zero; `out` is that read's own
 // result, before it was added to anything.
-template <int NB, bool CROSS>
+// PAIR (NB = 1, up to 16 tokens, an even number of heads): two heads of one environment share the tile, as
+// in the forward kernel for small fleets.  Row r of every staged operand is token r % 16 of head
+// 2 * pair + r / 16, and the score blocks between the two heads start at -inf like a dead key, so P and
+// dS are exactly zero there and every second product returns each head's gradient in its own columns.
+template <int NB, bool CROSS, bool PAIR>
 __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
     const uint16_t *__restrict__ q, int64_t q_row_stride, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
     int64_t kv_row_stride, const uint8_t *__restrict__ alive, const int32_t *__restrict__ ranges, int64_t kv_capacity,
@@ -274,9 +278,14 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
 
     const int chunk = gridDim.x >> 3;
     const int logical = (blockIdx.x & 7) * chunk + (blockIdx.x >> 3);  // the heads of an environment on one XCD
-    if (logical >= B * H) return;
-    const int env = logical / H, head = logical - env * H;
+    const int per_env = PAIR ? H >> 1 : H;  // work-groups per environment
+    if (logical >= B * per_env) return;
+    const int env = logical / per_env, head = (logical - env * per_env) * (PAIR ? 2 : 1);  // PAIR: the first head of the pair
     const int D = H * kSbDh;
+    static_assert(!PAIR || (NB == 1 && !CROSS), "two heads share one 32 x 32 tile of self-attention");
+    // tile row -> (token, first channel of its head)
+    auto tok_of = [&](int r) { return PAIR ? r & 15 : r; };
+    auto ch_of = [&](int r) { return (head + (PAIR ? r >> 4 : 0)) * kSbDh; };
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int m = lane & 31, half = lane >> 5;
@@ -304,11 +313,11 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
             const int item = tid + it * NT;
-            const int tok = item >> 2, c8 = (item & 3) * 8;
+            const int tile_row = item >> 2, tok = tok_of(tile_row), c8 = (item & 3) * 8 + ch_of(tile_row);
             const int safe = tok < n ? tok : (n > 0 ? n - 1 : 0);
             const int64_t row = n > 0 ? base + safe : 0;  // an empty range reads row 0 of the buffer and discards it
-            const u32x4 aw = *reinterpret_cast<const u32x4 *>(a + row * a_stride + head * kSbDh + c8);
-            const u32x4 bw = *reinterpret_cast<const u32x4 *>(b + row * b_stride + head * kSbDh + c8);
+            const u32x4 aw = *reinterpret_cast<const u32x4 *>(a + row * a_stride + c8);
+            const u32x4 bw = *reinterpret_cast<const u32x4 *>(b + row * b_stride + c8);
             r.a[it] = tok < n ? aw : zero4;
             r.b[it] = tok < n ? bw : zero4;
         }
@@ -349,26 +358,31 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
         return r;
     };
     // a (32 channels x 32 tokens) accumulator to rows of a gradient tensor: lane = token, rows = channels 8i + 4*half + j
-    auto store_grad = [&](const f32x16 &acc, uint16_t *base, int64_t row_stride, int64_t first_row, int tok, int n) {
+    auto store_grad = [&](const f32x16 &acc, uint16_t *base, int64_t row_stride, int64_t first_row, int tile_row, int n) {
+        const int tok = tok_of(tile_row);
         if (tok >= n) return;
-        uint16_t *dst = base + (first_row + tok) * row_stride + head * kSbDh + 4 * half;
+        uint16_t *dst = base + (first_row + tok) * row_stride + ch_of(tile_row) + 4 * half;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             *reinterpret_cast<u32x2 *>(dst + 8 * i) = u32x2{pack_bf16x2(acc[4 * i], acc[4 * i + 1]), pack_bf16x2(acc[4 * i + 2], acc[4 * i + 3])};
     };
 
     // ---- every global load of the kernel ----
-    const int own = wave * 32 + m;  // this lane's query in pass 1, its key in pass 2
+    const int own = wave * 32 + m;  // this lane's query in pass 1, its key in pass 2 (a tile row)
+    const int own_tok = tok_of(own), own_ch = ch_of(own);
     const int64_t q_base = (int64_t)env * NQ;
-    const int64_t q_row = q_base + (own < NQ ? own : NQ - 1);
-    const int64_t k_row = NK > 0 ? k_base + (own < NK ? own : NK - 1) : 0;
-    const int64_t own_q = q_row * q_row_stride + head * kSbDh + half * 8, own_o = q_row * D + head * kSbDh + half * 8;
-    const int64_t own_k = k_row * kv_row_stride + head * kSbDh + half * 8;
+    const int64_t q_row = q_base + (own_tok < NQ ? own_tok : NQ - 1);
+    const int64_t k_row = NK > 0 ? k_base + (own_tok < NK ? own_tok : NK - 1) : 0;
+    const int64_t own_q = q_row * q_row_stride + own_ch + half * 8, own_o = q_row * D + own_ch + half * 8;
+    const int64_t own_k = k_row * kv_row_stride + own_ch + half * 8;
     bool any_live = false, my_live = false;
     if (tid < CAP) {  // CAP <= NT
-        my_live = tid < NK && (alive == nullptr || ranges != nullptr || alive[k_base + tid] != 0);
+        const int t = tok_of(tid);
+        my_live = t < NK && (alive == nullptr || ranges != nullptr || alive[k_base + t] != 0);
         any_live = my_live;
     }
+    // PAIR: accumulator rows 0..15 (v < 8) belong to the first head, 16..31 to the second; a lane's column to head m / 16
+    auto other_head = [&](int vv) { return PAIR && ((vv >> 3) != (m >> 4)); };
     const Staged kv_in = stage_load(k, kv_row_stride, v, kv_row_stride, k_base, NK);
     u32x4 w0 = *reinterpret_cast<const u32x4 *>(q + own_q), w1 = *reinterpret_cast<const u32x4 *>(q + own_q + 16);
     u32x4 g0 = *reinterpret_cast<const u32x4 *>(dout + own_o), g1 = *reinterpret_cast<const u32x4 *>(dout + own_o + 16);
@@ -390,7 +404,7 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
         return;
     }
     const bool uniform = none_live;  // self-attention without a live key: equal weights over all keys
-    if (tid < CAP) s_bias[tid] = (uniform ? tid < NK : my_live) ? 0.0f : -INFINITY;
+    if (tid < CAP) s_bias[tid] = (uniform ? tok_of(tid) < NK : my_live) ? 0.0f : -INFINITY;
     stage_store(kv_in, true, false);
     __syncthreads();
 
@@ -408,7 +422,7 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
         for (int e = 0; e < 8; ++e) d = fmaf(a0.v[e], o0.v[e], fmaf(a1.v[e], o1.v[e], d));
         delta = d + __shfl_xor(d, 32);
     }
-    if (own >= NQ) w0 = w1 = g0 = g1 = zero4, delta = 0.0f;  // padding queries: nothing flows through them
+    if (own_tok >= NQ) w0 = w1 = g0 = g1 = zero4, delta = 0.0f;  // padding queries: nothing flows through them
     const bf16x8 qs0 = __builtin_bit_cast(bf16x8, uniform ? zero4 : w0), qs1 = __builtin_bit_cast(bf16x8, uniform ? zero4 : w1);
     const bf16x8 gb0 = __builtin_bit_cast(bf16x8, g0), gb1 = __builtin_bit_cast(bf16x8, g1);
 
@@ -419,6 +433,10 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
             for (int i = 0; i < 4; ++i) {
                 const f32x4 b4 = *reinterpret_cast<const f32x4 *>(s_bias + kb * 32 + 8 * i + 4 * half);
                 z[4 * i] = b4.x, z[4 * i + 1] = b4.y, z[4 * i + 2] = b4.z, z[4 * i + 3] = b4.w;
+            }
+            if (PAIR) {
+#pragma unroll
+                for (int vv = 0; vv < 16; ++vv) z[vv] = other_head(vv) ? -INFINITY : z[vv];
             }
             bf16x8 k0, k1;
             row_operand(s_rows[0], kb * 32 + m, k0, k1);
@@ -464,7 +482,7 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
     // ---- pass 2: this wave's keys ----
     stage_store(qd_in, true, true);
     const float col_bias = s_bias[own];
-    if (own >= NK) kw0 = kw1 = vw0 = vw1 = zero4;
+    if (own_tok >= NK) kw0 = kw1 = vw0 = vw1 = zero4;
     const bf16x8 ks0 = __builtin_bit_cast(bf16x8, uniform ? zero4 : kw0), ks1 = __builtin_bit_cast(bf16x8, uniform ? zero4 : kw1);
     const bf16x8 vb0 = __builtin_bit_cast(bf16x8, vw0), vb1 = __builtin_bit_cast(bf16x8, vw1);
     __syncthreads();
@@ -474,7 +492,7 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
     for (int qb = 0; qb < nqb; ++qb) {
         f32x16 z;
 #pragma unroll
-        for (int vv = 0; vv < 16; ++vv) z[vv] = col_bias;
+        for (int vv = 0; vv < 16; ++vv) z[vv] = other_head(vv) ? -INFINITY : col_bias;
         bf16x8 a0, a1;
         row_operand(s_rows[0], qb * 32 + m, a0, a1);
         z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, ks0, z, 0, 0, 0);
@@ -505,15 +523,15 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
     store_grad(dv, dv_out, dkv_row_stride, k_base, own, NK);
 }
 
-template <int NB, bool CROSS>
+template <int NB, bool CROSS, bool PAIR = false>
 static int launch_sdpa_bwd_mfma(const void *q, int64_t q_row_stride, const void *k, const void *v, int64_t kv_row_stride,
                                 const uint8_t *alive, const int32_t *ranges, int64_t kv_capacity, const void *out, const void *dout,
                                 void *dq, int64_t dq_row_stride, void *dk, void *dv, int64_t dkv_row_stride, int64_t B, int NQ,
                                 int NK, int H, hipStream_t stream)
 {
-    const int64_t groups = (B * H + 7) / 8 * 8;  // a multiple of 8: the XCD mapping deals whole rounds
+    const int64_t groups = (B * (PAIR ? H / 2 : H) + 7) / 8 * 8;  // a multiple of 8: the XCD mapping deals whole rounds
     if (groups > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<NB, CROSS>), dim3((unsigned)groups), dim3(kWave * NB), 0, stream, (const uint16_t *)q,
+    hipLaunchKernelGGL((sdpa_bwd_mfma_kernel<NB, CROSS, PAIR>), dim3((unsigned)groups), dim3(kWave * NB), 0, stream, (const uint16_t *)q,
                        q_row_stride, (const uint16_t *)k, (const uint16_t *)v, kv_row_stride, alive, ranges, kv_capacity,
                        (const uint16_t *)out, (const uint16_t *)dout, (uint16_t *)dq, dq_row_stride, (uint16_t *)dk, (uint16_t *)dv, dkv_row_stride, (int)B,
                        NQ, NK, H, 1.0f / sqrtf((float)kSbDh));
@@ -527,6 +545,9 @@ static int dispatch_sdpa_bwd_mfma(const void *q, int64_t q_row_stride, const voi
                                   int NK, int H, hipStream_t s)
 {
     const int nb = ((NQ > NK ? NQ : NK) + 31) / 32;
+    if (!CROSS && NQ <= 16 && H % 2 == 0)
+        return launch_sdpa_bwd_mfma<1, false, true>(q, q_row_stride, k, v, kv_row_stride, alive, ranges, kv_capacity, out, dout, dq,
+                                                    dq_row_stride, dk, dv, dkv_row_stride, B, NQ, NK, H, s);
 #define BNB_SBM(NBV) \
     return launch_sdpa_bwd_mfma<NBV, CROSS>(q, q_row_stride, k, v, kv_row_stride, alive, ranges, kv_capacity, out, dout, dq, \
                                             dq_row_stride, dk, dv, dkv_row_stride, B, NQ, NK, H, s)

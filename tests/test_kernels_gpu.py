@@ -1758,7 +1758,9 @@ def test_gelu_mul_packed_train_equals_the_two_operand_form():
 
 
 @pytest.mark.parametrize("B,NM,H", [(3, 12, 4), (5, 27, 4), (4, 1, 4), (6, 32, 4), (5, 33, 4), (4, 64, 4), (3, 84, 4), (2, 152, 4),
-                                    (2, 160, 4), (3, 100, 2), (300, 40, 4)])
+                                    (2, 160, 4), (3, 100, 2), (300, 40, 4),
+                                    # two heads per tile (up to 16 tokens, even head count) and its neighbours
+                                    (70, 12, 4), (9, 7, 2), (5, 16, 4), (3, 15, 8), (4, 17, 4), (6, 12, 3), (1001, 12, 4)])
 @pytest.mark.parametrize("p_alive", [1.0, 0.7, 0.0])
 def test_sdpa_masked_bwd_on_the_matrix_cores_matches_autograd_of_the_oracle(B, NM, H, p_alive):
     D = 32 * H
