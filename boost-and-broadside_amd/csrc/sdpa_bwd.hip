@@ -261,7 +261,7 @@ constexpr int kMbPitch = kSbDh + 8;  // halfs per token row in LDS (80 bytes: 16
 // 2 * pair + r / 16, and the score blocks between the two heads start at -inf like a dead key, so P and
 // dS are exactly zero there and every second product returns each head's gradient in its own columns.
 template <int NB, bool CROSS, bool PAIR>
-__global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
+__global__ __launch_bounds__(kWave * NB) __attribute__((amdgpu_waves_per_eu(NB == 1 && !PAIR ? 3 : 4))) void sdpa_bwd_mfma_kernel(
     const uint16_t *__restrict__ q, int64_t q_row_stride, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
     int64_t kv_row_stride, const uint8_t *__restrict__ alive, const int32_t *__restrict__ ranges, int64_t kv_capacity,
     const uint16_t *__restrict__ out, const uint16_t *__restrict__ dout, uint16_t *__restrict__ dq_out, int64_t dq_row_stride,
@@ -271,7 +271,10 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
     constexpr int CAP = NB * 32;
     constexpr int TP = CAP + 4;  // halfs per row of a transposed copy
     constexpr int NT = kWave * NB;
-    __shared__ __align__(16) uint16_t s_rows[2][CAP * kMbPitch];  // [K | V], later [Q | dO]: token-major
+    // with one block of 32 tokens a lane's own rows (loaded below for the other orientation) are the
+    // token-major operands too, so no token-major copy is staged
+    constexpr bool OWN_ROWS = NB == 1;
+    __shared__ __align__(16) uint16_t s_rows[2][OWN_ROWS ? 8 : CAP * kMbPitch];  // [K | V], later [Q | dO]: token-major
     __shared__ __align__(16) uint16_t s_tr[2][kSbDh * TP];        // K^T, later [Q^T | dO^T]: channel-major
     __shared__ __align__(16) float s_lse[CAP], s_delta[CAP];
     __shared__ __align__(16) float s_bias[CAP];  // 0 for a key that takes part, -inf for a dead or padding key
@@ -308,7 +311,8 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
     struct Staged {
         u32x4 a[2], b[2];
     };
-    auto stage_load = [&](const uint16_t *a, int64_t a_stride, const uint16_t *b, int64_t b_stride, int64_t base, int n) -> Staged {
+    auto stage_load = [&](const uint16_t *a, int64_t a_stride, const uint16_t *b, int64_t b_stride, int64_t base, int n,
+                          bool need_b) -> Staged {
         Staged r;
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
@@ -317,9 +321,12 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
             const int safe = tok < n ? tok : (n > 0 ? n - 1 : 0);
             const int64_t row = n > 0 ? base + safe : 0;  // an empty range reads row 0 of the buffer and discards it
             const u32x4 aw = *reinterpret_cast<const u32x4 *>(a + row * a_stride + c8);
-            const u32x4 bw = *reinterpret_cast<const u32x4 *>(b + row * b_stride + c8);
             r.a[it] = tok < n ? aw : zero4;
-            r.b[it] = tok < n ? bw : zero4;
+            r.b[it] = zero4;
+            if (need_b) {
+                const u32x4 bw = *reinterpret_cast<const u32x4 *>(b + row * b_stride + c8);
+                r.b[it] = tok < n ? bw : zero4;
+            }
         }
         return r;
     };
@@ -328,8 +335,10 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
         for (int it = 0; it < 2; ++it) {
             const int item = tid + it * NT;
             const int tok = item >> 2, c8 = (item & 3) * 8;
-            *reinterpret_cast<u32x4 *>(s_rows[0] + tok * kMbPitch + c8) = r.a[it];
-            *reinterpret_cast<u32x4 *>(s_rows[1] + tok * kMbPitch + c8) = r.b[it];
+            if (!OWN_ROWS) {
+                *reinterpret_cast<u32x4 *>(s_rows[0] + tok * kMbPitch + c8) = r.a[it];
+                *reinterpret_cast<u32x4 *>(s_rows[1] + tok * kMbPitch + c8) = r.b[it];
+            }
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const uint32_t wa = r.a[it][e >> 1], wb = r.b[it][e >> 1];
@@ -383,13 +392,13 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
     }
     // PAIR: accumulator rows 0..15 (v < 8) belong to the first head, 16..31 to the second; a lane's column to head m / 16
     auto other_head = [&](int vv) { return PAIR && ((vv >> 3) != (m >> 4)); };
-    const Staged kv_in = stage_load(k, kv_row_stride, v, kv_row_stride, k_base, NK);
+    const Staged kv_in = stage_load(k, kv_row_stride, v, kv_row_stride, k_base, NK, !OWN_ROWS);
     u32x4 w0 = *reinterpret_cast<const u32x4 *>(q + own_q), w1 = *reinterpret_cast<const u32x4 *>(q + own_q + 16);
     u32x4 g0 = *reinterpret_cast<const u32x4 *>(dout + own_o), g1 = *reinterpret_cast<const u32x4 *>(dout + own_o + 16);
     const Row8 o0 = load8(out + own_o), o1 = load8(out + own_o + 16);
     u32x4 kw0 = *reinterpret_cast<const u32x4 *>(k + own_k), kw1 = *reinterpret_cast<const u32x4 *>(k + own_k + 16);
     u32x4 vw0 = *reinterpret_cast<const u32x4 *>(v + own_k), vw1 = *reinterpret_cast<const u32x4 *>(v + own_k + 16);
-    const Staged qd_in = stage_load(q, q_row_stride, dout, D, q_base, NQ);
+    const Staged qd_in = stage_load(q, q_row_stride, dout, D, q_base, NQ, true);
 
     // ---- live keys ----
     const bool none_live = __syncthreads_or(any_live ? 1 : 0) == 0;
@@ -423,6 +432,7 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
         delta = d + __shfl_xor(d, 32);
     }
     if (own_tok >= NQ) w0 = w1 = g0 = g1 = zero4, delta = 0.0f;  // padding queries: nothing flows through them
+    if (own_tok >= NK) kw0 = kw1 = vw0 = vw1 = zero4;
     const bf16x8 qs0 = __builtin_bit_cast(bf16x8, uniform ? zero4 : w0), qs1 = __builtin_bit_cast(bf16x8, uniform ? zero4 : w1);
     const bf16x8 gb0 = __builtin_bit_cast(bf16x8, g0), gb1 = __builtin_bit_cast(bf16x8, g1);
 
@@ -439,7 +449,10 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
                 for (int vv = 0; vv < 16; ++vv) z[vv] = other_head(vv) ? -INFINITY : z[vv];
             }
             bf16x8 k0, k1;
-            row_operand(s_rows[0], kb * 32 + m, k0, k1);
+            if (OWN_ROWS)
+                k0 = __builtin_bit_cast(bf16x8, kw0), k1 = __builtin_bit_cast(bf16x8, kw1);
+            else
+                row_operand(s_rows[0], kb * 32 + m, k0, k1);
             z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k0, qs0, z, 0, 0, 0);
             return __builtin_amdgcn_mfma_f32_32x32x16_bf16(k1, qs1, z, 0, 0, 0);
         };
@@ -465,7 +478,10 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
         for (int kb = 0; kb < nkb; ++kb) {
             const f32x16 z = scores_t(kb);
             bf16x8 v0, v1;
-            row_operand(s_rows[1], kb * 32 + m, v0, v1);
+            if (OWN_ROWS)
+                v0 = __builtin_bit_cast(bf16x8, vw0), v1 = __builtin_bit_cast(bf16x8, vw1);
+            else
+                row_operand(s_rows[1], kb * 32 + m, v0, v1);
             f32x16 dp = {0.0f};
             dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, gb0, dp, 0, 0, 0);
             dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, gb1, dp, 0, 0, 0);
@@ -482,7 +498,6 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
     // ---- pass 2: this wave's keys ----
     stage_store(qd_in, true, true);
     const float col_bias = s_bias[own];
-    if (own_tok >= NK) kw0 = kw1 = vw0 = vw1 = zero4;
     const bf16x8 ks0 = __builtin_bit_cast(bf16x8, uniform ? zero4 : kw0), ks1 = __builtin_bit_cast(bf16x8, uniform ? zero4 : kw1);
     const bf16x8 vb0 = __builtin_bit_cast(bf16x8, vw0), vb1 = __builtin_bit_cast(bf16x8, vw1);
     __syncthreads();
@@ -494,10 +509,16 @@ __global__ __launch_bounds__(kWave * NB) void sdpa_bwd_mfma_kernel(
 #pragma unroll
         for (int vv = 0; vv < 16; ++vv) z[vv] = other_head(vv) ? -INFINITY : col_bias;
         bf16x8 a0, a1;
-        row_operand(s_rows[0], qb * 32 + m, a0, a1);
+        if (OWN_ROWS)
+            a0 = __builtin_bit_cast(bf16x8, w0), a1 = __builtin_bit_cast(bf16x8, w1);
+        else
+            row_operand(s_rows[0], qb * 32 + m, a0, a1);
         z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, ks0, z, 0, 0, 0);
         z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, ks1, z, 0, 0, 0);
-        row_operand(s_rows[1], qb * 32 + m, a0, a1);
+        if (OWN_ROWS)
+            a0 = gb0, a1 = gb1;
+        else
+            row_operand(s_rows[1], qb * 32 + m, a0, a1);
         f32x16 dp = {0.0f};
         dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, vb0, dp, 0, 0, 0);
         dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, vb1, dp, 0, 0, 0);
