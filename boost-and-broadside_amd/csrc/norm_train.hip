@@ -19,7 +19,7 @@
 namespace bnb {
 
 constexpr int kNbThreads = 256;
-constexpr int kNbMaxBlocks = 2048;  // eight work-groups per CU keep enough loads in flight
+constexpr int kNbMaxBlocks = 1280;  // five work-groups per CU: what 80-98 registers per lane let run at once, so no work-group waits for a free slot
 
 template <int LANES, typename GT, bool HAS_SUM>
 __global__ __launch_bounds__(kNbThreads) void rmsnorm_bwd_kernel(
@@ -41,14 +41,17 @@ __global__ __launch_bounds__(kNbThreads) void rmsnorm_bwd_kernel(
     int64_t row = (int64_t)blockIdx.x * ROWS + local_row;
     int64_t r = row < R ? row : R - 1;
     Row8 xn = load8_stream(x + r * x_stride + d0), gn = load8_stream(dy + r * dy_stride + d0);
+    Row8 sn = xn;  // the bypass gradient travels with the other two rows, one iteration ahead
+    if (HAS_SUM) sn = load8_stream(grad_sum + r * D + d0);
     for (int64_t base = (int64_t)blockIdx.x * ROWS; base < R; base += step) {
-        const Row8 xv = xn, gv = gn;
+        const Row8 xv = xn, gv = gn, sv = sn;
         const int64_t cur = row;
         const bool valid = cur < R;
         row += step;
         if (base + step < R) {
             r = row < R ? row : R - 1;
             xn = load8_stream(x + r * x_stride + d0), gn = load8_stream(dy + r * dy_stride + d0);
+            if (HAS_SUM) sn = load8_stream(grad_sum + r * D + d0);
         }
         float ss = 0.0f, dot = 0.0f;
         Row8 g;
@@ -73,12 +76,12 @@ __global__ __launch_bounds__(kNbThreads) void rmsnorm_bwd_kernel(
             dw[e] = fmaf(gv.v[e] * rstd, xv.v[e], dw[e]);
         }
         if (HAS_SUM) {
-            const Row8 s = load8_stream(grad_sum + cur * D + d0);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o.v[e] += s.v[e];
+            for (int e = 0; e < 8; ++e) o.v[e] += sv.v[e];
         }
         store8_stream(dx + cur * D + d0, o);
-        if (dx_bf16 != nullptr) store8_stream(dx_bf16 + cur * D + d0, o);
+        // an ordinary store: as a third nontemporal stream this copy cost 50 us more on some allocations
+        if (dx_bf16 != nullptr) store8(dx_bf16 + cur * D + d0, o);
     }
 
 #pragma unroll
