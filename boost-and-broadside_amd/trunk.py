@@ -746,6 +746,30 @@ class TeamPMA(nn.Module):
         return pool.gather(1, team_id.clamp(0, 1).long().unsqueeze(-1).expand(B, N, D))
 
 
+class _SplitTokens(torch.autograd.Function):
+    """``(x[:, :, :n], x[:, :, n:])`` of a (T, B, NM, D) tensor as two contiguous tensors.  The backward is one
+    concatenation; autograd's own slicing would fill two full-size zero tensors, copy a slice into each and
+    add them."""
+
+    @staticmethod
+    def forward(ctx, x, n):
+        ctx.n = n
+        ctx.shape = x.shape
+        return x[:, :, :n].contiguous(), x[:, :, n:].contiguous()
+
+    @staticmethod
+    def backward(ctx, d_first, d_rest):
+        T, B, NM, D = ctx.shape
+        if d_first is None and d_rest is None:
+            return None, None
+        like = d_first if d_first is not None else d_rest
+        if d_first is None:
+            d_first = like.new_zeros(T, B, ctx.n, D)
+        if d_rest is None:
+            d_rest = like.new_zeros(T, B, NM - ctx.n, D)
+        return torch.cat([d_first, d_rest], dim=2), None
+
+
 class YemongBlock(nn.Module):
     """``n_spatial_per_block`` attention sublayers, then ``n_temporal_per_block`` recurrent ones."""
 
@@ -831,11 +855,15 @@ class YemongBlock(nn.Module):
         new_h, new_cb = [], []
         for j, layer in enumerate(self.temporal):
             # the sequence kernels read (T, rows, D) as stored: no transposed copies of the rollout
-            ships = x[:, :, :n_rec].reshape(T, B * n_rec, D)
-            out, h_j, cb_j = layer.forward_sequence(ships, h0[j], conv_buf0[j], done_rows, time_major=True)
+            if NM > n_rec and x.requires_grad:
+                ships, fields = _SplitTokens.apply(x, n_rec)
+            else:
+                ships, fields = x[:, :, :n_rec], x[:, :, n_rec:]
+            out, h_j, cb_j = layer.forward_sequence(ships.reshape(T, B * n_rec, D), h0[j], conv_buf0[j], done_rows,
+                                                    time_major=True)
             parts = [out.reshape(T, B, n_rec, D)]
             if NM > n_rec:
-                parts.append(layer.forward_nonrecurrent(x[:, :, n_rec:], self.field_sub[j]))
+                parts.append(layer.forward_nonrecurrent(fields, self.field_sub[j]))
             x = torch.cat(parts, dim=2) if len(parts) > 1 else parts[0]
             new_h.append(h_j)
             new_cb.append(cb_j)
