@@ -419,7 +419,10 @@ class RGLRU(nn.Module):
 
         ``x_act``: the same rows already in the projection dtype (saves the cast)."""
         if torch.is_grad_enabled():
-            return torch.cat([_project(self.linear_a, x), _project(self.linear_x, x)], dim=-1)
+            # the (small) weights are concatenated, not the activations: one cast of x, one GEMM, one weight gradient
+            w = torch.cat([self.linear_a.weight, self.linear_x.weight], dim=0)
+            b = torch.cat([self.linear_a.bias, self.linear_x.bias], dim=0)
+            return _grad_linear(x, w, b)
         act = _projection_dtype()
         if x_act is None or x_act.dtype != act:
             x_act = x.to(act)
