@@ -153,3 +153,30 @@ def test_inputs_are_seeded_and_typed():
     assert t1.dtype == torch.bfloat16 and s1.dtype == torch.float32 and s1.shape == (64, 128)
     p = harness.make_weights(w.seed, w.dtype)
     assert p["qkv.weight"].shape == (384, 128) and p["log_lambda"].dtype == torch.float32
+
+
+@pytest.mark.parametrize("use", ["both", "first", "rest"])
+def test_token_split_has_the_gradient_of_plain_slicing(use):
+    """The ship/field split of the update path (one concatenation in its backward) against autograd's own slicing."""
+    from boost_and_broadside_amd.trunk import _SplitTokens
+
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(3, 2, 5, 4, generator=g, dtype=torch.float64)
+    wa, wb = torch.randn(3, 2, 3, 4, generator=g, dtype=torch.float64), torch.randn(3, 2, 2, 4, generator=g, dtype=torch.float64)
+
+    def loss(first, rest):
+        total = x.new_zeros(())
+        if use in ("both", "first"):
+            total = total + (first * wa).sum()
+        if use in ("both", "rest"):
+            total = total + (rest.square() * wb).sum()
+        return total
+
+    xs = x.clone().requires_grad_()
+    first, rest = _SplitTokens.apply(xs, 3)
+    assert first.is_contiguous() and rest.is_contiguous()
+    assert torch.equal(first, x[:, :, :3]) and torch.equal(rest, x[:, :, 3:])
+    loss(first, rest).backward()
+    xr = x.clone().requires_grad_()
+    loss(xr[:, :, :3], xr[:, :, 3:]).backward()
+    assert torch.equal(xs.grad, xr.grad)

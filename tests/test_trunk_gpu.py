@@ -480,6 +480,56 @@ def test_block_sequence_trains_and_matches_the_no_grad_path():
     assert block.temporal[0].rg_lru.log_lambda.grad.abs().max() > 0
 
 
+@pytest.mark.parametrize("N,M", [(4, 2), (5, 0)])
+def test_block_sequence_gradients_match_autograd_through_the_oracle_step_loop(N, M):
+    """Gradients of every parameter, of x and of the initial state through ``YemongBlock.sequence`` (float32: norm,
+    conv, gelu-gate, attention and recurrence backward kernels, ship/field split) against autograd in float64 through
+    the oracle's one-step block applied T times with the state carried and cut at episode ends."""
+    D, H, T, B, spatial, temporal = 128, 4, 7, 3, 2, 1
+    gen = torch.Generator().manual_seed(41 + N)
+    p = block_params(gen, "b.", D, spatial, temporal)
+    block = bnb.YemongBlock(_cfg(D, H, 1, spatial, temporal))
+    block.load_state_dict(_strip(p, "b."))
+    block.to(DEV)
+    x = torch.randn(T, B, N + M, D, generator=gen)
+    alive = torch.rand(T, B, N + M, generator=gen) < 0.8
+    alive[..., 0] = True
+    h0 = 0.5 * torch.randn(temporal, B * N, D, generator=gen)
+    cb0 = torch.randn(temporal, B * N, 3, D, generator=gen)
+    done = torch.rand(T, B, generator=gen) < 0.3
+    # the sequence form returns the last three conv inputs as they are (griffin.py:275-277), the step loop the buffer
+    # it zeroed at an episode end: the two agree once three steps have followed the last end
+    done[T - 3:] = False
+    done[1, 0] = True
+    up = torch.randn(T, B, N + M, D, generator=gen)
+
+    xg, hg, cg = (t.to(DEV).requires_grad_() for t in (x, h0, cb0))
+    out, h1, cb1 = block.sequence(xg, alive.to(DEV), hg, cg, done.to(DEV), N)
+    ((out * up.to(DEV)).sum() + h1.square().sum() + cb1.sum()).backward()
+
+    pd = {k: v.double().requires_grad_() for k, v in p.items()}
+    xr, hr, cr = (t.double().requires_grad_() for t in (x, h0, cb0))
+    h, cb, outs = hr, cr, []
+    for t in range(T):
+        if t > 0:  # a step that follows the end of an episode starts from the zero state (policy.py:268-285)
+            keep = (~done[t - 1]).double().repeat_interleave(N)
+            h, cb = h * keep[None, :, None], cb * keep[None, :, None, None]
+        o, h, cb = torch_ref.block_step(pd, "b.", spatial, temporal, H, xr[t], alive[t], h, cb, N)
+        outs.append(o)
+    ref = torch.stack(outs)
+    ((ref * up.double()).sum() + h.square().sum() + cb.sum()).backward()
+
+    assert max_rel(out.detach().cpu(), ref.detach()) <= 2e-5
+    assert max_rel(xg.grad.cpu(), xr.grad) <= 1e-4
+    assert max_rel(hg.grad.cpu(), hr.grad) <= 1e-4 and max_rel(cg.grad.cpu(), cr.grad) <= 1e-4
+    for name, param in block.named_parameters():
+        want = pd["b." + name].grad
+        if want is None:  # without field tokens their projection takes no part
+            assert M == 0 and name.startswith("field_sub") and (param.grad is None or not param.grad.any()), name
+            continue
+        assert max_rel(param.grad.cpu(), want) <= 2e-4, name
+
+
 @pytest.mark.parametrize("autocast", [False, True])
 @pytest.mark.parametrize("D,H", [(128, 4), (64, 4)])
 def test_team_pooling_layer_matches_oracle(autocast, D, H):
