@@ -19,16 +19,20 @@ from .trunk import (
     GatedMLP,
     GraphedTrunk,
     GriffinTemporalBlock,
+    LibraryDispatchWarning,
     ModelConfig,
     RGLRU,
     TeamPMA,
     TransformerBlock,
     YemongBlock,
     YemongTrunk,
+    forbid_library_dispatch,
+    invalidate_weight_caches,
+    library_dispatches,
 )
 
 __all__ = [
     "CONV_KERNEL", "GatedMLP", "GraphedTrunk", "GriffinTemporalBlock", "ModelConfig", "RGLRU", "TeamPMA", "TransformerBlock",
     "YemongBlock", "YemongTrunk", "conv_seq", "conv_step", "rglru_scan", "rglru_step", "sdpa_cross", "sdpa_masked", "ops",
-    "trunk", "harness",
+    "trunk", "harness", "LibraryDispatchWarning", "forbid_library_dispatch", "invalidate_weight_caches", "library_dispatches",
 ]

@@ -14,18 +14,31 @@ Every class keeps the constructor arguments, method signatures, tensor layouts a
     YemongTrunk             the block loop and hidden-state handling of
                             models/yemong/policy.py:234-254, 268-285, 311-354
 
-What runs where: the attention core (key masking, softmax, head merge), the RG-LRU
-element-wise recurrence and the one-step causal conv with its buffer shift are the HIP
-kernels in ``ops``; projections, norms and GELUs are torch library calls on the same stream
-(so is the conv over longer sequences).  ``YemongTrunk.forward`` steps the packed hidden
-tensor in place of the reference's unpack / ``cat`` / re-pack and can fold the done-environment
-reset into the same kernels.  The layers are forward-only (rollout / evaluation); they refuse
-tensors that need gradients and they refuse to run off-GPU.
+What runs where.  Without gradients (rollout, evaluation) every sublayer runs on the HIP
+kernels in ``ops``: attention core, recurrence, conv taps with the buffer shift, and under
+bfloat16 autocast at width 128 also the norms, projections and the gated MLP (fused kernels).
+``YemongTrunk.forward`` steps the packed hidden tensor in place of the reference's unpack /
+``cat`` / re-pack and can fold the done-environment reset into the same kernels.  With
+gradients enabled (the PPO update) the same layers run on forward + backward kernels behind
+``torch.autograd.Function``s, with the forward and input-gradient GEMMs on the library.
+The layers refuse to run off-GPU.
+
+Shapes outside what the kernels cover run the same mathematics through torch's library on the
+device.  Every such dispatch is counted in ``library_dispatches`` and warned about once per
+site (``LibraryDispatchWarning``); ``forbid_library_dispatch()`` turns them into errors.
+
+Derived weights (bfloat16 copies, concatenations, matrix-core operand packings) are cached per
+layer and rebuilt when a source parameter's version counter, address or device changes, when
+the module is moved / cast (``.to()``), on ``load_state_dict`` and on ``train()`` / ``eval()``.
+A write through ``param.data`` changes none of these: call ``invalidate_weight_caches(module)``
+(or the method of that name on any layer here) after such a write.
 """
 
 from __future__ import annotations
 
+import collections
 import contextlib
+import warnings
 from dataclasses import dataclass
 
 import torch
@@ -51,10 +64,12 @@ def _projection_dtype() -> torch.dtype:
 def _fused_ok(x: torch.Tensor, act: torch.dtype) -> bool:
     """Whether the fused norm / gelu kernels apply: fp32 residual stream on the GPU, a covered
     width, fp32 or bf16 projections.  Anything else takes the plain torch composition."""
-    return (
-        not torch.is_grad_enabled() and x.is_cuda and x.dtype == torch.float32 and x.shape[-1] in _FUSED_WIDTHS
-        and act in (torch.float32, torch.bfloat16)
-    )
+    if torch.is_grad_enabled():
+        return False
+    ok = x.is_cuda and x.dtype == torch.float32 and x.shape[-1] in _FUSED_WIDTHS and act in (torch.float32, torch.bfloat16)
+    if not ok and x.is_cuda:
+        _note_library("norm_and_gate_kernels", f"rows {x.dtype} of width {x.shape[-1]}, projections in {act}")
+    return ok
 
 
 _TRAIN_KERNELS = True  # grad-mode norms, gates, conv, attention and weight gradients on the library's own kernels when False
@@ -72,17 +87,133 @@ def library_update_path():
         _TRAIN_KERNELS = keep
 
 
-def _cached_cast(owner: nn.Module, slot: str, tensors: tuple, dtype: torch.dtype, build):
-    """``build()`` (a tensor derived from ``tensors`` in ``dtype``) cached on ``owner`` until one
-    of the source tensors is modified or replaced.  Saves the per-step weight casts autocast
-    would otherwise repeat."""
-    key = (dtype,) + tuple((t._version, t.data_ptr(), t.device) for t in tensors)
-    hit = owner.__dict__.get(slot)
-    if hit is None or hit[0] != key:
+class LibraryDispatchWarning(UserWarning):
+    """A shape outside what the kernels cover ran through torch's library on the device."""
+
+
+library_dispatches: collections.Counter = collections.Counter()  # site -> calls that took the library path
+_FORBID_LIBRARY = False
+
+
+def _note_library(site: str, why: str) -> None:
+    """Record that ``site`` runs on torch's library for this call (counter + one warning per site)."""
+    if _FORBID_LIBRARY:
+        raise RuntimeError(f"library dispatch at {site} ({why}) inside forbid_library_dispatch()")
+    if not library_dispatches[site]:
+        warnings.warn(f"{site}: {why}; running torch's library on the device instead of the gfx950 kernels",
+                      LibraryDispatchWarning, stacklevel=3)
+    library_dispatches[site] += 1
+
+
+@contextlib.contextmanager
+def forbid_library_dispatch():
+    """Inside the block a call that would leave the kernels for torch's library raises instead."""
+    global _FORBID_LIBRARY
+    keep, _FORBID_LIBRARY = _FORBID_LIBRARY, True
+    try:
+        yield
+    finally:
+        _FORBID_LIBRARY = keep
+
+
+_CACHE_PREFIX = "_bnb_"
+
+
+class _DerivedWeight:
+    """One cached tensor derived from parameters: the value, how to rebuild it, what it depends on."""
+
+    __slots__ = ("key", "value", "build", "tensors", "dtype")
+
+    def __init__(self, key, value, build, tensors, dtype):
+        self.key, self.value, self.build, self.tensors, self.dtype = key, value, build, tensors, dtype
+
+    def refresh(self) -> None:
+        """Rebuild from the source tensors into the same memory (addresses stay valid)."""
         with torch.no_grad():
-            hit = (key, build())
+            _copy_into(self.value, self.build())
+        self.key = _cache_key(self.tensors, self.dtype)
+
+
+def _same_layout(a, b) -> bool:
+    if isinstance(a, tuple) or isinstance(b, tuple):
+        return (isinstance(a, tuple) and isinstance(b, tuple) and len(a) == len(b)
+                and all(_same_layout(x, y) for x, y in zip(a, b)))
+    return a.shape == b.shape and a.dtype == b.dtype and a.device == b.device
+
+
+def _copy_into(dst, src) -> None:
+    if isinstance(dst, tuple):
+        for d, s in zip(dst, src):
+            d.copy_(s)
+    else:
+        dst.copy_(src)
+
+
+def _cache_key(tensors: tuple, dtype: torch.dtype):
+    return (dtype,) + tuple((t._version, t.data_ptr(), t.device) for t in tensors)
+
+
+def _cached_cast(owner: nn.Module, slot: str, tensors: tuple, dtype: torch.dtype, build):
+    """``build()`` (a tensor derived from ``tensors`` in ``dtype``) cached on ``owner`` until one of the
+    source tensors is modified in place, replaced or moved, or the cache is invalidated.  A rebuild
+    of the same shape is written into the existing memory, so an address captured into a HIP graph
+    stays valid.  Saves the per-step weight casts autocast would otherwise repeat."""
+    key = _cache_key(tensors, dtype)
+    hit = owner.__dict__.get(slot)
+    if hit is not None and hit.key == key:
+        return hit.value
+    with torch.no_grad():
+        value = build()
+    if hit is not None and _same_layout(hit.value, value):
+        _copy_into(hit.value, value)
+        hit.key, hit.build, hit.tensors, hit.dtype = key, build, tensors, dtype
+    else:
+        hit = _DerivedWeight(key, value, build, tensors, dtype)
         owner.__dict__[slot] = hit
-    return hit[1]
+    return hit.value
+
+
+def derived_weights(module: nn.Module) -> list:
+    """Every cached derived-weight entry below ``module``."""
+    return [v for m in module.modules() for k, v in m.__dict__.items()
+            if k.startswith(_CACHE_PREFIX) and isinstance(v, _DerivedWeight)]
+
+
+def invalidate_weight_caches(module: nn.Module, *, drop: bool = False) -> None:
+    """Mark every cached derived weight below ``module`` stale, so the next forward rebuilds it.
+
+    Needed after a write the caches cannot see: ``param.data.copy_(...)`` and other writes through
+    ``.data`` leave the parameter's version counter unchanged.  ``drop=True`` frees the cached
+    tensors instead of keeping their memory for the rebuild."""
+    for m in module.modules():
+        for k in [k for k, v in m.__dict__.items() if k.startswith(_CACHE_PREFIX) and isinstance(v, _DerivedWeight)]:
+            if drop:
+                del m.__dict__[k]
+            else:
+                m.__dict__[k].key = None
+
+
+class _WeightCaches:
+    """Mixin of the layers: keeps the derived-weight caches in step with what ``nn.Module`` does to
+    the parameters behind the caches' back (moves and casts, state-dict loads, mode switches)."""
+
+    def invalidate_weight_caches(self, *, drop: bool = False) -> None:
+        invalidate_weight_caches(self, drop=drop)
+
+    def _apply(self, fn, *args, **kwargs):
+        out = super()._apply(fn, *args, **kwargs)
+        invalidate_weight_caches(self, drop=True)  # device or dtype may have changed
+        return out
+
+    def load_state_dict(self, *args, **kwargs):
+        out = super().load_state_dict(*args, **kwargs)
+        invalidate_weight_caches(self)
+        return out
+
+    def train(self, mode: bool = True):
+        out = super().train(mode)
+        invalidate_weight_caches(self)
+        return out
 
 
 def _grad_linear(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None) -> torch.Tensor:
@@ -103,8 +234,9 @@ def _project(layer: nn.Linear, x: torch.Tensor) -> torch.Tensor:
         return _grad_linear(x, w, b)
     if x.dtype == w.dtype:
         return F.linear(x, w, b)
-    wc = _cached_cast(layer, "_bnb_w", (w,), x.dtype, lambda: w.detach().to(x.dtype))
-    bc = None if b is None else _cached_cast(layer, "_bnb_b", (b,), x.dtype, lambda: b.detach().to(x.dtype))
+    dt = x.dtype  # the builders must not keep the activation alive
+    wc = _cached_cast(layer, "_bnb_w", (w,), dt, lambda: w.detach().to(dt))
+    bc = None if b is None else _cached_cast(layer, "_bnb_b", (b,), dt, lambda: b.detach().to(dt))
     return F.linear(x, wc, bc)
 
 
@@ -132,6 +264,8 @@ def _train_norm(norm: nn.RMSNorm, x: torch.Tensor, delta: torch.Tensor | None = 
         and (delta is None or (delta.shape == x.shape and delta.dtype in (torch.float32, torch.bfloat16)))
     ):
         return ops.rmsnorm_train(x, norm.weight, delta=delta, eps=norm.eps, out_dtype=act)
+    if _TRAIN_KERNELS and torch.is_grad_enabled() and x.is_cuda:
+        _note_library("rmsnorm_backward", f"rows {x.dtype} of width {x.shape[-1]}, projections in {act}")
     s = x if delta is None else x + delta
     return s, norm(s)
 
@@ -171,7 +305,7 @@ class ModelConfig:
             )
 
 
-class GatedMLP(nn.Module):
+class GatedMLP(_WeightCaches, nn.Module):
     """``down_proj(gelu(gate_proj(x)) * up_proj(x))`` with a 4x hidden width by default."""
 
     def __init__(self, d_model: int, expand: int = 4) -> None:
@@ -225,12 +359,13 @@ class GatedMLP(nn.Module):
             return _project(self.down_proj, _gelu_gate(_project(self.gate_proj, x), _project(self.up_proj, x)))
         # one GEMM for [gate | up], one kernel for gelu(gate) * up, one GEMM down
         wg, wu = self.gate_proj.weight, self.up_proj.weight
-        w = _cached_cast(self, "_bnb_gate_up", (wg, wu), x.dtype, lambda: torch.cat([wg, wu], dim=0).detach().to(x.dtype))
+        dt = x.dtype
+        w = _cached_cast(self, "_bnb_gate_up", (wg, wu), dt, lambda: torch.cat([wg, wu], dim=0).detach().to(dt))
         gu = F.linear(x, w)
         return _project(self.down_proj, ops.gelu_mul(gu[..., :hidden], gu[..., hidden:], out_dtype=x.dtype))
 
 
-class TransformerBlock(nn.Module):
+class TransformerBlock(_WeightCaches, nn.Module):
     """Pre-norm attention + FFN over the entity tokens of each environment.
 
     ``forward(x (B,N,D), alive_mask (B,N) bool | None, bullets, bullet_mask) -> (B,N,D)``.
@@ -292,6 +427,9 @@ class TransformerBlock(nn.Module):
             if _TRAIN_KERNELS and ops.sdpa_train_supported(qkv, self.n_heads):
                 merged = ops.sdpa_train(qkv, alive_mask, self.n_heads)
             else:
+                if _TRAIN_KERNELS and qkv.is_cuda:
+                    _note_library("TransformerBlock.self_attention_backward",
+                                  f"qkv {tuple(qkv.shape)} {qkv.dtype}, {self.n_heads} heads")
                 merged = self._self_attention_autograd(qkv, alive_mask)
             if self.reads_bullets and bullets is not None:
                 merged = merged + self._bullet_branch_autograd(qkv, bullets, bullet_mask)
@@ -303,6 +441,7 @@ class TransformerBlock(nn.Module):
                 raise
             # a shape the kernels do not cover (head sizes other than 8/16/32/64, more than 512
             # tokens, float32 keys beyond what fits LDS): the library's attention on the device
+            _note_library("TransformerBlock.self_attention", f"qkv {tuple(qkv.shape)} {qkv.dtype}, {self.n_heads} heads")
             merged = self._self_attention_autograd(qkv, alive_mask)
         if self.reads_bullets and bullets is not None:
             rows = bullet_mask if isinstance(bullet_mask, ops.CompactRows) else None
@@ -322,6 +461,7 @@ class TransformerBlock(nn.Module):
             if ops.cross_supported(qkv, kv, self.n_heads):
                 merged = ops.sdpa_cross(qkv, kv, bullet_mask, self.n_heads, accum=merged)
             else:
+                _note_library("TransformerBlock.bullet_read", f"queries {tuple(qkv.shape)} {qkv.dtype}, keys {tuple(kv.shape)}")
                 merged = merged + self._bullet_read(qkv, kv, bullet_mask)
         return _project(self.out_proj, merged) if project else merged
 
@@ -331,6 +471,8 @@ class TransformerBlock(nn.Module):
         return (
             qkv.dtype == torch.bfloat16 and self.d_model == ops.FFN_WIDTH and self.head_dim == 32 and qkv.shape[1] <= 160
             and bullets.is_cuda and bullets.dtype == torch.float32 and self.kv_bullet.bias is None
+            # the compacted [K | V] rows are addressed with 32-bit element offsets over the full slot capacity
+            and bullets.shape[0] * bullets.shape[1] * 2 * self.d_model < 2 ** 32
         )
 
     def _bullet_branch_autograd(self, qkv, bullets, bullet_mask):
@@ -362,6 +504,8 @@ class TransformerBlock(nn.Module):
         kv = _project(self.kv_bullet, _train_norm(self.norm_bullet, bullets)[1])
         if _TRAIN_KERNELS and ops.sdpa_cross_train_supported(qkv, kv, self.n_heads):
             return ops.sdpa_cross_train(qkv, kv, mask, self.n_heads)
+        if _TRAIN_KERNELS and qkv.is_cuda:
+            _note_library("TransformerBlock.bullet_read_backward", f"queries {tuple(qkv.shape)} {qkv.dtype}, keys {tuple(kv.shape)}")
         return self._bullet_read(qkv, kv, mask)
 
     def _self_attention_autograd(self, qkv, alive_mask):
@@ -404,7 +548,7 @@ class TransformerBlock(nn.Module):
         return o.transpose(1, 2).reshape(B, N, D)
 
 
-class RGLRU(nn.Module):
+class RGLRU(_WeightCaches, nn.Module):
     """Real-gated linear recurrent unit; parameters ``log_lambda``, ``linear_a``, ``linear_x``."""
 
     def __init__(self, d_model: int, c: float = 8.0) -> None:
@@ -462,7 +606,7 @@ class RGLRU(nn.Module):
                               time_major=time_major)
 
 
-class GriffinTemporalBlock(nn.Module):
+class GriffinTemporalBlock(_WeightCaches, nn.Module):
     """norm -> (linear1 -> causal conv -> RG-LRU) * gelu(linear2) -> linear_out, then a gated MLP."""
 
     def __init__(self, d_model: int) -> None:
@@ -482,7 +626,7 @@ class GriffinTemporalBlock(nn.Module):
         ``time_major``: ``x_seq`` and ``out`` are (T,R,D), the layout stored rollouts have.
         """
         T = x_seq.shape[0] if time_major else x_seq.shape[1]
-        if T == 1 and done_mask is None and not time_major:
+        if T == 1 and done_mask is None and not time_major and not torch.is_grad_enabled():
             # rollout: the conv taps and the buffer shift are one kernel, the recurrence another
             x = x_seq[:, 0]
             out, new_h, new_conv_buf = self._step(x, h0, conv_buf, None, None, None, 1)
@@ -693,7 +837,7 @@ def _conv_within_episodes(padded, w, bias, done_mask):
     return out + bias
 
 
-class TeamPMA(nn.Module):
+class TeamPMA(_WeightCaches, nn.Module):
     """Pooling by multi-head attention over each team's alive ships (policy.py:78-120).
 
     Parameters and ``state_dict`` keys as in the reference: ``seeds`` (2, D), ``attn``
@@ -745,6 +889,8 @@ class TeamPMA(nn.Module):
                 u, folded = ops.team_pool_constants(self.seeds, self.attn.in_proj_weight, self.attn.out_proj.weight, self.n_heads)
                 return ops.team_pool_train(x, team_id, alive, u, folded, self.norm.weight, self.norm.eps, self.n_heads)
         B, N, D = x.shape
+        if x.is_cuda and _TRAIN_KERNELS:
+            _note_library("TeamPMA.forward", f"rows {tuple(x.shape)} {x.dtype}, {self.n_heads} heads")
         pool = self._pooled_library(x, team_id, alive)
         return pool.gather(1, team_id.clamp(0, 1).long().unsqueeze(-1).expand(B, N, D))
 
@@ -773,7 +919,7 @@ class _SplitTokens(torch.autograd.Function):
         return torch.cat([d_first, d_rest], dim=2), None
 
 
-class YemongBlock(nn.Module):
+class YemongBlock(_WeightCaches, nn.Module):
     """``n_spatial_per_block`` attention sublayers, then ``n_temporal_per_block`` recurrent ones."""
 
     def __init__(self, model_config: ModelConfig) -> None:
@@ -875,7 +1021,21 @@ class YemongBlock(nn.Module):
         return x, torch.stack(new_h), torch.stack(new_cb)
 
 
-class YemongTrunk(nn.Module):
+def _byte_range(t: torch.Tensor) -> tuple[int, int]:
+    """[first, last) byte addresses a (possibly strided) tensor can touch."""
+    if t.numel() == 0:
+        return (0, 0)
+    span = sum((n - 1) * abs(st) for n, st in zip(t.shape, t.stride())) + 1
+    return t.data_ptr(), t.data_ptr() + span * t.element_size()
+
+
+def _overlap(a: torch.Tensor, b: torch.Tensor) -> bool:
+    """Whether the address ranges of two tensors intersect (a view at another offset included)."""
+    (a0, a1), (b0, b1) = _byte_range(a), _byte_range(b)
+    return a0 < b1 and b0 < a1
+
+
+class YemongTrunk(_WeightCaches, nn.Module):
     """The recurrent trunk: ``forward(tokens, alive_mask, recurrent_state) -> (hidden, new_state)``.
 
     ``recurrent_state`` is the packed tensor (n_layers, B*n_rec, 4*D) float32 of the
@@ -961,10 +1121,8 @@ class YemongTrunk(nn.Module):
         n_t = self.config.n_temporal_per_block
         if out_state is None:
             out_state = torch.empty_like(recurrent_state)
-        elif out_state.shape != recurrent_state.shape or out_state.dtype != torch.float32 or (
-            out_state.data_ptr() == recurrent_state.data_ptr() and L
-        ):
-            raise ValueError("out_state must be a separate float32 tensor shaped like recurrent_state")
+        elif out_state.shape != recurrent_state.shape or out_state.dtype != torch.float32 or _overlap(out_state, recurrent_state):
+            raise ValueError("out_state must be a float32 tensor shaped like recurrent_state that shares no memory with it")
         if reset_mask is not None:
             reset_mask = reset_mask.contiguous()
         # the list of bullets in flight is built once and shared by every layer that reads them
@@ -993,9 +1151,16 @@ class GraphedTrunk:
     The packed state lives in two buffers that alternate as input and output, hence two
     graphs.  Outputs are overwritten by the next ``step``; clone what must outlive it.
 
+    Weights: the captured kernels read the parameters themselves (norm weights, float32 GEMM operands)
+    and the derived copies the layers cache (bfloat16 casts, concatenations, operand packings) at the
+    addresses they had at capture time.  A replay runs no Python, so after a weight update (optimizer
+    step, ``load_state_dict``, a write through ``.data``) call ``refresh_weights()``: it rebuilds
+    every derived copy into the same memory.  This object keeps those copies alive, so nothing the
+    graphs read is ever returned to the allocator.  Replacing parameter tensors, moving or casting
+    the module requires a new capture.
+
     Args:
-        trunk: the module to capture (weights are read at replay time, so in-place weight
-            updates are seen; replacing parameter tensors requires a new capture).
+        trunk: the module to capture.
         num_envs, num_tokens, num_recurrent: B, N+M and n_rec of every later call.
         autocast_dtype: ``torch.bfloat16`` to capture under autocast, None for fp32.
         use_reset: capture with a ``reset_mask`` input (all-False masks are then cheap no-ops).
@@ -1028,6 +1193,14 @@ class GraphedTrunk:
             self.outputs.append(out)
         for s in self.states:
             s.zero_()
+        # the derived weights the captured kernels read: held here so their memory outlives any cache
+        # invalidation on the module, and rebuilt in place by refresh_weights()
+        self._derived = derived_weights(trunk)
+
+    def refresh_weights(self) -> None:
+        """Rebuild every derived weight copy the graphs read from the current parameters, in place."""
+        for entry in self._derived:
+            entry.refresh()
 
     def _run(self, src: int) -> torch.Tensor:
         with torch.autocast("cuda", dtype=self.autocast_dtype or torch.bfloat16, enabled=self.autocast_dtype is not None):

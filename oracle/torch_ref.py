@@ -342,16 +342,20 @@ def block_step(
     h: torch.Tensor,
     conv_buf: torch.Tensor,
     n_rec: int | None = None,
+    bullets: torch.Tensor | None = None,
+    bullet_mask: torch.Tensor | None = None,
 ):
     """One Yemong block for one timestep; models/yemong/griffin.py:376-417.
 
     x (B,NM,D), alive (B,NM), h (n_temporal, B*n_rec, D), conv_buf
-    (n_temporal, B*n_rec, 3, D).  Recurrent rows are env-major (b*n_rec + n).
+    (n_temporal, B*n_rec, 3, D).  Recurrent rows are env-major (b*n_rec + n).  ``bullets``
+    (B,NB,D) / ``bullet_mask`` (B,NB) reach every spatial sublayer (griffin.py:400-401); the
+    ones that own ``kv_bullet`` weights read them (attention.py:149).
     """
     B, NM, D = x.shape
     n_rec = NM if n_rec is None else n_rec
     for s in range(n_spatial):
-        x = spatial_sublayer(p, f"{prefix}spatial.{s}.", x, alive, n_heads)
+        x = spatial_sublayer(p, f"{prefix}spatial.{s}.", x, alive, n_heads, bullets, bullet_mask)
     hs, cbs = [], []
     for j in range(n_temporal):
         tp = f"{prefix}temporal.{j}."
@@ -395,8 +399,11 @@ def trunk_step(
     x: torch.Tensor,
     alive: torch.Tensor,
     hidden: torch.Tensor,
+    bullets: torch.Tensor | None = None,
+    bullet_mask: torch.Tensor | None = None,
 ):
-    """The block loop of ``get_action_and_value``; models/yemong/policy.py:311-354."""
+    """The block loop of ``get_action_and_value``; models/yemong/policy.py:311-354 (bullets handed to
+    every block, :327-340)."""
     B, NM, D = x.shape
     n_rec = hidden.shape[1] // B
     h_all, cb_all = unpack_hidden(hidden, D)
@@ -404,7 +411,8 @@ def trunk_step(
     for i in range(n_blocks):
         sl = slice(i * n_temporal, (i + 1) * n_temporal)
         x, h_new, cb_new = block_step(
-            p, f"yemong_layers.{i}.", n_spatial, n_temporal, n_heads, x, alive, h_all[sl], cb_all[sl], n_rec
+            p, f"yemong_layers.{i}.", n_spatial, n_temporal, n_heads, x, alive, h_all[sl], cb_all[sl], n_rec,
+            bullets, bullet_mask,
         )
         hs.append(h_new)
         cbs.append(cb_new)

@@ -865,3 +865,148 @@ def test_trunk_sequence_with_bullets_shares_one_list_and_matches_the_block_loop(
         out = trunk.sequence(xin, alive, hidden0, done, bullets, bmask, grad_checkpoint=True)
     out.float().square().mean().backward()
     assert torch.isfinite(xin.grad).all() and all(q.grad is not None and torch.isfinite(q.grad).all() for q in trunk.parameters())
+
+
+# ------------------------------------------------------------------ weights that change after the first forward
+
+
+def _rollout_trunk(seed=51, D=128, H=4):
+    p = trunk_params(seed, D, 2, 2, 1)
+    trunk = bnb.YemongTrunk(_cfg(D, H, 2, 2, 1)).eval()
+    trunk.load_state_dict(p)
+    return trunk.to(DEV), p
+
+
+@pytest.mark.parametrize("autocast", [False, True])
+def test_weight_updates_after_the_first_forward_reach_the_cached_copies(autocast):
+    # the averaged-opponent policy is overwritten through .data every update (train/rl/opponents.py:112);
+    # the live policy by an optimizer step: after either, a no-grad forward must use the new weights
+    D, H, B, N, M = 128, 4, 8, 8, 4
+    trunk, _ = _rollout_trunk()
+    gen = torch.Generator().manual_seed(52)
+    x = torch.randn(B, N + M, D, generator=gen)
+    alive = torch.ones(B, N + M, dtype=torch.bool)
+    hidden = torch.randn(2, B * N, 4 * D, generator=gen)
+    tol = BF16_TOL if autocast else 5e-5
+
+    def run_and_check(p_now):
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+            out, new_hidden = trunk(x.to(DEV), alive.to(DEV), hidden.to(DEV))
+        ref_out, ref_hidden = torch_ref.trunk_step(p_now, 2, 2, 1, H, x, alive, hidden)
+        assert max_rel(out.cpu(), ref_out) <= tol and max_rel(new_hidden.cpu(), ref_hidden) <= tol
+        return out
+
+    first = run_and_check({k: v.detach().cpu() for k, v in trunk.state_dict().items()})
+
+    # 1. a write through .data, then the documented call
+    other = trunk_params(77, D, 2, 2, 1)
+    for name, param in trunk.named_parameters():
+        param.data.copy_(other[name])
+    trunk.invalidate_weight_caches()
+    second = run_and_check(other)
+    assert not torch.equal(first, second)
+
+    # 2. an optimizer step (in-place on the parameters: seen without any call)
+    opt = torch.optim.SGD(trunk.parameters(), lr=0.05)
+    for param in trunk.parameters():
+        param.grad = torch.randn(param.shape, generator=gen).to(DEV)
+    opt.step()
+    third = run_and_check({k: v.detach().cpu() for k, v in trunk.state_dict().items()})
+    assert not torch.equal(second, third)
+
+    # 3. load_state_dict, also through a parent module that is not one of these layers
+    holder = torch.nn.Module()
+    holder.trunk = trunk
+    holder.load_state_dict({"trunk." + k: v for k, v in trunk_params(78, D, 2, 2, 1).items()})
+    run_and_check(trunk_params(78, D, 2, 2, 1))
+
+
+@pytest.mark.parametrize("autocast_dtype", [None, torch.bfloat16])
+def test_graphed_trunk_sees_new_weights_after_refresh(autocast_dtype):
+    D, H, B, N, M = 128, 4, 16, 8, 4
+    trunk, _ = _rollout_trunk(61)
+    graphed = bnb.GraphedTrunk(trunk, B, N + M, N, autocast_dtype=autocast_dtype)
+    gen = torch.Generator().manual_seed(62)
+    alive = torch.ones(B, N + M, dtype=torch.bool, device=DEV)
+    eager_state = trunk.initial_hidden(B, N, DEV)
+
+    def both(t):
+        nonlocal eager_state
+        x = torch.randn(B, N + M, D, generator=gen).to(DEV)
+        out, state = graphed.step(x, alive)
+        out, state = out.clone(), state.clone()
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast_dtype is not None):
+            ref_out, eager_state = trunk(x, alive, eager_state)
+        assert torch.equal(out, ref_out) and torch.equal(state, eager_state), t
+
+    both(0)
+    # an optimizer-style in-place update and a write through .data, with no eager forward in between
+    other = trunk_params(63, D, 2, 2, 1)
+    for i, (name, param) in enumerate(trunk.named_parameters()):
+        if i % 2:
+            param.data.copy_(other[name])
+        else:
+            with torch.no_grad():
+                param.copy_(other[name])
+    graphed.refresh_weights()
+    trunk.invalidate_weight_caches()  # for the eager side of the comparison (the .data writes)
+    both(1)
+    both(2)
+    # the module dropping its caches must not take away memory the graphs read
+    trunk.invalidate_weight_caches(drop=True)
+    torch.cuda.empty_cache()
+    scratch = [torch.randn(1 << 16, device=DEV) for _ in range(64)]  # reuses whatever was freed
+    both(3)
+    del scratch
+
+
+def test_block_step_and_single_step_sequence_work_in_grad_mode_and_match_autograd_through_the_oracle():
+    # griffin.py:376-417 is differentiable in the reference; a T = 1 sequence in grad mode must not take
+    # the inference kernels
+    D, H, B, N, M = 64, 4, 3, 4, 2
+    gen = torch.Generator().manual_seed(71)
+    p = block_params(gen, "b.", D, 1, 1)
+    block = bnb.YemongBlock(_cfg(D, H, 1, 1, 1))
+    block.load_state_dict(_strip(p, "b."))
+    block.to(DEV)
+    x = torch.randn(B, N + M, D, generator=gen)
+    alive = torch.rand(B, N + M, generator=gen) < 0.8
+    alive[:, N:] = True
+    h = 0.5 * torch.randn(1, B * N, D, generator=gen)
+    cb = torch.randn(1, B * N, 3, D, generator=gen)
+    wo = torch.randn(B, N + M, D, generator=gen)
+    xd = x.to(DEV).requires_grad_(True)
+    out, h1, cb1 = block.step(xd, alive.to(DEV), h.to(DEV), cb.to(DEV), N)
+    assert out.requires_grad
+    ((out * wo.to(DEV)).sum() + h1.sum() + 0.5 * cb1.sum()).backward()
+    pr = {k: v.clone().double().requires_grad_(True) for k, v in p.items()}
+    xr = x.double().requires_grad_(True)
+    ro, rh, rcb = torch_ref.block_step(pr, "b.", 1, 1, H, xr, alive, h.double(), cb.double(), N)
+    ((ro * wo.double()).sum() + rh.sum() + 0.5 * rcb.sum()).backward()
+    assert max_rel(out.detach().cpu(), ro.detach()) <= 5e-5
+    assert max_rel(xd.grad.cpu(), xr.grad) <= 2e-4
+    for name, param in block.named_parameters():
+        assert param.grad is not None, name
+        assert max_rel(param.grad.cpu(), pr["b." + name].grad) <= 2e-4, name
+    # the temporal layer alone, T = 1
+    layer = block.temporal[0]
+    xs = torch.randn(5, 1, D, generator=gen).to(DEV).requires_grad_(True)
+    o, _, _ = layer.forward_sequence(xs, torch.zeros(5, D, device=DEV), torch.zeros(5, 3, D, device=DEV))
+    o.sum().backward()
+    assert xs.grad is not None and torch.isfinite(xs.grad).all()
+
+
+def test_out_state_overlapping_the_input_state_at_an_offset_is_refused():
+    D, H, B, N, M = 128, 4, 4, 8, 4
+    trunk, _ = _rollout_trunk(81)
+    x = torch.randn(B, N + M, D, device=DEV)
+    alive = torch.ones(B, N + M, dtype=torch.bool, device=DEV)
+    rows = B * N
+    big = torch.zeros(2 * 2 * rows + 2 * rows, 4 * D, device=DEV)
+    state = big[: 2 * rows].view(2, rows, 4 * D)
+    shifted = big[rows: 3 * rows].view(2, rows, 4 * D)  # same storage, one layer's worth of rows further on
+    with pytest.raises(ValueError, match="shares no memory"):
+        trunk(x, alive, state, out_state=shifted)
+    apart = big[2 * rows: 4 * rows].view(2, rows, 4 * D)
+    _, new_state = trunk(x, alive, state, out_state=apart)  # adjacent but disjoint: fine
+    assert new_state.data_ptr() == apart.data_ptr()
