@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_library_identity_and_error_names():
     lib = _native.load()
-    assert lib.bnb_abi_version() == _native.ABI_VERSION == 17
+    assert lib.bnb_abi_version() == _native.ABI_VERSION  # the header's value is checked below
     assert lib.bnb_build_arch() == b"gfx950"
     assert lib.bnb_error_string(0) == b"success"
     assert b"NULL" in lib.bnb_error_string(10001)
