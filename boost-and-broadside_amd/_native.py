@@ -12,7 +12,7 @@ import os
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "_lib", "libbnb_amd.so")
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 F32, BF16 = 0, 1
 PATH_AUTO, PATH_VALU, PATH_MFMA = 0, 1, 2
 
@@ -46,6 +46,8 @@ SIGNATURES = {
     "bnb_sdpa_masked_bwd_path": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _vp]),
     "bnb_rmsnorm_bwd_blocks": (_i, [_i64, _i]),
     "bnb_rmsnorm_bwd": (_i, [_vp, _i64, _vp, _i, _i64, _vp, _f, _vp, _vp, _vp, _vp, _i, _vp, _i64, _i, _vp]),
+    "bnb_rmsnorm_bwd_static_limit": (_i64, []),
+    "bnb_rmsnorm_bwd_static": (_i, [_vp, _i64, _vp, _i, _i64, _vp, _f, _vp, _vp, _vp, _vp, _i64, _i, _vp]),
     "bnb_team_attend_fwd": (_i, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i, _i, _i, _i, _vp]),
     "bnb_team_attend_bwd": (_i, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "bnb_team_attend_bwd_partial_rows": (_i, []),
@@ -83,6 +85,7 @@ class NativeLibraryError(RuntimeError):
 
 
 ERR_UNSUPPORTED = 10004  # BNB_ERR_UNSUPPORTED: a shape outside what the kernels cover
+ERR_SCRATCH_LIMIT = 10006  # BNB_ERR_SCRATCH_LIMIT: more workspace needed than the built-in buffer holds
 
 
 def load() -> ctypes.CDLL:

@@ -30,6 +30,7 @@ extern "C" const char *bnb_error_string(int code)
         case BNB_ERR_BAD_SHAPE: return "negative size, inconsistent dimensions or a stride smaller than a row";
         case BNB_ERR_UNSUPPORTED: return "shape or path outside what the kernels cover";
         case BNB_ERR_MISALIGNED: return "pointer or stride breaks the required alignment";
+        case BNB_ERR_SCRATCH_LIMIT: return "the call needs more workspace than the library's built-in buffer holds";
         default: return hipGetErrorString((hipError_t)code);
     }
 }

@@ -16,10 +16,42 @@
 
 #include "common.h"
 
+#include <mutex>
+
 namespace bnb {
 
 constexpr int kNbThreads = 256;
 constexpr int kNbMaxBlocks = 1280;  // five work-groups per CU: what 80-98 registers per lane let run at once, so no work-group waits for a free slot
+
+// Workspace of the entry point that allocates nothing (bnb_rmsnorm_bwd_static): the per-work-group
+// partial weight gradients, kNbMaxBlocks rows of at most kNbStaticMaxD floats = 2.5 MiB.  Every GPU
+// the library runs on holds its own copy at its own address until the process ends.  In host
+// code this name is only a handle for hipGetSymbolAddress, never a device address.
+constexpr int kNbStaticMaxD = 512;
+static __device__ __align__(256) float scratch[kNbMaxBlocks * kNbStaticMaxD];
+
+constexpr int kMaxDevices = 64;
+static float *g_scratch_ptr[kMaxDevices];  // device address of `scratch` per device, looked up once
+static std::mutex g_scratch_mutex;
+
+// Device address of this device's `scratch`, resolved on the first call with that device current.
+static int scratch_address(float **out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return BNB_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        float *ptr = nullptr;
+        e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (ptr == nullptr) return (int)hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
 
 template <int LANES, typename GT, bool HAS_SUM>
 __global__ __launch_bounds__(kNbThreads) void rmsnorm_bwd_kernel(
@@ -158,4 +190,22 @@ extern "C" int bnb_rmsnorm_bwd(const float *x, int64_t x_row_stride, const void 
                                            partials, blocks, dw, R, s);
     return dispatch_norm_bwd<float>(D, x, x_row_stride, dy, dy_row_stride, weight, eps, grad_sum, dx, (uint16_t *)dx_bf16, partials,
                                     blocks, dw, R, s);
+}
+
+extern "C" int64_t bnb_rmsnorm_bwd_static_limit(void) { return (int64_t)bnb::kNbMaxBlocks * bnb::kNbStaticMaxD * (int64_t)sizeof(float); }
+
+extern "C" int bnb_rmsnorm_bwd_static(const float *x, int64_t x_row_stride, const void *dy, int dy_dtype, int64_t dy_row_stride,
+                                      const float *weight, float eps, const float *grad_sum, float *dx, void *dx_bf16,
+                                      float *dw, int64_t R, int D, void *stream)
+{
+    using namespace bnb;
+    if (D > kNbStaticMaxD) return BNB_ERR_SCRATCH_LIMIT;
+    const int blocks = bnb_rmsnorm_bwd_blocks(R, D);
+    if ((int64_t)blocks * D > (int64_t)kNbMaxBlocks * kNbStaticMaxD) return BNB_ERR_SCRATCH_LIMIT;
+    float *partials = nullptr;
+    const int rc = scratch_address(&partials);
+    if (rc != 0) return rc;
+    // every partial row that is summed is written by this launch first: nothing to clear
+    return bnb_rmsnorm_bwd(x, x_row_stride, dy, dy_dtype, dy_row_stride, weight, eps, grad_sum, dx, dx_bf16, partials, blocks, dw,
+                           R, D, stream);
 }

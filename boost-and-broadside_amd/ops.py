@@ -1350,6 +1350,35 @@ def rmsnorm_bwd(x: torch.Tensor, dy: torch.Tensor, weight: torch.Tensor, *, eps:
     return dx.reshape(x.shape), dw
 
 
+def rmsnorm_bwd_static(x: torch.Tensor, dy: torch.Tensor, weight: torch.Tensor, dx: torch.Tensor, dw: torch.Tensor, *,
+                       eps: float | None = None, grad_sum: torch.Tensor | None = None,
+                       dx_bf16: torch.Tensor | None = None) -> None:
+    """``rmsnorm_bwd`` into the caller's ``dx`` (R, D) float32, ``dw`` (D,) float32 and optional ``dx_bf16``,
+    allocating nothing: the partial weight gradients use the library's built-in buffer (one per GPU,
+    shared by all calls on that GPU, so concurrent calls on one GPU must be ordered by the caller).
+    For code that cannot allocate around the call, e.g. under HIP graph capture.  All tensors must
+    have contiguous (R, D) rows already; nothing is copied."""
+    D = x.shape[-1]
+    R = x.numel() // D if D else 0
+    for t, name, dt in ((x, "x", torch.float32), (weight, "weight", torch.float32), (dx, "dx", torch.float32),
+                        (dw, "dw", torch.float32)):
+        _need_device(t, name)
+        if t.dtype != dt or not t.is_contiguous():
+            raise TypeError(f"{name} must be contiguous {dt}")
+    _need_device(dy, "dy")
+    if not dy.is_contiguous() or dy.shape != x.shape or dx.shape != x.shape or weight.shape != (D,) or dw.shape != (D,):
+        raise ValueError("dy and dx must be contiguous with x's shape, weight and dw (D,)")
+    for t, name, dt in ((grad_sum, "grad_sum", torch.float32), (dx_bf16, "dx_bf16", torch.bfloat16)):
+        if t is not None and (t.dtype != dt or not t.is_contiguous() or t.shape != x.shape or not t.is_cuda):
+            raise TypeError(f"{name} must be a contiguous {dt} device tensor with x's shape")
+    with torch.cuda.device(x.device):
+        rc = _native.load().bnb_rmsnorm_bwd_static(
+            x.data_ptr(), D, dy.data_ptr(), _code(dy, "dy"), D, weight.data_ptr(), _F32_EPS if eps is None else float(eps),
+            None if grad_sum is None else grad_sum.data_ptr(), dx.data_ptr(), None if dx_bf16 is None else dx_bf16.data_ptr(),
+            dw.data_ptr(), R, D, _stream())
+    _native.check(rc, "bnb_rmsnorm_bwd_static")
+
+
 class _RmsNormTrain(torch.autograd.Function):
     """``(x, rmsnorm(x) * weight)``: x is handed through so that the gradient arriving on the residual
     branch reaches the backward kernel, which adds it in the same pass."""

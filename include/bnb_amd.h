@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 17
+#define BNB_ABI_VERSION 18
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -36,6 +36,7 @@ extern "C" {
 #define BNB_ERR_BAD_SHAPE 10003     /* negative size, H*dh mismatch, stride smaller than a row */
 #define BNB_ERR_UNSUPPORTED 10004   /* shape outside what the kernels cover (see each entry point) */
 #define BNB_ERR_MISALIGNED 10005    /* pointer or stride breaks the stated alignment */
+#define BNB_ERR_SCRATCH_LIMIT 10006 /* the call needs more workspace than the library's built-in buffer holds */
 
 /* Bumped on any change of a signature or of the meaning of an argument. */
 int bnb_abi_version(void);
@@ -336,6 +337,27 @@ int bnb_rmsnorm_bwd_blocks(int64_t R, int D);
 int bnb_rmsnorm_bwd(const float *x, int64_t x_row_stride, const void *dy, int dy_dtype, int64_t dy_row_stride,
                     const float *weight, float eps, const float *grad_sum, float *dx, void *dx_bf16,
                     float *partials, int blocks, float *dw, int64_t R, int D, void *stream);
+
+/*
+ * bnb_rmsnorm_bwd without the caller's workspace and without any allocation.
+ *
+ * No counterpart in the reference.  It is for callers that cannot allocate device memory around the
+ * call: code under HIP graph capture, tight loops that must not touch the allocator, harnesses that
+ * forbid hipMalloc.  The per-work-group partial weight gradients (the `partials` argument of
+ * bnb_rmsnorm_bwd) live in a buffer built into the library, bnb_rmsnorm_bwd_static_limit() bytes
+ * (2.5 MiB) per GPU, held until the process ends; its device address is looked up once per device on
+ * the first call made with that device current.  The call itself calls no hipMalloc / hipFree.
+ *
+ * Arguments and results as bnb_rmsnorm_bwd (the number of work-groups is chosen as
+ * bnb_rmsnorm_bwd_blocks(R, D) would).  D above 512 returns BNB_ERR_SCRATCH_LIMIT: the partials of one
+ * launch would not fit the buffer.  All calls on one GPU share that GPU's buffer: two calls that
+ * may run at the same time on one GPU (different streams, different threads) race on it and must be
+ * ordered by the caller; calls on one stream are ordered already.
+ */
+int64_t bnb_rmsnorm_bwd_static_limit(void);
+int bnb_rmsnorm_bwd_static(const float *x, int64_t x_row_stride, const void *dy, int dy_dtype, int64_t dy_row_stride,
+                           const float *weight, float eps, const float *grad_sum, float *dx, void *dx_bf16,
+                           float *dw, int64_t R, int D, void *stream);
 
 /*
  * Pooling by multi-head attention over each team's alive ships, broadcast back to the ships:
