@@ -1133,6 +1133,10 @@ static int dispatch_cross_stream(const void *q, int64_t q_stride, const void *k,
     }
 }
 
+// defined in sdpa_cross_f32.hip
+int launch_cross_f32(const void *q, int64_t q_stride, const void *k, const void *v, int64_t kv_stride, const uint8_t *key_mask,
+                     const void *accum, void *out, int B, int NQ, int NK, int H, hipStream_t stream);
+
 }  // namespace bnb
 
 extern "C" int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive,
@@ -1210,8 +1214,19 @@ extern "C" int bnb_sdpa_cross_fwd(const void *q, int64_t q_row_stride, int NQ, c
 {
     using namespace bnb;
     if (B < 0 || NQ < 0 || NK < 0 || H < 1 || dh < 1) return BNB_ERR_BAD_SHAPE;
-    if (dtype != BNB_BF16 || dh != kDh || NQ > 160 || NK > kStreamMaxKeys) return BNB_ERR_UNSUPPORTED;
-    if (NK == 0) return BNB_ERR_UNSUPPORTED;  // nothing to read: the caller keeps `accum` as it is
+    if (dtype != BNB_BF16 && dtype != BNB_F32) return BNB_ERR_BAD_DTYPE;
+    if (dh != kDh || NK == 0) return BNB_ERR_UNSUPPORTED;  // NK == 0: nothing to read, the caller keeps `accum` as it is
+    if (dtype == BNB_F32) {
+        if (NQ > 512 || NK > 4096) return BNB_ERR_UNSUPPORTED;
+        if (B == 0 || NQ == 0) return 0;
+        if (!q || !out || !k || !v) return BNB_ERR_NULL_POINTER;
+        if (q_row_stride < (int64_t)H * dh || kv_row_stride < (int64_t)H * dh) return BNB_ERR_BAD_SHAPE;
+        if (!aligned16(q) || !aligned16(out) || (accum && !aligned16(accum)) || (q_row_stride * 4) % 16 != 0 || !aligned16(k) ||
+            !aligned16(v) || (kv_row_stride * 4) % 16 != 0)
+            return BNB_ERR_MISALIGNED;
+        return launch_cross_f32(q, q_row_stride, k, v, kv_row_stride, key_mask, accum, out, B, NQ, NK, H, (hipStream_t)stream);
+    }
+    if (NQ > 160 || NK > kStreamMaxKeys) return BNB_ERR_UNSUPPORTED;
     if (B == 0 || NQ == 0) return 0;
     if (!q || !out || !k || !v) return BNB_ERR_NULL_POINTER;
     if (q_row_stride < (int64_t)H * dh || kv_row_stride < (int64_t)H * dh) return BNB_ERR_BAD_SHAPE;

@@ -183,12 +183,14 @@ def sdpa_train(qkv: torch.Tensor, alive: torch.Tensor | None, n_heads: int) -> t
 
 
 def cross_supported(q: torch.Tensor, kv: torch.Tensor, n_heads: int) -> bool:
-    """Whether ``sdpa_cross`` covers these shapes (bf16, head size 32, 1..2048 keys, <= 160 queries)."""
+    """Whether ``sdpa_cross`` covers these shapes: head size 32 and either bfloat16 with 1..2048 keys and
+    at most 160 queries, or float32 with 1..4096 keys and at most 512 queries."""
     D = kv.shape[-1] // 2
-    return (
-        q.is_cuda and q.dtype == torch.bfloat16 and kv.dtype == torch.bfloat16 and D % n_heads == 0
-        and D // n_heads == 32 and 1 <= kv.shape[1] <= 2048 and q.shape[1] <= 160
-    )
+    if not (q.is_cuda and q.dtype == kv.dtype and D % n_heads == 0 and D // n_heads == 32):
+        return False
+    if q.dtype == torch.bfloat16:
+        return 1 <= kv.shape[1] <= 2048 and q.shape[1] <= 160
+    return q.dtype == torch.float32 and 1 <= kv.shape[1] <= 4096 and q.shape[1] <= 512
 
 
 def sdpa_cross(
@@ -200,7 +202,8 @@ def sdpa_cross(
     accum: torch.Tensor | None = None,
     out: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """Entity queries reading a second key/value set (the bullet read), on the matrix-core kernel.
+    """Entity queries reading a second key/value set (the bullet read), on the matrix-core kernels
+    (bfloat16, or float32 with true float32 products for evaluation without autocast).
 
     Args:
         qkv:      (B, NQ, 3*D) packed entity projection; only its Q third is read.
@@ -209,9 +212,9 @@ def sdpa_cross(
                   environment with no active key contributes exactly zero.
         accum:    optional (B, NQ, D) contiguous tensor the result is added to (and, unless
                   ``out`` is given, written into); default: the bare result in a new tensor.
-        out:      optional (B, NQ, D) contiguous bfloat16 destination.
+        out:      optional (B, NQ, D) contiguous destination.
 
-    Returns (B, NQ, D) bfloat16.
+    Returns (B, NQ, D) in ``qkv``'s dtype.
     """
     B, NQ, D3 = qkv.shape
     D = D3 // 3
@@ -219,7 +222,8 @@ def sdpa_cross(
     if kv.shape != (B, NK, 2 * D):
         raise ValueError(f"kv must be {(B, NK, 2 * D)}, got {tuple(kv.shape)}")
     if not cross_supported(qkv, kv, n_heads):
-        raise RuntimeError("sdpa_cross covers bfloat16, head size 32, 1..2048 keys and at most 160 queries")
+        raise RuntimeError("sdpa_cross covers head size 32 with bfloat16 (1..2048 keys, <= 160 queries) or "
+                           "float32 (1..4096 keys, <= 512 queries), queries and keys in one dtype")
     if torch.is_grad_enabled() and (qkv.requires_grad or kv.requires_grad):
         raise RuntimeError("sdpa_cross is forward-only; call it under torch.no_grad()")
     if B and NQ and (qkv.stride(-1) != 1 or (B > 1 and qkv.stride(0) != NQ * qkv.stride(1))):
@@ -232,19 +236,19 @@ def sdpa_cross(
             raise ValueError(f"key_mask must be a bool {(B, NK)} tensor")
         key_mask = key_mask.contiguous()
         mask_ptr = key_mask.data_ptr()
-    if accum is not None and (accum.shape != (B, NQ, D) or accum.dtype != torch.bfloat16 or not accum.is_contiguous()):
-        raise ValueError("accum must be a contiguous bfloat16 (B, NQ, D) tensor")
-    if out is not None and (out.shape != (B, NQ, D) or out.dtype != torch.bfloat16 or not out.is_contiguous()):
-        raise ValueError("out must be a contiguous bfloat16 (B, NQ, D) tensor")
+    if accum is not None and (accum.shape != (B, NQ, D) or accum.dtype != qkv.dtype or not accum.is_contiguous()):
+        raise ValueError("accum must be a contiguous (B, NQ, D) tensor in qkv's dtype")
+    if out is not None and (out.shape != (B, NQ, D) or out.dtype != qkv.dtype or not out.is_contiguous()):
+        raise ValueError("out must be a contiguous (B, NQ, D) tensor in qkv's dtype")
     if out is None:
-        out = accum if accum is not None else torch.empty((B, NQ, D), dtype=torch.bfloat16, device=qkv.device)
+        out = accum if accum is not None else torch.empty((B, NQ, D), dtype=qkv.dtype, device=qkv.device)
     if B == 0 or NQ == 0:
         return out
     with torch.cuda.device(qkv.device):
         rc = _native.load().bnb_sdpa_cross_fwd(
             qkv.data_ptr(), qkv.stride(1), NQ, kv.data_ptr(), kv.data_ptr() + D * kv.element_size(), kv.stride(1), NK,
             mask_ptr, None if accum is None else accum.data_ptr(), out.data_ptr(), B, n_heads, D // n_heads,
-            _native.BF16, _stream(),
+            _code(qkv, "qkv"), _stream(),
         )
     _native.check(rc, "bnb_sdpa_cross_fwd")
     return out
@@ -252,7 +256,8 @@ def sdpa_cross(
 
 def sdpa_cross_train_supported(qkv: torch.Tensor, kv: torch.Tensor, n_heads: int) -> bool:
     """Whether ``sdpa_cross_train`` covers these shapes: what ``sdpa_cross`` covers with at most 160 keys."""
-    return cross_supported(qkv, kv, n_heads) and kv.shape[1] <= 160 and kv.dim() == 3 and qkv.dim() == 3
+    return (cross_supported(qkv, kv, n_heads) and qkv.dtype == torch.bfloat16 and kv.shape[1] <= 160 and kv.dim() == 3
+            and qkv.dim() == 3)
 
 
 def sdpa_cross_bwd(qkv, kv, key_mask, n_heads, out, dout) -> tuple[torch.Tensor, torch.Tensor]:

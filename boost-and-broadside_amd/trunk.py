@@ -529,9 +529,9 @@ class TransformerBlock(_WeightCaches, nn.Module):
 
     def _bullet_read(self, qkv, kv, bullet_mask):
         """Cross-attention of the entity queries to bullet key/values (attention.py:149-166) for
-        the shapes the matrix-core kernel does not cover (fp32, more than 2048 bullets, other
-        head sizes): torch's SDPA on the device, with the reference's additive bias and its
-        all-inactive gate.  ``kv`` is ``kv_bullet(norm_bullet(bullets))``."""
+        the shapes the matrix-core kernels do not cover (head sizes other than 32, more than 2048
+        bullet slots in bf16 or 4096 in fp32): torch's SDPA on the device, with the reference's
+        additive bias and its all-inactive gate.  ``kv`` is ``kv_bullet(norm_bullet(bullets))``."""
         B, N, _ = qkv.shape
         H, dh, D = self.n_heads, self.head_dim, self.d_model
         NB = kv.shape[1]

@@ -106,11 +106,13 @@ int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride, const uint
  *   accum    optional (B, NQ, H*dh) contiguous: the self-attention output to add to (bf16
  *            addition as torch performs it); may equal out
  *   out      (B, NQ, H*dh) contiguous
- * Requirements: dtype BNB_BF16, dh == 32, 1 <= NK <= 2048, NQ <= 160, 16-byte aligned rows;
- * anything else returns BNB_ERR_UNSUPPORTED and the caller keeps its library path.  Up to
- * 160 keys are staged in LDS at once; longer key axes (the shipped scenarios have 10 bullet
- * slots per ship, 80 .. 1520 keys) are streamed in tiles of the active keys only, so the
- * cost follows the number of bullets in flight, not the number of slots.
+ * Requirements: dh == 32, 16-byte aligned rows; BNB_BF16 with 1 <= NK <= 2048, NQ <= 160, or
+ * BNB_F32 (evaluation without autocast, evaluation/agents.py:214-219; true fp32 products on the
+ * matrix cores, fp32 addition into accum) with 1 <= NK <= 4096, NQ <= 512; anything else returns
+ * BNB_ERR_UNSUPPORTED and the caller keeps its library path.  Up to 160 keys are staged in LDS at
+ * once; longer key axes (the shipped scenarios have 10 bullet slots per ship, 80 .. 1520 keys)
+ * are streamed in tiles of the active keys only, so the cost follows the number of bullets in
+ * flight, not the number of slots.
  */
 int bnb_sdpa_cross_fwd(const void *q, int64_t q_row_stride, int NQ, const void *k, const void *v,
                        int64_t kv_row_stride, int NK, const uint8_t *key_mask, const void *accum,

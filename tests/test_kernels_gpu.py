@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from helpers import max_rel, team_case, team_pool_params
-from oracle import c_ref, torch_ref
+from oracle import bruteforce, c_ref, torch_ref
 
 from boost_and_broadside_amd import harness, ops
 
@@ -379,10 +379,49 @@ def test_sdpa_cross_streams_long_key_axes(B, NQ, NK, p_live):
     assert max_rel(no_mask, torch_ref.bullet_read(qkv.float(), kv.float(), None, H)) <= BF16_TOL
 
 
+@pytest.mark.parametrize("B,NQ,NK,p_live", [(4, 12, 80, 0.5), (3, 20, 160, 0.25), (5, 12, 7, 0.5), (2, 84, 800, 0.3),
+                                           (2, 160, 1520, 1.0), (3, 160, 1520, 0.1), (2, 320, 3200, 0.25), (2, 33, 4096, 0.7),
+                                           (3, 20, 500, 0.02), (2, 160, 1, 1.0), (2, 512, 97, 0.6)])
+def test_sdpa_cross_fp32_matches_oracle(B, NQ, NK, p_live):
+    # evaluation without autocast: the same read on the fp32 matrix cores, float32 bar
+    H, D = 4, 128
+    g = torch.Generator().manual_seed(NQ * 5000 + NK)
+    qkv = torch.randn(B, NQ, 3 * D, generator=g)
+    kv = torch.randn(B, NK, 2 * D, generator=g)
+    kv[:, :, :D] *= 2.0  # peaked rows: the running maximum moves between tiles
+    mask = torch.rand(B, NK, generator=g) < p_live
+    mask[0] = False  # nothing active in env 0
+    mask[1, NK - 1] = True
+    merged = torch.randn(B, NQ, D, generator=g)
+    truth = torch_ref.bullet_read(qkv, kv, mask, H)
+    bare = ops.sdpa_cross(qkv.to(DEV), kv.to(DEV), mask.to(DEV), H).cpu()
+    assert bare.dtype == torch.float32 and bare[0].abs().max() == 0  # gated off exactly
+    assert max_rel(bare, truth) <= F32_TOL
+    if NK <= 200:  # the float64 loop statement on a few queries
+        brute = bruteforce.bullet_read_loops(qkv[1:2, :3, :D].numpy(), kv[1:2].numpy(), mask[1:2].numpy(), H)
+        assert max_rel(bare[1:2, :3].double(), torch.as_tensor(brute)) <= F32_TOL
+    acc = merged.to(DEV).clone()
+    out = ops.sdpa_cross(qkv.to(DEV), kv.to(DEV), mask.to(DEV), H, accum=acc)
+    assert out.data_ptr() == acc.data_ptr()
+    assert torch.equal(out.cpu(), merged + bare)  # one float32 addition
+    assert torch.equal(out[0].cpu(), merged[0])  # env 0 untouched
+    other = torch.empty_like(acc)
+    got = ops.sdpa_cross(qkv.to(DEV), kv.to(DEV), mask.to(DEV), H, accum=merged.to(DEV), out=other)
+    assert torch.equal(got.cpu(), out.cpu())
+    # inactive slots cannot influence the result; strided views of wider buffers work
+    kv2 = kv.clone()
+    kv2[~mask] = kv2[~mask] * -2.0 + 9.0
+    assert torch.equal(ops.sdpa_cross(qkv.to(DEV), kv2.to(DEV), mask.to(DEV), H).cpu(), bare)
+    no_mask = ops.sdpa_cross(qkv.to(DEV), kv.to(DEV), None, H).cpu()
+    assert max_rel(no_mask, torch_ref.bullet_read(qkv, kv, None, H)) <= F32_TOL
+
+
 def test_sdpa_cross_limits():
     qkv = torch.zeros(1, 12, 384, device=DEV, dtype=torch.bfloat16)
     assert not ops.cross_supported(qkv, torch.zeros(1, 2049, 256, device=DEV, dtype=torch.bfloat16), 4)
-    assert not ops.cross_supported(qkv.float(), torch.zeros(1, 80, 256, device=DEV), 4)
+    assert ops.cross_supported(qkv.float(), torch.zeros(1, 80, 256, device=DEV), 4)  # float32 has its own kernel
+    assert not ops.cross_supported(qkv.float(), torch.zeros(1, 80, 256, device=DEV, dtype=torch.bfloat16), 4)  # one dtype
+    assert not ops.cross_supported(qkv.float(), torch.zeros(1, 4097, 256, device=DEV), 4)
     with pytest.raises(RuntimeError):
         ops.sdpa_cross(qkv, torch.zeros(1, 2100, 256, device=DEV, dtype=torch.bfloat16), None, 4)
 
