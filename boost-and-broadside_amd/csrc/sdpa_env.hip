@@ -1,0 +1,276 @@
+// Masked self-attention, one work-group per environment, heads streamed through LDS (gfx950).
+//
+// Same function as sdpa_mfma_kernel (models/yemong/attention.py:101-112,136-147,168): bf16, four
+// heads of 32 channels, up to 160 tokens, dead keys compacted away, an environment without a live
+// key averages V over all keys.  What differs is how the data gets to the matrix cores:
+//
+//   * The work-group owns ALL heads of its environment.  The alive row is read once and the list
+//     of live keys (position -> token index) is built once, instead of once per head.
+//   * K and V rows travel global -> LDS directly (global_load_lds_dwordx4: a wave moves 1 KB per
+//     instruction, lane l filling LDS bytes 16 l .. 16 l + 15 of the wave's kilobyte), never
+//     through registers, so the next head's rows are in flight while the current head is being
+//     computed and no lane spends instructions on staging.  Two LDS buffers alternate.
+//   * A staged key is 128 bytes: [K 64 B | V 64 B] of one head, i.e. eight 16-byte chunks.  A
+//     lane may fetch ANY global chunk into its fixed LDS slot, so chunk c of position p is kept in
+//     slot c ^ f(p), f(p) = 2 (p%4) + (p/4)%2: eight consecutive keys put one chunk into eight
+//     different slots (K operand reads: 16 B of each of 32 keys), and four consecutive keys put a
+//     32-byte chunk pair into four different pairs (V operand reads: 32 B of each of 4 keys per
+//     16 lanes), so both spread over all banks although the key pitch is a power of two.
+//   * V stays row-major.  The A operand of O^T = V^T P^T needs, per lane, eight keys of ONE
+//     channel; ds_read_b64_tr_b16 delivers exactly that from row-major data: inside a group of 16
+//     lanes, lane i receives element i%4 of the 8-byte pieces addressed by lanes i/4, i/4 + 4,
+//     i/4 + 8, i/4 + 12.  Source lane r therefore points at key (r/4) of the four keys wanted and
+//     at the 4-channel block r%4 of the group's 16 output rows.  The eight 2-byte LDS writes per
+//     item that a transposed copy of V costs are gone.
+//
+// Thread roles: wave w owns queries 32w .. 32w+31 (S^T = K Q^T with keys on the M axis, so a lane
+// holds 16 scores of one query per key block; softmax reductions are in-lane plus one exchange
+// between the wave's halves), for every head in turn.  Padding (positions [0, pad) of key block 0)
+// is filled with a copy of the first live key and enters as -inf through the initial accumulator.
+
+#include "common.h"
+
+#include <type_traits>
+
+namespace bnb {
+
+constexpr int kEnvDh = 32;
+constexpr int kEnvHeads = 4;
+constexpr int kEnvD = kEnvDh * kEnvHeads;
+constexpr int kEnvKeyBytes = 128;  // one staged key of one head: [K | V]
+
+// 16 bytes per lane from `sbase + voff` to LDS byte address lds_base + 16 * lane.  No immediate
+// offset: the instruction would add it to the LDS address as well as to the global one.
+__device__ __forceinline__ void dma_row16(const void *sbase, uint32_t voff, uint32_t lds_base)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
+                 :
+                 : "s"(sbase), "v"(voff), "s"(lds_base)
+                 : "memory");
+}
+
+// slot permutation of the eight 16-byte chunks of staged key p (p % 8 passed in)
+__device__ __forceinline__ int swizzle(int p8) { return ((p8 & 3) << 1) | ((p8 >> 2) & 1); }
+
+__device__ __forceinline__ bf16x8 lds_tr_pair(const uint16_t *p)
+{
+    typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+    typedef bf16x4_t __attribute__((address_space(3))) * lds_ptr;
+    const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_ptr)p);
+    const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_ptr)(p + 8 * kEnvKeyBytes / 2));  // eight keys further on
+    return bf16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+}
+
+template <int NQB>
+__global__ __launch_bounds__(kWave * NQB) void sdpa_env_kernel(const uint16_t *__restrict__ qkv, int64_t stride,
+                                                              const uint8_t *__restrict__ alive, uint16_t *__restrict__ out,
+                                                              int B, int NM, float scale_log2e)
+{
+    constexpr int KCAP = NQB * 32;
+    constexpr int H = kEnvHeads, D = kEnvD;
+    __shared__ __align__(1024) uint16_t s_buf[2][KCAP * kEnvKeyBytes / 2];
+    __shared__ uint16_t s_idx[KCAP];
+    __shared__ int s_cnt[NQB];
+
+    const int env = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m = lane & 31;
+    const int half = lane >> 5;
+    const uint16_t *env_base = qkv + (int64_t)env * NM * stride;
+
+    // ---- this lane's query, all heads: column m of every S^T block this wave forms ----
+    const int qrow = wave * 32 + m;
+    const int qsafe = qrow < NM ? qrow : NM - 1;
+    const uint16_t *qp = env_base + (uint32_t)qsafe * (uint32_t)stride + half * 8;
+    u32x4 qw[H][2];
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+        qw[h][0] = *reinterpret_cast<const u32x4 *>(qp + h * kEnvDh);
+        qw[h][1] = *reinterpret_cast<const u32x4 *>(qp + h * kEnvDh + 16);
+    }
+
+    // ---- list of live keys (position -> token), once for all heads ----
+    uint32_t a = 1u;
+    if (alive != nullptr) a = alive[(int64_t)env * NM + (tid < NM ? tid : NM - 1)];
+    bool live = tid < NM && a != 0;
+    const uint64_t lmask = __ballot(live);
+    const int before = (int)__popcll(lmask & ((1ull << lane) - 1ull));
+    if (lane == 0) s_cnt[wave] = (int)__popcll(lmask);
+    __syncthreads();
+    int base = 0, cnt = 0;
+#pragma unroll
+    for (int w = 0; w < NQB; ++w) {
+        const int c = s_cnt[w];
+        if (w < wave) base += c;
+        cnt += c;
+    }
+    // no live key at all: every key takes part with the same weight (all scores equal)
+    const bool uniform = cnt == 0;
+    int pos = base + before;
+    if (uniform) {
+        live = tid < NM;
+        pos = tid;
+        cnt = NM;
+    }
+    if (live) s_idx[pos] = (uint16_t)tid;
+    __syncthreads();
+    const int nkb = (cnt + 31) >> 5;
+    const int pad = nkb * 32 - cnt;  // positions [0, pad) of key block 0 hold a copy of the first live key
+
+    // ---- the load instructions this wave issues per head: j = wave, wave + NQB, ... < 4 nkb ----
+    // instruction j fills LDS kilobyte j of the buffer: lane l -> position 8j + l/8, slot l%8, which
+    // holds global chunk (l%8) ^ f(position % 8) = (l%8) ^ f((l/8)%8)
+    const int chunk = (lane & 7) ^ swizzle((lane >> 3) & 7);
+    const uint32_t chan_bytes = (uint32_t)(((1 + (chunk >> 2)) * D + (chunk & 3) * 8) * 2);
+    uint32_t voff[4];
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+        const int j = wave + jj * NQB;
+        int li = j * 8 + (lane >> 3) - pad;
+        li = li > 0 ? li : 0;
+        li = li < cnt ? li : cnt - 1;  // instructions past 4 nkb are never issued; keep the read in range
+        voff[jj] = (uint32_t)s_idx[li] * (uint32_t)stride * 2u + chan_bytes;
+    }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)&s_buf[0][0];
+    constexpr uint32_t kBufBytes = KCAP * kEnvKeyBytes;
+    const int ninstr = nkb * 4;
+
+    auto issue = [&](auto head_tag, int buf) {
+        constexpr int h = decltype(head_tag)::value;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int j = wave + jj * NQB;
+            if (j < ninstr) dma_row16(env_base + h * kEnvDh, voff[jj], lds0 + (uint32_t)buf * kBufBytes + (uint32_t)j * 1024u);
+        }
+    };
+
+    // ---- per-lane LDS offsets (halfs) of the operands inside a buffer, key block 0 ----
+    // K (A operand of S^T): key m, channels 8 half .. (first product) and 16 + 8 half .. (second)
+    const int ksw = swizzle(m & 7);
+    const int k_off0 = m * (kEnvKeyBytes / 2) + ((half ^ ksw) * 8);
+    const int k_off1 = m * (kEnvKeyBytes / 2) + (((2 + half) ^ ksw) * 8);
+    // V (A operand of O^T through the transposing read): as SOURCE lane r = lane % 16 of group g = lane / 16
+    // this lane points at key 4 (g/2) + r/4 of the 16 keys of one product and at output-row block
+    // rb = 4 (g%2) + r%4, which is channel block cb(rb) (see the output stage: MFMA row 8i + 4 half + j
+    // is channel 16 (i/2) + 8 half + 4 (i%2) + j, i.e. row block 2i + half -> channel block 4 (i/2) + 2 half + i%2)
+    const int grp = lane >> 4, r = lane & 15;
+    const int rb = 4 * (grp & 1) + (r & 3);
+    const int cb = 4 * (rb >> 2) + 2 * (rb & 1) + ((rb >> 1) & 1);
+    const int vkey = 4 * (grp >> 1) + (r >> 2);  // + 16 t + 32 kb (+ 8 for the second half of the operand)
+    const int v_off = vkey * (kEnvKeyBytes / 2) + (((4 + (cb >> 1)) ^ swizzle(vkey & 7)) * 8) + (cb & 1) * 4;
+
+    f32x16 bias0;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) bias0[v] = (8 * (v >> 2) + 4 * half + (v & 3) < pad) ? -INFINITY : 0.0f;
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    const int64_t o_row = ((int64_t)env * NM + qsafe) * D + 8 * half;
+
+    issue(std::integral_constant<int, 0>{}, 0);
+    issue(std::integral_constant<int, 1>{}, 1);
+
+    u32x4 held[2];  // the previous head's output, stored after the next barrier
+    auto compute = [&](auto head_tag) {
+        constexpr int h = decltype(head_tag)::value;
+        const uint16_t *buf = &s_buf[h & 1][0];
+        const bf16x8 qb0 = __builtin_bit_cast(bf16x8, uniform ? zero4 : qw[h][0]);
+        const bf16x8 qb1 = __builtin_bit_cast(bf16x8, uniform ? zero4 : qw[h][1]);
+        auto scores = [&](int kb) -> f32x16 {
+            const uint16_t *kp = buf + kb * 32 * (kEnvKeyBytes / 2);
+            const bf16x8 ka0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + k_off0));
+            const bf16x8 ka1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + k_off1));
+            f32x16 z = {0.0f};
+            if (kb == 0) z = bias0;
+            z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0, qb0, z, 0, 0, 0);
+            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka1, qb1, z, 0, 0, 0);
+        };
+        float mx = -INFINITY;
+        for (int kb = 0; kb < nkb; ++kb) {
+            const f32x16 z = scores(kb);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float mc = mx * scale_log2e;
+        float sum = 0.0f;
+        f32x16 o = {0.0f};
+        for (int kb = 0; kb < nkb; ++kb) {
+            const f32x16 z = scores(kb);
+            float p[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                p[v] = __builtin_amdgcn_exp2f(fmaf(z[v], scale_log2e, -mc));
+                sum += p[v];
+            }
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                bf16x8 pb;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * t + e];
+                const bf16x8 va = lds_tr_pair(buf + (kb * 32 + 16 * t) * (kEnvKeyBytes / 2) + v_off);
+                o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb, o, 0, 0, 0);
+            }
+        }
+        sum += __shfl_xor(sum, 32);
+        const float inv = __builtin_amdgcn_rcpf(sum);
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+            held[g] = u32x4{pack_bf16x2(o[8 * g + 0] * inv, o[8 * g + 1] * inv), pack_bf16x2(o[8 * g + 2] * inv, o[8 * g + 3] * inv),
+                            pack_bf16x2(o[8 * g + 4] * inv, o[8 * g + 5] * inv), pack_bf16x2(o[8 * g + 6] * inv, o[8 * g + 7] * inv)};
+    };
+    auto store = [&](int h) {
+        if (qrow < NM) {
+            *reinterpret_cast<u32x4 *>(out + o_row + h * kEnvDh) = held[0];
+            *reinterpret_cast<u32x4 *>(out + o_row + h * kEnvDh + 16) = held[1];
+        }
+    };
+
+    // Head h is computed out of buffer h%2 while head h+1 lands in the other one.  One barrier per
+    // head: it says both "everybody's rows of head h have landed" (each wave waits for its own loads
+    // first) and "everybody is done reading head h-1", after which head h+1 may overwrite that buffer.
+    // The only vector-memory traffic issued between a head's loads and the wait for them is nothing
+    // at all (the previous head's output is stored right after the barrier, before the next loads),
+    // so every wait is a plain vmcnt(0) for work issued a whole head earlier.
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the queries and heads 0 and 1 of this wave's rows
+    __syncthreads();
+    compute(std::integral_constant<int, 0>{});
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    store(0);
+    issue(std::integral_constant<int, 2>{}, 0);
+    compute(std::integral_constant<int, 1>{});
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    store(1);
+    issue(std::integral_constant<int, 3>{}, 1);
+    compute(std::integral_constant<int, 2>{});
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    store(2);
+    compute(std::integral_constant<int, 3>{});
+    store(3);
+}
+
+template <int NQB>
+static int launch_env(const void *qkv, int64_t stride, const uint8_t *alive, void *out, int B, int NM, hipStream_t stream)
+{
+    hipLaunchKernelGGL((sdpa_env_kernel<NQB>), dim3((unsigned)B), dim3(kWave * NQB), 0, stream, (const uint16_t *)qkv, stride, alive,
+                       (uint16_t *)out, B, NM, 1.4426950408889634f / sqrtf((float)kEnvDh));
+    return (int)hipGetLastError();
+}
+
+// bf16, 4 heads of 32 channels, 1 <= NM <= 160, rows of one environment within 2^31 bytes.
+int dispatch_env(const void *qkv, int64_t stride, const uint8_t *alive, void *out, int B, int NM, hipStream_t stream)
+{
+    switch ((NM + 31) / 32) {
+        case 1: return launch_env<1>(qkv, stride, alive, out, B, NM, stream);
+        case 2: return launch_env<2>(qkv, stride, alive, out, B, NM, stream);
+        case 3: return launch_env<3>(qkv, stride, alive, out, B, NM, stream);
+        case 4: return launch_env<4>(qkv, stride, alive, out, B, NM, stream);
+        case 5: return launch_env<5>(qkv, stride, alive, out, B, NM, stream);
+        default: return BNB_ERR_UNSUPPORTED;
+    }
+}
+
+}  // namespace bnb

@@ -1133,6 +1133,9 @@ static int dispatch_cross_stream(const void *q, int64_t q_stride, const void *k,
     }
 }
 
+// defined in sdpa_env.hip: bf16, 4 heads of 32 channels, NM <= 160, one work-group per environment
+int dispatch_env(const void *qkv, int64_t stride, const uint8_t *alive, void *out, int B, int NM, hipStream_t stream);
+
 // defined in sdpa_cross_f32.hip
 int launch_cross_f32(const void *q, int64_t q_stride, const void *k, const void *v, int64_t kv_stride, const uint8_t *key_mask,
                      const void *accum, void *out, int B, int NQ, int NK, int H, hipStream_t stream);
@@ -1146,7 +1149,7 @@ extern "C" int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride,
     using namespace bnb;
     if (B < 0 || NM < 0 || H < 1 || dh < 1) return BNB_ERR_BAD_SHAPE;
     if (dtype != BNB_F32 && dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
-    if (path < BNB_SDPA_PATH_AUTO || path > BNB_SDPA_PATH_MFMA) return BNB_ERR_UNSUPPORTED;
+    if (path < BNB_SDPA_PATH_AUTO || path > BNB_SDPA_PATH_ENV) return BNB_ERR_UNSUPPORTED;
     if (B == 0 || NM == 0) return 0;
     if (!qkv || !out) return BNB_ERR_NULL_POINTER;
     if (qkv_row_stride < (int64_t)3 * H * dh) return BNB_ERR_BAD_SHAPE;
@@ -1158,6 +1161,11 @@ extern "C" int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride,
     // the matrix-core kernel addresses rows inside one environment with 32-bit offsets
     const bool mfma_ok = dtype == BNB_BF16 && dh == kDh && NM <= 160 && (int64_t)NM * qkv_row_stride < (1LL << 30);
     if (path == BNB_SDPA_PATH_MFMA && !mfma_ok) return BNB_ERR_UNSUPPORTED;
+    // one work-group per environment, rows straight into LDS: four heads only, byte offsets inside an environment in 32 bits
+    const bool env_ok = mfma_ok && H == 4 && (int64_t)NM * qkv_row_stride < (1LL << 30);
+    if (path == BNB_SDPA_PATH_ENV && !env_ok) return BNB_ERR_UNSUPPORTED;
+    if (path == BNB_SDPA_PATH_ENV)
+        return dispatch_env(qkv, qkv_row_stride, alive, out, B, NM, s);
     // measured on MI355X the matrix-core kernel wins at every token count it covers, 4v4 included
     // (12 tokens: 24.7 us vs 45.5 us for 8192 environments), so AUTO takes it whenever it applies
     const bool use_mfma = path == BNB_SDPA_PATH_MFMA || (path == BNB_SDPA_PATH_AUTO && mfma_ok);

@@ -30,7 +30,7 @@ def _outside_autocast(backward):
     return wrapped
 
 
-_PATH_CODE = {"auto": _native.PATH_AUTO, "valu": _native.PATH_VALU, "mfma": _native.PATH_MFMA}
+_PATH_CODE = {"auto": _native.PATH_AUTO, "valu": _native.PATH_VALU, "mfma": _native.PATH_MFMA, "env": _native.PATH_ENV}
 
 
 def _need_device(t: torch.Tensor, name: str) -> None:
@@ -70,7 +70,8 @@ def sdpa_masked(
                  Dead keys get weight 0; an environment with no live key averages V over
                  all keys; dead queries are still computed.
         n_heads: H; D must be divisible by it.
-        path:    "auto" | "valu" | "mfma" — kernel selection, for tests and benchmarks.
+        path:    "auto" | "valu" | "mfma" | "env" — kernel selection, for tests and benchmarks ("mfma": one
+                 work-group per (environment, head); "env": one per environment, heads streamed through LDS).
         out:     optional preallocated contiguous (B, NM, D) destination in qkv's dtype.
 
     Returns:

@@ -81,11 +81,15 @@ int bnb_sdpa_masked_fwd(const void *qkv, int64_t qkv_row_stride, const uint8_t *
  *                       dh == 32 and NM <= 160; the fp32 matrix-core kernel for fp32, dh == 32
  *                       and NM <= 512; the vector-ALU kernel otherwise
  *   BNB_SDPA_PATH_VALU  vector-ALU kernel (any supported shape and dtype)
- *   BNB_SDPA_PATH_MFMA  bf16 matrix-core kernel (bf16, dh == 32, NM <= 160; else BNB_ERR_UNSUPPORTED)
+ *   BNB_SDPA_PATH_MFMA  bf16 matrix-core kernel, one work-group per (environment, head) (bf16, dh == 32,
+ *                       NM <= 160; else BNB_ERR_UNSUPPORTED)
+ *   BNB_SDPA_PATH_ENV   bf16 matrix-core kernel, one work-group per environment with the heads streamed
+ *                       through LDS (bf16, H == 4, dh == 32, NM <= 160; else BNB_ERR_UNSUPPORTED)
  */
 #define BNB_SDPA_PATH_AUTO 0
 #define BNB_SDPA_PATH_VALU 1
 #define BNB_SDPA_PATH_MFMA 2
+#define BNB_SDPA_PATH_ENV 3
 int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, void *out,
                              int B, int NM, int H, int dh, int dtype, int path, void *stream);
 

@@ -224,6 +224,65 @@ def test_sdpa_mfma_live_counts_across_block_edges():
         assert max_rel(got[b], truth[b]) <= BF16_TOL, counts[b]
 
 
+@pytest.mark.parametrize("NM", [1, 7, 12, 23, 31, 32, 33, 64, 65, 84, 96, 97, 128, 129, 159, 160])
+def test_sdpa_environment_kernel_matches_oracle_and_the_per_head_kernel(NM):
+    # one work-group per environment, K/V rows straight into LDS, V read through the transposing LDS load.
+    # Per environment: mixed, all alive, all dead, only the first and only the last token alive, then
+    # random live counts that cross every key-block edge
+    B, H, D = 24, 4, 128
+    qkv = _qkv(700 + NM, B, NM, D, torch.bfloat16)
+    g = torch.Generator().manual_seed(700 + NM)
+    alive = _alive(701 + NM, B, NM, 0.6)
+    alive[0] = True
+    alive[1] = False
+    alive[2] = False
+    alive[2, 0] = True
+    alive[3] = False
+    alive[3, NM - 1] = True
+    for b in range(4, B):
+        alive[b] = False
+        alive[b, torch.randperm(NM, generator=g)[: int(torch.randint(1, NM + 1, (1,), generator=g))]] = True
+    got = _run_sdpa(qkv, alive, H, "env").float()
+    truth = torch_ref.sdpa_masked(qkv.float(), alive, H)
+    assert torch.isfinite(got).all()
+    for b in range(B):
+        assert max_rel(got[b], truth[b]) <= BF16_TOL, (b, int(alive[b].sum()))
+    mean_v = qkv[1, :, 2 * D:].float().mean(dim=0, keepdim=True).expand(NM, D)
+    assert (got[1] - mean_v).abs().max() <= 1.6e-2
+    assert torch.equal(got[3], qkv[3, NM - 1, 2 * D:].float().expand(NM, D))  # one live key: its V row, exactly
+    # the same arithmetic in the same order as the per-head kernel: identical bits
+    assert torch.equal(got, _run_sdpa(qkv, alive, H, "mfma").float())
+    # dead keys weigh exactly nothing: rewriting their K and V rows changes no output bit
+    pert = qkv.clone()
+    dead = ~alive
+    dead[~alive.any(dim=1)] = False  # an all-dead environment averages every row
+    pert[..., D:][dead] = pert[..., D:][dead] * -3.0 + 17.0
+    assert torch.equal(_run_sdpa(pert, alive, H, "env").float(), got)
+    # heads do not leak into each other
+    other = qkv.clone()
+    for part in range(3):
+        other[..., part * D + 64: part * D + 96] = other[..., part * D + 64: part * D + 96] * 2.0 + 1.0
+    again = _run_sdpa(other, alive, H, "env").float()
+    keep = torch.ones(D, dtype=torch.bool)
+    keep[64:96] = False
+    assert torch.equal(again[..., keep], got[..., keep]) and not torch.equal(again[..., 64:96], got[..., 64:96])
+    # no mask, and rows that are a view of a wider buffer
+    wide = torch.zeros(B, NM, 3 * D + 64, dtype=torch.bfloat16)
+    wide[..., : 3 * D] = qkv
+    view = wide.to(DEV)[..., : 3 * D]
+    assert torch.equal(ops.sdpa_masked(view, alive.to(DEV), H, path="env").float().cpu(), got)
+    assert max_rel(ops.sdpa_masked(view, None, H, path="env").float().cpu(), torch_ref.sdpa_masked(qkv.float(), None, H)) <= BF16_TOL
+
+
+def test_sdpa_environment_kernel_limits():
+    with pytest.raises(RuntimeError, match="outside what the kernels cover"):
+        ops.sdpa_masked(torch.zeros(1, 12, 192, device=DEV, dtype=torch.bfloat16), None, 2, path="env")  # two heads
+    with pytest.raises(RuntimeError, match="outside what the kernels cover"):
+        ops.sdpa_masked(torch.zeros(1, 161, 384, device=DEV, dtype=torch.bfloat16), None, 4, path="env")
+    with pytest.raises(RuntimeError, match="outside what the kernels cover"):
+        ops.sdpa_masked(torch.zeros(1, 12, 384, device=DEV), None, 4, path="env")  # float32
+
+
 @pytest.mark.parametrize("NM", [1, 2, 5, 12, 15, 16])
 @pytest.mark.parametrize("H", [2, 4, 8, 3])
 def test_sdpa_two_heads_per_wave_for_up_to_16_tokens(NM, H):
