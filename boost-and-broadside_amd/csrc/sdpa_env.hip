@@ -30,6 +30,8 @@
 
 #include "common.h"
 
+#include <stdlib.h>
+
 #include <type_traits>
 
 namespace bnb {
@@ -62,62 +64,95 @@ __device__ __forceinline__ bf16x8 lds_tr_pair(const uint16_t *p)
 }
 
 template <int NQB>
-__global__ __launch_bounds__(kWave * NQB) void sdpa_env_kernel(const uint16_t *__restrict__ qkv, int64_t stride,
+__global__ __launch_bounds__(kWave * NQB, 4) void sdpa_env_kernel(const uint16_t *__restrict__ qkv, int64_t stride,
                                                               const uint8_t *__restrict__ alive, uint16_t *__restrict__ out,
-                                                              int B, int NM, float scale_log2e)
+                                                              int B, int NM, int envs_per_group, float scale_log2e)
 {
     constexpr int KCAP = NQB * 32;
     constexpr int H = kEnvHeads, D = kEnvD;
+    // exactly 2 x 20 KB at 160 tokens: three work-groups share a CU only up to 40 KB each (measured), so the
+    // list of live keys is kept out of LDS memory (every wave derives its part from the alive row by itself)
     __shared__ __align__(1024) uint16_t s_buf[2][KCAP * kEnvKeyBytes / 2];
-    __shared__ uint16_t s_idx[KCAP];
-    __shared__ int s_cnt[NQB];
 
-    const int env = blockIdx.x;
+    // A work-group walks environments first, first + step, ...; while it computes one, the next one's
+    // alive row, key list, queries and first head are already on their way.
+    const int first = blockIdx.x;
+    const int step = envs_per_group;  // = gridDim.x
+    const int last = B;               // exclusive
+    if (first >= B) return;
+
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int m = lane & 31;
     const int half = lane >> 5;
-    const uint16_t *env_base = qkv + (int64_t)env * NM * stride;
+    const int64_t env_pitch = (int64_t)NM * stride * step;
 
-    // ---- this lane's query, all heads: column m of every S^T block this wave forms ----
+    // this lane's query: column m of every S^T block this wave forms
     const int qrow = wave * 32 + m;
     const int qsafe = qrow < NM ? qrow : NM - 1;
-    const uint16_t *qp = env_base + (uint32_t)qsafe * (uint32_t)stride + half * 8;
+    const uint32_t q_off = (uint32_t)qsafe * (uint32_t)stride + half * 8;
     u32x4 qw[H][2];
-#pragma unroll
-    for (int h = 0; h < H; ++h) {
-        qw[h][0] = *reinterpret_cast<const u32x4 *>(qp + h * kEnvDh);
-        qw[h][1] = *reinterpret_cast<const u32x4 *>(qp + h * kEnvDh + 16);
-    }
+    auto load_q = [&](const uint16_t *base, auto head_tag) {
+        constexpr int h = decltype(head_tag)::value;
+        qw[h][0] = *reinterpret_cast<const u32x4 *>(base + q_off + h * kEnvDh);
+        qw[h][1] = *reinterpret_cast<const u32x4 *>(base + q_off + h * kEnvDh + 16);
+    };
 
-    // ---- list of live keys (position -> token), once for all heads ----
-    uint32_t a = 1u;
-    if (alive != nullptr) a = alive[(int64_t)env * NM + (tid < NM ? tid : NM - 1)];
-    bool live = tid < NM && a != 0;
-    const uint64_t lmask = __ballot(live);
-    const int before = (int)__popcll(lmask & ((1ull << lane) - 1ull));
-    if (lane == 0) s_cnt[wave] = (int)__popcll(lmask);
-    __syncthreads();
-    int base = 0, cnt = 0;
+    // ---- list of live keys (position -> token), once per environment, per wave, without LDS memory ----
+    // Every wave reads the whole alive row (lane l: tokens l, l + 64, l + 128) and keeps it as three
+    // 64-bit masks; the token at live position n is the index of the n-th set bit.
+    struct AliveRow { uint32_t a[3]; };
+    auto load_alive = [&](int env) -> AliveRow {
+        AliveRow r;
 #pragma unroll
-    for (int w = 0; w < NQB; ++w) {
-        const int c = s_cnt[w];
-        if (w < wave) base += c;
-        cnt += c;
-    }
-    // no live key at all: every key takes part with the same weight (all scores equal)
-    const bool uniform = cnt == 0;
-    int pos = base + before;
-    if (uniform) {
-        live = tid < NM;
-        pos = tid;
-        cnt = NM;
-    }
-    if (live) s_idx[pos] = (uint16_t)tid;
-    __syncthreads();
-    const int nkb = (cnt + 31) >> 5;
-    const int pad = nkb * 32 - cnt;  // positions [0, pad) of key block 0 hold a copy of the first live key
+        for (int w = 0; w < 3; ++w) {
+            const int tok = lane + 64 * w;
+            r.a[w] = 0u;
+            if (w * 64 < KCAP) {
+                const uint32_t in = tok < NM ? 1u : 0u;
+                r.a[w] = alive == nullptr ? in : (in ? (uint32_t)alive[(int64_t)env * NM + tok] : 0u);
+            }
+        }
+        return r;
+    };
+    struct KeyList { uint64_t m[3]; int c0, c1, cnt; bool uniform; };
+    auto make_list = [&](const AliveRow &r) -> KeyList {
+        KeyList k;
+#pragma unroll
+        for (int w = 0; w < 3; ++w) k.m[w] = __ballot(r.a[w] != 0);
+        k.c0 = (int)__popcll(k.m[0]);
+        k.c1 = (int)__popcll(k.m[1]);
+        k.cnt = k.c0 + k.c1 + (int)__popcll(k.m[2]);
+        // no live key at all: every key takes part with the same weight (all scores equal)
+        k.uniform = k.cnt == 0;
+        if (k.uniform) {
+#pragma unroll
+            for (int w = 0; w < 3; ++w) k.m[w] = __ballot(lane + 64 * w < NM);
+            k.c0 = (int)__popcll(k.m[0]);
+            k.c1 = (int)__popcll(k.m[1]);
+            k.cnt = NM;
+        }
+        return k;
+    };
+    // index of the n-th set bit (n counted from 0, n < cnt) of the 160-bit row
+    auto nth_live = [&](const KeyList &k, int n) -> int {
+        uint64_t w = k.m[0];
+        int base = 0;
+        if (n >= k.c0) {
+            n -= k.c0, w = k.m[1], base = 64;
+            if (n >= k.c1) n -= k.c1, w = k.m[2], base = 128;
+        }
+        uint32_t x = (uint32_t)w;
+        int c = __popc(x);
+        if (n >= c) n -= c, x = (uint32_t)(w >> 32), base += 32;
+#pragma unroll
+        for (int width = 16; width >= 1; width >>= 1) {
+            c = __popc(x & ((1u << width) - 1u));
+            if (n >= c) n -= c, x >>= width, base += width;
+        }
+        return base;
+    };
 
     // ---- the load instructions this wave issues per head: j = wave, wave + NQB, ... < 4 nkb ----
     // instruction j fills LDS kilobyte j of the buffer: lane l -> position 8j + l/8, slot l%8, which
@@ -125,24 +160,28 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_env_kernel(const uint16_t *_
     const int chunk = (lane & 7) ^ swizzle((lane >> 3) & 7);
     const uint32_t chan_bytes = (uint32_t)(((1 + (chunk >> 2)) * D + (chunk & 3) * 8) * 2);
     uint32_t voff[4];
+    auto make_offsets = [&](const KeyList &k, int pad) {
+        // lane t (and t + 32) works out the token of the wave's t-th position: instruction t/8, position t%8 in it;
+        // padding positions hold a copy of the first live key; instructions past 4 nkb are never issued
+        const int t = lane & 31;
+        int n = (wave + (t >> 3) * NQB) * 8 + (t & 7) - pad;
+        n = n > 0 ? n : 0;
+        n = n < k.cnt ? n : k.cnt - 1;
+        const int token = nth_live(k, n);
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-        const int j = wave + jj * NQB;
-        int li = j * 8 + (lane >> 3) - pad;
-        li = li > 0 ? li : 0;
-        li = li < cnt ? li : cnt - 1;  // instructions past 4 nkb are never issued; keep the read in range
-        voff[jj] = (uint32_t)s_idx[li] * (uint32_t)stride * 2u + chan_bytes;
-    }
+        for (int jj = 0; jj < 4; ++jj) {
+            const int tok = __builtin_amdgcn_ds_bpermute((jj * 8 + (lane >> 3)) * 4, token);
+            voff[jj] = (uint32_t)tok * (uint32_t)stride * 2u + chan_bytes;
+        }
+    };
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)&s_buf[0][0];
     constexpr uint32_t kBufBytes = KCAP * kEnvKeyBytes;
-    const int ninstr = nkb * 4;
-
-    auto issue = [&](auto head_tag, int buf) {
+    auto issue = [&](const uint16_t *base, auto head_tag, int ninstr) {
         constexpr int h = decltype(head_tag)::value;
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
             const int j = wave + jj * NQB;
-            if (j < ninstr) dma_row16(env_base + h * kEnvDh, voff[jj], lds0 + (uint32_t)buf * kBufBytes + (uint32_t)j * 1024u);
+            if (j < ninstr) dma_row16(base + h * kEnvDh, voff[jj], lds0 + (uint32_t)(h & 1) * kBufBytes + (uint32_t)j * 1024u);
         }
     };
 
@@ -161,19 +200,23 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_env_kernel(const uint16_t *_
     const int vkey = 4 * (grp >> 1) + (r >> 2);  // + 16 t + 32 kb (+ 8 for the second half of the operand)
     const int v_off = vkey * (kEnvKeyBytes / 2) + (((4 + (cb >> 1)) ^ swizzle(vkey & 7)) * 8) + (cb & 1) * 4;
 
-    f32x16 bias0;
+    // ---- state of the environment being computed ----
+    int nkb, pad;
+    bool uniform;
+    f32x16 bias0;  // -inf for the padding positions of key block 0, as the initial accumulator there
+    auto set_padding = [&](int cnt) {
+        nkb = (cnt + 31) >> 5;
+        pad = nkb * 32 - cnt;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) bias0[v] = (8 * (v >> 2) + 4 * half + (v & 3) < pad) ? -INFINITY : 0.0f;
+        for (int v = 0; v < 16; ++v) bias0[v] = (8 * (v >> 2) + 4 * half + (v & 3) < pad) ? -INFINITY : 0.0f;
+    };
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
-    const int64_t o_row = ((int64_t)env * NM + qsafe) * D + 8 * half;
 
-    issue(std::integral_constant<int, 0>{}, 0);
-    issue(std::integral_constant<int, 1>{}, 1);
-
-    u32x4 held[2];  // the previous head's output, stored after the next barrier
+    u32x4 held[2];  // the last computed head's output, stored after the next barrier
     auto compute = [&](auto head_tag) {
         constexpr int h = decltype(head_tag)::value;
         const uint16_t *buf = &s_buf[h & 1][0];
+        // with no live key every score is the same constant: zero queries give exactly that
         const bf16x8 qb0 = __builtin_bit_cast(bf16x8, uniform ? zero4 : qw[h][0]);
         const bf16x8 qb1 = __builtin_bit_cast(bf16x8, uniform ? zero4 : qw[h][1]);
         auto scores = [&](int kb) -> f32x16 {
@@ -219,44 +262,100 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_env_kernel(const uint16_t *_
             held[g] = u32x4{pack_bf16x2(o[8 * g + 0] * inv, o[8 * g + 1] * inv), pack_bf16x2(o[8 * g + 2] * inv, o[8 * g + 3] * inv),
                             pack_bf16x2(o[8 * g + 4] * inv, o[8 * g + 5] * inv), pack_bf16x2(o[8 * g + 6] * inv, o[8 * g + 7] * inv)};
     };
-    auto store = [&](int h) {
+    auto store = [&](int env, int h) {
         if (qrow < NM) {
-            *reinterpret_cast<u32x4 *>(out + o_row + h * kEnvDh) = held[0];
-            *reinterpret_cast<u32x4 *>(out + o_row + h * kEnvDh + 16) = held[1];
+            uint16_t *op = out + ((int64_t)env * NM + qrow) * D + h * kEnvDh + 8 * half;
+            *reinterpret_cast<u32x4 *>(op) = held[0];
+            *reinterpret_cast<u32x4 *>(op + 16) = held[1];
         }
     };
+    // Everything a wave has in flight (its share of a head's rows, queries of the next environment,
+    // the previous head's output) was issued a whole head earlier, so the wait is a plain vmcnt(0);
+    // the barrier then says both "everybody's rows of this head have landed" and "everybody is done
+    // with the previous head", whose buffer the head after this one may now overwrite.
+    auto next_head = [&]() {
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+        __syncthreads();
+    };
+    using H0 = std::integral_constant<int, 0>;
+    using H1 = std::integral_constant<int, 1>;
+    using H2 = std::integral_constant<int, 2>;
+    using H3 = std::integral_constant<int, 3>;
 
-    // Head h is computed out of buffer h%2 while head h+1 lands in the other one.  One barrier per
-    // head: it says both "everybody's rows of head h have landed" (each wave waits for its own loads
-    // first) and "everybody is done reading head h-1", after which head h+1 may overwrite that buffer.
-    // The only vector-memory traffic issued between a head's loads and the wait for them is nothing
-    // at all (the previous head's output is stored right after the barrier, before the next loads),
-    // so every wait is a plain vmcnt(0) for work issued a whole head earlier.
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the queries and heads 0 and 1 of this wave's rows
-    __syncthreads();
-    compute(std::integral_constant<int, 0>{});
-    __builtin_amdgcn_s_waitcnt(0x0f70);
-    __syncthreads();
-    store(0);
-    issue(std::integral_constant<int, 2>{}, 0);
-    compute(std::integral_constant<int, 1>{});
-    __builtin_amdgcn_s_waitcnt(0x0f70);
-    __syncthreads();
-    store(1);
-    issue(std::integral_constant<int, 3>{}, 1);
-    compute(std::integral_constant<int, 2>{});
-    __builtin_amdgcn_s_waitcnt(0x0f70);
-    __syncthreads();
-    store(2);
-    compute(std::integral_constant<int, 3>{});
-    store(3);
+    // ---- first environment of the run: nothing to hide the set-up behind ----
+    int env = first;
+    const uint16_t *env_base = qkv + (int64_t)env * NM * stride;
+    load_q(env_base, H0{});
+    load_q(env_base, H1{});
+    load_q(env_base, H2{});
+    load_q(env_base, H3{});
+    {
+        const KeyList k = make_list(load_alive(env));
+        uniform = k.uniform;
+        set_padding(k.cnt);
+        make_offsets(k, pad);
+        issue(env_base, H0{}, nkb * 4);
+    }
+
+    AliveRow row_next = {{0u, 0u, 0u}};
+    for (;;) {
+        const bool more = env + step < last;
+        const uint16_t *next_base = env_base + env_pitch;
+        // ---- head 0 (buffer 0); head 1 starts to land in buffer 1 ----
+        next_head();
+        if (env != first) store(env - step, 3);
+        issue(env_base, H1{}, nkb * 4);
+        if (more) row_next = load_alive(env + step);
+        compute(H0{});
+        // ---- head 1; head 2 into buffer 0 ----
+        next_head();
+        store(env, 0);
+        issue(env_base, H2{}, nkb * 4);
+        if (more) load_q(next_base, H0{});
+        compute(H1{});
+        // ---- head 2; head 3 into buffer 1 ----
+        next_head();
+        store(env, 1);
+        issue(env_base, H3{}, nkb * 4);
+        if (more) load_q(next_base, H1{});
+        compute(H2{});
+        // ---- head 3; the next environment's key list, and its head 0 into buffer 0 ----
+        next_head();
+        store(env, 2);
+        bool uniform_next = false;
+        int cnt_next = 0;
+        if (more) {
+            load_q(next_base, H2{});
+            const KeyList k = make_list(row_next);
+            uniform_next = k.uniform;
+            cnt_next = k.cnt;
+            const int nkb_next = (cnt_next + 31) >> 5;
+            make_offsets(k, nkb_next * 32 - cnt_next);
+            issue(next_base, H0{}, nkb_next * 4);
+        }
+        compute(H3{});
+        if (!more) break;
+        load_q(next_base, H3{});
+        uniform = uniform_next;
+        set_padding(cnt_next);
+        env_base = next_base;
+        env += step;
+    }
+    store(env, 3);
 }
 
 template <int NQB>
 static int launch_env(const void *qkv, int64_t stride, const uint8_t *alive, void *out, int B, int NM, hipStream_t stream)
 {
-    hipLaunchKernelGGL((sdpa_env_kernel<NQB>), dim3((unsigned)B), dim3(kWave * NQB), 0, stream, (const uint16_t *)qkv, stride, alive,
-                       (uint16_t *)out, B, NM, 1.4426950408889634f / sqrtf((float)kEnvDh));
+    // environments per work-group: long enough runs to hide each environment's set-up behind the one before,
+    // short enough that the hardware still has several times more work-groups than slots to balance with
+    // (BNB_ENV_GROUP overrides the choice: a tuning and testing knob)
+    int groups = B;
+    if (const char *e = getenv("BNB_ENV_GROUP")) groups = atoi(e) > 0 ? atoi(e) : groups;
+    if (groups > B) groups = B;
+    const int per = groups;
+    hipLaunchKernelGGL((sdpa_env_kernel<NQB>), dim3((unsigned)groups), dim3(kWave * NQB), 0, stream, (const uint16_t *)qkv, stride,
+                       alive, (uint16_t *)out, B, NM, per, 1.4426950408889634f / sqrtf((float)kEnvDh));
     return (int)hipGetLastError();
 }
 

@@ -225,7 +225,11 @@ def test_sdpa_mfma_live_counts_across_block_edges():
 
 
 @pytest.mark.parametrize("NM", [1, 7, 12, 23, 31, 32, 33, 64, 65, 84, 96, 97, 128, 129, 159, 160])
-def test_sdpa_environment_kernel_matches_oracle_and_the_per_head_kernel(NM):
+@pytest.mark.parametrize("groups", [24, 7, 3])
+def test_sdpa_environment_kernel_matches_oracle_and_the_per_head_kernel(NM, groups, monkeypatch):
+    # groups = work-groups the 24 environments are dealt to (each walks its environments with the next one's
+    # set-up overlapped with the current one's arithmetic): one each, 3-4 each (ragged), 8 each
+    monkeypatch.setenv("BNB_ENV_GROUP", str(groups))
     # one work-group per environment, K/V rows straight into LDS, V read through the transposing LDS load.
     # Per environment: mixed, all alive, all dead, only the first and only the last token alive, then
     # random live counts that cross every key-block edge
@@ -272,6 +276,8 @@ def test_sdpa_environment_kernel_matches_oracle_and_the_per_head_kernel(NM):
     view = wide.to(DEV)[..., : 3 * D]
     assert torch.equal(ops.sdpa_masked(view, alive.to(DEV), H, path="env").float().cpu(), got)
     assert max_rel(ops.sdpa_masked(view, None, H, path="env").float().cpu(), torch_ref.sdpa_masked(qkv.float(), None, H)) <= BF16_TOL
+    # a batch that does not fill the last run
+    assert torch.equal(_run_sdpa(qkv[: B - 1], alive[: B - 1], H, "env").float(), got[: B - 1])
 
 
 def test_sdpa_environment_kernel_limits():
