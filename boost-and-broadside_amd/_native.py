@@ -12,7 +12,7 @@ import os
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "_lib", "libbnb_amd.so")
 
-ABI_VERSION = 18
+ABI_VERSION = 19
 F32, BF16 = 0, 1
 PATH_AUTO, PATH_VALU, PATH_MFMA, PATH_ENV = 0, 1, 2, 3
 
@@ -65,6 +65,7 @@ SIGNATURES = {
     ),
     "bnb_add_rmsnorm_fwd": (_i, [_vp, _i64, _vp, _i, _vp, _f, _vp, _vp, _i, _i64, _i, _vp]),
     "bnb_norm_linear_fwd": (_i, [_vp, _i64, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i64, _i, _i, _vp]),
+    "bnb_linear_f32_fwd": (_i, [_vp, _i64, _vp, _i64, _vp, _f, _vp, _vp, _vp, _i64, _vp, _i64, _i64, _i, _i, _i, _vp]),
     "bnb_mask_count": (_i, [_vp, _vp, _i, _i, _vp]),
     "bnb_mask_fill": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "bnb_ffn_fused_fwd": (_i, [_vp, _i64, _vp, _i, _vp, _f, _vp, _vp, _i64, _i, _i, _vp]),

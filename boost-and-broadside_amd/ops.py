@@ -1751,6 +1751,83 @@ def ffn_fused(
     return out.reshape(x.shape)
 
 
+def pack_linear_f32(weight: torch.Tensor, up_weight: torch.Tensor | None = None) -> torch.Tensor:
+    """A float32 Linear weight (N, K), N % 32 == 0, K % 128 == 0, as the operand stream of ``linear_f32``:
+    ``[fb][s4][l][e] = W[32 fb + l%32][(l/32) K/2 + 4 s4 + e]`` (a lane's four next contraction steps are one
+    16-byte piece of a 1 KB contiguous wave read).  With ``up_weight`` (same shape) the two matrices are
+    interleaved in blocks of 32 rows, ``[gate block u, up block u]``, for the gated form."""
+    w = weight.detach().float()
+    N, K = w.shape
+    if N % 32 or K % 128 or (up_weight is not None and up_weight.shape != weight.shape):
+        raise ValueError("linear_f32 covers (N, K) weights with N % 32 == 0 and K % 128 == 0 (gate and up of one shape)")
+    if up_weight is not None:
+        u = up_weight.detach().float()
+        w = torch.stack([w.view(N // 32, 32, K), u.view(N // 32, 32, K)], dim=1).reshape(2 * N, K)
+        N = 2 * N
+    dev = w.device
+    lane = torch.arange(64, device=dev)
+    rows = (32 * torch.arange(N // 32, device=dev)[:, None, None, None] + (lane % 32)[None, None, :, None]).expand(-1, K // 8, -1, 4)
+    cols = ((lane // 32)[None, None, :, None] * (K // 2) + 4 * torch.arange(K // 8, device=dev)[None, :, None, None]
+            + torch.arange(4, device=dev)[None, None, None, :]).expand(N // 32, -1, -1, -1)
+    return w[rows, cols].contiguous()
+
+
+def linear_f32_supported(x: torch.Tensor, n_features: int) -> bool:
+    """Whether ``linear_f32`` covers this input: float32 rows on the GPU, K % 128 == 0, N % 32 == 0."""
+    return (x.is_cuda and x.dtype == torch.float32 and x.shape[-1] % 128 == 0 and n_features % 32 == 0
+            and x.stride(-1) == 1)
+
+
+def linear_f32(x: torch.Tensor, weight_packed: torch.Tensor, *, bias: torch.Tensor | None = None,
+               norm_weight: torch.Tensor | None = None, eps: float | None = None, gelu_times: torch.Tensor | None = None,
+               gate: bool = False, resid: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+    """A float32 Linear with its neighbours folded in, one kernel on the fp32 matrix cores.
+
+    ``out = A W^T + bias (+ resid)`` with ``A = x``, or ``rmsnorm(x) * norm_weight`` (K = 128), or
+    ``gelu(x) * gelu_times``; with ``gate`` the packed weight holds gate and up projections
+    (``pack_linear_f32(gate_w, up_w)``) and ``out = gelu(A Wg^T) * (A Wu^T)``.  ``x`` (..., K) float32 with
+    unit-stride channels and evenly spaced rows; ``resid`` / ``out`` (..., N_out) float32 contiguous."""
+    K = x.shape[-1]
+    _need_device(x, "x")
+    if x.dtype != torch.float32 or weight_packed.dtype != torch.float32:
+        raise TypeError("linear_f32 takes float32 rows and a float32 packed weight")
+    n_blocks = weight_packed.shape[0]
+    if weight_packed.dim() != 4 or weight_packed.shape[1:] != (K // 8, 64, 4) or not weight_packed.is_contiguous():
+        raise ValueError("weight_packed must come from pack_linear_f32 for this contraction width")
+    N = 32 * n_blocks
+    n_out = N // 2 if gate else N
+    if torch.is_grad_enabled() and x.requires_grad:
+        raise RuntimeError("linear_f32 is forward-only; call it under torch.no_grad()")
+    x2 = x.reshape(-1, K) if _uniform_rows(x, K) else x.reshape(-1, K).contiguous()
+    R = x2.shape[0]
+    y2 = None
+    if gelu_times is not None:
+        if gelu_times.shape != x.shape or gelu_times.dtype != torch.float32:
+            raise ValueError("gelu_times must be float32 with x's shape")
+        y2 = gelu_times.reshape(-1, K) if _uniform_rows(gelu_times, K) else gelu_times.reshape(-1, K).contiguous()
+    lead = x.shape[:-1]
+    if out is None:
+        out = torch.empty((*lead, n_out), dtype=torch.float32, device=x.device)
+    elif out.shape != (*lead, n_out) or out.dtype != torch.float32 or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous float32 {(*lead, n_out)} tensor")
+    r2 = None
+    if resid is not None:
+        if resid.shape != (*lead, n_out) or resid.dtype != torch.float32:
+            raise ValueError(f"resid must be float32 {(*lead, n_out)}")
+        r2 = resid.reshape(-1, n_out) if _uniform_rows(resid, n_out) else resid.reshape(-1, n_out).contiguous()
+    if R == 0:
+        return out
+    with torch.cuda.device(x.device):
+        rc = _native.load().bnb_linear_f32_fwd(
+            x2.data_ptr(), x2.stride(0) if R > 1 else K, None if y2 is None else y2.data_ptr(),
+            0 if y2 is None else (y2.stride(0) if R > 1 else K), None if norm_weight is None else norm_weight.detach().contiguous().data_ptr(),
+            float(_F32_EPS if eps is None else eps), weight_packed.data_ptr(), None if bias is None else bias.detach().contiguous().data_ptr(),
+            None if r2 is None else r2.data_ptr(), 0 if r2 is None else (r2.stride(0) if R > 1 else n_out), out.data_ptr(), n_out, R, K, N,
+            1 if gate else 0, _stream())
+    _native.check(rc, "bnb_linear_f32_fwd")
+    return out
+
+
 def pack_linear_weights(weight: torch.Tensor) -> torch.Tensor:
     """A Linear weight (N, 128), N a multiple of 64, as the bfloat16 operand stream of
     ``norm_linear``: ``[fb][ks][l][e]`` with the index meaning given in ``include/bnb_amd.h``
@@ -1775,9 +1852,14 @@ def pack_linear_weights(weight: torch.Tensor) -> torch.Tensor:
 class CompactRows:
     """The set entries of a (B, n) bool mask as a device-side list: ``index`` (capacity B*n,
     int32 flat positions b*n + j, ascending, the first ``offsets[B]`` valid) and ``offsets``
-    (B+1, int32 exclusive prefix of the per-row counts).  Built without any copy to the host."""
+    (B+1, int32 exclusive prefix of the per-row counts).  Built without any copy to the host.
 
-    def __init__(self, mask: torch.Tensor) -> None:
+    ``total`` / ``max_count`` (optional Python ints): the number of set entries and the largest count of
+    one row, for a caller that knows them already (e.g. counted when the rollout was stored).  The
+    update path sizes gathered tensors with them; without the hint ``total_host()`` copies them from
+    the device once, which makes the host wait for everything queued before."""
+
+    def __init__(self, mask: torch.Tensor, *, total: int | None = None, max_count: int | None = None) -> None:
         if mask.dim() != 2 or mask.dtype not in (torch.bool, torch.uint8):
             raise ValueError("mask must be a bool (B, n) tensor")
         _need_device(mask, "mask")
@@ -1787,6 +1869,9 @@ class CompactRows:
             raise ValueError("mask too large for 32-bit row positions")
         self.shape = (B, n)
         self.mask = mask
+        if (total is None) != (max_count is None):
+            raise ValueError("give both total and max_count, or neither")
+        self._host = None if total is None else (int(total), int(max_count))
         counts = torch.empty(B, dtype=torch.int32, device=mask.device)
         self.offsets = torch.zeros(B + 1, dtype=torch.int32, device=mask.device)
         self.index = torch.empty(max(B * n, 1), dtype=torch.int32, device=mask.device)

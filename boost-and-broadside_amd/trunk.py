@@ -482,7 +482,8 @@ class TransformerBlock(_WeightCaches, nn.Module):
         flight are normalised and projected: the list of live slots is built on the device, its
         length read back once (torch needs it to size the gathered rows), ``norm_bullet`` and
         ``kv_bullet`` run on the gathered rows and the read and its backward take the compacted
-        ``[K | V]`` rows with per-environment ranges.  Otherwise every slot is projected and the
+        ``[K | V]`` rows with per-environment ranges (a ``CompactRows`` built with ``total=`` /
+        ``max_count=`` by a caller that knows the counts needs no read-back).  Otherwise every slot is projected and the
         read is the masked kernel pair, or torch's SDPA for the shapes the kernels do not cover."""
         rows = bullet_mask if isinstance(bullet_mask, ops.CompactRows) else None
         mask = rows.mask if rows is not None else bullet_mask

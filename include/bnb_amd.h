@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 18
+#define BNB_ABI_VERSION 19
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -615,6 +615,33 @@ int bnb_norm_linear_fwd(const float *x, int64_t x_row_stride, const int32_t *row
                         const int32_t *n_rows, const float *norm_weight, float eps,
                         const void *weight_packed, const float *bias, void *out,
                         int64_t R, int D, int N, void *stream);
+
+/*
+ * A float32 Linear layer with its neighbours folded in, on the fp32 matrix cores (true fp32 products):
+ *     out[r] = A[r] W^T + bias (+ resid[r]),   A[r] = x[r]                          (norm_weight, x2 NULL)
+ *                                                   | rmsnorm(x[r]) * norm_weight     (norm_weight given; K == 128)
+ *                                                   | gelu(x[r]) * x2[r]              (x2 given)
+ *     gate != 0: W holds gate_proj and up_proj interleaved in blocks of 32 rows, out[r][u] = gelu(g[r][u]) * up[r][u]
+ * Replaces, for a policy that runs without autocast (evaluation/agents.py:214-219), every Linear of the trunk
+ * together with the element-wise passes around it: `self.qkv(self.norm1(x))` (models/yemong/attention.py:94-96,
+ * 132-135), `x + self.out_proj(..)` (:97,168-169), `F.gelu(gate_proj(n)) * up_proj(n)` on `norm2(x)` (:36-37,98),
+ * `x + down_proj(..)` (:37,98); `linear1` / `linear2` on `norm1(x)` (models/yemong/griffin.py:269-272,279),
+ * `linear_a` / `linear_x` (:166-167,208-209), `x + linear_out(b1_out * gelu(linear2(..)))` (:281-284) and the same
+ * gated MLP (:285-286).
+ *
+ *   x, x2          (R, K) fp32 rows, x_row_stride / x2_row_stride floats apart (multiples of 4, 16-byte aligned)
+ *   norm_weight    (128) fp32 or NULL; eps as in nn.RMSNorm
+ *   weight_packed  W (N, K) as [fb][s4][l][e] = W[32 fb + l%32][(l/32) K/2 + 4 s4 + e], fb < N/32, s4 < K/8,
+ *                  l < 64, e < 4 (with gate: blocks 2u, 2u+1 = rows 32u.. of gate_proj, of up_proj)
+ *   bias           (N) fp32 or NULL (not with gate)
+ *   resid          optional (R, N_out) fp32 rows added to the result; may equal out
+ *   out            (R, N_out) fp32 rows, N_out = N, or N/2 with gate
+ * Requirements: K % 128 == 0, N % 32 == 0 (N % 64 with gate); anything else returns BNB_ERR_UNSUPPORTED.
+ */
+int bnb_linear_f32_fwd(const float *x, int64_t x_row_stride, const float *x2, int64_t x2_row_stride,
+                       const float *norm_weight, float eps, const float *weight_packed, const float *bias,
+                       const float *resid, int64_t resid_row_stride, float *out, int64_t out_row_stride, int64_t R,
+                       int K, int N, int gate, void *stream);
 
 /*
  * Compact list of the set entries of a byte mask (B, n), e.g. the bullets in flight of

@@ -2137,3 +2137,83 @@ def test_rollout_and_inference_kernels_index_rows_whose_element_offsets_pass_2_3
         assert max_rel(out[sl], s + F.linear(hidden, dw.bfloat16()).float()) <= BF16_TOL
         r = F.linear(F.rms_norm(xs[sl], (128,), nw, eps).bfloat16(), wq.bfloat16())
         assert max_rel(q[sl].float(), r.float()) <= BF16_TOL
+
+
+# ------------------------------------------------------------------ float32 Linear layers with their neighbours folded in
+
+
+def _gelu64(t):
+    return 0.5 * t * (1.0 + torch.erf(t / 2 ** 0.5))
+
+
+@pytest.mark.parametrize("R", [1, 31, 32, 33, 1000, 12288])
+@pytest.mark.parametrize("mode", ["plain", "bias_resid", "norm", "norm_gate", "mulgelu_resid", "gate", "k512_resid"])
+def test_linear_f32_matches_the_float64_statement(R, mode):
+    # every float32 Linear of the trunk as evaluation runs it (no autocast), with the passes around it folded in
+    g = torch.Generator().manual_seed(R * 13 + len(mode))
+    K = 512 if mode == "k512_resid" else 128
+    N = {"plain": 384, "bias_resid": 256, "norm": 384, "norm_gate": 512, "mulgelu_resid": 128, "gate": 512, "k512_resid": 128}[mode]
+    x = torch.randn(R, K, generator=g) * (0.3 + 2.0 * torch.rand(R, 1, generator=g))
+    w = torch.randn(N, K, generator=g) / K ** 0.5
+    xd, wd = x.double(), w.double()
+    kw, ref = {}, None
+    if mode == "plain":
+        ref = xd @ wd.t()
+        packed = ops.pack_linear_f32(w.to(DEV))
+    elif mode == "bias_resid":
+        b, res = torch.randn(N, generator=g), torch.randn(R, N, generator=g)
+        ref = xd @ wd.t() + b.double() + res.double()
+        packed = ops.pack_linear_f32(w.to(DEV))
+        kw = dict(bias=b.to(DEV), resid=res.to(DEV))
+    elif mode in ("norm", "norm_gate"):
+        nw = 1.0 + 0.2 * torch.randn(K, generator=g)
+        eps = float(torch.finfo(torch.float32).eps)
+        n = xd * torch.rsqrt(xd.pow(2).mean(-1, keepdim=True) + eps) * nw.double()
+        kw = dict(norm_weight=nw.to(DEV))
+        if mode == "norm":
+            ref = n @ wd.t()
+            packed = ops.pack_linear_f32(w.to(DEV))
+        else:
+            up = torch.randn(N, K, generator=g) / K ** 0.5
+            ref = _gelu64(n @ wd.t()) * (n @ up.double().t())
+            packed = ops.pack_linear_f32(w.to(DEV), up.to(DEV))
+            kw["gate"] = True
+    elif mode == "gate":
+        up = torch.randn(N, K, generator=g) / K ** 0.5
+        ref = _gelu64(xd @ wd.t()) * (xd @ up.double().t())
+        packed = ops.pack_linear_f32(w.to(DEV), up.to(DEV))
+        kw = dict(gate=True)
+    elif mode == "mulgelu_resid":
+        y, res = torch.randn(R, K, generator=g), torch.randn(R, N, generator=g)
+        ref = (_gelu64(xd) * y.double()) @ wd.t() + res.double()
+        packed = ops.pack_linear_f32(w.to(DEV))
+        kw = dict(gelu_times=y.to(DEV), resid=res.to(DEV))
+    else:
+        res = torch.randn(R, N, generator=g)
+        ref = xd @ wd.t() + res.double()
+        packed = ops.pack_linear_f32(w.to(DEV))
+        kw = dict(resid=res.to(DEV))
+    got = ops.linear_f32(x.to(DEV), packed, **kw)
+    assert got.shape == ref.shape and got.dtype == torch.float32
+    assert max_rel(got.cpu().double(), ref) <= F32_TOL
+    # repeated calls give identical bits; a leading shape is kept
+    again = ops.linear_f32(x.to(DEV).reshape(R, 1, K), packed, **{k: (v.reshape(R, 1, -1) if k in ("resid", "gelu_times") else v) for k, v in kw.items()})
+    assert torch.equal(again.reshape(got.shape), got)
+
+
+def test_linear_f32_reads_column_blocks_in_place_and_writes_into_the_residual():
+    g = torch.Generator().manual_seed(5)
+    R, K = 777, 128
+    wide = torch.randn(R, 3 * K, generator=g).to(DEV)
+    w = (torch.randn(K, K, generator=g) / K ** 0.5).to(DEV)
+    packed = ops.pack_linear_f32(w)
+    x = wide[:, K:2 * K]  # a column block: no copy is made
+    res = torch.randn(R, K, generator=g).to(DEV)
+    want = (x.double() @ w.double().t() + res.double()).cpu()
+    got = ops.linear_f32(x, packed, resid=res, out=res)  # in place on the residual stream
+    assert got.data_ptr() == res.data_ptr() and max_rel(got.cpu().double(), want) <= F32_TOL
+    with pytest.raises(RuntimeError, match="outside what the kernels cover"):
+        ops.linear_f32(torch.zeros(4, 256, device=DEV), ops.pack_linear_f32(torch.zeros(32, 256, device=DEV)),
+                       norm_weight=torch.ones(256, device=DEV))  # the norm prologue is for width 128
+    with pytest.raises(ValueError):
+        ops.pack_linear_f32(torch.zeros(48, 128))
