@@ -27,18 +27,21 @@ namespace bnb {
 constexpr int kLfSlab = 64;  // steps per slab: 128 channels (64 per half wave)
 
 template <bool NORM, bool MULGELU, bool GATE>
-__global__ __launch_bounds__(256, 2) void linear_f32_kernel(
+__global__ __launch_bounds__(64, 2) void linear_f32_kernel(
     const float *__restrict__ x, int64_t x_stride, const float *__restrict__ x2, int64_t x2_stride,
     const float *__restrict__ norm_w, float eps, const float *__restrict__ w_packed, const float *__restrict__ bias,
     const float *resid, int64_t resid_stride, float *out, int64_t out_stride, int64_t R, int K, int n_blocks,
     int blocks_per_wave)
 {
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // one wave per work-group: the waves that share a row tile (consecutive work-groups, each a run of feature blocks) are
+    // independent, so a finished wave's slot is refilled at once
+    const int lane = threadIdx.x;
     const int m = lane & 31, half = lane >> 5;
-    const int64_t row0 = (int64_t)blockIdx.x * 32;
     const int unit = GATE ? 2 : 1;  // weight blocks per output block
-    const int first = (blockIdx.y * 4 + wave) * blocks_per_wave;  // first OUTPUT block of this wave
+    const int n_out_all = n_blocks / unit;
+    const int waves_per_tile = (n_out_all + blocks_per_wave - 1) / blocks_per_wave;
+    const int64_t row0 = (int64_t)(blockIdx.x / waves_per_tile) * 32;
+    const int first = (blockIdx.x % waves_per_tile) * blocks_per_wave;  // first OUTPUT block of this wave
     const int n_out_blocks = n_blocks / unit;
     if (first >= n_out_blocks) return;
     const int last = first + blocks_per_wave < n_out_blocks ? first + blocks_per_wave : n_out_blocks;
@@ -84,55 +87,79 @@ __global__ __launch_bounds__(256, 2) void linear_f32_kernel(
     };
     if (slabs == 1) load_slab(0);  // a 128-wide contraction keeps its operand across all feature blocks
 
+    // Weight groups (one 16-byte load per lane = four contraction steps) are requested AHEAD groups before
+    // they are used, across slab and block boundaries, so that the matrix cores never wait for L2 at
+    // the start of a block: the ring wq/wq2 is carried through all loops.
+    constexpr int GROUPS = kLfSlab / 4;  // 16 groups per slab
+    constexpr int AHEAD = GATE ? 4 : 8;  // divides GROUPS, so a group's ring slot is the same in every slab
+    static_assert(GROUPS % AHEAD == 0, "the ring slot of a group must not depend on the slab");
+    f32x4 wq[AHEAD], wq2[AHEAD];
+    const int64_t block_floats = (int64_t)s4_per_block * 256;  // one packed 32-feature block
+    const float *w_lane = w_packed + lane * 4;
+    {
+        const float *ws = w_lane + (int64_t)first * unit * block_floats;
+#pragma unroll
+        for (int i = 0; i < AHEAD; ++i) {
+            wq[i] = *reinterpret_cast<const f32x4 *>(ws + (int64_t)i * 256);
+            if (GATE) wq2[i] = *reinterpret_cast<const f32x4 *>(ws + block_floats + (int64_t)i * 256);
+        }
+    }
+
     for (int ob = first; ob < last; ++ob) {
         f32x16 acc = {0.0f}, acc2 = {0.0f};
-        const float *wp = w_packed + ((int64_t)ob * unit * s4_per_block * 64 + lane) * 4;
-        const float *wp2 = wp + (int64_t)s4_per_block * 64 * 4;  // the up block of a gate pair
         for (int t = 0; t < slabs; ++t) {
             if (slabs > 1) load_slab(t);
-            // ---- 64 steps of the slab, four per 16-byte weight load, loads kept four ahead ----
-            const float *ws = wp + (int64_t)t * (kLfSlab / 4) * 64 * 4;
-            const float *ws2 = wp2 + (int64_t)t * (kLfSlab / 4) * 64 * 4;
-            constexpr int AHEAD = 4;
-            f32x4 wq[AHEAD], wq2[AHEAD];
+            // this slab's groups, and where the groups after it live (the next slab of this block, else the
+            // first slab of the next block; after the very last one the loads repeat this slab and are dropped)
+            const float *ws = w_lane + (int64_t)ob * unit * block_floats + (int64_t)t * GROUPS * 256;
+            const float *wn = ws;
+            if (t + 1 < slabs) wn = ws + (int64_t)GROUPS * 256;
+            else if (ob + 1 < last) wn = w_lane + (int64_t)(ob + 1) * unit * block_floats;
 #pragma unroll
-            for (int i = 0; i < AHEAD; ++i) {
-                wq[i] = *reinterpret_cast<const f32x4 *>(ws + (int64_t)i * 256);
-                if (GATE) wq2[i] = *reinterpret_cast<const f32x4 *>(ws2 + (int64_t)i * 256);
-            }
-#pragma unroll
-            for (int s4 = 0; s4 < kLfSlab / 4; ++s4) {
-                const f32x4 b = wq[s4 % AHEAD];
+            for (int s4 = 0; s4 < GROUPS; ++s4) {
+                const int slot = s4 % AHEAD;
+                const f32x4 b = wq[slot];
                 f32x4 b2 = {0.0f, 0.0f, 0.0f, 0.0f};
-                if (GATE) b2 = wq2[s4 % AHEAD];
-                if (s4 + AHEAD < kLfSlab / 4) {
-                    wq[s4 % AHEAD] = *reinterpret_cast<const f32x4 *>(ws + (int64_t)(s4 + AHEAD) * 256);
-                    if (GATE) wq2[s4 % AHEAD] = *reinterpret_cast<const f32x4 *>(ws2 + (int64_t)(s4 + AHEAD) * 256);
-                }
+                if (GATE) b2 = wq2[slot];
+                const float *src = s4 + AHEAD < GROUPS ? ws + (int64_t)(s4 + AHEAD) * 256 : wn + (int64_t)(s4 + AHEAD - GROUPS) * 256;
+                wq[slot] = *reinterpret_cast<const f32x4 *>(src);
+                if (GATE) wq2[slot] = *reinterpret_cast<const f32x4 *>(src + block_floats);
                 acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * s4 + 0], b.x, acc, 0, 0, 0);
+                if (GATE) acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * s4 + 0], b2.x, acc2, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * s4 + 1], b.y, acc, 0, 0, 0);
+                if (GATE) acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * s4 + 1], b2.y, acc2, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * s4 + 2], b.z, acc, 0, 0, 0);
+                if (GATE) acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * s4 + 2], b2.z, acc2, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * s4 + 3], b.w, acc, 0, 0, 0);
-                if (GATE) {
-                    acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * s4 + 0], b2.x, acc2, 0, 0, 0);
-                    acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * s4 + 1], b2.y, acc2, 0, 0, 0);
-                    acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * s4 + 2], b2.z, acc2, 0, 0, 0);
-                    acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * s4 + 3], b2.w, acc2, 0, 0, 0);
-                }
+                if (GATE) acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * s4 + 3], b2.w, acc2, 0, 0, 0);
+                // keep the request for group s4 + AHEAD in front of group s4's products: left to itself the
+                // scheduler sinks the loads until just before their use and the matrix cores wait for L2
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         // ---- epilogue: the lane holds feature 32 ob + m of rows 8 i + 4 half + j ----
         const int feat = ob * 32 + m;
         const float bv = bias != nullptr ? bias[feat] : 0.0f;
+        float res[16];
+        if (resid != nullptr) {
+            // all sixteen requests first: one round trip instead of sixteen
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int64_t r = row0 + 8 * (v >> 2) + 4 * half + (v & 3);
+                res[v] = resid[(r < R ? r : R - 1) * resid_stride + feat];
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            float o = acc[v] + bv;
+            if (GATE) o = gelu_erf(o) * acc2[v];
+            if (resid != nullptr) o += res[v];
+            acc[v] = o;
+        }
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int64_t r = row0 + 8 * (v >> 2) + 4 * half + (v & 3);
-            if (r < R) {
-                float o = acc[v] + bv;
-                if (GATE) o = gelu_erf(o) * acc2[v];
-                if (resid != nullptr) o += resid[r * resid_stride + feat];
-                out[r * out_stride + feat] = o;
-            }
+            if (r < R) out[r * out_stride + feat] = acc[v];
         }
     }
 }
@@ -145,12 +172,12 @@ static int launch_linear_f32(const float *x, int64_t x_stride, const float *x2, 
     const int n_blocks = N / 32;
     const int n_out_blocks = GATE ? n_blocks / 2 : n_blocks;
     const int64_t tiles = (R + 31) / 32;
-    // split the features over enough waves to give every SIMD a couple of tasks when the row count is small
+    // split the features over enough waves to give every SIMD several tasks (1024 SIMDs) when the row count is small
     int per = n_out_blocks;
-    while (per > 1 && tiles * ((n_out_blocks + per - 1) / per) < 2048) per = (per + 1) / 2;
+    while (per > 1 && tiles * ((n_out_blocks + per - 1) / per) < 8192) per = (per + 1) / 2;
     const int waves = (n_out_blocks + per - 1) / per;
-    if (tiles > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((linear_f32_kernel<NORM, MULGELU, GATE>), dim3((unsigned)tiles, (unsigned)((waves + 3) / 4)), dim3(256), 0, stream,
+    if (tiles * waves > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((linear_f32_kernel<NORM, MULGELU, GATE>), dim3((unsigned)(tiles * waves)), dim3(64), 0, stream,
                        x, x_stride, x2, x2_stride, norm_w, eps, w_packed, bias, resid, resid_stride, out, out_stride, R, K, n_blocks,
                        per);
     return (int)hipGetLastError();

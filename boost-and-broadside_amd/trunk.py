@@ -72,6 +72,20 @@ def _fused_ok(x: torch.Tensor, act: torch.dtype) -> bool:
     return ok
 
 
+def _f32_fused_ok(x: torch.Tensor, act: torch.dtype, *layers: nn.Linear) -> bool:
+    """Whether the float32 matrix-core Linear kernel applies: no gradients, float32 projections over float32 rows
+    of width 128 on the GPU, float32 weights."""
+    return (
+        not torch.is_grad_enabled() and act == torch.float32 and x.is_cuda and x.dtype == torch.float32
+        and x.shape[-1] == ops.FFN_WIDTH and all(l.weight.dtype == torch.float32 for l in layers)
+    )
+
+
+def _packed_f32(layer: nn.Module, slot: str, *weights: torch.Tensor) -> torch.Tensor:
+    """The float32 operand stream of ``ops.linear_f32`` for one weight, or for a (gate, up) pair (cached)."""
+    return _cached_cast(layer, slot, weights, torch.float32, lambda: ops.pack_linear_f32(*weights))
+
+
 _TRAIN_KERNELS = True  # grad-mode norms, gates, conv, attention and weight gradients on the library's own kernels when False
 
 
@@ -345,6 +359,17 @@ class GatedMLP(_WeightCaches, nn.Module):
         proj = (delta, wp) if gate is None else (gate, delta, wp)
         return ops.ffn_fused(x, None, norm.weight, self.packed_weights(), eps=norm.eps, proj=proj)
 
+    def tail_f32(self, x1: torch.Tensor, norm: nn.RMSNorm) -> torch.Tensor | None:
+        """``x1 + self(norm(x1))`` in float32 as two kernels (norm + gate/up + gelu gate; down + residual), or None
+        when that does not apply (other widths, biases)."""
+        if (self.gate_proj.bias is not None or self.up_proj.bias is not None or self.down_proj.bias is not None
+                or self.gate_proj.out_features % 128 or norm.weight is None
+                or not _f32_fused_ok(x1, torch.float32, self.gate_proj, self.up_proj, self.down_proj)):
+            return None
+        gu = _packed_f32(self, "_bnb_f32_gate_up", self.gate_proj.weight, self.up_proj.weight)
+        hid = ops.linear_f32(x1, gu, norm_weight=norm.weight, eps=norm.eps, gate=True)
+        return ops.linear_f32(hid, _packed_f32(self.down_proj, "_bnb_f32_pack", self.down_proj.weight), resid=x1)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         hidden = self.gate_proj.out_features
         if not x.is_cuda or hidden % 8 or x.dtype not in (torch.float32, torch.bfloat16) or torch.is_grad_enabled():
@@ -407,6 +432,19 @@ class TransformerBlock(_WeightCaches, nn.Module):
                 attn = _project(self.out_proj, merged)
             else:
                 attn = self._attn(None, alive_mask, bullets, bullet_mask, qkv=qkv)
+        elif (_f32_fused_ok(x, act, self.qkv, self.out_proj) and self.qkv.bias is None and self.out_proj.bias is None
+              and self.norm1.weight is not None):
+            # float32 (evaluation without autocast): every Linear on the fp32 matrix cores with its norm, gate and
+            # residual folded in: norm1 + qkv, attention, out_proj + residual, norm2 + gate/up + gelu gate, down + residual
+            qkv = ops.linear_f32(x, _packed_f32(self.qkv, "_bnb_f32_pack", self.qkv.weight), norm_weight=self.norm1.weight,
+                                 eps=self.norm1.eps)
+            merged = self._attn(None, alive_mask, bullets, bullet_mask, qkv=qkv, project=False)
+            x1 = ops.linear_f32(merged, _packed_f32(self.out_proj, "_bnb_f32_pack", self.out_proj.weight), resid=x)
+            tail = self.ffn.tail_f32(x1, self.norm2)
+            if tail is not None:
+                return tail
+            _, n2 = ops.add_rmsnorm(x1, self.norm2.weight, eps=self.norm2.eps, out_dtype=act)
+            return x1 + self.ffn(n2)
         else:
             _, n1 = ops.add_rmsnorm(x, self.norm1.weight, eps=self.norm1.eps, out_dtype=act)
             attn = self._attn(n1, alive_mask, bullets, bullet_mask)
@@ -457,7 +495,12 @@ class TransformerBlock(_WeightCaches, nn.Module):
                 return _project(self.out_proj, merged) if project else merged
             if rows is not None:
                 bullet_mask = rows.mask
-            kv = _project(self.kv_bullet, self._norm_bullets(bullets, qkv.dtype))
+            if (_f32_fused_ok(bullets, qkv.dtype, self.kv_bullet) and self.kv_bullet.bias is None
+                    and self.norm_bullet.weight is not None):
+                kv = ops.linear_f32(bullets, _packed_f32(self.kv_bullet, "_bnb_f32_pack", self.kv_bullet.weight),
+                                    norm_weight=self.norm_bullet.weight, eps=self.norm_bullet.eps)
+            else:
+                kv = _project(self.kv_bullet, self._norm_bullets(bullets, qkv.dtype))
             if ops.cross_supported(qkv, kv, self.n_heads):
                 merged = ops.sdpa_cross(qkv, kv, bullet_mask, self.n_heads, accum=merged)
             else:
@@ -569,9 +612,16 @@ class RGLRU(_WeightCaches, nn.Module):
             b = torch.cat([self.linear_a.bias, self.linear_x.bias], dim=0)
             return _grad_linear(x, w, b)
         act = _projection_dtype()
+        wa, wx, ba, bx = self.linear_a.weight, self.linear_x.weight, self.linear_a.bias, self.linear_x.bias
+        if _f32_fused_ok(x, act, self.linear_a, self.linear_x) and x.dim() == 2 and ba is not None and bx is not None:
+            # float32: both gate projections and their biases as one kernel on the fp32 matrix cores
+            pk = _cached_cast(self, "_bnb_f32_gates", (wa, wx), torch.float32,
+                              lambda: ops.pack_linear_f32(torch.cat([wa.detach(), wx.detach()], dim=0)))
+            bias = _cached_cast(self, "_bnb_f32_gate_bias", (ba, bx), torch.float32,
+                                lambda: torch.cat([ba.detach(), bx.detach()], dim=0).float())
+            return ops.linear_f32(x, pk, bias=bias)
         if x_act is None or x_act.dtype != act:
             x_act = x.to(act)
-        wa, wx, ba, bx = self.linear_a.weight, self.linear_x.weight, self.linear_a.bias, self.linear_x.bias
         w = _cached_cast(self, "_bnb_gw", (wa, wx), act, lambda: torch.cat([wa, wx], dim=0).detach().to(act))
         b = _cached_cast(self, "_bnb_gb", (ba, bx), act, lambda: torch.cat([ba, bx], dim=0).detach().to(act))
         return F.linear(x_act, w, b)
@@ -680,6 +730,16 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
         act = _projection_dtype()
         if gate_in is None:
             gate_in = _project(self.linear2, normed)
+        if (_f32_fused_ok(x, act, self.linear_out) and self.linear_out.bias is None and gate_in.dtype == torch.float32
+                and y.dtype == torch.float32 and y.shape == gate_in.shape):
+            # float32: gelu(linear2) * y, linear_out and the residual in one kernel, then the gated MLP's two
+            x1 = ops.linear_f32(gate_in, _packed_f32(self.linear_out, "_bnb_f32_pack", self.linear_out.weight), gelu_times=y,
+                                resid=x)
+            tail = self.gated_mlp.tail_f32(x1, self.norm2)
+            if tail is not None:
+                return tail
+            _, n2 = ops.add_rmsnorm(x1, self.norm2.weight, eps=self.norm2.eps, out_dtype=act)
+            return x1 + self.gated_mlp(n2)
         if _fused_ok(x, act) and gate_in.dtype == act:
             if y.dtype == torch.bfloat16 and y.shape == gate_in.shape:
                 # gelu(linear2) * y, linear_out, both residual adds, norm2 and the gated MLP in one kernel
@@ -764,6 +824,21 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
             b1, gate_in = both[..., :D], both[..., D:2 * D]
             if fold:
                 y = both[..., 2 * D:]
+        elif (_f32_fused_ok(x, act, self.linear1, self.linear2) and self.linear1.bias is None and self.linear2.bias is None
+              and self.norm1.weight is not None):
+            # float32: norm1 and [linear1 | linear2] as one kernel; with field tokens field_sub(linear1(.)) is one more
+            # projection of the same normed rows (field_sub . linear1 folded in float32), written for every token and
+            # then overwritten on the ship rows by the recurrence
+            w12 = (self.linear1.weight, self.linear2.weight)
+            pk = _cached_cast(self, "_bnb_f32_l12", w12, torch.float32,
+                              lambda: ops.pack_linear_f32(torch.cat([w12[0].detach(), w12[1].detach()], dim=0)))
+            both = ops.linear_f32(x, pk, norm_weight=self.norm1.weight, eps=self.norm1.eps)  # (B, NM, 2D)
+            b1, gate_in = both[..., :D], both[..., D:]
+            if NM > n_rec and field_sub is not None and field_sub.bias is None and field_sub.weight.dtype == torch.float32:
+                ws = (field_sub.weight, self.linear1.weight)
+                pf = _cached_cast(self, "_bnb_f32_fsub", ws, torch.float32,
+                                  lambda: ops.pack_linear_f32(ws[0].detach().float() @ ws[1].detach().float()))
+                y = ops.linear_f32(x, pf, norm_weight=self.norm1.weight, eps=self.norm1.eps)  # (B, NM, D)
         else:
             x, normed = self._norm_in(x)
             b1 = _project(self.linear1, normed)
@@ -793,7 +868,7 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
                             reset=reset, rows_per_env=n_rec, also_bf16=want_lp)
         self.rg_lru.step(res[0], state_in[:, :D], h_out=state_out[:, :D], reset=reset, rows_per_env=n_rec,
                          x_act=res[2] if want_lp else None, y_out=y[:, :n_rec] if NM > n_rec else y.view(R, D))
-        if NM > n_rec:
+        if NM > n_rec and not fields_done:
             # gathered into one (B*M, D) matrix first: on the strided view the library would run a
             # batch of B tiny GEMMs
             y[:, n_rec:] = _project(field_sub, b1[:, n_rec:].reshape(-1, D)).view(B, NM - n_rec, D)
