@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(PKG_DIR, "_lib", "libbnb_amd.so")
 
 ABI_VERSION = 19
 F32, BF16 = 0, 1
-PATH_AUTO, PATH_VALU, PATH_MFMA, PATH_ENV = 0, 1, 2, 3
+PATH_AUTO, PATH_VALU, PATH_MFMA, PATH_ENV, PATH_HEAD = 0, 1, 2, 3, 4
 
 _vp, _i, _i64, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
 

@@ -344,6 +344,193 @@ __global__ __launch_bounds__(kWave * NQB, 4) void sdpa_env_kernel(const uint16_t
     store(env, 3);
 }
 
+// ------------------------------------------------------------------------------------
+// One work-group per (environment, head): the same data path (rows straight into LDS, key list per wave from
+// the alive row, V through the transposing read) with the occupancy of the small work-group: 20 KB of LDS and
+// 64 registers, so six work-groups of five waves share a CU and one's loads hide behind the others' arithmetic.
+// One barrier per work-group; nothing is staged by the lanes.
+// ------------------------------------------------------------------------------------
+template <int NQB>
+__global__ __launch_bounds__(kWave * NQB, 8) void sdpa_head_kernel(const uint16_t *__restrict__ qkv, int64_t stride,
+                                                                  const uint8_t *__restrict__ alive, uint16_t *__restrict__ out,
+                                                                  int B, int NM, int H, float scale_log2e)
+{
+    constexpr int KCAP = NQB * 32;
+    __shared__ __align__(1024) uint16_t s_buf[KCAP * kEnvKeyBytes / 2];
+
+    // work-groups are dealt round-robin to the 8 XCDs; hand each XCD a contiguous run of (environment, head)
+    // pairs so the heads of an environment (adjacent 64-byte segments of the same rows) share one L2
+    const int chunk_wg = gridDim.x >> 3;
+    const int logical = (blockIdx.x & 7) * chunk_wg + (blockIdx.x >> 3);
+    if (logical >= B * H) return;
+    const int env = logical / H;
+    const int head = logical - env * H;
+    const int D = H * kEnvDh;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m = lane & 31;
+    const int half = lane >> 5;
+    const uint16_t *env_base = qkv + (int64_t)env * NM * stride + head * kEnvDh;
+
+    // this lane's query
+    const int qrow = wave * 32 + m;
+    const int qsafe = qrow < NM ? qrow : NM - 1;
+    const uint16_t *qp = env_base + (uint32_t)qsafe * (uint32_t)stride + half * 8;
+    u32x4 qw0 = *reinterpret_cast<const u32x4 *>(qp);
+    u32x4 qw1 = *reinterpret_cast<const u32x4 *>(qp + 16);
+
+    // the alive row as three 64-bit masks (lane l: tokens l, l + 64, l + 128)
+    uint64_t mk[3];
+#pragma unroll
+    for (int w = 0; w < 3; ++w) {
+        const int tok = lane + 64 * w;
+        uint32_t a = 0u;
+        if (w * 64 < KCAP) {
+            const uint32_t in = tok < NM ? 1u : 0u;
+            a = alive == nullptr ? in : (in ? (uint32_t)alive[(int64_t)env * NM + tok] : 0u);
+        }
+        mk[w] = __ballot(a != 0);
+    }
+    int c0 = (int)__popcll(mk[0]), c1 = (int)__popcll(mk[1]);
+    int cnt = c0 + c1 + (int)__popcll(mk[2]);
+    // no live key at all: every key takes part with the same weight (all scores equal)
+    const bool uniform = cnt == 0;
+    if (uniform) {
+#pragma unroll
+        for (int w = 0; w < 3; ++w) mk[w] = __ballot(lane + 64 * w < NM);
+        c0 = (int)__popcll(mk[0]), c1 = (int)__popcll(mk[1]);
+        cnt = NM;
+    }
+    const int nkb = (cnt + 31) >> 5;
+    const int pad = nkb * 32 - cnt;  // positions [0, pad) of key block 0 hold a copy of the first live key
+
+    // the token of this wave's t-th staged position (t = lane % 32: instruction t/8, position t%8 in it)
+    int token;
+    {
+        const int t = lane & 31;
+        int n = (wave + (t >> 3) * NQB) * 8 + (t & 7) - pad;
+        n = n > 0 ? n : 0;
+        n = n < cnt ? n : cnt - 1;
+        uint64_t w = mk[0];
+        int base = 0;
+        if (n >= c0) {
+            n -= c0, w = mk[1], base = 64;
+            if (n >= c1) n -= c1, w = mk[2], base = 128;
+        }
+        uint32_t x = (uint32_t)w;
+        int c = __popc(x);
+        if (n >= c) n -= c, x = (uint32_t)(w >> 32), base += 32;
+#pragma unroll
+        for (int width = 16; width >= 1; width >>= 1) {
+            c = __popc(x & ((1u << width) - 1u));
+            if (n >= c) n -= c, x >>= width, base += width;
+        }
+        token = base;
+    }
+    // instruction j = wave + jj * NQB fills LDS kilobyte j: lane l -> position 8j + l/8, slot l%8 = chunk ^ f(position)
+    const int chunk = (lane & 7) ^ swizzle((lane >> 3) & 7);
+    const uint32_t chan_bytes = (uint32_t)(((1 + (chunk >> 2)) * D + (chunk & 3) * 8) * 2);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)&s_buf[0];
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+        const int j = wave + jj * NQB;
+        const int tok = __builtin_amdgcn_ds_bpermute((jj * 8 + (lane >> 3)) * 4, token);
+        if (j < nkb * 4) dma_row16(env_base, (uint32_t)tok * (uint32_t)stride * 2u + chan_bytes, lds0 + (uint32_t)j * 1024u);
+    }
+
+    const int ksw = swizzle(m & 7);
+    const int k_off0 = m * (kEnvKeyBytes / 2) + ((half ^ ksw) * 8);
+    const int k_off1 = m * (kEnvKeyBytes / 2) + (((2 + half) ^ ksw) * 8);
+    const int grp = lane >> 4, r = lane & 15;
+    const int rb = 4 * (grp & 1) + (r & 3);
+    const int cb = 4 * (rb >> 2) + 2 * (rb & 1) + ((rb >> 1) & 1);
+    const int vkey = 4 * (grp >> 1) + (r >> 2);
+    const int v_off = vkey * (kEnvKeyBytes / 2) + (((4 + (cb >> 1)) ^ swizzle(vkey & 7)) * 8) + (cb & 1) * 4;
+
+    if (uniform) qw0 = qw1 = u32x4{0u, 0u, 0u, 0u};
+    const bf16x8 qb0 = __builtin_bit_cast(bf16x8, qw0);
+    const bf16x8 qb1 = __builtin_bit_cast(bf16x8, qw1);
+    f32x16 bias0;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) bias0[v] = (8 * (v >> 2) + 4 * half + (v & 3) < pad) ? -INFINITY : 0.0f;
+
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's rows and its queries
+    __syncthreads();                      // everybody's rows
+
+    auto scores = [&](int kb) -> f32x16 {
+        const uint16_t *kp = s_buf + kb * 32 * (kEnvKeyBytes / 2);
+        const bf16x8 ka0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + k_off0));
+        const bf16x8 ka1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + k_off1));
+        f32x16 z = {0.0f};
+        if (kb == 0) z = bias0;
+        z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0, qb0, z, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka1, qb1, z, 0, 0, 0);
+    };
+    float mx = -INFINITY;
+    for (int kb = 0; kb < nkb; ++kb) {
+        const f32x16 z = scores(kb);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float mc = mx * scale_log2e;
+    float sum = 0.0f;
+    f32x16 o = {0.0f};
+    for (int kb = 0; kb < nkb; ++kb) {
+        const f32x16 z = scores(kb);
+        float p[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            p[v] = __builtin_amdgcn_exp2f(fmaf(z[v], scale_log2e, -mc));
+            sum += p[v];
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            bf16x8 pb;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * t + e];
+            const bf16x8 va = lds_tr_pair(s_buf + (kb * 32 + 16 * t) * (kEnvKeyBytes / 2) + v_off);
+            o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb, o, 0, 0, 0);
+        }
+    }
+    sum += __shfl_xor(sum, 32);
+    const float inv = __builtin_amdgcn_rcpf(sum);
+    if (qrow < NM) {
+        uint16_t *op = out + ((int64_t)env * NM + qrow) * D + head * kEnvDh + 8 * half;
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+            *reinterpret_cast<u32x4 *>(op + 16 * g) =
+                u32x4{pack_bf16x2(o[8 * g + 0] * inv, o[8 * g + 1] * inv), pack_bf16x2(o[8 * g + 2] * inv, o[8 * g + 3] * inv),
+                      pack_bf16x2(o[8 * g + 4] * inv, o[8 * g + 5] * inv), pack_bf16x2(o[8 * g + 6] * inv, o[8 * g + 7] * inv)};
+    }
+}
+
+template <int NQB>
+static int launch_head(const void *qkv, int64_t stride, const uint8_t *alive, void *out, int B, int NM, int H, hipStream_t stream)
+{
+    const int64_t pairs = (int64_t)B * H;
+    const int64_t blocks = (pairs + 7) / 8 * 8;
+    if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((sdpa_head_kernel<NQB>), dim3((unsigned)blocks), dim3(kWave * NQB), 0, stream, (const uint16_t *)qkv, stride,
+                       alive, (uint16_t *)out, B, NM, H, 1.4426950408889634f / sqrtf((float)kEnvDh));
+    return (int)hipGetLastError();
+}
+
+// bf16, heads of 32 channels, 1 <= NM <= 160, rows of one environment within 2^31 bytes.
+int dispatch_head(const void *qkv, int64_t stride, const uint8_t *alive, void *out, int B, int NM, int H, hipStream_t stream)
+{
+    switch ((NM + 31) / 32) {
+        case 1: return launch_head<1>(qkv, stride, alive, out, B, NM, H, stream);
+        case 2: return launch_head<2>(qkv, stride, alive, out, B, NM, H, stream);
+        case 3: return launch_head<3>(qkv, stride, alive, out, B, NM, H, stream);
+        case 4: return launch_head<4>(qkv, stride, alive, out, B, NM, H, stream);
+        case 5: return launch_head<5>(qkv, stride, alive, out, B, NM, H, stream);
+        default: return BNB_ERR_UNSUPPORTED;
+    }
+}
+
 template <int NQB>
 static int launch_env(const void *qkv, int64_t stride, const uint8_t *alive, void *out, int B, int NM, hipStream_t stream)
 {

@@ -1136,6 +1136,9 @@ static int dispatch_cross_stream(const void *q, int64_t q_stride, const void *k,
 // defined in sdpa_env.hip: bf16, 4 heads of 32 channels, NM <= 160, one work-group per environment
 int dispatch_env(const void *qkv, int64_t stride, const uint8_t *alive, void *out, int B, int NM, hipStream_t stream);
 
+// defined in sdpa_env.hip: bf16, heads of 32 channels, NM <= 160, one work-group per (environment, head), rows straight into LDS
+int dispatch_head(const void *qkv, int64_t stride, const uint8_t *alive, void *out, int B, int NM, int H, hipStream_t stream);
+
 // defined in sdpa_cross_f32.hip
 int launch_cross_f32(const void *q, int64_t q_stride, const void *k, const void *v, int64_t kv_stride, const uint8_t *key_mask,
                      const void *accum, void *out, int B, int NQ, int NK, int H, hipStream_t stream);
@@ -1149,7 +1152,7 @@ extern "C" int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride,
     using namespace bnb;
     if (B < 0 || NM < 0 || H < 1 || dh < 1) return BNB_ERR_BAD_SHAPE;
     if (dtype != BNB_F32 && dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
-    if (path < BNB_SDPA_PATH_AUTO || path > BNB_SDPA_PATH_ENV) return BNB_ERR_UNSUPPORTED;
+    if (path < BNB_SDPA_PATH_AUTO || path > BNB_SDPA_PATH_HEAD) return BNB_ERR_UNSUPPORTED;
     if (B == 0 || NM == 0) return 0;
     if (!qkv || !out) return BNB_ERR_NULL_POINTER;
     if (qkv_row_stride < (int64_t)3 * H * dh) return BNB_ERR_BAD_SHAPE;
@@ -1166,6 +1169,8 @@ extern "C" int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride,
     if (path == BNB_SDPA_PATH_ENV && !env_ok) return BNB_ERR_UNSUPPORTED;
     if (path == BNB_SDPA_PATH_ENV)
         return dispatch_env(qkv, qkv_row_stride, alive, out, B, NM, s);
+    if (path == BNB_SDPA_PATH_HEAD && !mfma_ok) return BNB_ERR_UNSUPPORTED;
+    if (path == BNB_SDPA_PATH_HEAD) return dispatch_head(qkv, qkv_row_stride, alive, out, B, NM, H, s);
     // measured on MI355X the matrix-core kernel wins at every token count it covers, 4v4 included
     // (12 tokens: 24.7 us vs 45.5 us for 8192 environments), so AUTO takes it whenever it applies
     const bool use_mfma = path == BNB_SDPA_PATH_MFMA || (path == BNB_SDPA_PATH_AUTO && mfma_ok);

@@ -30,7 +30,8 @@ def _outside_autocast(backward):
     return wrapped
 
 
-_PATH_CODE = {"auto": _native.PATH_AUTO, "valu": _native.PATH_VALU, "mfma": _native.PATH_MFMA, "env": _native.PATH_ENV}
+_PATH_CODE = {"auto": _native.PATH_AUTO, "valu": _native.PATH_VALU, "mfma": _native.PATH_MFMA, "env": _native.PATH_ENV,
+              "head": _native.PATH_HEAD}
 
 
 def _need_device(t: torch.Tensor, name: str) -> None:

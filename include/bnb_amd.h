@@ -90,6 +90,7 @@ int bnb_sdpa_masked_fwd(const void *qkv, int64_t qkv_row_stride, const uint8_t *
 #define BNB_SDPA_PATH_VALU 1
 #define BNB_SDPA_PATH_MFMA 2
 #define BNB_SDPA_PATH_ENV 3
+#define BNB_SDPA_PATH_HEAD 4 /* one work-group per (environment, head) with the rows loaded straight into LDS (bf16, dh == 32, NM <= 160) */
 int bnb_sdpa_masked_fwd_path(const void *qkv, int64_t qkv_row_stride, const uint8_t *alive, void *out,
                              int B, int NM, int H, int dh, int dtype, int path, void *stream);
 

@@ -280,6 +280,43 @@ def test_sdpa_environment_kernel_matches_oracle_and_the_per_head_kernel(NM, grou
     assert torch.equal(_run_sdpa(qkv[: B - 1], alive[: B - 1], H, "env").float(), got[: B - 1])
 
 
+@pytest.mark.parametrize("NM", [1, 12, 23, 32, 33, 84, 97, 129, 160])
+@pytest.mark.parametrize("H", [4, 2, 8, 3])
+def test_sdpa_head_kernel_with_rows_loaded_straight_into_lds_matches_oracle_and_the_staged_kernel(NM, H):
+    # one work-group per (environment, head) like the staged kernel, but K/V rows go global -> LDS directly, the key
+    # list comes from the alive row per wave, V is read through the transposing LDS load: same arithmetic, same bits
+    B, D = 21, 32 * H
+    qkv = _qkv(900 + NM + H, B, NM, D, torch.bfloat16)
+    g = torch.Generator().manual_seed(900 + NM)
+    alive = _alive(901 + NM, B, NM, 0.6)
+    alive[0] = True
+    alive[1] = False
+    alive[2] = False
+    alive[2, 0] = True
+    alive[3] = False
+    alive[3, NM - 1] = True
+    for b in range(4, B):
+        alive[b] = False
+        alive[b, torch.randperm(NM, generator=g)[: int(torch.randint(1, NM + 1, (1,), generator=g))]] = True
+    got = _run_sdpa(qkv, alive, H, "head").float()
+    truth = torch_ref.sdpa_masked(qkv.float(), alive, H)
+    assert torch.isfinite(got).all()
+    for b in range(B):
+        assert max_rel(got[b], truth[b]) <= BF16_TOL, (b, int(alive[b].sum()))
+    assert torch.equal(got, _run_sdpa(qkv, alive, H, "mfma").float())
+    assert torch.equal(got[3], qkv[3, NM - 1, 2 * D:].float().expand(NM, D))
+    pert = qkv.clone()
+    dead = ~alive
+    dead[~alive.any(dim=1)] = False
+    pert[..., D:][dead] = pert[..., D:][dead] * -3.0 + 17.0
+    assert torch.equal(_run_sdpa(pert, alive, H, "head").float(), got)
+    wide = torch.zeros(B, NM, 3 * D + 64, dtype=torch.bfloat16)
+    wide[..., : 3 * D] = qkv
+    view = wide.to(DEV)[..., : 3 * D]
+    assert torch.equal(ops.sdpa_masked(view, alive.to(DEV), H, path="head").float().cpu(), got)
+    assert max_rel(ops.sdpa_masked(view, None, H, path="head").float().cpu(), torch_ref.sdpa_masked(qkv.float(), None, H)) <= BF16_TOL
+
+
 def test_sdpa_environment_kernel_limits():
     with pytest.raises(RuntimeError, match="outside what the kernels cover"):
         ops.sdpa_masked(torch.zeros(1, 12, 192, device=DEV, dtype=torch.bfloat16), None, 2, path="env")  # two heads
