@@ -257,9 +257,52 @@ def sdpa_cross(
 
 
 def sdpa_cross_train_supported(qkv: torch.Tensor, kv: torch.Tensor, n_heads: int) -> bool:
-    """Whether ``sdpa_cross_train`` covers these shapes: what ``sdpa_cross`` covers with at most 160 keys."""
-    return (cross_supported(qkv, kv, n_heads) and qkv.dtype == torch.bfloat16 and kv.shape[1] <= 160 and kv.dim() == 3
-            and qkv.dim() == 3)
+    """Whether ``sdpa_cross_train`` covers these shapes: what ``sdpa_cross`` covers in bfloat16 (up to 2048 keys,
+    160 queries)."""
+    return cross_supported(qkv, kv, n_heads) and qkv.dtype == torch.bfloat16 and kv.dim() == 3 and qkv.dim() == 3
+
+
+def sdpa_cross_stream_bwd(qkv, kv, rows: "CompactRows", n_heads, out, dout, *, indexed: bool):
+    """Gradients ``(dq (B, NQ, D), dkv)`` of the bullet read for any number of listed keys per environment.
+
+    ``indexed=False``: ``kv`` (capacity, 2D) holds ``[K | V]`` of the entries of ``rows`` in list order and
+    ``dkv`` has that layout.  ``indexed=True``: ``kv`` is the (B, NK, 2D) buffer the mask of ``rows`` was
+    taken over, read in place through the list; ``dkv`` (B, NK, 2D) is zero where the mask is."""
+    B, NQ, D3 = qkv.shape
+    D = D3 // 3
+    for name, t in (("qkv", qkv), ("kv", kv), ("out", out), ("dout", dout)):
+        _need_device(t, name)
+        if t.dtype != torch.bfloat16:
+            raise TypeError(f"{name} must be bfloat16")
+    if rows.shape[0] != B or out.shape != (B, NQ, D) or dout.shape != (B, NQ, D) or NQ > 160 or D // n_heads != 32:
+        raise ValueError("rows lists the keys of the B environments; out and dout are (B, NQ <= 160, D), heads of 32")
+    if indexed:
+        if kv.shape != (B, rows.shape[1], 2 * D):
+            raise ValueError(f"kv must be {(B, rows.shape[1], 2 * D)}")
+        if B and (kv.stride(-1) != 1 or kv.stride(1) != 2 * D or (B > 1 and kv.stride(0) != kv.shape[1] * 2 * D)):
+            kv = kv.contiguous()
+        dkv = torch.zeros_like(kv, memory_format=torch.contiguous_format)
+        capacity = B * rows.shape[1]
+    else:
+        if kv.dim() != 2 or kv.shape[1] != 2 * D or not kv.is_contiguous():
+            raise ValueError(f"kv must be a contiguous (capacity, {2 * D}) tensor")
+        dkv = torch.empty_like(kv)
+        capacity = kv.shape[0]
+    if B and NQ and (qkv.stride(-1) != 1 or (B > 1 and qkv.stride(0) != NQ * qkv.stride(1))):
+        qkv = qkv.contiguous()
+    out, dout = out.contiguous(), dout.contiguous()
+    dq = torch.empty((B, NQ, D), dtype=torch.bfloat16, device=qkv.device)
+    if capacity == 0:
+        return dq.zero_(), dkv
+    if B and NQ:
+        stats = torch.empty((B, n_heads, NQ, 2), dtype=torch.float32, device=qkv.device)
+        with torch.cuda.device(qkv.device):
+            rc = _native.load().bnb_sdpa_cross_stream_bwd(
+                qkv.data_ptr(), qkv.stride(1), NQ, kv.data_ptr(), 2 * D, rows.offsets.data_ptr(),
+                rows.index.data_ptr() if indexed else None, capacity, out.data_ptr(), dout.data_ptr(), dq.data_ptr(),
+                dkv.data_ptr(), stats.data_ptr(), B, n_heads, D // n_heads, _native.BF16, _stream())
+        _native.check(rc, "bnb_sdpa_cross_stream_bwd")
+    return dq, dkv
 
 
 def sdpa_cross_bwd(qkv, kv, key_mask, n_heads, out, dout) -> tuple[torch.Tensor, torch.Tensor]:
@@ -312,7 +355,14 @@ class _SdpaCrossTrain(torch.autograd.Function):
     @_outside_autocast
     def backward(ctx, dout):
         qkv, kv, out = ctx.saved_tensors
-        dq, dkv = sdpa_cross_bwd(qkv, kv, ctx.key_mask, ctx.n_heads, out, dout.to(torch.bfloat16))
+        if kv.shape[1] <= 160:
+            dq, dkv = sdpa_cross_bwd(qkv, kv, ctx.key_mask, ctx.n_heads, out, dout.to(torch.bfloat16))
+        else:
+            # long key axes: through the device-side list of the live slots (no copy to the host)
+            mask = ctx.key_mask
+            if mask is None:
+                mask = torch.ones(kv.shape[:2], dtype=torch.bool, device=kv.device)
+            dq, dkv = sdpa_cross_stream_bwd(qkv, kv, CompactRows(mask), ctx.n_heads, out, dout.to(torch.bfloat16), indexed=True)
         dqkv = torch.zeros_like(qkv)
         dqkv[..., : dq.shape[-1]] = dq
         return dqkv, dkv, None, None
@@ -335,8 +385,10 @@ def sdpa_cross_rows_bwd(qkv, kv_rows, rows: "CompactRows", n_heads, out, dout, t
             raise TypeError(f"{name} must be bfloat16")
     if kv_rows.dim() != 2 or kv_rows.shape[1] != 2 * D or not kv_rows.is_contiguous() or kv_rows.shape[0] < total:
         raise ValueError(f"kv_rows must be a contiguous (>= {total}, {2 * D}) tensor")
-    if rows.shape[0] != B or rows.shape[1] > 160 or out.shape != (B, NQ, D) or dout.shape != (B, NQ, D):
-        raise ValueError("rows must list at most 160 entries for each of the B environments; out and dout are (B, NQ, D)")
+    if rows.shape[0] != B or out.shape != (B, NQ, D) or dout.shape != (B, NQ, D):
+        raise ValueError("rows must list the entries of the B environments; out and dout are (B, NQ, D)")
+    if rows.max_count_host() > 160:
+        return sdpa_cross_stream_bwd(qkv, kv_rows[:total], rows, n_heads, out, dout, indexed=False)
     if B and NQ and (qkv.stride(-1) != 1 or (B > 1 and qkv.stride(0) != NQ * qkv.stride(1))):
         qkv = qkv.contiguous()
     out, dout = out.contiguous(), dout.contiguous()
@@ -377,7 +429,8 @@ class _SdpaCrossRowsTrain(torch.autograd.Function):
 
 def sdpa_cross_rows_train(qkv: torch.Tensor, kv_rows: torch.Tensor, rows: "CompactRows", n_heads: int) -> torch.Tensor:
     """Differentiable ``sdpa_cross_rows``: ``kv_rows`` holds exactly ``rows.total_host()`` rows, ``[K | V]`` of the
-    listed entries in list order (bfloat16).  Needs head size 32, at most 160 queries and 160 entries per row of the mask."""
+    listed entries in list order (bfloat16).  Needs head size 32 and at most 160 queries; any number of entries per
+    row of the mask (up to 160 on the single-tile backward kernel, more on the streaming one)."""
     total = rows.total_host()
     if kv_rows.shape[0] != total:
         raise ValueError(f"kv_rows must hold the {total} listed rows")

@@ -521,7 +521,7 @@ class TransformerBlock(_WeightCaches, nn.Module):
     def _bullet_branch_autograd(self, qkv, bullets, bullet_mask):
         """The bullet read in grad mode, (B, N, D) to be added to the self-attention output.
 
-        With a mask, bf16 projections and at most 160 slots per environment only the bullets in
+        With a mask, bf16 projections and at most 2048 slots per environment only the bullets in
         flight are normalised and projected: the list of live slots is built on the device, its
         length read back once (torch needs it to size the gathered rows), ``norm_bullet`` and
         ``kv_bullet`` run on the gathered rows and the read and its backward take the compacted
@@ -532,8 +532,8 @@ class TransformerBlock(_WeightCaches, nn.Module):
         mask = rows.mask if rows is not None else bullet_mask
         B, NB, D = bullets.shape
         compact_ok = (
-            _TRAIN_KERNELS and mask is not None and qkv.is_cuda and qkv.dtype == torch.bfloat16 and NB <= 160
-            and self.head_dim == 32 and qkv.shape[1] <= 160 and self.kv_bullet.bias is None
+            _TRAIN_KERNELS and mask is not None and qkv.is_cuda and qkv.dtype == torch.bfloat16 and NB <= 2048
+            and self.head_dim == 32 and qkv.shape[1] <= 160 and self.kv_bullet.bias is None and B * NB < 2 ** 31
         )
         if compact_ok:
             if rows is None:

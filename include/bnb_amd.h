@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 19
+#define BNB_ABI_VERSION 20
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -319,6 +319,25 @@ int bnb_sdpa_cross_bwd(const void *q, int64_t q_row_stride, int NQ, const void *
 int bnb_sdpa_cross_ranges_bwd(const void *q, int64_t q_row_stride, int NQ, const void *kv_rows, int64_t kv_row_stride,
                               const int32_t *ranges, int64_t capacity, int max_keys, const void *out, const void *dout,
                               void *dq, void *dkv_rows, int64_t B, int H, int dh, int dtype, void *stream);
+
+/*
+ * The bullet read's backward for ANY number of live keys per environment (bf16, dh = 32, NQ <= 160):
+ * what autograd computes through models/yemong/attention.py:149-166 when the bullet axis is longer
+ * than 160 slots (10 slots per ship, config/defaults.py:29; caller train/rl/ppo.py:1417-1425).
+ * Environment b's keys are list entries ranges[b] .. ranges[b+1]-1 (clamped to `capacity` entries in
+ * all).  row_index == NULL: entry e is row e of kv (rows compacted beforehand, as for
+ * bnb_sdpa_cross_ranges_bwd).  row_index != NULL: entry e is row row_index[e] of kv, i.e. the (B, NK, 2D)
+ * buffer is read in place through the list of its live slots (bnb_mask_count / bnb_mask_fill); dkv then
+ * has that layout too and the rows of slots that are not listed are NOT written (zero them beforehand).
+ * out is the read's own result (nothing accumulated), dq (B, NQ, D) contiguous, dkv has kv's row
+ * stride 2D.  stats: workspace of 2 * B * H * NQ floats (per query and head: log2-sum-exp and
+ * rowsum(dout * out), written by the first kernel, read by the second).  An environment with an
+ * empty range gets a zero dq.
+ */
+int bnb_sdpa_cross_stream_bwd(const void *q, int64_t q_row_stride, int NQ, const void *kv, int64_t kv_row_stride,
+                              const int32_t *ranges, const int32_t *row_index, int64_t capacity, const void *out,
+                              const void *dout, void *dq, void *dkv, float *stats, int64_t B, int H, int dh, int dtype,
+                              void *stream);
 
 /*
  * RMSNorm backward:  y = x * rsqrt(mean(x^2) + eps) * weight

@@ -1985,7 +1985,82 @@ def test_sdpa_cross_train_is_differentiable():
     (torch_ref.bullet_read(xq, xkv, mask.cpu(), H) * up.bfloat16().cpu().double()).sum().backward()
     assert max_rel(qkv.grad.float().cpu().double(), xq.grad) <= BF16_TOL
     assert max_rel(kv.grad.float().cpu().double(), xkv.grad) <= BF16_TOL
-    assert not ops.sdpa_cross_train_supported(qkv, torch.zeros(B, 200, 2 * D, device=DEV, dtype=torch.bfloat16), H)
+    assert ops.sdpa_cross_train_supported(qkv, torch.zeros(B, 200, 2 * D, device=DEV, dtype=torch.bfloat16), H)
+    assert not ops.sdpa_cross_train_supported(qkv, torch.zeros(B, 2049, 2 * D, device=DEV, dtype=torch.bfloat16), H)
+    assert not ops.sdpa_cross_train_supported(qkv.float(), torch.zeros(B, 80, 2 * D, device=DEV), H)
+
+
+@pytest.mark.parametrize("B,NQ,NK,p_live", [
+    (3, 12, 200, 0.5), (4, 23, 480, 0.3), (2, 160, 1520, 0.25), (3, 84, 800, 1.0), (5, 152, 2048, 0.05), (3, 33, 161, 1.0),
+    (4, 12, 80, 0.25), (6, 64, 1520, 0.02), (2, 97, 2048, 1.0),
+])
+def test_sdpa_cross_streaming_backward_matches_autograd_of_the_oracle(B, NQ, NK, p_live):
+    """The bullet read's backward over long slot axes (10 slots per ship: 1520 at 64v88), in both forms: the
+    (B, NK, 2D) buffer read in place through the list of its live slots, and rows compacted beforehand."""
+    H, D = 4, 128
+    g = torch.Generator().manual_seed(B * 17 + NQ + NK)
+    qkv = (1.2 * torch.randn(B, NQ, 3 * D, generator=g)).bfloat16()
+    kv = (1.2 * torch.randn(B, NK, 2 * D, generator=g)).bfloat16()
+    mask = torch.rand(B, NK, generator=g) < p_live
+    if B > 2:
+        mask[1] = False  # an environment without an active bullet among active ones
+    mask[0, 0] = True
+    mask[0, NK - 1] = True
+    up = torch.randn(B, NQ, D, generator=g).bfloat16()
+    xq = qkv.double().requires_grad_()
+    xkv = kv.double().requires_grad_()
+    ref = torch_ref.bullet_read(xq, xkv, mask, H)
+    (ref * up.double()).sum().backward()
+    dmask = mask.to(DEV)
+    dqkv, dkv_in, dup = qkv.to(DEV), kv.to(DEV), up.to(DEV)
+    out = ops.sdpa_cross(dqkv, dkv_in, dmask, H)
+    rows = ops.CompactRows(dmask)
+    dq, dkv = ops.sdpa_cross_stream_bwd(dqkv, dkv_in, rows, H, out, dup, indexed=True)
+    torch.cuda.synchronize()
+    for name, got, want in (("dQ", dq, xq.grad[..., :D]), ("dK", dkv[..., :D], xkv.grad[..., :D]), ("dV", dkv[..., D:], xkv.grad[..., D:])):
+        assert max_rel(got.float().cpu().double(), want) <= BF16_TOL, name
+    off = ~mask.any(dim=1)
+    assert not dq.cpu()[off].any() and not dkv.cpu()[off].any()  # gated off: exactly nothing
+    assert not dkv.cpu()[~mask].any()  # dead slots receive exact zeros
+    # rows compacted beforehand: the same keys in the same order, so the same numbers
+    total = rows.total_host()
+    kv_rows = dkv_in.reshape(B * NK, 2 * D)[dmask.reshape(-1)].contiguous()
+    dq_r, dkv_r = ops.sdpa_cross_stream_bwd(dqkv, kv_rows, rows, H, out, dup, indexed=False)
+    assert torch.equal(dq_r, dq)
+    assert torch.equal(dkv_r, dkv.reshape(B * NK, 2 * D)[dmask.reshape(-1)])
+    if rows.max_count_host() > 160:  # what the rows form of the update path dispatches to above one tile of keys
+        dq_d, dkv_d = ops.sdpa_cross_rows_bwd(dqkv, kv_rows, rows, H, out, dup, total)
+        assert torch.equal(dq_d, dq) and torch.equal(dkv_d, dkv_r)
+    elif NK <= 160:  # one tile: the single-tile kernel answers the same question
+        dq_s, dkv_s = ops.sdpa_cross_bwd(dqkv, dkv_in, dmask, H, out, dup)
+        assert max_rel(dq_s.float().cpu(), dq.float().cpu()) <= BF16_TOL
+        assert max_rel(dkv_s.float().cpu(), dkv.float().cpu()) <= BF16_TOL
+    again = ops.sdpa_cross_stream_bwd(dqkv, dkv_in, rows, H, out, dup, indexed=True)
+    assert torch.equal(dq, again[0]) and torch.equal(dkv, again[1])
+
+
+def test_sdpa_cross_train_over_a_long_slot_axis_is_differentiable():
+    B, NQ, NK, H, D = 5, 84, 800, 4, 128
+    g = torch.Generator().manual_seed(3)
+    qkv = torch.randn(B, NQ, 3 * D, generator=g).bfloat16().to(DEV).requires_grad_()
+    kv = torch.randn(B, NK, 2 * D, generator=g).bfloat16().to(DEV).requires_grad_()
+    mask = (torch.rand(B, NK, generator=g) < 0.3).to(DEV)
+    up = torch.randn(B, NQ, D, generator=g).to(DEV)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = ops.sdpa_cross_train(qkv, kv, mask, H)
+        (out.float() * up).sum().backward()
+    xq = qkv.detach().cpu().double().requires_grad_()
+    xkv = kv.detach().cpu().double().requires_grad_()
+    (torch_ref.bullet_read(xq, xkv, mask.cpu(), H) * up.bfloat16().cpu().double()).sum().backward()
+    assert max_rel(qkv.grad.float().cpu().double(), xq.grad) <= BF16_TOL
+    assert max_rel(kv.grad.float().cpu().double(), xkv.grad) <= BF16_TOL
+    # rows form with more than one tile of keys per environment
+    rows = ops.CompactRows(mask)
+    kv_rows = kv.detach().reshape(B * NK, 2 * D)[mask.reshape(-1)].clone().requires_grad_()
+    q2 = qkv.detach().clone().requires_grad_()
+    (ops.sdpa_cross_rows_train(q2, kv_rows, rows, H).float() * up).sum().backward()
+    assert max_rel(q2.grad.float().cpu().double(), xq.grad) <= BF16_TOL
+    assert max_rel(kv_rows.grad.float().cpu().double(), xkv.grad.reshape(B * NK, 2 * D)[mask.cpu().reshape(-1)]) <= BF16_TOL
 
 
 @pytest.mark.parametrize("B,NQ,NK,p_live", [(4, 12, 80, 0.25), (3, 23, 160, 0.1), (5, 12, 40, 1.0), (6, 84, 33, 0.5), (300, 12, 80, 0.25)])

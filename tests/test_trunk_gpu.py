@@ -841,6 +841,52 @@ def test_update_path_with_the_bullet_read_agrees_with_the_library_ops(p_live):
         assert not fast["bullets"].reshape(-1, D)[dead_rows].any()  # bullets that are not in flight receive nothing
 
 
+def test_update_path_reads_more_than_one_tile_of_bullets_on_the_kernels():
+    """32 ships = 320 bullet slots with most of them in flight: more live keys per environment than one tile
+    of the attention backward holds.  The read and its backward stay on the kernels (no library dispatch is
+    recorded) and every gradient agrees with torch's own differentiable ops."""
+    from boost_and_broadside_amd import trunk
+
+    cfg = _cfg(128, 4, spatial=2, temporal=1, bullets=1)
+    torch.manual_seed(21)
+    block = bnb.YemongBlock(cfg).to(DEV)
+    T, B, N, M, D = 3, 6, 32, 4, 128
+    NB = N * 10
+    gen = torch.Generator().manual_seed(22)
+    x = torch.randn(T, B, N + M, D, generator=gen).to(DEV).requires_grad_()
+    alive = (torch.rand(T, B, N + M, generator=gen) < 0.85).to(DEV)
+    alive[..., 0] = True
+    bullets = torch.randn(T * B, NB, D, generator=gen).to(DEV).requires_grad_()
+    bmask = (torch.rand(T * B, NB, generator=gen) < 0.7).to(DEV)
+    bmask[2] = False
+    bmask[4, 40:] = False  # one environment with few bullets among crowded ones
+    assert int(bmask.sum(dim=1).max()) > 160
+    h0 = torch.zeros(1, B * N, D, device=DEV)
+    cb0 = torch.zeros(1, B * N, 3, D, device=DEV)
+    done = torch.zeros(T, B, dtype=torch.bool, device=DEV)
+
+    def grads():
+        block.zero_grad(set_to_none=True)
+        x.grad = bullets.grad = None
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = block.sequence(x, alive, h0, cb0, done, N, bullets, bmask)[0]
+        out.float().square().mean().backward()
+        named = {n: p.grad for n, p in block.named_parameters() if p.grad is not None}
+        named["x"], named["bullets"] = x.grad, bullets.grad
+        return {k: v.detach().clone() for k, v in named.items()}
+
+    before = sum(trunk.library_dispatches.values())
+    with trunk.forbid_library_dispatch():
+        fast = grads()
+    assert sum(trunk.library_dispatches.values()) == before
+    with trunk.library_update_path():
+        slow = grads()
+    for name, g in slow.items():
+        assert torch.isfinite(fast[name]).all(), name
+        assert max_rel(fast[name].float().cpu(), g.float().cpu()) <= BF16_TOL, name
+    assert not fast["bullets"].reshape(-1, D)[~bmask.reshape(-1)].any()
+
+
 def test_trunk_sequence_with_bullets_shares_one_list_and_matches_the_block_loop():
     D, H, B, N, M, T = 128, 4, 10, 8, 4, 6
     torch.manual_seed(41)
