@@ -26,6 +26,23 @@ namespace bnb {
 
 constexpr int kLfSlab = 64;  // steps per slab: 128 channels (64 per half wave)
 
+// erf-GELU without branches: erf from the five-term Abramowitz-Stegun form 7.1.26 (|error| <= 1.5e-7,
+// |error of gelu| <= 5e-7 over |v| <= 12, far inside the float32 bar), 14 vector instructions against
+// about 30 for the library's erff.  gelu(v) = v/2 + |v|/2 * erf(|v| / sqrt 2).
+__device__ __forceinline__ float gelu_erf_lf(float v)
+{
+    const float x = fabsf(v) * 0.70710678118654752f;
+    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, x, 1.0f));
+    float poly = fmaf(1.061405429f, t, -1.453152027f);
+    poly = fmaf(poly, t, 1.421413741f);
+    poly = fmaf(poly, t, -0.284496736f);
+    poly = fmaf(poly, t, 0.254829592f);
+    const float e = __builtin_amdgcn_exp2f((x * x) * -1.4426950408889634f);
+    const float erf_abs = fmaf(-(poly * t), e, 1.0f);
+    const float hv = 0.5f * v;
+    return fmaf(fabsf(hv), erf_abs, hv);
+}
+
 template <bool NORM, bool MULGELU, bool GATE>
 __global__ __launch_bounds__(64, 2) void linear_f32_kernel(
     const float *__restrict__ x, int64_t x_stride, const float *__restrict__ x2, int64_t x2_stride,
@@ -80,8 +97,8 @@ __global__ __launch_bounds__(64, 2) void linear_f32_kernel(
 #pragma unroll
             for (int i = 0; i < kLfSlab / 4; ++i) {
                 const f32x4 v = *reinterpret_cast<const f32x4 *>(yp + 4 * i);
-                a[4 * i] = gelu_erf(a[4 * i]) * v.x, a[4 * i + 1] = gelu_erf(a[4 * i + 1]) * v.y;
-                a[4 * i + 2] = gelu_erf(a[4 * i + 2]) * v.z, a[4 * i + 3] = gelu_erf(a[4 * i + 3]) * v.w;
+                a[4 * i] = gelu_erf_lf(a[4 * i]) * v.x, a[4 * i + 1] = gelu_erf_lf(a[4 * i + 1]) * v.y;
+                a[4 * i + 2] = gelu_erf_lf(a[4 * i + 2]) * v.z, a[4 * i + 3] = gelu_erf_lf(a[4 * i + 3]) * v.w;
             }
         }
     };
@@ -152,7 +169,7 @@ __global__ __launch_bounds__(64, 2) void linear_f32_kernel(
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             float o = acc[v] + bv;
-            if (GATE) o = gelu_erf(o) * acc2[v];
+            if (GATE) o = gelu_erf_lf(o) * acc2[v];
             if (resid != nullptr) o += res[v];
             acc[v] = o;
         }
