@@ -173,6 +173,21 @@ def update() -> None:
         dq, dkv = bruteforce.bullet_read_grad_loops(qkv[..., :D], kv, active, H, dout)
         out.update({f"{tag}_qkv": qkv, f"{tag}_kv": kv, f"{tag}_active": active, f"{tag}_heads": np.int64(H), f"{tag}_dout": dout,
                     f"{tag}_dq": dq, f"{tag}_dkv": dkv})
+    # the same over a long slot axis (more live bullets than one 160-key tile of the backward kernels), from its
+    # own generator so that the vectors above and below do not depend on it
+    rng_long = np.random.default_rng(20260)
+    B, N, NB, H = 3, 12, 200, 1
+    D = 32 * H
+    qkv = bf16(1.2 * rng_long.standard_normal((B, N, 3 * D)))
+    kv = bf16(1.2 * rng_long.standard_normal((B, NB, 2 * D)))
+    active = rng_long.random((B, NB)) < 0.9
+    active[0] = False
+    active[1] = False
+    active[1, NB // 3] = True
+    dout = bf16(rng_long.standard_normal((B, N, D)))
+    dq, dkv = bruteforce.bullet_read_grad_loops(qkv[..., :D], kv, active, H, dout)
+    out.update({"cross_long_qkv": qkv, "cross_long_kv": kv, "cross_long_active": active, "cross_long_heads": np.int64(H),
+                "cross_long_dout": dout, "cross_long_dq": dq, "cross_long_dkv": dkv})
     # sequence conv backward with episode ends and a gradient on the handed-on inputs
     R, T, D = 5, 11, 128
     b1 = bf16(rng.standard_normal((R, T, D)))

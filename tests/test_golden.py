@@ -239,7 +239,7 @@ def test_kernels_reproduce_conv_and_norm_gradient_vectors(b_dtype):
     assert max_rel(dw.cpu().double(), torch.from_numpy(UPD["norm_dw"])) <= 1e-5
 
 
-UPD_CROSS = ("cross_4v4", "cross_wide")
+UPD_CROSS = ("cross_4v4", "cross_wide", "cross_long")
 
 
 @pytest.mark.parametrize("tag", UPD_CROSS)
@@ -267,7 +267,10 @@ def test_kernels_reproduce_bullet_read_gradient_vectors(tag, form):
     B, NB, D2 = kv.shape
     if form == "mask":
         out = ops.sdpa_cross(qkv, kv, act, H)
-        dq, dkv = ops.sdpa_cross_bwd(qkv, kv, act, H, out, dout)
+        if NB <= 160:
+            dq, dkv = ops.sdpa_cross_bwd(qkv, kv, act, H, out, dout)
+        else:  # long slot axes: the streaming pair, reading the buffer in place through the list of live slots
+            dq, dkv = ops.sdpa_cross_stream_bwd(qkv, kv, ops.CompactRows(act), H, out, dout, indexed=True)
         dkv = dkv.float().cpu()
     else:
         rows = ops.CompactRows(act)
