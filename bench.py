@@ -370,7 +370,8 @@ def main():
     if bf16 and w.NM <= 160:
         attn_kernel = "sdpa_mfma_pair_kernel" if (w.NM <= 16 and H % 2 == 0) else "sdpa_mfma_kernel"
     roofs = {"attention": roof(attn_kernel, ab["attn"], t_attn, med_attn),
-             "rglru": roof("rglru_step_vec8_kernel", ab["rglru"], t_rglru, med_rglru)}
+             # the lane map with dense memory instructions covers the widths that divide 512
+             "rglru": roof("rglru_step_dense_kernel" if 512 % D == 0 else "rglru_step_vec8_kernel", ab["rglru"], t_rglru, med_rglru)}
     dominant = "attention" if t_attn >= t_rglru else "rglru"
 
     result = {

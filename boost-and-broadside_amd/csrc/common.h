@@ -113,6 +113,42 @@ __device__ __forceinline__ void store8_stream(uint16_t *p, const Row8 &r)
                                 reinterpret_cast<u32x4 *>(p));
 }
 
+// Four consecutive channels of one row, widened to fp32 (an 8-byte access in bf16, 16 bytes in fp32).
+struct Row4 {
+    float v[4];
+};
+
+template <bool STREAM>
+__device__ __forceinline__ Row4 load4(const float *p)
+{
+    const f32x4 a = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p)) : *reinterpret_cast<const f32x4 *>(p);
+    return Row4{{a.x, a.y, a.z, a.w}};
+}
+
+template <bool STREAM>
+__device__ __forceinline__ Row4 load4(const uint16_t *p)
+{
+    const u32x2 w = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(p)) : *reinterpret_cast<const u32x2 *>(p);
+    return Row4{{__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u), __uint_as_float(w.y << 16),
+                 __uint_as_float(w.y & 0xffff0000u)}};
+}
+
+template <bool STREAM>
+__device__ __forceinline__ void store4(float *p, const Row4 &r)
+{
+    const f32x4 v = {r.v[0], r.v[1], r.v[2], r.v[3]};
+    if (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(p));
+    else *reinterpret_cast<f32x4 *>(p) = v;
+}
+
+template <bool STREAM>
+__device__ __forceinline__ void store4(uint16_t *p, const Row4 &r)
+{
+    const u32x2 v = {pack_bf16x2(r.v[0], r.v[1]), pack_bf16x2(r.v[2], r.v[3])};
+    if (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<u32x2 *>(p));
+    else *reinterpret_cast<u32x2 *>(p) = v;
+}
+
 __device__ __forceinline__ float load1(const float *p) { return *p; }
 __device__ __forceinline__ float load1(const uint16_t *p) { return bf16_bits_to_f32(*p); }
 __device__ __forceinline__ void store1(float *p, float v) { *p = v; }

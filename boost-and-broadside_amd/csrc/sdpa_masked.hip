@@ -395,11 +395,13 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
 
     // The MFMA leaves a lane with rows 8i + 4*half + j (i, j = 0..3) of O^T.  V^T was stored
     // with its rows permuted so that MFMA row 8i + 4*half + j is channel
-    // 16*(i/2) + 8*half + 4*(i%2) + j: the lane then owns two runs of 8 consecutive channels
-    // and stores 16 bytes at a time, lanes m and m+32 side by side (32 contiguous bytes per
-    // row and store instruction instead of scattered 8-byte pieces).
-    if (qrow < NQ) {
-        const int64_t o_off = ((int64_t)env * NQ + qrow) * D + head * kDh + 8 * half;
+    // 16*(i/2) + 8*half + 4*(i%2) + j: the lane then owns two runs of 8 consecutive channels,
+    // 16 bytes each.  Stored as they are, one instruction would write 32 bytes of each of 32 rows.
+    // Lanes m and m + 16 first trade runs (v_permlane16_swap: the second run of query m goes to the
+    // lane of query m + 16, whose first run comes back), so that one store instruction writes the
+    // whole 64-byte head row of 16 queries and the other the rows of the other 16.
+    {
+        u32x4 w[2];
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
             float r[8];
@@ -407,14 +409,24 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
             for (int e = 0; e < 8; ++e) r[e] = o[8 * g + e] * inv;
             if (CROSS && accum != nullptr) {
                 // bf16 + bf16 as torch adds them: the read result is rounded first, then the sum
-                const Row8 a = load8(accum + o_off + 16 * g);
+                const int qs = qrow < NQ ? qrow : NQ - 1;
+                const Row8 a = load8(accum + ((int64_t)env * NQ + qs) * D + head * kDh + 8 * half + 16 * g);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) r[e] = a.v[e] + round_to_bf16(r[e]);
             }
-            const u32x4 w = {pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3]), pack_bf16x2(r[4], r[5]),
-                             pack_bf16x2(r[6], r[7])};
-            *reinterpret_cast<u32x4 *>(out + o_off + 16 * g) = w;
+            w[g] = u32x4{pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3]), pack_bf16x2(r[4], r[5]), pack_bf16x2(r[6], r[7])};
         }
+#pragma unroll
+        for (int cdw = 0; cdw < 4; ++cdw) {
+            const u32x2 t = __builtin_amdgcn_permlane16_swap(w[0][cdw], w[1][cdw], false, false);
+            w[0][cdw] = t.x, w[1][cdw] = t.y;
+        }
+        // lane (m, half) now holds, of query 32 wave + m%16: channels 16 (m/16) + 8 half .. +7 in w[0];
+        // of query 32 wave + 16 + m%16: the same channels in w[1]
+        const int row_a = wave * 32 + (m & 15);
+        const int ch = head * kDh + 16 * (m >> 4) + 8 * half;
+        if (row_a < NQ) *reinterpret_cast<u32x4 *>(out + ((int64_t)env * NQ + row_a) * D + ch) = w[0];
+        if (row_a + 16 < NQ) *reinterpret_cast<u32x4 *>(out + ((int64_t)env * NQ + row_a + 16) * D + ch) = w[1];
     }
 }
 
@@ -548,16 +560,24 @@ __global__ __launch_bounds__(kWave) void sdpa_mfma_pair_kernel(
     }
     sum += __shfl_xor(sum, 32);
     const float inv = __builtin_amdgcn_rcpf(sum);
-    if (qi < NM) {
-        const int64_t o_off = ((int64_t)env * NM + qi) * D + qhead * kDh + 8 * half;
+    // Lanes m and m + 16 hold the same token of the pair's two heads.  They trade runs as in
+    // sdpa_mfma_kernel, so that one store instruction writes the whole 64-byte row of the first
+    // head for every token and the other the row of the second head (instead of 32 bytes of each).
+    u32x4 w[2];
 #pragma unroll
-        for (int g = 0; g < 2; ++g) {
-            const u32x4 w = {pack_bf16x2(o[8 * g + 0] * inv, o[8 * g + 1] * inv),
-                             pack_bf16x2(o[8 * g + 2] * inv, o[8 * g + 3] * inv),
-                             pack_bf16x2(o[8 * g + 4] * inv, o[8 * g + 5] * inv),
-                             pack_bf16x2(o[8 * g + 6] * inv, o[8 * g + 7] * inv)};
-            *reinterpret_cast<u32x4 *>(out + o_off + 16 * g) = w;
-        }
+    for (int g = 0; g < 2; ++g)
+        w[g] = u32x4{pack_bf16x2(o[8 * g + 0] * inv, o[8 * g + 1] * inv), pack_bf16x2(o[8 * g + 2] * inv, o[8 * g + 3] * inv),
+                     pack_bf16x2(o[8 * g + 4] * inv, o[8 * g + 5] * inv), pack_bf16x2(o[8 * g + 6] * inv, o[8 * g + 7] * inv)};
+#pragma unroll
+    for (int cdw = 0; cdw < 4; ++cdw) {
+        const u32x2 t = __builtin_amdgcn_permlane16_swap(w[0][cdw], w[1][cdw], false, false);
+        w[0][cdw] = t.x, w[1][cdw] = t.y;
+    }
+    if (qi < NM) {
+        // w[0]: head head0, w[1]: head head0 + 1; channels 16 (m/16) + 8 half .. +7 of each
+        const int64_t o_off = ((int64_t)env * NM + qi) * D + head0 * kDh + 16 * (m >> 4) + 8 * half;
+        *reinterpret_cast<u32x4 *>(out + o_off) = w[0];
+        *reinterpret_cast<u32x4 *>(out + o_off + kDh) = w[1];
     }
 }
 
@@ -993,7 +1013,8 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
     sum += __shfl_xor(sum, 32);
     const float inv = cnt == 0 ? 0.0f : __builtin_amdgcn_rcpf(sum);
 
-    if (qrow < NQ) {
+    {
+        u32x4 w[2];
 #pragma unroll
         for (int g = 0; g < 2; ++g) {
             float r[8];
@@ -1009,10 +1030,18 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
                     r[e] = a + round_to_bf16(r[e]);
                 }
             }
-            const u32x4 w = {pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3]), pack_bf16x2(r[4], r[5]),
-                             pack_bf16x2(r[6], r[7])};
-            *reinterpret_cast<u32x4 *>(out + o_off + 16 * g) = w;
+            w[g] = u32x4{pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3]), pack_bf16x2(r[4], r[5]), pack_bf16x2(r[6], r[7])};
         }
+        // whole 64-byte head rows per store instruction (lanes m and m + 16 trade runs, see sdpa_mfma_kernel)
+#pragma unroll
+        for (int cdw = 0; cdw < 4; ++cdw) {
+            const u32x2 t = __builtin_amdgcn_permlane16_swap(w[0][cdw], w[1][cdw], false, false);
+            w[0][cdw] = t.x, w[1][cdw] = t.y;
+        }
+        const int row_a = wave * 32 + (m & 15);
+        const int ch = head * kDh + 16 * (m >> 4) + 8 * half;
+        if (row_a < NQ) *reinterpret_cast<u32x4 *>(out + ((int64_t)env * NQ + row_a) * D + ch) = w[0];
+        if (row_a + 16 < NQ) *reinterpret_cast<u32x4 *>(out + ((int64_t)env * NQ + row_a + 16) * D + ch) = w[1];
     }
 }
 

@@ -73,7 +73,19 @@ __global__ __launch_bounds__(kTsMaxWaves * kWave) __attribute__((amdgpu_waves_pe
     uint16_t *tile = s_tiles + wave * kTsTileHalfs;
     // row mapping
     const int sub = lane >> 3;       // row inside a pass of 8 rows
-    const int f8 = (lane & 7) * 8;   // first of the lane's 8 channels inside a half of 64
+    // The lane's 8 channels inside a half of 64 are two runs of four, c4 .. c4+3 and 32+c4 .. 32+c4+3, so that the
+    // eight lanes of a row cover 128 contiguous bytes of fp32 with EACH 16-byte access (64 bytes of bf16 with each
+    // 8-byte access): a 16-byte access whose lanes sit 32 bytes apart streams a third slower on this memory system.
+    const int c4 = (lane & 7) * 4;
+    auto ch = [&](int e) { return c4 + (e & 3) + 32 * (e >> 2); };  // channel of element e inside the half
+    auto ld8 = [&](auto *half_base) -> Row8 {
+        const Row4 a = load4<false>(half_base + c4), b = load4<false>(half_base + c4 + 32);
+        return Row8{{a.v[0], a.v[1], a.v[2], a.v[3], b.v[0], b.v[1], b.v[2], b.v[3]}};
+    };
+    auto st8 = [&](auto *half_base, const Row8 &r) {
+        store4<false>(half_base + c4, Row4{{r.v[0], r.v[1], r.v[2], r.v[3]}});
+        store4<false>(half_base + c4 + 32, Row4{{r.v[4], r.v[5], r.v[6], r.v[7]}});
+    };
     // matrix-core mapping
     const int m = lane & 31;
     const int half = lane >> 5;
@@ -82,7 +94,7 @@ __global__ __launch_bounds__(kTsMaxWaves * kWave) __attribute__((amdgpu_waves_pe
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) l2s[hf][e] = s_l2sig[64 * hf + f8 + e];
+        for (int e = 0; e < 8; ++e) l2s[hf][e] = s_l2sig[64 * hf + ch(e)];
 
     // Rounds of whole tiles are dealt to the waves of the grid in turn (at any time the grid works
     // on one compact window of rows); what is left after the last whole round is split evenly
@@ -117,13 +129,13 @@ __global__ __launch_bounds__(kTsMaxWaves * kWave) __attribute__((amdgpu_waves_pe
         float v[2][4][8];
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-            const int d0 = 64 * hf + f8;
+            const int d0 = 64 * hf;  // first channel of the half
             float w[8][4], beta[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const f32x4 q = *reinterpret_cast<const f32x4 *>(s_conv_w + (d0 + e) * 4);
+                const f32x4 q = *reinterpret_cast<const f32x4 *>(s_conv_w + (d0 + ch(e)) * 4);
                 w[e][0] = q.x, w[e][1] = q.y, w[e][2] = q.z, w[e][3] = q.w;
-                beta[e] = s_conv_b[d0 + e];
+                beta[e] = s_conv_b[d0 + ch(e)];
             }
             // two rows at a time: all loads of the pair, then arithmetic and stores
 #pragma unroll
@@ -136,11 +148,11 @@ __global__ __launch_bounds__(kTsMaxWaves * kWave) __attribute__((amdgpu_waves_pe
                     const int64_t b1_off = b1_group_stride != 0
                                                ? env[p] * b1_group_stride + (row[p] - env[p] * rows_per_env) * b1_row_stride
                                                : row[p] * b1_row_stride;
-                    cur[i] = load8(b1 + b1_off + d0);
+                    cur[i] = ld8(b1 + b1_off + d0);
                     const float *pin = conv_in + row[p] * conv_in_stride + d0;
-                    p0[i] = load8(pin);
-                    p1[i] = load8(pin + kTsD);
-                    p2[i] = load8(pin + 2 * kTsD);
+                    p0[i] = ld8(pin);
+                    p1[i] = ld8(pin + kTsD);
+                    p2[i] = ld8(pin + 2 * kTsD);
                 }
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
@@ -160,14 +172,14 @@ __global__ __launch_bounds__(kTsMaxWaves * kWave) __attribute__((amdgpu_waves_pe
                     }
                     if (valid[p]) {
                         float *pout = conv_out + row[p] * conv_out_stride + d0;
-                        store8(pout, p1[i]);
-                        store8(pout + kTsD, p2[i]);
-                        store8(pout + 2 * kTsD, cur[i]);
+                        st8(pout, p1[i]);
+                        st8(pout + kTsD, p2[i]);
+                        st8(pout + 2 * kTsD, cur[i]);
                     }
                     const float *vv = v[hf][p];
-                    *reinterpret_cast<u32x4 *>(tile + (8 * p + sub) * kTsPitch + d0) =
-                        u32x4{pack_bf16x2(vv[0], vv[1]), pack_bf16x2(vv[2], vv[3]), pack_bf16x2(vv[4], vv[5]),
-                              pack_bf16x2(vv[6], vv[7])};
+                    uint16_t *tp = tile + (8 * p + sub) * kTsPitch + d0 + c4;
+                    *reinterpret_cast<u32x2 *>(tp) = u32x2{pack_bf16x2(vv[0], vv[1]), pack_bf16x2(vv[2], vv[3])};
+                    *reinterpret_cast<u32x2 *>(tp + 32) = u32x2{pack_bf16x2(vv[4], vv[5]), pack_bf16x2(vv[6], vv[7])};
                 }
             }
         }
@@ -182,11 +194,11 @@ __global__ __launch_bounds__(kTsMaxWaves * kWave) __attribute__((amdgpu_waves_pe
 
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-            const int d0 = 64 * hf + f8;
+            const int d0 = 64 * hf;
             // previous state of this half's channels: in flight while the matrix cores work
             Row8 hv[4];
 #pragma unroll
-            for (int p = 0; p < 4; ++p) hv[p] = load8(h_in + row[p] * h_in_stride + d0);
+            for (int p = 0; p < 4; ++p) hv[p] = ld8(h_in + row[p] * h_in_stride + d0);
 
             // ---- gate pre-activations of channels 64*hf .. +63: blocks q = 0,1 of Wa, 2,3 of Wx ----
             // A lane ends up with 16 consecutive channels per block: 32*(q%2) + 16*half + 0..15.
@@ -229,20 +241,20 @@ __global__ __launch_bounds__(kTsMaxWaves * kWave) __attribute__((amdgpu_waves_pe
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
                 if (8 * p >= tile_rows) break;
-                const uint16_t *gp = tile + (8 * p + sub) * kTsPitch + f8;
-                const Row8 ga = load8(gp);
-                const Row8 gx = load8(gp + 64);
+                const uint16_t *gp = tile + (8 * p + sub) * kTsPitch;
+                const Row8 ga = ld8(gp);
+                const Row8 gx = ld8(gp + 64);
                 Row8 out;
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
                     out.v[e] = rglru_element<true, false>(v[hf][p][e], ga.v[e], gx.v[e], l2s[hf][e], c,
                                                           zero[p] ? 0.0f : hv[p].v[e]);
                 if (valid[p]) {
-                    store8(h_out + row[p] * h_out_stride + d0, out);
+                    st8(h_out + row[p] * h_out_stride + d0, out);
                     const int64_t y_off = y_group_stride != 0
                                               ? env[p] * y_group_stride + (row[p] - env[p] * rows_per_env) * y_row_stride
                                               : row[p] * y_row_stride;
-                    store8(y + y_off + d0, out);
+                    st8(y + y_off + d0, out);
                 }
             }
             wave_lds_handover();
