@@ -16,9 +16,10 @@
 // life and its 8 waves walk over tiles of 32 rows independently (no work-group barrier inside
 // the loop).  A wave alternates between two thread-to-data mappings and exchanges only the small
 // operands through its private 8.5 KB LDS tile:
-//   * row mapping (global memory side): 8 lanes cover 64 consecutive channels of a row with
-//     16-byte accesses, 8 rows per instruction; conv, buffer shift and the recurrence run here,
-//     v stays in registers between them;
+//   * row mapping (global memory side): 8 lanes cover 64 consecutive channels of a row, each lane
+//     two runs of four channels 32 apart, so that every 16-byte (fp32) or 8-byte (bf16) access
+//     instruction covers dense 128-byte / 64-byte runs, 8 rows per instruction; conv, buffer
+//     shift and the recurrence run here, v stays in registers between them;
 //   * matrix-core mapping: G^T = W v^T per 32 gate features x 32 rows, v^T read from the LDS
 //     tile as the B operand, W as the A operand straight from the packed stream; the result
 //     (bias added, rounded to bf16 like the library GEMM's output) goes back through the same
