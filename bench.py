@@ -568,6 +568,17 @@ def main():
         t_branch = timed_loop(branch_compact, n_b, 3) / n_b
         t_branch_all = timed_loop(branch_all_slots, 4, 2) / 4
         del bullets_f, layer_b
+
+        # the read over rows compacted beforehand (what the trunk calls), and its backward (the PPO update's
+        # kernels for this read: one tile of keys up to 160 live bullets per environment, the streaming pair above)
+        rows_b = ops.CompactRows(b_mask)
+        total_b = rows_b.total_host()
+        kv_rows_b = kv_b.reshape(w.B * NB, 2 * D)[b_mask.reshape(-1)].contiguous()
+        t_rows = timed_loop(lambda t: ops.sdpa_cross_rows(qkv_b, kv_rows_b, rows_b, H, accum=merged[t & 1], total=total_b), n_b, 3) / n_b
+        out_b = ops.sdpa_cross_rows(qkv_b, kv_rows_b, rows_b, H, total=total_b)
+        dout_b = (0.5 * torch.randn(w.B, w.NM, D, device=dev, generator=gen)).to(w.dtype)
+        t_bwd = timed_loop(lambda t: ops.sdpa_cross_rows_bwd(qkv_b, kv_rows_b, rows_b, H, out_b, dout_b, total_b), n_b, 3) / n_b
+        del kv_rows_b, out_b, dout_b
         read_bytes = live * 2 * D * 2 + w.B * NB + 3 * w.B * w.NM * D * 2
         result["bullet_read"] = {
             "avg_launch_us": t_read * 1e6, "slots_per_env": NB, "live_fraction": live_p,
@@ -575,6 +586,7 @@ def main():
             "frac_of_hbm_peak": read_bytes / t_read / peak,
             "tflops": 4 * live * w.NM * D / t_read / 1e12,
             "eager_torch_us": None if t_read_torch is None else t_read_torch * 1e6,
+            "rows_form_us": t_rows * 1e6, "rows_form_backward_us": t_bwd * 1e6, "max_live_per_env": rows_b.max_count_host(),
             "branch_compact_us": t_branch * 1e6, "branch_all_slots_us": t_branch_all * 1e6,
             "branch_what": "norm_bullet + kv_bullet + read from fp32 bullet tokens: compact = device-side list of the "
                            "live bullets, bnb_norm_linear_fwd over it, bnb_sdpa_cross_ranges_fwd; all_slots = "
