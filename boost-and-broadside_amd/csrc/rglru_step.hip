@@ -78,7 +78,7 @@ template <int THREADS, typename XT, typename GT, typename YT, bool HAS_Y, bool S
 __global__ __launch_bounds__(THREADS) void rglru_step_dense_kernel(
     const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
     const float *h_in, int64_t h_in_stride, float *h_out, int64_t h_out_stride, YT *__restrict__ y,
-    int64_t R, int D, const uint8_t *__restrict__ reset, int rows_per_env, int64_t y_group_stride)
+    int64_t R, int D, int log2_d, const uint8_t *__restrict__ reset, int rows_per_env, int64_t y_group_stride)
 {
     extern __shared__ float s_l2sig[];  // D entries
     for (int d = threadIdx.x; d < D; d += THREADS) s_l2sig[d] = log2_sigmoid(log_lambda[d]);
@@ -89,14 +89,17 @@ __global__ __launch_bounds__(THREADS) void rglru_step_dense_kernel(
 #pragma unroll
     for (int part = 0; part < 2; ++part) {
         const int64_t e = first + 256 * part;
-        const int64_t row = e / D;
+        const int64_t row = e >> log2_d;  // D divides 512: a power of two
         if (row >= R) continue;
-        const int d0 = (int)(e - row * D);
+        const int d0 = (int)e & (D - 1);
         const Row4 xv = load4<STREAM>(x + row * D + d0);
         const Row4 ga = load4<STREAM>(gates + row * 2 * D + d0);
         const Row4 gx = load4<STREAM>(gates + row * 2 * D + D + d0);
         Row4 hv = load4<STREAM>(h_in + row * h_in_stride + d0);
-        const int64_t env = (reset != nullptr || y_group_stride != 0) ? row / rows_per_env : 0;
+        // rows fit 32 bits wherever a packed state of that many rows exists at all: one 32-bit division
+        const int64_t env = (reset != nullptr || y_group_stride != 0)
+                                ? (row <= 0xffffffffLL ? (int64_t)((uint32_t)row / (uint32_t)rows_per_env) : row / rows_per_env)
+                                : 0;
         if (reset != nullptr && reset[env]) {
 #pragma unroll
             for (int k = 0; k < 4; ++k) hv.v[k] = 0.0f;
@@ -165,17 +168,19 @@ static int launch_rglru(const void *x, const void *gates, const float *log_lambd
         // there and faster on mid-sized inputs (327,680 rows: 107 against 111 us).
         if (512 % D == 0) {
             const int64_t waves = (R * (int64_t)D + 511) / 512;
+            int log2_d = 0;
+            while ((1 << log2_d) < D) ++log2_d;
             const int64_t dblocks = (waves + (kRglruThreads >> 6) - 1) / (kRglruThreads >> 6);
             if (dblocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
             if (stream_hint)
                 hipLaunchKernelGGL((rglru_step_dense_kernel<kRglruThreads, XT, GT, YT, HAS_Y, true>), dim3((unsigned)dblocks),
                                    dim3(kRglruThreads), (size_t)D * sizeof(float), stream, (const XT *)x, (const GT *)gates,
-                                   log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D, reset, rows_per_env,
+                                   log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D, log2_d, reset, rows_per_env,
                                    y_group_stride);
             else
                 hipLaunchKernelGGL((rglru_step_dense_kernel<kRglruThreads, XT, GT, YT, HAS_Y, false>), dim3((unsigned)dblocks),
                                    dim3(kRglruThreads), (size_t)D * sizeof(float), stream, (const XT *)x, (const GT *)gates,
-                                   log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D, reset, rows_per_env,
+                                   log_lambda, c, h_in, h_in_stride, h_out, h_out_stride, (YT *)y, R, D, log2_d, reset, rows_per_env,
                                    y_group_stride);
             return (int)hipGetLastError();
         }
