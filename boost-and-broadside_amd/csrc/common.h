@@ -149,6 +149,24 @@ __device__ __forceinline__ void store4(uint16_t *p, const Row4 &r)
     else *reinterpret_cast<u32x2 *>(p) = v;
 }
 
+// Eight channels of one row as two runs of four, `gap` elements apart (p points at the first run): with
+// lane j of a row on channels 4j..4j+3 and gap + 4j..gap + 4j+3, every access instruction of the lanes
+// of a row covers one dense run of bytes, which streams markedly faster than eight consecutive
+// channels per lane (two 16-byte accesses whose lanes sit 32 bytes apart).
+template <bool STREAM, typename T>
+__device__ __forceinline__ Row8 load8_split(const T *p, int gap)
+{
+    const Row4 a = load4<STREAM>(p), b = load4<STREAM>(p + gap);
+    return Row8{{a.v[0], a.v[1], a.v[2], a.v[3], b.v[0], b.v[1], b.v[2], b.v[3]}};
+}
+
+template <bool STREAM, typename T>
+__device__ __forceinline__ void store8_split(T *p, int gap, const Row8 &r)
+{
+    store4<STREAM>(p, Row4{{r.v[0], r.v[1], r.v[2], r.v[3]}});
+    store4<STREAM>(p + gap, Row4{{r.v[4], r.v[5], r.v[6], r.v[7]}});
+}
+
 __device__ __forceinline__ float load1(const float *p) { return *p; }
 __device__ __forceinline__ float load1(const uint16_t *p) { return bf16_bits_to_f32(*p); }
 __device__ __forceinline__ void store1(float *p, float v) { *p = v; }

@@ -40,12 +40,13 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_vec8_kernel(
     const int local_row = threadIdx.x / vecs_per_row;
     const int64_t row = (int64_t)blockIdx.x * rows_per_block + local_row;
     if (local_row >= rows_per_block || row >= R) return;
-    const int d0 = (threadIdx.x - local_row * vecs_per_row) << 3;
+    const int d0 = (threadIdx.x - local_row * vecs_per_row) << 2;  // first of the lane's two runs of four channels
+    const int gap = D >> 1;        // the second run starts here: every access of a row's lanes is one dense run
 
     float l2[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) l2[e] = s_l2sig[d0 + e];
-    Row8 h = load8(h0 + row * h0_stride + d0);
+    for (int e = 0; e < 8; ++e) l2[e] = s_l2sig[d0 + (e & 3) + (e >> 2) * gap];
+    Row8 h = load8_split<false>(h0 + row * h0_stride + d0, gap);
     const XT *xp = x + row * rs + d0;
     const GT *gp = gates + row * 2 * rs + d0;
     YT *yp = y + row * rs + d0;
@@ -58,9 +59,9 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_vec8_kernel(
         for (int u = 0; u < kSeqAhead; ++u) {
             // past the end: re-read the last step (discarded) so the loads stay branch-free
             const int t = t0 + u < T ? t0 + u : T - 1;
-            xv[u] = load8_stream(xp + t * ts);
-            ga[u] = load8_stream(gp + t * 2 * ts);
-            gx[u] = load8_stream(gp + t * 2 * ts + D);
+            xv[u] = load8_split<true>(xp + t * ts, gap);
+            ga[u] = load8_split<true>(gp + t * 2 * ts, gap);
+            gx[u] = load8_split<true>(gp + t * 2 * ts + D, gap);
             cut[u] = 0;
             if (dn != nullptr) cut[u] = dn[t > 0 ? t - 1 : 0];
             if (t == 0) cut[u] = 0;  // the first step continues the stored state
@@ -74,11 +75,11 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_vec8_kernel(
                     h.v[e] = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(xv[u].v[e], ga[u].v[e], gx[u].v[e],
                                                                                     l2[e], c, prev);
                 }
-                store8_stream(yp + (t0 + u) * ts, h);
+                store8_split<true>(yp + (t0 + u) * ts, gap, h);
             }
         }
     }
-    store8(h_last + row * h_last_stride + d0, h);
+    store8_split<false>(h_last + row * h_last_stride + d0, gap, h);
 }
 
 // Any D, any alignment, and small inputs (eight times the lanes): one lane per (row, channel).
@@ -294,13 +295,14 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_bwd_vec8_kernel(
     const int local_row = threadIdx.x / vecs_per_row;
     const int64_t row = (int64_t)blockIdx.x * rows_per_block + local_row;
     if (local_row >= rows_per_block || row >= R) return;
-    const int d0 = (threadIdx.x - local_row * vecs_per_row) << 3;
+    const int d0 = (threadIdx.x - local_row * vecs_per_row) << 2;  // first of the lane's two runs of four channels
+    const int gap = D >> 1;        // the second run starts here: every access of a row's lanes is one dense run
 
     float l2[8], oms[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        l2[e] = s_lam[d0 + e];
-        oms[e] = s_lam[D + d0 + e];
+        l2[e] = s_lam[d0 + (e & 3) + (e >> 2) * gap];
+        oms[e] = s_lam[D + d0 + (e & 3) + (e >> 2) * gap];
     }
     const XT *xp = x + row * rs + d0;
     const GT *gp = gates + row * 2 * rs + d0;
@@ -309,11 +311,11 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_bwd_vec8_kernel(
     XT *dxp = dx + row * rs + d0;
     GT *dgp = dgates + row * 2 * rs + d0;
     const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
-    const Row8 h_first = load8(h0 + row * h0_stride + d0);
+    const Row8 h_first = load8_split<false>(h0 + row * h0_stride + d0, gap);
     Row8 carry, dlam;
 #pragma unroll
     for (int e = 0; e < 8; ++e) carry.v[e] = dlam.v[e] = 0.0f;
-    if (dh_last != nullptr) carry = load8(dh_last + row * dh_last_stride + d0);
+    if (dh_last != nullptr) carry = load8_split<false>(dh_last + row * dh_last_stride + d0, gap);
 
     constexpr int AHEAD = 2;  // five operand rows per step: keep the register footprint moderate
     for (int t1 = T; t1 > 0; t1 -= AHEAD) {
@@ -322,16 +324,16 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_bwd_vec8_kernel(
 #pragma unroll
         for (int u = 0; u < AHEAD; ++u) {
             const int t = t1 - 1 - u > 0 ? t1 - 1 - u : 0;
-            xv[u] = load8_stream(xp + t * ts);
-            ga[u] = load8_stream(gp + t * 2 * ts);
-            gx[u] = load8_stream(gp + t * 2 * ts + D);
+            xv[u] = load8_split<true>(xp + t * ts, gap);
+            ga[u] = load8_split<true>(gp + t * 2 * ts, gap);
+            gx[u] = load8_split<true>(gp + t * 2 * ts + D, gap);
             if (dyp != nullptr) {
-                dyv[u] = load8_stream(dyp + t * ts);
+                dyv[u] = load8_split<true>(dyp + t * ts, gap);
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) dyv[u].v[e] = 0.0f;
             }
-            hp[u] = load8(yp + (t > 0 ? t - 1 : 0) * ts);
+            hp[u] = load8_split<false>(yp + (t > 0 ? t - 1 : 0) * ts, gap);
             cut[u] = 0;
             if (dn != nullptr) cut[u] = dn[t > 0 ? t - 1 : 0];
             if (t == 0) {
@@ -355,14 +357,14 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_bwd_vec8_kernel(
                     dlam.v[e] += g.dlam;
                     carry.v[e] = cut[u] ? 0.0f : g.carry;
                 }
-                store8_stream(dxp + t * ts, ox);
-                store8_stream(dgp + t * 2 * ts, oa);
-                store8_stream(dgp + t * 2 * ts + D, og);
+                store8_split<true>(dxp + t * ts, gap, ox);
+                store8_split<true>(dgp + t * 2 * ts, gap, oa);
+                store8_split<true>(dgp + t * 2 * ts + D, gap, og);
             }
         }
     }
-    store8(dh0 + row * D + d0, carry);
-    store8(dlam_rows + row * D + d0, dlam);
+    store8_split<false>(dh0 + row * D + d0, gap, carry);
+    store8_split<false>(dlam_rows + row * D + d0, gap, dlam);
 }
 
 template <typename XT, typename GT, typename YT>
@@ -425,20 +427,21 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_vec8_kernel(
     const int local_row = threadIdx.x / vecs_per_row;
     const int64_t row = (int64_t)blockIdx.x * rows_per_block + local_row;
     if (local_row >= rows_per_block || row >= R) return;
-    const int d0 = (threadIdx.x - local_row * vecs_per_row) << 3;
+    const int d0 = (threadIdx.x - local_row * vecs_per_row) << 2;  // first of the lane's two runs of four channels
+    const int gap = D >> 1;        // the second run starts here: every access of a row's lanes is one dense run
 
     float w[8][kSeqTaps], bs[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        const f32x4 wv = *reinterpret_cast<const f32x4 *>(weight + (int64_t)(d0 + e) * kSeqTaps);
+        const f32x4 wv = *reinterpret_cast<const f32x4 *>(weight + (int64_t)(d0 + (e & 3) + (e >> 2) * gap) * kSeqTaps);
         w[e][0] = wv.x;
         w[e][1] = wv.y;
         w[e][2] = wv.z;
         w[e][3] = wv.w;
-        bs[e] = bias != nullptr ? bias[d0 + e] : 0.0f;
+        bs[e] = bias != nullptr ? bias[d0 + (e & 3) + (e >> 2) * gap] : 0.0f;
     }
     const float *pin = conv_in + row * conv_in_stride + d0;
-    Row8 p0 = load8(pin), p1 = load8(pin + D), p2 = load8(pin + 2 * D);
+    Row8 p0 = load8_split<false>(pin, gap), p1 = load8_split<false>(pin + D, gap), p2 = load8_split<false>(pin + 2 * D, gap);
     const BT *bp = b1 + row * rs + d0;
     const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
     int hist = 3;
@@ -449,7 +452,7 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_vec8_kernel(
 #pragma unroll
         for (int u = 0; u < kSeqAhead; ++u) {
             const int t = t0 + u < T ? t0 + u : T - 1;
-            cur[u] = load8_stream(bp + t * ts);
+            cur[u] = load8_split<true>(bp + t * ts, gap);
             cut[u] = 0;
             if (dn != nullptr) cut[u] = dn[t > 0 ? t - 1 : 0];
             if (t == 0) cut[u] = 0;
@@ -470,8 +473,8 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_vec8_kernel(
                     v.v[e] = acc + bs[e];
                 }
                 const int64_t off = row * rs + (t0 + u) * ts + d0;
-                store8_stream(v_out + off, v);
-                if (v_bf16_out != nullptr) store8_stream(v_bf16_out + off, v);
+                store8_split<true>(v_out + off, gap, v);
+                if (v_bf16_out != nullptr) store8_split<true>(v_bf16_out + off, gap, v);
                 p0 = p1;
                 p1 = p2;
                 p2 = cur[u];
@@ -481,9 +484,9 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_vec8_kernel(
     }
     // the last three inputs, whatever episode they belong to (griffin.py:277)
     float *pout = conv_out + row * conv_out_stride + d0;
-    store8(pout, p0);
-    store8(pout + D, p1);
-    store8(pout + 2 * D, p2);
+    store8_split<false>(pout, gap, p0);
+    store8_split<false>(pout + D, gap, p1);
+    store8_split<false>(pout + 2 * D, gap, p2);
 }
 
 template <typename BT>
@@ -581,12 +584,13 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_bwd_kernel(
     const int vecs = D >> 3;
     const int rows_per_block = kSeqThreads / vecs;
     const int local_row = threadIdx.x / vecs;
-    const int d0 = (threadIdx.x - local_row * vecs) << 3;
+    const int d0 = (threadIdx.x - local_row * vecs) << 2;  // first of the lane's two runs of four channels
+    const int gap = D >> 1;        // the second run starts here: every access of a row's lanes is one dense run
 
     float w[8][kSeqTaps], dw[8][kSeqTaps], db[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        const f32x4 wv = *reinterpret_cast<const f32x4 *>(weight + (int64_t)(d0 + e) * kSeqTaps);
+        const f32x4 wv = *reinterpret_cast<const f32x4 *>(weight + (int64_t)(d0 + (e & 3) + (e >> 2) * gap) * kSeqTaps);
         w[e][0] = wv.x, w[e][1] = wv.y, w[e][2] = wv.z, w[e][3] = wv.w;
         dw[e][0] = dw[e][1] = dw[e][2] = dw[e][3] = 0.0f;
         db[e] = 0.0f;
@@ -601,7 +605,7 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_bwd_kernel(
         const float *dvp = dv + row * rs + d0;
         const BT *bp = b1 + row * rs + d0;
         const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
-        auto grad_row = [&](int t) -> Row8 { return t >= 0 && t < T ? load8_stream(dvp + t * ts) : zero; };
+        auto grad_row = [&](int t) -> Row8 { return t >= 0 && t < T ? load8_split<true>(dvp + t * ts, gap) : zero; };
         auto ended = [&](int t) -> bool { return dn != nullptr && t >= 0 && t < T && dn[t] != 0; };
 
         Row8 g0 = grad_row(s0), g1 = grad_row(s0 + 1), g2 = grad_row(s0 + 2);
@@ -615,9 +619,9 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_bwd_kernel(
                 gn[u] = grad_row(s + 3);
                 fn[u] = ended(s + 2);
                 if (s < 0)
-                    in[u] = load8(conv_in + row * conv_in_stride + (int64_t)(s + 3) * D + d0);
+                    in[u] = load8_split<false>(conv_in + row * conv_in_stride + (int64_t)(s + 3) * D + d0, gap);
                 else
-                    in[u] = s < T ? load8_stream(bp + s * ts) : zero;
+                    in[u] = s < T ? load8_split<true>(bp + s * ts, gap) : zero;
             }
 #pragma unroll
             for (int u = 0; u < kSeqAhead; ++u) {
@@ -640,14 +644,14 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_bwd_kernel(
                     }
                     if (dconv_out != nullptr && s >= T - 3) {
                         // this input is also entry s - (T - 3) of the stored inputs handed on
-                        const Row8 h = load8(dconv_out + row * 3 * (int64_t)D + (int64_t)(s - (T - 3)) * D + d0);
+                        const Row8 h = load8_split<false>(dconv_out + row * 3 * (int64_t)D + (int64_t)(s - (T - 3)) * D + d0, gap);
 #pragma unroll
                         for (int e = 0; e < 8; ++e) o.v[e] += h.v[e];
                     }
                     if (s < 0)
-                        store8(dconv_in + row * 3 * (int64_t)D + (int64_t)(s + 3) * D + d0, o);
+                        store8_split<false>(dconv_in + row * 3 * (int64_t)D + (int64_t)(s + 3) * D + d0, gap, o);
                     else
-                        store8_stream(db1 + row * rs + s * ts + d0, o);
+                        store8_split<true>(db1 + row * rs + s * ts + d0, gap, o);
                     g0 = g1, g1 = g2, g2 = g3;
                     f0 = f1, f1 = f2;
                 }
@@ -661,7 +665,7 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_bwd_kernel(
 #pragma unroll
     for (int q = 0; q < 5; ++q) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) s_red[local_row * D + d0 + e] = q < 4 ? dw[e][q < 4 ? q : 0] : db[e];
+        for (int e = 0; e < 8; ++e) s_red[local_row * D + d0 + (e & 3) + (e >> 2) * gap] = q < 4 ? dw[e][q < 4 ? q : 0] : db[e];
         __syncthreads();
         for (int d = threadIdx.x; d < D; d += kSeqThreads) {
             float t = 0.0f;
