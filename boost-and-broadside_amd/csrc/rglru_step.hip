@@ -36,14 +36,16 @@ __global__ __launch_bounds__(THREADS) void rglru_step_vec8_kernel(
     const int local_row = threadIdx.x / vecs_per_row;
     const int64_t row = (int64_t)blockIdx.x * rows_per_block + local_row;
     if (local_row >= rows_per_block || row >= R) return;
-    const int d0 = (threadIdx.x - local_row * vecs_per_row) << 3;
+    // two runs of four channels per lane (d0.. and gap + d0..): every access of a row's lanes is one dense run
+    const int d0 = (threadIdx.x - local_row * vecs_per_row) << 2;
+    const int gap = D >> 1;
 
     // STREAM: nontemporal accesses, best once the rows no longer fit the last-level cache; below
     // that size cached accesses let the producer's output be picked up on chip
-    const Row8 xv = STREAM ? load8_stream(x + row * D + d0) : load8(x + row * D + d0);
-    const Row8 ga = STREAM ? load8_stream(gates + row * 2 * D + d0) : load8(gates + row * 2 * D + d0);
-    const Row8 gx = STREAM ? load8_stream(gates + row * 2 * D + D + d0) : load8(gates + row * 2 * D + D + d0);
-    Row8 hv = STREAM ? load8_stream(h_in + row * h_in_stride + d0) : load8(h_in + row * h_in_stride + d0);
+    const Row8 xv = load8_split<STREAM>(x + row * D + d0, gap);
+    const Row8 ga = load8_split<STREAM>(gates + row * 2 * D + d0, gap);
+    const Row8 gx = load8_split<STREAM>(gates + row * 2 * D + D + d0, gap);
+    Row8 hv = load8_split<STREAM>(h_in + row * h_in_stride + d0, gap);
     // environment of the row: for the reset flag and for an output laid out per environment
     const int64_t env = (reset != nullptr || y_group_stride != 0) ? row / rows_per_env : 0;
     if (reset != nullptr && reset[env]) {
@@ -56,14 +58,12 @@ __global__ __launch_bounds__(THREADS) void rglru_step_vec8_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e)
         out.v[e] = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(xv.v[e], ga.v[e], gx.v[e],
-                                                                          s_l2sig[d0 + e], c, hv.v[e]);
-    if (STREAM) store8_stream(h_out + row * h_out_stride + d0, out);
-    else store8(h_out + row * h_out_stride + d0, out);
+                                                                          s_l2sig[d0 + (e & 3) + (e >> 2) * gap], c, hv.v[e]);
+    store8_split<STREAM>(h_out + row * h_out_stride + d0, gap, out);
     if (HAS_Y) {
         // y rows either back to back or in groups of rows_per_env, y_group_stride elements apart
         const int64_t y_off = y_group_stride != 0 ? env * y_group_stride + (row - env * rows_per_env) * D : row * D;
-        if (STREAM) store8_stream(y + y_off + d0, out);
-        else store8(y + y_off + d0, out);
+        store8_split<STREAM>(y + y_off + d0, gap, out);
     }
 }
 
