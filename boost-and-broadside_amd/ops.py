@@ -49,8 +49,44 @@ def _code(t: torch.Tensor, name: str) -> int:
         raise TypeError(f"{name} must be float32 or bfloat16, got {t.dtype}") from None
 
 
+_get_device = getattr(torch._C, "_cuda_getDevice", None)
+_set_device = getattr(torch._C, "_cuda_setDevice", None)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """Raw handle of torch's current stream on the current device.  The direct query is what
+    ``torch.cuda.current_stream().cuda_stream`` ends in, without building a Stream object on every launch
+    (about 9 us of host time each; a small rollout step is bound by exactly that)."""
+    if _raw_stream is not None and _get_device is not None:
+        return _raw_stream(_get_device())
     return torch.cuda.current_stream().cuda_stream
+
+
+class _on_device:
+    """``with torch.cuda.device(d)`` that does nothing when ``d`` is already the current device, the usual case."""
+
+    __slots__ = ("idx", "prev", "ctx")
+
+    def __init__(self, device: torch.device) -> None:
+        self.idx = device.index
+        self.ctx = None
+
+    def __enter__(self):
+        if _get_device is None or _set_device is None or self.idx is None:
+            self.ctx = torch.cuda.device(self.idx)
+            return self.ctx.__enter__()
+        self.prev = _get_device()
+        if self.prev != self.idx:
+            _set_device(self.idx)
+        return None
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            return self.ctx.__exit__(*exc)
+        if self.prev != self.idx:
+            _set_device(self.prev)
+        return False
 
 
 def sdpa_masked(
@@ -108,7 +144,7 @@ def sdpa_masked(
         raise ValueError(f"out must be a contiguous {(B, NM, D)} {qkv.dtype} tensor on {qkv.device}")
     if B == 0 or NM == 0:
         return out
-    with torch.cuda.device(qkv.device):
+    with _on_device(qkv.device):
         rc = _native.load().bnb_sdpa_masked_fwd_path(
             qkv.data_ptr(), qkv.stride(1), mask_ptr, out.data_ptr(), B, NM, n_heads, D // n_heads, dtype,
             _PATH_CODE[path], _stream(),
@@ -151,7 +187,7 @@ def sdpa_masked_bwd(qkv: torch.Tensor, alive: torch.Tensor | None, n_heads: int,
         mask_ptr = alive.data_ptr()
     dqkv = torch.empty((B, NM, D3), dtype=qkv.dtype, device=qkv.device)
     if B:
-        with torch.cuda.device(qkv.device):
+        with _on_device(qkv.device):
             rc = _native.load().bnb_sdpa_masked_bwd_path(qkv.data_ptr(), qkv.stride(1), mask_ptr, out.data_ptr(), dout.data_ptr(),
                                                          dqkv.data_ptr(), B, NM, n_heads, D // n_heads, _code(qkv, "qkv"),
                                                          _PATH_CODE[path], _stream())
@@ -246,7 +282,7 @@ def sdpa_cross(
         out = accum if accum is not None else torch.empty((B, NQ, D), dtype=qkv.dtype, device=qkv.device)
     if B == 0 or NQ == 0:
         return out
-    with torch.cuda.device(qkv.device):
+    with _on_device(qkv.device):
         rc = _native.load().bnb_sdpa_cross_fwd(
             qkv.data_ptr(), qkv.stride(1), NQ, kv.data_ptr(), kv.data_ptr() + D * kv.element_size(), kv.stride(1), NK,
             mask_ptr, None if accum is None else accum.data_ptr(), out.data_ptr(), B, n_heads, D // n_heads,
@@ -296,7 +332,7 @@ def sdpa_cross_stream_bwd(qkv, kv, rows: "CompactRows", n_heads, out, dout, *, i
         return dq.zero_(), dkv
     if B and NQ:
         stats = torch.empty((B, n_heads, NQ, 2), dtype=torch.float32, device=qkv.device)
-        with torch.cuda.device(qkv.device):
+        with _on_device(qkv.device):
             rc = _native.load().bnb_sdpa_cross_stream_bwd(
                 qkv.data_ptr(), qkv.stride(1), NQ, kv.data_ptr(), 2 * D, rows.offsets.data_ptr(),
                 rows.index.data_ptr() if indexed else None, capacity, out.data_ptr(), dout.data_ptr(), dq.data_ptr(),
@@ -331,7 +367,7 @@ def sdpa_cross_bwd(qkv, kv, key_mask, n_heads, out, dout) -> tuple[torch.Tensor,
     dq = torch.empty((B, NQ, D), dtype=torch.bfloat16, device=qkv.device)
     dkv = torch.empty((B, NK, 2 * D), dtype=torch.bfloat16, device=qkv.device)
     if B:
-        with torch.cuda.device(qkv.device):
+        with _on_device(qkv.device):
             rc = _native.load().bnb_sdpa_cross_bwd(qkv.data_ptr(), qkv.stride(1), NQ, kv.data_ptr(), kv.stride(1), NK, mask_ptr,
                                                    out.data_ptr(), dout.data_ptr(), dq.data_ptr(), dkv.data_ptr(), B, n_heads,
                                                    D // n_heads, _native.BF16, _stream())
@@ -397,7 +433,7 @@ def sdpa_cross_rows_bwd(qkv, kv_rows, rows: "CompactRows", n_heads, out, dout, t
     if total == 0:
         return dq.zero_(), dkv
     if B:
-        with torch.cuda.device(qkv.device):
+        with _on_device(qkv.device):
             rc = _native.load().bnb_sdpa_cross_ranges_bwd(qkv.data_ptr(), qkv.stride(1), NQ, kv_rows.data_ptr(), kv_rows.stride(0),
                                                           rows.offsets.data_ptr(), total, max(1, rows.max_count_host()), out.data_ptr(),
                                                           dout.data_ptr(),
@@ -521,7 +557,7 @@ def rglru_step(
     reset_ptr = _reset_pointer(reset, R, rows_per_env, x.device)
     if R == 0:
         return (h_out if y is None else y), h_out
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = _native.load().bnb_rglru_step_rows_fwd(
             x.data_ptr(), x_code, gates_pre.data_ptr(), g_code, log_lambda.data_ptr(), float(c),
             h.data_ptr(), h.stride(0), h_out.data_ptr(), h_out.stride(0),
@@ -629,7 +665,7 @@ def conv_step(
     v_lp = torch.empty((R, D), dtype=torch.bfloat16, device=b1.device) if also_bf16 else None
     reset_ptr = _reset_pointer(reset, R, rows_per_env, b1.device)
     if R:
-        with torch.cuda.device(b1.device):
+        with _on_device(b1.device):
             rc = _native.load().bnb_conv_step_rows_fwd(
                 b1.data_ptr(), b_code, int(b1_group), int(b1_row), conv_buf.data_ptr(), conv_buf.stride(0), weight.data_ptr(), bias_ptr,
                 reset_ptr, int(rows_per_env), v.data_ptr(), None if v_lp is None else v_lp.data_ptr(),
@@ -669,7 +705,7 @@ def linear_wgrad(dy: torch.Tensor, x: torch.Tensor, out: torch.Tensor | None = N
     lib = _native.load()
     slices = int(lib.bnb_linear_wgrad_slices(R, N, K))
     partials = torch.empty((slices, N, K), dtype=torch.float32, device=dy.device)
-    with torch.cuda.device(dy.device):
+    with _on_device(dy.device):
         rc = lib.bnb_linear_wgrad_fwd(dy2.data_ptr(), dy2.stride(0) if R else N, x2.data_ptr(), x2.stride(0) if R else K,
                                       partials.data_ptr(), slices, out.data_ptr(), int(bool(accumulate)), R, N, K, _stream())
     _native.check(rc, "bnb_linear_wgrad_fwd")
@@ -794,7 +830,7 @@ def team_pool(x: torch.Tensor, team_id: torch.Tensor, alive: torch.Tensor, score
 
         z = torch.empty((B * 2, n_heads * D), dtype=torch.float32, device=dev)
         lib = _native.load()
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             rc = lib.bnb_team_attend_fwd(
                 x.data_ptr(), env_stride(x), x.stride(1) if N else D, team_id.data_ptr(), env_stride(team_id) if N else 0,
                 alive.data_ptr(), env_stride(alive) if N else 0, score_vectors.contiguous().data_ptr(), z.data_ptr(),
@@ -869,7 +905,7 @@ class _TeamPoolTrain(torch.autograd.Function):
             return t.stride(0) if B > 1 else t.shape[1] * (t.stride(1) if N else 1)
 
         dpool = torch.empty((B, 2, D), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             rc = lib.bnb_team_gather_bwd(dships.data_ptr(), team_id.data_ptr(), env_stride(team_id) if N else 0, alive.data_ptr(),
                                          env_stride(alive) if N else 0, dpool.data_ptr(), B, N, D, _stream())
         _native.check(rc, "bnb_team_gather_bwd")
@@ -890,7 +926,7 @@ class _TeamPoolTrain(torch.autograd.Function):
         ds = torch.empty((B * N, 2 * H), dtype=torch.float32, device=dev)
         du = torch.empty((2 * H, D), dtype=torch.float32, device=dev)
         partials = torch.empty((int(lib.bnb_team_attend_bwd_partial_rows()), 2 * H, D), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             rc = lib.bnb_team_attend_bwd(
                 x.data_ptr(), env_stride(x) if N else 0, x.stride(1) if N else D, team_id.data_ptr(), env_stride(team_id) if N else 0,
                 alive.data_ptr(), env_stride(alive) if N else 0, u.data_ptr(), z.data_ptr(), dz.data_ptr(),
@@ -1031,7 +1067,7 @@ def temporal_step(
     if (b1_group or y_group) and (rows_per_env < 1 or R % rows_per_env):
         raise ValueError(f"rows_per_env={rows_per_env} does not divide the {R} rows")
     if R:
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             rc = _native.load().bnb_temporal_step_fwd(
                 b1.data_ptr(), int(b1_group), int(b1_row), conv_buf.data_ptr(), conv_buf.stride(0),
                 conv_out.data_ptr(), conv_out.stride(0), h.data_ptr(), h.stride(0), h_out.data_ptr(), h_out.stride(0),
@@ -1118,7 +1154,7 @@ def conv_seq(
     v_lp = torch.empty(b1.shape, dtype=torch.bfloat16, device=b1.device) if also_bf16 else None
     keep, done_ptr = _done_pointer(done, R, T, b1.device)
     if R:
-        with torch.cuda.device(b1.device):
+        with _on_device(b1.device):
             rc = _native.load().bnb_conv_seq_fwd(
                 b1.data_ptr(), b_code, conv_buf.data_ptr(), conv_buf.stride(0), weight.data_ptr(), bias_ptr, done_ptr,
                 v.data_ptr(), None if v_lp is None else v_lp.data_ptr(), conv_out.data_ptr(), conv_out.stride(0),
@@ -1161,7 +1197,7 @@ def conv_seq_bwd(b1, conv_buf, weight, done, dv, dconv_out=None, *, time_major: 
     blocks = int(lib.bnb_conv_seq_bwd_blocks(R, T, D))
     partials = torch.empty((blocks, 5 * D), dtype=torch.float32, device=b1.device)
     keep, done_ptr = _done_pointer(done, R, T, b1.device)
-    with torch.cuda.device(b1.device):
+    with _on_device(b1.device):
         rc = lib.bnb_conv_seq_bwd(b1.data_ptr(), _code(b1, "b1"), conv_buf.data_ptr(), conv_buf.stride(0) if R else 3 * D,
                                   weight.data_ptr(), done_ptr, dv.data_ptr(), None if dconv_out is None else dconv_out.data_ptr(),
                                   db1.data_ptr(), dconv.data_ptr(), partials.data_ptr(), blocks, dwb.data_ptr(), R, T, D,
@@ -1267,7 +1303,7 @@ def rglru_scan(
     y = torch.empty(x.shape, dtype=y_dtype, device=x.device)
     keep, done_ptr = _done_pointer(done, R, T, x.device)
     if R:
-        with torch.cuda.device(x.device):
+        with _on_device(x.device):
             rc = _native.load().bnb_rglru_scan_fwd(
                 x.data_ptr(), x_code, gates_pre.data_ptr(), g_code, log_lambda.data_ptr(), float(c), h0.data_ptr(),
                 h0.stride(0), done_ptr, y.data_ptr(), _DTYPE_CODE[y_dtype], h_out.data_ptr(), h_out.stride(0),
@@ -1305,7 +1341,7 @@ class _RglruScan(torch.autograd.Function):
         dh0 = torch.empty((R, D), dtype=torch.float32, device=x.device)
         dlam_rows = torch.empty((R, D), dtype=torch.float32, device=x.device)
         done_ptr = None if ctx.done is None else ctx.done.data_ptr()
-        with torch.cuda.device(x.device):
+        with _on_device(x.device):
             rc = _native.load().bnb_rglru_scan_bwd(
                 x_c.data_ptr(), _DTYPE_CODE[x.dtype], g_c.data_ptr(), _DTYPE_CODE[gates_pre.dtype],
                 log_lambda.data_ptr(), ctx.c, h0_c.data_ptr(), h0_c.stride(0), done_ptr, y.data_ptr(),
@@ -1356,7 +1392,7 @@ def add_rmsnorm(
     normed = torch.empty((R, D), dtype=out_dtype, device=x.device)
     o_code = _code(normed, "out_dtype")
     if R:
-        with torch.cuda.device(x.device):
+        with _on_device(x.device):
             rc = _native.load().bnb_add_rmsnorm_fwd(
                 x2.data_ptr(), x2.stride(0), d_ptr, d_code, weight.detach().contiguous().data_ptr(),
                 _F32_EPS if eps is None else float(eps), None if s_out is None else s_out.data_ptr(),
@@ -1398,7 +1434,7 @@ def rmsnorm_bwd(x: torch.Tensor, dy: torch.Tensor, weight: torch.Tensor, *, eps:
     lib = _native.load()
     blocks = int(lib.bnb_rmsnorm_bwd_blocks(R, D))
     partials = torch.empty((blocks, D), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = lib.bnb_rmsnorm_bwd(x2.data_ptr(), x2.stride(0) if R else D, dy2.data_ptr(), _code(dy2, "dy"),
                                  dy2.stride(0) if R else D, weight.detach().contiguous().data_ptr(),
                                  _F32_EPS if eps is None else float(eps), None if gs is None else gs.data_ptr(),
@@ -1431,7 +1467,7 @@ def rmsnorm_bwd_static(x: torch.Tensor, dy: torch.Tensor, weight: torch.Tensor, 
     for t, name, dt in ((grad_sum, "grad_sum", torch.float32), (dx_bf16, "dx_bf16", torch.bfloat16)):
         if t is not None and (t.dtype != dt or not t.is_contiguous() or t.shape != x.shape or not t.is_cuda):
             raise TypeError(f"{name} must be a contiguous {dt} device tensor with x's shape")
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = _native.load().bnb_rmsnorm_bwd_static(
             x.data_ptr(), D, dy.data_ptr(), _code(dy, "dy"), D, weight.data_ptr(), _F32_EPS if eps is None else float(eps),
             None if grad_sum is None else grad_sum.data_ptr(), dx.data_ptr(), None if dx_bf16 is None else dx_bf16.data_ptr(),
@@ -1533,7 +1569,7 @@ def gelu_mul(a: torch.Tensor, b: torch.Tensor, *, out_dtype: torch.dtype | None 
     R = a2.shape[0]
     out = torch.empty((R, H), dtype=out_dtype, device=a.device)
     if R:
-        with torch.cuda.device(a.device):
+        with _on_device(a.device):
             rc = _native.load().bnb_gelu_mul_fwd(
                 a2.data_ptr(), _code(a2, "a"), a2.stride(0), b2.data_ptr(), _code(b2, "b"), b2.stride(0),
                 out.data_ptr(), _code(out, "out_dtype"), R, H, _stream(),
@@ -1561,7 +1597,7 @@ def gelu_mul_bwd(a: torch.Tensor, b: torch.Tensor, dout: torch.Tensor) -> tuple[
     da = torch.empty((R, H), dtype=a.dtype, device=a.device)
     db = torch.empty((R, H), dtype=b.dtype, device=a.device)
     if R:
-        with torch.cuda.device(a.device):
+        with _on_device(a.device):
             rc = _native.load().bnb_gelu_mul_bwd(
                 a2.data_ptr(), _code(a2, "a"), a2.stride(0), b2.data_ptr(), _code(b2, "b"), b2.stride(0),
                 g2.data_ptr(), _code(g2, "dout"), da.data_ptr(), H, db.data_ptr(), H, R, H, _stream(),
@@ -1613,7 +1649,7 @@ class _GeluMulPackedTrain(torch.autograd.Function):
         dgu = torch.empty((R, 2 * H), dtype=gu.dtype, device=gu.device)
         if R:
             code = _code(g2, "gu")
-            with torch.cuda.device(gu.device):
+            with _on_device(gu.device):
                 rc = _native.load().bnb_gelu_mul_bwd(
                     g2.data_ptr(), code, g2.stride(0), g2.data_ptr() + H * g2.element_size(), code, g2.stride(0),
                     d2.data_ptr(), _code(d2, "dout"), dgu.data_ptr(), 2 * H, dgu.data_ptr() + H * dgu.element_size(), 2 * H,
@@ -1653,7 +1689,7 @@ def copy_bytes(src: torch.Tensor, dst: torch.Tensor) -> None:
     n = src.numel() * src.element_size()
     if n != dst.numel() * dst.element_size() or not (src.is_contiguous() and dst.is_contiguous()):
         raise ValueError("src and dst must be contiguous and of equal byte size")
-    with torch.cuda.device(src.device):
+    with _on_device(src.device):
         rc = _native.load().bnb_copy_bytes(src.data_ptr(), dst.data_ptr(), n, _stream())
     _native.check(rc, "bnb_copy_bytes")
 
@@ -1785,7 +1821,7 @@ def ffn_fused(
                 raise RuntimeError("ffn_fused is forward-only; call it under torch.no_grad()")
             flat.append(t.view(-1, D) if _uniform_rows(t, D) else t.reshape(-1, D).contiguous())
         if R:
-            with torch.cuda.device(x.device):
+            with _on_device(x.device):
                 rc = _native.load().bnb_ffn_fused_proj_fwd(
                     x2.data_ptr(), x2.stride(0), flat[0].data_ptr(), flat[0].stride(0),
                     flat[1].data_ptr() if len(flat) == 2 else None, flat[1].stride(0) if len(flat) == 2 else 0,
@@ -1795,7 +1831,7 @@ def ffn_fused(
             _native.check(rc, "bnb_ffn_fused_proj_fwd")
         return out.reshape(x.shape)
     if R:
-        with torch.cuda.device(x.device):
+        with _on_device(x.device):
             rc = _native.load().bnb_ffn_fused_fwd(
                 x2.data_ptr(), x2.stride(0), delta_ptr, _native.BF16, norm_weight.data_ptr(),
                 float(_F32_EPS if eps is None else eps), weights_packed.data_ptr(), out.data_ptr(), R, D, FFN_HIDDEN,
@@ -1871,7 +1907,7 @@ def linear_f32(x: torch.Tensor, weight_packed: torch.Tensor, *, bias: torch.Tens
         r2 = resid.reshape(-1, n_out) if _uniform_rows(resid, n_out) else resid.reshape(-1, n_out).contiguous()
     if R == 0:
         return out
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = _native.load().bnb_linear_f32_fwd(
             x2.data_ptr(), x2.stride(0) if R > 1 else K, None if y2 is None else y2.data_ptr(),
             0 if y2 is None else (y2.stride(0) if R > 1 else K), None if norm_weight is None else norm_weight.detach().contiguous().data_ptr(),
@@ -1931,7 +1967,7 @@ class CompactRows:
         self.index = torch.empty(max(B * n, 1), dtype=torch.int32, device=mask.device)
         if B and n:
             lib = _native.load()
-            with torch.cuda.device(mask.device):
+            with _on_device(mask.device):
                 _native.check(lib.bnb_mask_count(mask.data_ptr(), counts.data_ptr(), B, n, _stream()), "bnb_mask_count")
                 torch.cumsum(counts, dim=0, dtype=torch.int32, out=self.offsets[1:])
                 _native.check(lib.bnb_mask_fill(mask.data_ptr(), self.offsets.data_ptr(), self.index.data_ptr(), B, n,
@@ -2004,7 +2040,7 @@ def norm_linear(
     out = torch.empty((R, N), dtype=torch.bfloat16, device=x.device)
     norm_weight = norm_weight.detach().contiguous()
     if R:
-        with torch.cuda.device(x.device):
+        with _on_device(x.device):
             rc = _native.load().bnb_norm_linear_fwd(
                 x2.data_ptr(), x2.stride(0), None if rows is None else rows.index.data_ptr(),
                 None if rows is None else rows.total.data_ptr(), norm_weight.data_ptr(),
@@ -2049,7 +2085,7 @@ def sdpa_cross_rows(
         return out
     if kv_rows.shape[0] == 0:  # an empty list: every environment reads nothing
         return out if accum is not None else out.zero_()
-    with torch.cuda.device(qkv.device):
+    with _on_device(qkv.device):
         rc = _native.load().bnb_sdpa_cross_ranges_fwd(
             qkv.data_ptr(), qkv.stride(1), NQ, kv_rows.data_ptr(), kv_rows.stride(0), rows.offsets.data_ptr(),
             kv_rows.shape[0], None if accum is None else accum.data_ptr(), out.data_ptr(), B, n_heads, D // n_heads,
