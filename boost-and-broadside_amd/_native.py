@@ -12,7 +12,7 @@ import os
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "_lib", "libbnb_amd.so")
 
-ABI_VERSION = 20
+ABI_VERSION = 21
 F32, BF16 = 0, 1
 PATH_AUTO, PATH_VALU, PATH_MFMA, PATH_ENV, PATH_HEAD = 0, 1, 2, 3, 4
 
@@ -37,6 +37,7 @@ SIGNATURES = {
     "bnb_conv_step_rows_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _vp]),
     "bnb_linear_wgrad_slices": (_i, [_i64, _i, _i]),
     "bnb_linear_wgrad_fwd": (_i, [_vp, _i64, _vp, _i64, _vp, _i, _vp, _i, _i64, _i, _i, _vp]),
+    "bnb_linear_wgrad_tiled_fwd": (_i, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i, _vp, _i, _i64, _i, _i, _vp]),
     "bnb_conv_seq_bwd_blocks": (_i, [_i64, _i, _i]),
     "bnb_conv_seq_bwd": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _vp]),
     "bnb_gelu_mul_bwd": (_i, [_vp, _i, _i64, _vp, _i, _i64, _vp, _i, _vp, _i64, _vp, _i64, _i64, _i, _vp]),
@@ -70,6 +71,8 @@ SIGNATURES = {
     "bnb_mask_count": (_i, [_vp, _vp, _i, _i, _vp]),
     "bnb_mask_fill": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "bnb_ffn_fused_fwd": (_i, [_vp, _i64, _vp, _i, _vp, _f, _vp, _vp, _i64, _i, _i, _vp]),
+    "bnb_ffn_fused_train_fwd": (_i, [_vp, _i64, _vp, _i, _vp, _f, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp]),
+    "bnb_ffn_bwd": (_i, [_vp, _vp, _i, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i, _vp]),
     "bnb_ffn_fused_proj_fwd": (_i, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _f, _vp, _vp, _i64, _i, _i, _vp]),
     "bnb_gelu_mul_fwd": (_i, [_vp, _i, _i64, _vp, _i, _i64, _vp, _i, _i64, _i, _vp]),
     "bnb_copy_bytes": (_i, [_vp, _vp, _i64, _vp]),

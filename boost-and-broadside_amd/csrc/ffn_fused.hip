@@ -40,29 +40,14 @@
 #include <type_traits>
 
 #include "common.h"
+#include "ffn_math.h"
 
 namespace bnb {
 
-constexpr int kFfnD = 128;
-constexpr int kFfnHidden = 512;
-constexpr int kFfnChunks = kFfnHidden / 32;
 constexpr int kFfnChunkHalfs = 3 * 32 * kFfnD;  // 12288 bf16 = 24 KB
 constexpr int kFfnWaves = 4;
 constexpr int kFfnThreads = kFfnWaves * kWave;
 constexpr int kFfnPrefetch = kFfnChunkHalfs / 8 / kFfnThreads;  // 16-byte pieces per thread per chunk
-
-// erf-GELU as v * Phi(v) with Phi(v) ~ 1 / (1 + 2^(-v p(v^2))), p a quadratic fitted (minimax over
-// |v| <= 9) to the normal distribution function: |error of gelu| <= 2.6e-5, two orders of
-// magnitude below the bf16 rounding of the product that follows.  v^2 is clamped at 64, beyond
-// which the quadratic would turn over (there Phi is 0 or 1 to 1e-15 anyway).  Eight vector-ALU
-// instructions per element, two of them transcendental; the three-term Abramowitz-Stegun erfc
-// form used before had the same error at eleven.
-__device__ __forceinline__ float gelu_phi(float v)
-{
-    const float v2 = fminf(v * v, 64.0f);
-    const float p = fmaf(fmaf(v2, -0.0010142630628405414f, 0.10677572405393032f), v2, 2.3011213393619663f);
-    return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-(p * v)));
-}
 
 // What is added to x before the norm (the output of the sublayer the tail belongs to):
 //   kDeltaNone  nothing;  kDeltaRows  the bf16 rows `delta`;
@@ -75,11 +60,14 @@ __device__ __forceinline__ float gelu_phi(float v)
 enum { kDeltaNone = 0, kDeltaRows = 1, kDeltaProj = 2, kDeltaGate = 3 };
 constexpr int kProjPitch = kFfnD + 8;  // halfs per staged operand row (bank spread, 16-byte aligned)
 
-template <int MODE>
+// TRAIN: the update path's forward.  It also writes what the backward needs and nothing else saves: the
+// residual sum `s` (when there is a delta; otherwise s is x) and the normalised rows `n` in bf16.
+template <int MODE, bool TRAIN = false>
 __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void ffn_fused_kernel(
     const float *__restrict__ x, int64_t x_stride, const uint16_t *__restrict__ delta,
     const uint16_t *__restrict__ rows_b, const uint16_t *__restrict__ wproj, const float *__restrict__ norm_w,
-    float eps, const uint16_t *__restrict__ wpack, float *__restrict__ out, int64_t R, int64_t rows_a_stride, int64_t rows_b_stride, unsigned first_round)
+    float eps, const uint16_t *__restrict__ wpack, float *__restrict__ out, int64_t R, int64_t rows_a_stride, int64_t rows_b_stride, unsigned first_round,
+    float *__restrict__ s_out = nullptr, uint16_t *__restrict__ n_out = nullptr)
 {
     constexpr bool HAS_DELTA = MODE == kDeltaRows;
     // three weight buffers: chunk c is used while chunk c+1 is already complete (its operands
@@ -181,6 +169,7 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
             sv.y += __uint_as_float(dv.x & 0xffff0000u);
             sv.z += __uint_as_float(dv.y << 16);
             sv.w += __uint_as_float(dv.y & 0xffff0000u);
+            if (TRAIN && r < R) __builtin_nontemporal_store(sv, reinterpret_cast<f32x4 *>(s_out + r * kFfnD + io_col));
         }
         *reinterpret_cast<f32x4 *>(stage + (2 * j + io_row) * kRowPitch + io_col) = sv;
     }
@@ -243,6 +232,26 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
         for (int e = 0; e < 8; ++e) nb[ks][e] = (__bf16)((acc[ks >> 1][8 * (ks & 1) + e] * rstd) * wv[e]);
     }
 
+    if (TRAIN) {
+        // n leaves as whole 256-byte rows through this wave's slice of the staging area
+        uint16_t *stage_n = reinterpret_cast<uint16_t *>(stage);
+        wave_lds_handover();
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            const u32x4 v = __builtin_bit_cast(u32x4, nb[ks]);
+            uint16_t *sp = stage_n + m * kProjPitch + 16 * ks + 4 * half;
+            *reinterpret_cast<u32x2 *>(sp) = u32x2{v.x, v.y};
+            *reinterpret_cast<u32x2 *>(sp + 8) = u32x2{v.z, v.w};
+        }
+        wave_lds_handover();
+        const int a_row = lane >> 4, a_col = (lane & 15) * 8;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int64_t r = row0 + 4 * j + a_row;
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(stage_n + (4 * j + a_row) * kProjPitch + a_col);
+            if (r < R) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(n_out + r * kFfnD + a_col));
+        }
+    }
     __syncthreads();  // every wave has its tokens out of the staging area
     stash(0, pre);
     stash(1, pre1);
@@ -362,10 +371,11 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
 
 namespace bnb {
 
-template <int MODE>
+template <int MODE, bool TRAIN = false>
 static int launch_ffn(const float *x, int64_t x_stride, const void *rows_a, const void *rows_b, const void *wproj,
                       const float *norm_weight, float eps, const void *weights_packed, float *out, int64_t R,
-                      int64_t rows_a_stride, int64_t rows_b_stride, hipStream_t s)
+                      int64_t rows_a_stride, int64_t rows_b_stride, hipStream_t s, float *s_out = nullptr,
+                      uint16_t *n_out = nullptr)
 {
     const int64_t blocks = (R + kFfnWaves * 32 - 1) / (kFfnWaves * 32);
     if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
@@ -378,9 +388,9 @@ static int launch_ffn(const float *x, int64_t x_stride, const void *rows_a, cons
             cus = 256;
         first_round = 2u * (unsigned)cus;
     }
-    hipLaunchKernelGGL((ffn_fused_kernel<MODE>), dim3((unsigned)blocks), dim3(kFfnThreads), 0, s, x, x_stride,
+    hipLaunchKernelGGL((ffn_fused_kernel<MODE, TRAIN>), dim3((unsigned)blocks), dim3(kFfnThreads), 0, s, x, x_stride,
                        (const uint16_t *)rows_a, (const uint16_t *)rows_b, (const uint16_t *)wproj, norm_weight, eps,
-                       (const uint16_t *)weights_packed, out, R, rows_a_stride, rows_b_stride, first_round);
+                       (const uint16_t *)weights_packed, out, R, rows_a_stride, rows_b_stride, first_round, s_out, n_out);
     return (int)hipGetLastError();
 }
 
@@ -414,6 +424,24 @@ extern "C" int bnb_ffn_fused_fwd(const float *x, int64_t x_row_stride, const voi
                                       R, kFfnD, kFfnD, s);
     return launch_ffn<kDeltaNone>(x, x_row_stride, nullptr, nullptr, nullptr, norm_weight, eps, weights_packed, out, R,
                                   kFfnD, kFfnD, s);
+}
+
+extern "C" int bnb_ffn_fused_train_fwd(const float *x, int64_t x_row_stride, const void *delta, int delta_dtype,
+                                       const float *norm_weight, float eps, const void *weights_packed, float *out,
+                                       float *s_out, void *n_out, int64_t R, int D, int hidden, void *stream)
+{
+    using namespace bnb;
+    const int rc = ffn_common_checks(x, x_row_stride, norm_weight, weights_packed, out, R, D, hidden);
+    if (rc != 0 || R == 0) return rc;
+    if (delta && delta_dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
+    if (!n_out || (delta && !s_out)) return BNB_ERR_NULL_POINTER;
+    if ((delta && !aligned16(delta)) || !aligned16(n_out) || (s_out && !aligned16(s_out))) return BNB_ERR_MISALIGNED;
+    hipStream_t s = (hipStream_t)stream;
+    if (delta)
+        return launch_ffn<kDeltaRows, true>(x, x_row_stride, delta, nullptr, nullptr, norm_weight, eps, weights_packed,
+                                            out, R, kFfnD, kFfnD, s, s_out, (uint16_t *)n_out);
+    return launch_ffn<kDeltaNone, true>(x, x_row_stride, nullptr, nullptr, nullptr, norm_weight, eps, weights_packed,
+                                        out, R, kFfnD, kFfnD, s, nullptr, (uint16_t *)n_out);
 }
 
 extern "C" int bnb_ffn_fused_proj_fwd(const float *x, int64_t x_row_stride, const void *rows_a, int64_t rows_a_stride,

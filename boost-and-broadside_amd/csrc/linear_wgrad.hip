@@ -35,7 +35,8 @@ __device__ __forceinline__ int wg_slot(int c, int rb) { return c * kWgRows + 8 *
 
 __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
     const uint16_t *__restrict__ dy, int64_t dy_stride, const uint16_t *__restrict__ x, int64_t x_stride,
-    float *__restrict__ partials, int64_t R, int N, int K, int64_t rows_per_slice, int slices)
+    float *__restrict__ partials, int64_t R, int N, int K, int64_t rows_per_slice, int slices, int64_t dy_tile_stride,
+    int64_t x_tile_stride)
 {
     __shared__ __align__(16) uint16_t s_t[2][kWgTile * kWgRows];  // [operand: dy, x][column][row], swizzled
 
@@ -68,7 +69,9 @@ __global__ __launch_bounds__(kWgThreads) void linear_wgrad_kernel(
     const int operand = tid >> 7;  // uniform per wave
     const int rg = (tid & 127) >> 4;
     const int cb = tid & 15;
-    const uint16_t *src = operand ? x + k0 + 8 * cb : dy + n0 + 8 * cb;
+    // the 128 columns of a tile start `tile stride` elements after those of the tile before (128 for plain row-major
+    // operands; R * 128 for operands stored tile by tile)
+    const uint16_t *src = operand ? x + (k0 / kWgTile) * x_tile_stride + 8 * cb : dy + (n0 / kWgTile) * dy_tile_stride + 8 * cb;
     const int64_t src_stride = operand ? x_stride : dy_stride;
     uint16_t *dst = s_t[operand];
 
@@ -190,25 +193,37 @@ extern "C" int bnb_linear_wgrad_slices(int64_t R, int N, int K)
     return (int)s;
 }
 
-extern "C" int bnb_linear_wgrad_fwd(const void *dy, int64_t dy_row_stride, const void *x, int64_t x_row_stride,
-                                    float *partials, int slices, float *dw, int accumulate, int64_t R, int N, int K,
-                                    void *stream)
+extern "C" int bnb_linear_wgrad_tiled_fwd(const void *dy, int64_t dy_row_stride, int64_t dy_tile_stride, const void *x,
+                                          int64_t x_row_stride, int64_t x_tile_stride, float *partials, int slices, float *dw,
+                                          int accumulate, int64_t R, int N, int K, void *stream)
 {
     using namespace bnb;
     if (R < 0 || N < 1 || K < 1 || slices < 1) return BNB_ERR_BAD_SHAPE;
     if (N % kWgTile != 0 || K % kWgTile != 0 || slices > 65535) return BNB_ERR_UNSUPPORTED;
     if (!dw || !partials || (R > 0 && (!dy || !x))) return BNB_ERR_NULL_POINTER;
-    if (dy_row_stride < N || x_row_stride < K) return BNB_ERR_BAD_SHAPE;
+    // row-major operands hold all their columns in a row; tile-by-tile ones 128 per row
+    if (dy_row_stride < (dy_tile_stride == kWgTile ? N : kWgTile) || x_row_stride < (x_tile_stride == kWgTile ? K : kWgTile) ||
+        dy_tile_stride < kWgTile || x_tile_stride < kWgTile)
+        return BNB_ERR_BAD_SHAPE;
     if ((R > 0 && (!aligned16(dy) || !aligned16(x))) || !aligned16(partials) || !aligned16(dw) || dy_row_stride % 8 != 0 ||
-        x_row_stride % 8 != 0)
+        x_row_stride % 8 != 0 || dy_tile_stride % 8 != 0 || x_tile_stride % 8 != 0)
         return BNB_ERR_MISALIGNED;
     hipStream_t s = (hipStream_t)stream;
     const int64_t rows_per_slice = ((R + slices - 1) / slices + kWgRows - 1) / kWgRows * kWgRows;
     const int64_t groups = (int64_t)(N / kWgTile) * (K / kWgTile) * slices;
     if (groups > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(linear_wgrad_kernel, dim3((unsigned)groups), dim3(kWgThreads), 0, s, (const uint16_t *)dy, dy_row_stride,
-                       (const uint16_t *)x, x_row_stride, partials, R, N, K, rows_per_slice > 0 ? rows_per_slice : kWgRows, slices);
+                       (const uint16_t *)x, x_row_stride, partials, R, N, K, rows_per_slice > 0 ? rows_per_slice : kWgRows, slices,
+                       dy_tile_stride, x_tile_stride);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
     return launch_sum_slices(partials, dw, (int64_t)N * K, slices, accumulate, s);
+}
+
+extern "C" int bnb_linear_wgrad_fwd(const void *dy, int64_t dy_row_stride, const void *x, int64_t x_row_stride,
+                                    float *partials, int slices, float *dw, int accumulate, int64_t R, int N, int K,
+                                    void *stream)
+{
+    return bnb_linear_wgrad_tiled_fwd(dy, dy_row_stride, bnb::kWgTile, x, x_row_stride, bnb::kWgTile, partials, slices, dw,
+                                      accumulate, R, N, K, stream);
 }

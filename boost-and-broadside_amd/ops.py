@@ -712,6 +712,30 @@ def linear_wgrad(dy: torch.Tensor, x: torch.Tensor, out: torch.Tensor | None = N
     return out
 
 
+def _linear_wgrad_tiled(dy_tiles: torch.Tensor, x_tiles: torch.Tensor, R: int) -> torch.Tensor:
+    """``dW = dy^T x`` over the first R rows of operands stored tile by tile: ``dy_tiles`` (N/128, >= R, 128) and
+    ``x_tiles`` (K/128, >= R, 128) contiguous bfloat16 (a plain (>= R, 128) matrix is one tile).  Returns (N, K) float32."""
+    if dy_tiles.dim() == 2:
+        dy_tiles = dy_tiles.unsqueeze(0)
+    if x_tiles.dim() == 2:
+        x_tiles = x_tiles.unsqueeze(0)
+    for t, name in ((dy_tiles, "dy_tiles"), (x_tiles, "x_tiles")):
+        _need_device(t, name)
+        if t.dtype != torch.bfloat16 or not t.is_contiguous() or t.dim() != 3 or t.shape[2] != 128 or t.shape[1] < R:
+            raise ValueError(f"{name} must be a contiguous bfloat16 (tiles, >= {R}, 128) tensor")
+    N, K = 128 * dy_tiles.shape[0], 128 * x_tiles.shape[0]
+    out = torch.empty((N, K), dtype=torch.float32, device=dy_tiles.device)
+    lib = _native.load()
+    slices = int(lib.bnb_linear_wgrad_slices(R, N, K))
+    partials = torch.empty((slices, N, K), dtype=torch.float32, device=dy_tiles.device)
+    with _on_device(dy_tiles.device):
+        rc = lib.bnb_linear_wgrad_tiled_fwd(dy_tiles.data_ptr(), 128, max(dy_tiles.shape[1], 1) * 128, x_tiles.data_ptr(), 128,
+                                            max(x_tiles.shape[1], 1) * 128, partials.data_ptr(), slices, out.data_ptr(), 0, R, N, K,
+                                            _stream())
+    _native.check(rc, "bnb_linear_wgrad_tiled_fwd")
+    return out
+
+
 class _LinearTrain(torch.autograd.Function):
     """``F.linear`` under bfloat16 autocast whose weight gradient runs on ``linear_wgrad``."""
 
@@ -1741,6 +1765,152 @@ def pack_proj_weights(weight: torch.Tensor) -> torch.Tensor:
     cols = (16 * ks[None, :, None, None] + 8 * (e // 4)[None, None, None, :] + 4 * half[None, None, :, None]
             + (e % 4)[None, None, None, :]).expand(4, -1, -1, -1)
     return weight.detach().to(torch.bfloat16)[rows, cols].contiguous()
+
+
+def pack_ffn_bwd_weights(gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor) -> torch.Tensor:
+    """The three GatedMLP weights as the bfloat16 operand stream of ``ffn_bwd``: 16 chunks of 32 hidden
+    units, each ``[gate (8, 64, 8) | up (8, 64, 8) | down^T (8, 64, 8) | gate^T (4, 2, 64, 8) | up^T (4, 2, 64, 8)]``
+    with the index meaning given in ``include/bnb_amd.h``."""
+    D, Hd = FFN_WIDTH, FFN_HIDDEN
+    if gate_w.shape != (Hd, D) or up_w.shape != (Hd, D) or down_w.shape != (D, Hd):
+        raise ValueError("ffn_bwd covers d_model 128 with a hidden width of 512")
+    dev = gate_w.device
+    lane = torch.arange(64, device=dev)
+    m, b = lane % 32, lane // 32
+    pi = 16 * (m // 16) + 8 * ((m // 4) % 2) + 4 * ((m // 8) % 2) + m % 4  # unit that matrix-core row m stands for
+    e = torch.arange(8, device=dev)
+    c = torch.arange(Hd // 32, device=dev)
+    ks = torch.arange(8, device=dev)
+    # sections 0-2: (16, 8, 64, 8), rows = hidden unit, columns = channel
+    hid = (32 * c[:, None, None, None] + pi[None, None, :, None]).expand(-1, 8, -1, 8)
+    ch = (16 * ks[None, :, None, None] + 8 * b[None, None, :, None] + e[None, None, None, :]).expand(16, -1, -1, -1)
+    wg, wu, wd = (w.detach().to(torch.bfloat16) for w in (gate_w, up_w, down_w))
+    s0, s1, s2 = wg[hid, ch], wu[hid, ch], wd[ch, hid]
+    # sections 3-4: (16, 4, 2, 64, 8), contraction over the chunk's hidden units, rows = channel
+    cb = torch.arange(4, device=dev)
+    t = torch.arange(2, device=dev)
+    k_hid = (32 * c[:, None, None, None, None] + 16 * t[None, None, :, None, None] + 8 * b[None, None, None, :, None]
+             + e[None, None, None, None, :]).expand(-1, 4, -1, -1, -1)
+    r_ch = (32 * cb[None, :, None, None, None] + pi[None, None, None, :, None]).expand(16, -1, 2, -1, 8)
+    s3, s4 = wg[k_hid, r_ch], wu[k_hid, r_ch]
+    return torch.cat([x.reshape(16, -1) for x in (s0, s1, s2, s3, s4)], dim=1).contiguous()
+
+
+def ffn_bwd(n: torch.Tensor, dy: torch.Tensor, weights_packed: torch.Tensor):
+    """Backward of ``y = down(gelu(gate(n)) * up(n))`` with the gate/up activations recomputed on chip.
+
+    n (R, 128) bfloat16 contiguous, dy (R, 128) float32 or bfloat16, ``weights_packed`` from
+    ``pack_ffn_bwd_weights``.  Returns ``(dn, dgu, h, dy_bf16)``: dn (R, 128) bfloat16; ``dgu`` (8, Rp, 128) and
+    ``h`` (4, Rp, 128) bfloat16, the tile-by-tile operands of the weight gradients (see ``ffn_weight_grads``;
+    Rp is R rounded up to a multiple of 256, rows past R are don't-cares); dy rounded to bfloat16 (dy itself
+    when it already is)."""
+    D = FFN_WIDTH
+    _need_device(n, "n")
+    _need_device(dy, "dy")
+    if n.dim() != 2 or n.shape[1] != D or n.dtype != torch.bfloat16 or not n.is_contiguous():
+        raise ValueError("n must be a contiguous bfloat16 (R, 128) tensor")
+    if dy.shape != n.shape or dy.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("dy must be a float32 or bfloat16 tensor of n's shape")
+    if weights_packed.dtype != torch.bfloat16 or weights_packed.numel() != 5 * FFN_HIDDEN * D or not weights_packed.is_contiguous():
+        raise ValueError("weights_packed must come from pack_ffn_bwd_weights")
+    if not _uniform_rows(dy, D):
+        dy = dy.contiguous()
+    R = n.shape[0]
+    Rp = (R + 255) // 256 * 256
+    dev = n.device
+    dn = torch.empty((Rp, D), dtype=torch.bfloat16, device=dev)
+    dgu = torch.empty((8, Rp, 128), dtype=torch.bfloat16, device=dev)
+    h = torch.empty((4, Rp, 128), dtype=torch.bfloat16, device=dev)
+    dy_lp = torch.empty((Rp, D), dtype=torch.bfloat16, device=dev) if dy.dtype == torch.float32 else None
+    if R:
+        with _on_device(dev):
+            rc = _native.load().bnb_ffn_bwd(n.data_ptr(), dy.data_ptr(), _code(dy, "dy"), dy.stride(0), weights_packed.data_ptr(),
+                                            dn.data_ptr(), dgu.data_ptr(), h.data_ptr(),
+                                            None if dy_lp is None else dy_lp.data_ptr(), R, Rp, D, FFN_HIDDEN, _stream())
+        _native.check(rc, "bnb_ffn_bwd")
+    return dn[:R], dgu, h, (dy if dy_lp is None else dy_lp[:R])
+
+
+def ffn_weight_grads(n: torch.Tensor, dgu: torch.Tensor, h: torch.Tensor, dy_bf16: torch.Tensor):
+    """``(d gate_proj.weight, d up_proj.weight, d down_proj.weight)`` (float32) from ``ffn_bwd``'s operands."""
+    R = n.shape[0]
+    dw = _linear_wgrad_tiled(dgu, n, R).view(8, 2, 2, 32, FFN_WIDTH)  # [pair][chunk in pair][gate, up][unit][channel]
+    d_gate = dw[:, :, 0].reshape(FFN_HIDDEN, FFN_WIDTH)
+    d_up = dw[:, :, 1].reshape(FFN_HIDDEN, FFN_WIDTH)
+    return d_gate, d_up, _linear_wgrad_tiled(dy_bf16, h, R)
+
+
+class _FfnTailTrain(torch.autograd.Function):
+    """``s = x + delta; s + mlp(rmsnorm(s) * w)`` for the update path: forward on the fused sublayer-tail kernel
+    (which also writes ``s`` and the normalised rows), backward on ``ffn_bwd``, the weight-gradient kernel and the
+    norm's backward kernel.  Only ``s`` (float32) and the normalised rows (bfloat16) are kept between the two."""
+
+    @staticmethod
+    def forward(ctx, x, delta, norm_weight, gate_w, up_w, down_w, eps, packed_fwd, packed_bwd):
+        D = x.shape[-1]
+        x2 = x.reshape(-1, D)
+        if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) % 4):
+            x2 = x2.contiguous()
+        R = x2.shape[0]
+        dev = x.device
+        out = torch.empty((R, D), dtype=torch.float32, device=dev)
+        n = torch.empty((R, D), dtype=torch.bfloat16, device=dev)
+        s, d_ptr = None, None
+        if delta is not None:
+            delta2 = delta.reshape(-1, D).contiguous()
+            d_ptr = delta2.data_ptr()
+            s = torch.empty((R, D), dtype=torch.float32, device=dev)
+        nw = norm_weight.detach().contiguous()
+        if R:
+            with _on_device(dev):
+                rc = _native.load().bnb_ffn_fused_train_fwd(
+                    x2.data_ptr(), x2.stride(0), d_ptr, _native.BF16, nw.data_ptr(), float(eps), packed_fwd.data_ptr(),
+                    out.data_ptr(), None if s is None else s.data_ptr(), n.data_ptr(), R, D, FFN_HIDDEN, _stream())
+            _native.check(rc, "bnb_ffn_fused_train_fwd")
+        ctx.save_for_backward(x2 if s is None else s, n, nw, packed_bwd)
+        ctx.eps = eps
+        ctx.has_delta = delta is not None
+        ctx.shape = x.shape
+        return out.reshape(x.shape)
+
+    @staticmethod
+    @_outside_autocast
+    def backward(ctx, dout):
+        s, n, nw, packed_bwd = ctx.saved_tensors
+        D = s.shape[-1]
+        dout2 = dout.reshape(-1, D)
+        if dout2.dtype != torch.float32:
+            dout2 = dout2.float()
+        dout2 = dout2.contiguous()
+        dn, dgu, h, dy_lp = ffn_bwd(n, dout2, packed_bwd)
+        need_w = ctx.needs_input_grad[3] or ctx.needs_input_grad[4] or ctx.needs_input_grad[5]
+        d_gate = d_up = d_down = None
+        if need_w:
+            d_gate, d_up, d_down = ffn_weight_grads(n, dgu, h, dy_lp)
+        del dgu, h
+        if ctx.has_delta:
+            dx, dw, ddelta = rmsnorm_bwd(s, dn, nw, eps=ctx.eps, grad_sum=dout2, also_bf16=True)
+            ddelta = ddelta.reshape(ctx.shape)
+        else:
+            dx, dw = rmsnorm_bwd(s, dn, nw, eps=ctx.eps, grad_sum=dout2)
+            ddelta = None
+        return dx.reshape(ctx.shape), ddelta, dw, d_gate, d_up, d_down, None, None, None
+
+
+def ffn_tail_train_supported(x: torch.Tensor, delta: torch.Tensor | None, hidden: int) -> bool:
+    """Whether ``ffn_tail_train`` covers this sublayer tail: float32 (..., 128) residual stream on the GPU,
+    hidden width 512, ``delta`` bfloat16 of x's shape or absent."""
+    return ffn_supported(x, hidden) and (delta is None or (delta.dtype == torch.bfloat16 and delta.shape == x.shape))
+
+
+def ffn_tail_train(x, delta, norm_weight, gate_w, up_w, down_w, *, eps: float | None, packed_fwd: torch.Tensor,
+                   packed_bwd: torch.Tensor) -> torch.Tensor:
+    """Differentiable ``s = x + delta; s + down(gelu(gate(n)) * up(n))`` with ``n = rmsnorm(s) * norm_weight``, as
+    bfloat16 autocast computes it, without saving the 512/1024-wide activations (``packed_fwd`` from
+    ``pack_ffn_weights``, ``packed_bwd`` from ``pack_ffn_bwd_weights``, both of the current weights)."""
+    with torch.autocast("cuda", enabled=False):
+        return _FfnTailTrain.apply(x, delta, norm_weight, gate_w, up_w, down_w, _F32_EPS if eps is None else float(eps),
+                                   packed_fwd, packed_bwd)
 
 
 def _uniform_rows(t: torch.Tensor, D: int) -> bool:

@@ -359,6 +359,22 @@ class GatedMLP(_WeightCaches, nn.Module):
         proj = (delta, wp) if gate is None else (gate, delta, wp)
         return ops.ffn_fused(x, None, norm.weight, self.packed_weights(), eps=norm.eps, proj=proj)
 
+    def train_tail(self, x: torch.Tensor, delta: torch.Tensor | None, norm: nn.RMSNorm) -> torch.Tensor | None:
+        """``s = x + delta; s + self(norm(s))`` in grad mode under bfloat16 autocast as one kernel forward and one
+        matrix-core kernel backward that recomputes the 512/1024-wide activations instead of saving them
+        (plus the weight-gradient and norm-backward kernels); None when that does not apply."""
+        ws = (self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight)
+        if not (
+            _TRAIN_KERNELS and torch.is_grad_enabled() and _projection_dtype() == torch.bfloat16
+            and ops.ffn_tail_train_supported(x, delta, self.gate_proj.out_features)
+            and self.gate_proj.bias is None and self.up_proj.bias is None and self.down_proj.bias is None
+            and norm.weight is not None and norm.weight.dtype == torch.float32 and all(w.dtype == torch.float32 for w in ws)
+        ):
+            return None
+        packed_bwd = _cached_cast(self, "_bnb_ffn_bwd_pack", ws, torch.bfloat16, lambda: ops.pack_ffn_bwd_weights(*ws))
+        return ops.ffn_tail_train(x, delta, norm.weight, *ws, eps=norm.eps, packed_fwd=self.packed_weights(),
+                                  packed_bwd=packed_bwd)
+
     def tail_f32(self, x1: torch.Tensor, norm: nn.RMSNorm) -> torch.Tensor | None:
         """``x1 + self(norm(x1))`` in float32 as two kernels (norm + gate/up + gelu gate; down + residual), or None
         when that does not apply (other widths, biases)."""
@@ -416,7 +432,11 @@ class TransformerBlock(_WeightCaches, nn.Module):
         act = _projection_dtype()
         if not _fused_ok(x, act):
             x0, n1 = _train_norm(self.norm1, x)
-            x1, n2 = _train_norm(self.norm2, x0, self._attn(n1, alive_mask, bullets, bullet_mask))
+            attn = self._attn(n1, alive_mask, bullets, bullet_mask)
+            tail = self.ffn.train_tail(x0, attn, self.norm2)
+            if tail is not None:
+                return tail
+            x1, n2 = _train_norm(self.norm2, x0, attn)
             return x1 + self.ffn(n2)
         # norm + qkv (one kernel under bf16) -> attention kernel -> out_proj -> fused sublayer tail
         if act == torch.bfloat16 and self.d_model == ops.FFN_WIDTH and self.qkv.bias is None:
@@ -753,7 +773,11 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
                 return fused
             x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=r, eps=self.norm2.eps, out_dtype=act)
             return x1 + self.gated_mlp(n2)
-        x1, n2 = _train_norm(self.norm2, x, _project(self.linear_out, _gelu_gate(gate_in, y)))
+        r = _project(self.linear_out, _gelu_gate(gate_in, y))
+        tail = self.gated_mlp.train_tail(x, r, self.norm2)
+        if tail is not None:
+            return tail
+        x1, n2 = _train_norm(self.norm2, x, r)
         return x1 + self.gated_mlp(n2)
 
     def _step(self, x, h_in, conv_in, h_out, conv_out, reset, rows_per_env):

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 20
+#define BNB_ABI_VERSION 21
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -271,6 +271,14 @@ int bnb_linear_wgrad_slices(int64_t R, int N, int K);
 int bnb_linear_wgrad_fwd(const void *dy, int64_t dy_row_stride, const void *x, int64_t x_row_stride,
                          float *partials, int slices, float *dw, int accumulate,
                          int64_t R, int N, int K, void *stream);
+/*
+ * The same with operands that may be stored tile by tile: the 128 columns 128j .. 128j+127 of dy
+ * start dy_tile_stride elements after those of tile j-1 (128 = plain row-major rows; R * 128 with
+ * dy_row_stride 128 = a (N/128, R, 128) array), likewise x.  bnb_ffn_bwd writes such operands.
+ */
+int bnb_linear_wgrad_tiled_fwd(const void *dy, int64_t dy_row_stride, int64_t dy_tile_stride, const void *x,
+                               int64_t x_row_stride, int64_t x_tile_stride, float *partials, int slices, float *dw,
+                               int accumulate, int64_t R, int N, int K, void *stream);
 
 /*
  * Backward of bnb_sdpa_masked_fwd for small token counts: what autograd computes through
@@ -699,6 +707,49 @@ int bnb_mask_fill(const uint8_t *mask, const int32_t *offsets, int32_t *index, i
 int bnb_ffn_fused_fwd(const float *x, int64_t x_row_stride, const void *delta, int delta_dtype,
                       const float *norm_weight, float eps, const void *weights_packed, float *out,
                       int64_t R, int D, int hidden, void *stream);
+
+/*
+ * bnb_ffn_fused_fwd for the PPO update (train/rl/ppo.py:1417-1425 evaluating the trunk in grad mode):
+ * the same kernel also writes what the backward needs and the forward would otherwise not keep,
+ *   s_out  (R, 128) fp32 contiguous: s = x + delta (required with a delta; ignored without, where s is x)
+ *   n_out  (R, 128) bf16 contiguous: the normalised rows that entered gate_proj / up_proj
+ * so that none of the 512/1024-wide activations has to be saved (bnb_ffn_bwd recomputes them).
+ */
+int bnb_ffn_fused_train_fwd(const float *x, int64_t x_row_stride, const void *delta, int delta_dtype,
+                            const float *norm_weight, float eps, const void *weights_packed, float *out,
+                            float *s_out, void *n_out, int64_t R, int D, int hidden, void *stream);
+
+/*
+ * Backward of the gated MLP  y = Wd (gelu(Wg n) * (Wu n))  of models/yemong/attention.py:21-37 (what autograd
+ * runs through GatedMLP.forward under bf16 autocast) as one matrix-core kernel that recomputes the
+ * gate/up activations from n:
+ *     g, u = Wg n, Wu n;   dh = Wd^T dy;   h = bf16(gelu(g) u);
+ *     dg = bf16(dh u gelu'(g));  du = bf16(dh gelu(g));   dn = bf16(Wg^T dg + Wu^T du)
+ *
+ *   n    (R, 128) bf16 contiguous (bnb_ffn_fused_train_fwd's n_out)
+ *   dy   (R, 128) fp32 or bf16 (dy_dtype), rows dy_row_stride elements apart; used rounded to bf16
+ *   weights_packed  the three matrices in bf16 in the kernel's operand order, 16 chunks of 32 hidden
+ *        units, 40 KB each; with l = 0..63, m = l%32, b = l/32, e = 0..7,
+ *        pi(m) = 16(m/16) + 8((m/4)%2) + 4((m/8)%2) + m%4:
+ *          [c][0][ks][l][e] = Wg[32c + pi(m)][16ks + 8b + e]      ks = 0..7
+ *          [c][1][ks][l][e] = Wu[32c + pi(m)][16ks + 8b + e]
+ *          [c][2][ks][l][e] = Wd[16ks + 8b + e][32c + pi(m)]
+ *          [c][3][cb][t][l][e] = Wg[32c + 16t + 8b + e][32cb + pi(m)]   cb = 0..3, t = 0..1
+ *          [c][4][cb][t][l][e] = Wu[32c + 16t + 8b + e][32cb + pi(m)]
+ *   out_rows  rows that every result has room for: a multiple of 256, >= R.  The kernel stores whole
+ *        work-groups of 256 rows without a bounds test (rows R .. out_rows-1 receive don't-care values)
+ *   dn   (out_rows, 128) bf16 contiguous: gradient of n in rows 0 .. R-1
+ *   dgu  (8, out_rows, 128) bf16: tile p holds, for hidden chunks 2p and 2p+1 (32 units each),
+ *        [dg chunk 2p | du chunk 2p | dg chunk 2p+1 | du chunk 2p+1]
+ *   h    (4, out_rows, 128) bf16: tile q holds hidden units 128q .. 128q+127
+ *        (both are operands for bnb_linear_wgrad_tiled_fwd with tile stride out_rows * 128: dW(gate,up) =
+ *        dgu^T n in dgu's column order, dWd = dy^T h)
+ *   dy_bf16  optional (out_rows, 128) bf16 contiguous: dy rounded to bf16, when dy is fp32 (the other operand of dWd)
+ * Requirements: D == 128, hidden == 512 (else BNB_ERR_UNSUPPORTED), 16-byte aligned pointers.
+ */
+int bnb_ffn_bwd(const void *n, const void *dy, int dy_dtype, int64_t dy_row_stride, const void *weights_packed,
+                void *dn, void *dgu, void *h, void *dy_bf16, int64_t R, int64_t out_rows, int D, int hidden,
+                void *stream);
 
 /*
  * bnb_ffn_fused_fwd with the sublayer's output projection folded in: the tensor added to x

@@ -180,3 +180,29 @@ def test_token_split_has_the_gradient_of_plain_slicing(use):
     xr = x.clone().requires_grad_()
     loss(xr[:, :, :3], xr[:, :, 3:]).backward()
     assert torch.equal(xs.grad, xr.grad)
+
+
+def test_backward_weight_pack_follows_the_documented_operand_order():
+    # include/bnb_amd.h, bnb_ffn_bwd: sampled entries of the five sections against the index formulas written out
+    from boost_and_broadside_amd import ops
+
+    g = torch.Generator().manual_seed(3)
+    wg, wu, wd = torch.randn(512, 128, generator=g), torch.randn(512, 128, generator=g), torch.randn(128, 512, generator=g)
+    pk = ops.pack_ffn_bwd_weights(wg, wu, wd).view(16, 5, 4096).float()
+
+    def pi(m):
+        return 16 * (m // 16) + 8 * ((m // 4) % 2) + 4 * ((m // 8) % 2) + m % 4
+
+    assert sorted(pi(m) for m in range(32)) == list(range(32))
+    rnd = torch.randint(0, 1 << 30, (200, 5), generator=g).tolist()
+    for a, b_, c_, d, e_ in rnd:
+        c, ks, l, e = a % 16, b_ % 8, c_ % 64, d % 8
+        m, b = l % 32, l // 32
+        at = (ks * 64 + l) * 8 + e
+        assert pk[c, 0, at] == wg.bfloat16().float()[32 * c + pi(m), 16 * ks + 8 * b + e]
+        assert pk[c, 1, at] == wu.bfloat16().float()[32 * c + pi(m), 16 * ks + 8 * b + e]
+        assert pk[c, 2, at] == wd.bfloat16().float()[16 * ks + 8 * b + e, 32 * c + pi(m)]
+        cb, t = ks // 2, ks % 2
+        at = ((cb * 2 + t) * 64 + l) * 8 + e
+        assert pk[c, 3, at] == wg.bfloat16().float()[32 * c + 16 * t + 8 * b + e, 32 * cb + pi(m)]
+        assert pk[c, 4, at] == wu.bfloat16().float()[32 * c + 16 * t + 8 * b + e, 32 * cb + pi(m)]

@@ -6,6 +6,8 @@ alive-masking behaviour (dead keys weigh exactly nothing, an all-dead environmen
 mean of V, dead queries are computed).
 """
 
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -1020,6 +1022,119 @@ def test_ffn_fused_every_weight_reaches_its_output():
         want[k] = 3.0 * h
         assert torch.allclose(got[0], want, rtol=1e-2, atol=1e-6), (j, k)
         assert torch.equal(got[0], got[63])
+
+
+# ------------------------------------------------------------------ the gated MLP in the update: fused forward, recompute-backward
+
+
+def _ffn_bwd_reference(n, dy, p):
+    """float64 autograd through the oracle's gated MLP on the bf16-rounded operands the kernel sees."""
+    w = {k: v.bfloat16().double().requires_grad_() for k, v in p.items()}
+    nd = n.double().requires_grad_()
+    a = torch.nn.functional.linear(nd, w["f.gate_proj.weight"])
+    b = torch.nn.functional.linear(nd, w["f.up_proj.weight"])
+    a.retain_grad(), b.retain_grad()
+    hid = torch.nn.functional.gelu(a) * b
+    y = torch.nn.functional.linear(hid, w["f.down_proj.weight"])
+    assert torch.allclose(y, torch_ref.gated_mlp({k: v.detach() for k, v in w.items()}, "f.", nd.detach()), rtol=1e-12, atol=1e-12)
+    y.backward(dy.bfloat16().double())
+    return hid.detach(), a.grad, b.grad, nd.grad, w
+
+
+@pytest.mark.parametrize("R", [1, 31, 256, 257, 1000, 20000])
+@pytest.mark.parametrize("dy_dtype", [torch.float32, torch.bfloat16])
+def test_ffn_bwd_matches_autograd_of_the_oracle(R, dy_dtype):
+    _, _, _, p = _ffn_case(R + 3, R)
+    g = torch.Generator().manual_seed(R)
+    n = torch.randn(R, 128, generator=g).bfloat16()
+    dy = torch.randn(R, 128, generator=g).to(dy_dtype)
+    hid, da, db, dn_ref, w = _ffn_bwd_reference(n, dy.float(), p)
+    pk = ops.pack_ffn_bwd_weights(*(p[k].to(DEV) for k in ("f.gate_proj.weight", "f.up_proj.weight", "f.down_proj.weight")))
+    dn, dgu, h, dy_lp = ops.ffn_bwd(n.to(DEV), dy.to(DEV), pk)
+    assert dn.shape == (R, 128) and dn.dtype == torch.bfloat16 and dgu.shape[0] == 8 and h.shape[0] == 4
+    assert torch.equal(dy_lp.cpu(), dy.bfloat16())
+    h_rows = h[:, :R].permute(1, 0, 2).reshape(R, 512).float().cpu()
+    t = dgu[:, :R].permute(1, 0, 2).reshape(R, 8, 2, 2, 32).float().cpu()  # [row][pair][chunk in pair][gate, up][unit]
+    assert max_rel(h_rows, hid.float()) <= BF16_TOL
+    assert max_rel(t[:, :, :, 0].reshape(R, 512), da.float()) <= BF16_TOL
+    assert max_rel(t[:, :, :, 1].reshape(R, 512), db.float()) <= BF16_TOL
+    assert max_rel(dn.float().cpu(), dn_ref.float()) <= BF16_TOL
+    d_gate, d_up, d_down = ops.ffn_weight_grads(n.to(DEV), dgu, h, dy_lp)
+    assert max_rel(d_gate.cpu(), w["f.gate_proj.weight"].grad.float()) <= BF16_TOL
+    assert max_rel(d_up.cpu(), w["f.up_proj.weight"].grad.float()) <= BF16_TOL
+    assert max_rel(d_down.cpu(), w["f.down_proj.weight"].grad.float()) <= BF16_TOL
+    # fixed-order reductions: repeated calls give identical bits
+    again = ops.ffn_bwd(n.to(DEV), dy.to(DEV), pk)
+    assert torch.equal(again[0], dn) and torch.equal(again[1][:, :R], dgu[:, :R]) and torch.equal(again[2][:, :R], h[:, :R])
+
+
+def test_ffn_bwd_every_weight_reaches_its_gradient():
+    # one-hot weights: the packed operand order, the tile layout of the results and the weight-gradient un-permutation
+    # must each put hidden unit j and channel k where the layout says
+    D, Hd, R = 128, 512, 64
+    n = torch.zeros(R, D)
+    n[:, 5] = 1.5
+    dy = torch.zeros(R, D)
+    for j, k in [(0, 0), (37, 100), (511, 127), (300, 9), (140, 64)]:
+        wg, wu, wd = torch.zeros(Hd, D), torch.zeros(Hd, D), torch.zeros(D, Hd)
+        wg[j, 5], wu[j, 5], wd[k, j] = 1.0, 2.0, 3.0
+        dy.zero_()
+        dy[:, k] = 0.5
+        pk = ops.pack_ffn_bwd_weights(wg.to(DEV), wu.to(DEV), wd.to(DEV))
+        dn, dgu, h, dy_lp = ops.ffn_bwd(n.bfloat16().to(DEV), dy.to(DEV), pk)
+        a, b, dh = 1.5, 3.0, 1.5  # gate, up, gradient of the hidden unit
+        cdf = 0.5 * (1.0 + math.erf(a / 2 ** 0.5))
+        pdf = math.exp(-a * a / 2) / (2 * math.pi) ** 0.5
+        h_rows = h[:, :R].permute(1, 0, 2).reshape(R, Hd).float().cpu()
+        want_h = torch.zeros(Hd)
+        want_h[j] = a * cdf * b
+        assert torch.allclose(h_rows[0], want_h, rtol=1e-2, atol=1e-6), (j, k)
+        t = dgu[:, :R].permute(1, 0, 2).reshape(R, 8, 2, 2, 32).float().cpu()
+        want_g, want_u = torch.zeros(Hd), torch.zeros(Hd)
+        want_g[j], want_u[j] = dh * b * (cdf + a * pdf), dh * a * cdf
+        assert torch.allclose(t[0, :, :, 0].reshape(Hd), want_g, rtol=1e-2, atol=1e-6), (j, k)
+        assert torch.allclose(t[0, :, :, 1].reshape(Hd), want_u, rtol=1e-2, atol=1e-6), (j, k)
+        want_n = torch.zeros(D)
+        want_n[5] = float(want_g[j]) * 1.0 + float(want_u[j]) * 2.0
+        assert torch.allclose(dn[0].float().cpu(), want_n, rtol=2e-2, atol=1e-6), (j, k)
+        assert torch.equal(dn[0], dn[R - 1])
+        d_gate, d_up, d_down = ops.ffn_weight_grads(n.bfloat16().to(DEV), dgu, h, dy_lp)
+        hot = torch.zeros(Hd, D)
+        hot[j, 5] = 1.0
+        got_g = t[0, :, :, 0].reshape(Hd)[j].item()
+        assert torch.allclose(d_gate.cpu(), hot * (R * 1.5 * got_g), rtol=1e-2, atol=1e-5), (j, k)
+        assert d_down.cpu()[k, j] != 0 and d_down.cpu().count_nonzero() == 1, (j, k)
+
+
+@pytest.mark.parametrize("R", [1, 300, 5000])
+@pytest.mark.parametrize("with_delta", [True, False])
+def test_ffn_tail_train_matches_the_inference_kernel_and_autograd_of_the_oracle(R, with_delta):
+    x, delta, nw, p = _ffn_case(R + 11, R)
+    names = ("f.gate_proj.weight", "f.up_proj.weight", "f.down_proj.weight")
+    ws = [p[k].to(DEV).requires_grad_() for k in names]
+    pf, pb = ops.pack_ffn_weights(*ws), ops.pack_ffn_bwd_weights(*ws)
+    xg = x.to(DEV).requires_grad_()
+    dg = delta.to(DEV).requires_grad_() if with_delta else None
+    nwg = nw.to(DEV).requires_grad_()
+    out = ops.ffn_tail_train(xg, dg, nwg, *ws, eps=None, packed_fwd=pf, packed_bwd=pb)
+    with torch.no_grad():
+        assert torch.equal(out, ops.ffn_fused(x.to(DEV), delta.to(DEV) if with_delta else None, nw.to(DEV), pf))
+    g = torch.Generator().manual_seed(R + 1)
+    up = torch.randn(R, 128, generator=g)
+    out.backward(up.to(DEV))
+    # float64 autograd through the oracle on the bf16-rounded weights
+    wd = {k: p[k].bfloat16().double().requires_grad_() for k in names}
+    xd = x.double().requires_grad_()
+    dd = delta.double().requires_grad_()
+    nwd = nw.double().requires_grad_()
+    s = xd + dd if with_delta else xd
+    (s + torch_ref.gated_mlp(wd, "f.", torch_ref.rms_norm(s, nwd))).backward(up.double())
+    assert max_rel(xg.grad.cpu(), xd.grad.float()) <= BF16_TOL
+    if with_delta:
+        assert dg.grad.dtype == torch.bfloat16 and max_rel(dg.grad.float().cpu(), dd.grad.float()) <= BF16_TOL
+    assert max_rel(nwg.grad.cpu(), nwd.grad.float()) <= BF16_TOL
+    for w_, k in zip(ws, names):
+        assert max_rel(w_.grad.cpu(), wd[k].grad.float()) <= BF16_TOL, k
 
 
 # ------------------------------------------------------------------ rows addressed inside a wider (B, N+M, D) token tensor
