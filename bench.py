@@ -789,6 +789,26 @@ def main():
             dg = torch.randn(Rw, 4 * D, device=dev, generator=gen).to(torch.bfloat16)
             kern["gelu_mul_bwd"] = stream_leg(lambda t: ops.gelu_mul_bwd(ag, bg, dg), Rw * 4 * D * 2 * 5)
             del ag, bg, dg
+            # the gated MLP of the update: fused tail forward that keeps s and n, and the recompute-backward
+            # (n 256 B + dy 512 B in, dn 256 B + dy bf16 256 B + [dg | du] 2 KB + h 1 KB out per row; 2 * 2560 * 128 flops
+            # per row: gate/up again, dh, dn)
+            mlp_u = bnb.GatedMLP(D).to(dev)
+            ws_u = (mlp_u.gate_proj.weight, mlp_u.up_proj.weight, mlp_u.down_proj.weight)
+            pf_u, pb_u = ops.pack_ffn_weights(*ws_u), ops.pack_ffn_bwd_weights(*ws_u)
+            nn_u = torch.randn(Rw, D, device=dev, generator=gen).to(torch.bfloat16)
+            dy_u = torch.randn(Rw, D, device=dev, generator=gen)
+            kern["ffn_bwd"] = stream_leg(lambda t: ops.ffn_bwd(nn_u, dy_u, pb_u), Rw * (256 + 512 + 256 + 256 + 2048 + 1024))
+            kern["ffn_bwd"]["tflops"] = 2.0 * Rw * 2560 * D / (kern["ffn_bwd"]["us"] * 1e-6) / 1e12
+            xt_u = torch.randn(Rw, D, device=dev, generator=gen, requires_grad=True)
+            dl_u = torch.randn(Rw, D, device=dev, generator=gen).to(torch.bfloat16).requires_grad_()
+            nw_u = torch.ones(D, device=dev, requires_grad=True)
+
+            def tail_fwd(t):
+                with torch.enable_grad():
+                    ops.ffn_tail_train(xt_u, dl_u, nw_u, *ws_u, eps=None, packed_fwd=pf_u, packed_bwd=pb_u)
+
+            kern["ffn_tail_train_fwd"] = stream_leg(tail_fwd, Rw * (512 + 256 + 512 + 256 + 512))
+            del mlp_u, nn_u, dy_u, xt_u, dl_u
             Ba = Tu * Bu
             qa = torch.randn(Ba, Nu + Mu, 3 * D, device=dev, generator=gen).to(torch.bfloat16)
             aa = torch.rand(Ba, Nu + Mu, device=dev, generator=gen) < 0.9
@@ -834,7 +854,7 @@ def main():
                 "team_pool_fwd_bwd_library_ms": None if t_pool_up_lib is None else t_pool_up_lib * 1e3,
                 "block_fwd_bwd_library_ms": None if t_up_lib is None else t_up_lib * 1e3,
                 "what": "bnb_linear_wgrad_fwd (dW = dy^T x, bf16 in, fp32 out, rows split over the chip) beside the library "
-                        "GEMM on the same operands; kernels = the norm, gelu-gate, attention and conv backward kernels at the "
+                        "GEMM on the same operands; kernels = the norm, gelu-gate, gated-MLP, attention and conv backward kernels at the "
                         "sizes of the block below; block = one YemongBlock (2 attention + 1 temporal sublayer), T = 128 x 256 "
                         "environments of 4v4, forward + backward under bf16 autocast, on the update-path kernels and with "
                         "torch's own differentiable ops in their place (the recurrence keeps its kernels in both); block_with_bullets = "
