@@ -72,6 +72,7 @@ SIGNATURES = {
     "bnb_mask_fill": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "bnb_ffn_fused_fwd": (_i, [_vp, _i64, _vp, _i, _vp, _f, _vp, _vp, _i64, _i, _i, _vp]),
     "bnb_ffn_fused_train_fwd": (_i, [_vp, _i64, _vp, _i, _vp, _f, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp]),
+    "bnb_ffn_fused_proj_train_fwd": (_i, [_vp, _i64, _vp, _i64, _vp, _vp, _f, _vp, _vp, _vp, _vp, _i64, _i, _i, _vp]),
     "bnb_ffn_bwd": (_i, [_vp, _vp, _i, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i, _vp]),
     "bnb_ffn_fused_proj_fwd": (_i, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _f, _vp, _vp, _i64, _i, _i, _vp]),
     "bnb_gelu_mul_fwd": (_i, [_vp, _i, _i64, _vp, _i, _i64, _vp, _i, _i64, _i, _vp]),

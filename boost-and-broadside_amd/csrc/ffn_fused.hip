@@ -213,6 +213,25 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
             }
         }
     }
+    if (TRAIN && (MODE == kDeltaProj || MODE == kDeltaGate)) {
+        // s exists only in the accumulators here: out through the staging area as whole rows, like `out` at the end
+        __syncthreads();  // every wave is done reading Wp out of the weight buffers
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            const f32x16 &a = acc[ks >> 1];
+            const int v0 = 8 * (ks & 1);
+            float *sp = stage + m * kRowPitch + 16 * ks + 4 * half;
+            *reinterpret_cast<f32x4 *>(sp) = f32x4{a[v0], a[v0 + 1], a[v0 + 2], a[v0 + 3]};
+            *reinterpret_cast<f32x4 *>(sp + 8) = f32x4{a[v0 + 4], a[v0 + 5], a[v0 + 6], a[v0 + 7]};
+        }
+        wave_lds_handover();
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int64_t r = row0 + 2 * j + io_row;
+            const f32x4 sv = *reinterpret_cast<const f32x4 *>(stage + (2 * j + io_row) * kRowPitch + io_col);
+            if (r < R) __builtin_nontemporal_store(sv, reinterpret_cast<f32x4 *>(s_out + r * kFfnD + io_col));
+        }
+    }
 #pragma unroll
     for (int cb = 0; cb < 4; ++cb) {
 #pragma unroll
@@ -442,6 +461,23 @@ extern "C" int bnb_ffn_fused_train_fwd(const float *x, int64_t x_row_stride, con
                                             out, R, kFfnD, kFfnD, s, s_out, (uint16_t *)n_out);
     return launch_ffn<kDeltaNone, true>(x, x_row_stride, nullptr, nullptr, nullptr, norm_weight, eps, weights_packed,
                                         out, R, kFfnD, kFfnD, s, nullptr, (uint16_t *)n_out);
+}
+
+extern "C" int bnb_ffn_fused_proj_train_fwd(const float *x, int64_t x_row_stride, const void *rows_a, int64_t rows_a_stride,
+                                            const void *proj_packed, const float *norm_weight, float eps,
+                                            const void *weights_packed, float *out, float *s_out, void *n_out, int64_t R,
+                                            int D, int hidden, void *stream)
+{
+    using namespace bnb;
+    const int rc = ffn_common_checks(x, x_row_stride, norm_weight, weights_packed, out, R, D, hidden);
+    if (rc != 0 || R == 0) return rc;
+    if (!rows_a || !proj_packed || !s_out || !n_out) return BNB_ERR_NULL_POINTER;
+    if (rows_a_stride == 0) rows_a_stride = kFfnD;
+    if (rows_a_stride < kFfnD) return BNB_ERR_BAD_SHAPE;
+    if (!aligned16(rows_a) || rows_a_stride % 8 != 0 || !aligned16(proj_packed) || !aligned16(s_out) || !aligned16(n_out))
+        return BNB_ERR_MISALIGNED;
+    return launch_ffn<kDeltaProj, true>(x, x_row_stride, rows_a, nullptr, proj_packed, norm_weight, eps, weights_packed, out,
+                                        R, rows_a_stride, kFfnD, (hipStream_t)stream, s_out, (uint16_t *)n_out);
 }
 
 extern "C" int bnb_ffn_fused_proj_fwd(const float *x, int64_t x_row_stride, const void *rows_a, int64_t rows_a_stride,

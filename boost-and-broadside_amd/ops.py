@@ -1841,12 +1841,13 @@ def ffn_weight_grads(n: torch.Tensor, dgu: torch.Tensor, h: torch.Tensor, dy_bf1
 
 
 class _FfnTailTrain(torch.autograd.Function):
-    """``s = x + delta; s + mlp(rmsnorm(s) * w)`` for the update path: forward on the fused sublayer-tail kernel
-    (which also writes ``s`` and the normalised rows), backward on ``ffn_bwd``, the weight-gradient kernel and the
-    norm's backward kernel.  Only ``s`` (float32) and the normalised rows (bfloat16) are kept between the two."""
+    """``s = x + d; s + mlp(rmsnorm(s) * w)`` for the update path, with ``d`` = ``delta`` or, with a projection weight,
+    ``delta @ proj_w^T`` formed inside the kernel: forward on the fused sublayer-tail kernel (which also writes
+    ``s`` and the normalised rows), backward on ``ffn_bwd``, the weight-gradient kernel and the norm's backward
+    kernel.  Only ``s`` (float32), the normalised rows (bfloat16) and the projection's operand rows are kept."""
 
     @staticmethod
-    def forward(ctx, x, delta, norm_weight, gate_w, up_w, down_w, eps, packed_fwd, packed_bwd):
+    def forward(ctx, x, delta, proj_w, norm_weight, gate_w, up_w, down_w, eps, packed_fwd, packed_bwd, proj_packed):
         D = x.shape[-1]
         x2 = x.reshape(-1, D)
         if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) % 4):
@@ -1855,46 +1856,67 @@ class _FfnTailTrain(torch.autograd.Function):
         dev = x.device
         out = torch.empty((R, D), dtype=torch.float32, device=dev)
         n = torch.empty((R, D), dtype=torch.bfloat16, device=dev)
-        s, d_ptr = None, None
+        s, delta2 = None, None
         if delta is not None:
-            delta2 = delta.reshape(-1, D).contiguous()
-            d_ptr = delta2.data_ptr()
+            delta2 = delta.reshape(-1, D)
+            if proj_w is None or not _uniform_rows(delta2, D):
+                delta2 = delta2.contiguous()
             s = torch.empty((R, D), dtype=torch.float32, device=dev)
         nw = norm_weight.detach().contiguous()
         if R:
+            lib = _native.load()
             with _on_device(dev):
-                rc = _native.load().bnb_ffn_fused_train_fwd(
-                    x2.data_ptr(), x2.stride(0), d_ptr, _native.BF16, nw.data_ptr(), float(eps), packed_fwd.data_ptr(),
-                    out.data_ptr(), None if s is None else s.data_ptr(), n.data_ptr(), R, D, FFN_HIDDEN, _stream())
-            _native.check(rc, "bnb_ffn_fused_train_fwd")
-        ctx.save_for_backward(x2 if s is None else s, n, nw, packed_bwd)
+                if proj_w is None:
+                    rc = lib.bnb_ffn_fused_train_fwd(
+                        x2.data_ptr(), x2.stride(0), None if delta2 is None else delta2.data_ptr(), _native.BF16, nw.data_ptr(),
+                        float(eps), packed_fwd.data_ptr(), out.data_ptr(), None if s is None else s.data_ptr(), n.data_ptr(), R, D,
+                        FFN_HIDDEN, _stream())
+                else:
+                    rc = lib.bnb_ffn_fused_proj_train_fwd(
+                        x2.data_ptr(), x2.stride(0), delta2.data_ptr(), delta2.stride(0), proj_packed.data_ptr(), nw.data_ptr(),
+                        float(eps), packed_fwd.data_ptr(), out.data_ptr(), s.data_ptr(), n.data_ptr(), R, D, FFN_HIDDEN, _stream())
+            _native.check(rc, "bnb_ffn_fused_train_fwd" if proj_w is None else "bnb_ffn_fused_proj_train_fwd")
+        if proj_w is None:
+            ctx.save_for_backward(x2 if s is None else s, n, nw, packed_bwd)
+        else:
+            ctx.save_for_backward(s, n, nw, packed_bwd, delta2, proj_w)
         ctx.eps = eps
         ctx.has_delta = delta is not None
+        ctx.has_proj = proj_w is not None
         ctx.shape = x.shape
         return out.reshape(x.shape)
 
     @staticmethod
     @_outside_autocast
     def backward(ctx, dout):
-        s, n, nw, packed_bwd = ctx.saved_tensors
+        saved = ctx.saved_tensors  # read once: activation checkpointing unpacks on every access
+        s, n, nw, packed_bwd = saved[:4]
         D = s.shape[-1]
         dout2 = dout.reshape(-1, D)
         if dout2.dtype != torch.float32:
             dout2 = dout2.float()
         dout2 = dout2.contiguous()
         dn, dgu, h, dy_lp = ffn_bwd(n, dout2, packed_bwd)
-        need_w = ctx.needs_input_grad[3] or ctx.needs_input_grad[4] or ctx.needs_input_grad[5]
+        need_w = ctx.needs_input_grad[4] or ctx.needs_input_grad[5] or ctx.needs_input_grad[6]
         d_gate = d_up = d_down = None
         if need_w:
             d_gate, d_up, d_down = ffn_weight_grads(n, dgu, h, dy_lp)
         del dgu, h
+        ddelta = d_proj = None
         if ctx.has_delta:
-            dx, dw, ddelta = rmsnorm_bwd(s, dn, nw, eps=ctx.eps, grad_sum=dout2, also_bf16=True)
-            ddelta = ddelta.reshape(ctx.shape)
+            dx, dw, ds_lp = rmsnorm_bwd(s, dn, nw, eps=ctx.eps, grad_sum=dout2, also_bf16=True)
+            if ctx.has_proj:
+                # the projection's output gradient is the bfloat16 rounding of ds, as autograd hands it to a bf16 Linear
+                rows, proj_w = saved[4:]
+                if ctx.needs_input_grad[1]:
+                    ddelta = torch.matmul(ds_lp, proj_w.to(torch.bfloat16)).reshape(ctx.shape)
+                if ctx.needs_input_grad[2]:
+                    d_proj = linear_wgrad(ds_lp, rows)
+            else:
+                ddelta = ds_lp.reshape(ctx.shape)
         else:
             dx, dw = rmsnorm_bwd(s, dn, nw, eps=ctx.eps, grad_sum=dout2)
-            ddelta = None
-        return dx.reshape(ctx.shape), ddelta, dw, d_gate, d_up, d_down, None, None, None
+        return dx.reshape(ctx.shape), ddelta, d_proj, dw, d_gate, d_up, d_down, None, None, None, None
 
 
 def ffn_tail_train_supported(x: torch.Tensor, delta: torch.Tensor | None, hidden: int) -> bool:
@@ -1904,13 +1926,23 @@ def ffn_tail_train_supported(x: torch.Tensor, delta: torch.Tensor | None, hidden
 
 
 def ffn_tail_train(x, delta, norm_weight, gate_w, up_w, down_w, *, eps: float | None, packed_fwd: torch.Tensor,
-                   packed_bwd: torch.Tensor) -> torch.Tensor:
+                   packed_bwd: torch.Tensor, proj_weight: torch.Tensor | None = None,
+                   proj_packed: torch.Tensor | None = None) -> torch.Tensor:
     """Differentiable ``s = x + delta; s + down(gelu(gate(n)) * up(n))`` with ``n = rmsnorm(s) * norm_weight``, as
     bfloat16 autocast computes it, without saving the 512/1024-wide activations (``packed_fwd`` from
-    ``pack_ffn_weights``, ``packed_bwd`` from ``pack_ffn_bwd_weights``, both of the current weights)."""
+    ``pack_ffn_weights``, ``packed_bwd`` from ``pack_ffn_bwd_weights``, both of the current weights).
+
+    With ``proj_weight`` (128, 128) and its ``pack_proj_weights`` arrangement, ``delta`` is the operand of a bias-free
+    projection that runs inside the kernel: ``s = x + delta @ proj_weight^T`` (accumulated in float32 onto x, not
+    rounded to bfloat16 first)."""
+    if (proj_weight is None) != (proj_packed is None):
+        raise ValueError("give proj_weight and proj_packed together")
+    if proj_weight is not None and (delta is None or proj_weight.shape != (FFN_WIDTH, FFN_WIDTH) or proj_packed.dtype != torch.bfloat16
+                                    or proj_packed.numel() != FFN_WIDTH * FFN_WIDTH or not proj_packed.is_contiguous()):
+        raise ValueError("the folded projection needs its operand rows, a (128, 128) weight and pack_proj_weights' output")
     with torch.autocast("cuda", enabled=False):
-        return _FfnTailTrain.apply(x, delta, norm_weight, gate_w, up_w, down_w, _F32_EPS if eps is None else float(eps),
-                                   packed_fwd, packed_bwd)
+        return _FfnTailTrain.apply(x, delta, proj_weight, norm_weight, gate_w, up_w, down_w, _F32_EPS if eps is None else float(eps),
+                                   packed_fwd, packed_bwd, proj_packed)
 
 
 def _uniform_rows(t: torch.Tensor, D: int) -> bool:

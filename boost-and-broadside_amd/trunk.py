@@ -359,11 +359,16 @@ class GatedMLP(_WeightCaches, nn.Module):
         proj = (delta, wp) if gate is None else (gate, delta, wp)
         return ops.ffn_fused(x, None, norm.weight, self.packed_weights(), eps=norm.eps, proj=proj)
 
-    def train_tail(self, x: torch.Tensor, delta: torch.Tensor | None, norm: nn.RMSNorm) -> torch.Tensor | None:
+    def train_tail(self, x: torch.Tensor, delta: torch.Tensor | None, norm: nn.RMSNorm, *,
+                   proj_layer: nn.Linear | None = None) -> torch.Tensor | None:
         """``s = x + delta; s + self(norm(s))`` in grad mode under bfloat16 autocast as one kernel forward and one
         matrix-core kernel backward that recomputes the 512/1024-wide activations instead of saving them
-        (plus the weight-gradient and norm-backward kernels); None when that does not apply."""
+        (plus the weight-gradient and norm-backward kernels); None when that does not apply.  With ``proj_layer``
+        (a bias-free 128 x 128 Linear with float32 weights) ``s = x + proj_layer(delta)``, the projection inside the kernel."""
         ws = (self.gate_proj.weight, self.up_proj.weight, self.down_proj.weight)
+        if proj_layer is not None and (proj_layer.bias is not None or proj_layer.weight.dtype != torch.float32
+                                       or tuple(proj_layer.weight.shape) != (ops.FFN_WIDTH, ops.FFN_WIDTH)):
+            return None
         if not (
             _TRAIN_KERNELS and torch.is_grad_enabled() and _projection_dtype() == torch.bfloat16
             and ops.ffn_tail_train_supported(x, delta, self.gate_proj.out_features)
@@ -372,8 +377,13 @@ class GatedMLP(_WeightCaches, nn.Module):
         ):
             return None
         packed_bwd = _cached_cast(self, "_bnb_ffn_bwd_pack", ws, torch.bfloat16, lambda: ops.pack_ffn_bwd_weights(*ws))
+        if proj_layer is None:
+            return ops.ffn_tail_train(x, delta, norm.weight, *ws, eps=norm.eps, packed_fwd=self.packed_weights(),
+                                      packed_bwd=packed_bwd)
+        w = proj_layer.weight
+        wp = _cached_cast(proj_layer, "_bnb_proj_pack", (w,), torch.bfloat16, lambda: ops.pack_proj_weights(w))
         return ops.ffn_tail_train(x, delta, norm.weight, *ws, eps=norm.eps, packed_fwd=self.packed_weights(),
-                                  packed_bwd=packed_bwd)
+                                  packed_bwd=packed_bwd, proj_weight=w, proj_packed=wp)
 
     def tail_f32(self, x1: torch.Tensor, norm: nn.RMSNorm) -> torch.Tensor | None:
         """``x1 + self(norm(x1))`` in float32 as two kernels (norm + gate/up + gelu gate; down + residual), or None
@@ -432,7 +442,17 @@ class TransformerBlock(_WeightCaches, nn.Module):
         act = _projection_dtype()
         if not _fused_ok(x, act):
             x0, n1 = _train_norm(self.norm1, x)
-            attn = self._attn(n1, alive_mask, bullets, bullet_mask)
+            if torch.is_grad_enabled():
+                # out_proj inside the tail kernel, on the merged heads, when the tail kernel applies
+                merged = self._attn(n1, alive_mask, bullets, bullet_mask, project=False)
+                tail = None
+                if merged.dtype == torch.bfloat16:
+                    tail = self.ffn.train_tail(x0, merged, self.norm2, proj_layer=self.out_proj)
+                if tail is not None:
+                    return tail
+                attn = _project(self.out_proj, merged)
+            else:
+                attn = self._attn(n1, alive_mask, bullets, bullet_mask)
             tail = self.ffn.train_tail(x0, attn, self.norm2)
             if tail is not None:
                 return tail
@@ -476,7 +496,7 @@ class TransformerBlock(_WeightCaches, nn.Module):
 
     def _attn(self, x, alive_mask, bullets=None, bullet_mask=None, qkv=None, project=True):
         """Attention sublayer without the residual; ``project=False`` returns the merged heads
-        before ``out_proj`` (inference path only)."""
+        before ``out_proj``."""
         if qkv is None:
             qkv = _project(self.qkv, x)  # (B, N, 3D), fp32 or bf16 under autocast
         if torch.is_grad_enabled():
@@ -491,7 +511,7 @@ class TransformerBlock(_WeightCaches, nn.Module):
                 merged = self._self_attention_autograd(qkv, alive_mask)
             if self.reads_bullets and bullets is not None:
                 merged = merged + self._bullet_branch_autograd(qkv, bullets, bullet_mask)
-            return _project(self.out_proj, merged)
+            return _project(self.out_proj, merged) if project else merged
         try:
             merged = ops.sdpa_masked(qkv, alive_mask, self.n_heads)  # (B, N, D) head-major
         except _native.NativeLibraryError as err:
@@ -911,7 +931,11 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
                 return fused
             x1, n2 = ops.add_rmsnorm(x, self.norm2.weight, delta=r, eps=self.norm2.eps, out_dtype=act)
             return x1 + self.gated_mlp(n2)
-        x1, n2 = _train_norm(self.norm2, x, _project(self.linear_out, _gelu_gate(gate_in, b1)))
+        r = _project(self.linear_out, _gelu_gate(gate_in, b1))
+        tail = self.gated_mlp.train_tail(x, r, self.norm2)
+        if tail is not None:
+            return tail
+        x1, n2 = _train_norm(self.norm2, x, r)
         return x1 + self.gated_mlp(n2)
 
 

@@ -720,6 +720,17 @@ int bnb_ffn_fused_train_fwd(const float *x, int64_t x_row_stride, const void *de
                             float *s_out, void *n_out, int64_t R, int D, int hidden, void *stream);
 
 /*
+ * bnb_ffn_fused_train_fwd with the sublayer's output projection inside, as bnb_ffn_fused_proj_fwd has it
+ * (rows_b == NULL form): s = x + rows_a Wp^T is formed on the matrix cores and written to s_out; the
+ * projection's output never exists in memory.  For `x + out_proj(merged heads)` followed by the gated-MLP
+ * tail (models/yemong/attention.py:97-99,168-169) in the PPO update.
+ */
+int bnb_ffn_fused_proj_train_fwd(const float *x, int64_t x_row_stride, const void *rows_a, int64_t rows_a_stride,
+                                 const void *proj_packed, const float *norm_weight, float eps,
+                                 const void *weights_packed, float *out, float *s_out, void *n_out, int64_t R,
+                                 int D, int hidden, void *stream);
+
+/*
  * Backward of the gated MLP  y = Wd (gelu(Wg n) * (Wu n))  of models/yemong/attention.py:21-37 (what autograd
  * runs through GatedMLP.forward under bf16 autocast) as one matrix-core kernel that recomputes the
  * gate/up activations from n:

@@ -1137,6 +1137,35 @@ def test_ffn_tail_train_matches_the_inference_kernel_and_autograd_of_the_oracle(
         assert max_rel(w_.grad.cpu(), wd[k].grad.float()) <= BF16_TOL, k
 
 
+@pytest.mark.parametrize("R", [1, 300, 5000])
+def test_ffn_tail_train_with_the_output_projection_inside_matches_autograd_of_the_oracle(R):
+    x, _, nw, p = _ffn_case(R + 17, R)
+    g = torch.Generator().manual_seed(R + 2)
+    names = ("f.gate_proj.weight", "f.up_proj.weight", "f.down_proj.weight")
+    Wp = torch.randn(128, 128, generator=g) / 128 ** 0.5
+    rows = torch.randn(R, 128, generator=g).bfloat16()
+    ws = [p[k].to(DEV).requires_grad_() for k in names]
+    wp = Wp.to(DEV).requires_grad_()
+    pf, pb, pp = ops.pack_ffn_weights(*ws), ops.pack_ffn_bwd_weights(*ws), ops.pack_proj_weights(wp)
+    xg, rg, nwg = x.to(DEV).requires_grad_(), rows.to(DEV).requires_grad_(), nw.to(DEV).requires_grad_()
+    out = ops.ffn_tail_train(xg, rg, nwg, *ws, eps=None, packed_fwd=pf, packed_bwd=pb, proj_weight=wp, proj_packed=pp)
+    with torch.no_grad():
+        assert torch.equal(out, ops.ffn_fused(x.to(DEV), None, nw.to(DEV), pf, proj=(rows.to(DEV), pp)))
+    up = torch.randn(R, 128, generator=g)
+    out.backward(up.to(DEV))
+    wd = {k: p[k].bfloat16().double().requires_grad_() for k in names}
+    xd, rd, nwd = x.double().requires_grad_(), rows.double().requires_grad_(), nw.double().requires_grad_()
+    wpd = Wp.bfloat16().double().requires_grad_()
+    s = xd + rd @ wpd.t()
+    (s + torch_ref.gated_mlp(wd, "f.", torch_ref.rms_norm(s, nwd))).backward(up.double())
+    assert max_rel(xg.grad.cpu(), xd.grad.float()) <= BF16_TOL
+    assert rg.grad.dtype == torch.bfloat16 and max_rel(rg.grad.float().cpu(), rd.grad.float()) <= BF16_TOL
+    assert max_rel(wp.grad.cpu(), wpd.grad.float()) <= BF16_TOL
+    assert max_rel(nwg.grad.cpu(), nwd.grad.float()) <= BF16_TOL
+    for w_, k in zip(ws, names):
+        assert max_rel(w_.grad.cpu(), wd[k].grad.float()) <= BF16_TOL, k
+
+
 # ------------------------------------------------------------------ rows addressed inside a wider (B, N+M, D) token tensor
 
 
