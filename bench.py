@@ -398,6 +398,9 @@ def main():
             "bound": "hbm", "achieved": ab["step"] / (t_attn + t_rglru) / 1e9, "peak": peak / 1e9, "unit": "GB/s",
             "frac": ab["step"] / (t_attn + t_rglru) / peak, "algorithmic_bytes_per_step": ab["step"],
             "kernel_us_per_step": (t_attn + t_rglru) * 1e6, "median_kernel_us_per_step": (med_attn + med_rglru) * 1e6,
+            # the same bytes over the wall-clock step of the timed region above (what `value` and `ms_per_step` are from);
+            # the event figures carry the two event records per launch as well, which shows on launches of ~20 us
+            "wall_us_per_step": wall / steps * 1e6, "frac_by_wall_clock": ab["step"] / (wall / steps) / peak,
         },
         "kernels": roofs,
     }
