@@ -61,6 +61,19 @@ def _projection_dtype() -> torch.dtype:
     return torch.float32
 
 
+def _widen_tokens(x: torch.Tensor) -> tuple[torch.Tensor, bool]:
+    """``(tokens for the kernels, whether they were widened)``.
+
+    Under bfloat16 autocast the reference's encoder ends in ``Linear -> RMSNorm`` (models/yemong/encoder.py:82-101),
+    which hands the trunk bfloat16 tokens, and its residual stream then stays bfloat16.  The kernels carry the
+    residual stream in float32 (every sublayer adds its bfloat16 output onto float32 rows), so such tokens are
+    widened once on entry and the result is rounded back to bfloat16 once on exit: the same function with fewer
+    roundings in between, instead of torch's library composition for a bfloat16 stream."""
+    if x.dtype == torch.bfloat16 and x.is_cuda and _projection_dtype() == torch.bfloat16:
+        return x.float(), True
+    return x, False
+
+
 def _fused_ok(x: torch.Tensor, act: torch.dtype) -> bool:
     """Whether the fused norm / gelu kernels apply: fp32 residual stream on the GPU, a covered
     width, fp32 or bf16 projections.  Anything else takes the plain torch composition."""
@@ -1072,6 +1085,10 @@ class YemongBlock(_WeightCaches, nn.Module):
         """
         B, NM, D = x.shape
         n_rec = NM if num_recurrent is None else num_recurrent
+        x, widened = _widen_tokens(x)
+        if widened:
+            out, new_h, new_cb = self.step(x, alive, h, conv_buf, num_recurrent, bullets, bullet_mask)
+            return out.to(torch.bfloat16), new_h, new_cb
         for layer in self.spatial:
             x = layer(x, alive, bullets, bullet_mask)
         new_h, new_cb = [], []
@@ -1097,6 +1114,9 @@ class YemongBlock(_WeightCaches, nn.Module):
         """
         B, NM, D = x.shape
         n_rec = num_recurrent
+        x, widened = _widen_tokens(x)
+        if widened:
+            return self.step_packed(x, alive, state_in, state_out, num_recurrent, reset, bullets, bullet_mask).to(torch.bfloat16)
         for layer in self.spatial:
             x = layer(x, alive, bullets, bullet_mask)
         act = _projection_dtype()
@@ -1121,6 +1141,10 @@ class YemongBlock(_WeightCaches, nn.Module):
         input-gradient GEMMs stay with the library."""
         T, B, NM, D = x.shape
         n_rec = NM if num_recurrent is None else num_recurrent
+        x, widened = _widen_tokens(x)
+        if widened:
+            out, new_h, new_cb = self.sequence(x, alive_mask, h0, conv_buf0, done_mask, num_recurrent, bullets, bullet_mask)
+            return out.to(torch.bfloat16), new_h, new_cb
         for layer in self.spatial:
             x = layer(x.reshape(T * B, NM, D), alive_mask.reshape(T * B, NM), bullets, bullet_mask)
             x = x.reshape(T, B, NM, D)
@@ -1198,6 +1222,10 @@ class YemongTrunk(_WeightCaches, nn.Module):
         recomputes each block in the backward pass instead of keeping its activations, as the
         reference's ``grad_checkpoint`` option does."""
         T, B, NM, D = x.shape
+        x, widened = _widen_tokens(x)
+        if widened:
+            return self.sequence(x, alive_mask, initial_hidden, done_mask, bullets, bullet_mask,
+                                 grad_checkpoint=grad_checkpoint).to(torch.bfloat16)
         n_layers, rows = initial_hidden.shape[0], initial_hidden.shape[1]
         if n_layers != self.n_hidden_layers or rows % B:
             raise ValueError(f"initial_hidden must be ({self.n_hidden_layers}, B*n_rec, {CONV_KERNEL * D})")
@@ -1257,12 +1285,12 @@ class YemongTrunk(_WeightCaches, nn.Module):
             and D // self.config.n_heads == 32 and NM <= 160
         ):
             bullet_rows = ops.CompactRows(bullet_mask)
-        x = tokens
+        x, widened = _widen_tokens(tokens)
         for i, block in enumerate(self.yemong_layers):
             sl = slice(i * n_t, (i + 1) * n_t)
             x = block.step_packed(x, alive_mask, recurrent_state[sl], out_state[sl], n_rec, reset_mask, bullets,
                                   bullet_rows)
-        return x, out_state
+        return (x.to(torch.bfloat16) if widened else x), out_state
 
 
 class GraphedTrunk:

@@ -1056,3 +1056,115 @@ def test_out_state_overlapping_the_input_state_at_an_offset_is_refused():
     apart = big[2 * rows: 4 * rows].view(2, rows, 4 * D)
     _, new_state = trunk(x, alive, state, out_state=apart)  # adjacent but disjoint: fine
     assert new_state.data_ptr() == apart.data_ptr()
+
+
+def test_a_policy_around_the_trunk_runs_under_torch_compile():
+    """The reference wraps its policies in torch.compile (train/rl/ppo.py:396-400, policy_io.py:354-358).  The
+    kernels are reached through ctypes, which the tracer cannot follow: it must break the graph there, run the
+    trunk as it is and give the eager result, for the rollout step and for the update (gradients included).
+    The encoder ends in Linear -> RMSNorm as the reference's does (encoder.py:82-101), so under autocast the trunk
+    is handed bfloat16 tokens."""
+    import torch._dynamo
+
+    from boost_and_broadside_amd import trunk as trunk_module
+
+    cfg = _cfg(128, 4, blocks=2, spatial=2, temporal=1)
+    torch.manual_seed(21)
+    trunk = bnb.YemongTrunk(cfg).to(DEV)
+
+    class Policy(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.enc = torch.nn.Sequential(torch.nn.Linear(20, 128), torch.nn.RMSNorm(128))
+            self.trunk = trunk
+            self.head = torch.nn.Linear(128, 6)
+
+        def forward(self, obs, alive, state):  # rollout step
+            hidden, new_state = self.trunk(self.enc(obs), alive, state)
+            return self.head(hidden), new_state
+
+    class Evaluate(torch.nn.Module):  # the update's re-evaluation of a stored rollout
+        def __init__(self, policy):
+            super().__init__()
+            self.policy = policy
+
+        def forward(self, obs_seq, alive_seq, state, done):
+            return self.policy.head(self.policy.trunk.sequence(self.policy.enc(obs_seq), alive_seq, state, done))
+
+    policy = Policy().to(DEV)
+    B, N, M, T = 24, 8, 4, 6
+    g = torch.Generator().manual_seed(22)
+    obs = torch.randn(T, B, N + M, 20, generator=g).to(DEV)
+    alive = (torch.rand(T, B, N + M, generator=g) < 0.8).to(DEV)
+    alive[..., N:] = True
+    done = (torch.rand(T, B, generator=g) < 0.1).to(DEV)
+    state = trunk.initial_hidden(B, N, DEV)
+    torch._dynamo.reset()
+    compiled = torch.compile(policy, backend="aot_eager")
+    evaluate = Evaluate(policy)
+    compiled_evaluate = torch.compile(evaluate, backend="aot_eager")
+    try:
+        with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16), trunk_module.forbid_library_dispatch():
+            want = policy(obs[0], alive[0], state)
+            got = compiled(obs[0], alive[0], state)
+            again = compiled(obs[0], alive[0], state)
+        for a, b, c in zip(want, got, again):
+            assert torch.equal(a, b) and torch.equal(a, c)
+
+        def grads(fn):
+            policy.zero_grad(set_to_none=True)
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                logits = fn(obs, alive, state, done)
+            logits.float().square().mean().backward()
+            return [q.grad.clone() for q in policy.parameters()]
+
+        for a, b in zip(grads(evaluate), grads(compiled_evaluate)):
+            assert torch.isfinite(b).all() and max_rel(b.float().cpu(), a.float().cpu()) <= BF16_TOL
+    finally:
+        torch._dynamo.reset()
+
+
+@pytest.mark.parametrize("bullets", [0, 1])
+def test_bfloat16_tokens_under_autocast_run_on_the_kernels_and_match_the_oracle(bullets):
+    """Linear -> RMSNorm at the end of the reference's encoder (encoder.py:82-101) emits bfloat16 under bf16 autocast,
+    so that is what the trunk is handed there.  The tokens are widened on entry, every sublayer runs on the kernels
+    (no library dispatch) and the result comes back in bfloat16, within the bf16 bar of the oracle's float32 evaluation
+    of the same (already rounded) tokens."""
+    from boost_and_broadside_amd import trunk as trunk_module
+
+    D, H, B, N, M = 128, 4, 12, 8, 4
+    p = trunk_params(33, D, 2, 2, 1)
+    if bullets:
+        pg = torch.Generator().manual_seed(35)
+        for i in range(2):
+            p[f"yemong_layers.{i}.spatial.0.norm_bullet.weight"] = 1.0 + 0.1 * torch.randn(D, generator=pg)
+            p[f"yemong_layers.{i}.spatial.0.kv_bullet.weight"] = 0.15 * torch.randn(2 * D, D, generator=pg)
+    trunk = bnb.YemongTrunk(_cfg(D, H, 2, 2, 1, bullets=bullets)).eval()
+    trunk.load_state_dict(p)
+    trunk.to(DEV)
+    gen = torch.Generator().manual_seed(34)
+    hidden, ref_hidden = trunk.initial_hidden(B, N, DEV), torch.zeros(2, B * N, 4 * D)
+    alive = torch.ones(B, N + M, dtype=torch.bool)
+    for t in range(3):
+        x = torch.randn(B, N + M, D, generator=gen).bfloat16()
+        alive[:, :N] &= torch.rand(B, N, generator=gen) > 0.1
+        kw, ref_kw = {}, {}
+        if bullets:
+            bul = torch.randn(B, 10 * N, D, generator=gen)
+            bm = torch.rand(B, 10 * N, generator=gen) < 0.3
+            kw = {"bullets": bul.to(DEV), "bullet_mask": bm.to(DEV)}
+            ref_kw = {"bullets": bul, "bullet_mask": bm}
+        with torch.autocast("cuda", dtype=torch.bfloat16), trunk_module.forbid_library_dispatch():
+            out, hidden = trunk(x.to(DEV), alive.to(DEV), hidden, **kw)
+        assert out.dtype == torch.bfloat16 and hidden.dtype == torch.float32
+        ref_out, ref_hidden = torch_ref.trunk_step(p, 2, 2, 1, H, x.float(), alive, ref_hidden, **ref_kw)
+        assert max_rel(out.float().cpu(), ref_out) <= BF16_TOL, t
+        assert max_rel(hidden.cpu(), ref_hidden) <= BF16_TOL, t
+    # the update's re-evaluation takes the same tokens, differentiably
+    xs = torch.randn(4, B, N + M, D, generator=gen).bfloat16().to(DEV).requires_grad_()
+    al = torch.ones(4, B, N + M, dtype=torch.bool, device=DEV)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        seq = trunk.sequence(xs, al, trunk.initial_hidden(B, N, DEV))
+    assert seq.dtype == torch.bfloat16
+    seq.float().square().mean().backward()
+    assert xs.grad.dtype == torch.bfloat16 and torch.isfinite(xs.grad).all() and xs.grad.abs().max() > 0
