@@ -1001,6 +1001,9 @@ class TeamPMA(_WeightCaches, nn.Module):
 
     def pooled(self, x: torch.Tensor, team_id: torch.Tensor, alive: torch.Tensor) -> torch.Tensor:
         """(B, 2, D) pooled team vectors without the broadcast back to the ships."""
+        x, widened = _widen_tokens(x)
+        if widened:
+            return self.pooled(x, team_id, alive).to(torch.bfloat16)
         if not torch.is_grad_enabled() and ops.team_pool_supported(x, self.n_heads):
             return ops.team_pool(x, team_id, alive, *self._folded(), self.norm.weight, self.norm.eps, self.n_heads,
                                  broadcast=False)[1]
@@ -1018,6 +1021,9 @@ class TeamPMA(_WeightCaches, nn.Module):
         return self.norm(out).to(x.dtype)
 
     def forward(self, x: torch.Tensor, team_id: torch.Tensor, alive: torch.Tensor) -> torch.Tensor:
+        x, widened = _widen_tokens(x)
+        if widened:  # a bfloat16 stream under autocast: the kernels read float32 rows, the result is rounded back
+            return self.forward(x, team_id, alive).to(torch.bfloat16)
         if ops.team_pool_supported(x, self.n_heads):
             if not torch.is_grad_enabled():
                 return ops.team_pool(x, team_id, alive, *self._folded(), self.norm.weight, self.norm.eps, self.n_heads)[0]

@@ -1168,3 +1168,28 @@ def test_bfloat16_tokens_under_autocast_run_on_the_kernels_and_match_the_oracle(
     assert seq.dtype == torch.bfloat16
     seq.float().square().mean().backward()
     assert xs.grad.dtype == torch.bfloat16 and torch.isfinite(xs.grad).all() and xs.grad.abs().max() > 0
+
+
+def test_team_pooling_takes_a_bfloat16_stream_under_autocast_on_the_kernels():
+    from boost_and_broadside_amd import trunk as trunk_module
+
+    D, H, B, N = 128, 4, 40, 8
+    torch.manual_seed(41)
+    layer = bnb.TeamPMA(D, H).to(DEV)
+    with torch.no_grad():
+        layer.seeds.normal_(0.0, 0.02)
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(B, N, D, generator=g).bfloat16().to(DEV)
+    team = torch.randint(0, 2, (B, N), generator=g, dtype=torch.int32).to(DEV)
+    alive = (torch.rand(B, N, generator=g) < 0.8).to(DEV)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        with trunk_module.forbid_library_dispatch():
+            got = layer(x, team, alive)
+            pooled = layer.pooled(x, team, alive)
+        want = layer(x.float(), team, alive)
+    assert got.dtype == torch.bfloat16 and pooled.dtype == torch.bfloat16
+    assert torch.equal(got, want.to(torch.bfloat16))
+    xg = x.clone().requires_grad_()
+    with torch.autocast("cuda", dtype=torch.bfloat16), trunk_module.forbid_library_dispatch():
+        layer(xg, team, alive).float().square().mean().backward()
+    assert xg.grad.dtype == torch.bfloat16 and torch.isfinite(xg.grad).all()
