@@ -823,6 +823,11 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
         const int key0 = wave * J * 64 + lane;
         uint32_t bits = 0;
         int mine = 0;
+        // without a mask every slot is a key: the scan reads a byte that is never zero (a branch on the pointer
+        // between the loads would make the compiler wait for each load inside its own branch, one round trip per byte)
+        static __device__ const uint8_t kAllAlive[1] = {1};
+        const uint8_t *alive_src = alive_env != nullptr ? alive_env : kAllAlive;
+        const int alive_last = alive_env != nullptr ? NK - 1 : 0;
         for (int j0 = 0; j0 < J; j0 += 8) {
             // eight independent byte loads in flight, then their ballots
             uint32_t a[8];
@@ -830,8 +835,7 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
             for (int u = 0; u < 8; ++u) {
                 const int key = key0 + (j0 + u) * 64;
                 const bool in = j0 + u < J && key < NK;
-                a[u] = 1u;
-                if (alive_env != nullptr) a[u] = alive_env[key < NK ? key : NK - 1];  // branch-free: no wait between the loads
+                a[u] = alive_src[key < alive_last ? key : alive_last];
                 a[u] = in ? a[u] : 0u;
             }
 #pragma unroll
