@@ -12,9 +12,10 @@ import os
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "_lib", "libbnb_amd.so")
 
-ABI_VERSION = 21
+ABI_VERSION = 22
 F32, BF16 = 0, 1
 PATH_AUTO, PATH_VALU, PATH_MFMA, PATH_ENV, PATH_HEAD = 0, 1, 2, 3, 4
+WGRAD_PATH_AUTO, WGRAD_PATH_STAGED, WGRAD_PATH_DMA = 0, 1, 2
 
 _vp, _i, _i64, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
 
@@ -36,6 +37,7 @@ SIGNATURES = {
     ),
     "bnb_conv_step_rows_fwd": (_i, [_vp, _i, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _vp]),
     "bnb_linear_wgrad_slices": (_i, [_i64, _i, _i]),
+    "bnb_linear_wgrad_path": (_i, [_i]),
     "bnb_linear_wgrad_fwd": (_i, [_vp, _i64, _vp, _i64, _vp, _i, _vp, _i, _i64, _i, _i, _vp]),
     "bnb_linear_wgrad_tiled_fwd": (_i, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i, _vp, _i, _i64, _i, _i, _vp]),
     "bnb_conv_seq_bwd_blocks": (_i, [_i64, _i, _i]),

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 21
+#define BNB_ABI_VERSION 22
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -268,6 +268,13 @@ int bnb_conv_step_rows_fwd(const void *b1, int b1_dtype, int64_t b1_group_stride
  * Requirements: N % 128 == 0, K % 128 == 0, 16-byte aligned pointers, strides multiples of 8.
  */
 int bnb_linear_wgrad_slices(int64_t R, int N, int K);
+/* Which kernel computes the product, for tests and benchmarks: AUTO = DMA (operand rows global -> LDS directly,
+ * transposed by the LDS read); STAGED = through registers with a transpose in registers.  Changes what
+ * bnb_linear_wgrad_slices returns: set it before sizing the workspace. */
+#define BNB_WGRAD_PATH_AUTO 0
+#define BNB_WGRAD_PATH_STAGED 1
+#define BNB_WGRAD_PATH_DMA 2
+int bnb_linear_wgrad_path(int path);
 int bnb_linear_wgrad_fwd(const void *dy, int64_t dy_row_stride, const void *x, int64_t x_row_stride,
                          float *partials, int slices, float *dw, int accumulate,
                          int64_t R, int N, int K, void *stream);

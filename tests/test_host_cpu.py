@@ -45,6 +45,8 @@ def test_header_constants_match_loader():
     assert int(consts["BNB_ERR_UNSUPPORTED"]) == _native.ERR_UNSUPPORTED
     assert (int(consts["BNB_F32"]), int(consts["BNB_BF16"])) == (_native.F32, _native.BF16)
     assert [int(consts[f"BNB_SDPA_PATH_{n}"]) for n in ("AUTO", "VALU", "MFMA")] == [0, 1, 2]
+    assert [int(consts[f"BNB_WGRAD_PATH_{n}"]) for n in ("AUTO", "STAGED", "DMA")] == [
+        _native.WGRAD_PATH_AUTO, _native.WGRAD_PATH_STAGED, _native.WGRAD_PATH_DMA]
 
 
 def test_ops_refuse_host_tensors_and_bad_arguments():

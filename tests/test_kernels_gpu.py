@@ -1667,9 +1667,21 @@ def _wgrad_case(seed, R, N, K):
     return torch.randn(R, N, generator=g).bfloat16(), torch.randn(R, K, generator=g).bfloat16()
 
 
-@pytest.mark.parametrize("R", [0, 1, 63, 64, 65, 1000, 20011, 140000])
+@pytest.fixture(params=["dma", "staged"])
+def wgrad_path(request):
+    """Both kernels behind bnb_linear_wgrad_fwd: operand rows global -> LDS directly with the transposing LDS
+    read (the default), and through registers with the transpose in registers."""
+    from boost_and_broadside_amd import _native
+
+    lib = _native.load()
+    assert lib.bnb_linear_wgrad_path(_native.WGRAD_PATH_DMA if request.param == "dma" else _native.WGRAD_PATH_STAGED) == 0
+    yield request.param
+    assert lib.bnb_linear_wgrad_path(_native.WGRAD_PATH_AUTO) == 0
+
+
+@pytest.mark.parametrize("R", [0, 1, 31, 33, 63, 64, 65, 1000, 20011, 140000])
 @pytest.mark.parametrize("N,K", [(128, 128), (384, 128), (128, 512), (256, 256)])
-def test_linear_wgrad_matches_float64_product(R, N, K):
+def test_linear_wgrad_matches_float64_product(R, N, K, wgrad_path):
     """dW = dy^T x is fixed by the mathematics: the float64 product of the same bf16 operands is the truth
     (what nn.Linear's backward, reference models/yemong/attention.py:60-74, computes for its weight)."""
     if R == 140000 and (N, K) != (128, 128):
