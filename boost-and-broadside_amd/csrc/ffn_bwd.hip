@@ -20,7 +20,7 @@
 // a lane holds one row's column of every result, so dG^T and dU^T go from the accumulators straight
 // into the B operands of the last product.  The weights (640 KB bf16 in this arrangement) stream
 // through LDS in 16 chunks of 32 hidden units (40 KB) with two buffers; the next chunk travels
-// from L2 through registers while the current one is used; one barrier per chunk.  One work-group of
+// from L2 straight into LDS while the current one is used; one barrier per chunk.  One work-group of
 // eight waves per CU (80 KB of LDS, 256 registers per lane).
 //
 // Which hidden unit an MFMA row stands for is free, and chosen so that stores are dense without a
@@ -141,8 +141,22 @@ __global__ __launch_bounds__(kFbThreads) void ffn_bwd_kernel(
 
     __syncthreads();  // every wave has its rows out of the staging area
     stash(0);
-    fetch(1);
     __syncthreads();
+
+    // from here on a chunk travels global -> LDS directly (global_load_lds_dwordx4: a wave moves 1 KB per
+    // instruction, lane l filling bytes 16 l .. 16 l + 15 of its kilobyte): no registers, no LDS store instructions
+    const uint32_t lds_w = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)&s_w[0][0];
+    constexpr int kDmaPerWave = kFbChunkHalfs / 512 / kFbWaves;  // 1 KB pieces per wave and chunk: 5
+    auto dma_chunk = [&](int c, int buf) {
+        const uint16_t *src = wpack + (int64_t)c * kFbChunkHalfs + wave * (kDmaPerWave * 512);  // wave-uniform
+        const uint32_t dst = lds_w + (uint32_t)(buf * kFbChunkHalfs * 2 + wave * (kDmaPerWave * 1024));
+#pragma unroll
+        for (int q = 0; q < kDmaPerWave; ++q)
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
+                         :
+                         : "s"(src + q * 512), "v"((uint32_t)(lane * 16)), "s"(dst + (uint32_t)(q * 1024))
+                         : "memory");
+    };
 
     f32x16 acc[4];
 #pragma unroll
@@ -168,6 +182,8 @@ __global__ __launch_bounds__(kFbThreads) void ffn_bwd_kernel(
 
 #pragma unroll 1
     for (int c = 0; c < kFfnChunks; ++c) {
+        // chunk c + 1 into the buffer that chunk c - 1 was read from (everyone is past the barrier that ended it)
+        if (c + 1 < kFfnChunks) dma_chunk(c + 1, (c + 1) & 1);
         const uint16_t *wb = s_w[c & 1] + lane * 8;
         f32x16 g, u, dh;
 #pragma unroll
@@ -225,9 +241,9 @@ __global__ __launch_bounds__(kFbThreads) void ffn_bwd_kernel(
             __builtin_nontemporal_store(gw[1], reinterpret_cast<u32x4 *>(gp + 16 * 128));
             __builtin_nontemporal_store(uw[1], reinterpret_cast<u32x4 *>(gp + 16 * 128 + 32));
         }
-        // chunk c + 1 into the buffer that chunk c - 1 was read from (everyone is past the barrier that ended it)
-        if (c + 1 < kFfnChunks) stash((c + 1) & 1);
-        if (c + 2 < kFfnChunks) fetch(c + 2);
+        // this wave's part of chunk c + 1 has landed when at most the six stores above (issued after it) are
+        // outstanding: vmcnt counts loads and stores in issue order
+        __builtin_amdgcn_s_waitcnt(0x0f76);  // vmcnt(6)
         __syncthreads();
     }
 

@@ -20,8 +20,9 @@
 // out^T, so `s` is simply the initial accumulator, and with the channel order chosen in the
 // pack the same registers are the B operand of the first GEMM after normalisation.
 // The weights (384 KB bf16) stream through LDS in 16 chunks of 32 hidden units (24 KB) with
-// three buffers: chunk c+2 travels from L2 through registers into LDS while the down projection
-// of chunk c and the gate/up products of chunk c+1 are formed; one barrier per chunk.
+// three buffers: chunk c+2 travels from L2 straight into LDS (global_load_lds_dwordx4, no registers and
+// no LDS store instructions) while the down projection of chunk c and the gate/up products of chunk c+1
+// are formed; one barrier per chunk.
 //
 // Channel order: k-slot e of contraction step ks in a lane of half h stands for channel
 //   ch(ks, h, e) = 16ks + 8(e/4) + 4h + e%4
@@ -91,18 +92,19 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
 #pragma unroll
         for (int q = 0; q < kFfnPrefetch; ++q) dst[tid + q * kFfnThreads] = src[q];
     };
-    // inside the loop a chunk comes in as two halves, so that only half of it occupies registers
-    constexpr int kHalfPre = kFfnPrefetch / 2;
-    u32x4 hp[kHalfPre];
-    auto fetch_half = [&](int c, int part) {
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(wpack + (int64_t)c * kFfnChunkHalfs);
+    // inside the loop a chunk travels global -> LDS directly (global_load_lds_dwordx4: a wave moves 1 KB per
+    // instruction, lane l filling bytes 16 l .. 16 l + 15 of its kilobyte): no registers, no LDS store instructions
+    const uint32_t lds_w = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)&s_w[0][0];
+    constexpr int kDmaPerWave = kFfnChunkHalfs / 512 / kFfnWaves;  // 1 KB pieces per wave and chunk: 6
+    auto dma_chunk = [&](int c, int buf) {
+        const uint16_t *src = wpack + (int64_t)c * kFfnChunkHalfs + wave * (kDmaPerWave * 512);  // wave-uniform
+        const uint32_t dst = lds_w + (uint32_t)(buf * kFfnChunkHalfs * 2 + wave * (kDmaPerWave * 1024));
 #pragma unroll
-        for (int q = 0; q < kHalfPre; ++q) hp[q] = src[tid + (part * kHalfPre + q) * kFfnThreads];
-    };
-    auto stash_half = [&](int buf, int part) {
-        u32x4 *dst = reinterpret_cast<u32x4 *>(s_w[buf]);
-#pragma unroll
-        for (int q = 0; q < kHalfPre; ++q) dst[tid + (part * kHalfPre + q) * kFfnThreads] = hp[q];
+        for (int q = 0; q < kDmaPerWave; ++q)
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
+                         :
+                         : "s"(src + q * 512), "v"((uint32_t)(lane * 16)), "s"(dst + (uint32_t)(q * 1024))
+                         : "memory");
     };
     // Every work-group takes the same time, so the two that share a CU would move in lockstep for
     // the whole launch: both reading rows, then both on the matrix cores, then both writing,
@@ -301,7 +303,7 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
         constexpr bool FETCH = decltype(fetch_tag)::value, NEXT = decltype(next_tag)::value;
         const int buf1 = buf == 2 ? 0 : buf + 1;
         const int buf2 = buf1 == 2 ? 0 : buf1 + 1;
-        if (FETCH) fetch_half(c + 2, 0);
+        if (FETCH) dma_chunk(c + 2, buf2);  // the buffer chunk c - 1 was read from: everyone is past the barrier that ended it
         const uint16_t *wgu = s_w[buf1] + lane * 8;
         const uint16_t *wd = s_w[buf] + lane * 8 + 8192;
         bf16x8 hb[2];
@@ -336,10 +338,6 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
             }
             a0 = n0;
             a1 = n1;
-            if (FETCH && ks == 3) {
-                stash_half(buf2, 0);
-                fetch_half(c + 2, 1);
-            }
         }
         // operand (cb, t) sits at index 2cb + t; blocks 0 and 1 are in, 2 and 3 follow while those MFMAs run
 #pragma unroll
@@ -351,7 +349,7 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
                 acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ad[cb * 2 + t]), hb[t],
                                                                   acc[cb], 0, 0, 0);
         }
-        if (FETCH) stash_half(buf2, 1);
+        if (FETCH) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of chunk c + 2 is in LDS
         __syncthreads();
     };
     using yes = std::integral_constant<bool, true>;
