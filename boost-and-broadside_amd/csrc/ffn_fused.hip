@@ -135,7 +135,7 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
                 const Row8 y = load8_stream(rows_b + rs * rows_b_stride + a_col);
                 float p[8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) p[e] = round_to_bf16(gelu_erf(g.v[e])) * y.v[e];
+                for (int e = 0; e < 8; ++e) p[e] = round_to_bf16(gelu_phi(g.v[e])) * y.v[e];  // 2.6e-5 from erf-GELU, far below the bf16 rounding that follows
                 av = u32x4{pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
                            pack_bf16x2(p[6], p[7])};
             }
