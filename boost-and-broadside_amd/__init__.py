@@ -27,6 +27,7 @@ from .trunk import (
     YemongBlock,
     YemongTrunk,
     forbid_library_dispatch,
+    separate_heads,
     invalidate_weight_caches,
     library_dispatches,
 )
@@ -34,5 +35,5 @@ from .trunk import (
 __all__ = [
     "CONV_KERNEL", "GatedMLP", "GraphedTrunk", "GriffinTemporalBlock", "ModelConfig", "RGLRU", "TeamPMA", "TransformerBlock",
     "YemongBlock", "YemongTrunk", "conv_seq", "conv_step", "rglru_scan", "rglru_step", "sdpa_cross", "sdpa_masked", "ops",
-    "trunk", "harness", "LibraryDispatchWarning", "forbid_library_dispatch", "invalidate_weight_caches", "library_dispatches",
+    "trunk", "harness", "LibraryDispatchWarning", "forbid_library_dispatch", "separate_heads", "invalidate_weight_caches", "library_dispatches",
 ]

@@ -63,12 +63,23 @@ constexpr int kProjPitch = kFfnD + 8;  // halfs per staged operand row (bank spr
 
 // TRAIN: the update path's forward.  It also writes what the backward needs and nothing else saves: the
 // residual sum `s` (when there is a delta; otherwise s is x) and the normalised rows `n` in bf16.
-template <int MODE, bool TRAIN = false>
+// HEAD: the kernel goes on to the head of the NEXT sublayer, which is a norm and a projection of the rows it has
+// just produced (`qkv(norm1(x))` of models/yemong/attention.py:94-96,132, `[linear1 | linear2](norm1(x))` of
+// griffin.py:269-283): head = bf16(rmsnorm(out) * next_norm_w) Wh^T, N_h features (a multiple of 64), written
+// as bf16 rows.  The rows never come back from memory for it, and one launch with its own row I/O disappears.
+// Wh streams through the same three weight buffers as chunks 16, 17, ... of the pipeline, 64 features (16 KB) at
+// a time: [c][b][ks][l][e] = Wh[64c + 32b + pi(l%32)][16ks + 8(e/4) + 4(l/32) + e%4] with
+// pi(m) = 16(m/16) + 8((m/4)%2) + 4((m/8)%2) + m%4, the row order that leaves a lane with two runs of eight
+// consecutive features, which lanes m and m + 16 trade (v_permlane16_swap) so that a store instruction writes whole
+// 64-byte pieces of 16 rows.  The stores are unconditional: next_out has room for whole work-groups of 128 rows.
+template <int MODE, bool TRAIN = false, bool HEAD = false>
 __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void ffn_fused_kernel(
     const float *__restrict__ x, int64_t x_stride, const uint16_t *__restrict__ delta,
     const uint16_t *__restrict__ rows_b, const uint16_t *__restrict__ wproj, const float *__restrict__ norm_w,
     float eps, const uint16_t *__restrict__ wpack, float *__restrict__ out, int64_t R, int64_t rows_a_stride, int64_t rows_b_stride, unsigned first_round,
-    float *__restrict__ s_out = nullptr, uint16_t *__restrict__ n_out = nullptr)
+    float *__restrict__ s_out = nullptr, uint16_t *__restrict__ n_out = nullptr, const float *__restrict__ next_norm_w = nullptr,
+    float next_eps = 0.0f, const uint16_t *__restrict__ next_wpack = nullptr, uint16_t *__restrict__ next_out = nullptr,
+    int next_features = 0)
 {
     constexpr bool HAS_DELTA = MODE == kDeltaRows;
     // three weight buffers: chunk c is used while chunk c+1 is already complete (its operands
@@ -101,6 +112,18 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
         const uint32_t dst = lds_w + (uint32_t)(buf * kFfnChunkHalfs * 2 + wave * (kDmaPerWave * 1024));
 #pragma unroll
         for (int q = 0; q < kDmaPerWave; ++q)
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
+                         :
+                         : "s"(src + q * 512), "v"((uint32_t)(lane * 16)), "s"(dst + (uint32_t)(q * 1024))
+                         : "memory");
+    };
+    // a chunk of the next sublayer's head: 64 features = 16 KB, four 1 KB pieces per wave, into the front of a buffer
+    constexpr int kHeadChunkHalfs = 64 * kFfnD;
+    auto dma_head = [&](int hc, int buf) {
+        const uint16_t *src = next_wpack + (int64_t)hc * kHeadChunkHalfs + wave * (4 * 512);  // wave-uniform
+        const uint32_t dst = lds_w + (uint32_t)(buf * kFfnChunkHalfs * 2 + wave * (4 * 1024));
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
             asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
                          :
                          : "s"(src + q * 512), "v"((uint32_t)(lane * 16)), "s"(dst + (uint32_t)(q * 1024))
@@ -303,7 +326,10 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
         constexpr bool FETCH = decltype(fetch_tag)::value, NEXT = decltype(next_tag)::value;
         const int buf1 = buf == 2 ? 0 : buf + 1;
         const int buf2 = buf1 == 2 ? 0 : buf1 + 1;
-        if (FETCH) dma_chunk(c + 2, buf2);  // the buffer chunk c - 1 was read from: everyone is past the barrier that ended it
+        if (FETCH) {  // into the buffer chunk c - 1 was read from: everyone is past the barrier that ended it
+            if (!HEAD || c + 2 < kFfnChunks) dma_chunk(c + 2, buf2);
+            else dma_head(c + 2 - kFfnChunks, buf2);  // the pipeline goes on with the head's weights
+        }
         const uint16_t *wgu = s_w[buf1] + lane * 8;
         const uint16_t *wd = s_w[buf] + lane * 8 + 8192;
         bf16x8 hb[2];
@@ -361,9 +387,70 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
         step(yes{}, yes{}, c + 1, buf, gB, uB, gA, uA);
         buf = buf == 2 ? 0 : buf + 1;
     }
-    step(no{}, yes{}, kFfnChunks - 2, buf, gA, uA, gB, uB);
+    using more = std::integral_constant<bool, HEAD>;
+    step(more{}, yes{}, kFfnChunks - 2, buf, gA, uA, gB, uB);
     buf = buf == 2 ? 0 : buf + 1;
-    step(no{}, no{}, kFfnChunks - 1, buf, gB, uB, gA, uA);
+    step(more{}, no{}, kFfnChunks - 1, buf, gB, uB, gA, uA);
+
+    if constexpr (HEAD) {
+        // ---- head of the next sublayer: n2 = rmsnorm(out) as B operand, as n was formed from s above ----
+        float ss2 = 0.0f;
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) ss2 = fmaf(acc[cb][v], acc[cb][v], ss2);
+        }
+        ss2 += __shfl_xor(ss2, 32);
+        const float rstd2 = rsqrtf(ss2 * (1.0f / kFfnD) + next_eps);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            const f32x4 wl = *reinterpret_cast<const f32x4 *>(next_norm_w + 16 * ks + 4 * half);
+            const f32x4 wh = *reinterpret_cast<const f32x4 *>(next_norm_w + 16 * ks + 8 + 4 * half);
+            const float wv[8] = {wl.x, wl.y, wl.z, wl.w, wh.x, wh.y, wh.z, wh.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) nb[ks][e] = (__bf16)((acc[ks >> 1][8 * (ks & 1) + e] * rstd2) * wv[e]);
+        }
+        const int nhc = next_features >> 6;
+        const int64_t out_row = row0 + (m & 15);
+        for (int hc = 0; hc < nhc; ++hc) {
+            buf = buf == 2 ? 0 : buf + 1;  // buffer of pipeline chunk 16 + hc
+            const int buf1 = buf == 2 ? 0 : buf + 1;
+            const int buf2 = buf1 == 2 ? 0 : buf1 + 1;
+            if (hc + 2 < nhc) dma_head(hc + 2, buf2);
+            const uint16_t *wb = s_w[buf] + lane * 8;
+            f32x16 z0 = {0.0f}, z1 = {0.0f};
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                const bf16x8 a0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(wb + ks * 512));
+                const bf16x8 a1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(wb + 4096 + ks * 512));
+                z0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, nb[ks], z0, 0, 0, 0);
+                z1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, nb[ks], z1, 0, 0, 0);
+            }
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const f32x16 &z = b ? z1 : z0;
+                // registers 0..7: features 8 half .. + 7 of the block, registers 8..15: 16 + 8 half ..
+                u32x4 w[2];
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    w[t] = u32x4{pack_bf16x2(z[8 * t], z[8 * t + 1]), pack_bf16x2(z[8 * t + 2], z[8 * t + 3]),
+                                 pack_bf16x2(z[8 * t + 4], z[8 * t + 5]), pack_bf16x2(z[8 * t + 6], z[8 * t + 7])};
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const u32x2 t = __builtin_amdgcn_permlane16_swap(w[0][q], w[1][q], false, false);
+                    w[0][q] = t.x, w[1][q] = t.y;
+                }
+                // w[0]: row m % 16, w[1]: row 16 + m % 16; features 16 (m / 16) + 8 half .. + 7 of the block
+                uint16_t *p = next_out + out_row * next_features + hc * 64 + 32 * b + 16 * (m >> 4) + 8 * half;
+                *reinterpret_cast<u32x4 *>(p) = w[0];
+                *reinterpret_cast<u32x4 *>(p + 16 * (int64_t)next_features) = w[1];
+            }
+            // this wave's part of head chunk hc + 2 has landed when at most the four stores above (issued after
+            // it) are outstanding: vmcnt counts loads and stores in issue order
+            __builtin_amdgcn_s_waitcnt(0x0f74);  // vmcnt(4)
+            __syncthreads();
+        }
+    }
 
     // ---- out: back through the staging area (the loop's last barrier has freed the weight
     //      buffers) so that rows leave as whole 512-byte runs ----
@@ -388,11 +475,19 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
 
 namespace bnb {
 
-template <int MODE, bool TRAIN = false>
+struct NextHead {
+    const float *norm_weight = nullptr;
+    float eps = 0.0f;
+    const void *packed = nullptr;
+    void *out = nullptr;
+    int features = 0;
+};
+
+template <int MODE, bool TRAIN = false, bool HEAD = false>
 static int launch_ffn(const float *x, int64_t x_stride, const void *rows_a, const void *rows_b, const void *wproj,
                       const float *norm_weight, float eps, const void *weights_packed, float *out, int64_t R,
                       int64_t rows_a_stride, int64_t rows_b_stride, hipStream_t s, float *s_out = nullptr,
-                      uint16_t *n_out = nullptr)
+                      uint16_t *n_out = nullptr, NextHead next = NextHead())
 {
     const int64_t blocks = (R + kFfnWaves * 32 - 1) / (kFfnWaves * 32);
     if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
@@ -405,9 +500,10 @@ static int launch_ffn(const float *x, int64_t x_stride, const void *rows_a, cons
             cus = 256;
         first_round = 2u * (unsigned)cus;
     }
-    hipLaunchKernelGGL((ffn_fused_kernel<MODE, TRAIN>), dim3((unsigned)blocks), dim3(kFfnThreads), 0, s, x, x_stride,
+    hipLaunchKernelGGL((ffn_fused_kernel<MODE, TRAIN, HEAD>), dim3((unsigned)blocks), dim3(kFfnThreads), 0, s, x, x_stride,
                        (const uint16_t *)rows_a, (const uint16_t *)rows_b, (const uint16_t *)wproj, norm_weight, eps,
-                       (const uint16_t *)weights_packed, out, R, rows_a_stride, rows_b_stride, first_round, s_out, n_out);
+                       (const uint16_t *)weights_packed, out, R, rows_a_stride, rows_b_stride, first_round, s_out, n_out,
+                       next.norm_weight, next.eps, (const uint16_t *)next.packed, (uint16_t *)next.out, next.features);
     return (int)hipGetLastError();
 }
 
@@ -459,6 +555,37 @@ extern "C" int bnb_ffn_fused_train_fwd(const float *x, int64_t x_row_stride, con
                                             out, R, kFfnD, kFfnD, s, s_out, (uint16_t *)n_out);
     return launch_ffn<kDeltaNone, true>(x, x_row_stride, nullptr, nullptr, nullptr, norm_weight, eps, weights_packed,
                                         out, R, kFfnD, kFfnD, s, nullptr, (uint16_t *)n_out);
+}
+
+extern "C" int bnb_ffn_fused_proj_next_fwd(const float *x, int64_t x_row_stride, const void *rows_a, int64_t rows_a_stride,
+                                           const void *rows_b, int64_t rows_b_stride, const void *proj_packed,
+                                           const float *norm_weight, float eps, const void *weights_packed, float *out,
+                                           const float *next_norm_weight, float next_eps, const void *next_packed,
+                                           void *next_out, int next_features, int64_t next_out_rows, int64_t R, int D,
+                                           int hidden, void *stream)
+{
+    using namespace bnb;
+    const int rc = ffn_common_checks(x, x_row_stride, norm_weight, weights_packed, out, R, D, hidden);
+    if (rc != 0 || R == 0) return rc;
+    if (!rows_a || !proj_packed || !next_norm_weight || !next_packed || !next_out) return BNB_ERR_NULL_POINTER;
+    if (rows_a_stride == 0) rows_a_stride = kFfnD;
+    if (rows_b_stride == 0) rows_b_stride = kFfnD;
+    if (rows_a_stride < kFfnD || rows_b_stride < kFfnD) return BNB_ERR_BAD_SHAPE;
+    // the head's stores are unconditional: room for every row of every work-group
+    if (next_features < 128 || next_features % 64 != 0 || next_out_rows < (R + kFfnWaves * 32 - 1) / (kFfnWaves * 32) * (kFfnWaves * 32))
+        return BNB_ERR_BAD_SHAPE;
+    if (!aligned16(rows_a) || rows_a_stride % 8 != 0 || !aligned16(proj_packed) ||
+        (rows_b && (!aligned16(rows_b) || rows_b_stride % 8 != 0)) || !aligned16(next_norm_weight) || !aligned16(next_packed) ||
+        !aligned16(next_out))
+        return BNB_ERR_MISALIGNED;
+    NextHead next;
+    next.norm_weight = next_norm_weight, next.eps = next_eps, next.packed = next_packed, next.out = next_out, next.features = next_features;
+    hipStream_t s = (hipStream_t)stream;
+    if (rows_b)
+        return launch_ffn<kDeltaGate, false, true>(x, x_row_stride, rows_a, rows_b, proj_packed, norm_weight, eps, weights_packed,
+                                                   out, R, rows_a_stride, rows_b_stride, s, nullptr, nullptr, next);
+    return launch_ffn<kDeltaProj, false, true>(x, x_row_stride, rows_a, nullptr, proj_packed, norm_weight, eps, weights_packed, out,
+                                               R, rows_a_stride, kFfnD, s, nullptr, nullptr, next);
 }
 
 extern "C" int bnb_ffn_fused_proj_train_fwd(const float *x, int64_t x_row_stride, const void *rows_a, int64_t rows_a_stride,

@@ -1767,6 +1767,27 @@ def pack_proj_weights(weight: torch.Tensor) -> torch.Tensor:
     return weight.detach().to(torch.bfloat16)[rows, cols].contiguous()
 
 
+def pack_head_weights(weight: torch.Tensor) -> torch.Tensor:
+    """A (N, 128) projection weight (N a multiple of 64, at least 128) as the bfloat16 operand stream of the
+    next-sublayer head folded into ``ffn_fused``: chunks of 64 features,
+    ``[c][b][ks][l][e] = W[64c + 32b + pi(l%32)][16ks + 8(e/4) + 4(l/32) + e%4]`` with
+    ``pi(m) = 16(m/16) + 8((m/4)%2) + 4((m/8)%2) + m%4``."""
+    N, D = weight.shape
+    if D != FFN_WIDTH or N % 64 or N < 128:
+        raise ValueError("the folded head covers (N, 128) weights with N a multiple of 64, at least 128")
+    dev = weight.device
+    lane = torch.arange(64, device=dev)
+    m, half = lane % 32, lane // 32
+    pi = 16 * (m // 16) + 8 * ((m // 4) % 2) + 4 * ((m // 8) % 2) + m % 4
+    e = torch.arange(8, device=dev)
+    blk = torch.arange(N // 32, device=dev)
+    ks = torch.arange(8, device=dev)
+    rows = (32 * blk[:, None, None, None] + pi[None, None, :, None]).expand(-1, 8, -1, 8)
+    cols = (16 * ks[None, :, None, None] + 8 * (e // 4)[None, None, None, :] + 4 * half[None, None, :, None]
+            + (e % 4)[None, None, None, :]).expand(N // 32, -1, -1, -1)
+    return weight.detach().to(torch.bfloat16)[rows, cols].contiguous()
+
+
 def pack_ffn_bwd_weights(gate_w: torch.Tensor, up_w: torch.Tensor, down_w: torch.Tensor) -> torch.Tensor:
     """The three GatedMLP weights as the bfloat16 operand stream of ``ffn_bwd``: 16 chunks of 32 hidden
     units, each ``[gate (8, 64, 8) | up (8, 64, 8) | down^T (8, 64, 8) | gate^T (4, 2, 64, 8) | up^T (4, 2, 64, 8)]``
@@ -1971,7 +1992,8 @@ def ffn_fused(
     eps: float | None = None,
     out: torch.Tensor | None = None,
     proj: tuple | None = None,
-) -> torch.Tensor:
+    next_head: tuple | None = None,
+):
     """``s = x + delta; s + down(gelu(gate(n)) * up(n))`` with ``n = rmsnorm(s) * norm_weight``,
     one matrix-core kernel with bfloat16 projections (what the sublayer tail computes under
     bfloat16 autocast).
@@ -1983,8 +2005,14 @@ def ffn_fused(
     ``(rows, wp)`` adds ``rows @ W^T``, ``(rows_g, rows_y, wp)`` adds
     ``(gelu(rows_g) * rows_y) @ W^T``; rows are bfloat16 with x's shape, ``wp`` from
     ``pack_proj_weights``.
+
+    ``next_head = (next_norm_weight, next_eps, packed, N)`` (only with ``proj``) makes the same launch go on to
+    the head of the next sublayer, ``bf16(rmsnorm(out) * next_norm_weight) @ Wh^T`` with ``packed`` from
+    ``pack_head_weights`` (N features); the call then returns ``(out, head)`` with head (..., N) bfloat16.
     """
     D = x.shape[-1]
+    if next_head is not None and proj is None:
+        raise ValueError("next_head needs the folded projection form (proj=...)")
     if not ffn_supported(x, FFN_HIDDEN):
         raise RuntimeError("ffn_fused covers float32 (..., 128) residual streams on the GPU")
     _need_device(x, "x")
@@ -2022,6 +2050,25 @@ def ffn_fused(
             if torch.is_grad_enabled() and t.requires_grad:
                 raise RuntimeError("ffn_fused is forward-only; call it under torch.no_grad()")
             flat.append(t.view(-1, D) if _uniform_rows(t, D) else t.reshape(-1, D).contiguous())
+        if next_head is not None:
+            nw2, eps2, hp, N2 = next_head
+            if (nw2.shape != (D,) or nw2.dtype != torch.float32 or hp.dtype != torch.bfloat16 or hp.numel() != N2 * D
+                    or not hp.is_contiguous() or N2 % 64 or N2 < 128):
+                raise ValueError("next_head must be (float32 (128,) norm weight, eps, pack_head_weights output, N)")
+            Rp = (R + 127) // 128 * 128  # the head's stores are unconditional: room for whole work-groups
+            head = torch.empty((Rp, N2), dtype=torch.bfloat16, device=x.device)
+            if R:
+                with _on_device(x.device):
+                    rc = _native.load().bnb_ffn_fused_proj_next_fwd(
+                        x2.data_ptr(), x2.stride(0), flat[0].data_ptr(), flat[0].stride(0),
+                        flat[1].data_ptr() if len(flat) == 2 else None, flat[1].stride(0) if len(flat) == 2 else 0,
+                        wp.data_ptr(), norm_weight.data_ptr(), float(_F32_EPS if eps is None else eps),
+                        weights_packed.data_ptr(), out.data_ptr(), nw2.detach().contiguous().data_ptr(),
+                        float(_F32_EPS if eps2 is None else eps2), hp.data_ptr(), head.data_ptr(), N2, Rp, R, D, FFN_HIDDEN,
+                        _stream(),
+                    )
+                _native.check(rc, "bnb_ffn_fused_proj_next_fwd")
+            return out.reshape(x.shape), head[:R].reshape(*x.shape[:-1], N2)
         if R:
             with _on_device(x.device):
                 rc = _native.load().bnb_ffn_fused_proj_fwd(

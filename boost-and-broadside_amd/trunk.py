@@ -99,6 +99,21 @@ def _packed_f32(layer: nn.Module, slot: str, *weights: torch.Tensor) -> torch.Te
     return _cached_cast(layer, slot, weights, torch.float32, lambda: ops.pack_linear_f32(*weights))
 
 
+_HEAD_FUSION = True  # the sublayer tail also forms the next sublayer's norm + projection (bf16 inference, width 128)
+
+
+@contextlib.contextmanager
+def separate_heads():
+    """Inside the block every sublayer forms its own norm + projection (one more launch per sublayer) instead of
+    receiving it from the tail kernel of the sublayer before.  For comparisons."""
+    global _HEAD_FUSION
+    keep, _HEAD_FUSION = _HEAD_FUSION, False
+    try:
+        yield
+    finally:
+        _HEAD_FUSION = keep
+
+
 _TRAIN_KERNELS = True  # grad-mode norms, gates, conv, attention and weight gradients on the library's own kernels when False
 
 
@@ -353,12 +368,14 @@ class GatedMLP(_WeightCaches, nn.Module):
             and ops.ffn_supported(x, self.gate_proj.out_features)
         )
 
-    def fused_tail(self, x, delta, norm: nn.RMSNorm, *, proj_layer: nn.Linear | None = None, gate=None):
+    def fused_tail(self, x, delta, norm: nn.RMSNorm, *, proj_layer: nn.Linear | None = None, gate=None, next_head=None):
         """``s = x + d; s + self(norm(s))`` as one kernel, or None when it does not apply.
 
         ``d`` is ``delta`` itself, or with ``proj_layer`` (a bias-free 128 x 128 Linear)
         ``proj_layer(delta)``, or with ``gate`` as well ``proj_layer(gelu(gate) * delta)``,
-        the projection then running inside the kernel."""
+        the projection then running inside the kernel.  With ``next_head`` (``head_spec`` of the sublayer that
+        follows) and a folded projection the same launch also forms that sublayer's norm + projection, and the
+        result is the pair ``(out, head)``."""
         if not self.fused_tail_ok(x) or (delta is not None and delta.dtype != torch.bfloat16):
             return None
         if proj_layer is None:
@@ -370,7 +387,7 @@ class GatedMLP(_WeightCaches, nn.Module):
             return None
         wp = _cached_cast(proj_layer, "_bnb_proj_pack", (w,), torch.bfloat16, lambda: ops.pack_proj_weights(w))
         proj = (delta, wp) if gate is None else (gate, delta, wp)
-        return ops.ffn_fused(x, None, norm.weight, self.packed_weights(), eps=norm.eps, proj=proj)
+        return ops.ffn_fused(x, None, norm.weight, self.packed_weights(), eps=norm.eps, proj=proj, next_head=next_head)
 
     def train_tail(self, x: torch.Tensor, delta: torch.Tensor | None, norm: nn.RMSNorm, *,
                    proj_layer: nn.Linear | None = None) -> torch.Tensor | None:
@@ -451,7 +468,28 @@ class TransformerBlock(_WeightCaches, nn.Module):
         self.norm2 = nn.RMSNorm(D)
         self.ffn = GatedMLP(D)
 
-    def forward(self, x, alive_mask=None, bullets=None, bullet_mask=None):
+    def head_spec(self, x: torch.Tensor):
+        """``(norm weight, eps, packed weight, features)`` of this sublayer's head ``qkv(norm1(x))`` for the tail
+        kernel of the sublayer before (``ops.ffn_fused(next_head=...)``), or None when this sublayer would not take
+        the bfloat16 kernel path for rows like ``x``."""
+        if not (_HEAD_FUSION and not torch.is_grad_enabled() and _projection_dtype() == torch.bfloat16 and x.is_cuda
+                and x.dtype == torch.float32 and self.d_model == ops.FFN_WIDTH and self.qkv.bias is None
+                and self.norm1.weight is not None and self.norm1.weight.dtype == torch.float32):
+            return None
+        w = self.qkv.weight
+        hp = _cached_cast(self.qkv, "_bnb_head_pack", (w,), torch.bfloat16, lambda: ops.pack_head_weights(w))
+        return (self.norm1.weight, self.norm1.eps, hp, 3 * self.d_model)
+
+    def forward(self, x, alive_mask=None, bullets=None, bullet_mask=None, *, head=None, next_head=None):
+        """``head``: this sublayer's ``qkv(norm1(x))`` when the sublayer before has already formed it;
+        ``next_head``: the ``head_spec`` of the sublayer that follows: the result is then the pair
+        ``(out, that head or None)``.  Both are internal to the trunk's step."""
+        if next_head is not None:
+            out = self._forward(x, alive_mask, bullets, bullet_mask, head, next_head)
+            return out if isinstance(out, tuple) else (out, None)
+        return self._forward(x, alive_mask, bullets, bullet_mask, head, None)
+
+    def _forward(self, x, alive_mask, bullets, bullet_mask, head, next_head):
         act = _projection_dtype()
         if not _fused_ok(x, act):
             x0, n1 = _train_norm(self.norm1, x)
@@ -474,12 +512,15 @@ class TransformerBlock(_WeightCaches, nn.Module):
         # norm + qkv (one kernel under bf16) -> attention kernel -> out_proj -> fused sublayer tail
         if act == torch.bfloat16 and self.d_model == ops.FFN_WIDTH and self.qkv.bias is None:
             w = self.qkv.weight
-            pk = _cached_cast(self.qkv, "_bnb_pack", (w,), torch.bfloat16, lambda: ops.pack_linear_weights(w))
-            qkv = ops.norm_linear(x, self.norm1.weight, pk, eps=self.norm1.eps)
+            if head is not None:
+                qkv = head  # formed by the tail kernel of the sublayer before
+            else:
+                pk = _cached_cast(self.qkv, "_bnb_pack", (w,), torch.bfloat16, lambda: ops.pack_linear_weights(w))
+                qkv = ops.norm_linear(x, self.norm1.weight, pk, eps=self.norm1.eps)
             if self.ffn.fused_tail_ok(x) and self.out_proj.bias is None:
                 # the output projection runs inside the tail kernel, on the merged heads
                 merged = self._attn(None, alive_mask, bullets, bullet_mask, qkv=qkv, project=False)
-                fused = self.ffn.fused_tail(x, merged, self.norm2, proj_layer=self.out_proj)
+                fused = self.ffn.fused_tail(x, merged, self.norm2, proj_layer=self.out_proj, next_head=next_head)
                 if fused is not None:
                     return fused
                 attn = _project(self.out_proj, merged)
@@ -778,8 +819,15 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
             return x, ops.add_rmsnorm(x, self.norm1.weight, eps=self.norm1.eps, out_dtype=act)[1]
         return _train_norm(self.norm1, x)
 
-    def _finish(self, x, normed, y, gate_in=None):
-        """Gate branch, output projection and the gated MLP, both residuals."""
+    def _finish(self, x, normed, y, gate_in=None, next_head=None):
+        """Gate branch, output projection and the gated MLP, both residuals.  With ``next_head`` (the ``head_spec``
+        of the sublayer that follows) the result is ``(out, that head or None)``."""
+        if next_head is not None:
+            out = self._finish_sublayer(x, normed, y, gate_in, next_head)
+            return out if isinstance(out, tuple) else (out, None)
+        return self._finish_sublayer(x, normed, y, gate_in, None)
+
+    def _finish_sublayer(self, x, normed, y, gate_in, next_head):
         act = _projection_dtype()
         if gate_in is None:
             gate_in = _project(self.linear2, normed)
@@ -796,7 +844,8 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
         if _fused_ok(x, act) and gate_in.dtype == act:
             if y.dtype == torch.bfloat16 and y.shape == gate_in.shape:
                 # gelu(linear2) * y, linear_out, both residual adds, norm2 and the gated MLP in one kernel
-                fused = self.gated_mlp.fused_tail(x, y, self.norm2, proj_layer=self.linear_out, gate=gate_in)
+                fused = self.gated_mlp.fused_tail(x, y, self.norm2, proj_layer=self.linear_out, gate=gate_in,
+                                                  next_head=next_head)
                 if fused is not None:
                     return fused
             # gelu(linear2) * y in one kernel, residual add + norm2 (+ cast) in one kernel
@@ -842,7 +891,37 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
             state_out[:, D:].view(R, CONV_KERNEL - 1, D), reset, rows_per_env,
         )[0]
 
-    def step_tokens(self, x, n_rec, state_in, state_out, reset, field_sub):
+    def _head_weights(self, NM, n_rec, field_sub):
+        """``(fold, weights)`` of the bfloat16 head ``[linear1 | linear2 (| field_sub . linear1)](norm1(x))``:
+        with field tokens a third block carries field_sub(linear1(.)) as ONE projection (exact while field_sub is
+        the identity it starts as, a bf16 rounding of b1 apart otherwise)."""
+        rg = self.rg_lru
+        fold = (NM > n_rec and field_sub is not None and field_sub.bias is None
+                and rg.linear_a.bias is not None and rg.linear_x.bias is not None)
+        return fold, (self.linear1.weight, self.linear2.weight) + ((field_sub.weight,) if fold else ())
+
+    @staticmethod
+    def _head_matrix(ws):
+        blocks = [ws[0].detach().float(), ws[1].detach().float()]
+        if len(ws) == 3:
+            with torch.autocast("cuda", enabled=False):  # the folded product is formed in float32
+                blocks.append(ws[2].detach().float() @ blocks[0])
+        return torch.cat(blocks, dim=0)
+
+    def head_spec(self, x: torch.Tensor, n_rec: int, field_sub):
+        """``(norm weight, eps, packed weight, features)`` of this sublayer's head as ``step_tokens`` forms it, for the
+        tail kernel of the sublayer before (``ops.ffn_fused(next_head=...)``), or None when ``step_tokens`` would not
+        take the bfloat16 kernel path for tokens like ``x`` (B, NM, D)."""
+        if not (_HEAD_FUSION and not torch.is_grad_enabled() and _projection_dtype() == torch.bfloat16 and x.is_cuda
+                and x.dtype == torch.float32 and x.shape[-1] == ops.FFN_WIDTH and self.linear1.bias is None
+                and self.linear2.bias is None and self.norm1.weight is not None and self.norm1.weight.dtype == torch.float32):
+            return None
+        fold, ws = self._head_weights(x.shape[1], n_rec, field_sub)
+        hp = _cached_cast(self, "_bnb_l12f_head_pack" if fold else "_bnb_l12_head_pack", ws, torch.bfloat16,
+                          lambda: ops.pack_head_weights(self._head_matrix(ws)))
+        return (self.norm1.weight, self.norm1.eps, hp, len(ws) * ops.FFN_WIDTH)
+
+    def step_tokens(self, x, n_rec, state_in, state_out, reset, field_sub, *, head=None, next_head=None):
         """One timestep over all tokens of every environment at once.
 
         x (B, NM, D): the first ``n_rec`` tokens of an environment are recurrent (state rows
@@ -852,6 +931,9 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
         and the recurrence writes its output into the (B, NM, D) gate operand in place, so the
         reference's slicing and concatenation of ship and field tokens (griffin.py:390-417)
         costs nothing.  Returns (B, NM, D).
+
+        ``head``: this sublayer's head (``head_spec``) when the sublayer before has already formed it;
+        ``next_head``: the ``head_spec`` of the sublayer that follows: the result is then ``(out, that head or None)``.
         """
         B, NM, D = x.shape
         R = B * n_rec
@@ -860,24 +942,15 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
         y = None
         if act == torch.bfloat16 and D == ops.FFN_WIDTH and self.linear1.bias is None and self.linear2.bias is None:
             # norm1, linear1 and linear2 as one kernel: [b1 | gate_in] side by side, read in place.
-            # With field tokens a third block carries field_sub(linear1(.)) as ONE projection
-            # (field_sub . linear1 folded; exact while field_sub is the identity it starts as, a
-            # bf16 rounding of b1 apart otherwise): the recurrence then writes the ship rows of the
-            # same block, and no gather, GEMM and scatter of the field rows remain.
-            rg = self.rg_lru
-            fold = (NM > n_rec and field_sub is not None and field_sub.bias is None
-                    and rg.linear_a.bias is not None and rg.linear_x.bias is not None)
-            ws = (self.linear1.weight, self.linear2.weight) + ((field_sub.weight,) if fold else ())
-
-            def packed():
-                blocks = [ws[0].detach().float(), ws[1].detach().float()]
-                if fold:
-                    with torch.autocast("cuda", enabled=False):  # the folded product is formed in float32
-                        blocks.append(ws[2].detach().float() @ blocks[0])
-                return ops.pack_linear_weights(torch.cat(blocks, dim=0))
-
-            pk = _cached_cast(self, "_bnb_l12f_pack" if fold else "_bnb_l12_pack", ws, torch.bfloat16, packed)
-            both = ops.norm_linear(x, self.norm1.weight, pk, eps=self.norm1.eps)  # (B, NM, 2D or 3D)
+            # With field tokens the third block (field_sub . linear1) gives the field rows of y; the recurrence
+            # then writes the ship rows of the same block, and no gather, GEMM and scatter of the field rows remain.
+            fold, ws = self._head_weights(NM, n_rec, field_sub)
+            if head is not None:
+                both = head  # formed by the tail kernel of the sublayer before
+            else:
+                pk = _cached_cast(self, "_bnb_l12f_pack" if fold else "_bnb_l12_pack", ws, torch.bfloat16,
+                                  lambda: ops.pack_linear_weights(self._head_matrix(ws)))
+                both = ops.norm_linear(x, self.norm1.weight, pk, eps=self.norm1.eps)  # (B, NM, 2D or 3D)
             b1, gate_in = both[..., :D], both[..., D:2 * D]
             if fold:
                 y = both[..., 2 * D:]
@@ -919,7 +992,7 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
                               y_out=y[:, :n_rec] if NM > n_rec else y.view(R, D), reset=reset, rows_per_env=n_rec)
             if NM > n_rec and not fields_done:
                 y[:, n_rec:] = _project(field_sub, b1[:, n_rec:].reshape(-1, D)).view(B, NM - n_rec, D)
-            return self._finish(x, normed, y, gate_in)
+            return self._finish(x, normed, y, gate_in, next_head)
         res = ops.conv_step(ships_b1, state_in[:, D:].view(R, CONV_KERNEL - 1, D),
                             self.conv.weight, self.conv.bias, conv_out=state_out[:, D:].view(R, CONV_KERNEL - 1, D),
                             reset=reset, rows_per_env=n_rec, also_bf16=want_lp)
@@ -929,7 +1002,7 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
             # gathered into one (B*M, D) matrix first: on the strided view the library would run a
             # batch of B tiny GEMMs
             y[:, n_rec:] = _project(field_sub, b1[:, n_rec:].reshape(-1, D)).view(B, NM - n_rec, D)
-        return self._finish(x, normed, y, gate_in)
+        return self._finish(x, normed, y, gate_in, next_head)
 
     def forward_nonrecurrent(self, x, sub):
         """Same block with ``sub`` (a Linear) in place of conv + RG-LRU; no state."""
@@ -1111,31 +1184,61 @@ class YemongBlock(_WeightCaches, nn.Module):
             return x, h[:0], conv_buf[:0]
         return x, torch.stack(new_h), torch.stack(new_cb)
 
+    def first_head_spec(self, x, num_recurrent):
+        """``head_spec`` of this block's first sublayer for tokens like ``x`` (B, NM, D), or None."""
+        if len(self.spatial):
+            return self.spatial[0].head_spec(x)
+        if len(self.temporal):
+            return self.temporal[0].head_spec(x, num_recurrent, self.field_sub[0] if x.shape[1] > num_recurrent else None)
+        return None
+
     def step_packed(self, x, alive, state_in, state_out, num_recurrent, reset=None, bullets=None,
-                    bullet_mask=None):
+                    bullet_mask=None, *, head=None, after=None):
         """``step`` on this block's slots of the packed hidden tensor.
 
         ``state_in`` / ``state_out`` are (n_temporal, B*n_rec, 4*D) views; the new state is
         written into ``state_out`` by the kernels.  Returns the updated tokens (B, NM, D).
+
+        Under bfloat16 autocast each sublayer's tail kernel also forms the norm + projection the next sublayer
+        starts with.  Across blocks: ``head`` is that product for this block's first sublayer when the block before
+        has formed it, and ``after`` (the next block's ``first_head_spec``) asks the last sublayer here for the next
+        block's; with ``after`` the result is ``(tokens, that head or None)``.
         """
         B, NM, D = x.shape
         n_rec = num_recurrent
         x, widened = _widen_tokens(x)
         if widened:
-            return self.step_packed(x, alive, state_in, state_out, num_recurrent, reset, bullets, bullet_mask).to(torch.bfloat16)
-        for layer in self.spatial:
-            x = layer(x, alive, bullets, bullet_mask)
+            out = self.step_packed(x, alive, state_in, state_out, num_recurrent, reset, bullets, bullet_mask, head=head,
+                                   after=after)
+            return (out[0].to(torch.bfloat16), out[1]) if after is not None else out.to(torch.bfloat16)
         act = _projection_dtype()
+        n_s, n_t = len(self.spatial), len(self.temporal)
+
+        def spec_of(k, x):  # head_spec of sublayer k of this block (spatial first), of the next block's first past the end
+            if k < n_s:
+                return self.spatial[k].head_spec(x)
+            if k < n_s + n_t:
+                return self.temporal[k - n_s].head_spec(x, n_rec, self.field_sub[k - n_s] if NM > n_rec else None)
+            return after(x) if after is not None else None
+
+        for k, layer in enumerate(self.spatial):
+            nxt = spec_of(k + 1, x)
+            out = layer(x, alive, bullets, bullet_mask, head=head, next_head=nxt)
+            x, head = out if nxt is not None else (out, None)
         for j, layer in enumerate(self.temporal):
             if _fused_ok(x, act):
-                x = layer.step_tokens(x, n_rec, state_in[j], state_out[j], reset, self.field_sub[j] if NM > n_rec else None)
+                fsub = self.field_sub[j] if NM > n_rec else None
+                nxt = spec_of(n_s + j + 1, x)
+                out = layer.step_tokens(x, n_rec, state_in[j], state_out[j], reset, fsub, head=head, next_head=nxt)
+                x, head = out if nxt is not None else (out, None)
                 continue
+            head = None
             ships = layer.step_packed(x[:, :n_rec].reshape(B * n_rec, D), state_in[j], state_out[j], reset, n_rec)
             parts = [ships.reshape(B, n_rec, D)]
             if NM > n_rec:
                 parts.append(layer.forward_nonrecurrent(x[:, n_rec:], self.field_sub[j]))
             x = torch.cat(parts, dim=1) if len(parts) > 1 else parts[0]
-        return x
+        return (x, head) if after is not None else x
 
     def sequence(self, x, alive_mask, h0, conv_buf0, done_mask=None, num_recurrent=None, bullets=None,
                  bullet_mask=None):
@@ -1292,10 +1395,18 @@ class YemongTrunk(_WeightCaches, nn.Module):
         ):
             bullet_rows = ops.CompactRows(bullet_mask)
         x, widened = _widen_tokens(tokens)
-        for i, block in enumerate(self.yemong_layers):
+        blocks = list(self.yemong_layers)
+        head = None
+        for i, block in enumerate(blocks):
             sl = slice(i * n_t, (i + 1) * n_t)
-            x = block.step_packed(x, alive_mask, recurrent_state[sl], out_state[sl], n_rec, reset_mask, bullets,
-                                  bullet_rows)
+            if i + 1 < len(blocks):
+                # the last sublayer of this block also forms the norm + projection the next block starts with
+                nxt = blocks[i + 1]
+                x, head = block.step_packed(x, alive_mask, recurrent_state[sl], out_state[sl], n_rec, reset_mask, bullets,
+                                            bullet_rows, head=head, after=lambda t, nxt=nxt: nxt.first_head_spec(t, n_rec))
+            else:
+                x = block.step_packed(x, alive_mask, recurrent_state[sl], out_state[sl], n_rec, reset_mask, bullets,
+                                      bullet_rows, head=head)
         return (x.to(torch.bfloat16) if widened else x), out_state
 
 

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 22
+#define BNB_ABI_VERSION 23
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -714,6 +714,28 @@ int bnb_mask_fill(const uint8_t *mask, const int32_t *offsets, int32_t *index, i
 int bnb_ffn_fused_fwd(const float *x, int64_t x_row_stride, const void *delta, int delta_dtype,
                       const float *norm_weight, float eps, const void *weights_packed, float *out,
                       int64_t R, int D, int hidden, void *stream);
+
+/*
+ * bnb_ffn_fused_proj_fwd that goes on to the head of the NEXT sublayer: a norm and a projection of the rows it
+ * has just produced (`self.qkv(self.norm1(x))`, models/yemong/attention.py:94-96,132; `linear1` / `linear2` of
+ * `self.norm1(x)`, models/yemong/griffin.py:269-283), so that those rows do not come back from memory for it and
+ * the separate norm + projection launch (bnb_norm_linear_fwd) disappears:
+ *     next_out = bf16( bf16(rmsnorm(out) * next_norm_weight) Wh^T )
+ *
+ *   next_packed    Wh (next_features, 128) in bf16, 64 features per chunk:
+ *                  [c][b][ks][l][e] = Wh[64c + 32b + pi(l%32)][16ks + 8(e/4) + 4(l/32) + e%4],
+ *                  b = 0..1, ks = 0..7, l = 0..63, e = 0..7, pi(m) = 16(m/16) + 8((m/4)%2) + 4((m/8)%2) + m%4
+ *   next_out       (next_out_rows, next_features) bf16 contiguous; next_out_rows >= R rounded up to a multiple of
+ *                  128: the kernel stores whole work-groups of 128 rows (rows past R receive don't-care values)
+ *   next_features  a multiple of 64, at least 128
+ *   other arguments as bnb_ffn_fused_proj_fwd (rows_b == NULL: plain projection; else the gelu-gate form)
+ */
+int bnb_ffn_fused_proj_next_fwd(const float *x, int64_t x_row_stride, const void *rows_a, int64_t rows_a_stride,
+                                const void *rows_b, int64_t rows_b_stride, const void *proj_packed,
+                                const float *norm_weight, float eps, const void *weights_packed, float *out,
+                                const float *next_norm_weight, float next_eps, const void *next_packed,
+                                void *next_out, int next_features, int64_t next_out_rows, int64_t R, int D,
+                                int hidden, void *stream);
 
 /*
  * bnb_ffn_fused_fwd for the PPO update (train/rl/ppo.py:1417-1425 evaluating the trunk in grad mode):

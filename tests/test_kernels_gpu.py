@@ -1442,6 +1442,82 @@ def test_ffn_fused_with_folded_projection_matches_oracle(R, gated):
     assert max_rel(got.cpu(), two_step.cpu()) <= 1e-2
 
 
+@pytest.mark.parametrize("R,N", [(1, 128), (37, 384), (128, 256), (130, 384), (5000, 256), (4096, 384)])
+@pytest.mark.parametrize("gated", [False, True])
+def test_ffn_fused_with_the_next_sublayers_head_matches_oracle(R, N, gated):
+    # the same launch goes on to rmsnorm(out) * w2 -> bf16 -> @ Wh^T, the projection the next sublayer starts with
+    x, _, nw, p = _ffn_case(R + N, R)
+    g = torch.Generator().manual_seed(R * 3 + N)
+    D = 128
+    Wp = torch.randn(D, D, generator=g) / D ** 0.5
+    Wh = torch.randn(N, D, generator=g) / D ** 0.5
+    nw2 = 1.0 + 0.2 * torch.randn(D, generator=g)
+    rows_a = torch.randn(R, D, generator=g).bfloat16()
+    rows_y = torch.randn(R, D, generator=g).bfloat16()
+    pk = ops.pack_ffn_weights(p["f.gate_proj.weight"].to(DEV), p["f.up_proj.weight"].to(DEV), p["f.down_proj.weight"].to(DEV))
+    wp = ops.pack_proj_weights(Wp.to(DEV))
+    proj = (rows_a.to(DEV), rows_y.to(DEV), wp) if gated else (rows_a.to(DEV), wp)
+    plain = ops.ffn_fused(x.to(DEV), None, nw.to(DEV), pk, proj=proj)
+    out, head = ops.ffn_fused(x.to(DEV), None, nw.to(DEV), pk, proj=proj,
+                              next_head=(nw2.to(DEV), None, ops.pack_head_weights(Wh.to(DEV)), N))
+    assert torch.equal(out, plain)  # the tail itself is the same arithmetic
+    assert head.shape == (R, N) and head.dtype == torch.bfloat16 and head.is_contiguous()
+    # the oracle's norm + Linear on the rows the kernel produced
+    want = torch.nn.functional.linear(torch_ref.rms_norm(plain.cpu(), nw2), Wh.bfloat16().float())
+    assert max_rel(head.float().cpu(), want) <= BF16_TOL
+    # and against the stand-alone norm + projection kernel on the same rows: two bf16 roundings of one product
+    alone = ops.norm_linear(plain, nw2.to(DEV), ops.pack_linear_weights(Wh.to(DEV)))
+    assert max_rel(head.float().cpu(), alone.float().cpu()) <= BF16_TOL
+
+
+def test_next_head_one_hot_weights_hit_the_documented_positions():
+    D, N, R = 128, 384, 70
+    x, _, nw, p = _ffn_case(11, R)
+    g = torch.Generator().manual_seed(5)
+    rows_a = torch.randn(R, D, generator=g).bfloat16().to(DEV)
+    pk = ops.pack_ffn_weights(p["f.gate_proj.weight"].to(DEV), p["f.up_proj.weight"].to(DEV), p["f.down_proj.weight"].to(DEV))
+    wp = ops.pack_proj_weights((torch.randn(D, D, generator=g) / D ** 0.5).to(DEV))
+    nw2 = torch.ones(D)
+    plain = ops.ffn_fused(x.to(DEV), None, nw.to(DEV), pk, proj=(rows_a, wp)).cpu()
+    normed = torch_ref.rms_norm(plain, nw2).bfloat16().float()
+    for f, k in ((0, 0), (5, 77), (63, 127), (64, 3), (200, 64), (383, 31)):
+        Wh = torch.zeros(N, D)
+        Wh[f, k] = 1.0
+        _, head = ops.ffn_fused(x.to(DEV), None, nw.to(DEV), pk, proj=(rows_a, wp),
+                                next_head=(nw2.to(DEV), None, ops.pack_head_weights(Wh.to(DEV)), N))
+        head = head.float().cpu()
+        assert torch.allclose(head[:, f], normed[:, k], rtol=1e-2, atol=1e-6), (f, k)
+        head[:, f] = 0
+        assert head.abs().max() == 0, (f, k)
+
+
+def test_next_head_refuses_what_the_kernel_does_not_cover():
+    x, _, nw, p = _ffn_case(2, 16)
+    pk = ops.pack_ffn_weights(p["f.gate_proj.weight"].to(DEV), p["f.up_proj.weight"].to(DEV), p["f.down_proj.weight"].to(DEV))
+    nw2 = torch.ones(128, device=DEV)
+    hp = ops.pack_head_weights(torch.zeros(256, 128, device=DEV))
+    with pytest.raises(ValueError):  # only with the folded projection
+        ops.ffn_fused(x.to(DEV), None, nw.to(DEV), pk, next_head=(nw2, None, hp, 256))
+    wp = ops.pack_proj_weights(torch.zeros(128, 128, device=DEV))
+    rows = torch.zeros(16, 128, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError):  # feature count and pack disagree
+        ops.ffn_fused(x.to(DEV), None, nw.to(DEV), pk, proj=(rows, wp), next_head=(nw2, None, hp, 384))
+    with pytest.raises(ValueError):
+        ops.pack_head_weights(torch.zeros(96, 128, device=DEV))
+    from boost_and_broadside_amd import _native
+
+    lib = _native.load()
+    out = torch.empty(16, 128, device=DEV)
+    head = torch.empty(128, 256, dtype=torch.bfloat16, device=DEV)
+    args = lambda feats, rows_out: (x.to(DEV).data_ptr(), 128, rows.data_ptr(), 128, None, 0, wp.data_ptr(), nw.to(DEV).data_ptr(),
+                                    1e-6, pk.data_ptr(), out.data_ptr(), nw2.data_ptr(), 1e-6, hp.data_ptr(), head.data_ptr(),
+                                    feats, rows_out, 16, 128, 512, None)
+    bad_shape = 10003  # BNB_ERR_BAD_SHAPE
+    assert lib.bnb_ffn_fused_proj_next_fwd(*args(96, 128)) == bad_shape  # not a multiple of 64
+    assert lib.bnb_ffn_fused_proj_next_fwd(*args(256, 16)) == bad_shape  # the head needs whole work-groups of rows
+    assert lib.bnb_ffn_fused_proj_next_fwd(*args(256, 128)) == 0
+
+
 def test_column_block_operands_are_read_in_place():
     # [linear1 | linear2] outputs side by side: the conv reads the left block, the tail's gate the right one
     B, n, NM, D = 6, 8, 12, 128

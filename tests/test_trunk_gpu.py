@@ -1193,3 +1193,86 @@ def test_team_pooling_takes_a_bfloat16_stream_under_autocast_on_the_kernels():
     with torch.autocast("cuda", dtype=torch.bfloat16), trunk_module.forbid_library_dispatch():
         layer(xg, team, alive).float().square().mean().backward()
     assert xg.grad.dtype == torch.bfloat16 and torch.isfinite(xg.grad).all()
+
+
+@pytest.mark.parametrize("blocks,spatial,temporal,M,bullets", [
+    (2, 2, 1, 4, 0), (2, 2, 1, 0, 0), (2, 2, 1, 4, 1), (2, 1, 2, 4, 0), (1, 0, 2, 0, 0), (3, 1, 0, 4, 0), (2, 0, 1, 4, 0),
+])
+def test_sublayer_tails_hand_the_next_sublayer_its_projection(monkeypatch, blocks, spatial, temporal, M, bullets):
+    """Under bf16 autocast the tail kernel of every sublayer but the last also forms the norm + projection the next
+    sublayer starts with (within a block and across blocks): one stand-alone norm + projection launch is left, the
+    first sublayer's.  Same result as with every sublayer forming its own, within the bf16 bar, and as the oracle."""
+    from boost_and_broadside_amd import trunk as trunk_module
+
+    D, H, B, N = 128, 4, 11, 8
+    p = trunk_params(50 + blocks + 3 * spatial + 7 * temporal, D, blocks, spatial, temporal)
+    pg = torch.Generator().manual_seed(51)
+    for i in range(blocks):
+        for j in range(temporal):  # field tokens' stand-in for the recurrence away from the identity it starts as
+            p[f"yemong_layers.{i}.field_sub.{j}.weight"] = torch.eye(D) + 0.05 * torch.randn(D, D, generator=pg)
+        if bullets:
+            p[f"yemong_layers.{i}.spatial.0.norm_bullet.weight"] = 1.0 + 0.1 * torch.randn(D, generator=pg)
+            p[f"yemong_layers.{i}.spatial.0.kv_bullet.weight"] = 0.15 * torch.randn(2 * D, D, generator=pg)
+    trunk = bnb.YemongTrunk(_cfg(D, H, blocks, spatial, temporal, bullets=bullets)).eval()
+    trunk.load_state_dict(p)
+    trunk.to(DEV)
+    calls = []
+    ops = trunk_module.ops
+    real = ops.norm_linear
+    monkeypatch.setattr(ops, "norm_linear", lambda x, *a, **k: (calls.append(k.get("rows") is None), real(x, *a, **k))[1])
+    gen = torch.Generator().manual_seed(52)
+    L = blocks * temporal
+    state_a = state_b = torch.randn(L, B * N, 4 * D, generator=gen).to(DEV)
+    ref_state = state_a.cpu()
+    alive = torch.ones(B, N + M, dtype=torch.bool)
+    for t in range(3):
+        x = torch.randn(B, N + M, D, generator=gen)
+        alive[:, :N] &= torch.rand(B, N, generator=gen) > 0.1
+        reset = torch.rand(B, generator=gen) < 0.2
+        kw, ref_kw = {}, {}
+        if bullets:
+            bul = torch.randn(B, 10 * N, D, generator=gen)
+            bm = torch.rand(B, 10 * N, generator=gen) < 0.3
+            kw = {"bullets": bul.to(DEV), "bullet_mask": bm.to(DEV)}
+            ref_kw = {"bullets": bul, "bullet_mask": bm}
+        with torch.autocast("cuda", dtype=torch.bfloat16), trunk_module.forbid_library_dispatch():
+            calls.clear()
+            out_a, state_a = trunk(x.to(DEV), alive.to(DEV), state_a, reset_mask=reset.to(DEV), **kw)
+            handed_over = sum(calls)  # launches over all rows of the residual stream (the bullets' own do not count)
+            with trunk_module.separate_heads():
+                calls.clear()
+                out_b, state_b = trunk(x.to(DEV), alive.to(DEV), state_b, reset_mask=reset.to(DEV), **kw)
+                on_their_own = sum(calls)
+        assert handed_over == 1 and on_their_own == blocks * (spatial + temporal)
+        assert max_rel(out_a.cpu(), out_b.cpu()) <= BF16_TOL, t
+        if L:
+            assert max_rel(state_a.cpu(), state_b.cpu()) <= BF16_TOL, t
+        ref_out, ref_state = torch_ref.trunk_step(p, blocks, spatial, temporal, H, x, alive,
+                                                  torch_ref.reset_hidden(ref_state, reset, N), **ref_kw)
+        assert max_rel(out_a.cpu(), ref_out) <= BF16_TOL, t
+        if L:
+            assert max_rel(state_a.cpu(), ref_state) <= BF16_TOL, t
+
+
+def test_graphed_trunk_with_handed_over_projections_replays_like_the_eager_step():
+    from boost_and_broadside_amd import trunk as trunk_module
+
+    D, H, B, N, M = 128, 4, 24, 8, 4
+    p = trunk_params(61, D, 2, 2, 1)
+    trunk = bnb.YemongTrunk(_cfg(D, H, 2, 2, 1)).eval()
+    trunk.load_state_dict(p)
+    trunk.to(DEV)
+    graphed = bnb.GraphedTrunk(trunk, B, N + M, N, autocast_dtype=torch.bfloat16)
+    gen = torch.Generator().manual_seed(62)
+    state = trunk.initial_hidden(B, N, DEV)
+    alive = torch.ones(B, N + M, dtype=torch.bool, device=DEV)
+    for t in range(4):
+        x = torch.randn(B, N + M, D, generator=gen).to(DEV)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            eager, state = trunk(x, alive, state)
+            with trunk_module.separate_heads():
+                apart, _ = trunk(x, alive, graphed.state.clone())
+        torch.cuda.synchronize()
+        out, new_state = graphed.step(x, alive)
+        assert torch.equal(out, eager) and torch.equal(new_state, state), t
+        assert max_rel(out.cpu(), apart.cpu()) <= BF16_TOL
