@@ -1068,6 +1068,37 @@ def test_ffn_bwd_matches_autograd_of_the_oracle(R, dy_dtype):
     assert torch.equal(again[0], dn) and torch.equal(again[1][:, :R], dgu[:, :R]) and torch.equal(again[2][:, :R], h[:, :R])
 
 
+def test_ffn_bwd_at_update_size_on_sampled_rows():
+    # the update's row count at 4v4 (128 steps x 256 environments x 12 tokens): six rounds of resident work-groups
+    R = 128 * 256 * 12
+    _, _, _, p = _ffn_case(77, 1)
+    g = torch.Generator(device=DEV).manual_seed(78)
+    n = torch.randn(R, 128, device=DEV, generator=g).bfloat16()
+    dy = torch.randn(R, 128, device=DEV, generator=g)
+    pk = ops.pack_ffn_bwd_weights(*(p[k].to(DEV) for k in ("f.gate_proj.weight", "f.up_proj.weight", "f.down_proj.weight")))
+    dn, dgu, h, dy_lp = ops.ffn_bwd(n, dy, pk)
+    pick = torch.arange(0, R, 3001, device=DEV)
+    hid, da, db, dn_ref, _ = _ffn_bwd_reference(n[pick].cpu(), dy[pick].cpu(), p)
+    P = pick.numel()
+    assert max_rel(h[:, pick].permute(1, 0, 2).reshape(P, 512).float().cpu(), hid.float()) <= BF16_TOL
+    t = dgu[:, pick].permute(1, 0, 2).reshape(P, 8, 2, 2, 32).float().cpu()
+    assert max_rel(t[:, :, :, 0].reshape(P, 512), da.float()) <= BF16_TOL
+    assert max_rel(t[:, :, :, 1].reshape(P, 512), db.float()) <= BF16_TOL
+    assert max_rel(dn[pick].float().cpu(), dn_ref.float()) <= BF16_TOL
+    assert torch.isfinite(dn.float()).all()
+    # a row's results do not depend on where or when it is computed: bit for bit under a row permutation
+    perm = torch.randperm(R, device=DEV, generator=g)
+    dn_p, dgu_p, h_p, _ = ops.ffn_bwd(n[perm], dy[perm], pk)
+    assert torch.equal(dn_p, dn[perm]) and torch.equal(dgu_p[:, :R], dgu[:, perm]) and torch.equal(h_p[:, :R], h[:, perm])
+    # weight gradients against float32 products of the very operands the kernel stored
+    d_gate, d_up, d_down = ops.ffn_weight_grads(n, dgu, h, dy_lp)
+    tt = dgu[:, :R].permute(1, 0, 2).reshape(R, 8, 2, 2, 32).float()
+    nf = n.float()
+    assert max_rel(d_gate, tt[:, :, :, 0].reshape(R, 512).t() @ nf) <= 1e-3
+    assert max_rel(d_up, tt[:, :, :, 1].reshape(R, 512).t() @ nf) <= 1e-3
+    assert max_rel(d_down, dy_lp.float().t() @ h[:, :R].permute(1, 0, 2).reshape(R, 512).float()) <= 1e-3
+
+
 def test_ffn_bwd_every_weight_reaches_its_gradient():
     # one-hot weights: the packed operand order, the tile layout of the results and the weight-gradient un-permutation
     # must each put hidden unit j and channel k where the layout says
@@ -1715,6 +1746,39 @@ def test_full_size_sublayer_tail_and_projection_on_sampled_rows():
     qkv = ops.norm_linear(x, nw.to(DEV), ops.pack_linear_weights(wq.to(DEV)))
     want = torch_ref.rms_norm(x[pick].cpu(), nw) @ wq.bfloat16().float().t()
     assert max_rel(qkv[pick].float().cpu(), want) <= BF16_TOL
+
+
+@pytest.mark.parametrize("gated,N", [(False, 384), (True, 256)])
+def test_full_size_tail_with_the_next_sublayers_head_on_sampled_rows(gated, N):
+    # 64v88: 655,360 token rows, ten rounds of resident work-groups: every weight buffer is recycled many times
+    w = harness.WORKLOADS["c4_64v88_bf16"]
+    R, D = w.B * w.NM, 128
+    g = torch.Generator(device=DEV).manual_seed(29 + N)
+    cg = torch.Generator().manual_seed(30 + N)
+    _, _, nw, p = _ffn_case(29, 1)
+    x = torch.randn(R, D, device=DEV, generator=g)
+    rows_a = torch.randn(R, D, device=DEV, generator=g).bfloat16()
+    rows_y = torch.randn(R, D, device=DEV, generator=g).bfloat16()
+    Wp = torch.randn(D, D, generator=cg) / D ** 0.5
+    Wh = torch.randn(N, D, generator=cg) / D ** 0.5
+    nw2 = 1.0 + 0.2 * torch.randn(D, generator=cg)
+    pk = ops.pack_ffn_weights(p["f.gate_proj.weight"].to(DEV), p["f.up_proj.weight"].to(DEV), p["f.down_proj.weight"].to(DEV))
+    wp = ops.pack_proj_weights(Wp.to(DEV))
+    spec = (nw2.to(DEV), None, ops.pack_head_weights(Wh.to(DEV)), N)
+    proj = (rows_a, rows_y, wp) if gated else (rows_a, wp)
+    out, head = ops.ffn_fused(x, None, nw.to(DEV), pk, proj=proj, next_head=spec)
+    assert torch.equal(out, ops.ffn_fused(x, None, nw.to(DEV), pk, proj=proj))
+    assert torch.isfinite(head.float()).all()
+    pick = torch.arange(0, R, 5003, device=DEV)
+    want = torch.nn.functional.linear(torch_ref.rms_norm(out[pick].cpu(), nw2), Wh.bfloat16().float())
+    assert max_rel(head[pick].float().cpu(), want) <= BF16_TOL
+    alone = ops.norm_linear(out, nw2.to(DEV), ops.pack_linear_weights(Wh.to(DEV)))
+    assert max_rel(head.float(), alone.float()) <= BF16_TOL
+    # row permutation equivariance, bit for bit: a row's result does not depend on where or when it is computed
+    perm = torch.randperm(R, device=DEV, generator=g)
+    proj_p = (rows_a[perm], rows_y[perm], wp) if gated else (rows_a[perm], wp)
+    out_p, head_p = ops.ffn_fused(x[perm], None, nw.to(DEV), pk, proj=proj_p, next_head=spec)
+    assert torch.equal(out_p, out[perm]) and torch.equal(head_p, head[perm])
 
 
 def test_full_size_team_pool_on_sampled_environments():
