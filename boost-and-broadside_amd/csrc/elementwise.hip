@@ -9,7 +9,7 @@
 //                 (reference: GatedMLP, attention.py:36-37; the gate branch of the temporal
 //                 block, griffin.py:281-282)
 //
-// Both are pure streaming kernels: 8 channels per lane, 16-byte nontemporal accesses, fp32
+// Both are pure streaming kernels: 8 channels per lane, nontemporal accesses, fp32
 // arithmetic, roundings placed where torch's type promotion places them.
 
 #include "common.h"
@@ -29,14 +29,17 @@ __global__ __launch_bounds__(kEwThreads) void add_rmsnorm_kernel(
     constexpr int D = LANES * 8;
     constexpr int ROWS = kEwThreads / LANES;
     const int local_row = threadIdx.x / LANES;
-    const int d0 = (threadIdx.x - local_row * LANES) << 3;
+    // a lane's eight channels are two runs of four, d0 .. d0 + 3 and D/2 + d0 ..: every access of a row's lanes is one
+    // dense run of bytes
+    const int d0 = (threadIdx.x - local_row * LANES) << 2;
+    constexpr int gap = D / 2;
     const int64_t row = (int64_t)blockIdx.x * ROWS + local_row;
     const bool valid = row < R;  // keep every lane in the butterfly
     const int64_t r = valid ? row : R - 1;
 
-    Row8 s = load8_stream(x + r * x_stride + d0);
+    Row8 s = load8_split<true>(x + r * x_stride + d0, gap);
     if (HAS_DELTA) {
-        const Row8 dl = load8_stream(delta + r * D + d0);
+        const Row8 dl = load8_split<true>(delta + r * D + d0, gap);
 #pragma unroll
         for (int e = 0; e < 8; ++e) s.v[e] += dl.v[e];
     }
@@ -48,12 +51,12 @@ __global__ __launch_bounds__(kEwThreads) void add_rmsnorm_kernel(
     const float rstd = rsqrtf(ss * (1.0f / D) + eps);
 
     if (!valid) return;
-    if (HAS_SUM) store8_stream(sum_out + row * D + d0, s);
-    const Row8 w = load8(weight + d0);
+    if (HAS_SUM) store8_split<true>(sum_out + row * D + d0, gap, s);
+    const Row8 w = load8_split<false>(weight + d0, gap);
     Row8 n;
 #pragma unroll
     for (int e = 0; e < 8; ++e) n.v[e] = (s.v[e] * rstd) * w.v[e];
-    store8_stream(norm_out + row * D + d0, n);
+    store8_split<true>(norm_out + row * D + d0, gap, n);
 }
 
 // ---- out = gelu(a) * b -----------------------------------------------------------------------

@@ -64,17 +64,21 @@ __global__ __launch_bounds__(kNbThreads) void rmsnorm_bwd_kernel(
     __shared__ float s_dw[ROWS * D];
 
     const int local_row = threadIdx.x / LANES;
-    const int d0 = (threadIdx.x - local_row * LANES) << 3;
+    // a lane's eight channels are two runs of four, d0 .. d0 + 3 and D/2 + d0 ..: each access of a row's lanes is
+    // then one dense run of bytes (eight consecutive float32 channels per lane put the lanes of an instruction 32
+    // bytes apart, which streams at two thirds of the rate)
+    const int d0 = (threadIdx.x - local_row * LANES) << 2;
+    constexpr int gap = D / 2;
     const int64_t step = (int64_t)gridDim.x * ROWS;
-    const Row8 w = load8(weight + d0);
+    const Row8 w = load8_split<false>(weight + d0, gap);
     float dw[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 
     // every lane of a row group walks the same number of iterations (the butterflies need all of them)
     int64_t row = (int64_t)blockIdx.x * ROWS + local_row;
     int64_t r = row < R ? row : R - 1;
-    Row8 xn = load8_stream(x + r * x_stride + d0), gn = load8_stream(dy + r * dy_stride + d0);
+    Row8 xn = load8_split<true>(x + r * x_stride + d0, gap), gn = load8_split<true>(dy + r * dy_stride + d0, gap);
     Row8 sn = xn;  // the bypass gradient travels with the other two rows, one iteration ahead
-    if (HAS_SUM) sn = load8_stream(grad_sum + r * D + d0);
+    if (HAS_SUM) sn = load8_split<true>(grad_sum + r * D + d0, gap);
     for (int64_t base = (int64_t)blockIdx.x * ROWS; base < R; base += step) {
         const Row8 xv = xn, gv = gn, sv = sn;
         const int64_t cur = row;
@@ -82,8 +86,8 @@ __global__ __launch_bounds__(kNbThreads) void rmsnorm_bwd_kernel(
         row += step;
         if (base + step < R) {
             r = row < R ? row : R - 1;
-            xn = load8_stream(x + r * x_stride + d0), gn = load8_stream(dy + r * dy_stride + d0);
-            if (HAS_SUM) sn = load8_stream(grad_sum + r * D + d0);
+            xn = load8_split<true>(x + r * x_stride + d0, gap), gn = load8_split<true>(dy + r * dy_stride + d0, gap);
+            if (HAS_SUM) sn = load8_split<true>(grad_sum + r * D + d0, gap);
         }
         float ss = 0.0f, dot = 0.0f;
         Row8 g;
@@ -111,13 +115,13 @@ __global__ __launch_bounds__(kNbThreads) void rmsnorm_bwd_kernel(
 #pragma unroll
             for (int e = 0; e < 8; ++e) o.v[e] += sv.v[e];
         }
-        store8_stream(dx + cur * D + d0, o);
+        store8_split<true>(dx + cur * D + d0, gap, o);
         // an ordinary store: as a third nontemporal stream this copy cost 50 us more on some allocations
-        if (dx_bf16 != nullptr) store8(dx_bf16 + cur * D + d0, o);
+        if (dx_bf16 != nullptr) store8_split<false>(dx_bf16 + cur * D + d0, gap, o);
     }
 
 #pragma unroll
-    for (int e = 0; e < 8; ++e) s_dw[local_row * D + d0 + e] = dw[e];
+    for (int e = 0; e < 8; ++e) s_dw[local_row * D + d0 + (e & 3) + (e >> 2) * gap] = dw[e];
     __syncthreads();
     for (int d = threadIdx.x; d < D; d += kNbThreads) {
         float t = 0.0f;
