@@ -919,10 +919,13 @@ def main():
             wall_te = timed_loop(trunk_step_eager, n_tr, 10)
         graphed = bnb.GraphedTrunk(trunk, w.B, w.NM, w.N, autocast_dtype=torch.bfloat16 if bf16 else None)
         wall_g = timed_loop(lambda t: graphed.step(x32[t & 1], alive_steps[t % n_alive]), n_tr, 4)
+        # a producer that writes tokens and mask straight into the capture's input buffers: no staging copies
+        wall_gi = timed_loop(lambda t: graphed.step(graphed.tokens, graphed.alive, graphed.reset), n_tr, 4)
         del graphed
         result["trunk"] = {
             "value": tokens * n_tr / wall_tr, "unit": "entity-tokens/s", "ms_per_step": wall_tr / n_tr * 1e3,
             "hip_graph_ms_per_step": wall_g / n_tr * 1e3,
+            "hip_graph_inputs_in_place_ms_per_step": wall_gi / n_tr * 1e3,
             "steps": n_tr, "eager_torch_ms_per_step": wall_te / n_tr * 1e3, "speedup_over_eager_torch": wall_te / wall_tr,
             "what": "YemongTrunk.forward, 2 blocks x (2 attention + 1 temporal sublayer), d_model 128, packed fp32 state "
                     "carried, " + ("bf16 autocast" if bf16 else "fp32") + "; eager = same modules with the kernels "

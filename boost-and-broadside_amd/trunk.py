@@ -1487,13 +1487,19 @@ class GraphedTrunk:
 
     @torch.no_grad()
     def step(self, tokens, alive_mask, reset_mask=None):
-        """One trunk step on the captured shape; returns (hidden, new_state) static tensors."""
-        self.tokens.copy_(tokens)
-        self.alive.copy_(alive_mask)
+        """One trunk step on the captured shape; returns (hidden, new_state) static tensors.
+
+        The inputs are copied into the static buffers ``self.tokens`` / ``self.alive`` / ``self.reset``; a producer that
+        writes its result straight into those buffers passes the buffers themselves and no copy is made
+        (at 4096 environments x 160 tokens the token copy alone is 0.13 ms of a 4.5 ms step)."""
+        if tokens is not self.tokens:
+            self.tokens.copy_(tokens)
+        if alive_mask is not self.alive:
+            self.alive.copy_(alive_mask)
         if self.reset is not None:
             if reset_mask is None:
                 self.reset.fill_(False)
-            else:
+            elif reset_mask is not self.reset:
                 self.reset.copy_(reset_mask)
         elif reset_mask is not None:
             raise ValueError("this capture was made without a reset input")
