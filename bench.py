@@ -774,8 +774,17 @@ def main():
                     out_u = blk.sequence(xu, au, hu, cu, du, num_recurrent=Nu)[0]
                 out_u.float().square().mean().backward()
 
+            go_blk = torch.randn(Tu, Bu, Nu + Mu, D, device=dev, generator=gen)
+
+            def update_step_given_grad(t):  # the block alone: the gradient of its output is handed in, no loss kernels
+                blk.zero_grad(set_to_none=True)
+                with torch.enable_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+                    out_u = blk.sequence(xu, au, hu, cu, du, num_recurrent=Nu)[0]
+                out_u.backward(go_blk)
+
             from boost_and_broadside_amd import trunk as trunk_module
             t_up = timed_loop(update_step, 3, 2) / 3
+            t_up_g = timed_loop(update_step_given_grad, 3, 2) / 3
             t_up_lib = None
             if not args.no_torch_baseline:
                 with trunk_module.library_update_path():
@@ -879,6 +888,7 @@ def main():
             del pma_u, xs_u, tm_u, al_u, go_u
             result["update_path"] = {
                 "rows": Rw, "linear_wgrad": wg, "kernels": kern, "block_fwd_bwd_ms": t_up * 1e3,
+                "block_fwd_bwd_given_grad_ms": t_up_g * 1e3,
                 "block_with_bullets_fwd_bwd_ms": t_upb * 1e3,
                 "block_with_bullets_fwd_bwd_library_ms": None if t_upb_lib is None else t_upb_lib * 1e3,
                 "team_pool_fwd_bwd_ms": t_pool_up * 1e3,
@@ -887,7 +897,8 @@ def main():
                 "what": "bnb_linear_wgrad_fwd (dW = dy^T x, bf16 in, fp32 out, rows split over the chip) beside the library "
                         "GEMM on the same operands; kernels = the norm, gelu-gate, gated-MLP, attention and conv backward kernels at the "
                         "sizes of the block below; block = one YemongBlock (2 attention + 1 temporal sublayer), T = 128 x 256 "
-                        "environments of 4v4, forward + backward under bf16 autocast, on the update-path kernels and with "
+                        "environments of 4v4, forward + backward of mean(out^2) under bf16 autocast (given_grad: backward from a "
+                        "given gradient of the output instead, i.e. without the loss's own kernels), on the update-path kernels and with "
                         "torch's own differentiable ops in their place (the recurrence keeps its kernels in both); block_with_bullets = "
                         "the same with one attention sublayer reading 80 bullet slots per environment, 25 % live; team_pool = TeamPMA "
                         "forward + backward over the ships of the same rollout (32,768 environments x 8 ships), kernels and library",

@@ -811,6 +811,37 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
         y, new_h = self.rg_lru.forward_sequence(v, h0, done_mask, time_major=time_major)
         return self._finish(x_seq, normed, y), new_h, padded[:, T:]
 
+    def sequence_tokens(self, x, n_rec, h0, conv_buf, done_rows, field_sub):
+        """The update's form of this sublayer over ALL tokens of a stored rollout at once, or None when it does not apply.
+
+        x (T, B, NM, D) float32, the first ``n_rec`` tokens of an environment recurrent (state rows env-major,
+        ``h0`` (B*n_rec, D), ``conv_buf`` (B*n_rec, 3, D), ``done_rows`` (B*n_rec, T) or None), the rest going through
+        ``field_sub`` instead of conv + RG-LRU (griffin.py:288-317, :406-413).  The reference runs the block twice, on the
+        ship rows and on the field rows, and concatenates the results; every row-wise part (both norms, linear1,
+        linear2, the gate, linear_out, the gated MLP and all their backward kernels) is the same function of a row
+        either way, so here it runs once over all rows, and only conv + recurrence (ship rows) and ``field_sub``
+        (field rows) see a part of them.  Returns ``(out (T, B, NM, D), new_h, new_conv_buf)``."""
+        T, B, NM, D = x.shape
+        if not (_TRAIN_KERNELS and torch.is_grad_enabled() and x.is_cuda and NM > n_rec and field_sub is not None
+                and _projection_dtype() == torch.bfloat16 and conv_buf.dtype == torch.float32
+                and self.conv.weight.dtype == torch.float32):
+            return None
+        x, normed = _train_norm(self.norm1, x)
+        b1 = _project(self.linear1, normed)
+        if b1.dtype != torch.bfloat16 or b1.shape[-1] != ops.FFN_WIDTH:
+            return None
+        ships_b1, fields_b1 = _SplitTokens.apply(b1, n_rec)
+        ships_b1 = ships_b1.reshape(T, B * n_rec, D)
+        if not ops.conv_seq_train_supported(ships_b1):
+            return None
+        v, new_buf = ops.conv_seq_train(ships_b1, conv_buf, self.conv.weight, self.conv.bias, done_rows, time_major=True)
+        y_ships, new_h = self.rg_lru.forward_sequence(v, h0, done_rows, time_major=True)
+        y_fields = _project(field_sub, fields_b1)
+        # the recurrence's output is float32 (the conv buffer promotes its input, griffin.py:275); the field rows'
+        # bfloat16 values are exact in it, and the gate kernel rounds the product once either way
+        y = torch.cat([y_ships.reshape(T, B, n_rec, D), y_fields.to(y_ships.dtype)], dim=2)
+        return self._finish(x, normed, y), new_h, new_buf
+
     def _norm_in(self, x):
         """``(x, norm1(x))`` with the norm in the projection dtype (one kernel with the cast when the fused
         path applies); the returned x is the one to use for the residual connection."""
@@ -1260,6 +1291,14 @@ class YemongBlock(_WeightCaches, nn.Module):
         done_rows = None if done_mask is None else done_mask.t().repeat_interleave(n_rec, dim=0)  # (B*n_rec, T)
         new_h, new_cb = [], []
         for j, layer in enumerate(self.temporal):
+            if NM > n_rec and torch.is_grad_enabled():
+                # the update: every row-wise part of the sublayer once over all tokens
+                whole = layer.sequence_tokens(x, n_rec, h0[j], conv_buf0[j], done_rows, self.field_sub[j])
+                if whole is not None:
+                    x = whole[0]
+                    new_h.append(whole[1])
+                    new_cb.append(whole[2])
+                    continue
             # the sequence kernels read (T, rows, D) as stored: no transposed copies of the rollout
             if NM > n_rec and x.requires_grad:
                 ships, fields = _SplitTokens.apply(x, n_rec)
