@@ -36,7 +36,8 @@ constexpr int kNlHalfPitch = 64 + 4;                                   // floats
 __global__ __launch_bounds__(kNlThreads) void norm_linear_kernel(
     const float *__restrict__ x, int64_t x_stride, const int32_t *__restrict__ row_index,
     const int32_t *__restrict__ n_rows, const float *__restrict__ norm_w, float eps,
-    const uint16_t *__restrict__ wpack, const float *__restrict__ bias, uint16_t *__restrict__ out, int64_t R, int N)
+    const uint16_t *__restrict__ wpack, const float *__restrict__ bias, uint16_t *__restrict__ out, int64_t R, int N,
+    uint16_t *__restrict__ n_out = nullptr)
 {
     // staging area for the rows (prologue) and the two weight buffers (loop) share this space
     constexpr int kStageFloats = kNlWaves * 32 * kNlHalfPitch;                       // 8704 floats = 34 KB
@@ -114,6 +115,33 @@ __global__ __launch_bounds__(kNlThreads) void norm_linear_kernel(
     }
     ss += __shfl_xor(ss, 32);
     const float rstd = rsqrtf(ss * (1.0f / kNlD) + eps);
+
+    if (n_out != nullptr) {
+        // The update keeps the normalised rows for the weight gradient: the operand this kernel multiplies is
+        // rstd * bf16(x * w_norm); its bfloat16 rounding leaves as whole 256-byte rows through this wave's slice
+        // of the staging area (32 rows x 136 halfs fit in the 32 x 68 floats of the slice).
+        constexpr int kNPitch = kNlD + 8;
+        static_assert(kNPitch * 2 <= kNlHalfPitch * 4, "a staged bf16 row fits the slice's row pitch");
+        uint16_t *stage_n = reinterpret_cast<uint16_t *>(stage);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            float t[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) t[e] = (float)nb[ks][e] * rstd;
+            uint16_t *sp = stage_n + m * kNPitch + 16 * ks + 4 * half;
+            *reinterpret_cast<u32x2 *>(sp) = u32x2{pack_bf16x2(t[0], t[1]), pack_bf16x2(t[2], t[3])};
+            *reinterpret_cast<u32x2 *>(sp + 8) = u32x2{pack_bf16x2(t[4], t[5]), pack_bf16x2(t[6], t[7])};
+        }
+        wave_lds_handover();
+        const int a_row = lane >> 4, a_col = (lane & 15) * 8;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int64_t r = row0 + 4 * j + a_row;
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(stage_n + (4 * j + a_row) * kNPitch + a_col);
+            if (r < rows) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(n_out + r * kNlD + a_col));
+        }
+        __syncthreads();  // the slices are read out before the weights move in
+    }
 
     stash(0);
     __builtin_amdgcn_s_waitcnt(0x0f70);
@@ -217,6 +245,26 @@ extern "C" int bnb_norm_linear_fwd(const float *x, int64_t x_row_stride, const i
     hipLaunchKernelGGL(norm_linear_kernel, dim3((unsigned)blocks), dim3(kNlThreads), 0, (hipStream_t)stream, x,
                        x_row_stride, row_index, n_rows, norm_weight, eps, (const uint16_t *)weight_packed, bias,
                        (uint16_t *)out, R, N);
+    return (int)hipGetLastError();
+}
+
+extern "C" int bnb_norm_linear_train_fwd(const float *x, int64_t x_row_stride, const float *norm_weight, float eps,
+                                         const void *weight_packed, void *out, void *n_out, int64_t R, int D, int N,
+                                         void *stream)
+{
+    using namespace bnb;
+    if (R < 0 || x_row_stride < D || N < 1) return BNB_ERR_BAD_SHAPE;
+    if (D != kNlD || N % kNlChunkFeatures != 0) return BNB_ERR_UNSUPPORTED;
+    if (R == 0) return 0;
+    if (!x || !norm_weight || !weight_packed || !out || !n_out) return BNB_ERR_NULL_POINTER;
+    if (!aligned16(x) || !aligned16(out) || !aligned16(n_out) || !aligned16(norm_weight) || !aligned16(weight_packed) ||
+        (x_row_stride % 4) != 0)
+        return BNB_ERR_MISALIGNED;
+    const int64_t blocks = (R + kNlWaves * 32 - 1) / (kNlWaves * 32);
+    if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(norm_linear_kernel, dim3((unsigned)blocks), dim3(kNlThreads), 0, (hipStream_t)stream, x,
+                       x_row_stride, (const int32_t *)nullptr, (const int32_t *)nullptr, norm_weight, eps,
+                       (const uint16_t *)weight_packed, (const float *)nullptr, (uint16_t *)out, R, N, (uint16_t *)n_out);
     return (int)hipGetLastError();
 }
 

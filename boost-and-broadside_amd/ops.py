@@ -1548,6 +1548,77 @@ class _AddRmsNormTrain(torch.autograd.Function):
         return dx, ddelta, dw, None, None
 
 
+class _NormLinearTrain(torch.autograd.Function):
+    """``(x, linear(rmsnorm(x) * norm_weight), rmsnorm(x) * norm_weight)`` under bfloat16 autocast as one
+    kernel forward: the projection's launch also writes the normalised rows, which are all the backward keeps
+    besides x.  Backward: the library's input-gradient GEMM, the weight-gradient kernel and the norm's backward
+    kernel, which adds the gradients reaching x (residual branch) and the normalised rows (their other users)
+    in the same pass."""
+
+    @staticmethod
+    def forward(ctx, x, norm_weight, weight, eps, packed):
+        D = x.shape[-1]
+        x2 = x.reshape(-1, D)
+        if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) % 4):
+            x2 = x2.contiguous()
+        R, N = x2.shape[0], weight.shape[0]
+        y = torch.empty((R, N), dtype=torch.bfloat16, device=x.device)
+        n = torch.empty((R, D), dtype=torch.bfloat16, device=x.device)
+        if R:
+            with _on_device(x.device):
+                rc = _native.load().bnb_norm_linear_train_fwd(
+                    x2.data_ptr(), x2.stride(0), norm_weight.detach().contiguous().data_ptr(),
+                    float(_F32_EPS if eps is None else eps), packed.data_ptr(), y.data_ptr(), n.data_ptr(), R, D, N, _stream())
+            _native.check(rc, "bnb_norm_linear_train_fwd")
+        ctx.save_for_backward(x, norm_weight, weight, n)
+        ctx.eps = eps
+        n_out = n.view(x.shape)
+        return x.view_as(x), y.view(*x.shape[:-1], N), n_out
+
+    @staticmethod
+    @_outside_autocast
+    def backward(ctx, ds, dy, dn_other):
+        x, norm_weight, weight, n = ctx.saved_tensors
+        D = x.shape[-1]
+        dn = None
+        d_weight = None
+        if dy is not None:
+            dy2 = dy.reshape(-1, dy.shape[-1])
+            dyb = dy2 if dy2.dtype == torch.bfloat16 else dy2.to(torch.bfloat16)
+            if dyb.stride(-1) != 1:
+                dyb = dyb.contiguous()
+            dn = torch.matmul(dyb, weight.detach().to(torch.bfloat16))
+            if ctx.needs_input_grad[2]:
+                d_weight = linear_wgrad(dyb, n)
+        if dn_other is not None:
+            dn_other = dn_other.reshape(-1, D)
+            dn = dn_other if dn is None else dn + dn_other.to(dn.dtype)
+        if dn is None:
+            dn = torch.zeros_like(n)
+        dx, d_norm = rmsnorm_bwd(x, dn.view(x.shape), norm_weight, eps=ctx.eps, grad_sum=ds)
+        return dx, d_norm, d_weight, None, None
+
+
+def norm_linear_train_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether ``norm_linear_train`` covers this projection: float32 (..., 128) rows on the GPU, a float32 (N, 128)
+    weight with N a multiple of 64, enough rows for the weight-gradient kernel."""
+    return (x.is_cuda and x.dtype == torch.float32 and x.shape[-1] == FFN_WIDTH and weight.dtype == torch.float32
+            and weight.dim() == 2 and weight.shape[1] == FFN_WIDTH and weight.shape[0] % 64 == 0
+            and linear_wgrad_supported(x, weight))
+
+
+def norm_linear_train(x: torch.Tensor, norm_weight: torch.Tensor, weight: torch.Tensor, *, eps: float | None = None,
+                      packed: torch.Tensor | None = None):
+    """Differentiable ``norm_linear`` for the update under bfloat16 autocast: returns ``(x, y, n)`` with
+    ``n = bf16(rmsnorm(x) * norm_weight)`` and ``y = n @ weight^T`` (bfloat16, float32 accumulation).  Use the returned
+    x for the residual connection (its gradient is then added inside the norm's backward kernel) and ``n`` for any other
+    projection of the same normalised rows.  ``packed``: ``pack_linear_weights(weight)``, if the caller caches it."""
+    if packed is None:
+        packed = pack_linear_weights(weight)
+    with torch.autocast("cuda", enabled=False):
+        return _NormLinearTrain.apply(x, norm_weight, weight, eps, packed)
+
+
 def rmsnorm_train_supported(x: torch.Tensor) -> bool:
     """Whether ``rmsnorm_train`` covers this input: float32 rows of a covered width on the GPU."""
     return x.is_cuda and x.dtype == torch.float32 and x.shape[-1] in _NORM_TRAIN_WIDTHS

@@ -292,6 +292,22 @@ def _gelu_gate(gate: torch.Tensor, value: torch.Tensor) -> torch.Tensor:
     return F.gelu(gate) * value
 
 
+def _norm_linear_train_ok(x: torch.Tensor, act: torch.dtype, norm: nn.RMSNorm, layer: nn.Linear) -> bool:
+    """Whether ``layer(norm(x))`` of the update runs as one forward kernel (``ops.norm_linear_train``)."""
+    return (
+        _TRAIN_KERNELS and torch.is_grad_enabled() and act == torch.bfloat16 and layer.bias is None
+        and norm.weight is not None and norm.weight.dtype == torch.float32 and layer.weight.requires_grad
+        and x.numel() >= _WGRAD_MIN_ROWS * x.shape[-1] and ops.norm_linear_train_supported(x, layer.weight)
+    )
+
+
+def _norm_linear_train(x: torch.Tensor, norm: nn.RMSNorm, layer: nn.Linear):
+    """``(x, layer(norm(x)), norm(x))`` through ``ops.norm_linear_train``; use the returned x for the residual."""
+    w = layer.weight
+    pk = _cached_cast(layer, "_bnb_pack", (w,), torch.bfloat16, lambda: ops.pack_linear_weights(w))
+    return ops.norm_linear_train(x, norm.weight, w, eps=norm.eps, packed=pk)
+
+
 def _train_norm(norm: nn.RMSNorm, x: torch.Tensor, delta: torch.Tensor | None = None):
     """``(s, norm(s))`` with ``s = x + delta`` (``s`` = x without ``delta``), differentiable.  Use the
     returned ``s`` for the residual connection.
@@ -492,10 +508,15 @@ class TransformerBlock(_WeightCaches, nn.Module):
     def _forward(self, x, alive_mask, bullets, bullet_mask, head, next_head):
         act = _projection_dtype()
         if not _fused_ok(x, act):
-            x0, n1 = _train_norm(self.norm1, x)
+            qkv = None
+            if _norm_linear_train_ok(x, act, self.norm1, self.qkv):
+                # the update: norm1 and qkv as one kernel that also leaves the normalised rows for the weight gradient
+                x0, qkv, n1 = _norm_linear_train(x, self.norm1, self.qkv)
+            else:
+                x0, n1 = _train_norm(self.norm1, x)
             if torch.is_grad_enabled():
                 # out_proj inside the tail kernel, on the merged heads, when the tail kernel applies
-                merged = self._attn(n1, alive_mask, bullets, bullet_mask, project=False)
+                merged = self._attn(n1, alive_mask, bullets, bullet_mask, qkv=qkv, project=False)
                 tail = None
                 if merged.dtype == torch.bfloat16:
                     tail = self.ffn.train_tail(x0, merged, self.norm2, proj_layer=self.out_proj)
@@ -794,8 +815,11 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
     def _sequence_autograd(self, x_seq, h0, conv_buf, done_mask, time_major):
         """Training path: torch ops (differentiable) around the recurrence, which runs on its
         forward and backward kernels."""
-        x_seq, normed = _train_norm(self.norm1, x_seq)
-        b1 = _project(self.linear1, normed)
+        if _norm_linear_train_ok(x_seq, _projection_dtype(), self.norm1, self.linear1):
+            x_seq, b1, normed = _norm_linear_train(x_seq, self.norm1, self.linear1)
+        else:
+            x_seq, normed = _train_norm(self.norm1, x_seq)
+            b1 = _project(self.linear1, normed)
         if (_TRAIN_KERNELS and ops.conv_seq_train_supported(b1) and conv_buf.dtype == torch.float32
                 and self.conv.weight.dtype == torch.float32):
             # conv forward and backward on their kernels (one pass each instead of a dozen element-wise ops per tap)
@@ -826,8 +850,11 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
                 and _projection_dtype() == torch.bfloat16 and conv_buf.dtype == torch.float32
                 and self.conv.weight.dtype == torch.float32):
             return None
-        x, normed = _train_norm(self.norm1, x)
-        b1 = _project(self.linear1, normed)
+        if _norm_linear_train_ok(x, torch.bfloat16, self.norm1, self.linear1):
+            x, b1, normed = _norm_linear_train(x, self.norm1, self.linear1)
+        else:
+            x, normed = _train_norm(self.norm1, x)
+            b1 = _project(self.linear1, normed)
         if b1.dtype != torch.bfloat16 or b1.shape[-1] != ops.FFN_WIDTH:
             return None
         ships_b1, fields_b1 = _SplitTokens.apply(b1, n_rec)

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 23
+#define BNB_ABI_VERSION 24
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -650,6 +650,18 @@ int bnb_norm_linear_fwd(const float *x, int64_t x_row_stride, const int32_t *row
                         const int32_t *n_rows, const float *norm_weight, float eps,
                         const void *weight_packed, const float *bias, void *out,
                         int64_t R, int D, int N, void *stream);
+
+/*
+ * bnb_norm_linear_fwd for the PPO update (train/rl/ppo.py:1417-1425 re-evaluates the rollout in grad mode): the same
+ * launch also writes the normalised rows the projection multiplied, n = bf16(rmsnorm(x) * norm_weight), which are what
+ * autograd would keep of `self.qkv(self.norm1(x))` (models/yemong/attention.py:94-96,132) and
+ * `self.linear1(self.norm1(x))` (models/yemong/griffin.py:269-272) for the weight gradient; the norm's own forward
+ * launch and the re-read of n by the projection disappear.
+ *   n_out   (R, 128) bf16 contiguous
+ *   other arguments as bnb_norm_linear_fwd (all rows, no bias)
+ */
+int bnb_norm_linear_train_fwd(const float *x, int64_t x_row_stride, const float *norm_weight, float eps,
+                              const void *weight_packed, void *out, void *n_out, int64_t R, int D, int N, void *stream);
 
 /*
  * A float32 Linear layer with its neighbours folded in, on the fp32 matrix cores (true fp32 products):

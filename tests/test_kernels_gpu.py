@@ -2625,3 +2625,54 @@ def test_linear_f32_reads_column_blocks_in_place_and_writes_into_the_residual():
                        norm_weight=torch.ones(256, device=DEV))  # the norm prologue is for width 128
     with pytest.raises(ValueError):
         ops.pack_linear_f32(torch.zeros(48, 128))
+
+
+# ------------------------------------------------------------------ norm + projection of the update (forward kernel writes n)
+
+
+@pytest.mark.parametrize("R,N", [(1, 128), (130, 384), (8192, 384), (20000, 128)])
+def test_norm_linear_train_forward_and_gradients_match_autograd_of_the_oracle(R, N):
+    g = torch.Generator().manual_seed(R + N)
+    D = 128
+    x = 2.0 * torch.randn(R, D, generator=g)
+    nw = 1.0 + 0.1 * torch.randn(D, generator=g)
+    W = torch.randn(N, D, generator=g) / D ** 0.5
+    dy = torch.randn(R, N, generator=g).bfloat16()
+    ds = torch.randn(R, D, generator=g)
+    dn_other = torch.randn(R, D, generator=g).bfloat16()
+    xd, nwd, Wd = x.to(DEV).requires_grad_(), nw.to(DEV).requires_grad_(), W.to(DEV).requires_grad_()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        x_out, y, n = ops.norm_linear_train(xd, nwd, Wd)
+    assert y.dtype == torch.bfloat16 and n.dtype == torch.bfloat16 and x_out.data_ptr() == xd.data_ptr()
+    # forward: the inference kernel bit for bit; n the bf16 rows of the oracle's norm
+    with torch.no_grad():
+        assert torch.equal(y, ops.norm_linear(xd.detach(), nwd.detach(), ops.pack_linear_weights(Wd.detach())))
+    n_ref = torch_ref.rms_norm(x, nw)
+    assert max_rel(n.float().cpu(), n_ref) <= BF16_TOL
+    # backward against float64 autograd through the oracle on the bf16-rounded weight
+    xr, nwr = x.double().requires_grad_(), nw.double().requires_grad_()
+    Wr = W.bfloat16().double().requires_grad_()
+    nr = torch_ref.rms_norm(xr, nwr)
+    yr = nr @ Wr.t()
+    (yr * dy.double()).sum().add((xr * ds.double()).sum()).add((nr * dn_other.double()).sum()).backward()
+    torch.autograd.backward([x_out, y, n], [ds.to(DEV), dy.to(DEV), dn_other.to(DEV)])
+    assert max_rel(xd.grad.cpu(), xr.grad.float()) <= BF16_TOL
+    assert max_rel(Wd.grad.cpu(), Wr.grad.float()) <= BF16_TOL
+    assert max_rel(nwd.grad.cpu(), nwr.grad.float()) <= BF16_TOL
+
+
+def test_norm_linear_train_refuses_what_the_kernel_does_not_cover():
+    from boost_and_broadside_amd import _native
+
+    lib = _native.load()
+    x = torch.zeros(16, 128, device=DEV)
+    w = torch.ones(128, device=DEV)
+    pk = ops.pack_linear_weights(torch.zeros(128, 128, device=DEV))
+    y = torch.empty(16, 128, dtype=torch.bfloat16, device=DEV)
+    n = torch.empty(16, 128, dtype=torch.bfloat16, device=DEV)
+    args = lambda D, N, n_ptr: (x.data_ptr(), 128, w.data_ptr(), 1e-6, pk.data_ptr(), y.data_ptr(), n_ptr, 16, D, N, None)
+    assert lib.bnb_norm_linear_train_fwd(*args(128, 128, n.data_ptr())) == 0
+    assert lib.bnb_norm_linear_train_fwd(*args(64, 128, n.data_ptr())) == _native.ERR_UNSUPPORTED
+    assert lib.bnb_norm_linear_train_fwd(*args(128, 96, n.data_ptr())) == _native.ERR_UNSUPPORTED
+    assert lib.bnb_norm_linear_train_fwd(*args(128, 128, None)) == 10001  # BNB_ERR_NULL_POINTER
+    assert not ops.norm_linear_train_supported(x, torch.zeros(64, 128, device=DEV))  # the weight-gradient kernel wants 128s
