@@ -1473,7 +1473,8 @@ def test_ffn_fused_with_folded_projection_matches_oracle(R, gated):
     assert max_rel(got.cpu(), two_step.cpu()) <= 1e-2
 
 
-@pytest.mark.parametrize("R,N", [(1, 128), (37, 384), (128, 256), (130, 384), (5000, 256), (4096, 384)])
+@pytest.mark.parametrize("R,N", [(1, 128), (37, 384), (128, 256), (130, 384), (5000, 256), (4096, 384), (700, 192), (3000, 320),
+                                 (260, 640)])
 @pytest.mark.parametrize("gated", [False, True])
 def test_ffn_fused_with_the_next_sublayers_head_matches_oracle(R, N, gated):
     # the same launch goes on to rmsnorm(out) * w2 -> bf16 -> @ Wh^T, the projection the next sublayer starts with
