@@ -234,3 +234,42 @@ def test_a_shape_outside_the_kernels_is_counted_and_warned_about_once():
         assert bnb.library_dispatches[site] == 2
         with bnb.forbid_library_dispatch(), pytest.raises(RuntimeError, match="library dispatch"):
             layer(x)
+
+
+@pytest.mark.parametrize("with_bullets", [False, True])
+def test_full_batch_trunk_steps_checked_on_sampled_environments(with_bullets):
+    # 64v88 x 4096 environments through the whole trunk (every kernel ten rounds of resident work-groups deep, the
+    # sublayer tails handing their successors the norm + projection), three carried steps with a reset folded into
+    # the last; environments are independent, so the oracle follows a sample of them
+    w = harness.WORKLOADS["c4_64v88_bf16"]
+    B, N, NM = w.B, w.N, w.NM
+    p = _params(400, with_bullets, round_bf16=True)
+    trunk = _trunk(p, with_bullets)
+    g = torch.Generator().manual_seed(9)
+    sample = torch.randperm(B, generator=g)[:6].sort().values
+    sample[0], sample[-1] = 0, B - 1
+    rows = (sample[:, None] * N + torch.arange(N)[None, :]).reshape(-1)  # state rows of the sampled environments
+    gd = torch.Generator(device=DEV).manual_seed(10)
+    hidden = trunk.initial_hidden(B, N, DEV)
+    ref_hidden = torch.zeros(2, sample.numel() * N, 4 * D)
+    alive = torch.rand(B, NM, device=DEV, generator=gd) < 0.8
+    alive[:, N:] = True
+    for t in range(3):
+        x = torch.randn(B, NM, D, device=DEV, generator=gd).bfloat16().float()
+        reset = torch.rand(B, device=DEV, generator=gd) < 0.3 if t == 2 else None
+        kw, ref_kw = {}, {}
+        if with_bullets:
+            bul = torch.randn(B, 10 * N, D, device=DEV, generator=gd).bfloat16().float()
+            bm = torch.rand(B, 10 * N, device=DEV, generator=gd) < 0.25
+            kw = {"bullets": bul, "bullet_mask": bm}
+            ref_kw = {"bullets": bul[sample.to(DEV)].cpu(), "bullet_mask": bm[sample.to(DEV)].cpu()}
+        with warnings.catch_warnings(), bnb.forbid_library_dispatch(), torch.autocast("cuda", dtype=torch.bfloat16):
+            warnings.simplefilter("error", bnb.LibraryDispatchWarning)
+            out, hidden = trunk(x, alive, hidden, reset_mask=reset, **kw)
+        if reset is not None:
+            ref_hidden = torch_ref.reset_hidden(ref_hidden, reset[sample.to(DEV)].cpu(), N)
+        ref_out, ref_hidden = torch_ref.trunk_step(p, 2, 2, 1, H, x[sample.to(DEV)].cpu(), alive[sample.to(DEV)].cpu(),
+                                                   ref_hidden, **ref_kw)
+        assert torch.isfinite(out).all() and torch.isfinite(hidden).all()
+        assert max_rel(out[sample.to(DEV)].cpu(), ref_out) <= BF16_TOL, t
+        assert max_rel(hidden[:, rows.to(DEV)].cpu(), ref_hidden) <= BF16_TOL, t

@@ -1281,3 +1281,49 @@ def test_graphed_trunk_with_handed_over_projections_replays_like_the_eager_step(
             out, new_state = graphed.step(x, alive)
         assert torch.equal(out, eager) and torch.equal(new_state, state), t
         assert max_rel(out.cpu(), apart.cpu()) <= BF16_TOL
+
+
+@pytest.mark.parametrize("bullets", [0, 1])
+def test_update_path_at_the_rollouts_size_agrees_with_the_library_ops(bullets):
+    """One block forward + backward at the size of a stored 4v4 rollout (128 steps x 256 environments x 12 tokens:
+    393,216 token rows, every update kernel several rounds of resident work-groups deep): every parameter gradient and
+    the input gradient agree with the same update through torch's own differentiable ops, twice in a row bit for bit."""
+    from boost_and_broadside_amd import trunk
+
+    cfg = _cfg(128, 4, spatial=2, temporal=1, bullets=bullets)
+    torch.manual_seed(70 + bullets)
+    block = bnb.YemongBlock(cfg).to(DEV)
+    T, B, N, M, D = 128, 256, 8, 4, 128
+    gen = torch.Generator(device=DEV).manual_seed(71)
+    x = torch.randn(T, B, N + M, D, device=DEV, generator=gen).requires_grad_()
+    alive = torch.rand(T, B, N + M, device=DEV, generator=gen) < 0.9
+    alive[..., 0] = True
+    h0 = torch.zeros(1, B * N, D, device=DEV)
+    cb0 = torch.zeros(1, B * N, 3, D, device=DEV)
+    done = torch.rand(T, B, device=DEV, generator=gen) < 0.02
+    go = torch.randn(T, B, N + M, D, device=DEV, generator=gen)
+    kw = {}
+    if bullets:
+        kw = {"bullets": torch.randn(T * B, N * 10, D, device=DEV, generator=gen),
+              "bullet_mask": torch.rand(T * B, N * 10, device=DEV, generator=gen) < 0.25}
+
+    def grads():
+        block.zero_grad(set_to_none=True)
+        x.grad = None
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = block.sequence(x, alive, h0, cb0, done, N, **kw)[0]
+        out.backward(go)
+        found = {n: p.grad.detach().clone() for n, p in block.named_parameters() if p.grad is not None}
+        found["tokens"] = x.grad.detach().clone()
+        return found
+
+    with trunk.forbid_library_dispatch():
+        routed = grads()
+        again = grads()
+    with trunk.library_update_path():
+        library = grads()
+    assert set(routed) == set(library)
+    for name, g in routed.items():
+        assert torch.isfinite(g).all(), name
+        assert torch.equal(g, again[name]), name  # fixed-order reductions everywhere
+        assert max_rel(g, library[name]) <= BF16_TOL, name
