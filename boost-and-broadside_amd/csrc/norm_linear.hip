@@ -86,14 +86,20 @@ __global__ __launch_bounds__(kNlThreads) void norm_linear_kernel(
     // channels arrive (the row never sits in registers as fp32), same relative rounding.
     bf16x8 nb[8];
     float ss = 0.0f;
+    // both passes' rows are requested before the first one is staged: one round trip to memory instead of two
+    f32x4 xv[2][8];
 #pragma unroll
     for (int pass = 0; pass < 2; ++pass) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const f32x4 v = __builtin_nontemporal_load(
+        for (int j = 0; j < 8; ++j)
+            xv[pass][j] = __builtin_nontemporal_load(
                 reinterpret_cast<const f32x4 *>(x + src_row[j] * x_stride + 64 * pass + io_col));
-            *reinterpret_cast<f32x4 *>(stage + (4 * j + io_row) * kNlHalfPitch + io_col) = v;
-        }
+    }
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            *reinterpret_cast<f32x4 *>(stage + (4 * j + io_row) * kNlHalfPitch + io_col) = xv[pass][j];
         __syncthreads();
 #pragma unroll
         for (int k4 = 0; k4 < 4; ++k4) {  // contraction step ks = 4 pass + k4: channels 16 ks + ...
