@@ -17,6 +17,7 @@ from .ops import conv_seq, conv_step, rglru_scan, rglru_step, sdpa_cross, sdpa_m
 from .trunk import (
     CONV_KERNEL,
     GatedMLP,
+    EagerTrunkStepper,
     GraphedTrunk,
     GriffinTemporalBlock,
     LibraryDispatchWarning,
@@ -28,12 +29,13 @@ from .trunk import (
     YemongTrunk,
     forbid_library_dispatch,
     separate_heads,
+    trunk_stepper,
     invalidate_weight_caches,
     library_dispatches,
 )
 
 __all__ = [
-    "CONV_KERNEL", "GatedMLP", "GraphedTrunk", "GriffinTemporalBlock", "ModelConfig", "RGLRU", "TeamPMA", "TransformerBlock",
+    "CONV_KERNEL", "GatedMLP", "GraphedTrunk", "EagerTrunkStepper", "trunk_stepper", "GriffinTemporalBlock", "ModelConfig", "RGLRU", "TeamPMA", "TransformerBlock",
     "YemongBlock", "YemongTrunk", "conv_seq", "conv_step", "rglru_scan", "rglru_step", "sdpa_cross", "sdpa_masked", "ops",
     "trunk", "harness", "LibraryDispatchWarning", "forbid_library_dispatch", "separate_heads", "invalidate_weight_caches", "library_dispatches",
 ]

@@ -1573,3 +1573,52 @@ class GraphedTrunk:
         out = self.outputs[self.cur]
         self.cur = 1 - self.cur
         return out, self.states[self.cur]
+
+
+class EagerTrunkStepper:
+    """``GraphedTrunk``'s interface on plain launches: the packed state alternates between two buffers it owns and
+    ``step(tokens, alive_mask, reset_mask)`` returns ``(hidden, new_state)``.  For batches large enough that the
+    kernels, not their launches, set the pace of a step."""
+
+    def __init__(self, trunk: YemongTrunk, num_envs: int, num_tokens: int, num_recurrent: int, *,
+                 autocast_dtype: torch.dtype | None = None, device=None) -> None:
+        dev = torch.device(device) if device is not None else next(trunk.parameters()).device
+        self.trunk, self.autocast_dtype = trunk, autocast_dtype
+        self.states = [trunk.initial_hidden(num_envs, num_recurrent, dev) for _ in range(2)]
+        self.cur = 0
+
+    def refresh_weights(self) -> None:
+        """Nothing to do: every step looks the weights up (the derived copies follow the parameters' version counters)."""
+
+    @property
+    def state(self) -> torch.Tensor:
+        return self.states[self.cur]
+
+    def load_state(self, state: torch.Tensor) -> None:
+        self.states[self.cur].copy_(state)
+
+    @torch.no_grad()
+    def step(self, tokens, alive_mask, reset_mask=None):
+        with torch.autocast("cuda", dtype=self.autocast_dtype or torch.bfloat16, enabled=self.autocast_dtype is not None):
+            out, new_state = self.trunk(tokens, alive_mask, self.states[self.cur], reset_mask=reset_mask,
+                                        out_state=self.states[1 - self.cur])
+        self.cur = 1 - self.cur
+        return out, new_state
+
+
+# tokens per step below which a captured step beats plain launches (measured on MI355X with the default trunk of
+# 2 blocks x (2 attention + 1 temporal sublayer)): the launches of a step take the host ~0.4 ms
+GRAPH_BELOW_TOKENS = {torch.float32: 10_000, torch.bfloat16: 40_000}
+
+
+def trunk_stepper(trunk: YemongTrunk, num_envs: int, num_tokens: int, num_recurrent: int, *,
+                  autocast_dtype: torch.dtype | None = None, graph: bool | None = None, device=None):
+    """The rollout's way to step the trunk for one fixed shape: a ``GraphedTrunk`` (the step captured into HIP graphs)
+    when ``num_envs * num_tokens`` is small enough that launches set the pace (``GRAPH_BELOW_TOKENS``), an
+    ``EagerTrunkStepper`` above that; ``graph`` forces either.  Both own the packed state and share
+    ``step`` / ``state`` / ``load_state`` / ``refresh_weights``."""
+    if graph is None:
+        graph = num_envs * num_tokens < GRAPH_BELOW_TOKENS[torch.float32 if autocast_dtype is None else torch.bfloat16]
+    if graph:
+        return GraphedTrunk(trunk, num_envs, num_tokens, num_recurrent, autocast_dtype=autocast_dtype, device=device)
+    return EagerTrunkStepper(trunk, num_envs, num_tokens, num_recurrent, autocast_dtype=autocast_dtype, device=device)

@@ -1327,3 +1327,28 @@ def test_update_path_at_the_rollouts_size_agrees_with_the_library_ops(bullets):
         assert torch.isfinite(g).all(), name
         assert torch.equal(g, again[name]), name  # fixed-order reductions everywhere
         assert max_rel(g, library[name]) <= BF16_TOL, name
+
+
+def test_trunk_stepper_picks_the_captured_step_for_small_batches_and_both_kinds_agree():
+    D, H, N, M = 128, 4, 8, 4
+    p = trunk_params(81, D, 2, 2, 1)
+    trunk = bnb.YemongTrunk(_cfg(D, H, 2, 2, 1)).eval()
+    trunk.load_state_dict(p)
+    trunk.to(DEV)
+    small = bnb.trunk_stepper(trunk, 16, N + M, N, autocast_dtype=torch.bfloat16)
+    assert isinstance(small, bnb.GraphedTrunk)
+    assert isinstance(bnb.trunk_stepper(trunk, 4096, N + M, N, autocast_dtype=torch.bfloat16), bnb.EagerTrunkStepper)
+    assert isinstance(bnb.trunk_stepper(trunk, 1024, N + M, N), bnb.EagerTrunkStepper)  # 12,288 tokens in float32
+    plain = bnb.trunk_stepper(trunk, 16, N + M, N, autocast_dtype=torch.bfloat16, graph=False)
+    assert isinstance(plain, bnb.EagerTrunkStepper)
+    gen = torch.Generator().manual_seed(82)
+    alive = torch.ones(16, N + M, dtype=torch.bool, device=DEV)
+    for t in range(4):
+        x = torch.randn(16, N + M, D, generator=gen).to(DEV)
+        done = (torch.rand(16, generator=gen) < 0.3).to(DEV) if t == 2 else None
+        out_a, state_a = small.step(x, alive, done)
+        out_b, state_b = plain.step(x, alive, done)
+        assert torch.equal(out_a, out_b) and torch.equal(state_a, state_b), t
+        assert torch.equal(plain.state, state_b)
+    plain.load_state(torch.zeros_like(plain.state))
+    assert plain.state.abs().max() == 0
