@@ -933,13 +933,32 @@ def main():
         # a producer that writes tokens and mask straight into the capture's input buffers: no staging copies
         wall_gi = timed_loop(lambda t: graphed.step(graphed.tokens, graphed.alive, graphed.reset), n_tr, 4)
         del graphed
+        # the shipped default (config/defaults.py:21-31) also reads the bullets in flight in the first attention sublayer
+        # of each block: 10 slots per ship, a quarter of them live here
+        wall_tb = None
+        if not args.no_bullets and bf16:
+            cfg_tb = bnb.ModelConfig(d_model=D, n_heads=H, n_yemong_blocks=2, n_spatial_per_block=2, n_temporal_per_block=1,
+                                     n_bullet_cross_per_block=1)
+            torch.manual_seed(w.seed)
+            trunk_b = bnb.YemongTrunk(cfg_tb).to(dev).eval()
+            bul_t = torch.randn(w.B, w.N * 10, D, device=dev, generator=gen)
+            bm_t = torch.rand(w.B, w.N * 10, device=dev, generator=gen) < 0.25
+
+            def trunk_step_bullets(t):
+                with torch.autocast("cuda", dtype=torch.bfloat16):
+                    trunk_b(x32[t & 1], alive_steps[t % n_alive], hid[t & 1], bul_t, bm_t, out_state=hid[(t + 1) & 1])
+
+            wall_tb = timed_loop(trunk_step_bullets, n_tr, 6)
+            del trunk_b, bul_t, bm_t
         result["trunk"] = {
             "value": tokens * n_tr / wall_tr, "unit": "entity-tokens/s", "ms_per_step": wall_tr / n_tr * 1e3,
             "hip_graph_ms_per_step": wall_g / n_tr * 1e3,
             "hip_graph_inputs_in_place_ms_per_step": wall_gi / n_tr * 1e3,
+            "with_bullet_read_ms_per_step": None if wall_tb is None else wall_tb / n_tr * 1e3,
             "steps": n_tr, "eager_torch_ms_per_step": wall_te / n_tr * 1e3, "speedup_over_eager_torch": wall_te / wall_tr,
             "what": "YemongTrunk.forward, 2 blocks x (2 attention + 1 temporal sublayer), d_model 128, packed fp32 state "
-                    "carried, " + ("bf16 autocast" if bf16 else "fp32") + "; eager = same modules with the kernels "
+                    "carried, " + ("bf16 autocast" if bf16 else "fp32") + "; with_bullet_read = the shipped default, whose first "
+                    "attention sublayer of each block also reads the bullets in flight (10 slots per ship, 25 % live); eager = same modules with the kernels "
                     "replaced by the reference's torch ops and its unpack/cat/re-pack of the state",
         }
         del trunk, hid, ref_h

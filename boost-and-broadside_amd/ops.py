@@ -2282,6 +2282,7 @@ class CompactRows:
         if (total is None) != (max_count is None):
             raise ValueError("give both total and max_count, or neither")
         self._host = None if total is None else (int(total), int(max_count))
+        self.shared_kv = None  # set by the trunk: {id(layer): [K | V] rows of the listed entries}, one projection pass for all readers
         counts = torch.empty(B, dtype=torch.int32, device=mask.device)
         self.offsets = torch.zeros(B + 1, dtype=torch.int32, device=mask.device)
         self.index = torch.empty(max(B * n, 1), dtype=torch.int32, device=mask.device)
@@ -2389,8 +2390,8 @@ def sdpa_cross_rows(
     if not (qkv.is_cuda and qkv.dtype == torch.bfloat16 and kv_rows.dtype == torch.bfloat16 and D % n_heads == 0
             and D // n_heads == 32 and NQ <= 160):
         raise RuntimeError("sdpa_cross_rows covers bfloat16, head size 32 and at most 160 queries")
-    if kv_rows.dim() != 2 or kv_rows.shape[1] != 2 * D or not kv_rows.is_contiguous():
-        raise ValueError(f"kv_rows must be a contiguous (capacity, {2 * D}) tensor")
+    if kv_rows.dim() != 2 or kv_rows.shape[1] != 2 * D or kv_rows.stride(1) != 1 or kv_rows.stride(0) % 8:
+        raise ValueError(f"kv_rows must be a (capacity, {2 * D}) tensor with unit column stride (a column block of a wider one is fine)")
     need = rows.shape[0] * rows.shape[1] if total is None else total  # without the host-side count: room for every entry
     if rows.shape[0] != B or kv_rows.shape[0] < need:
         raise ValueError("rows was built for a different batch, or kv_rows is smaller than its capacity")

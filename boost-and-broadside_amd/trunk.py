@@ -603,9 +603,11 @@ class TransformerBlock(_WeightCaches, nn.Module):
             if rows is not None and self._compact_read_ok(qkv, bullets):
                 # only the bullets in flight are normalised and projected (one kernel over a
                 # device-side list of them), and the read walks each environment's run of rows
-                w = self.kv_bullet.weight
-                pk = _cached_cast(self.kv_bullet, "_bnb_pack", (w,), torch.bfloat16, lambda: ops.pack_linear_weights(w))
-                kv_rows = ops.norm_linear(bullets, self.norm_bullet.weight, pk, eps=self.norm_bullet.eps, rows=rows)
+                kv_rows = rows.shared_kv.get(id(self)) if rows.shared_kv is not None else None
+                if kv_rows is None:
+                    w = self.kv_bullet.weight
+                    pk = _cached_cast(self.kv_bullet, "_bnb_pack", (w,), torch.bfloat16, lambda: ops.pack_linear_weights(w))
+                    kv_rows = ops.norm_linear(bullets, self.norm_bullet.weight, pk, eps=self.norm_bullet.eps, rows=rows)
                 merged = ops.sdpa_cross_rows(qkv, kv_rows, rows, self.n_heads, accum=merged)
                 return _project(self.out_proj, merged) if project else merged
             if rows is not None:
@@ -1424,6 +1426,37 @@ class YemongTrunk(_WeightCaches, nn.Module):
                 x = run(x)
         return x
 
+    def _bullet_kv_of_all_layers(self, bullets, rows):
+        """``{id(layer): [K | V] rows}`` of every bullet-reading sublayer of the step from ONE pass over the bullets in
+        flight, or None when there are fewer than two such sublayers (or their norms differ in eps).
+
+        Every reading sublayer normalises the same bullet tokens with its own ``norm_bullet`` weight and projects them
+        with its own ``kv_bullet`` (attention.py:149-151).  The normalised row is the same up to that weight, which
+        folds into the projection's columns: ``(x^ * w) W^T = x^ (W * w)^T``.  So the live bullets are gathered and
+        normalised once and projected onto the folded weights of all layers side by side; a layer reads its column
+        block.  (The operand is then ``bf16(x^)`` against ``bf16(W * w)`` instead of ``bf16(x^ * w)`` against
+        ``bf16(W)``: a bfloat16 rounding apart, like the other folded products.)"""
+        readers = [layer for block in self.yemong_layers for layer in block.spatial if layer.reads_bullets]
+        if (len(readers) < 2 or torch.is_grad_enabled() or any(l.kv_bullet.bias is not None for l in readers)
+                or any(l.norm_bullet.weight is None or l.norm_bullet.eps != readers[0].norm_bullet.eps for l in readers)):
+            return None
+        D = self.config.d_model
+        # a layer's column block is addressed with 32-bit element offsets over the full slot capacity
+        if bullets.shape[0] * bullets.shape[1] * 2 * D * len(readers) >= 2 ** 32:
+            return None
+        ws = tuple(t for l in readers for t in (l.kv_bullet.weight, l.norm_bullet.weight))
+
+        def folded():
+            with torch.autocast("cuda", enabled=False):
+                return ops.pack_linear_weights(torch.cat(
+                    [l.kv_bullet.weight.detach().float() * l.norm_bullet.weight.detach().float()[None, :] for l in readers], dim=0))
+
+        pk = _cached_cast(self, "_bnb_bullet_kv_pack", ws, torch.bfloat16, folded)
+        ones = _cached_cast(self, "_bnb_unit_norm", (readers[0].norm_bullet.weight,), torch.float32,
+                            lambda: torch.ones(D, dtype=torch.float32, device=bullets.device))
+        kv = ops.norm_linear(bullets, ones, pk, eps=readers[0].norm_bullet.eps, rows=rows)  # (capacity, 2 D x layers)
+        return {id(l): kv[:, 2 * D * i:2 * D * (i + 1)] for i, l in enumerate(readers)}
+
     @torch.no_grad()
     def forward(self, tokens, alive_mask, recurrent_state, bullets=None, bullet_mask=None, *, reset_mask=None,
                 out_state=None):
@@ -1460,6 +1493,7 @@ class YemongTrunk(_WeightCaches, nn.Module):
             and D // self.config.n_heads == 32 and NM <= 160
         ):
             bullet_rows = ops.CompactRows(bullet_mask)
+            bullet_rows.shared_kv = self._bullet_kv_of_all_layers(bullets, bullet_rows)
         x, widened = _widen_tokens(tokens)
         blocks = list(self.yemong_layers)
         head = None

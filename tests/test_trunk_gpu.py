@@ -1352,3 +1352,42 @@ def test_trunk_stepper_picks_the_captured_step_for_small_batches_and_both_kinds_
         assert torch.equal(plain.state, state_b)
     plain.load_state(torch.zeros_like(plain.state))
     assert plain.state.abs().max() == 0
+
+
+def test_bullet_reading_layers_share_one_projection_pass_over_the_live_bullets(monkeypatch):
+    """Two blocks, each with one bullet-reading sublayer: the live bullets are gathered, normalised and projected once
+    per step (the layers' norm weights folded into their projections), and the result stays within the bf16 bar of the
+    oracle and of the step in which every layer projects for itself."""
+    from boost_and_broadside_amd import trunk as trunk_module
+
+    D, H, B, N, M = 128, 4, 9, 8, 4
+    p = trunk_params(91, D, 2, 2, 1)
+    pg = torch.Generator().manual_seed(92)
+    for i in range(2):
+        p[f"yemong_layers.{i}.spatial.0.norm_bullet.weight"] = 1.0 + 0.3 * torch.randn(D, generator=pg)
+        p[f"yemong_layers.{i}.spatial.0.kv_bullet.weight"] = 0.15 * torch.randn(2 * D, D, generator=pg)
+    trunk = bnb.YemongTrunk(_cfg(D, H, 2, 2, 1, bullets=1)).eval()
+    trunk.load_state_dict(p)
+    trunk.to(DEV)
+    ops = trunk_module.ops
+    calls = []
+    real = ops.norm_linear
+    monkeypatch.setattr(ops, "norm_linear", lambda x, *a, **k: (calls.append(k.get("rows") is not None), real(x, *a, **k))[1])
+    gen = torch.Generator().manual_seed(93)
+    x = torch.randn(B, N + M, D, generator=gen)
+    alive = torch.rand(B, N + M, generator=gen) < 0.9
+    alive[:, 0] = True
+    bul = torch.randn(B, 10 * N, D, generator=gen)
+    bm = torch.rand(B, 10 * N, generator=gen) < 0.3
+    bm[2] = False  # an environment with nothing in flight
+    hidden = trunk.initial_hidden(B, N, DEV)
+    with torch.autocast("cuda", dtype=torch.bfloat16), trunk_module.forbid_library_dispatch():
+        out, state = trunk(x.to(DEV), alive.to(DEV), hidden, bul.to(DEV), bm.to(DEV))
+        assert sum(calls) == 1  # one pass over the bullets in flight for both readers
+        calls.clear()
+        monkeypatch.setattr(bnb.YemongTrunk, "_bullet_kv_of_all_layers", lambda self, bullets, rows: None)
+        apart, state_b = trunk(x.to(DEV), alive.to(DEV), hidden, bul.to(DEV), bm.to(DEV))
+        assert sum(calls) == 2
+    ref_out, ref_state = torch_ref.trunk_step(p, 2, 2, 1, H, x, alive, torch.zeros(2, B * N, 4 * D), bullets=bul, bullet_mask=bm)
+    assert max_rel(out.cpu(), ref_out) <= BF16_TOL and max_rel(state.cpu(), ref_state) <= BF16_TOL
+    assert max_rel(out.cpu(), apart.cpu()) <= BF16_TOL and max_rel(state.cpu(), state_b.cpu()) <= BF16_TOL
