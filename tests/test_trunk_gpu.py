@@ -1381,6 +1381,7 @@ def test_bullet_reading_layers_share_one_projection_pass_over_the_live_bullets(m
     bm = torch.rand(B, 10 * N, generator=gen) < 0.3
     bm[2] = False  # an environment with nothing in flight
     hidden = trunk.initial_hidden(B, N, DEV)
+    shared = bnb.YemongTrunk._bullet_kv_of_all_layers
     with torch.autocast("cuda", dtype=torch.bfloat16), trunk_module.forbid_library_dispatch():
         out, state = trunk(x.to(DEV), alive.to(DEV), hidden, bul.to(DEV), bm.to(DEV))
         assert sum(calls) == 1  # one pass over the bullets in flight for both readers
@@ -1391,3 +1392,15 @@ def test_bullet_reading_layers_share_one_projection_pass_over_the_live_bullets(m
     ref_out, ref_state = torch_ref.trunk_step(p, 2, 2, 1, H, x, alive, torch.zeros(2, B * N, 4 * D), bullets=bul, bullet_mask=bm)
     assert max_rel(out.cpu(), ref_out) <= BF16_TOL and max_rel(state.cpu(), ref_state) <= BF16_TOL
     assert max_rel(out.cpu(), apart.cpu()) <= BF16_TOL and max_rel(state.cpu(), state_b.cpu()) <= BF16_TOL
+
+    # an optimizer-style update of one reader's bullet weights: the folded matrix is rebuilt for the next step
+    monkeypatch.setattr(bnb.YemongTrunk, "_bullet_kv_of_all_layers", shared)
+    with torch.no_grad():
+        trunk.yemong_layers[1].spatial[0].norm_bullet.weight.mul_(-0.5)
+        trunk.yemong_layers[0].spatial[0].kv_bullet.weight.add_(0.05)
+    p2 = {k: v.detach().cpu().clone() for k, v in trunk.state_dict().items()}
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out2, state2 = trunk(x.to(DEV), alive.to(DEV), hidden, bul.to(DEV), bm.to(DEV))
+    ref2, ref_state2 = torch_ref.trunk_step(p2, 2, 2, 1, H, x, alive, torch.zeros(2, B * N, 4 * D), bullets=bul, bullet_mask=bm)
+    assert max_rel(out2.cpu(), ref2) <= BF16_TOL and max_rel(state2.cpu(), ref_state2) <= BF16_TOL
+    assert max_rel(ref2, ref_out) > 10 * BF16_TOL  # the update did change the result
