@@ -763,28 +763,41 @@ __global__ __launch_bounds__(1024) void sdpa_mfma_f32_kernel(
 // The bullet axis is N*K slots long (80 .. 1520 in the shipped scenarios) and mostly
 // empty: only bullets in flight are keys.  One work-group per (environment, head), one
 // wave per 32 queries.  The work-group first compacts the indices of the live bullets
-// into LDS, then walks them in tiles of 32*NQB keys: the K rows and transposed V rows of
+// into LDS, then walks them in tiles of 32 keys per wave: the K rows and transposed V rows of
 // the next tile are gathered from global memory into registers while the matrix cores
 // work on the current tile out of LDS (two LDS buffers, one barrier per tile), with the
 // running maximum / sum / output of an online softmax carried across tiles.  Key
 // positions, operand layouts and the output stage are those of sdpa_mfma_kernel.
 
+//
+// Waves per work-group: a CU places a work-group only while every one of its four SIMDs has room for
+// ceil(waves / 4) more waves, and the waves of a work-group move in step (one barrier per tile), so a
+// work-group of five waves runs at the pace of the SIMD that holds two of them.  Hence never more than
+// four waves: with five blocks of queries (129 .. 160 queries) waves 0..3 own blocks 0..3, and the fifth
+// block is shared - in every tile of 128 keys wave w takes its key block w for those 32 queries, with its
+// own running maximum, sum and output, and the four partial results are merged through LDS at the end.
+
 constexpr int kStreamMaxKeys = 2048;
 
 template <int NQB>
-__global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
+__global__ __launch_bounds__(kWave *(NQB < 4 ? NQB : 4), 3) void sdpa_cross_stream_kernel(
     const uint16_t *__restrict__ q, int64_t q_stride, const uint16_t *__restrict__ k,
     const uint16_t *__restrict__ v, int64_t kv_stride, const uint8_t *__restrict__ alive,
     const int32_t *__restrict__ ranges, const uint16_t *accum, uint16_t *out, int B, int NQ, int NK, int H,
     float scale_log2e)
 {
-    constexpr int TK = 32 * NQB;  // keys per tile
+    constexpr int NW = NQB < 4 ? NQB : 4;  // waves, and key blocks per tile
+    constexpr bool SPLIT = NQB > NW;       // a fifth block of queries, shared by the four waves
+    static_assert(NQB <= 5, "at most one shared block of queries");
+    constexpr int TK = 32 * NW;   // keys per tile
     constexpr int VP = TK + 4;    // halfs per V^T row: 8-byte aligned, bank-spread
-    constexpr int NT = kWave * NQB;
+    constexpr int NT = kWave * NW;
     __shared__ __align__(16) uint16_t s_k[2][TK * kKeyPitch];
     __shared__ __align__(16) uint16_t s_vt[2][kDh * VP];
     __shared__ uint16_t s_idx[kStreamMaxKeys];  // indices of the live keys, ascending
-    __shared__ int s_wcnt[NQB];
+    __shared__ int s_wcnt[NW];
+    static_assert(!SPLIT || sizeof(s_k) >= (size_t)NW * (16 * kWave + 2 * 32) * sizeof(float),
+                  "the partial results of the shared block are merged through the K buffers");
 
     const int chunk = gridDim.x >> 3;
     const int logical = (blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
@@ -806,6 +819,16 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
                          (uint32_t)(head * kDh + half * 8);
     const u32x4 qw0 = *reinterpret_cast<const u32x4 *>(qp);
     const u32x4 qw1 = *reinterpret_cast<const u32x4 *>(qp + 16);
+    // the shared block of queries (rows 32 NW ..)
+    const int srow = NW * 32 + m;
+    const int ssafe = srow < NQ ? srow : NQ - 1;
+    u32x4 sw0 = {0u, 0u, 0u, 0u}, sw1 = {0u, 0u, 0u, 0u};
+    if (SPLIT) {
+        const uint16_t *sp = q + (int64_t)env * NQ * q_stride + (uint32_t)ssafe * (uint32_t)q_stride +
+                             (uint32_t)(head * kDh + half * 8);
+        sw0 = *reinterpret_cast<const u32x4 *>(sp);
+        sw1 = *reinterpret_cast<const u32x4 *>(sp + 16);
+    }
 
     // Two ways to name the live keys of the environment: `ranges` (the K/V rows were already
     // compacted: rows ranges[env] .. ranges[env+1]-1 of one list for all environments), or a
@@ -850,7 +873,7 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
         int base = 0;
         cnt = 0;
 #pragma unroll
-        for (int w = 0; w < NQB; ++w) {
+        for (int w = 0; w < NW; ++w) {
             const int c = s_wcnt[w];
             if (w < wave) base += c;
             cnt += c;
@@ -868,7 +891,7 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
 
     const int nkb = (cnt + 31) >> 5;
     const int pad = nkb * 32 - cnt;  // positions [0, pad) of the first key block hold no key
-    const int ntiles = (nkb + NQB - 1) / NQB;
+    const int ntiles = (nkb + NW - 1) / NW;
 
     // thread -> (position in tile, 8 channels), two items per thread
     const uint32_t stride32 = (uint32_t)kv_stride;
@@ -912,8 +935,13 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
 
     const bf16x8 qb0 = __builtin_bit_cast(bf16x8, qw0);
     const bf16x8 qb1 = __builtin_bit_cast(bf16x8, qw1);
+    const bf16x8 sb0 = __builtin_bit_cast(bf16x8, sw0);
+    const bf16x8 sb1 = __builtin_bit_cast(bf16x8, sw1);
     float mx = -INFINITY, sum = 0.0f;
     f32x16 o = {0.0f};
+    // this wave's part of the shared block: its own maximum, sum and output over the key blocks it takes
+    float smx = -INFINITY, ssum = 0.0f;
+    f32x16 so = {0.0f};
 
     // the rows this lane will add its result to, fetched while the first tile is gathered
     const int64_t o_off = ((int64_t)env * NQ + qsafe) * D + head * kDh + 8 * half;
@@ -934,31 +962,32 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
     for (int t = 0; t < ntiles; ++t) {
         const int buf = t & 1;
         if (t + 1 < ntiles) gather(t + 1);
-        int nb = nkb - t * NQB;
-        nb = nb < NQB ? nb : NQB;
+        int nb = nkb - t * NW;
+        nb = nb < NW ? nb : NW;
         // K Q^T of key block kb.  Only the very first key block can hold padding positions; they
         // get -inf there.  The empty asm keeps that rare fix-up a real branch: folded into
         // selects it would cost 16 extra instructions in every key block.
-        auto scores = [&](int kb) -> f32x16 {
+        auto scores_of = [&](int kb, const bf16x8 &q0, const bf16x8 &q1) -> f32x16 {
             const uint16_t *kp = &s_k[buf][(kb * 32 + m) * kKeyPitch + half * 8];
             const bf16x8 ka0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp));
             const bf16x8 ka1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + 16));
             f32x16 z = {0.0f};
-            z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0, qb0, z, 0, 0, 0);
-            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka1, qb1, z, 0, 0, 0);
+            z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0, q0, z, 0, 0, 0);
+            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka1, q1, z, 0, 0, 0);
         };
+        auto scores = [&](int kb) -> f32x16 { return scores_of(kb, qb0, qb1); };
         auto mask_padding = [&](f32x16 &z) {
             asm volatile("" ::: "memory");
 #pragma unroll
             for (int e = 0; e < 16; ++e)
                 if (8 * (e >> 2) + 4 * half + (e & 3) < pad) z[e] = -INFINITY;
         };
-        auto weigh = [&](int kb, const f32x16 &z, float mc) {
+        auto weigh_into = [&](int kb, const f32x16 &z, float mc, float &total, f32x16 &acc) {
             float p[16];
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 p[e] = __builtin_amdgcn_exp2f(fmaf(z[e], scale_log2e, -mc));
-                sum += p[e];
+                total += p[e];
             }
 #pragma unroll
             for (int h2 = 0; h2 < 2; ++h2) {
@@ -969,9 +998,10 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
                 const u32x2 lo = *reinterpret_cast<const u32x2 *>(vp);
                 const u32x2 hi = *reinterpret_cast<const u32x2 *>(vp + 8);
                 const u32x4 vq = {lo.x, lo.y, hi.x, hi.y};
-                o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vq), pb, o, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vq), pb, acc, 0, 0, 0);
             }
         };
+        auto weigh = [&](int kb, const f32x16 &z, float mc) { weigh_into(kb, z, mc, sum, o); };
         if (wave * 32 < NQ) {
             // two key blocks per iteration: two independent MFMA chains in flight
             float tmx = -INFINITY;
@@ -1011,11 +1041,73 @@ __global__ __launch_bounds__(kWave * NQB) void sdpa_cross_stream_kernel(
                 weigh(kb, z0, mc);
             }
         }
+        if (SPLIT && wave < nb) {
+            // the shared block of queries against key block `wave` of the tile: one online-softmax step
+            f32x16 z = scores_of(wave, sb0, sb1);
+            if (t == 0 && wave == 0 && pad != 0) mask_padding(z);
+            float tmx = z[0];
+#pragma unroll
+            for (int e = 1; e < 16; ++e) tmx = fmaxf(tmx, z[e]);
+            tmx = fmaxf(tmx, __shfl_xor(tmx, 32));
+            const float mnew = fmaxf(smx, tmx);  // finite: the key block holds at least one live key
+            const float alpha = __builtin_amdgcn_exp2f((smx - mnew) * scale_log2e);  // 0 the first time
+            smx = mnew;
+            ssum *= alpha;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) so[e] *= alpha;
+            weigh_into(wave, z, smx * scale_log2e, ssum, so);
+        }
         if (t + 1 < ntiles) stash(t + 1, buf ^ 1);
         __syncthreads();
     }
     sum += __shfl_xor(sum, 32);
     const float inv = cnt == 0 ? 0.0f : __builtin_amdgcn_rcpf(sum);
+
+    if (SPLIT) {
+        // Merge the four partial results of the shared block.  Every wave has passed the barrier of the last tile,
+        // so the K buffers are free: o as [wave][e][lane], then maximum and sum as [wave][query].
+        float *part = reinterpret_cast<float *>(&s_k[0][0]);
+        float *stat = part + NW * 16 * kWave;
+        ssum += __shfl_xor(ssum, 32);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) part[(wave * 16 + e) * kWave + lane] = so[e];
+        if (half == 0) {
+            stat[(wave * 2 + 0) * 32 + m] = smx;
+            stat[(wave * 2 + 1) * 32 + m] = ssum;
+        }
+        __syncthreads();
+        // wave w finishes accumulator registers 4w .. 4w+3 of the 32 queries: rows 8w + 4*half + 0..3 of V^T as it
+        // lies in LDS, which the stash fills so that they are channels 16 (w / 2) + 8*half + 4 (w % 2) + 0..3
+        float mall = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < NW; ++j) mall = fmaxf(mall, stat[(j * 2 + 0) * 32 + m]);
+        float total = 0.0f;
+        float r[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < NW; ++j) {
+            const float mj = stat[(j * 2 + 0) * 32 + m];
+            // a wave that met no key block holds (-inf, 0, 0); with no key at all every part is like that
+            const float f = mj == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f((mj - mall) * scale_log2e);
+            total = fmaf(f, stat[(j * 2 + 1) * 32 + m], total);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) r[i] = fmaf(f, part[(j * 16 + wave * 4 + i) * kWave + lane], r[i]);
+        }
+        const float sinv = cnt == 0 ? 0.0f : __builtin_amdgcn_rcpf(total);
+        if (srow < NQ) {
+            const int64_t at = ((int64_t)env * NQ + srow) * D + head * kDh + 16 * (wave >> 1) + 8 * half + 4 * (wave & 1);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) r[i] *= sinv;
+            if (accum != nullptr) {
+                // bf16 + bf16 as torch adds them: the read result is rounded first, then the sum
+                const u32x2 aw = *reinterpret_cast<const u32x2 *>(accum + at);
+                r[0] = __uint_as_float(aw.x << 16) + round_to_bf16(r[0]);
+                r[1] = __uint_as_float(aw.x & 0xffff0000u) + round_to_bf16(r[1]);
+                r[2] = __uint_as_float(aw.y << 16) + round_to_bf16(r[2]);
+                r[3] = __uint_as_float(aw.y & 0xffff0000u) + round_to_bf16(r[3]);
+            }
+            *reinterpret_cast<u32x2 *>(out + at) = u32x2{pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
+        }
+    }
 
     {
         u32x4 w[2];
@@ -1146,7 +1238,7 @@ static int launch_cross_stream(const void *q, int64_t q_stride, const void *k, c
     const int64_t blocks = (pairs + 7) / 8 * 8;
     if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
     const float scale_log2e = kLog2eA / sqrtf((float)kDh);
-    hipLaunchKernelGGL((sdpa_cross_stream_kernel<NQB>), dim3((unsigned)blocks), dim3(kWave * NQB), 0, stream,
+    hipLaunchKernelGGL((sdpa_cross_stream_kernel<NQB>), dim3((unsigned)blocks), dim3(kWave * (NQB < 4 ? NQB : 4)), 0, stream,
                        (const uint16_t *)q, q_stride, (const uint16_t *)k, (const uint16_t *)v, kv_stride, alive,
                        ranges, (const uint16_t *)accum, (uint16_t *)out, B, NQ, NK, H, scale_log2e);
     return (int)hipGetLastError();

@@ -453,7 +453,9 @@ def test_sdpa_cross_matches_oracle(B, NQ, NK):
 
 
 @pytest.mark.parametrize("B,NQ,NK,p_live", [(4, 12, 161, 0.5), (3, 84, 800, 0.3), (2, 156, 1520, 1.0), (3, 156, 1520, 0.1),
-                                           (2, 33, 2048, 0.7), (3, 20, 500, 0.02), (2, 160, 193, 0.17)])
+                                           (2, 33, 2048, 0.7), (3, 20, 500, 0.02), (2, 160, 193, 0.17),
+                                           # a fifth block of queries, shared by the waves: 2 rows of it, few keys, many keys
+                                           (3, 130, 700, 0.3), (3, 129, 300, 0.05), (2, 145, 2048, 0.9)])
 def test_sdpa_cross_streams_long_key_axes(B, NQ, NK, p_live):
     # more keys than fit in LDS at once: tiles of live keys with an online softmax across them
     H, D = 4, 128
@@ -1419,7 +1421,8 @@ def test_compact_rows_and_gathered_projection(B, n, p):
         assert max_rel(out[:total].float().cpu(), want) <= BF16_TOL
 
 
-@pytest.mark.parametrize("B,NQ,NK,p", [(4, 12, 80, 0.5), (3, 84, 800, 0.3), (3, 156, 1520, 0.1), (2, 33, 3000, 0.6), (5, 20, 190, 0.0)])
+@pytest.mark.parametrize("B,NQ,NK,p", [(4, 12, 80, 0.5), (3, 84, 800, 0.3), (3, 156, 1520, 0.1), (2, 33, 3000, 0.6), (5, 20, 190, 0.0),
+                                       (3, 131, 900, 0.4), (4, 160, 1520, 0.02)])
 def test_sdpa_cross_over_compacted_rows_equals_the_masked_form(B, NQ, NK, p):
     H, D = 4, 128
     g = torch.Generator().manual_seed(NQ * 13 + NK)
