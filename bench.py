@@ -606,10 +606,13 @@ def main():
         total_b = rows_b.total_host()
         kv_rows_b = kv_b.reshape(w.B * NB, 2 * D)[b_mask.reshape(-1)].contiguous()
         t_rows = timed_loop(lambda t: ops.sdpa_cross_rows(qkv_b, kv_rows_b, rows_b, H, accum=merged[t & 1], total=total_b), n_b, 3) / n_b
-        out_b = ops.sdpa_cross_rows(qkv_b, kv_rows_b, rows_b, H, total=total_b)
+        # as the update runs it: the forward hands its log-sum-exp to the backward when the streaming kernels apply
+        lse_b = torch.empty((w.B, H, w.NM), dtype=torch.float32, device=dev) if rows_b.max_count_host() > 160 else None
+        out_b = ops.sdpa_cross_rows(qkv_b, kv_rows_b, rows_b, H, total=total_b, lse=lse_b)
         dout_b = (0.5 * torch.randn(w.B, w.NM, D, device=dev, generator=gen)).to(w.dtype)
-        t_bwd = timed_loop(lambda t: ops.sdpa_cross_rows_bwd(qkv_b, kv_rows_b, rows_b, H, out_b, dout_b, total_b), n_b, 3) / n_b
-        del kv_rows_b, out_b, dout_b
+        t_bwd = timed_loop(lambda t: ops.sdpa_cross_rows_bwd(qkv_b, kv_rows_b, rows_b, H, out_b, dout_b, total_b, lse=lse_b), n_b, 3) / n_b
+        t_bwd_alone = timed_loop(lambda t: ops.sdpa_cross_rows_bwd(qkv_b, kv_rows_b, rows_b, H, out_b, dout_b, total_b), n_b, 3) / n_b
+        del kv_rows_b, out_b, dout_b, lse_b
         read_bytes = live * 2 * D * 2 + w.B * NB + 3 * w.B * w.NM * D * 2
         result["bullet_read"] = {
             "avg_launch_us": t_read * 1e6, "slots_per_env": NB, "live_fraction": live_p,
@@ -617,7 +620,8 @@ def main():
             "frac_of_hbm_peak": read_bytes / t_read / peak,
             "tflops": 4 * live * w.NM * D / t_read / 1e12,
             "eager_torch_us": None if t_read_torch is None else t_read_torch * 1e6,
-            "rows_form_us": t_rows * 1e6, "rows_form_backward_us": t_bwd * 1e6, "max_live_per_env": rows_b.max_count_host(),
+            "rows_form_us": t_rows * 1e6, "rows_form_backward_us": t_bwd * 1e6,
+            "rows_form_backward_recomputing_lse_us": t_bwd_alone * 1e6, "max_live_per_env": rows_b.max_count_host(),
             "branch_compact_us": t_branch * 1e6, "branch_all_slots_us": t_branch_all * 1e6,
             "branch_what": "norm_bullet + kv_bullet + read from fp32 bullet tokens: compact = device-side list of the "
                            "live bullets, bnb_norm_linear_fwd over it, bnb_sdpa_cross_ranges_fwd; all_slots = "

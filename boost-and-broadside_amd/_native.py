@@ -12,7 +12,7 @@ import os
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "_lib", "libbnb_amd.so")
 
-ABI_VERSION = 24
+ABI_VERSION = 25
 F32, BF16 = 0, 1
 PATH_AUTO, PATH_VALU, PATH_MFMA, PATH_ENV, PATH_HEAD = 0, 1, 2, 3, 4
 WGRAD_PATH_AUTO, WGRAD_PATH_STAGED, WGRAD_PATH_DMA = 0, 1, 2
@@ -28,6 +28,7 @@ SIGNATURES = {
     "bnb_sdpa_masked_fwd_path": (_i, [_vp, _i64, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "bnb_sdpa_cross_fwd": (_i, [_vp, _i64, _i, _vp, _vp, _i64, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "bnb_sdpa_cross_ranges_fwd": (_i, [_vp, _i64, _i, _vp, _i64, _vp, _i64, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "bnb_sdpa_cross_ranges_fwd_lse": (_i, [_vp, _i64, _i, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "bnb_rglru_step_fwd": (_i, [_vp, _i, _vp, _i, _vp, _f, _vp, _i64, _vp, _i64, _vp, _i, _i64, _i, _vp]),
     "bnb_rglru_step_reset_fwd": (
         _i, [_vp, _i, _vp, _i, _vp, _f, _vp, _i64, _vp, _i64, _vp, _i, _vp, _i, _i64, _i, _vp]
@@ -47,6 +48,7 @@ SIGNATURES = {
     "bnb_sdpa_cross_bwd": (_i, [_vp, _i64, _i, _vp, _i64, _i, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
     "bnb_sdpa_cross_ranges_bwd": (_i, [_vp, _i64, _i, _vp, _i64, _vp, _i64, _i, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
     "bnb_sdpa_cross_stream_bwd": (_i, [_vp, _i64, _i, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
+    "bnb_sdpa_cross_stream_bwd_lse": (_i, [_vp, _i64, _i, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]),
     "bnb_sdpa_masked_bwd_path": (_i, [_vp, _i64, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _vp]),
     "bnb_rmsnorm_bwd_blocks": (_i, [_i64, _i]),
     "bnb_rmsnorm_bwd": (_i, [_vp, _i64, _vp, _i, _i64, _vp, _f, _vp, _vp, _vp, _vp, _i, _vp, _i64, _i, _vp]),

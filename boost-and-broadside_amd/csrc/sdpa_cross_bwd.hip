@@ -75,12 +75,14 @@ __device__ __forceinline__ void cb_store_row(const f32x16 &acc, uint16_t *dst)
         *reinterpret_cast<u32x2 *>(dst + 8 * i) = u32x2{pack_bf16x2(acc[4 * i], acc[4 * i + 1]), pack_bf16x2(acc[4 * i + 2], acc[4 * i + 3])};
 }
 
-template <int NB>
-__global__ __launch_bounds__(kWave *NB) void cross_bwd_dq_kernel(
+// HAVE_LSE: the forward pass handed over the log2-sum-exp of every query (`lse_in`, (B, H, NQ) floats); pass A,
+// which otherwise recomputes it from the keys (all the scores twice), is skipped.
+template <int NB, bool HAVE_LSE>
+__global__ __launch_bounds__(kWave *NB, 3) void cross_bwd_dq_kernel(
     const uint16_t *__restrict__ q, int64_t q_row_stride, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
     int64_t kv_row_stride, const int32_t *__restrict__ ranges, const int32_t *__restrict__ row_index, int64_t capacity,
     const uint16_t *__restrict__ out, const uint16_t *__restrict__ dout, uint16_t *__restrict__ dq_out, float *__restrict__ stats,
-    int B, int NQ, int H, float scale)
+    const float *__restrict__ lse_in, int B, int NQ, int H, float scale)
 {
     constexpr int CAP = NB * 32;  // keys per tile
     constexpr int TP = CAP + 4;   // halfs per row of the transposed copy
@@ -199,10 +201,11 @@ __global__ __launch_bounds__(kWave *NB) void cross_bwd_dq_kernel(
     };
 
     // ---- pass A: log2-sum-exp of every query over all keys ----
-    const bool single = ntiles == 1;  // one tile: staged once, with V and K^T, for both passes
+    const bool single = !HAVE_LSE && ntiles == 1;  // one tile: staged once, with V and K^T, for both passes
     float mx = -INFINITY, sum = 0.0f;
-    CbStaged cur = stage_load(0, single);
-    for (int t = 0; t < ntiles; ++t) {
+    CbStaged cur;
+    if (!HAVE_LSE) cur = stage_load(0, single);
+    for (int t = 0; !HAVE_LSE && t < ntiles; ++t) {
         __syncthreads();  // the previous tile has been read by every wave
         stage_store(cur, single);
         __syncthreads();
@@ -228,7 +231,8 @@ __global__ __launch_bounds__(kWave *NB) void cross_bwd_dq_kernel(
         }
     }
     sum += __shfl_xor(sum, 32);
-    const float lse = mx * c + __builtin_amdgcn_logf(sum);  // log2 of the sum of exp2(z c)
+    // log2 of the sum of exp2(z c)
+    const float lse = HAVE_LSE ? lse_in[((int64_t)env * H + head) * NQ + (own < NQ ? own : NQ - 1)] : mx * c + __builtin_amdgcn_logf(sum);
     if (own < NQ && half == 0) stat_row[0] = lse, stat_row[1] = delta;
 
     // ---- pass B: dQ ----
@@ -262,8 +266,11 @@ __global__ __launch_bounds__(kWave *NB) void cross_bwd_dq_kernel(
     if (own < NQ) cb_store_row(dq, dq_row);
 }
 
+// Waves: the key blocks are dealt to the waves in turn, so their number is free; never more than four.  A CU places
+// a work-group only while each of its four SIMDs has room for ceil(waves / 4) more waves: at this kernel's
+// register count a work-group of five waves came out as the only one on its CU, four-wave ones are three.
 template <int NB>
-__global__ __launch_bounds__(kWave *NB) void cross_bwd_dkv_kernel(
+__global__ __launch_bounds__(kWave *(NB < 4 ? NB : 4), 3) void cross_bwd_dkv_kernel(
     const uint16_t *__restrict__ q, int64_t q_row_stride, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
     int64_t kv_row_stride, const int32_t *__restrict__ ranges, const int32_t *__restrict__ row_index, int64_t capacity,
     const uint16_t *__restrict__ dout, const float *__restrict__ stats, uint16_t *__restrict__ dk_out, uint16_t *__restrict__ dv_out,
@@ -271,7 +278,8 @@ __global__ __launch_bounds__(kWave *NB) void cross_bwd_dkv_kernel(
 {
     constexpr int CAP = NB * 32;  // queries staged
     constexpr int TP = CAP + 4;
-    constexpr int NT = kWave * NB;
+    constexpr int NW = NB < 4 ? NB : 4;
+    constexpr int NT = kWave * NW;
     __shared__ __align__(16) uint16_t s_rows[2][CAP * kCbPitch];  // Q and dO, token-major
     __shared__ __align__(16) uint16_t s_tr[2][kCbDh * TP];        // Q^T and dO^T
     __shared__ __align__(16) float s_lse[CAP], s_delta[CAP];
@@ -318,8 +326,9 @@ __global__ __launch_bounds__(kWave *NB) void cross_bwd_dkv_kernel(
 
     // ---- Q, dO of the environment: token-major and channel-major copies; rows past NQ are zero ----
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
+    for (int it = 0; it < (4 * CAP + NT - 1) / NT; ++it) {
         const int item = tid + it * NT;
+        if (item >= 4 * CAP) break;
         const int tok = item >> 2, c8 = (item & 3) * 8;
         const bool valid = tok < NQ;
         const int64_t row = q_base + (valid ? tok : NQ - 1);
@@ -343,9 +352,9 @@ __global__ __launch_bounds__(kWave *NB) void cross_bwd_dkv_kernel(
     __syncthreads();
 
     // ---- this wave's key blocks ----
-    for (int kb = wave; kb < nkb; kb += NB) {
+    for (int kb = wave; kb < nkb; kb += NW) {
         const KeyRows cur = nxt;
-        if (kb + NB < nkb) nxt = load_keys(kb + NB);
+        if (kb + NW < nkb) nxt = load_keys(kb + NW);
         const bf16x8 ks0 = __builtin_bit_cast(bf16x8, cur.valid ? cur.k0 : zero4), ks1 = __builtin_bit_cast(bf16x8, cur.valid ? cur.k1 : zero4);
         const bf16x8 vb0 = __builtin_bit_cast(bf16x8, cur.valid ? cur.v0 : zero4), vb1 = __builtin_bit_cast(bf16x8, cur.valid ? cur.v1 : zero4);
         const float col_bias = cur.valid ? 0.0f : -INFINITY;
@@ -391,7 +400,7 @@ __global__ __launch_bounds__(kWave *NB) void cross_bwd_dkv_kernel(
 template <int NB>
 static int launch_cross_stream_bwd(const void *q, int64_t q_row_stride, const void *kv, int64_t kv_row_stride, const int32_t *ranges,
                                    const int32_t *row_index, int64_t capacity, const void *out, const void *dout, void *dq, void *dkv,
-                                   float *stats, int64_t B, int NQ, int H, hipStream_t stream)
+                                   float *stats, const float *lse, int64_t B, int NQ, int H, hipStream_t stream)
 {
     const int64_t groups = (B * H + 7) / 8 * 8;  // a multiple of 8: the XCD mapping deals whole rounds
     if (groups > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
@@ -399,12 +408,17 @@ static int launch_cross_stream_bwd(const void *q, int64_t q_row_stride, const vo
     const uint16_t *kp = (const uint16_t *)kv;
     uint16_t *g = (uint16_t *)dkv;
     const float scale = 1.0f / sqrtf((float)kCbDh);
-    hipLaunchKernelGGL((cross_bwd_dq_kernel<NB>), dim3((unsigned)groups), dim3(kWave * NB), 0, stream, (const uint16_t *)q, q_row_stride, kp,
-                       kp + D, kv_row_stride, ranges, row_index, capacity, (const uint16_t *)out, (const uint16_t *)dout, (uint16_t *)dq,
-                       stats, (int)B, NQ, H, scale);
+    if (lse != nullptr)
+        hipLaunchKernelGGL((cross_bwd_dq_kernel<NB, true>), dim3((unsigned)groups), dim3(kWave * NB), 0, stream, (const uint16_t *)q,
+                           q_row_stride, kp, kp + D, kv_row_stride, ranges, row_index, capacity, (const uint16_t *)out,
+                           (const uint16_t *)dout, (uint16_t *)dq, stats, lse, (int)B, NQ, H, scale);
+    else
+        hipLaunchKernelGGL((cross_bwd_dq_kernel<NB, false>), dim3((unsigned)groups), dim3(kWave * NB), 0, stream, (const uint16_t *)q,
+                           q_row_stride, kp, kp + D, kv_row_stride, ranges, row_index, capacity, (const uint16_t *)out,
+                           (const uint16_t *)dout, (uint16_t *)dq, stats, lse, (int)B, NQ, H, scale);
     int rc = (int)hipGetLastError();
     if (rc != 0) return rc;
-    hipLaunchKernelGGL((cross_bwd_dkv_kernel<NB>), dim3((unsigned)groups), dim3(kWave * NB), 0, stream, (const uint16_t *)q, q_row_stride, kp,
+    hipLaunchKernelGGL((cross_bwd_dkv_kernel<NB>), dim3((unsigned)groups), dim3(kWave * (NB < 4 ? NB : 4)), 0, stream, (const uint16_t *)q, q_row_stride, kp,
                        kp + D, kv_row_stride, ranges, row_index, capacity, (const uint16_t *)dout, (const float *)stats, g, g + D,
                        2 * (int64_t)D, (int)B, NQ, H, scale);
     return (int)hipGetLastError();
@@ -412,12 +426,11 @@ static int launch_cross_stream_bwd(const void *q, int64_t q_row_stride, const vo
 
 }  // namespace bnb
 
-extern "C" int bnb_sdpa_cross_stream_bwd(const void *q, int64_t q_row_stride, int NQ, const void *kv, int64_t kv_row_stride,
-                                         const int32_t *ranges, const int32_t *row_index, int64_t capacity, const void *out,
-                                         const void *dout, void *dq, void *dkv, float *stats, int64_t B, int H, int dh, int dtype,
-                                         void *stream)
+namespace bnb {
+static int cross_stream_bwd(const void *q, int64_t q_row_stride, int NQ, const void *kv, int64_t kv_row_stride,
+                            const int32_t *ranges, const int32_t *row_index, int64_t capacity, const void *out, const void *dout,
+                            void *dq, void *dkv, float *stats, const float *lse, int64_t B, int H, int dh, int dtype, void *stream)
 {
-    using namespace bnb;
     if (B < 0 || NQ < 1 || H < 1 || dh < 1 || capacity < 1) return BNB_ERR_BAD_SHAPE;
     if (dtype != BNB_BF16 || dh != kCbDh || NQ > 160) return BNB_ERR_UNSUPPORTED;
     const int D = H * dh;
@@ -429,7 +442,7 @@ extern "C" int bnb_sdpa_cross_stream_bwd(const void *q, int64_t q_row_stride, in
         return BNB_ERR_MISALIGNED;
     if (B > 0x7fffffffLL / H) return BNB_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
-#define BNB_CSB(NBV) return launch_cross_stream_bwd<NBV>(q, q_row_stride, kv, kv_row_stride, ranges, row_index, capacity, out, dout, dq, dkv, stats, B, NQ, H, s)
+#define BNB_CSB(NBV) return launch_cross_stream_bwd<NBV>(q, q_row_stride, kv, kv_row_stride, ranges, row_index, capacity, out, dout, dq, dkv, stats, lse, B, NQ, H, s)
     switch ((NQ + 31) / 32) {
         case 1: BNB_CSB(1);
         case 2: BNB_CSB(2);
@@ -439,4 +452,25 @@ extern "C" int bnb_sdpa_cross_stream_bwd(const void *q, int64_t q_row_stride, in
         default: return BNB_ERR_UNSUPPORTED;
     }
 #undef BNB_CSB
+}
+}  // namespace bnb
+
+extern "C" int bnb_sdpa_cross_stream_bwd(const void *q, int64_t q_row_stride, int NQ, const void *kv, int64_t kv_row_stride,
+                                         const int32_t *ranges, const int32_t *row_index, int64_t capacity, const void *out,
+                                         const void *dout, void *dq, void *dkv, float *stats, int64_t B, int H, int dh, int dtype,
+                                         void *stream)
+{
+    return bnb::cross_stream_bwd(q, q_row_stride, NQ, kv, kv_row_stride, ranges, row_index, capacity, out, dout, dq, dkv, stats,
+                                 nullptr, B, H, dh, dtype, stream);
+}
+
+extern "C" int bnb_sdpa_cross_stream_bwd_lse(const void *q, int64_t q_row_stride, int NQ, const void *kv, int64_t kv_row_stride,
+                                             const int32_t *ranges, const int32_t *row_index, int64_t capacity, const void *out,
+                                             const void *dout, const float *lse, void *dq, void *dkv, float *stats, int64_t B,
+                                             int H, int dh, int dtype, void *stream)
+{
+    if (lse == nullptr && B > 0) return BNB_ERR_NULL_POINTER;
+    if (reinterpret_cast<uintptr_t>(lse) & 3u) return BNB_ERR_MISALIGNED;
+    return bnb::cross_stream_bwd(q, q_row_stride, NQ, kv, kv_row_stride, ranges, row_index, capacity, out, dout, dq, dkv, stats,
+                                 lse, B, H, dh, dtype, stream);
 }

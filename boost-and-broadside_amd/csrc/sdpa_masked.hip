@@ -783,8 +783,8 @@ template <int NQB>
 __global__ __launch_bounds__(kWave *(NQB < 4 ? NQB : 4), 3) void sdpa_cross_stream_kernel(
     const uint16_t *__restrict__ q, int64_t q_stride, const uint16_t *__restrict__ k,
     const uint16_t *__restrict__ v, int64_t kv_stride, const uint8_t *__restrict__ alive,
-    const int32_t *__restrict__ ranges, const uint16_t *accum, uint16_t *out, int B, int NQ, int NK, int H,
-    float scale_log2e)
+    const int32_t *__restrict__ ranges, const uint16_t *accum, uint16_t *out, float *__restrict__ lse_out, int B, int NQ,
+    int NK, int H, float scale_log2e)
 {
     constexpr int NW = NQB < 4 ? NQB : 4;  // waves, and key blocks per tile
     constexpr bool SPLIT = NQB > NW;       // a fifth block of queries, shared by the four waves
@@ -1062,6 +1062,10 @@ __global__ __launch_bounds__(kWave *(NQB < 4 ? NQB : 4), 3) void sdpa_cross_stre
     }
     sum += __shfl_xor(sum, 32);
     const float inv = cnt == 0 ? 0.0f : __builtin_amdgcn_rcpf(sum);
+    // log2 of the sum over the keys of exp2(score * scale_log2e), for a backward pass that would otherwise recompute it
+    // (meaningless for an environment without keys, which that pass does not read)
+    float *lse_env = lse_out == nullptr ? nullptr : lse_out + ((int64_t)env * H + head) * NQ;
+    if (lse_env != nullptr && qrow < NQ && half == 0) lse_env[qrow] = fmaf(mx, scale_log2e, __builtin_amdgcn_logf(sum));
 
     if (SPLIT) {
         // Merge the four partial results of the shared block.  Every wave has passed the barrier of the last tile,
@@ -1093,6 +1097,8 @@ __global__ __launch_bounds__(kWave *(NQB < 4 ? NQB : 4), 3) void sdpa_cross_stre
             for (int i = 0; i < 4; ++i) r[i] = fmaf(f, part[(j * 16 + wave * 4 + i) * kWave + lane], r[i]);
         }
         const float sinv = cnt == 0 ? 0.0f : __builtin_amdgcn_rcpf(total);
+        if (lse_env != nullptr && wave == 0 && srow < NQ && half == 0)
+            lse_env[srow] = fmaf(mall, scale_log2e, __builtin_amdgcn_logf(total));
         if (srow < NQ) {
             const int64_t at = ((int64_t)env * NQ + srow) * D + head * kDh + 16 * (wave >> 1) + 8 * half + 4 * (wave & 1);
 #pragma unroll
@@ -1231,7 +1237,7 @@ static int dispatch_mfma(const void *q, int64_t q_stride, const void *k, const v
 
 template <int NQB>
 static int launch_cross_stream(const void *q, int64_t q_stride, const void *k, const void *v, int64_t kv_stride,
-                               const uint8_t *alive, const int32_t *ranges, const void *accum, void *out, int B,
+                               const uint8_t *alive, const int32_t *ranges, const void *accum, void *out, float *lse, int B,
                                int NQ, int NK, int H, hipStream_t stream)
 {
     const int64_t pairs = (int64_t)B * H;
@@ -1240,20 +1246,20 @@ static int launch_cross_stream(const void *q, int64_t q_stride, const void *k, c
     const float scale_log2e = kLog2eA / sqrtf((float)kDh);
     hipLaunchKernelGGL((sdpa_cross_stream_kernel<NQB>), dim3((unsigned)blocks), dim3(kWave * (NQB < 4 ? NQB : 4)), 0, stream,
                        (const uint16_t *)q, q_stride, (const uint16_t *)k, (const uint16_t *)v, kv_stride, alive,
-                       ranges, (const uint16_t *)accum, (uint16_t *)out, B, NQ, NK, H, scale_log2e);
+                       ranges, (const uint16_t *)accum, (uint16_t *)out, lse, B, NQ, NK, H, scale_log2e);
     return (int)hipGetLastError();
 }
 
 static int dispatch_cross_stream(const void *q, int64_t q_stride, const void *k, const void *v, int64_t kv_stride,
-                                 const uint8_t *alive, const int32_t *ranges, const void *accum, void *out, int B,
-                                 int NQ, int NK, int H, hipStream_t stream)
+                                 const uint8_t *alive, const int32_t *ranges, const void *accum, void *out, float *lse,
+                                 int B, int NQ, int NK, int H, hipStream_t stream)
 {
     switch ((NQ + 31) / 32) {
-        case 1: return launch_cross_stream<1>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, B, NQ, NK, H, stream);
-        case 2: return launch_cross_stream<2>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, B, NQ, NK, H, stream);
-        case 3: return launch_cross_stream<3>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, B, NQ, NK, H, stream);
-        case 4: return launch_cross_stream<4>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, B, NQ, NK, H, stream);
-        case 5: return launch_cross_stream<5>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, B, NQ, NK, H, stream);
+        case 1: return launch_cross_stream<1>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, lse, B, NQ, NK, H, stream);
+        case 2: return launch_cross_stream<2>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, lse, B, NQ, NK, H, stream);
+        case 3: return launch_cross_stream<3>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, lse, B, NQ, NK, H, stream);
+        case 4: return launch_cross_stream<4>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, lse, B, NQ, NK, H, stream);
+        case 5: return launch_cross_stream<5>(q, q_stride, k, v, kv_stride, alive, ranges, accum, out, lse, B, NQ, NK, H, stream);
         default: return BNB_ERR_UNSUPPORTED;
     }
 }
@@ -1374,18 +1380,17 @@ extern "C" int bnb_sdpa_cross_fwd(const void *q, int64_t q_row_stride, int NQ, c
         !aligned16(k) || !aligned16(v) || (kv_row_stride * 2) % 16 != 0)
         return BNB_ERR_MISALIGNED;
     if (NK > 160)
-        return dispatch_cross_stream(q, q_row_stride, k, v, kv_row_stride, key_mask, nullptr, accum, out, B, NQ, NK,
+        return dispatch_cross_stream(q, q_row_stride, k, v, kv_row_stride, key_mask, nullptr, accum, out, nullptr, B, NQ, NK,
                                      H, (hipStream_t)stream);
     return dispatch_mfma<true>(q, q_row_stride, k, v, kv_row_stride, key_mask, accum, out, B, NQ, NK, H,
                                (hipStream_t)stream);
 }
 
-extern "C" int bnb_sdpa_cross_ranges_fwd(const void *q, int64_t q_row_stride, int NQ, const void *kv_rows,
-                                         int64_t kv_row_stride, const int32_t *ranges, int64_t kv_capacity,
-                                         const void *accum, void *out, int B, int H, int dh, int dtype,
-                                         void *stream)
+namespace bnb {
+static int cross_ranges_fwd(const void *q, int64_t q_row_stride, int NQ, const void *kv_rows, int64_t kv_row_stride,
+                            const int32_t *ranges, int64_t kv_capacity, const void *accum, void *out, float *lse, int B, int H,
+                            int dh, int dtype, void *stream)
 {
-    using namespace bnb;
     if (B < 0 || NQ < 0 || H < 1 || dh < 1 || kv_capacity < 0) return BNB_ERR_BAD_SHAPE;
     if (dtype != BNB_BF16 || dh != kDh || NQ > 160) return BNB_ERR_UNSUPPORTED;
     if (B == 0 || NQ == 0) return 0;
@@ -1398,6 +1403,27 @@ extern "C" int bnb_sdpa_cross_ranges_fwd(const void *q, int64_t q_row_stride, in
         !aligned16(kv_rows) || (kv_row_stride * 2) % 16 != 0 || (reinterpret_cast<uintptr_t>(ranges) & 3u))
         return BNB_ERR_MISALIGNED;
     const uint16_t *kp = (const uint16_t *)kv_rows;
-    return dispatch_cross_stream(q, q_row_stride, kp, kp + (int64_t)H * dh, kv_row_stride, nullptr, ranges, accum, out, B,
-                                 NQ, 0, H, (hipStream_t)stream);
+    return dispatch_cross_stream(q, q_row_stride, kp, kp + (int64_t)H * dh, kv_row_stride, nullptr, ranges, accum, out, lse,
+                                 B, NQ, 0, H, (hipStream_t)stream);
+}
+}  // namespace bnb
+
+extern "C" int bnb_sdpa_cross_ranges_fwd(const void *q, int64_t q_row_stride, int NQ, const void *kv_rows,
+                                         int64_t kv_row_stride, const int32_t *ranges, int64_t kv_capacity,
+                                         const void *accum, void *out, int B, int H, int dh, int dtype,
+                                         void *stream)
+{
+    return bnb::cross_ranges_fwd(q, q_row_stride, NQ, kv_rows, kv_row_stride, ranges, kv_capacity, accum, out, nullptr, B, H, dh,
+                                 dtype, stream);
+}
+
+extern "C" int bnb_sdpa_cross_ranges_fwd_lse(const void *q, int64_t q_row_stride, int NQ, const void *kv_rows,
+                                             int64_t kv_row_stride, const int32_t *ranges, int64_t kv_capacity,
+                                             const void *accum, void *out, float *lse, int B, int H, int dh, int dtype,
+                                             void *stream)
+{
+    if (lse == nullptr && B > 0 && NQ > 0) return BNB_ERR_NULL_POINTER;
+    if (reinterpret_cast<uintptr_t>(lse) & 3u) return BNB_ERR_MISALIGNED;
+    return bnb::cross_ranges_fwd(q, q_row_stride, NQ, kv_rows, kv_row_stride, ranges, kv_capacity, accum, out, lse, B, H, dh,
+                                 dtype, stream);
 }

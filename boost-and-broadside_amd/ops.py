@@ -298,8 +298,10 @@ def sdpa_cross_train_supported(qkv: torch.Tensor, kv: torch.Tensor, n_heads: int
     return cross_supported(qkv, kv, n_heads) and qkv.dtype == torch.bfloat16 and kv.dim() == 3 and qkv.dim() == 3
 
 
-def sdpa_cross_stream_bwd(qkv, kv, rows: "CompactRows", n_heads, out, dout, *, indexed: bool):
+def sdpa_cross_stream_bwd(qkv, kv, rows: "CompactRows", n_heads, out, dout, *, indexed: bool, lse: torch.Tensor | None = None):
     """Gradients ``(dq (B, NQ, D), dkv)`` of the bullet read for any number of listed keys per environment.
+    ``lse`` (B, n_heads, NQ) float32, optional: the log-sum-exp ``sdpa_cross_rows(..., lse=...)`` wrote in the forward
+    pass over the same queries and keys; without it the first kernel recomputes it (a second pass over every key).
 
     ``indexed=False``: ``kv`` (capacity, 2D) holds ``[K | V]`` of the entries of ``rows`` in list order and
     ``dkv`` has that layout.  ``indexed=True``: ``kv`` is the (B, NK, 2D) buffer the mask of ``rows`` was
@@ -330,13 +332,23 @@ def sdpa_cross_stream_bwd(qkv, kv, rows: "CompactRows", n_heads, out, dout, *, i
     dq = torch.empty((B, NQ, D), dtype=torch.bfloat16, device=qkv.device)
     if capacity == 0:
         return dq.zero_(), dkv
+    if lse is not None and (lse.shape != (B, n_heads, NQ) or lse.dtype != torch.float32 or not lse.is_contiguous()
+                            or lse.device != qkv.device):
+        raise ValueError(f"lse must be a contiguous float32 {(B, n_heads, NQ)} tensor on the queries' device")
     if B and NQ:
         stats = torch.empty((B, n_heads, NQ, 2), dtype=torch.float32, device=qkv.device)
+        lib = _native.load()
         with _on_device(qkv.device):
-            rc = _native.load().bnb_sdpa_cross_stream_bwd(
-                qkv.data_ptr(), qkv.stride(1), NQ, kv.data_ptr(), 2 * D, rows.offsets.data_ptr(),
-                rows.index.data_ptr() if indexed else None, capacity, out.data_ptr(), dout.data_ptr(), dq.data_ptr(),
-                dkv.data_ptr(), stats.data_ptr(), B, n_heads, D // n_heads, _native.BF16, _stream())
+            if lse is None:
+                rc = lib.bnb_sdpa_cross_stream_bwd(
+                    qkv.data_ptr(), qkv.stride(1), NQ, kv.data_ptr(), 2 * D, rows.offsets.data_ptr(),
+                    rows.index.data_ptr() if indexed else None, capacity, out.data_ptr(), dout.data_ptr(), dq.data_ptr(),
+                    dkv.data_ptr(), stats.data_ptr(), B, n_heads, D // n_heads, _native.BF16, _stream())
+            else:
+                rc = lib.bnb_sdpa_cross_stream_bwd_lse(
+                    qkv.data_ptr(), qkv.stride(1), NQ, kv.data_ptr(), 2 * D, rows.offsets.data_ptr(),
+                    rows.index.data_ptr() if indexed else None, capacity, out.data_ptr(), dout.data_ptr(), lse.data_ptr(),
+                    dq.data_ptr(), dkv.data_ptr(), stats.data_ptr(), B, n_heads, D // n_heads, _native.BF16, _stream())
         _native.check(rc, "bnb_sdpa_cross_stream_bwd")
     return dq, dkv
 
@@ -410,9 +422,10 @@ def sdpa_cross_train(qkv: torch.Tensor, kv: torch.Tensor, key_mask: torch.Tensor
         return _SdpaCrossTrain.apply(qkv, kv, key_mask, n_heads)
 
 
-def sdpa_cross_rows_bwd(qkv, kv_rows, rows: "CompactRows", n_heads, out, dout, total: int):
+def sdpa_cross_rows_bwd(qkv, kv_rows, rows: "CompactRows", n_heads, out, dout, total: int, lse: torch.Tensor | None = None):
     """Gradients ``(dq (B, NQ, D), dkv_rows (total, 2D))`` of ``sdpa_cross_rows`` (without accumulator);
-    ``total`` = ``rows.total_host()`` rows of ``kv_rows`` are valid."""
+    ``total`` = ``rows.total_host()`` rows of ``kv_rows`` are valid.  ``lse``: what the forward wrote with
+    ``sdpa_cross_rows(..., lse=...)``; used when some environment lists more than 160 keys (the streaming kernels)."""
     B, NQ, D3 = qkv.shape
     D = D3 // 3
     for name, t in (("qkv", qkv), ("kv_rows", kv_rows), ("out", out), ("dout", dout)):
@@ -424,7 +437,7 @@ def sdpa_cross_rows_bwd(qkv, kv_rows, rows: "CompactRows", n_heads, out, dout, t
     if rows.shape[0] != B or out.shape != (B, NQ, D) or dout.shape != (B, NQ, D):
         raise ValueError("rows must list the entries of the B environments; out and dout are (B, NQ, D)")
     if rows.max_count_host() > 160:
-        return sdpa_cross_stream_bwd(qkv, kv_rows[:total], rows, n_heads, out, dout, indexed=False)
+        return sdpa_cross_stream_bwd(qkv, kv_rows[:total], rows, n_heads, out, dout, indexed=False, lse=lse)
     if B and NQ and (qkv.stride(-1) != 1 or (B > 1 and qkv.stride(0) != NQ * qkv.stride(1))):
         qkv = qkv.contiguous()
     out, dout = out.contiguous(), dout.contiguous()
@@ -447,17 +460,21 @@ class _SdpaCrossRowsTrain(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, qkv, kv_rows, rows, n_heads, total):
+        B, NQ, _ = qkv.shape
+        # more keys than the single-tile backward takes: its streaming counterpart reuses the forward's log-sum-exp
+        lse = (torch.empty((B, n_heads, NQ), dtype=torch.float32, device=qkv.device)
+               if B and NQ and total and rows.max_count_host() > 160 else None)
         with torch.no_grad():
-            out = sdpa_cross_rows(qkv, kv_rows, rows, n_heads, total=total)
+            out = sdpa_cross_rows(qkv, kv_rows, rows, n_heads, total=total, lse=lse)
         ctx.save_for_backward(qkv, kv_rows, out)
-        ctx.rows, ctx.n_heads, ctx.total = rows, n_heads, total
+        ctx.rows, ctx.n_heads, ctx.total, ctx.lse = rows, n_heads, total, lse
         return out
 
     @staticmethod
     @_outside_autocast
     def backward(ctx, dout):
         qkv, kv_rows, out = ctx.saved_tensors
-        dq, dkv = sdpa_cross_rows_bwd(qkv, kv_rows, ctx.rows, ctx.n_heads, out, dout.to(torch.bfloat16), ctx.total)
+        dq, dkv = sdpa_cross_rows_bwd(qkv, kv_rows, ctx.rows, ctx.n_heads, out, dout.to(torch.bfloat16), ctx.total, ctx.lse)
         dqkv = torch.zeros_like(qkv)
         dqkv[..., : dq.shape[-1]] = dq
         return dqkv, dkv, None, None, None
@@ -2380,11 +2397,15 @@ def sdpa_cross_rows(
     *,
     accum: torch.Tensor | None = None,
     total: int | None = None,
+    lse: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """``sdpa_cross`` over key/value rows compacted beforehand: ``kv_rows`` (capacity, 2*D)
     holds ``[K | V]`` of the entries listed in ``rows`` (e.g. ``norm_linear(bullets, ..., rows=rows)``),
     environment b reading the rows ``rows.offsets[b] .. rows.offsets[b+1]-1``.  Same result as
-    ``sdpa_cross`` with the mask the list was built from, without scanning the mask again."""
+    ``sdpa_cross`` with the mask the list was built from, without scanning the mask again.
+
+    ``lse``: optional contiguous float32 (B, n_heads, NQ) tensor that receives the base-2 log-sum-exp of every
+    query's scaled scores, which ``sdpa_cross_stream_bwd`` takes instead of recomputing it."""
     B, NQ, D3 = qkv.shape
     D = D3 // 3
     if not (qkv.is_cuda and qkv.dtype == torch.bfloat16 and kv_rows.dtype == torch.bfloat16 and D % n_heads == 0
@@ -2401,16 +2422,27 @@ def sdpa_cross_rows(
         qkv = qkv.contiguous()
     if accum is not None and (accum.shape != (B, NQ, D) or accum.dtype != torch.bfloat16 or not accum.is_contiguous()):
         raise ValueError("accum must be a contiguous bfloat16 (B, NQ, D) tensor")
+    if lse is not None and (lse.shape != (B, n_heads, NQ) or lse.dtype != torch.float32 or not lse.is_contiguous()
+                            or lse.device != qkv.device):
+        raise ValueError(f"lse must be a contiguous float32 {(B, n_heads, NQ)} tensor on the queries' device")
     out = accum if accum is not None else torch.empty((B, NQ, D), dtype=torch.bfloat16, device=qkv.device)
     if B == 0 or NQ == 0:
         return out
     if kv_rows.shape[0] == 0:  # an empty list: every environment reads nothing
         return out if accum is not None else out.zero_()
+    lib = _native.load()
     with _on_device(qkv.device):
-        rc = _native.load().bnb_sdpa_cross_ranges_fwd(
-            qkv.data_ptr(), qkv.stride(1), NQ, kv_rows.data_ptr(), kv_rows.stride(0), rows.offsets.data_ptr(),
-            kv_rows.shape[0], None if accum is None else accum.data_ptr(), out.data_ptr(), B, n_heads, D // n_heads,
-            _native.BF16, _stream(),
-        )
+        if lse is None:
+            rc = lib.bnb_sdpa_cross_ranges_fwd(
+                qkv.data_ptr(), qkv.stride(1), NQ, kv_rows.data_ptr(), kv_rows.stride(0), rows.offsets.data_ptr(),
+                kv_rows.shape[0], None if accum is None else accum.data_ptr(), out.data_ptr(), B, n_heads, D // n_heads,
+                _native.BF16, _stream(),
+            )
+        else:
+            rc = lib.bnb_sdpa_cross_ranges_fwd_lse(
+                qkv.data_ptr(), qkv.stride(1), NQ, kv_rows.data_ptr(), kv_rows.stride(0), rows.offsets.data_ptr(),
+                kv_rows.shape[0], None if accum is None else accum.data_ptr(), out.data_ptr(), lse.data_ptr(), B, n_heads,
+                D // n_heads, _native.BF16, _stream(),
+            )
     _native.check(rc, "bnb_sdpa_cross_ranges_fwd")
     return out

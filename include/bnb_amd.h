@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 24
+#define BNB_ABI_VERSION 25
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -136,6 +136,18 @@ int bnb_sdpa_cross_fwd(const void *q, int64_t q_row_stride, int NQ, const void *
 int bnb_sdpa_cross_ranges_fwd(const void *q, int64_t q_row_stride, int NQ, const void *kv_rows,
                               int64_t kv_row_stride, const int32_t *ranges, int64_t kv_capacity,
                               const void *accum, void *out, int B, int H, int dh, int dtype, void *stream);
+
+/*
+ * bnb_sdpa_cross_ranges_fwd that also hands over what the update needs from this pass: lse, (B, H, NQ)
+ * float32, the base-2 logarithm of the sum over an environment's keys of exp2(score * log2(e) / sqrt(dh))
+ * per head and query, for bnb_sdpa_cross_stream_bwd_lse (the backward of the same read,
+ * models/yemong/attention.py:149-166 under train/rl/ppo.py:1417-1425), which otherwise recomputes it
+ * from every key.  Entries of environments with an empty range carry no meaning and are not read there.
+ */
+int bnb_sdpa_cross_ranges_fwd_lse(const void *q, int64_t q_row_stride, int NQ, const void *kv_rows,
+                                  int64_t kv_row_stride, const int32_t *ranges, int64_t kv_capacity,
+                                  const void *accum, void *out, float *lse, int B, int H, int dh, int dtype,
+                                  void *stream);
 
 /*
  * One RG-LRU recurrence step over R = B*n_rec entity rows of D channels.
@@ -353,6 +365,17 @@ int bnb_sdpa_cross_stream_bwd(const void *q, int64_t q_row_stride, int NQ, const
                               const int32_t *ranges, const int32_t *row_index, int64_t capacity, const void *out,
                               const void *dout, void *dq, void *dkv, float *stats, int64_t B, int H, int dh, int dtype,
                               void *stream);
+
+/*
+ * bnb_sdpa_cross_stream_bwd with the log2-sum-exp of every query taken from the forward pass
+ * (lse as written by bnb_sdpa_cross_ranges_fwd_lse over the same q, keys and ranges) instead of being
+ * recomputed: the first kernel then passes over the keys once instead of twice.  Everything else,
+ * stats included, as bnb_sdpa_cross_stream_bwd.
+ */
+int bnb_sdpa_cross_stream_bwd_lse(const void *q, int64_t q_row_stride, int NQ, const void *kv, int64_t kv_row_stride,
+                                  const int32_t *ranges, const int32_t *row_index, int64_t capacity, const void *out,
+                                  const void *dout, const float *lse, void *dq, void *dkv, float *stats, int64_t B,
+                                  int H, int dh, int dtype, void *stream);
 
 /*
  * RMSNorm backward:  y = x * rsqrt(mean(x^2) + eps) * weight

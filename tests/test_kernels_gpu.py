@@ -2408,6 +2408,54 @@ def test_sdpa_cross_rows_train_matches_autograd_of_the_oracle():
     assert max_rel(kv_rows.grad.float().cpu().double(), xkv.grad.reshape(B * NK, 2 * D)[mask.reshape(-1)]) <= BF16_TOL
 
 
+@pytest.mark.parametrize("B,NQ,NK,p_live", [(5, 12, 400, 0.6), (4, 84, 800, 0.3), (3, 156, 1520, 0.25), (3, 130, 700, 0.5)])
+def test_streamed_read_hands_its_log_sum_exp_to_the_backward(B, NQ, NK, p_live):
+    """More than 160 listed keys per environment: the forward writes every query's log2-sum-exp, the backward takes it
+    instead of passing over the keys twice.  Pinned three ways: the values against float64 scores of the same
+    bfloat16 operands, the gradients against the backward that recomputes them, and, through autograd, against the
+    oracle's."""
+    H, D = 4, 128
+    g = torch.Generator().manual_seed(B * 1000 + NQ + NK)
+    qkv = torch.randn(B, NQ, 3 * D, generator=g).bfloat16()
+    kv = torch.randn(B, NK, 2 * D, generator=g).bfloat16()
+    kv[:, :, :D] *= 2.0
+    mask = torch.rand(B, NK, generator=g) < p_live
+    mask[1] = False
+    up = torch.randn(B, NQ, D, generator=g).bfloat16()
+    rows = ops.CompactRows(mask.to(DEV))
+    total = rows.total_host()
+    assert rows.max_count_host() > 160
+    kv_rows = kv.reshape(B * NK, 2 * D)[mask.reshape(-1)].contiguous().to(DEV)
+    q_d = qkv.to(DEV)
+    lse = torch.full((B, H, NQ), float("nan"), device=DEV)
+    out = ops.sdpa_cross_rows(q_d, kv_rows, rows, H, total=total, lse=lse)
+    assert torch.equal(out, ops.sdpa_cross_rows(q_d, kv_rows, rows, H, total=total))  # the same forward either way
+    # log2 sum_k exp2(q.k log2(e) / sqrt(32)) over the live keys
+    qh = qkv[..., :D].double().reshape(B, NQ, H, 32).transpose(1, 2)
+    kh = kv[..., :D].double().reshape(B, NK, H, 32).transpose(1, 2)
+    scores = (qh @ kh.transpose(-1, -2)) / 32 ** 0.5
+    scores = scores.masked_fill(~mask[:, None, None, :], float("-inf"))
+    want = torch.logsumexp(scores, dim=-1) / math.log(2.0)
+    live = mask.any(dim=1)
+    assert (lse[live.to(DEV)].double().cpu() - want[live]).abs().max() <= 1e-4
+
+    dq0, dkv0 = ops.sdpa_cross_rows_bwd(q_d, kv_rows, rows, H, out, up.to(DEV), total)
+    dq1, dkv1 = ops.sdpa_cross_rows_bwd(q_d, kv_rows, rows, H, out, up.to(DEV), total, lse=lse)
+    assert max_rel(dq1.float().cpu(), dq0.float().cpu()) <= 2e-3 and max_rel(dkv1.float().cpu(), dkv0.float().cpu()) <= 2e-3
+    assert not dq1[~live.to(DEV)].any()
+
+    qg = q_d.clone().requires_grad_()
+    kvg = kv_rows.clone().requires_grad_()
+    (ops.sdpa_cross_rows_train(qg, kvg, rows, H).float() * up.to(DEV).float()).sum().backward()
+    xq = qkv.double().requires_grad_()
+    xkv = kv.double().requires_grad_()
+    (torch_ref.bullet_read(xq, xkv, mask, H) * up.double()).sum().backward()
+    assert max_rel(qg.grad.float().cpu().double(), xq.grad) <= BF16_TOL
+    assert max_rel(kvg.grad.float().cpu().double(), xkv.grad.reshape(B * NK, 2 * D)[mask.reshape(-1)]) <= BF16_TOL
+    with pytest.raises(ValueError):
+        ops.sdpa_cross_rows(q_d, kv_rows, rows, H, total=total, lse=lse[:, :, :-1])
+
+
 # ------------------------------------------------------------------ element offsets past 2^31
 
 
