@@ -77,8 +77,11 @@ __device__ __forceinline__ void cb_store_row(const f32x16 &acc, uint16_t *dst)
 
 // HAVE_LSE: the forward pass handed over the log2-sum-exp of every query (`lse_in`, (B, H, NQ) floats); pass A,
 // which otherwise recomputes it from the keys (all the scores twice), is skipped.
+// Registers: five waves per work-group only come three to a CU at 96 registers or fewer (a CU wants room for two more
+// waves on every SIMD before it takes such a work-group); the handful of values that spills at that bound costs less
+// than the third work-group brings (kernel trace at 4096 environments x 160 queries x 380 keys: 701 -> 637..658 us).
 template <int NB, bool HAVE_LSE>
-__global__ __launch_bounds__(kWave *NB, 3) void cross_bwd_dq_kernel(
+__global__ __launch_bounds__(kWave *NB, NB == 5 ? 5 : 3) void cross_bwd_dq_kernel(
     const uint16_t *__restrict__ q, int64_t q_row_stride, const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
     int64_t kv_row_stride, const int32_t *__restrict__ ranges, const int32_t *__restrict__ row_index, int64_t capacity,
     const uint16_t *__restrict__ out, const uint16_t *__restrict__ dout, uint16_t *__restrict__ dq_out, float *__restrict__ stats,
