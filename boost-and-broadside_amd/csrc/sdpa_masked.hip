@@ -1011,7 +1011,9 @@ __global__ __launch_bounds__(kWave *(NQB < 4 ? NQB : 4), 3) void sdpa_cross_stre
                 const f32x16 z1 = scores(kb + 1);
                 if (t == 0 && kb == 0 && pad != 0) mask_padding(z0);
 #pragma unroll
-                for (int e = 0; e < 16; ++e) tmx = fmaxf(tmx, fmaxf(z0[e], z1[e]));
+                for (int e = 0; e < 16; ++e) tmx = fmaxf(tmx, z0[e]);  // one chain: max(z0[e], z1[e]) first would have both
+#pragma unroll
+                for (int e = 0; e < 16; ++e) tmx = fmaxf(tmx, z1[e]);  // operands quieted by a v_max x, x each (56 ops, not 16)
             }
             if (kb < nb) {
                 f32x16 z0 = scores(kb);
