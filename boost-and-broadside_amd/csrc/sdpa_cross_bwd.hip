@@ -259,13 +259,15 @@ __global__ __launch_bounds__(kWave *NB, NB == 5 ? 5 : 3) void cross_bwd_dq_kerne
                 dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, gb1, dp, 0, 0, 0);
                 float ds[16];
 #pragma unroll
-                for (int vv = 0; vv < 16; ++vv) ds[vv] = __builtin_amdgcn_exp2f(fmaf(z[vv], c, -lse)) * (dp[vv] - delta) * scale;
+                for (int vv = 0; vv < 16; ++vv) ds[vv] = __builtin_amdgcn_exp2f(fmaf(z[vv], c, -lse)) * (dp[vv] - delta);  // * scale: once, on dq
 #pragma unroll
                 for (int t2 = 0; t2 < 2; ++t2)
                     dq = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cb_tr_operand<TP>(s_kt, m, half, kb, t2), cb_pack8(ds, t2), dq, 0, 0, 0);
             }
         }
     }
+#pragma unroll
+    for (int vv = 0; vv < 16; ++vv) dq[vv] *= scale;
     if (own < NQ) cb_store_row(dq, dq_row);
 }
 
@@ -383,7 +385,7 @@ __global__ __launch_bounds__(kWave *(NB < 4 ? NB : 4), 3) void cross_bwd_dkv_ker
                 for (int j = 0; j < 4; ++j) {
                     const int vv = 4 * i + j;
                     p[vv] = __builtin_amdgcn_exp2f(fmaf(z[vv], c, -l4[j]));
-                    ds[vv] = p[vv] * (dp[vv] - d4[j]) * scale;
+                    ds[vv] = p[vv] * (dp[vv] - d4[j]);  // * scale: once per key block, on dk
                 }
             }
 #pragma unroll
@@ -394,6 +396,8 @@ __global__ __launch_bounds__(kWave *(NB < 4 ? NB : 4), 3) void cross_bwd_dkv_ker
         }
         if (cur.valid) {
             const int64_t off = cur.row * dkv_row_stride + head * kCbDh + 4 * half;
+#pragma unroll
+            for (int vv = 0; vv < 16; ++vv) dk[vv] *= scale;
             cb_store_row(dk, dk_out + off);
             cb_store_row(dv, dv_out + off);
         }
