@@ -762,13 +762,12 @@ __global__ __launch_bounds__(1024) void sdpa_mfma_f32_kernel(
 //
 // The bullet axis is N*K slots long (80 .. 1520 in the shipped scenarios) and mostly
 // empty: only bullets in flight are keys.  One work-group per (environment, head), one
-// wave per 32 queries.  The work-group first compacts the indices of the live bullets
-// into LDS, then walks them in tiles of 32 keys per wave: the K rows and transposed V rows of
-// the next tile are gathered from global memory into registers while the matrix cores
-// work on the current tile out of LDS (two LDS buffers, one barrier per tile), with the
-// running maximum / sum / output of an online softmax carried across tiles.  Key
+// wave per 32 queries (up to four waves, see below).  The work-group first compacts the indices
+// of the live bullets into LDS, then walks them in tiles of 32 keys per wave: the K rows and
+// transposed V rows of the next tile are gathered from global memory into registers while the
+// matrix cores work on the current tile out of LDS (two LDS buffers, one barrier per tile), with
+// the running maximum / sum / output of an online softmax carried across tiles.  Key
 // positions, operand layouts and the output stage are those of sdpa_mfma_kernel.
-
 //
 // Waves per work-group: a CU places a work-group only while every one of its four SIMDs has room for
 // ceil(waves / 4) more waves, and the waves of a work-group move in step (one barrier per tile), so a
