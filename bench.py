@@ -35,6 +35,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default: the workload's rollout length, at least 32)")
     ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--repeats", type=int, default=9, help="the K-step loop is run this many times after the warm-up; the median loop is reported")
     ap.add_argument("--workload", default=None, help="one of the harness workloads (default: the 64v88 headline)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU-baseline leg; 0 skips it")
     ap.add_argument("--no-graph", action="store_true", help="time the step loop as eager launches only (no HIP graph replay)")
@@ -187,6 +188,25 @@ def timed_loop(fn, steps, warmup):
         fn(warmup + t)
     torch.cuda.synchronize()
     return time.perf_counter() - t0
+
+
+def median_loop(fn, steps, warmup, repeats):
+    """``warmup`` untimed iterations, then ``repeats`` loops of exactly ``steps`` iterations, each bracketed by a
+    device synchronisation on both sides: (median loop seconds, all loop seconds in run order).  The step index keeps
+    counting through the loops, so carried state and the input rotation go on as in one long rollout."""
+    for t in range(warmup):
+        fn(t)
+    walls = []
+    t = warmup
+    for _ in range(max(1, repeats)):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn(t)
+            t += 1
+        torch.cuda.synchronize()
+        walls.append(time.perf_counter() - t0)
+    return sorted(walls)[len(walls) // 2], walls
 
 
 def event_split(launch_a, launch_b, steps, warmup):
@@ -349,24 +369,21 @@ def main():
         launch_attn(t)
         launch_rglru(t)
 
-    wall_eager = timed_loop(kernel_step, steps, warmup)
+    # `value` is the median of `repeats` loops of exactly K steps: one loop of a few milliseconds reads the device
+    # clock wherever it happens to be on its ramp, and a short run then reports less than a long one
+    wall_eager, walls_eager = median_loop(kernel_step, steps, warmup, args.repeats)
     # The same K steps (same inputs, masks and state buffers in the same order) recorded once into a HIP graph and
     # replayed: the 2 K launches reach the GPU as one submission, without the 8 us between two launches that the
     # host-side launch path leaves at the long shapes.  `value` is the faster of the two ways to launch the K steps;
     # both times are reported.
-    wall_graph = None
+    wall_graph, walls_graph = None, None
     if not args.no_graph:
         try:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 for t in range(steps):
                     kernel_step(warmup + t)
-            graph.replay()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            graph.replay()
-            torch.cuda.synchronize()
-            wall_graph = time.perf_counter() - t0
+            wall_graph, walls_graph = median_loop(lambda t: graph.replay(), 1, 1, args.repeats)
             del graph
         except RuntimeError as err:  # capture refused: the eager figure stands
             print(f"bench: HIP graph capture of the step loop failed ({err}); timing eager launches", file=sys.stderr)
@@ -386,6 +403,8 @@ def main():
             "kernel": kernel, "bound": "hbm", "achieved": nbytes / seconds / 1e9, "peak": peak / 1e9, "unit": "GB/s",
             "frac": nbytes / seconds / peak, "algorithmic_bytes_per_launch": nbytes, "avg_launch_us": seconds * 1e6,
             "median_launch_us": median * 1e6, "traffic": traffic,
+            # a stored figure (two counter runs of this kernel at this workload), not something this run measured
+            "traffic_source": None if traffic is None else "profiles/hbm_traffic.json",
             # the same fraction on the bytes the kernel actually moves (dead K/V rows are never read)
             "frac_of_measured_traffic": None if traffic is None else traffic / seconds / peak,
         }
@@ -409,6 +428,10 @@ def main():
         "launch": launch_mode,
         "eager_launch_ms_per_step": wall_eager / steps * 1e3,
         "hip_graph_ms_per_step": None if wall_graph is None else wall_graph / steps * 1e3,
+        "repeats": len(walls_eager),
+        "loops_ms_per_step": {"eager_launches": [round(x / steps * 1e3, 5) for x in walls_eager],
+                              "hip_graph_replay": None if walls_graph is None else [round(x / steps * 1e3, 5) for x in walls_graph],
+                              "reported": "median of each list; `value` is from the faster of the two medians"},
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -418,7 +441,8 @@ def main():
             "workload": f"{w.name}: {w.B} environments x ({w.N} ship + {w.M} field tokens), d_model {D}, "
                         f"{H} heads x {D // H}, alive mask '{w.alive}', fp32 recurrent state carried over the steps",
             "region": "masked attention kernel + RG-LRU step kernel (the 4 projections are reported under 'module'); the K timed "
-                      "steps are launched one by one and, recorded once, as one HIP graph replay: the faster is `value`",
+                      "steps are launched one by one and, recorded once, as one HIP graph replay, `repeats` loops of K steps each way: "
+                      "`value` is the median loop of the faster way",
             "tokens_per_step": tokens,
         },
         "roofline": roofs[dominant],
@@ -973,6 +997,14 @@ def main():
     else:
         result["cpu_baseline"] = None
 
+    # the figures a reader of the last few hundred characters of the line needs
+    trunk_leg = result.get("trunk") or {}
+    result["summary"] = {
+        "value": result["value"], "ms_per_step": result["ms_per_step"], "roofline_frac": result["roofline"]["frac"],
+        "roofline_step_frac": result["roofline_step"]["frac"], "vs_torch_gpu_baseline": result.get("vs_torch_gpu_baseline"),
+        "trunk_ms_per_step": trunk_leg.get("ms_per_step"),
+        "trunk_with_bullet_read_ms_per_step": trunk_leg.get("with_bullet_read_ms_per_step"),
+    }
     print(json.dumps(result))
 
 

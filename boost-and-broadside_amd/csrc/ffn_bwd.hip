@@ -155,7 +155,7 @@ __global__ __launch_bounds__(kFbThreads) void ffn_bwd_kernel(
             asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
                          :
                          : "s"(src + q * 512), "v"((uint32_t)(lane * 16)), "s"(dst + (uint32_t)(q * 1024))
-                         : "memory");
+                         : "memory", "m0");
     };
 
     f32x16 acc[4];

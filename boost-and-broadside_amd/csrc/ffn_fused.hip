@@ -115,7 +115,7 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
             asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
                          :
                          : "s"(src + q * 512), "v"((uint32_t)(lane * 16)), "s"(dst + (uint32_t)(q * 1024))
-                         : "memory");
+                         : "memory", "m0");
     };
     // a chunk of the next sublayer's head: 64 features = 16 KB, four 1 KB pieces per wave, into the front of a buffer
     constexpr int kHeadChunkHalfs = 64 * kFfnD;
@@ -127,7 +127,7 @@ __global__ __launch_bounds__(kFfnThreads) __attribute__((amdgpu_waves_per_eu(2, 
             asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
                          :
                          : "s"(src + q * 512), "v"((uint32_t)(lane * 16)), "s"(dst + (uint32_t)(q * 1024))
-                         : "memory");
+                         : "memory", "m0");
     };
     // Every work-group takes the same time, so the two that share a CU would move in lockstep for
     // the whole launch: both reading rows, then both on the matrix cores, then both writing,

@@ -160,7 +160,7 @@ __device__ __forceinline__ void wd_dma16(const void *sbase, uint32_t voff, uint3
 {
     // 16 bytes per lane from sbase + voff to LDS byte address lds_base + 16 * lane (no immediate offset: the
     // instruction would add it to the LDS address as well as to the global one)
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(sbase), "v"(voff), "s"(lds_base) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(sbase), "v"(voff), "s"(lds_base) : "memory", "m0");
 }
 
 __device__ __forceinline__ bf16x8 wd_operand(const unsigned char *p)

@@ -48,7 +48,7 @@ __device__ __forceinline__ void dma_row16(const void *sbase, uint32_t voff, uint
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0"
                  :
                  : "s"(sbase), "v"(voff), "s"(lds_base)
-                 : "memory");
+                 : "memory", "m0");
 }
 
 // slot permutation of the eight 16-byte chunks of staged key p (p % 8 passed in)

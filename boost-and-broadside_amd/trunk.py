@@ -30,8 +30,12 @@ site (``LibraryDispatchWarning``); ``forbid_library_dispatch()`` turns them into
 Derived weights (bfloat16 copies, concatenations, matrix-core operand packings) are cached per
 layer and rebuilt when a source parameter's version counter, address or device changes, when
 the module is moved / cast (``.to()``), on ``load_state_dict`` and on ``train()`` / ``eval()``.
-A write through ``param.data`` changes none of these: call ``invalidate_weight_caches(module)``
-(or the method of that name on any layer here) after such a write.
+A write through ``param.data`` (``avg_parameter.data.copy_(...)``, train/rl/opponents.py:107-112)
+leaves the version counter alone, so the layers hold their parameters as ``WatchedParameter``s:
+every access to ``.data`` counts as a possible write and the caches that depend on that parameter
+are rebuilt by the next forward.  No call by the trainer is needed.  What still escapes is a write
+through an alias taken earlier and kept (``alias = p.data`` once, ``alias.copy_(...)`` many times):
+``invalidate_weight_caches(module)`` covers that, and ``verify_weight_caches(module)`` finds it.
 """
 
 from __future__ import annotations
@@ -192,7 +196,48 @@ def _copy_into(dst, src) -> None:
 
 
 def _cache_key(tensors: tuple, dtype: torch.dtype):
-    return (dtype,) + tuple((t._version, t.data_ptr(), t.device) for t in tensors)
+    return (dtype,) + tuple((t._version, t.data_ptr(), t.device, getattr(t, "_bnb_touch", 0)) for t in tensors)
+
+
+class WatchedParameter(nn.Parameter):
+    """An ``nn.Parameter`` that counts accesses to ``.data``.
+
+    ``p.data`` hands out an alias with a version counter of its own, so ``p.data.copy_(w)`` changes the weights
+    without changing ``p._version``, and a cache keyed on the version would keep serving the old weights.  Here
+    the ``.data`` attribute itself is the signal: reading or assigning it bumps ``_bnb_touch``, which is part
+    of every derived weight's key.  A read that wrote nothing costs one rebuild of the copies derived from
+    that parameter; optimizers and ``load_state_dict`` write under ``no_grad`` and do not come this way.
+    Everything else (autograd, ``state_dict``, ``deepcopy``, ``.to()``) behaves as for ``nn.Parameter``."""
+
+    __torch_function__ = torch._C._disabled_torch_function_impl
+
+    def __new__(cls, data=None, requires_grad=True):
+        if data is None:
+            data = torch.empty(0)
+        out = torch.Tensor._make_subclass(cls, data, requires_grad)
+        out._bnb_touch = 0
+        return out
+
+    @property
+    def data(self):
+        self._bnb_touch = getattr(self, "_bnb_touch", 0) + 1
+        return torch._C.TensorBase.data.__get__(self)
+
+    @data.setter
+    def data(self, value):
+        self._bnb_touch = getattr(self, "_bnb_touch", 0) + 1
+        torch._C.TensorBase.data.__set__(self, value)
+
+
+def watch_parameters(module: nn.Module) -> None:
+    """Replace every plain ``nn.Parameter`` below ``module`` by a ``WatchedParameter`` over the same memory."""
+    for m in module.modules():
+        for name, p in m._parameters.items():
+            if p is not None and type(p) is nn.Parameter:
+                watched = WatchedParameter(torch._C.TensorBase.data.__get__(p), p.requires_grad)
+                if p.grad is not None:
+                    watched.grad = p.grad
+                m._parameters[name] = watched
 
 
 def _cached_cast(owner: nn.Module, slot: str, tensors: tuple, dtype: torch.dtype, build):
@@ -224,9 +269,10 @@ def derived_weights(module: nn.Module) -> list:
 def invalidate_weight_caches(module: nn.Module, *, drop: bool = False) -> None:
     """Mark every cached derived weight below ``module`` stale, so the next forward rebuilds it.
 
-    Needed after a write the caches cannot see: ``param.data.copy_(...)`` and other writes through
-    ``.data`` leave the parameter's version counter unchanged.  ``drop=True`` frees the cached
-    tensors instead of keeping their memory for the rebuild."""
+    Only needed after a write the caches cannot see: one through an alias of the weights that was taken
+    earlier and kept (``alias = p.data`` once, then ``alias.copy_(...)``), or through a view of the storage made
+    outside autograd.  ``p.data.copy_(...)`` itself is seen (``WatchedParameter``).  ``drop=True`` frees the
+    cached tensors instead of keeping their memory for the rebuild."""
     for m in module.modules():
         for k in [k for k, v in m.__dict__.items() if k.startswith(_CACHE_PREFIX) and isinstance(v, _DerivedWeight)]:
             if drop:
@@ -235,20 +281,54 @@ def invalidate_weight_caches(module: nn.Module, *, drop: bool = False) -> None:
                 m.__dict__[k].key = None
 
 
+def verify_weight_caches(module: nn.Module) -> list[str]:
+    """Names (``module path:slot``) of cached derived weights that no longer equal a fresh build from their
+    sources although their key says they are current.  Compares on the device and copies one flag per entry
+    to the host: a debugging aid for a trainer suspected of writing weights where the caches cannot see it."""
+    stale = []
+    for name, m in module.named_modules():
+        for slot, entry in m.__dict__.items():
+            if not (slot.startswith(_CACHE_PREFIX) and isinstance(entry, _DerivedWeight)):
+                continue
+            if entry.key != _cache_key(entry.tensors, entry.dtype):
+                continue  # known to be stale: the next forward rebuilds it
+            with torch.no_grad():
+                fresh = entry.build()
+            have = entry.value if isinstance(entry.value, tuple) else (entry.value,)
+            want = fresh if isinstance(fresh, tuple) else (fresh,)
+            if not all(torch.equal(a, b) for a, b in zip(have, want)):
+                stale.append(f"{name}:{slot}")
+    return stale
+
+
 class _WeightCaches:
     """Mixin of the layers: keeps the derived-weight caches in step with what ``nn.Module`` does to
-    the parameters behind the caches' back (moves and casts, state-dict loads, mode switches)."""
+    the parameters behind the caches' back (moves and casts, state-dict loads, mode switches), and
+    keeps the parameters below the layer ``WatchedParameter``s, so writes through ``.data`` are seen."""
 
     def invalidate_weight_caches(self, *, drop: bool = False) -> None:
         invalidate_weight_caches(self, drop=drop)
 
+    def __setattr__(self, name, value):
+        super().__setattr__(name, value)
+        if isinstance(value, nn.Module):
+            watch_parameters(value)
+        elif type(value) is nn.Parameter:
+            watch_parameters(self)
+
+    def __setstate__(self, state):
+        super().__setstate__(state)
+        watch_parameters(self)  # unpickling rebuilds plain Parameters
+
     def _apply(self, fn, *args, **kwargs):
         out = super()._apply(fn, *args, **kwargs)
+        watch_parameters(self)
         invalidate_weight_caches(self, drop=True)  # device or dtype may have changed
         return out
 
     def load_state_dict(self, *args, **kwargs):
         out = super().load_state_dict(*args, **kwargs)
+        watch_parameters(self)  # assign=True swaps the Parameter objects
         invalidate_weight_caches(self)
         return out
 
@@ -1510,39 +1590,68 @@ class YemongTrunk(_WeightCaches, nn.Module):
         return (x.to(torch.bfloat16) if widened else x), out_state
 
 
+def _bullet_buffers(trunk, num_envs: int, num_bullet_slots: int | None, dev, dtype):
+    """Static ``(bullets, bullet_mask)`` inputs of a stepper, or ``(None, None)`` for a trunk that reads none.
+
+    A trunk whose configuration reads bullets skips the read silently when it is handed none
+    (attention.py:149), which is a different policy: a stepper over such a trunk therefore wants the slot
+    count spelled out, 0 meaning that the policy has no bullet encoder and steps without them on purpose."""
+    if not trunk.config.reads_bullets:
+        if num_bullet_slots:
+            raise ValueError("this trunk has no bullet-reading sublayer")
+        return None, None
+    if num_bullet_slots is None:
+        raise ValueError("the trunk reads bullets: pass num_bullet_slots (0 to step without them on purpose)")
+    if num_bullet_slots == 0:
+        return None, None
+    bullets = torch.zeros(num_envs, num_bullet_slots, trunk.config.d_model, device=dev, dtype=dtype)
+    return bullets, torch.zeros(num_envs, num_bullet_slots, dtype=torch.bool, device=dev)
+
+
+def _weights_stamp(params) -> int:
+    """Changes whenever a parameter is written in place or touched through ``.data``."""
+    return sum(p._version + getattr(p, "_bnb_touch", 0) for p in params)
+
+
 class GraphedTrunk:
     """``YemongTrunk.forward`` for one fixed shape, captured into two HIP graphs and replayed.
 
     At rollout scale of a few thousand tokens a trunk step is ~100 short launches and the
     host, not the GPU, sets the pace (the reference notes the same of its own rollout).
-    Capturing the step removes that: ``step(tokens, alive_mask, reset_mask)`` copies the inputs
-    into static buffers, replays one graph and returns the static output and state tensors.
+    Capturing the step removes that: ``step(tokens, alive_mask, reset_mask, bullets, bullet_mask)`` copies
+    the inputs into static buffers, replays one graph and returns the static output and state tensors.
     The packed state lives in two buffers that alternate as input and output, hence two
     graphs.  Outputs are overwritten by the next ``step``; clone what must outlive it.
 
     Weights: the captured kernels read the parameters themselves (norm weights, float32 GEMM operands)
     and the derived copies the layers cache (bfloat16 casts, concatenations, operand packings) at the
-    addresses they had at capture time.  A replay runs no Python, so after a weight update (optimizer
-    step, ``load_state_dict``, a write through ``.data``) call ``refresh_weights()``: it rebuilds
-    every derived copy into the same memory.  This object keeps those copies alive, so nothing the
-    graphs read is ever returned to the allocator.  Replacing parameter tensors, moving or casting
-    the module requires a new capture.
+    addresses they had at capture time.  A replay runs no Python, so ``step`` first compares a stamp of the
+    parameters (version counters and ``.data`` accesses) with the one of the last step and, when it moved
+    (optimizer step, ``load_state_dict``, a write through ``.data``), rebuilds the derived copies whose
+    sources changed into the same memory; ``refresh_weights()`` rebuilds all of them unconditionally.
+    This object keeps those copies alive, so nothing the graphs read is ever returned to the allocator.
+    Replacing parameter tensors, moving or casting the module requires a new capture.
 
     Args:
         trunk: the module to capture.
         num_envs, num_tokens, num_recurrent: B, N+M and n_rec of every later call.
         autocast_dtype: ``torch.bfloat16`` to capture under autocast, None for fp32.
         use_reset: capture with a ``reset_mask`` input (all-False masks are then cheap no-ops).
+        num_bullet_slots: length of the bullet axis (ships x ring-buffer slots); required for a trunk whose
+            configuration reads bullets, 0 to step such a trunk without bullets on purpose.
+        bullet_dtype: dtype of the bullet tokens the caller's encoder emits (float32 by default).
     """
 
     def __init__(self, trunk: YemongTrunk, num_envs: int, num_tokens: int, num_recurrent: int, *,
-                 autocast_dtype: torch.dtype | None = None, use_reset: bool = True, device=None) -> None:
+                 autocast_dtype: torch.dtype | None = None, use_reset: bool = True, device=None,
+                 num_bullet_slots: int | None = None, bullet_dtype: torch.dtype = torch.float32) -> None:
         dev = torch.device(device) if device is not None else next(trunk.parameters()).device
         D = trunk.config.d_model
         self.trunk, self.autocast_dtype = trunk, autocast_dtype
         self.tokens = torch.zeros(num_envs, num_tokens, D, device=dev)
         self.alive = torch.ones(num_envs, num_tokens, dtype=torch.bool, device=dev)
         self.reset = torch.zeros(num_envs, dtype=torch.bool, device=dev) if use_reset else None
+        self.bullets, self.bullet_mask = _bullet_buffers(trunk, num_envs, num_bullet_slots, dev, bullet_dtype)
         self.states = [trunk.initial_hidden(num_envs, num_recurrent, dev) for _ in range(2)]
         self.cur = 0  # index of the buffer holding the current state
         self.graphs, self.outputs = [], []
@@ -1563,18 +1672,29 @@ class GraphedTrunk:
         for s in self.states:
             s.zero_()
         # the derived weights the captured kernels read: held here so their memory outlives any cache
-        # invalidation on the module, and rebuilt in place by refresh_weights()
+        # invalidation on the module, and rebuilt in place when their sources change
         self._derived = derived_weights(trunk)
+        self._params = list(trunk.parameters())
+        self._stamp = _weights_stamp(self._params)
 
     def refresh_weights(self) -> None:
         """Rebuild every derived weight copy the graphs read from the current parameters, in place."""
         for entry in self._derived:
             entry.refresh()
+        self._stamp = _weights_stamp(self._params)
+
+    def _follow_weights(self) -> None:
+        stamp = _weights_stamp(self._params)
+        if stamp != self._stamp:
+            for entry in self._derived:
+                if entry.key != _cache_key(entry.tensors, entry.dtype):
+                    entry.refresh()
+            self._stamp = stamp
 
     def _run(self, src: int) -> torch.Tensor:
         with torch.autocast("cuda", dtype=self.autocast_dtype or torch.bfloat16, enabled=self.autocast_dtype is not None):
-            out, _ = self.trunk(self.tokens, self.alive, self.states[src], reset_mask=self.reset,
-                                out_state=self.states[1 - src])
+            out, _ = self.trunk(self.tokens, self.alive, self.states[src], self.bullets, self.bullet_mask,
+                                reset_mask=self.reset, out_state=self.states[1 - src])
         return out
 
     @property
@@ -1586,12 +1706,14 @@ class GraphedTrunk:
         self.states[self.cur].copy_(state)
 
     @torch.no_grad()
-    def step(self, tokens, alive_mask, reset_mask=None):
+    def step(self, tokens, alive_mask, reset_mask=None, bullets=None, bullet_mask=None):
         """One trunk step on the captured shape; returns (hidden, new_state) static tensors.
 
-        The inputs are copied into the static buffers ``self.tokens`` / ``self.alive`` / ``self.reset``; a producer that
-        writes its result straight into those buffers passes the buffers themselves and no copy is made
-        (at 4096 environments x 160 tokens the token copy alone is 0.13 ms of a 4.5 ms step)."""
+        The inputs are copied into the static buffers ``self.tokens`` / ``self.alive`` / ``self.reset`` /
+        ``self.bullets`` / ``self.bullet_mask``; a producer that writes its result straight into those buffers
+        passes the buffers themselves and no copy is made (at 4096 environments x 160 tokens the token copy
+        alone is 0.13 ms of a 4.5 ms step).  A capture with bullet inputs needs them at every step;
+        ``bullet_mask=None`` then means every slot holds a bullet, as in the reference."""
         if tokens is not self.tokens:
             self.tokens.copy_(tokens)
         if alive_mask is not self.alive:
@@ -1603,6 +1725,18 @@ class GraphedTrunk:
                 self.reset.copy_(reset_mask)
         elif reset_mask is not None:
             raise ValueError("this capture was made without a reset input")
+        if self.bullets is not None:
+            if bullets is None:
+                raise ValueError("this capture reads bullets: pass bullets (and bullet_mask) at every step")
+            if bullets is not self.bullets:
+                self.bullets.copy_(bullets)
+            if bullet_mask is None:
+                self.bullet_mask.fill_(True)
+            elif bullet_mask is not self.bullet_mask:
+                self.bullet_mask.copy_(bullet_mask)
+        elif bullets is not None:
+            raise ValueError("this capture was made without bullet inputs")
+        self._follow_weights()
         self.graphs[self.cur].replay()
         out = self.outputs[self.cur]
         self.cur = 1 - self.cur
@@ -1611,13 +1745,19 @@ class GraphedTrunk:
 
 class EagerTrunkStepper:
     """``GraphedTrunk``'s interface on plain launches: the packed state alternates between two buffers it owns and
-    ``step(tokens, alive_mask, reset_mask)`` returns ``(hidden, new_state)``.  For batches large enough that the
-    kernels, not their launches, set the pace of a step."""
+    ``step(tokens, alive_mask, reset_mask, bullets, bullet_mask)`` returns ``(hidden, new_state)``.  For batches
+    large enough that the kernels, not their launches, set the pace of a step."""
 
     def __init__(self, trunk: YemongTrunk, num_envs: int, num_tokens: int, num_recurrent: int, *,
-                 autocast_dtype: torch.dtype | None = None, device=None) -> None:
+                 autocast_dtype: torch.dtype | None = None, device=None, num_bullet_slots: int | None = None,
+                 bullet_dtype: torch.dtype = torch.float32) -> None:
         dev = torch.device(device) if device is not None else next(trunk.parameters()).device
         self.trunk, self.autocast_dtype = trunk, autocast_dtype
+        if trunk.config.reads_bullets and num_bullet_slots is None:
+            raise ValueError("the trunk reads bullets: pass num_bullet_slots (0 to step without them on purpose)")
+        if num_bullet_slots and not trunk.config.reads_bullets:
+            raise ValueError("this trunk has no bullet-reading sublayer")
+        self.reads_bullets = bool(num_bullet_slots)
         self.states = [trunk.initial_hidden(num_envs, num_recurrent, dev) for _ in range(2)]
         self.cur = 0
 
@@ -1632,10 +1772,14 @@ class EagerTrunkStepper:
         self.states[self.cur].copy_(state)
 
     @torch.no_grad()
-    def step(self, tokens, alive_mask, reset_mask=None):
+    def step(self, tokens, alive_mask, reset_mask=None, bullets=None, bullet_mask=None):
+        if self.reads_bullets and bullets is None:
+            raise ValueError("this stepper reads bullets: pass bullets (and bullet_mask) at every step")
+        if not self.reads_bullets and bullets is not None:
+            raise ValueError("this stepper was made without bullet inputs")
         with torch.autocast("cuda", dtype=self.autocast_dtype or torch.bfloat16, enabled=self.autocast_dtype is not None):
-            out, new_state = self.trunk(tokens, alive_mask, self.states[self.cur], reset_mask=reset_mask,
-                                        out_state=self.states[1 - self.cur])
+            out, new_state = self.trunk(tokens, alive_mask, self.states[self.cur], bullets, bullet_mask,
+                                        reset_mask=reset_mask, out_state=self.states[1 - self.cur])
         self.cur = 1 - self.cur
         return out, new_state
 
@@ -1646,13 +1790,17 @@ GRAPH_BELOW_TOKENS = {torch.float32: 10_000, torch.bfloat16: 40_000}
 
 
 def trunk_stepper(trunk: YemongTrunk, num_envs: int, num_tokens: int, num_recurrent: int, *,
-                  autocast_dtype: torch.dtype | None = None, graph: bool | None = None, device=None):
+                  autocast_dtype: torch.dtype | None = None, graph: bool | None = None, device=None,
+                  num_bullet_slots: int | None = None, bullet_dtype: torch.dtype = torch.float32):
     """The rollout's way to step the trunk for one fixed shape: a ``GraphedTrunk`` (the step captured into HIP graphs)
     when ``num_envs * num_tokens`` is small enough that launches set the pace (``GRAPH_BELOW_TOKENS``), an
     ``EagerTrunkStepper`` above that; ``graph`` forces either.  Both own the packed state and share
-    ``step`` / ``state`` / ``load_state`` / ``refresh_weights``."""
+    ``step`` / ``state`` / ``load_state`` / ``refresh_weights``.  A trunk whose configuration reads bullets needs
+    ``num_bullet_slots`` (the length of the bullet axis; 0 to step without bullets on purpose)."""
     if graph is None:
         graph = num_envs * num_tokens < GRAPH_BELOW_TOKENS[torch.float32 if autocast_dtype is None else torch.bfloat16]
     if graph:
-        return GraphedTrunk(trunk, num_envs, num_tokens, num_recurrent, autocast_dtype=autocast_dtype, device=device)
-    return EagerTrunkStepper(trunk, num_envs, num_tokens, num_recurrent, autocast_dtype=autocast_dtype, device=device)
+        return GraphedTrunk(trunk, num_envs, num_tokens, num_recurrent, autocast_dtype=autocast_dtype, device=device,
+                            num_bullet_slots=num_bullet_slots, bullet_dtype=bullet_dtype)
+    return EagerTrunkStepper(trunk, num_envs, num_tokens, num_recurrent, autocast_dtype=autocast_dtype, device=device,
+                             num_bullet_slots=num_bullet_slots, bullet_dtype=bullet_dtype)

@@ -42,6 +42,7 @@ How each function is pinned (see tests/test_oracle_pins.py):
 
 from __future__ import annotations
 
+import contextlib
 import math
 
 import torch
@@ -150,9 +151,28 @@ def rglru_step(
 # Level M pieces (torch library ops around the two kernels)
 # --------------------------------------------------------------------------
 
+_NORM_EPS_DTYPE = None  # set by norm_eps_of(): the dtype whose eps the norms use, whatever dtype they compute in
+
+
+@contextlib.contextmanager
+def norm_eps_of(dtype: torch.dtype):
+    """Inside the block every ``rms_norm`` uses ``finfo(dtype).eps`` instead of the eps of the dtype it is handed.
+
+    ``nn.RMSNorm(D)`` takes its eps from the input's dtype, so the float32 module and the same formulas typed in
+    float64 are two slightly different functions.  A float64 evaluation that is to serve as the exact value of the
+    float32 module (the yardstick of the composed float32 tests) keeps the float32 eps: ``norm_eps_of(torch.float32)``."""
+    global _NORM_EPS_DTYPE
+    keep, _NORM_EPS_DTYPE = _NORM_EPS_DTYPE, dtype
+    try:
+        yield
+    finally:
+        _NORM_EPS_DTYPE = keep
+
+
 def rms_norm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``nn.RMSNorm(D)`` with its default ``eps=None`` (=> finfo(x.dtype).eps)."""
-    return F.rms_norm(x, (x.shape[-1],), weight, None)
+    eps = None if _NORM_EPS_DTYPE is None else torch.finfo(_NORM_EPS_DTYPE).eps
+    return F.rms_norm(x, (x.shape[-1],), weight, eps)
 
 
 def gated_mlp(p: dict, prefix: str, x: torch.Tensor) -> torch.Tensor:

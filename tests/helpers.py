@@ -109,3 +109,40 @@ def team_case(seed: int, B: int, N: int, p_alive: float = 0.7):
         alive[3] = False
         alive[3, N - 1] = True
     return team, alive
+
+
+F32_COMPOSED_TOL = 1e-5  # the float32 bar of the step, applied to compositions through ``assert_float32_bar``
+
+
+def as_float64(p: dict) -> dict:
+    return {k: v.double() for k, v in p.items()}
+
+
+def float64_truth(fn, *args, **kwargs):
+    """``fn`` of the torch oracle evaluated in float64 on the same (float32) numbers, with the float32 module's
+    norm eps: the exact value of the function the float32 module computes, up to float64 rounding."""
+    from oracle import torch_ref
+
+    def widen(a):
+        if isinstance(a, dict):
+            return as_float64(a)
+        if isinstance(a, torch.Tensor) and a.is_floating_point():
+            return a.double()
+        return a
+
+    with torch_ref.norm_eps_of(torch.float32):
+        return fn(*[widen(a) for a in args], **{k: widen(v) for k, v in kwargs.items()})
+
+
+def assert_float32_bar(got: torch.Tensor, ref32: torch.Tensor, ref64: torch.Tensor, what, tol: float = F32_COMPOSED_TOL):
+    """The bar of a float32 composition several sublayers deep.
+
+    ``ref64`` is the exact value (``float64_truth``), ``ref32`` what the float32 torch oracle makes of the same
+    inputs.  The kernels pass when they are within ``tol`` (max |error| / max |value|) of the exact value, or
+    no further from it than the float32 oracle is: a composition cannot be asked to round better than the
+    reference's own arithmetic does.  Both errors are printed (``pytest -s`` shows them)."""
+    scale = ref64.abs().max().clamp_min(1e-30)
+    err_kernels = float((got.double() - ref64).abs().max() / scale)
+    err_oracle = float((ref32.double() - ref64).abs().max() / scale)
+    print(f"float32 bar [{what}]: kernels vs float64 {err_kernels:.2e}, float32 oracle vs float64 {err_oracle:.2e}", flush=True)
+    assert err_kernels <= max(tol, err_oracle), (what, err_kernels, err_oracle)

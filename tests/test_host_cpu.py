@@ -208,3 +208,66 @@ def test_backward_weight_pack_follows_the_documented_operand_order():
         at = ((cb * 2 + t) * 64 + l) * 8 + e
         assert pk[c, 3, at] == wg.bfloat16().float()[32 * c + 16 * t + 8 * b + e, 32 * cb + pi(m)]
         assert pk[c, 4, at] == wu.bfloat16().float()[32 * c + 16 * t + 8 * b + e, 32 * cb + pi(m)]
+
+
+def test_layer_parameters_notice_writes_through_data_and_stay_ordinary_parameters():
+    # train/rl/opponents.py:107-112 overwrites the averaged policy with avg_parameter.data.copy_(...), which
+    # leaves the version counter alone: the layers' parameters count .data accesses instead
+    import copy
+    import io
+
+    from boost_and_broadside_amd import trunk as trunk_module
+
+    cfg = bnb.ModelConfig(d_model=32, n_heads=4, n_yemong_blocks=2, n_spatial_per_block=2, n_bullet_cross_per_block=1)
+    trunk = bnb.YemongTrunk(cfg)
+    params = dict(trunk.named_parameters())
+    assert params and all(type(p) is trunk_module.WatchedParameter for p in params.values())
+    assert all(isinstance(p, torch.nn.Parameter) and p.is_leaf and p.requires_grad for p in params.values())
+    w = params["yemong_layers.0.spatial.0.qkv.weight"]
+    key = trunk_module._cache_key((w,), torch.bfloat16)
+    w.data.copy_(torch.ones_like(w))
+    assert w._version == 0 and float(w.detach()[0, 0]) == 1.0
+    assert trunk_module._cache_key((w,), torch.bfloat16) != key  # the write is seen although the version is not
+    key = trunk_module._cache_key((w,), torch.bfloat16)
+    with torch.no_grad():
+        w.mul_(2.0)
+    assert trunk_module._cache_key((w,), torch.bfloat16) != key
+    # state_dict, deepcopy, pickling, casts and assign-loading keep the names, the values and the watching
+    assert sorted(trunk.state_dict()) == sorted(params)
+    for other in (copy.deepcopy(trunk), torch.load(_pickled(trunk), weights_only=False), copy.deepcopy(trunk).double()):
+        assert all(type(p) is trunk_module.WatchedParameter for p in other.parameters())
+        assert all(torch.equal(a.float(), b) for a, b in zip(other.parameters(), trunk.parameters()))
+    fresh = bnb.YemongTrunk(cfg)
+    fresh.load_state_dict({k: v.clone() for k, v in trunk.state_dict().items()}, assign=True)
+    assert all(type(p) is trunk_module.WatchedParameter for p in fresh.parameters())
+    assert float(fresh.yemong_layers[0].spatial[0].qkv.weight.detach()[0, 0]) == 2.0
+    # gradients and optimizers see ordinary leaves
+    lin = trunk.yemong_layers[0].spatial[0].out_proj
+    lin(torch.ones(2, 32)).sum().backward()
+    assert lin.weight.grad is not None and type(lin.weight.grad) is torch.Tensor
+    torch.optim.SGD(trunk.parameters(), lr=0.1).step()
+
+
+def _pickled(module):
+    import io
+
+    buf = io.BytesIO()
+    torch.save(module, buf)
+    buf.seek(0)
+    return buf
+
+
+def test_steppers_refuse_to_drop_the_bullets_of_a_bullet_reading_trunk():
+    from boost_and_broadside_amd import trunk as trunk_module
+
+    cfg = bnb.ModelConfig(d_model=32, n_heads=4, n_yemong_blocks=1, n_spatial_per_block=1, n_bullet_cross_per_block=1)
+    trunk = bnb.YemongTrunk(cfg)
+    with pytest.raises(ValueError, match="num_bullet_slots"):
+        trunk_module._bullet_buffers(trunk, 4, None, "cpu", torch.float32)
+    assert trunk_module._bullet_buffers(trunk, 4, 0, "cpu", torch.float32) == (None, None)
+    bullets, mask = trunk_module._bullet_buffers(trunk, 4, 80, "cpu", torch.float32)
+    assert bullets.shape == (4, 80, 32) and mask.shape == (4, 80) and mask.dtype == torch.bool and not mask.any()
+    plain = bnb.YemongTrunk(bnb.ModelConfig(d_model=32, n_heads=4, n_yemong_blocks=1))
+    with pytest.raises(ValueError, match="no bullet-reading"):
+        trunk_module._bullet_buffers(plain, 4, 80, "cpu", torch.float32)
+    assert trunk_module._bullet_buffers(plain, 4, None, "cpu", torch.float32) == (None, None)

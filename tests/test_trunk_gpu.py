@@ -11,7 +11,8 @@ norms and GELUs are library calls on both sides.
 import pytest
 import torch
 
-from helpers import block_params, max_rel, team_case, team_pool_params, temporal_params, trunk_params
+from helpers import (assert_float32_bar, block_params, float64_truth, max_rel, team_case, team_pool_params, temporal_params,
+                     trunk_params)
 from oracle import torch_ref
 
 import boost_and_broadside_amd as bnb
@@ -199,8 +200,10 @@ def test_temporal_block_sequence_with_done_matches_oracle_sequence():
     with torch.no_grad():
         out, h1, cb1 = layer.forward_sequence(x_seq.to(DEV), h0.to(DEV), cb.to(DEV), done.to(DEV))
     ref_out, ref_h, ref_cb = torch_ref.temporal_sequence(p, "t.", x_seq, h0, cb, done)
-    assert max_rel(out.cpu(), ref_out) <= 2e-5
-    assert max_rel(h1.cpu(), ref_h) <= 2e-5 and torch.allclose(cb1.cpu(), ref_cb, atol=1e-5)
+    t_out, t_h, t_cb = float64_truth(torch_ref.temporal_sequence, p, "t.", x_seq, h0, cb, done)
+    assert_float32_bar(out.cpu(), ref_out, t_out, "temporal sequence, output")
+    assert_float32_bar(h1.cpu(), ref_h, t_h, "temporal sequence, state")
+    assert_float32_bar(cb1.cpu(), ref_cb, t_cb, "temporal sequence, conv inputs")
 
 
 @pytest.mark.parametrize("time_major", [False, True])
@@ -247,10 +250,12 @@ def test_block_step_matches_oracle(spatial, temporal, N, M):
     with torch.no_grad():
         out, h1, cb1 = block.step(x.to(DEV), alive.to(DEV), h.to(DEV), cb.to(DEV), N)
     ref_out, ref_h, ref_cb = torch_ref.block_step(p, "b.", spatial, temporal, H, x, alive, h, cb, N)
+    t_out, t_h, t_cb = float64_truth(torch_ref.block_step, p, "b.", spatial, temporal, H, x, alive, h, cb, N)
     assert out.shape == x.shape and h1.shape == h.shape and cb1.shape == cb.shape
-    assert max_rel(out.cpu(), ref_out) <= 2e-5
+    assert_float32_bar(out.cpu(), ref_out, t_out, f"block step {spatial}+{temporal}, output")
     if temporal:
-        assert max_rel(h1.cpu(), ref_h) <= 2e-5 and max_rel(cb1.cpu(), ref_cb) <= 2e-5
+        assert_float32_bar(h1.cpu(), ref_h, t_h, f"block step {spatial}+{temporal}, state")
+        assert_float32_bar(cb1.cpu(), ref_cb, t_cb, f"block step {spatial}+{temporal}, conv inputs")
 
 
 @pytest.mark.parametrize("blocks,spatial,temporal", [(2, 1, 1), (2, 2, 1), (1, 3, 2)])
@@ -269,13 +274,14 @@ def test_trunk_step_equals_sequence_and_oracle(blocks, spatial, temporal):
     hidden0 = trunk.initial_hidden(B, N, DEV)
     assert hidden0.shape == (blocks * temporal, B * N, 4 * D)
 
-    hidden, ref_hidden, outs = hidden0, hidden0.cpu(), []
+    hidden, ref_hidden, true_hidden, outs = hidden0, hidden0.cpu(), hidden0.cpu().double(), []
     for t in range(T):
         out, hidden = trunk(xs[t].to(DEV), alive[t].to(DEV), hidden)
         ref_out, ref_hidden = torch_ref.trunk_step(p, blocks, spatial, temporal, H, xs[t], alive[t], ref_hidden)
-        assert max_rel(out.cpu(), ref_out) <= 5e-5, t
+        true_out, true_hidden = float64_truth(torch_ref.trunk_step, p, blocks, spatial, temporal, H, xs[t], alive[t], true_hidden)
+        assert_float32_bar(out.cpu(), ref_out, true_out, f"trunk {blocks}x({spatial}+{temporal}) step {t}, output")
         outs.append(out)
-    assert max_rel(hidden.cpu(), ref_hidden) <= 5e-5
+    assert_float32_bar(hidden.cpu(), ref_hidden, true_hidden, f"trunk {blocks}x({spatial}+{temporal}) after {T} steps, state")
 
     # sequence path over the same inputs
     x = xs.to(DEV)
@@ -326,8 +332,10 @@ def test_state_sized_with_all_tokens_makes_fields_recurrent():
     hidden = torch.randn(1, B * (N + M), 4 * D, generator=gen)
     out, new_hidden = trunk(x.to(DEV), alive.to(DEV), hidden.to(DEV))
     ref_out, ref_hidden = torch_ref.trunk_step(p, 1, 1, 1, H, x, alive, hidden)
+    true_out, true_hidden = float64_truth(torch_ref.trunk_step, p, 1, 1, 1, H, x, alive, hidden)
     assert new_hidden.shape == hidden.shape
-    assert max_rel(out.cpu(), ref_out) <= 2e-5 and max_rel(new_hidden.cpu(), ref_hidden) <= 2e-5
+    assert_float32_bar(out.cpu(), ref_out, true_out, "trunk with recurrent fields, output")
+    assert_float32_bar(new_hidden.cpu(), ref_hidden, true_hidden, "trunk with recurrent fields, state")
 
 
 def test_trunk_under_autocast_matches_oracle_within_bf16_bar():
@@ -371,7 +379,9 @@ def test_trunk_folded_reset_equals_reset_then_step_and_leaves_input_state_alone(
     out_b, state_b = trunk(x.to(DEV), alive.to(DEV), trunk.reset_hidden_for_envs(dev_hidden, done.to(DEV), N))
     assert torch.equal(out_a, out_b) and torch.equal(state_a, state_b)
     ref_out, ref_state = torch_ref.trunk_step(p, 2, 2, 1, H, x, alive, torch_ref.reset_hidden(hidden, done, N))
-    assert max_rel(out_a.cpu(), ref_out) <= 5e-5 and max_rel(state_a.cpu(), ref_state) <= 5e-5
+    true_out, true_state = float64_truth(torch_ref.trunk_step, p, 2, 2, 1, H, x, alive, torch_ref.reset_hidden(hidden, done, N))
+    assert_float32_bar(out_a.cpu(), ref_out, true_out, "trunk with folded reset, output")
+    assert_float32_bar(state_a.cpu(), ref_state, true_state, "trunk with folded reset, state")
     # preallocated destination
     dest = torch.empty_like(dev_hidden)
     _, state_c = trunk(x.to(DEV), alive.to(DEV), dev_hidden, reset_mask=done.to(DEV), out_state=dest)
@@ -933,24 +943,41 @@ def test_weight_updates_after_the_first_forward_reach_the_cached_copies(autocast
     x = torch.randn(B, N + M, D, generator=gen)
     alive = torch.ones(B, N + M, dtype=torch.bool)
     hidden = torch.randn(2, B * N, 4 * D, generator=gen)
-    tol = BF16_TOL if autocast else 5e-5
 
     def run_and_check(p_now):
         with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
             out, new_hidden = trunk(x.to(DEV), alive.to(DEV), hidden.to(DEV))
         ref_out, ref_hidden = torch_ref.trunk_step(p_now, 2, 2, 1, H, x, alive, hidden)
-        assert max_rel(out.cpu(), ref_out) <= tol and max_rel(new_hidden.cpu(), ref_hidden) <= tol
+        if autocast:
+            assert max_rel(out.cpu(), ref_out) <= BF16_TOL and max_rel(new_hidden.cpu(), ref_hidden) <= BF16_TOL
+        else:
+            true_out, true_hidden = float64_truth(torch_ref.trunk_step, p_now, 2, 2, 1, H, x, alive, hidden)
+            assert_float32_bar(out.cpu(), ref_out, true_out, "trunk after a weight update, output")
+            assert_float32_bar(new_hidden.cpu(), ref_hidden, true_hidden, "trunk after a weight update, state")
         return out
 
     first = run_and_check({k: v.detach().cpu() for k, v in trunk.state_dict().items()})
 
-    # 1. a write through .data, then the documented call
+    # 1. a write through .data exactly as the trainer's running average does it, and no call after it
     other = trunk_params(77, D, 2, 2, 1)
-    for name, param in trunk.named_parameters():
-        param.data.copy_(other[name])
-    trunk.invalidate_weight_caches()
+    cumsum = [2.0 * other[name].to(DEV) for name, _ in trunk.named_parameters()]
+    for avg_parameter, cumulative in zip(trunk.parameters(), cumsum):
+        avg_parameter.data.copy_(cumulative / 2)
+    assert bnb.trunk.verify_weight_caches(trunk) == []  # every cache already knows it is out of date
     second = run_and_check(other)
     assert not torch.equal(first, second)
+    assert bnb.trunk.verify_weight_caches(trunk) == []
+
+    # 1b. a write the layers cannot see (through an alias taken earlier) is what verify_weight_caches reports
+    #     and invalidate_weight_caches repairs
+    aliases = [param.data for param in trunk.parameters()]
+    run_and_check(other)  # the caches are rebuilt once more (the .data reads above) and are current again
+    stale_free = trunk_params(79, D, 2, 2, 1)
+    for (name, _), alias in zip(trunk.named_parameters(), aliases):
+        alias.copy_(stale_free[name])
+    assert bnb.trunk.verify_weight_caches(trunk) != []
+    trunk.invalidate_weight_caches()
+    run_and_check(stale_free)
 
     # 2. an optimizer step (in-place on the parameters: seen without any call)
     opt = torch.optim.SGD(trunk.parameters(), lr=0.05)
@@ -994,16 +1021,84 @@ def test_graphed_trunk_sees_new_weights_after_refresh(autocast_dtype):
         else:
             with torch.no_grad():
                 param.copy_(other[name])
-    graphed.refresh_weights()
-    trunk.invalidate_weight_caches()  # for the eager side of the comparison (the .data writes)
-    both(1)
+    both(1)  # no refresh_weights(), no invalidate call: the step follows the parameters by itself
     both(2)
+    # the trainer's running average once more, between two replays
+    for param in trunk.parameters():
+        param.data.copy_(0.5 * param.detach() + 0.01)
+    both(21)
+    # and the explicit call still works
+    with torch.no_grad():
+        for param in trunk.parameters():
+            param.mul_(1.01)
+    graphed.refresh_weights()
+    both(22)
     # the module dropping its caches must not take away memory the graphs read
     trunk.invalidate_weight_caches(drop=True)
     torch.cuda.empty_cache()
     scratch = [torch.randn(1 << 16, device=DEV) for _ in range(64)]  # reuses whatever was freed
     both(3)
     del scratch
+
+
+def _bullet_trunk(seed, D=128, H=4):
+    p = trunk_params(seed, D, 2, 2, 1)
+    gen = torch.Generator().manual_seed(seed + 1000)
+    for b in range(2):
+        p[f"yemong_layers.{b}.spatial.0.norm_bullet.weight"] = 1.0 + 0.1 * torch.randn(D, generator=gen)
+        p[f"yemong_layers.{b}.spatial.0.kv_bullet.weight"] = 0.1 * torch.randn(2 * D, D, generator=gen)
+    trunk = bnb.YemongTrunk(_cfg(D, H, 2, 2, 1, bullets=1)).eval()
+    trunk.load_state_dict(p)
+    return trunk.to(DEV), p
+
+
+@pytest.mark.parametrize("graph", [True, False])
+@pytest.mark.parametrize("autocast_dtype", [None, torch.bfloat16])
+def test_steppers_over_a_bullet_reading_trunk_take_the_bullets_and_match_the_plain_forward(graph, autocast_dtype):
+    # the shipped default reads bullets (config/defaults.py:29): a stepper that dropped them would step another policy
+    D, H, B, N, M, K = 128, 4, 16, 8, 4, 10
+    trunk, p = _bullet_trunk(91)
+    with pytest.raises(ValueError, match="num_bullet_slots"):
+        bnb.trunk_stepper(trunk, B, N + M, N, autocast_dtype=autocast_dtype, graph=graph)
+    stepper = bnb.trunk_stepper(trunk, B, N + M, N, autocast_dtype=autocast_dtype, graph=graph, num_bullet_slots=N * K)
+    gen = torch.Generator().manual_seed(92)
+    eager_state = trunk.initial_hidden(B, N, DEV)
+    alive = torch.ones(B, N + M, dtype=torch.bool)
+    with pytest.raises(ValueError, match="bullets"):
+        stepper.step(torch.zeros(B, N + M, D, device=DEV), alive.to(DEV))
+    for t in range(5):
+        x = torch.randn(B, N + M, D, generator=gen).to(DEV)
+        alive[:, :N] &= torch.rand(B, N, generator=gen) > 0.1
+        bullets = torch.randn(B, N * K, D, generator=gen).to(DEV)
+        bmask = torch.rand(B, N * K, generator=gen) < (0.0 if t == 1 else 0.3)  # one step with nothing in flight
+        bmask[3] = False
+        done = torch.rand(B, generator=gen) < 0.2 if t == 2 else None
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast_dtype is not None):
+            ref_out, eager_state = trunk(x, alive.to(DEV), eager_state, bullets, bmask.to(DEV),
+                                         reset_mask=None if done is None else done.to(DEV))
+            no_read, _ = trunk(x, alive.to(DEV), stepper.state.clone(), reset_mask=None if done is None else done.to(DEV))
+        torch.cuda.synchronize()
+        out, state = stepper.step(x, alive.to(DEV), None if done is None else done.to(DEV), bullets, bmask.to(DEV))
+        assert torch.equal(out, ref_out), t
+        assert torch.equal(state, eager_state), t
+        if t != 1:
+            assert not torch.equal(out, no_read), t  # the read does change the result
+    # and against the oracle on the last step's inputs
+    hidden0 = torch.randn(2, B * N, 4 * D, generator=gen)
+    stepper.load_state(hidden0.to(DEV))
+    out, state = stepper.step(x, alive.to(DEV), None, bullets, bmask.to(DEV))
+    ref_out, ref_hidden = torch_ref.trunk_step(p, 2, 2, 1, H, x.cpu(), alive, hidden0, bullets=bullets.cpu(), bullet_mask=bmask)
+    if autocast_dtype is not None:
+        assert max_rel(out.float().cpu(), ref_out) <= BF16_TOL and max_rel(state.cpu(), ref_hidden) <= BF16_TOL
+    else:
+        true_out, true_hidden = float64_truth(torch_ref.trunk_step, p, 2, 2, 1, H, x.cpu(), alive, hidden0, bullets=bullets.cpu(),
+                                              bullet_mask=bmask)
+        assert_float32_bar(out.cpu(), ref_out, true_out, "stepper with bullets, output")
+        assert_float32_bar(state.cpu(), ref_hidden, true_hidden, "stepper with bullets, state")
+    # a stepper without bullets over a trunk that reads none keeps its old signature
+    plain_trunk, _ = _rollout_trunk(93)
+    with pytest.raises(ValueError, match="no bullet-reading"):
+        bnb.trunk_stepper(plain_trunk, B, N + M, N, graph=False, num_bullet_slots=80)
 
 
 def test_block_step_and_single_step_sequence_work_in_grad_mode_and_match_autograd_through_the_oracle():
