@@ -41,6 +41,7 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="time the step loop as eager launches only (no HIP graph replay)")
     ap.add_argument("--no-torch-baseline", action="store_true")
     ap.add_argument("--no-module", action="store_true")
+    ap.add_argument("--no-issue-probe", action="store_true", help="skip the matrix-core / vector-ALU issue-rate yardstick")
     ap.add_argument("--no-ffn", action="store_true", help="skip the fused sublayer-tail leg")
     ap.add_argument("--no-bullets", action="store_true", help="skip the bullet-read leg")
     ap.add_argument("--no-sequence", action="store_true", help="skip the update-path (T = 128) recurrence leg")
@@ -464,6 +465,23 @@ def main():
     t_copy = timed_loop(lambda t: ops.copy_bytes(src, dst), 20, 3) / 20
     result["copy_kernel"] = {"GBps_read_plus_write": 2 * n_copy / t_copy / 1e9, "bytes": n_copy}
     del src, dst
+
+    # ---- yardstick of the issue-bound kernels: how a SIMD's issue is shared by matrix products and vector arithmetic ----
+    if not args.no_issue_probe:
+        mfma_only = ops.issue_probe(0)
+        fma16 = ops.issue_probe(16, mfma=False)
+        sweep = {str(m): ops.issue_probe(m) for m in (2, 4, 8, 12, 16)}
+        mixed = ops.issue_probe(10, transcendentals=True)
+        mixed_alone = ops.issue_probe(10, mfma=False, transcendentals=True)
+        result["issue_probe"] = {
+            "ns_per_slot": {"mfma_only": mfma_only, "16_fma_only": fma16, "mfma_plus_n_fma": sweep,
+                            "mfma_plus_8_fma_2_exp": mixed, "8_fma_2_exp_only": mixed_alone},
+            # 1 = the matrix product and the vector work take as long together as one after the other, 0 = the shorter
+            # of the two disappears under the longer
+            "serial_fraction_mfma_plus_16_fma": (sweep["16"] - max(mfma_only, fma16)) / min(mfma_only, fma16),
+            "what": "bnb_issue_probe at two waves per SIMD: one 32x32x16 bf16 matrix product followed by n independent "
+                    "vector instructions, order pinned; nanoseconds per such slot on one SIMD",
+        }
 
     # ---- the same two regions through eager PyTorch on the GPU ----
     if not args.no_torch_baseline:

@@ -12,7 +12,7 @@ import os
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "_lib", "libbnb_amd.so")
 
-ABI_VERSION = 25
+ABI_VERSION = 26
 F32, BF16 = 0, 1
 PATH_AUTO, PATH_VALU, PATH_MFMA, PATH_ENV, PATH_HEAD = 0, 1, 2, 3, 4
 WGRAD_PATH_AUTO, WGRAD_PATH_STAGED, WGRAD_PATH_DMA = 0, 1, 2
@@ -84,6 +84,7 @@ SIGNATURES = {
     "bnb_ffn_fused_proj_fwd": (_i, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _f, _vp, _vp, _i64, _i, _i, _vp]),
     "bnb_gelu_mul_fwd": (_i, [_vp, _i, _i64, _vp, _i, _i64, _vp, _i, _i64, _i, _vp]),
     "bnb_copy_bytes": (_i, [_vp, _vp, _i64, _vp]),
+    "bnb_issue_probe": (_i, [_i, _i, _i, _i, _i, _vp, _vp]),
 }
 
 _lib = None

@@ -16,7 +16,7 @@ INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_DIR = os.path.join(PKG_DIR, "_lib")
 LIB_PATH = os.path.join(LIB_DIR, "libbnb_amd.so")
 SOURCES = ("abi.hip", "conv_step.hip", "elementwise.hip", "ffn_bwd.hip", "ffn_fused.hip", "linear_f32.hip", "linear_wgrad.hip",
-    "norm_train.hip", "norm_linear.hip", "rglru_step.hip", "sdpa_bwd.hip", "sdpa_cross_bwd.hip", "sdpa_cross_f32.hip", "sdpa_env.hip", "sdpa_masked.hip", "team_pool.hip", "temporal_seq.hip", "temporal_step.hip")
+    "norm_train.hip", "norm_linear.hip", "probe.hip", "rglru_step.hip", "sdpa_bwd.hip", "sdpa_cross_bwd.hip", "sdpa_cross_f32.hip", "sdpa_env.hip", "sdpa_masked.hip", "team_pool.hip", "temporal_seq.hip", "temporal_step.hip")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -1806,6 +1806,28 @@ def copy_bytes(src: torch.Tensor, dst: torch.Tensor) -> None:
     _native.check(rc, "bnb_copy_bytes")
 
 
+def issue_probe(valu_per_mfma: int, *, mfma: bool = True, transcendentals: bool = False, waves_per_simd: int = 2,
+                iters: int = 20000, device=None) -> float:
+    """Issue time in nanoseconds of one slot = one 32x32x16 bfloat16 matrix product (``mfma``) followed by
+    ``valu_per_mfma`` independent vector instructions (multiply-adds, every fifth one an exp2 with
+    ``transcendentals``) on one SIMD carrying ``waves_per_simd`` waves: the yardstick for the kernels that are bound
+    by instruction issue rather than by bandwidth (``bnb_issue_probe``).  Synchronises the device."""
+    dev = torch.device(device if device is not None else "cuda")
+    sink = torch.zeros(256, dtype=torch.float32, device=dev)
+    lib = _native.load()
+    with _on_device(sink.device):
+        def launch(n):
+            _native.check(lib.bnb_issue_probe(int(valu_per_mfma), int(mfma), int(transcendentals), int(waves_per_simd), n,
+                                              sink.data_ptr(), _stream()), "bnb_issue_probe")
+        launch(200)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        launch(iters)
+        stop.record()
+        stop.synchronize()
+    return start.elapsed_time(stop) * 1e6 / (4.0 * iters * waves_per_simd)
+
+
 FFN_WIDTH, FFN_HIDDEN = 128, 512
 
 

@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 25
+#define BNB_ABI_VERSION 26
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -873,6 +873,19 @@ int bnb_gelu_mul_bwd(const void *a, int a_dtype, int64_t a_row_stride, const voi
  * byte counters.
  */
 int bnb_copy_bytes(const void *src, void *dst, int64_t bytes, void *stream);
+
+/*
+ * Issue-rate yardstick.  It has no counterpart in the reference: like bnb_copy_bytes for the bandwidth-bound
+ * kernels, it gives the benchmark the hardware figure that bounds the matrix-core kernels of this library (the
+ * gated MLP of models/yemong/attention.py:21-37 and the attention of :147 spend their time issuing matrix
+ * products and vector arithmetic on the same SIMDs).  One launch runs, on `waves_per_simd` (1 or 2) waves per SIMD
+ * of every compute unit, `iters` rounds of four slots; a slot is one 32x32x16 bf16 matrix product (if
+ * `with_mfma`) followed by `valu_per_mfma` (0, 2, 4, 8, 10, 12 or 16) independent vector instructions:
+ * multiply-adds, every fifth one an exp2 if `with_transcendentals`.  The caller times the launch; time /
+ * (4 iters waves_per_simd) is the issue time of one slot on one SIMD.  `sink` (>= 1 KiB) is never written.
+ */
+int bnb_issue_probe(int valu_per_mfma, int with_mfma, int with_transcendentals, int waves_per_simd, int iters,
+                    float *sink, void *stream);
 
 #ifdef __cplusplus
 }

@@ -2728,3 +2728,22 @@ def test_norm_linear_train_refuses_what_the_kernel_does_not_cover():
     assert lib.bnb_norm_linear_train_fwd(*args(128, 96, n.data_ptr())) == _native.ERR_UNSUPPORTED
     assert lib.bnb_norm_linear_train_fwd(*args(128, 128, None)) == 10001  # BNB_ERR_NULL_POINTER
     assert not ops.norm_linear_train_supported(x, torch.zeros(64, 128, device=DEV))  # the weight-gradient kernel wants 128s
+
+
+def test_issue_probe_reports_a_plausible_matrix_product_time_and_rejects_bad_arguments():
+    # the yardstick of the issue-bound kernels: a 32x32x16 bf16 matrix product occupies a SIMD's matrix core for 32
+    # cycles, i.e. 13-20 ns at the clocks this part runs at; vector work added to it can only make a slot longer
+    from boost_and_broadside_amd import _native
+
+    alone = ops.issue_probe(0, iters=4000)
+    with_valu = ops.issue_probe(16, iters=4000)
+    valu_alone = ops.issue_probe(16, mfma=False, iters=4000)
+    assert 8.0 < alone < 40.0, alone
+    assert with_valu >= alone and with_valu >= valu_alone
+    assert with_valu <= 1.2 * (alone + valu_alone)
+    lib = _native.load()
+    sink = torch.zeros(256, device=DEV)
+    assert lib.bnb_issue_probe(3, 1, 0, 2, 10, sink.data_ptr(), None) == _native.ERR_UNSUPPORTED
+    assert lib.bnb_issue_probe(8, 1, 0, 3, 10, sink.data_ptr(), None) == 10003  # BNB_ERR_BAD_SHAPE
+    assert lib.bnb_issue_probe(8, 1, 0, 2, 10, None, None) == 10001  # BNB_ERR_NULL_POINTER
+    assert not sink.any()
