@@ -11,6 +11,8 @@ synchronise.  They are forward-only and run on a ROCm device only: anything else
 
 from __future__ import annotations
 
+import os
+
 import functools
 import math
 
@@ -2305,8 +2307,13 @@ class CompactRows:
 
     ``total`` / ``max_count`` (optional Python ints): the number of set entries and the largest count of
     one row, for a caller that knows them already (e.g. counted when the rollout was stored).  The
-    update path sizes gathered tensors with them; without the hint ``total_host()`` copies them from
-    the device once, which makes the host wait for everything queued before."""
+    update path sizes gathered tensors with them and picks the single-tile or the streaming backward by
+    ``max_count``; without the hint ``total_host()`` copies them from the device once, which makes the host
+    wait for everything queued before.  The hints are taken on trust: a ``total`` below the true count makes
+    the gathered tensors too small for what the kernels write, a ``max_count`` below the true one sends a row with
+    more than 160 entries to the single-tile backward, and either is undefined behaviour.  ``check_hints()``
+    compares them with the device's counts (one copy to the host); with ``BNB_CHECK_HINTS=1`` in the environment
+    every construction with hints does that."""
 
     def __init__(self, mask: torch.Tensor, *, total: int | None = None, max_count: int | None = None) -> None:
         if mask.dim() != 2 or mask.dtype not in (torch.bool, torch.uint8):
@@ -2321,6 +2328,7 @@ class CompactRows:
         if (total is None) != (max_count is None):
             raise ValueError("give both total and max_count, or neither")
         self._host = None if total is None else (int(total), int(max_count))
+        self._hinted = total is not None
         self.shared_kv = None  # set by the trunk: {id(layer): [K | V] rows of the listed entries}, one projection pass for all readers
         counts = torch.empty(B, dtype=torch.int32, device=mask.device)
         self.offsets = torch.zeros(B + 1, dtype=torch.int32, device=mask.device)
@@ -2332,6 +2340,25 @@ class CompactRows:
                 torch.cumsum(counts, dim=0, dtype=torch.int32, out=self.offsets[1:])
                 _native.check(lib.bnb_mask_fill(mask.data_ptr(), self.offsets.data_ptr(), self.index.data_ptr(), B, n,
                                                 _stream()), "bnb_mask_fill")
+
+        if self._hinted and os.environ.get("BNB_CHECK_HINTS") == "1":
+            self.check_hints()
+
+    def check_hints(self) -> None:
+        """Raise ``ValueError`` unless the ``total`` / ``max_count`` given at construction equal the device's counts
+        (``total``) or bound them from above (``max_count``).  Copies two integers to the host."""
+        if not self._hinted:
+            return
+        B = self.shape[0]
+        if B == 0:
+            true_total, true_max = 0, 0
+        else:
+            per_row = self.offsets[1:] - self.offsets[:-1]
+            true_total, true_max = (int(v) for v in torch.stack([self.offsets[-1], per_row.max()]).tolist())
+        total, max_count = self._host
+        if total != true_total or max_count < true_max:
+            raise ValueError(f"CompactRows hints total={total}, max_count={max_count} do not fit the mask: it has "
+                             f"{true_total} set entries, at most {true_max} in one row")
 
     @property
     def total(self) -> torch.Tensor:

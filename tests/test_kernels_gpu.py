@@ -2747,3 +2747,21 @@ def test_issue_probe_reports_a_plausible_matrix_product_time_and_rejects_bad_arg
     assert lib.bnb_issue_probe(8, 1, 0, 3, 10, sink.data_ptr(), None) == 10003  # BNB_ERR_BAD_SHAPE
     assert lib.bnb_issue_probe(8, 1, 0, 2, 10, None, None) == 10001  # BNB_ERR_NULL_POINTER
     assert not sink.any()
+
+
+def test_compact_rows_hints_are_checked_on_request(monkeypatch):
+    # a caller that counted the live bullets when the rollout was stored hands the counts over; wrong ones are
+    # undefined behaviour in the kernels, so there is a way to find them
+    gen = torch.Generator().manual_seed(5)
+    mask = (torch.rand(9, 40, generator=gen) < 0.3).to(DEV)
+    total, most = int(mask.sum()), int(mask.sum(dim=1).max())
+    ops.CompactRows(mask, total=total, max_count=most).check_hints()
+    ops.CompactRows(mask, total=total, max_count=most + 7).check_hints()  # an upper bound on the row count is fine
+    ops.CompactRows(mask).check_hints()  # nothing to check without hints
+    for bad_total, bad_most in ((total - 1, most), (total + 1, most), (total, most - 1)):
+        with pytest.raises(ValueError, match="do not fit the mask"):
+            ops.CompactRows(mask, total=bad_total, max_count=bad_most).check_hints()
+    monkeypatch.setenv("BNB_CHECK_HINTS", "1")
+    with pytest.raises(ValueError, match="do not fit the mask"):
+        ops.CompactRows(mask, total=total - 1, max_count=most)
+    ops.CompactRows(mask, total=total, max_count=most)
