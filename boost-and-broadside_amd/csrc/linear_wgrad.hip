@@ -336,7 +336,84 @@ int launch_sum_slices(const float *partials, float *out, int64_t elems, int slic
     return (int)hipGetLastError();
 }
 
+// Column sums of a (R, N) matrix (a bias gradient): a work-group owns a run of consecutive rows, a lane eight
+// consecutive columns of every (256 / (N / 8))-th row of the run; the lanes of a column group are added in lane order
+// through LDS into one partial row per work-group, the partial rows by sum_slices.
+constexpr int kColSumMaxSlices = 1024;
+
+template <typename T>
+__global__ __launch_bounds__(256) void column_sums_kernel(const T *__restrict__ x, int64_t row_stride, float *__restrict__ partials,
+                                                          int64_t R, int N, int64_t rows_per_slice)
+{
+    __shared__ float s_part[256 * 8];
+    const int groups = N >> 3;                    // lanes per row
+    const int lanes_rows = 256 / groups;          // rows in flight per pass
+    const int local_row = threadIdx.x / groups, c0 = (threadIdx.x - local_row * groups) << 3;
+    const int64_t first = (int64_t)blockIdx.x * rows_per_slice;
+    const int64_t last = first + rows_per_slice < R ? first + rows_per_slice : R;
+    float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    if (local_row < lanes_rows) {
+        int64_t r = first + local_row;
+        for (; r + 3 * lanes_rows < last; r += 4 * lanes_rows) {
+            Row8 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = load8_stream(x + (r + (int64_t)u * lanes_rows) * row_stride + c0);
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[e] += v[u].v[e];
+        }
+        for (; r < last; r += lanes_rows) {
+            const Row8 v = load8_stream(x + r * row_stride + c0);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] += v.v[e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s_part[threadIdx.x * 8 + e] = acc[e];
+    __syncthreads();
+    for (int c = threadIdx.x; c < N; c += 256) {
+        const int g = c >> 3, e = c & 7;
+        float t = 0.0f;
+        for (int j = 0; j < lanes_rows; ++j) t += s_part[(j * groups + g) * 8 + e];
+        partials[(int64_t)blockIdx.x * N + c] = t;
+    }
+}
+
 }  // namespace bnb
+
+extern "C" int bnb_column_sums_slices(int64_t R, int N)
+{
+    if (R <= 0 || N < 8) return 1;
+    const int64_t lanes_rows = 256 / (N / 8) > 0 ? 256 / (N / 8) : 1;
+    int64_t s = (R + 16 * lanes_rows - 1) / (16 * lanes_rows);  // at least sixteen passes per work-group
+    if (s > bnb::kColSumMaxSlices) s = bnb::kColSumMaxSlices;
+    return (int)(s < 1 ? 1 : s);
+}
+
+extern "C" int bnb_column_sums(const void *x, int x_dtype, int64_t x_row_stride, float *partials, int slices, float *out,
+                               int accumulate, int64_t R, int N, void *stream)
+{
+    using namespace bnb;
+    if (R < 0 || N < 1 || slices < 1 || slices > kColSumMaxSlices || x_row_stride < N) return BNB_ERR_BAD_SHAPE;
+    if (N % 64 != 0 || N > 2048) return BNB_ERR_UNSUPPORTED;
+    if (x_dtype != BNB_F32 && x_dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
+    if (!out || !partials || (R > 0 && !x)) return BNB_ERR_NULL_POINTER;
+    if ((R > 0 && !aligned16(x)) || !aligned16(partials) || !aligned16(out) || x_row_stride % 8 != 0) return BNB_ERR_MISALIGNED;
+    hipStream_t s = (hipStream_t)stream;
+    if (R == 0) return launch_sum_slices(partials, out, N, 0, accumulate, s);
+    const int64_t rows_per_slice = (R + slices - 1) / slices;
+    const int used = (int)((R + rows_per_slice - 1) / rows_per_slice);  // trailing work-groups without rows are not launched
+    if (x_dtype == BNB_BF16)
+        hipLaunchKernelGGL((column_sums_kernel<uint16_t>), dim3((unsigned)used), dim3(256), 0, s, (const uint16_t *)x, x_row_stride,
+                           partials, R, N, rows_per_slice);
+    else
+        hipLaunchKernelGGL((column_sums_kernel<float>), dim3((unsigned)used), dim3(256), 0, s, (const float *)x, x_row_stride, partials,
+                           R, N, rows_per_slice);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    return launch_sum_slices(partials, out, N, used, accumulate, s);
+}
 
 namespace bnb {
 // BNB_WGRAD_PATH_AUTO picks the direct-to-LDS kernel; the register-staged one stays selectable for comparisons

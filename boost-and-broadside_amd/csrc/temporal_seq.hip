@@ -576,9 +576,9 @@ constexpr int kCbMaxBlocks = 2048;
 template <typename BT>
 __global__ __launch_bounds__(kSeqThreads) void conv_seq_bwd_kernel(
     const BT *__restrict__ b1, const float *__restrict__ conv_in, int64_t conv_in_stride, const float *__restrict__ weight,
-    const uint8_t *__restrict__ done, const float *__restrict__ dv, const float *__restrict__ dconv_out,
-    BT *__restrict__ db1, float *__restrict__ dconv_in, float *__restrict__ partials, int64_t R, int T, int D, int64_t rs,
-    int64_t ts, int chunks, int64_t items)
+    const uint8_t *__restrict__ done, const float *__restrict__ dv, const uint16_t *__restrict__ dv_lp,
+    const float *__restrict__ dconv_out, BT *__restrict__ db1, float *__restrict__ dconv_in, float *__restrict__ partials,
+    int64_t R, int T, int D, int64_t rs, int64_t ts, int chunks, int64_t items)
 {
     __shared__ float s_red[kSeqThreads * 8];
     const int vecs = D >> 3;
@@ -603,9 +603,20 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_bwd_kernel(
         const int64_t row = group * rows_per_block + local_row;
         if (row >= R) continue;
         const float *dvp = dv + row * rs + d0;
+        const uint16_t *dlp = dv_lp == nullptr ? nullptr : dv_lp + row * rs + d0;
         const BT *bp = b1 + row * rs + d0;
         const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
-        auto grad_row = [&](int t) -> Row8 { return t >= 0 && t < T ? load8_split<true>(dvp + t * ts, gap) : zero; };
+        // the output's gradient: the float32 part plus, when the output also went out in bfloat16, that copy's
+        auto grad_row = [&](int t) -> Row8 {
+            if (t < 0 || t >= T) return zero;
+            Row8 g = load8_split<true>(dvp + t * ts, gap);
+            if (dlp != nullptr) {
+                const Row8 l = load8_split<true>(dlp + t * ts, gap);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) g.v[e] += l.v[e];
+            }
+            return g;
+        };
         auto ended = [&](int t) -> bool { return dn != nullptr && t >= 0 && t < T && dn[t] != 0; };
 
         Row8 g0 = grad_row(s0), g1 = grad_row(s0 + 1), g2 = grad_row(s0 + 2);
@@ -678,16 +689,17 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_bwd_kernel(
 
 template <typename BT>
 static int launch_conv_seq_bwd(const void *b1, const float *conv_in, int64_t conv_in_stride, const float *weight,
-                               const uint8_t *done, const float *dv, const float *dconv_out, void *db1, float *dconv_in,
-                               float *partials, int blocks, float *dwb, int64_t R, int T, int D, int time_major,
-                               hipStream_t stream)
+                               const uint8_t *done, const float *dv, const uint16_t *dv_lp, const float *dconv_out, void *db1,
+                               float *dconv_in, float *partials, int blocks, float *dwb, int64_t R, int T, int D,
+                               int time_major, hipStream_t stream)
 {
     const int64_t rs = time_major ? D : (int64_t)T * D, ts = time_major ? R * D : D;
     const int rows_per_block = kSeqThreads / (D / 8);
     const int chunks = (T + (kSeqTaps - 1) + kCbChunk - 1) / kCbChunk;
     const int64_t items = (R + rows_per_block - 1) / rows_per_block * chunks;
     hipLaunchKernelGGL((conv_seq_bwd_kernel<BT>), dim3((unsigned)blocks), dim3(kSeqThreads), 0, stream, (const BT *)b1, conv_in,
-                       conv_in_stride, weight, done, dv, dconv_out, (BT *)db1, dconv_in, partials, R, T, D, rs, ts, chunks, items);
+                       conv_in_stride, weight, done, dv, dv_lp, dconv_out, (BT *)db1, dconv_in, partials, R, T, D, rs, ts, chunks,
+                       items);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
     return launch_sum_slices(partials, dwb, 5 * (int64_t)D, blocks, 0, stream);
@@ -803,9 +815,9 @@ extern "C" int bnb_conv_seq_bwd_blocks(int64_t R, int T, int D)
 }
 
 extern "C" int bnb_conv_seq_bwd(const void *b1, int b1_dtype, const float *conv_in, int64_t conv_in_row_stride,
-                                const float *weight, const uint8_t *done, const float *dv, const float *dconv_out,
-                                void *db1, float *dconv_in, float *partials, int blocks, float *dwb, int64_t R, int T,
-                                int D, int time_major, void *stream)
+                                const float *weight, const uint8_t *done, const float *dv, const void *dv_bf16,
+                                const float *dconv_out, void *db1, float *dconv_in, float *partials, int blocks, float *dwb,
+                                int64_t R, int T, int D, int time_major, void *stream)
 {
     using namespace bnb;
     if (R < 0 || T < 1 || D < 1) return BNB_ERR_BAD_SHAPE;
@@ -815,14 +827,14 @@ extern "C" int bnb_conv_seq_bwd(const void *b1, int b1_dtype, const float *conv_
     if (conv_in_row_stride < 3 * (int64_t)D || blocks < 1 || blocks > kCbMaxBlocks) return BNB_ERR_BAD_SHAPE;
     if (!aligned16(weight) || !aligned16(partials) || !aligned16(dwb) ||
         (R > 0 && (!aligned16(b1) || !aligned16(conv_in) || !aligned16(dv) || !aligned16(db1) || !aligned16(dconv_in) ||
-                   (dconv_out && !aligned16(dconv_out)))) ||
+                   (dconv_out && !aligned16(dconv_out)) || (dv_bf16 && !aligned16(dv_bf16)))) ||
         conv_in_row_stride % 4 != 0)
         return BNB_ERR_MISALIGNED;
     hipStream_t s = (hipStream_t)stream;
     if (R == 0) return launch_sum_slices(partials, dwb, 5 * (int64_t)D, 0, 0, s);
     if (b1_dtype == BNB_BF16)
-        return launch_conv_seq_bwd<uint16_t>(b1, conv_in, conv_in_row_stride, weight, done, dv, dconv_out, db1, dconv_in,
-                                             partials, blocks, dwb, R, T, D, time_major != 0, s);
-    return launch_conv_seq_bwd<float>(b1, conv_in, conv_in_row_stride, weight, done, dv, dconv_out, db1, dconv_in, partials,
-                                      blocks, dwb, R, T, D, time_major != 0, s);
+        return launch_conv_seq_bwd<uint16_t>(b1, conv_in, conv_in_row_stride, weight, done, dv, (const uint16_t *)dv_bf16,
+                                             dconv_out, db1, dconv_in, partials, blocks, dwb, R, T, D, time_major != 0, s);
+    return launch_conv_seq_bwd<float>(b1, conv_in, conv_in_row_stride, weight, done, dv, (const uint16_t *)dv_bf16, dconv_out,
+                                      db1, dconv_in, partials, blocks, dwb, R, T, D, time_major != 0, s);
 }

@@ -755,6 +755,30 @@ def _linear_wgrad_tiled(dy_tiles: torch.Tensor, x_tiles: torch.Tensor, R: int) -
     return out
 
 
+def column_sums_supported(x: torch.Tensor) -> bool:
+    """Whether ``column_sums`` covers this matrix: bfloat16 or float32 rows on the GPU, a width that is a
+    multiple of 64 up to 2048, rows a multiple of 8 elements apart."""
+    return (x.is_cuda and x.dim() == 2 and x.dtype in (torch.bfloat16, torch.float32) and x.shape[1] % 64 == 0
+            and 0 < x.shape[1] <= 2048 and x.stride(1) == 1 and (x.shape[0] <= 1 or x.stride(0) % 8 == 0)
+            and x.data_ptr() % 16 == 0)
+
+
+def column_sums(x: torch.Tensor) -> torch.Tensor:
+    """``x.sum(dim=0, dtype=float32)`` of a (R, N) matrix (a bias gradient) with the rows added in a fixed order."""
+    if not column_sums_supported(x):
+        raise ValueError(f"column_sums does not cover {x.dtype} {tuple(x.shape)} with strides {x.stride()}")
+    R, N = x.shape
+    lib = _native.load()
+    slices = int(lib.bnb_column_sums_slices(R, N))
+    partials = torch.empty((slices, N), dtype=torch.float32, device=x.device)
+    out = torch.empty((N,), dtype=torch.float32, device=x.device)
+    with _on_device(x.device):
+        rc = lib.bnb_column_sums(x.data_ptr(), _DTYPE_CODE[x.dtype], x.stride(0) if R > 1 else N, partials.data_ptr(), slices,
+                                 out.data_ptr(), 0, R, N, _stream())
+    _native.check(rc, "bnb_column_sums")
+    return out
+
+
 class _LinearTrain(torch.autograd.Function):
     """``F.linear`` under bfloat16 autocast whose weight gradient runs on ``linear_wgrad``."""
 
@@ -781,7 +805,8 @@ class _LinearTrain(torch.autograd.Function):
         if ctx.needs_input_grad[1]:
             dw = linear_wgrad(dyb, xb)
         if ctx.has_bias and ctx.needs_input_grad[2]:
-            db = dyb.reshape(-1, dyb.shape[-1]).sum(dim=0, dtype=torch.float32)
+            rows = dyb.reshape(-1, dyb.shape[-1])
+            db = column_sums(rows) if column_sums_supported(rows) else rows.sum(dim=0, dtype=torch.float32)
         return dx, dw, db
 
 
@@ -1211,11 +1236,12 @@ def conv_seq(
 _CONV_TRAIN_WIDTHS = (64, 128, 256, 512)
 
 
-def conv_seq_bwd(b1, conv_buf, weight, done, dv, dconv_out=None, *, time_major: bool = False):
+def conv_seq_bwd(b1, conv_buf, weight, done, dv, dconv_out=None, *, time_major: bool = False, dv_bf16=None):
     """Backward of ``conv_seq``: returns ``(db1, dconv_buf, dweight (D, 4), dbias (D,))``.
 
     ``dv`` is the float32 gradient of the conv output (b1's layout), ``dconv_out`` the optional
-    gradient of the returned stored inputs; ``db1`` has b1's dtype.  Sums run in a fixed order."""
+    gradient of the returned stored inputs, ``dv_bf16`` the optional gradient of the output's bfloat16
+    copy (added to ``dv`` in the kernel); ``db1`` has b1's dtype.  Sums run in a fixed order."""
     R, T, D = b1.shape
     if time_major:
         T, R = R, T
@@ -1227,6 +1253,11 @@ def conv_seq_bwd(b1, conv_buf, weight, done, dv, dconv_out=None, *, time_major: 
         _need_device(t, name)
     b1 = b1.contiguous()
     dv = dv.contiguous()
+    if dv_bf16 is not None:
+        if dv_bf16.shape != b1.shape or dv_bf16.dtype != torch.bfloat16:
+            raise ValueError("dv_bf16 must be bfloat16 with b1's shape")
+        _need_device(dv_bf16, "dv_bf16")
+        dv_bf16 = dv_bf16.contiguous()
     conv_buf = conv_buf if (R == 0 or (conv_buf.stride(2) == 1 and conv_buf.stride(1) == D)) else conv_buf.contiguous()
     weight = weight.detach().reshape(D, 4).contiguous()
     if dconv_out is not None:
@@ -1242,9 +1273,9 @@ def conv_seq_bwd(b1, conv_buf, weight, done, dv, dconv_out=None, *, time_major: 
     keep, done_ptr = _done_pointer(done, R, T, b1.device)
     with _on_device(b1.device):
         rc = lib.bnb_conv_seq_bwd(b1.data_ptr(), _code(b1, "b1"), conv_buf.data_ptr(), conv_buf.stride(0) if R else 3 * D,
-                                  weight.data_ptr(), done_ptr, dv.data_ptr(), None if dconv_out is None else dconv_out.data_ptr(),
-                                  db1.data_ptr(), dconv.data_ptr(), partials.data_ptr(), blocks, dwb.data_ptr(), R, T, D,
-                                  int(time_major), _stream())
+                                  weight.data_ptr(), done_ptr, dv.data_ptr(), None if dv_bf16 is None else dv_bf16.data_ptr(),
+                                  None if dconv_out is None else dconv_out.data_ptr(), db1.data_ptr(), dconv.data_ptr(),
+                                  partials.data_ptr(), blocks, dwb.data_ptr(), R, T, D, int(time_major), _stream())
     _native.check(rc, "bnb_conv_seq_bwd")
     del keep
     return db1, dconv, dwb[:4 * D].view(D, 4), dwb[4 * D:]
@@ -1254,23 +1285,24 @@ class _ConvSeqTrain(torch.autograd.Function):
     """``conv_seq`` with its backward kernel."""
 
     @staticmethod
-    def forward(ctx, b1, conv_buf, weight, bias, done, time_major):
+    def forward(ctx, b1, conv_buf, weight, bias, done, time_major, also_bf16):
         with torch.no_grad():
-            v, new_buf = conv_seq(b1, conv_buf, weight, bias, done, time_major=time_major)
+            res = conv_seq(b1, conv_buf, weight, bias, done, time_major=time_major, also_bf16=also_bf16)
         ctx.save_for_backward(b1, conv_buf, weight)
+        ctx.set_materialize_grads(False)
         ctx.done = done
         ctx.time_major = time_major
         ctx.has_bias = bias is not None
-        return v, new_buf
+        return res[0], res[1], (res[2] if also_bf16 else None)
 
     @staticmethod
     @_outside_autocast
-    def backward(ctx, dv, dbuf):
+    def backward(ctx, dv, dbuf, dv_lp):
         b1, conv_buf, weight = ctx.saved_tensors
         if dv is None:
             dv = torch.zeros(b1.shape, dtype=torch.float32, device=b1.device)
-        db1, dconv, dw, db = conv_seq_bwd(b1, conv_buf, weight, ctx.done, dv, dbuf, time_major=ctx.time_major)
-        return db1, dconv, dw.reshape(weight.shape), db if ctx.has_bias else None, None, None
+        db1, dconv, dw, db = conv_seq_bwd(b1, conv_buf, weight, ctx.done, dv, dbuf, time_major=ctx.time_major, dv_bf16=dv_lp)
+        return db1, dconv, dw.reshape(weight.shape), db if ctx.has_bias else None, None, None, None
 
 
 def conv_seq_train_supported(b1: torch.Tensor) -> bool:
@@ -1278,10 +1310,14 @@ def conv_seq_train_supported(b1: torch.Tensor) -> bool:
     return b1.is_cuda and b1.dim() == 3 and b1.shape[-1] in _CONV_TRAIN_WIDTHS and b1.dtype in (torch.float32, torch.bfloat16)
 
 
-def conv_seq_train(b1, conv_buf, weight, bias, done=None, *, time_major: bool = False):
-    """Differentiable ``conv_seq``: ``(v, new_conv_buf)`` with gradients for b1, conv_buf, weight and bias."""
+def conv_seq_train(b1, conv_buf, weight, bias, done=None, *, time_major: bool = False, also_bf16: bool = False):
+    """Differentiable ``conv_seq``: ``(v, new_conv_buf)`` with gradients for b1, conv_buf, weight and bias.
+
+    ``also_bf16``: a third result, the bfloat16 rounding of ``v`` written by the same launch (what a bfloat16
+    projection of ``v`` would cast for itself); its gradient is added to ``v``'s inside the backward kernel."""
     with torch.autocast("cuda", enabled=False):
-        return _ConvSeqTrain.apply(b1, conv_buf, weight, bias, done, time_major)
+        v, new_buf, v_lp = _ConvSeqTrain.apply(b1, conv_buf, weight, bias, done, time_major, also_bf16)
+    return (v, new_buf, v_lp) if also_bf16 else (v, new_buf)
 
 
 def rglru_scan(
@@ -1366,6 +1402,7 @@ class _RglruScan(torch.autograd.Function):
         with torch.no_grad():
             y, h_last = rglru_scan(x, gates_pre, log_lambda, c, h0, done, time_major=time_major)
         ctx.save_for_backward(x, gates_pre, log_lambda, h0, y)
+        ctx.set_materialize_grads(False)
         ctx.done, ctx.c, ctx.time_major = done, c, time_major
         return y, h_last
 
@@ -1377,8 +1414,9 @@ class _RglruScan(torch.autograd.Function):
         D = x.shape[2]
         x_c, g_c = x.contiguous(), gates_pre.contiguous()
         h0_c = h0 if h0.stride(1) == 1 else h0.contiguous()
-        dy = dy.to(y.dtype).contiguous()          # the kernel reads dy in y's dtype and dh_last as float32
-        dh_last = dh_last.float().contiguous()
+        # the kernel reads dy in y's dtype and dh_last as float32; an output nobody differentiated arrives as None
+        dy = torch.zeros_like(y) if dy is None else dy.to(y.dtype).contiguous()
+        dh_last = torch.zeros((R, D), dtype=torch.float32, device=x.device) if dh_last is None else dh_last.float().contiguous()
         dx = torch.empty_like(x_c)
         dgates = torch.empty_like(g_c)
         dh0 = torch.empty((R, D), dtype=torch.float32, device=x.device)
@@ -1527,6 +1565,7 @@ class _RmsNormTrain(torch.autograd.Function):
         with torch.no_grad():
             n = add_rmsnorm(x, weight, eps=eps, out_dtype=out_dtype)[1]
         ctx.save_for_backward(x, weight)
+        ctx.set_materialize_grads(False)
         ctx.eps = eps
         return x.view_as(x), n
 
@@ -1549,6 +1588,7 @@ class _AddRmsNormTrain(torch.autograd.Function):
         with torch.no_grad():
             s, n = add_rmsnorm(x, weight, delta=delta, eps=eps, out_dtype=out_dtype)
         ctx.save_for_backward(s, weight)
+        ctx.set_materialize_grads(False)
         ctx.eps = eps
         ctx.delta_dtype = delta.dtype
         return s, n
@@ -1590,6 +1630,7 @@ class _NormLinearTrain(torch.autograd.Function):
                     float(_F32_EPS if eps is None else eps), packed.data_ptr(), y.data_ptr(), n.data_ptr(), R, D, N, _stream())
             _native.check(rc, "bnb_norm_linear_train_fwd")
         ctx.save_for_backward(x, norm_weight, weight, n)
+        ctx.set_materialize_grads(False)
         ctx.eps = eps
         n_out = n.view(x.shape)
         return x.view_as(x), y.view(*x.shape[:-1], N), n_out
@@ -1601,17 +1642,23 @@ class _NormLinearTrain(torch.autograd.Function):
         D = x.shape[-1]
         dn = None
         d_weight = None
+        if dn_other is not None:
+            dn_other = dn_other.reshape(-1, D)
         if dy is not None:
             dy2 = dy.reshape(-1, dy.shape[-1])
             dyb = dy2 if dy2.dtype == torch.bfloat16 else dy2.to(torch.bfloat16)
             if dyb.stride(-1) != 1:
                 dyb = dyb.contiguous()
-            dn = torch.matmul(dyb, weight.detach().to(torch.bfloat16))
+            wb = weight.detach().to(torch.bfloat16)
+            if dn_other is None:
+                dn = torch.matmul(dyb, wb)
+            else:
+                # one rounding of (dy W + the other users' gradient) in the GEMM's epilogue instead of a second pass
+                dn = torch.addmm(dn_other.to(torch.bfloat16), dyb, wb)
             if ctx.needs_input_grad[2]:
                 d_weight = linear_wgrad(dyb, n)
-        if dn_other is not None:
-            dn_other = dn_other.reshape(-1, D)
-            dn = dn_other if dn is None else dn + dn_other.to(dn.dtype)
+        elif dn_other is not None:
+            dn = dn_other
         if dn is None:
             dn = torch.zeros_like(n)
         dx, d_norm = rmsnorm_bwd(x, dn.view(x.shape), norm_weight, eps=ctx.eps, grad_sum=ds)

@@ -807,6 +807,8 @@ class RGLRU(_WeightCaches, nn.Module):
             # the (small) weights are concatenated, not the activations: one cast of x, one GEMM, one weight gradient
             w = torch.cat([self.linear_a.weight, self.linear_x.weight], dim=0)
             b = torch.cat([self.linear_a.bias, self.linear_x.bias], dim=0)
+            if x_act is not None and x_act.dtype == _projection_dtype():
+                x = x_act  # the producer's own copy in the projection dtype: no cast here, no cast back in the backward
             return _grad_linear(x, w, b)
         act = _projection_dtype()
         wa, wx, ba, bx = self.linear_a.weight, self.linear_x.weight, self.linear_a.bias, self.linear_x.bias
@@ -905,9 +907,12 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
         if (_TRAIN_KERNELS and ops.conv_seq_train_supported(b1) and conv_buf.dtype == torch.float32
                 and self.conv.weight.dtype == torch.float32):
             # conv forward and backward on their kernels (one pass each instead of a dozen element-wise ops per tap)
-            v, new_buf = ops.conv_seq_train(b1, conv_buf, self.conv.weight, self.conv.bias, done_mask, time_major=time_major)
-            y, new_h = self.rg_lru.forward_sequence(v, h0, done_mask, time_major=time_major)
-            return self._finish(x_seq, normed, y), new_h, new_buf
+            want_lp = _projection_dtype() == torch.bfloat16
+            res = ops.conv_seq_train(b1, conv_buf, self.conv.weight, self.conv.bias, done_mask, time_major=time_major,
+                                     also_bf16=want_lp)
+            y, new_h = self.rg_lru.forward_sequence(res[0], h0, done_mask, time_major=time_major,
+                                                    x_act=res[2] if want_lp else None)
+            return self._finish(x_seq, normed, y), new_h, res[1]
         rows_first = b1.transpose(0, 1) if time_major else b1  # (R, T, D) view
         T = rows_first.shape[1]
         padded = torch.cat([conv_buf, rows_first], dim=1)  # fp32 buffer promotes a bf16 b1
@@ -943,8 +948,10 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
         ships_b1 = ships_b1.reshape(T, B * n_rec, D)
         if not ops.conv_seq_train_supported(ships_b1):
             return None
-        v, new_buf = ops.conv_seq_train(ships_b1, conv_buf, self.conv.weight, self.conv.bias, done_rows, time_major=True)
-        y_ships, new_h = self.rg_lru.forward_sequence(v, h0, done_rows, time_major=True)
+        # the conv launch also writes its output in bfloat16 for the gate projections (the backward kernel adds the two gradients)
+        v, new_buf, v_lp = ops.conv_seq_train(ships_b1, conv_buf, self.conv.weight, self.conv.bias, done_rows, time_major=True,
+                                              also_bf16=True)
+        y_ships, new_h = self.rg_lru.forward_sequence(v, h0, done_rows, time_major=True, x_act=v_lp)
         y_fields = _project(field_sub, fields_b1)
         # the recurrence's output is float32 (the conv buffer promotes its input, griffin.py:275); the field rows'
         # bfloat16 values are exact in it, and the gate kernel rounds the product once either way
@@ -1260,6 +1267,7 @@ class _SplitTokens(torch.autograd.Function):
     def forward(ctx, x, n):
         ctx.n = n
         ctx.shape = x.shape
+        ctx.set_materialize_grads(False)
         return x[:, :, :n].contiguous(), x[:, :, n:].contiguous()
 
     @staticmethod

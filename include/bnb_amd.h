@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 26
+#define BNB_ABI_VERSION 27
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -300,6 +300,24 @@ int bnb_linear_wgrad_tiled_fwd(const void *dy, int64_t dy_row_stride, int64_t dy
                                int accumulate, int64_t R, int N, int K, void *stream);
 
 /*
+ * Bias gradient of a Linear layer:  out[n] (+)= sum_r x[r][n], fp32 sums of bf16 or fp32 rows.
+ *
+ * Replaces what autograd computes for `bias.grad` of the RG-LRU's two gate projections
+ * (models/yemong/griffin.py:165-167) in the PPO update (train/rl/ppo.py:1417-1425): a column sum over
+ * several hundred thousand rows of the (R, 256) gate gradient.
+ *
+ *   x        (R, N) bf16 or fp32 (x_dtype), rows x_row_stride elements apart
+ *   partials (slices, N) fp32 workspace owned by the caller; slices from bnb_column_sums_slices(R, N)
+ *   out      (N) fp32: overwritten, or added to when accumulate != 0
+ *
+ * Each work-group adds a run of consecutive rows, a second kernel the work-groups' rows, both in a fixed order.
+ * Requirements: N % 64 == 0, N <= 2048, 16-byte aligned pointers, x_row_stride a multiple of 8.
+ */
+int bnb_column_sums_slices(int64_t R, int N);
+int bnb_column_sums(const void *x, int x_dtype, int64_t x_row_stride, float *partials, int slices, float *out,
+                    int accumulate, int64_t R, int N, void *stream);
+
+/*
  * Backward of bnb_sdpa_masked_fwd for small token counts: what autograd computes through
  * models/yemong/attention.py:136-147 (head split, key bias on dead entities, SDPA, head merge)
  * in the PPO update (train/rl/ppo.py:1417-1425).
@@ -564,6 +582,7 @@ int bnb_conv_seq_fwd(const void *b1, int b1_dtype,
  *
  *   b1, conv_in, weight, done, time_major  as passed to the forward
  *   dv         gradient of v_out, fp32, b1's layout
+ *   dv_bf16    gradient of v_bf16_out (bf16, b1's layout), added to dv element by element, or NULL
  *   dconv_out  gradient of conv_out, (R, 3, D) fp32 contiguous, or NULL
  *   db1        gradient of b1, b1's dtype and layout
  *   dconv_in   gradient of conv_in, (R, 3, D) fp32 contiguous
@@ -574,8 +593,8 @@ int bnb_conv_seq_fwd(const void *b1, int b1_dtype,
  */
 int bnb_conv_seq_bwd_blocks(int64_t R, int T, int D);
 int bnb_conv_seq_bwd(const void *b1, int b1_dtype, const float *conv_in, int64_t conv_in_row_stride,
-                     const float *weight, const uint8_t *done, const float *dv, const float *dconv_out,
-                     void *db1, float *dconv_in, float *partials, int blocks, float *dwb,
+                     const float *weight, const uint8_t *done, const float *dv, const void *dv_bf16,
+                     const float *dconv_out, void *db1, float *dconv_in, float *partials, int blocks, float *dwb,
                      int64_t R, int T, int D, int time_major, void *stream);
 
 /*

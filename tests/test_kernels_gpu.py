@@ -1922,6 +1922,49 @@ def test_linear_train_gradients_match_autograd_of_the_same_bf16_linear(with_bias
         assert max_rel(b.grad.cpu().double(), bd.grad) <= F32_TOL
 
 
+@pytest.mark.parametrize("R,N", [(1, 64), (7, 256), (300, 384), (9001, 256), (70000, 128), (513, 2048), (0, 256)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_column_sums_match_the_float64_sums_and_repeat_exactly(R, N, dtype):
+    g = torch.Generator().manual_seed(R + N)
+    x = (torch.randn(R, N, generator=g) + 0.25).to(dtype)
+    xd = x.to(DEV)
+    got = ops.column_sums(xd)
+    torch.cuda.synchronize()
+    assert got.dtype == torch.float32 and got.shape == (N,)
+    want = x.double().sum(dim=0)
+    scale = max(float(x.double().abs().sum(dim=0).max()), 1.0)  # float32 sums of R terms: error against the terms' size
+    assert float((got.cpu().double() - want).abs().max()) / scale <= F32_TOL
+    assert torch.equal(got, ops.column_sums(xd))
+    # rows further apart than their width (a column slice of a wider matrix)
+    if R:
+        wide = torch.zeros(R, N + 64, dtype=dtype, device=DEV)
+        wide[:, :N] = xd
+        assert torch.equal(ops.column_sums(wide[:, :N]), got)
+
+
+def test_column_sums_find_a_single_entry_in_its_column_and_refuse_other_shapes():
+    x = torch.zeros(5000, 256, dtype=torch.bfloat16, device=DEV)
+    x[4321, 77] = 3.0
+    x[0, 255] = -2.0
+    got = ops.column_sums(x).cpu()
+    want = torch.zeros(256)
+    want[77], want[255] = 3.0, -2.0
+    assert torch.equal(got, want)
+    for bad in (torch.zeros(10, 100, device=DEV), torch.zeros(10, 4096, device=DEV), torch.zeros(10, 128, device=DEV).half(),
+                torch.zeros(10, 128, 2, device=DEV)):
+        assert not ops.column_sums_supported(bad)
+        with pytest.raises(ValueError):
+            ops.column_sums(bad)
+    from boost_and_broadside_amd import _native
+
+    lib = _native.load()
+    out = torch.zeros(256, device=DEV)
+    part = torch.zeros(4, 256, device=DEV)
+    assert lib.bnb_column_sums(None, _native.BF16, 256, part.data_ptr(), 4, out.data_ptr(), 0, 10, 256, None) == 10001
+    assert lib.bnb_column_sums(x.data_ptr(), _native.BF16, 256, part.data_ptr(), 4, out.data_ptr(), 0, 10, 100, None) != 0
+    assert lib.bnb_column_sums(x.data_ptr(), _native.BF16, 100, part.data_ptr(), 4, out.data_ptr(), 0, 10, 256, None) == 10003
+
+
 # ------------------------------------------------------------------ RMSNorm backward
 
 
@@ -2084,6 +2127,57 @@ def test_conv_seq_train_is_differentiable_and_equals_the_forward_kernel():
     assert max_rel(buf.grad.cpu().double(), want[1]) <= F32_TOL
     assert max_rel(w.grad.cpu().double(), want[2]) <= F32_TOL
     assert max_rel(bias.grad.cpu().double(), want[3]) <= F32_TOL
+
+
+@pytest.mark.parametrize("R,T,time_major", [(40, 24, True), (9, 35, False), (2100, 29, True)])
+def test_conv_seq_bwd_adds_the_gradient_of_the_bfloat16_copy_in_the_same_pass(R, T, time_major):
+    D = 128
+    g = torch.Generator().manual_seed(R + T)
+    shape = (T, R, D) if time_major else (R, T, D)
+    b1 = torch.randn(shape, generator=g).bfloat16().to(DEV)
+    buf = torch.randn(R, 3, D, generator=g).to(DEV)
+    w = (0.5 * torch.randn(D, 1, 4, generator=g)).to(DEV)
+    done = (torch.rand(R, T, generator=g) < 0.2).to(DEV)
+    dv = torch.randn(shape, generator=g).to(DEV)
+    dv_lp = torch.randn(shape, generator=g).bfloat16().to(DEV)
+    got = ops.conv_seq_bwd(b1, buf, w, done, dv, None, time_major=time_major, dv_bf16=dv_lp)
+    want = ops.conv_seq_bwd(b1, buf, w, done, dv + dv_lp.float(), None, time_major=time_major)
+    assert all(torch.equal(a, b) for a, b in zip(got, want))  # the same float32 addition, inside the kernel
+    with pytest.raises(ValueError):
+        ops.conv_seq_bwd(b1, buf, w, done, dv, None, time_major=time_major, dv_bf16=dv_lp.float())
+
+
+def test_conv_seq_train_hands_out_a_bfloat16_copy_whose_gradient_reaches_the_input():
+    R, T, D = 40, 24, 128
+    g = torch.Generator().manual_seed(22)
+    b1 = torch.randn(T, R, D, generator=g).bfloat16().to(DEV).requires_grad_()
+    buf = torch.randn(R, 3, D, generator=g).to(DEV).requires_grad_()
+    w = (0.5 * torch.randn(D, 1, 4, generator=g)).to(DEV).requires_grad_()
+    bias = (0.1 * torch.randn(D, generator=g)).to(DEV).requires_grad_()
+    done = (torch.rand(R, T, generator=g) < 0.2).to(DEV)
+    up_v = torch.randn(T, R, D, generator=g).to(DEV)
+    up_lp = torch.randn(T, R, D, generator=g).bfloat16().to(DEV)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        v, tail, v_lp = ops.conv_seq_train(b1, buf, w, bias, done, time_major=True, also_bf16=True)
+    assert v_lp.dtype == torch.bfloat16 and torch.equal(v_lp, v.detach().bfloat16())
+    ((v * up_v).sum() + (v_lp.float() * up_lp.float()).sum()).backward()
+    got = [t.grad.clone() for t in (b1, buf, w, bias)]
+    for t in (b1, buf, w, bias):
+        t.grad = None
+    # the same loss with the copy made by autograd's own cast
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        v2, _ = ops.conv_seq_train(b1, buf, w, bias, done, time_major=True)
+    ((v2 * up_v).sum() + (v2.bfloat16().float() * up_lp.float()).sum()).backward()
+    for a, t in zip(got, (b1, buf, w, bias)):
+        assert torch.equal(a, t.grad)
+    # only the copy used: the float32 output's gradient is absent, not a tensor of zeros
+    for t in (b1, buf, w, bias):
+        t.grad = None
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        _, _, v_lp3 = ops.conv_seq_train(b1, buf, w, bias, done, time_major=True, also_bf16=True)
+    (v_lp3.float() * up_lp.float()).sum().backward()
+    want = ops.conv_seq_bwd(b1.detach(), buf.detach(), w.detach(), done, up_lp.float(), None, time_major=True)
+    assert torch.equal(b1.grad, want[0]) and torch.equal(buf.grad, want[1])
 
 
 # ------------------------------------------------------------------ gelu(a) * b backward
