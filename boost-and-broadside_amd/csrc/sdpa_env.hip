@@ -203,12 +203,16 @@ __global__ __launch_bounds__(kWave * NQB, 4) void sdpa_env_kernel(const uint16_t
     // ---- state of the environment being computed ----
     int nkb, pad;
     bool uniform;
-    f32x16 bias0;  // -inf for the padding positions of key block 0, as the initial accumulator there
     auto set_padding = [&](int cnt) {
         nkb = (cnt + 31) >> 5;
         pad = nkb * 32 - cnt;
+    };
+    // -inf for the padding positions of key block 0, as the initial accumulator there (made where it is used)
+    auto pad_bias = [&](int pad_rows) -> f32x16 {
+        f32x16 b;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) bias0[v] = (8 * (v >> 2) + 4 * half + (v & 3) < pad) ? -INFINITY : 0.0f;
+        for (int v = 0; v < 16; ++v) b[v] = (8 * (v >> 2) + 4 * half + (v & 3) < pad_rows) ? -INFINITY : 0.0f;
+        return b;
     };
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
 
@@ -219,43 +223,58 @@ __global__ __launch_bounds__(kWave * NQB, 4) void sdpa_env_kernel(const uint16_t
         // with no live key every score is the same constant: zero queries give exactly that
         const bf16x8 qb0 = __builtin_bit_cast(bf16x8, uniform ? zero4 : qw[h][0]);
         const bf16x8 qb1 = __builtin_bit_cast(bf16x8, uniform ? zero4 : qw[h][1]);
-        auto scores = [&](int kb) -> f32x16 {
+        auto scores = [&](int kb, int pad_rows) -> f32x16 {
             const uint16_t *kp = buf + kb * 32 * (kEnvKeyBytes / 2);
             const bf16x8 ka0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + k_off0));
             const bf16x8 ka1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + k_off1));
             f32x16 z = {0.0f};
-            if (kb == 0) z = bias0;
+            if (kb == 0) z = pad_bias(pad_rows);
             z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0, qb0, z, 0, 0, 0);
             return __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka1, qb1, z, 0, 0, 0);
         };
-        float mx = -INFINITY;
-        for (int kb = 0; kb < nkb; ++kb) {
-            const f32x16 z = scores(kb);
-#pragma unroll
-            for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float mc = mx * scale_log2e;
+        // weights without a shift first (one sweep), with the maximum as shift when a query's sum leaves the safe
+        // exponent range: the same arithmetic as sdpa_mfma_kernel, whose results this kernel repeats bit for bit
+        const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
         float sum = 0.0f;
         f32x16 o = {0.0f};
-        for (int kb = 0; kb < nkb; ++kb) {
-            const f32x16 z = scores(kb);
-            float p[16];
+        auto sweep = [&](auto shifted, float mc, int pad_rows) {
+            sum = 0.0f;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                p[v] = __builtin_amdgcn_exp2f(fmaf(z[v], scale_log2e, -mc));
-                sum += p[v];
+            for (int v = 0; v < 16; ++v) o[v] = 0.0f;
+            for (int kb = 0; kb < nkb; ++kb) {
+                const f32x16 z = scores(kb, pad_rows);
+                float p[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    if constexpr (decltype(shifted)::value) p[v] = __builtin_amdgcn_exp2f(fmaf(z[v], scale_log2e, -mc));
+                    else p[v] = __builtin_amdgcn_exp2f(z[v] * scale_log2e);
+                }
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    bf16x8 pb;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * t + e];
+#pragma unroll
+                    for (int e = 0; e < 8; e += 2) sum = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{pb[e], pb[e + 1]}, ones, sum, false);
+                    const bf16x8 va = lds_tr_pair(buf + (kb * 32 + 16 * t) * (kEnvKeyBytes / 2) + v_off);
+                    o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb, o, 0, 0, 0);
+                }
             }
+            sum += __shfl_xor(sum, 32);
+        };
+        sweep(std::false_type{}, 0.0f, pad);
+        if (!__all(sum >= 0x1p-60f && sum <= 0x1p60f)) {
+            int pad_again = pad;
+            asm volatile("" : "+v"(pad_again));  // a value of its own: nothing of the first try is kept for this one
+            float mx = -INFINITY;
+            for (int kb = 0; kb < nkb; ++kb) {
+                const f32x16 z = scores(kb, pad_again);
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                bf16x8 pb;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * t + e];
-                const bf16x8 va = lds_tr_pair(buf + (kb * 32 + 16 * t) * (kEnvKeyBytes / 2) + v_off);
-                o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb, o, 0, 0, 0);
+                for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
             }
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            sweep(std::true_type{}, mx * scale_log2e, pad_again);
         }
-        sum += __shfl_xor(sum, 32);
         const float inv = __builtin_amdgcn_rcpf(sum);
 #pragma unroll
         for (int g = 0; g < 2; ++g)
@@ -452,50 +471,68 @@ __global__ __launch_bounds__(kWave * NQB, 8) void sdpa_head_kernel(const uint16_
     if (uniform) qw0 = qw1 = u32x4{0u, 0u, 0u, 0u};
     const bf16x8 qb0 = __builtin_bit_cast(bf16x8, qw0);
     const bf16x8 qb1 = __builtin_bit_cast(bf16x8, qw1);
-    f32x16 bias0;
+    auto pad_bias = [&](int pad_rows) -> f32x16 {
+        f32x16 b;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) bias0[v] = (8 * (v >> 2) + 4 * half + (v & 3) < pad) ? -INFINITY : 0.0f;
+        for (int v = 0; v < 16; ++v) b[v] = (8 * (v >> 2) + 4 * half + (v & 3) < pad_rows) ? -INFINITY : 0.0f;
+        return b;
+    };
 
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's rows and its queries
     __syncthreads();                      // everybody's rows
 
-    auto scores = [&](int kb) -> f32x16 {
+    auto scores = [&](int kb, int pad_rows) -> f32x16 {
         const uint16_t *kp = s_buf + kb * 32 * (kEnvKeyBytes / 2);
         const bf16x8 ka0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + k_off0));
         const bf16x8 ka1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + k_off1));
         f32x16 z = {0.0f};
-        if (kb == 0) z = bias0;
+        if (kb == 0) z = pad_bias(pad_rows);
         z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0, qb0, z, 0, 0, 0);
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka1, qb1, z, 0, 0, 0);
     };
-    float mx = -INFINITY;
-    for (int kb = 0; kb < nkb; ++kb) {
-        const f32x16 z = scores(kb);
-#pragma unroll
-        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float mc = mx * scale_log2e;
+    // weights without a shift first (one sweep), with the maximum as shift when a query's sum leaves the safe
+    // exponent range: the same arithmetic as sdpa_mfma_kernel, whose results this kernel repeats bit for bit
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
     float sum = 0.0f;
     f32x16 o = {0.0f};
-    for (int kb = 0; kb < nkb; ++kb) {
-        const f32x16 z = scores(kb);
-        float p[16];
+    auto sweep = [&](auto shifted, float mc, int pad_rows) {
+        sum = 0.0f;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            p[v] = __builtin_amdgcn_exp2f(fmaf(z[v], scale_log2e, -mc));
-            sum += p[v];
+        for (int v = 0; v < 16; ++v) o[v] = 0.0f;
+        for (int kb = 0; kb < nkb; ++kb) {
+            const f32x16 z = scores(kb, pad_rows);
+            float p[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                if constexpr (decltype(shifted)::value) p[v] = __builtin_amdgcn_exp2f(fmaf(z[v], scale_log2e, -mc));
+                else p[v] = __builtin_amdgcn_exp2f(z[v] * scale_log2e);
+            }
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                bf16x8 pb;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * t + e];
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) sum = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{pb[e], pb[e + 1]}, ones, sum, false);
+                const bf16x8 va = lds_tr_pair(s_buf + (kb * 32 + 16 * t) * (kEnvKeyBytes / 2) + v_off);
+                o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb, o, 0, 0, 0);
+            }
         }
+        sum += __shfl_xor(sum, 32);
+    };
+    sweep(std::false_type{}, 0.0f, pad);
+    if (!__all(sum >= 0x1p-60f && sum <= 0x1p60f)) {
+        int pad_again = pad;
+        asm volatile("" : "+v"(pad_again));  // a value of its own: nothing of the first try is kept for this one
+        float mx = -INFINITY;
+        for (int kb = 0; kb < nkb; ++kb) {
+            const f32x16 z = scores(kb, pad_again);
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            bf16x8 pb;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * t + e];
-            const bf16x8 va = lds_tr_pair(s_buf + (kb * 32 + 16 * t) * (kEnvKeyBytes / 2) + v_off);
-            o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb, o, 0, 0, 0);
+            for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
         }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        sweep(std::true_type{}, mx * scale_log2e, pad_again);
     }
-    sum += __shfl_xor(sum, 32);
     const float inv = __builtin_amdgcn_rcpf(sum);
     if (qrow < NM) {
         uint16_t *op = out + ((int64_t)env * NM + qrow) * D + head * kEnvDh + 8 * half;

@@ -21,6 +21,8 @@
 //                      v_mfma_f32_32x32x16_bf16 so that the softmax reductions over keys
 //                      stay inside a lane.
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace bnb {
@@ -207,7 +209,7 @@ constexpr int kKeyPitch = kDh + 8;  // halfs per K row in LDS: 80 bytes, 16-byte
 // instead of letting the uniform average through), and the result is added to `accum`.
 // NKB = key blocks and waves of the work-group: max(ceil(NK/32), ceil(NQ/32)).
 template <int NKB, bool CROSS>
-__global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
+__global__ __launch_bounds__(kWave * NKB) __attribute__((amdgpu_waves_per_eu(8, 8))) void sdpa_mfma_kernel(
     const uint16_t *__restrict__ q, int64_t q_stride, const uint16_t *__restrict__ k,
     const uint16_t *__restrict__ v, int64_t kv_stride, const uint8_t *__restrict__ alive,
     const uint16_t *accum, uint16_t *out, int B, int NQ, int NK, int H, float scale_log2e)
@@ -339,57 +341,77 @@ __global__ __launch_bounds__(kWave * NKB) void sdpa_mfma_kernel(
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
     const bf16x8 qb0 = __builtin_bit_cast(bf16x8, uniform ? zero4 : qw0);
     const bf16x8 qb1 = __builtin_bit_cast(bf16x8, uniform ? zero4 : qw1);
-    // Padding is confined to key block 0, where it enters as the initial accumulator.
-    f32x16 bias0;
+    // Padding is confined to key block 0, where it enters as the initial accumulator (made where it is used: sixteen
+    // registers that would otherwise stay occupied from here to the rarely taken second try).
+    auto pad_bias = [&](int pad_rows) -> f32x16 {
+        f32x16 b;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) bias0[v] = (8 * (v >> 2) + 4 * half + (v & 3) < pad) ? -INFINITY : 0.0f;
+        for (int v = 0; v < 16; ++v) b[v] = (8 * (v >> 2) + 4 * half + (v & 3) < pad_rows) ? -INFINITY : 0.0f;
+        return b;
+    };
 
-    // Two sweeps over the key blocks instead of keeping all NKB*16 scores per lane: the
-    // matrix cores idle most of the time, registers are what limits the work-groups in
-    // flight, and a second K Q^T costs less than the occupancy the scores would take.
-    auto scores = [&](int kb) -> f32x16 {
+    auto scores = [&](int kb, int pad_rows) -> f32x16 {
         const uint16_t *kp = s_k + (kb * 32 + m) * kKeyPitch + half * 8;
         const bf16x8 ka0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp));
         const bf16x8 ka1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + 16));
         f32x16 z = {0.0f};
-        if (kb == 0) z = bias0;
+        if (kb == 0) z = pad_bias(pad_rows);
         z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0, qb0, z, 0, 0, 0);
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka1, qb1, z, 0, 0, 0);
     };
 
-    float mx = -INFINITY;
-    for (int kb = 0; kb < nkb; ++kb) {
-        const f32x16 z = scores(kb);
-#pragma unroll
-        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float mc = mx * scale_log2e;
-
-    // ---- P = exp2(scale (S - max)), O^T = V^T P^T ----
+    // ---- P = exp2(scale S - shift), O^T = V^T P^T ----
+    // Softmax does not depend on the shift, only the exponent range does.  First try: no shift at all, one sweep
+    // (no K Q^T just to find the maximum).  That is exact to rounding whenever the sum of a query's weights stays
+    // well inside the float32 range; a wave with a query whose sum does not (scores beyond +-60 in log2 units, or not
+    // finite) throws the try away and takes the two sweeps with the true maximum as shift.
     float sum = 0.0f;
     f32x16 o = {0.0f};
-    for (int kb = 0; kb < nkb; ++kb) {
-        const f32x16 z = scores(kb);
-        float p[16];
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    auto sweep = [&](auto shifted, float mc, int pad_rows) {
+        sum = 0.0f;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            p[v] = __builtin_amdgcn_exp2f(fmaf(z[v], scale_log2e, -mc));
-            sum += p[v];
+        for (int v = 0; v < 16; ++v) o[v] = 0.0f;
+        for (int kb = 0; kb < nkb; ++kb) {
+            const f32x16 z = scores(kb, pad_rows);
+            float p[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                if constexpr (decltype(shifted)::value) p[v] = __builtin_amdgcn_exp2f(fmaf(z[v], scale_log2e, -mc));
+                else p[v] = __builtin_amdgcn_exp2f(z[v] * scale_log2e);
+            }
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                bf16x8 pb;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * t + e];
+                // the normaliser adds the weights as the matrix product sees them (rounded to bfloat16), a pair per
+                // instruction: a query with one live key then gets that key's value row back exactly
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) sum = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{pb[e], pb[e + 1]}, ones, sum, false);
+                const uint16_t *vp = s_vt + m * VP + kb * 32 + 16 * t + 4 * half;
+                const u32x2 lo = *reinterpret_cast<const u32x2 *>(vp);
+                const u32x2 hi = *reinterpret_cast<const u32x2 *>(vp + 8);
+                const u32x4 vw = {lo.x, lo.y, hi.x, hi.y};
+                o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vw), pb, o, 0, 0, 0);
+            }
         }
+        sum += __shfl_xor(sum, 32);
+    };
+    sweep(std::false_type{}, 0.0f, pad);
+    const bool in_range = (sum >= 0x1p-60f && sum <= 0x1p60f) || (CROSS && cnt == 0);  // false for NaN
+    if (!__all(in_range)) {
+        int pad_again = pad;
+        asm volatile("" : "+v"(pad_again));  // a value of its own: nothing of the first try is kept for this one
+        float mx = -INFINITY;
+        for (int kb = 0; kb < nkb; ++kb) {
+            const f32x16 z = scores(kb, pad_again);
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            bf16x8 pb;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * t + e];
-            const uint16_t *vp = s_vt + m * VP + kb * 32 + 16 * t + 4 * half;
-            const u32x2 lo = *reinterpret_cast<const u32x2 *>(vp);
-            const u32x2 hi = *reinterpret_cast<const u32x2 *>(vp + 8);
-            const u32x4 vw = {lo.x, lo.y, hi.x, hi.y};
-            o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vw), pb, o, 0, 0, 0);
+            for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
         }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        sweep(std::true_type{}, mx * scale_log2e, pad_again);
     }
-    sum += __shfl_xor(sum, 32);
     // CROSS with no live key: nkb == 0, o == 0 and the contribution is exactly zero
     const float inv = (CROSS && cnt == 0) ? 0.0f : __builtin_amdgcn_rcpf(sum);
 
@@ -534,31 +556,45 @@ __global__ __launch_bounds__(kWave) void sdpa_mfma_pair_kernel(
         z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0, __builtin_bit_cast(bf16x8, qw0), z, 0, 0, 0);
         z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka1, __builtin_bit_cast(bf16x8, qw1), z, 0, 0, 0);
     }
-    float mx = -INFINITY;
+    // weights without a shift first, with the maximum as shift when a query's sum leaves the safe exponent range
+    // (see sdpa_mfma_kernel); the scores stay in registers here, so the second try costs no matrix product
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    float sum;
+    bf16x8 pb[2];
+    auto weights = [&](auto shifted, float mc) {
+        sum = 0.0f;
+        float p[16];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float mc = mx * scale_log2e;
-    float sum = 0.0f;
-    float p[16];
+        for (int v = 0; v < 16; ++v) {
+            if constexpr (decltype(shifted)::value) p[v] = __builtin_amdgcn_exp2f(fmaf(z[v], scale_log2e, -mc));
+            else p[v] = __builtin_amdgcn_exp2f(z[v] * scale_log2e);
+        }
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        p[v] = __builtin_amdgcn_exp2f(fmaf(z[v], scale_log2e, -mc));
-        sum += p[v];
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pb[t][e] = (__bf16)p[8 * t + e];
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) sum = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{pb[t][e], pb[t][e + 1]}, ones, sum, false);
+        }
+        sum += __shfl_xor(sum, 32);
+    };
+    weights(std::false_type{}, 0.0f);
+    if (!__all(sum >= 0x1p-60f && sum <= 0x1p60f)) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, z[v]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        weights(std::true_type{}, mx * scale_log2e);
     }
     f32x16 o = {0.0f};
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-        bf16x8 pb;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * t + e];
         const uint16_t *vp = s_vt + m * VP + 16 * t + 4 * half;
         const u32x2 lo = *reinterpret_cast<const u32x2 *>(vp);
         const u32x2 hi = *reinterpret_cast<const u32x2 *>(vp + 8);
         const u32x4 vq = {lo.x, lo.y, hi.x, hi.y};
-        o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vq), pb, o, 0, 0, 0);
+        o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vq), pb[t], o, 0, 0, 0);
     }
-    sum += __shfl_xor(sum, 32);
     const float inv = __builtin_amdgcn_rcpf(sum);
     // Lanes m and m + 16 hold the same token of the pair's two heads.  They trade runs as in
     // sdpa_mfma_kernel, so that one store instruction writes the whole 64-byte row of the first
@@ -778,7 +814,7 @@ __global__ __launch_bounds__(1024) void sdpa_mfma_f32_kernel(
 
 constexpr int kStreamMaxKeys = 2048;
 
-template <int NQB>
+template <int NQB, bool LSE>
 __global__ __launch_bounds__(kWave *(NQB < 4 ? NQB : 4), 3) void sdpa_cross_stream_kernel(
     const uint16_t *__restrict__ q, int64_t q_stride, const uint16_t *__restrict__ k,
     const uint16_t *__restrict__ v, int64_t kv_stride, const uint8_t *__restrict__ alive,
@@ -795,7 +831,7 @@ __global__ __launch_bounds__(kWave *(NQB < 4 ? NQB : 4), 3) void sdpa_cross_stre
     __shared__ __align__(16) uint16_t s_vt[2][kDh * VP];
     __shared__ uint16_t s_idx[kStreamMaxKeys];  // indices of the live keys, ascending
     __shared__ int s_wcnt[NW];
-    static_assert(!SPLIT || sizeof(s_k) >= (size_t)NW * (16 * kWave + 2 * 32) * sizeof(float),
+    static_assert(!SPLIT || sizeof(s_k) >= (size_t)NW * (16 * kWave + 3 * 32) * sizeof(float),
                   "the partial results of the shared block are merged through the K buffers");
 
     const int chunk = gridDim.x >> 3;
@@ -949,124 +985,177 @@ __global__ __launch_bounds__(kWave *(NQB < 4 ? NQB : 4), 3) void sdpa_cross_stre
         acc0 = *reinterpret_cast<const u32x4 *>(accum + o_off);
         acc1 = *reinterpret_cast<const u32x4 *>(accum + o_off + 16);
     }
-    if (ntiles > 0) {
-        gather(0);
-        stash(0, 0);
-    }
-    // Every load issued so far has to be back before the loop: otherwise the compiler guards
-    // the first use of the query registers inside the loop with a wait for ALL outstanding
-    // loads, and that wait would also stall every iteration on the next tile's gather.
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), expcnt/lgkmcnt untouched
-    __syncthreads();
-    for (int t = 0; t < ntiles; ++t) {
-        const int buf = t & 1;
-        if (t + 1 < ntiles) gather(t + 1);
-        int nb = nkb - t * NW;
-        nb = nb < NW ? nb : NW;
-        // K Q^T of key block kb.  Only the very first key block can hold padding positions; they
-        // get -inf there.  The empty asm keeps that rare fix-up a real branch: folded into
-        // selects it would cost 16 extra instructions in every key block.
-        auto scores_of = [&](int kb, const bf16x8 &q0, const bf16x8 &q1) -> f32x16 {
-            const uint16_t *kp = &s_k[buf][(kb * 32 + m) * kKeyPitch + half * 8];
-            const bf16x8 ka0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp));
-            const bf16x8 ka1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + 16));
-            f32x16 z = {0.0f};
-            z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0, q0, z, 0, 0, 0);
-            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka1, q1, z, 0, 0, 0);
-        };
-        auto scores = [&](int kb) -> f32x16 { return scores_of(kb, qb0, qb1); };
-        auto mask_padding = [&](f32x16 &z) {
-            asm volatile("" ::: "memory");
-#pragma unroll
-            for (int e = 0; e < 16; ++e)
-                if (8 * (e >> 2) + 4 * half + (e & 3) < pad) z[e] = -INFINITY;
-        };
-        auto weigh_into = [&](int kb, const f32x16 &z, float mc, float &total, f32x16 &acc) {
-            float p[16];
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                p[e] = __builtin_amdgcn_exp2f(fmaf(z[e], scale_log2e, -mc));
-                total += p[e];
-            }
-#pragma unroll
-            for (int h2 = 0; h2 < 2; ++h2) {
-                bf16x8 pb;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * h2 + e];
-                const uint16_t *vp = &s_vt[buf][m * VP + kb * 32 + 16 * h2 + 4 * half];
-                const u32x2 lo = *reinterpret_cast<const u32x2 *>(vp);
-                const u32x2 hi = *reinterpret_cast<const u32x2 *>(vp + 8);
-                const u32x4 vq = {lo.x, lo.y, hi.x, hi.y};
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vq), pb, acc, 0, 0, 0);
-            }
-        };
-        auto weigh = [&](int kb, const f32x16 &z, float mc) { weigh_into(kb, z, mc, sum, o); };
-        if (wave * 32 < NQ) {
-            // two key blocks per iteration: two independent MFMA chains in flight
-            float tmx = -INFINITY;
-            int kb = 0;
-            for (; kb + 1 < nb; kb += 2) {
-                f32x16 z0 = scores(kb);
-                const f32x16 z1 = scores(kb + 1);
-                if (t == 0 && kb == 0 && pad != 0) mask_padding(z0);
-#pragma unroll
-                for (int e = 0; e < 16; ++e) tmx = fmaxf(tmx, z0[e]);  // one chain: max(z0[e], z1[e]) first would have both
-#pragma unroll
-                for (int e = 0; e < 16; ++e) tmx = fmaxf(tmx, z1[e]);  // operands quieted by a v_max x, x each (56 ops, not 16)
-            }
-            if (kb < nb) {
-                f32x16 z0 = scores(kb);
-                if (t == 0 && kb == 0 && pad != 0) mask_padding(z0);
-#pragma unroll
-                for (int e = 0; e < 16; ++e) tmx = fmaxf(tmx, z0[e]);
-            }
-            tmx = fmaxf(tmx, __shfl_xor(tmx, 32));
-            const float mnew = fmaxf(mx, tmx);  // finite: every key block holds at least one live key
-            const float alpha = __builtin_amdgcn_exp2f((mx - mnew) * scale_log2e);
-            mx = mnew;
-            sum *= alpha;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) o[e] *= alpha;
-            const float mc = mx * scale_log2e;
-            kb = 0;
-            for (; kb + 1 < nb; kb += 2) {
-                f32x16 z0 = scores(kb);
-                const f32x16 z1 = scores(kb + 1);
-                if (t == 0 && kb == 0 && pad != 0) mask_padding(z0);
-                weigh(kb, z0, mc);
-                weigh(kb + 1, z1, mc);
-            }
-            if (kb < nb) {
-                f32x16 z0 = scores(kb);
-                if (t == 0 && kb == 0 && pad != 0) mask_padding(z0);
-                weigh(kb, z0, mc);
-            }
+    // The walk over the tiles, in two forms.  First try (`shifted` false): weights exp2(scale S) without any shift - no
+    // sweep for the maximum, no rescaling between tiles, one K Q^T per key block.  Softmax does not depend on the
+    // shift, only the exponent range does: when a query's sum of weights leaves the safe float32 range (scores beyond
+    // +-60 in log2 units, or not finite), the whole work-group throws the try away and walks the tiles again in the
+    // second form, an online softmax with the running maximum as shift (two sweeps per tile).
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    float esum = 0.0f, sesum = 0.0f;  // the weights before rounding, for the log-sum-exp a backward pass asks for (LSE)
+    auto walk = [&](auto shifted) {
+        constexpr bool SHIFT = decltype(shifted)::value;
+        if (ntiles > 0) {
+            gather(0);
+            stash(0, 0);
         }
-        if (SPLIT && wave < nb) {
-            // the shared block of queries against key block `wave` of the tile: one online-softmax step
-            f32x16 z = scores_of(wave, sb0, sb1);
-            if (t == 0 && wave == 0 && pad != 0) mask_padding(z);
-            float tmx = z[0];
-#pragma unroll
-            for (int e = 1; e < 16; ++e) tmx = fmaxf(tmx, z[e]);
-            tmx = fmaxf(tmx, __shfl_xor(tmx, 32));
-            const float mnew = fmaxf(smx, tmx);  // finite: the key block holds at least one live key
-            const float alpha = __builtin_amdgcn_exp2f((smx - mnew) * scale_log2e);  // 0 the first time
-            smx = mnew;
-            ssum *= alpha;
-#pragma unroll
-            for (int e = 0; e < 16; ++e) so[e] *= alpha;
-            weigh_into(wave, z, smx * scale_log2e, ssum, so);
-        }
-        if (t + 1 < ntiles) stash(t + 1, buf ^ 1);
+        // Every load issued so far has to be back before the loop: otherwise the compiler guards
+        // the first use of the query registers inside the loop with a wait for ALL outstanding
+        // loads, and that wait would also stall every iteration on the next tile's gather.
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), expcnt/lgkmcnt untouched
         __syncthreads();
+        for (int t = 0; t < ntiles; ++t) {
+            const int buf = t & 1;
+            if (t + 1 < ntiles) gather(t + 1);
+            int nb = nkb - t * NW;
+            nb = nb < NW ? nb : NW;
+            // K Q^T of key block kb.  Only the very first key block can hold padding positions; they
+            // get -inf there.  The empty asm keeps that rare fix-up a real branch: folded into
+            // selects it would cost 16 extra instructions in every key block.
+            auto scores_of = [&](int kb, const bf16x8 &q0, const bf16x8 &q1) -> f32x16 {
+                const uint16_t *kp = &s_k[buf][(kb * 32 + m) * kKeyPitch + half * 8];
+                const bf16x8 ka0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp));
+                const bf16x8 ka1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(kp + 16));
+                f32x16 z = {0.0f};
+                z = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0, q0, z, 0, 0, 0);
+                return __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka1, q1, z, 0, 0, 0);
+            };
+            auto scores = [&](int kb) -> f32x16 { return scores_of(kb, qb0, qb1); };
+            auto mask_padding = [&](f32x16 &z) {
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    if (8 * (e >> 2) + 4 * half + (e & 3) < pad) z[e] = -INFINITY;
+            };
+            // the normaliser adds the weights as the matrix product sees them (rounded to bfloat16, a pair per
+            // instruction): a query with one live key gets that key's value row back exactly
+            auto weigh_into = [&](int kb, const f32x16 &z, float mc, float &total, float &exact, f32x16 &acc) {
+                float p[16];
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    if constexpr (SHIFT) p[e] = __builtin_amdgcn_exp2f(fmaf(z[e], scale_log2e, -mc));
+                    else p[e] = __builtin_amdgcn_exp2f(z[e] * scale_log2e);
+                    if (LSE) exact += p[e];
+                }
+#pragma unroll
+                for (int h2 = 0; h2 < 2; ++h2) {
+                    bf16x8 pb;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * h2 + e];
+#pragma unroll
+                    for (int e = 0; e < 8; e += 2) total = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{pb[e], pb[e + 1]}, ones, total, false);
+                    const uint16_t *vp = &s_vt[buf][m * VP + kb * 32 + 16 * h2 + 4 * half];
+                    const u32x2 lo = *reinterpret_cast<const u32x2 *>(vp);
+                    const u32x2 hi = *reinterpret_cast<const u32x2 *>(vp + 8);
+                    const u32x4 vq = {lo.x, lo.y, hi.x, hi.y};
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vq), pb, acc, 0, 0, 0);
+                }
+            };
+            auto weigh = [&](int kb, const f32x16 &z, float mc) { weigh_into(kb, z, mc, sum, esum, o); };
+            if (wave * 32 < NQ) {
+                float mc = 0.0f;
+                int kb = 0;
+                if constexpr (SHIFT) {
+                    // two key blocks per iteration: two independent MFMA chains in flight
+                    float tmx = -INFINITY;
+                    for (; kb + 1 < nb; kb += 2) {
+                        f32x16 z0 = scores(kb);
+                        const f32x16 z1 = scores(kb + 1);
+                        if (t == 0 && kb == 0 && pad != 0) mask_padding(z0);
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) tmx = fmaxf(tmx, z0[e]);  // one chain: max(z0[e], z1[e]) first would have both
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) tmx = fmaxf(tmx, z1[e]);  // operands quieted by a v_max x, x each (56 ops, not 16)
+                    }
+                    if (kb < nb) {
+                        f32x16 z0 = scores(kb);
+                        if (t == 0 && kb == 0 && pad != 0) mask_padding(z0);
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) tmx = fmaxf(tmx, z0[e]);
+                    }
+                    tmx = fmaxf(tmx, __shfl_xor(tmx, 32));
+                    const float mnew = fmaxf(mx, tmx);  // finite: every key block holds at least one live key
+                    const float alpha = __builtin_amdgcn_exp2f((mx - mnew) * scale_log2e);
+                    mx = mnew;
+                    sum *= alpha;
+                    if (LSE) esum *= alpha;
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) o[e] *= alpha;
+                    mc = mx * scale_log2e;
+                    kb = 0;
+                }
+                for (; kb + 1 < nb; kb += 2) {
+                    f32x16 z0 = scores(kb);
+                    const f32x16 z1 = scores(kb + 1);
+                    if (t == 0 && kb == 0 && pad != 0) mask_padding(z0);
+                    weigh(kb, z0, mc);
+                    weigh(kb + 1, z1, mc);
+                }
+                if (kb < nb) {
+                    f32x16 z0 = scores(kb);
+                    if (t == 0 && kb == 0 && pad != 0) mask_padding(z0);
+                    weigh(kb, z0, mc);
+                }
+            }
+            if (SPLIT && wave < nb) {
+                // the shared block of queries against key block `wave` of the tile
+                f32x16 z = scores_of(wave, sb0, sb1);
+                if (t == 0 && wave == 0 && pad != 0) mask_padding(z);
+                if constexpr (SHIFT) {
+                    // one online-softmax step
+                    float tmx = z[0];
+#pragma unroll
+                    for (int e = 1; e < 16; ++e) tmx = fmaxf(tmx, z[e]);
+                    tmx = fmaxf(tmx, __shfl_xor(tmx, 32));
+                    const float mnew = fmaxf(smx, tmx);  // finite: the key block holds at least one live key
+                    const float alpha = __builtin_amdgcn_exp2f((smx - mnew) * scale_log2e);  // 0 the first time
+                    smx = mnew;
+                    ssum *= alpha;
+                    if (LSE) sesum *= alpha;
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) so[e] *= alpha;
+                } else {
+                    smx = 0.0f;  // this wave met a key block: its part counts, with shift zero
+                }
+                weigh_into(wave, z, smx * scale_log2e, ssum, sesum, so);
+            }
+            if (t + 1 < ntiles) stash(t + 1, buf ^ 1);
+            __syncthreads();
+        }
+    };
+    walk(std::false_type{});
+    {
+        // one vote of the work-group: the second walk shares tiles and barriers, so all waves take it or none does
+        const float whole = sum + __shfl_xor(sum, 32);
+        bool fine = (whole >= 0x1p-60f && whole <= 0x1p60f) || cnt == 0 || wave * 32 >= NQ;  // false for NaN
+        if (SPLIT) {
+            const float part = ssum + __shfl_xor(ssum, 32);
+            // a part may be empty (no key block met); one that is merely tiny next to the others also sends the
+            // work-group to the second walk, which is always right
+            fine = fine && ((part >= 0x1p-60f && part <= 0x1p60f) || smx == -INFINITY);
+        }
+        if (lane == 0) s_wcnt[wave] = __all(fine) ? 1 : 0;
+        __syncthreads();
+        bool redo = false;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) redo = redo || s_wcnt[w] == 0;
+        if (redo) {
+            mx = -INFINITY, sum = 0.0f, esum = 0.0f, smx = -INFINITY, ssum = 0.0f, sesum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[e] = 0.0f, so[e] = 0.0f;
+            walk(std::true_type{});
+        } else {
+            mx = 0.0f;
+        }
     }
     sum += __shfl_xor(sum, 32);
     const float inv = cnt == 0 ? 0.0f : __builtin_amdgcn_rcpf(sum);
     // log2 of the sum over the keys of exp2(score * scale_log2e), for a backward pass that would otherwise recompute it
     // (meaningless for an environment without keys, which that pass does not read)
     float *lse_env = lse_out == nullptr ? nullptr : lse_out + ((int64_t)env * H + head) * NQ;
-    if (lse_env != nullptr && qrow < NQ && half == 0) lse_env[qrow] = fmaf(mx, scale_log2e, __builtin_amdgcn_logf(sum));
+    if (LSE) {
+        esum += __shfl_xor(esum, 32);
+        if (lse_env != nullptr && qrow < NQ && half == 0) lse_env[qrow] = fmaf(mx, scale_log2e, __builtin_amdgcn_logf(esum));
+    }
 
     if (SPLIT) {
         // Merge the four partial results of the shared block.  Every wave has passed the barrier of the last tile,
@@ -1074,32 +1163,35 @@ __global__ __launch_bounds__(kWave *(NQB < 4 ? NQB : 4), 3) void sdpa_cross_stre
         float *part = reinterpret_cast<float *>(&s_k[0][0]);
         float *stat = part + NW * 16 * kWave;
         ssum += __shfl_xor(ssum, 32);
+        if (LSE) sesum += __shfl_xor(sesum, 32);
 #pragma unroll
         for (int e = 0; e < 16; ++e) part[(wave * 16 + e) * kWave + lane] = so[e];
         if (half == 0) {
-            stat[(wave * 2 + 0) * 32 + m] = smx;
-            stat[(wave * 2 + 1) * 32 + m] = ssum;
+            stat[(wave * 3 + 0) * 32 + m] = smx;
+            stat[(wave * 3 + 1) * 32 + m] = ssum;
+            if (LSE) stat[(wave * 3 + 2) * 32 + m] = sesum;
         }
         __syncthreads();
         // wave w finishes accumulator registers 4w .. 4w+3 of the 32 queries: rows 8w + 4*half + 0..3 of V^T as it
         // lies in LDS, which the stash fills so that they are channels 16 (w / 2) + 8*half + 4 (w % 2) + 0..3
         float mall = -INFINITY;
 #pragma unroll
-        for (int j = 0; j < NW; ++j) mall = fmaxf(mall, stat[(j * 2 + 0) * 32 + m]);
-        float total = 0.0f;
+        for (int j = 0; j < NW; ++j) mall = fmaxf(mall, stat[(j * 3 + 0) * 32 + m]);
+        float total = 0.0f, etotal = 0.0f;
         float r[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int j = 0; j < NW; ++j) {
-            const float mj = stat[(j * 2 + 0) * 32 + m];
+            const float mj = stat[(j * 3 + 0) * 32 + m];
             // a wave that met no key block holds (-inf, 0, 0); with no key at all every part is like that
             const float f = mj == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f((mj - mall) * scale_log2e);
-            total = fmaf(f, stat[(j * 2 + 1) * 32 + m], total);
+            total = fmaf(f, stat[(j * 3 + 1) * 32 + m], total);
+            if (LSE) etotal = fmaf(f, stat[(j * 3 + 2) * 32 + m], etotal);
 #pragma unroll
             for (int i = 0; i < 4; ++i) r[i] = fmaf(f, part[(j * 16 + wave * 4 + i) * kWave + lane], r[i]);
         }
         const float sinv = cnt == 0 ? 0.0f : __builtin_amdgcn_rcpf(total);
-        if (lse_env != nullptr && wave == 0 && srow < NQ && half == 0)
-            lse_env[srow] = fmaf(mall, scale_log2e, __builtin_amdgcn_logf(total));
+        if (LSE && lse_env != nullptr && wave == 0 && srow < NQ && half == 0)
+            lse_env[srow] = fmaf(mall, scale_log2e, __builtin_amdgcn_logf(etotal));
         if (srow < NQ) {
             const int64_t at = ((int64_t)env * NQ + srow) * D + head * kDh + 16 * (wave >> 1) + 8 * half + 4 * (wave & 1);
 #pragma unroll
@@ -1245,9 +1337,15 @@ static int launch_cross_stream(const void *q, int64_t q_stride, const void *k, c
     const int64_t blocks = (pairs + 7) / 8 * 8;
     if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
     const float scale_log2e = kLog2eA / sqrtf((float)kDh);
-    hipLaunchKernelGGL((sdpa_cross_stream_kernel<NQB>), dim3((unsigned)blocks), dim3(kWave * (NQB < 4 ? NQB : 4)), 0, stream,
-                       (const uint16_t *)q, q_stride, (const uint16_t *)k, (const uint16_t *)v, kv_stride, alive,
-                       ranges, (const uint16_t *)accum, (uint16_t *)out, lse, B, NQ, NK, H, scale_log2e);
+    // the log-sum-exp (asked for by the update's forward) costs sixteen additions per key block: a form of its own
+    if (lse != nullptr)
+        hipLaunchKernelGGL((sdpa_cross_stream_kernel<NQB, true>), dim3((unsigned)blocks), dim3(kWave * (NQB < 4 ? NQB : 4)), 0,
+                           stream, (const uint16_t *)q, q_stride, (const uint16_t *)k, (const uint16_t *)v, kv_stride, alive,
+                           ranges, (const uint16_t *)accum, (uint16_t *)out, lse, B, NQ, NK, H, scale_log2e);
+    else
+        hipLaunchKernelGGL((sdpa_cross_stream_kernel<NQB, false>), dim3((unsigned)blocks), dim3(kWave * (NQB < 4 ? NQB : 4)), 0,
+                           stream, (const uint16_t *)q, q_stride, (const uint16_t *)k, (const uint16_t *)v, kv_stride, alive,
+                           ranges, (const uint16_t *)accum, (uint16_t *)out, lse, B, NQ, NK, H, scale_log2e);
     return (int)hipGetLastError();
 }
 

@@ -200,6 +200,55 @@ def test_sdpa_bf16_matches_fp32_oracle(B, NM, path):
     assert max_rel(got.float(), truth) <= max_rel(lib16, truth) + 8e-3
 
 
+@pytest.mark.parametrize("NM,path", [(12, "mfma"), (12, "auto"), (84, "mfma"), (160, "mfma"), (84, "env"), (84, "head"), (160, "head")])
+@pytest.mark.parametrize("case", ["large", "huge", "all_negative", "mixed"])
+def test_sdpa_bf16_scores_beyond_the_exponent_range_take_the_shifted_sweep(NM, path, case):
+    """The matrix-core kernels first form the weights without subtracting the maximum; scores whose weights leave
+    float32's safe range (|score| / sqrt(dh) beyond ~40) must fall back to the shifted form and stay at the bar."""
+    B, H, D = 4, 4, 128
+    g = torch.Generator().manual_seed(NM + len(case))
+    qkv = torch.randn(B, NM, 3 * D, generator=g)
+    if case == "large":        # weights up to 2^150: overflow without the shift
+        qkv[..., : 2 * D] *= 6.0
+    elif case == "huge":       # nearly one-hot rows
+        qkv[..., : 2 * D] *= 40.0
+    elif case == "all_negative":
+        # every key points against every query: all weights underflow without the shift, yet they differ by O(1)
+        u = torch.randn(H, 32, generator=g)
+        u = u / u.norm(dim=-1, keepdim=True)
+        k = 30.0 * u.view(1, 1, H, 32) + 0.3 * torch.randn(B, NM, H, 32, generator=g)
+        qkv[..., D:2 * D] = k.reshape(B, NM, D)
+        qkv[..., :D] = (-30.0 * u.view(1, 1, H, 32) + 0.3 * torch.randn(B, NM, H, 32, generator=g)).reshape(B, NM, D)
+    else:                      # one environment out of range, the others ordinary: the choice is made per wave
+        qkv[1, :, : 2 * D] *= 25.0
+    qkv = qkv.bfloat16()
+    alive = _alive(NM, B, NM, 0.7)
+    alive[:, NM // 3] = True
+    got = _run_sdpa(qkv, alive, H, path).float()
+    assert torch.isfinite(got).all()
+    truth = torch_ref.sdpa_masked(qkv.double(), alive, H).float()
+    for b in range(B):
+        assert max_rel(got[b], truth[b]) <= BF16_TOL, (case, b)
+    lib16 = torch_ref.sdpa_masked(qkv, alive, H).float()
+    assert max_rel(got, truth) <= max_rel(lib16, truth) + 8e-3
+
+
+def test_sdpa_bf16_one_live_key_returns_its_value_row_exactly_on_every_kernel():
+    # the normaliser is the sum of the weights as the matrix product sees them, so a single weight cancels exactly
+    B, NM, H, D = 3, 84, 4, 128
+    qkv = _qkv(5, B, NM, D, torch.bfloat16, scale=2.0)
+    alive = torch.zeros(B, NM, dtype=torch.bool)
+    alive[0, 7], alive[1, NM - 1], alive[2, 40] = True, True, True
+    for path in ("mfma", "env", "head"):
+        got = _run_sdpa(qkv, alive, H, path)
+        for b, key in enumerate((7, NM - 1, 40)):
+            assert torch.equal(got[b], qkv[b, key, 2 * D:].expand(NM, D)), (path, b)
+    small = _qkv(6, B, 12, D, torch.bfloat16, scale=2.0)
+    one = torch.zeros(B, 12, dtype=torch.bool)
+    one[:, 5] = True
+    assert torch.equal(_run_sdpa(small, one, H, "auto"), small[:, 5:6, 2 * D:].expand(B, 12, D))
+
+
 def test_sdpa_bf16_both_kernels_agree():
     B, NM, H, D = 6, 84, 4, 128
     qkv = _qkv(21, B, NM, D, torch.bfloat16)
