@@ -12,7 +12,7 @@ import os
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "_lib", "libbnb_amd.so")
 
-ABI_VERSION = 27
+ABI_VERSION = 28
 F32, BF16 = 0, 1
 PATH_AUTO, PATH_VALU, PATH_MFMA, PATH_ENV, PATH_HEAD = 0, 1, 2, 3, 4
 WGRAD_PATH_AUTO, WGRAD_PATH_STAGED, WGRAD_PATH_DMA = 0, 1, 2
@@ -42,7 +42,7 @@ SIGNATURES = {
     "bnb_linear_wgrad_fwd": (_i, [_vp, _i64, _vp, _i64, _vp, _i, _vp, _i, _i64, _i, _i, _vp]),
     "bnb_linear_wgrad_tiled_fwd": (_i, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i, _vp, _i, _i64, _i, _i, _vp]),
     "bnb_conv_seq_bwd_blocks": (_i, [_i64, _i, _i]),
-    "bnb_conv_seq_bwd": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _vp]),
+    "bnb_conv_seq_bwd": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i64, _i, _i, _i, _i, _i, _vp]),
     "bnb_column_sums_slices": (_i, [_i64, _i]),
     "bnb_column_sums": (_i, [_vp, _i, _i64, _vp, _i, _vp, _i, _i64, _i, _vp]),
     "bnb_gelu_mul_bwd": (_i, [_vp, _i, _i64, _vp, _i, _i64, _vp, _i, _vp, _i64, _vp, _i64, _i64, _i, _vp]),
@@ -66,10 +66,10 @@ SIGNATURES = {
              _vp, _i, _i64, _i, _vp]
     ),
     "bnb_conv_step_fwd": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i64, _i64, _i, _vp]),
-    "bnb_conv_seq_fwd": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i, _i, _vp]),
-    "bnb_rglru_scan_fwd": (_i, [_vp, _i, _vp, _i, _vp, _f, _vp, _i64, _vp, _vp, _i, _vp, _i64, _i64, _i, _i, _i, _vp]),
+    "bnb_conv_seq_fwd": (_i, [_vp, _i, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i, _i, _i, _i, _i, _vp]),
+    "bnb_rglru_scan_fwd": (_i, [_vp, _i, _vp, _i, _vp, _f, _vp, _i64, _vp, _vp, _i, _vp, _i64, _i64, _i, _i, _i, _i, _i, _vp]),
     "bnb_rglru_scan_bwd": (
-        _i, [_vp, _i, _vp, _i, _vp, _f, _vp, _i64, _vp, _vp, _i, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _vp]
+        _i, [_vp, _i, _vp, _i, _vp, _f, _vp, _i64, _vp, _vp, _i, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _i, _vp]
     ),
     "bnb_add_rmsnorm_fwd": (_i, [_vp, _i64, _vp, _i, _vp, _f, _vp, _vp, _i, _i64, _i, _vp]),
     "bnb_norm_linear_fwd": (_i, [_vp, _i64, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i64, _i, _i, _vp]),

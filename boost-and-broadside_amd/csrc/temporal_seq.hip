@@ -22,6 +22,16 @@ constexpr int kSeqThreads = 256;
 constexpr int kSeqTaps = 4;
 constexpr int kSeqAhead = 4;  // timesteps whose operands are in flight together
 
+// A time-major tensor may hold this call's rows inside a wider token tensor (T, environments * pitch, D): the rows of
+// environment b are then rows b * pitch .. b * pitch + group - 1 of every step (group == 0: the tensor holds this
+// call's rows only).  The update path keeps ship and field tokens of a sublayer in one tensor that way.
+__device__ __forceinline__ int64_t placed_row(int64_t row, int group, int pitch)
+{
+    if (group <= 0) return row;
+    const int64_t b = row / group;
+    return b * pitch + (row - b * group);
+}
+
 // ------------------------------------------------------------------------------------
 // RG-LRU over T steps
 // ------------------------------------------------------------------------------------
@@ -30,7 +40,8 @@ template <typename XT, typename GT, typename YT>
 __global__ __launch_bounds__(kSeqThreads) void rglru_scan_vec8_kernel(
     const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
     const float *__restrict__ h0, int64_t h0_stride, const uint8_t *__restrict__ done, YT *__restrict__ y,
-    float *__restrict__ h_last, int64_t h_last_stride, int64_t R, int T, int D, int64_t rs, int64_t ts, int rows_per_block)
+    float *__restrict__ h_last, int64_t h_last_stride, int64_t R, int T, int D, int64_t rs, int64_t ts, int rows_per_block,
+    int y_group, int y_pitch, int64_t ts_y)
 {
     extern __shared__ float s_l2sig[];  // D entries
     for (int d = threadIdx.x; d < D; d += kSeqThreads) s_l2sig[d] = log2_sigmoid(log_lambda[d]);
@@ -49,7 +60,7 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_vec8_kernel(
     Row8 h = load8_split<false>(h0 + row * h0_stride + d0, gap);
     const XT *xp = x + row * rs + d0;
     const GT *gp = gates + row * 2 * rs + d0;
-    YT *yp = y + row * rs + d0;
+    YT *yp = y + placed_row(row, y_group, y_pitch) * rs + d0;
     const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
 
     for (int t0 = 0; t0 < T; t0 += kSeqAhead) {
@@ -75,7 +86,7 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_vec8_kernel(
                     h.v[e] = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(xv[u].v[e], ga[u].v[e], gx[u].v[e],
                                                                                     l2[e], c, prev);
                 }
-                store8_split<true>(yp + (t0 + u) * ts, gap, h);
+                store8_split<true>(yp + (t0 + u) * ts_y, gap, h);
             }
         }
     }
@@ -87,7 +98,8 @@ template <typename XT, typename GT, typename YT>
 __global__ __launch_bounds__(kSeqThreads) void rglru_scan_scalar_kernel(
     const XT *__restrict__ x, const GT *__restrict__ gates, const float *__restrict__ log_lambda, float c,
     const float *__restrict__ h0, int64_t h0_stride, const uint8_t *__restrict__ done, YT *__restrict__ y,
-    float *__restrict__ h_last, int64_t h_last_stride, int64_t R, int T, int D, int64_t rs, int64_t ts)
+    float *__restrict__ h_last, int64_t h_last_stride, int64_t R, int T, int D, int64_t rs, int64_t ts, int y_group,
+    int y_pitch, int64_t ts_y)
 {
     const int64_t idx = (int64_t)blockIdx.x * kSeqThreads + threadIdx.x;
     if (idx >= R * D) return;
@@ -97,7 +109,7 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_scalar_kernel(
     float h = h0[row * h0_stride + d];
     const XT *xp = x + row * rs + d;
     const GT *gp = gates + row * 2 * rs + d;
-    YT *yp = y + row * rs + d;
+    YT *yp = y + placed_row(row, y_group, y_pitch) * rs + d;
     const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
     for (int t0 = 0; t0 < T; t0 += kSeqAhead) {
         float xv[kSeqAhead], ga[kSeqAhead], gx[kSeqAhead];
@@ -117,7 +129,7 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_scalar_kernel(
             if (t0 + u < T) {
                 h = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(xv[u], ga[u], gx[u], l2, c,
                                                                           cut[u] ? 0.0f : h);
-                store1(yp + (t0 + u) * ts, h);
+                store1(yp + (t0 + u) * ts_y, h);
             }
         }
     }
@@ -127,10 +139,11 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_scalar_kernel(
 template <typename XT, typename GT, typename YT>
 static int launch_scan(const void *x, const void *gates, const float *log_lambda, float c, const float *h0,
                        int64_t h0_stride, const uint8_t *done, void *y, float *h_last, int64_t h_last_stride,
-                       int64_t R, int T, int D, int time_major, hipStream_t stream)
+                       int64_t R, int T, int D, int time_major, int y_group, int y_pitch, hipStream_t stream)
 {
     // element strides of one row / one timestep: (R, T, D) or (T, R, D)
     const int64_t rs = time_major ? D : (int64_t)T * D, ts = time_major ? R * D : D;
+    const int64_t ts_y = y_group > 0 ? R / y_group * y_pitch * D : ts;
     const bool vec_ok = (D % 8 == 0) && (D / 8 <= kSeqThreads) && aligned16(x) && aligned16(gates) && aligned16(h0) &&
                         aligned16(h_last) && aligned16(y) && (h0_stride % 4 == 0) && (h_last_stride % 4 == 0);
     // the wide lanes need enough rows to fill the chip; below that one lane per channel
@@ -141,13 +154,14 @@ static int launch_scan(const void *x, const void *gates, const float *log_lambda
         if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
         hipLaunchKernelGGL((rglru_scan_vec8_kernel<XT, GT, YT>), dim3((unsigned)blocks), dim3(kSeqThreads),
                            (size_t)D * sizeof(float), stream, (const XT *)x, (const GT *)gates, log_lambda, c, h0,
-                           h0_stride, done, (YT *)y, h_last, h_last_stride, R, T, D, rs, ts, rows_per_block);
+                           h0_stride, done, (YT *)y, h_last, h_last_stride, R, T, D, rs, ts, rows_per_block, y_group, y_pitch,
+                           ts_y);
     } else {
         const int64_t blocks = (R * D + kSeqThreads - 1) / kSeqThreads;
         if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
         hipLaunchKernelGGL((rglru_scan_scalar_kernel<XT, GT, YT>), dim3((unsigned)blocks), dim3(kSeqThreads), 0,
                            stream, (const XT *)x, (const GT *)gates, log_lambda, c, h0, h0_stride, done, (YT *)y,
-                           h_last, h_last_stride, R, T, D, rs, ts);
+                           h_last, h_last_stride, R, T, D, rs, ts, y_group, y_pitch, ts_y);
     }
     return (int)hipGetLastError();
 }
@@ -155,13 +169,14 @@ static int launch_scan(const void *x, const void *gates, const float *log_lambda
 template <typename XT, typename GT>
 static int scan_dispatch_y(const void *x, const void *gates, const float *log_lambda, float c, const float *h0,
                            int64_t h0_stride, const uint8_t *done, void *y, int y_dtype, float *h_last,
-                           int64_t h_last_stride, int64_t R, int T, int D, int time_major, hipStream_t stream)
+                           int64_t h_last_stride, int64_t R, int T, int D, int time_major, int y_group, int y_pitch,
+                           hipStream_t stream)
 {
     if (y_dtype == BNB_F32)
         return launch_scan<XT, GT, float>(x, gates, log_lambda, c, h0, h0_stride, done, y, h_last, h_last_stride, R,
-                                          T, D, time_major, stream);
+                                          T, D, time_major, y_group, y_pitch, stream);
     return launch_scan<XT, GT, uint16_t>(x, gates, log_lambda, c, h0, h0_stride, done, y, h_last, h_last_stride, R, T,
-                                         D, time_major, stream);
+                                         D, time_major, y_group, y_pitch, stream);
 }
 
 // ------------------------------------------------------------------------------------
@@ -220,7 +235,7 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_bwd_scalar_kernel(
     const float *__restrict__ h0, int64_t h0_stride, const uint8_t *__restrict__ done, const YT *__restrict__ y,
     const YT *__restrict__ dy, const float *__restrict__ dh_last, int64_t dh_last_stride, XT *__restrict__ dx,
     GT *__restrict__ dgates, float *__restrict__ dh0, float *__restrict__ dlam_rows, int64_t R, int T, int D,
-    int64_t rs, int64_t ts)
+    int64_t rs, int64_t ts, int y_group, int y_pitch, int64_t ts_y)
 {
     const int64_t idx = (int64_t)blockIdx.x * kSeqThreads + threadIdx.x;
     if (idx >= R * D) return;
@@ -230,8 +245,9 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_bwd_scalar_kernel(
     const float l2 = log2_sigmoid(lam), oms = sigmoid_neg(lam);
     const XT *xp = x + row * rs + d;
     const GT *gp = gates + row * 2 * rs + d;
-    const YT *yp = y + row * rs + d;
-    const YT *dyp = dy == nullptr ? nullptr : dy + row * rs + d;
+    const int64_t at_y = placed_row(row, y_group, y_pitch) * rs;  // y and dy: possibly rows of a wider token tensor
+    const YT *yp = y + at_y + d;
+    const YT *dyp = dy == nullptr ? nullptr : dy + at_y + d;
     XT *dxp = dx + row * rs + d;
     GT *dgp = dgates + row * 2 * rs + d;
     const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
@@ -247,8 +263,8 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_bwd_scalar_kernel(
             xv[u] = load1(xp + t * ts);
             ga[u] = load1(gp + t * 2 * ts);
             gx[u] = load1(gp + t * 2 * ts + D);
-            dyv[u] = dyp == nullptr ? 0.0f : load1(dyp + t * ts);
-            hp[u] = load1(yp + (t > 0 ? t - 1 : 0) * ts);
+            dyv[u] = dyp == nullptr ? 0.0f : load1(dyp + t * ts_y);
+            hp[u] = load1(yp + (t > 0 ? t - 1 : 0) * ts_y);
             cut[u] = 0;
             if (dn != nullptr) cut[u] = dn[t > 0 ? t - 1 : 0];
             if (t == 0) {
@@ -281,7 +297,7 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_bwd_vec8_kernel(
     const float *__restrict__ h0, int64_t h0_stride, const uint8_t *__restrict__ done, const YT *__restrict__ y,
     const YT *__restrict__ dy, const float *__restrict__ dh_last, int64_t dh_last_stride, XT *__restrict__ dx,
     GT *__restrict__ dgates, float *__restrict__ dh0, float *__restrict__ dlam_rows, int64_t R, int T, int D,
-    int64_t rs, int64_t ts, int rows_per_block)
+    int64_t rs, int64_t ts, int rows_per_block, int y_group, int y_pitch, int64_t ts_y)
 {
     extern __shared__ float s_lam[];  // D entries of log2 sigmoid(lambda), then D of 1 - sigmoid(lambda)
     for (int d = threadIdx.x; d < D; d += kSeqThreads) {
@@ -306,8 +322,9 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_bwd_vec8_kernel(
     }
     const XT *xp = x + row * rs + d0;
     const GT *gp = gates + row * 2 * rs + d0;
-    const YT *yp = y + row * rs + d0;
-    const YT *dyp = dy == nullptr ? nullptr : dy + row * rs + d0;
+    const int64_t at_y = placed_row(row, y_group, y_pitch) * rs;  // y and dy: possibly rows of a wider token tensor
+    const YT *yp = y + at_y + d0;
+    const YT *dyp = dy == nullptr ? nullptr : dy + at_y + d0;
     XT *dxp = dx + row * rs + d0;
     GT *dgp = dgates + row * 2 * rs + d0;
     const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
@@ -328,12 +345,12 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_bwd_vec8_kernel(
             ga[u] = load8_split<true>(gp + t * 2 * ts, gap);
             gx[u] = load8_split<true>(gp + t * 2 * ts + D, gap);
             if (dyp != nullptr) {
-                dyv[u] = load8_split<true>(dyp + t * ts, gap);
+                dyv[u] = load8_split<true>(dyp + t * ts_y, gap);
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) dyv[u].v[e] = 0.0f;
             }
-            hp[u] = load8_split<false>(yp + (t > 0 ? t - 1 : 0) * ts, gap);
+            hp[u] = load8_split<false>(yp + (t > 0 ? t - 1 : 0) * ts_y, gap);
             cut[u] = 0;
             if (dn != nullptr) cut[u] = dn[t > 0 ? t - 1 : 0];
             if (t == 0) {
@@ -371,9 +388,11 @@ template <typename XT, typename GT, typename YT>
 static int launch_scan_bwd(const void *x, const void *gates, const float *log_lambda, float c, const float *h0,
                            int64_t h0_stride, const uint8_t *done, const void *y, const void *dy,
                            const float *dh_last, int64_t dh_last_stride, void *dx, void *dgates, float *dh0,
-                           float *dlam_rows, int64_t R, int T, int D, int time_major, hipStream_t stream)
+                           float *dlam_rows, int64_t R, int T, int D, int time_major, int y_group, int y_pitch,
+                           hipStream_t stream)
 {
     const int64_t rs = time_major ? D : (int64_t)T * D, ts = time_major ? R * D : D;
+    const int64_t ts_y = y_group > 0 ? R / y_group * y_pitch * D : ts;
     const bool vec_ok = (D % 8 == 0) && (D / 8 <= kSeqThreads) && aligned16(x) && aligned16(gates) && aligned16(h0) &&
                         aligned16(y) && aligned16(dy) && aligned16(dh_last) && aligned16(dx) && aligned16(dgates) &&
                         aligned16(dh0) && aligned16(dlam_rows) && (h0_stride % 4 == 0) && (dh_last_stride % 4 == 0);
@@ -385,14 +404,14 @@ static int launch_scan_bwd(const void *x, const void *gates, const float *log_la
         hipLaunchKernelGGL((rglru_scan_bwd_vec8_kernel<XT, GT, YT>), dim3((unsigned)blocks), dim3(kSeqThreads),
                            (size_t)2 * D * sizeof(float), stream, (const XT *)x, (const GT *)gates, log_lambda, c, h0,
                            h0_stride, done, (const YT *)y, (const YT *)dy, dh_last, dh_last_stride, (XT *)dx,
-                           (GT *)dgates, dh0, dlam_rows, R, T, D, rs, ts, rows_per_block);
+                           (GT *)dgates, dh0, dlam_rows, R, T, D, rs, ts, rows_per_block, y_group, y_pitch, ts_y);
     } else {
         const int64_t blocks = (R * D + kSeqThreads - 1) / kSeqThreads;
         if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
         hipLaunchKernelGGL((rglru_scan_bwd_scalar_kernel<XT, GT, YT>), dim3((unsigned)blocks), dim3(kSeqThreads), 0,
                            stream, (const XT *)x, (const GT *)gates, log_lambda, c, h0, h0_stride, done,
                            (const YT *)y, (const YT *)dy, dh_last, dh_last_stride, (XT *)dx, (GT *)dgates, dh0,
-                           dlam_rows, R, T, D, rs, ts);
+                           dlam_rows, R, T, D, rs, ts, y_group, y_pitch, ts_y);
     }
     return (int)hipGetLastError();
 }
@@ -401,13 +420,14 @@ template <typename XT, typename GT>
 static int scan_bwd_dispatch_y(const void *x, const void *gates, const float *log_lambda, float c, const float *h0,
                                int64_t h0_stride, const uint8_t *done, const void *y, int y_dtype, const void *dy,
                                const float *dh_last, int64_t dh_last_stride, void *dx, void *dgates, float *dh0,
-                               float *dlam_rows, int64_t R, int T, int D, int time_major, hipStream_t stream)
+                               float *dlam_rows, int64_t R, int T, int D, int time_major, int y_group, int y_pitch,
+                               hipStream_t stream)
 {
     if (y_dtype == BNB_F32)
-        return launch_scan_bwd<XT, GT, float>(x, gates, log_lambda, c, h0, h0_stride, done, y, dy, dh_last,
-                                              dh_last_stride, dx, dgates, dh0, dlam_rows, R, T, D, time_major, stream);
-    return launch_scan_bwd<XT, GT, uint16_t>(x, gates, log_lambda, c, h0, h0_stride, done, y, dy, dh_last,
-                                             dh_last_stride, dx, dgates, dh0, dlam_rows, R, T, D, time_major, stream);
+        return launch_scan_bwd<XT, GT, float>(x, gates, log_lambda, c, h0, h0_stride, done, y, dy, dh_last, dh_last_stride,
+                                              dx, dgates, dh0, dlam_rows, R, T, D, time_major, y_group, y_pitch, stream);
+    return launch_scan_bwd<XT, GT, uint16_t>(x, gates, log_lambda, c, h0, h0_stride, done, y, dy, dh_last, dh_last_stride,
+                                             dx, dgates, dh0, dlam_rows, R, T, D, time_major, y_group, y_pitch, stream);
 }
 
 // ------------------------------------------------------------------------------------
@@ -421,7 +441,8 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_vec8_kernel(
     const BT *__restrict__ b1, const float *__restrict__ conv_in, int64_t conv_in_stride,
     const float *__restrict__ weight, const float *__restrict__ bias, const uint8_t *__restrict__ done,
     float *__restrict__ v_out, uint16_t *__restrict__ v_bf16_out, float *__restrict__ conv_out,
-    int64_t conv_out_stride, int64_t R, int T, int D, int64_t rs, int64_t ts, int rows_per_block)
+    int64_t conv_out_stride, int64_t R, int T, int D, int64_t rs, int64_t ts, int rows_per_block, int b_group, int b_pitch,
+    int64_t ts_b)
 {
     const int vecs_per_row = D >> 3;
     const int local_row = threadIdx.x / vecs_per_row;
@@ -442,7 +463,7 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_vec8_kernel(
     }
     const float *pin = conv_in + row * conv_in_stride + d0;
     Row8 p0 = load8_split<false>(pin, gap), p1 = load8_split<false>(pin + D, gap), p2 = load8_split<false>(pin + 2 * D, gap);
-    const BT *bp = b1 + row * rs + d0;
+    const BT *bp = b1 + placed_row(row, b_group, b_pitch) * rs + d0;
     const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
     int hist = 3;
 
@@ -452,7 +473,7 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_vec8_kernel(
 #pragma unroll
         for (int u = 0; u < kSeqAhead; ++u) {
             const int t = t0 + u < T ? t0 + u : T - 1;
-            cur[u] = load8_split<true>(bp + t * ts, gap);
+            cur[u] = load8_split<true>(bp + t * ts_b, gap);
             cut[u] = 0;
             if (dn != nullptr) cut[u] = dn[t > 0 ? t - 1 : 0];
             if (t == 0) cut[u] = 0;
@@ -494,7 +515,7 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_scalar_kernel(
     const BT *__restrict__ b1, const float *__restrict__ conv_in, int64_t conv_in_stride,
     const float *__restrict__ weight, const float *__restrict__ bias, const uint8_t *__restrict__ done,
     float *__restrict__ v_out, uint16_t *__restrict__ v_bf16_out, float *__restrict__ conv_out,
-    int64_t conv_out_stride, int64_t R, int T, int D, int64_t rs, int64_t ts)
+    int64_t conv_out_stride, int64_t R, int T, int D, int64_t rs, int64_t ts, int b_group, int b_pitch, int64_t ts_b)
 {
     const int64_t idx = (int64_t)blockIdx.x * kSeqThreads + threadIdx.x;
     if (idx >= R * D) return;
@@ -505,11 +526,11 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_scalar_kernel(
     const float bs = bias != nullptr ? bias[d] : 0.0f;
     const float *pin = conv_in + row * conv_in_stride + d;
     float p0 = pin[0], p1 = pin[D], p2 = pin[2 * D];
-    const BT *bp = b1 + row * rs + d;
+    const BT *bp = b1 + placed_row(row, b_group, b_pitch) * rs + d;
     const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
     int hist = 3;
     for (int t = 0; t < T; ++t) {
-        const float cur = load1(bp + t * ts);
+        const float cur = load1(bp + t * ts_b);
         if (dn != nullptr && t > 0 && dn[t - 1]) hist = 0;
         float acc = (hist >= 3 ? p0 : 0.0f) * w0;
         acc += (hist >= 2 ? p1 : 0.0f) * w1;
@@ -533,9 +554,10 @@ template <typename BT>
 static int launch_conv_seq(const void *b1, const float *conv_in, int64_t conv_in_stride, const float *weight,
                            const float *bias, const uint8_t *done, float *v_out, uint16_t *v_bf16_out,
                            float *conv_out, int64_t conv_out_stride, int64_t R, int T, int D, int time_major,
-                           hipStream_t stream)
+                           int b_group, int b_pitch, hipStream_t stream)
 {
     const int64_t rs = time_major ? D : (int64_t)T * D, ts = time_major ? R * D : D;
+    const int64_t ts_b = b_group > 0 ? R / b_group * b_pitch * D : ts;
     const bool vec_ok = (D % 8 == 0) && (D / 8 <= kSeqThreads) && aligned16(b1) && aligned16(conv_in) &&
                         aligned16(conv_out) && aligned16(v_out) && aligned16(v_bf16_out) && aligned16(weight) &&
                         (conv_in_stride % 4 == 0) && (conv_out_stride % 4 == 0);
@@ -546,13 +568,13 @@ static int launch_conv_seq(const void *b1, const float *conv_in, int64_t conv_in
         if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
         hipLaunchKernelGGL((conv_seq_vec8_kernel<BT>), dim3((unsigned)blocks), dim3(kSeqThreads), 0, stream,
                            (const BT *)b1, conv_in, conv_in_stride, weight, bias, done, v_out, v_bf16_out, conv_out,
-                           conv_out_stride, R, T, D, rs, ts, rows_per_block);
+                           conv_out_stride, R, T, D, rs, ts, rows_per_block, b_group, b_pitch, ts_b);
     } else {
         const int64_t blocks = (R * D + kSeqThreads - 1) / kSeqThreads;
         if (blocks > 0x7fffffffLL) return BNB_ERR_UNSUPPORTED;
         hipLaunchKernelGGL((conv_seq_scalar_kernel<BT>), dim3((unsigned)blocks), dim3(kSeqThreads), 0, stream,
                            (const BT *)b1, conv_in, conv_in_stride, weight, bias, done, v_out, v_bf16_out, conv_out,
-                           conv_out_stride, R, T, D, rs, ts);
+                           conv_out_stride, R, T, D, rs, ts, b_group, b_pitch, ts_b);
     }
     return (int)hipGetLastError();
 }
@@ -578,7 +600,7 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_bwd_kernel(
     const BT *__restrict__ b1, const float *__restrict__ conv_in, int64_t conv_in_stride, const float *__restrict__ weight,
     const uint8_t *__restrict__ done, const float *__restrict__ dv, const uint16_t *__restrict__ dv_lp,
     const float *__restrict__ dconv_out, BT *__restrict__ db1, float *__restrict__ dconv_in, float *__restrict__ partials,
-    int64_t R, int T, int D, int64_t rs, int64_t ts, int chunks, int64_t items)
+    int64_t R, int T, int D, int64_t rs, int64_t ts, int chunks, int64_t items, int b_group, int b_pitch, int64_t ts_b)
 {
     __shared__ float s_red[kSeqThreads * 8];
     const int vecs = D >> 3;
@@ -604,7 +626,8 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_bwd_kernel(
         if (row >= R) continue;
         const float *dvp = dv + row * rs + d0;
         const uint16_t *dlp = dv_lp == nullptr ? nullptr : dv_lp + row * rs + d0;
-        const BT *bp = b1 + row * rs + d0;
+        const int64_t at_b = placed_row(row, b_group, b_pitch) * rs;  // b1 and db1: possibly rows of a wider token tensor
+        const BT *bp = b1 + at_b + d0;
         const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
         // the output's gradient: the float32 part plus, when the output also went out in bfloat16, that copy's
         auto grad_row = [&](int t) -> Row8 {
@@ -632,7 +655,7 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_bwd_kernel(
                 if (s < 0)
                     in[u] = load8_split<false>(conv_in + row * conv_in_stride + (int64_t)(s + 3) * D + d0, gap);
                 else
-                    in[u] = s < T ? load8_split<true>(bp + s * ts, gap) : zero;
+                    in[u] = s < T ? load8_split<true>(bp + s * ts_b, gap) : zero;
             }
 #pragma unroll
             for (int u = 0; u < kSeqAhead; ++u) {
@@ -662,7 +685,7 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_bwd_kernel(
                     if (s < 0)
                         store8_split<false>(dconv_in + row * 3 * (int64_t)D + (int64_t)(s + 3) * D + d0, gap, o);
                     else
-                        store8_split<true>(db1 + row * rs + s * ts + d0, gap, o);
+                        store8_split<true>(db1 + at_b + s * ts_b + d0, gap, o);
                     g0 = g1, g1 = g2, g2 = g3;
                     f0 = f1, f1 = f2;
                 }
@@ -691,18 +714,28 @@ template <typename BT>
 static int launch_conv_seq_bwd(const void *b1, const float *conv_in, int64_t conv_in_stride, const float *weight,
                                const uint8_t *done, const float *dv, const uint16_t *dv_lp, const float *dconv_out, void *db1,
                                float *dconv_in, float *partials, int blocks, float *dwb, int64_t R, int T, int D,
-                               int time_major, hipStream_t stream)
+                               int time_major, int b_group, int b_pitch, hipStream_t stream)
 {
     const int64_t rs = time_major ? D : (int64_t)T * D, ts = time_major ? R * D : D;
+    const int64_t ts_b = b_group > 0 ? R / b_group * b_pitch * D : ts;
     const int rows_per_block = kSeqThreads / (D / 8);
     const int chunks = (T + (kSeqTaps - 1) + kCbChunk - 1) / kCbChunk;
     const int64_t items = (R + rows_per_block - 1) / rows_per_block * chunks;
     hipLaunchKernelGGL((conv_seq_bwd_kernel<BT>), dim3((unsigned)blocks), dim3(kSeqThreads), 0, stream, (const BT *)b1, conv_in,
                        conv_in_stride, weight, done, dv, dv_lp, dconv_out, (BT *)db1, dconv_in, partials, R, T, D, rs, ts, chunks,
-                       items);
+                       items, b_group, b_pitch, ts_b);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
     return launch_sum_slices(partials, dwb, 5 * (int64_t)D, blocks, 0, stream);
+}
+
+// rows_per_env / env_row_pitch of the entry points below: both zero, or a time-major call whose rows are the first
+// rows_per_env of every env_row_pitch rows of a wider tensor
+static int check_token_rows(int64_t R, int time_major, int rows_per_env, int env_row_pitch)
+{
+    if (rows_per_env == 0 && env_row_pitch == 0) return 0;
+    if (rows_per_env < 1 || env_row_pitch < rows_per_env || !time_major || R % rows_per_env != 0) return BNB_ERR_BAD_SHAPE;
+    return 0;
 }
 
 }  // namespace bnb
@@ -710,10 +743,12 @@ static int launch_conv_seq_bwd(const void *b1, const float *conv_in, int64_t con
 extern "C" int bnb_rglru_scan_fwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
                                   const float *log_lambda, float c, const float *h0, int64_t h0_row_stride,
                                   const uint8_t *done, void *y, int y_dtype, float *h_last,
-                                  int64_t h_last_row_stride, int64_t R, int T, int D, int time_major, void *stream)
+                                  int64_t h_last_row_stride, int64_t R, int T, int D, int time_major, int rows_per_env,
+                                  int env_row_pitch, void *stream)
 {
     using namespace bnb;
     if (R < 0 || T < 0 || D < 1) return BNB_ERR_BAD_SHAPE;
+    if (check_token_rows(R, time_major, rows_per_env, env_row_pitch)) return BNB_ERR_BAD_SHAPE;
     if (R == 0) return 0;
     if (!log_lambda || !h0 || !h_last) return BNB_ERR_NULL_POINTER;
     if (h0_row_stride < D || h_last_row_stride < D) return BNB_ERR_BAD_SHAPE;
@@ -734,15 +769,15 @@ extern "C" int bnb_rglru_scan_fwd(const void *x, int x_dtype, const void *gates_
     const bool xb = x_dtype == BNB_BF16, gb = g_dtype == BNB_BF16;
     if (!xb && !gb)
         return scan_dispatch_y<float, float>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype, h_last,
-                                             h_last_row_stride, R, T, D, time_major != 0, s);
+                                             h_last_row_stride, R, T, D, time_major != 0, rows_per_env, env_row_pitch, s);
     if (xb && gb)
         return scan_dispatch_y<uint16_t, uint16_t>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype,
-                                                   h_last, h_last_row_stride, R, T, D, time_major != 0, s);
+                                                   h_last, h_last_row_stride, R, T, D, time_major != 0, rows_per_env, env_row_pitch, s);
     if (!xb && gb)
         return scan_dispatch_y<float, uint16_t>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype,
-                                                h_last, h_last_row_stride, R, T, D, time_major != 0, s);
+                                                h_last, h_last_row_stride, R, T, D, time_major != 0, rows_per_env, env_row_pitch, s);
     return scan_dispatch_y<uint16_t, float>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype, h_last,
-                                            h_last_row_stride, R, T, D, time_major != 0, s);
+                                            h_last_row_stride, R, T, D, time_major != 0, rows_per_env, env_row_pitch, s);
 }
 
 extern "C" int bnb_rglru_scan_bwd(const void *x, int x_dtype, const void *gates_pre, int g_dtype,
@@ -750,10 +785,11 @@ extern "C" int bnb_rglru_scan_bwd(const void *x, int x_dtype, const void *gates_
                                   const uint8_t *done, const void *y, int y_dtype, const void *dy,
                                   const float *dh_last, int64_t dh_last_row_stride, void *dx, void *dgates,
                                   float *dh0, float *dlam_rows, int64_t R, int T, int D, int time_major,
-                                  void *stream)
+                                  int rows_per_env, int env_row_pitch, void *stream)
 {
     using namespace bnb;
     if (R < 0 || T < 1 || D < 1) return BNB_ERR_BAD_SHAPE;
+    if (check_token_rows(R, time_major, rows_per_env, env_row_pitch)) return BNB_ERR_BAD_SHAPE;
     if (R == 0) return 0;
     if (!x || !gates_pre || !log_lambda || !h0 || !y || !dx || !dgates || !dh0 || !dlam_rows)
         return BNB_ERR_NULL_POINTER;
@@ -769,27 +805,28 @@ extern "C" int bnb_rglru_scan_bwd(const void *x, int x_dtype, const void *gates_
     if (!xb && !gb)
         return scan_bwd_dispatch_y<float, float>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype, dy,
                                                  dh_last, dh_last_row_stride, dx, dgates, dh0, dlam_rows, R, T, D,
-                                                 time_major != 0, s);
+                                                 time_major != 0, rows_per_env, env_row_pitch, s);
     if (xb && gb)
         return scan_bwd_dispatch_y<uint16_t, uint16_t>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y,
                                                        y_dtype, dy, dh_last, dh_last_row_stride, dx, dgates, dh0,
-                                                       dlam_rows, R, T, D, time_major != 0, s);
+                                                       dlam_rows, R, T, D, time_major != 0, rows_per_env, env_row_pitch, s);
     if (!xb && gb)
         return scan_bwd_dispatch_y<float, uint16_t>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype,
                                                     dy, dh_last, dh_last_row_stride, dx, dgates, dh0, dlam_rows, R, T,
-                                                    D, time_major != 0, s);
+                                                    D, time_major != 0, rows_per_env, env_row_pitch, s);
     return scan_bwd_dispatch_y<uint16_t, float>(x, gates_pre, log_lambda, c, h0, h0_row_stride, done, y, y_dtype, dy,
                                                 dh_last, dh_last_row_stride, dx, dgates, dh0, dlam_rows, R, T, D,
-                                                time_major != 0, s);
+                                                time_major != 0, rows_per_env, env_row_pitch, s);
 }
 
 extern "C" int bnb_conv_seq_fwd(const void *b1, int b1_dtype, const float *conv_in, int64_t conv_in_row_stride,
                                 const float *weight, const float *bias, const uint8_t *done, float *v_out,
                                 void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride, int64_t R, int T,
-                                int D, int time_major, void *stream)
+                                int D, int time_major, int rows_per_env, int env_row_pitch, void *stream)
 {
     using namespace bnb;
     if (R < 0 || T < 1 || D < 1) return BNB_ERR_BAD_SHAPE;
+    if (check_token_rows(R, time_major, rows_per_env, env_row_pitch)) return BNB_ERR_BAD_SHAPE;
     if (R == 0) return 0;
     if (!b1 || !conv_in || !weight || !v_out || !conv_out) return BNB_ERR_NULL_POINTER;
     if (b1_dtype != BNB_F32 && b1_dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
@@ -801,9 +838,10 @@ extern "C" int bnb_conv_seq_fwd(const void *b1, int b1_dtype, const float *conv_
     hipStream_t s = (hipStream_t)stream;
     if (b1_dtype == BNB_BF16)
         return launch_conv_seq<uint16_t>(b1, conv_in, conv_in_row_stride, weight, bias, done, v_out,
-                                         (uint16_t *)v_bf16_out, conv_out, conv_out_row_stride, R, T, D, time_major != 0, s);
+                                         (uint16_t *)v_bf16_out, conv_out, conv_out_row_stride, R, T, D, time_major != 0,
+                                         rows_per_env, env_row_pitch, s);
     return launch_conv_seq<float>(b1, conv_in, conv_in_row_stride, weight, bias, done, v_out, (uint16_t *)v_bf16_out,
-                                  conv_out, conv_out_row_stride, R, T, D, time_major != 0, s);
+                                  conv_out, conv_out_row_stride, R, T, D, time_major != 0, rows_per_env, env_row_pitch, s);
 }
 
 extern "C" int bnb_conv_seq_bwd_blocks(int64_t R, int T, int D)
@@ -817,10 +855,11 @@ extern "C" int bnb_conv_seq_bwd_blocks(int64_t R, int T, int D)
 extern "C" int bnb_conv_seq_bwd(const void *b1, int b1_dtype, const float *conv_in, int64_t conv_in_row_stride,
                                 const float *weight, const uint8_t *done, const float *dv, const void *dv_bf16,
                                 const float *dconv_out, void *db1, float *dconv_in, float *partials, int blocks, float *dwb,
-                                int64_t R, int T, int D, int time_major, void *stream)
+                                int64_t R, int T, int D, int time_major, int rows_per_env, int env_row_pitch, void *stream)
 {
     using namespace bnb;
     if (R < 0 || T < 1 || D < 1) return BNB_ERR_BAD_SHAPE;
+    if (check_token_rows(R, time_major, rows_per_env, env_row_pitch)) return BNB_ERR_BAD_SHAPE;
     if (D != 64 && D != 128 && D != 256 && D != 512) return BNB_ERR_UNSUPPORTED;
     if (b1_dtype != BNB_F32 && b1_dtype != BNB_BF16) return BNB_ERR_BAD_DTYPE;
     if (!weight || !partials || !dwb || (R > 0 && (!b1 || !conv_in || !dv || !db1 || !dconv_in))) return BNB_ERR_NULL_POINTER;
@@ -834,7 +873,9 @@ extern "C" int bnb_conv_seq_bwd(const void *b1, int b1_dtype, const float *conv_
     if (R == 0) return launch_sum_slices(partials, dwb, 5 * (int64_t)D, 0, 0, s);
     if (b1_dtype == BNB_BF16)
         return launch_conv_seq_bwd<uint16_t>(b1, conv_in, conv_in_row_stride, weight, done, dv, (const uint16_t *)dv_bf16,
-                                             dconv_out, db1, dconv_in, partials, blocks, dwb, R, T, D, time_major != 0, s);
+                                             dconv_out, db1, dconv_in, partials, blocks, dwb, R, T, D, time_major != 0,
+                                             rows_per_env, env_row_pitch, s);
     return launch_conv_seq_bwd<float>(b1, conv_in, conv_in_row_stride, weight, done, dv, (const uint16_t *)dv_bf16, dconv_out,
-                                      db1, dconv_in, partials, blocks, dwb, R, T, D, time_major != 0, s);
+                                      db1, dconv_in, partials, blocks, dwb, R, T, D, time_major != 0, rows_per_env,
+                                      env_row_pitch, s);
 }

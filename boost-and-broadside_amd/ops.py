@@ -1159,6 +1159,19 @@ def _done_pointer(done, R, T, device):
     return done, done.data_ptr()
 
 
+def _token_rows(t: torch.Tensor, token_rows: int | None, time_major: bool, name: str):
+    """``(rows_per_env, env_row_pitch, dense shape)`` of a kernel operand that may be a (T, B, NM, D) token tensor of
+    which a call covers the first ``token_rows`` tokens per environment; (0, 0, t.shape) for a plain operand."""
+    if token_rows is None:
+        return 0, 0, tuple(t.shape)
+    if not time_major or t.dim() != 4 or not 1 <= token_rows <= t.shape[2]:
+        raise ValueError(f"token_rows needs time_major and a (T, B, NM, D) {name} with NM >= token_rows, got {tuple(t.shape)}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous when token_rows is given")
+    T, B, NM, D = t.shape
+    return int(token_rows), int(NM), (T, B * token_rows, D)
+
+
 def conv_seq(
     b1: torch.Tensor,
     conv_buf: torch.Tensor,
@@ -1169,6 +1182,7 @@ def conv_seq(
     conv_out: torch.Tensor | None = None,
     also_bf16: bool = False,
     time_major: bool = False,
+    token_rows: int | None = None,
 ):
     """Causal depthwise conv over a sequence, taps cut at episode ends (griffin.py:67-140).
 
@@ -1181,14 +1195,18 @@ def conv_seq(
         also_bf16: also return a bfloat16 copy of the conv output.
         time_major: ``b1`` and the returned conv output are (T, R, D) instead of (R, T, D);
                   ``done`` stays (R, T).
+        token_rows: with ``time_major``, ``b1`` is a (T, B, NM, D) token tensor and the conv runs over its first
+                  ``token_rows`` tokens of every environment, read where they lie (R = B * token_rows, env-major);
+                  the outputs are dense, (T, R, D).
 
     Returns:
         (v, new_conv_buf[, v_bf16]): conv output (R, T, D) float32 and the last three entries
         of ``[conv_buf, b1]``.
     """
-    if b1.dim() != 3 or conv_buf.dim() != 3:
+    group, pitch, v_shape = _token_rows(b1, token_rows, time_major, "b1")
+    if (b1.dim() != 3 and not group) or conv_buf.dim() != 3:
         raise ValueError("b1 must be (R, T, D) and conv_buf (R, 3, D)")
-    R, T, D = b1.shape
+    R, T, D = v_shape
     if time_major:
         T, R = R, T
     if T < 1:
@@ -1218,15 +1236,15 @@ def conv_seq(
         conv_out = torch.empty((R, 3, D), dtype=torch.float32, device=b1.device)
     elif conv_out.shape != (R, 3, D) or conv_out.dtype != torch.float32 or conv_out.device != b1.device or not rows_ok(conv_out):
         raise ValueError("conv_out must be a float32 (R, 3, D) tensor on b1's device with contiguous rows")
-    v = torch.empty(b1.shape, dtype=torch.float32, device=b1.device)
-    v_lp = torch.empty(b1.shape, dtype=torch.bfloat16, device=b1.device) if also_bf16 else None
+    v = torch.empty(v_shape, dtype=torch.float32, device=b1.device)
+    v_lp = torch.empty(v_shape, dtype=torch.bfloat16, device=b1.device) if also_bf16 else None
     keep, done_ptr = _done_pointer(done, R, T, b1.device)
     if R:
         with _on_device(b1.device):
             rc = _native.load().bnb_conv_seq_fwd(
                 b1.data_ptr(), b_code, conv_buf.data_ptr(), conv_buf.stride(0), weight.data_ptr(), bias_ptr, done_ptr,
                 v.data_ptr(), None if v_lp is None else v_lp.data_ptr(), conv_out.data_ptr(), conv_out.stride(0),
-                R, T, D, int(time_major), _stream(),
+                R, T, D, int(time_major), group, pitch, _stream(),
             )
         _native.check(rc, "bnb_conv_seq_fwd")
     del keep
@@ -1236,26 +1254,32 @@ def conv_seq(
 _CONV_TRAIN_WIDTHS = (64, 128, 256, 512)
 
 
-def conv_seq_bwd(b1, conv_buf, weight, done, dv, dconv_out=None, *, time_major: bool = False, dv_bf16=None):
+def conv_seq_bwd(b1, conv_buf, weight, done, dv, dconv_out=None, *, time_major: bool = False, dv_bf16=None,
+                 token_rows: int | None = None, db1_out: torch.Tensor | None = None):
     """Backward of ``conv_seq``: returns ``(db1, dconv_buf, dweight (D, 4), dbias (D,))``.
 
     ``dv`` is the float32 gradient of the conv output (b1's layout), ``dconv_out`` the optional
     gradient of the returned stored inputs, ``dv_bf16`` the optional gradient of the output's bfloat16
-    copy (added to ``dv`` in the kernel); ``db1`` has b1's dtype.  Sums run in a fixed order."""
-    R, T, D = b1.shape
+    copy (added to ``dv`` in the kernel); ``db1`` has b1's dtype.  Sums run in a fixed order.
+
+    ``token_rows`` as in ``conv_seq``: b1 is a (T, B, NM, D) token tensor, ``dv`` dense (T, B * token_rows, D), and
+    ``db1`` is a token tensor like b1 (``db1_out`` if given) in which ONLY the first ``token_rows`` tokens of every
+    environment are written."""
+    group, pitch, v_shape = _token_rows(b1, token_rows, time_major, "b1")
+    R, T, D = v_shape
     if time_major:
         T, R = R, T
     if D not in _CONV_TRAIN_WIDTHS:
         raise ValueError(f"conv_seq_bwd supports D in {_CONV_TRAIN_WIDTHS}, got {D}")
-    if dv.shape != b1.shape or dv.dtype != torch.float32:
-        raise ValueError("dv must be float32 with b1's shape")
+    if tuple(dv.shape) != v_shape or dv.dtype != torch.float32:
+        raise ValueError("dv must be float32 with the conv output's shape")
     for name, t in (("b1", b1), ("conv_buf", conv_buf), ("weight", weight), ("dv", dv)):
         _need_device(t, name)
     b1 = b1.contiguous()
     dv = dv.contiguous()
     if dv_bf16 is not None:
-        if dv_bf16.shape != b1.shape or dv_bf16.dtype != torch.bfloat16:
-            raise ValueError("dv_bf16 must be bfloat16 with b1's shape")
+        if tuple(dv_bf16.shape) != v_shape or dv_bf16.dtype != torch.bfloat16:
+            raise ValueError("dv_bf16 must be bfloat16 with the conv output's shape")
         _need_device(dv_bf16, "dv_bf16")
         dv_bf16 = dv_bf16.contiguous()
     conv_buf = conv_buf if (R == 0 or (conv_buf.stride(2) == 1 and conv_buf.stride(1) == D)) else conv_buf.contiguous()
@@ -1264,7 +1288,12 @@ def conv_seq_bwd(b1, conv_buf, weight, done, dv, dconv_out=None, *, time_major: 
         if dconv_out.shape != (R, 3, D):
             raise ValueError(f"dconv_out must be {(R, 3, D)}")
         dconv_out = dconv_out.to(torch.float32).contiguous()
-    db1 = torch.empty_like(b1)
+    if db1_out is None:
+        db1 = torch.empty_like(b1)
+    elif db1_out.shape != b1.shape or db1_out.dtype != b1.dtype or db1_out.device != b1.device or not db1_out.is_contiguous():
+        raise ValueError("db1_out must be a contiguous tensor like b1")
+    else:
+        db1 = db1_out
     dconv = torch.empty((R, 3, D), dtype=torch.float32, device=b1.device)
     dwb = torch.empty((5 * D,), dtype=torch.float32, device=b1.device)
     lib = _native.load()
@@ -1275,7 +1304,7 @@ def conv_seq_bwd(b1, conv_buf, weight, done, dv, dconv_out=None, *, time_major: 
         rc = lib.bnb_conv_seq_bwd(b1.data_ptr(), _code(b1, "b1"), conv_buf.data_ptr(), conv_buf.stride(0) if R else 3 * D,
                                   weight.data_ptr(), done_ptr, dv.data_ptr(), None if dv_bf16 is None else dv_bf16.data_ptr(),
                                   None if dconv_out is None else dconv_out.data_ptr(), db1.data_ptr(), dconv.data_ptr(),
-                                  partials.data_ptr(), blocks, dwb.data_ptr(), R, T, D, int(time_major), _stream())
+                                  partials.data_ptr(), blocks, dwb.data_ptr(), R, T, D, int(time_major), group, pitch, _stream())
     _native.check(rc, "bnb_conv_seq_bwd")
     del keep
     return db1, dconv, dwb[:4 * D].view(D, 4), dwb[4 * D:]
@@ -1331,6 +1360,7 @@ def rglru_scan(
     y_dtype: torch.dtype = torch.float32,
     h_out: torch.Tensor | None = None,
     time_major: bool = False,
+    y_tokens: tuple[torch.Tensor, int] | None = None,
 ):
     """RG-LRU over a whole sequence in one pass (griffin.py:188-219 without the log-depth scan).
 
@@ -1344,6 +1374,9 @@ def rglru_scan(
         h_out:      optional (R, D) float32 destination of the final state.
         time_major: ``x``, ``gates_pre`` and the returned states are (T, R, .) instead of
                     (R, T, .); ``done`` stays (R, T).
+        y_tokens:   ``(tokens, n)``: with ``time_major`` and no gradient, the states go into the first ``n`` tokens of
+                    every environment of the (T, B, NM, D) tensor ``tokens`` (R = B * n, env-major), which is returned
+                    in place of ``y``; its other tokens are left alone.
 
     Returns:
         (y, h_last): all states (R, T, D) in ``y_dtype`` and the final state (R, D) float32.
@@ -1365,7 +1398,7 @@ def rglru_scan(
         raise TypeError(f"y_dtype must be float32 or bfloat16, got {y_dtype}")
     if torch.is_grad_enabled() and (x.requires_grad or gates_pre.requires_grad or h0.requires_grad or log_lambda.requires_grad):
         # training: forward and backward kernels behind autograd
-        if y_dtype != torch.float32 or h_out is not None:
+        if y_dtype != torch.float32 or h_out is not None or y_tokens is not None:
             raise RuntimeError("rglru_scan under autograd returns float32 states and owns its outputs")
         keep, _ = _done_pointer(done, R, T, x.device)
         return _RglruScan.apply(x, gates_pre, log_lambda, h0, keep, float(c), bool(time_major))
@@ -1379,14 +1412,21 @@ def rglru_scan(
         h_out = torch.empty((R, D), dtype=torch.float32, device=x.device)
     elif h_out.shape != (R, D) or h_out.dtype != torch.float32 or h_out.device != x.device or (R and h_out.stride(1) != 1):
         raise ValueError("h_out must be a float32 (R, D) tensor on x's device with contiguous rows")
-    y = torch.empty(x.shape, dtype=y_dtype, device=x.device)
+    group = pitch = 0
+    if y_tokens is None:
+        y = torch.empty(x.shape, dtype=y_dtype, device=x.device)
+    else:
+        y, n = y_tokens
+        group, pitch, dense = _token_rows(y, n, time_major, "y_tokens[0]")
+        if dense != tuple(x.shape) or y.dtype != y_dtype or y.device != x.device:
+            raise ValueError(f"y_tokens must hold {tuple(x.shape)} {y_dtype} states on x's device")
     keep, done_ptr = _done_pointer(done, R, T, x.device)
     if R:
         with _on_device(x.device):
             rc = _native.load().bnb_rglru_scan_fwd(
                 x.data_ptr(), x_code, gates_pre.data_ptr(), g_code, log_lambda.data_ptr(), float(c), h0.data_ptr(),
                 h0.stride(0), done_ptr, y.data_ptr(), _DTYPE_CODE[y_dtype], h_out.data_ptr(), h_out.stride(0),
-                R, T, D, int(time_major), _stream(),
+                R, T, D, int(time_major), group, pitch, _stream(),
             )
         _native.check(rc, "bnb_rglru_scan_fwd")
     del keep
@@ -1410,27 +1450,134 @@ class _RglruScan(torch.autograd.Function):
     @_outside_autocast
     def backward(ctx, dy, dh_last):
         x, gates_pre, log_lambda, h0, y = ctx.saved_tensors
-        T, R = (x.shape[0], x.shape[1]) if ctx.time_major else (x.shape[1], x.shape[0])
-        D = x.shape[2]
-        x_c, g_c = x.contiguous(), gates_pre.contiguous()
-        h0_c = h0 if h0.stride(1) == 1 else h0.contiguous()
-        # the kernel reads dy in y's dtype and dh_last as float32; an output nobody differentiated arrives as None
-        dy = torch.zeros_like(y) if dy is None else dy.to(y.dtype).contiguous()
-        dh_last = torch.zeros((R, D), dtype=torch.float32, device=x.device) if dh_last is None else dh_last.float().contiguous()
-        dx = torch.empty_like(x_c)
-        dgates = torch.empty_like(g_c)
-        dh0 = torch.empty((R, D), dtype=torch.float32, device=x.device)
-        dlam_rows = torch.empty((R, D), dtype=torch.float32, device=x.device)
-        done_ptr = None if ctx.done is None else ctx.done.data_ptr()
+        dx, dgates, dh0, dlam_rows = rglru_scan_bwd(x, gates_pre, log_lambda, ctx.c, h0, ctx.done, y, dy, dh_last,
+                                                    time_major=ctx.time_major)
+        return dx, dgates, dlam_rows.sum(dim=0), dh0, None, None, None
+
+
+def rglru_scan_bwd(x, gates_pre, log_lambda, c, h0, done, y, dy, dh_last=None, *, time_major: bool = False,
+                   token_rows: int | None = None):
+    """Backward of ``rglru_scan``: ``(dx, dgates, dh0, dlog_lambda per row (R, D))`` from the saved inputs, the saved
+    states ``y`` and the gradients of the states (``dy``, in y's dtype; None = zero) and of the final state.
+
+    ``done`` is the (R, T) uint8/bool tensor the forward saw, or None.  ``token_rows``: with ``time_major``, ``y`` and
+    ``dy`` are (T, B, NM, D) token tensors whose first ``token_rows`` tokens per environment are this call's rows."""
+    group, pitch, dense = _token_rows(y, token_rows, time_major, "y")
+    if dense != tuple(x.shape) or (dy is not None and dy.shape != y.shape):
+        raise ValueError("y (and dy) must hold x's rows")
+    T, R = (x.shape[0], x.shape[1]) if time_major else (x.shape[1], x.shape[0])
+    D = x.shape[2]
+    x_c, g_c = x.contiguous(), gates_pre.contiguous()
+    h0_c = h0 if h0.stride(1) == 1 else h0.contiguous()
+    y = y.contiguous()
+    # the kernel reads dy in y's dtype and dh_last as float32; a gradient nobody produced arrives as None
+    if dy is not None:
+        dy = dy.to(y.dtype).contiguous()
+    elif group:
+        raise ValueError("dy is required with token_rows")
+    else:
+        dy = torch.zeros_like(y)
+    if dh_last is not None:
+        dh_last = dh_last.float().contiguous()
+    dx = torch.empty_like(x_c)
+    dgates = torch.empty_like(g_c)
+    dh0 = torch.empty((R, D), dtype=torch.float32, device=x.device)
+    dlam_rows = torch.empty((R, D), dtype=torch.float32, device=x.device)
+    keep, done_ptr = _done_pointer(done, R, T, x.device)
+    if R:
         with _on_device(x.device):
             rc = _native.load().bnb_rglru_scan_bwd(
                 x_c.data_ptr(), _DTYPE_CODE[x.dtype], g_c.data_ptr(), _DTYPE_CODE[gates_pre.dtype],
-                log_lambda.data_ptr(), ctx.c, h0_c.data_ptr(), h0_c.stride(0), done_ptr, y.data_ptr(),
-                _DTYPE_CODE[y.dtype], dy.data_ptr(), dh_last.data_ptr(), dh_last.stride(0), dx.data_ptr(),
-                dgates.data_ptr(), dh0.data_ptr(), dlam_rows.data_ptr(), R, T, D, int(ctx.time_major), _stream(),
+                log_lambda.detach().contiguous().data_ptr(), float(c), h0_c.data_ptr(), h0_c.stride(0), done_ptr, y.data_ptr(),
+                _DTYPE_CODE[y.dtype], dy.data_ptr(), None if dh_last is None else dh_last.data_ptr(),
+                0 if dh_last is None else dh_last.stride(0), dx.data_ptr(), dgates.data_ptr(), dh0.data_ptr(),
+                dlam_rows.data_ptr(), R, T, D, int(time_major), group, pitch, _stream(),
             )
         _native.check(rc, "bnb_rglru_scan_bwd")
-        return dx, dgates, dlam_rows.sum(dim=0), dh0, None, None, None
+    else:
+        dlam_rows.zero_()
+    del keep
+    return dx, dgates, dh0, dlam_rows
+
+
+class _TemporalMixTrain(torch.autograd.Function):
+    """The middle of the temporal sublayer over a stored rollout's (T, B, NM, D) bfloat16 token tensor ``b1`` (the
+    ``linear1`` outputs), as the update runs it under bfloat16 autocast: causal conv, the two gate projections and the
+    RG-LRU over the first ``n`` tokens of every environment (griffin.py:267-283), a bias-free Linear ``field_w`` over
+    the others (griffin.py:406-413), both results in ONE float32 (T, B, NM, D) tensor.
+
+    The reference slices the tokens, runs the two branches and concatenates; here the conv and scan kernels read and
+    write the ship rows where they lie in the token tensors (forward and backward), so neither the split, nor the
+    concatenation, nor their backward copies exist.  Values and gradients equal those of the separate steps
+    (``conv_seq_train`` with its bfloat16 copy, ``linear_train``, ``rglru_scan``, ``linear_train``, ``torch.cat``)."""
+
+    @staticmethod
+    def forward(ctx, b1, n, conv_buf, conv_w, conv_b, gate_w, gate_b, log_lambda, c, h0, done, field_w):
+        T, B, NM, D = b1.shape
+        bf16 = torch.bfloat16
+        with torch.no_grad():
+            v, new_buf, v_lp = conv_seq(b1, conv_buf, conv_w, conv_b, done, also_bf16=True, time_major=True, token_rows=n)
+            wb = gate_w.to(bf16)
+            gates = torch.nn.functional.linear(v_lp.view(-1, D), wb, gate_b.to(bf16)).view(T, B * n, 2 * D)
+            y = torch.empty((T, B, NM, D), dtype=torch.float32, device=b1.device)
+            _, h_last = rglru_scan(v, gates, log_lambda, c, h0, done, time_major=True, y_tokens=(y, n))
+            fields = b1[:, :, n:].contiguous()
+            fw = field_w.to(bf16)
+            y[:, :, n:].copy_(torch.nn.functional.linear(fields, fw))  # bfloat16 values are exact in float32
+        ctx.save_for_backward(b1, conv_buf, conv_w, wb, log_lambda, h0, v, v_lp, gates, y, fields, fw)
+        ctx.set_materialize_grads(False)
+        ctx.n, ctx.c, ctx.done = n, c, done
+        ctx.conv_w_shape = conv_w.shape
+        ctx.has_conv_bias = conv_b is not None
+        return y, h_last, new_buf
+
+    @staticmethod
+    @_outside_autocast
+    def backward(ctx, dy, dh_last, dbuf):
+        b1, conv_buf, conv_w, wb, log_lambda, h0, v, v_lp, gates, y, fields, fw = ctx.saved_tensors
+        T, B, NM, D = b1.shape
+        n = ctx.n
+        bf16 = torch.bfloat16
+        dy = torch.zeros_like(y) if dy is None else dy.float().contiguous()
+        dx, dgates, dh0, dlam_rows = rglru_scan_bwd(v, gates, log_lambda, ctx.c, h0, ctx.done, y, dy, dh_last, time_major=True,
+                                                    token_rows=n)
+        dg = dgates.view(-1, 2 * D)
+        dv_lp = torch.matmul(dg, wb).view(T, B * n, D)
+        d_gate_w = linear_wgrad(dg, v_lp.view(-1, D)) if ctx.needs_input_grad[5] else None
+        d_gate_b = None
+        if ctx.needs_input_grad[6]:
+            d_gate_b = column_sums(dg) if column_sums_supported(dg) else dg.sum(dim=0, dtype=torch.float32)
+        db1 = torch.empty_like(b1)
+        _, dconv, dw, db = conv_seq_bwd(b1, conv_buf, conv_w, ctx.done, dx, dbuf, time_major=True, dv_bf16=dv_lp, token_rows=n,
+                                        db1_out=db1)
+        # the other tokens: one strided read of their gradient (rounded to bfloat16, as a bfloat16 Linear receives it),
+        # the input-gradient GEMM, one strided write into the token tensor the conv backward filled the ship rows of
+        dyf = torch.empty((T, B, NM - n, D), dtype=bf16, device=b1.device)
+        dyf.copy_(dy[:, :, n:])
+        db1[:, :, n:].copy_(torch.matmul(dyf.view(-1, D), fw).view(T, B, NM - n, D))
+        d_field_w = linear_wgrad(dyf.view(-1, D), fields.view(-1, D)) if ctx.needs_input_grad[11] else None
+        return (db1, None, dconv, dw.reshape(ctx.conv_w_shape), db if ctx.has_conv_bias else None, d_gate_w, d_gate_b,
+                dlam_rows.sum(dim=0), None, dh0, None, d_field_w)
+
+
+def temporal_mix_train_supported(b1: torch.Tensor, n: int, gate_w: torch.Tensor, field_w: torch.Tensor) -> bool:
+    """Whether ``temporal_mix_train`` covers this token tensor: bfloat16 (T, B, NM, 128) on the GPU with recurrent and
+    other tokens in every environment, float32 weights of the widths the weight-gradient kernel covers."""
+    return (b1.is_cuda and b1.dim() == 4 and b1.dtype == torch.bfloat16 and b1.shape[-1] in _CONV_TRAIN_WIDTHS
+            and 0 < n < b1.shape[2] and gate_w.dtype == field_w.dtype == torch.float32
+            and linear_wgrad_supported(b1, gate_w) and linear_wgrad_supported(b1, field_w))
+
+
+def temporal_mix_train(b1, n, conv_buf, conv_weight, conv_bias, gate_weight, gate_bias, log_lambda, c, h0, done, field_weight):
+    """Differentiable conv + gate projections + RG-LRU over the first ``n`` tokens of every environment of the
+    (T, B, NM, D) bfloat16 tensor ``b1`` and ``F.linear(., field_weight)`` over the others:
+    ``(y (T, B, NM, D) float32, h_last (B*n, D), new_conv_buf (B*n, 3, D))``.
+
+    ``gate_weight`` (2D, D) and ``gate_bias`` (2D,) are ``[linear_a | linear_x]``; ``h0`` (B*n, D), ``conv_buf``
+    (B*n, 3, D) float32 and ``done`` ((B*n, T) or None) are env-major like the recurrent state."""
+    with torch.autocast("cuda", enabled=False):
+        return _TemporalMixTrain.apply(b1.contiguous(), int(n), conv_buf, conv_weight, conv_bias, gate_weight, gate_bias, log_lambda,
+                                       float(c), h0, done, field_weight)
 
 
 _F32_EPS = float(torch.finfo(torch.float32).eps)

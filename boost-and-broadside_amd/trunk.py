@@ -944,6 +944,16 @@ class GriffinTemporalBlock(_WeightCaches, nn.Module):
             b1 = _project(self.linear1, normed)
         if b1.dtype != torch.bfloat16 or b1.shape[-1] != ops.FFN_WIDTH:
             return None
+        rows = T * B * min(n_rec, NM - n_rec)
+        if (rows >= _WGRAD_MIN_ROWS and field_sub.bias is None and self.rg_lru.linear_a.bias is not None
+                and self.rg_lru.linear_x.bias is not None):
+            gate_w = torch.cat([self.rg_lru.linear_a.weight, self.rg_lru.linear_x.weight], dim=0)
+            gate_b = torch.cat([self.rg_lru.linear_a.bias, self.rg_lru.linear_x.bias], dim=0)
+            if ops.temporal_mix_train_supported(b1, n_rec, gate_w, field_sub.weight):
+                # conv, gates, recurrence (ship tokens) and field_sub (the others) read and write the token tensors in place
+                y, new_h, new_buf = ops.temporal_mix_train(b1, n_rec, conv_buf, self.conv.weight, self.conv.bias, gate_w, gate_b,
+                                                           self.rg_lru.log_lambda, self.rg_lru.c, h0, done_rows, field_sub.weight)
+                return self._finish(x, normed, y), new_h, new_buf
         ships_b1, fields_b1 = _SplitTokens.apply(b1, n_rec)
         ships_b1 = ships_b1.reshape(T, B * n_rec, D)
         if not ops.conv_seq_train_supported(ships_b1):

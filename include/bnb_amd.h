@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define BNB_ABI_VERSION 27
+#define BNB_ABI_VERSION 28
 
 /* element types of activation buffers */
 #define BNB_F32 0
@@ -568,12 +568,19 @@ int bnb_temporal_step_fwd(const void *b1, int64_t b1_group_stride, int64_t b1_ro
  *             the reference); may equal conv_in
  * Requirements: T >= 1, strides >= 3*D; vector path as for bnb_conv_step_fwd (weight 16-byte
  * aligned), scalar path otherwise.
+ *
+ * rows_per_env, env_row_pitch (both 0: b1 holds exactly the R rows): with time_major, b1 may be a wider token
+ * tensor (T, R / rows_per_env * env_row_pitch, D) of which this call's rows are the first rows_per_env of every
+ * env_row_pitch rows; the reference runs its temporal block on the ship tokens of a (ships | fields) tensor
+ * (models/yemong/policy.py: the split before the temporal sublayer), this reads them where they lie.  The
+ * outputs stay dense (R rows).  bnb_conv_seq_bwd: b1 and db1 are placed that way (db1's other rows are not written);
+ * bnb_rglru_scan_fwd: y; bnb_rglru_scan_bwd: y and dy.
  */
 int bnb_conv_seq_fwd(const void *b1, int b1_dtype,
                      const float *conv_in, int64_t conv_in_row_stride,
                      const float *weight, const float *bias, const uint8_t *done,
                      float *v_out, void *v_bf16_out, float *conv_out, int64_t conv_out_row_stride,
-                     int64_t R, int T, int D, int time_major, void *stream);
+                     int64_t R, int T, int D, int time_major, int rows_per_env, int env_row_pitch, void *stream);
 
 /*
  * Backward of bnb_conv_seq_fwd: what autograd computes through griffin.py:67-140,275-277 in the
@@ -595,7 +602,7 @@ int bnb_conv_seq_bwd_blocks(int64_t R, int T, int D);
 int bnb_conv_seq_bwd(const void *b1, int b1_dtype, const float *conv_in, int64_t conv_in_row_stride,
                      const float *weight, const uint8_t *done, const float *dv, const void *dv_bf16,
                      const float *dconv_out, void *db1, float *dconv_in, float *partials, int blocks, float *dwb,
-                     int64_t R, int T, int D, int time_major, void *stream);
+                     int64_t R, int T, int D, int time_major, int rows_per_env, int env_row_pitch, void *stream);
 
 /*
  * RG-LRU over a whole sequence: T recurrence steps per row in one pass.
@@ -621,7 +628,7 @@ int bnb_rglru_scan_fwd(const void *x, int x_dtype, const void *gates_pre, int g_
                        const float *log_lambda, float c,
                        const float *h0, int64_t h0_row_stride, const uint8_t *done,
                        void *y, int y_dtype, float *h_last, int64_t h_last_row_stride,
-                       int64_t R, int T, int D, int time_major, void *stream);
+                       int64_t R, int T, int D, int time_major, int rows_per_env, int env_row_pitch, void *stream);
 
 /*
  * Backward of bnb_rglru_scan_fwd: what autograd computes through the reference's coefficient
@@ -646,7 +653,7 @@ int bnb_rglru_scan_bwd(const void *x, int x_dtype, const void *gates_pre, int g_
                        const void *y, int y_dtype, const void *dy,
                        const float *dh_last, int64_t dh_last_row_stride,
                        void *dx, void *dgates, float *dh0, float *dlam_rows,
-                       int64_t R, int T, int D, int time_major, void *stream);
+                       int64_t R, int T, int D, int time_major, int rows_per_env, int env_row_pitch, void *stream);
 
 /*
  * Residual add + RMSNorm (+ the cast in front of the next projection) in one pass:

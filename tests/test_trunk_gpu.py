@@ -1424,6 +1424,99 @@ def test_update_path_at_the_rollouts_size_agrees_with_the_library_ops(bullets):
         assert max_rel(g, library[name]) <= BF16_TOL, name
 
 
+@pytest.mark.parametrize("N,M,with_done", [(8, 4, True), (8, 4, False), (3, 9, True)])
+def test_temporal_mix_in_place_of_split_and_concatenation_gives_the_same_bits(N, M, with_done, monkeypatch):
+    """The update's temporal sublayer reads the ship rows of the token tensor where they lie and writes its states (and
+    their gradients) back into token tensors; with that switched off the same kernels run on split copies and the
+    results are concatenated.  Same arithmetic either way: outputs, states and every gradient must be identical."""
+    from boost_and_broadside_amd import ops
+
+    cfg = _cfg(128, 4, spatial=1, temporal=1)
+    torch.manual_seed(90 + N)
+    block = bnb.YemongBlock(cfg).to(DEV)
+    T, B, D = 32, 96, 128
+    gen = torch.Generator(device=DEV).manual_seed(91)
+    x = torch.randn(T, B, N + M, D, device=DEV, generator=gen).requires_grad_()
+    alive = torch.rand(T, B, N + M, device=DEV, generator=gen) < 0.9
+    alive[..., 0] = True
+    h0 = torch.randn(1, B * N, D, device=DEV, generator=gen).requires_grad_()
+    cb0 = torch.randn(1, B * N, 3, D, device=DEV, generator=gen).requires_grad_()
+    done = (torch.rand(T, B, device=DEV, generator=gen) < 0.05) if with_done else None
+    go = torch.randn(T, B, N + M, D, device=DEV, generator=gen)
+    gh = torch.randn(1, B * N, D, device=DEV, generator=gen)
+    gc = torch.randn(1, B * N, 3, D, device=DEV, generator=gen)
+
+    used = []
+    real = ops.temporal_mix_train
+    monkeypatch.setattr(ops, "temporal_mix_train", lambda *a, **k: (used.append(1), real(*a, **k))[1])
+
+    def run():
+        block.zero_grad(set_to_none=True)
+        for t in (x, h0, cb0):
+            t.grad = None
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out, h, cb = block.sequence(x, alive, h0, cb0, done, N)
+        torch.autograd.backward([out, h, cb], [go, gh, gc])
+        found = {n: p.grad.detach().clone() for n, p in block.named_parameters() if p.grad is not None}
+        found.update(tokens=x.grad.clone(), h0=h0.grad.clone(), cb0=cb0.grad.clone(), out=out.detach().clone(),
+                     h=h.detach().clone(), cb=cb.detach().clone())
+        return found
+
+    in_place = run()
+    assert used, "the token-tensor form did not run"
+    n_used = len(used)
+    monkeypatch.setattr(ops, "temporal_mix_train_supported", lambda *a, **k: False)
+    apart = run()
+    assert len(used) == n_used
+    assert set(in_place) == set(apart)
+    for name, g in in_place.items():
+        assert torch.equal(g, apart[name]), name
+
+
+def test_kernels_over_token_tensors_touch_only_their_rows_and_refuse_other_layouts():
+    from boost_and_broadside_amd import ops
+
+    T, B, n, NM, D = 9, 5, 3, 7, 128
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    b1 = torch.randn(T, B, NM, D, device=DEV, generator=gen).bfloat16()
+    buf = torch.randn(B * n, 3, D, device=DEV, generator=gen)
+    w = 0.5 * torch.randn(D, 1, 4, device=DEV, generator=gen)
+    bias = 0.1 * torch.randn(D, device=DEV, generator=gen)
+    done = torch.rand(B * n, T, device=DEV, generator=gen) < 0.2
+    ships = b1[:, :, :n].reshape(T, B * n, D).contiguous()
+    want = ops.conv_seq(ships, buf, w, bias, done, time_major=True, also_bf16=True)
+    got = ops.conv_seq(b1, buf, w, bias, done, time_major=True, also_bf16=True, token_rows=n)
+    assert all(torch.equal(a, b) for a, b in zip(got, want))
+    # the recurrence writes its states into the first n tokens and leaves the others as they were
+    gates = torch.randn(T, B * n, 2 * D, device=DEV, generator=gen).bfloat16()
+    lam = torch.linspace(0, 4, D, device=DEV)
+    h0 = torch.randn(B * n, D, device=DEV, generator=gen)
+    y_want, h_want = ops.rglru_scan(want[0], gates, lam, 8.0, h0, done, time_major=True)
+    tokens = torch.full((T, B, NM, D), 7.0, device=DEV)
+    y_got, h_got = ops.rglru_scan(want[0], gates, lam, 8.0, h0, done, time_major=True, y_tokens=(tokens, n))
+    assert y_got is tokens and torch.equal(h_got, h_want)
+    assert torch.equal(tokens[:, :, :n].reshape(T, B * n, D), y_want) and bool((tokens[:, :, n:] == 7.0).all())
+    # backward kernels: gradients of the ship rows from / into token tensors, the other rows untouched
+    dy_tok = torch.randn(T, B, NM, D, device=DEV, generator=gen)
+    dh = torch.randn(B * n, D, device=DEV, generator=gen)
+    a = ops.rglru_scan_bwd(want[0], gates, lam, 8.0, h0, done, tokens, dy_tok, dh, time_major=True, token_rows=n)
+    b = ops.rglru_scan_bwd(want[0], gates, lam, 8.0, h0, done, y_want, dy_tok[:, :, :n].reshape(T, B * n, D).contiguous(), dh,
+                           time_major=True)
+    assert all(torch.equal(p, q) for p, q in zip(a, b))
+    dv = torch.randn(T, B * n, D, device=DEV, generator=gen)
+    db1_tok = torch.full((T, B, NM, D), 3.0, device=DEV).bfloat16()
+    c = ops.conv_seq_bwd(b1, buf, w, done, dv, None, time_major=True, token_rows=n, db1_out=db1_tok)
+    d = ops.conv_seq_bwd(ships, buf, w, done, dv, None, time_major=True)
+    assert c[0] is db1_tok and torch.equal(db1_tok[:, :, :n].reshape(T, B * n, D), d[0]) and bool((db1_tok[:, :, n:] == 3.0).all())
+    assert all(torch.equal(p, q) for p, q in zip(c[1:], d[1:]))
+    with pytest.raises(ValueError):
+        ops.conv_seq(b1, buf, w, bias, done, token_rows=n)  # batch-major
+    with pytest.raises(ValueError):
+        ops.conv_seq(b1, buf, w, bias, done, time_major=True, token_rows=NM + 1)
+    with pytest.raises(ValueError):
+        ops.conv_seq(b1.transpose(1, 2), buf, w, bias, done, time_major=True, token_rows=n)
+
+
 def test_trunk_stepper_picks_the_captured_step_for_small_batches_and_both_kinds_agree():
     D, H, N, M = 128, 4, 8, 4
     p = trunk_params(81, D, 2, 2, 1)
