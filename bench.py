@@ -48,6 +48,9 @@ def parse_args():
     ap.add_argument("--no-team-pool", action="store_true", help="skip the team pooling leg")
     ap.add_argument("--no-fp32-attention", action="store_true", help="skip the float32 attention leg")
     ap.add_argument("--no-trunk", action="store_true", help="skip the whole-trunk leg (2 blocks x (2 spatial + 1 temporal))")
+    ap.add_argument("--only-update-step", action="store_true",
+                    help="run nothing but the update-path block step (forward + backward from a given gradient, T = 128 x 256 "
+                         "environments of 4v4) a few times and print its time: the command a kernel trace of one step is taken from")
     return ap.parse_args()
 
 
@@ -308,6 +311,37 @@ def load_traffic(kernel, workload):
     return None if entry is None else entry["total_bytes"]
 
 
+def only_update_step():
+    """One YemongBlock (2 attention + 1 temporal sublayer) forward + backward over a stored 4v4 rollout, as the
+    `update_path` leg times it, and nothing else: `--only-update-step` under a kernel trace lists one step's launches."""
+    import boost_and_broadside_amd as bnb
+    from boost_and_broadside_amd import harness
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    H, D = harness.N_HEADS, harness.D_MODEL
+    gen = torch.Generator(device=dev).manual_seed(1234)
+    torch.manual_seed(1234)
+    blk = bnb.YemongBlock(bnb.ModelConfig(d_model=D, n_heads=H, n_yemong_blocks=1, n_spatial_per_block=2,
+                                          n_temporal_per_block=1)).to(dev)
+    Tu, Bu, Nu, Mu = 128, 256, 8, 4
+    xu = torch.randn(Tu, Bu, Nu + Mu, D, device=dev, generator=gen)
+    au = torch.rand(Tu, Bu, Nu + Mu, device=dev, generator=gen) < 0.9
+    hu = torch.zeros(1, Bu * Nu, D, device=dev)
+    cu = torch.zeros(1, Bu * Nu, 3, D, device=dev)
+    du = torch.rand(Tu, Bu, device=dev, generator=gen) < 0.02
+    go = torch.randn(Tu, Bu, Nu + Mu, D, device=dev, generator=gen)
+
+    def step(t):
+        blk.zero_grad(set_to_none=True)
+        with torch.enable_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+            out = blk.sequence(xu, au, hu, cu, du, num_recurrent=Nu)[0]
+        out.backward(go)
+
+    ms = timed_loop(step, 4, 3) / 4 * 1e3
+    print(json.dumps({"leg": "update_step", "rows": Tu * Bu * (Nu + Mu), "block_fwd_bwd_given_grad_ms": ms, "steps": 4, "warmup": 3}))
+
+
 def main():
     args = parse_args()
     world = int(os.environ.get("WORLD_SIZE", "1"))
@@ -326,6 +360,9 @@ def main():
     from boost_and_broadside_amd import harness, ops
 
     bnb._native.load()
+    if args.only_update_step:
+        only_update_step()
+        return
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     w = harness.WORKLOADS[args.workload or harness.HEADLINE]
