@@ -1515,6 +1515,21 @@ def test_kernels_over_token_tensors_touch_only_their_rows_and_refuse_other_layou
         ops.conv_seq(b1, buf, w, bias, done, time_major=True, token_rows=NM + 1)
     with pytest.raises(ValueError):
         ops.conv_seq(b1.transpose(1, 2), buf, w, bias, done, time_major=True, token_rows=n)
+    # the C entry points refuse a placement that is not time-major, a pitch below the group, rows that are no multiple of it
+    from boost_and_broadside_amd import _native
+
+    lib = _native.load()
+    v = torch.empty(T, B * n, D, device=DEV)
+    nb = torch.empty(B * n, 3, D, device=DEV)
+    w4 = w.reshape(D, 4).contiguous()
+
+    def conv(time_major, group, pitch, rows=B * n):
+        return lib.bnb_conv_seq_fwd(b1.data_ptr(), _native.BF16, buf.data_ptr(), 3 * D, w4.data_ptr(), bias.data_ptr(), None,
+                                    v.data_ptr(), None, nb.data_ptr(), 3 * D, rows, T, D, time_major, group, pitch, None)
+
+    assert conv(1, n, NM) == 0
+    for bad in ((0, n, NM), (1, n, n - 1), (1, 0, NM), (1, 2, NM)):  # B * n = 15 rows are no multiple of 2
+        assert conv(*bad) == 10003, bad
 
 
 def test_trunk_stepper_picks_the_captured_step_for_small_batches_and_both_kinds_agree():
