@@ -199,6 +199,29 @@ __global__ __launch_bounds__(kValuThreads) void sdpa_valu_kernel(
 constexpr int kDh = 32;
 constexpr int kKeyPitch = kDh + 8;  // halfs per K row in LDS: 80 bytes, 16-byte aligned, bank-spread
 
+// The A operand of O^T = V^T P^T (per lane eight keys of ONE channel) out of ROW-MAJOR V rows in LDS (32 channels = 64
+// bytes per key, keys dense): ds_read_b64_tr_b16 hands lane i of a group of 16 lanes element i%4 of the 8-byte pieces
+// that lanes i/4, i/4 + 4, i/4 + 8, i/4 + 12 of the group address.  As SOURCE lane r = lane%16 of group g = lane/16 a
+// lane therefore points at key 4 (g/2) + r/4 of the 16 keys of one product and at the four channels of output-row
+// block rb = 4 (g%2) + r%4; MFMA row 8i + 4 half + j is channel 16 (i/2) + 8 half + 4 (i%2) + j (the output stage's
+// order), i.e. row block rb is channel block 4 (rb/4) + 2 (rb%2) + (rb/2)%2.  No transposed copy of V is written.
+__device__ __forceinline__ int v_tr_offset(int lane)
+{
+    const int grp = lane >> 4, r = lane & 15;
+    const int rb = 4 * (grp & 1) + (r & 3);
+    const int cb = 4 * (rb >> 2) + 2 * (rb & 1) + ((rb >> 1) & 1);
+    return (4 * (grp >> 1) + (r >> 2)) * kDh + cb * 4;  // halfs; + 16 t + 32 kb keys, + 8 keys for the operand's second half
+}
+
+__device__ __forceinline__ bf16x8 v_tr_operand(const uint16_t *p)
+{
+    typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+    typedef bf16x4_t __attribute__((address_space(3))) * lds_ptr;
+    const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_ptr)p);
+    const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_ptr)(p + 8 * kDh));
+    return bf16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+}
+
 // One work-group per (environment, head); wave w owns queries 32w .. 32w+31 and all waves
 // share the K rows and the transposed V rows of the live keys in LDS.
 //
@@ -825,10 +848,9 @@ __global__ __launch_bounds__(kWave *(NQB < 4 ? NQB : 4), 3) void sdpa_cross_stre
     constexpr bool SPLIT = NQB > NW;       // a fifth block of queries, shared by the four waves
     static_assert(NQB <= 5, "at most one shared block of queries");
     constexpr int TK = 32 * NW;   // keys per tile
-    constexpr int VP = TK + 4;    // halfs per V^T row: 8-byte aligned, bank-spread
     constexpr int NT = kWave * NW;
     __shared__ __align__(16) uint16_t s_k[2][TK * kKeyPitch];
-    __shared__ __align__(16) uint16_t s_vt[2][kDh * VP];
+    __shared__ __align__(16) uint16_t s_v[2][TK * kDh];  // V rows as they come, 64 bytes per key
     __shared__ uint16_t s_idx[kStreamMaxKeys];  // indices of the live keys, ascending
     __shared__ int s_wcnt[NW];
     static_assert(!SPLIT || sizeof(s_k) >= (size_t)NW * (16 * kWave + 3 * 32) * sizeof(float),
@@ -955,15 +977,7 @@ __global__ __launch_bounds__(kWave *(NQB < 4 ? NQB : 4), 3) void sdpa_cross_stre
                 const u32x4 vv = li >= 0 ? vw[it] : zero4;
                 const int c8 = (tid & 3) * 8;
                 *reinterpret_cast<u32x4 *>(&s_k[buf][lp * kKeyPitch + c8]) = kk;
-                uint16_t *dst = &s_vt[buf][(16 * (c8 >> 4) + 4 * ((c8 >> 3) & 1)) * VP + lp];
-                dst[0 * VP] = (uint16_t)(vv.x & 0xffffu);
-                dst[1 * VP] = (uint16_t)(vv.x >> 16);
-                dst[2 * VP] = (uint16_t)(vv.y & 0xffffu);
-                dst[3 * VP] = (uint16_t)(vv.y >> 16);
-                dst[8 * VP] = (uint16_t)(vv.z & 0xffffu);
-                dst[9 * VP] = (uint16_t)(vv.z >> 16);
-                dst[10 * VP] = (uint16_t)(vv.w & 0xffffu);
-                dst[11 * VP] = (uint16_t)(vv.w >> 16);
+                *reinterpret_cast<u32x4 *>(&s_v[buf][lp * kDh + c8]) = vv;
             }
         }
     };
@@ -991,6 +1005,7 @@ __global__ __launch_bounds__(kWave *(NQB < 4 ? NQB : 4), 3) void sdpa_cross_stre
     // +-60 in log2 units, or not finite), the whole work-group throws the try away and walks the tiles again in the
     // second form, an online softmax with the running maximum as shift (two sweeps per tile).
     const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    const int v_off = v_tr_offset(lane);
     float esum = 0.0f, sesum = 0.0f;  // the weights before rounding, for the log-sum-exp a backward pass asks for (LSE)
     auto walk = [&](auto shifted) {
         constexpr bool SHIFT = decltype(shifted)::value;
@@ -1043,11 +1058,8 @@ __global__ __launch_bounds__(kWave *(NQB < 4 ? NQB : 4), 3) void sdpa_cross_stre
                     for (int e = 0; e < 8; ++e) pb[e] = (__bf16)p[8 * h2 + e];
 #pragma unroll
                     for (int e = 0; e < 8; e += 2) total = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{pb[e], pb[e + 1]}, ones, total, false);
-                    const uint16_t *vp = &s_vt[buf][m * VP + kb * 32 + 16 * h2 + 4 * half];
-                    const u32x2 lo = *reinterpret_cast<const u32x2 *>(vp);
-                    const u32x2 hi = *reinterpret_cast<const u32x2 *>(vp + 8);
-                    const u32x4 vq = {lo.x, lo.y, hi.x, hi.y};
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vq), pb, acc, 0, 0, 0);
+                    const bf16x8 va = v_tr_operand(&s_v[buf][(kb * 32 + 16 * h2) * kDh + v_off]);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb, acc, 0, 0, 0);
                 }
             };
             auto weigh = [&](int kb, const f32x16 &z, float mc) { weigh_into(kb, z, mc, sum, esum, o); };
