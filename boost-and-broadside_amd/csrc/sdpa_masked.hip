@@ -238,10 +238,9 @@ __global__ __launch_bounds__(kWave * NKB) __attribute__((amdgpu_waves_per_eu(8, 
     const uint16_t *accum, uint16_t *out, int B, int NQ, int NK, int H, float scale_log2e)
 {
     constexpr int KCAP = NKB * 32;
-    constexpr int VP = KCAP + 4;  // halfs per V^T row: 8-byte aligned, bank-spread
     constexpr int NT = kWave * NKB;
     __shared__ __align__(16) uint16_t s_k[KCAP * kKeyPitch];
-    __shared__ __align__(16) uint16_t s_vt[kDh * VP];
+    __shared__ __align__(16) uint16_t s_v[KCAP * kDh];  // V rows as they come, 64 bytes per key (see v_tr_offset)
     __shared__ uint16_t s_cnt[2 * NKB];  // live keys per 16-key slice, in key order
 
     // Work-groups are dealt round-robin to the 8 XCDs; hand each XCD a contiguous run of
@@ -330,16 +329,7 @@ __global__ __launch_bounds__(kWave * NKB) __attribute__((amdgpu_waves_per_eu(8, 
                 const int pos = (((cnt + 31) & ~31) - cnt) + (it ? base1 : base0) + before[it];
                 const int c8 = (tid & 3) * 8;
                 *reinterpret_cast<u32x4 *>(s_k + pos * kKeyPitch + c8) = kw[it];
-                // channel d = c8 + e goes to V^T row vt_row(d) (see the output stage)
-                uint16_t *dst = s_vt + (16 * (c8 >> 4) + 4 * ((c8 >> 3) & 1)) * VP + pos;
-                dst[0 * VP] = (uint16_t)(vw[it].x & 0xffffu);
-                dst[1 * VP] = (uint16_t)(vw[it].x >> 16);
-                dst[2 * VP] = (uint16_t)(vw[it].y & 0xffffu);
-                dst[3 * VP] = (uint16_t)(vw[it].y >> 16);
-                dst[8 * VP] = (uint16_t)(vw[it].z & 0xffffu);
-                dst[9 * VP] = (uint16_t)(vw[it].z >> 16);
-                dst[10 * VP] = (uint16_t)(vw[it].w & 0xffffu);
-                dst[11 * VP] = (uint16_t)(vw[it].w >> 16);
+                *reinterpret_cast<u32x4 *>(s_v + pos * kDh + c8) = vw[it];
             }
         }
         if (cnt != 0 || CROSS) break;
@@ -353,8 +343,7 @@ __global__ __launch_bounds__(kWave * NKB) __attribute__((amdgpu_waves_per_eu(8, 
         const int pos = idx >> 2;
         const int c8 = (idx & 3) * 8;
         *reinterpret_cast<u32x4 *>(s_k + pos * kKeyPitch + c8) = u32x4{0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int e = 0; e < 8; ++e) s_vt[(c8 + e) * VP + pos] = 0;
+        *reinterpret_cast<u32x4 *>(s_v + pos * kDh + c8) = u32x4{0u, 0u, 0u, 0u};
     }
     __syncthreads();
     if (wave * 32 >= NQ) return;  // waves that only helped staging (more key blocks than query blocks)
@@ -391,6 +380,7 @@ __global__ __launch_bounds__(kWave * NKB) __attribute__((amdgpu_waves_per_eu(8, 
     float sum = 0.0f;
     f32x16 o = {0.0f};
     const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    const int v_off = v_tr_offset(lane);
     auto sweep = [&](auto shifted, float mc, int pad_rows) {
         sum = 0.0f;
 #pragma unroll
@@ -412,11 +402,8 @@ __global__ __launch_bounds__(kWave * NKB) __attribute__((amdgpu_waves_per_eu(8, 
                 // instruction: a query with one live key then gets that key's value row back exactly
 #pragma unroll
                 for (int e = 0; e < 8; e += 2) sum = __builtin_amdgcn_fdot2_f32_bf16(bf16x2{pb[e], pb[e + 1]}, ones, sum, false);
-                const uint16_t *vp = s_vt + m * VP + kb * 32 + 16 * t + 4 * half;
-                const u32x2 lo = *reinterpret_cast<const u32x2 *>(vp);
-                const u32x2 hi = *reinterpret_cast<const u32x2 *>(vp + 8);
-                const u32x4 vw = {lo.x, lo.y, hi.x, hi.y};
-                o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vw), pb, o, 0, 0, 0);
+                const bf16x8 va = v_tr_operand(s_v + (kb * 32 + 16 * t) * kDh + v_off);
+                o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb, o, 0, 0, 0);
             }
         }
         sum += __shfl_xor(sum, 32);

@@ -21,6 +21,7 @@ namespace bnb {
 constexpr int kSeqThreads = 256;
 constexpr int kSeqTaps = 4;
 constexpr int kSeqAhead = 4;  // timesteps whose operands are in flight together
+constexpr int kScalarAhead = 16;  // the same for the forward one-lane-per-channel forms (few waves per SIMD there: more steps per lane)
 
 // A time-major tensor may hold this call's rows inside a wider token tensor (T, environments * pitch, D): the rows of
 // environment b are then rows b * pitch .. b * pitch + group - 1 of every step (group == 0: the tensor holds this
@@ -111,11 +112,11 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_scalar_kernel(
     const GT *gp = gates + row * 2 * rs + d;
     YT *yp = y + placed_row(row, y_group, y_pitch) * rs + d;
     const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
-    for (int t0 = 0; t0 < T; t0 += kSeqAhead) {
-        float xv[kSeqAhead], ga[kSeqAhead], gx[kSeqAhead];
-        uint32_t cut[kSeqAhead];
+    for (int t0 = 0; t0 < T; t0 += kScalarAhead) {
+        float xv[kScalarAhead], ga[kScalarAhead], gx[kScalarAhead];
+        uint32_t cut[kScalarAhead];
 #pragma unroll
-        for (int u = 0; u < kSeqAhead; ++u) {
+        for (int u = 0; u < kScalarAhead; ++u) {
             const int t = t0 + u < T ? t0 + u : T - 1;
             xv[u] = load1(xp + t * ts);
             ga[u] = load1(gp + t * 2 * ts);
@@ -125,7 +126,7 @@ __global__ __launch_bounds__(kSeqThreads) void rglru_scan_scalar_kernel(
             if (t == 0) cut[u] = 0;
         }
 #pragma unroll
-        for (int u = 0; u < kSeqAhead; ++u) {
+        for (int u = 0; u < kScalarAhead; ++u) {
             if (t0 + u < T) {
                 h = rglru_element<is_bf16<GT>::value, is_bf16<XT>::value>(xv[u], ga[u], gx[u], l2, c,
                                                                           cut[u] ? 0.0f : h);
@@ -529,20 +530,34 @@ __global__ __launch_bounds__(kSeqThreads) void conv_seq_scalar_kernel(
     const BT *bp = b1 + placed_row(row, b_group, b_pitch) * rs + d;
     const uint8_t *dn = done == nullptr ? nullptr : done + row * T;
     int hist = 3;
-    for (int t = 0; t < T; ++t) {
-        const float cur = load1(bp + t * ts_b);
-        if (dn != nullptr && t > 0 && dn[t - 1]) hist = 0;
-        float acc = (hist >= 3 ? p0 : 0.0f) * w0;
-        acc += (hist >= 2 ? p1 : 0.0f) * w1;
-        acc += (hist >= 1 ? p2 : 0.0f) * w2;
-        acc += cur * w3;
-        const float v = acc + bs;
-        v_out[row * rs + t * ts + d] = v;
-        if (v_bf16_out != nullptr) store1(v_bf16_out + row * rs + t * ts + d, v);
-        p0 = p1;
-        p1 = p2;
-        p2 = cur;
-        hist = hist < 3 ? hist + 1 : 3;
+    for (int t0 = 0; t0 < T; t0 += kScalarAhead) {
+        float in[kScalarAhead];
+        uint32_t cut[kScalarAhead];
+#pragma unroll
+        for (int u = 0; u < kScalarAhead; ++u) {
+            const int t = t0 + u < T ? t0 + u : T - 1;  // past the end: re-read the last step (discarded)
+            in[u] = load1(bp + t * ts_b);
+            cut[u] = (dn != nullptr && t > 0) ? dn[t - 1] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < kScalarAhead; ++u) {
+            const int t = t0 + u;
+            if (t < T) {
+                const float cur = in[u];
+                if (cut[u]) hist = 0;
+                float acc = (hist >= 3 ? p0 : 0.0f) * w0;
+                acc += (hist >= 2 ? p1 : 0.0f) * w1;
+                acc += (hist >= 1 ? p2 : 0.0f) * w2;
+                acc += cur * w3;
+                const float v = acc + bs;
+                v_out[row * rs + t * ts + d] = v;
+                if (v_bf16_out != nullptr) store1(v_bf16_out + row * rs + t * ts + d, v);
+                p0 = p1;
+                p1 = p2;
+                p2 = cur;
+                hist = hist < 3 ? hist + 1 : 3;
+            }
+        }
     }
     float *pout = conv_out + row * conv_out_stride + d;
     pout[0] = p0;
