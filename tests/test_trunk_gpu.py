@@ -1473,6 +1473,46 @@ def test_temporal_mix_in_place_of_split_and_concatenation_gives_the_same_bits(N,
         assert torch.equal(g, apart[name]), name
 
 
+@pytest.mark.parametrize("T,B,n,NM,D", [(5, 2048, 8, 12, 128), (3, 4100, 5, 6, 128), (6, 1100, 3, 4, 256), (7, 33, 2, 9, 64)])
+def test_kernels_over_token_tensors_equal_the_dense_calls_on_the_wide_lane_forms_too(T, B, n, NM, D):
+    """Enough rows for the eight-channels-per-lane kernels (and a few shapes of the one-lane-per-channel ones): the four
+    sequence kernels over the ship rows of a token tensor give the bits of the same calls on sliced copies."""
+    from boost_and_broadside_amd import ops
+
+    gen = torch.Generator(device=DEV).manual_seed(T * B + n)
+    R = B * n
+    b1 = torch.randn(T, B, NM, D, device=DEV, generator=gen).bfloat16()
+    buf = torch.randn(R, 3, D, device=DEV, generator=gen)
+    w = 0.5 * torch.randn(D, 1, 4, device=DEV, generator=gen)
+    bias = 0.1 * torch.randn(D, device=DEV, generator=gen)
+    done = torch.rand(R, T, device=DEV, generator=gen) < 0.2
+    ships = b1[:, :, :n].reshape(T, R, D).contiguous()
+    want = ops.conv_seq(ships, buf, w, bias, done, time_major=True, also_bf16=True)
+    got = ops.conv_seq(b1, buf, w, bias, done, time_major=True, also_bf16=True, token_rows=n)
+    assert all(torch.equal(a, b) for a, b in zip(got, want))
+    gates = torch.randn(T, R, 2 * D, device=DEV, generator=gen).bfloat16()
+    lam = torch.linspace(0, 4, D, device=DEV)
+    h0 = torch.randn(R, D, device=DEV, generator=gen)
+    y_want, h_want = ops.rglru_scan(want[0], gates, lam, 8.0, h0, done, time_major=True)
+    tokens = torch.full((T, B, NM, D), -3.0, device=DEV)
+    _, h_got = ops.rglru_scan(want[0], gates, lam, 8.0, h0, done, time_major=True, y_tokens=(tokens, n))
+    assert torch.equal(h_got, h_want) and torch.equal(tokens[:, :, :n].reshape(T, R, D), y_want)
+    assert bool((tokens[:, :, n:] == -3.0).all())
+    dy_tok = torch.randn(T, B, NM, D, device=DEV, generator=gen)
+    dh = torch.randn(R, D, device=DEV, generator=gen)
+    a = ops.rglru_scan_bwd(want[0], gates, lam, 8.0, h0, done, tokens, dy_tok, dh, time_major=True, token_rows=n)
+    b = ops.rglru_scan_bwd(want[0], gates, lam, 8.0, h0, done, y_want, dy_tok[:, :, :n].reshape(T, R, D).contiguous(), dh,
+                           time_major=True)
+    assert all(torch.equal(p, q) for p, q in zip(a, b))
+    dv = torch.randn(T, R, D, device=DEV, generator=gen)
+    dv_lp = torch.randn(T, R, D, device=DEV, generator=gen).bfloat16()
+    db1_tok = torch.full((T, B, NM, D), 3.0, device=DEV).bfloat16()
+    c = ops.conv_seq_bwd(b1, buf, w, done, dv, None, time_major=True, dv_bf16=dv_lp, token_rows=n, db1_out=db1_tok)
+    d = ops.conv_seq_bwd(ships, buf, w, done, dv, None, time_major=True, dv_bf16=dv_lp)
+    assert torch.equal(db1_tok[:, :, :n].reshape(T, R, D), d[0]) and bool((db1_tok[:, :, n:] == 3.0).all())
+    assert all(torch.equal(p, q) for p, q in zip(c[1:], d[1:]))
+
+
 def test_kernels_over_token_tensors_touch_only_their_rows_and_refuse_other_layouts():
     from boost_and_broadside_amd import ops
 
